@@ -1,0 +1,47 @@
+"""Builds libhemm.so (HIP kernels + C ABI + C++ host layer) for gfx950 with hipcc, in-tree."""
+import glob
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libhemm.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wno-unused-value",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def sources():
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "host", "*.cpp")))
+
+
+def _compile(src):
+    obj = os.path.splitext(src)[0] + ".o"
+    cmd = [HIPCC] + FLAGS + ["-I", os.path.join(HERE, "..", "include"), "-I", CSRC, "-c", src, "-o", obj]
+    if src.endswith(".cpp"):
+        cmd = [HIPCC] + FLAGS + ["-x", "hip", "-I", os.path.join(HERE, "..", "include"), "-I", CSRC,
+                                 "-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    return obj
+
+
+def build(verbose=False):
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        objs = list(ex.map(_compile, srcs))
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-o", LIB] + objs,
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)

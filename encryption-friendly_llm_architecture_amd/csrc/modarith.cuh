@@ -1,0 +1,78 @@
+// Device-side modular arithmetic for RNS primes below 2^61 on gfx950.
+//
+// gfx950 has no 64x64->128 multiplier: every 64-bit product below is assembled by the
+// compiler from 32-bit v_mad_u64_u32 / v_mul_hi_u32 pieces, so the code is written to keep
+// the number of wide products per modular multiplication minimal:
+//   * constant multiplicands (NTT twiddles, 1/N, P^-1, q_l^-1, basis-conversion factors) carry a
+//     precomputed Shoup quotient floor(w * 2^64 / q): one high product + two low products;
+//   * data x data products are kept as 128-bit values, summed lazily, and reduced once with a
+//     Barrett step sized to the prime's bit length.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef unsigned long long u64;
+typedef unsigned int u32;
+
+struct u128_t {
+    u64 lo, hi;
+};
+
+__device__ __forceinline__ u128_t mul64wide(u64 a, u64 b) {
+    u128_t r;
+    r.lo = a * b;
+    r.hi = __umul64hi(a, b);
+    return r;
+}
+__device__ __forceinline__ void add128(u128_t &acc, const u128_t &x) {
+    u64 lo = acc.lo + x.lo;
+    acc.hi += x.hi + (lo < acc.lo ? 1ull : 0ull);
+    acc.lo = lo;
+}
+
+// Per-prime constants, passed to kernels by value or read from a small device table.
+struct ModQ {
+    u64 q;     // the prime
+    u64 mu;    // floor(2^(2k) / q), k = bit length of q
+    u32 k;     // bit length of q (q < 2^k, k <= 61)
+    u32 pad;
+};
+
+// x * w mod q for a constant w with ws = floor(w * 2^64 / q); result in [0, 2q).
+__device__ __forceinline__ u64 mul_shoup_lazy(u64 x, u64 w, u64 ws, u64 q) {
+    return x * w - __umul64hi(x, ws) * q;
+}
+__device__ __forceinline__ u64 mul_shoup(u64 x, u64 w, u64 ws, u64 q) {
+    u64 r = mul_shoup_lazy(x, w, ws, q);
+    return r >= q ? r - q : r;
+}
+
+// Barrett reduction of a 128-bit value T < 6 * 2^(2k) to [0, q).
+__device__ __forceinline__ u64 barrett128(u128_t t, const ModQ &m) {
+    const u32 k = m.k;
+    u64 t1 = (t.hi << (65 - k)) | (t.lo >> (k - 1));
+    u128_t p = mul64wide(t1, m.mu);
+    u64 qhat = (p.hi << (63 - k)) | (p.lo >> (k + 1));
+    u64 r = t.lo - qhat * m.q;
+    const u64 q = m.q;
+    if (r >= 4 * q) r -= 4 * q;
+    if (r >= 2 * q) r -= 2 * q;
+    if (r >= q) r -= q;
+    return r;
+}
+__device__ __forceinline__ u64 mulmod(u64 a, u64 b, const ModQ &m) {
+    return barrett128(mul64wide(a, b), m);
+}
+// reduce an arbitrary 64-bit value
+__device__ __forceinline__ u64 reduce64(u64 a, const ModQ &m) {
+    u128_t t;
+    t.lo = a;
+    t.hi = 0;
+    return barrett128(t, m);
+}
+__device__ __forceinline__ u64 addmod(u64 a, u64 b, u64 q) {
+    u64 s = a + b;
+    return s >= q ? s - q : s;
+}
+__device__ __forceinline__ u64 submod(u64 a, u64 b, u64 q) { return a >= b ? a - b : a + q - b; }
+__device__ __forceinline__ u64 negmod(u64 a, u64 q) { return a ? q - a : 0; }

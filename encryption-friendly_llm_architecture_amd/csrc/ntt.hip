@@ -1,0 +1,327 @@
+// Batched negacyclic NTT / INTT over RNS primes < 2^61 for gfx950.
+//
+// Forward: merged-twiddle Cooley-Tukey, natural order in, bit-reversed order out
+//   out[k] = sum_j a[j] psi^{(2 bitrev(k)+1) j};  inverse: Gentleman-Sande with the 1/N factor.
+// Twiddle table per prime: tw[i] = (psi^bitrev(i), floor(that * 2^64 / q)) as one 16-byte entry.
+//
+// N = 2^16 does not fit a CU's LDS (512 KiB per limb), so a transform is two launches over the
+// 256 x 256 view  index = r*256 + c:
+//   forward pass 1: stages 0..7  act down columns  (butterfly distance >= 256)
+//   forward pass 2: stages 8..15 act inside rows   (distance <= 128)
+// and mirrored for the inverse.  Each workgroup (256 threads = 4 wavefronts) owns a 16-column
+// (or 16-row) slab; a thread keeps 16 residues in registers, runs a radix-16 block (4 stages)
+// on them, swaps through LDS once and runs the second radix-16 block.  All global accesses
+// are 128-byte row segments shared by 16 adjacent lanes.
+//
+// Other sizes (2^6 .. 2^15, used by the small-parameter tests) run a plain LDS kernel with the
+// same butterfly network, so residues are identical for every N.
+#include "hemm_internal.hpp"
+
+namespace {
+
+struct __align__(16) Tw {
+    u64 w, ws;
+};
+
+__device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q2) {
+    u64 u = x;
+    if (u >= q2) u -= q2;
+    u64 v = mul_shoup_lazy(y, tw.w, tw.ws, q);
+    x = u + v;
+    y = u - v + q2;
+}
+__device__ __forceinline__ void gs_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q2) {
+    u64 u = x, v = y;
+    u64 s = u + v;
+    if (s >= q2) s -= q2;
+    x = s;
+    y = mul_shoup_lazy(u - v + q2, tw.w, tw.ws, q);
+}
+
+// ------------------------------------------------------------------------------------------
+// generic LDS kernel: tile [R rows][CW cols], global index = r*rowstride + c0 + cc
+// ------------------------------------------------------------------------------------------
+struct GenericPass {
+    int logN;
+    int R, CW;          // tile shape (powers of two)
+    int rowstride;      // distance between tile rows in the limb
+    int s_begin, s_end; // forward: stages s_begin..s_end-1 ascending; inverse: descending
+    int tiles_per_limb;
+    int first, last;    // first / last pass of the transform
+};
+
+template <bool INV>
+__global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                          const ModQ *__restrict__ modq,
+                                                          const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
+                                                          LimbList ll, int n_limbs, size_t poly_stride,
+                                                          GenericPass gp) {
+    extern __shared__ u64 lds[];
+    const int N = 1 << gp.logN;
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + (size_t)prime * N;
+    const u64 q = modq[prime].q, q2 = 2 * q;
+    u64 *base = data + (size_t)poly * poly_stride + (size_t)limb * N;
+    const int tile = blockIdx.x;
+    // tile origin: strided pass tiles walk the columns; contiguous pass tiles walk the limb
+    const int c0 = (gp.rowstride == 1) ? tile * gp.R * gp.CW : tile * gp.CW;
+    const int elems = gp.R * gp.CW;
+    for (int e = threadIdx.x; e < elems; e += blockDim.x) {
+        int r = e / gp.CW, cc = e % gp.CW;
+        lds[e] = base[(size_t)r * gp.rowstride + c0 + cc];
+    }
+    __syncthreads();
+    const int half = elems / 2;
+    if (!INV) {
+        for (int s = gp.s_begin; s < gp.s_end; s++) {
+            const int t = N >> (s + 1);
+            const int tr = t / gp.rowstride;  // row distance inside the tile
+            for (int b = threadIdx.x; b < half; b += blockDim.x) {
+                int cc = b % gp.CW, rb = b / gp.CW;
+                int r = (rb / tr) * 2 * tr + rb % tr;
+                int i = r * gp.CW + cc, j = i + tr * gp.CW;
+                int gidx = r * gp.rowstride + c0 + cc;
+                Tw w = tw[(1 << s) + (gidx / (2 * t))];
+                u64 x = lds[i], y = lds[j];
+                ct_bfly(x, y, w, q, q2);
+                lds[i] = x;
+                lds[j] = y;
+            }
+            __syncthreads();
+        }
+    } else {
+        for (int s = gp.s_begin - 1; s >= gp.s_end; s--) {
+            const int t = N >> (s + 1);
+            const int tr = t / gp.rowstride;
+            for (int b = threadIdx.x; b < half; b += blockDim.x) {
+                int cc = b % gp.CW, rb = b / gp.CW;
+                int r = (rb / tr) * 2 * tr + rb % tr;
+                int i = r * gp.CW + cc, j = i + tr * gp.CW;
+                int gidx = r * gp.rowstride + c0 + cc;
+                Tw w = tw[(1 << s) + (gidx / (2 * t))];
+                u64 x = lds[i], y = lds[j];
+                gs_bfly(x, y, w, q, q2);
+                lds[i] = x;
+                lds[j] = y;
+            }
+            __syncthreads();
+        }
+    }
+    const u64 ni = ninv[prime], nis = ninv_s[prime];
+    for (int e = threadIdx.x; e < elems; e += blockDim.x) {
+        int r = e / gp.CW, cc = e % gp.CW;
+        u64 v = lds[e];
+        if (gp.last) {
+            if (INV) {
+                v = mul_shoup_lazy(v, ni, nis, q);
+            } else if (v >= q2)
+                v -= q2;
+            if (v >= q) v -= q;
+        }
+        base[(size_t)r * gp.rowstride + c0 + cc] = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// N = 2^16 kernels
+// ------------------------------------------------------------------------------------------
+// radix-16 block of 4 Cooley-Tukey stages on registers; stage s, group g uses twiddle
+// (X << s) + g.
+__device__ __forceinline__ void radix16_fwd(u64 (&x)[16], const Tw *__restrict__ tw, const u32 X, const u64 q) {
+    const u64 q2 = 2 * q;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int d = 8 >> s;
+#pragma unroll
+        for (int g = 0; g < (1 << s); g++) {
+            const Tw w = tw[(X << s) + g];
+#pragma unroll
+            for (int j = 0; j < d; j++) ct_bfly(x[g * 2 * d + j], x[g * 2 * d + j + d], w, q, q2);
+        }
+    }
+}
+// radix-16 block of 4 Gentleman-Sande stages; stage s (distance 1<<s), group g uses twiddle
+// (X << (3-s)) + g.
+__device__ __forceinline__ void radix16_inv(u64 (&x)[16], const Tw *__restrict__ tw, const u32 X, const u64 q) {
+    const u64 q2 = 2 * q;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int d = 1 << s;
+#pragma unroll
+        for (int g = 0; g < (8 >> s); g++) {
+            const Tw w = tw[(X << (3 - s)) + g];
+#pragma unroll
+            for (int j = 0; j < d; j++) gs_bfly(x[g * 2 * d + j], x[g * 2 * d + j + d], w, q, q2);
+        }
+    }
+}
+
+#define ROWPAD 272  // 256 residues of a row + one pad word per 16, so a 16-lane column read
+                    // (stride 17 words) hits 16 distinct bank pairs
+__device__ __forceinline__ int padc(int c) { return c + (c >> 4); }
+
+// forward pass 1 / inverse pass 2 work on a 256-row x 16-column slab.
+template <bool INV>
+__global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                         const ModQ *__restrict__ modq,
+                                                         const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
+                                                         LimbList ll, int n_limbs, size_t poly_stride) {
+    __shared__ u64 lds[256 * 16];
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const u64 q = modq[prime].q;
+    const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
+    u64 *base = data + (size_t)poly * poly_stride + ((size_t)limb << 16) + blockIdx.x * 16 + cc;
+    u64 x[16];
+    if (!INV) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = base[(size_t)(rh + 16 * k) << 8];
+        radix16_fwd(x, tw, 1u, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) lds[(rh + 16 * k) * 16 + cc] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = lds[(16 * rh + k) * 16 + cc];
+        radix16_fwd(x, tw, 16u + rh, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) base[(size_t)(16 * rh + k) << 8] = x[k];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = base[(size_t)(16 * rh + k) << 8];
+        radix16_inv(x, tw, 16u + rh, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) lds[(16 * rh + k) * 16 + cc] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = lds[(rh + 16 * k) * 16 + cc];
+        radix16_inv(x, tw, 1u, q);
+        const u64 ni = ninv[prime], nis = ninv_s[prime];
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            u64 v = mul_shoup_lazy(x[k], ni, nis, q);
+            if (v >= q) v -= q;
+            base[(size_t)(rh + 16 * k) << 8] = v;
+        }
+    }
+}
+
+// forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
+template <bool INV>
+__global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                         const ModQ *__restrict__ modq, LimbList ll, int n_limbs,
+                                                         size_t poly_stride) {
+    __shared__ u64 lds[16 * ROWPAD];
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const u64 q = modq[prime].q, q2 = 2 * q;
+    const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
+    const u32 r = blockIdx.x * 16 + rr;  // global row
+    u64 *row = data + (size_t)poly * poly_stride + ((size_t)limb << 16) + ((size_t)r << 8);
+    u64 *l = lds + rr * ROWPAD;
+    u64 x[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = row[c + 16 * k];
+    if (!INV) {
+        radix16_fwd(x, tw, 256u + r, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
+        radix16_fwd(x, tw, 16u * (256u + r) + c, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            u64 v = x[k];
+            if (v >= q2) v -= q2;
+            if (v >= q) v -= q;
+            x[k] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) row[c + 16 * k] = l[padc(c + 16 * k)];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
+        radix16_inv(x, tw, 16u * (256u + r) + c, q);
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = l[padc(c + 16 * k)];
+        radix16_inv(x, tw, 256u + r, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) row[c + 16 * k] = x[k];
+    }
+}
+
+}  // namespace
+
+void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
+                size_t poly_stride, bool inverse, hipStream_t s) {
+    if (n_limbs <= 0 || n_polys <= 0) return;
+    const Tw *tw = (const Tw *)(inverse ? c->d_iw : c->d_w);
+    const int lanes = n_limbs * n_polys;
+    if (c->logN == 16) {
+        dim3 grid(16, lanes), block(256);
+        if (!inverse) {
+            hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
+                               c->d_ninv_s, ll, n_limbs, poly_stride);
+            hipLaunchKernelGGL(ntt16_rows_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, ll, n_limbs,
+                               poly_stride);
+        } else {
+            hipLaunchKernelGGL(ntt16_rows_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, ll, n_limbs,
+                               poly_stride);
+            hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
+                               c->d_ninv_s, ll, n_limbs, poly_stride);
+        }
+        return;
+    }
+    // generic path
+    const int logN = c->logN, N = c->N;
+    GenericPass A{}, B{};
+    int n_pass;
+    if (logN <= 12) {
+        n_pass = 1;
+        B.logN = logN; B.R = N; B.CW = 1; B.rowstride = 1; B.s_begin = 0; B.s_end = logN;
+        B.tiles_per_limb = 1;
+    } else {
+        n_pass = 2;
+        const int sA = logN - 8;                 // strided stages
+        A.logN = logN; A.R = 1 << sA; A.CW = (4096 >> sA) > 256 ? 256 : (4096 >> sA);
+        A.rowstride = 256; A.s_begin = 0; A.s_end = sA; A.tiles_per_limb = 256 / A.CW;
+        B.logN = logN; B.R = 4096; B.CW = 1; B.rowstride = 1; B.s_begin = sA; B.s_end = logN;
+        B.tiles_per_limb = N / 4096;
+    }
+    auto run = [&](GenericPass gp, bool first, bool last) {
+        gp.first = first; gp.last = last;
+        dim3 grid(gp.tiles_per_limb, lanes), block(256);
+        size_t sh = (size_t)gp.R * gp.CW * sizeof(u64);
+        if (!inverse)
+            hipLaunchKernelGGL(ntt_generic_kernel<false>, grid, block, sh, s, data, tw, c->d_modq, c->d_ninv,
+                               c->d_ninv_s, ll, n_limbs, poly_stride, gp);
+        else {
+            std::swap(gp.s_begin, gp.s_end);     // inverse walks stages downwards
+            hipLaunchKernelGGL(ntt_generic_kernel<true>, grid, block, sh, s, data, tw, c->d_modq, c->d_ninv,
+                               c->d_ninv_s, ll, n_limbs, poly_stride, gp);
+        }
+    };
+    if (n_pass == 1) {
+        run(B, true, true);
+    } else if (!inverse) {
+        run(A, true, false);
+        run(B, false, true);
+    } else {
+        run(B, true, false);
+        run(A, false, true);
+    }
+}
