@@ -45,6 +45,19 @@ def _declare(L):
     L.hemm_context_psi.argtypes = [vp, ctypes.c_uint32]
     L.hemm_primes_below.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, u64p]
     L.hemm_ntt.argtypes = [vp, vp, u32p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, vp]
+    sz, u32, u64, ci = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int
+    L.hemm_pointwise.argtypes = [vp, ci, vp, sz, vp, sz, vp, sz, u32, ci, u32, vp]
+    L.hemm_mul_scalar.argtypes = [vp, vp, sz, u64p, vp, sz, u32, ci, u32, vp]
+    L.hemm_mul_imag_unit.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
+    L.hemm_tensor.argtypes = [vp, vp, sz, vp, sz, vp, sz, u32, ci, vp]
+    L.hemm_automorphism.argtypes = [vp, vp, sz, vp, sz, u64, u32, u32, vp]
+    L.hemm_modup.argtypes = [vp, vp, u32, vp, vp]
+    L.hemm_inner_product.argtypes = [vp, vp, vp, u32, vp, vp]
+    L.hemm_moddown.argtypes = [vp, vp, u32, u32, vp, sz, vp]
+    L.hemm_keyswitch.argtypes = [vp, vp, vp, u32, vp, sz, vp, vp]
+    L.hemm_rotate.argtypes = [vp, vp, sz, vp, u64, u32, vp, sz, vp]
+    L.hemm_relinearize.argtypes = [vp, vp, sz, vp, u32, vp, sz, vp]
+    L.hemm_rescale.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
 
 
 def check(rc):
@@ -93,6 +106,110 @@ class Context:
         check(lib().hemm_ntt(self.h, vp(data.data_ptr()), idx, n_limbs, n_polys, int(inverse),
                              vp(stream or 0)))
         return data
+
+
+    # ---- evaluator-level kernels on [polys][limbs][N] int64 CUDA tensors ---------------------
+    def _new(self, polys, limbs, like):
+        import torch
+        return torch.empty((polys, limbs, self.N), dtype=torch.int64, device=like.device)
+
+    @staticmethod
+    def _ps(t):
+        return t.stride(0) if t.dim() == 3 else 0
+
+    def pointwise(self, op, a, b, nq, with_p=False, out=None, stream=None):
+        """a: [P][>=nl][N]; b: same or a single [>=nl][N] polynomial (broadcast)."""
+        nl = nq + (self.nP if with_p else 0)
+        polys = a.shape[0]
+        if out is None:
+            out = self._new(polys, nl, a)
+        check(lib().hemm_pointwise(self.h, op, vp(a.data_ptr()), self._ps(a),
+                                   vp(b.data_ptr() if b is not None else 0),
+                                   self._ps(b) if b is not None else 0, vp(out.data_ptr()),
+                                   self._ps(out), nq, int(with_p), polys, vp(stream or 0)))
+        return out
+
+    def mul_scalar(self, a, scalars, nq, with_p=False, out=None):
+        nl = nq + (self.nP if with_p else 0)
+        if out is None:
+            out = self._new(a.shape[0], nl, a)
+        arr = (ctypes.c_uint64 * nl)(*[int(v) for v in scalars])
+        check(lib().hemm_mul_scalar(self.h, vp(a.data_ptr()), self._ps(a), arr, vp(out.data_ptr()),
+                                    self._ps(out), nq, int(with_p), a.shape[0], vp(0)))
+        return out
+
+    def mul_imag_unit(self, a, nq, out=None):
+        if out is None:
+            out = self._new(a.shape[0], nq, a)
+        check(lib().hemm_mul_imag_unit(self.h, vp(a.data_ptr()), self._ps(a), vp(out.data_ptr()),
+                                       self._ps(out), nq, a.shape[0], vp(0)))
+        return out
+
+    def tensor(self, c1, c2, nq, out=None, accumulate=False):
+        if out is None:
+            out = self._new(3, nq, c1)
+        check(lib().hemm_tensor(self.h, vp(c1.data_ptr()), self._ps(c1), vp(c2.data_ptr()),
+                                self._ps(c2), vp(out.data_ptr()), self._ps(out), nq,
+                                int(accumulate), vp(0)))
+        return out
+
+    def automorphism(self, a, galois, n_limbs):
+        polys = a.shape[0]
+        out = self._new(polys, n_limbs, a)
+        check(lib().hemm_automorphism(self.h, vp(a.data_ptr()), self._ps(a), vp(out.data_ptr()),
+                                      self._ps(out), galois, n_limbs, polys, vp(0)))
+        return out
+
+    def beta(self, nq):
+        alpha = -(-self.nQ // self.dnum)
+        return -(-nq // alpha)
+
+    def modup(self, poly, nq):
+        import torch
+        ext = torch.empty((self.beta(nq), nq + self.nP, self.N), dtype=torch.int64, device=poly.device)
+        check(lib().hemm_modup(self.h, vp(poly.data_ptr()), nq, vp(ext.data_ptr()), vp(0)))
+        return ext
+
+    def inner_product(self, ext, evk, nq):
+        acc = self._new(2, nq + self.nP, ext)
+        check(lib().hemm_inner_product(self.h, vp(ext.data_ptr()), vp(evk.data_ptr()), nq,
+                                       vp(acc.data_ptr()), vp(0)))
+        return acc
+
+    def moddown(self, acc, nq):
+        out = self._new(acc.shape[0], nq, acc)
+        check(lib().hemm_moddown(self.h, vp(acc.data_ptr()), nq, acc.shape[0], vp(out.data_ptr()),
+                                 self._ps(out), vp(0)))
+        return out
+
+    def keyswitch(self, poly, evk, nq, add_b=None):
+        out = self._new(2, nq, poly)
+        check(lib().hemm_keyswitch(self.h, vp(poly.data_ptr()), vp(evk.data_ptr()), nq,
+                                   vp(out.data_ptr()), self._ps(out),
+                                   vp(add_b.data_ptr() if add_b is not None else 0), vp(0)))
+        return out
+
+    def rotate(self, ct, evk, galois, nq, out=None):
+        if out is None:
+            out = self._new(2, nq, ct)
+        check(lib().hemm_rotate(self.h, vp(ct.data_ptr()), self._ps(ct), vp(evk.data_ptr()), galois,
+                                nq, vp(out.data_ptr()), self._ps(out), vp(0)))
+        return out
+
+    def relinearize(self, ct3, evk, nq):
+        out = self._new(2, nq, ct3)
+        check(lib().hemm_relinearize(self.h, vp(ct3.data_ptr()), self._ps(ct3), vp(evk.data_ptr()),
+                                     nq, vp(out.data_ptr()), self._ps(out), vp(0)))
+        return out
+
+    def rescale(self, ct, nq):
+        out = self._new(ct.shape[0], nq - 1, ct)
+        check(lib().hemm_rescale(self.h, vp(ct.data_ptr()), self._ps(ct), vp(out.data_ptr()),
+                                 self._ps(out), nq, ct.shape[0], vp(0)))
+        return out
+
+
+ADD, SUB, MUL, NEG, MAC = 0, 1, 2, 3, 4
 
 
 def primes_below(bits, log_n, count):

@@ -7,6 +7,7 @@
 hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, int dnum);
 void hemm_context_free(hemm_context *c);
 void hemm_primes_below_impl(int bits, int logN, int count, u64 *out);
+void hemm_keyswitch_tables_free(const hemm_context *c);
 
 static thread_local std::string g_err;
 void hemm_set_error(const std::string &m) { g_err = m; }
@@ -40,7 +41,10 @@ int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64
     *out = hemm_context_build((int)log_n, (int)n_q, (int)n_p, (const u64 *)primes, (int)dnum);
     HEMM_CATCH
 }
-void hemm_context_destroy(hemm_context *ctx) { hemm_context_free(ctx); }
+void hemm_context_destroy(hemm_context *ctx) {
+    if (ctx) hemm_keyswitch_tables_free(ctx);
+    hemm_context_free(ctx);
+}
 uint64_t hemm_context_psi(const hemm_context *ctx, uint32_t idx) { return ctx->psi.at(idx); }
 
 int hemm_primes_below(uint32_t bits, uint32_t log_n, uint32_t count, uint64_t *out) {
@@ -63,6 +67,169 @@ int hemm_ntt(hemm_context *ctx, uint64_t *data, const uint32_t *prime_idx, uint3
     }
     launch_ntt(ctx, (u64 *)data, ll, (int)n_limbs, (int)n_polys, (size_t)n_limbs * ctx->N, inverse != 0,
                (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+static LimbList chain_limbs(hemm_context *ctx, uint32_t nq, int with_p, int *n_limbs) {
+    need(ctx, "null context");
+    need(ctx->logN >= 9, "residue kernels need log_n >= 9");
+    need(nq >= 1 && nq <= (uint32_t)ctx->nQ, "nq out of range");
+    *n_limbs = (int)nq + (with_p ? ctx->nP : 0);
+    return limbs_default(ctx, (int)nq, with_p);
+}
+
+int hemm_pointwise(hemm_context *ctx, int op, const uint64_t *a, size_t a_stride, const uint64_t *b, size_t b_stride,
+                   uint64_t *out, size_t out_stride, uint32_t nq, int with_p, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
+    need(a && out && (b || op == HEMM_NEG), "null operand");
+    need(op >= 0 && op <= 4, "unknown op");
+    launch_binary(ctx, op, (const u64 *)a, a_stride, (const u64 *)b, b_stride, (u64 *)out, out_stride, ll, nl,
+                  (int)n_polys, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_mul_scalar(hemm_context *ctx, const uint64_t *a, size_t a_stride, const uint64_t *scalars, uint64_t *out,
+                    size_t out_stride, uint32_t nq, int with_p, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
+    need(a && out && scalars, "null operand");
+    launch_mul_scalar(ctx, (const u64 *)a, a_stride, (const u64 *)scalars, (u64 *)out, out_stride, ll, nl,
+                      (int)n_polys, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_mul_imag_unit(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out, size_t out_stride,
+                       uint32_t nq, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, 0, &nl);
+    need(a && out, "null operand");
+    launch_mul_imag(ctx, (const u64 *)a, a_stride, (u64 *)out, out_stride, ll, nl, (int)n_polys, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_tensor(hemm_context *ctx, const uint64_t *ct1, size_t stride1, const uint64_t *ct2, size_t stride2,
+                uint64_t *out, size_t out_stride, uint32_t nq, int accumulate, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 0, &nl);
+    need(ct1 && ct2 && out, "null operand");
+    launch_tensor(ctx, (const u64 *)ct1, stride1, (const u64 *)ct2, stride2, (u64 *)out, out_stride, (int)nq,
+                  accumulate != 0, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_automorphism(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out, size_t out_stride,
+                      uint64_t galois, uint32_t n_limbs, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    need(ctx && a && out, "null operand");
+    need(ctx->logN >= 9, "residue kernels need log_n >= 9");
+    need(a != out, "automorphism cannot run in place");
+    need((galois & 1) && galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
+    launch_galois(ctx, (const u64 *)a, a_stride, (u64 *)out, out_stride, galois, (int)n_limbs, (int)n_polys,
+                  (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_modup(hemm_context *ctx, const uint64_t *in, uint32_t nq, uint64_t *ext, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(in && ext, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    launch_modup(ctx, (const u64 *)in, (int)nq, (u64 *)ext, hemm_scratch(ctx), true, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_inner_product(hemm_context *ctx, const uint64_t *ext, const uint64_t *evk, uint32_t nq, uint64_t *acc,
+                       void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(ext && evk && acc, "null operand");
+    launch_inner_product(ctx, nullptr, (const u64 *)ext, (const u64 *)evk, (int)nq, (u64 *)acc, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_moddown(hemm_context *ctx, uint64_t *acc, uint32_t nq, uint32_t n_polys, uint64_t *out, size_t out_stride,
+                 void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(acc && out, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    need(n_polys >= 1 && n_polys <= 2, "n_polys must be 1 or 2");
+    launch_moddown(ctx, (u64 *)acc, (int)nq, (int)n_polys, (u64 *)out, out_stride, nullptr, 0, 0, hemm_scratch(ctx),
+                   (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_keyswitch(hemm_context *ctx, const uint64_t *in, const uint64_t *evk, uint32_t nq, uint64_t *out,
+                   size_t out_stride, const uint64_t *add_b, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(in && evk && out, "null operand");
+    launch_keyswitch(ctx, (const u64 *)in, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, (const u64 *)add_b,
+                     (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_rotate(hemm_context *ctx, const uint64_t *ct, size_t ct_stride, const uint64_t *evk, uint64_t galois,
+                uint32_t nq, uint64_t *out, size_t out_stride, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(ct && evk && out, "null operand");
+    need((galois & 1) && galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
+    const size_t N = ctx->N;
+    u64 *rot = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
+    launch_galois(ctx, (const u64 *)ct, ct_stride, rot, (size_t)nq * N, galois, (int)nq, 2, (hipStream_t)stream);
+    launch_keyswitch(ctx, rot + (size_t)nq * N, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, rot,
+                     (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, const uint64_t *evk, uint32_t nq,
+                     uint64_t *out, size_t out_stride, void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, 0, &nl);
+    need(ct3 && evk && out, "null operand");
+    const size_t N = ctx->N;
+    u64 *tmp = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
+    launch_keyswitch(ctx, (const u64 *)ct3 + 2 * ct_stride, (const u64 *)evk, (int)nq, tmp, (size_t)nq * N, nullptr,
+                     (hipStream_t)stream);
+    launch_binary(ctx, HEMM_ADD, (const u64 *)ct3, ct_stride, tmp, (size_t)nq * N, (u64 *)out, out_stride, ll, nl, 2,
+                  (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out, size_t out_stride,
+                 uint32_t nq, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 0, &nl);
+    need(in && out, "null operand");
+    need(nq >= 2, "rescale needs at least two limbs");
+    need(n_polys >= 1 && n_polys <= 3, "n_polys must be 1..3");
+    launch_rescale(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
+                   (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

@@ -54,3 +54,24 @@ LimbList limbs_default(const hemm_context *c, int nq, int with_p);
 // kernel launchers (defined in the .hip files)
 void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
                 size_t poly_stride, bool inverse, hipStream_t s);
+void launch_binary(const hemm_context *c, int op, const u64 *a, size_t a_stride, const u64 *b, size_t b_stride,
+                   u64 *out, size_t out_stride, const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
+void launch_mul_scalar(const hemm_context *c, const u64 *a, size_t a_stride, const u64 *scalars, u64 *out,
+                       size_t out_stride, const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
+void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride,
+                     const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
+void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c2, size_t s2, u64 *out,
+                   size_t out_stride, int nq, bool accumulate, hipStream_t s);
+void launch_galois(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride, u64 g,
+                   int n_limbs, int n_polys, hipStream_t s);
+size_t hemm_scratch_words(const hemm_context *c);
+u64 *hemm_scratch(hemm_context *c);
+void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, bool fill_own, hipStream_t s);
+void launch_inner_product(hemm_context *c, const u64 *in, const u64 *ext, const u64 *evk, int nq, u64 *acc,
+                          hipStream_t s);
+void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, size_t out_stride, const u64 *add,
+                    size_t add_stride, int add_polys, u64 *conv, hipStream_t s);
+void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
+                      const u64 *add_b, hipStream_t s);
+void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
+                    int n_polys, hipStream_t s);

@@ -1,0 +1,368 @@
+// Hybrid key switching (ModUp -> evaluation-key inner product -> ModDown) and rescale.
+//
+//   ModUp    : per digit d, coefficient-form fast basis conversion of the digit's limbs to every
+//              other active limb (chain + special), then NTT of the converted limbs.
+//   inner    : acc[pol][j] = sum_d ext_d[j] * evk[d][pol][prime(j)]   (128-bit lazy sum, one
+//              Barrett step per output residue).  Reads the key exactly once: this is the
+//              HBM-bound part, 2*beta*(nq+K) limbs of key per switch.
+//   ModDown  : INTT of the special limbs, basis conversion P -> Q, NTT, (acc - conv) * P^-1.
+//   rescale  : INTT of the last limb, reduce into every remaining prime, NTT, (c - t) * q_l^-1.
+// Basis conversion is the float-free form  y_j = sum_i [x_i * (S/q_i)^-1]_{q_i} * (S/q_i) mod q_j.
+#include <cstring>
+
+#include "hemm_internal.hpp"
+
+void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
+                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s);
+
+namespace {
+
+struct __align__(16) Cst {
+    u64 w, ws;
+};
+
+struct BConvArgs {
+    const u64 *src;        // coefficient form
+    u64 *dst;              // coefficient form
+    size_t src_poly_stride, dst_poly_stride;
+    const Cst *inv;        // [n_src]  (S/q_i)^-1 mod q_i
+    const Cst *hat;        // [n_src][hat_ld]  (S/q_i) mod prime, indexed by prime
+    int n_src, n_dst, hat_ld, logN;
+    uint8_t src_slot[32], src_prime[32];
+    uint8_t dst_slot[HEMM_MAX_PRIMES], dst_prime[HEMM_MAX_PRIMES];
+};
+
+// One thread owns one coefficient: the n_src scaled residues stay in LDS columns private to the
+// thread, then every target limb is a short Shoup multiply-accumulate chain.
+__global__ __launch_bounds__(256) void bconv_kernel(BConvArgs a, const ModQ *__restrict__ modq) {
+    extern __shared__ u64 v[];  // [n_src][256]
+    const int poly = blockIdx.y;
+    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const u64 *src = a.src + poly * a.src_poly_stride;
+    u64 *dst = a.dst + poly * a.dst_poly_stride;
+    for (int i = 0; i < a.n_src; i++) {
+        const u64 q = modq[a.src_prime[i]].q;
+        const Cst c = a.inv[i];
+        v[i * 256 + threadIdx.x] = mul_shoup(src[((size_t)a.src_slot[i] << a.logN) + n], c.w, c.ws, q);
+    }
+    for (int j = 0; j < a.n_dst; j++) {
+        const int pj = a.dst_prime[j];
+        const u64 q = modq[pj].q;
+        u64 acc = 0;
+        for (int i = 0; i < a.n_src; i++) {
+            const Cst c = a.hat[i * a.hat_ld + pj];
+            acc = addmod(acc, mul_shoup(v[i * 256 + threadIdx.x], c.w, c.ws, q), q);
+        }
+        dst[((size_t)a.dst_slot[j] << a.logN) + n] = acc;
+    }
+}
+
+struct DigitMap {
+    uint8_t digit_of[HEMM_MAX_PRIMES];  // for limb j < nq: owning digit; 255 for special limbs
+};
+
+// acc[pol][j][n] = sum_d x_d[j][n] * evk[d][pol][prime(j)][n],  x_d = in[j] when limb j belongs to
+// digit d (its residues were never converted), ext[d][j] otherwise.
+__global__ __launch_bounds__(256) void inner_product_kernel(const u64 *__restrict__ in, const u64 *__restrict__ ext,
+                                                            const u64 *__restrict__ evk, u64 *__restrict__ acc,
+                                                            const ModQ *__restrict__ modq, LimbList ll, DigitMap dm,
+                                                            int beta, int n_ext, int n_full, int logN) {
+    const int j = blockIdx.y;
+    const int prime = ll.idx[j];
+    const ModQ m = modq[prime];
+    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t N = (size_t)1 << logN;
+    u128_t sb = {0, 0}, sa = {0, 0};
+    for (int d = 0; d < beta; d++) {
+        const u64 x = (dm.digit_of[j] == d) ? in[(size_t)j * N + n] : ext[((size_t)d * n_ext + j) * N + n];
+        const u64 kb = evk[(((size_t)d * 2 + 0) * n_full + prime) * N + n];
+        const u64 ka = evk[(((size_t)d * 2 + 1) * n_full + prime) * N + n];
+        add128(sb, mul64wide(x, kb));
+        add128(sa, mul64wide(x, ka));
+    }
+    acc[(size_t)j * N + n] = barrett128(sb, m);
+    acc[((size_t)n_ext + j) * N + n] = barrett128(sa, m);
+}
+
+struct CstList {
+    Cst c[HEMM_MAX_PRIMES];
+};
+
+// out[p][j] = (a[p][j] - t[p][j]) * cst[j]  (+ add[p][j] when add != nullptr)
+__global__ __launch_bounds__(256) void sub_scale_kernel(const u64 *__restrict__ a, size_t a_stride,
+                                                        const u64 *__restrict__ t, size_t t_stride,
+                                                        const u64 *__restrict__ add, size_t add_stride,
+                                                        int add_polys, u64 *__restrict__ out, size_t out_stride,
+                                                        const ModQ *__restrict__ modq, CstList cl, int n_limbs,
+                                                        int logN) {
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const u64 q = modq[limb].q;
+    const size_t e = ((size_t)limb << logN) + (size_t)blockIdx.x * 256 + threadIdx.x;
+    u64 r = mul_shoup(submod(a[poly * a_stride + e], t[poly * t_stride + e], q), cl.c[limb].w, cl.c[limb].ws, q);
+    if (add != nullptr && poly < add_polys) r = addmod(r, add[poly * add_stride + e], q);
+    out[poly * out_stride + e] = r;
+}
+
+// t[p][j][n] = last[p][n] mod q_j
+__global__ __launch_bounds__(256) void spread_kernel(const u64 *__restrict__ last, u64 *__restrict__ t,
+                                                     size_t t_stride, const ModQ *__restrict__ modq, int n_limbs,
+                                                     int logN) {
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const u64 x = last[((size_t)poly << logN) + n];
+    t[poly * t_stride + ((size_t)limb << logN) + n] = reduce64(x, modq[limb]);
+}
+
+u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
+
+}  // namespace
+
+// ---- tables -----------------------------------------------------------------------------------
+// For every active chain length nq and digit d: inv[i] and hat[i][prime] of the digit's limbs;
+// for ModDown: the same for the special basis.  Laid out in one device array of (w, ws) pairs.
+struct KsTables {
+    std::vector<Cst> host;
+    Cst *dev = nullptr;
+    std::vector<std::vector<size_t>> inv_off, hat_off;  // [nq][d]
+    size_t p_inv_off = 0, p_hat_off = 0;
+    std::vector<Cst> pinv;                               // P^-1 mod q_j
+    std::vector<std::vector<Cst>> qlinv;                 // [l][j<l]  q_l^-1 mod q_j
+};
+
+static KsTables *g_tables_of(const hemm_context *c);
+
+static void build_tables(const hemm_context *c, KsTables &t) {
+    const int nQ = c->nQ, K = c->nP, T = nQ + K, alpha = c->alpha;
+    auto push_basis = [&](const std::vector<int> &src, size_t &inv_off, size_t &hat_off) {
+        inv_off = t.host.size();
+        for (size_t i = 0; i < src.size(); i++) {
+            u64 qi = c->primes[src[i]], prod = 1;
+            for (size_t k = 0; k < src.size(); k++)
+                if (k != i) prod = h_mulmod(prod, c->primes[src[k]] % qi, qi);
+            u64 inv = h_invmod(prod, qi);
+            t.host.push_back(Cst{inv, shoup_h(inv, qi)});
+        }
+        hat_off = t.host.size();
+        for (size_t i = 0; i < src.size(); i++)
+            for (int pj = 0; pj < T; pj++) {
+                u64 tq = c->primes[pj], prod = 1;
+                for (size_t k = 0; k < src.size(); k++)
+                    if (k != i) prod = h_mulmod(prod, c->primes[src[k]] % tq, tq);
+                t.host.push_back(Cst{prod, shoup_h(prod, tq)});
+            }
+    };
+    t.inv_off.assign(nQ + 1, {});
+    t.hat_off.assign(nQ + 1, {});
+    for (int nq = 1; nq <= nQ; nq++) {
+        int beta = (nq + alpha - 1) / alpha;
+        t.inv_off[nq].resize(beta);
+        t.hat_off[nq].resize(beta);
+        for (int d = 0; d < beta; d++) {
+            std::vector<int> src;
+            for (int j = d * alpha; j < std::min(nq, (d + 1) * alpha); j++) src.push_back(j);
+            push_basis(src, t.inv_off[nq][d], t.hat_off[nq][d]);
+        }
+    }
+    if (K > 0) {
+        std::vector<int> src;
+        for (int k = 0; k < K; k++) src.push_back(nQ + k);
+        push_basis(src, t.p_inv_off, t.p_hat_off);
+    }
+    t.pinv.resize(nQ);
+    for (int j = 0; j < nQ; j++) {
+        u64 q = c->primes[j], P = 1;
+        for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[nQ + k] % q, q);
+        u64 inv = h_invmod(P, q);
+        t.pinv[j] = Cst{inv, shoup_h(inv, q)};
+    }
+    t.qlinv.assign(nQ, {});
+    for (int l = 1; l < nQ; l++)
+        for (int j = 0; j < l; j++) {
+            u64 q = c->primes[j];
+            u64 inv = h_invmod(c->primes[l] % q, q);
+            t.qlinv[l].push_back(Cst{inv, shoup_h(inv, q)});
+        }
+    HEMM_HIP(hipMalloc((void **)&t.dev, t.host.size() * sizeof(Cst)));
+    HEMM_HIP(hipMemcpy(t.dev, t.host.data(), t.host.size() * sizeof(Cst), hipMemcpyHostToDevice));
+}
+
+// tables live beside the context (created on first use, destroyed with it)
+#include <map>
+#include <mutex>
+static std::map<const hemm_context *, KsTables *> g_tabs;
+static std::mutex g_tabs_mu;
+static KsTables *g_tables_of(const hemm_context *c) {
+    std::lock_guard<std::mutex> lk(g_tabs_mu);
+    auto it = g_tabs.find(c);
+    if (it != g_tabs.end()) return it->second;
+    KsTables *t = new KsTables();
+    build_tables(c, *t);
+    g_tabs[c] = t;
+    return t;
+}
+void hemm_keyswitch_tables_free(const hemm_context *c) {
+    std::lock_guard<std::mutex> lk(g_tabs_mu);
+    auto it = g_tabs.find(c);
+    if (it == g_tabs.end()) return;
+    (void)hipFree(it->second->dev);
+    delete it->second;
+    g_tabs.erase(it);
+}
+
+// scratch (u64 words) needed by key switching / rescale at full width
+size_t hemm_scratch_words(const hemm_context *c) {
+    const size_t N = c->N, T = c->nQ + c->nP;
+    return ((size_t)c->dnum + 7) * T * N;
+}
+u64 *hemm_scratch(hemm_context *c) {
+    if (!c->d_scratch) {
+        c->scratch_bytes = hemm_scratch_words(c) * sizeof(u64);
+        HEMM_HIP(hipMalloc((void **)&c->d_scratch, c->scratch_bytes));
+    }
+    return c->d_scratch;
+}
+
+// ---- ModUp ------------------------------------------------------------------------------------
+// in: [nq][N] NTT form.  ext: [beta][nq+K][N]; limbs owned by digit d are NOT written in ext[d]
+// unless fill_own is set (they equal `in`).  coef: scratch [nq][N].
+void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, bool fill_own, hipStream_t s) {
+    KsTables *t = g_tables_of(c);
+    const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
+    const size_t N = c->N;
+    HEMM_HIP(hipMemcpyAsync(coef, in, (size_t)nq * N * 8, hipMemcpyDeviceToDevice, s));
+    launch_ntt(c, coef, limbs_default(c, nq, 0), nq, 1, (size_t)nq * N, true, s);
+    for (int d = 0; d < beta; d++) {
+        const int lo = d * alpha, hi = std::min(nq, lo + alpha);
+        BConvArgs a;
+        memset(&a, 0, sizeof(a));
+        a.src = coef;
+        a.dst = ext + (size_t)d * E * N;
+        a.inv = t->dev + t->inv_off[nq][d];
+        a.hat = t->dev + t->hat_off[nq][d];
+        a.n_src = hi - lo;
+        a.hat_ld = c->nQ + c->nP;
+        a.logN = c->logN;
+        if (a.n_src > 32) throw std::invalid_argument("digit wider than 32 limbs");
+        LimbList pl, sl;
+        memset(&pl, 0, sizeof(pl));
+        memset(&sl, 0, sizeof(sl));
+        for (int i = 0; i < a.n_src; i++) {
+            a.src_slot[i] = (uint8_t)(lo + i);
+            a.src_prime[i] = (uint8_t)(lo + i);
+        }
+        int nd = 0;
+        for (int j = 0; j < E; j++) {
+            if (j >= lo && j < hi) continue;
+            a.dst_slot[nd] = (uint8_t)j;
+            a.dst_prime[nd] = (uint8_t)(j < nq ? j : c->nQ + (j - nq));
+            pl.idx[nd] = a.dst_prime[nd];
+            sl.idx[nd] = (uint8_t)j;
+            nd++;
+        }
+        a.n_dst = nd;
+        if (nd > 0) {
+            dim3 grid(N / 256, 1), block(256);
+            hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)a.n_src * 256 * 8, s, a, c->d_modq);
+            launch_ntt_slots(c, a.dst, pl, sl, nd, 1, (size_t)E * N, false, s);
+        }
+        if (fill_own)
+            HEMM_HIP(hipMemcpyAsync(a.dst + (size_t)lo * N, in + (size_t)lo * N, (size_t)(hi - lo) * N * 8,
+                                    hipMemcpyDeviceToDevice, s));
+    }
+}
+
+// acc: [2][nq+K][N]
+void launch_inner_product(hemm_context *c, const u64 *in, const u64 *ext, const u64 *evk, int nq, u64 *acc,
+                          hipStream_t s) {
+    const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
+    DigitMap dm;
+    memset(&dm, 255, sizeof(dm));
+    if (in != nullptr)
+        for (int j = 0; j < nq; j++) dm.digit_of[j] = (uint8_t)(j / alpha);
+    dim3 grid(c->N / 256, E), block(256);
+    hipLaunchKernelGGL(inner_product_kernel, grid, block, 0, s, in, ext, evk, acc, c->d_modq,
+                       limbs_default(c, nq, 1), dm, beta, E, c->nQ + c->nP, c->logN);
+}
+
+// acc: [n_polys][nq+K][N] NTT (special limbs are overwritten with their coefficient form).
+// out[p] = ModDown(acc[p]) (+ add[p] for p < add_polys).  conv: scratch [n_polys][nq][N].
+void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, size_t out_stride, const u64 *add,
+                    size_t add_stride, int add_polys, u64 *conv, hipStream_t s) {
+    KsTables *t = g_tables_of(c);
+    const int K = c->nP, E = nq + K;
+    const size_t N = c->N;
+    LimbList pl;
+    memset(&pl, 0, sizeof(pl));
+    for (int k = 0; k < K; k++) pl.idx[k] = (uint8_t)(c->nQ + k);
+    launch_ntt(c, acc + (size_t)nq * N, pl, K, n_polys, (size_t)E * N, true, s);
+    BConvArgs a;
+    memset(&a, 0, sizeof(a));
+    a.src = acc;
+    a.src_poly_stride = (size_t)E * N;
+    a.dst = conv;
+    a.dst_poly_stride = (size_t)nq * N;
+    a.inv = t->dev + t->p_inv_off;
+    a.hat = t->dev + t->p_hat_off;
+    a.n_src = K;
+    a.n_dst = nq;
+    a.hat_ld = c->nQ + c->nP;
+    a.logN = c->logN;
+    if (K > 32) throw std::invalid_argument("more than 32 special primes");
+    for (int k = 0; k < K; k++) {
+        a.src_slot[k] = (uint8_t)(nq + k);
+        a.src_prime[k] = (uint8_t)(c->nQ + k);
+    }
+    for (int j = 0; j < nq; j++) {
+        a.dst_slot[j] = (uint8_t)j;
+        a.dst_prime[j] = (uint8_t)j;
+    }
+    dim3 grid(N / 256, n_polys), block(256);
+    hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)K * 256 * 8, s, a, c->d_modq);
+    launch_ntt(c, conv, limbs_default(c, nq, 0), nq, n_polys, (size_t)nq * N, false, s);
+    CstList cl;
+    for (int j = 0; j < nq; j++) cl.c[j] = t->pinv[j];
+    dim3 g2(N / 256, nq * n_polys);
+    hipLaunchKernelGGL(sub_scale_kernel, g2, block, 0, s, acc, (size_t)E * N, conv, (size_t)nq * N, add, add_stride,
+                       add_polys, out, out_stride, c->d_modq, cl, nq, c->logN);
+}
+
+// Full key switch of `in` ([nq][N], NTT) with `evk` ([dnum][2][nQ+K][N]):
+// out[0] = ks_b (+ add_b), out[1] = ks_a; out poly stride out_stride.
+void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
+                      const u64 *add_b, hipStream_t s) {
+    if (c->nP < 1) throw std::invalid_argument("key switching needs special primes");
+    const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+    const size_t N = c->N;
+    u64 *sc = hemm_scratch(c);
+    u64 *coef = sc;                              // [nq][N]   (reused as conv[2][nq] needs 2*nq)
+    u64 *ext = coef + (size_t)2 * (c->nQ) * N;   // [beta][E][N]
+    u64 *acc = ext + (size_t)beta * E * N;       // [2][E][N]
+    launch_modup(c, in, nq, ext, coef, false, s);
+    launch_inner_product(c, in, ext, evk, nq, acc, s);
+    launch_moddown(c, acc, nq, 2, out, out_stride, add_b, 0, add_b ? 1 : 0, coef, s);
+}
+
+// in: [n_polys][nq][N] -> out: [n_polys][nq-1][N]
+void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
+                    int n_polys, hipStream_t s) {
+    if (nq < 2) throw std::invalid_argument("rescale needs at least two limbs");
+    KsTables *t = g_tables_of(c);
+    const size_t N = c->N;
+    u64 *sc = hemm_scratch(c);
+    u64 *last = sc;                               // [n_polys][N]
+    u64 *tt = sc + (size_t)n_polys * N;           // [n_polys][nq-1][N]
+    for (int p = 0; p < n_polys; p++)
+        HEMM_HIP(hipMemcpyAsync(last + (size_t)p * N, in + p * in_stride + (size_t)(nq - 1) * N, N * 8,
+                                hipMemcpyDeviceToDevice, s));
+    LimbList pl;
+    memset(&pl, 0, sizeof(pl));
+    pl.idx[0] = (uint8_t)(nq - 1);
+    launch_ntt(c, last, pl, 1, n_polys, N, true, s);
+    dim3 grid(N / 256, (nq - 1) * n_polys), block(256);
+    hipLaunchKernelGGL(spread_kernel, grid, block, 0, s, last, tt, (size_t)(nq - 1) * N, c->d_modq, nq - 1, c->logN);
+    launch_ntt(c, tt, limbs_default(c, nq - 1, 0), nq - 1, n_polys, (size_t)(nq - 1) * N, false, s);
+    CstList cl;
+    for (int j = 0; j < nq - 1; j++) cl.c[j] = t->qlinv[nq - 1][j];
+    hipLaunchKernelGGL(sub_scale_kernel, grid, block, 0, s, in, in_stride, tt, (size_t)(nq - 1) * N,
+                       (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq - 1, c->logN);
+}

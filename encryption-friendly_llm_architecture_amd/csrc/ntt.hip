@@ -54,7 +54,7 @@ template <bool INV>
 __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
                                                           const ModQ *__restrict__ modq,
                                                           const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
-                                                          LimbList ll, int n_limbs, size_t poly_stride,
+                                                          LimbList ll, LimbList sl, int n_limbs, size_t poly_stride,
                                                           GenericPass gp) {
     extern __shared__ u64 lds[];
     const int N = 1 << gp.logN;
@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + (size_t)prime * N;
     const u64 q = modq[prime].q, q2 = 2 * q;
-    u64 *base = data + (size_t)poly * poly_stride + (size_t)limb * N;
+    u64 *base = data + (size_t)poly * poly_stride + (size_t)sl.idx[limb] * N;
     const int tile = blockIdx.x;
     // tile origin: strided pass tiles walk the columns; contiguous pass tiles walk the limb
     const int c0 = (gp.rowstride == 1) ? tile * gp.R * gp.CW : tile * gp.CW;
@@ -166,14 +166,14 @@ template <bool INV>
 __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
                                                          const ModQ *__restrict__ modq,
                                                          const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
-                                                         LimbList ll, int n_limbs, size_t poly_stride) {
+                                                         LimbList ll, LimbList sl, int n_limbs, size_t poly_stride) {
     __shared__ u64 lds[256 * 16];
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
     const u64 q = modq[prime].q;
     const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
-    u64 *base = data + (size_t)poly * poly_stride + ((size_t)limb << 16) + blockIdx.x * 16 + cc;
+    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + blockIdx.x * 16 + cc;
     u64 x[16];
     if (!INV) {
 #pragma unroll
@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
 template <bool INV>
 __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
-                                                         const ModQ *__restrict__ modq, LimbList ll, int n_limbs,
+                                                         const ModQ *__restrict__ modq, LimbList ll, LimbList sl, int n_limbs,
                                                          size_t poly_stride) {
     __shared__ u64 lds[16 * ROWPAD];
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
     const u64 q = modq[prime].q, q2 = 2 * q;
     const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
     const u32 r = blockIdx.x * 16 + rr;  // global row
-    u64 *row = data + (size_t)poly * poly_stride + ((size_t)limb << 16) + ((size_t)r << 8);
+    u64 *row = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     u64 *l = lds + rr * ROWPAD;
     u64 x[16];
 #pragma unroll
@@ -266,8 +266,8 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
 
 }  // namespace
 
-void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
-                size_t poly_stride, bool inverse, hipStream_t s) {
+void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
+                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s) {
     if (n_limbs <= 0 || n_polys <= 0) return;
     const Tw *tw = (const Tw *)(inverse ? c->d_iw : c->d_w);
     const int lanes = n_limbs * n_polys;
@@ -275,14 +275,14 @@ void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limb
         dim3 grid(16, lanes), block(256);
         if (!inverse) {
             hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, n_limbs, poly_stride);
-            hipLaunchKernelGGL(ntt16_rows_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, ll, n_limbs,
+                               c->d_ninv_s, ll, sl, n_limbs, poly_stride);
+            hipLaunchKernelGGL(ntt16_rows_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
                                poly_stride);
         } else {
-            hipLaunchKernelGGL(ntt16_rows_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, ll, n_limbs,
+            hipLaunchKernelGGL(ntt16_rows_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
                                poly_stride);
             hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, n_limbs, poly_stride);
+                               c->d_ninv_s, ll, sl, n_limbs, poly_stride);
         }
         return;
     }
@@ -308,11 +308,11 @@ void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limb
         size_t sh = (size_t)gp.R * gp.CW * sizeof(u64);
         if (!inverse)
             hipLaunchKernelGGL(ntt_generic_kernel<false>, grid, block, sh, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, n_limbs, poly_stride, gp);
+                               c->d_ninv_s, ll, sl, n_limbs, poly_stride, gp);
         else {
             std::swap(gp.s_begin, gp.s_end);     // inverse walks stages downwards
             hipLaunchKernelGGL(ntt_generic_kernel<true>, grid, block, sh, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, n_limbs, poly_stride, gp);
+                               c->d_ninv_s, ll, sl, n_limbs, poly_stride, gp);
         }
     };
     if (n_pass == 1) {
@@ -324,4 +324,11 @@ void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limb
         run(B, true, false);
         run(A, false, true);
     }
+}
+
+void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
+                size_t poly_stride, bool inverse, hipStream_t s) {
+    LimbList sl;
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) sl.idx[j] = (uint8_t)j;
+    launch_ntt_slots(c, data, ll, sl, n_limbs, n_polys, poly_stride, inverse, s);
 }

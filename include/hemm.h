@@ -44,6 +44,60 @@ int hemm_primes_below(uint32_t bits, uint32_t log_n, uint32_t count, uint64_t *o
 int hemm_ntt(hemm_context *ctx, uint64_t *data, const uint32_t *prime_idx, uint32_t n_limbs,
              uint32_t n_polys, int inverse, void *stream);
 
+/* ---- streaming residue kernels -------------------------------------------------------------
+ * Operands are [n_polys][n_limbs][N] with their own polynomial stride (in uint64 words), so a
+ * higher-level operand can be read at a lower level ("levels auto-adjust to the lower operand",
+ * HomEvaluator.hpp:128-129); stride 0 broadcasts one polynomial (a plaintext).  n_limbs =
+ * nq + (with_p ? n_p : 0).  `out` may alias an input element-for-element. */
+enum { HEMM_ADD = 0, HEMM_SUB = 1, HEMM_MUL = 2, HEMM_NEG = 3, HEMM_MAC = 4 };
+/* HomEvaluator::add :144 / sub :223 / negate :67 / multWithoutRescale(ct, pt) :491 (HEMM_MUL with
+ * b_stride = 0) / multiply-accumulate for the diagonal accumulation of matmul :600 */
+int hemm_pointwise(hemm_context *ctx, int op, const uint64_t *a, size_t a_stride, const uint64_t *b,
+                   size_t b_stride, uint64_t *out, size_t out_stride, uint32_t nq, int with_p,
+                   uint32_t n_polys, void *stream);
+/* HomEvaluator::multInteger :347 / constant multiply :276,:478: residue-wise product with one
+ * host-side scalar per limb (scalars[j] is reduced modulo limb j's prime). */
+int hemm_mul_scalar(hemm_context *ctx, const uint64_t *a, size_t a_stride, const uint64_t *scalars,
+                    uint64_t *out, size_t out_stride, uint32_t nq, int with_p, uint32_t n_polys,
+                    void *stream);
+/* HomEvaluator::multImagUnit :330: multiply by the monomial X^(N/2) in NTT form. */
+int hemm_mul_imag_unit(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out,
+                       size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
+/* HomEvaluator::tensor :518: (b1,a1) x (b2,a2) -> (b1 b2, a1 b2 + a2 b1, a1 a2); accumulate != 0
+ * adds into `out` (the running 3-polynomial sum of the CCMM loop, MatrixUtils.cpp:1434-1439). */
+int hemm_tensor(hemm_context *ctx, const uint64_t *ct1, size_t stride1, const uint64_t *ct2,
+                size_t stride2, uint64_t *out, size_t out_stride, uint32_t nq, int accumulate,
+                void *stream);
+/* Galois automorphism X -> X^galois on NTT-form limbs (the keyless half of leftRotate :370-403 and
+ * conjugate :465; all of leftRotate(Plaintext) :376).  `out` must not alias `a`. */
+int hemm_automorphism(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out,
+                      size_t out_stride, uint64_t galois, uint32_t n_limbs, uint32_t n_polys,
+                      void *stream);
+
+/* ---- hybrid key switching (inside leftRotate/rightRotate :383-403, conjugate :465, relinearize
+ * :524).  Evaluation key layout: [dnum][2 (b, a)][n_q + n_p][N], NTT form.  The stages are exposed
+ * one by one so each can be checked against the CPU oracle; hemm_keyswitch chains them. ---- */
+/* in [nq][N] -> ext [beta][nq + n_p][N], beta = ceil(nq / alpha), alpha = ceil(n_q / dnum) */
+int hemm_modup(hemm_context *ctx, const uint64_t *in, uint32_t nq, uint64_t *ext, void *stream);
+/* ext [beta][nq + n_p][N], evk -> acc [2][nq + n_p][N] */
+int hemm_inner_product(hemm_context *ctx, const uint64_t *ext, const uint64_t *evk, uint32_t nq,
+                       uint64_t *acc, void *stream);
+/* acc [n_polys][nq + n_p][N] (clobbered) -> out [n_polys][nq][N] = acc / P */
+int hemm_moddown(hemm_context *ctx, uint64_t *acc, uint32_t nq, uint32_t n_polys, uint64_t *out,
+                 size_t out_stride, void *stream);
+/* in [nq][N], evk -> out[0] = ks_b (+ add_b[nq][N] when not NULL), out[1] = ks_a */
+int hemm_keyswitch(hemm_context *ctx, const uint64_t *in, const uint64_t *evk, uint32_t nq,
+                   uint64_t *out, size_t out_stride, const uint64_t *add_b, void *stream);
+/* HomEvaluator::leftRotate(ct) :383 / conjugate :465: automorphism of (b, a) + key switch of a. */
+int hemm_rotate(hemm_context *ctx, const uint64_t *ct, size_t ct_stride, const uint64_t *evk,
+                uint64_t galois, uint32_t nq, uint64_t *out, size_t out_stride, void *stream);
+/* HomEvaluator::relinearize :524: (d0, d1, d2) -> (d0 + ks_b(d2), d1 + ks_a(d2)) */
+int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, const uint64_t *evk,
+                     uint32_t nq, uint64_t *out, size_t out_stride, void *stream);
+/* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last */
+int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
+                 size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,173 @@
+"""GPU parity, stage by stage, of the evaluator kernels (pointwise, tensor, automorphism, ModUp,
+evk inner product, ModDown, key switch, rotate, relinearize, rescale) against the CPU oracle:
+bit-exact residues on identical primes, keys and inputs."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle import oracle as O
+from oracle.oracle import _p
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int64)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy().view(np.uint64)
+
+
+def rand_limbs(rng, mods, shape_prefix, N):
+    out = np.empty(tuple(shape_prefix) + (len(mods), N), dtype=np.uint64)
+    for j, q in enumerate(mods):
+        out[..., j, :] = rng.integers(0, q, tuple(shape_prefix) + (N,), dtype=np.uint64)
+    return out
+
+
+class Setup:
+    def __init__(self, log_n, n_q, n_p, dnum, seed):
+        pkg = load_package()
+        self.pkg = pkg
+        qs, ps = O.ckks_chain(log_n, n_q, n_p)
+        self.orc = O.Oracle(log_n, qs, ps, dnum)
+        self.ctx = pkg.Context(log_n, qs, ps, dnum)
+        self.rng = np.random.default_rng(seed)
+        self.N = 1 << log_n
+        self.orc.gen_secret(3, hw=min(192, self.N // 4))
+
+
+@pytest.fixture(scope="module", params=[(10, 6, 2, 3), (12, 7, 4, 2), (16, 5, 3, 2)],
+                ids=["N1024", "N4096", "N65536"])
+def S(request):
+    return Setup(*request.param, seed=request.param[0])
+
+
+def test_pointwise_ops(S):
+    orc, ctx, pkg, N = S.orc, S.ctx, S.pkg, S.N
+    nq = orc.nQ - 1
+    mods = [orc.mods[orc.prime_of(j, nq)] for j in range(nq + orc.nP)]
+    a = rand_limbs(S.rng, mods, (2,), N)
+    b = rand_limbs(S.rng, mods, (2,), N)
+    a[0, 0, :3] = [0, mods[0] - 1, 1]
+    b[0, 0, :3] = [0, mods[0] - 1, mods[0] - 1]
+    da, db = dev(a), dev(b)
+    ref = {}
+    for op in (0, 1, 2):
+        ref[op] = np.empty_like(a)
+        for p in range(2):
+            for j in range(nq + orc.nP):
+                orc.L.orc_pointwise(orc.h, op, _p(a[p, j]), _p(b[p, j]), _p(ref[op][p, j]), orc.prime_of(j, nq))
+        assert np.array_equal(host(ctx.pointwise(op, da, db, nq, with_p=True)), ref[op])
+    # negate, broadcast multiply (ct x pt), multiply-accumulate, aliasing output
+    neg = host(ctx.pointwise(pkg.NEG, da, None, nq, with_p=True))
+    assert np.array_equal((neg.astype(object) + a.astype(object)) % np.array(mods, dtype=object)[None, :, None], 0 * a)
+    pt = db[0].contiguous()
+    got = host(ctx.pointwise(pkg.MUL, da, pt, nq, with_p=True))
+    want = np.empty_like(a)
+    for p in range(2):
+        for j in range(nq + orc.nP):
+            orc.L.orc_pointwise(orc.h, 2, _p(a[p, j]), _p(b[0, j]), _p(want[p, j]), orc.prime_of(j, nq))
+    assert np.array_equal(got, want)
+    acc = da.clone()
+    ctx.pointwise(pkg.MAC, da, db, nq, with_p=True, out=acc)
+    want = (ref[2].astype(object) + a.astype(object)) % np.array(mods, dtype=object)[None, :, None]
+    assert np.array_equal(host(acc).astype(object), want)
+    # reading a 2-poly operand at a lower level through its stride
+    lo = ctx.pointwise(pkg.ADD, da, db, 2, with_p=False)
+    assert np.array_equal(host(lo), ref[0][:, :2])
+
+
+def test_scalar_imag_tensor_automorphism(S):
+    orc, ctx, N = S.orc, S.ctx, S.N
+    nq = orc.nQ
+    mods = orc.q[:nq]
+    c1 = rand_limbs(S.rng, mods, (2,), N)
+    c2 = rand_limbs(S.rng, mods, (2,), N)
+    d1, d2 = dev(c1), dev(c2)
+    want = np.empty((3, nq, N), dtype=np.uint64)
+    orc.L.orc_tensor(orc.h, _p(c1), _p(c2), nq, _p(want))
+    t = ctx.tensor(d1, d2, nq)
+    assert np.array_equal(host(t), want)
+    ctx.tensor(d2, d1, nq, out=t, accumulate=True)
+    dbl = (want.astype(object) * 2) % np.array(mods, dtype=object)[None, :, None]
+    assert np.array_equal(host(t).astype(object), dbl)
+    # scalar (negative integer and a 60-bit constant) and imaginary unit
+    for val in (-2, 123456789012345678):
+        sc = [val % q for q in mods]
+        got = host(ctx.mul_scalar(d1, sc, nq))
+        assert np.array_equal(got, orc.mult_scalar_residues(O.Ct(c1, 1.0), val))
+    assert np.array_equal(host(ctx.mul_imag_unit(d1, nq)), orc.mult_imag_unit(O.Ct(c1, 1.0)).data)
+    for g in (5, pow(5, 77, 2 * N), 2 * N - 1):
+        got = host(ctx.automorphism(d1, g, nq))
+        want = np.empty_like(c1)
+        for p in range(2):
+            for j in range(nq):
+                orc.L.orc_automorphism_ntt(orc.h, _p(c1[p, j]), _p(want[p, j]), g)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("drop", [0, 1, 2])
+def test_keyswitch_stages(S, drop):
+    """ModUp, inner product and ModDown one at a time, then the fused chain, at several levels
+    (drop = limbs removed from the top, so partial last digits are covered)."""
+    orc, ctx, N = S.orc, S.ctx, S.N
+    nq = orc.nQ - drop
+    E = nq + orc.nP
+    if "mult" not in orc.keys:
+        orc.gen_mult_key(6)
+    evk = orc.keys["mult"]
+    devk = dev(evk)
+    x = rand_limbs(S.rng, orc.q[:nq], (), N)
+    dx = dev(x)
+    beta = (nq + orc.alpha - 1) // orc.alpha
+    ext = np.empty((beta, E, N), dtype=np.uint64)
+    orc.L.orc_modup(orc.h, _p(x), nq, _p(ext))
+    dext = ctx.modup(dx, nq)
+    assert np.array_equal(host(dext), ext)
+    acc = np.empty((2, E, N), dtype=np.uint64)
+    orc.L.orc_inner_product(orc.h, _p(ext), _p(evk), nq, _p(acc))
+    dacc = ctx.inner_product(dext, devk, nq)
+    assert np.array_equal(host(dacc), acc)
+    want = np.empty((2, nq, N), dtype=np.uint64)
+    for p in range(2):
+        orc.L.orc_moddown(orc.h, _p(acc[p]), nq, _p(want[p]))
+    assert np.array_equal(host(ctx.moddown(dacc, nq)), want)
+    assert np.array_equal(host(ctx.keyswitch(dx, devk, nq)), want)
+    ob, oa = orc.keyswitch(x, evk)
+    assert np.array_equal(want[0], ob) and np.array_equal(want[1], oa)
+
+
+def test_rotate_relinearize_rescale(S):
+    orc, ctx, N = S.orc, S.ctx, S.N
+    nq = orc.nQ - 1
+    if "mult" not in orc.keys:
+        orc.gen_mult_key(6)
+    rng = S.rng
+    z = rng.uniform(-1, 1, orc.slots) + 1j * rng.uniform(-1, 1, orc.slots)
+    ct = orc.encrypt(orc.encode(z, nq - 1), 4)
+    dct = dev(ct.data)
+    for r in (1, 7):
+        orc.gen_rot_key(6, r)
+        g = orc.galois(r)
+        want = orc.left_rotate(ct, r)
+        got = host(ctx.rotate(dct, dev(orc.keys[("gal", g)]), g, nq))
+        assert np.array_equal(got, want.data)
+        assert np.abs(orc.decrypt(O.Ct(got, ct.scale)) - np.roll(z, -r)).max() < 1e-6
+    orc.gen_conj_key(6)
+    g = 2 * N - 1
+    assert np.array_equal(host(ctx.rotate(dct, dev(orc.keys[("gal", g)]), g, nq)), orc.conjugate(ct).data)
+    t3 = orc.tensor(ct, ct)
+    d3 = ctx.tensor(dct, dct, nq)
+    assert np.array_equal(host(d3), t3.data)
+    rl = orc.relinearize(t3)
+    drl = ctx.relinearize(d3, dev(orc.keys["mult"]), nq)
+    assert np.array_equal(host(drl), rl.data)
+    rs = orc.rescale(rl)
+    drs = ctx.rescale(drl, nq)
+    assert np.array_equal(host(drs), rs.data)
+    assert np.abs(orc.decrypt(O.Ct(host(drs), rs.scale)) - z * z).max() < 1e-6
+    # 3-polynomial rescale (used on un-relinearised sums)
+    assert np.array_equal(host(ctx.rescale(d3, nq)), orc.rescale(t3).data)
