@@ -19,10 +19,11 @@ def sources():
 
 def _compile(src):
     obj = os.path.splitext(src)[0] + ".o"
-    cmd = [HIPCC] + FLAGS + ["-I", os.path.join(HERE, "..", "include"), "-I", CSRC, "-c", src, "-o", obj]
+    inc = ["-I", os.path.join(HERE, "..", "include"), "-I", CSRC, "-I", os.path.join(CSRC, "host")]
+    cmd = [HIPCC] + FLAGS + inc + ["-c", src, "-o", obj]
     if src.endswith(".cpp"):
-        cmd = [HIPCC] + FLAGS + ["-x", "hip", "-I", os.path.join(HERE, "..", "include"), "-I", CSRC,
-                                 "-c", src, "-o", obj]
+        # host layer: no fused multiply-adds, so the embedding FFT rounds the same everywhere
+        cmd = [HIPCC] + FLAGS + ["-x", "hip", "-ffp-contract=off"] + inc + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

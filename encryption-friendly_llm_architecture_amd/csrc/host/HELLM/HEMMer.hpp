@@ -1,0 +1,127 @@
+// HEMMer: owns the context, keys and evaluator and exposes the matrix-multiplication entry points
+// (reference: ciphertext/include/HELLM/HEMMer.hpp:33-351, matmul / packing / codec part).
+// Where the reference takes torch::Tensor, this build takes a plain row-major Matrix of doubles:
+// tensors are only a container on that path (HEMMer.cpp:232-275 copy them straight into a Message).
+//
+// Tile side n is fixed by the ring: n * n * 2 = N / 2 slots (n = 128 for N = 2^16, the reference's
+// ModelArgs::HEAD_DIM).  "Single" layout: one n x n tile in rows of n slots (lower half of the slot
+// vector).  "Pair" layout: two tiles side by side in rows of 2n slots (all slots).
+#pragma once
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "HELLM/MatrixUtils.hpp"
+
+namespace HELLM {
+
+struct Matrix {
+    i64 rows = 0, cols = 0;
+    std::vector<double> v;  // row-major
+    Matrix() = default;
+    Matrix(i64 r, i64 c, double fill = 0.0) : rows(r), cols(c), v((size_t)(r * c), fill) {}
+    double &at(i64 r, i64 c) { return v[(size_t)(r * cols + c)]; }
+    double at(i64 r, i64 c) const { return v[(size_t)(r * cols + c)]; }
+};
+
+void cleanUpMatrixTransformer();
+
+class HEMMer final {
+public:
+    static HEMMer genHEMMer(int device_id = 0, ParameterPreset preset = ParameterPreset::FGb,
+                            const bool is_multi_gpu = false);
+    explicit HEMMer(int device_id = 0, ParameterPreset preset = ParameterPreset::FGb);
+    // any context (small rings for tests); min_bootstrap_level feeds the level checks
+    HEMMer(const Context &context, u64 min_bootstrap_level);
+    HEMMer(const std::string &key_path, int device_id = 0, ParameterPreset preset = ParameterPreset::FGb);
+    ~HEMMer();
+    HEMMer(const HEMMer &) = delete;
+
+    const Context &getContext() const { return context_; }
+    const HomEvaluator &getEval() const { return eval_; }
+    const Bootstrapper &getBtp() const { return btp_; }
+    const EnDecoder &getEnDec() const { return endec_; }
+    const Decryptor &getDec() const { return dec_; }
+    const SecretKey &getsk() const { return sk_; }
+    i64 dim() const { return dim_; }
+    const KeyPack &keyPack() const { return pack_; }
+    // sigma / tau on their own (MatrixTransformer::diagonalToColumn / diagonalToRow with this HEMMer's keys)
+    CtxtTensor diagonalToColumn(const CtxtTensor &a) const;
+    CtxtTensor diagonalToRow(const CtxtTensor &b) const;
+
+    void save(const std::string &keys_path);
+
+    Message message2(const Matrix &a, const Matrix &b) const;
+    PtxtTensor encode(const Matrix &data, u64 level = 0) const;
+    PtxtTensor encode2(const Matrix &a, const Matrix &b, u64 level = 0) const;
+    Message msgDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4) const;
+    PtxtTensor encodeDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4,
+                                    u64 level = 0) const;
+    CtxtTensor encrypt(const Matrix &data) const;
+    CtxtTensor encrypt2(const Matrix &a, const Matrix &b) const;
+    Matrix decrypt(const CtxtTensor &t) const;
+    std::vector<Matrix> decrypt2(const CtxtTensor &t) const;
+
+    template <class T>
+    void addInplace(CtxtTensor &a, const HETensor<T> &b) const {
+        eval_.add(a.get(), b.get(), a.get());
+    }
+    template <class T>
+    void hadamardMultInplace(CtxtTensor &a, const HETensor<T> &b) const {
+        eval_.mult(a.get(), b.get(), a.get());
+    }
+
+    void transposeInplace(CtxtTensor &t, u64 target_level = 0) const;
+    void complexPackingInplace(CtxtTensor &t) const;
+    void complexPackingRowInplace(CtxtTensor &t) const;
+    void transposeComplexPackingInplace(CtxtTensor &t, u64 target_level = 0) const;
+    void splitInTwo(CtxtTensor &t, CtxtTensor &t1, CtxtTensor &t2) const;
+
+    CtxtTensor packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 target_level = 4) const;
+    CtxtTensor packedMatMulPre(const CtxtTensor &a, u64 target_level = 4) const;
+    void packedMatMulPreRot(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level = 4) const;
+    CtxtTensor packedMatMulPreRev(const CtxtTensor &b, u64 target_level = 4) const;
+    CtxtTensor packedMatMulCCReuse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
+                                   u64 target_level = 4) const;
+    CtxtTensor singleMatMul(const CtxtTensor &a, const PtxtTensor &b, u64 target_level = 4) const;
+    CtxtTensor singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 target_level = 4) const;
+
+    CtxtTensor repackCC(CtxtTensor &t) const;
+    PtxtTensor complexPacking(const PtxtTensor &a, const PtxtTensor &b) const;
+    CtxtTensor complexPacking(const CtxtTensor &a, const CtxtTensor &b) const;
+    CtxtTensor complexPackingRev(const CtxtTensor &a, const CtxtTensor &b) const;
+    CtxtTensor repack(CtxtTensor &t1, CtxtTensor &t2) const;         // needs bootstrapping: throws
+    CtxtTensor repack_notBTS(CtxtTensor &t1, CtxtTensor &t2) const;
+
+    void matMulPre(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level = 4) const;
+    CtxtTensor matMulReUse(const std::vector<Ciphertext> &tmp, const PtxtTensor &b, u64 target_level = 4) const;
+    CtxtTensor matMulPreRev(const CtxtTensor &b, u64 target_level = 4) const;
+    CtxtTensor matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 target_level = 4) const;
+
+    // generate (once) the direct rotation keys a routine needs; rotations are left shifts in slots
+    void ensureRotationKeys(const std::vector<u64> &left_rotations) const;
+    size_t rotationKeyCount() const { return have_rot_.size(); }
+
+private:
+    void init();
+    const Plaintext &cachedMask(int id, u64 level) const;
+    std::vector<u64> transformRotations(MaskKind kind, i64 width) const;
+
+    int device_id_ = 0;
+    Context context_;
+    u64 log_slots_;
+    i64 dim_;
+    SecretKey sk_;
+    Encryptor enc_;
+    Decryptor dec_;
+    EnDecoder endec_;
+    mutable KeyPack pack_;
+    HomEvaluator eval_;
+    Bootstrapper btp_;
+    Message col_mask_even_, row_mask_even_, mask_left_half_, mask_matmul_;
+    mutable std::map<std::pair<int, u64>, Plaintext> mask_cache_;
+    mutable std::set<u64> have_rot_;
+};
+
+}  // namespace HELLM

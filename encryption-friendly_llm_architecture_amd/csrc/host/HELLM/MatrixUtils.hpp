@@ -1,0 +1,95 @@
+// Homomorphic matrix products on packed tiles: the sigma/tau diagonal transforms, transpose, and the
+// ciphertext x ciphertext / plaintext x ciphertext multiplications built on them.
+// Mirrors the call surface of the reference's ciphertext/include/HELLM/MatrixUtils.hpp:130-215
+// (free functions taking the evaluator, the operands, the target level and the transformer) and the
+// MatrixTransformer methods of ciphertext/src/MatrixUtils.cpp:584-1098.
+//
+// Slot layout: value (r, c) of a tile lives in slot r * block_width + c; tiles repeat over the whole
+// slot vector, and every mask below is tiled the same way, so one ciphertext may carry several tiles.
+//
+// Differences from the reference that do not change the decrypted result: transform masks are
+// encoded once per (kind, shape, level) and stay resident in HBM in NTT form instead of being
+// re-encoded from a Message on every multiplication, and a transform sums its masked rotations
+// before a single rescale instead of rescaling each term.
+#pragma once
+#include <map>
+#include <vector>
+
+#include "HELLM/HETensor.hpp"
+
+namespace HELLM {
+
+enum class MaskKind { Horizontal, Vertical, PackedHorizontal, PackedVertical, Diagonal };
+
+// 0/1 (or 0.5) slot pattern of diagonal `idx` for a transform kind, before any pre-rotation.
+// Horizontal (sigma): rows r with r mod n == idx take columns [0, n - idx); negative idx = the wrapped
+// part.  Vertical (tau): the same with rows and columns swapped.  Packed kinds work on 2 x 2 cells.
+// Diagonal (transpose): output positions (r, c) with r - c == idx.
+Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, i64 idx);
+
+class MatrixTransformer {
+public:
+    // mask `idx` of `kind`, pre-rotated for its baby-step/giant-step group and encoded at `level`
+    const Plaintext &transformMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape, u64 level,
+                                   i64 idx);
+    // assemble masks of a cyclic shift by i inside each tile row (columns) / tile column (rows):
+    // [2i] selects the wrapped part, [2i+1] its complement; encoded at `level`
+    std::vector<Plaintext> &getColMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
+    std::vector<Plaintext> &getRowMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
+
+    template <class T>
+    HETensor<T> transpose(const HomEvaluator &eval, const HETensor<T> &op);
+    // sigma(A)[i, j] = A[i, (i + j) mod n]
+    template <class T>
+    HETensor<T> diagonalToColumn(const HomEvaluator &eval, const HETensor<T> &op);
+    // tau(B)[i, j] = B[(i + j) mod n, j]
+    template <class T>
+    HETensor<T> diagonalToRow(const HomEvaluator &eval, const HETensor<T> &op);
+    CtxtTensor packedDiagonalToColumn(const HomEvaluator &eval, const CtxtTensor &op);
+    CtxtTensor packedDiagonalToRow(const HomEvaluator &eval, const CtxtTensor &op);
+
+    void cleanUp();
+    size_t cachedMasks() const;
+
+private:
+    struct Key {
+        int kind;
+        TileTensorShape shape;
+        u64 level;
+        i64 idx;
+        bool operator<(const Key &o) const {
+            return std::tie(kind, shape, level, idx) < std::tie(o.kind, o.shape, o.level, o.idx);
+        }
+    };
+    Ciphertext diagonalTransform(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                 const TileTensorShape &shape);
+    std::map<Key, Plaintext> masks_;
+    std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
+};
+
+// A x B for two encrypted tiles (HEMMer::singleCCMatMul); output level = target_level.
+template <class T>
+CtxtTensor multMatMat(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                      const HETensor<T> &op2, u64 target_level, MatrixTransformer &transformer);
+// two products per call on complex-packed operands (HEMMer::packedMatMul)
+CtxtTensor multPackedMatMat(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                            const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer);
+CtxtTensor multPackedMatMatPre(const HomEvaluator &eval, const CtxtTensor &a, u64 target_level,
+                               MatrixTransformer &transformer);
+void multPackedMatMatPreRot(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp,
+                            u64 target_level, MatrixTransformer &transformer);
+CtxtTensor multPackedMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b, u64 target_level,
+                                  MatrixTransformer &transformer);
+CtxtTensor multPackedMatMatCCReuse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
+                                   u64 target_level, MatrixTransformer &transformer);
+// hoisted form: all column shifts of sigma(A) once, then one accumulation per weight tile
+void multMatMatPre(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
+                   MatrixTransformer &transformer);
+CtxtTensor multMatMatReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const PtxtTensor &b,
+                           u64 target_level, MatrixTransformer &transformer);
+CtxtTensor multMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b, u64 target_level,
+                            MatrixTransformer &transformer);
+CtxtTensor multMatMatCCReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
+                             u64 target_level, MatrixTransformer &transformer);
+
+}  // namespace HELLM

@@ -1,0 +1,422 @@
+// extern "C" facade over HELLM::HEMMer (declared in include/hellm.h).
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "../../../include/hellm.h"
+#include "HELLM/HEMMer.hpp"
+#include "context_content.hpp"
+
+void hemm_set_error(const std::string &msg);
+
+using namespace HELLM;
+
+struct hellm_hemmer {
+    HEMMer *m;
+};
+struct hellm_ct {
+    CtxtTensor t;
+};
+struct hellm_pt {
+    PtxtTensor t;
+};
+struct hellm_ctvec {
+    std::vector<Ciphertext> v;
+};
+
+#define FACADE_TRY try {
+#define FACADE_CATCH                           \
+    }                                          \
+    catch (const std::invalid_argument &e) {   \
+        hemm_set_error(e.what());              \
+        return 1;                              \
+    }                                          \
+    catch (const std::exception &e) {          \
+        hemm_set_error(e.what());              \
+        return 2;                              \
+    }                                          \
+    return 0;
+
+static Matrix mat(const double *p, uint32_t rows, uint32_t cols) {
+    if (!p) throw std::invalid_argument("null matrix");
+    Matrix m(rows, cols);
+    memcpy(m.v.data(), p, sizeof(double) * m.v.size());
+    return m;
+}
+static void need(bool ok, const char *msg) {
+    if (!ok) throw std::invalid_argument(msg);
+}
+
+extern "C" {
+
+int hellm_hemmer_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64_t *primes, uint32_t dnum,
+                        uint32_t log_scale, uint32_t min_boot, uint64_t seed, hellm_hemmer **out) {
+    FACADE_TRY
+    need(primes && out, "null argument");
+    HEaaN::setSeed(seed);
+    std::vector<u64> q(primes, primes + n_q), p(primes + n_q, primes + n_q + n_p);
+    Context c = makeContextCustom(log_n, q, p, dnum, log_scale);
+    *out = new hellm_hemmer{new HEMMer(c, min_boot)};
+    FACADE_CATCH
+}
+int hellm_hemmer_create_preset(uint64_t seed, hellm_hemmer **out) {
+    FACADE_TRY
+    need(out, "null argument");
+    HEaaN::setSeed(seed);
+    *out = new hellm_hemmer{new HEMMer(0, ParameterPreset::FGb)};
+    FACADE_CATCH
+}
+void hellm_hemmer_destroy(hellm_hemmer *h) {
+    if (!h) return;
+    delete h->m;
+    delete h;
+}
+int hellm_hemmer_info(hellm_hemmer *h, uint32_t *log_n, uint32_t *n_q, uint32_t *n_p, uint32_t *dnum, uint32_t *dim,
+                      uint64_t *primes) {
+    FACADE_TRY
+    need(h, "null argument");
+    const Context &c = h->m->getContext();
+    if (log_n) *log_n = (uint32_t)c->logN;
+    if (n_q) *n_q = (uint32_t)c->nQ;
+    if (n_p) *n_p = (uint32_t)c->nP;
+    if (dnum) *dnum = (uint32_t)c->dnum;
+    if (dim) *dim = (uint32_t)h->m->dim();
+    if (primes) {
+        auto l = getPrimeList(c);
+        memcpy(primes, l.data(), l.size() * 8);
+    }
+    FACADE_CATCH
+}
+int hellm_secret_coeffs(hellm_hemmer *h, int32_t *out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    const auto &v = h->m->getsk().getCoefficients();
+    for (size_t i = 0; i < v.size(); i++) out[i] = v[i];
+    FACADE_CATCH
+}
+int hellm_export_key(hellm_hemmer *h, uint64_t galois, uint64_t *out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    const Context &c = h->m->getContext();
+    const size_t words = c->dnum * 2 * (c->nQ + c->nP) * c->N;
+    // the key pack is reachable through the evaluator's relinearize / rotate only; export via a friend path
+    const u64 *src = galois == 0 ? h->m->keyPack().multKey() : h->m->keyPack().galoisKey(galois);
+    if (hipMemcpy(out, src, words * 8, hipMemcpyDeviceToHost) != hipSuccess) throw RuntimeException("hipMemcpy failed");
+    FACADE_CATCH
+}
+int hellm_ensure_rotation_keys(hellm_hemmer *h, const uint64_t *rots, uint32_t count) {
+    FACADE_TRY
+    need(h && rots, "null argument");
+    h->m->ensureRotationKeys(std::vector<u64>(rots, rots + count));
+    FACADE_CATCH
+}
+int hellm_sync(void) {
+    FACADE_TRY
+    CudaTools::cudaDeviceSynchronize();
+    FACADE_CATCH
+}
+
+int hellm_encrypt(hellm_hemmer *h, const double *m, uint32_t rows, uint32_t cols, hellm_ct **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    *out = new hellm_ct{h->m->encrypt(mat(m, rows, cols))};
+    FACADE_CATCH
+}
+int hellm_encrypt2(hellm_hemmer *h, const double *a, const double *b, uint32_t rows, uint32_t cols, hellm_ct **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    *out = new hellm_ct{h->m->encrypt2(mat(a, rows, cols), mat(b, rows, cols))};
+    FACADE_CATCH
+}
+int hellm_encode(hellm_hemmer *h, const double *m, uint32_t rows, uint32_t cols, uint32_t level, hellm_pt **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    *out = new hellm_pt{h->m->encode(mat(m, rows, cols), level)};
+    FACADE_CATCH
+}
+int hellm_encode2(hellm_hemmer *h, const double *a, const double *b, uint32_t rows, uint32_t cols, uint32_t level,
+                  hellm_pt **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    *out = new hellm_pt{h->m->encode2(mat(a, rows, cols), mat(b, rows, cols), level)};
+    FACADE_CATCH
+}
+int hellm_encode_diagonal_to_row4(hellm_hemmer *h, const double *w1, const double *w2, const double *w3,
+                                  const double *w4, uint32_t rows, uint32_t cols, uint32_t level, hellm_pt **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    *out = new hellm_pt{h->m->encodeDiagonalToRow4(mat(w1, rows, cols), mat(w2, rows, cols), mat(w3, rows, cols),
+                                                   mat(w4, rows, cols), level)};
+    FACADE_CATCH
+}
+int hellm_decrypt(hellm_hemmer *h, const hellm_ct *ct, double *out) {
+    FACADE_TRY
+    need(h && ct && out, "null argument");
+    Matrix m = h->m->decrypt(ct->t);
+    memcpy(out, m.v.data(), m.v.size() * sizeof(double));
+    FACADE_CATCH
+}
+int hellm_decrypt2(hellm_hemmer *h, const hellm_ct *ct, double *out) {
+    FACADE_TRY
+    need(h && ct && out, "null argument");
+    auto ms = h->m->decrypt2(ct->t);
+    memcpy(out, ms[0].v.data(), ms[0].v.size() * sizeof(double));
+    memcpy(out + ms[0].v.size(), ms[1].v.data(), ms[1].v.size() * sizeof(double));
+    FACADE_CATCH
+}
+int hellm_decrypt_slots(hellm_hemmer *h, const hellm_ct *ct, double *re_im) {
+    FACADE_TRY
+    need(h && ct && re_im, "null argument");
+    Message msg(getLogFullSlots(h->m->getContext()));
+    h->m->getDec().decrypt(ct->t.get(), h->m->getsk(), msg);
+    for (u64 i = 0; i < msg.getSize(); i++) {
+        re_im[2 * i] = msg[i].real();
+        re_im[2 * i + 1] = msg[i].imag();
+    }
+    FACADE_CATCH
+}
+
+int hellm_ct_info(const hellm_ct *ct, uint32_t *num_poly, uint32_t *level, uint32_t *rc, uint32_t *rows,
+                  uint32_t *cols, uint32_t *bw) {
+    FACADE_TRY
+    need(ct, "null argument");
+    if (num_poly) *num_poly = (uint32_t)ct->t.get().getNumPoly();
+    if (level) *level = (uint32_t)ct->t.get().getLevel();
+    if (rc) *rc = (uint32_t)ct->t.get().getRescaleCounter();
+    if (rows) *rows = (uint32_t)ct->t.getHeight();
+    if (cols) *cols = (uint32_t)ct->t.getWidth();
+    if (bw) *bw = (uint32_t)ct->t.getBlockWidth();
+    FACADE_CATCH
+}
+int hellm_ct_download(const hellm_ct *ct, uint64_t *out) {
+    FACADE_TRY
+    need(ct && out, "null argument");
+    const Ciphertext &c = ct->t.get();
+    if (hipMemcpy(out, c.buf_.data(), c.buf_.words() * 8, hipMemcpyDeviceToHost) != hipSuccess)
+        throw RuntimeException("hipMemcpy failed");
+    FACADE_CATCH
+}
+int hellm_ct_upload(hellm_hemmer *h, const uint64_t *residues, uint32_t num_poly, uint32_t level, uint32_t rc,
+                    uint32_t rows, uint32_t cols, uint32_t bw, hellm_ct **out) {
+    FACADE_TRY
+    need(h && residues && out, "null argument");
+    const Context &c = h->m->getContext();
+    need(num_poly >= 1 && num_poly <= 3 && level < c->nQ, "bad ciphertext shape");
+    Ciphertext ct(c);
+    ct.allocate(num_poly, level, rc);
+    if (hipMemcpy(ct.buf_.data(), residues, ct.buf_.words() * 8, hipMemcpyHostToDevice) != hipSuccess)
+        throw RuntimeException("hipMemcpy failed");
+    *out = new hellm_ct{CtxtTensor(TileTensorShape(rows, cols, bw), ct)};
+    FACADE_CATCH
+}
+int hellm_ct_clone(const hellm_ct *ct, hellm_ct **out) {
+    FACADE_TRY
+    need(ct && out, "null argument");
+    *out = new hellm_ct{ct->t};
+    FACADE_CATCH
+}
+void hellm_ct_destroy(hellm_ct *ct) { delete ct; }
+void hellm_pt_destroy(hellm_pt *pt) { delete pt; }
+int hellm_pt_download(const hellm_pt *pt, uint32_t *level, uint64_t *out) {
+    FACADE_TRY
+    need(pt, "null argument");
+    if (level) *level = (uint32_t)pt->t.getLevel();
+    if (out && hipMemcpy(out, pt->t.get().buf_.data(), pt->t.get().buf_.words() * 8, hipMemcpyDeviceToHost) != hipSuccess)
+        throw RuntimeException("hipMemcpy failed");
+    FACADE_CATCH
+}
+void hellm_ctvec_destroy(hellm_ctvec *v) { delete v; }
+int hellm_ctvec_size(const hellm_ctvec *v, uint32_t *out) {
+    FACADE_TRY
+    need(v && out, "null argument");
+    *out = (uint32_t)v->v.size();
+    FACADE_CATCH
+}
+int hellm_ctvec_get(const hellm_ctvec *v, uint32_t i, uint32_t rows, uint32_t cols, uint32_t bw, hellm_ct **out) {
+    FACADE_TRY
+    need(v && out && i < v->v.size(), "bad argument");
+    *out = new hellm_ct{CtxtTensor(TileTensorShape(rows, cols, bw), v->v[i])};
+    FACADE_CATCH
+}
+
+#define UNARY_EVAL(name, expr)                                        \
+    int name(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out) {    \
+        FACADE_TRY                                                    \
+        need(h && a && out, "null argument");                         \
+        hellm_ct *r = new hellm_ct{a->t};                             \
+        try {                                                         \
+            expr;                                                     \
+        } catch (...) {                                               \
+            delete r;                                                 \
+            throw;                                                    \
+        }                                                             \
+        *out = r;                                                     \
+        FACADE_CATCH                                                  \
+    }
+
+int hellm_left_rotate(hellm_hemmer *h, const hellm_ct *a, uint64_t rot, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    h->m->ensureRotationKeys({rot});
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().leftRotate(a->t.get(), rot, r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+UNARY_EVAL(hellm_conjugate, h->m->getEval().conjugate(a->t.get(), r->t.get()))
+UNARY_EVAL(hellm_mult_imag_unit, h->m->getEval().multImagUnit(a->t.get(), r->t.get()))
+UNARY_EVAL(hellm_diagonal_to_column, r->t = h->m->diagonalToColumn(a->t))
+UNARY_EVAL(hellm_diagonal_to_row, r->t = h->m->diagonalToRow(a->t))
+
+int hellm_mult(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().mult(a->t.get(), b->t.get(), r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().add(a->t.get(), b->t.get(), r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().levelDown(a->t.get(), target, r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+
+int hellm_transpose_inplace(hellm_hemmer *h, hellm_ct *a, uint32_t T) {
+    FACADE_TRY
+    need(h && a, "null argument");
+    h->m->transposeInplace(a->t, T);
+    FACADE_CATCH
+}
+int hellm_complex_packing_inplace(hellm_hemmer *h, hellm_ct *a) {
+    FACADE_TRY
+    need(h && a, "null argument");
+    h->m->complexPackingInplace(a->t);
+    FACADE_CATCH
+}
+int hellm_complex_packing_row_inplace(hellm_hemmer *h, hellm_ct *a) {
+    FACADE_TRY
+    need(h && a, "null argument");
+    h->m->complexPackingRowInplace(a->t);
+    FACADE_CATCH
+}
+int hellm_transpose_complex_packing_inplace(hellm_hemmer *h, hellm_ct *a, uint32_t T) {
+    FACADE_TRY
+    need(h && a, "null argument");
+    h->m->transposeComplexPackingInplace(a->t, T);
+    FACADE_CATCH
+}
+int hellm_split_in_two(hellm_hemmer *h, hellm_ct *a, hellm_ct **o1, hellm_ct **o2) {
+    FACADE_TRY
+    need(h && a && o1 && o2, "null argument");
+    hellm_ct *r1 = new hellm_ct{a->t}, *r2 = new hellm_ct{a->t};
+    h->m->splitInTwo(a->t, r1->t, r2->t);
+    *o1 = r1;
+    *o2 = r2;
+    FACADE_CATCH
+}
+
+#define BINARY_MM(name, BT, call)                                                                   \
+    int name(hellm_hemmer *h, const hellm_ct *a, const BT *b, uint32_t T, hellm_ct **out) {          \
+        FACADE_TRY                                                                                   \
+        need(h && a && b && out, "null argument");                                                   \
+        *out = new hellm_ct{h->m->call(a->t, b->t, T)};                                              \
+        FACADE_CATCH                                                                                 \
+    }
+BINARY_MM(hellm_single_cc_matmul, hellm_ct, singleCCMatMul)
+BINARY_MM(hellm_single_matmul, hellm_pt, singleMatMul)
+BINARY_MM(hellm_packed_matmul, hellm_ct, packedMatMul)
+
+#define UNARY_MM(name, call)                                                      \
+    int name(hellm_hemmer *h, const hellm_ct *a, uint32_t T, hellm_ct **out) {    \
+        FACADE_TRY                                                                \
+        need(h && a && out, "null argument");                                     \
+        *out = new hellm_ct{h->m->call(a->t, T)};                                 \
+        FACADE_CATCH                                                              \
+    }
+UNARY_MM(hellm_packed_matmul_pre, packedMatMulPre)
+UNARY_MM(hellm_packed_matmul_pre_rev, packedMatMulPreRev)
+UNARY_MM(hellm_matmul_pre_rev, matMulPreRev)
+
+int hellm_packed_matmul_pre_rot(hellm_hemmer *h, const hellm_ct *a, uint32_t T, hellm_ctvec **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ctvec *v = new hellm_ctvec();
+    try {
+        h->m->packedMatMulPreRot(a->t, v->v, T);
+    } catch (...) {
+        delete v;
+        throw;
+    }
+    *out = v;
+    FACADE_CATCH
+}
+int hellm_matmul_pre(hellm_hemmer *h, const hellm_ct *a, uint32_t T, hellm_ctvec **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ctvec *v = new hellm_ctvec();
+    try {
+        h->m->matMulPre(a->t, v->v, T);
+    } catch (...) {
+        delete v;
+        throw;
+    }
+    *out = v;
+    FACADE_CATCH
+}
+int hellm_packed_matmul_cc_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const hellm_ct *b, uint32_t T,
+                                 hellm_ct **out) {
+    FACADE_TRY
+    need(h && tmp && b && out, "null argument");
+    *out = new hellm_ct{h->m->packedMatMulCCReuse(tmp->v, b->t, T)};
+    FACADE_CATCH
+}
+int hellm_matmul_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const hellm_pt *b, uint32_t T, hellm_ct **out) {
+    FACADE_TRY
+    need(h && tmp && b && out, "null argument");
+    *out = new hellm_ct{h->m->matMulReUse(tmp->v, b->t, T)};
+    FACADE_CATCH
+}
+int hellm_matmul_cc_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const hellm_ct *b, uint32_t T, hellm_ct **out) {
+    FACADE_TRY
+    need(h && tmp && b && out, "null argument");
+    *out = new hellm_ct{h->m->matMulCCReUse(tmp->v, b->t, T)};
+    FACADE_CATCH
+}
+int hellm_repack_cc(hellm_hemmer *h, hellm_ct *a, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    *out = new hellm_ct{h->m->repackCC(a->t)};
+    FACADE_CATCH
+}
+int hellm_complex_packing(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->complexPacking(a->t, b->t)};
+    FACADE_CATCH
+}
+int hellm_complex_packing_rev(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->complexPackingRev(a->t, b->t)};
+    FACADE_CATCH
+}
+int hellm_repack_not_bts(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->repack_notBTS(a->t, b->t)};
+    FACADE_CATCH
+}
+
+}  // extern "C"

@@ -1,0 +1,380 @@
+// HEMMer facade (reference: ciphertext/src/HEMMer.cpp, codec :232-416,:579-638, packing :764-831,
+// matmul entry points :833-880,:964-1124, transpose :1166-1172, masks :2336-2400).
+#include <cmath>
+
+#include "HELLM/HEMMer.hpp"
+
+namespace HELLM {
+
+static MatrixTransformer matrix_transformer;
+void cleanUpMatrixTransformer() { matrix_transformer.cleanUp(); }
+
+namespace {
+enum { MASK_COL_EVEN = 0, MASK_ROW_EVEN = 1, MASK_LEFT_HALF = 2, MASK_MATMUL = 3 };
+
+i64 tileDim(u64 log_slots) {
+    if (log_slots < 3 || (log_slots & 1) == 0)
+        throw RuntimeException("HEMMer needs 2 * n * n slots: the number of slots must be an odd power of two");
+    return i64(1) << ((log_slots - 1) / 2);
+}
+i64 pow2ceil(i64 v) {
+    i64 p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+}  // namespace
+
+HEMMer HEMMer::genHEMMer(int device_id, ParameterPreset preset, const bool) { return HEMMer(device_id, preset); }
+
+HEMMer::HEMMer(int device_id, ParameterPreset preset)
+    : device_id_(device_id), context_(makeContext(preset, {device_id})), log_slots_(getLogFullSlots(context_)),
+      dim_(tileDim(log_slots_)), sk_(context_), enc_(context_), dec_(context_), endec_(context_), pack_(context_),
+      eval_(context_, pack_), btp_(eval_, 3) {
+    init();
+}
+HEMMer::HEMMer(const Context &context, u64 min_bootstrap_level)
+    : context_(context), log_slots_(getLogFullSlots(context_)), dim_(tileDim(log_slots_)), sk_(context_),
+      enc_(context_), dec_(context_), endec_(context_), pack_(context_), eval_(context_, pack_),
+      btp_(eval_, min_bootstrap_level) {
+    init();
+}
+HEMMer::HEMMer(const std::string &key_path, int device_id, ParameterPreset preset)
+    : device_id_(device_id), context_(makeContext(preset, {device_id})), log_slots_(getLogFullSlots(context_)),
+      dim_(tileDim(log_slots_)), sk_(context_, key_path + "/SecretKey.bin"), enc_(context_), dec_(context_),
+      endec_(context_), pack_(context_, key_path), eval_(context_, pack_), btp_(eval_, 3) {
+    init();
+}
+HEMMer::~HEMMer() = default;
+
+void HEMMer::init() {
+    KeyGenerator keygen(context_, sk_, pack_);
+    if (!pack_.hasMultKey()) keygen.genMultKey();
+    keygen.genConjKey();
+    const i64 n = dim_;
+    Matrix even(n, n), tr_even(n, n), ones(n, n, 1.0), zeros(n, n, 0.0);
+    for (i64 r = 0; r < n; r++)
+        for (i64 c = 0; c < n; c++) {
+            even.at(r, c) = (c % 2 == 0) ? 1.0 : 0.0;
+            tr_even.at(r, c) = (r % 2 == 0) ? 1.0 : 0.0;
+        }
+    col_mask_even_ = message2(even, even);
+    row_mask_even_ = message2(tr_even, tr_even);
+    mask_left_half_ = message2(ones, zeros);
+    mask_matmul_ = message2(ones, zeros);
+}
+
+void HEMMer::save(const std::string &keys_path) {
+    sk_.save(keys_path + "/SecretKey.bin");
+    pack_.save(keys_path);
+}
+
+const Plaintext &HEMMer::cachedMask(int id, u64 level) const {
+    auto key = std::make_pair(id, level);
+    auto it = mask_cache_.find(key);
+    if (it != mask_cache_.end()) return it->second;
+    const Message *m = id == MASK_COL_EVEN ? &col_mask_even_
+                       : id == MASK_ROW_EVEN ? &row_mask_even_
+                       : id == MASK_LEFT_HALF ? &mask_left_half_
+                                              : &mask_matmul_;
+    return mask_cache_.emplace(key, endec_.encode(*m, level)).first->second;
+}
+
+void HEMMer::ensureRotationKeys(const std::vector<u64> &rots) const {
+    const u64 slots = u64(1) << log_slots_;
+    KeyGenerator keygen(context_, sk_, pack_);
+    for (u64 r : rots) {
+        r %= slots;
+        if (r == 0 || have_rot_.count(r)) continue;
+        keygen.genLeftRotKey(r);
+        have_rot_.insert(r);
+    }
+}
+
+// rotations issued by a diagonal transform of `kind` on tiles in rows of `width` slots
+std::vector<u64> HEMMer::transformRotations(MaskKind kind, i64 width) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 n = dim_;
+    std::vector<u64> r;
+    auto left = [&](i64 v) { r.push_back((u64)(((v % (i64)slots) + (i64)slots) % (i64)slots)); };
+    if (kind == MaskKind::Diagonal) {
+        const i64 count = 2 * n - 1, bs = (i64)std::ceil(std::sqrt((double)count)),
+                  gs = (i64)std::ceil((double)count / (double)bs), step = width - 1;
+        left(-(n - 1) * step);
+        left(step);
+        for (i64 i = 1; i < gs; i++) left(i * bs * step);
+        return r;
+    }
+    const bool packed = kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical;
+    const bool vertical = kind == MaskKind::Vertical || kind == MaskKind::PackedVertical;
+    const i64 cell = packed ? 2 : 1, units = n / cell, step = cell * (vertical ? width : 1);
+    const i64 bs = (i64)std::ceil(std::sqrt((double)(2 * units - 1))),
+              gs = (i64)std::ceil((double)(units - 1) / (double)bs);
+    left(step);
+    for (i64 i = 0; i < gs; i++) {
+        left(-(units - i * bs) * step);
+        if (i > 0) left(i * bs * step);
+    }
+    return r;
+}
+
+// ---- codec ---------------------------------------------------------------------------------------------
+Message HEMMer::message2(const Matrix &a, const Matrix &b) const {
+    if (a.rows != b.rows || a.cols != b.cols) throw RuntimeException("message2: shapes differ");
+    Message msg(log_slots_, 0);
+    if ((u64)(2 * a.rows * a.cols) > msg.getSize()) throw RuntimeException("message2: matrices do not fit");
+    for (i64 r = 0; r < a.rows; r++)
+        for (i64 c = 0; c < a.cols; c++) {
+            msg[(u64)(r * 2 * a.cols + c)] = a.at(r, c);
+            msg[(u64)(r * 2 * a.cols + a.cols + c)] = b.at(r, c);
+        }
+    return msg;
+}
+PtxtTensor HEMMer::encode(const Matrix &data, u64 level) const {
+    Message msg(log_slots_, 0);
+    if (data.v.size() > msg.getSize()) throw RuntimeException("encode: matrix does not fit");
+    for (size_t i = 0; i < data.v.size(); i++) msg[i] = data.v[i];
+    if (level == 0) level = getEncryptionLevel(context_);
+    return PtxtTensor(data.rows, data.cols, endec_.encode(msg, level));
+}
+PtxtTensor HEMMer::encode2(const Matrix &a, const Matrix &b, u64 level) const {
+    Message msg = message2(a, b);
+    if (level == 0) level = getEncryptionLevel(context_);
+    return PtxtTensor(a.rows, a.cols, endec_.encode(msg, level), a.cols * 2);
+}
+// weight layout of the hoisted plaintext product: 0.5 (W1 - i W3) | 0.5 (W2 - i W4), column j of each
+// half rolled up by j (the tau layout)
+Message HEMMer::msgDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4) const {
+    const i64 h = w1.rows, w = w1.cols;
+    Message msg(log_slots_, 0);
+    if ((u64)(2 * h * w) > msg.getSize()) throw RuntimeException("msgDiagonalToRow4: matrices do not fit");
+    for (i64 r = 0; r < h; r++)
+        for (i64 c = 0; c < w; c++) {
+            const i64 src = (r + c) % h;
+            msg[(u64)(r * 2 * w + c)] = Complex(0.5 * w1.at(src, c), -0.5 * w3.at(src, c));
+            msg[(u64)(r * 2 * w + w + c)] = Complex(0.5 * w2.at(src, c), -0.5 * w4.at(src, c));
+        }
+    return msg;
+}
+PtxtTensor HEMMer::encodeDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4,
+                                        u64 level) const {
+    Message msg = msgDiagonalToRow4(w1, w2, w3, w4);
+    if (level == 0) level = getEncryptionLevel(context_);
+    return PtxtTensor(w1.rows, w1.cols, endec_.encode(msg, level), w1.cols * 2);
+}
+CtxtTensor HEMMer::encrypt(const Matrix &data) const {
+    PtxtTensor p = encode(data);
+    CtxtTensor ret(context_, p.getShape());
+    enc_.encrypt(p.get(), sk_, ret.get());
+    return ret;
+}
+CtxtTensor HEMMer::encrypt2(const Matrix &a, const Matrix &b) const {
+    PtxtTensor p = encode2(a, b);
+    CtxtTensor ret(context_, p.getShape());
+    enc_.encrypt(p.get(), sk_, ret.get());
+    return ret;
+}
+Matrix HEMMer::decrypt(const CtxtTensor &t) const {
+    Message msg(log_slots_);
+    dec_.decrypt(t.get(), sk_, msg);
+    Matrix m(t.getHeight(), t.getWidth());
+    for (size_t i = 0; i < m.v.size(); i++) m.v[i] = msg[i].real();
+    return m;
+}
+std::vector<Matrix> HEMMer::decrypt2(const CtxtTensor &t) const {
+    Message msg(log_slots_);
+    dec_.decrypt(t.get(), sk_, msg);
+    const i64 h = t.getHeight(), w = t.getWidth();
+    std::vector<Matrix> out(2, Matrix(h, w));
+    for (i64 r = 0; r < h; r++)
+        for (i64 c = 0; c < w; c++) {
+            out[0].at(r, c) = msg[(u64)(r * 2 * w + c)].real();
+            out[1].at(r, c) = msg[(u64)(r * 2 * w + w + c)].real();
+        }
+    return out;
+}
+
+// ---- packing ---------------------------------------------------------------------------------------------
+void HEMMer::transposeInplace(CtxtTensor &t, u64 target_level) const {
+    ensureRotationKeys(transformRotations(MaskKind::Diagonal, t.getBlockWidth()));
+    if (target_level > 0) eval_.levelDown(t.get(), 1 + target_level, t.get());
+    t = matrix_transformer.transpose(eval_, t);
+}
+
+// adjacent columns (2c, 2c+1) -> a + i b, written to both slots of the pair
+void HEMMer::complexPackingInplace(CtxtTensor &t) const {
+    const u64 slots = u64(1) << log_slots_;
+    ensureRotationKeys({1, slots - 1});
+    Ciphertext odd(context_), even(context_), fus(context_);
+    const Plaintext &m = cachedMask(MASK_COL_EVEN, t.getLevel());
+    eval_.mult(t.get(), m, even);
+    eval_.leftRotate(t.get(), 1, odd);
+    eval_.multImagUnit(odd, odd);
+    eval_.mult(odd, m, odd);
+    eval_.add(odd, even, fus);
+    eval_.rightRotate(fus, 1, t.get());
+    eval_.add(t.get(), fus, t.get());
+}
+void HEMMer::transposeComplexPackingInplace(CtxtTensor &t, u64 target_level) const {
+    const u64 slots = u64(1) << log_slots_;
+    ensureRotationKeys({1, slots - 1});
+    Ciphertext odd(context_), even(context_), fus(context_);
+    const Plaintext &m = cachedMask(MASK_COL_EVEN, t.getLevel());
+    eval_.mult(t.get(), m, even);
+    eval_.leftRotate(t.get(), 1, odd);
+    eval_.multImagUnit(odd, odd);
+    eval_.negate(odd, odd);
+    eval_.mult(odd, m, odd);
+    eval_.add(odd, even, fus);
+    eval_.rightRotate(fus, 1, t.get());
+    eval_.add(t.get(), fus, t.get());
+    if (target_level > 0) eval_.levelDown(t.get(), 1 + target_level, t.get());
+    transposeInplace(t);
+}
+// adjacent rows (2k, 2k+1) -> a - i b, written to both rows of the pair
+void HEMMer::complexPackingRowInplace(CtxtTensor &t) const {
+    const u64 slots = u64(1) << log_slots_, w = (u64)t.getBlockWidth();
+    ensureRotationKeys({w, slots - w});
+    Ciphertext odd(context_), even(context_), fus(context_);
+    const Plaintext &m = cachedMask(MASK_ROW_EVEN, t.getLevel());
+    eval_.mult(t.get(), m, even);
+    eval_.leftRotate(t.get(), w, odd);
+    eval_.multImagUnit(odd, odd);
+    eval_.negate(odd, odd);
+    eval_.mult(odd, m, odd);
+    eval_.add(even, odd, fus);
+    eval_.rightRotate(fus, w, t.get());
+    eval_.add(t.get(), fus, t.get());
+}
+void HEMMer::splitInTwo(CtxtTensor &t, CtxtTensor &t1, CtxtTensor &t2) const {
+    const u64 slots = u64(1) << log_slots_, width = (u64)t.getWidth();
+    ensureRotationKeys({width, slots - width});
+    Ciphertext tmp(context_), low(context_);
+    eval_.mult(t.get(), cachedMask(MASK_LEFT_HALF, t.getLevel()), tmp);
+    eval_.levelDown(t.get(), tmp.getLevel(), low);
+    eval_.sub(low, tmp, t2.get());
+    eval_.rightRotate(tmp, width, t1.get());
+    eval_.add(t1.get(), tmp, t1.get());
+    eval_.leftRotate(t2.get(), width, tmp);
+    eval_.add(t2.get(), tmp, t2.get());
+}
+
+// ---- products ---------------------------------------------------------------------------------------------
+CtxtTensor HEMMer::diagonalToColumn(const CtxtTensor &a) const {
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getBlockWidth()));
+    return matrix_transformer.diagonalToColumn(eval_, a);
+}
+CtxtTensor HEMMer::diagonalToRow(const CtxtTensor &b) const {
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, b.getBlockWidth()));
+    return matrix_transformer.diagonalToRow(eval_, b);
+}
+CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
+    ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});
+    return multMatMat(eval_, btp_, a, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::singleMatMul(const CtxtTensor &a, const PtxtTensor &b, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
+    ensureRotationKeys({1, slots - (u64)n});
+    return multMatMat(eval_, btp_, a, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
+    ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
+    ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
+    ensureRotationKeys({2, (u64)(2 * w), slots - (u64)n});
+    return multPackedMatMat(eval_, btp_, a, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::packedMatMulPre(const CtxtTensor &a, u64 T) const {
+    ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, a.getBlockWidth()));
+    return multPackedMatMatPre(eval_, a, T, matrix_transformer);
+}
+void HEMMer::packedMatMulPreRot(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    ensureRotationKeys({2, slots - (u64)a.getHeight()});
+    multPackedMatMatPreRot(eval_, a, tmp, T, matrix_transformer);
+}
+CtxtTensor HEMMer::packedMatMulPreRev(const CtxtTensor &b, u64 T) const {
+    ensureRotationKeys(transformRotations(MaskKind::PackedVertical, b.getBlockWidth()));
+    return multPackedMatMatPreRev(eval_, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::packedMatMulCCReuse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 T) const {
+    ensureRotationKeys({(u64)(2 * b.getBlockWidth())});
+    return multPackedMatMatCCReuse(eval_, tmp, b, T, matrix_transformer);
+}
+void HEMMer::matMulPre(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getBlockWidth()));
+    ensureRotationKeys({1, slots - (u64)a.getHeight()});
+    multMatMatPre(eval_, a, tmp, T, matrix_transformer);
+}
+CtxtTensor HEMMer::matMulReUse(const std::vector<Ciphertext> &tmp, const PtxtTensor &b, u64 T) const {
+    return multMatMatReUse(eval_, tmp, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::matMulPreRev(const CtxtTensor &b, u64 T) const {
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, b.getBlockWidth()));
+    return multMatMatPreRev(eval_, b, T, matrix_transformer);
+}
+CtxtTensor HEMMer::matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 T) const {
+    ensureRotationKeys({(u64)b.getBlockWidth()});
+    return multMatMatCCReUse(eval_, tmp, b, T, matrix_transformer);
+}
+
+// x + conj(x) = 2 Re(x)
+CtxtTensor HEMMer::repackCC(CtxtTensor &t) const {
+    CtxtTensor out(t);
+    eval_.conjugate(t.get(), out.get());
+    eval_.add(t.get(), out.get(), out.get());
+    return out;
+}
+PtxtTensor HEMMer::complexPacking(const PtxtTensor &a, const PtxtTensor &b) const {
+    // 0.5 a - 0.5 i b on the decoded values
+    Message ma = endec_.decode(a.get()), mb = endec_.decode(b.get());
+    for (u64 i = 0; i < ma.getSize(); i++) ma[i] = 0.5 * ma[i] - Complex(0, 0.5) * mb[i];
+    return PtxtTensor(a.getShape(), endec_.encode(ma, std::min(a.getLevel(), b.getLevel())));
+}
+CtxtTensor HEMMer::complexPacking(const CtxtTensor &a, const CtxtTensor &b) const {
+    CtxtTensor res(b);
+    eval_.multImagUnit(b.get(), res.get());
+    eval_.add(a.get(), res.get(), res.get());
+    return res;
+}
+CtxtTensor HEMMer::complexPackingRev(const CtxtTensor &a, const CtxtTensor &b) const {
+    CtxtTensor res(b);
+    eval_.multImagUnit(b.get(), res.get());
+    eval_.sub(a.get(), res.get(), res.get());
+    return res;
+}
+CtxtTensor HEMMer::repack_notBTS(CtxtTensor &t1, CtxtTensor &t2) const {
+    const u64 slots = u64(1) << log_slots_, n = (u64)dim_;
+    ensureRotationKeys({n, slots - n});
+    CtxtTensor out(t1), tmp(t2);
+    if (t1.get().getRescaleCounter() > 0) eval_.rescale(t1.get());
+    if (t2.get().getRescaleCounter() > 0) eval_.rescale(t2.get());
+    eval_.conjugate(t1.get(), out.get());
+    eval_.add(t1.get(), out.get(), out.get());
+    eval_.conjugate(t2.get(), tmp.get());
+    eval_.add(t2.get(), tmp.get(), tmp.get());
+    eval_.multImagUnit(tmp.get(), tmp.get());
+    eval_.add(out.get(), tmp.get(), out.get());
+    eval_.leftRotate(out.get(), n, tmp.get());
+    eval_.add(out.get(), tmp.get(), out.get());
+    const Plaintext &m = cachedMask(MASK_MATMUL, out.getLevel());
+    eval_.mult(tmp.get(), m, tmp.get());
+    eval_.mult(out.get(), m, out.get());
+    eval_.rightRotate(tmp.get(), n, tmp.get());
+    addInplace(out, tmp);
+    return out;
+}
+CtxtTensor HEMMer::repack(CtxtTensor &t1, CtxtTensor &) const {
+    Ciphertext dummy(context_);
+    btp_.bootstrapExtended(t1.get(), dummy);  // throws: bootstrapping is outside this build
+    return t1;
+}
+
+}  // namespace HELLM

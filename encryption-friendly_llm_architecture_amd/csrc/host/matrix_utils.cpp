@@ -1,0 +1,611 @@
+// sigma / tau / transpose transforms and the matrix products of HELLM/MatrixUtils.hpp.
+// Follows the algorithm of the reference's ciphertext/src/MatrixUtils.cpp (mask families :90-578,
+// transforms :671-1098, products :1100-1679) restated over this build's evaluator.
+#include <cmath>
+
+#include "HELLM/MatrixUtils.hpp"
+
+namespace HELLM {
+
+namespace {
+
+i64 pow2ceil(i64 v) {
+    i64 p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+// baby-step / giant-step geometry of a transform kind
+struct Geometry {
+    i64 n;       // tile side (values)
+    i64 units;   // diagonals counted in cells: n (plain) or n / 2 (packed)
+    i64 cell;    // 1 or 2
+    i64 bs, gs;
+    i64 step;    // slots moved per unit diagonal
+};
+
+Geometry geometry(MaskKind kind, const TileTensorShape &s) {
+    Geometry g{};
+    const i64 rows = s.getNumRows(), cols = s.getNumCols(), w = s.getBlockWidth();
+    if (rows != cols) throw std::invalid_argument("[MatrixTransformer] only square tiles are supported");
+    g.n = rows;
+    if (kind == MaskKind::Diagonal) {
+        g.units = g.n;
+        g.cell = 1;
+        const i64 count = 2 * g.n - 1;
+        g.bs = (i64)std::ceil(std::sqrt((double)count));
+        g.gs = (i64)std::ceil((double)count / (double)g.bs);
+        g.step = w - 1;
+        return g;
+    }
+    const bool packed = (kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical);
+    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
+    g.cell = packed ? 2 : 1;
+    g.units = g.n / g.cell;
+    g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.units - 1)));
+    g.gs = (i64)std::ceil((double)(g.units - 1) / (double)g.bs);
+    g.step = g.cell * (vertical ? w : 1);
+    return g;
+}
+
+}  // namespace
+
+Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, i64 idx) {
+    const Geometry g = geometry(kind, shape);
+    const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, height = slots / w;
+    Message m(log_slots, 0);
+    const double value = (kind == MaskKind::PackedHorizontal) ? 0.5 : 1.0;
+    for (i64 r = 0; r < height; r++)
+        for (i64 c = 0; c < w; c++) {
+            const i64 R = (r % g.n) / g.cell, C = (c % g.n) / g.cell;
+            bool on;
+            switch (kind) {
+                case MaskKind::Horizontal:
+                case MaskKind::PackedHorizontal:
+                    on = idx >= 0 ? (R == idx && C < g.units - idx) : (R == g.units + idx && C >= -idx);
+                    break;
+                case MaskKind::Vertical:
+                case MaskKind::PackedVertical:
+                    on = idx >= 0 ? (C == idx && R < g.units - idx) : (C == g.units + idx && R >= -idx);
+                    break;
+                default:  // Diagonal: output positions with column - row == idx
+                    on = (C - R == idx);
+            }
+            if (on) m[(u64)(r * w + c)] = value;
+        }
+    return m;
+}
+
+const Plaintext &MatrixTransformer::transformMask(const HomEvaluator &eval, MaskKind kind,
+                                                  const TileTensorShape &shape, u64 level, i64 idx) {
+    Key key{(int)kind, shape, level, idx};
+    auto it = masks_.find(key);
+    if (it != masks_.end()) return it->second;
+    const Context &ctx = eval.getContext();
+    const u64 log_slots = getLogFullSlots(ctx);
+    const Geometry g = geometry(kind, shape);
+    Message m = transformMaskMessage(kind, shape, log_slots, idx);
+    // pre-rotation so the mask can be applied before the giant-step rotation of its group
+    if (kind == MaskKind::Diagonal) {
+        const i64 i = (idx + (g.n - 1)) / g.bs;
+        eval.rightRotate(m, (u64)(i * g.bs * g.step), m);
+    } else if (idx > 0) {
+        const i64 i = (idx - 1) / g.bs;
+        eval.rightRotate(m, (u64)(i * g.bs * g.step), m);
+    } else if (idx < 0) {
+        const i64 i = (idx + g.units - 1) / g.bs;
+        eval.leftRotate(m, (u64)((g.units - i * g.bs) * g.step), m);
+    }
+    auto res = masks_.emplace(key, EnDecoder(ctx).encode(m, level));
+    return res.first->second;
+}
+
+std::vector<Plaintext> &MatrixTransformer::getColMask(const HomEvaluator &eval, const TileTensorShape &shape,
+                                                      u64 level) {
+    auto key = std::make_pair(shape, level);
+    auto it = col_masks_.find(key);
+    if (it != col_masks_.end()) return it->second;
+    const Context &ctx = eval.getContext();
+    const u64 log_slots = getLogFullSlots(ctx);
+    const i64 n = shape.getNumCols(), slots = i64(1) << log_slots;
+    EnDecoder endec(ctx);
+    std::vector<Plaintext> v;
+    v.reserve((size_t)(2 * n));
+    for (i64 i = 0; i < n; i++) {
+        Message wrap(log_slots, 0), main(log_slots, 0);
+        for (i64 j = 0; j < slots; j++) {
+            if (j % n < n - i)
+                main[(u64)j] = 1;
+            else
+                wrap[(u64)j] = 1;
+        }
+        v.push_back(endec.encode(wrap, level));
+        v.push_back(endec.encode(main, level));
+    }
+    return col_masks_.emplace(key, std::move(v)).first->second;
+}
+
+std::vector<Plaintext> &MatrixTransformer::getRowMask(const HomEvaluator &eval, const TileTensorShape &shape,
+                                                      u64 level) {
+    auto key = std::make_pair(shape, level);
+    auto it = row_masks_.find(key);
+    if (it != row_masks_.end()) return it->second;
+    const Context &ctx = eval.getContext();
+    const u64 log_slots = getLogFullSlots(ctx);
+    const i64 n = shape.getNumRows(), w = shape.getBlockWidth(), slots = i64(1) << log_slots;
+    EnDecoder endec(ctx);
+    std::vector<Plaintext> v;
+    v.reserve((size_t)(2 * n));
+    for (i64 i = 0; i < n; i++) {
+        Message wrap(log_slots, 0), main(log_slots, 0);
+        for (i64 j = 0; j < slots; j++) {
+            if ((j / w) % n < n - i)
+                main[(u64)j] = 1;
+            else
+                wrap[(u64)j] = 1;
+        }
+        v.push_back(endec.encode(wrap, level));
+        v.push_back(endec.encode(main, level));
+    }
+    return row_masks_.emplace(key, std::move(v)).first->second;
+}
+
+void MatrixTransformer::cleanUp() {
+    masks_.clear();
+    col_masks_.clear();
+    row_masks_.clear();
+}
+size_t MatrixTransformer::cachedMasks() const {
+    size_t n = masks_.size();
+    for (auto &kv : col_masks_) n += kv.second.size();
+    for (auto &kv : row_masks_) n += kv.second.size();
+    return n;
+}
+
+// T(A) = M_0 * A + sum_{d != 0} M_d * rot_{d step}(A), d in (-units, units), grouped so that only
+// bs baby rotations of A and 2 gs giant rotations of partial sums are key switched.  All products
+// are summed at the doubled scale and rescaled once.
+Ciphertext MatrixTransformer::diagonalTransform(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                                const TileTensorShape &shape) {
+    const Context &ctx = eval.getContext();
+    const Geometry g = geometry(kind, shape);
+    const u64 level = in.getLevel();
+    if (level == 0) throw std::invalid_argument("[diagonalTransform] level >= 1 is needed.");
+    std::vector<Ciphertext> baby;
+    baby.reserve((size_t)g.bs);
+    for (i64 j = 0; j < g.bs; j++) {
+        baby.emplace_back(ctx);
+        eval.leftRotate(j == 0 ? in : baby[(size_t)j - 1], (u64)g.step, baby[(size_t)j]);
+    }
+    Ciphertext res(ctx), group(ctx), tmp(ctx);
+    eval.multWithoutRescale(in, transformMask(eval, kind, shape, level, 0), res);
+    for (i64 i = 0; i < g.gs; i++) {
+        // wrapped diagonals d = 1 + i bs + j - units < 0
+        bool any = false;
+        for (i64 j = 0; j < g.bs; j++) {
+            const i64 d = 1 + i * g.bs + j - g.units;
+            if (d >= 0) break;
+            eval.multWithoutRescale(baby[(size_t)j], transformMask(eval, kind, shape, level, d), any ? tmp : group);
+            if (any) eval.add(group, tmp, group);
+            any = true;
+        }
+        if (any) {
+            eval.rightRotate(group, (u64)((g.units - i * g.bs) * g.step), group);
+            eval.add(res, group, res);
+        }
+        // diagonals d = 1 + i bs + j > 0
+        any = false;
+        for (i64 j = 0; j < g.bs; j++) {
+            const i64 d = 1 + i * g.bs + j;
+            if (d >= g.units) break;
+            eval.multWithoutRescale(baby[(size_t)j], transformMask(eval, kind, shape, level, d), any ? tmp : group);
+            if (any) eval.add(group, tmp, group);
+            any = true;
+        }
+        if (any) {
+            if (i > 0) eval.leftRotate(group, (u64)(i * g.bs * g.step), group);
+            eval.add(res, group, res);
+        }
+    }
+    eval.rescale(res);
+    return res;
+}
+
+template <>
+CtxtTensor MatrixTransformer::diagonalToColumn<Ciphertext>(const HomEvaluator &eval, const CtxtTensor &op) {
+    return CtxtTensor(op.getShape(), diagonalTransform(eval, op.get(), MaskKind::Horizontal, op.getShape()));
+}
+template <>
+CtxtTensor MatrixTransformer::diagonalToRow<Ciphertext>(const HomEvaluator &eval, const CtxtTensor &op) {
+    return CtxtTensor(op.getShape(), diagonalTransform(eval, op.get(), MaskKind::Vertical, op.getShape()));
+}
+CtxtTensor MatrixTransformer::packedDiagonalToColumn(const HomEvaluator &eval, const CtxtTensor &op) {
+    return CtxtTensor(op.getShape(), diagonalTransform(eval, op.get(), MaskKind::PackedHorizontal, op.getShape()));
+}
+CtxtTensor MatrixTransformer::packedDiagonalToRow(const HomEvaluator &eval, const CtxtTensor &op) {
+    return CtxtTensor(op.getShape(), diagonalTransform(eval, op.get(), MaskKind::PackedVertical, op.getShape()));
+}
+
+// plaintext operands are permuted on the host (decode -> permute -> encode)
+template <>
+PtxtTensor MatrixTransformer::diagonalToRow<Plaintext>(const HomEvaluator &eval, const PtxtTensor &op) {
+    const Context &ctx = eval.getContext();
+    EnDecoder endec(ctx);
+    const Message src = endec.decode(op.get());
+    Message dst(src.getLogSlots(), 0);
+    const i64 n = op.getHeight(), w = op.getBlockWidth(), height = (i64)src.getSize() / w;
+    for (i64 r = 0; r < height; r++)
+        for (i64 c = 0; c < w; c++) {
+            const i64 rb = r - r % n, cb = c - c % n, i = r % n, j = c % n;
+            dst[(u64)(r * w + c)] = src[(u64)((rb + (i + j) % n) * w + cb + j)];
+        }
+    return PtxtTensor(op.getShape(), endec.encode(dst, op.getLevel()));
+}
+template <>
+PtxtTensor MatrixTransformer::diagonalToColumn<Plaintext>(const HomEvaluator &eval, const PtxtTensor &op) {
+    const Context &ctx = eval.getContext();
+    EnDecoder endec(ctx);
+    const Message src = endec.decode(op.get());
+    Message dst(src.getLogSlots(), 0);
+    const i64 n = op.getHeight(), w = op.getBlockWidth(), height = (i64)src.getSize() / w;
+    for (i64 r = 0; r < height; r++)
+        for (i64 c = 0; c < w; c++) {
+            const i64 cb = c - c % n, i = r % n, j = c % n;
+            dst[(u64)(r * w + c)] = src[(u64)(r * w + cb + (i + j) % n)];
+        }
+    return PtxtTensor(op.getShape(), endec.encode(dst, op.getLevel()));
+}
+
+// out(r, c) = in(c, r): sum over e = c - r of M_e * rot_{e (w - 1)}(in)
+template <>
+CtxtTensor MatrixTransformer::transpose<Ciphertext>(const HomEvaluator &eval, const CtxtTensor &op) {
+    const Context &ctx = eval.getContext();
+    const i64 n_out_cols = op.getHeight(), n_out_rows = op.getWidth(), w = op.getBlockWidth();
+    if (n_out_cols > w) throw std::invalid_argument("[transpose] num_cols > width.");
+    const TileTensorShape shape(n_out_rows, n_out_cols, w);
+    const Geometry g = geometry(MaskKind::Diagonal, shape);
+    const u64 level = op.getLevel();
+    if (level == 0) throw std::invalid_argument("[transpose] level >= 1 is needed.");
+    std::vector<Ciphertext> baby;
+    baby.reserve((size_t)g.bs);
+    for (i64 j = 0; j < g.bs; j++) {
+        baby.emplace_back(ctx);
+        if (j == 0)
+            eval.rightRotate(op.get(), (u64)((g.n - 1) * g.step), baby[0]);
+        else
+            eval.leftRotate(baby[(size_t)j - 1], (u64)g.step, baby[(size_t)j]);
+    }
+    Ciphertext res(ctx), group(ctx), tmp(ctx);
+    bool first = true;
+    for (i64 i = 0; i < g.gs; i++) {
+        bool any = false;
+        for (i64 j = 0; j < g.bs; j++) {
+            const i64 e = 1 - g.n + i * g.bs + j;
+            if (e >= g.n) break;
+            eval.multWithoutRescale(baby[(size_t)j], transformMask(eval, MaskKind::Diagonal, shape, level, e),
+                                    any ? tmp : group);
+            if (any) eval.add(group, tmp, group);
+            any = true;
+        }
+        if (!any) continue;
+        if (i > 0) eval.leftRotate(group, (u64)(i * g.bs * g.step), group);
+        if (first)
+            res = group;
+        else
+            eval.add(res, group, res);
+        first = false;
+    }
+    eval.rescale(res);
+    return CtxtTensor(shape, res);
+}
+template <>
+PtxtTensor MatrixTransformer::transpose<Plaintext>(const HomEvaluator &eval, const PtxtTensor &op) {
+    const Context &ctx = eval.getContext();
+    const i64 n = op.getHeight(), w = op.getBlockWidth();
+    if (n > w) throw std::invalid_argument("[transpose] num_cols > width.");
+    EnDecoder endec(ctx);
+    const Message src = endec.decode(op.get());
+    Message dst(src.getLogSlots(), 0);
+    const i64 height = (i64)src.getSize() / w;
+    for (i64 r = 0; r < height; r++)
+        for (i64 c = 0; c < w; c++) {
+            const i64 rb = r - r % n, cb = c - c % n;
+            dst[(u64)(r * w + c)] = src[(u64)((rb + c % n) * w + cb + r % n)];
+        }
+    return PtxtTensor(TileTensorShape(op.getWidth(), op.getHeight(), w), endec.encode(dst, op.getLevel()));
+}
+
+// ---- products ----------------------------------------------------------------------------------------
+namespace {
+template <class T1, class T2>
+i64 commonInside(const HETensor<T1> &a, const HETensor<T2> &b) {
+    if (a.getWidth() != b.getHeight()) throw std::invalid_argument("[getCommonInsideLength] different inside length.");
+    return a.getWidth();
+}
+template <class T1, class T2>
+i64 commonBlockWidth(const HETensor<T1> &a, const HETensor<T2> &b) {
+    if (a.getBlockWidth() != b.getBlockWidth())
+        throw std::invalid_argument("[getCommonBlockWidth] different block width");
+    return a.getBlockWidth();
+}
+void checkLevel(u64 level, const Bootstrapper &btp) {
+    if (level < 1 + btp.getMinLevelForBootstrap())
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(1 + btp.getMinLevelForBootstrap()) +
+                                    " is needed.");
+}
+}  // namespace
+
+template <>
+CtxtTensor multMatMat<Ciphertext>(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                                  const CtxtTensor &op2, u64 T, MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = op1.getHeight(), cols = op2.getWidth();
+    const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
+    checkLevel(std::min(op1.getLevel(), op2.getLevel()), btp);
+    CtxtTensor a{op1}, b{op2};
+    a.setShape(rows, k);
+    b.setShape(k, cols);
+    if (std::min(a.getLevel(), b.getLevel()) < 4 + btp.getMinLevelForBootstrap()) {
+        eval.multImagUnit(b.get(), b.get());
+        eval.add(a.get(), b.get(), a.get());
+        btp.bootstrapExtended(a.get(), a.get(), b.get());
+    }
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, a.getShape(), T + 2);
+    std::vector<Plaintext> &row_mask = tr.getRowMask(eval, b.getShape(), T + 2);
+    a = tr.diagonalToColumn(eval, a);
+    b = tr.diagonalToRow(eval, b);
+    if (std::min(a.getLevel(), b.getLevel()) < T + 2)
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
+    eval.levelDown(a.get(), T + 2, a.get());
+    eval.levelDown(b.get(), T + 2, b.get());
+
+    const i64 rows_p = std::max(k, pow2ceil(rows)), cols_p = std::max(k, pow2ceil(cols));
+    CtxtTensor res(ctx, rows, cols, w);
+    eval.mult(a.get(), b.get(), res.get());
+
+    eval.leftRotate(a.get(), 1, a.get());
+    eval.leftRotate(b.get(), (u64)w, b.get());
+    Ciphertext a_wrap(ctx), b_wrap(ctx);
+    eval.rightRotate(a.get(), (u64)cols_p, a_wrap);
+    eval.rightRotate(b.get(), (u64)(rows_p * w), b_wrap);
+
+    Ciphertext t1(ctx), t2(ctx), acc(ctx);
+    for (i64 i = 1; i < k; i++) {
+        if (i > 1) {
+            eval.leftRotate(a.get(), 1, a.get());
+            eval.leftRotate(a_wrap, 1, a_wrap);
+            eval.leftRotate(b.get(), (u64)w, b.get());
+            eval.leftRotate(b_wrap, (u64)w, b_wrap);
+        }
+        eval.maskedSum(a.get(), col_mask[(size_t)(2 * i + 1)], a_wrap, col_mask[(size_t)(2 * i)], t1);
+        eval.rescale(t1);
+        eval.maskedSum(b.get(), row_mask[(size_t)(2 * i + 1)], b_wrap, row_mask[(size_t)(2 * i)], t2);
+        eval.rescale(t2);
+        eval.tensorAccumulate(t1, t2, acc, i == 1);
+    }
+    if (k > 1) {
+        eval.relinearize(acc, t1);
+        eval.rescale(t1);
+        eval.add(res.get(), t1, res.get());
+    }
+    return res;
+}
+
+template <>
+CtxtTensor multMatMat<Plaintext>(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                                 const PtxtTensor &op2, u64 T, MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = op1.getHeight(), cols = op2.getWidth();
+    const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
+    checkLevel(std::min(op1.getLevel(), op2.getLevel()), btp);
+    CtxtTensor a{op1};
+    PtxtTensor b{op2};
+    a.setShape(rows, k);
+    b.setShape(k, cols);
+    if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
+    a = tr.diagonalToColumn(eval, a);
+    b = tr.diagonalToRow(eval, b);
+    if (a.getLevel() < T + 2)
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
+    eval.levelDown(a.get(), T + 2, a.get());
+    EnDecoder endec(ctx);
+    b.get() = endec.encode(endec.decode(b.get()), T + 2);
+
+    const i64 rows_p = std::max(k, pow2ceil(rows)), cols_p = std::max(k, pow2ceil(cols));
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, a.getShape(), T + 2);
+    std::vector<Plaintext> &row_mask = tr.getRowMask(eval, b.getShape(), T + 2);
+    CtxtTensor res(ctx, rows, cols, w);
+    eval.mult(a.get(), b.get(), res.get());
+
+    eval.leftRotate(a.get(), 1, a.get());
+    eval.leftRotate(b.get(), (u64)w, b.get());
+    Ciphertext a_wrap(ctx);
+    Plaintext b_wrap(ctx);
+    eval.rightRotate(a.get(), (u64)cols_p, a_wrap);
+    eval.rightRotate(b.get(), (u64)(rows_p * w), b_wrap);
+
+    Ciphertext t1(ctx), prod(ctx), acc(ctx);
+    Plaintext p1(ctx), p2(ctx);
+    for (i64 i = 1; i < k; i++) {
+        if (i > 1) {
+            eval.leftRotate(a.get(), 1, a.get());
+            eval.leftRotate(a_wrap, 1, a_wrap);
+            eval.leftRotate(b.get(), (u64)w, b.get());
+            eval.leftRotate(b_wrap, (u64)w, b_wrap);
+        }
+        eval.maskedSum(a.get(), col_mask[(size_t)(2 * i + 1)], a_wrap, col_mask[(size_t)(2 * i)], t1);
+        eval.rescale(t1);
+        eval.mult(b.get(), row_mask[(size_t)(2 * i + 1)], p1);
+        eval.mult(b_wrap, row_mask[(size_t)(2 * i)], p2);
+        eval.add(p1, p2, p1);
+        eval.mult(t1, p1, prod);
+        if (i == 1)
+            acc = prod;
+        else
+            eval.add(acc, prod, acc);
+    }
+    if (k > 1) eval.add(res.get(), acc, res.get());
+    return res;
+}
+
+CtxtTensor multPackedMatMat(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = op1.getHeight(), cols = op2.getWidth();
+    const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
+    checkLevel(std::min(op1.getLevel(), op2.getLevel()), btp);
+    if (op1.getLevel() < T + 3 || op2.getLevel() < T + 2)
+        throw std::invalid_argument("[multPackedMatMat] levels >= " + std::to_string(T + 3) + " / " +
+                                    std::to_string(T + 2) + " are needed.");
+    CtxtTensor a{op1}, b{op2};
+    a.setShape(rows, k);
+    b.setShape(k, cols);
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, a.getShape(), T + 2);
+    eval.levelDown(a.get(), T + 3, a.get());
+    eval.levelDown(b.get(), T + 2, b.get());
+    a = tr.packedDiagonalToColumn(eval, a);
+    b = tr.packedDiagonalToRow(eval, b);
+
+    const i64 cols_p = std::max(k, pow2ceil(cols));
+    CtxtTensor res(ctx, rows, cols, w);
+    eval.mult(a.get(), b.get(), res.get());
+    eval.leftRotate(a.get(), 2, a.get());
+    eval.leftRotate(b.get(), (u64)(2 * w), b.get());
+    Ciphertext a_wrap(ctx);
+    eval.rightRotate(a.get(), (u64)cols_p, a_wrap);
+    Ciphertext t1(ctx), acc(ctx);
+    for (i64 i = 1; i < k / 2; i++) {
+        if (i > 1) {
+            eval.leftRotate(a.get(), 2, a.get());
+            eval.leftRotate(a_wrap, 2, a_wrap);
+            eval.leftRotate(b.get(), (u64)(2 * w), b.get());
+        }
+        eval.maskedSum(a.get(), col_mask[(size_t)(4 * i + 1)], a_wrap, col_mask[(size_t)(4 * i)], t1);
+        eval.rescale(t1);
+        eval.tensorAccumulate(t1, b.get(), acc, i == 1);
+    }
+    if (k / 2 > 1) {
+        eval.relinearize(acc, t1);
+        eval.rescale(t1);
+        eval.add(res.get(), t1, res.get());
+    }
+    return res;
+}
+
+CtxtTensor multPackedMatMatPre(const HomEvaluator &eval, const CtxtTensor &a_in, u64 T, MatrixTransformer &tr) {
+    CtxtTensor a(a_in);
+    eval.levelDown(a.get(), T + 3, a.get());
+    return tr.packedDiagonalToColumn(eval, a);
+}
+
+void multPackedMatMatPreRot(const HomEvaluator &eval, const CtxtTensor &a_in, std::vector<Ciphertext> &tmp, u64 T,
+                            MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    tmp.clear();
+    const i64 n = a_in.getHeight();
+    CtxtTensor a(a_in);
+    Ciphertext first(ctx);
+    eval.levelDownOne(a.get(), first);
+    tmp.push_back(first);
+    eval.leftRotate(a.get(), 2, a.get());
+    Ciphertext a_wrap(ctx), t1(ctx);
+    eval.rightRotate(a.get(), (u64)n, a_wrap);
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, a.getShape(), T + 2);
+    for (i64 i = 1; i < n / 2; i++) {
+        if (i > 1) {
+            eval.leftRotate(a.get(), 2, a.get());
+            eval.leftRotate(a_wrap, 2, a_wrap);
+        }
+        eval.maskedSum(a.get(), col_mask[(size_t)(4 * i + 1)], a_wrap, col_mask[(size_t)(4 * i)], t1);
+        eval.rescale(t1);
+        tmp.push_back(t1);
+    }
+}
+
+CtxtTensor multPackedMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b_in, u64 T, MatrixTransformer &tr) {
+    CtxtTensor b(b_in);
+    eval.levelDown(b.get(), T + 2, b.get());
+    return tr.packedDiagonalToRow(eval, b);
+}
+
+CtxtTensor multPackedMatMatCCReuse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp,
+                                   const CtxtTensor &b_in, u64, MatrixTransformer &) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = b_in.getHeight(), cols = b_in.getWidth(), w = b_in.getBlockWidth();
+    CtxtTensor b(b_in);
+    b.setShape(pow2ceil(rows), cols);
+    CtxtTensor res(ctx, rows, cols, w);
+    Ciphertext acc(ctx);
+    for (size_t i = 0; i < tmp.size(); i++) {
+        if (i > 0) eval.leftRotate(b.get(), (u64)(2 * w), b.get());
+        eval.tensorAccumulate(tmp[i], b.get(), acc, i == 0);
+    }
+    eval.relinearize(acc, res.get());
+    eval.rescale(res.get());
+    return res;
+}
+
+void multMatMatPre(const HomEvaluator &eval, const CtxtTensor &a_in, std::vector<Ciphertext> &tmp, u64 T,
+                   MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    tmp.clear();
+    const i64 n = a_in.getHeight();
+    CtxtTensor a(a_in);
+    if (a.getLevel() < T + 3)
+        throw std::invalid_argument("[multMatMatPre] level >= " + std::to_string(T + 3) + " is needed.");
+    eval.levelDown(a.get(), T + 3, a.get());
+    a = tr.diagonalToColumn(eval, a);
+    Ciphertext first(ctx);
+    eval.levelDownOne(a.get(), first);
+    tmp.push_back(first);
+    eval.leftRotate(a.get(), 1, a.get());
+    Ciphertext a_wrap(ctx), t1(ctx);
+    eval.rightRotate(a.get(), (u64)n, a_wrap);
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, a.getShape(), T + 2);
+    for (i64 i = 1; i < n; i++) {
+        if (i > 1) {
+            eval.leftRotate(a.get(), 1, a.get());
+            eval.leftRotate(a_wrap, 1, a_wrap);
+        }
+        eval.maskedSum(a.get(), col_mask[(size_t)(2 * i + 1)], a_wrap, col_mask[(size_t)(2 * i)], t1);
+        eval.rescale(t1);
+        tmp.push_back(t1);
+    }
+}
+
+CtxtTensor multMatMatReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const PtxtTensor &b_in,
+                           u64 T, MatrixTransformer &) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = b_in.getHeight(), cols = b_in.getWidth(), w = b_in.getBlockWidth();
+    PtxtTensor b(b_in);
+    if (b.getLevel() != T + 1) {
+        EnDecoder endec(ctx);
+        b.get() = endec.encode(endec.decode(b.get()), T + 1);
+    }
+    CtxtTensor res(ctx, rows, cols, w);
+    eval.matmul(tmp, b.get(), res.get());
+    return res;
+}
+
+CtxtTensor multMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b_in, u64 T, MatrixTransformer &tr) {
+    CtxtTensor b(b_in);
+    eval.levelDown(b.get(), T + 2, b.get());
+    return tr.diagonalToRow(eval, b);
+}
+
+CtxtTensor multMatMatCCReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b_in,
+                             u64, MatrixTransformer &) {
+    const Context &ctx = eval.getContext();
+    const i64 rows = b_in.getHeight(), cols = b_in.getWidth(), w = b_in.getBlockWidth();
+    CtxtTensor b(b_in);
+    CtxtTensor res(ctx, rows, cols, w);
+    Ciphertext acc(ctx);
+    for (size_t i = 0; i < tmp.size(); i++) {
+        if (i > 0) eval.leftRotate(b.get(), (u64)w, b.get());
+        eval.tensorAccumulate(tmp[i], b.get(), acc, i == 0);
+    }
+    eval.relinearize(acc, res.get());
+    return res;
+}
+
+}  // namespace HELLM

@@ -1,0 +1,334 @@
+"""ctypes binding of the HEMMer facade (include/hellm.h): the Python mirror of HELLM::HEMMer used by
+the tests and bench.py.  Matrices are numpy float64 arrays; tensors are opaque device handles."""
+import ctypes
+
+import numpy as np
+
+from . import check, lib
+
+vp = ctypes.c_void_p
+u32 = ctypes.c_uint32
+u64 = ctypes.c_uint64
+f64p = ctypes.POINTER(ctypes.c_double)
+u64p = ctypes.POINTER(ctypes.c_uint64)
+u32p = ctypes.POINTER(ctypes.c_uint32)
+_declared = False
+
+
+def _L():
+    global _declared
+    L = lib()
+    if not _declared:
+        pvp = ctypes.POINTER(vp)
+        L.hellm_hemmer_create.argtypes = [u32, u32, u32, u64p, u32, u32, u32, u64, pvp]
+        L.hellm_hemmer_create_preset.argtypes = [u64, pvp]
+        L.hellm_hemmer_destroy.argtypes = [vp]
+        L.hellm_hemmer_info.argtypes = [vp, u32p, u32p, u32p, u32p, u32p, u64p]
+        L.hellm_secret_coeffs.argtypes = [vp, ctypes.POINTER(ctypes.c_int32)]
+        L.hellm_export_key.argtypes = [vp, u64, u64p]
+        L.hellm_ensure_rotation_keys.argtypes = [vp, u64p, u32]
+        L.hellm_encrypt.argtypes = [vp, f64p, u32, u32, pvp]
+        L.hellm_encrypt2.argtypes = [vp, f64p, f64p, u32, u32, pvp]
+        L.hellm_encode.argtypes = [vp, f64p, u32, u32, u32, pvp]
+        L.hellm_encode2.argtypes = [vp, f64p, f64p, u32, u32, u32, pvp]
+        L.hellm_encode_diagonal_to_row4.argtypes = [vp, f64p, f64p, f64p, f64p, u32, u32, u32, pvp]
+        L.hellm_decrypt.argtypes = [vp, vp, f64p]
+        L.hellm_decrypt2.argtypes = [vp, vp, f64p]
+        L.hellm_decrypt_slots.argtypes = [vp, vp, f64p]
+        L.hellm_ct_info.argtypes = [vp, u32p, u32p, u32p, u32p, u32p, u32p]
+        L.hellm_ct_download.argtypes = [vp, u64p]
+        L.hellm_ct_upload.argtypes = [vp, u64p, u32, u32, u32, u32, u32, u32, pvp]
+        L.hellm_ct_clone.argtypes = [vp, pvp]
+        L.hellm_ct_destroy.argtypes = [vp]
+        L.hellm_pt_destroy.argtypes = [vp]
+        L.hellm_pt_download.argtypes = [vp, u32p, u64p]
+        L.hellm_ctvec_destroy.argtypes = [vp]
+        L.hellm_ctvec_size.argtypes = [vp, u32p]
+        L.hellm_ctvec_get.argtypes = [vp, u32, u32, u32, u32, pvp]
+        L.hellm_left_rotate.argtypes = [vp, vp, u64, pvp]
+        for n in ("hellm_conjugate", "hellm_mult_imag_unit", "hellm_diagonal_to_column",
+                  "hellm_diagonal_to_row"):
+            getattr(L, n).argtypes = [vp, vp, pvp]
+        for n in ("hellm_mult", "hellm_add", "hellm_complex_packing", "hellm_complex_packing_rev",
+                  "hellm_repack_not_bts"):
+            getattr(L, n).argtypes = [vp, vp, vp, pvp]
+        L.hellm_level_down.argtypes = [vp, vp, u32, pvp]
+        L.hellm_transpose_inplace.argtypes = [vp, vp, u32]
+        L.hellm_complex_packing_inplace.argtypes = [vp, vp]
+        L.hellm_complex_packing_row_inplace.argtypes = [vp, vp]
+        L.hellm_transpose_complex_packing_inplace.argtypes = [vp, vp, u32]
+        L.hellm_split_in_two.argtypes = [vp, vp, pvp, pvp]
+        for n in ("hellm_single_cc_matmul", "hellm_single_matmul", "hellm_packed_matmul",
+                  "hellm_packed_matmul_cc_reuse", "hellm_matmul_reuse", "hellm_matmul_cc_reuse"):
+            getattr(L, n).argtypes = [vp, vp, vp, u32, pvp]
+        for n in ("hellm_packed_matmul_pre", "hellm_packed_matmul_pre_rot", "hellm_packed_matmul_pre_rev",
+                  "hellm_matmul_pre", "hellm_matmul_pre_rev"):
+            getattr(L, n).argtypes = [vp, vp, u32, pvp]
+        L.hellm_repack_cc.argtypes = [vp, vp, pvp]
+        _declared = True
+    return L
+
+
+def _m(a):
+    a = np.ascontiguousarray(a, dtype=np.float64)
+    return a, a.ctypes.data_as(f64p)
+
+
+class _Handle:
+    _destroy = None
+
+    def __init__(self, owner, h):
+        self.owner, self.h = owner, h
+
+    def free(self):
+        if self.h:
+            getattr(_L(), self._destroy)(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Ct(_Handle):
+    _destroy = "hellm_ct_destroy"
+
+    def info(self):
+        v = [u32() for _ in range(6)]
+        check(_L().hellm_ct_info(self.h, *[ctypes.byref(x) for x in v]))
+        return dict(zip(("num_poly", "level", "rescale_counter", "rows", "cols", "block_width"),
+                        [x.value for x in v]))
+
+    @property
+    def level(self):
+        return self.info()["level"]
+
+    def residues(self):
+        i = self.info()
+        out = np.empty((i["num_poly"], i["level"] + 1, self.owner.N), dtype=np.uint64)
+        check(_L().hellm_ct_download(self.h, out.ctypes.data_as(u64p)))
+        return out
+
+    def clone(self):
+        h = vp()
+        check(_L().hellm_ct_clone(self.h, ctypes.byref(h)))
+        return Ct(self.owner, h)
+
+
+class Pt(_Handle):
+    _destroy = "hellm_pt_destroy"
+
+    def residues(self):
+        lvl = u32()
+        check(_L().hellm_pt_download(self.h, ctypes.byref(lvl), None))
+        out = np.empty((lvl.value + 1, self.owner.N), dtype=np.uint64)
+        check(_L().hellm_pt_download(self.h, ctypes.byref(lvl), out.ctypes.data_as(u64p)))
+        return out
+
+
+class CtVec(_Handle):
+    _destroy = "hellm_ctvec_destroy"
+
+    def __len__(self):
+        n = u32()
+        check(_L().hellm_ctvec_size(self.h, ctypes.byref(n)))
+        return n.value
+
+    def get(self, i, rows, cols, block_width):
+        h = vp()
+        check(_L().hellm_ctvec_get(self.h, i, rows, cols, block_width, ctypes.byref(h)))
+        return Ct(self.owner, h)
+
+
+class HEMMer:
+    """HELLM::HEMMer on the GPU.  preset=True builds the FGb-sized context (N = 2^16)."""
+
+    def __init__(self, log_n=None, q_primes=None, p_primes=None, dnum=None, log_scale=42,
+                 min_bootstrap_level=0, seed=0x5EED, preset=False):
+        L = _L()
+        h = vp()
+        if preset:
+            check(L.hellm_hemmer_create_preset(seed, ctypes.byref(h)))
+        else:
+            mods = [int(x) for x in q_primes] + [int(x) for x in p_primes]
+            arr = (ctypes.c_uint64 * len(mods))(*mods)
+            check(L.hellm_hemmer_create(log_n, len(q_primes), len(p_primes), arr, dnum, log_scale,
+                                        min_bootstrap_level, seed, ctypes.byref(h)))
+        self.h = h
+        self.seed = seed
+        v = [u32() for _ in range(5)]
+        check(L.hellm_hemmer_info(h, *[ctypes.byref(x) for x in v], None))
+        self.log_n, self.nQ, self.nP, self.dnum, self.dim = [x.value for x in v]
+        self.N = 1 << self.log_n
+        pr = (ctypes.c_uint64 * (self.nQ + self.nP))()
+        check(L.hellm_hemmer_info(h, None, None, None, None, None, pr))
+        self.q, self.p = list(pr)[: self.nQ], list(pr)[self.nQ:]
+
+    def close(self):
+        if getattr(self, "h", None):
+            _L().hellm_hemmer_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def sync(self):
+        check(_L().hellm_sync())
+
+    def secret_coeffs(self):
+        out = np.empty(self.N, dtype=np.int32)
+        check(_L().hellm_secret_coeffs(self.h, out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))))
+        return out
+
+    def export_key(self, galois=0):
+        out = np.empty((self.dnum, 2, self.nQ + self.nP, self.N), dtype=np.uint64)
+        check(_L().hellm_export_key(self.h, galois, out.ctypes.data_as(u64p)))
+        return out
+
+    def ensure_rotation_keys(self, rots):
+        arr = (ctypes.c_uint64 * len(rots))(*[int(r) for r in rots])
+        check(_L().hellm_ensure_rotation_keys(self.h, arr, len(rots)))
+
+    # ---- codec ------------------------------------------------------------------------------
+    def _new(self, cls, fn, *args):
+        h = vp()
+        check(getattr(_L(), fn)(self.h, *args, ctypes.byref(h)))
+        return cls(self, h)
+
+    def encrypt(self, m):
+        a, pa = _m(m)
+        return self._new(Ct, "hellm_encrypt", pa, a.shape[0], a.shape[1])
+
+    def encrypt2(self, m1, m2):
+        a, pa = _m(m1)
+        b, pb = _m(m2)
+        return self._new(Ct, "hellm_encrypt2", pa, pb, a.shape[0], a.shape[1])
+
+    def encode(self, m, level=0):
+        a, pa = _m(m)
+        return self._new(Pt, "hellm_encode", pa, a.shape[0], a.shape[1], level)
+
+    def encode2(self, m1, m2, level=0):
+        a, pa = _m(m1)
+        b, pb = _m(m2)
+        return self._new(Pt, "hellm_encode2", pa, pb, a.shape[0], a.shape[1], level)
+
+    def encode_diagonal_to_row4(self, w1, w2, w3, w4, level=0):
+        ms = [_m(w) for w in (w1, w2, w3, w4)]
+        return self._new(Pt, "hellm_encode_diagonal_to_row4", *[p for _, p in ms],
+                         ms[0][0].shape[0], ms[0][0].shape[1], level)
+
+    def decrypt(self, ct):
+        i = ct.info()
+        out = np.empty((i["rows"], i["cols"]), dtype=np.float64)
+        check(_L().hellm_decrypt(self.h, ct.h, out.ctypes.data_as(f64p)))
+        return out
+
+    def decrypt2(self, ct):
+        i = ct.info()
+        out = np.empty((2, i["rows"], i["cols"]), dtype=np.float64)
+        check(_L().hellm_decrypt2(self.h, ct.h, out.ctypes.data_as(f64p)))
+        return out
+
+    def decrypt_slots(self, ct):
+        out = np.empty(self.N, dtype=np.float64)
+        check(_L().hellm_decrypt_slots(self.h, ct.h, out.ctypes.data_as(f64p)))
+        return out.view(np.complex128).copy()
+
+    def upload(self, residues, rows, cols, block_width, rescale_counter=0):
+        r = np.ascontiguousarray(residues, dtype=np.uint64)
+        return self._new(Ct, "hellm_ct_upload", r.ctypes.data_as(u64p), r.shape[0], r.shape[1] - 1,
+                         rescale_counter, rows, cols, block_width)
+
+    # ---- evaluator ----------------------------------------------------------------------------
+    def left_rotate(self, a, rot):
+        return self._new(Ct, "hellm_left_rotate", a.h, rot)
+
+    def conjugate(self, a):
+        return self._new(Ct, "hellm_conjugate", a.h)
+
+    def mult_imag_unit(self, a):
+        return self._new(Ct, "hellm_mult_imag_unit", a.h)
+
+    def mult(self, a, b):
+        return self._new(Ct, "hellm_mult", a.h, b.h)
+
+    def add(self, a, b):
+        return self._new(Ct, "hellm_add", a.h, b.h)
+
+    def level_down(self, a, target):
+        return self._new(Ct, "hellm_level_down", a.h, target)
+
+    # ---- transforms and products -----------------------------------------------------------------
+    def diagonal_to_column(self, a):
+        return self._new(Ct, "hellm_diagonal_to_column", a.h)
+
+    def diagonal_to_row(self, a):
+        return self._new(Ct, "hellm_diagonal_to_row", a.h)
+
+    def transpose_inplace(self, a, target_level=0):
+        check(_L().hellm_transpose_inplace(self.h, a.h, target_level))
+
+    def complex_packing_inplace(self, a):
+        check(_L().hellm_complex_packing_inplace(self.h, a.h))
+
+    def complex_packing_row_inplace(self, a):
+        check(_L().hellm_complex_packing_row_inplace(self.h, a.h))
+
+    def transpose_complex_packing_inplace(self, a, target_level=0):
+        check(_L().hellm_transpose_complex_packing_inplace(self.h, a.h, target_level))
+
+    def split_in_two(self, a):
+        h1, h2 = vp(), vp()
+        check(_L().hellm_split_in_two(self.h, a.h, ctypes.byref(h1), ctypes.byref(h2)))
+        return Ct(self, h1), Ct(self, h2)
+
+    def single_cc_matmul(self, a, b, target_level=4):
+        return self._new(Ct, "hellm_single_cc_matmul", a.h, b.h, target_level)
+
+    def single_matmul(self, a, b_pt, target_level=4):
+        return self._new(Ct, "hellm_single_matmul", a.h, b_pt.h, target_level)
+
+    def packed_matmul(self, a, b, target_level=4):
+        return self._new(Ct, "hellm_packed_matmul", a.h, b.h, target_level)
+
+    def packed_matmul_pre(self, a, target_level=4):
+        return self._new(Ct, "hellm_packed_matmul_pre", a.h, target_level)
+
+    def packed_matmul_pre_rot(self, a, target_level=4):
+        return self._new(CtVec, "hellm_packed_matmul_pre_rot", a.h, target_level)
+
+    def packed_matmul_pre_rev(self, b, target_level=4):
+        return self._new(Ct, "hellm_packed_matmul_pre_rev", b.h, target_level)
+
+    def packed_matmul_cc_reuse(self, tmp, b, target_level=4):
+        return self._new(Ct, "hellm_packed_matmul_cc_reuse", tmp.h, b.h, target_level)
+
+    def repack_cc(self, a):
+        return self._new(Ct, "hellm_repack_cc", a.h)
+
+    def complex_packing(self, a, b):
+        return self._new(Ct, "hellm_complex_packing", a.h, b.h)
+
+    def complex_packing_rev(self, a, b):
+        return self._new(Ct, "hellm_complex_packing_rev", a.h, b.h)
+
+    def repack_not_bts(self, a, b):
+        return self._new(Ct, "hellm_repack_not_bts", a.h, b.h)
+
+    def matmul_pre(self, a, target_level=4):
+        return self._new(CtVec, "hellm_matmul_pre", a.h, target_level)
+
+    def matmul_reuse(self, tmp, b_pt, target_level=4):
+        return self._new(Ct, "hellm_matmul_reuse", tmp.h, b_pt.h, target_level)
+
+    def matmul_pre_rev(self, b, target_level=4):
+        return self._new(Ct, "hellm_matmul_pre_rev", b.h, target_level)
+
+    def matmul_cc_reuse(self, tmp, b, target_level=4):
+        return self._new(Ct, "hellm_matmul_cc_reuse", tmp.h, b.h, target_level)
