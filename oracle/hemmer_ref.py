@@ -1,0 +1,508 @@
+"""TEST INFRASTRUCTURE ONLY -- CPU restatement of HEMMer's matrix-multiplication algorithms.
+
+Restates, over an abstract evaluator, the slot-level algorithms of the reference's
+ciphertext/src/MatrixUtils.cpp (mask families :90-578, sigma/tau transforms :776-1098, transpose
+:671-739, multMatMat<Ciphertext> :1307-1446, multMatMat<Plaintext> :1448-1570, multPackedMatMat
+:1100-1216, the Pre/ReUse family :1218-1305,:1572-1679) and the packing helpers of
+ciphertext/src/HEMMer.cpp (:764-831, :964-1053).  Two evaluators run the same code:
+
+  * SlotSim   -- "ciphertexts" are plain complex slot vectors (np.roll for rotations).  Pins every
+                 mask and rotation index against float64 matrix algebra, independent of any crypto.
+  * oracle.Oracle -- the CPU RNS-CKKS oracle; gives the residues the GPU path must reproduce bit
+                 for bit when it issues the same operation sequence.
+
+The operation order (masked rotations summed before one rescale; masks pre-rotated per
+baby-step/giant-step group) is the one the GPU build documents for itself; decrypted results equal
+the reference's A*B either way.
+"""
+import math
+
+import numpy as np
+
+
+def pow2ceil(v):
+    p = 1
+    while p < v:
+        p <<= 1
+    return p
+
+
+# --------------------------------------------------------------------------------------------
+# slot simulator
+# --------------------------------------------------------------------------------------------
+class SimCt:
+    def __init__(self, z, level, rc=0):
+        self.z, self.level, self.rc = np.asarray(z, dtype=np.complex128), level, rc
+
+
+class SlotSim:
+    """Evaluator over exact slot vectors, with the same level / rescale-counter bookkeeping."""
+
+    def __init__(self, log_slots, top_level):
+        self.slots = 1 << log_slots
+        self.top = top_level
+
+    def encrypt(self, z, level=None):
+        v = np.zeros(self.slots, dtype=np.complex128)
+        z = np.asarray(z).reshape(-1)
+        v[: z.size] = z
+        return SimCt(v, self.top if level is None else level)
+
+    def encode(self, msg, level):
+        return SimCt(np.asarray(msg, dtype=np.complex128).copy(), level)
+
+    def decrypt(self, ct):
+        return ct.z.copy()
+
+    def level_of(self, x):
+        return x.level
+
+    def _lv(self, x, y):
+        lo = min(x.level, y.level)
+        return lo
+
+    def add(self, x, y):
+        assert x.rc == y.rc
+        return SimCt(x.z + y.z, self._lv(x, y), x.rc)
+
+    def sub(self, x, y):
+        assert x.rc == y.rc
+        return SimCt(x.z - y.z, self._lv(x, y), x.rc)
+
+    def negate(self, x):
+        return SimCt(-x.z, x.level, x.rc)
+
+    def mult_plain_no_rescale(self, x, pt):
+        assert x.rc == 0 and pt.level >= x.level
+        return SimCt(x.z * pt.z, x.level, 1)
+
+    def masked_sum(self, a, ma, b, mb):
+        assert a.level == b.level
+        return self.add(self.mult_plain_no_rescale(a, ma), self.mult_plain_no_rescale(b, mb))
+
+    def rescale(self, x):
+        assert x.rc >= 1 and x.level >= 1
+        return SimCt(x.z, x.level - 1, x.rc - 1)
+
+    def tensor(self, x, y):
+        assert x.rc == 0 and y.rc == 0
+        return SimCt(x.z * y.z, self._lv(x, y), 1)
+
+    def relinearize(self, x):
+        return x
+
+    def mult(self, x, y):
+        if isinstance(y, SimCt) and getattr(y, "is_pt", False):
+            return self.rescale(self.mult_plain_no_rescale(x, y))
+        return self.rescale(self.tensor(x, y))
+
+    def mult_pt(self, x, pt):
+        return self.rescale(self.mult_plain_no_rescale(x, pt))
+
+    def mult_imag_unit(self, x):
+        return SimCt(1j * x.z, x.level, x.rc)
+
+    def left_rotate(self, x, r):
+        return SimCt(np.roll(x.z, -(r % self.slots)), x.level, x.rc)
+
+    def right_rotate(self, x, r):
+        return SimCt(np.roll(x.z, r % self.slots), x.level, x.rc)
+
+    def conjugate(self, x):
+        return SimCt(np.conj(x.z), x.level, x.rc)
+
+    def level_down(self, x, target):
+        assert target <= x.level
+        return SimCt(x.z, target, x.rc)
+
+    def level_down_one(self, x):
+        return self.level_down(x, x.level - 1)
+
+    # plaintext helpers (plaintexts are SimCt too)
+    def pt_mult(self, a, b):
+        return SimCt(a.z * b.z, min(a.level, b.level) - 1)
+
+    def pt_add(self, a, b):
+        return SimCt(a.z + b.z, min(a.level, b.level))
+
+    def pt_reencode(self, pt, level):
+        return SimCt(pt.z, level)
+
+    def pt_values(self, pt):
+        return pt.z
+
+
+class OracleEval:
+    """Adapter giving oracle.Oracle the interface the algorithms below use."""
+
+    def __init__(self, orc):
+        self.o = orc
+        self.slots = orc.slots
+
+    def encode(self, msg, level):
+        return self.o.encode(msg, level)
+
+    def level_of(self, x):
+        return x.level
+
+    def _same_level(self, x, y):
+        if x.level > y.level:
+            x = self.o.level_down(x, y.level)
+        elif y.level > x.level:
+            y = self.o.level_down(y, x.level)
+        return x, y
+
+    def add(self, x, y):
+        x, y = self._same_level(x, y)
+        return self.o.add(x, y)
+
+    def sub(self, x, y):
+        x, y = self._same_level(x, y)
+        return self.o.sub(x, y)
+
+    def negate(self, x):
+        return self.o.negate(x)
+
+    def mult_plain_no_rescale(self, x, pt):
+        assert pt.level >= x.level
+        return self.o.mult_plain_no_rescale(x, pt)
+
+    def masked_sum(self, a, ma, b, mb):
+        return self.o.add(self.o.mult_plain_no_rescale(a, ma), self.o.mult_plain_no_rescale(b, mb))
+
+    def rescale(self, x):
+        return self.o.rescale(x)
+
+    def tensor(self, x, y):
+        x, y = self._same_level(x, y)
+        return self.o.tensor(x, y)
+
+    def relinearize(self, x):
+        return self.o.relinearize(x)
+
+    def mult(self, x, y):
+        return self.rescale(self.relinearize(self.tensor(x, y)))
+
+    def mult_pt(self, x, pt):
+        return self.rescale(self.mult_plain_no_rescale(x, pt))
+
+    def mult_imag_unit(self, x):
+        return self.o.mult_imag_unit(x)
+
+    def left_rotate(self, x, r):
+        return self.o.left_rotate(x, r)
+
+    def right_rotate(self, x, r):
+        return self.o.right_rotate(x, r)
+
+    def conjugate(self, x):
+        return self.o.conjugate(x)
+
+    def level_down(self, x, target):
+        return self.o.level_down(x, target)
+
+    def level_down_one(self, x):
+        return self.o.level_down_one(x)
+
+    def pt_mult(self, a, b):
+        from .oracle import Ct, Pt
+        lv = min(a.level, b.level)
+        prod = self.o._binary(2, a.data[: lv + 1], b.data[: lv + 1])
+        r = self.o.rescale(Ct(prod[None], a.scale * b.scale))
+        return Pt(r.data[0], r.scale)
+
+    def pt_add(self, a, b):
+        from .oracle import Pt
+        lv = min(a.level, b.level)
+        return Pt(self.o._binary(0, a.data[: lv + 1], b.data[: lv + 1]), a.scale)
+
+    def pt_reencode(self, pt, level):
+        return self.o.encode(self.o.decode(pt), level)
+
+    def pt_values(self, pt):
+        return self.o.decode(pt)
+
+
+# --------------------------------------------------------------------------------------------
+# masks  (MatrixUtils.cpp:90-578)
+# --------------------------------------------------------------------------------------------
+H, V, PH, PV, DIAG = "horizontal", "vertical", "packed_horizontal", "packed_vertical", "diagonal"
+
+
+def geometry(kind, n, w):
+    """(units, cell, bs, gs, step): diagonals in cells, cell size, BSGS sizes, slots per diagonal."""
+    if kind == DIAG:
+        count = 2 * n - 1
+        bs = math.ceil(math.sqrt(count))
+        return n, 1, bs, math.ceil(count / bs), w - 1
+    cell = 2 if kind in (PH, PV) else 1
+    units = n // cell
+    bs = math.ceil(math.sqrt(2 * units - 1))
+    gs = math.ceil((units - 1) / bs)
+    step = cell * (w if kind in (V, PV) else 1)
+    return units, cell, bs, gs, step
+
+
+def transform_mask(kind, n, w, slots, idx):
+    """Slot pattern of diagonal idx (no pre-rotation)."""
+    units, cell, _, _, _ = geometry(kind, n, w)
+    r = np.arange(slots) // w
+    c = np.arange(slots) % w
+    R = (r % n) // cell
+    C = (c % n) // cell
+    if kind in (H, PH):
+        on = (R == idx) & (C < units - idx) if idx >= 0 else (R == units + idx) & (C >= -idx)
+    elif kind in (V, PV):
+        on = (C == idx) & (R < units - idx) if idx >= 0 else (C == units + idx) & (R >= -idx)
+    else:
+        on = (C - R) == idx
+    return np.where(on, 0.5 if kind == PH else 1.0, 0.0).astype(np.complex128)
+
+
+def prerotated_mask(kind, n, w, slots, idx):
+    units, _, bs, _, step = geometry(kind, n, w)
+    m = transform_mask(kind, n, w, slots, idx)
+    if kind == DIAG:
+        i = (idx + n - 1) // bs
+        return np.roll(m, i * bs * step)
+    if idx > 0:
+        i = (idx - 1) // bs
+        return np.roll(m, i * bs * step)
+    if idx < 0:
+        i = (idx + units - 1) // bs
+        return np.roll(m, -((units - i * bs) * step))
+    return m
+
+
+def col_masks(n, slots):
+    """[2i] wrapped part, [2i+1] main part of a cyclic column shift by i (generateColMask :554-578)."""
+    j = np.arange(slots)
+    out = []
+    for i in range(n):
+        main = (j % n < n - i)
+        out += [(~main).astype(np.complex128), main.astype(np.complex128)]
+    return out
+
+
+def row_masks(n, w, slots):
+    j = np.arange(slots)
+    out = []
+    for i in range(n):
+        main = ((j // w) % n < n - i)
+        out += [(~main).astype(np.complex128), main.astype(np.complex128)]
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# transforms  (MatrixUtils.cpp:671-1098)
+# --------------------------------------------------------------------------------------------
+def diagonal_transform(ev, ct, kind, n, w):
+    units, _, bs, gs, step = geometry(kind, n, w)
+    level = ev.level_of(ct)
+    enc = lambda idx: ev.encode(prerotated_mask(kind, n, w, ev.slots, idx), level)
+    baby = []
+    for j in range(bs):
+        baby.append(ev.left_rotate(ct if j == 0 else baby[j - 1], step))
+    res = ev.mult_plain_no_rescale(ct, enc(0))
+    for i in range(gs):
+        group = None
+        for j in range(bs):
+            d = 1 + i * bs + j - units
+            if d >= 0:
+                break
+            t = ev.mult_plain_no_rescale(baby[j], enc(d))
+            group = t if group is None else ev.add(group, t)
+        if group is not None:
+            res = ev.add(res, ev.right_rotate(group, (units - i * bs) * step))
+        group = None
+        for j in range(bs):
+            d = 1 + i * bs + j
+            if d >= units:
+                break
+            t = ev.mult_plain_no_rescale(baby[j], enc(d))
+            group = t if group is None else ev.add(group, t)
+        if group is not None:
+            if i > 0:
+                group = ev.left_rotate(group, i * bs * step)
+            res = ev.add(res, group)
+    return ev.rescale(res)
+
+
+def transpose(ev, ct, n, w):
+    _, _, bs, gs, step = geometry(DIAG, n, w)
+    level = ev.level_of(ct)
+    baby = []
+    for j in range(bs):
+        baby.append(ev.right_rotate(ct, (n - 1) * step) if j == 0 else ev.left_rotate(baby[j - 1], step))
+    res = None
+    for i in range(gs):
+        group = None
+        for j in range(bs):
+            e = 1 - n + i * bs + j
+            if e >= n:
+                break
+            t = ev.mult_plain_no_rescale(baby[j], ev.encode(prerotated_mask(DIAG, n, w, ev.slots, e), level))
+            group = t if group is None else ev.add(group, t)
+        if group is None:
+            continue
+        if i > 0:
+            group = ev.left_rotate(group, i * bs * step)
+        res = group if res is None else ev.add(res, group)
+    return ev.rescale(res)
+
+
+# --------------------------------------------------------------------------------------------
+# products  (MatrixUtils.cpp:1100-1679)
+# --------------------------------------------------------------------------------------------
+def mult_mat_mat_cc(ev, a, b, T, n, w):
+    """multMatMat<Ciphertext> (:1307-1446): sum_k phi^k(sigma A) * psi^k(tau B)."""
+    cm = [ev.encode(m, T + 2) for m in col_masks(n, ev.slots)]
+    rm = [ev.encode(m, T + 2) for m in row_masks(n, w, ev.slots)]
+    a = diagonal_transform(ev, a, H, n, w)
+    b = diagonal_transform(ev, b, V, n, w)
+    a = ev.level_down(a, T + 2)
+    b = ev.level_down(b, T + 2)
+    res = ev.mult(a, b)
+    a = ev.left_rotate(a, 1)
+    b = ev.left_rotate(b, w)
+    a_wrap = ev.right_rotate(a, n)
+    b_wrap = ev.right_rotate(b, n * w)
+    acc = None
+    for i in range(1, n):
+        if i > 1:
+            a = ev.left_rotate(a, 1)
+            a_wrap = ev.left_rotate(a_wrap, 1)
+            b = ev.left_rotate(b, w)
+            b_wrap = ev.left_rotate(b_wrap, w)
+        t1 = ev.rescale(ev.masked_sum(a, cm[2 * i + 1], a_wrap, cm[2 * i]))
+        t2 = ev.rescale(ev.masked_sum(b, rm[2 * i + 1], b_wrap, rm[2 * i]))
+        t = ev.tensor(t1, t2)
+        acc = t if acc is None else ev.add(acc, t)
+    out = ev.rescale(ev.relinearize(acc))
+    return ev.add(res, out)
+
+
+def tau_plain(values, n, w):
+    """diagonalToRow<Plaintext> (:1072-1098): host permutation tau(B)[i,j] = B[(i+j) mod n, j]."""
+    slots = values.size
+    r = np.arange(slots) // w
+    c = np.arange(slots) % w
+    src = ((r - r % n) + (r % n + c % n) % n) * w + c
+    return values[src]
+
+
+def mult_mat_mat_pc(ev, a, b_pt, T, n, w):
+    """multMatMat<Plaintext> (:1448-1570)."""
+    cm = [ev.encode(m, T + 2) for m in col_masks(n, ev.slots)]
+    rm = [ev.encode(m, T + 2) for m in row_masks(n, w, ev.slots)]
+    a = diagonal_transform(ev, a, H, n, w)
+    b = ev.encode(tau_plain(ev.pt_values(b_pt), n, w), ev.level_of(b_pt))
+    a = ev.level_down(a, T + 2)
+    b = ev.pt_reencode(b, T + 2)
+    res = ev.mult_pt(a, b)
+    a = ev.left_rotate(a, 1)
+    b = ev.left_rotate(b, w)
+    a_wrap = ev.right_rotate(a, n)
+    b_wrap = ev.right_rotate(b, n * w)
+    acc = None
+    for i in range(1, n):
+        if i > 1:
+            a = ev.left_rotate(a, 1)
+            a_wrap = ev.left_rotate(a_wrap, 1)
+            b = ev.left_rotate(b, w)
+            b_wrap = ev.left_rotate(b_wrap, w)
+        t1 = ev.rescale(ev.masked_sum(a, cm[2 * i + 1], a_wrap, cm[2 * i]))
+        p = ev.pt_add(ev.pt_mult(b, rm[2 * i + 1]), ev.pt_mult(b_wrap, rm[2 * i]))
+        t = ev.mult_pt(t1, p)
+        acc = t if acc is None else ev.add(acc, t)
+    return ev.add(res, acc)
+
+
+def complex_packing_cols(ev, t, n, w):
+    """HEMMer::complexPackingInplace (HEMMer.cpp:764-777): columns (2c, 2c+1) -> a + i b in both."""
+    even = (np.arange(ev.slots) % 2 == 0).astype(np.complex128)
+    m = ev.encode(even, ev.level_of(t))
+    e = ev.mult_pt(t, m)
+    o = ev.mult_pt(ev.mult_imag_unit(ev.left_rotate(t, 1)), m)
+    fus = ev.add(o, e)
+    return ev.add(ev.right_rotate(fus, 1), fus)
+
+
+def complex_packing_rows(ev, t, n, w):
+    """HEMMer::complexPackingRowInplace (HEMMer.cpp:801-817): rows (2k, 2k+1) -> a - i b in both."""
+    even = ((np.arange(ev.slots) // w) % 2 == 0).astype(np.complex128)
+    m = ev.encode(even, ev.level_of(t))
+    e = ev.mult_pt(t, m)
+    o = ev.mult_pt(ev.negate(ev.mult_imag_unit(ev.left_rotate(t, w))), m)
+    fus = ev.add(e, o)
+    return ev.add(ev.right_rotate(fus, w), fus)
+
+
+def mult_packed_mat_mat(ev, a, b, T, n, w):
+    """multPackedMatMat (:1100-1216) on complex-packed operands."""
+    cm = [ev.encode(m, T + 2) for m in col_masks(n, ev.slots)]
+    a = ev.level_down(a, T + 3)
+    b = ev.level_down(b, T + 2)
+    a = diagonal_transform(ev, a, PH, n, w)
+    b = diagonal_transform(ev, b, PV, n, w)
+    res = ev.mult(a, b)
+    a = ev.left_rotate(a, 2)
+    b = ev.left_rotate(b, 2 * w)
+    a_wrap = ev.right_rotate(a, n)
+    acc = None
+    for i in range(1, n // 2):
+        if i > 1:
+            a = ev.left_rotate(a, 2)
+            a_wrap = ev.left_rotate(a_wrap, 2)
+            b = ev.left_rotate(b, 2 * w)
+        t1 = ev.rescale(ev.masked_sum(a, cm[4 * i + 1], a_wrap, cm[4 * i]))
+        t = ev.tensor(t1, b)
+        acc = t if acc is None else ev.add(acc, t)
+    out = ev.rescale(ev.relinearize(acc))
+    return ev.add(res, out)
+
+
+def repack_cc(ev, t):
+    """HEMMer::repackCC (HEMMer.cpp:964-969): x + conj(x)."""
+    return ev.add(t, ev.conjugate(t))
+
+
+def mult_mat_mat_pre(ev, a, T, n, w):
+    """multMatMatPre (:1572-1610): all column shifts of sigma(A), at level T+1."""
+    cm = [ev.encode(m, T + 2) for m in col_masks(n, ev.slots)]
+    a = ev.level_down(a, T + 3)
+    a = diagonal_transform(ev, a, H, n, w)
+    tmp = [ev.level_down_one(a)]
+    a = ev.left_rotate(a, 1)
+    a_wrap = ev.right_rotate(a, n)
+    for i in range(1, n):
+        if i > 1:
+            a = ev.left_rotate(a, 1)
+            a_wrap = ev.left_rotate(a_wrap, 1)
+        tmp.append(ev.rescale(ev.masked_sum(a, cm[2 * i + 1], a_wrap, cm[2 * i])))
+    return tmp
+
+
+def mult_mat_mat_reuse(ev, tmp, b_pt, T):
+    """multMatMatReUse (:1612-1639) with eval.matmul spelled out:
+    rescale(sum_k tmp[k] * leftRotate(pt, k * slots / len(tmp)))."""
+    if ev.level_of(b_pt) != T + 1:
+        b_pt = ev.pt_reencode(b_pt, T + 1)
+    step = ev.slots // len(tmp)
+    acc = None
+    for k, c in enumerate(tmp):
+        t = ev.mult_plain_no_rescale(c, ev.left_rotate(b_pt, k * step))
+        acc = t if acc is None else ev.add(acc, t)
+    return ev.rescale(acc)
+
+
+def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
+    """HEMMer::msgDiagonalToRow4 (HEMMer.cpp:353-399)."""
+    h, w = w1.shape
+    msg = np.zeros(slots, dtype=np.complex128)
+    left = 0.5 * (w1 - 1j * w3)
+    right = 0.5 * (w2 - 1j * w4)
+    for c in range(w):
+        msg[np.arange(h) * 2 * w + c] = np.roll(left[:, c], -c)
+        msg[np.arange(h) * 2 * w + w + c] = np.roll(right[:, c], -c)
+    return msg

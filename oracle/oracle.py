@@ -504,6 +504,9 @@ class Oracle:
         for i in range(nq):
             self.L.orc_automorphism_ntt(self.h, _p(np.ascontiguousarray(x.data[0, i])), _p(rb[i]), g)
             self.L.orc_automorphism_ntt(self.h, _p(np.ascontiguousarray(x.data[1, i])), _p(ra[i]), g)
+        if ("gal", g) not in self.keys and getattr(self, "key_seed", None) is not None:
+            # keys are a deterministic function of (seed, Galois element): derive on first use
+            self.keys[("gal", g)] = self._gen_switch_key(self.key_seed, g, self._sk_automorphism(g))
         ob, oa = self.keyswitch(ra, self.keys[("gal", g)])
         out = np.empty((2, nq, self.N), dtype=np.uint64)
         out[0] = self._binary(0, rb, ob)
@@ -536,7 +539,7 @@ class Oracle:
             return x.copy()
         assert x.level > target
         t = Ct(np.ascontiguousarray(x.data[:, : target + 2]), x.scale)
-        c = int(round(self.delta[target] * float(self.q[target + 1]) / x.scale))
+        c = int(math.floor(self.delta[target] * float(self.q[target + 1]) / x.scale + 0.5))
         t = Ct(self.mult_scalar_residues(t, c), t.scale * c)
         r = self.rescale(t)
         r.scale = self.delta[target]

@@ -1,0 +1,228 @@
+"""GPU parity of the HEMMer layer.
+
+Small ring (N = 1024, 16 x 16 tiles): the GPU path and the CPU oracle share primes, seed-derived
+secret / evaluation keys and input ciphertexts, run the same operation sequence, and must agree on
+every residue (bit-exact).  Full ring (N = 2^16, 128 x 128 tiles, 13 + 4 primes, dnum 3, scale 2^42):
+decrypted products are checked against float64 A @ B within 2^-12 max-abs (tolerance asked for the
+128 x 128 CCMM on U(-1,1) inputs; the reference's own checks use 2^-15 .. 2^-10)."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle import hemmer_ref as R
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 2.0 ** -12
+
+
+def gen_oracle_keys(orc, seed, n):
+    orc.gen_secret(seed)
+    orc.gen_mult_key(seed)
+    orc.gen_conj_key(seed)
+    orc.key_seed = seed          # rotation keys are derived from (seed, Galois element) on first use
+
+
+@pytest.fixture(scope="module")
+def small():
+    pkg = load_package()
+    from efla_amd import hellm
+    qs, ps = O.ckks_chain(10, 8, 3)
+    H = hellm.HEMMer(10, qs, ps, dnum=3, min_bootstrap_level=0, seed=7)
+    orc = O.Oracle(10, qs, ps, dnum=3)
+    gen_oracle_keys(orc, 7, H.dim)
+    return H, orc, R.OracleEval(orc)
+
+
+@pytest.fixture(scope="module")
+def full():
+    load_package()
+    from efla_amd import hellm
+    return hellm.HEMMer(preset=True, seed=3)
+
+
+def to_oracle(orc, ct):
+    i = ct.info()
+    assert i["rescale_counter"] == 0
+    return O.Ct(ct.residues(), orc.delta[i["level"]])
+
+
+def test_keys_and_encoding_match_oracle(small):
+    H, orc, _ = small
+    assert np.array_equal(H.secret_coeffs(), orc.sk_coeffs)
+    assert np.array_equal(H.export_key(0), orc.keys["mult"])
+    H.ensure_rotation_keys([1, 5])
+    for r in (1, 5):
+        orc.gen_rot_key(7, r)
+        g = orc.galois(r)
+        assert np.array_equal(H.export_key(g), orc.keys[("gal", g)])
+    assert np.array_equal(H.export_key(2 * H.N - 1), orc.keys[("gal", 2 * H.N - 1)])
+    # host-side encoding (embedding FFT + rounding) gives the oracle's residues
+    rng = np.random.default_rng(1)
+    M = rng.uniform(-1, 1, (16, 16))
+    z = np.zeros(orc.slots, dtype=np.complex128)
+    z[:256] = M.reshape(-1)
+    for level in (7, 3):
+        assert np.array_equal(H.encode(M, level).residues(), orc.encode(z, level).data)
+
+
+def test_evaluator_calls_bit_exact(small):
+    H, orc, ev = small
+    rng = np.random.default_rng(2)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    oa, ob = to_oracle(orc, ca), to_oracle(orc, cb)
+    assert np.abs(orc.decrypt(oa)[:256].real.reshape(16, 16) - A).max() < 1e-8
+    assert np.array_equal(H.left_rotate(ca, 1).residues(), ev.left_rotate(oa, 1).data)
+    assert np.array_equal(H.conjugate(ca).residues(), ev.conjugate(oa).data)
+    assert np.array_equal(H.mult(ca, cb).residues(), ev.mult(oa, ob).data)
+    assert np.array_equal(H.level_down(ca, 3).residues(), ev.level_down(oa, 3).data)
+    assert np.array_equal(H.mult_imag_unit(ca).residues(), ev.mult_imag_unit(oa).data)
+    lo = H.level_down(cb, 4)
+    assert np.array_equal(H.add(ca, lo).residues(), ev.add(oa, ev.level_down(ob, 4)).data)
+
+
+def test_sigma_tau_bit_exact(small):
+    H, orc, ev = small
+    rng = np.random.default_rng(3)
+    A = rng.uniform(-1, 1, (16, 16))
+    ca = H.encrypt(A)
+    oa = to_oracle(orc, ca)
+    s = H.diagonal_to_column(ca)
+    assert np.array_equal(s.residues(), R.diagonal_transform(ev, oa, R.H, 16, 16).data)
+    t = H.diagonal_to_row(ca)
+    assert np.array_equal(t.residues(), R.diagonal_transform(ev, oa, R.V, 16, 16).data)
+    i, j = np.meshgrid(np.arange(16), np.arange(16), indexing="ij")
+    assert np.abs(H.decrypt(s) - A[i, (i + j) % 16]).max() < 1e-7
+    tr = ca.clone()
+    H.transpose_inplace(tr)
+    assert np.array_equal(tr.residues(), R.transpose(ev, oa, 16, 16).data)
+
+
+def test_ccmm_residues_bit_exact_and_decrypts(small):
+    H, orc, ev = small
+    rng = np.random.default_rng(4)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    c = H.single_cc_matmul(ca, cb, 2)
+    want = R.mult_mat_mat_cc(ev, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16)
+    assert c.info()["level"] == 2
+    assert np.array_equal(c.residues(), want.data)
+    assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
+
+
+def test_pcmm_and_packed_bit_exact(small):
+    H, orc, ev = small
+    rng = np.random.default_rng(5)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ca = H.encrypt(A)
+    pb = H.encode(B)
+    c = H.single_matmul(ca, pb, 2)
+    opb = O.Pt(pb.residues(), orc.delta[orc.nQ - 1])
+    want = R.mult_mat_mat_pc(ev, to_oracle(orc, ca), opb, 2, 16, 16)
+    assert np.array_equal(c.residues(), want.data)
+    assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
+    A2, B2 = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    pa, pbb = H.encrypt2(A, A2), H.encrypt2(B, B2)
+    oa, ob = to_oracle(orc, pa), to_oracle(orc, pbb)
+    H.complex_packing_inplace(pa)
+    H.complex_packing_row_inplace(pbb)
+    oa = R.complex_packing_cols(ev, oa, 16, 32)
+    ob = R.complex_packing_rows(ev, ob, 16, 32)
+    assert np.array_equal(pa.residues(), oa.data) and np.array_equal(pbb.residues(), ob.data)
+    pc = H.repack_cc(H.packed_matmul(pa, pbb, 2))
+    want = R.repack_cc(ev, R.mult_packed_mat_mat(ev, oa, ob, 2, 16, 32))
+    assert np.array_equal(pc.residues(), want.data)
+    d = H.decrypt2(pc)
+    assert np.abs(d[0] - A @ B).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
+
+
+def test_hoisted_products_bit_exact(small):
+    H, orc, ev = small
+    n = 16
+    rng = np.random.default_rng(6)
+    X0, X1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    W = [rng.normal(0, 0.02, (n, n)) for _ in range(4)]
+    x = H.complex_packing(H.encrypt2(X0, X0), H.encrypt2(X1, X1))
+    ox = to_oracle(orc, x)
+    tmp = H.matmul_pre(x, 2)
+    otmp = R.mult_mat_mat_pre(ev, ox, 2, n, 2 * n)
+    assert len(tmp) == n
+    for k in (0, 1, n - 1):
+        assert np.array_equal(tmp.get(k, n, n, 2 * n).residues(), otmp[k].data)
+    wp = H.encode_diagonal_to_row4(*W, level=3)
+    owp = orc.encode(R.weights_diagonal_to_row4(*W, orc.slots), 3)
+    assert np.array_equal(wp.residues(), owp.data)
+    y = H.matmul_reuse(tmp, wp, 2)
+    assert np.array_equal(y.residues(), R.mult_mat_mat_reuse(ev, otmp, owp, 2).data)
+    z = H.decrypt2(H.repack_cc(y))
+    assert np.abs(z[0] - (X0 @ W[0] + X1 @ W[2])).max() < 2 ** -18
+    assert np.abs(z[1] - (X0 @ W[1] + X1 @ W[3])).max() < 2 ** -18
+
+
+def test_error_behaviour(small):
+    H, _, _ = small
+    A = np.ones((16, 16))
+    ca = H.encrypt(A)
+    low = H.level_down(ca, 3)
+    zero = H.level_down(ca, 0)
+    with pytest.raises(ValueError):            # std::invalid_argument("[multMatMat] level >= 1 is needed.")
+        H.single_cc_matmul(zero, zero, 2)
+    with pytest.raises(pkg_error()):           # level < 4 + minimum bootstrap level: the reference would
+        H.single_cc_matmul(low, low, 2)        # bootstrap here; this build raises instead
+    mid = H.level_down(ca, 4)
+    with pytest.raises(ValueError):            # enough to skip bootstrapping, too low for target level 2
+        H.single_cc_matmul(mid, mid, 2)
+    pa = H.encrypt2(A, A)
+    with pytest.raises(ValueError):            # block widths differ
+        H.single_cc_matmul(ca, pa, 2)
+    with pytest.raises(pkg_error()):           # rescale / level errors surface as runtime errors
+        H.level_down(low, 5)
+
+
+def pkg_error():
+    return load_package().HemmError
+
+
+# ---- full size -----------------------------------------------------------------------------------
+def test_full_ccmm_128(full):
+    H = full
+    rng = np.random.default_rng(1)
+    A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    assert ca.info()["level"] == 12
+    c = H.single_cc_matmul(ca, cb, 4)
+    assert c.info()["level"] == 4
+    err = np.abs(H.decrypt(c) - A @ B).max()
+    assert err < TOL, err
+    z = H.decrypt_slots(c)
+    assert np.abs(z[128 * 128:]).max() < TOL           # upper half of the slots stays empty
+    # linearity in the encrypted operand: (2A) B = 2 (A B)
+    c2 = H.single_cc_matmul(H.add(ca, ca), cb, 4)
+    assert np.abs(H.decrypt(c2) - 2 * (A @ B)).max() < TOL
+
+
+def test_full_pcmm_packed_and_hoisted(full):
+    H = full
+    rng = np.random.default_rng(2)
+    A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    A2, B2 = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    c = H.single_matmul(H.encrypt(A), H.encode(B), 4)
+    assert np.abs(H.decrypt(c) - A @ B).max() < TOL
+    pa, pb = H.encrypt2(A, A2), H.encrypt2(B, B2)
+    H.complex_packing_inplace(pa)
+    H.complex_packing_row_inplace(pb)
+    d = H.decrypt2(H.repack_cc(H.packed_matmul(pa, pb, 4)))
+    assert np.abs(d[0] - A @ B).max() < TOL and np.abs(d[1] - A2 @ B2).max() < TOL
+    W = [rng.normal(0, 0.02, (128, 128)) for _ in range(4)]
+    X0, X1 = 0.1 * rng.normal(size=(128, 128)), 0.1 * rng.normal(size=(128, 128))
+    x = H.complex_packing(H.encrypt2(X0, X0), H.encrypt2(X1, X1))
+    tmp = H.matmul_pre(x, 4)
+    y = H.matmul_reuse(tmp, H.encode_diagonal_to_row4(*W, level=5), 4)
+    z = H.decrypt2(H.repack_cc(y))
+    assert np.abs(z[0] - (X0 @ W[0] + X1 @ W[2])).max() < 2 ** -10
+    assert np.abs(z[1] - (X0 @ W[1] + X1 @ W[3])).max() < 2 ** -10
+    t = H.encrypt2(A, A2)
+    H.transpose_inplace(t)
+    d = H.decrypt2(t)
+    assert np.abs(d[0] - A.T).max() < TOL and np.abs(d[1] - A2.T).max() < TOL

@@ -1,0 +1,110 @@
+"""Pins the restated HEMMer algorithms (oracle/hemmer_ref.py) on exact slot vectors: every mask and
+rotation index must reproduce float64 matrix algebra, at the reference's 128 x 128 / 2^15-slot shape
+and on a small tile.  No cryptography involved."""
+import numpy as np
+import pytest
+
+from oracle import hemmer_ref as R
+
+
+def setup(n, top=12):
+    slots = 2 * n * n
+    ev = R.SlotSim(slots.bit_length() - 1, top)
+    rng = np.random.default_rng(n)
+    return ev, rng
+
+
+def single(ev, M, n):
+    return ev.encrypt(M.reshape(-1))
+
+
+def pair(ev, M1, M2):
+    return ev.encrypt(np.concatenate([M1, M2], axis=1).reshape(-1))
+
+
+@pytest.mark.parametrize("n", [8, 128])
+def test_sigma_tau_transpose(n):
+    ev, rng = setup(n)
+    A = rng.uniform(-1, 1, (n, n))
+    i, j = np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
+    for w, enc in ((n, lambda M: single(ev, M, n)), (2 * n, lambda M: pair(ev, M, 2 * M))):
+        s = R.diagonal_transform(ev, enc(A), R.H, n, w)
+        got = ev.decrypt(s).real.reshape(-1, w)[:n, :n]
+        assert np.array_equal(got, A[i, (i + j) % n]) and s.level == 11 and s.rc == 0
+        t = R.diagonal_transform(ev, enc(A), R.V, n, w)
+        assert np.array_equal(ev.decrypt(t).real.reshape(-1, w)[:n, :n], A[(i + j) % n, j])
+        tr = R.transpose(ev, enc(A), n, w)
+        assert np.array_equal(ev.decrypt(tr).real.reshape(-1, w)[:n, :n], A.T)
+        if w == 2 * n:   # the second tile of the pair is transformed independently
+            assert np.array_equal(ev.decrypt(tr).real.reshape(-1, w)[:n, n:], 2 * A.T)
+
+
+@pytest.mark.parametrize("n", [8, 128])
+def test_ccmm_single_and_pair_layout(n):
+    ev, rng = setup(n)
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    c = R.mult_mat_mat_cc(ev, single(ev, A, n), single(ev, B, n), 4, n, n)
+    z = ev.decrypt(c)
+    assert c.level == 4 and c.rc == 0
+    assert np.abs(z[: n * n].real.reshape(n, n) - A @ B).max() < 1e-12
+    assert np.abs(z[n * n:]).max() == 0           # upper half of the slots stays empty
+    A2, B2 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    c = R.mult_mat_mat_cc(ev, pair(ev, A, A2), pair(ev, B, B2), 4, n, 2 * n)
+    z = ev.decrypt(c).real.reshape(n, 2 * n)
+    assert np.abs(z[:, :n] - A @ B).max() < 1e-12 and np.abs(z[:, n:] - A2 @ B2).max() < 1e-12
+
+
+@pytest.mark.parametrize("n", [8, 128])
+def test_pcmm_unhoisted(n):
+    ev, rng = setup(n)
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    bp = ev.encode(single(ev, B, n).z, 12)
+    c = R.mult_mat_mat_pc(ev, single(ev, A, n), bp, 4, n, n)
+    assert np.abs(ev.decrypt(c)[: n * n].real.reshape(n, n) - A @ B).max() < 1e-12
+
+
+@pytest.mark.parametrize("n", [8, 128])
+def test_packed_ccmm_two_products_per_call(n):
+    ev, rng = setup(n)
+    A1, A2, B1, B2 = (rng.uniform(-1, 1, (n, n)) for _ in range(4))
+    a = R.complex_packing_cols(ev, pair(ev, A1, A2), n, 2 * n)
+    b = R.complex_packing_rows(ev, pair(ev, B1, B2), n, 2 * n)
+    # packing: both slots of a column pair hold a + i b; both rows of a row pair hold a - i b
+    za = ev.decrypt(a).reshape(n, 2 * n)
+    assert np.allclose(za[:, 0:n:2], A1[:, 0::2] + 1j * A1[:, 1::2]) and np.allclose(za[:, 0:n:2], za[:, 1:n:2])
+    zb = ev.decrypt(b).reshape(n, 2 * n)
+    assert np.allclose(zb[0::2, :n], B1[0::2] - 1j * B1[1::2]) and np.allclose(zb[0::2], zb[1::2])
+    c = R.repack_cc(ev, R.mult_packed_mat_mat(ev, a, b, 4, n, 2 * n))
+    z = ev.decrypt(c).reshape(n, 2 * n)
+    assert np.abs(z.imag).max() < 1e-12
+    assert np.abs(z.real[:, :n] - A1 @ B1).max() < 1e-12 and np.abs(z.real[:, n:] - A2 @ B2).max() < 1e-12
+    assert c.level == 4
+
+
+@pytest.mark.parametrize("n", [8, 128])
+def test_hoisted_plaintext_product(n):
+    """complexPacking(x0, x1) -> matMulPre -> matMulReUse(encodeDiagonalToRow4(W..)) gives
+    Re = X0 W1 + X1 W3 (left) | X0 W2 + X1 W4 (right) after x + conj(x)."""
+    ev, rng = setup(n)
+    X0, X1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    W = [rng.normal(0, 0.02, (n, n)) for _ in range(4)]
+    x0 = pair(ev, X0, X0)
+    x1 = pair(ev, X1, X1)
+    x = ev.add(x0, ev.mult_imag_unit(x1))                     # HEMMer::complexPacking(ct, ct)
+    tmp = R.mult_mat_mat_pre(ev, x, 4, n, 2 * n)
+    assert len(tmp) == n and all(t.level == 5 for t in tmp)
+    wp = ev.encode(R.weights_diagonal_to_row4(*W, ev.slots), 5)
+    y = R.mult_mat_mat_reuse(ev, tmp, wp, 4)
+    z = ev.decrypt(R.repack_cc(ev, y)).real.reshape(n, 2 * n)
+    assert y.level == 4
+    assert np.abs(z[:, :n] - (X0 @ W[0] + X1 @ W[2])).max() < 1e-12
+    assert np.abs(z[:, n:] - (X0 @ W[1] + X1 @ W[3])).max() < 1e-12
+
+
+def test_assemble_masks_are_complementary():
+    n, slots = 8, 128
+    cm, rm = R.col_masks(n, slots), R.row_masks(n, n, slots)
+    for i in range(n):
+        assert np.array_equal(cm[2 * i] + cm[2 * i + 1], np.ones(slots))
+        assert np.array_equal(rm[2 * i] + rm[2 * i + 1], np.ones(slots))
+        assert cm[2 * i].sum() == i * slots // n and rm[2 * i].sum() == i * slots // n

@@ -1,0 +1,50 @@
+"""The restated algorithms over the CPU RNS-CKKS oracle (N = 1024, 16 x 16 tiles): decrypted
+products equal float64 A @ B, which pins the composition of oracle primitives that the GPU residues
+are later compared against."""
+import numpy as np
+import pytest
+
+from oracle import hemmer_ref as R
+from oracle import oracle as O
+
+
+@pytest.fixture(scope="module")
+def env():
+    qs, ps = O.ckks_chain(10, 8, 3)
+    orc = O.Oracle(10, qs, ps, dnum=3)
+    orc.gen_secret(7)
+    orc.gen_mult_key(7)
+    orc.gen_conj_key(7)
+    n = 16
+    orc.key_seed = 7
+    return orc, R.OracleEval(orc), n
+
+
+def enc(orc, M, seed):
+    z = np.zeros(orc.slots, dtype=np.complex128)
+    z[: M.size] = M.reshape(-1)
+    return orc.encrypt(orc.encode(z, orc.nQ - 1), seed)
+
+
+def test_ccmm_over_oracle(env):
+    orc, ev, n = env
+    rng = np.random.default_rng(0)
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    c = R.mult_mat_mat_cc(ev, enc(orc, A, 11), enc(orc, B, 12), 2, n, n)
+    assert c.level == 2
+    z = orc.decrypt(c)
+    assert np.abs(z[: n * n].real.reshape(n, n) - A @ B).max() < 2 ** -20
+    assert np.abs(z[n * n:]).max() < 2 ** -20
+
+
+def test_packed_ccmm_over_oracle(env):
+    orc, ev, n = env
+    rng = np.random.default_rng(1)
+    A1, A2, B1, B2 = (rng.uniform(-1, 1, (n, n)) for _ in range(4))
+    a = R.complex_packing_cols(ev, enc(orc, np.concatenate([A1, A2], 1), 13), n, 2 * n)
+    b = R.complex_packing_rows(ev, enc(orc, np.concatenate([B1, B2], 1), 14), n, 2 * n)
+    c = R.repack_cc(ev, R.mult_packed_mat_mat(ev, a, b, 2, n, 2 * n))
+    z = orc.decrypt(c).reshape(n, 2 * n)
+    assert np.abs(z.real[:, :n] - A1 @ B1).max() < 2 ** -18
+    assert np.abs(z.real[:, n:] - A2 @ B2).max() < 2 ** -18
+    assert np.abs(z.imag).max() < 2 ** -18
