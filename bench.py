@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the HEMMer hot path on one MI355X.
+
+Headline (the metric BASELINE.json names): ms per 128 x 128 ciphertext-ciphertext matrix product
+(HEMMer::singleCCMatMul, N = 2^16, 13 + 4 primes, dnum 3, scale 2^42, inputs fresh at level 12,
+target level 4), inputs and keys resident in HBM.  Also reported in the same JSON line: batched
+NTT limb-transforms/s (32 polys x 24 limbs x 2^16, 60-bit primes), one key-switched rotation at
+level 12, the roofline of the NTT kernels (HBM bound) and the CPU oracle timed on the host cores.
+
+A "step" is one full CCMM.  Everything runs on one GPU; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+LIMB_BYTES = (1 << 16) * 8
+
+
+def gpu_ccmm(args, out):
+    import numpy as np
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    from efla_amd import hellm
+    H = hellm.HEMMer(preset=True, seed=3)
+    rng = np.random.default_rng(1)
+    A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    T = 4
+    t0 = time.perf_counter()
+    c = H.single_cc_matmul(ca, cb, T)          # first call also builds keys and masks
+    H.sync()
+    out["setup_s"] = round(time.perf_counter() - t0, 3)
+    for _ in range(args.warmup):
+        c = H.single_cc_matmul(ca, cb, T)
+    H.sync()
+    timer = pkg.Timer()
+    t0 = time.perf_counter()
+    timer.start()
+    for _ in range(args.steps):
+        c = H.single_cc_matmul(ca, cb, T)
+    ev_ms = timer.stop()
+    H.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    err = float(np.abs(H.decrypt(c) - A @ B).max())
+    out["ms_per_step"] = wall_ms / args.steps
+    out["value"] = wall_ms / args.steps
+    out["gpu_event_ms_per_step"] = ev_ms / args.steps
+    out["max_abs_err"] = err
+    out["max_abs_err_ok"] = bool(err <= 2.0 ** -12)
+    # one rotation (automorphism + hybrid key switch) at the top level
+    r = H.left_rotate(ca, 1)
+    H.sync()
+    timer.start()
+    for _ in range(50):
+        r = H.left_rotate(ca, 1)
+    out["rotation_level12_us"] = timer.stop() / 50 * 1e3
+    low = H.level_down(ca, 6)
+    r = H.left_rotate(low, 1)
+    H.sync()
+    timer.start()
+    for _ in range(50):
+        r = H.left_rotate(low, 1)
+    out["rotation_level6_us"] = timer.stop() / 50 * 1e3
+    return H
+
+
+def gpu_ntt(args, out):
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    qs = pkg.primes_below(60, 16, 24)
+    ctx = pkg.Context(16, qs, [], 1)
+    q_t = torch.tensor(qs, dtype=torch.int64, device="cuda").view(1, 24, 1)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    d = torch.randint(0, 2 ** 62, (32, 24, 1 << 16), dtype=torch.int64, device="cuda", generator=g) % q_t
+    ref = d.clone()
+    idx = list(range(24))
+    for _ in range(3):
+        ctx.ntt(d, idx)
+        ctx.ntt(d, idx, inverse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(d, ref), "NTT round trip is not bit-exact"
+    timer = pkg.Timer()
+    iters = 20
+    timer.start()
+    for _ in range(iters):
+        ctx.ntt(d, idx)
+    fwd_ms = timer.stop() / iters
+    timer.start()
+    for _ in range(iters):
+        ctx.ntt(d, idx, inverse=True)
+    inv_ms = timer.stop() / iters
+    limbs = 32 * 24
+    out["ntt_forward_limbs_per_s"] = limbs / fwd_ms * 1e3
+    out["ntt_inverse_limbs_per_s"] = limbs / inv_ms * 1e3
+    out["ntt_limbs_per_s"] = 2 * limbs / (fwd_ms + inv_ms) * 1e3
+    # roofline of the dominant kernel family: one forward transform of the batch = one launch of
+    # ntt16_cols_kernel + one of ntt16_rows_kernel; algorithmic traffic = read + write of every limb
+    # once = 1 MiB per limb-transform
+    alg_bytes = limbs * 2 * LIMB_BYTES
+    achieved = alg_bytes / (fwd_ms * 1e-3) / 1e9
+    out["roofline"] = {
+        "kernel": "ntt16_cols_kernel<false> + ntt16_rows_kernel<false> (one forward transform of "
+                  "32x24 limbs = 2 launches)",
+        "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+        "algorithmic_bytes_per_launch_pair": alg_bytes, "avg_ms_per_launch_pair": fwd_ms,
+    }
+
+
+def cpu_baseline(out, budget_s=25.0):
+    """The CPU oracle (scalar C++ port, one thread) on a bounded sample of the CCMM's operation mix,
+    scaled by the per-product operation counts."""
+    import numpy as np
+    from oracle import oracle as O
+    qs, ps = O.ckks_chain(16, 13, 4)
+    orc = O.Oracle(16, qs, ps, dnum=3, threads=1)
+    orc.gen_secret(3)
+    orc.key_seed = 3
+    orc.gen_mult_key(3)
+    rng = np.random.default_rng(0)
+    z = rng.uniform(-1, 1, orc.slots).astype(np.complex128)
+    ct12 = orc.encrypt(orc.encode(z, 12), 4)
+    ct6 = orc.level_down(ct12, 6)
+    ct5 = orc.level_down(ct12, 5)
+    m12, m6 = orc.encode(z, 12), orc.encode(z, 6)
+    orc.left_rotate(ct6, 1)   # derive the key outside the timed region
+
+    def t(fn, reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    t_rot12 = t(lambda: orc.left_rotate(ct12, 1), 2)
+    t_rot6 = t(lambda: orc.left_rotate(ct6, 1), 4)
+    t_mul12 = t(lambda: orc.mult_plain_no_rescale(ct12, m12), 2)
+    t_mul6 = t(lambda: orc.mult_plain_no_rescale(ct6, m6), 4)
+    pre = orc.mult_plain_no_rescale(ct6, m6)
+    t_res6 = t(lambda: orc.rescale(pre), 4)
+    t_tensor5 = t(lambda: orc.tensor(ct5, ct5), 4)
+    t3 = orc.tensor(ct5, ct5)
+    t_relin5 = t(lambda: orc.relinearize(t3), 2)
+    # operation counts of one 128 x 128 CCMM: 2 transforms (32 rotations + 255 mask products each at
+    # level 12), 508 rotations + 508 mask products + 254 rescales at level 6, 127 tensor products,
+    # 2 relinearisations
+    total = (64 * t_rot12 + 510 * t_mul12 + 508 * t_rot6 + 508 * t_mul6 + 254 * t_res6 +
+             128 * t_tensor5 + 2 * t_relin5)
+    out["cpu_baseline"] = {
+        "value": total * 1e3, "unit": "ms", "cores": 1, "kind": "port",
+        "sample": "CPU oracle, 1 thread: timed 2 rotations + 2 mask products at level 12, 4 rotations, "
+                  "4 mask products, 4 rescales at level 6, 4 tensor products + 2 relinearisations at "
+                  "level 5; scaled by the operation counts of one CCMM (64/510/508/508/254/128/2)",
+        "rotation_level12_ms": t_rot12 * 1e3, "rotation_level6_ms": t_rot6 * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU hot path only: run it with --gpus 1 "
+              "(no multi-GPU figure is produced by this build)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback for the product path)", file=sys.stderr)
+        sys.exit(3)
+    out = {
+        "metric": "ms per 128x128 CCMM (N=2^16) on 1 GPU", "value": None, "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u64", "data": "synthetic",
+        "config": {"workload": "singleCCMatMul 128x128 U(-1,1) seeded, N=2^16, 13 chain (60-bit + 12x42-bit) "
+                               "+ 4 special 60-bit primes, dnum=3, scale 2^42, inputs fresh at level 12, "
+                               "target level 4, all keys and masks resident in HBM"},
+    }
+    gpu_ccmm(args, out)
+    gpu_ntt(args, out)
+    if not args.no_cpu:
+        cpu_baseline(out)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

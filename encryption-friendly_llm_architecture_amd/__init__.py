@@ -212,6 +212,34 @@ class Context:
 ADD, SUB, MUL, NEG, MAC = 0, 1, 2, 3, 4
 
 
+class Timer:
+    """HIP-event stopwatch on the stream the kernels are launched on (default: the null stream)."""
+
+    def __init__(self, stream=None):
+        L = lib()
+        L.hemm_timer_create.argtypes = [ctypes.POINTER(vp)]
+        L.hemm_timer_start.argtypes = [vp, vp]
+        L.hemm_timer_stop.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+        L.hemm_timer_destroy.argtypes = [vp]
+        self.t = vp()
+        self.stream = vp(stream or 0)
+        check(L.hemm_timer_create(ctypes.byref(self.t)))
+
+    def start(self):
+        check(lib().hemm_timer_start(self.t, self.stream))
+
+    def stop(self):
+        ms = ctypes.c_float()
+        check(lib().hemm_timer_stop(self.t, self.stream, ctypes.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            lib().hemm_timer_destroy(self.t)
+        except Exception:
+            pass
+
+
 def primes_below(bits, log_n, count):
     out = (ctypes.c_uint64 * count)()
     check(lib().hemm_primes_below(bits, log_n, count, out))

@@ -47,6 +47,41 @@ void hemm_context_destroy(hemm_context *ctx) {
 }
 uint64_t hemm_context_psi(const hemm_context *ctx, uint32_t idx) { return ctx->psi.at(idx); }
 
+struct hemm_timer {
+    hipEvent_t a, b;
+};
+int hemm_timer_create(void **timer) {
+    HEMM_TRY
+    need(timer, "null argument");
+    hemm_timer *t = new hemm_timer();
+    HEMM_HIP(hipEventCreate(&t->a));
+    HEMM_HIP(hipEventCreate(&t->b));
+    *timer = t;
+    HEMM_CATCH
+}
+int hemm_timer_start(void *timer, void *stream) {
+    HEMM_TRY
+    need(timer, "null argument");
+    HEMM_HIP(hipEventRecord(((hemm_timer *)timer)->a, (hipStream_t)stream));
+    HEMM_CATCH
+}
+int hemm_timer_stop(void *timer, void *stream, float *ms) {
+    HEMM_TRY
+    need(timer && ms, "null argument");
+    hemm_timer *t = (hemm_timer *)timer;
+    HEMM_HIP(hipEventRecord(t->b, (hipStream_t)stream));
+    HEMM_HIP(hipEventSynchronize(t->b));
+    HEMM_HIP(hipEventElapsedTime(ms, t->a, t->b));
+    HEMM_CATCH
+}
+void hemm_timer_destroy(void *timer) {
+    if (!timer) return;
+    hemm_timer *t = (hemm_timer *)timer;
+    (void)hipEventDestroy(t->a);
+    (void)hipEventDestroy(t->b);
+    delete t;
+}
+
 int hemm_primes_below(uint32_t bits, uint32_t log_n, uint32_t count, uint64_t *out) {
     HEMM_TRY
     need(out && bits >= 21 && bits <= 61 && log_n >= 1 && log_n + 2 <= bits, "bad arguments");

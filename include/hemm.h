@@ -38,6 +38,13 @@ uint64_t hemm_context_psi(const hemm_context *ctx, uint32_t idx);
  * (HEaaN::getPrimeList, Context.hpp:201, is a fixed preset; this build takes explicit lists). */
 int hemm_primes_below(uint32_t bits, uint32_t log_n, uint32_t count, uint64_t *out);
 
+/* HIP-event stopwatch on `stream` (the reference times with cudaDeviceSynchronize + std::chrono,
+ * ciphertext/src/TransformerBlock.cpp:101-112).  stop() waits for the stream and returns ms. */
+int hemm_timer_create(void **timer);
+int hemm_timer_start(void *timer, void *stream);
+int hemm_timer_stop(void *timer, void *stream, float *ms);
+void hemm_timer_destroy(void *timer);
+
 /* Batched negacyclic NTT (inverse = 0: natural -> bit-reversed order) or INTT (inverse = 1,
  * including 1/N) in place over data[n_polys][n_limbs][N]; limb j uses prime prime_idx[j]
  * (host array).  Every NTT-form operand of HomEvaluator goes through this. */
