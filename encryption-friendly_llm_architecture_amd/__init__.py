@@ -36,6 +36,14 @@ u32p = ctypes.POINTER(ctypes.c_uint32)
 vp = ctypes.c_void_p
 
 
+class RotTerm(ctypes.Structure):
+    _fields_ = [("ext", vp), ("b", vp), ("evk", vp), ("mask", vp), ("galois", ctypes.c_uint64)]
+
+
+class LinTerm(ctypes.Structure):
+    _fields_ = [("ct", vp), ("mask", vp), ("stride", ctypes.c_uint64)]
+
+
 def _declare(L):
     L.hemm_last_error.restype = ctypes.c_char_p
     L.hemm_context_create.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, u64p,
@@ -58,6 +66,11 @@ def _declare(L):
     L.hemm_rotate.argtypes = [vp, vp, sz, vp, u64, u32, vp, sz, vp]
     L.hemm_relinearize.argtypes = [vp, vp, sz, vp, u32, vp, sz, vp]
     L.hemm_rescale.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
+    L.hemm_modup_batch.argtypes = [vp, vp, sz, u32, u32, vp, vp, vp]
+    L.hemm_hoisted_terms.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, vp, vp]
+    L.hemm_moddown_batch.argtypes = [vp, vp, u32, u32, ci, vp, sz, vp, vp]
+    L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
+    L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
 
 
 def check(rc):
@@ -207,6 +220,69 @@ class Context:
         check(lib().hemm_rescale(self.h, vp(ct.data_ptr()), self._ps(ct), vp(out.data_ptr()),
                                  self._ps(out), nq, ct.shape[0], vp(0)))
         return out
+
+
+    # ---- batched / hoisted forms ------------------------------------------------------------
+    def modup_batch(self, polys, nq):
+        """polys: [n_in][>=nq][N] -> ext [n_in][beta][nq+K][N]"""
+        import torch
+        n_in = polys.shape[0]
+        ext = torch.empty((n_in, self.beta(nq), nq + self.nP, self.N), dtype=torch.int64, device=polys.device)
+        ws = torch.empty((n_in, nq, self.N), dtype=torch.int64, device=polys.device)
+        check(lib().hemm_modup_batch(self.h, vp(polys.data_ptr()), polys.stride(0), nq, n_in,
+                                     vp(ext.data_ptr()), vp(ws.data_ptr()), vp(0)))
+        return ext
+
+    def hoisted_terms(self, groups, nq):
+        """groups: list of lists of (ext, b, evk, mask or None, galois) -> y [n_out][2][nq+K][N]"""
+        import torch
+        flat = [t for g in groups for t in g]
+        arr = (RotTerm * len(flat))()
+        for i, (ext, b, evk, mask, gal) in enumerate(flat):
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
+                             mask.data_ptr() if mask is not None else None, gal)
+        offs = [0]
+        for g in groups:
+            offs.append(offs[-1] + len(g))
+        off = (ctypes.c_uint32 * len(offs))(*offs)
+        y = torch.empty((len(groups), 2, nq + self.nP, self.N), dtype=torch.int64, device=flat[0][0].device)
+        check(lib().hemm_hoisted_terms(self.h, arr, off, len(groups), nq, vp(y.data_ptr()), vp(0)))
+        return y
+
+    def moddown_batch(self, y, nq, drop_last):
+        """y: [..., nq+K, N] (clobbered) -> [..., nq - drop_last, N]"""
+        import torch
+        n_polys = y.numel() // ((nq + self.nP) * self.N)
+        nq_out = nq - 1 if drop_last else nq
+        out = torch.empty(tuple(y.shape[:-2]) + (nq_out, self.N), dtype=torch.int64, device=y.device)
+        ws = torch.empty_like(out)
+        check(lib().hemm_moddown_batch(self.h, vp(y.data_ptr()), nq, n_polys, int(drop_last),
+                                       vp(out.data_ptr()), nq_out * self.N, vp(ws.data_ptr()), vp(0)))
+        return out
+
+    def masked_sum_batch(self, groups, nq, n_polys):
+        """groups: list of lists of (ct [n_polys][>=nq][N], mask [>=nq][N] or None)"""
+        import torch
+        flat = [t for g in groups for t in g]
+        arr = (LinTerm * len(flat))()
+        for i, (ct, mask) in enumerate(flat):
+            arr[i] = LinTerm(ct.data_ptr(), mask.data_ptr() if mask is not None else None, ct.stride(0))
+        offs = [0]
+        for g in groups:
+            offs.append(offs[-1] + len(g))
+        off = (ctypes.c_uint32 * len(offs))(*offs)
+        out = torch.empty((len(groups), n_polys, nq, self.N), dtype=torch.int64, device=flat[0][0].device)
+        check(lib().hemm_masked_sum_batch(self.h, arr, off, len(groups), nq, n_polys, vp(out.data_ptr()), vp(0)))
+        return out
+
+    def tensor_batch(self, t1, t2, nq, acc=None):
+        import torch
+        accumulate = acc is not None
+        if acc is None:
+            acc = torch.empty((3, nq, self.N), dtype=torch.int64, device=t1.device)
+        check(lib().hemm_tensor_batch(self.h, vp(t1.data_ptr()), vp(t2.data_ptr()), t1.shape[0], nq,
+                                      vp(acc.data_ptr()), int(accumulate), vp(0)))
+        return acc
 
 
 ADD, SUB, MUL, NEG, MAC = 0, 1, 2, 3, 4

@@ -1,5 +1,6 @@
 // extern "C" boundary (declared in include/hemm.h).
 #include <cstring>
+#include <vector>
 
 #include "../../include/hemm.h"
 #include "hemm_internal.hpp"
@@ -251,6 +252,101 @@ int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, c
                      (hipStream_t)stream);
     launch_binary(ctx, HEMM_ADD, (const u64 *)ct3, ct_stride, tmp, (size_t)nq * N, (u64 *)out, out_stride, ll, nl, 2,
                   (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+// descriptor staging: one device region reused by every call (copies and kernels are ordered on the stream)
+static void *upload_desc(hemm_context *ctx, const void *a, size_t na, const void *b, size_t nb, void **second,
+                         hipStream_t s) {
+    const size_t cap = 4u << 20;
+    if (!ctx->d_desc) HEMM_HIP(hipMalloc(&ctx->d_desc, cap));
+    const size_t off_b = (na + 255) & ~(size_t)255;
+    if (off_b + nb > cap) throw std::invalid_argument("too many terms in one batched call");
+    HEMM_HIP(hipMemcpyAsync(ctx->d_desc, a, na, hipMemcpyHostToDevice, s));
+    HEMM_HIP(hipMemcpyAsync((char *)ctx->d_desc + off_b, b, nb, hipMemcpyHostToDevice, s));
+    *second = (char *)ctx->d_desc + off_b;
+    return ctx->d_desc;
+}
+
+int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint32_t nq, uint32_t n_in,
+                     uint64_t *ext, uint64_t *workspace, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(in && ext && workspace && n_in >= 1, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    launch_modup_batch(ctx, (const u64 *)in, in_stride, (int)nq, (int)n_in, (u64 *)ext, (u64 *)workspace,
+                       (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                       uint32_t nq, uint64_t *y, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(terms && group_offsets && y && n_out >= 1, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    const uint32_t n_terms = group_offsets[n_out];
+    struct Dev {
+        const u64 *ext, *b, *evk, *mask;
+        u32 galois, pad;
+    };
+    std::vector<Dev> d(n_terms);
+    for (uint32_t t = 0; t < n_terms; t++) {
+        need(terms[t].ext && terms[t].b && terms[t].evk, "null pointer in a rotation term");
+        need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
+        d[t] = Dev{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
+                   (const u64 *)terms[t].mask, (u32)terms[t].galois, 0};
+    }
+    void *off_dev = nullptr;
+    void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), group_offsets, (n_out + 1) * sizeof(uint32_t),
+                                  &off_dev, (hipStream_t)stream);
+    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_moddown_batch(hemm_context *ctx, uint64_t *y, uint32_t nq, uint32_t n_polys, int drop_last, uint64_t *out,
+                       size_t out_stride, uint64_t *workspace, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(y && out && workspace && n_polys >= 1, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    launch_moddown_batch(ctx, (u64 *)y, (int)nq, (int)n_polys, drop_last != 0, (u64 *)out, out_stride,
+                         (u64 *)workspace, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                          uint32_t nq, uint32_t n_polys, uint64_t *out, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 0, &nl);
+    need(terms && group_offsets && out && n_out >= 1 && n_polys >= 1, "null operand");
+    const uint32_t n_terms = group_offsets[n_out];
+    for (uint32_t t = 0; t < n_terms; t++) need(terms[t].ct != nullptr, "null pointer in a term");
+    void *off_dev = nullptr;
+    void *terms_dev = upload_desc(ctx, terms, n_terms * sizeof(hemm_lin_term), group_offsets,
+                                  (n_out + 1) * sizeof(uint32_t), &off_dev, (hipStream_t)stream);
+    launch_masked_sum(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
+                      (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_tensor_batch(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
+                      uint64_t *acc3, int accumulate, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 0, &nl);
+    need(t1 && t2 && acc3 && n_pairs >= 1, "null operand");
+    launch_tensor_batch(ctx, (const u64 *)t1, (const u64 *)t2, (int)n_pairs, (int)nq, (u64 *)acc3, accumulate != 0,
+                        (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

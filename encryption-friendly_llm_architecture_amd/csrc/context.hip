@@ -154,6 +154,7 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_imag_s = (u64 *)up(im_s.data(), T * 8);
     c->d_modq = (ModQ *)up(c->modq.data(), T * sizeof(ModQ));
     c->d_scratch = nullptr;
+    c->d_desc = nullptr;
     c->scratch_bytes = 0;
     return c;
 }
@@ -168,5 +169,6 @@ void hemm_context_free(hemm_context *c) {
     hipFree(c->d_imag_s);
     hipFree(c->d_modq);
     if (c->d_scratch) hipFree(c->d_scratch);
+    if (c->d_desc) hipFree(c->d_desc);
     delete c;
 }

@@ -33,6 +33,7 @@ struct hemm_context {
     // scratch owned by the context (single stream use)
     u64 *d_scratch;
     size_t scratch_bytes;
+    void *d_desc;                   // staging for the term lists of batched calls
 };
 
 void hemm_set_error(const std::string &msg);
@@ -75,3 +76,13 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
                       const u64 *add_b, hipStream_t s);
 void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
                     int n_polys, hipStream_t s);
+void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
+                        hipStream_t s);
+void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
+                          hipStream_t s);
+void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
+                          u64 *conv, hipStream_t s);
+void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
+                       u64 *out, hipStream_t s);
+void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
+                         hipStream_t s);

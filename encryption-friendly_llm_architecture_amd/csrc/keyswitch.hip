@@ -115,6 +115,112 @@ __global__ __launch_bounds__(256) void spread_kernel(const u64 *__restrict__ las
 
 u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 
+// NTT-domain index of the automorphism X -> X^g: out[k] = in[galois_index(k)]
+__device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
+    const u32 br = __brev(k) >> (32 - logN);
+    const u32 e = ((2 * br + 1) * g) & ((2u << logN) - 1);
+    return __brev(e >> 1) >> (32 - logN);
+}
+
+struct RotTermDev {
+    const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
+    const u64 *b;     // [nq][N] b-polynomial of the source
+    const u64 *evk;   // [dnum][2][nQ+K][N]
+    const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
+    u32 galois, pad;
+};
+
+// Hoisted rotations, several per output, combined with masks in the extended basis:
+//   y[o][pol][j][n] = sum_{t in group o} mask_t[j][n] * ( sum_d ext_t[d][j][pi_t(n)] * evk_t[d][pol][j][n]
+//                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
+// The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
+// bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
+__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
+                                                            const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                            const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
+                                                            int nq, int E, int beta, int n_full, int logN) {
+    const int j = blockIdx.y, o = blockIdx.z;
+    const int prime = ll.idx[j];
+    const ModQ m = modq[prime];
+    const u32 n = blockIdx.x * 256 + threadIdx.x;
+    const size_t N = (size_t)1 << logN;
+    u64 acc_b = 0, acc_a = 0;
+    for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
+        const RotTermDev T = terms[t];
+        const u32 np = galois_index(n, T.galois, logN);
+        u128_t sb = {0, 0}, sa = {0, 0};
+        for (int d = 0; d < beta; d++) {
+            const u64 x = T.ext[((size_t)d * E + j) * N + np];
+            const u64 kb = T.evk[(((size_t)d * 2 + 0) * n_full + prime) * N + n];
+            const u64 ka = T.evk[(((size_t)d * 2 + 1) * n_full + prime) * N + n];
+            add128(sb, mul64wide(x, kb));
+            add128(sa, mul64wide(x, ka));
+        }
+        u64 rb = barrett128(sb, m), ra = barrett128(sa, m);
+        if (j < nq) rb = addmod(rb, mul_shoup(T.b[(size_t)j * N + np], pmod.c[j].w, pmod.c[j].ws, m.q), m.q);
+        if (T.mask != nullptr) {
+            const u64 mk = T.mask[(size_t)j * N + n];
+            rb = mulmod(rb, mk, m);
+            ra = mulmod(ra, mk, m);
+        }
+        acc_b = addmod(acc_b, rb, m.q);
+        acc_a = addmod(acc_a, ra, m.q);
+    }
+    y[(((size_t)o * 2 + 0) * E + j) * N + n] = acc_b;
+    y[(((size_t)o * 2 + 1) * E + j) * N + n] = acc_a;
+}
+
+struct LinTermDev {
+    const u64 *ct;    // [n_polys][.][N]
+    const u64 *mask;  // [nq][N] or nullptr (factor 1)
+    u64 stride;       // polynomial stride of ct
+};
+// out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j]
+__global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
+                                                         const u32 *__restrict__ group_off, u64 *__restrict__ out,
+                                                         const ModQ *__restrict__ modq, int nq, int n_polys, int logN) {
+    const int j = blockIdx.y % nq, p = blockIdx.y / nq, o = blockIdx.z;
+    const ModQ m = modq[j];
+    const size_t N = (size_t)1 << logN;
+    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
+    u64 acc = 0;
+    for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
+        const LinTermDev T = terms[t];
+        u64 x = T.ct[p * T.stride + (size_t)j * N + n];
+        if (T.mask != nullptr) x = mulmod(x, T.mask[(size_t)j * N + n], m);
+        acc = addmod(acc, x, m.q);
+    }
+    out[(((size_t)o * n_polys + p) * nq + j) * N + n] = acc;
+}
+
+// acc3 (+)= sum_{g < G} (b1 b2, a1 b2 + a2 b1, a1 a2) of t1[g], t2[g], each [2][nq][N]
+__global__ __launch_bounds__(256) void tensor_batch_kernel(const u64 *__restrict__ t1, const u64 *__restrict__ t2,
+                                                           int G, u64 *__restrict__ acc3, int accumulate,
+                                                           const ModQ *__restrict__ modq, int nq, int logN) {
+    const int j = blockIdx.y;
+    const ModQ m = modq[j];
+    const size_t N = (size_t)1 << logN, P = (size_t)nq * N;
+    const size_t e = (size_t)j * N + (size_t)blockIdx.x * 256 + threadIdx.x;
+    u64 d0 = 0, d1 = 0, d2 = 0;
+    if (accumulate) {
+        d0 = acc3[e];
+        d1 = acc3[P + e];
+        d2 = acc3[2 * P + e];
+    }
+    for (int g = 0; g < G; g++) {
+        const u64 b1 = t1[(size_t)g * 2 * P + e], a1 = t1[(size_t)g * 2 * P + P + e];
+        const u64 b2 = t2[(size_t)g * 2 * P + e], a2 = t2[(size_t)g * 2 * P + P + e];
+        d0 = addmod(d0, mulmod(b1, b2, m), m.q);
+        u128_t t = mul64wide(a1, b2);
+        add128(t, mul64wide(a2, b1));
+        d1 = addmod(d1, barrett128(t, m), m.q);
+        d2 = addmod(d2, mulmod(a1, a2, m), m.q);
+    }
+    acc3[e] = d0;
+    acc3[P + e] = d1;
+    acc3[2 * P + e] = d2;
+}
+
 }  // namespace
 
 // ---- tables -----------------------------------------------------------------------------------
@@ -127,6 +233,9 @@ struct KsTables {
     size_t p_inv_off = 0, p_hat_off = 0;
     std::vector<Cst> pinv;                               // P^-1 mod q_j
     std::vector<std::vector<Cst>> qlinv;                 // [l][j<l]  q_l^-1 mod q_j
+    // merged ModDown + rescale: basis {q_{nq-1}} U P dropped at once
+    std::vector<size_t> drop_inv_off, drop_hat_off;      // [nq]
+    std::vector<std::vector<Cst>> dropinv;               // [nq][j<nq-1]  (P q_{nq-1})^-1 mod q_j
 };
 
 static KsTables *g_tables_of(const hemm_context *c);
@@ -181,6 +290,22 @@ static void build_tables(const hemm_context *c, KsTables &t) {
             u64 q = c->primes[j];
             u64 inv = h_invmod(c->primes[l] % q, q);
             t.qlinv[l].push_back(Cst{inv, shoup_h(inv, q)});
+        }
+    t.drop_inv_off.assign(nQ + 1, 0);
+    t.drop_hat_off.assign(nQ + 1, 0);
+    t.dropinv.assign(nQ + 1, {});
+    if (K > 0)
+        for (int nq = 2; nq <= nQ; nq++) {
+            std::vector<int> src;
+            src.push_back(nq - 1);
+            for (int k = 0; k < K; k++) src.push_back(nQ + k);
+            push_basis(src, t.drop_inv_off[nq], t.drop_hat_off[nq]);
+            for (int j = 0; j < nq - 1; j++) {
+                u64 q = c->primes[j], prod = c->primes[nq - 1] % q;
+                for (int k = 0; k < K; k++) prod = h_mulmod(prod, c->primes[nQ + k] % q, q);
+                u64 inv = h_invmod(prod, q);
+                t.dropinv[nq].push_back(Cst{inv, shoup_h(inv, q)});
+            }
         }
     HEMM_HIP(hipMalloc((void **)&t.dev, t.host.size() * sizeof(Cst)));
     HEMM_HIP(hipMemcpy(t.dev, t.host.data(), t.host.size() * sizeof(Cst), hipMemcpyHostToDevice));
@@ -365,4 +490,141 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
     for (int j = 0; j < nq - 1; j++) cl.c[j] = t->qlinv[nq - 1][j];
     hipLaunchKernelGGL(sub_scale_kernel, grid, block, 0, s, in, in_stride, tt, (size_t)(nq - 1) * N,
                        (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq - 1, c->logN);
+}
+
+// ---- batched / hoisted forms ---------------------------------------------------------------------
+// in: [n_in][.][N] (polynomial stride in_stride, first nq limbs used) -> ext [n_in][beta][nq+K][N], own
+// limbs of every digit filled.  coef: workspace [n_in][nq][N].
+void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
+                        hipStream_t s) {
+    KsTables *t = g_tables_of(c);
+    const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
+    const size_t N = c->N;
+    HEMM_HIP(hipMemcpy2DAsync(coef, (size_t)nq * N * 8, in, in_stride * 8, (size_t)nq * N * 8, n_in,
+                              hipMemcpyDeviceToDevice, s));
+    launch_ntt(c, coef, limbs_default(c, nq, 0), nq, n_in, (size_t)nq * N, true, s);
+    for (int d = 0; d < beta; d++) {
+        const int lo = d * alpha, hi = std::min(nq, lo + alpha);
+        BConvArgs a;
+        memset(&a, 0, sizeof(a));
+        a.src = coef;
+        a.src_poly_stride = (size_t)nq * N;
+        a.dst = ext + (size_t)d * E * N;
+        a.dst_poly_stride = (size_t)beta * E * N;
+        a.inv = t->dev + t->inv_off[nq][d];
+        a.hat = t->dev + t->hat_off[nq][d];
+        a.n_src = hi - lo;
+        a.hat_ld = c->nQ + c->nP;
+        a.logN = c->logN;
+        if (a.n_src > 32) throw std::invalid_argument("digit wider than 32 limbs");
+        LimbList pl, sl;
+        memset(&pl, 0, sizeof(pl));
+        memset(&sl, 0, sizeof(sl));
+        for (int i = 0; i < a.n_src; i++) {
+            a.src_slot[i] = (uint8_t)(lo + i);
+            a.src_prime[i] = (uint8_t)(lo + i);
+        }
+        int nd = 0;
+        for (int j = 0; j < E; j++) {
+            if (j >= lo && j < hi) continue;
+            a.dst_slot[nd] = (uint8_t)j;
+            a.dst_prime[nd] = (uint8_t)(j < nq ? j : c->nQ + (j - nq));
+            pl.idx[nd] = a.dst_prime[nd];
+            sl.idx[nd] = (uint8_t)j;
+            nd++;
+        }
+        a.n_dst = nd;
+        if (nd > 0) {
+            dim3 grid(N / 256, n_in), block(256);
+            hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)a.n_src * 256 * 8, s, a, c->d_modq);
+            launch_ntt_slots(c, a.dst, pl, sl, nd, n_in, (size_t)beta * E * N, false, s);
+        }
+        HEMM_HIP(hipMemcpy2DAsync(a.dst + (size_t)lo * N, (size_t)beta * E * N * 8, in + (size_t)lo * N, in_stride * 8,
+                                  (size_t)(hi - lo) * N * 8, n_in, hipMemcpyDeviceToDevice, s));
+    }
+}
+
+// terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]
+void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
+                          hipStream_t s) {
+    const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+    CstList pm;
+    memset(&pm, 0, sizeof(pm));
+    for (int j = 0; j < nq; j++) {
+        u64 q = c->primes[j], P = 1;
+        for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
+        pm.c[j] = Cst{P, shoup_h(P, q)};
+    }
+    dim3 grid(c->N / 256, E, n_out), block(256);
+    hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
+                       c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN);
+}
+
+// y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;
+// drop_last = 1: out[p] = y[p] / (P q_{nq-1}) over nq-1 limbs (ModDown and rescale in one conversion).
+// conv: workspace [n_polys][nq_out][N].
+void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
+                          u64 *conv, hipStream_t s) {
+    KsTables *t = g_tables_of(c);
+    const int K = c->nP, E = nq + K, nq_out = drop_last ? nq - 1 : nq;
+    const size_t N = c->N;
+    if (drop_last && nq < 2) throw std::invalid_argument("merged rescale needs at least two limbs");
+    BConvArgs a;
+    memset(&a, 0, sizeof(a));
+    LimbList pl, sl;
+    memset(&pl, 0, sizeof(pl));
+    memset(&sl, 0, sizeof(sl));
+    int ns = 0;
+    if (drop_last) {
+        a.src_slot[ns] = (uint8_t)(nq - 1);
+        a.src_prime[ns] = (uint8_t)(nq - 1);
+        ns++;
+    }
+    for (int k = 0; k < K; k++) {
+        a.src_slot[ns] = (uint8_t)(nq + k);
+        a.src_prime[ns] = (uint8_t)(c->nQ + k);
+        ns++;
+    }
+    if (ns > 32) throw std::invalid_argument("more than 32 limbs dropped");
+    for (int i = 0; i < ns; i++) {
+        pl.idx[i] = a.src_prime[i];
+        sl.idx[i] = a.src_slot[i];
+    }
+    launch_ntt_slots(c, y, pl, sl, ns, n_polys, (size_t)E * N, true, s);
+    a.src = y;
+    a.src_poly_stride = (size_t)E * N;
+    a.dst = conv;
+    a.dst_poly_stride = (size_t)nq_out * N;
+    a.inv = t->dev + (drop_last ? t->drop_inv_off[nq] : t->p_inv_off);
+    a.hat = t->dev + (drop_last ? t->drop_hat_off[nq] : t->p_hat_off);
+    a.n_src = ns;
+    a.n_dst = nq_out;
+    a.hat_ld = c->nQ + c->nP;
+    a.logN = c->logN;
+    for (int j = 0; j < nq_out; j++) {
+        a.dst_slot[j] = (uint8_t)j;
+        a.dst_prime[j] = (uint8_t)j;
+    }
+    dim3 grid(N / 256, n_polys), block(256);
+    hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)ns * 256 * 8, s, a, c->d_modq);
+    launch_ntt(c, conv, limbs_default(c, nq_out, 0), nq_out, n_polys, (size_t)nq_out * N, false, s);
+    CstList cl;
+    for (int j = 0; j < nq_out; j++) cl.c[j] = drop_last ? t->dropinv[nq][j] : t->pinv[j];
+    dim3 g2(N / 256, nq_out * n_polys);
+    hipLaunchKernelGGL(sub_scale_kernel, g2, block, 0, s, y, (size_t)E * N, conv, (size_t)nq_out * N,
+                       (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq_out, c->logN);
+}
+
+void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
+                       u64 *out, hipStream_t s) {
+    dim3 grid(c->N / 256, nq * n_polys, n_out), block(256);
+    hipLaunchKernelGGL(masked_sum_kernel, grid, block, 0, s, (const LinTermDev *)terms_dev, group_off_dev, out,
+                       c->d_modq, nq, n_polys, c->logN);
+}
+
+void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
+                         hipStream_t s) {
+    dim3 grid(c->N / 256, nq), block(256);
+    hipLaunchKernelGGL(tensor_batch_kernel, grid, block, 0, s, t1, t2, G, acc3, accumulate ? 1 : 0, c->d_modq, nq,
+                       c->logN);
 }

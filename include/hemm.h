@@ -101,6 +101,45 @@ int hemm_rotate(hemm_context *ctx, const uint64_t *ct, size_t ct_stride, const u
 /* HomEvaluator::relinearize :524: (d0, d1, d2) -> (d0 + ks_b(d2), d1 + ks_a(d2)) */
 int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, const uint64_t *evk,
                      uint32_t nq, uint64_t *out, size_t out_stride, void *stream);
+/* ---- batched / hoisted forms: what one GPU-sized launch does where the reference issues one
+ * evaluator call per rotation.  They have no single counterpart in HomEvaluator; each replaces a
+ * run of leftRotate / multWithoutRescale / add / rescale calls of the matmul loops
+ * (MatrixUtils.cpp:800-845, 1413-1433). ---- */
+/* ModUp of n_in polynomials at once: in [n_in][.][N] (stride in_stride, nq limbs used) ->
+ * ext [n_in][beta][nq+n_p][N]; workspace >= n_in*nq*N words. */
+int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint32_t nq, uint32_t n_in,
+                     uint64_t *ext, uint64_t *workspace, void *stream);
+/* One hoisted rotation term: automorphism `galois` applied to an already extended source (ext, b),
+ * inner product with evk, optional plaintext mask over the extended basis (NULL = 1). */
+typedef struct {
+    const uint64_t *ext;  /* [beta][nq+n_p][N] */
+    const uint64_t *b;    /* [nq][N] */
+    const uint64_t *evk;  /* [dnum][2][n_q+n_p][N] */
+    const uint64_t *mask; /* [nq+n_p][N] or NULL */
+    uint64_t galois;
+} hemm_rot_term;
+/* y[o] = sum over terms[group_offsets[o] .. group_offsets[o+1]) of
+ *        mask * ( <galois(ext), evk> + P * galois(b) )      in the extended basis, y: [n_out][2][nq+n_p][N].
+ * terms / group_offsets are host arrays. */
+int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
+                       uint32_t n_out, uint32_t nq, uint64_t *y, void *stream);
+/* y [n_polys][nq+n_p][N] (clobbered) -> out [n_polys][nq - drop_last][N]: division by P (drop_last = 0)
+ * or by P*q_{nq-1} (drop_last = 1, ModDown and rescale in one basis conversion);
+ * workspace >= n_polys*(nq-drop_last)*N words. */
+int hemm_moddown_batch(hemm_context *ctx, uint64_t *y, uint32_t nq, uint32_t n_polys, int drop_last,
+                       uint64_t *out, size_t out_stride, uint64_t *workspace, void *stream);
+typedef struct {
+    const uint64_t *ct;   /* [n_polys][.][N] */
+    const uint64_t *mask; /* [nq][N] or NULL */
+    uint64_t stride;      /* polynomial stride of ct in words */
+} hemm_lin_term;
+/* out[o][p] = sum over the terms of group o of mask * ct[p]; out: [n_out][n_polys][nq][N] */
+int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const uint32_t *group_offsets,
+                          uint32_t n_out, uint32_t nq, uint32_t n_polys, uint64_t *out, void *stream);
+/* acc3 [3][nq][N] (+)= sum_g tensor(t1[g], t2[g]); t1, t2: [n_pairs][2][nq][N] */
+int hemm_tensor_batch(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
+                      uint64_t *acc3, int accumulate, void *stream);
+
 /* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last */
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
                  size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);

@@ -533,6 +533,80 @@ void orc_tensor(void *h, const u64 *ct1, const u64 *ct2, int nq, u64 *out) {
     }
 }
 
+// ---- hoisted rotation term: y (+)= mask * ( <galois(ext), evk> + P * galois(b) ) -----------------
+// ext [beta][nq+K][N] (ModUp output), b [nq][N], evk [dnum][2][nQ+nP][N], mask [nq+K][N] or null,
+// y [2][nq+K][N].  The automorphism acts on the NTT-form limbs as the index map of
+// orc_automorphism_ntt.
+void orc_hoisted_term(void *h, const u64 *ext, const u64 *b, const u64 *evk, const u64 *mask, u64 g, int nq,
+                      u64 *y, int accumulate) {
+    Ctx *c = (Ctx *)h;
+    const int N = c->N, K = c->nP, E = nq + K, full = c->nQ + c->nP;
+    const int beta = (nq + c->alpha - 1) / c->alpha;
+    const u64 M = 2 * (u64)N;
+    std::vector<int> perm(N);
+    for (int k = 0; k < N; k++) {
+        u64 e = (2 * (u64)bitrev((unsigned)k, c->logN) + 1) * g % M;
+        perm[k] = (int)bitrev((unsigned)((e - 1) / 2), c->logN);
+    }
+    for (int j = 0; j < E; j++) {
+        const int pi = prime_of(c, j, nq);
+        const u64 q = c->pr[pi].q;
+        u64 P = 1;
+        for (int k = 0; k < K; k++) P = mulmod(P, c->pr[c->nQ + k].q % q, q);
+        for (int pol = 0; pol < 2; pol++) {
+            u64 *o = y + ((size_t)pol * E + j) * N;
+            for (int n = 0; n < N; n++) {
+                u64 s = 0;
+                for (int d = 0; d < beta; d++)
+                    s = addmod(s, mulmod(ext[((size_t)d * E + j) * N + perm[n]],
+                                         evk[(((size_t)d * 2 + pol) * full + pi) * N + n], q), q);
+                if (pol == 0 && j < nq) s = addmod(s, mulmod(b[(size_t)j * N + perm[n]], P, q), q);
+                if (mask) s = mulmod(s, mask[(size_t)j * N + n], q);
+                o[n] = accumulate ? addmod(o[n], s, q) : s;
+            }
+        }
+    }
+}
+
+// Division of an extended polynomial y [nq+K][N] (NTT) by P (drop_last = 0, result over nq limbs) or by
+// P * q_{nq-1} (drop_last = 1, result over nq-1 limbs): out_j = (y_j - BConv_{D->q_j}(y_D)) * D^{-1}.
+void orc_moddown_drop(void *h, const u64 *y, int nq, int drop_last, u64 *out) {
+    Ctx *c = (Ctx *)h;
+    const int N = c->N, K = c->nP, nq_out = drop_last ? nq - 1 : nq;
+    std::vector<int> src, slot, dst;
+    if (drop_last) {
+        src.push_back(nq - 1);
+        slot.push_back(nq - 1);
+    }
+    for (int k = 0; k < K; k++) {
+        src.push_back(c->nQ + k);
+        slot.push_back(nq + k);
+    }
+    std::vector<u64> dc(src.size() * (size_t)N);
+    std::vector<const u64 *> ip;
+    std::vector<u64 *> op;
+    for (size_t i = 0; i < src.size(); i++) {
+        memcpy(dc.data() + i * N, y + (size_t)slot[i] * N, sizeof(u64) * N);
+        ntt_inv(c->pr[src[i]], dc.data() + i * N, N);
+        ip.push_back(dc.data() + i * N);
+    }
+    for (int j = 0; j < nq_out; j++) {
+        dst.push_back(j);
+        op.push_back(out + (size_t)j * N);
+    }
+    BConv bc = make_bconv(c, src, dst);
+    run_bconv(c, bc, ip.data(), op.data());
+    for (int j = 0; j < nq_out; j++) {
+        const u64 q = c->pr[j].q;
+        ntt_fwd(c->pr[j], op[j], N);
+        u64 D = 1;
+        for (int s : src) D = mulmod(D, c->pr[s].q % q, q);
+        const u64 dinv = invmod(D, q);
+        const u64 *a = y + (size_t)j * N;
+        for (int n = 0; n < N; n++) op[j][n] = mulmod(submod(a[n], op[j][n], q), dinv, q);
+    }
+}
+
 // ---- encode / decode ---------------------------------------------------------------------
 // slots: n = N/2 complex values (re, im interleaved).  Produces signed integer coefficients
 // round(scale * coeff) as int64 (caller reduces per prime with orc_lift_i64).

@@ -70,6 +70,9 @@ def lib():
         L.orc_moddown.argtypes = [ctypes.c_void_p, u64p, ctypes.c_int, u64p]
         L.orc_keyswitch.argtypes = [ctypes.c_void_p, u64p, u64p, ctypes.c_int, u64p, u64p]
         L.orc_rescale.argtypes = [ctypes.c_void_p, u64p, ctypes.c_int, u64p]
+        L.orc_hoisted_term.argtypes = [ctypes.c_void_p, u64p, u64p, u64p, u64p, ctypes.c_uint64,
+                                       ctypes.c_int, u64p, ctypes.c_int]
+        L.orc_moddown_drop.argtypes = [ctypes.c_void_p, u64p, ctypes.c_int, ctypes.c_int, u64p]
         L.orc_tensor.argtypes = [ctypes.c_void_p, u64p, u64p, ctypes.c_int, u64p]
         L.orc_encode_coeffs.argtypes = [ctypes.c_void_p, f64p, ctypes.c_double, i64p]
         L.orc_decode_coeffs.argtypes = [ctypes.c_void_p, f64p, f64p]
@@ -547,3 +550,60 @@ class Oracle:
 
     def level_down_one(self, x):
         return self.level_down(x, x.level - 1)
+
+    # ---- hoisted / merged forms (what the batched GPU launches compute) -------------------------
+    def encode_ext(self, msg, level):
+        """Plaintext over the extended basis: limbs q_0..q_level then the special primes."""
+        z = np.zeros(self.slots, dtype=np.complex128)
+        m = np.asarray(msg)
+        z[: m.size] = m.reshape(-1)
+        sl = np.ascontiguousarray(z.view(np.float64))
+        co = np.empty(self.N, dtype=np.int64)
+        scale = self.delta[level]
+        self.L.orc_encode_coeffs(self.h, _p(sl, f64p), float(scale), _p(co, i64p))
+        primes = list(range(level + 1)) + [self.nQ + k for k in range(self.nP)]
+        out = np.empty((len(primes), self.N), dtype=np.uint64)
+        for j, pi in enumerate(primes):
+            self.L.orc_lift_i64(self.h, _p(co, i64p), pi, _p(out[j]))
+        self.ntt(out, primes)
+        return Pt(out, float(scale))
+
+    def modup(self, poly):
+        nq = poly.shape[0]
+        beta = (nq + self.alpha - 1) // self.alpha
+        ext = np.empty((beta, nq + self.nP, self.N), dtype=np.uint64)
+        self.L.orc_modup(self.h, _p(np.ascontiguousarray(poly)), nq, _p(ext))
+        return ext
+
+    def galois_key(self, g):
+        if ("gal", g) not in self.keys and getattr(self, "key_seed", None) is not None:
+            self.keys[("gal", g)] = self._gen_switch_key(self.key_seed, g, self._sk_automorphism(g))
+        return self.keys[("gal", g)]
+
+    def hoisted_sum(self, terms, nq):
+        """terms: (ext, b, rotation r (left, in slots) or ('g', galois), mask Pt over the extended basis
+        or None).  Returns y[2][nq+K][N] = sum mask * (<galois(ext), evk> + P galois(b))."""
+        y = np.zeros((2, nq + self.nP, self.N), dtype=np.uint64)
+        for i, (ext, b, rot, mask) in enumerate(terms):
+            g = rot[1] if isinstance(rot, tuple) else self.galois(rot)
+            evk = self.galois_key(g)
+            mk = _p(np.ascontiguousarray(mask.data)) if mask is not None else None
+            self.L.orc_hoisted_term(self.h, _p(np.ascontiguousarray(ext)), _p(np.ascontiguousarray(b)),
+                                    _p(evk), mk, g, nq, _p(y), int(i > 0))
+        return y
+
+    def moddown_drop(self, y, nq, drop_last):
+        nq_out = nq - 1 if drop_last else nq
+        out = np.empty((y.shape[0], nq_out, self.N), dtype=np.uint64)
+        for p in range(y.shape[0]):
+            self.L.orc_moddown_drop(self.h, _p(np.ascontiguousarray(y[p])), nq, int(drop_last), _p(out[p]))
+        return out
+
+    def rotate_hoisted(self, x, r):
+        """Rotation with the automorphism applied after ModUp (the order the batched launches use)."""
+        r %= self.slots
+        if r == 0:
+            return x.copy()
+        ext = self.modup(x.data[1])
+        y = self.hoisted_sum([(ext, x.data[0], r, None)], x.nq)
+        return Ct(self.moddown_drop(y, x.nq, False), x.scale)

@@ -171,3 +171,62 @@ def test_rotate_relinearize_rescale(S):
     assert np.abs(orc.decrypt(O.Ct(host(drs), rs.scale)) - z * z).max() < 1e-6
     # 3-polynomial rescale (used on un-relinearised sums)
     assert np.array_equal(host(ctx.rescale(d3, nq)), orc.rescale(t3).data)
+
+
+def test_batched_hoisted_forms(S):
+    """ModUp of several polynomials, hoisted masked rotation terms, merged ModDown + rescale, masked
+    sums and batched tensor accumulation against the oracle's one-at-a-time forms."""
+    import torch
+    orc, ctx, N = S.orc, S.ctx, S.N
+    rng = S.rng
+    nq = orc.nQ - 1
+    orc.key_seed = 6
+    E = nq + orc.nP
+    mods = orc.q[:nq]
+    cts = [rand_limbs(rng, mods, (2,), N) for _ in range(3)]
+    dcts = [dev(c) for c in cts]
+    # batched ModUp of the three a-polynomials == three single ModUps
+    a_stack = torch.stack([d[1] for d in dcts]).contiguous()
+    dext = ctx.modup_batch(a_stack, nq)
+    exts = [orc.modup(c[1]) for c in cts]
+    for k in range(3):
+        assert np.array_equal(host(dext[k]), exts[k])
+    # hoisted terms: group 0 = two masked rotations of ct0, group 1 = one unmasked rotation of ct1,
+    # group 2 = conjugation of ct2
+    z1 = rng.uniform(-1, 1, orc.slots)
+    z2 = rng.uniform(-1, 1, orc.slots)
+    m1, m2 = orc.encode_ext(z1, nq - 1), orc.encode_ext(z2, nq - 1)
+    g1, g2, g3, gc = orc.galois(1), orc.galois(orc.slots - 5), orc.galois(16), 2 * N - 1
+    dk = {g: dev(orc.galois_key(g)) for g in (g1, g2, g3, gc)}
+    dm1, dm2 = dev(m1.data), dev(m2.data)
+    groups = [[(dext[0], dcts[0][0], dk[g1], dm1, g1), (dext[0], dcts[0][0], dk[g2], dm2, g2)],
+              [(dext[1], dcts[1][0], dk[g3], None, g3)],
+              [(dext[2], dcts[2][0], dk[gc], None, gc)]]
+    y = ctx.hoisted_terms(groups, nq)
+    want = [orc.hoisted_sum([(exts[0], cts[0][0], ("g", g1), m1), (exts[0], cts[0][0], ("g", g2), m2)], nq),
+            orc.hoisted_sum([(exts[1], cts[1][0], ("g", g3), None)], nq),
+            orc.hoisted_sum([(exts[2], cts[2][0], ("g", gc), None)], nq)]
+    for k in range(3):
+        assert np.array_equal(host(y[k]), want[k])
+    # plain ModDown and ModDown merged with the rescale, batched over all outputs
+    for drop in (False, True):
+        got = host(ctx.moddown_batch(y.clone(), nq, drop))
+        for k in range(3):
+            assert np.array_equal(got[k], orc.moddown_drop(want[k], nq, drop))
+    # masked sums: out0 = m*ct0 + ct1, out1 = m'*ct2
+    p1, p2 = orc.encode(z1, nq - 1), orc.encode(z2, nq - 1)
+    dp1, dp2 = dev(p1.data), dev(p2.data)
+    ms = host(ctx.masked_sum_batch([[(dcts[0], dp1), (dcts[1], None)], [(dcts[2], dp2)]], nq, 2))
+    w0 = orc.add(orc.mult_plain_no_rescale(O.Ct(cts[0], 1.0), p1), O.Ct(cts[1], 1.0)).data
+    w1 = orc.mult_plain_no_rescale(O.Ct(cts[2], 1.0), p2).data
+    assert np.array_equal(ms[0], w0) and np.array_equal(ms[1], w1)
+    # batched tensor accumulation
+    t1 = torch.stack(dcts).contiguous()
+    t2 = torch.stack(dcts[::-1]).contiguous()
+    acc = ctx.tensor_batch(t1, t2, nq)
+    ctx.tensor_batch(t1[:1].contiguous(), t1[:1].contiguous(), nq, acc=acc)
+    want3 = None
+    for a, b in list(zip(cts, cts[::-1])) + [(cts[0], cts[0])]:
+        t = orc.tensor(O.Ct(a, 1.0), O.Ct(b, 1.0))
+        want3 = t if want3 is None else orc.add(want3, t)
+    assert np.array_equal(host(acc), want3.data)
