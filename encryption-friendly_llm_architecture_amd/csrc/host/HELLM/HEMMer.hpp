@@ -99,6 +99,14 @@ public:
     CtxtTensor matMulPreRev(const CtxtTensor &b, u64 target_level = 4) const;
     CtxtTensor matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 target_level = 4) const;
 
+    // Schedule of singleCCMatMul / packedMatMul / matMulPre: batched launches with hoisted rotations
+    // (default) or one evaluator call per step in the reference's order.  `batch` = shifts per launch.
+    void setFused(bool on, u64 batch = 16) {
+        fused_ = on;
+        batch_ = batch;
+    }
+    bool fused() const { return fused_; }
+
     // generate (once) the direct rotation keys a routine needs; rotations are left shifts in slots
     void ensureRotationKeys(const std::vector<u64> &left_rotations) const;
     size_t rotationKeyCount() const { return have_rot_.size(); }
@@ -122,6 +130,8 @@ private:
     Message col_mask_even_, row_mask_even_, mask_left_half_, mask_matmul_;
     mutable std::map<std::pair<int, u64>, Plaintext> mask_cache_;
     mutable std::set<u64> have_rot_;
+    bool fused_ = true;
+    u64 batch_ = 16;
 };
 
 }  // namespace HELLM

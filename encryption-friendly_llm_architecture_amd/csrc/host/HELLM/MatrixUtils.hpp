@@ -48,6 +48,15 @@ public:
     CtxtTensor packedDiagonalToColumn(const HomEvaluator &eval, const CtxtTensor &op);
     CtxtTensor packedDiagonalToRow(const HomEvaluator &eval, const CtxtTensor &op);
 
+    // The same transforms and assemble masks for the batched launches: masks over the extended basis
+    // (chain limbs + special primes) so they can be applied before ModDown.
+    std::vector<Plaintext> &getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
+    std::vector<Plaintext> &getRowMaskExt(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
+    // sigma / tau / packed variants with hoisted baby steps (one ModUp, all baby rotations in one launch
+    // chain) and all giant-step rotations batched and summed in the extended basis
+    Ciphertext diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                      const TileTensorShape &shape);
+
     void cleanUp();
     size_t cachedMasks() const;
 
@@ -65,6 +74,7 @@ private:
                                  const TileTensorShape &shape);
     std::map<Key, Plaintext> masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
+    std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_;
 };
 
 // A x B for two encrypted tiles (HEMMer::singleCCMatMul); output level = target_level.
@@ -91,5 +101,19 @@ CtxtTensor multMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b, u64 t
                             MatrixTransformer &transformer);
 CtxtTensor multMatMatCCReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
                              u64 target_level, MatrixTransformer &transformer);
+
+// Batched schedules of the same products (same decrypted results, far fewer and larger launches):
+// every column / row shift of the main loop is a direct hoisted rotation of sigma(A) / tau(B) (one ModUp
+// per operand), the two masked halves of a shift are combined before one merged ModDown + rescale, and
+// `batch` shifts are processed per launch.
+CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                           const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16);
+CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                                 const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer,
+                                 u64 batch = 16);
+void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
+                        MatrixTransformer &transformer, u64 batch = 16);
+// left rotations (in slots) whose direct keys the batched schedules use
+std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 
 }  // namespace HELLM

@@ -221,6 +221,9 @@ public:
     Plaintext encode(const Message &msg, u64 level, u64 rescale_counter = 0) const;
     Plaintext encode(const Message &msg) const;
     Message decode(const Plaintext &pt) const;
+    // plaintext over the extended basis (limbs q_0..q_level then the special primes), for masks that
+    // are applied before ModDown
+    Plaintext encodeExtended(const Message &msg, u64 level) const;
 
 private:
     Context ctx_;
@@ -250,6 +253,7 @@ class HomEvaluator {
 public:
     HomEvaluator(const Context &c, const KeyPack &pack) : ctx_(c), pack_(pack) {}
     const Context &getContext() const { return ctx_; }
+    const KeyPack &getKeyPack() const { return pack_; }
 
     void negate(const Ciphertext &a, Ciphertext &out) const;
     void add(const Ciphertext &a, const Ciphertext &b, Ciphertext &out) const;

@@ -550,8 +550,7 @@ void bitrev_perm(std::vector<double> &re, std::vector<double> &im) {
 }
 }  // namespace
 
-Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) const {
-    const Context &c = ctx_;
+static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u64 rescale_counter, bool extended) {
     if (level >= c->nQ) throw RuntimeException("encode: level above the encryption level");
     if (rescale_counter != 0) throw RuntimeException("encode: only rescale counter 0 is supported");
     const size_t n = c->N / 2, M = 2 * c->N;
@@ -585,8 +584,19 @@ Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) 
     }
     Plaintext pt(c);
     pt.allocate(level, 0);
-    lift_and_ntt(c, coeffs, chain_primes(level + 1), pt.buf_.data());
+    std::vector<uint32_t> primes = chain_primes(level + 1);
+    if (extended) {
+        for (u64 k = 0; k < c->nP; k++) primes.push_back((uint32_t)(c->nQ + k));
+        pt.buf_.resize(c, primes.size() * c->N);
+    }
+    lift_and_ntt(c, coeffs, primes, pt.buf_.data());
     return pt;
+}
+Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) const {
+    return encode_impl(ctx_, msg, level, rescale_counter, false);
+}
+Plaintext EnDecoder::encodeExtended(const Message &msg, u64 level) const {
+    return encode_impl(ctx_, msg, level, 0, true);
 }
 Plaintext EnDecoder::encode(const Message &msg) const { return encode(msg, getEncryptionLevel(ctx_)); }
 

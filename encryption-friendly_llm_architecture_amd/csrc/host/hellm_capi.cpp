@@ -110,6 +110,12 @@ int hellm_ensure_rotation_keys(hellm_hemmer *h, const uint64_t *rots, uint32_t c
     h->m->ensureRotationKeys(std::vector<u64>(rots, rots + count));
     FACADE_CATCH
 }
+int hellm_set_schedule(hellm_hemmer *h, int fused, uint32_t batch) {
+    FACADE_TRY
+    need(h && batch >= 1, "bad argument");
+    h->m->setFused(fused != 0, batch);
+    FACADE_CATCH
+}
 int hellm_sync(void) {
     FACADE_TRY
     CudaTools::cudaDeviceSynchronize();

@@ -272,6 +272,10 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
+    if (fused_) {
+        ensureRotationKeys(fusedRotations(TileTensorShape(n, n, w), log_slots_, false, true));
+        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
+    }
     ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});
     return multMatMat(eval_, btp_, a, b, T, matrix_transformer);
 }
@@ -287,6 +291,10 @@ CtxtTensor HEMMer::packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T)
     const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
     ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
+    if (fused_ && (u64)(n * w) == slots) {
+        ensureRotationKeys(fusedRotations(TileTensorShape(n, n, w), log_slots_, true, true));
+        return multPackedMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
+    }
     ensureRotationKeys({2, (u64)(2 * w), slots - (u64)n});
     return multPackedMatMat(eval_, btp_, a, b, T, matrix_transformer);
 }
@@ -310,6 +318,11 @@ CtxtTensor HEMMer::packedMatMulCCReuse(const std::vector<Ciphertext> &tmp, const
 void HEMMer::matMulPre(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 T) const {
     const u64 slots = u64(1) << log_slots_;
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getBlockWidth()));
+    if (fused_) {
+        ensureRotationKeys(fusedRotations(a.getShape(), log_slots_, false, false));
+        multMatMatPreFused(eval_, a, tmp, T, matrix_transformer, batch_);
+        return;
+    }
     ensureRotationKeys({1, slots - (u64)a.getHeight()});
     multMatMatPre(eval_, a, tmp, T, matrix_transformer);
 }
