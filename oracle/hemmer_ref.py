@@ -496,6 +496,113 @@ def mult_mat_mat_reuse(ev, tmp, b_pt, T):
     return ev.rescale(acc)
 
 
+# --------------------------------------------------------------------------------------------
+# batched schedule of the same products, over the oracle only (residue-level definition of what the
+# GPU's batched launches compute): rotations are applied after ModUp ("hoisted"), the two masked
+# halves of a shift are combined in the extended basis and ModDown is merged with the rescale.
+# --------------------------------------------------------------------------------------------
+def diagonal_transform_fused(orc, ct, kind, n, w):
+    from .oracle import Ct
+    units, _, bs, gs, step = geometry(kind, n, w)
+    level, nq = ct.level, ct.nq
+    enc = lambda idx: orc.encode(prerotated_mask(kind, n, w, orc.slots, idx), level)
+    ext = orc.modup(ct.data[1])
+    baby = [Ct(orc.moddown_drop(orc.hoisted_sum([(ext, ct.data[0], (j + 1) * step, None)], nq), nq, False),
+               ct.scale) for j in range(bs)]
+    groups, rots = [[(ct, 0)]], [0]
+
+    def push(terms, r):
+        if not terms:
+            return
+        if r % orc.slots == 0:
+            groups[0].extend(terms)
+        else:
+            groups.append(terms)
+            rots.append(r)
+
+    for i in range(gs):
+        neg = [(baby[j], 1 + i * bs + j - units) for j in range(bs) if 1 + i * bs + j - units < 0]
+        push(neg, -(units - i * bs) * step)
+        pos = [(baby[j], 1 + i * bs + j) for j in range(bs) if 1 + i * bs + j < units]
+        push(pos, i * bs * step)
+    sums = []
+    for terms in groups:
+        acc = None
+        for c, d in terms:
+            t = orc.mult_plain_no_rescale(c, enc(d))
+            acc = t if acc is None else orc.add(acc, t)
+        sums.append(acc)
+    res = sums[0]
+    if len(sums) > 1:
+        terms = [(orc.modup(s.data[1]), s.data[0], r % orc.slots, None) for s, r in zip(sums[1:], rots[1:])]
+        y = orc.hoisted_sum(terms, nq)
+        res = orc.add(Ct(orc.moddown_drop(y, nq, False), res.scale), res)
+    return orc.rescale(res)
+
+
+def _assemble_shifts(orc, src, ext, shifts):
+    """shifts: (rot1, mask1_ext, rot2, mask2_ext) -> ciphertexts one level down."""
+    from .oracle import Ct
+    nq = src.nq
+    out = []
+    for r1, m1, r2, m2 in shifts:
+        terms = [(ext, src.data[0], r1 % orc.slots, m1)]
+        if m2 is not None:
+            terms.append((ext, src.data[0], r2 % orc.slots, m2))
+        y = orc.hoisted_sum(terms, nq)
+        out.append(Ct(orc.moddown_drop(y, nq, True), orc.delta[src.level - 1]))
+    return out
+
+
+def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
+    ev = OracleEval(orc)
+    a = orc.level_down(a, T + 3)
+    b = orc.level_down(b, T + 3)
+    cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+    rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
+    a = diagonal_transform_fused(orc, a, H, n, w)
+    b = diagonal_transform_fused(orc, b, V, n, w)
+    res = ev.mult(a, b)
+    ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
+    ta = _assemble_shifts(orc, a, ext_a, [(i, cm[2 * i + 1], i - n, cm[2 * i]) for i in range(1, n)])
+    tb = _assemble_shifts(orc, b, ext_b, [(i * w, rm[2 * i + 1], (i - n) * w, rm[2 * i]) for i in range(1, n)])
+    acc = None
+    for x, y in zip(ta, tb):
+        t = orc.tensor(x, y)
+        acc = t if acc is None else orc.add(acc, t)
+    out = orc.rescale(orc.relinearize(acc))
+    return ev.add(res, out)
+
+
+def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
+    from .oracle import Ct
+    ev = OracleEval(orc)
+    cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+    a = orc.level_down(a, T + 3)
+    b = orc.level_down(b, T + 2)
+    a = diagonal_transform_fused(orc, a, PH, n, w)
+    b = diagonal_transform_fused(orc, b, PV, n, w)
+    res = ev.mult(a, b)
+    ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
+    ta = _assemble_shifts(orc, a, ext_a, [(2 * i, cm[4 * i + 1], 2 * i - n, cm[4 * i]) for i in range(1, n // 2)])
+    acc = None
+    for i, x in zip(range(1, n // 2), ta):
+        y = orc.hoisted_sum([(ext_b, b.data[0], (2 * i * w) % orc.slots, None)], b.nq)
+        t = orc.tensor(x, Ct(orc.moddown_drop(y, b.nq, False), b.scale))
+        acc = t if acc is None else orc.add(acc, t)
+    out = orc.rescale(orc.relinearize(acc))
+    return ev.add(res, out)
+
+
+def mult_mat_mat_pre_fused(orc, a, T, n, w):
+    cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+    a = orc.level_down(a, T + 3)
+    a = diagonal_transform_fused(orc, a, H, n, w)
+    ext = orc.modup(a.data[1])
+    return [orc.level_down_one(a)] + _assemble_shifts(
+        orc, a, ext, [(i, cm[2 * i + 1], i - n, cm[2 * i]) for i in range(1, n)])
+
+
 def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
     """HEMMer::msgDiagonalToRow4 (HEMMer.cpp:353-399)."""
     h, w = w1.shape

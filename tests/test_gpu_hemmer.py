@@ -99,20 +99,42 @@ def test_sigma_tau_bit_exact(small):
     assert np.array_equal(tr.residues(), R.transpose(ev, oa, 16, 16).data)
 
 
-def test_ccmm_residues_bit_exact_and_decrypts(small):
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_ccmm_residues_bit_exact_and_decrypts(small, fused):
+    """Both schedules of singleCCMatMul against the oracle running the same schedule."""
     H, orc, ev = small
     rng = np.random.default_rng(4)
     A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
     ca, cb = H.encrypt(A), H.encrypt(B)
-    c = H.single_cc_matmul(ca, cb, 2)
-    want = R.mult_mat_mat_cc(ev, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16)
+    H.set_schedule(fused, batch=4)
+    try:
+        c = H.single_cc_matmul(ca, cb, 2)
+    finally:
+        H.set_schedule(True)
+    oa, ob = to_oracle(orc, ca), to_oracle(orc, cb)
+    want = R.mult_mat_mat_cc_fused(orc, oa, ob, 2, 16, 16) if fused else R.mult_mat_mat_cc(ev, oa, ob, 2, 16, 16)
     assert c.info()["level"] == 2
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
 
 
-def test_pcmm_and_packed_bit_exact(small):
+def test_batch_size_does_not_change_residues(small):
+    H, _, _ = small
+    rng = np.random.default_rng(14)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    outs = []
+    for batch in (1, 5, 16):
+        H.set_schedule(True, batch=batch)
+        outs.append(H.single_cc_matmul(ca, cb, 2).residues())
+    H.set_schedule(True)
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_pcmm_and_packed_bit_exact(small, fused):
     H, orc, ev = small
+    H.set_schedule(fused, batch=3)
     rng = np.random.default_rng(5)
     A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
     ca = H.encrypt(A)
@@ -131,22 +153,27 @@ def test_pcmm_and_packed_bit_exact(small):
     ob = R.complex_packing_rows(ev, ob, 16, 32)
     assert np.array_equal(pa.residues(), oa.data) and np.array_equal(pbb.residues(), ob.data)
     pc = H.repack_cc(H.packed_matmul(pa, pbb, 2))
-    want = R.repack_cc(ev, R.mult_packed_mat_mat(ev, oa, ob, 2, 16, 32))
+    H.set_schedule(True)
+    prod = R.mult_packed_mat_mat_fused(orc, oa, ob, 2, 16, 32) if fused else R.mult_packed_mat_mat(ev, oa, ob, 2, 16, 32)
+    want = R.repack_cc(ev, prod)
     assert np.array_equal(pc.residues(), want.data)
     d = H.decrypt2(pc)
     assert np.abs(d[0] - A @ B).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
 
 
-def test_hoisted_products_bit_exact(small):
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_hoisted_products_bit_exact(small, fused):
     H, orc, ev = small
     n = 16
+    H.set_schedule(fused, batch=6)
     rng = np.random.default_rng(6)
     X0, X1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
     W = [rng.normal(0, 0.02, (n, n)) for _ in range(4)]
     x = H.complex_packing(H.encrypt2(X0, X0), H.encrypt2(X1, X1))
     ox = to_oracle(orc, x)
     tmp = H.matmul_pre(x, 2)
-    otmp = R.mult_mat_mat_pre(ev, ox, 2, n, 2 * n)
+    H.set_schedule(True)
+    otmp = R.mult_mat_mat_pre_fused(orc, ox, 2, n, 2 * n) if fused else R.mult_mat_mat_pre(ev, ox, 2, n, 2 * n)
     assert len(tmp) == n
     for k in (0, 1, n - 1):
         assert np.array_equal(tmp.get(k, n, n, 2 * n).residues(), otmp[k].data)
@@ -185,8 +212,10 @@ def pkg_error():
 
 
 # ---- full size -----------------------------------------------------------------------------------
-def test_full_ccmm_128(full):
+@pytest.mark.parametrize("fused", [True, False], ids=["batched", "reference-order"])
+def test_full_ccmm_128(full, fused):
     H = full
+    H.set_schedule(fused)
     rng = np.random.default_rng(1)
     A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
     ca, cb = H.encrypt(A), H.encrypt(B)
@@ -199,6 +228,7 @@ def test_full_ccmm_128(full):
     assert np.abs(z[128 * 128:]).max() < TOL           # upper half of the slots stays empty
     # linearity in the encrypted operand: (2A) B = 2 (A B)
     c2 = H.single_cc_matmul(H.add(ca, ca), cb, 4)
+    H.set_schedule(True)
     assert np.abs(H.decrypt(c2) - 2 * (A @ B)).max() < TOL
 
 
