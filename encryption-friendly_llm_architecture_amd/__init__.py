@@ -41,7 +41,7 @@ class RotTerm(ctypes.Structure):
 
 
 class LinTerm(ctypes.Structure):
-    _fields_ = [("ct", vp), ("mask", vp), ("stride", ctypes.c_uint64)]
+    _fields_ = [("ct", vp), ("mask", vp), ("stride", ctypes.c_uint64), ("galois", ctypes.c_uint64)]
 
 
 def _declare(L):
@@ -265,8 +265,10 @@ class Context:
         import torch
         flat = [t for g in groups for t in g]
         arr = (LinTerm * len(flat))()
-        for i, (ct, mask) in enumerate(flat):
-            arr[i] = LinTerm(ct.data_ptr(), mask.data_ptr() if mask is not None else None, ct.stride(0))
+        for i, term in enumerate(flat):
+            ct, mask = term[0], term[1]
+            gal = term[2] if len(term) > 2 else 0
+            arr[i] = LinTerm(ct.data_ptr(), mask.data_ptr() if mask is not None else None, ct.stride(0), gal)
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))

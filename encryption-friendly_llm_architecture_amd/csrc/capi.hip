@@ -329,7 +329,11 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
     chain_limbs(ctx, nq, 0, &nl);
     need(terms && group_offsets && out && n_out >= 1 && n_polys >= 1, "null operand");
     const uint32_t n_terms = group_offsets[n_out];
-    for (uint32_t t = 0; t < n_terms; t++) need(terms[t].ct != nullptr, "null pointer in a term");
+    for (uint32_t t = 0; t < n_terms; t++) {
+        need(terms[t].ct != nullptr, "null pointer in a term");
+        need(terms[t].galois == 0 || ((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N),
+             "galois element must be odd and < 2N");
+    }
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, terms, n_terms * sizeof(hemm_lin_term), group_offsets,
                                   (n_out + 1) * sizeof(uint32_t), &off_dev, (hipStream_t)stream);

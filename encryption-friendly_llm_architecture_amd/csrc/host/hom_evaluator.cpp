@@ -415,15 +415,20 @@ void HomEvaluator::matmul(const std::vector<Ciphertext> &cts, const Plaintext &p
     if (cts.empty()) throw RuntimeException("matmul: empty operand list");
     const u64 slots = ctx_->N / 2, step = slots / cts.size(), lvl = cts[0].level_;
     if (pt.level_ < lvl) throw RuntimeException("matmul: plaintext level below the ciphertext level");
+    // one launch: every term reads its ciphertext and the plaintext through that term's automorphism
     Ciphertext acc(ctx_);
     acc.allocate(2, lvl, 1);
-    Plaintext rot(ctx_);
+    std::vector<hemm_lin_term> terms(cts.size());
     for (size_t k = 0; k < cts.size(); k++) {
         if (cts[k].level_ != lvl || cts[k].rescale_counter_ != 0) throw RuntimeException("matmul: level mismatch");
-        leftRotate(pt, k * step, rot);
-        ck(hemm_pointwise(ctx_->dev, k == 0 ? HEMM_MUL : HEMM_MAC, cts[k].buf_.data(), cts[k].polyStride(),
-                          rot.buf_.data(), 0, acc.buf_.data(), acc.polyStride(), (uint32_t)lvl + 1, 0, 2, nullptr));
+        terms[k].ct = cts[k].buf_.data();
+        terms[k].mask = pt.buf_.data();
+        terms[k].stride = cts[k].polyStride();
+        const u64 r = (k * step) % slots;
+        terms[k].galois = r == 0 ? 0 : powmod(5, r, 2 * ctx_->N);
     }
+    const uint32_t off[2] = {0, (uint32_t)cts.size()};
+    ck(hemm_masked_sum_batch(ctx_->dev, terms.data(), off, 1, (uint32_t)lvl + 1, 2, acc.buf_.data(), nullptr));
     rescale(acc);
     out = std::move(acc);
 }

@@ -187,6 +187,7 @@ Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, c
         t.ct = ct;
         t.mask = transformMask(eval, kind, shape, level, d).buf_.data();
         t.stride = nq * N;
+        t.galois = 0;
         return t;
     };
     auto push_group = [&](std::vector<hemm_lin_term> &&g_terms, i64 r) {

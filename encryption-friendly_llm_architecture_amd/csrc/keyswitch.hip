@@ -139,10 +139,11 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
                                                             int nq, int E, int beta, int n_full, int logN) {
-    const int j = blockIdx.y, o = blockIdx.z;
+    // blockIdx.x = output (fastest): workgroups that gather from the same 2 KiB source run back to back
+    const int j = blockIdx.z, o = blockIdx.x;
     const int prime = ll.idx[j];
     const ModQ m = modq[prime];
-    const u32 n = blockIdx.x * 256 + threadIdx.x;
+    const u32 n = blockIdx.y * 256 + threadIdx.x;
     const size_t N = (size_t)1 << logN;
     u64 acc_b = 0, acc_a = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
@@ -174,23 +175,42 @@ struct LinTermDev {
     const u64 *ct;    // [n_polys][.][N]
     const u64 *mask;  // [nq][N] or nullptr (factor 1)
     u64 stride;       // polynomial stride of ct
+    u64 galois;       // 0: mask used as is; else the mask is read through the automorphism X -> X^galois
 };
-// out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j]
+// out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j], p < n_polys (<= 3).  A thread owns one
+// (limb, coefficient) for every polynomial, so each mask residue is read once; products are summed as
+// 128-bit values and reduced every 4 terms.
 __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
                                                          const u32 *__restrict__ group_off, u64 *__restrict__ out,
                                                          const ModQ *__restrict__ modq, int nq, int n_polys, int logN) {
-    const int j = blockIdx.y % nq, p = blockIdx.y / nq, o = blockIdx.z;
+    const int j = blockIdx.y, o = blockIdx.z;
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN;
-    const size_t n = (size_t)blockIdx.x * 256 + threadIdx.x;
-    u64 acc = 0;
+    const size_t e = (size_t)j * N + (size_t)blockIdx.x * 256 + threadIdx.x;
+    u64 acc[3] = {0, 0, 0};
+    u128_t lazy[3] = {{0, 0}, {0, 0}, {0, 0}};
+    int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const LinTermDev T = terms[t];
-        u64 x = T.ct[p * T.stride + (size_t)j * N + n];
-        if (T.mask != nullptr) x = mulmod(x, T.mask[(size_t)j * N + n], m);
-        acc = addmod(acc, x, m.q);
+        if (T.mask != nullptr) {
+            const u64 mk = T.galois ? T.mask[(size_t)j * N + galois_index((u32)(e - (size_t)j * N), (u32)T.galois, logN)]
+                                    : T.mask[e];
+            for (int p = 0; p < n_polys; p++) add128(lazy[p], mul64wide(T.ct[p * T.stride + e], mk));
+            if (++pending == 4) {
+                for (int p = 0; p < n_polys; p++) {
+                    acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
+                    lazy[p].lo = lazy[p].hi = 0;
+                }
+                pending = 0;
+            }
+        } else {
+            for (int p = 0; p < n_polys; p++) acc[p] = addmod(acc[p], T.ct[p * T.stride + e], m.q);
+        }
     }
-    out[(((size_t)o * n_polys + p) * nq + j) * N + n] = acc;
+    for (int p = 0; p < n_polys; p++) {
+        if (pending) acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
+        out[((size_t)o * n_polys + p) * nq * N + e] = acc[p];
+    }
 }
 
 // acc3 (+)= sum_{g < G} (b1 b2, a1 b2 + a2 b1, a1 a2) of t1[g], t2[g], each [2][nq][N]
@@ -555,7 +575,7 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
         for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
         pm.c[j] = Cst{P, shoup_h(P, q)};
     }
-    dim3 grid(c->N / 256, E, n_out), block(256);
+    dim3 grid(n_out, c->N / 256, E), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN);
 }
@@ -617,7 +637,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
 
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s) {
-    dim3 grid(c->N / 256, nq * n_polys, n_out), block(256);
+    if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
+    dim3 grid(c->N / 256, nq, n_out), block(256);
     hipLaunchKernelGGL(masked_sum_kernel, grid, block, 0, s, (const LinTermDev *)terms_dev, group_off_dev, out,
                        c->d_modq, nq, n_polys, c->logN);
 }

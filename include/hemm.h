@@ -132,6 +132,8 @@ typedef struct {
     const uint64_t *ct;   /* [n_polys][.][N] */
     const uint64_t *mask; /* [nq][N] or NULL */
     uint64_t stride;      /* polynomial stride of ct in words */
+    uint64_t galois;      /* 0, or the mask is read through X -> X^galois (a rotated plaintext:
+                             leftRotate(Plaintext), HomEvaluator.hpp:376, without materialising it) */
 } hemm_lin_term;
 /* out[o][p] = sum over the terms of group o of mask * ct[p]; out: [n_out][n_polys][nq][N] */
 int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const uint32_t *group_offsets,
