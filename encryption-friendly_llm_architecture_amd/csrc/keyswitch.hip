@@ -14,6 +14,8 @@
 
 void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
                       int n_polys, size_t poly_stride, bool inverse, hipStream_t s);
+bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
+                          size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 
 namespace {
 
@@ -256,6 +258,8 @@ struct KsTables {
     // merged ModDown + rescale: basis {q_{nq-1}} U P dropped at once
     std::vector<size_t> drop_inv_off, drop_hat_off;      // [nq]
     std::vector<std::vector<Cst>> dropinv;               // [nq][j<nq-1]  (P q_{nq-1})^-1 mod q_j
+    size_t pinv_off = 0;                                 // device copies of pinv / dropinv[nq] / qlinv[l]
+    std::vector<size_t> dropinv_off, qlinv_off;
 };
 
 static KsTables *g_tables_of(const hemm_context *c);
@@ -327,6 +331,18 @@ static void build_tables(const hemm_context *c, KsTables &t) {
                 t.dropinv[nq].push_back(Cst{inv, shoup_h(inv, q)});
             }
         }
+    t.pinv_off = t.host.size();
+    for (auto &x : t.pinv) t.host.push_back(x);
+    t.dropinv_off.assign(nQ + 1, 0);
+    for (int nq = 0; nq <= nQ; nq++) {
+        t.dropinv_off[nq] = t.host.size();
+        for (auto &x : t.dropinv[nq]) t.host.push_back(x);
+    }
+    t.qlinv_off.assign(nQ, 0);
+    for (int l = 0; l < nQ; l++) {
+        t.qlinv_off[l] = t.host.size();
+        for (auto &x : t.qlinv[l]) t.host.push_back(x);
+    }
     HEMM_HIP(hipMalloc((void **)&t.dev, t.host.size() * sizeof(Cst)));
     HEMM_HIP(hipMemcpy(t.dev, t.host.data(), t.host.size() * sizeof(Cst), hipMemcpyHostToDevice));
 }
@@ -505,6 +521,8 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
     launch_ntt(c, last, pl, 1, n_polys, N, true, s);
     dim3 grid(N / 256, (nq - 1) * n_polys), block(256);
     hipLaunchKernelGGL(spread_kernel, grid, block, 0, s, last, tt, (size_t)(nq - 1) * N, c->d_modq, nq - 1, c->logN);
+    if (launch_ntt_sub_scale(c, tt, nq - 1, n_polys, in, in_stride, out, out_stride, t->dev + t->qlinv_off[nq - 1], s))
+        return;
     launch_ntt(c, tt, limbs_default(c, nq - 1, 0), nq - 1, n_polys, (size_t)(nq - 1) * N, false, s);
     CstList cl;
     for (int j = 0; j < nq - 1; j++) cl.c[j] = t->qlinv[nq - 1][j];
@@ -627,6 +645,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
     }
     dim3 grid(N / 256, n_polys), block(256);
     hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)ns * 256 * 8, s, a, c->d_modq);
+    const Cst *cst_dev = t->dev + (drop_last ? t->dropinv_off[nq] : t->pinv_off);
+    if (launch_ntt_sub_scale(c, conv, nq_out, n_polys, y, (size_t)E * N, out, out_stride, cst_dev, s)) return;
     launch_ntt(c, conv, limbs_default(c, nq_out, 0), nq_out, n_polys, (size_t)nq_out * N, false, s);
     CstList cl;
     for (int j = 0; j < nq_out; j++) cl.c[j] = drop_last ? t->dropinv[nq][j] : t->pinv[j];

@@ -207,11 +207,30 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
     }
 }
 
+// A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
+// the row kernel never cross a wavefront: ordering them needs no workgroup barrier, only a fence that
+// keeps the compiler from moving LDS accesses across it.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Optional tail of a forward transform: instead of storing the transformed residues v in place, store
+// (minuend - v) * cst[limb] to `out` -- the last step of ModDown / rescale, folded into the pass that
+// already holds v in registers (saves one read and one write of every limb and a launch).
+struct NttEpilogue {
+    const u64 *minuend;
+    u64 *out;
+    const Tw *cst;  // per limb: constant and Shoup quotient
+    size_t minuend_stride, out_stride;
+};
+
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
-template <bool INV>
+template <bool INV, bool EPI>
 __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
                                                          const ModQ *__restrict__ modq, LimbList ll, LimbList sl, int n_limbs,
-                                                         size_t poly_stride) {
+                                                         size_t poly_stride, NttEpilogue ep) {
     __shared__ u64 lds[16 * ROWPAD];
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
@@ -228,7 +247,7 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
         radix16_fwd(x, tw, 256u + r, q);
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
         radix16_fwd(x, tw, 16u * (256u + r) + c, q);
@@ -239,23 +258,38 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
             if (v >= q) v -= q;
             x[k] = v;
         }
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
-        __syncthreads();
+        wave_sync();
+        if (EPI) {
+            const size_t off = ((size_t)limb << 16) + ((size_t)r << 8);
+            const u64 *mn = ep.minuend + (size_t)poly * ep.minuend_stride + off;
+            u64 *o = ep.out + (size_t)poly * ep.out_stride + off;
+            const Tw cst = ep.cst[limb];
 #pragma unroll
-        for (int k = 0; k < 16; k++) row[c + 16 * k] = l[padc(c + 16 * k)];
+            for (int k = 0; k < 16; k++) {
+                const u64 v = l[padc(c + 16 * k)], y = mn[c + 16 * k];
+                const u64 d = y >= v ? y - v : y + q - v;
+                u64 t = mul_shoup_lazy(d, cst.w, cst.ws, q);
+                if (t >= q) t -= q;
+                o[c + 16 * k] = t;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) row[c + 16 * k] = l[padc(c + 16 * k)];
+        }
     } else {
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
         radix16_inv(x, tw, 16u * (256u + r) + c, q);
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(c + 16 * k)];
         radix16_inv(x, tw, 256u + r, q);
@@ -265,6 +299,27 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
 }
 
 }  // namespace
+
+// Forward transform of data[n_polys][n_limbs][N] (limb j = chain prime j) whose result is consumed as
+// out = (minuend - NTT(data)) * cst[j]; returns false when this ring size has no fused tail (the caller
+// then runs the transform and the subtraction separately).
+bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
+                          size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s) {
+    if (c->logN != 16) return false;
+    LimbList ll, sl;
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) ll.idx[j] = sl.idx[j] = (uint8_t)j;
+    const Tw *tw = (const Tw *)c->d_w;
+    dim3 grid(16, n_limbs * n_polys), block(256);
+    const size_t poly_stride = (size_t)n_limbs << 16;
+    NttEpilogue none{};
+    NttEpilogue ep{minuend, out, (const Tw *)cst_dev, minuend_stride, out_stride};
+    hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, ll, sl,
+                       n_limbs, poly_stride);
+    (void)none;
+    hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
+                       poly_stride, ep);
+    return true;
+}
 
 void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
                       int n_polys, size_t poly_stride, bool inverse, hipStream_t s) {
@@ -276,11 +331,11 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
         if (!inverse) {
             hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
                                c->d_ninv_s, ll, sl, n_limbs, poly_stride);
-            hipLaunchKernelGGL(ntt16_rows_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
-                               poly_stride);
+            hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
+                               poly_stride, NttEpilogue{});
         } else {
-            hipLaunchKernelGGL(ntt16_rows_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
-                               poly_stride);
+            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
+                               poly_stride, NttEpilogue{});
             hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
                                c->d_ninv_s, ll, sl, n_limbs, poly_stride);
         }
