@@ -67,7 +67,7 @@ def _declare(L):
     L.hemm_relinearize.argtypes = [vp, vp, sz, vp, u32, vp, sz, vp]
     L.hemm_rescale.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
     L.hemm_modup_batch.argtypes = [vp, vp, sz, u32, u32, vp, vp, vp]
-    L.hemm_hoisted_terms.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, vp, vp]
+    L.hemm_hoisted_terms.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, vp, ci, vp]
     L.hemm_moddown_batch.argtypes = [vp, vp, u32, u32, ci, vp, sz, vp, vp]
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
@@ -233,7 +233,7 @@ class Context:
                                      vp(ext.data_ptr()), vp(ws.data_ptr()), vp(0)))
         return ext
 
-    def hoisted_terms(self, groups, nq):
+    def hoisted_terms(self, groups, nq, b_premultiplied=False):
         """groups: list of lists of (ext, b, evk, mask or None, galois) -> y [n_out][2][nq+K][N]"""
         import torch
         flat = [t for g in groups for t in g]
@@ -246,7 +246,7 @@ class Context:
             offs.append(offs[-1] + len(g))
         off = (ctypes.c_uint32 * len(offs))(*offs)
         y = torch.empty((len(groups), 2, nq + self.nP, self.N), dtype=torch.int64, device=flat[0][0].device)
-        check(lib().hemm_hoisted_terms(self.h, arr, off, len(groups), nq, vp(y.data_ptr()), vp(0)))
+        check(lib().hemm_hoisted_terms(self.h, arr, off, len(groups), nq, vp(y.data_ptr()), int(b_premultiplied), vp(0)))
         return y
 
     def moddown_batch(self, y, nq, drop_last):

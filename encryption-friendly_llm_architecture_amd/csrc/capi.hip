@@ -283,7 +283,7 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
 }
 
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
-                       uint32_t nq, uint64_t *y, void *stream) {
+                       uint32_t nq, uint64_t *y, int b_premultiplied, void *stream) {
     HEMM_TRY
     int nl;
     chain_limbs(ctx, nq, 1, &nl);
@@ -304,7 +304,8 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), group_offsets, (n_out + 1) * sizeof(uint32_t),
                                   &off_dev, (hipStream_t)stream);
-    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, (hipStream_t)stream);
+    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
+                         (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

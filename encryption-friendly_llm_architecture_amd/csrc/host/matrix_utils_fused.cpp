@@ -74,6 +74,19 @@ hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois
     return t;
 }
 
+// P * b of a ciphertext's b-polynomial (limb j times P mod q_j), computed once per rotation source
+DeviceBuffer timesP(const Context &c, const u64 *b, u64 nq) {
+    DeviceBuffer out(c, nq * c->N);
+    std::vector<u64> sc(nq);
+    for (u64 j = 0; j < nq; j++) {
+        u64 P = 1;
+        for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+        sc[j] = P;
+    }
+    ck(hemm_mul_scalar(c->dev, b, 0, sc.data(), out.data(), 0, (uint32_t)nq, 0, 1, nullptr));
+    return out;
+}
+
 // ModUp of the a-polynomial of one ciphertext
 DeviceBuffer modUpOne(const Context &c, const Ciphertext &ct) {
     const u64 nq = ct.level_ + 1, E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha;
@@ -167,14 +180,15 @@ Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, c
 
     // 1. baby steps
     DeviceBuffer ext = modUpOne(c, in);
+    DeviceBuffer pb = timesP(c, in.getPolyData(0), nq);
     std::vector<hemm_rot_term> terms;
     std::vector<uint32_t> off{0};
     for (i64 j = 0; j < g.bs; j++) {
-        terms.push_back(term(ext.data(), in.getPolyData(0), pack, rot.galois((j + 1) * g.step), nullptr));
+        terms.push_back(term(ext.data(), pb.data(), pack, rot.galois((j + 1) * g.step), nullptr));
         off.push_back((uint32_t)terms.size());
     }
     DeviceBuffer y(c, (size_t)g.bs * 2 * E * N), baby(c, (size_t)g.bs * ctw), ws(c, (size_t)g.bs * ctw);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)g.bs, (uint32_t)nq, y.data(), nullptr));
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)g.bs, (uint32_t)nq, y.data(), 1, nullptr));
     ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * g.bs), 0, baby.data(), nq * N, ws.data(),
                           nullptr));
 
@@ -240,7 +254,7 @@ Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, c
                               rot.galois(group_rot[k + 1]), nullptr));
         uint32_t goff[2] = {0, (uint32_t)ng};
         DeviceBuffer y2(c, 2 * E * N), ws3(c, ctw);
-        ck(hemm_hoisted_terms(c->dev, gt.data(), goff, 1, (uint32_t)nq, y2.data(), nullptr));
+        ck(hemm_hoisted_terms(c->dev, gt.data(), goff, 1, (uint32_t)nq, y2.data(), 0, nullptr));
         ck(hemm_moddown_batch(c->dev, y2.data(), (uint32_t)nq, 2, 0, res.buf_.data(), nq * N, ws3.data(), nullptr));
         ck(hemm_pointwise(c->dev, HEMM_ADD, res.buf_.data(), nq * N, sums.data(), nq * N, res.buf_.data(), nq * N,
                           (uint32_t)nq, 0, 2, nullptr));
@@ -263,7 +277,7 @@ struct Shift {
     const Plaintext *mask2;  // nullptr: single-term shift
     bool two;
 };
-void assembleShifts(const HomEvaluator &eval, const Ciphertext &src, const DeviceBuffer &ext,
+void assembleShifts(const HomEvaluator &eval, const Ciphertext &src, const DeviceBuffer &ext, const DeviceBuffer &pb,
                     const std::vector<Shift> &shifts, size_t first, size_t count, u64 *y, u64 *out, u64 *ws) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
@@ -273,11 +287,11 @@ void assembleShifts(const HomEvaluator &eval, const Ciphertext &src, const Devic
     std::vector<uint32_t> off{0};
     for (size_t k = first; k < first + count; k++) {
         const Shift &s = shifts[k];
-        terms.push_back(term(ext.data(), src.getPolyData(0), pack, rot.galois(s.rot1), s.mask1));
-        if (s.two) terms.push_back(term(ext.data(), src.getPolyData(0), pack, rot.galois(s.rot2), s.mask2));
+        terms.push_back(term(ext.data(), pb.data(), pack, rot.galois(s.rot1), s.mask1));
+        if (s.two) terms.push_back(term(ext.data(), pb.data(), pack, rot.galois(s.rot2), s.mask2));
         off.push_back((uint32_t)terms.size());
     }
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)count, (uint32_t)nq, y, nullptr));
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)count, (uint32_t)nq, y, 1, nullptr));
     ck(hemm_moddown_batch(c->dev, y, (uint32_t)nq, (uint32_t)(2 * count), 1, out, (nq - 1) * N, ws, nullptr));
 }
 
@@ -330,14 +344,15 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     }
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
     DeviceBuffer extA = modUpOne(c, a.get()), extB = modUpOne(c, b.get());
+    DeviceBuffer pbA = timesP(c, a.get().getPolyData(0), nq), pbB = timesP(c, b.get().getPolyData(0), nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
     Ciphertext acc(c);
     acc.allocate(3, T + 1, 1);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), extA, sa, first, cnt, y.data(), t.data(), ws.data());
-        assembleShifts(eval, b.get(), extB, sb, first, cnt, y.data() + G * 2 * E * N, t.data() + G * 2 * lo * N,
+        assembleShifts(eval, a.get(), extA, pbA, sa, first, cnt, y.data(), t.data(), ws.data());
+        assembleShifts(eval, b.get(), extB, pbB, sb, first, cnt, y.data() + G * 2 * E * N, t.data() + G * 2 * lo * N,
                        ws.data() + G * 2 * lo * N);
         ck(hemm_tensor_batch(c->dev, t.data(), t.data() + G * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
                              first == 0 ? 0 : 1, nullptr));
@@ -380,6 +395,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
         sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], 2 * i - n, &cm[(size_t)(4 * i)], true});
     const u64 nqa = T + 3, nqb = T + 2, N = c->N, K = c->nP, lo = T + 2;  // both sides end at T+1 (lo limbs)
     DeviceBuffer extA = modUpOne(c, a.get()), extB = modUpOne(c, b.get());
+    DeviceBuffer pbA = timesP(c, a.get().getPolyData(0), nqa), pbB = timesP(c, b.get().getPolyData(0), nqb);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
@@ -389,15 +405,15 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     acc.allocate(3, T + 1, 1);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), extA, sa, first, cnt, ya.data(), t1.data(), ws.data());
+        assembleShifts(eval, a.get(), extA, pbA, sa, first, cnt, ya.data(), t1.data(), ws.data());
         // row shifts are exact rotations here: one unmasked hoisted term each, plain ModDown
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         for (size_t q = first; q < first + cnt; q++) {
-            terms.push_back(term(extB.data(), b.get().getPolyData(0), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
+            terms.push_back(term(extB.data(), pbB.data(), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
             off.push_back((uint32_t)terms.size());
         }
-        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, yb.data(), nullptr));
+        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, yb.data(), 1, nullptr));
         ck(hemm_moddown_batch(c->dev, yb.data(), (uint32_t)nqb, (uint32_t)(2 * cnt), 0, t2.data(), lo * N, ws.data(),
                               nullptr));
         ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
@@ -428,11 +444,12 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     for (i64 i = 1; i < n; i++) sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], i - n, &cm[(size_t)(2 * i)], true});
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
     DeviceBuffer ext = modUpOne(c, a.get());
+    DeviceBuffer pb = timesP(c, a.get().getPolyData(0), nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
     DeviceBuffer y(c, G * 2 * E * N), t(c, G * 2 * lo * N), ws(c, G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), ext, sa, first, cnt, y.data(), t.data(), ws.data());
+        assembleShifts(eval, a.get(), ext, pb, sa, first, cnt, y.data(), t.data(), ws.data());
         for (size_t q = 0; q < cnt; q++) {
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);

@@ -140,14 +140,18 @@ struct RotTermDev {
 __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
-                                                            int nq, int E, int beta, int n_full, int logN) {
+                                                            int nq, int E, int beta, int n_full, int logN,
+                                                            int b_premultiplied) {
     // blockIdx.x = output (fastest): workgroups that gather from the same 2 KiB source run back to back
     const int j = blockIdx.z, o = blockIdx.x;
     const int prime = ll.idx[j];
     const ModQ m = modq[prime];
     const u32 n = blockIdx.y * 256 + threadIdx.x;
     const size_t N = (size_t)1 << logN;
+    // masked terms are summed as 128-bit products and reduced once; unmasked terms are added directly
     u64 acc_b = 0, acc_a = 0;
+    u128_t lazy_b = {0, 0}, lazy_a = {0, 0};
+    int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const RotTermDev T = terms[t];
         const u32 np = galois_index(n, T.galois, logN);
@@ -160,14 +164,28 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
             add128(sa, mul64wide(x, ka));
         }
         u64 rb = barrett128(sb, m), ra = barrett128(sa, m);
-        if (j < nq) rb = addmod(rb, mul_shoup(T.b[(size_t)j * N + np], pmod.c[j].w, pmod.c[j].ws, m.q), m.q);
+        if (j < nq) {
+            const u64 bv = T.b[(size_t)j * N + np];
+            rb = addmod(rb, b_premultiplied ? bv : mul_shoup(bv, pmod.c[j].w, pmod.c[j].ws, m.q), m.q);
+        }
         if (T.mask != nullptr) {
             const u64 mk = T.mask[(size_t)j * N + n];
-            rb = mulmod(rb, mk, m);
-            ra = mulmod(ra, mk, m);
+            add128(lazy_b, mul64wide(rb, mk));
+            add128(lazy_a, mul64wide(ra, mk));
+            if (++pending == 4) {
+                acc_b = addmod(acc_b, barrett128(lazy_b, m), m.q);
+                acc_a = addmod(acc_a, barrett128(lazy_a, m), m.q);
+                lazy_b.lo = lazy_b.hi = lazy_a.lo = lazy_a.hi = 0;
+                pending = 0;
+            }
+        } else {
+            acc_b = addmod(acc_b, rb, m.q);
+            acc_a = addmod(acc_a, ra, m.q);
         }
-        acc_b = addmod(acc_b, rb, m.q);
-        acc_a = addmod(acc_a, ra, m.q);
+    }
+    if (pending) {
+        acc_b = addmod(acc_b, barrett128(lazy_b, m), m.q);
+        acc_a = addmod(acc_a, barrett128(lazy_a, m), m.q);
     }
     y[(((size_t)o * 2 + 0) * E + j) * N + n] = acc_b;
     y[(((size_t)o * 2 + 1) * E + j) * N + n] = acc_a;
@@ -584,7 +602,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
 
 // terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          hipStream_t s) {
+                          bool b_premultiplied, hipStream_t s) {
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     CstList pm;
     memset(&pm, 0, sizeof(pm));
@@ -595,7 +613,8 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     }
     dim3 grid(n_out, c->N / 256, E), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
-                       c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN);
+                       c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
+                       b_premultiplied ? 1 : 0);
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;

@@ -120,9 +120,10 @@ typedef struct {
 } hemm_rot_term;
 /* y[o] = sum over terms[group_offsets[o] .. group_offsets[o+1]) of
  *        mask * ( <galois(ext), evk> + P * galois(b) )      in the extended basis, y: [n_out][2][nq+n_p][N].
- * terms / group_offsets are host arrays. */
+ * terms / group_offsets are host arrays.  b_premultiplied != 0: every term's b already holds P*b
+ * (hemm_mul_scalar with P mod q_j once per source instead of once per term). */
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
-                       uint32_t n_out, uint32_t nq, uint64_t *y, void *stream);
+                       uint32_t n_out, uint32_t nq, uint64_t *y, int b_premultiplied, void *stream);
 /* y [n_polys][nq+n_p][N] (clobbered) -> out [n_polys][nq - drop_last][N]: division by P (drop_last = 0)
  * or by P*q_{nq-1} (drop_last = 1, ModDown and rescale in one basis conversion);
  * workspace >= n_polys*(nq-drop_last)*N words. */
