@@ -103,6 +103,7 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->modq.resize(T);
     std::vector<u64> w((size_t)T * N * 2), iw((size_t)T * N * 2), ninv(T), ninv_s(T), im(T), im_s(T);
     std::vector<u64> pw(N), ipw(N);
+    std::vector<double> fpc((size_t)T * 4);
     for (int i = 0; i < T; i++) {
         const u64 q = primes[i];
         u64 psi = 0;
@@ -121,14 +122,26 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
             ipw[j] = h_mulmod(ipw[j - 1], ipsi, q);
         }
         u64 *wt = w.data() + (size_t)i * N * 2, *iwt = iw.data() + (size_t)i * N * 2;
+        // Primes below 2^44 run the 2^16-point transform in double precision (exact: see ntt.hip); their
+        // table entries are the doubles (w, w / q) instead of (w, Shoup quotient).
+        const bool fp = (logN == 16) && (q >> 44) == 0;
+        auto as_bits = [](double d) {
+            u64 b;
+            memcpy(&b, &d, 8);
+            return b;
+        };
         for (int j = 0; j < N; j++) {
             unsigned r = bitrev((unsigned)j, logN);
-            wt[2 * j] = pw[r];
-            wt[2 * j + 1] = h_shoup(pw[r], q);
-            iwt[2 * j] = ipw[r];
-            iwt[2 * j + 1] = h_shoup(ipw[r], q);
+            wt[2 * j] = fp ? as_bits((double)pw[r]) : pw[r];
+            wt[2 * j + 1] = fp ? as_bits((double)pw[r] / (double)q) : h_shoup(pw[r], q);
+            iwt[2 * j] = fp ? as_bits((double)ipw[r]) : ipw[r];
+            iwt[2 * j + 1] = fp ? as_bits((double)ipw[r] / (double)q) : h_shoup(ipw[r], q);
         }
         ninv[i] = h_invmod((u64)N, q);
+        fpc[4 * i + 0] = fp ? (double)q : 0.0;
+        fpc[4 * i + 1] = fp ? 1.0 / (double)q : 0.0;
+        fpc[4 * i + 2] = (double)ninv[i];
+        fpc[4 * i + 3] = (double)ninv[i] / (double)q;
         ninv_s[i] = h_shoup(ninv[i], q);
         im[i] = pw[N / 2];
         im_s[i] = h_shoup(im[i], q);
@@ -153,6 +166,7 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_imag = (u64 *)up(im.data(), T * 8);
     c->d_imag_s = (u64 *)up(im_s.data(), T * 8);
     c->d_modq = (ModQ *)up(c->modq.data(), T * sizeof(ModQ));
+    c->d_fp = (double *)up(fpc.data(), fpc.size() * 8);
     c->d_scratch = nullptr;
     c->d_desc = nullptr;
     c->scratch_bytes = 0;
@@ -168,6 +182,7 @@ void hemm_context_free(hemm_context *c) {
     hipFree(c->d_imag);
     hipFree(c->d_imag_s);
     hipFree(c->d_modq);
+    hipFree(c->d_fp);
     if (c->d_scratch) hipFree(c->d_scratch);
     if (c->d_desc) hipFree(c->d_desc);
     delete c;

@@ -142,53 +142,82 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
                                                             const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
                                                             int nq, int E, int beta, int n_full, int logN,
                                                             int b_premultiplied) {
-    // blockIdx.x = output (fastest): workgroups that gather from the same 2 KiB source run back to back
+    // blockIdx.x = output (fastest): workgroups that gather from the same source tile run back to back.
+    // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
+    // (possibly swapped), so every access is a 16-byte load or store.
     const int j = blockIdx.z, o = blockIdx.x;
     const int prime = ll.idx[j];
     const ModQ m = modq[prime];
-    const u32 n = blockIdx.y * 256 + threadIdx.x;
+    const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
     const size_t N = (size_t)1 << logN;
-    // masked terms are summed as 128-bit products and reduced once; unmasked terms are added directly
-    u64 acc_b = 0, acc_a = 0;
-    u128_t lazy_b = {0, 0}, lazy_a = {0, 0};
+    u64 acc_b[2] = {0, 0}, acc_a[2] = {0, 0};
+    u128_t lazy_b[2] = {{0, 0}, {0, 0}}, lazy_a[2] = {{0, 0}, {0, 0}};
     int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const RotTermDev T = terms[t];
         const u32 np = galois_index(n, T.galois, logN);
-        u128_t sb = {0, 0}, sa = {0, 0};
+        const u32 base = np & ~1u;
+        const bool swap = (np & 1u) != 0;
+        u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
         for (int d = 0; d < beta; d++) {
-            const u64 x = T.ext[((size_t)d * E + j) * N + np];
-            const u64 kb = T.evk[(((size_t)d * 2 + 0) * n_full + prime) * N + n];
-            const u64 ka = T.evk[(((size_t)d * 2 + 1) * n_full + prime) * N + n];
-            add128(sb, mul64wide(x, kb));
-            add128(sa, mul64wide(x, ka));
+            ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
+            if (swap) {
+                const u64 tmp = x.x;
+                x.x = x.y;
+                x.y = tmp;
+            }
+            const ulonglong2 kb = *(const ulonglong2 *)(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
+            const ulonglong2 ka = *(const ulonglong2 *)(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+            add128(sb[0], mul64wide(x.x, kb.x));
+            add128(sb[1], mul64wide(x.y, kb.y));
+            add128(sa[0], mul64wide(x.x, ka.x));
+            add128(sa[1], mul64wide(x.y, ka.y));
         }
-        u64 rb = barrett128(sb, m), ra = barrett128(sa, m);
+        u64 rb[2] = {barrett128(sb[0], m), barrett128(sb[1], m)};
+        u64 ra[2] = {barrett128(sa[0], m), barrett128(sa[1], m)};
         if (j < nq) {
-            const u64 bv = T.b[(size_t)j * N + np];
-            rb = addmod(rb, b_premultiplied ? bv : mul_shoup(bv, pmod.c[j].w, pmod.c[j].ws, m.q), m.q);
+            ulonglong2 bv = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
+            if (swap) {
+                const u64 tmp = bv.x;
+                bv.x = bv.y;
+                bv.y = tmp;
+            }
+            if (!b_premultiplied) {
+                bv.x = mul_shoup(bv.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+                bv.y = mul_shoup(bv.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            }
+            rb[0] = addmod(rb[0], bv.x, m.q);
+            rb[1] = addmod(rb[1], bv.y, m.q);
         }
         if (T.mask != nullptr) {
-            const u64 mk = T.mask[(size_t)j * N + n];
-            add128(lazy_b, mul64wide(rb, mk));
-            add128(lazy_a, mul64wide(ra, mk));
+            const ulonglong2 mk = *(const ulonglong2 *)(T.mask + (size_t)j * N + n);
+            add128(lazy_b[0], mul64wide(rb[0], mk.x));
+            add128(lazy_b[1], mul64wide(rb[1], mk.y));
+            add128(lazy_a[0], mul64wide(ra[0], mk.x));
+            add128(lazy_a[1], mul64wide(ra[1], mk.y));
             if (++pending == 4) {
-                acc_b = addmod(acc_b, barrett128(lazy_b, m), m.q);
-                acc_a = addmod(acc_a, barrett128(lazy_a, m), m.q);
-                lazy_b.lo = lazy_b.hi = lazy_a.lo = lazy_a.hi = 0;
+                for (int i = 0; i < 2; i++) {
+                    acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
+                    acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
+                    lazy_b[i].lo = lazy_b[i].hi = lazy_a[i].lo = lazy_a[i].hi = 0;
+                }
                 pending = 0;
             }
         } else {
-            acc_b = addmod(acc_b, rb, m.q);
-            acc_a = addmod(acc_a, ra, m.q);
+            for (int i = 0; i < 2; i++) {
+                acc_b[i] = addmod(acc_b[i], rb[i], m.q);
+                acc_a[i] = addmod(acc_a[i], ra[i], m.q);
+            }
         }
     }
     if (pending) {
-        acc_b = addmod(acc_b, barrett128(lazy_b, m), m.q);
-        acc_a = addmod(acc_a, barrett128(lazy_a, m), m.q);
+        for (int i = 0; i < 2; i++) {
+            acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
+            acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
+        }
     }
-    y[(((size_t)o * 2 + 0) * E + j) * N + n] = acc_b;
-    y[(((size_t)o * 2 + 1) * E + j) * N + n] = acc_a;
+    *(ulonglong2 *)(y + (((size_t)o * 2 + 0) * E + j) * N + n) = make_ulonglong2(acc_b[0], acc_b[1]);
+    *(ulonglong2 *)(y + (((size_t)o * 2 + 1) * E + j) * N + n) = make_ulonglong2(acc_a[0], acc_a[1]);
 }
 
 struct LinTermDev {
@@ -611,7 +640,7 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
         for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
         pm.c[j] = Cst{P, shoup_h(P, q)};
     }
-    dim3 grid(n_out, c->N / 256, E), block(256);
+    dim3 grid(n_out, c->N / 512, E), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
                        b_premultiplied ? 1 : 0);

@@ -126,33 +126,121 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
 // ------------------------------------------------------------------------------------------
 // N = 2^16 kernels
 // ------------------------------------------------------------------------------------------
+// Two arithmetic back ends share the kernels below.
+//
+// IntField: 64-bit Shoup butterflies with values kept in [0, 4q) (Harvey), for primes up to 2^61.
+//
+// FpField: primes below 2^44 in double precision.  gfx950 issues one FP64 FMA per lane per clock but
+// has to assemble every 64-bit integer product from 32-bit pieces, so for residues that fit a double
+// exactly the floating-point butterfly is about a third of the instructions.  A product y*w mod q is
+//     c = rint(y * (w/q));  h = fl(y*w);  l = fma(y, w, -h)  [exact low part];  r = fma(-c, q, h) + l
+// Both h - c*q and the final sum are integers far below 2^53, so r is the exact centred residue
+// (|r| <= 0.54 q for |y| < 2^48).  Values stay signed and unreduced through the forward stages (growth
+// 0.54 q per stage); the inverse stages double the sums, so a radix-16 block first reduces its inputs.
+// The last pass maps to [0, q), which makes the stored result identical to the integer path's.
+// Between the two launches of one transform the buffer holds the raw doubles.
+#pragma clang fp contract(off)
+
+struct IntField {
+    typedef u64 E;
+    typedef Tw W;
+    u64 q, q2, ni, nis;
+    __device__ __forceinline__ IntField(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
+        q = modq[prime].q;
+        q2 = 2 * q;
+        ni = ninv[prime];
+        nis = ninv_s[prime];
+    }
+    __device__ __forceinline__ E from_canonical(u64 v) const { return v; }
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q2); }
+    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q2); }
+    __device__ __forceinline__ void before_inverse_block(E (&)[16]) const {}
+    __device__ __forceinline__ u64 to_canonical(E v) const {
+        if (v >= q2) v -= q2;
+        return v >= q ? v - q : v;
+    }
+    __device__ __forceinline__ u64 scale_to_canonical(E v) const {
+        u64 t = mul_shoup_lazy(v, ni, nis, q);
+        return t >= q ? t - q : t;
+    }
+};
+
+struct __align__(16) TwF {
+    double w, winv;
+};
+
+struct FpField {
+    typedef double E;
+    typedef TwF W;
+    double q, qinv, ni, niinv;
+    __device__ __forceinline__ FpField(const ModQ *, const u64 *, const u64 *, const double *fp, int prime) {
+        q = fp[4 * prime];
+        qinv = fp[4 * prime + 1];
+        ni = fp[4 * prime + 2];
+        niinv = fp[4 * prime + 3];
+    }
+    __device__ __forceinline__ E mulmod(E y, E w, E winv) const {
+        const double c = __builtin_rint(y * winv);
+        const double h = y * w;
+        const double l = __builtin_fma(y, w, -h);
+        return __builtin_fma(-c, q, h) + l;
+    }
+    __device__ __forceinline__ E reduce(E x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
+    __device__ __forceinline__ E from_canonical(u64 v) const {
+        return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - 4503599627370496.0;
+    }
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const {
+        const double v = mulmod(y, tw.w, tw.winv);
+        const double u = x;
+        x = u + v;
+        y = u - v;
+    }
+    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const {
+        const double u = x, v = y;
+        x = u + v;
+        y = mulmod(u - v, tw.w, tw.winv);
+    }
+    __device__ __forceinline__ void before_inverse_block(E (&x)[16]) const {
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = reduce(x[k]);
+    }
+    __device__ __forceinline__ u64 centred_to_canonical(E r) const {
+        r += r < 0.0 ? q : 0.0;
+        return (u64)__double_as_longlong(r + 4503599627370496.0) & 0x000fffffffffffffull;
+    }
+    __device__ __forceinline__ u64 to_canonical(E v) const { return centred_to_canonical(reduce(v)); }
+    __device__ __forceinline__ u64 scale_to_canonical(E v) const { return centred_to_canonical(mulmod(v, ni, niinv)); }
+};
+
 // radix-16 block of 4 Cooley-Tukey stages on registers; stage s, group g uses twiddle
 // (X << s) + g.
-__device__ __forceinline__ void radix16_fwd(u64 (&x)[16], const Tw *__restrict__ tw, const u32 X, const u64 q) {
-    const u64 q2 = 2 * q;
+template <class F>
+__device__ __forceinline__ void radix16_fwd(const F &f, typename F::E (&x)[16], const typename F::W *__restrict__ tw,
+                                            const u32 X) {
 #pragma unroll
     for (int s = 0; s < 4; s++) {
         const int d = 8 >> s;
 #pragma unroll
         for (int g = 0; g < (1 << s); g++) {
-            const Tw w = tw[(X << s) + g];
+            const typename F::W w = tw[(X << s) + g];
 #pragma unroll
-            for (int j = 0; j < d; j++) ct_bfly(x[g * 2 * d + j], x[g * 2 * d + j + d], w, q, q2);
+            for (int j = 0; j < d; j++) f.ct(x[g * 2 * d + j], x[g * 2 * d + j + d], w);
         }
     }
 }
 // radix-16 block of 4 Gentleman-Sande stages; stage s (distance 1<<s), group g uses twiddle
 // (X << (3-s)) + g.
-__device__ __forceinline__ void radix16_inv(u64 (&x)[16], const Tw *__restrict__ tw, const u32 X, const u64 q) {
-    const u64 q2 = 2 * q;
+template <class F>
+__device__ __forceinline__ void radix16_inv(const F &f, typename F::E (&x)[16], const typename F::W *__restrict__ tw,
+                                            const u32 X) {
 #pragma unroll
     for (int s = 0; s < 4; s++) {
         const int d = 1 << s;
 #pragma unroll
         for (int g = 0; g < (8 >> s); g++) {
-            const Tw w = tw[(X << (3 - s)) + g];
+            const typename F::W w = tw[(X << (3 - s)) + g];
 #pragma unroll
-            for (int j = 0; j < d; j++) gs_bfly(x[g * 2 * d + j], x[g * 2 * d + j + d], w, q, q2);
+            for (int j = 0; j < d; j++) f.gs(x[g * 2 * d + j], x[g * 2 * d + j + d], w);
         }
     }
 }
@@ -162,49 +250,58 @@ __device__ __forceinline__ void radix16_inv(u64 (&x)[16], const Tw *__restrict__
 __device__ __forceinline__ int padc(int c) { return c + (c >> 4); }
 
 // forward pass 1 / inverse pass 2 work on a 256-row x 16-column slab.
-template <bool INV>
-__global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
-                                                         const ModQ *__restrict__ modq,
-                                                         const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
-                                                         LimbList ll, LimbList sl, int n_limbs, size_t poly_stride) {
-    __shared__ u64 lds[256 * 16];
-    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
-    const int prime = ll.idx[limb];
-    const Tw *tw = tw_all + ((size_t)prime << 16);
-    const u64 q = modq[prime].q;
+template <bool INV, class F>
+__device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw) {
+    typedef typename F::E E;
+    const typename F::W *tw = (const typename F::W *)tw_int;
+    E *lds = (E *)lds_raw;
+    E *mem = (E *)base;
     const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
-    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + blockIdx.x * 16 + cc;
-    u64 x[16];
+    E x[16];
     if (!INV) {
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = base[(size_t)(rh + 16 * k) << 8];
-        radix16_fwd(x, tw, 1u, q);
+        for (int k = 0; k < 16; k++) x[k] = f.from_canonical(base[(size_t)(rh + 16 * k) << 8]);
+        radix16_fwd(f, x, tw, 1u);
 #pragma unroll
         for (int k = 0; k < 16; k++) lds[(rh + 16 * k) * 16 + cc] = x[k];
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = lds[(16 * rh + k) * 16 + cc];
-        radix16_fwd(x, tw, 16u + rh, q);
+        radix16_fwd(f, x, tw, 16u + rh);
 #pragma unroll
-        for (int k = 0; k < 16; k++) base[(size_t)(16 * rh + k) << 8] = x[k];
+        for (int k = 0; k < 16; k++) mem[(size_t)(16 * rh + k) << 8] = x[k];
     } else {
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = base[(size_t)(16 * rh + k) << 8];
-        radix16_inv(x, tw, 16u + rh, q);
+        for (int k = 0; k < 16; k++) x[k] = mem[(size_t)(16 * rh + k) << 8];
+        f.before_inverse_block(x);
+        radix16_inv(f, x, tw, 16u + rh);
 #pragma unroll
         for (int k = 0; k < 16; k++) lds[(16 * rh + k) * 16 + cc] = x[k];
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = lds[(rh + 16 * k) * 16 + cc];
-        radix16_inv(x, tw, 1u, q);
-        const u64 ni = ninv[prime], nis = ninv_s[prime];
+        f.before_inverse_block(x);
+        radix16_inv(f, x, tw, 1u);
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            u64 v = mul_shoup_lazy(x[k], ni, nis, q);
-            if (v >= q) v -= q;
-            base[(size_t)(rh + 16 * k) << 8] = v;
-        }
+        for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = f.scale_to_canonical(x[k]);
     }
+}
+
+template <bool INV>
+__global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                         const ModQ *__restrict__ modq,
+                                                         const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
+                                                         const double *__restrict__ fp, LimbList ll, LimbList sl,
+                                                         int n_limbs, size_t poly_stride) {
+    __shared__ u64 lds[256 * 16];
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
+    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + blockIdx.x * 16 + (threadIdx.x & 15);
+    if (fp[4 * prime] != 0.0)
+        cols_body<INV>(base, tw, FpField(modq, ninv, ninv_s, fp, prime), lds);
+    else
+        cols_body<INV>(base, tw, IntField(modq, ninv, ninv_s, fp, prime), lds);
 }
 
 // A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
@@ -227,49 +324,35 @@ struct NttEpilogue {
 };
 
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
-template <bool INV, bool EPI>
-__global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
-                                                         const ModQ *__restrict__ modq, LimbList ll, LimbList sl, int n_limbs,
-                                                         size_t poly_stride, NttEpilogue ep) {
-    __shared__ u64 lds[16 * ROWPAD];
-    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
-    const int prime = ll.idx[limb];
-    const Tw *tw = tw_all + ((size_t)prime << 16);
-    const u64 q = modq[prime].q, q2 = 2 * q;
+template <bool INV, bool EPI, class F>
+__device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw,
+                                          const u32 r, const u64 q, const u64 *__restrict__ mn, u64 *__restrict__ o,
+                                          const Tw cst) {
+    typedef typename F::E E;
+    const typename F::W *tw = (const typename F::W *)tw_int;
     const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
-    const u32 r = blockIdx.x * 16 + rr;  // global row
-    u64 *row = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
-    u64 *l = lds + rr * ROWPAD;
-    u64 x[16];
-#pragma unroll
-    for (int k = 0; k < 16; k++) x[k] = row[c + 16 * k];
+    E *l = (E *)lds_raw + rr * ROWPAD;
+    u64 *lc = lds_raw + rr * ROWPAD;
+    E *mem = (E *)row;
+    E x[16];
     if (!INV) {
-        radix16_fwd(x, tw, 256u + r, q);
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = mem[c + 16 * k];
+        radix16_fwd(f, x, tw, 256u + r);
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
-        radix16_fwd(x, tw, 16u * (256u + r) + c, q);
-#pragma unroll
-        for (int k = 0; k < 16; k++) {
-            u64 v = x[k];
-            if (v >= q2) v -= q2;
-            if (v >= q) v -= q;
-            x[k] = v;
-        }
+        radix16_fwd(f, x, tw, 16u * (256u + r) + c);
         wave_sync();
 #pragma unroll
-        for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
+        for (int k = 0; k < 16; k++) lc[padc(16 * c + k)] = f.to_canonical(x[k]);
         wave_sync();
         if (EPI) {
-            const size_t off = ((size_t)limb << 16) + ((size_t)r << 8);
-            const u64 *mn = ep.minuend + (size_t)poly * ep.minuend_stride + off;
-            u64 *o = ep.out + (size_t)poly * ep.out_stride + off;
-            const Tw cst = ep.cst[limb];
 #pragma unroll
             for (int k = 0; k < 16; k++) {
-                const u64 v = l[padc(c + 16 * k)], y = mn[c + 16 * k];
+                const u64 v = lc[padc(c + 16 * k)], y = mn[c + 16 * k];
                 const u64 d = y >= v ? y - v : y + q - v;
                 u64 t = mul_shoup_lazy(d, cst.w, cst.ws, q);
                 if (t >= q) t -= q;
@@ -277,25 +360,53 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
             }
         } else {
 #pragma unroll
-            for (int k = 0; k < 16; k++) row[c + 16 * k] = l[padc(c + 16 * k)];
+            for (int k = 0; k < 16; k++) row[c + 16 * k] = lc[padc(c + 16 * k)];
         }
     } else {
 #pragma unroll
-        for (int k = 0; k < 16; k++) l[padc(c + 16 * k)] = x[k];
+        for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = row[c + 16 * k];
         wave_sync();
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
-        radix16_inv(x, tw, 16u * (256u + r) + c, q);
+        for (int k = 0; k < 16; k++) x[k] = f.from_canonical(lc[padc(16 * c + k)]);
+        radix16_inv(f, x, tw, 16u * (256u + r) + c);
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(c + 16 * k)];
-        radix16_inv(x, tw, 256u + r, q);
+        f.before_inverse_block(x);
+        radix16_inv(f, x, tw, 256u + r);
 #pragma unroll
-        for (int k = 0; k < 16; k++) row[c + 16 * k] = x[k];
+        for (int k = 0; k < 16; k++) mem[c + 16 * k] = x[k];
     }
+}
+
+template <bool INV, bool EPI>
+__global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                         const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                         LimbList ll, LimbList sl, int n_limbs, size_t poly_stride,
+                                                         NttEpilogue ep) {
+    __shared__ u64 lds[16 * ROWPAD];
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const u32 r = blockIdx.x * 16 + (threadIdx.x >> 4);  // global row
+    u64 *row = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
+    const u64 *mn = nullptr;
+    u64 *o = nullptr;
+    Tw cst{0, 0};
+    if (EPI) {
+        const size_t off = ((size_t)limb << 16) + ((size_t)r << 8);
+        mn = ep.minuend + (size_t)poly * ep.minuend_stride + off;
+        o = ep.out + (size_t)poly * ep.out_stride + off;
+        cst = ep.cst[limb];
+    }
+    const u64 q = modq[prime].q;
+    if (fp[4 * prime] != 0.0)
+        rows_body<INV, EPI>(row, tw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst);
+    else
+        rows_body<INV, EPI>(row, tw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst);
 }
 
 }  // namespace
@@ -313,10 +424,10 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
     const size_t poly_stride = (size_t)n_limbs << 16;
     NttEpilogue none{};
     NttEpilogue ep{minuend, out, (const Tw *)cst_dev, minuend_stride, out_stride};
-    hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, ll, sl,
-                       n_limbs, poly_stride);
+    hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ll,
+                       sl, n_limbs, poly_stride);
     (void)none;
-    hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
+    hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl, n_limbs,
                        poly_stride, ep);
     return true;
 }
@@ -330,14 +441,14 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
         dim3 grid(16, lanes), block(256);
         if (!inverse) {
             hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, sl, n_limbs, poly_stride);
-            hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
-                               poly_stride, NttEpilogue{});
+                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
+            hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
+                               n_limbs, poly_stride, NttEpilogue{});
         } else {
-            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), grid, block, 0, s, data, tw, c->d_modq, ll, sl, n_limbs,
-                               poly_stride, NttEpilogue{});
+            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
+                               n_limbs, poly_stride, NttEpilogue{});
             hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, ll, sl, n_limbs, poly_stride);
+                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
         }
         return;
     }
