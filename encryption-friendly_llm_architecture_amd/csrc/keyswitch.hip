@@ -59,6 +59,57 @@ __global__ __launch_bounds__(256) void bconv_kernel(BConvArgs a, const ModQ *__r
     }
 }
 
+// Register form of the same conversion for up to 8 source limbs: a thread owns two adjacent coefficients
+// (16-byte accesses), keeps the scaled source residues in registers and sums the Shoup products of a
+// target limb lazily (each below 2q; reduced every 3 terms, which cannot overflow for q < 2^61).
+template <int NS>
+__global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ *__restrict__ modq) {
+    const int poly = blockIdx.y;
+    const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const u64 *src = a.src + poly * a.src_poly_stride;
+    u64 *dst = a.dst + poly * a.dst_poly_stride;
+    u64 v0[NS], v1[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        const u64 q = modq[a.src_prime[i]].q;
+        const Cst c = a.inv[i];
+        const ulonglong2 x = *(const ulonglong2 *)(src + ((size_t)a.src_slot[i] << a.logN) + n);
+        v0[i] = mul_shoup(x.x, c.w, c.ws, q);
+        v1[i] = mul_shoup(x.y, c.w, c.ws, q);
+    }
+    for (int j = 0; j < a.n_dst; j++) {
+        const int pj = a.dst_prime[j];
+        const u64 q = modq[pj].q;
+        u64 acc0 = 0, acc1 = 0;
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            const Cst c = a.hat[i * a.hat_ld + pj];
+            acc0 += mul_shoup_lazy(v0[i], c.w, c.ws, q);
+            acc1 += mul_shoup_lazy(v1[i], c.w, c.ws, q);
+            if (i % 3 == 2 || i == NS - 1) {
+                if (acc0 >= 4 * q) acc0 -= 4 * q;
+                if (acc1 >= 4 * q) acc1 -= 4 * q;
+                if (acc0 >= 2 * q) acc0 -= 2 * q;
+                if (acc1 >= 2 * q) acc1 -= 2 * q;
+                if (acc0 >= q) acc0 -= q;
+                if (acc1 >= q) acc1 -= q;
+            }
+        }
+        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
+    }
+}
+
+// grid = (N / 256, n_polys) coefficients x polynomials
+void launch_bconv(const BConvArgs &a, const ModQ *modq, int N, int n_polys, hipStream_t s) {
+    dim3 block(256), wide(N / 256, n_polys), pair(N / 512, n_polys);
+    switch (a.n_src) {
+#define BCONV_CASE(K) case K: hipLaunchKernelGGL(bconv_reg_kernel<K>, pair, block, 0, s, a, modq); break;
+        BCONV_CASE(1) BCONV_CASE(2) BCONV_CASE(3) BCONV_CASE(4) BCONV_CASE(5) BCONV_CASE(6) BCONV_CASE(7) BCONV_CASE(8)
+#undef BCONV_CASE
+        default: hipLaunchKernelGGL(bconv_kernel, wide, block, (size_t)a.n_src * 256 * 8, s, a, modq);
+    }
+}
+
 struct DigitMap {
     uint8_t digit_of[HEMM_MAX_PRIMES];  // for limb j < nq: owning digit; 255 for special limbs
 };
@@ -231,11 +282,25 @@ struct LinTermDev {
 // 128-bit values and reduced every 4 terms.
 __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
                                                          const u32 *__restrict__ group_off, u64 *__restrict__ out,
-                                                         const ModQ *__restrict__ modq, int nq, int n_polys, int logN) {
-    const int j = blockIdx.y, o = blockIdx.z;
+                                                         const ModQ *__restrict__ modq, int nq, int n_polys, int logN,
+                                                         int n_out) {
+    // Workgroups go round-robin over the 8 XCDs, each with its own L2.  The outputs of one launch mostly
+    // sum the same ciphertexts under different masks, so all outputs of a (limb, 256-coefficient) tile are
+    // placed back to back on one XCD: the ciphertext tile is fetched from HBM once instead of once per output.
+    const u32 tiles = (u32)nq << (logN - 8);
+    u32 o, tile;
+    if ((tiles & 7u) == 0) {
+        const u32 xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+        o = slot % (u32)n_out;
+        tile = (slot / (u32)n_out) * 8u + xcd;
+    } else {
+        o = blockIdx.x % (u32)n_out;
+        tile = blockIdx.x / (u32)n_out;
+    }
+    const int j = (int)(tile >> (logN - 8));
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN;
-    const size_t e = (size_t)j * N + (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t e = (size_t)j * N + (size_t)(tile & ((1u << (logN - 8)) - 1)) * 256 + threadIdx.x;
     u64 acc[3] = {0, 0, 0};
     u128_t lazy[3] = {{0, 0}, {0, 0}, {0, 0}};
     int pending = 0;
@@ -469,8 +534,7 @@ void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, b
         }
         a.n_dst = nd;
         if (nd > 0) {
-            dim3 grid(N / 256, 1), block(256);
-            hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)a.n_src * 256 * 8, s, a, c->d_modq);
+            launch_bconv(a, c->d_modq, (int)N, 1, s);
             launch_ntt_slots(c, a.dst, pl, sl, nd, 1, (size_t)E * N, false, s);
         }
         if (fill_own)
@@ -524,8 +588,8 @@ void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, si
         a.dst_slot[j] = (uint8_t)j;
         a.dst_prime[j] = (uint8_t)j;
     }
-    dim3 grid(N / 256, n_polys), block(256);
-    hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)K * 256 * 8, s, a, c->d_modq);
+    launch_bconv(a, c->d_modq, (int)N, n_polys, s);
+    const dim3 block(256);
     launch_ntt(c, conv, limbs_default(c, nq, 0), nq, n_polys, (size_t)nq * N, false, s);
     CstList cl;
     for (int j = 0; j < nq; j++) cl.c[j] = t->pinv[j];
@@ -620,8 +684,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         }
         a.n_dst = nd;
         if (nd > 0) {
-            dim3 grid(N / 256, n_in), block(256);
-            hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)a.n_src * 256 * 8, s, a, c->d_modq);
+            launch_bconv(a, c->d_modq, (int)N, n_in, s);
             launch_ntt_slots(c, a.dst, pl, sl, nd, n_in, (size_t)beta * E * N, false, s);
         }
         HEMM_HIP(hipMemcpy2DAsync(a.dst + (size_t)lo * N, (size_t)beta * E * N * 8, in + (size_t)lo * N, in_stride * 8,
@@ -691,8 +754,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
         a.dst_slot[j] = (uint8_t)j;
         a.dst_prime[j] = (uint8_t)j;
     }
-    dim3 grid(N / 256, n_polys), block(256);
-    hipLaunchKernelGGL(bconv_kernel, grid, block, (size_t)ns * 256 * 8, s, a, c->d_modq);
+    launch_bconv(a, c->d_modq, (int)N, n_polys, s);
+    const dim3 block(256);
     const Cst *cst_dev = t->dev + (drop_last ? t->dropinv_off[nq] : t->pinv_off);
     if (launch_ntt_sub_scale(c, conv, nq_out, n_polys, y, (size_t)E * N, out, out_stride, cst_dev, s)) return;
     launch_ntt(c, conv, limbs_default(c, nq_out, 0), nq_out, n_polys, (size_t)nq_out * N, false, s);
@@ -706,9 +769,9 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s) {
     if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
-    dim3 grid(c->N / 256, nq, n_out), block(256);
+    dim3 grid((unsigned)(c->N / 256) * nq * n_out), block(256);
     hipLaunchKernelGGL(masked_sum_kernel, grid, block, 0, s, (const LinTermDev *)terms_dev, group_off_dev, out,
-                       c->d_modq, nq, n_polys, c->logN);
+                       c->d_modq, nq, n_polys, c->logN, n_out);
 }
 
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
