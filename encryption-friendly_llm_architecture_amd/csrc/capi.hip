@@ -363,7 +363,8 @@ int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64
     chain_limbs(ctx, nq, 0, &nl);
     need(in && out, "null operand");
     need(nq >= 2, "rescale needs at least two limbs");
-    need(n_polys >= 1 && n_polys <= 3, "n_polys must be 1..3");
+    need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_scratch_words(ctx),
+         "n_polys * nq limbs must fit the context's scratch ((dnum + 7) * (nQ + nP) limbs)");
     launch_rescale(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
                    (hipStream_t)stream);
     check_launch();

@@ -57,6 +57,11 @@ public:
     Ciphertext diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
                                       const TileTensorShape &shape);
 
+    // the same for n_jobs operands at one level through shared launches: in [job][2][level+1][N] -> out
+    // [job][2][level][N] (one level lower, rescaled)
+    void diagonalTransformBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
+                                const TileTensorShape *shapes, u64 *out);
+
     void cleanUp();
     size_t cachedMasks() const;
 

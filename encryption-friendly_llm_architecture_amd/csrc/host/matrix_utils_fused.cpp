@@ -167,101 +167,145 @@ std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, boo
 //   one masked-sum launch for every (giant index, sign) group;
 //   1 batched ModUp of the group sums, every giant rotation as a hoisted term of ONE output, so the
 //   groups are summed in the extended basis and share a single ModDown; one rescale at the end.
-Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
-                                                     const TileTensorShape &shape) {
+// Several transforms of operands at the same level (sigma(A) and tau(B) of one product) go through the
+// same launches: `in` holds n_jobs ciphertexts [job][2][nq][N], `out` receives [job][2][nq-1][N].
+void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
+                                               const MaskKind *kinds, const TileTensorShape *shapes, u64 *out) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
-    const Geo g = geo(kind, shape);
     const Rot rot(c);
-    const u64 level = in.getLevel(), nq = level + 1, N = c->N, K = c->nP, E = nq + K;
+    const u64 nq = level + 1, N = c->N, K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     if (level == 0) throw std::invalid_argument("[diagonalTransform] level >= 1 is needed.");
-    if (in.getRescaleCounter() != 0) throw RuntimeException("diagonalTransform: operand must be rescaled first");
     const size_t ctw = 2 * nq * N;  // words per 2-poly ciphertext at this level
+    std::vector<Geo> g;
+    std::vector<size_t> baby_first{0};  // index of a job's first baby ciphertext
+    for (size_t q = 0; q < n_jobs; q++) {
+        g.push_back(geo(kinds[q], shapes[q]));
+        baby_first.push_back(baby_first.back() + (size_t)g[q].bs);
+    }
+    const size_t n_baby = baby_first.back();
 
     // 1. baby steps
-    DeviceBuffer ext = modUpOne(c, in);
-    DeviceBuffer pb = timesP(c, in.getPolyData(0), nq);
+    DeviceBuffer ext(c, n_jobs * beta * E * N), pb(c, n_jobs * nq * N);
+    {
+        DeviceBuffer ws(c, n_jobs * nq * N);
+        ck(hemm_modup_batch(c->dev, in + nq * N, ctw, (uint32_t)nq, (uint32_t)n_jobs, ext.data(), ws.data(), nullptr));
+        std::vector<u64> sc(nq);
+        for (u64 j = 0; j < nq; j++) {
+            u64 P = 1;
+            for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+            sc[j] = P;
+        }
+        ck(hemm_mul_scalar(c->dev, in, ctw, sc.data(), pb.data(), nq * N, (uint32_t)nq, 0, (uint32_t)n_jobs, nullptr));
+    }
     std::vector<hemm_rot_term> terms;
     std::vector<uint32_t> off{0};
-    for (i64 j = 0; j < g.bs; j++) {
-        terms.push_back(term(ext.data(), pb.data(), pack, rot.galois((j + 1) * g.step), nullptr));
-        off.push_back((uint32_t)terms.size());
-    }
-    DeviceBuffer y(c, (size_t)g.bs * 2 * E * N), baby(c, (size_t)g.bs * ctw), ws(c, (size_t)g.bs * ctw);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)g.bs, (uint32_t)nq, y.data(), 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * g.bs), 0, baby.data(), nq * N, ws.data(),
+    for (size_t q = 0; q < n_jobs; q++)
+        for (i64 j = 0; j < g[q].bs; j++) {
+            terms.push_back(term(ext.data() + q * beta * E * N, pb.data() + q * nq * N, pack,
+                                 rot.galois((j + 1) * g[q].step), nullptr));
+            off.push_back((uint32_t)terms.size());
+        }
+    DeviceBuffer y(c, n_baby * 2 * E * N), baby(c, n_baby * ctw), ws(c, n_baby * ctw);
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)n_baby, (uint32_t)nq, y.data(), 1, nullptr));
+    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * n_baby), 0, baby.data(), nq * N, ws.data(),
                           nullptr));
 
-    // 2. group sums: group 0 needs no rotation (d = 0, the positive diagonals of giant index 0, and any
-    //    group whose rotation is a whole turn)
-    std::vector<std::vector<hemm_lin_term>> groups(1);
-    std::vector<i64> group_rot{0};  // left rotation still to apply to each group
-    auto lin = [&](const u64 *ct, i64 d) {
-        hemm_lin_term t;
-        t.ct = ct;
-        t.mask = transformMask(eval, kind, shape, level, d).buf_.data();
-        t.stride = nq * N;
-        t.galois = 0;
-        return t;
-    };
-    auto push_group = [&](std::vector<hemm_lin_term> &&g_terms, i64 r) {
-        if (g_terms.empty()) return;
-        if (rot.norm(r) == 0) {
-            for (auto &t : g_terms) groups[0].push_back(t);
-        } else {
-            groups.push_back(std::move(g_terms));
-            group_rot.push_back(r);
+    // 2. group sums: a job's group 0 needs no rotation (d = 0, the positive diagonals of giant index 0, and
+    //    any group whose rotation is a whole turn).  The unrotated groups of all jobs come first in `sums`,
+    //    then every rotated group, so the rotated ones form one contiguous ModUp batch.
+    std::vector<std::vector<hemm_lin_term>> plain(n_jobs), rotated;
+    std::vector<i64> rotated_by;        // left rotation still to apply to each rotated group
+    std::vector<size_t> rotated_first{0};
+    for (size_t q = 0; q < n_jobs; q++) {
+        const Geo &gq = g[q];
+        const u64 *ct = in + q * ctw;
+        const u64 *bb = baby.data() + baby_first[q] * ctw;
+        auto lin = [&](const u64 *src, i64 d) {
+            hemm_lin_term t;
+            t.ct = src;
+            t.mask = transformMask(eval, kinds[q], shapes[q], level, d).buf_.data();
+            t.stride = nq * N;
+            t.galois = 0;
+            return t;
+        };
+        auto push_group = [&](std::vector<hemm_lin_term> &&g_terms, i64 r) {
+            if (g_terms.empty()) return;
+            if (rot.norm(r) == 0) {
+                for (auto &t : g_terms) plain[q].push_back(t);
+            } else {
+                rotated.push_back(std::move(g_terms));
+                rotated_by.push_back(r);
+            }
+        };
+        plain[q].push_back(lin(ct, 0));
+        for (i64 i = 0; i < gq.gs; i++) {
+            std::vector<hemm_lin_term> neg, pos;
+            for (i64 j = 0; j < gq.bs; j++) {
+                const i64 d = 1 + i * gq.bs + j - gq.units;
+                if (d >= 0) break;
+                neg.push_back(lin(bb + (size_t)j * ctw, d));
+            }
+            push_group(std::move(neg), -(gq.units - i * gq.bs) * gq.step);
+            for (i64 j = 0; j < gq.bs; j++) {
+                const i64 d = 1 + i * gq.bs + j;
+                if (d >= gq.units) break;
+                pos.push_back(lin(bb + (size_t)j * ctw, d));
+            }
+            push_group(std::move(pos), i * gq.bs * gq.step);
         }
-    };
-    groups[0].push_back(lin(in.buf_.data(), 0));
-    for (i64 i = 0; i < g.gs; i++) {
-        std::vector<hemm_lin_term> neg, pos;
-        for (i64 j = 0; j < g.bs; j++) {
-            const i64 d = 1 + i * g.bs + j - g.units;
-            if (d >= 0) break;
-            neg.push_back(lin(baby.data() + (size_t)j * ctw, d));
-        }
-        push_group(std::move(neg), -(g.units - i * g.bs) * g.step);
-        for (i64 j = 0; j < g.bs; j++) {
-            const i64 d = 1 + i * g.bs + j;
-            if (d >= g.units) break;
-            pos.push_back(lin(baby.data() + (size_t)j * ctw, d));
-        }
-        push_group(std::move(pos), i * g.bs * g.step);
+        rotated_first.push_back(rotated.size());
     }
     std::vector<hemm_lin_term> lt;
     std::vector<uint32_t> loff{0};
-    for (auto &gr : groups) {
+    for (auto &gr : plain) {
         for (auto &t : gr) lt.push_back(t);
         loff.push_back((uint32_t)lt.size());
     }
-    const size_t n_groups = group_rot.size();
+    for (auto &gr : rotated) {
+        for (auto &t : gr) lt.push_back(t);
+        loff.push_back((uint32_t)lt.size());
+    }
+    const size_t ng = rotated.size(), n_groups = n_jobs + ng;
     DeviceBuffer sums(c, n_groups * ctw);
     ck(hemm_masked_sum_batch(c->dev, lt.data(), loff.data(), (uint32_t)n_groups, (uint32_t)nq, 2, sums.data(), nullptr));
 
-    // 3. giant steps: every rotated group is a term of one output
-    Ciphertext res(c);
-    res.allocate(2, level, 1);
-    if (n_groups > 1) {
-        const size_t ng = n_groups - 1;
-        const u64 beta = (nq + c->alpha - 1) / c->alpha;
+    // 3. giant steps: every rotated group is a term of its job's output
+    DeviceBuffer res(c, n_jobs * ctw);
+    bool every_job_rotates = ng > 0;
+    for (size_t q = 0; q < n_jobs; q++) every_job_rotates = every_job_rotates && rotated_first[q + 1] > rotated_first[q];
+    if (every_job_rotates) {
+        const u64 *rs = sums.data() + n_jobs * ctw;
         DeviceBuffer ext2(c, ng * beta * E * N), ws2(c, ng * nq * N);
-        ck(hemm_modup_batch(c->dev, sums.data() + ctw + nq * N, ctw, (uint32_t)nq, (uint32_t)ng, ext2.data(), ws2.data(),
-                            nullptr));
+        ck(hemm_modup_batch(c->dev, rs + nq * N, ctw, (uint32_t)nq, (uint32_t)ng, ext2.data(), ws2.data(), nullptr));
         std::vector<hemm_rot_term> gt;
-        for (size_t k = 0; k < ng; k++)
-            gt.push_back(term(ext2.data() + k * beta * E * N, sums.data() + (k + 1) * ctw, pack,
-                              rot.galois(group_rot[k + 1]), nullptr));
-        uint32_t goff[2] = {0, (uint32_t)ng};
-        DeviceBuffer y2(c, 2 * E * N), ws3(c, ctw);
-        ck(hemm_hoisted_terms(c->dev, gt.data(), goff, 1, (uint32_t)nq, y2.data(), 0, nullptr));
-        ck(hemm_moddown_batch(c->dev, y2.data(), (uint32_t)nq, 2, 0, res.buf_.data(), nq * N, ws3.data(), nullptr));
-        ck(hemm_pointwise(c->dev, HEMM_ADD, res.buf_.data(), nq * N, sums.data(), nq * N, res.buf_.data(), nq * N,
-                          (uint32_t)nq, 0, 2, nullptr));
+        std::vector<uint32_t> goff{0};
+        for (size_t q = 0; q < n_jobs; q++) {
+            for (size_t k = rotated_first[q]; k < rotated_first[q + 1]; k++)
+                gt.push_back(term(ext2.data() + k * beta * E * N, rs + k * ctw, pack, rot.galois(rotated_by[k]), nullptr));
+            goff.push_back((uint32_t)gt.size());
+        }
+        DeviceBuffer y2(c, n_jobs * 2 * E * N), ws3(c, n_jobs * ctw);
+        ck(hemm_hoisted_terms(c->dev, gt.data(), goff.data(), (uint32_t)n_jobs, (uint32_t)nq, y2.data(), 0, nullptr));
+        ck(hemm_moddown_batch(c->dev, y2.data(), (uint32_t)nq, (uint32_t)(2 * n_jobs), 0, res.data(), nq * N, ws3.data(),
+                              nullptr));
+        ck(hemm_pointwise(c->dev, HEMM_ADD, res.data(), nq * N, sums.data(), nq * N, res.data(), nq * N, (uint32_t)nq, 0,
+                          (uint32_t)(2 * n_jobs), nullptr));
+    } else if (ng == 0) {
+        (void)hipMemcpyAsync(res.data(), sums.data(), n_jobs * ctw * 8, hipMemcpyDeviceToDevice, nullptr);
     } else {
-        (void)hipMemcpyAsync(res.buf_.data(), sums.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+        throw RuntimeException("diagonalTransformBatch: jobs with and without giant steps cannot share a batch");
     }
-    eval.rescale(res);
+    ck(hemm_rescale(c->dev, res.data(), nq * N, out, (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
+}
+
+Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                                     const TileTensorShape &shape) {
+    if (in.getRescaleCounter() != 0) throw RuntimeException("diagonalTransform: operand must be rescaled first");
+    if (in.getLevel() == 0) throw std::invalid_argument("[diagonalTransform] level >= 1 is needed.");
+    Ciphertext res(eval.getContext());
+    res.allocate(2, in.getLevel() - 1, 0);
+    diagonalTransformBatch(eval, in.buf_.data(), 1, in.getLevel(), &kind, &shape, res.buf_.data());
     return res;
 }
 
@@ -277,18 +321,18 @@ struct Shift {
     const Plaintext *mask2;  // nullptr: single-term shift
     bool two;
 };
-void assembleShifts(const HomEvaluator &eval, const Ciphertext &src, const DeviceBuffer &ext, const DeviceBuffer &pb,
+void assembleShifts(const HomEvaluator &eval, u64 src_level, const u64 *ext, const u64 *pb,
                     const std::vector<Shift> &shifts, size_t first, size_t count, u64 *y, u64 *out, u64 *ws) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    const u64 nq = src.getLevel() + 1, N = c->N;
+    const u64 nq = src_level + 1, N = c->N;
     std::vector<hemm_rot_term> terms;
     std::vector<uint32_t> off{0};
     for (size_t k = first; k < first + count; k++) {
         const Shift &s = shifts[k];
-        terms.push_back(term(ext.data(), pb.data(), pack, rot.galois(s.rot1), s.mask1));
-        if (s.two) terms.push_back(term(ext.data(), pb.data(), pack, rot.galois(s.rot2), s.mask2));
+        terms.push_back(term(ext, pb, pack, rot.galois(s.rot1), s.mask1));
+        if (s.two) terms.push_back(term(ext, pb, pack, rot.galois(s.rot2), s.mask2));
         off.push_back((uint32_t)terms.size());
     }
     ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)count, (uint32_t)nq, y, 1, nullptr));
@@ -329,8 +373,22 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     eval.levelDown(b.get(), T + 3, b.get());
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
     std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);
-    a.get() = tr.diagonalTransformFused(eval, a.get(), MaskKind::Horizontal, a.getShape());
-    b.get() = tr.diagonalTransformFused(eval, b.get(), MaskKind::Vertical, b.getShape());
+    // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
+    const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
+    DeviceBuffer ab(c, 2 * ctw);
+    {
+        const u64 ctw_in = 2 * (nq + 1) * N;
+        DeviceBuffer joint(c, 2 * ctw_in);
+        (void)hipMemcpyAsync(joint.data(), a.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(joint.data() + ctw_in, b.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        const MaskKind kinds[2] = {MaskKind::Horizontal, MaskKind::Vertical};
+        const TileTensorShape shapes[2] = {a.getShape(), b.getShape()};
+        tr.diagonalTransformBatch(eval, joint.data(), 2, T + 3, kinds, shapes, ab.data());
+    }
+    a.get().allocate(2, T + 2, 0);
+    b.get().allocate(2, T + 2, 0);
+    (void)hipMemcpyAsync(a.get().buf_.data(), ab.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipMemcpyAsync(b.get().buf_.data(), ab.data() + ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
 
     CtxtTensor res(c, rows, cols, w);
     eval.mult(a.get(), b.get(), res.get());  // k = 0 term, level T+1
@@ -342,19 +400,45 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], i - n, &cm[(size_t)(2 * i)], true});
         sb.push_back(Shift{i * w, &rm[(size_t)(2 * i + 1)], (i - n) * w, &rm[(size_t)(2 * i)], true});
     }
-    const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
-    DeviceBuffer extA = modUpOne(c, a.get()), extB = modUpOne(c, b.get());
-    DeviceBuffer pbA = timesP(c, a.get().getPolyData(0), nq), pbB = timesP(c, b.get().getPolyData(0), nq);
+    // ModUp and P * b of both rotation sources in one batch each
+    const u64 beta = (nq + c->alpha - 1) / c->alpha;
+    DeviceBuffer extAB(c, 2 * beta * E * N), pbAB(c, 2 * nq * N);
+    {
+        DeviceBuffer mws(c, 2 * nq * N);
+        ck(hemm_modup_batch(c->dev, ab.data() + nq * N, ctw, (uint32_t)nq, 2, extAB.data(), mws.data(), nullptr));
+        std::vector<u64> sc(nq);
+        for (u64 j = 0; j < nq; j++) {
+            u64 P = 1;
+            for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+            sc[j] = P;
+        }
+        ck(hemm_mul_scalar(c->dev, ab.data(), ctw, sc.data(), pbAB.data(), nq * N, (uint32_t)nq, 0, 2, nullptr));
+    }
+    const u64 *extA = extAB.data(), *extB = extAB.data() + beta * E * N;
+    const u64 *pbA = pbAB.data(), *pbB = pbAB.data() + nq * N;
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
     Ciphertext acc(c);
     acc.allocate(3, T + 1, 1);
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
     for (size_t first = 0; first < sa.size(); first += G) {
+        // cnt column shifts of sigma(A), then cnt row shifts of tau(B): one launch chain for all 2 cnt outputs
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), extA, pbA, sa, first, cnt, y.data(), t.data(), ws.data());
-        assembleShifts(eval, b.get(), extB, pbB, sb, first, cnt, y.data() + G * 2 * E * N, t.data() + G * 2 * lo * N,
-                       ws.data() + G * 2 * lo * N);
-        ck(hemm_tensor_batch(c->dev, t.data(), t.data() + G * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        for (int side = 0; side < 2; side++) {
+            const std::vector<Shift> &sh = side ? sb : sa;
+            const u64 *ext = side ? extB : extA, *pb = side ? pbB : pbA;
+            for (size_t q = first; q < first + cnt; q++) {
+                terms.push_back(term(ext, pb, pack, rot.galois(sh[q].rot1), sh[q].mask1));
+                terms.push_back(term(ext, pb, pack, rot.galois(sh[q].rot2), sh[q].mask2));
+                off.push_back((uint32_t)terms.size());
+            }
+        }
+        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)(2 * cnt), (uint32_t)nq, y.data(), 1, nullptr));
+        ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(4 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
+        ck(hemm_tensor_batch(c->dev, t.data(), t.data() + cnt * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
                              first == 0 ? 0 : 1, nullptr));
     }
     Ciphertext out(c);
@@ -405,7 +489,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     acc.allocate(3, T + 1, 1);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), extA, pbA, sa, first, cnt, ya.data(), t1.data(), ws.data());
+        assembleShifts(eval, a.get().getLevel(), extA.data(), pbA.data(), sa, first, cnt, ya.data(), t1.data(), ws.data());
         // row shifts are exact rotations here: one unmasked hoisted term each, plain ModDown
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
@@ -449,7 +533,7 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     DeviceBuffer y(c, G * 2 * E * N), t(c, G * 2 * lo * N), ws(c, G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get(), ext, pb, sa, first, cnt, y.data(), t.data(), ws.data());
+        assembleShifts(eval, a.get().getLevel(), ext.data(), pb.data(), sa, first, cnt, y.data(), t.data(), ws.data());
         for (size_t q = 0; q < cnt; q++) {
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);
