@@ -339,6 +339,18 @@ void assembleShifts(const HomEvaluator &eval, u64 src_level, const u64 *ext, con
     ck(hemm_moddown_batch(c->dev, y, (uint32_t)nq, (uint32_t)(2 * count), 1, out, (nq - 1) * N, ws, nullptr));
 }
 
+// levelDown by one level of n_polys polynomials [n_polys][level+1][N] -> [n_polys][level][N]:
+// multiply by round(Delta_{level-1} q_level / Delta_level), rescale (HomEvaluator::levelDown on a batch)
+void levelDownOneBatch(const Context &c, const u64 *in, size_t n_polys, u64 level, u64 *out) {
+    const u64 nq = level + 1, N = c->N;
+    const i64 v = (i64)llround(c->delta[level - 1] * (Real)c->q[level] / c->delta[level]);
+    std::vector<u64> sc(nq);
+    for (u64 j = 0; j < nq; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
+    DeviceBuffer t(c, n_polys * nq * N);
+    ck(hemm_mul_scalar(c->dev, in, nq * N, sc.data(), t.data(), nq * N, (uint32_t)nq, 0, (uint32_t)n_polys, nullptr));
+    ck(hemm_rescale(c->dev, t.data(), nq * N, out, (nq - 1) * N, (uint32_t)nq, (uint32_t)n_polys, nullptr));
+}
+
 template <class T1, class T2>
 i64 commonInside(const HETensor<T1> &a, const HETensor<T2> &b) {
     if (a.getWidth() != b.getHeight()) throw std::invalid_argument("[getCommonInsideLength] different inside length.");
@@ -385,14 +397,23 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         const TileTensorShape shapes[2] = {a.getShape(), b.getShape()};
         tr.diagonalTransformBatch(eval, joint.data(), 2, T + 3, kinds, shapes, ab.data());
     }
-    a.get().allocate(2, T + 2, 0);
-    b.get().allocate(2, T + 2, 0);
-    (void)hipMemcpyAsync(a.get().buf_.data(), ab.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
-    (void)hipMemcpyAsync(b.get().buf_.data(), ab.data() + ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
-
+    // the k = 0 term sigma(A) (x) tau(B) joins the accumulator at the shifts' level T+1
+    Ciphertext acc(c);
+    acc.allocate(3, T + 1, 1);
+    {
+        DeviceBuffer low(c, 2 * 2 * lo * N);
+        levelDownOneBatch(c, ab.data(), 4, T + 2, low.data());
+        ck(hemm_tensor_batch(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
+    }
     CtxtTensor res(c, rows, cols, w);
-    eval.mult(a.get(), b.get(), res.get());  // k = 0 term, level T+1
-    if (k == 1) return res;
+    auto finish = [&]() {
+        eval.relinearize(acc, res.get());
+        eval.rescale(res.get());
+    };
+    if (k == 1) {
+        finish();
+        return res;
+    }
 
     const i64 n = k;
     std::vector<Shift> sa, sb;
@@ -418,8 +439,6 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     const u64 *pbA = pbAB.data(), *pbB = pbAB.data() + nq * N;
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
-    Ciphertext acc(c);
-    acc.allocate(3, T + 1, 1);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     for (size_t first = 0; first < sa.size(); first += G) {
@@ -439,12 +458,9 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)(2 * cnt), (uint32_t)nq, y.data(), 1, nullptr));
         ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(4 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
         ck(hemm_tensor_batch(c->dev, t.data(), t.data() + cnt * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
-                             first == 0 ? 0 : 1, nullptr));
+                             1, nullptr));
     }
-    Ciphertext out(c);
-    eval.relinearize(acc, out);
-    eval.rescale(out);
-    eval.add(res.get(), out, res.get());
+    finish();
     return res;
 }
 
@@ -469,15 +485,29 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     eval.levelDown(b.get(), T + 2, b.get());
     a.get() = tr.diagonalTransformFused(eval, a.get(), MaskKind::PackedHorizontal, a.getShape());  // T+2
     b.get() = tr.diagonalTransformFused(eval, b.get(), MaskKind::PackedVertical, b.getShape());    // T+1
+    const u64 nqa = T + 3, nqb = T + 2, N = c->N, K = c->nP, lo = T + 2;  // both sides end at T+1 (lo limbs)
+    // the k = 0 term joins the accumulator at level T+1: sigma(A) lowered one level, tau(B) as it is
+    Ciphertext acc(c);
+    acc.allocate(3, T + 1, 1);
+    {
+        DeviceBuffer low(c, 2 * lo * N);
+        levelDownOneBatch(c, a.get().buf_.data(), 2, T + 2, low.data());
+        ck(hemm_tensor_batch(c->dev, low.data(), b.get().buf_.data(), 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
+    }
     CtxtTensor res(c, rows, cols, w);
-    eval.mult(a.get(), b.get(), res.get());  // level T
-    if (k / 2 <= 1) return res;
+    auto finish = [&]() {
+        eval.relinearize(acc, res.get());
+        eval.rescale(res.get());
+    };
+    if (k / 2 <= 1) {
+        finish();
+        return res;
+    }
 
     const i64 n = k;
     std::vector<Shift> sa;
     for (i64 i = 1; i < n / 2; i++)
         sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], 2 * i - n, &cm[(size_t)(4 * i)], true});
-    const u64 nqa = T + 3, nqb = T + 2, N = c->N, K = c->nP, lo = T + 2;  // both sides end at T+1 (lo limbs)
     DeviceBuffer extA = modUpOne(c, a.get()), extB = modUpOne(c, b.get());
     DeviceBuffer pbA = timesP(c, a.get().getPolyData(0), nqa), pbB = timesP(c, b.get().getPolyData(0), nqb);
     const KeyPack &pack = eval.getKeyPack();
@@ -485,8 +515,6 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
     DeviceBuffer ya(c, G * 2 * (nqa + K) * N), yb(c, G * 2 * (nqb + K) * N), t1(c, G * 2 * lo * N), t2(c, G * 2 * lo * N),
         ws(c, G * 2 * lo * N);
-    Ciphertext acc(c);
-    acc.allocate(3, T + 1, 1);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
         assembleShifts(eval, a.get().getLevel(), extA.data(), pbA.data(), sa, first, cnt, ya.data(), t1.data(), ws.data());
@@ -500,13 +528,9 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
         ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, yb.data(), 1, nullptr));
         ck(hemm_moddown_batch(c->dev, yb.data(), (uint32_t)nqb, (uint32_t)(2 * cnt), 0, t2.data(), lo * N, ws.data(),
                               nullptr));
-        ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
-                             first == 0 ? 0 : 1, nullptr));
+        ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(), 1, nullptr));
     }
-    Ciphertext out(c);
-    eval.relinearize(acc, out);
-    eval.rescale(out);
-    eval.add(res.get(), out, res.get());
+    finish();
     return res;
 }
 

@@ -562,16 +562,14 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
     rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
     a = diagonal_transform_fused(orc, a, H, n, w)
     b = diagonal_transform_fused(orc, b, V, n, w)
-    res = ev.mult(a, b)
+    # the k = 0 term joins the accumulator at the shifts' level
+    acc = orc.tensor(orc.level_down_one(a), orc.level_down_one(b))
     ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
     ta = _assemble_shifts(orc, a, ext_a, [(i, cm[2 * i + 1], i - n, cm[2 * i]) for i in range(1, n)])
     tb = _assemble_shifts(orc, b, ext_b, [(i * w, rm[2 * i + 1], (i - n) * w, rm[2 * i]) for i in range(1, n)])
-    acc = None
     for x, y in zip(ta, tb):
-        t = orc.tensor(x, y)
-        acc = t if acc is None else orc.add(acc, t)
-    out = orc.rescale(orc.relinearize(acc))
-    return ev.add(res, out)
+        acc = orc.add(acc, orc.tensor(x, y))
+    return orc.rescale(orc.relinearize(acc))
 
 
 def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
@@ -582,16 +580,14 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     b = orc.level_down(b, T + 2)
     a = diagonal_transform_fused(orc, a, PH, n, w)
     b = diagonal_transform_fused(orc, b, PV, n, w)
-    res = ev.mult(a, b)
+    # the k = 0 term joins the accumulator at the shifts' level
+    acc = orc.tensor(orc.level_down_one(a), b)
     ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
     ta = _assemble_shifts(orc, a, ext_a, [(2 * i, cm[4 * i + 1], 2 * i - n, cm[4 * i]) for i in range(1, n // 2)])
-    acc = None
     for i, x in zip(range(1, n // 2), ta):
         y = orc.hoisted_sum([(ext_b, b.data[0], (2 * i * w) % orc.slots, None)], b.nq)
-        t = orc.tensor(x, Ct(orc.moddown_drop(y, b.nq, False), b.scale))
-        acc = t if acc is None else orc.add(acc, t)
-    out = orc.rescale(orc.relinearize(acc))
-    return ev.add(res, out)
+        acc = orc.add(acc, orc.tensor(x, Ct(orc.moddown_drop(y, b.nq, False), b.scale)))
+    return orc.rescale(orc.relinearize(acc))
 
 
 def mult_mat_mat_pre_fused(orc, a, T, n, w):
