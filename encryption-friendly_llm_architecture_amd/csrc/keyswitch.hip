@@ -280,10 +280,10 @@ struct LinTermDev {
 // out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j], p < n_polys (<= 3).  A thread owns one
 // (limb, coefficient) for every polynomial, so each mask residue is read once; products are summed as
 // 128-bit values and reduced every 4 terms.
+template <int n_polys>
 __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
                                                          const u32 *__restrict__ group_off, u64 *__restrict__ out,
-                                                         const ModQ *__restrict__ modq, int nq, int n_polys, int logN,
-                                                         int n_out) {
+                                                         const ModQ *__restrict__ modq, int nq, int logN, int n_out) {
     // Workgroups go round-robin over the 8 XCDs, each with its own L2.  The outputs of one launch mostly
     // sum the same ciphertexts under different masks, so all outputs of a (limb, 256-coefficient) tile are
     // placed back to back on one XCD: the ciphertext tile is fetched from HBM once instead of once per output.
@@ -301,27 +301,40 @@ __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__res
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN;
     const size_t e = (size_t)j * N + (size_t)(tile & ((1u << (logN - 8)) - 1)) * 256 + threadIdx.x;
-    u64 acc[3] = {0, 0, 0};
-    u128_t lazy[3] = {{0, 0}, {0, 0}, {0, 0}};
+    u64 acc[n_polys];
+    u128_t lazy[n_polys];
+#pragma unroll
+    for (int p = 0; p < n_polys; p++) {
+        acc[p] = 0;
+        lazy[p].lo = lazy[p].hi = 0;
+    }
     int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const LinTermDev T = terms[t];
         if (T.mask != nullptr) {
             const u64 mk = T.galois ? T.mask[(size_t)j * N + galois_index((u32)(e - (size_t)j * N), (u32)T.galois, logN)]
                                     : T.mask[e];
+            
+#pragma unroll
             for (int p = 0; p < n_polys; p++) add128(lazy[p], mul64wide(T.ct[p * T.stride + e], mk));
             if (++pending == 4) {
-                for (int p = 0; p < n_polys; p++) {
+                
+#pragma unroll
+            for (int p = 0; p < n_polys; p++) {
                     acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
                     lazy[p].lo = lazy[p].hi = 0;
                 }
                 pending = 0;
             }
         } else {
+            
+#pragma unroll
             for (int p = 0; p < n_polys; p++) acc[p] = addmod(acc[p], T.ct[p * T.stride + e], m.q);
         }
     }
-    for (int p = 0; p < n_polys; p++) {
+    
+#pragma unroll
+            for (int p = 0; p < n_polys; p++) {
         if (pending) acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
         out[((size_t)o * n_polys + p) * nq * N + e] = acc[p];
     }
@@ -770,8 +783,13 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
                        u64 *out, hipStream_t s) {
     if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
     dim3 grid((unsigned)(c->N / 256) * nq * n_out), block(256);
-    hipLaunchKernelGGL(masked_sum_kernel, grid, block, 0, s, (const LinTermDev *)terms_dev, group_off_dev, out,
-                       c->d_modq, nq, n_polys, c->logN, n_out);
+    const LinTermDev *td = (const LinTermDev *)terms_dev;
+    if (n_polys == 1)
+        hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
+    else if (n_polys == 2)
+        hipLaunchKernelGGL(masked_sum_kernel<2>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
+    else
+        hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
 }
 
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
