@@ -3,11 +3,14 @@
 
 Headline (the metric BASELINE.json names): ms per 128 x 128 ciphertext-ciphertext matrix product
 (HEMMer::singleCCMatMul, N = 2^16, 13 + 4 primes, dnum 3, scale 2^42, inputs fresh at level 12,
-target level 4), inputs and keys resident in HBM.  Also reported in the same JSON line: batched
-NTT limb-transforms/s (32 polys x 24 limbs x 2^16, 60-bit primes), one key-switched rotation at
-level 12, the roofline of the NTT kernels (HBM bound) and the CPU oracle timed on the host cores.
+target level 4), inputs and keys resident in HBM.  Also reported in the same JSON line: one
+key-switched rotation at levels 12 and 6, batched NTT limb-transforms/s, the roofline of the
+dominant kernel (the hoisted key-switch inner product, HBM bound) and of the NTT launch pair, and
+the CPU oracle timed on the host cores.
 
 A "step" is one full CCMM.  Everything runs on one GPU; --gpus above 1 is refused.
+--roofline-only runs just the roofline legs (used for the committed rocprofv3 summaries, so that a
+kernel's average in the profile is the average of exactly the launches timed here).
 """
 import argparse
 import json
@@ -74,44 +77,112 @@ def gpu_ntt(args, out):
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
-    qs = pkg.primes_below(60, 16, 24)
-    ctx = pkg.Context(16, qs, [], 1)
-    q_t = torch.tensor(qs, dtype=torch.int64, device="cuda").view(1, 24, 1)
-    g = torch.Generator(device="cuda").manual_seed(7)
-    d = torch.randint(0, 2 ** 62, (32, 24, 1 << 16), dtype=torch.int64, device="cuda", generator=g) % q_t
-    ref = d.clone()
-    idx = list(range(24))
-    for _ in range(3):
-        ctx.ntt(d, idx)
-        ctx.ntt(d, idx, inverse=True)
-    torch.cuda.synchronize()
-    assert torch.equal(d, ref), "NTT round trip is not bit-exact"
-    timer = pkg.Timer()
-    iters = 20
-    timer.start()
-    for _ in range(iters):
-        ctx.ntt(d, idx)
-    fwd_ms = timer.stop() / iters
-    timer.start()
-    for _ in range(iters):
-        ctx.ntt(d, idx, inverse=True)
-    inv_ms = timer.stop() / iters
     limbs = 32 * 24
+    res = {}
+    for bits in (60, 42):
+        qs = pkg.primes_below(bits, 16, 24)
+        ctx = pkg.Context(16, qs, [], 1)
+        q_t = torch.tensor(qs, dtype=torch.int64, device="cuda").view(1, 24, 1)
+        g = torch.Generator(device="cuda").manual_seed(7)
+        d = torch.randint(0, 2 ** 62, (32, 24, 1 << 16), dtype=torch.int64, device="cuda", generator=g) % q_t
+        ref = d.clone()
+        idx = list(range(24))
+        for _ in range(3):
+            ctx.ntt(d, idx)
+            ctx.ntt(d, idx, inverse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(d, ref), "NTT round trip is not bit-exact"
+        timer = pkg.Timer()
+        iters = 20
+        timer.start()
+        for _ in range(iters):
+            ctx.ntt(d, idx)
+        fwd_ms = timer.stop() / iters
+        timer.start()
+        for _ in range(iters):
+            ctx.ntt(d, idx, inverse=True)
+        inv_ms = timer.stop() / iters
+        res[bits] = (fwd_ms, inv_ms)
+        del ctx, d, ref
+    fwd_ms, inv_ms = res[60]
     out["ntt_forward_limbs_per_s"] = limbs / fwd_ms * 1e3
     out["ntt_inverse_limbs_per_s"] = limbs / inv_ms * 1e3
     out["ntt_limbs_per_s"] = 2 * limbs / (fwd_ms + inv_ms) * 1e3
-    # roofline of the dominant kernel family: one forward transform of the batch = one launch of
-    # ntt16_cols_kernel + one of ntt16_rows_kernel; algorithmic traffic = read + write of every limb
-    # once = 1 MiB per limb-transform
+    out["ntt_limbs_per_s_42bit_primes"] = 2 * limbs / (res[42][0] + res[42][1]) * 1e3
+    # one forward transform of the batch = one launch of ntt16_cols_kernel + one of ntt16_rows_kernel;
+    # algorithmic traffic = read + write of every limb once = 1 MiB per limb-transform (each of the two
+    # launches moves that much, so the pair cannot exceed half of the HBM roofline on this figure)
     alg_bytes = limbs * 2 * LIMB_BYTES
-    achieved = alg_bytes / (fwd_ms * 1e-3) / 1e9
-    out["roofline"] = {
+    out["roofline_ntt"] = {
         "kernel": "ntt16_cols_kernel<false> + ntt16_rows_kernel<false> (one forward transform of "
-                  "32x24 limbs = 2 launches)",
-        "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                  "32x24 limbs = 2 launches), 60-bit primes / 42-bit primes",
+        "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "achieved": alg_bytes / (fwd_ms * 1e-3) / 1e9, "frac": alg_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "achieved_42bit": alg_bytes / (res[42][0] * 1e-3) / 1e9,
+        "frac_42bit": alg_bytes / (res[42][0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_launch_pair": alg_bytes, "avg_ms_per_launch_pair": fwd_ms,
+        "avg_ms_per_launch_pair_42bit": res[42][0],
     }
+
+
+# HBM bytes per launch of hoisted_terms_kernel at the shape below, from two rocprofv3 --pmc runs of
+# `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
+# 1 GiB copy this mode also launches; None until measured.
+HOISTED_TRAFFIC_BYTES = None
+
+
+def gpu_hoisted(args, out):
+    """Roofline of the dominant kernel, hoisted_terms_kernel, at the shape of the CCMM's main loop: one
+    launch produces 16 column shifts of sigma(A) and 16 row shifts of tau(B) in the extended basis, each
+    the sum of two masked hoisted rotations (7 chain + 4 special limbs, 2 digits)."""
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    nq, K, dnum, n_out = 7, 4, 3, 32
+    big = pkg.primes_below(60, 16, 1 + K)
+    qs = [big[0]] + pkg.primes_below(42, 16, 12)
+    ps = big[1:]
+    ctx = pkg.Context(16, qs, ps, dnum)
+    N, E, T, beta = 1 << 16, nq + K, 13 + K, 2
+    g = torch.Generator(device="cuda").manual_seed(11)
+
+    def rnd(*shape):
+        # residues below 2^41 are valid for every prime of the set; the kernel's work does not depend on values
+        return torch.randint(0, 2 ** 41, shape, dtype=torch.int64, device="cuda", generator=g)
+
+    src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(2)]
+    groups = []
+    for o in range(n_out):
+        ext, pb = src[o // (n_out // 2)]
+        groups.append([(ext, pb, rnd(dnum, 2, T, N), rnd(E, N), 5 ** (2 * o + t + 1) % (2 * N)) for t in range(2)])
+    for _ in range(2):
+        ctx.hoisted_terms(groups, nq, b_premultiplied=True)
+    torch.cuda.synchronize()
+    timer = pkg.Timer()
+    iters = 10
+    timer.start()
+    for _ in range(iters):
+        ctx.hoisted_terms(groups, nq, b_premultiplied=True)
+    ms = timer.stop() / iters
+    # algorithmic bytes: per output 2 terms x (beta x 2 x E key limbs + E mask limbs) read + 2 x E limbs
+    # written; the two rotation sources (beta x E + nq limbs each) read once per launch
+    limbs = n_out * (2 * (beta * 2 * E + E) + 2 * E) + 2 * (beta * E + nq)
+    alg_bytes = limbs * LIMB_BYTES
+    achieved = alg_bytes / (ms * 1e-3) / 1e9
+    out["roofline"] = {
+        "kernel": "hoisted_terms_kernel (32 outputs x 2 masked rotation terms, 7+4 limbs, 2 digits: one "
+                  "batch of the CCMM main loop)",
+        "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS, "traffic": HOISTED_TRAFFIC_BYTES,
+        "algorithmic_bytes_per_launch": alg_bytes, "avg_ms_per_launch": ms,
+    }
+    if args.roofline_only:
+        # a plain copy of known size in the same process: the scale reference for the --pmc counters
+        a = torch.empty(1 << 27, dtype=torch.int64, device="cuda").fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(4):
+            b.copy_(a)
+        torch.cuda.synchronize()
 
 
 def cpu_baseline(out, budget_s=25.0):
@@ -167,6 +238,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--roofline-only", action="store_true", help="run only the roofline legs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run it with --gpus 1 "
@@ -184,7 +256,13 @@ def main():
                                "+ 4 special 60-bit primes, dnum=3, scale 2^42, inputs fresh at level 12, "
                                "target level 4, all keys and masks resident in HBM"},
     }
+    if args.roofline_only:
+        gpu_hoisted(args, out)
+        gpu_ntt(args, out)
+        print(json.dumps(out))
+        return
     gpu_ccmm(args, out)
+    gpu_hoisted(args, out)
     gpu_ntt(args, out)
     if not args.no_cpu:
         cpu_baseline(out)

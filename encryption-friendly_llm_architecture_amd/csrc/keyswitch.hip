@@ -188,6 +188,20 @@ struct RotTermDev {
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
+// 16-byte accesses to data that is touched once per launch (keys, masks, results): marked non-temporal so
+// they do not push the rotation sources, which every output gathers from, out of the L2.
+typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ ulonglong2 stream_load2(const u64 *p) {
+    const u64x2 v = __builtin_nontemporal_load((const u64x2 *)p);
+    return make_ulonglong2(v.x, v.y);
+}
+__device__ __forceinline__ void stream_store2(u64 *p, u64 a, u64 b) {
+    u64x2 v;
+    v.x = a;
+    v.y = b;
+    __builtin_nontemporal_store(v, (u64x2 *)p);
+}
+
 __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
@@ -217,8 +231,8 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
                 x.x = x.y;
                 x.y = tmp;
             }
-            const ulonglong2 kb = *(const ulonglong2 *)(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-            const ulonglong2 ka = *(const ulonglong2 *)(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+            const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
+            const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
             add128(sb[0], mul64wide(x.x, kb.x));
             add128(sb[1], mul64wide(x.y, kb.y));
             add128(sa[0], mul64wide(x.x, ka.x));
@@ -241,7 +255,7 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
             rb[1] = addmod(rb[1], bv.y, m.q);
         }
         if (T.mask != nullptr) {
-            const ulonglong2 mk = *(const ulonglong2 *)(T.mask + (size_t)j * N + n);
+            const ulonglong2 mk = stream_load2(T.mask + (size_t)j * N + n);
             add128(lazy_b[0], mul64wide(rb[0], mk.x));
             add128(lazy_b[1], mul64wide(rb[1], mk.y));
             add128(lazy_a[0], mul64wide(ra[0], mk.x));
@@ -267,8 +281,8 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
             acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
         }
     }
-    *(ulonglong2 *)(y + (((size_t)o * 2 + 0) * E + j) * N + n) = make_ulonglong2(acc_b[0], acc_b[1]);
-    *(ulonglong2 *)(y + (((size_t)o * 2 + 1) * E + j) * N + n) = make_ulonglong2(acc_a[0], acc_a[1]);
+    stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, acc_b[0], acc_b[1]);
+    stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, acc_a[0], acc_a[1]);
 }
 
 struct LinTermDev {

@@ -388,10 +388,18 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
                                                          LimbList ll, LimbList sl, int n_limbs, size_t poly_stride,
                                                          NttEpilogue ep) {
     __shared__ u64 lds[16 * ROWPAD];
-    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    // The second radix-16 block of a row pass walks 1/16 of the prime's twiddle table per 16-row slab (as
+    // many bytes as the slab's data), identical for every polynomial of the batch.  Workgroups are dealt
+    // round-robin to the 8 XCDs, so the polynomials of one (limb, slab) pair are placed back to back on
+    // one XCD and share those twiddles through its L2 instead of fetching them from HBM once each.
+    const u32 n_polys = gridDim.x / (16u * (u32)n_limbs);
+    const u32 xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const u32 poly = slot % n_polys, group = (slot / n_polys) * 8u + xcd;
+    const int limb = (int)(group >> 4);
+    const u32 slab = group & 15u;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
-    const u32 r = blockIdx.x * 16 + (threadIdx.x >> 4);  // global row
+    const u32 r = slab * 16 + (threadIdx.x >> 4);  // global row
     u64 *row = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     const u64 *mn = nullptr;
     u64 *o = nullptr;
@@ -427,7 +435,7 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
     hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ll,
                        sl, n_limbs, poly_stride);
     (void)none;
-    hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl, n_limbs,
+    hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl, n_limbs,
                        poly_stride, ep);
     return true;
 }
@@ -442,10 +450,10 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
         if (!inverse) {
             hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
                                c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
-            hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
+            hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
                                n_limbs, poly_stride, NttEpilogue{});
         } else {
-            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), grid, block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
+            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
                                n_limbs, poly_stride, NttEpilogue{});
             hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
                                c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
