@@ -293,16 +293,33 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     struct Dev {
         const u64 *ext, *b, *evk, *mask;
         u32 galois, pad;
+        const u64 *ext2, *b2, *mask2;
     };
-    std::vector<Dev> d(n_terms);
-    for (uint32_t t = 0; t < n_terms; t++) {
-        need(terms[t].ext && terms[t].b && terms[t].evk, "null pointer in a rotation term");
-        need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
-        d[t] = Dev{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
-                   (const u64 *)terms[t].mask, (u32)terms[t].galois, 0};
+    // Consecutive masked terms of a group that use the same key and Galois element are merged into one
+    // two-source term: the kernel then streams that key once for both.
+    std::vector<Dev> d;
+    std::vector<uint32_t> off{0};
+    d.reserve(n_terms);
+    for (uint32_t o = 0; o < n_out; o++) {
+        need(group_offsets[o + 1] >= group_offsets[o], "group offsets must not decrease");
+        for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
+            need(terms[t].ext && terms[t].b && terms[t].evk, "null pointer in a rotation term");
+            need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
+            Dev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
+                    (const u64 *)terms[t].mask, (u32)terms[t].galois, 0, nullptr, nullptr, nullptr};
+            if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t + 1].ext && terms[t + 1].b &&
+                terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois) {
+                cur.ext2 = (const u64 *)terms[t + 1].ext;
+                cur.b2 = (const u64 *)terms[t + 1].b;
+                cur.mask2 = (const u64 *)terms[t + 1].mask;
+                t++;
+            }
+            d.push_back(cur);
+        }
+        off.push_back((uint32_t)d.size());
     }
     void *off_dev = nullptr;
-    void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), group_offsets, (n_out + 1) * sizeof(uint32_t),
+    void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), off.data(), (n_out + 1) * sizeof(uint32_t),
                                   &off_dev, (hipStream_t)stream);
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
                          (hipStream_t)stream);

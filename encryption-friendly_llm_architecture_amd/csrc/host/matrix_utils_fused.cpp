@@ -74,27 +74,6 @@ hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois
     return t;
 }
 
-// P * b of a ciphertext's b-polynomial (limb j times P mod q_j), computed once per rotation source
-DeviceBuffer timesP(const Context &c, const u64 *b, u64 nq) {
-    DeviceBuffer out(c, nq * c->N);
-    std::vector<u64> sc(nq);
-    for (u64 j = 0; j < nq; j++) {
-        u64 P = 1;
-        for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
-        sc[j] = P;
-    }
-    ck(hemm_mul_scalar(c->dev, b, 0, sc.data(), out.data(), 0, (uint32_t)nq, 0, 1, nullptr));
-    return out;
-}
-
-// ModUp of the a-polynomial of one ciphertext
-DeviceBuffer modUpOne(const Context &c, const Ciphertext &ct) {
-    const u64 nq = ct.level_ + 1, E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha;
-    DeviceBuffer ext(c, beta * E * c->N), ws(c, nq * c->N);
-    ck(hemm_modup_batch(c->dev, ct.getPolyData(1), ct.polyStride(), (uint32_t)nq, 1, ext.data(), ws.data(), nullptr));
-    return ext;
-}
-
 }  // namespace
 
 std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
@@ -151,13 +130,11 @@ std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, boo
     std::vector<u64> r;
     auto left = [&](i64 v) { r.push_back((u64)(((v % slots) + slots) % slots)); };
     const i64 stride = packed ? 2 : 1, count = packed ? n / 2 : n;
+    left(-n);
+    if (need_rows && !packed) left(-n * w);
     for (i64 i = 1; i < count; i++) {
         left(stride * i);
-        left(stride * i - n);
-        if (need_rows) {
-            left(stride * i * w);
-            if (!packed) left((stride * i - n) * w);
-        }
+        if (need_rows) left(stride * i * w);
     }
     return r;
 }
@@ -311,32 +288,67 @@ Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, c
 
 namespace {
 
-// Shifts of `src` (level l, rescale counter 0): for every entry two hoisted rotations of src combined
-// with extended masks (second one optional), then ModDown merged with the rescale.  Output: entries.size()
-// ciphertexts [2][l][N] (level l-1) packed in `out`.
-struct Shift {
-    i64 rot1;
-    const Plaintext *mask1;
-    i64 rot2;
-    const Plaintext *mask2;  // nullptr: single-term shift
-    bool two;
+// Rotation sources in the form the hoisted launches read: ModUp of the a-polynomial and P * b of
+// n ciphertexts stored back to back ([n][2][nq][N]).
+struct Sources {
+    DeviceBuffer ext, pb;  // [n][beta][E][N], [n][nq][N]
+    u64 nq, ext_words;
+    const u64 *extOf(size_t q) const { return ext.data() + q * ext_words; }
+    const u64 *pbOf(size_t q) const { return pb.data() + q * nq * N_; }
+    u64 N_;
 };
-void assembleShifts(const HomEvaluator &eval, u64 src_level, const u64 *ext, const u64 *pb,
-                    const std::vector<Shift> &shifts, size_t first, size_t count, u64 *y, u64 *out, u64 *ws) {
+Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq) {
+    const u64 N = c->N, E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha, ctw = 2 * nq * N;
+    Sources s{DeviceBuffer(c, n * beta * E * N), DeviceBuffer(c, n * nq * N), nq, beta * E * N, N};
+    DeviceBuffer ws(c, n * nq * N);
+    ck(hemm_modup_batch(c->dev, cts + nq * N, ctw, (uint32_t)nq, (uint32_t)n, s.ext.data(), ws.data(), nullptr));
+    std::vector<u64> sc(nq);
+    for (u64 j = 0; j < nq; j++) {
+        u64 P = 1;
+        for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+        sc[j] = P;
+    }
+    ck(hemm_mul_scalar(c->dev, cts, ctw, sc.data(), s.pb.data(), nq * N, (uint32_t)nq, 0, (uint32_t)n, nullptr));
+    return s;
+}
+// The same sources rotated left by rots[q] slots, as ciphertexts [n][2][nq][N]: one hoisted launch and one
+// ModDown for all of them.
+DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, size_t n, const i64 *rots) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    const u64 nq = src_level + 1, N = c->N;
+    const u64 nq = src.nq, N = c->N, E = nq + c->nP;
     std::vector<hemm_rot_term> terms;
     std::vector<uint32_t> off{0};
-    for (size_t k = first; k < first + count; k++) {
-        const Shift &s = shifts[k];
-        terms.push_back(term(ext, pb, pack, rot.galois(s.rot1), s.mask1));
-        if (s.two) terms.push_back(term(ext, pb, pack, rot.galois(s.rot2), s.mask2));
+    for (size_t q = 0; q < n; q++) {
+        terms.push_back(term(src.extOf(q), src.pbOf(q), pack, rot.galois(rots[q]), nullptr));
         off.push_back((uint32_t)terms.size());
     }
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)count, (uint32_t)nq, y, 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, y, (uint32_t)nq, (uint32_t)(2 * count), 1, out, (nq - 1) * N, ws, nullptr));
+    DeviceBuffer y(c, n * 2 * E * N), ws(c, n * 2 * nq * N), out(c, n * 2 * nq * N);
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)n, (uint32_t)nq, y.data(), 1, nullptr));
+    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * n), 0, out.data(), nq * N, ws.data(), nullptr));
+    return out;
+}
+
+// A cyclic shift by r inside a tile of period n (columns: unit 1, rows: unit w) is
+//   main_mask * rot(X, r) + wrap_mask * rot(X, r - n unit)  =  main_mask * rot(X, r) + wrap_mask * rot(X', r)
+// with X' = rot(X, -n unit) prepared once: both halves then use the key of r, which is streamed once.
+struct Shift {
+    i64 rot;
+    const Plaintext *main_mask, *wrap_mask;
+};
+// terms of shifts[first, first + count) of source pair (x, x2) appended to `terms`
+void pushShifts(const HomEvaluator &eval, const Sources &x, size_t ix, const Sources &x2, size_t ix2,
+                const std::vector<Shift> &shifts, size_t first, size_t count, std::vector<hemm_rot_term> &terms,
+                std::vector<uint32_t> &off) {
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(eval.getContext());
+    for (size_t k = first; k < first + count; k++) {
+        const u64 g = rot.galois(shifts[k].rot);
+        terms.push_back(term(x.extOf(ix), x.pbOf(ix), pack, g, shifts[k].main_mask));
+        terms.push_back(term(x2.extOf(ix2), x2.pbOf(ix2), pack, g, shifts[k].wrap_mask));
+        off.push_back((uint32_t)terms.size());
+    }
 }
 
 // levelDown by one level of n_polys polynomials [n_polys][level+1][N] -> [n_polys][level][N]:
@@ -418,43 +430,23 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     const i64 n = k;
     std::vector<Shift> sa, sb;
     for (i64 i = 1; i < n; i++) {
-        sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], i - n, &cm[(size_t)(2 * i)], true});
-        sb.push_back(Shift{i * w, &rm[(size_t)(2 * i + 1)], (i - n) * w, &rm[(size_t)(2 * i)], true});
+        sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
+        sb.push_back(Shift{i * w, &rm[(size_t)(2 * i + 1)], &rm[(size_t)(2 * i)]});
     }
-    // ModUp and P * b of both rotation sources in one batch each
-    const u64 beta = (nq + c->alpha - 1) / c->alpha;
-    DeviceBuffer extAB(c, 2 * beta * E * N), pbAB(c, 2 * nq * N);
-    {
-        DeviceBuffer mws(c, 2 * nq * N);
-        ck(hemm_modup_batch(c->dev, ab.data() + nq * N, ctw, (uint32_t)nq, 2, extAB.data(), mws.data(), nullptr));
-        std::vector<u64> sc(nq);
-        for (u64 j = 0; j < nq; j++) {
-            u64 P = 1;
-            for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
-            sc[j] = P;
-        }
-        ck(hemm_mul_scalar(c->dev, ab.data(), ctw, sc.data(), pbAB.data(), nq * N, (uint32_t)nq, 0, 2, nullptr));
-    }
-    const u64 *extA = extAB.data(), *extB = extAB.data() + beta * E * N;
-    const u64 *pbA = pbAB.data(), *pbB = pbAB.data() + nq * N;
+    // rotation sources: sigma(A), tau(B) and their copies rotated by -n columns / -n rows
+    const Sources x = extendSources(c, ab.data(), 2, nq);
+    const i64 back[2] = {-n, -n * w};
+    const DeviceBuffer ab2 = rotateSources(eval, x, 2, back);
+    const Sources x2 = extendSources(c, ab2.data(), 2, nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
-    const KeyPack &pack = eval.getKeyPack();
-    const Rot rot(c);
     for (size_t first = 0; first < sa.size(); first += G) {
         // cnt column shifts of sigma(A), then cnt row shifts of tau(B): one launch chain for all 2 cnt outputs
         const size_t cnt = std::min(G, sa.size() - first);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
-        for (int side = 0; side < 2; side++) {
-            const std::vector<Shift> &sh = side ? sb : sa;
-            const u64 *ext = side ? extB : extA, *pb = side ? pbB : pbA;
-            for (size_t q = first; q < first + cnt; q++) {
-                terms.push_back(term(ext, pb, pack, rot.galois(sh[q].rot1), sh[q].mask1));
-                terms.push_back(term(ext, pb, pack, rot.galois(sh[q].rot2), sh[q].mask2));
-                off.push_back((uint32_t)terms.size());
-            }
-        }
+        pushShifts(eval, x, 0, x2, 0, sa, first, cnt, terms, off);
+        pushShifts(eval, x, 1, x2, 1, sb, first, cnt, terms, off);
         ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)(2 * cnt), (uint32_t)nq, y.data(), 1, nullptr));
         ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(4 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
         ck(hemm_tensor_batch(c->dev, t.data(), t.data() + cnt * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
@@ -506,10 +498,13 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
 
     const i64 n = k;
     std::vector<Shift> sa;
-    for (i64 i = 1; i < n / 2; i++)
-        sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], 2 * i - n, &cm[(size_t)(4 * i)], true});
-    DeviceBuffer extA = modUpOne(c, a.get()), extB = modUpOne(c, b.get());
-    DeviceBuffer pbA = timesP(c, a.get().getPolyData(0), nqa), pbB = timesP(c, b.get().getPolyData(0), nqb);
+    for (i64 i = 1; i < n / 2; i++) sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], &cm[(size_t)(4 * i)]});
+    // rotation sources: sigma(A), its copy rotated by -n columns, and tau(B)
+    const Sources xa = extendSources(c, a.get().buf_.data(), 1, nqa);
+    const i64 back = -n;
+    const DeviceBuffer a2 = rotateSources(eval, xa, 1, &back);
+    const Sources xa2 = extendSources(c, a2.data(), 1, nqa);
+    const Sources xb = extendSources(c, b.get().buf_.data(), 1, nqb);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
@@ -517,12 +512,19 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
         ws(c, G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get().getLevel(), extA.data(), pbA.data(), sa, first, cnt, ya.data(), t1.data(), ws.data());
+        {
+            std::vector<hemm_rot_term> terms;
+            std::vector<uint32_t> off{0};
+            pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
+            ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqa, ya.data(), 1, nullptr));
+            ck(hemm_moddown_batch(c->dev, ya.data(), (uint32_t)nqa, (uint32_t)(2 * cnt), 1, t1.data(), lo * N, ws.data(),
+                                  nullptr));
+        }
         // row shifts are exact rotations here: one unmasked hoisted term each, plain ModDown
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         for (size_t q = first; q < first + cnt; q++) {
-            terms.push_back(term(extB.data(), pbB.data(), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
+            terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
             off.push_back((uint32_t)terms.size());
         }
         ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, yb.data(), 1, nullptr));
@@ -549,15 +551,21 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     eval.levelDownOne(a.get(), first_ct);
     tmp.push_back(first_ct);
     std::vector<Shift> sa;
-    for (i64 i = 1; i < n; i++) sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], i - n, &cm[(size_t)(2 * i)], true});
+    for (i64 i = 1; i < n; i++) sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
-    DeviceBuffer ext = modUpOne(c, a.get());
-    DeviceBuffer pb = timesP(c, a.get().getPolyData(0), nq);
+    const Sources x = extendSources(c, a.get().buf_.data(), 1, nq);
+    const i64 back = -n;
+    const DeviceBuffer a2 = rotateSources(eval, x, 1, &back);
+    const Sources x2 = extendSources(c, a2.data(), 1, nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
     DeviceBuffer y(c, G * 2 * E * N), t(c, G * 2 * lo * N), ws(c, G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {
         const size_t cnt = std::min(G, sa.size() - first);
-        assembleShifts(eval, a.get().getLevel(), ext.data(), pb.data(), sa, first, cnt, y.data(), t.data(), ws.data());
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        pushShifts(eval, x, 0, x2, 0, sa, first, cnt, terms, off);
+        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, y.data(), 1, nullptr));
+        ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
         for (size_t q = 0; q < cnt; q++) {
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);

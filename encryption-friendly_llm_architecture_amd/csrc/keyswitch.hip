@@ -181,6 +181,9 @@ struct RotTermDev {
     const u64 *evk;   // [dnum][2][nQ+K][N]
     const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
     u32 galois, pad;
+    // optional second source rotated by the same Galois element with the same key (ext2 == nullptr: none):
+    // the term is mask * rot(source) + mask2 * rot(source 2) and the key is read once for both
+    const u64 *ext2, *b2, *mask2;
 };
 
 // Hoisted rotations, several per output, combined with masks in the extended basis:
@@ -223,6 +226,63 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
         const u32 np = galois_index(n, T.galois, logN);
         const u32 base = np & ~1u;
         const bool swap = (np & 1u) != 0;
+        if (T.ext2 != nullptr) {
+            // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
+            const ulonglong2 m1 = stream_load2(T.mask + (size_t)j * N + n);
+            const ulonglong2 m2 = stream_load2(T.mask2 + (size_t)j * N + n);
+            u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
+            for (int d = 0; d < beta; d++) {
+                ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
+                ulonglong2 x2 = *(const ulonglong2 *)(T.ext2 + ((size_t)d * E + j) * N + base);
+                if (swap) {
+                    u64 tmp = x1.x;
+                    x1.x = x1.y;
+                    x1.y = tmp;
+                    tmp = x2.x;
+                    x2.x = x2.y;
+                    x2.y = tmp;
+                }
+                u128_t t0 = mul64wide(m1.x, x1.x), t1 = mul64wide(m1.y, x1.y);
+                add128(t0, mul64wide(m2.x, x2.x));
+                add128(t1, mul64wide(m2.y, x2.y));
+                const u64 z0 = barrett128(t0, m), z1 = barrett128(t1, m);
+                const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
+                const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+                add128(pb[0], mul64wide(z0, kb.x));
+                add128(pb[1], mul64wide(z1, kb.y));
+                add128(pa[0], mul64wide(z0, ka.x));
+                add128(pa[1], mul64wide(z1, ka.y));
+            }
+            u64 rb0 = barrett128(pb[0], m), rb1 = barrett128(pb[1], m);
+            if (j < nq) {
+                ulonglong2 b1 = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
+                ulonglong2 b2 = *(const ulonglong2 *)(T.b2 + (size_t)j * N + base);
+                if (swap) {
+                    u64 tmp = b1.x;
+                    b1.x = b1.y;
+                    b1.y = tmp;
+                    tmp = b2.x;
+                    b2.x = b2.y;
+                    b2.y = tmp;
+                }
+                if (!b_premultiplied) {
+                    b1.x = mul_shoup(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+                    b1.y = mul_shoup(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+                    b2.x = mul_shoup(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+                    b2.y = mul_shoup(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+                }
+                u128_t t0 = mul64wide(m1.x, b1.x), t1 = mul64wide(m1.y, b1.y);
+                add128(t0, mul64wide(m2.x, b2.x));
+                add128(t1, mul64wide(m2.y, b2.y));
+                rb0 = addmod(rb0, barrett128(t0, m), m.q);
+                rb1 = addmod(rb1, barrett128(t1, m), m.q);
+            }
+            acc_b[0] = addmod(acc_b[0], rb0, m.q);
+            acc_b[1] = addmod(acc_b[1], rb1, m.q);
+            acc_a[0] = addmod(acc_a[0], barrett128(pa[0], m), m.q);
+            acc_a[1] = addmod(acc_a[1], barrett128(pa[1], m), m.q);
+            continue;
+        }
         u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
         for (int d = 0; d < beta; d++) {
             ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);

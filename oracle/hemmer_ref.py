@@ -540,15 +540,24 @@ def diagonal_transform_fused(orc, ct, kind, n, w):
     return orc.rescale(res)
 
 
-def _assemble_shifts(orc, src, ext, shifts):
-    """shifts: (rot1, mask1_ext, rot2, mask2_ext) -> ciphertexts one level down."""
+def _rotated_copy(orc, src, ext, r):
+    """rot(src, r) with the automorphism after ModUp (one hoisted term, plain ModDown)."""
+    from .oracle import Ct
+    y = orc.hoisted_sum([(ext, src.data[0], r % orc.slots, None)], src.nq)
+    return Ct(orc.moddown_drop(y, src.nq, False), src.scale)
+
+
+def _assemble_shifts(orc, src, ext, back, shifts):
+    """Cyclic shifts inside a tile: main_mask * rot(src, r) + wrap_mask * rot(src2, r) with
+    src2 = rot(src, back) prepared once, so both halves use the key of r.
+    shifts: (r, main_mask_ext, wrap_mask_ext) -> ciphertexts one level down."""
     from .oracle import Ct
     nq = src.nq
+    src2 = _rotated_copy(orc, src, ext, back)
+    ext2 = orc.modup(src2.data[1])
     out = []
-    for r1, m1, r2, m2 in shifts:
-        terms = [(ext, src.data[0], r1 % orc.slots, m1)]
-        if m2 is not None:
-            terms.append((ext, src.data[0], r2 % orc.slots, m2))
+    for r, m_main, m_wrap in shifts:
+        terms = [(ext, src.data[0], r % orc.slots, m_main), (ext2, src2.data[0], r % orc.slots, m_wrap)]
         y = orc.hoisted_sum(terms, nq)
         out.append(Ct(orc.moddown_drop(y, nq, True), orc.delta[src.level - 1]))
     return out
@@ -565,8 +574,8 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), orc.level_down_one(b))
     ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
-    ta = _assemble_shifts(orc, a, ext_a, [(i, cm[2 * i + 1], i - n, cm[2 * i]) for i in range(1, n)])
-    tb = _assemble_shifts(orc, b, ext_b, [(i * w, rm[2 * i + 1], (i - n) * w, rm[2 * i]) for i in range(1, n)])
+    ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
+    tb = _assemble_shifts(orc, b, ext_b, -n * w, [(i * w, rm[2 * i + 1], rm[2 * i]) for i in range(1, n)])
     for x, y in zip(ta, tb):
         acc = orc.add(acc, orc.tensor(x, y))
     return orc.rescale(orc.relinearize(acc))
@@ -583,7 +592,7 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
     ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
-    ta = _assemble_shifts(orc, a, ext_a, [(2 * i, cm[4 * i + 1], 2 * i - n, cm[4 * i]) for i in range(1, n // 2)])
+    ta = _assemble_shifts(orc, a, ext_a, -n, [(2 * i, cm[4 * i + 1], cm[4 * i]) for i in range(1, n // 2)])
     for i, x in zip(range(1, n // 2), ta):
         y = orc.hoisted_sum([(ext_b, b.data[0], (2 * i * w) % orc.slots, None)], b.nq)
         acc = orc.add(acc, orc.tensor(x, Ct(orc.moddown_drop(y, b.nq, False), b.scale)))
@@ -596,7 +605,7 @@ def mult_mat_mat_pre_fused(orc, a, T, n, w):
     a = diagonal_transform_fused(orc, a, H, n, w)
     ext = orc.modup(a.data[1])
     return [orc.level_down_one(a)] + _assemble_shifts(
-        orc, a, ext, [(i, cm[2 * i + 1], i - n, cm[2 * i]) for i in range(1, n)])
+        orc, a, ext, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
 
 
 def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
