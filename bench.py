@@ -134,7 +134,8 @@ HOISTED_TRAFFIC_BYTES = None
 def gpu_hoisted(args, out):
     """Roofline of the dominant kernel, hoisted_terms_kernel, at the shape of the CCMM's main loop: one
     launch produces 16 column shifts of sigma(A) and 16 row shifts of tau(B) in the extended basis, each
-    the sum of two masked hoisted rotations (7 chain + 4 special limbs, 2 digits)."""
+    the sum of two masked hoisted rotations (of the operand and of its copy rotated by -n) under one
+    key (7 chain + 4 special limbs, 2 digits)."""
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -150,11 +151,12 @@ def gpu_hoisted(args, out):
         # residues below 2^41 are valid for every prime of the set; the kernel's work does not depend on values
         return torch.randint(0, 2 ** 41, shape, dtype=torch.int64, device="cuda", generator=g)
 
-    src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(2)]
+    src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(4)]
     groups = []
     for o in range(n_out):
-        ext, pb = src[o // (n_out // 2)]
-        groups.append([(ext, pb, rnd(dnum, 2, T, N), rnd(E, N), 5 ** (2 * o + t + 1) % (2 * N)) for t in range(2)])
+        side = o // (n_out // 2)
+        evk, gal = rnd(dnum, 2, T, N), pow(5, o + 1, 2 * N)
+        groups.append([(src[2 * side + t][0], src[2 * side + t][1], evk, rnd(E, N), gal) for t in range(2)])
     for _ in range(2):
         ctx.hoisted_terms(groups, nq, b_premultiplied=True)
     torch.cuda.synchronize()
@@ -164,14 +166,14 @@ def gpu_hoisted(args, out):
     for _ in range(iters):
         ctx.hoisted_terms(groups, nq, b_premultiplied=True)
     ms = timer.stop() / iters
-    # algorithmic bytes: per output 2 terms x (beta x 2 x E key limbs + E mask limbs) read + 2 x E limbs
-    # written; the two rotation sources (beta x E + nq limbs each) read once per launch
-    limbs = n_out * (2 * (beta * 2 * E + E) + 2 * E) + 2 * (beta * E + nq)
+    # algorithmic bytes: per output beta x 2 x E key limbs + 2 x E mask limbs read + 2 x E limbs written;
+    # the four rotation sources (beta x E + nq limbs each) read once per launch
+    limbs = n_out * (beta * 2 * E + 2 * E + 2 * E) + 4 * (beta * E + nq)
     alg_bytes = limbs * LIMB_BYTES
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     out["roofline"] = {
-        "kernel": "hoisted_terms_kernel (32 outputs x 2 masked rotation terms, 7+4 limbs, 2 digits: one "
-                  "batch of the CCMM main loop)",
+        "kernel": "hoisted_terms_kernel (32 outputs x 2 masked sources under one key, 7+4 limbs, 2 digits: "
+                  "one batch of the CCMM main loop)",
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS, "traffic": HOISTED_TRAFFIC_BYTES,
         "algorithmic_bytes_per_launch": alg_bytes, "avg_ms_per_launch": ms,

@@ -138,8 +138,9 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
             iwt[2 * j + 1] = fp ? as_bits((double)ipw[r] / (double)q) : h_shoup(ipw[r], q);
         }
         ninv[i] = h_invmod((u64)N, q);
-        fpc[4 * i + 0] = fp ? (double)q : 0.0;
-        fpc[4 * i + 1] = fp ? 1.0 / (double)q : 0.0;
+        const bool small = (q >> 44) == 0;  // residues and products-by-parts are exact in double precision
+        fpc[4 * i + 0] = small ? (double)q : 0.0;
+        fpc[4 * i + 1] = small ? 1.0 / (double)q : 0.0;
         fpc[4 * i + 2] = (double)ninv[i];
         fpc[4 * i + 3] = (double)ninv[i] / (double)q;
         ninv_s[i] = h_shoup(ninv[i], q);

@@ -29,8 +29,8 @@ struct hemm_context {
     u64 *d_iw, *d_iws;              // inverse-transform twiddles
     u64 *d_ninv, *d_ninv_s;         // [prime]
     ModQ *d_modq;                   // [prime]
-    double *d_fp;                   // [prime][4]: q, 1/q, 1/N mod q, that / q as doubles; q = 0 marks a prime
-                                    // whose transform uses the integer path
+    double *d_fp;                   // [prime][4]: q, 1/q, 1/N mod q, that / q as doubles; q = 0 marks a prime of
+                                    // 44 bits or more, which only the integer code paths handle
     u64 *d_imag, *d_imag_s;         // [prime] psi^(N/2) and Shoup quotient
     // scratch owned by the context (single stream use)
     u64 *d_scratch;

@@ -205,18 +205,11 @@ __device__ __forceinline__ void stream_store2(u64 *p, u64 a, u64 b) {
     __builtin_nontemporal_store(v, (u64x2 *)p);
 }
 
-__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
-                                                            const u32 *__restrict__ group_off, u64 *__restrict__ y,
-                                                            const ModQ *__restrict__ modq, LimbList ll, CstList pmod,
-                                                            int nq, int E, int beta, int n_full, int logN,
-                                                            int b_premultiplied) {
-    // blockIdx.x = output (fastest): workgroups that gather from the same source tile run back to back.
-    // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
-    // (possibly swapped), so every access is a 16-byte load or store.
-    const int j = blockIdx.z, o = blockIdx.x;
-    const int prime = ll.idx[j];
-    const ModQ m = modq[prime];
-    const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
+__device__ __forceinline__ void hoisted_terms_int(const RotTermDev *__restrict__ terms,
+                                                  const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                  const ModQ m, const CstList &pmod, const int j, const int o,
+                                                  const int prime, const u32 n, int nq, int E, int beta, int n_full,
+                                                  int logN, int b_premultiplied) {
     const size_t N = (size_t)1 << logN;
     u64 acc_b[2] = {0, 0}, acc_a[2] = {0, 0};
     u128_t lazy_b[2] = {{0, 0}, {0, 0}}, lazy_a[2] = {{0, 0}, {0, 0}};
@@ -343,6 +336,147 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
     }
     stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, acc_b[0], acc_b[1]);
     stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, acc_a[0], acc_a[1]);
+}
+
+// The same sums in double precision for primes below 2^44 (exact, see the transform kernels): a product
+// mod q is 6 FP64 operations instead of ~40 integer ones for a wide product plus its Barrett step.
+struct D2 {
+    double x, y;
+};
+__device__ __forceinline__ D2 to_d2(const ulonglong2 v) {
+    D2 r;
+    r.x = __longlong_as_double((long long)(v.x | 0x4330000000000000ull)) - 4503599627370496.0;
+    r.y = __longlong_as_double((long long)(v.y | 0x4330000000000000ull)) - 4503599627370496.0;
+    return r;
+}
+__device__ __forceinline__ D2 gather_d2(const u64 *p, const bool swap) {
+    ulonglong2 v = *(const ulonglong2 *)p;
+    if (swap) {
+        const u64 tmp = v.x;
+        v.x = v.y;
+        v.y = tmp;
+    }
+    return to_d2(v);
+}
+#pragma clang fp contract(off)
+struct FpMod {
+    double q, qinv;
+    // a * b mod q as a centred residue (|r| <= 0.54 q) for integers |a| < 2^48, |b| < 2^44
+    __device__ __forceinline__ double mul(double a, double b) const {
+        const double h = a * b;
+        const double l = __builtin_fma(a, b, -h);
+        const double c = __builtin_rint(h * qinv);
+        return __builtin_fma(-c, q, h) + l;
+    }
+    __device__ __forceinline__ double reduce(double x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
+    __device__ __forceinline__ u64 canonical(double x) const {
+        double r = reduce(x);
+        r += r < 0.0 ? q : 0.0;
+        return (u64)__double_as_longlong(r + 4503599627370496.0) & 0x000fffffffffffffull;
+    }
+};
+__device__ __forceinline__ void hoisted_terms_fp(const RotTermDev *__restrict__ terms,
+                                                 const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                 const FpMod f, const double p_mod_q, const int j, const int o,
+                                                 const int prime, const u32 n, int nq, int E, int beta, int n_full,
+                                                 int logN, int b_premultiplied) {
+    const size_t N = (size_t)1 << logN;
+    double acc_b0 = 0, acc_b1 = 0, acc_a0 = 0, acc_a1 = 0;
+    int since = 0;
+    for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
+        const RotTermDev T = terms[t];
+        const u32 np = galois_index(n, T.galois, logN);
+        const u32 base = np & ~1u;
+        const bool swap = (np & 1u) != 0;
+        double sb0 = 0, sb1 = 0, sa0 = 0, sa1 = 0;
+        if (T.ext2 != nullptr) {
+            const D2 m1 = to_d2(stream_load2(T.mask + (size_t)j * N + n));
+            const D2 m2 = to_d2(stream_load2(T.mask2 + (size_t)j * N + n));
+            for (int d = 0; d < beta; d++) {
+                const D2 x1 = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
+                const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
+                const double z0 = f.mul(m1.x, x1.x) + f.mul(m2.x, x2.x);
+                const double z1 = f.mul(m1.y, x1.y) + f.mul(m2.y, x2.y);
+                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
+                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
+                sb0 += f.mul(z0, kb.x);
+                sb1 += f.mul(z1, kb.y);
+                sa0 += f.mul(z0, ka.x);
+                sa1 += f.mul(z1, ka.y);
+            }
+            if (j < nq) {
+                D2 b1 = gather_d2(T.b + (size_t)j * N + base, swap);
+                D2 b2 = gather_d2(T.b2 + (size_t)j * N + base, swap);
+                if (!b_premultiplied) {
+                    b1.x = f.mul(b1.x, p_mod_q);
+                    b1.y = f.mul(b1.y, p_mod_q);
+                    b2.x = f.mul(b2.x, p_mod_q);
+                    b2.y = f.mul(b2.y, p_mod_q);
+                }
+                sb0 += f.mul(m1.x, b1.x) + f.mul(m2.x, b2.x);
+                sb1 += f.mul(m1.y, b1.y) + f.mul(m2.y, b2.y);
+            }
+        } else {
+            for (int d = 0; d < beta; d++) {
+                const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
+                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
+                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
+                sb0 += f.mul(x.x, kb.x);
+                sb1 += f.mul(x.y, kb.y);
+                sa0 += f.mul(x.x, ka.x);
+                sa1 += f.mul(x.y, ka.y);
+            }
+            if (j < nq) {
+                D2 bv = gather_d2(T.b + (size_t)j * N + base, swap);
+                if (!b_premultiplied) {
+                    bv.x = f.mul(bv.x, p_mod_q);
+                    bv.y = f.mul(bv.y, p_mod_q);
+                }
+                sb0 += bv.x;
+                sb1 += bv.y;
+            }
+            if (T.mask != nullptr) {
+                const D2 mk = to_d2(stream_load2(T.mask + (size_t)j * N + n));
+                sb0 = f.mul(sb0, mk.x);
+                sb1 = f.mul(sb1, mk.y);
+                sa0 = f.mul(sa0, mk.x);
+                sa1 = f.mul(sa1, mk.y);
+            }
+        }
+        acc_b0 += sb0;
+        acc_b1 += sb1;
+        acc_a0 += sa0;
+        acc_a1 += sa1;
+        if (++since == 8) {  // a term adds at most (beta + 2) * 0.54 q: keep the running sums far below 2^52
+            acc_b0 = f.reduce(acc_b0);
+            acc_b1 = f.reduce(acc_b1);
+            acc_a0 = f.reduce(acc_a0);
+            acc_a1 = f.reduce(acc_a1);
+            since = 0;
+        }
+    }
+    stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, f.canonical(acc_b0), f.canonical(acc_b1));
+    stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, f.canonical(acc_a0), f.canonical(acc_a1));
+}
+
+__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
+                                                            const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                            const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                            LimbList ll, CstList pmod, int nq, int E, int beta,
+                                                            int n_full, int logN, int b_premultiplied) {
+    // blockIdx.x = output (fastest): workgroups that gather from the same source tile run back to back.
+    // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
+    // (possibly swapped), so every access is a 16-byte load or store.
+    const int j = blockIdx.z, o = blockIdx.x;
+    const int prime = ll.idx[j];
+    const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
+    const double fq = fp[4 * prime];
+    if (fq != 0.0 && beta <= 6)
+        hoisted_terms_fp(terms, group_off, y, FpMod{fq, fp[4 * prime + 1]}, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime,
+                         n, nq, E, beta, n_full, logN, b_premultiplied);
+    else
+        hoisted_terms_int(terms, group_off, y, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN,
+                          b_premultiplied);
 }
 
 struct LinTermDev {
@@ -792,7 +926,7 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     }
     dim3 grid(n_out, c->N / 512, E), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
-                       c->d_modq, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
+                       c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
                        b_premultiplied ? 1 : 0);
 }
 

@@ -208,6 +208,20 @@ def test_batched_hoisted_forms(S):
             orc.hoisted_sum([(exts[2], cts[2][0], ("g", gc), None)], nq)]
     for k in range(3):
         assert np.array_equal(host(y[k]), want[k])
+    # two masked sources under one key (the kernel reads that key once for both), followed by a third
+    # term of another key in the same group
+    shared = [[(dext[0], dcts[0][0], dk[g1], dm1, g1), (dext[1], dcts[1][0], dk[g1], dm2, g1),
+               (dext[2], dcts[2][0], dk[g3], dm1, g3)]]
+    want_shared = orc.hoisted_sum([(exts[0], cts[0][0], ("g", g1), m1), (exts[1], cts[1][0], ("g", g1), m2),
+                                   (exts[2], cts[2][0], ("g", g3), m1)], nq)
+    assert np.array_equal(host(ctx.hoisted_terms(shared, nq)[0]), want_shared)
+    # the same with P * b supplied by the caller
+    Pq = [int(np.prod([int(p) for p in orc.p], dtype=object) % q) for q in mods]
+    pbs = [dev(np.stack([(c[0][j].astype(object) * Pq[j] % mods[j]).astype(np.uint64) for j in range(nq)]))
+           for c in cts]
+    shared_pb = [[(dext[0], pbs[0], dk[g1], dm1, g1), (dext[1], pbs[1], dk[g1], dm2, g1),
+                  (dext[2], pbs[2], dk[g3], dm1, g3)]]
+    assert np.array_equal(host(ctx.hoisted_terms(shared_pb, nq, b_premultiplied=True)[0]), want_shared)
     # plain ModDown and ModDown merged with the rescale, batched over all outputs
     for drop in (False, True):
         got = host(ctx.moddown_batch(y.clone(), nq, drop))
