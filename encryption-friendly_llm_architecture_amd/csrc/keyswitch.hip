@@ -491,7 +491,8 @@ struct LinTermDev {
 template <int n_polys>
 __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
                                                          const u32 *__restrict__ group_off, u64 *__restrict__ out,
-                                                         const ModQ *__restrict__ modq, int nq, int logN, int n_out) {
+                                                         const ModQ *__restrict__ modq, const double *__restrict__ fp, int nq, int logN,
+                                                         int n_out) {
     // Workgroups go round-robin over the 8 XCDs, each with its own L2.  The outputs of one launch mostly
     // sum the same ciphertexts under different masks, so all outputs of a (limb, 256-coefficient) tile are
     // placed back to back on one XCD: the ciphertext tile is fetched from HBM once instead of once per output.
@@ -509,6 +510,42 @@ __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__res
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN;
     const size_t e = (size_t)j * N + (size_t)(tile & ((1u << (logN - 8)) - 1)) * 256 + threadIdx.x;
+    const double fq = fp[4 * j];
+    if (fq != 0.0) {
+        // primes below 2^44: exact double-precision products (6 FP64 operations each)
+        const FpMod f{fq, fp[4 * j + 1]};
+        double facc[n_polys];
+#pragma unroll
+        for (int p = 0; p < n_polys; p++) facc[p] = 0.0;
+        int since = 0;
+        for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
+            const LinTermDev T = terms[t];
+            if (T.mask != nullptr) {
+                const u64 mk = T.galois ? T.mask[(size_t)j * N + galois_index((u32)(e - (size_t)j * N), (u32)T.galois, logN)]
+                                        : T.mask[e];
+                const double dm = __longlong_as_double((long long)(mk | 0x4330000000000000ull)) - 4503599627370496.0;
+#pragma unroll
+                for (int p = 0; p < n_polys; p++) {
+                    const u64 cv = T.ct[p * T.stride + e];
+                    facc[p] += f.mul(__longlong_as_double((long long)(cv | 0x4330000000000000ull)) - 4503599627370496.0, dm);
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < n_polys; p++) {
+                    const u64 cv = T.ct[p * T.stride + e];
+                    facc[p] += __longlong_as_double((long long)(cv | 0x4330000000000000ull)) - 4503599627370496.0;
+                }
+            }
+            if (++since == 64) {  // a term adds at most q: keep the running sums far below 2^52
+#pragma unroll
+                for (int p = 0; p < n_polys; p++) facc[p] = f.reduce(facc[p]);
+                since = 0;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < n_polys; p++) out[((size_t)o * n_polys + p) * nq * N + e] = f.canonical(facc[p]);
+        return;
+    }
     u64 acc[n_polys];
     u128_t lazy[n_polys];
 #pragma unroll
@@ -993,11 +1030,14 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
     dim3 grid((unsigned)(c->N / 256) * nq * n_out), block(256);
     const LinTermDev *td = (const LinTermDev *)terms_dev;
     if (n_polys == 1)
-        hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
+        hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
+                           n_out);
     else if (n_polys == 2)
-        hipLaunchKernelGGL(masked_sum_kernel<2>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
+        hipLaunchKernelGGL(masked_sum_kernel<2>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
+                           n_out);
     else
-        hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, nq, c->logN, n_out);
+        hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
+                           n_out);
 }
 
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
