@@ -163,6 +163,13 @@ struct IntField {
         u64 t = mul_shoup_lazy(v, ni, nis, q);
         return t >= q ? t - q : t;
     }
+    // (y - v) * cst mod q for a transformed value v and a canonical minuend y
+    __device__ __forceinline__ u64 sub_scale(E v, u64 y, const Tw cst) const {
+        const u64 c = to_canonical(v);
+        const u64 d = y >= c ? y - c : y + q - c;
+        const u64 t = mul_shoup_lazy(d, cst.w, cst.ws, q);
+        return t >= q ? t - q : t;
+    }
 };
 
 struct __align__(16) TwF {
@@ -210,6 +217,10 @@ struct FpField {
     }
     __device__ __forceinline__ u64 to_canonical(E v) const { return centred_to_canonical(reduce(v)); }
     __device__ __forceinline__ u64 scale_to_canonical(E v) const { return centred_to_canonical(mulmod(v, ni, niinv)); }
+    __device__ __forceinline__ u64 sub_scale(E v, u64 y, const Tw cst) const {
+        const double w = (double)cst.w;
+        return centred_to_canonical(mulmod(from_canonical(y) - v, w, w * qinv));
+    }
 };
 
 // radix-16 block of 4 Cooley-Tukey stages on registers; stage s, group g uses twiddle
@@ -347,20 +358,14 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
         radix16_fwd(f, x, tw, 16u * (256u + r) + c);
         wave_sync();
 #pragma unroll
-        for (int k = 0; k < 16; k++) lc[padc(16 * c + k)] = f.to_canonical(x[k]);
+        for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
         wave_sync();
         if (EPI) {
 #pragma unroll
-            for (int k = 0; k < 16; k++) {
-                const u64 v = lc[padc(c + 16 * k)], y = mn[c + 16 * k];
-                const u64 d = y >= v ? y - v : y + q - v;
-                u64 t = mul_shoup_lazy(d, cst.w, cst.ws, q);
-                if (t >= q) t -= q;
-                o[c + 16 * k] = t;
-            }
+            for (int k = 0; k < 16; k++) o[c + 16 * k] = f.sub_scale(l[padc(c + 16 * k)], mn[c + 16 * k], cst);
         } else {
 #pragma unroll
-            for (int k = 0; k < 16; k++) row[c + 16 * k] = lc[padc(c + 16 * k)];
+            for (int k = 0; k < 16; k++) row[c + 16 * k] = f.to_canonical(l[padc(c + 16 * k)]);
         }
     } else {
 #pragma unroll
