@@ -321,8 +321,23 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), off.data(), (n_out + 1) * sizeof(uint32_t),
                                   &off_dev, (hipStream_t)stream);
+    // When the first and the second half of the outputs gather from disjoint sets of sources (column shifts
+    // of one operand, then row shifts of the other), the kernel walks the halves one after the other.
+    int phases = 1;
+    if (n_out % 2 == 0 && n_out >= 2) {
+        std::vector<const u64 *> first;
+        bool disjoint = true;
+        for (uint32_t t = 0; t < off[n_out / 2]; t++) first.push_back(d[t].ext);
+        for (uint32_t t = off[n_out / 2]; t < off[n_out] && disjoint; t++)
+            for (const u64 *p : first)
+                if (p == d[t].ext || p == d[t].ext2) {
+                    disjoint = false;
+                    break;
+                }
+        if (disjoint) phases = 2;
+    }
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
-                         (hipStream_t)stream);
+                         phases, (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

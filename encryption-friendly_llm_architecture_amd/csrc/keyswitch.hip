@@ -463,11 +463,14 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
-                                                            int n_full, int logN, int b_premultiplied) {
+                                                            int n_full, int logN, int b_premultiplied, int phases) {
     // blockIdx.x = output (fastest): workgroups that gather from the same source tile run back to back.
     // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
     // (possibly swapped), so every access is a 16-byte load or store.
-    const int j = blockIdx.z, o = blockIdx.x;
+    // The outputs are walked in `phases` equal runs per limb (blockIdx.z = limb * phases + run): when the
+    // runs gather from different sources, only one run's sources (1.5 MiB per source and limb) compete
+    // for an XCD's 4 MiB L2 at a time.
+    const int j = blockIdx.z / phases, o = blockIdx.x + (blockIdx.z % phases) * gridDim.x;
     const int prime = ll.idx[j];
     const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
     const double fq = fp[4 * prime];
@@ -952,7 +955,8 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
 
 // terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, hipStream_t s) {
+                          bool b_premultiplied, int phases, hipStream_t s) {
+    if (phases < 1 || n_out % phases != 0) phases = 1;
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     CstList pm;
     memset(&pm, 0, sizeof(pm));
@@ -961,10 +965,10 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
         for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
         pm.c[j] = Cst{P, shoup_h(P, q)};
     }
-    dim3 grid(n_out, c->N / 512, E), block(256);
+    dim3 grid(n_out / phases, c->N / 512, E * phases), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
-                       b_premultiplied ? 1 : 0);
+                       b_premultiplied ? 1 : 0, phases);
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;
