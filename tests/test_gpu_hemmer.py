@@ -187,6 +187,56 @@ def test_hoisted_products_bit_exact(small, fused):
     assert np.abs(z[1] - (X0 @ W[1] + X1 @ W[3])).max() < 2 ** -18
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_reuse_variants_and_repacking(small, fused):
+    """The ciphertext x ciphertext re-use forms (matMulPre + matMulPreRev + matMulCCReUse and their packed
+    counterparts), splitInTwo, complexPackingRev and repack_notBTS against float64 algebra on the slots."""
+    H, orc, ev = small
+    n, T = 16, 2
+    H.set_schedule(fused, batch=5)
+    rng = np.random.default_rng(8)
+    A0, A1, B0, B1 = (rng.uniform(-1, 1, (n, n)) for _ in range(4))
+    a, b = H.encrypt2(A0, A1), H.encrypt2(B0, B1)
+    # sigma(A) shifts once, tau(B) once, then sum_k shift_k(sigma A) (x) rowrot_k(tau B)
+    tmp = H.matmul_pre(a, T)
+    bt = H.matmul_pre_rev(b, T)
+    c = H.matmul_cc_reuse(tmp, bt, T)
+    d = H.decrypt2(c)
+    assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    # packed counterparts: the same product as packedMatMul
+    pa, pb = H.encrypt2(A0, A1), H.encrypt2(B0, B1)
+    H.complex_packing_inplace(pa)
+    H.complex_packing_row_inplace(pb)
+    sa = H.packed_matmul_pre(pa, T)
+    ptmp = H.packed_matmul_pre_rot(sa, T)
+    pbt = H.packed_matmul_pre_rev(pb, T)
+    pc = H.repack_cc(H.packed_matmul_cc_reuse(ptmp, pbt, T))
+    d = H.decrypt2(pc)
+    assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    H.set_schedule(True)
+    # splitInTwo: [A0 | A1] -> [A0 | A0], [A1 | A1]
+    t1, t2 = H.split_in_two(H.encrypt2(A0, A1))
+    d1, d2 = H.decrypt2(t1), H.decrypt2(t2)
+    for got, want in ((d1[0], A0), (d1[1], A0), (d2[0], A1), (d2[1], A1)):
+        assert np.abs(got - want).max() < 2 ** -20
+    # complexPackingRev: x - i y
+    z = H.decrypt_slots(H.complex_packing_rev(H.encrypt2(A0, A1), H.encrypt2(B0, B1)))
+    want = np.concatenate([A0, A1], axis=1).ravel() - 1j * np.concatenate([B0, B1], axis=1).ravel()
+    assert np.abs(z - want).max() < 2 ** -20
+    # repack_notBTS: o = 2 Re(t1) + 2i Re(t2); left half <- o + rot(o, n) on the left columns, right half <-
+    # the left columns of rot(o, n)
+    x1 = H.complex_packing(H.encrypt2(A0, A1), H.encrypt2(B0, B1))     # A + iB
+    x2 = H.complex_packing(H.encrypt2(B1, A0), H.encrypt2(A1, B0))
+    out = H.decrypt_slots(H.repack_not_bts(x1, x2))
+    s1 = np.concatenate([A0, A1], axis=1).ravel()
+    s2 = np.concatenate([B1, A0], axis=1).ravel()
+    o = 2 * s1 + 2j * s2
+    rot = np.roll(o, -n)
+    m = np.concatenate([np.ones((n, n)), np.zeros((n, n))], axis=1).ravel()
+    want = (o + rot) * m + np.roll(rot * m, n)
+    assert np.abs(out - want).max() < 2 ** -18
+
+
 def test_error_behaviour(small):
     H, _, _ = small
     A = np.ones((16, 16))
