@@ -188,6 +188,28 @@ def gpu_hoisted(args, out):
         torch.cuda.synchronize()
 
 
+def gpu_rotation_60bit(args, out):
+    """One key-switched rotation at the reference rotation benchmark's shape: chain of 24 60-bit primes + 4
+    special primes, dnum 3, ciphertext at level 20 (random residues and key: timing only)."""
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    primes = pkg.primes_below(60, 16, 28)
+    ctx = pkg.Context(16, primes[:24], primes[24:], 3)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    nq, N = 21, 1 << 16
+    ct = torch.randint(0, 2 ** 59, (2, nq, N), dtype=torch.int64, device="cuda", generator=g)
+    evk = torch.randint(0, 2 ** 59, (3, 2, 28, N), dtype=torch.int64, device="cuda", generator=g)
+    for _ in range(3):
+        ctx.rotate(ct, evk, 5, nq)
+    torch.cuda.synchronize()
+    timer = pkg.Timer()
+    timer.start()
+    for _ in range(30):
+        ctx.rotate(ct, evk, 5, nq)
+    out["rotation_24x60bit_level20_us"] = timer.stop() / 30 * 1e3
+
+
 def cpu_baseline(out, budget_s=25.0):
     """The CPU oracle (scalar C++ port, one thread) on a bounded sample of the CCMM's operation mix,
     scaled by the per-product operation counts."""
@@ -267,6 +289,7 @@ def main():
     gpu_ccmm(args, out)
     gpu_hoisted(args, out)
     gpu_ntt(args, out)
+    gpu_rotation_60bit(args, out)
     if not args.no_cpu:
         cpu_baseline(out)
     print(json.dumps(out))

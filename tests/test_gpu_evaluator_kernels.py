@@ -244,3 +244,29 @@ def test_batched_hoisted_forms(S):
         t = orc.tensor(O.Ct(a, 1.0), O.Ct(b, 1.0))
         want3 = t if want3 is None else orc.add(want3, t)
     assert np.array_equal(host(acc), want3.data)
+
+
+def test_rotation_24_limb_chain_of_60_bit_primes():
+    """One key-switched rotation at the shape of the reference's rotation benchmark: N = 2^16, a chain of 24
+    60-bit primes + 4 special primes, dnum = 3 (digits of 8 limbs), ciphertext at level 20, steps from the
+    power-of-two set HEMMer uses.  Residues bit-exact against the oracle, ModUp and ModDown included."""
+    pkg = load_package()
+    log_n, N = 16, 1 << 16
+    primes = pkg.primes_below(60, log_n, 28)
+    qs, ps = primes[:24], primes[24:]
+    orc = O.Oracle(log_n, qs, ps, 3)
+    ctx = pkg.Context(log_n, qs, ps, 3)
+    orc.gen_secret(3)
+    rng = np.random.default_rng(20)
+    nq = 21
+    ct = rand_limbs(rng, qs[:nq], (2,), N)
+    dct = dev(ct)
+    # stages on the a-polynomial
+    ext = orc.modup(ct[1])
+    assert np.array_equal(host(ctx.modup(dct[1].contiguous(), nq)), ext)
+    for r in (1, 64, 128 * 5):
+        orc.gen_rot_key(6, r)
+        g = orc.galois(r)
+        want = orc.left_rotate(O.Ct(ct, 1.0), r)
+        got = host(ctx.rotate(dct, dev(orc.keys[("gal", g)]), g, nq))
+        assert np.array_equal(got, want.data), r
