@@ -313,20 +313,31 @@ Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq) {
 }
 // The same sources rotated left by rots[q] slots, as ciphertexts [n][2][nq][N]: one hoisted launch and one
 // ModDown for all of them.
-DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, size_t n, const i64 *rots) {
+DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u64 *cts, size_t n, const i64 *rots) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    const u64 nq = src.nq, N = c->N, E = nq + c->nP;
+    const u64 nq = src.nq, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
+    DeviceBuffer out(c, n * ctw);
     std::vector<hemm_rot_term> terms;
     std::vector<uint32_t> off{0};
+    std::vector<size_t> which;
     for (size_t q = 0; q < n; q++) {
+        if (rot.norm(rots[q]) == 0) {  // a whole turn (rows of a tile that fills the slots): plain copy
+            (void)hipMemcpyAsync(out.data() + q * ctw, cts + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+            continue;
+        }
         terms.push_back(term(src.extOf(q), src.pbOf(q), pack, rot.galois(rots[q]), nullptr));
         off.push_back((uint32_t)terms.size());
+        which.push_back(q);
     }
-    DeviceBuffer y(c, n * 2 * E * N), ws(c, n * 2 * nq * N), out(c, n * 2 * nq * N);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)n, (uint32_t)nq, y.data(), 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * n), 0, out.data(), nq * N, ws.data(), nullptr));
+    if (which.empty()) return out;
+    const size_t m = which.size();
+    DeviceBuffer y(c, m * 2 * E * N), ws(c, m * ctw), tmp(c, m * ctw);
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, y.data(), 1, nullptr));
+    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * m), 0, tmp.data(), nq * N, ws.data(), nullptr));
+    for (size_t k = 0; k < m; k++)
+        (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
     return out;
 }
 
@@ -436,7 +447,7 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     // rotation sources: sigma(A), tau(B) and their copies rotated by -n columns / -n rows
     const Sources x = extendSources(c, ab.data(), 2, nq);
     const i64 back[2] = {-n, -n * w};
-    const DeviceBuffer ab2 = rotateSources(eval, x, 2, back);
+    const DeviceBuffer ab2 = rotateSources(eval, x, ab.data(), 2, back);
     const Sources x2 = extendSources(c, ab2.data(), 2, nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
@@ -502,7 +513,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     // rotation sources: sigma(A), its copy rotated by -n columns, and tau(B)
     const Sources xa = extendSources(c, a.get().buf_.data(), 1, nqa);
     const i64 back = -n;
-    const DeviceBuffer a2 = rotateSources(eval, xa, 1, &back);
+    const DeviceBuffer a2 = rotateSources(eval, xa, a.get().buf_.data(), 1, &back);
     const Sources xa2 = extendSources(c, a2.data(), 1, nqa);
     const Sources xb = extendSources(c, b.get().buf_.data(), 1, nqb);
     const KeyPack &pack = eval.getKeyPack();
@@ -555,7 +566,7 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
     const Sources x = extendSources(c, a.get().buf_.data(), 1, nq);
     const i64 back = -n;
-    const DeviceBuffer a2 = rotateSources(eval, x, 1, &back);
+    const DeviceBuffer a2 = rotateSources(eval, x, a.get().buf_.data(), 1, &back);
     const Sources x2 = extendSources(c, a2.data(), 1, nq);
     const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
     DeviceBuffer y(c, G * 2 * E * N), t(c, G * 2 * lo * N), ws(c, G * 2 * lo * N);

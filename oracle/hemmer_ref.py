@@ -543,6 +543,8 @@ def diagonal_transform_fused(orc, ct, kind, n, w):
 def _rotated_copy(orc, src, ext, r):
     """rot(src, r) with the automorphism after ModUp (one hoisted term, plain ModDown)."""
     from .oracle import Ct
+    if r % orc.slots == 0:      # a whole turn: rows of a tile that fills the slot vector
+        return src.copy()
     y = orc.hoisted_sum([(ext, src.data[0], r % orc.slots, None)], src.nq)
     return Ct(orc.moddown_drop(y, src.nq, False), src.scale)
 

@@ -118,6 +118,24 @@ def test_ccmm_residues_bit_exact_and_decrypts(small, fused):
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_ccmm_pair_layout(small, fused):
+    """Two products per call on the pair layout [A1 | A2] x [B1 | B2] (rows fill the slot vector, so the
+    row wrap is a whole turn)."""
+    H, orc, ev = small
+    H.set_schedule(fused, batch=4)
+    rng = np.random.default_rng(9)
+    A1, A2, B1, B2 = (rng.uniform(-1, 1, (16, 16)) for _ in range(4))
+    ca, cb = H.encrypt2(A1, A2), H.encrypt2(B1, B2)
+    c = H.single_cc_matmul(ca, cb, 2)
+    H.set_schedule(True)
+    oa, ob = to_oracle(orc, ca), to_oracle(orc, cb)
+    want = R.mult_mat_mat_cc_fused(orc, oa, ob, 2, 16, 32) if fused else R.mult_mat_mat_cc(ev, oa, ob, 2, 16, 32)
+    assert np.array_equal(c.residues(), want.data)
+    d = H.decrypt2(c)
+    assert np.abs(d[0] - A1 @ B1).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
+
+
 def test_batch_size_does_not_change_residues(small):
     H, _, _ = small
     rng = np.random.default_rng(14)
