@@ -69,6 +69,7 @@ def _declare(L):
     L.hemm_modup_batch.argtypes = [vp, vp, sz, u32, u32, vp, vp, vp]
     L.hemm_hoisted_terms.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, vp, ci, vp]
     L.hemm_moddown_batch.argtypes = [vp, vp, u32, u32, ci, vp, sz, vp, vp]
+    L.hemm_hoisted_moddown.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, ci, ci, vp, vp, sz, vp, vp]
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
 
@@ -248,6 +249,27 @@ class Context:
         y = torch.empty((len(groups), 2, nq + self.nP, self.N), dtype=torch.int64, device=flat[0][0].device)
         check(lib().hemm_hoisted_terms(self.h, arr, off, len(groups), nq, vp(y.data_ptr()), int(b_premultiplied), vp(0)))
         return y
+
+    def hoisted_moddown(self, groups, nq, drop_last, b_premultiplied=False):
+        """hoisted_terms + moddown_batch in one call -> [n_out][2][nq - drop_last][N]"""
+        import torch
+        flat = [t for g in groups for t in g]
+        arr = (RotTerm * len(flat))()
+        for i, (ext, b, evk, mask, gal) in enumerate(flat):
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
+                             mask.data_ptr() if mask is not None else None, gal)
+        offs = [0]
+        for g in groups:
+            offs.append(offs[-1] + len(g))
+        off = (ctypes.c_uint32 * len(offs))(*offs)
+        dev = flat[0][0].device
+        nq_out = nq - 1 if drop_last else nq
+        y = torch.empty((len(groups), 2, nq + self.nP, self.N), dtype=torch.int64, device=dev)
+        out = torch.empty((len(groups), 2, nq_out, self.N), dtype=torch.int64, device=dev)
+        ws = torch.empty_like(out)
+        check(lib().hemm_hoisted_moddown(self.h, arr, off, len(groups), nq, int(b_premultiplied), int(drop_last),
+                                         vp(y.data_ptr()), vp(out.data_ptr()), nq_out * self.N, vp(ws.data_ptr()), vp(0)))
+        return out
 
     def moddown_batch(self, y, nq, drop_last):
         """y: [..., nq+K, N] (clobbered) -> [..., nq - drop_last, N]"""

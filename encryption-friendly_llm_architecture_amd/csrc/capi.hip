@@ -282,22 +282,19 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
     HEMM_CATCH
 }
 
-int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
-                       uint32_t nq, uint64_t *y, int b_premultiplied, void *stream) {
-    HEMM_TRY
-    int nl;
-    chain_limbs(ctx, nq, 1, &nl);
-    need(terms && group_offsets && y && n_out >= 1, "null operand");
-    need(ctx->nP >= 1, "key switching needs special primes");
+// Validates a list of rotation terms, merges consecutive masked terms of a group that use the same key and
+// Galois element into one two-source term (the kernels then stream that key once for both), and uploads
+// the device descriptors.  *phases = 2 when the first and the second half of the outputs gather from
+// disjoint sets of sources (column shifts of one operand, then row shifts of the other).
+struct RotDev {
+    const u64 *ext, *b, *evk, *mask;
+    u32 galois, pad;
+    const u64 *ext2, *b2, *mask2;
+};
+static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
+                             uint32_t n_out, hipStream_t stream, void **terms_dev, void **off_dev, int *phases) {
     const uint32_t n_terms = group_offsets[n_out];
-    struct Dev {
-        const u64 *ext, *b, *evk, *mask;
-        u32 galois, pad;
-        const u64 *ext2, *b2, *mask2;
-    };
-    // Consecutive masked terms of a group that use the same key and Galois element are merged into one
-    // two-source term: the kernel then streams that key once for both.
-    std::vector<Dev> d;
+    std::vector<RotDev> d;
     std::vector<uint32_t> off{0};
     d.reserve(n_terms);
     for (uint32_t o = 0; o < n_out; o++) {
@@ -305,8 +302,8 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
         for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
             need(terms[t].ext && terms[t].b && terms[t].evk, "null pointer in a rotation term");
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
-            Dev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
-                    (const u64 *)terms[t].mask, (u32)terms[t].galois, 0, nullptr, nullptr, nullptr};
+            RotDev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
+                       (const u64 *)terms[t].mask, (u32)terms[t].galois, 0, nullptr, nullptr, nullptr};
             if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t + 1].ext && terms[t + 1].b &&
                 terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois) {
                 cur.ext2 = (const u64 *)terms[t + 1].ext;
@@ -318,12 +315,9 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
         }
         off.push_back((uint32_t)d.size());
     }
-    void *off_dev = nullptr;
-    void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(Dev), off.data(), (n_out + 1) * sizeof(uint32_t),
-                                  &off_dev, (hipStream_t)stream);
-    // When the first and the second half of the outputs gather from disjoint sets of sources (column shifts
-    // of one operand, then row shifts of the other), the kernel walks the halves one after the other.
-    int phases = 1;
+    *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t), off_dev,
+                             stream);
+    *phases = 1;
     if (n_out % 2 == 0 && n_out >= 2) {
         std::vector<const u64 *> first;
         bool disjoint = true;
@@ -334,10 +328,41 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
                     disjoint = false;
                     break;
                 }
-        if (disjoint) phases = 2;
+        if (disjoint) *phases = 2;
     }
+}
+
+int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                       uint32_t nq, uint64_t *y, int b_premultiplied, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(terms && group_offsets && y && n_out >= 1, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    void *terms_dev = nullptr, *off_dev = nullptr;
+    int phases = 1;
+    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev, &phases);
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
                          phases, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                         uint32_t nq, int b_premultiplied, int drop_last, uint64_t *y_workspace, uint64_t *out,
+                         size_t out_stride, uint64_t *workspace, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(terms && group_offsets && y_workspace && out && workspace && n_out >= 1, "null operand");
+    need(ctx->nP >= 1, "key switching needs special primes");
+    void *terms_dev = nullptr, *off_dev = nullptr;
+    int phases = 1;
+    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev, &phases);
+    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y_workspace,
+                         b_premultiplied != 0, phases, (hipStream_t)stream);
+    launch_moddown_batch(ctx, (u64 *)y_workspace, (int)nq, (int)(2 * n_out), drop_last != 0, (u64 *)out, out_stride,
+                         (u64 *)workspace, (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

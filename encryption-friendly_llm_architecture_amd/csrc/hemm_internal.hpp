@@ -38,6 +38,11 @@ struct hemm_context {
     void *d_desc;                   // staging for the term lists of batched calls
 };
 
+// a constant and its Shoup quotient floor(w * 2^64 / q)
+struct __align__(16) Cst {
+    u64 w, ws;
+};
+
 void hemm_set_error(const std::string &msg);
 
 #define HEMM_HIP(call)                                                                       \

@@ -184,9 +184,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
             off.push_back((uint32_t)terms.size());
         }
     DeviceBuffer y(c, n_baby * 2 * E * N), baby(c, n_baby * ctw), ws(c, n_baby * ctw);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)n_baby, (uint32_t)nq, y.data(), 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * n_baby), 0, baby.data(), nq * N, ws.data(),
-                          nullptr));
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_baby, (uint32_t)nq, 1, 0, y.data(), baby.data(), nq * N, ws.data(), nullptr));
 
     // 2. group sums: a job's group 0 needs no rotation (d = 0, the positive diagonals of giant index 0, and
     //    any group whose rotation is a whole turn).  The unrotated groups of all jobs come first in `sums`,
@@ -263,9 +261,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
             goff.push_back((uint32_t)gt.size());
         }
         DeviceBuffer y2(c, n_jobs * 2 * E * N), ws3(c, n_jobs * ctw);
-        ck(hemm_hoisted_terms(c->dev, gt.data(), goff.data(), (uint32_t)n_jobs, (uint32_t)nq, y2.data(), 0, nullptr));
-        ck(hemm_moddown_batch(c->dev, y2.data(), (uint32_t)nq, (uint32_t)(2 * n_jobs), 0, res.data(), nq * N, ws3.data(),
-                              nullptr));
+        ck(hemm_hoisted_moddown(c->dev, gt.data(), goff.data(), (uint32_t)n_jobs, (uint32_t)nq, 0, 0, y2.data(), res.data(), nq * N, ws3.data(), nullptr));
         ck(hemm_pointwise(c->dev, HEMM_ADD, res.data(), nq * N, sums.data(), nq * N, res.data(), nq * N, (uint32_t)nq, 0,
                           (uint32_t)(2 * n_jobs), nullptr));
     } else if (ng == 0) {
@@ -334,8 +330,7 @@ DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u
     if (which.empty()) return out;
     const size_t m = which.size();
     DeviceBuffer y(c, m * 2 * E * N), ws(c, m * ctw), tmp(c, m * ctw);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, y.data(), 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * m), 0, tmp.data(), nq * N, ws.data(), nullptr));
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, 1, 0, y.data(), tmp.data(), nq * N, ws.data(), nullptr));
     for (size_t k = 0; k < m; k++)
         (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
     return out;
@@ -458,8 +453,7 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         std::vector<uint32_t> off{0};
         pushShifts(eval, x, 0, x2, 0, sa, first, cnt, terms, off);
         pushShifts(eval, x, 1, x2, 1, sb, first, cnt, terms, off);
-        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)(2 * cnt), (uint32_t)nq, y.data(), 1, nullptr));
-        ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(4 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)(2 * cnt), (uint32_t)nq, 1, 1, y.data(), t.data(), lo * N, ws.data(), nullptr));
         ck(hemm_tensor_batch(c->dev, t.data(), t.data() + cnt * 2 * lo * N, (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(),
                              1, nullptr));
     }
@@ -527,9 +521,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
             std::vector<hemm_rot_term> terms;
             std::vector<uint32_t> off{0};
             pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
-            ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqa, ya.data(), 1, nullptr));
-            ck(hemm_moddown_batch(c->dev, ya.data(), (uint32_t)nqa, (uint32_t)(2 * cnt), 1, t1.data(), lo * N, ws.data(),
-                                  nullptr));
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqa, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
         }
         // row shifts are exact rotations here: one unmasked hoisted term each, plain ModDown
         std::vector<hemm_rot_term> terms;
@@ -538,9 +530,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
             terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
             off.push_back((uint32_t)terms.size());
         }
-        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, yb.data(), 1, nullptr));
-        ck(hemm_moddown_batch(c->dev, yb.data(), (uint32_t)nqb, (uint32_t)(2 * cnt), 0, t2.data(), lo * N, ws.data(),
-                              nullptr));
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, 1, 0, yb.data(), t2.data(), lo * N, ws.data(), nullptr));
         ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(), 1, nullptr));
     }
     finish();
@@ -575,8 +565,7 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         pushShifts(eval, x, 0, x2, 0, sa, first, cnt, terms, off);
-        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, y.data(), 1, nullptr));
-        ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, (uint32_t)(2 * cnt), 1, t.data(), lo * N, ws.data(), nullptr));
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, y.data(), t.data(), lo * N, ws.data(), nullptr));
         for (size_t q = 0; q < cnt; q++) {
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);

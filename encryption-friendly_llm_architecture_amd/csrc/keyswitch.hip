@@ -11,6 +11,7 @@
 #include <cstring>
 
 #include "hemm_internal.hpp"
+#include "hoisted.cuh"
 
 void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
                       int n_polys, size_t poly_stride, bool inverse, hipStream_t s);
@@ -18,10 +19,6 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
                           size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 
 namespace {
-
-struct __align__(16) Cst {
-    u64 w, ws;
-};
 
 struct BConvArgs {
     const u64 *src;        // coefficient form
@@ -137,10 +134,6 @@ __global__ __launch_bounds__(256) void inner_product_kernel(const u64 *__restric
     acc[((size_t)n_ext + j) * N + n] = barrett128(sa, m);
 }
 
-struct CstList {
-    Cst c[HEMM_MAX_PRIMES];
-};
-
 // out[p][j] = (a[p][j] - t[p][j]) * cst[j]  (+ add[p][j] when add != nullptr)
 __global__ __launch_bounds__(256) void sub_scale_kernel(const u64 *__restrict__ a, size_t a_stride,
                                                         const u64 *__restrict__ t, size_t t_stride,
@@ -168,297 +161,11 @@ __global__ __launch_bounds__(256) void spread_kernel(const u64 *__restrict__ las
 
 u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 
-// NTT-domain index of the automorphism X -> X^g: out[k] = in[galois_index(k)]
-__device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
-    const u32 br = __brev(k) >> (32 - logN);
-    const u32 e = ((2 * br + 1) * g) & ((2u << logN) - 1);
-    return __brev(e >> 1) >> (32 - logN);
-}
-
-struct RotTermDev {
-    const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
-    const u64 *b;     // [nq][N] b-polynomial of the source
-    const u64 *evk;   // [dnum][2][nQ+K][N]
-    const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
-    u32 galois, pad;
-    // optional second source rotated by the same Galois element with the same key (ext2 == nullptr: none):
-    // the term is mask * rot(source) + mask2 * rot(source 2) and the key is read once for both
-    const u64 *ext2, *b2, *mask2;
-};
-
 // Hoisted rotations, several per output, combined with masks in the extended basis:
 //   y[o][pol][j][n] = sum_{t in group o} mask_t[j][n] * ( sum_d ext_t[d][j][pi_t(n)] * evk_t[d][pol][j][n]
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
-// 16-byte accesses to data that is touched once per launch (keys, masks, results): marked non-temporal so
-// they do not push the rotation sources, which every output gathers from, out of the L2.
-typedef u64 u64x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ ulonglong2 stream_load2(const u64 *p) {
-    const u64x2 v = __builtin_nontemporal_load((const u64x2 *)p);
-    return make_ulonglong2(v.x, v.y);
-}
-__device__ __forceinline__ void stream_store2(u64 *p, u64 a, u64 b) {
-    u64x2 v;
-    v.x = a;
-    v.y = b;
-    __builtin_nontemporal_store(v, (u64x2 *)p);
-}
-
-__device__ __forceinline__ void hoisted_terms_int(const RotTermDev *__restrict__ terms,
-                                                  const u32 *__restrict__ group_off, u64 *__restrict__ y,
-                                                  const ModQ m, const CstList &pmod, const int j, const int o,
-                                                  const int prime, const u32 n, int nq, int E, int beta, int n_full,
-                                                  int logN, int b_premultiplied) {
-    const size_t N = (size_t)1 << logN;
-    u64 acc_b[2] = {0, 0}, acc_a[2] = {0, 0};
-    u128_t lazy_b[2] = {{0, 0}, {0, 0}}, lazy_a[2] = {{0, 0}, {0, 0}};
-    int pending = 0;
-    for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
-        const RotTermDev T = terms[t];
-        const u32 np = galois_index(n, T.galois, logN);
-        const u32 base = np & ~1u;
-        const bool swap = (np & 1u) != 0;
-        if (T.ext2 != nullptr) {
-            // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
-            const ulonglong2 m1 = stream_load2(T.mask + (size_t)j * N + n);
-            const ulonglong2 m2 = stream_load2(T.mask2 + (size_t)j * N + n);
-            u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
-            for (int d = 0; d < beta; d++) {
-                ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
-                ulonglong2 x2 = *(const ulonglong2 *)(T.ext2 + ((size_t)d * E + j) * N + base);
-                if (swap) {
-                    u64 tmp = x1.x;
-                    x1.x = x1.y;
-                    x1.y = tmp;
-                    tmp = x2.x;
-                    x2.x = x2.y;
-                    x2.y = tmp;
-                }
-                u128_t t0 = mul64wide(m1.x, x1.x), t1 = mul64wide(m1.y, x1.y);
-                add128(t0, mul64wide(m2.x, x2.x));
-                add128(t1, mul64wide(m2.y, x2.y));
-                const u64 z0 = barrett128(t0, m), z1 = barrett128(t1, m);
-                const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-                const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
-                add128(pb[0], mul64wide(z0, kb.x));
-                add128(pb[1], mul64wide(z1, kb.y));
-                add128(pa[0], mul64wide(z0, ka.x));
-                add128(pa[1], mul64wide(z1, ka.y));
-            }
-            u64 rb0 = barrett128(pb[0], m), rb1 = barrett128(pb[1], m);
-            if (j < nq) {
-                ulonglong2 b1 = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
-                ulonglong2 b2 = *(const ulonglong2 *)(T.b2 + (size_t)j * N + base);
-                if (swap) {
-                    u64 tmp = b1.x;
-                    b1.x = b1.y;
-                    b1.y = tmp;
-                    tmp = b2.x;
-                    b2.x = b2.y;
-                    b2.y = tmp;
-                }
-                if (!b_premultiplied) {
-                    b1.x = mul_shoup(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b1.y = mul_shoup(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b2.x = mul_shoup(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b2.y = mul_shoup(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-                }
-                u128_t t0 = mul64wide(m1.x, b1.x), t1 = mul64wide(m1.y, b1.y);
-                add128(t0, mul64wide(m2.x, b2.x));
-                add128(t1, mul64wide(m2.y, b2.y));
-                rb0 = addmod(rb0, barrett128(t0, m), m.q);
-                rb1 = addmod(rb1, barrett128(t1, m), m.q);
-            }
-            acc_b[0] = addmod(acc_b[0], rb0, m.q);
-            acc_b[1] = addmod(acc_b[1], rb1, m.q);
-            acc_a[0] = addmod(acc_a[0], barrett128(pa[0], m), m.q);
-            acc_a[1] = addmod(acc_a[1], barrett128(pa[1], m), m.q);
-            continue;
-        }
-        u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
-        for (int d = 0; d < beta; d++) {
-            ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
-            if (swap) {
-                const u64 tmp = x.x;
-                x.x = x.y;
-                x.y = tmp;
-            }
-            const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-            const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
-            add128(sb[0], mul64wide(x.x, kb.x));
-            add128(sb[1], mul64wide(x.y, kb.y));
-            add128(sa[0], mul64wide(x.x, ka.x));
-            add128(sa[1], mul64wide(x.y, ka.y));
-        }
-        u64 rb[2] = {barrett128(sb[0], m), barrett128(sb[1], m)};
-        u64 ra[2] = {barrett128(sa[0], m), barrett128(sa[1], m)};
-        if (j < nq) {
-            ulonglong2 bv = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
-            if (swap) {
-                const u64 tmp = bv.x;
-                bv.x = bv.y;
-                bv.y = tmp;
-            }
-            if (!b_premultiplied) {
-                bv.x = mul_shoup(bv.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                bv.y = mul_shoup(bv.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-            }
-            rb[0] = addmod(rb[0], bv.x, m.q);
-            rb[1] = addmod(rb[1], bv.y, m.q);
-        }
-        if (T.mask != nullptr) {
-            const ulonglong2 mk = stream_load2(T.mask + (size_t)j * N + n);
-            add128(lazy_b[0], mul64wide(rb[0], mk.x));
-            add128(lazy_b[1], mul64wide(rb[1], mk.y));
-            add128(lazy_a[0], mul64wide(ra[0], mk.x));
-            add128(lazy_a[1], mul64wide(ra[1], mk.y));
-            if (++pending == 4) {
-                for (int i = 0; i < 2; i++) {
-                    acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
-                    acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
-                    lazy_b[i].lo = lazy_b[i].hi = lazy_a[i].lo = lazy_a[i].hi = 0;
-                }
-                pending = 0;
-            }
-        } else {
-            for (int i = 0; i < 2; i++) {
-                acc_b[i] = addmod(acc_b[i], rb[i], m.q);
-                acc_a[i] = addmod(acc_a[i], ra[i], m.q);
-            }
-        }
-    }
-    if (pending) {
-        for (int i = 0; i < 2; i++) {
-            acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
-            acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
-        }
-    }
-    stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, acc_b[0], acc_b[1]);
-    stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, acc_a[0], acc_a[1]);
-}
-
-// The same sums in double precision for primes below 2^44 (exact, see the transform kernels): a product
-// mod q is 6 FP64 operations instead of ~40 integer ones for a wide product plus its Barrett step.
-struct D2 {
-    double x, y;
-};
-__device__ __forceinline__ D2 to_d2(const ulonglong2 v) {
-    D2 r;
-    r.x = __longlong_as_double((long long)(v.x | 0x4330000000000000ull)) - 4503599627370496.0;
-    r.y = __longlong_as_double((long long)(v.y | 0x4330000000000000ull)) - 4503599627370496.0;
-    return r;
-}
-__device__ __forceinline__ D2 gather_d2(const u64 *p, const bool swap) {
-    ulonglong2 v = *(const ulonglong2 *)p;
-    if (swap) {
-        const u64 tmp = v.x;
-        v.x = v.y;
-        v.y = tmp;
-    }
-    return to_d2(v);
-}
-#pragma clang fp contract(off)
-struct FpMod {
-    double q, qinv;
-    // a * b mod q as a centred residue (|r| <= 0.54 q) for integers |a| < 2^48, |b| < 2^44
-    __device__ __forceinline__ double mul(double a, double b) const {
-        const double h = a * b;
-        const double l = __builtin_fma(a, b, -h);
-        const double c = __builtin_rint(h * qinv);
-        return __builtin_fma(-c, q, h) + l;
-    }
-    __device__ __forceinline__ double reduce(double x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
-    __device__ __forceinline__ u64 canonical(double x) const {
-        double r = reduce(x);
-        r += r < 0.0 ? q : 0.0;
-        return (u64)__double_as_longlong(r + 4503599627370496.0) & 0x000fffffffffffffull;
-    }
-};
-__device__ __forceinline__ void hoisted_terms_fp(const RotTermDev *__restrict__ terms,
-                                                 const u32 *__restrict__ group_off, u64 *__restrict__ y,
-                                                 const FpMod f, const double p_mod_q, const int j, const int o,
-                                                 const int prime, const u32 n, int nq, int E, int beta, int n_full,
-                                                 int logN, int b_premultiplied) {
-    const size_t N = (size_t)1 << logN;
-    double acc_b0 = 0, acc_b1 = 0, acc_a0 = 0, acc_a1 = 0;
-    int since = 0;
-    for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
-        const RotTermDev T = terms[t];
-        const u32 np = galois_index(n, T.galois, logN);
-        const u32 base = np & ~1u;
-        const bool swap = (np & 1u) != 0;
-        double sb0 = 0, sb1 = 0, sa0 = 0, sa1 = 0;
-        if (T.ext2 != nullptr) {
-            const D2 m1 = to_d2(stream_load2(T.mask + (size_t)j * N + n));
-            const D2 m2 = to_d2(stream_load2(T.mask2 + (size_t)j * N + n));
-            for (int d = 0; d < beta; d++) {
-                const D2 x1 = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
-                const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
-                const double z0 = f.mul(m1.x, x1.x) + f.mul(m2.x, x2.x);
-                const double z1 = f.mul(m1.y, x1.y) + f.mul(m2.y, x2.y);
-                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
-                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
-                sb0 += f.mul(z0, kb.x);
-                sb1 += f.mul(z1, kb.y);
-                sa0 += f.mul(z0, ka.x);
-                sa1 += f.mul(z1, ka.y);
-            }
-            if (j < nq) {
-                D2 b1 = gather_d2(T.b + (size_t)j * N + base, swap);
-                D2 b2 = gather_d2(T.b2 + (size_t)j * N + base, swap);
-                if (!b_premultiplied) {
-                    b1.x = f.mul(b1.x, p_mod_q);
-                    b1.y = f.mul(b1.y, p_mod_q);
-                    b2.x = f.mul(b2.x, p_mod_q);
-                    b2.y = f.mul(b2.y, p_mod_q);
-                }
-                sb0 += f.mul(m1.x, b1.x) + f.mul(m2.x, b2.x);
-                sb1 += f.mul(m1.y, b1.y) + f.mul(m2.y, b2.y);
-            }
-        } else {
-            for (int d = 0; d < beta; d++) {
-                const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
-                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
-                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
-                sb0 += f.mul(x.x, kb.x);
-                sb1 += f.mul(x.y, kb.y);
-                sa0 += f.mul(x.x, ka.x);
-                sa1 += f.mul(x.y, ka.y);
-            }
-            if (j < nq) {
-                D2 bv = gather_d2(T.b + (size_t)j * N + base, swap);
-                if (!b_premultiplied) {
-                    bv.x = f.mul(bv.x, p_mod_q);
-                    bv.y = f.mul(bv.y, p_mod_q);
-                }
-                sb0 += bv.x;
-                sb1 += bv.y;
-            }
-            if (T.mask != nullptr) {
-                const D2 mk = to_d2(stream_load2(T.mask + (size_t)j * N + n));
-                sb0 = f.mul(sb0, mk.x);
-                sb1 = f.mul(sb1, mk.y);
-                sa0 = f.mul(sa0, mk.x);
-                sa1 = f.mul(sa1, mk.y);
-            }
-        }
-        acc_b0 += sb0;
-        acc_b1 += sb1;
-        acc_a0 += sa0;
-        acc_a1 += sa1;
-        if (++since == 8) {  // a term adds at most (beta + 2) * 0.54 q: keep the running sums far below 2^52
-            acc_b0 = f.reduce(acc_b0);
-            acc_b1 = f.reduce(acc_b1);
-            acc_a0 = f.reduce(acc_a0);
-            acc_a1 = f.reduce(acc_a1);
-            since = 0;
-        }
-    }
-    stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, f.canonical(acc_b0), f.canonical(acc_b1));
-    stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, f.canonical(acc_a0), f.canonical(acc_a1));
-}
-
 __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
@@ -474,12 +181,23 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
     const int prime = ll.idx[j];
     const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
     const double fq = fp[4 * prime];
-    if (fq != 0.0 && beta <= 6)
-        hoisted_terms_fp(terms, group_off, y, FpMod{fq, fp[4 * prime + 1]}, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime,
-                         n, nq, E, beta, n_full, logN, b_premultiplied);
-    else
-        hoisted_terms_int(terms, group_off, y, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN,
-                          b_premultiplied);
+    const size_t N = (size_t)1 << logN;
+    u64 rb[2], ra[2];
+    if (fq != 0.0 && beta <= 6) {
+        const FpMod f{fq, fp[4 * prime + 1]};
+        double fb[2], fa[2];
+        hoisted_pair_fp(terms, group_off, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E, beta, n_full, logN,
+                        b_premultiplied, fb, fa);
+        rb[0] = f.canonical(fb[0]);
+        rb[1] = f.canonical(fb[1]);
+        ra[0] = f.canonical(fa[0]);
+        ra[1] = f.canonical(fa[1]);
+    } else {
+        hoisted_pair_int(terms, group_off, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN, b_premultiplied,
+                         rb, ra);
+    }
+    stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, rb[0], rb[1]);
+    stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, ra[0], ra[1]);
 }
 
 struct LinTermDev {
@@ -954,17 +672,23 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
 }
 
 // terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]
-void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, int phases, hipStream_t s) {
-    if (phases < 1 || n_out % phases != 0) phases = 1;
-    const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+// P mod q_j (and Shoup quotient) for the chain limbs j < nq
+static CstList p_mod_chain(const hemm_context *c, int nq) {
     CstList pm;
     memset(&pm, 0, sizeof(pm));
     for (int j = 0; j < nq; j++) {
         u64 q = c->primes[j], P = 1;
-        for (int k = 0; k < K; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
+        for (int k = 0; k < c->nP; k++) P = h_mulmod(P, c->primes[c->nQ + k] % q, q);
         pm.c[j] = Cst{P, shoup_h(P, q)};
     }
+    return pm;
+}
+
+void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
+                          bool b_premultiplied, int phases, hipStream_t s) {
+    if (phases < 1 || n_out % phases != 0) phases = 1;
+    const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+    const CstList pm = p_mod_chain(c, nq);
     dim3 grid(n_out / phases, c->N / 512, E * phases), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,

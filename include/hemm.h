@@ -124,6 +124,14 @@ typedef struct {
  * (hemm_mul_scalar with P mod q_j once per source instead of once per term). */
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
                        uint32_t n_out, uint32_t nq, uint64_t *y, int b_premultiplied, void *stream);
+/* hemm_hoisted_terms followed by hemm_moddown_batch on all n_out outputs (one term upload, one call).
+ * y_workspace: [n_out][2][nq+K][N] receives the sums and is clobbered; out: [n_out][2][nq_out][N] with
+ * polynomial stride out_stride; workspace: [n_out][2][nq_out][N].  No counterpart in HEaaN's interface: it is
+ * the key-switch tail of HomEvaluator::leftRotate / multWithoutRescale + rescale for a batch of outputs. */
+int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
+                         uint32_t n_out, uint32_t nq, int b_premultiplied, int drop_last, uint64_t *y_workspace,
+                         uint64_t *out, size_t out_stride, uint64_t *workspace, void *stream);
+
 /* y [n_polys][nq+n_p][N] (clobbered) -> out [n_polys][nq - drop_last][N]: division by P (drop_last = 0)
  * or by P*q_{nq-1} (drop_last = 1, ModDown and rescale in one basis conversion);
  * workspace >= n_polys*(nq-drop_last)*N words. */

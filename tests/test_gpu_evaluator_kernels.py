@@ -227,6 +227,18 @@ def test_batched_hoisted_forms(S):
         got = host(ctx.moddown_batch(y.clone(), nq, drop))
         for k in range(3):
             assert np.array_equal(got[k], orc.moddown_drop(want[k], nq, drop))
+    # both calls in one
+    all_groups = (groups + shared) * 2
+    all_want = (want + [want_shared]) * 2
+    for drop in (False, True):
+        got = host(ctx.hoisted_moddown(all_groups, nq, drop))
+        for k in range(8):
+            assert np.array_equal(got[k], orc.moddown_drop(all_want[k], nq, drop)), (k, drop)
+    got = host(ctx.hoisted_moddown(shared_pb * 8, nq, True, b_premultiplied=True))
+    assert np.array_equal(got[0], orc.moddown_drop(want_shared, nq, True))
+    assert np.array_equal(got[7], got[0])
+    got = host(ctx.hoisted_moddown(shared_pb, nq, True, b_premultiplied=True))
+    assert np.array_equal(got[0], orc.moddown_drop(want_shared, nq, True))
     # masked sums: out0 = m*ct0 + ct1, out1 = m'*ct2
     p1, p2 = orc.encode(z1, nq - 1), orc.encode(z2, nq - 1)
     dp1, dp2 = dev(p1.data), dev(p2.data)
