@@ -5,6 +5,7 @@
 
 #include "../../../include/hellm.h"
 #include "HELLM/HEMMer.hpp"
+#include "HELLM/PolyEval.hpp"
 #include "context_content.hpp"
 
 void hemm_set_error(const std::string &msg);
@@ -295,6 +296,36 @@ int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target, hellm_
     need(h && a && out, "null argument");
     hellm_ct *r = new hellm_ct{a->t};
     h->m->getEval().levelDown(a->t.get(), target, r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+
+int hellm_exp_iter(hellm_hemmer *h, const hellm_ct *a, int num_iter, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out && num_iter >= 0, "bad argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    HELLM::Exp::exp_iter(h->m->getEval(), h->m->getBtp(), a->t.get(), r->t.get(), num_iter);
+    *out = r;
+    FACADE_CATCH
+}
+int hellm_eval_odd_polynomial(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, int k, int l,
+                              hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && coeffs && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    HEaaN::Ciphertext x(a->t.get());
+    HELLM::ReLU::evalOddPolynomial(h->m->getEval(), x, r->t.get(), std::vector<double>(coeffs, coeffs + n_coeffs), k, l);
+    *out = r;
+    FACADE_CATCH
+}
+int hellm_eval_chebyshev(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, uint32_t baby_steps,
+                         double multiplier, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && coeffs && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    r->t.get() = HEaaN::Math::evaluateChebyshevExpansion(
+        h->m->getEval(), h->m->getBtp(), a->t.get(),
+        HEaaN::Math::ChebyshevCoefficients(std::vector<HEaaN::Real>(coeffs, coeffs + n_coeffs), baby_steps), multiplier);
     *out = r;
     FACADE_CATCH
 }

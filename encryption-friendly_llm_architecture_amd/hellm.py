@@ -66,6 +66,10 @@ def _L():
                   "hellm_matmul_pre", "hellm_matmul_pre_rev"):
             getattr(L, n).argtypes = [vp, vp, u32, pvp]
         L.hellm_repack_cc.argtypes = [vp, vp, pvp]
+        dp = ctypes.POINTER(ctypes.c_double)
+        L.hellm_exp_iter.argtypes = [vp, vp, ctypes.c_int, pvp]
+        L.hellm_eval_odd_polynomial.argtypes = [vp, vp, dp, u32, ctypes.c_int, ctypes.c_int, pvp]
+        L.hellm_eval_chebyshev.argtypes = [vp, vp, dp, u32, u32, ctypes.c_double, pvp]
         _declared = True
     return L
 
@@ -265,6 +269,20 @@ class HEMMer:
 
     def add(self, a, b):
         return self._new(Ct, "hellm_add", a.h, b.h)
+
+    def exp_iter(self, a, num_iter):
+        """(1 + a / 2^num_iter)^(2^num_iter) on the slots (HELLM::Exp::exp_iter)"""
+        return self._new(Ct, "hellm_exp_iter", a.h, num_iter)
+
+    def eval_odd_polynomial(self, a, coeffs, k, l):
+        """sum over odd i of coeffs[i] a^i (HELLM::ReLU::evalOddPolynomial)"""
+        c = (ctypes.c_double * len(coeffs))(*[float(x) for x in coeffs])
+        return self._new(Ct, "hellm_eval_odd_polynomial", a.h, c, len(coeffs), k, l)
+
+    def eval_chebyshev(self, a, coeffs, baby_steps, multiplier=1.0):
+        """multiplier * sum_k coeffs[k] T_k(a) for slot values in [-1, 1]"""
+        c = (ctypes.c_double * len(coeffs))(*[float(x) for x in coeffs])
+        return self._new(Ct, "hellm_eval_chebyshev", a.h, c, len(coeffs), baby_steps, float(multiplier))
 
     def level_down(self, a, target):
         return self._new(Ct, "hellm_level_down", a.h, target)

@@ -73,6 +73,18 @@ int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **
 int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ct **out);
 int hellm_mult_imag_unit(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);
 
+/* polynomial evaluation on the slots
+ * exp_iter: HELLM::Exp::exp_iter (src/Exp.cpp:41-52), (1 + x / 2^k)^(2^k);
+ * eval_odd_polynomial: HELLM::ReLU::evalOddPolynomial (src/ReLU.cpp:165-188), coeffs[i] = coefficient of x^i,
+ *   k baby steps (power of two), l giant-step powers;
+ * eval_chebyshev: HEaaN::Math::evaluateChebyshevExpansion (external/include/HEaaN-math/tools/PolynomialEvaluator.hpp:49-63),
+ *   multiplier * sum_k coeffs[k] T_k(x) for slot values in [-1, 1]. */
+int hellm_exp_iter(hellm_hemmer *h, const hellm_ct *a, int num_iter, hellm_ct **out);
+int hellm_eval_odd_polynomial(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, int k, int l,
+                              hellm_ct **out);
+int hellm_eval_chebyshev(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs,
+                         uint32_t baby_steps, double multiplier, hellm_ct **out);
+
 /* transforms and products */
 int hellm_diagonal_to_column(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out); /* MatrixTransformer :776 */
 int hellm_diagonal_to_row(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);    /* :924 */

@@ -96,6 +96,16 @@ class SlotSim:
             return self.rescale(self.mult_plain_no_rescale(x, y))
         return self.rescale(self.tensor(x, y))
 
+    def mult_const(self, x, c):
+        """HomEvaluator::mult(ct, constant): constants within 1e-8 of an integer do not use a level."""
+        if abs(c - round(c)) <= 1e-8:
+            return SimCt(x.z * round(c), x.level, x.rc)
+        assert x.rc == 0 and x.level >= 1
+        return SimCt(x.z * c, x.level - 1, 0)
+
+    def add_const(self, x, c):
+        return SimCt(x.z + c, x.level, x.rc)
+
     def mult_pt(self, x, pt):
         return self.rescale(self.mult_plain_no_rescale(x, pt))
 
@@ -185,6 +195,21 @@ class OracleEval:
 
     def mult_pt(self, x, pt):
         return self.rescale(self.mult_plain_no_rescale(x, pt))
+
+    def mult_const(self, x, c):
+        """HomEvaluator::mult(ct, real constant): an integer (within 1e-8) multiplies the residues and keeps
+        the level; anything else is multiplied by round(c * Delta_level) and rescaled."""
+        from .oracle import Ct
+        r = math.floor(c + 0.5)
+        if abs(c - r) <= 1e-8:
+            return self.o.mult_integer(x, int(r))
+        d = c * self.o.delta[x.level]
+        v = int(math.floor(abs(d) + 0.5)) * (1 if d >= 0 else -1)      # llround: halves away from zero
+        return self.o.rescale(Ct(self.o.mult_scalar_residues(x, v), x.scale * self.o.delta[x.level]))
+
+    def add_const(self, x, c):
+        import numpy as _np
+        return self.o.add(x, self.o.encode(_np.full(self.o.slots, c, dtype=_np.complex128), x.level))
 
     def mult_imag_unit(self, x):
         return self.o.mult_imag_unit(x)
