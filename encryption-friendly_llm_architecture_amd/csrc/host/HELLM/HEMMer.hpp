@@ -56,6 +56,19 @@ public:
     PtxtTensor encode(const Matrix &data, u64 level = 0) const;
     PtxtTensor encode2(const Matrix &a, const Matrix &b, u64 level = 0) const;
     Message msgDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4) const;
+    // Weight store (reference HEMMer::encodeWeight, src/HEMMer.cpp:437-482, and TransformerBlock::getWeight,
+    // src/TransformerBlock.cpp:11009-11031).  A weight given as a height x width grid of tiles is written as
+    //   <save_path><i>_<j>.msg = msgDiagonalToRow4(tile[4i][j], tile[4i+1][j], tile[4i+2][j], tile[4i+3][j])
+    // (the last group takes tiles height-2, height-1 and two zero tiles when height is not a multiple of 4);
+    // a list of tiles is written pairwise as <save_path><i>.msg = message2(tile[2i], tile[2i+1]).
+    // File format (this build's own; HEaaN's is closed): u64 log_slots, then 2^log_slots complex128 values.
+    void encodeWeight(const std::vector<std::vector<Matrix>> &grid, const std::string &save_path) const;
+    void encodeWeight(const std::vector<Matrix> &tiles, const std::string &save_path) const;
+    // reads one .msg file and encodes it at `level` as a pair-layout plaintext tile
+    PtxtTensor getWeight(const std::string &file, u64 level) const;
+    // ciphertext store: u64 {polynomials, level, rescale counter, N, rows, cols, block width}, then the residues
+    void saveCtxtTensor(const CtxtTensor &t, const std::string &file) const;
+    CtxtTensor loadCtxtTensor(const std::string &file) const;
     PtxtTensor encodeDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4,
                                     u64 level = 0) const;
     CtxtTensor encrypt(const Matrix &data) const;

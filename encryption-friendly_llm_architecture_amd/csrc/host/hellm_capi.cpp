@@ -156,6 +156,44 @@ int hellm_encode_diagonal_to_row4(hellm_hemmer *h, const double *w1, const doubl
                                                    mat(w4, rows, cols), level)};
     FACADE_CATCH
 }
+int hellm_encode_weight_grid(hellm_hemmer *h, const double *tiles, uint32_t height, uint32_t width, uint32_t rows,
+                             uint32_t cols, const char *save_path) {
+    FACADE_TRY
+    need(h && tiles && save_path, "null argument");
+    std::vector<std::vector<Matrix>> grid(height);
+    for (uint32_t i = 0; i < height; i++)
+        for (uint32_t j = 0; j < width; j++)
+            grid[i].push_back(mat(tiles + ((size_t)i * width + j) * rows * cols, rows, cols));
+    h->m->encodeWeight(grid, save_path);
+    FACADE_CATCH
+}
+int hellm_encode_weight_list(hellm_hemmer *h, const double *tiles, uint32_t count, uint32_t rows, uint32_t cols,
+                             const char *save_path) {
+    FACADE_TRY
+    need(h && tiles && save_path, "null argument");
+    std::vector<Matrix> v;
+    for (uint32_t i = 0; i < count; i++) v.push_back(mat(tiles + (size_t)i * rows * cols, rows, cols));
+    h->m->encodeWeight(v, save_path);
+    FACADE_CATCH
+}
+int hellm_get_weight(hellm_hemmer *h, const char *file, uint32_t level, hellm_pt **out) {
+    FACADE_TRY
+    need(h && file && out, "null argument");
+    *out = new hellm_pt{h->m->getWeight(file, level)};
+    FACADE_CATCH
+}
+int hellm_ct_save(hellm_hemmer *h, const hellm_ct *ct, const char *file) {
+    FACADE_TRY
+    need(h && ct && file, "null argument");
+    h->m->saveCtxtTensor(ct->t, file);
+    FACADE_CATCH
+}
+int hellm_ct_load(hellm_hemmer *h, const char *file, hellm_ct **out) {
+    FACADE_TRY
+    need(h && file && out, "null argument");
+    *out = new hellm_ct{h->m->loadCtxtTensor(file)};
+    FACADE_CATCH
+}
 int hellm_decrypt(hellm_hemmer *h, const hellm_ct *ct, double *out) {
     FACADE_TRY
     need(h && ct && out, "null argument");

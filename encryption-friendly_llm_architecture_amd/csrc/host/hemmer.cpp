@@ -2,6 +2,8 @@
 // matmul entry points :833-880,:964-1124, transpose :1166-1172, masks :2336-2400).
 #include <cmath>
 
+#include <fstream>
+
 #include "HELLM/HEMMer.hpp"
 
 namespace HELLM {
@@ -161,6 +163,51 @@ PtxtTensor HEMMer::encodeDiagonalToRow4(const Matrix &w1, const Matrix &w2, cons
     if (level == 0) level = getEncryptionLevel(context_);
     return PtxtTensor(w1.rows, w1.cols, endec_.encode(msg, level), w1.cols * 2);
 }
+void HEMMer::encodeWeight(const std::vector<std::vector<Matrix>> &grid, const std::string &save_path) const {
+    const size_t height = grid.size();
+    if (height == 0) throw std::invalid_argument("[encodeWeight] empty weight");
+    const size_t width = grid[0].size();
+    for (const auto &row : grid)
+        if (row.size() != width) throw std::invalid_argument("[encodeWeight] ragged tile grid");
+    for (size_t i = 0; i < height / 4; i++)
+        for (size_t j = 0; j < width; j++)
+            msgDiagonalToRow4(grid[4 * i][j], grid[4 * i + 1][j], grid[4 * i + 2][j], grid[4 * i + 3][j])
+                .save(save_path + std::to_string(i) + "_" + std::to_string(j) + ".msg");
+    if (height % 4 > 0) {
+        if (height < 2) throw std::invalid_argument("[encodeWeight] a trailing group needs two tile rows");
+        const Matrix zero(dim_, dim_, 0.0);
+        for (size_t j = 0; j < width; j++)
+            msgDiagonalToRow4(grid[height - 2][j], grid[height - 1][j], zero, zero)
+                .save(save_path + std::to_string(height / 4) + "_" + std::to_string(j) + ".msg");
+    }
+}
+void HEMMer::encodeWeight(const std::vector<Matrix> &tiles, const std::string &save_path) const {
+    for (size_t i = 0; i < tiles.size() / 2; i++)
+        message2(tiles[2 * i], tiles[2 * i + 1]).save(save_path + std::to_string(i) + ".msg");
+}
+PtxtTensor HEMMer::getWeight(const std::string &file, u64 level) const {
+    Message msg(log_slots_);
+    msg.load(file);
+    if (msg.getLogSlots() != log_slots_) throw RuntimeException("weight file does not match the slot count: " + file);
+    return PtxtTensor(dim_, dim_, endec_.encode(msg, level), 2 * dim_);
+}
+void HEMMer::saveCtxtTensor(const CtxtTensor &t, const std::string &file) const {
+    t.get().save(file);
+    std::ofstream f(file + ".shape", std::ios::binary);
+    if (!f) throw RuntimeException("cannot open " + file + ".shape");
+    const i64 shape[3] = {t.getHeight(), t.getWidth(), t.getBlockWidth()};
+    f.write((const char *)shape, sizeof(shape));
+}
+CtxtTensor HEMMer::loadCtxtTensor(const std::string &file) const {
+    std::ifstream f(file + ".shape", std::ios::binary);
+    if (!f) throw RuntimeException("cannot open " + file + ".shape");
+    i64 shape[3];
+    f.read((char *)shape, sizeof(shape));
+    CtxtTensor t(context_, shape[0], shape[1], shape[2]);
+    t.get().load(file);
+    return t;
+}
+
 CtxtTensor HEMMer::encrypt(const Matrix &data) const {
     PtxtTensor p = encode(data);
     CtxtTensor ret(context_, p.getShape());

@@ -67,6 +67,11 @@ def _L():
             getattr(L, n).argtypes = [vp, vp, u32, pvp]
         L.hellm_repack_cc.argtypes = [vp, vp, pvp]
         dp = ctypes.POINTER(ctypes.c_double)
+        L.hellm_encode_weight_grid.argtypes = [vp, dp, u32, u32, u32, u32, ctypes.c_char_p]
+        L.hellm_encode_weight_list.argtypes = [vp, dp, u32, u32, u32, ctypes.c_char_p]
+        L.hellm_get_weight.argtypes = [vp, ctypes.c_char_p, u32, pvp]
+        L.hellm_ct_save.argtypes = [vp, vp, ctypes.c_char_p]
+        L.hellm_ct_load.argtypes = [vp, ctypes.c_char_p, pvp]
         L.hellm_exp_iter.argtypes = [vp, vp, ctypes.c_int, pvp]
         L.hellm_eval_odd_polynomial.argtypes = [vp, vp, dp, u32, ctypes.c_int, ctypes.c_int, pvp]
         L.hellm_eval_chebyshev.argtypes = [vp, vp, dp, u32, u32, ctypes.c_double, pvp]
@@ -269,6 +274,29 @@ class HEMMer:
 
     def add(self, a, b):
         return self._new(Ct, "hellm_add", a.h, b.h)
+
+    def encode_weight(self, tiles, save_path):
+        """HEMMer::encodeWeight: tiles [height][width][rows][cols] -> <save_path><i>_<j>.msg (diagonal-to-row
+        packing of four tile rows), or [count][rows][cols] -> <save_path><i>.msg (pairs of tiles)."""
+        import numpy as np
+        t = np.ascontiguousarray(tiles, dtype=np.float64)
+        p = t.ctypes.data_as(ctypes.POINTER(ctypes.c_double))
+        if t.ndim == 4:
+            check(_L().hellm_encode_weight_grid(self.h, p, t.shape[0], t.shape[1], t.shape[2], t.shape[3],
+                                                str(save_path).encode()))
+        elif t.ndim == 3:
+            check(_L().hellm_encode_weight_list(self.h, p, t.shape[0], t.shape[1], t.shape[2], str(save_path).encode()))
+        else:
+            raise ValueError("tiles must have 3 or 4 dimensions")
+
+    def get_weight(self, file, level):
+        return self._new(Pt, "hellm_get_weight", str(file).encode(), level)
+
+    def save_ct(self, ct, file):
+        check(_L().hellm_ct_save(self.h, ct.h, str(file).encode()))
+
+    def load_ct(self, file):
+        return self._new(Ct, "hellm_ct_load", str(file).encode())
 
     def exp_iter(self, a, num_iter):
         """(1 + a / 2^num_iter)^(2^num_iter) on the slots (HELLM::Exp::exp_iter)"""

@@ -73,6 +73,20 @@ int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **
 int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ct **out);
 int hellm_mult_imag_unit(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);
 
+/* weight and ciphertext stores (formats are this build's own; HEaaN's are closed).
+ * encode_weight_grid: HEMMer::encodeWeight on a height x width grid of rows x cols tiles (src/HEMMer.cpp:437-482):
+ *   writes <save_path><i>_<j>.msg = msgDiagonalToRow4 of tile rows 4i..4i+3 of column j;
+ * encode_weight_list: the 3-D case, <save_path><i>.msg = message2(tile[2i], tile[2i+1]);
+ * get_weight: TransformerBlock::getWeight (src/TransformerBlock.cpp:11009-11031): load one .msg file and encode it;
+ * ct_save / ct_load: the ciphertext store of src/LoRA.cpp:732-801 (file + file.shape). */
+int hellm_encode_weight_grid(hellm_hemmer *h, const double *tiles, uint32_t height, uint32_t width, uint32_t rows,
+                             uint32_t cols, const char *save_path);
+int hellm_encode_weight_list(hellm_hemmer *h, const double *tiles, uint32_t count, uint32_t rows, uint32_t cols,
+                             const char *save_path);
+int hellm_get_weight(hellm_hemmer *h, const char *file, uint32_t level, hellm_pt **out);
+int hellm_ct_save(hellm_hemmer *h, const hellm_ct *ct, const char *file);
+int hellm_ct_load(hellm_hemmer *h, const char *file, hellm_ct **out);
+
 /* polynomial evaluation on the slots
  * exp_iter: HELLM::Exp::exp_iter (src/Exp.cpp:41-52), (1 + x / 2^k)^(2^k);
  * eval_odd_polynomial: HELLM::ReLU::evalOddPolynomial (src/ReLU.cpp:165-188), coeffs[i] = coefficient of x^i,

@@ -255,6 +255,34 @@ def test_reuse_variants_and_repacking(small, fused):
     assert np.abs(out - want).max() < 2 ** -18
 
 
+def test_weight_and_ciphertext_stores(small, tmp_path):
+    """encodeWeight / getWeight and the ciphertext store: what is read back is what was written."""
+    H, orc, ev = small
+    n = 16
+    rng = np.random.default_rng(10)
+    grid = rng.normal(0, 0.02, (6, 2, n, n))                 # 6 tile rows (one full group of 4 + a trailing pair) x 2
+    H.encode_weight(grid, str(tmp_path / "w_"))
+    for i, j, rows in ((0, 0, (0, 1, 2, 3)), (0, 1, (0, 1, 2, 3)), (1, 0, (4, 5, None, None))):
+        w = [grid[r][j] if r is not None else np.zeros((n, n)) for r in rows]
+        got = H.get_weight(str(tmp_path / ("w_%d_%d.msg" % (i, j))), 3)
+        want = H.encode_diagonal_to_row4(*w, level=3)
+        assert np.array_equal(got.residues(), want.residues())
+    H.encode_weight(grid[:4, 0], str(tmp_path / "v_"))       # list of tiles -> pairs
+    got = H.get_weight(str(tmp_path / "v_1.msg"), 2)
+    assert np.array_equal(got.residues(), H.encode2(grid[2, 0], grid[3, 0], level=2).residues())
+    with pytest.raises(pkg_error()):
+        H.get_weight(str(tmp_path / "missing.msg"), 2)
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    ct = H.level_down(H.encrypt2(A, B), 5)
+    H.save_ct(ct, str(tmp_path / "ct.bin"))
+    back = H.load_ct(str(tmp_path / "ct.bin"))
+    assert back.info() == ct.info()
+    assert np.array_equal(back.residues(), ct.residues())
+    c = H.single_cc_matmul(back, H.encrypt2(B, A), 2)          # the loaded tensor keeps its tile shape
+    d = H.decrypt2(c)
+    assert np.abs(d[0] - A @ B).max() < 2 ** -18 and np.abs(d[1] - B @ A).max() < 2 ** -18
+
+
 def test_error_behaviour(small):
     H, _, _ = small
     A = np.ones((16, 16))
