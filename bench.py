@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HEMMer hot path on one MI355X.
 
-Headline (the metric BASELINE.json names): ms per 128 x 128 ciphertext-ciphertext matrix product
+Headline metric: ms per 128 x 128 ciphertext-ciphertext matrix product
 (HEMMer::singleCCMatMul, N = 2^16, 13 + 4 primes, dnum 3, scale 2^42, inputs fresh at level 12,
 target level 4), inputs and keys resident in HBM.  Also reported in the same JSON line: one
 key-switched rotation at levels 12 and 6, batched NTT limb-transforms/s, the roofline of the

@@ -64,7 +64,7 @@ inline unsigned bitrev(unsigned x, int bits) {
     return r;
 }
 
-// splitmix64 finaliser used as a counter-based generator (documented in DESIGN.md).
+// splitmix64 finaliser used as a counter-based generator: draw(key, ctr) = sm64(key + ctr * golden-ratio constant).
 inline u64 sm64(u64 x) {
     x += 0x9E3779B97F4A7C15ull;
     u64 z = x;
