@@ -56,6 +56,22 @@ public:
     PtxtTensor encode(const Matrix &data, u64 level = 0) const;
     PtxtTensor encode2(const Matrix &a, const Matrix &b, u64 level = 0) const;
     Message msgDiagonalToRow4(const Matrix &w1, const Matrix &w2, const Matrix &w3, const Matrix &w4) const;
+    // Rotate-and-sum reductions on the pair layout (reference src/HEMMer.cpp):
+    //   reduceRowSumWithScaledMask :2512-2530  sum every tile row over the block width (log-step left rotations),
+    //                                          multiply by `mask`, spread the kept values back over the row
+    //                                          (log-step right rotations);
+    //   oneMatRotSumInplace :882-919           row sums of a over half a row into column 0 / of b into the last
+    //                                          column, masked and spread over the whole row;
+    //   maskRightLeft :1245-1249, maskFirstColInplace :1251-1253;
+    //   rowMoments                             the first half of LayerNorm :1699-1760: over a list of tiles,
+    //                                          mean and mean of squares of every token row (scaled by `inv_count`
+    //                                          in column 0, then spread over the row), one level each.
+    void reduceRowSumWithScaledMask(CtxtTensor &tensor, const Message &mask) const;
+    void oneMatRotSumInplace(CtxtTensor &tensor_a, CtxtTensor &tensor_b) const;
+    void maskRightLeft(const CtxtTensor &tensor, CtxtTensor &out_left, CtxtTensor &out_right) const;
+    void maskFirstColInplace(CtxtTensor &tensor) const;
+    void rowMoments(const std::vector<CtxtTensor> &tiles, Real inv_count, CtxtTensor &mean, CtxtTensor &mean_square) const;
+
     // Weight store (reference HEMMer::encodeWeight, src/HEMMer.cpp:437-482, and TransformerBlock::getWeight,
     // src/TransformerBlock.cpp:11009-11031).  A weight given as a height x width grid of tiles is written as
     //   <save_path><i>_<j>.msg = msgDiagonalToRow4(tile[4i][j], tile[4i+1][j], tile[4i+2][j], tile[4i+3][j])

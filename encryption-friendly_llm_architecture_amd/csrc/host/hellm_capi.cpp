@@ -156,6 +156,49 @@ int hellm_encode_diagonal_to_row4(hellm_hemmer *h, const double *w1, const doubl
                                                    mat(w4, rows, cols), level)};
     FACADE_CATCH
 }
+int hellm_reduce_row_sum_with_scaled_mask(hellm_hemmer *h, hellm_ct *a, const double *mask_left, const double *mask_right,
+                                          uint32_t rows, uint32_t cols) {
+    FACADE_TRY
+    need(h && a && mask_left && mask_right, "null argument");
+    h->m->reduceRowSumWithScaledMask(a->t, h->m->message2(mat(mask_left, rows, cols), mat(mask_right, rows, cols)));
+    FACADE_CATCH
+}
+int hellm_one_mat_rot_sum_inplace(hellm_hemmer *h, hellm_ct *a, hellm_ct *b) {
+    FACADE_TRY
+    need(h && a && b, "null argument");
+    h->m->oneMatRotSumInplace(a->t, b->t);
+    FACADE_CATCH
+}
+int hellm_mask_right_left(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out_left, hellm_ct **out_right) {
+    FACADE_TRY
+    need(h && a && out_left && out_right, "null argument");
+    hellm_ct *l = new hellm_ct{a->t}, *r = new hellm_ct{a->t};
+    h->m->maskRightLeft(a->t, l->t, r->t);
+    *out_left = l;
+    *out_right = r;
+    FACADE_CATCH
+}
+int hellm_mask_first_col_inplace(hellm_hemmer *h, hellm_ct *a) {
+    FACADE_TRY
+    need(h && a, "null argument");
+    h->m->maskFirstColInplace(a->t);
+    FACADE_CATCH
+}
+int hellm_row_moments(hellm_hemmer *h, const hellm_ct *const *tiles, uint32_t count, double inv_count, hellm_ct **mean,
+                      hellm_ct **mean_square) {
+    FACADE_TRY
+    need(h && tiles && count >= 1 && mean && mean_square, "null argument");
+    std::vector<HELLM::CtxtTensor> v;
+    for (uint32_t i = 0; i < count; i++) {
+        need(tiles[i] != nullptr, "null tile");
+        v.push_back(tiles[i]->t);
+    }
+    hellm_ct *m = new hellm_ct{v[0]}, *sq = new hellm_ct{v[0]};
+    h->m->rowMoments(v, inv_count, m->t, sq->t);
+    *mean = m;
+    *mean_square = sq;
+    FACADE_CATCH
+}
 int hellm_encode_weight_grid(hellm_hemmer *h, const double *tiles, uint32_t height, uint32_t width, uint32_t rows,
                              uint32_t cols, const char *save_path) {
     FACADE_TRY

@@ -163,6 +163,95 @@ PtxtTensor HEMMer::encodeDiagonalToRow4(const Matrix &w1, const Matrix &w2, cons
     if (level == 0) level = getEncryptionLevel(context_);
     return PtxtTensor(w1.rows, w1.cols, endec_.encode(msg, level), w1.cols * 2);
 }
+// ---- rotate-and-sum reductions -----------------------------------------------------------------------
+namespace {
+std::vector<u64> logSteps(u64 bound, u64 slots) {
+    std::vector<u64> r;
+    for (u64 i = 1; i < bound; i <<= 1) {
+        r.push_back(i);
+        r.push_back(slots - i);
+    }
+    return r;
+}
+}  // namespace
+
+void HEMMer::reduceRowSumWithScaledMask(CtxtTensor &tensor, const Message &mask) const {
+    const u64 w = (u64)tensor.getBlockWidth(), slots = u64(1) << log_slots_;
+    ensureRotationKeys(logSteps(w, slots));
+    Ciphertext tmp(context_);
+    for (u64 i = 1; i < w; i <<= 1) {
+        eval_.leftRotate(tensor.get(), i, tmp);
+        eval_.add(tensor.get(), tmp, tensor.get());
+    }
+    eval_.mult(tensor.get(), mask, tensor.get());
+    for (u64 i = 1; i < w; i <<= 1) {
+        eval_.rightRotate(tensor.get(), i, tmp);
+        eval_.add(tensor.get(), tmp, tensor.get());
+    }
+}
+
+void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
+    const u64 n = (u64)dim_, slots = u64(1) << log_slots_;
+    ensureRotationKeys(logSteps(n, slots));
+    Ciphertext tmp(context_);
+    for (u64 rot = 1; rot < n / 2; rot <<= 1) {
+        eval_.leftRotate(a.get(), rot, tmp);
+        eval_.add(a.get(), tmp, a.get());
+        eval_.rightRotate(b.get(), rot, tmp);
+        eval_.add(b.get(), tmp, b.get());
+    }
+    Matrix first(dim_, dim_, 0.0), last(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++) {
+        first.at(r, 0) = 1.0;
+        last.at(r, dim_ - 1) = 1.0;
+    }
+    eval_.mult(a.get(), message2(first, first), a.get());
+    eval_.mult(b.get(), message2(last, last), b.get());
+    for (u64 rot = 1; rot < n; rot <<= 1) {
+        eval_.rightRotate(a.get(), rot, tmp);
+        eval_.add(a.get(), tmp, a.get());
+        eval_.leftRotate(b.get(), rot, tmp);
+        eval_.add(b.get(), tmp, b.get());
+    }
+}
+
+void HEMMer::maskRightLeft(const CtxtTensor &tensor, CtxtTensor &out_left, CtxtTensor &out_right) const {
+    Matrix left(dim_, dim_, 0.0), right(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++)
+        for (i64 c = 0; c < dim_; c++) (c < dim_ / 2 ? left : right).at(r, c) = 1.0;
+    eval_.mult(tensor.get(), message2(left, left), out_left.get());
+    eval_.mult(tensor.get(), message2(right, right), out_right.get());
+}
+
+void HEMMer::maskFirstColInplace(CtxtTensor &tensor) const {
+    Matrix first(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++) first.at(r, 0) = 1.0;
+    eval_.mult(tensor.get(), message2(first, first), tensor.get());
+}
+
+void HEMMer::rowMoments(const std::vector<CtxtTensor> &tiles, Real inv_count, CtxtTensor &mean,
+                        CtxtTensor &mean_square) const {
+    if (tiles.empty()) throw std::invalid_argument("[rowMoments] no tiles");
+    const u64 w = (u64)tiles[0].getBlockWidth(), slots = u64(1) << log_slots_;
+    ensureRotationKeys(logSteps(w, slots));
+    Ciphertext tmp(context_);
+    mean.get() = tiles[0].get();
+    eval_.tensor(tiles[0].get(), tiles[0].get(), mean_square.get());
+    for (size_t i = 1; i < tiles.size(); i++) {
+        eval_.tensor(tiles[i].get(), tiles[i].get(), tmp);
+        eval_.add(mean_square.get(), tmp, mean_square.get());
+        eval_.add(mean.get(), tiles[i].get(), mean.get());
+    }
+    eval_.relinearize(mean_square.get(), mean_square.get());
+    eval_.rescale(mean_square.get());
+    // both halves of the pair layout are summed together (one token row spans the whole block width)
+    Matrix scaled(dim_, dim_, 0.0), zero(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++) scaled.at(r, 0) = inv_count;
+    const Message mask = message2(scaled, zero);
+    reduceRowSumWithScaledMask(mean_square, mask);
+    reduceRowSumWithScaledMask(mean, mask);
+}
+
 void HEMMer::encodeWeight(const std::vector<std::vector<Matrix>> &grid, const std::string &save_path) const {
     const size_t height = grid.size();
     if (height == 0) throw std::invalid_argument("[encodeWeight] empty weight");

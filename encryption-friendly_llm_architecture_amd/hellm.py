@@ -67,6 +67,11 @@ def _L():
             getattr(L, n).argtypes = [vp, vp, u32, pvp]
         L.hellm_repack_cc.argtypes = [vp, vp, pvp]
         dp = ctypes.POINTER(ctypes.c_double)
+        L.hellm_reduce_row_sum_with_scaled_mask.argtypes = [vp, vp, dp, dp, u32, u32]
+        L.hellm_one_mat_rot_sum_inplace.argtypes = [vp, vp, vp]
+        L.hellm_mask_right_left.argtypes = [vp, vp, pvp, pvp]
+        L.hellm_mask_first_col_inplace.argtypes = [vp, vp]
+        L.hellm_row_moments.argtypes = [vp, ctypes.POINTER(vp), u32, ctypes.c_double, pvp, pvp]
         L.hellm_encode_weight_grid.argtypes = [vp, dp, u32, u32, u32, u32, ctypes.c_char_p]
         L.hellm_encode_weight_list.argtypes = [vp, dp, u32, u32, u32, ctypes.c_char_p]
         L.hellm_get_weight.argtypes = [vp, ctypes.c_char_p, u32, pvp]
@@ -274,6 +279,31 @@ class HEMMer:
 
     def add(self, a, b):
         return self._new(Ct, "hellm_add", a.h, b.h)
+
+    def reduce_row_sum_with_scaled_mask(self, a, mask_left, mask_right):
+        import numpy as np
+        ml = np.ascontiguousarray(mask_left, dtype=np.float64)
+        mr = np.ascontiguousarray(mask_right, dtype=np.float64)
+        dp = ctypes.POINTER(ctypes.c_double)
+        check(_L().hellm_reduce_row_sum_with_scaled_mask(self.h, a.h, ml.ctypes.data_as(dp), mr.ctypes.data_as(dp),
+                                                         ml.shape[0], ml.shape[1]))
+
+    def one_mat_rot_sum_inplace(self, a, b):
+        check(_L().hellm_one_mat_rot_sum_inplace(self.h, a.h, b.h))
+
+    def mask_right_left(self, a):
+        h1, h2 = vp(), vp()
+        check(_L().hellm_mask_right_left(self.h, a.h, ctypes.byref(h1), ctypes.byref(h2)))
+        return Ct(self, h1), Ct(self, h2)
+
+    def mask_first_col_inplace(self, a):
+        check(_L().hellm_mask_first_col_inplace(self.h, a.h))
+
+    def row_moments(self, tiles, inv_count):
+        arr = (vp * len(tiles))(*[t.h for t in tiles])
+        h1, h2 = vp(), vp()
+        check(_L().hellm_row_moments(self.h, arr, len(tiles), float(inv_count), ctypes.byref(h1), ctypes.byref(h2)))
+        return Ct(self, h1), Ct(self, h2)
 
     def encode_weight(self, tiles, save_path):
         """HEMMer::encodeWeight: tiles [height][width][rows][cols] -> <save_path><i>_<j>.msg (diagonal-to-row

@@ -73,6 +73,18 @@ int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **
 int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ct **out);
 int hellm_mult_imag_unit(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);
 
+/* rotate-and-sum reductions on the pair layout (src/HEMMer.cpp:2512-2530, 882-919, 1245-1253, 1699-1760):
+ * reduce_row_sum_with_scaled_mask: sum each tile row over the block width, multiply by message2(mask_left, mask_right),
+ *   spread the kept values over the row; one_mat_rot_sum_inplace; mask_right_left; mask_first_col_inplace;
+ * row_moments: per token row, mean and mean of squares over `count` tiles (scaled by inv_count), spread over the row. */
+int hellm_reduce_row_sum_with_scaled_mask(hellm_hemmer *h, hellm_ct *a, const double *mask_left,
+                                          const double *mask_right, uint32_t rows, uint32_t cols);
+int hellm_one_mat_rot_sum_inplace(hellm_hemmer *h, hellm_ct *a, hellm_ct *b);
+int hellm_mask_right_left(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out_left, hellm_ct **out_right);
+int hellm_mask_first_col_inplace(hellm_hemmer *h, hellm_ct *a);
+int hellm_row_moments(hellm_hemmer *h, const hellm_ct *const *tiles, uint32_t count, double inv_count, hellm_ct **mean,
+                      hellm_ct **mean_square);
+
 /* weight and ciphertext stores (formats are this build's own; HEaaN's are closed).
  * encode_weight_grid: HEMMer::encodeWeight on a height x width grid of rows x cols tiles (src/HEMMer.cpp:437-482):
  *   writes <save_path><i>_<j>.msg = msgDiagonalToRow4 of tile rows 4i..4i+3 of column j;

@@ -645,3 +645,66 @@ def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
         msg[np.arange(h) * 2 * w + c] = np.roll(left[:, c], -c)
         msg[np.arange(h) * 2 * w + w + c] = np.roll(right[:, c], -c)
     return msg
+
+
+# ---- rotate-and-sum reductions on the pair layout (HEMMer.cpp:2512-2530, 882-919, 1245-1253, 1699-1760) -----------
+def _message2(a, b, slots):
+    """HEMMer::message2 (HEMMer.cpp:243-262): [A | B] row-major with block width 2 * cols."""
+    n = a.shape[1]
+    m = np.zeros(slots, dtype=np.complex128)
+    m[: 2 * a.size] = np.concatenate([a, b], axis=1).reshape(-1)
+    return m
+
+
+def reduce_row_sum_with_scaled_mask(ev, x, mask_msg, w):
+    i = 1
+    while i < w:
+        x = ev.add(x, ev.left_rotate(x, i))
+        i <<= 1
+    x = ev.mult_pt(x, ev.encode(mask_msg, ev.level_of(x)))
+    i = 1
+    while i < w:
+        x = ev.add(x, ev.right_rotate(x, i))
+        i <<= 1
+    return x
+
+
+def one_mat_rot_sum(ev, a, b, n):
+    rot = 1
+    while rot < n // 2:
+        a = ev.add(a, ev.left_rotate(a, rot))
+        b = ev.add(b, ev.right_rotate(b, rot))
+        rot <<= 1
+    first, last = np.zeros((n, n)), np.zeros((n, n))
+    first[:, 0] = 1.0
+    last[:, n - 1] = 1.0
+    a = ev.mult_pt(a, ev.encode(_message2(first, first, ev.slots), ev.level_of(a)))
+    b = ev.mult_pt(b, ev.encode(_message2(last, last, ev.slots), ev.level_of(b)))
+    rot = 1
+    while rot < n:
+        a = ev.add(a, ev.right_rotate(a, rot))
+        b = ev.add(b, ev.left_rotate(b, rot))
+        rot <<= 1
+    return a, b
+
+
+def mask_right_left(ev, x, n):
+    left, right = np.zeros((n, n)), np.zeros((n, n))
+    left[:, : n // 2] = 1.0
+    right[:, n // 2:] = 1.0
+    return (ev.mult_pt(x, ev.encode(_message2(left, left, ev.slots), ev.level_of(x))),
+            ev.mult_pt(x, ev.encode(_message2(right, right, ev.slots), ev.level_of(x))))
+
+
+def row_moments(ev, tiles, inv_count, n):
+    mean = tiles[0]
+    sq = ev.tensor(tiles[0], tiles[0])
+    for t in tiles[1:]:
+        sq = ev.add(sq, ev.tensor(t, t))
+        mean = ev.add(mean, t)
+    sq = ev.rescale(ev.relinearize(sq))
+    scaled = np.zeros((n, n))
+    scaled[:, 0] = inv_count
+    mask = _message2(scaled, np.zeros((n, n)), ev.slots)
+    return (reduce_row_sum_with_scaled_mask(ev, mean, mask, 2 * n),
+            reduce_row_sum_with_scaled_mask(ev, sq, mask, 2 * n))

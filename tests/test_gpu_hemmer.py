@@ -255,6 +255,42 @@ def test_reuse_variants_and_repacking(small, fused):
     assert np.abs(out - want).max() < 2 ** -18
 
 
+def test_rotate_and_sum_reductions(small):
+    """Row reductions on the pair layout: residues against the oracle restatement, values against numpy."""
+    H, orc, ev = small
+    n = 16
+    rng = np.random.default_rng(13)
+    A, B = rng.normal(size=(n, n)), rng.normal(size=(n, n))
+    x = H.encrypt2(A, B)
+    ox = to_oracle(orc, x)
+    scaled = np.zeros((n, n))
+    scaled[:, 0] = 1.0 / (2 * n)
+    got = x.clone()
+    H.reduce_row_sum_with_scaled_mask(got, scaled, np.zeros((n, n)))
+    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n)
+    assert np.array_equal(got.residues(), want.data)
+    d = H.decrypt2(got)
+    mean = np.concatenate([A, B], axis=1).mean(axis=1, keepdims=True)
+    assert np.abs(d[0] - mean).max() < 2 ** -20 and np.abs(d[1] - mean).max() < 2 ** -20
+    a, b = x.clone(), x.clone()
+    H.one_mat_rot_sum_inplace(a, b)
+    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n)
+    assert np.array_equal(a.residues(), wa.data) and np.array_equal(b.residues(), wb.data)
+    assert np.abs(H.decrypt2(a)[1] - B[:, : n // 2].sum(axis=1, keepdims=True)).max() < 2 ** -18
+    l, r = H.mask_right_left(x)
+    wl, wr = R.mask_right_left(ev, ox, n)
+    assert np.array_equal(l.residues(), wl.data) and np.array_equal(r.residues(), wr.data)
+    assert np.abs(H.decrypt2(l)[0][:, : n // 2] - A[:, : n // 2]).max() < 2 ** -20
+    assert np.abs(H.decrypt2(l)[0][:, n // 2:]).max() < 2 ** -20
+    tiles = [H.encrypt2(rng.normal(size=(n, n)), rng.normal(size=(n, n))) for _ in range(3)]
+    rows = np.concatenate([np.concatenate(H.decrypt2(t), axis=1) for t in tiles], axis=1)
+    m, sq = H.row_moments(tiles, 1.0 / rows.shape[1])
+    wm, wsq = R.row_moments(ev, [to_oracle(orc, t) for t in tiles], 1.0 / rows.shape[1], n)
+    assert np.array_equal(m.residues(), wm.data) and np.array_equal(sq.residues(), wsq.data)
+    assert np.abs(H.decrypt2(m)[0] - rows.mean(axis=1, keepdims=True)).max() < 2 ** -18
+    assert np.abs(H.decrypt2(sq)[1] - (rows ** 2).mean(axis=1, keepdims=True)).max() < 2 ** -16
+
+
 def test_weight_and_ciphertext_stores(small, tmp_path):
     """encodeWeight / getWeight and the ciphertext store: what is read back is what was written."""
     H, orc, ev = small
