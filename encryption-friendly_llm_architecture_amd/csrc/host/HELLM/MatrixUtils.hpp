@@ -118,6 +118,9 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
                                  u64 batch = 16);
 void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
                         MatrixTransformer &transformer, u64 batch = 16);
+// plaintext x ciphertext product for tiles whose rows fill the slot vector (pair layout)
+CtxtTensor multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                                const PtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16);
 // left rotations (in slots) whose direct keys the batched schedules use
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 

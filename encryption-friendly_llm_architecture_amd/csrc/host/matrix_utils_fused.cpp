@@ -577,3 +577,36 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
 }
 
 }  // namespace HELLM
+
+namespace HELLM {
+
+// Plaintext x ciphertext product for tiles whose rows fill the slot vector (rows * block width == slots, the
+// pair layout): the row shifts of tau(B) are then whole rotations of one encoded plaintext, so the product is
+// the hoisted column shifts of sigma(A) (multMatMatPreFused) followed by one masked-sum launch that reads
+// tau(B) through each term's automorphism:  rescale(sum_k shift_k(sigma A) (.) rot(tau B, k w)).
+CtxtTensor multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
+                                const PtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch) {
+    const Context &c = eval.getContext();
+    const i64 rows = op1.getHeight(), cols = op2.getWidth();
+    const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
+    if (std::min(op1.getLevel(), op2.getLevel()) < 1 + btp.getMinLevelForBootstrap())
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(1 + btp.getMinLevelForBootstrap()) +
+                                    " is needed.");
+    if ((u64)(k * w) != c->N / 2)
+        throw std::invalid_argument("[multMatMatPlainFused] the row shift must be cyclic: rows * block width == slots");
+    CtxtTensor a{op1};
+    PtxtTensor b{op2};
+    a.setShape(rows, k);
+    b.setShape(k, cols);
+    if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
+    std::vector<Ciphertext> shifts;
+    multMatMatPreFused(eval, a, shifts, T, tr, batch);
+    b = tr.diagonalToRow(eval, b);
+    EnDecoder endec(c);
+    if (b.getLevel() != T + 1) b.get() = endec.encode(endec.decode(b.get()), T + 1);
+    CtxtTensor res(c, rows, cols, w);
+    eval.matmul(shifts, b.get(), res.get());   // rotation step slots / k == w
+    return res;
+}
+
+}  // namespace HELLM

@@ -635,6 +635,16 @@ def mult_mat_mat_pre_fused(orc, a, T, n, w):
         orc, a, ext, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
 
 
+def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
+    """Batched plaintext x ciphertext product for rows * block width == slots: hoisted column shifts of
+    sigma(A), then rescale(sum_k shift_k (.) rot(tau(B), k w))."""
+    ev = OracleEval(orc)
+    assert n * w == orc.slots
+    tmp = mult_mat_mat_pre_fused(orc, a, T, n, w)
+    b = ev.encode(tau_plain(ev.pt_values(b_pt), n, w), ev.level_of(b_pt))
+    return mult_mat_mat_reuse(ev, tmp, b, T)
+
+
 def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
     """HEMMer::msgDiagonalToRow4 (HEMMer.cpp:353-399)."""
     h, w = w1.shape

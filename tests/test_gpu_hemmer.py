@@ -136,6 +136,26 @@ def test_ccmm_pair_layout(small, fused):
     assert np.abs(d[0] - A1 @ B1).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_pcmm_pair_layout(small, fused):
+    """Plaintext x ciphertext product on the pair layout (two products per call); the batched schedule takes the
+    hoisted route because the plaintext's row shifts are whole rotations there."""
+    H, orc, ev = small
+    H.set_schedule(fused, batch=5)
+    rng = np.random.default_rng(14)
+    A1, A2, B1, B2 = (rng.uniform(-1, 1, (16, 16)) for _ in range(4))
+    ca = H.encrypt2(A1, A2)
+    pb = H.encode2(B1, B2)
+    c = H.single_matmul(ca, pb, 2)
+    H.set_schedule(True)
+    opb = O.Pt(pb.residues(), orc.delta[orc.nQ - 1])
+    oa = to_oracle(orc, ca)
+    want = R.mult_mat_mat_pc_fused(orc, oa, opb, 2, 16, 32) if fused else R.mult_mat_mat_pc(ev, oa, opb, 2, 16, 32)
+    assert np.array_equal(c.residues(), want.data)
+    d = H.decrypt2(c)
+    assert np.abs(d[0] - A1 @ B1).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
+
+
 def test_batch_size_does_not_change_residues(small):
     H, _, _ = small
     rng = np.random.default_rng(14)
