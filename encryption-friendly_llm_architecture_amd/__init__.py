@@ -66,6 +66,8 @@ def _declare(L):
     L.hemm_rotate.argtypes = [vp, vp, sz, vp, u64, u32, vp, sz, vp]
     L.hemm_relinearize.argtypes = [vp, vp, sz, vp, u32, vp, sz, vp]
     L.hemm_rescale.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
+    L.hemm_sample_uniform.argtypes = [vp, u64p, u32p, u32, vp, vp]
+    L.hemm_sample_error.argtypes = [vp, u64, u32p, u32, vp, vp]
     L.hemm_modup_batch.argtypes = [vp, vp, sz, u32, u32, vp, vp, vp]
     L.hemm_hoisted_terms.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, vp, ci, vp]
     L.hemm_moddown_batch.argtypes = [vp, vp, u32, u32, ci, vp, sz, vp, vp]
@@ -177,6 +179,25 @@ class Context:
     def beta(self, nq):
         alpha = -(-self.nQ // self.dnum)
         return -(-nq // alpha)
+
+    def sample_uniform(self, stream_keys, prime_idx):
+        """out[j] uniform mod prime prime_idx[j] from stream key stream_keys[j] (counter-based, masked rejection)"""
+        import torch
+        n = len(prime_idx)
+        out = torch.empty((n, self.N), dtype=torch.int64, device="cuda")
+        keys = (ctypes.c_uint64 * n)(*[int(k) for k in stream_keys])
+        idx = (ctypes.c_uint32 * n)(*prime_idx)
+        check(lib().hemm_sample_uniform(self.h, keys, idx, n, vp(out.data_ptr()), vp(0)))
+        return out
+
+    def sample_error(self, stream_key, prime_idx):
+        """residues of the centred-binomial error polynomial of a stream (coefficient form)"""
+        import torch
+        n = len(prime_idx)
+        out = torch.empty((n, self.N), dtype=torch.int64, device="cuda")
+        idx = (ctypes.c_uint32 * n)(*prime_idx)
+        check(lib().hemm_sample_error(self.h, int(stream_key), idx, n, vp(out.data_ptr()), vp(0)))
+        return out
 
     def modup(self, poly, nq):
         import torch

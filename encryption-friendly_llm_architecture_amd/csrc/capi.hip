@@ -107,6 +107,39 @@ int hemm_ntt(hemm_context *ctx, uint64_t *data, const uint32_t *prime_idx, uint3
     HEMM_CATCH
 }
 
+static LimbList explicit_limbs(hemm_context *ctx, const uint32_t *prime_idx, uint32_t n_limbs) {
+    need(ctx && prime_idx, "null argument");
+    need(ctx->logN >= 9, "residue kernels need log_n >= 9");
+    need(n_limbs >= 1 && n_limbs <= HEMM_MAX_PRIMES, "n_limbs out of range");
+    LimbList ll;
+    memset(&ll, 0, sizeof(ll));
+    for (uint32_t j = 0; j < n_limbs; j++) {
+        need(prime_idx[j] < (uint32_t)(ctx->nQ + ctx->nP), "prime index out of range");
+        ll.idx[j] = (uint8_t)prime_idx[j];
+    }
+    return ll;
+}
+
+int hemm_sample_uniform(hemm_context *ctx, const uint64_t *stream_keys, const uint32_t *prime_idx, uint32_t n_limbs,
+                        uint64_t *out, void *stream) {
+    HEMM_TRY
+    const LimbList ll = explicit_limbs(ctx, prime_idx, n_limbs);
+    need(stream_keys && out, "null operand");
+    launch_sample_uniform(ctx, (const u64 *)stream_keys, ll, (int)n_limbs, (u64 *)out, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_sample_error(hemm_context *ctx, uint64_t stream_key, const uint32_t *prime_idx, uint32_t n_limbs, uint64_t *out,
+                      void *stream) {
+    HEMM_TRY
+    const LimbList ll = explicit_limbs(ctx, prime_idx, n_limbs);
+    need(out, "null operand");
+    launch_sample_error(ctx, (u64)stream_key, ll, (int)n_limbs, (u64 *)out, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
 static LimbList chain_limbs(hemm_context *ctx, uint32_t nq, int with_p, int *n_limbs) {
     need(ctx, "null context");
     need(ctx->logN >= 9, "residue kernels need log_n >= 9");

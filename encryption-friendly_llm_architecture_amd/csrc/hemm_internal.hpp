@@ -72,6 +72,9 @@ void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c
                    size_t out_stride, int nq, bool accumulate, hipStream_t s);
 void launch_galois(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride, u64 g,
                    int n_limbs, int n_polys, hipStream_t s);
+void launch_sample_uniform(const hemm_context *c, const u64 *stream_keys, const LimbList &ll, int n_limbs, u64 *out,
+                           hipStream_t s);
+void launch_sample_error(const hemm_context *c, u64 stream_key, const LimbList &ll, int n_limbs, u64 *out, hipStream_t s);
 size_t hemm_scratch_words(const hemm_context *c);
 u64 *hemm_scratch(hemm_context *c);
 void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, bool fill_own, hipStream_t s);

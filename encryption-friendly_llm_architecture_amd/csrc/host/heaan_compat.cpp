@@ -341,29 +341,6 @@ std::vector<uint32_t> chain_primes(u64 count) {
     return r;
 }
 
-void sample_uniform(const Context &c, u64 key, u64 prime_idx, u64 *out) {
-    const u64 q = c->prime(prime_idx);
-    const int bits = 64 - __builtin_clzll(q);
-    const u64 mask = bits >= 64 ? ~0ull : ((1ull << bits) - 1);
-    for (u64 i = 0; i < c->N; i++)
-        for (u64 t = 0;; t++) {
-            u64 x = draw(sm64(key + t), i) & mask;
-            if (x < q) {
-                out[i] = x;
-                break;
-            }
-        }
-}
-std::vector<i64> sample_error(const Context &c, u64 key) {
-    const u64 M21 = (1ull << 21) - 1;
-    std::vector<i64> e(c->N);
-    for (u64 i = 0; i < c->N; i++) {
-        u64 x = draw(key, i);
-        e[i] = __builtin_popcountll(x & M21) - __builtin_popcountll((x >> 21) & M21);
-    }
-    return e;
-}
-
 u64 galois_of_rotation(const Context &c, u64 rot) { return powmod(5, rot % (c->N / 2), 2 * c->N); }
 
 }  // namespace
@@ -465,14 +442,16 @@ void KeyGenerator::genSwitchKey(u64 key_id, const u64 *s_from, DeviceBuffer &out
     const Context &c = ctx_;
     const size_t N = c->N, T = c->nQ + c->nP;
     out.resize(c, c->dnum * 2 * T * N);
-    std::vector<u64> ha(T * N);
     DeviceBuffer e(c, T * N), tmp(c, T * N);
     const auto primes = all_primes(c);
+    std::vector<u64> keys(T);
     for (u64 d = 0; d < c->dnum; d++) {
         u64 *b = out.data() + (d * 2 + 0) * T * N, *a = out.data() + (d * 2 + 1) * T * N;
-        lift_and_ntt(c, sample_error(c, stream_key(g_seed, TAG_EVK_E, key_id, d)), primes, e.data());
-        for (size_t i = 0; i < T; i++) sample_uniform(c, stream_key(g_seed, TAG_EVK_A, key_id, d * T + i), i, &ha[i * N]);
-        hip_ck(hipMemcpy(a, ha.data(), T * N * 8, hipMemcpyHostToDevice), "hipMemcpy");
+        // error and uniform part are sampled on the device (same counter-based streams as the host samplers)
+        ck(hemm_sample_error(c->dev, stream_key(g_seed, TAG_EVK_E, key_id, d), primes.data(), (uint32_t)T, e.data(), nullptr));
+        ck(hemm_ntt(c->dev, e.data(), primes.data(), (uint32_t)T, 1, 0, nullptr));
+        for (size_t i = 0; i < T; i++) keys[i] = stream_key(g_seed, TAG_EVK_A, key_id, d * T + i);
+        ck(hemm_sample_uniform(c->dev, keys.data(), primes.data(), (uint32_t)T, a, nullptr));
         // tmp = a*s ; b = e - tmp     (all T limbs: chain then special, i.e. nq = nQ with_p = 1)
         ck(hemm_pointwise(c->dev, HEMM_MUL, a, 0, sk_.ntt(), 0, tmp.data(), 0, (uint32_t)c->nQ, 1, 1, nullptr));
         ck(hemm_pointwise(c->dev, HEMM_SUB, e.data(), 0, tmp.data(), 0, b, 0, (uint32_t)c->nQ, 1, 1, nullptr));
@@ -672,12 +651,14 @@ void Encryptor::encrypt(const Plaintext &pt, const SecretKey &sk, Ciphertext &ct
     const u64 enc_id = g_enc_counter++;
     Ciphertext out(c);
     out.allocate(2, pt.level_, pt.rescale_counter_);
-    std::vector<u64> ha(nq * N);
-    for (size_t i = 0; i < nq; i++) sample_uniform(c, stream_key(g_seed + enc_id, TAG_ENC_A, i, 0), i, &ha[i * N]);
     u64 *b = out.buf_.data(), *a = b + nq * N;
-    hip_ck(hipMemcpy(a, ha.data(), nq * N * 8, hipMemcpyHostToDevice), "hipMemcpy");
+    const auto primes = chain_primes(nq);
+    std::vector<u64> keys(nq);
+    for (size_t i = 0; i < nq; i++) keys[i] = stream_key(g_seed + enc_id, TAG_ENC_A, i, 0);
+    ck(hemm_sample_uniform(c->dev, keys.data(), primes.data(), (uint32_t)nq, a, nullptr));
     DeviceBuffer e(c, nq * N), tmp(c, nq * N);
-    lift_and_ntt(c, sample_error(c, stream_key(g_seed + enc_id, TAG_ENC_E, 0, 0)), chain_primes(nq), e.data());
+    ck(hemm_sample_error(c->dev, stream_key(g_seed + enc_id, TAG_ENC_E, 0, 0), primes.data(), (uint32_t)nq, e.data(), nullptr));
+    ck(hemm_ntt(c->dev, e.data(), primes.data(), (uint32_t)nq, 1, 0, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_MUL, a, 0, sk.ntt(), 0, tmp.data(), 0, (uint32_t)nq, 0, 1, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_SUB, e.data(), 0, tmp.data(), 0, b, 0, (uint32_t)nq, 0, 1, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_ADD, b, 0, pt.buf_.data(), 0, b, 0, (uint32_t)nq, 0, 1, nullptr));

@@ -45,6 +45,17 @@ int hemm_timer_start(void *timer, void *stream);
 int hemm_timer_stop(void *timer, void *stream, float *ms);
 void hemm_timer_destroy(void *timer);
 
+/* Samplers behind KeyGenerator / Encryptor (HEaaN keeps them internal: KeyGenerator.hpp:31-95, Encryptor.hpp:32-49).
+ * Counter-based: value i of a stream is a function of (stream key, i) only.
+ *   hemm_sample_uniform: out[j][i] uniform in [0, q_{prime_idx[j]}) from stream_keys[j] (masked rejection);
+ *   hemm_sample_error:   out[j][i] = e_i mod q_{prime_idx[j]}, e centred binomial (21 bit pairs) from stream_key.
+ * Both write coefficient-order values [n_limbs][N]; the error is a coefficient vector (transform it with hemm_ntt),
+ * the uniform values are used directly as NTT-form residues. */
+int hemm_sample_uniform(hemm_context *ctx, const uint64_t *stream_keys, const uint32_t *prime_idx, uint32_t n_limbs,
+                        uint64_t *out, void *stream);
+int hemm_sample_error(hemm_context *ctx, uint64_t stream_key, const uint32_t *prime_idx, uint32_t n_limbs, uint64_t *out,
+                      void *stream);
+
 /* Batched negacyclic NTT (inverse = 0: natural -> bit-reversed order) or INTT (inverse = 1,
  * including 1/N) in place over data[n_polys][n_limbs][N]; limb j uses prime prime_idx[j]
  * (host array).  Every NTT-form operand of HomEvaluator goes through this. */

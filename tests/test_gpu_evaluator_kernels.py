@@ -282,3 +282,20 @@ def test_rotation_24_limb_chain_of_60_bit_primes():
         want = orc.left_rotate(O.Ct(ct, 1.0), r)
         got = host(ctx.rotate(dct, dev(orc.keys[("gal", g)]), g, nq))
         assert np.array_equal(got, want.data), r
+
+
+def test_device_samplers_match_oracle(S):
+    """The uniform and error samplers on the device reproduce the oracle's counter-based streams."""
+    orc, ctx, N = S.orc, S.ctx, S.N
+    tot = orc.nQ + orc.nP
+    idx = list(range(tot))
+    keys = [orc.stream(9, O.TAG_EVK_A, 77, j) for j in idx]
+    got = host(ctx.sample_uniform(keys, idx))
+    for j in idx:
+        assert np.array_equal(got[j], orc.uniform(keys[j], j)), j
+        assert got[j].max() < orc.mods[j]
+    ek = orc.stream(9, O.TAG_EVK_E, 77, 1)
+    e = orc.error(ek)
+    got = host(ctx.sample_error(ek, idx))
+    for j in idx:
+        assert np.array_equal(got[j], np.mod(e.astype(np.int64), orc.mods[j]).astype(np.uint64)), j
