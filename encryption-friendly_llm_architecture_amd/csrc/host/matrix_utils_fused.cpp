@@ -601,9 +601,20 @@ CtxtTensor multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &bt
     if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
     std::vector<Ciphertext> shifts;
     multMatMatPreFused(eval, a, shifts, T, tr, batch);
-    b = tr.diagonalToRow(eval, b);
-    EnDecoder endec(c);
-    if (b.getLevel() != T + 1) b.get() = endec.encode(endec.decode(b.get()), T + 1);
+    // tau on the plaintext: decode once, permute the values (MatrixTransformer::diagonalToRow<Plaintext>), encode
+    // directly at the level the shifts live at
+    {
+        EnDecoder endec(c);
+        const Message src = endec.decode(b.get());
+        Message dst(src.getLogSlots(), 0);
+        const i64 height = (i64)src.getSize() / w;
+        for (i64 r = 0; r < height; r++)
+            for (i64 cc = 0; cc < w; cc++) {
+                const i64 rb = r - r % k, cb = cc - cc % k, i = r % k, j = cc % k;
+                dst[(u64)(r * w + cc)] = src[(u64)((rb + (i + j) % k) * w + cb + j)];
+            }
+        b.get() = endec.encode(dst, T + 1);
+    }
     CtxtTensor res(c, rows, cols, w);
     eval.matmul(shifts, b.get(), res.get());   // rotation step slots / k == w
     return res;

@@ -641,7 +641,7 @@ def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
     ev = OracleEval(orc)
     assert n * w == orc.slots
     tmp = mult_mat_mat_pre_fused(orc, a, T, n, w)
-    b = ev.encode(tau_plain(ev.pt_values(b_pt), n, w), ev.level_of(b_pt))
+    b = ev.encode(tau_plain(ev.pt_values(b_pt), n, w), T + 1)
     return mult_mat_mat_reuse(ev, tmp, b, T)
 
 
