@@ -86,6 +86,8 @@ def gpu_ccmm(args, out):
     out["ccmm_pair_layout_two_products_ms"] = ms(lambda: H.single_cc_matmul(pa, pb, T))
     ppb = H.encode2(B, B2)
     out["pcmm_pair_layout_two_products_ms"] = ms(lambda: H.single_matmul(pa, ppb, T))
+    sb = H.encode(B)
+    out["pcmm_single_product_ms"] = ms(lambda: H.single_matmul(ca, sb, T))
     qa, qb = H.encrypt2(A, A2), H.encrypt2(B, B2)
     H.complex_packing_inplace(qa)
     H.complex_packing_row_inplace(qb)

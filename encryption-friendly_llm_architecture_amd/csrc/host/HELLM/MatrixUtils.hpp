@@ -50,7 +50,12 @@ public:
 
     // The same transforms and assemble masks for the batched launches: masks over the extended basis
     // (chain limbs + special primes) so they can be applied before ModDown.
-    std::vector<Plaintext> &getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
+    // first_block_only: the masks are additionally zero outside the first tile block (rows >= shape rows), which
+    // clears whatever the operand carries there
+    std::vector<Plaintext> &getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape, u64 level,
+                                          bool first_block_only = false);
+    // ones on the first tile block, zero elsewhere (ordinary plaintext at `level`)
+    const Plaintext &firstBlockMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
     std::vector<Plaintext> &getRowMaskExt(const HomEvaluator &eval, const TileTensorShape &shape, u64 level);
     // sigma / tau / packed variants with hoisted baby steps (one ModUp, all baby rotations in one launch
     // chain) and all giant-step rotations batched and summed in the extended basis
@@ -79,7 +84,8 @@ private:
                                  const TileTensorShape &shape);
     std::map<Key, Plaintext> masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
-    std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_;
+    std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_, col_masks_ext_first_;
+    std::map<std::pair<TileTensorShape, u64>, Plaintext> first_block_masks_;
 };
 
 // A x B for two encrypted tiles (HEMMer::singleCCMatMul); output level = target_level.
@@ -117,10 +123,10 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
                                  const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer,
                                  u64 batch = 16);
 void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
-                        MatrixTransformer &transformer, u64 batch = 16);
-// plaintext x ciphertext product for tiles whose rows fill the slot vector (pair layout)
-CtxtTensor multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
-                                const PtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16);
+                        MatrixTransformer &transformer, u64 batch = 16, bool first_block_only = false);
+// plaintext x ciphertext product through the hoisted column shifts (see matrix_utils_fused.cpp for the layouts it takes)
+bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const PtxtTensor &op2,
+                          u64 target_level, MatrixTransformer &transformer, u64 batch, CtxtTensor &res);
 // left rotations (in slots) whose direct keys the batched schedules use
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 

@@ -295,6 +295,8 @@ public:
     // out = rescale( sum_k cts[k] * leftRotate(pt, k * slots / cts.size()) )  -- the diagonal-packing
     // accumulation behind HEMMer::matMulReUse (MatrixUtils.cpp:1636)
     void matmul(const std::vector<Ciphertext> &cts, const Plaintext &pt, Ciphertext &out) const;
+    // the same with the plaintext rotated by k * step slots for term k (step = 0: slots / cts.size())
+    void matmul(const std::vector<Ciphertext> &cts, const Plaintext &pt, Ciphertext &out, u64 step) const;
     void modReduct(Ciphertext &) const {}  // residues here are always kept in [0, q)
 
     // extension used by the fused assemble step: out = a*ma + b*mb (no rescale)

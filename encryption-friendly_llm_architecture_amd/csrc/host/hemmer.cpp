@@ -419,9 +419,10 @@ CtxtTensor HEMMer::singleMatMul(const CtxtTensor &a, const PtxtTensor &b, u64 T)
     const u64 slots = u64(1) << log_slots_;
     const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
-    if (fused_ && (u64)(n * w) == slots) {  // rows fill the slot vector: the plaintext's row shifts are whole rotations
+    if (fused_) {
         ensureRotationKeys(fusedRotations(TileTensorShape(n, n, w), log_slots_, false, false));
-        return multMatMatPlainFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
+        CtxtTensor res(context_, a.getHeight(), b.getWidth(), w);
+        if (multMatMatPlainFused(eval_, btp_, a, b, T, matrix_transformer, batch_, res)) return res;
     }
     ensureRotationKeys({1, slots - (u64)n});
     return multMatMat(eval_, btp_, a, b, T, matrix_transformer);

@@ -412,8 +412,11 @@ void HomEvaluator::leftRotateReduce(const Ciphertext &a, u64 idx_interval, u64 n
 
 // out = rescale( sum_k cts[k] * leftRotate(pt, k * slots / cts.size()) )
 void HomEvaluator::matmul(const std::vector<Ciphertext> &cts, const Plaintext &pt, Ciphertext &out) const {
+    matmul(cts, pt, out, 0);
+}
+void HomEvaluator::matmul(const std::vector<Ciphertext> &cts, const Plaintext &pt, Ciphertext &out, u64 step_in) const {
     if (cts.empty()) throw RuntimeException("matmul: empty operand list");
-    const u64 slots = ctx_->N / 2, step = slots / cts.size(), lvl = cts[0].level_;
+    const u64 slots = ctx_->N / 2, step = step_in ? step_in : slots / cts.size(), lvl = cts[0].level_;
     if (pt.level_ < lvl) throw RuntimeException("matmul: plaintext level below the ciphertext level");
     // one launch: every term reads its ciphertext and the plaintext through that term's automorphism
     Ciphertext acc(ctx_);

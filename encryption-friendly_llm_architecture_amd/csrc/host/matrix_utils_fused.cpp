@@ -76,11 +76,24 @@ hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois
 
 }  // namespace
 
-std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
-                                                         u64 level) {
+const Plaintext &MatrixTransformer::firstBlockMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level) {
     auto key = std::make_pair(shape, level);
-    auto it = col_masks_ext_.find(key);
-    if (it != col_masks_ext_.end()) return it->second;
+    auto it = first_block_masks_.find(key);
+    if (it != first_block_masks_.end()) return it->second;
+    const Context &ctx = eval.getContext();
+    const u64 log_slots = getLogFullSlots(ctx);
+    const i64 first = shape.getNumRows() * shape.getBlockWidth(), slots = i64(1) << log_slots;
+    Message m(log_slots, 0);
+    for (i64 j = 0; j < std::min(first, slots); j++) m[(u64)j] = 1;
+    return first_block_masks_.emplace(key, EnDecoder(ctx).encode(m, level)).first->second;
+}
+
+std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
+                                                         u64 level, bool first_block_only) {
+    auto key = std::make_pair(shape, level);
+    auto &cache = first_block_only ? col_masks_ext_first_ : col_masks_ext_;
+    auto it = cache.find(key);
+    if (it != cache.end()) return it->second;
     const Context &ctx = eval.getContext();
     const u64 log_slots = getLogFullSlots(ctx);
     const i64 n = shape.getNumCols(), slots = i64(1) << log_slots;
@@ -89,7 +102,8 @@ std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eva
     v.reserve((size_t)(2 * n));
     for (i64 i = 0; i < n; i++) {
         Message wrap(log_slots, 0), main(log_slots, 0);
-        for (i64 j = 0; j < slots; j++) {
+        const i64 limit = first_block_only ? std::min(slots, shape.getNumRows() * shape.getBlockWidth()) : slots;
+        for (i64 j = 0; j < limit; j++) {
             if (j % n < n - i)
                 main[(u64)j] = 1;
             else
@@ -98,7 +112,7 @@ std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eva
         v.push_back(endec.encodeExtended(wrap, level));
         v.push_back(endec.encodeExtended(main, level));
     }
-    return col_masks_ext_.emplace(key, std::move(v)).first->second;
+    return cache.emplace(key, std::move(v)).first->second;
 }
 std::vector<Plaintext> &MatrixTransformer::getRowMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
                                                          u64 level) {
@@ -538,7 +552,7 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
 }
 
 void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::vector<Ciphertext> &tmp, u64 T,
-                        MatrixTransformer &tr, u64 batch) {
+                        MatrixTransformer &tr, u64 batch, bool first_block_only) {
     const Context &c = eval.getContext();
     tmp.clear();
     const i64 n = a_in.getHeight();
@@ -546,10 +560,13 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     if (a.getLevel() < T + 3)
         throw std::invalid_argument("[multMatMatPre] level >= " + std::to_string(T + 3) + " is needed.");
     eval.levelDown(a.get(), T + 3, a.get());
-    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
+    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2, first_block_only);
     a.get() = tr.diagonalTransformFused(eval, a.get(), MaskKind::Horizontal, a.getShape());
     Ciphertext first_ct(c);
-    eval.levelDownOne(a.get(), first_ct);
+    if (first_block_only)   // shift 0 is masked like the others so that it too is empty outside the first tile block
+        eval.mult(a.get(), tr.firstBlockMask(eval, a.getShape(), T + 2), first_ct);
+    else
+        eval.levelDownOne(a.get(), first_ct);
     tmp.push_back(first_ct);
     std::vector<Shift> sa;
     for (i64 i = 1; i < n; i++) sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
@@ -580,44 +597,61 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
 
 namespace HELLM {
 
-// Plaintext x ciphertext product for tiles whose rows fill the slot vector (rows * block width == slots, the
-// pair layout): the row shifts of tau(B) are then whole rotations of one encoded plaintext, so the product is
-// the hoisted column shifts of sigma(A) (multMatMatPreFused) followed by one masked-sum launch that reads
-// tau(B) through each term's automorphism:  rescale(sum_k shift_k(sigma A) (.) rot(tau B, k w)).
-CtxtTensor multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
-                                const PtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch) {
+// Plaintext x ciphertext product through the hoisted column shifts of sigma(A) (multMatMatPreFused) and one
+// masked-sum launch that reads tau(B) through each term's automorphism:
+//     rescale(sum_k shift_k(sigma A) (.) rot(tau B, k w)).
+// A row shift of tau(B) is a whole rotation when every tile block of the plaintext (rows * block width slots
+// each) is the same.  The plaintext is known to the host, so the layouts are told apart there:
+//   * one tile block fills the slot vector (pair layout), or all blocks are equal: as written above;
+//   * only the first block is non-zero (HEMMer::encode of a single matrix): tau(B) is copied into every block
+//     and the column-shift masks are restricted to the first block, so the product stays empty elsewhere
+//     whatever the ciphertext carries there;
+//   * anything else (different matrices stacked in one plaintext) returns false: the caller takes the
+//     reference-order product.
+bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const PtxtTensor &op2,
+                          u64 T, MatrixTransformer &tr, u64 batch, CtxtTensor &res_out) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
     if (std::min(op1.getLevel(), op2.getLevel()) < 1 + btp.getMinLevelForBootstrap())
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(1 + btp.getMinLevelForBootstrap()) +
                                     " is needed.");
-    if ((u64)(k * w) != c->N / 2)
-        throw std::invalid_argument("[multMatMatPlainFused] the row shift must be cyclic: rows * block width == slots");
+    const i64 slots = (i64)(c->N / 2), block = k * w;
+    if (block > slots || slots % block != 0) return false;
     CtxtTensor a{op1};
     PtxtTensor b{op2};
     a.setShape(rows, k);
     b.setShape(k, cols);
-    if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
-    std::vector<Ciphertext> shifts;
-    multMatMatPreFused(eval, a, shifts, T, tr, batch);
     // tau on the plaintext: decode once, permute the values (MatrixTransformer::diagonalToRow<Plaintext>), encode
     // directly at the level the shifts live at
-    {
-        EnDecoder endec(c);
-        const Message src = endec.decode(b.get());
-        Message dst(src.getLogSlots(), 0);
-        const i64 height = (i64)src.getSize() / w;
-        for (i64 r = 0; r < height; r++)
-            for (i64 cc = 0; cc < w; cc++) {
-                const i64 rb = r - r % k, cb = cc - cc % k, i = r % k, j = cc % k;
-                dst[(u64)(r * w + cc)] = src[(u64)((rb + (i + j) % k) * w + cb + j)];
-            }
-        b.get() = endec.encode(dst, T + 1);
+    EnDecoder endec(c);
+    const Message src = endec.decode(b.get());
+    // decoded values carry the encoding's rounding noise (about sqrt(N) / 2^43 at this scale): "zero" and "equal"
+    // are taken up to 2^-24
+    const double tol = std::ldexp(1.0, -24);
+    bool rest_zero = true, rest_equal = true;
+    for (i64 j = block; j < slots && (rest_zero || rest_equal); j++) {
+        if (std::abs(src[(u64)j]) >= tol) rest_zero = false;
+        if (std::abs(src[(u64)j] - src[(u64)(j % block)]) >= tol) rest_equal = false;
     }
+    if (!rest_zero && !rest_equal) return false;
+    const bool first_block_only = rest_zero && block < slots;
+    Message dst(src.getLogSlots(), 0);
+    const i64 height = slots / w;
+    for (i64 r = 0; r < height; r++)
+        for (i64 cc = 0; cc < w; cc++) {
+            const i64 cb = cc - cc % k, i = r % k, j = cc % k;
+            const i64 rb = first_block_only ? 0 : r - r % k;   // single matrix: every block takes the first one's tau
+            dst[(u64)(r * w + cc)] = src[(u64)((rb + (i + j) % k) * w + cb + j)];
+        }
+    b.get() = endec.encode(dst, T + 1);
+    if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
+    std::vector<Ciphertext> shifts;
+    multMatMatPreFused(eval, a, shifts, T, tr, batch, first_block_only);
     CtxtTensor res(c, rows, cols, w);
-    eval.matmul(shifts, b.get(), res.get());   // rotation step slots / k == w
-    return res;
+    eval.matmul(shifts, b.get(), res.get(), (u64)w);
+    res_out = res;
+    return true;
 }
 
 }  // namespace HELLM

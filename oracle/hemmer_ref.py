@@ -508,12 +508,12 @@ def mult_mat_mat_pre(ev, a, T, n, w):
     return tmp
 
 
-def mult_mat_mat_reuse(ev, tmp, b_pt, T):
+def mult_mat_mat_reuse(ev, tmp, b_pt, T, step=None):
     """multMatMatReUse (:1612-1639) with eval.matmul spelled out:
     rescale(sum_k tmp[k] * leftRotate(pt, k * slots / len(tmp)))."""
     if ev.level_of(b_pt) != T + 1:
         b_pt = ev.pt_reencode(b_pt, T + 1)
-    step = ev.slots // len(tmp)
+    step = ev.slots // len(tmp) if step is None else step
     acc = None
     for k, c in enumerate(tmp):
         t = ev.mult_plain_no_rescale(c, ev.left_rotate(b_pt, k * step))
@@ -626,23 +626,46 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     return orc.rescale(orc.relinearize(acc))
 
 
-def mult_mat_mat_pre_fused(orc, a, T, n, w):
-    cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+def mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only=False):
+    """first_block_only: every mask (shift 0 included) is zero outside the first n * w slots."""
+    masks = col_masks(n, orc.slots)
+    block = np.zeros(orc.slots, dtype=np.complex128)
+    block[: min(n * w, orc.slots)] = 1
+    if first_block_only:
+        masks = [m * block for m in masks]
+    cm = [orc.encode_ext(m, T + 2) for m in masks]
     a = orc.level_down(a, T + 3)
     a = diagonal_transform_fused(orc, a, H, n, w)
     ext = orc.modup(a.data[1])
-    return [orc.level_down_one(a)] + _assemble_shifts(
+    first = OracleEval(orc).mult_pt(a, orc.encode(block, T + 2)) if first_block_only else orc.level_down_one(a)
+    return [first] + _assemble_shifts(
         orc, a, ext, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
 
 
 def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
-    """Batched plaintext x ciphertext product for rows * block width == slots: hoisted column shifts of
-    sigma(A), then rescale(sum_k shift_k (.) rot(tau(B), k w))."""
+    """Batched plaintext x ciphertext product: hoisted column shifts of sigma(A), then
+    rescale(sum_k shift_k (.) rot(tau(B), k w)).  The row shift of tau(B) is a whole rotation when all
+    tile blocks (n * w slots) of the plaintext are equal; a plaintext that is zero outside its first block
+    gets tau of that block copied into every block and masks restricted to the first block ("zero" and "equal"
+    up to 2^-24).  Returns None
+    for plaintexts of any other form (the product then takes the reference order)."""
     ev = OracleEval(orc)
-    assert n * w == orc.slots
-    tmp = mult_mat_mat_pre_fused(orc, a, T, n, w)
-    b = ev.encode(tau_plain(ev.pt_values(b_pt), n, w), T + 1)
-    return mult_mat_mat_reuse(ev, tmp, b, T)
+    slots, block = orc.slots, n * w
+    if block > slots or slots % block:
+        return None
+    v = ev.pt_values(b_pt)
+    blocks = v.reshape(slots // block, block)
+    tol = 2.0 ** -24            # decoded values carry the encoding's rounding noise
+    rest_zero = bool(np.all(np.abs(blocks[1:]) < tol))
+    rest_equal = bool(np.all(np.abs(blocks[1:] - blocks[0]) < tol))
+    if not (rest_zero or rest_equal):
+        return None
+    first_block_only = rest_zero and block < slots
+    if first_block_only:
+        v = np.tile(blocks[0], slots // block)
+    tmp = mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only)
+    b = ev.encode(tau_plain(v, n, w), T + 1)
+    return mult_mat_mat_reuse(ev, tmp, b, T, step=w)
 
 
 def weights_diagonal_to_row4(w1, w2, w3, w4, slots):

@@ -179,9 +179,13 @@ def test_pcmm_and_packed_bit_exact(small, fused):
     pb = H.encode(B)
     c = H.single_matmul(ca, pb, 2)
     opb = O.Pt(pb.residues(), orc.delta[orc.nQ - 1])
-    want = R.mult_mat_mat_pc(ev, to_oracle(orc, ca), opb, 2, 16, 16)
+    if fused:   # single matrix in the first tile block: tau(B) copied into every block, masks on the first block
+        want = R.mult_mat_mat_pc_fused(orc, to_oracle(orc, ca), opb, 2, 16, 16)
+    else:
+        want = R.mult_mat_mat_pc(ev, to_oracle(orc, ca), opb, 2, 16, 16)
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
+    assert np.abs(H.decrypt_slots(c)[256:]).max() < 2 ** -20      # nothing outside the first tile block
     A2, B2 = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
     pa, pbb = H.encrypt2(A, A2), H.encrypt2(B, B2)
     oa, ob = to_oracle(orc, pa), to_oracle(orc, pbb)
