@@ -128,6 +128,28 @@ public:
     CtxtTensor matMulPreRev(const CtxtTensor &b, u64 target_level = 4) const;
     CtxtTensor matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 target_level = 4) const;
 
+    // LoRA low-rank path (reference src/HEMMer.cpp:2111-2332, 1055-1091; products in MatrixUtils.cpp:1681-1996).
+    // A rank-`LOW_DIM` factor occupies LOW_DIM columns (or rows) of a tile, at column (row) block `block`:
+    //   getLowColBlock / getLowRowBlock   keep that block of every tile;
+    //   matMulHighLow(a, b, in_col_block) partial sums of A x B_low spread over the column blocks;
+    //   matMulLowHigh(a, b, in_row_block) A_low x B, partial sums spread over the row blocks;
+    //   matMulLowLow(a, b, col, row)      (rows x LOW_DIM) x (LOW_DIM x cols), complete product;
+    //   repackToOneCol / OneRow           sum the partial sums of all blocks (both tiles of the pair layout
+    //                                     included) into block `out_block`, copied to every tile;
+    //   repackToMultiCol / MultiRow       the same per tile, without the copy.
+    CtxtTensor matMulHighLow(const CtxtTensor &a, const CtxtTensor &b, u64 in_col_block, u64 target_level) const;
+    CtxtTensor matMulLowHigh(const CtxtTensor &a, const CtxtTensor &b, u64 in_row_block, u64 target_level) const;
+    CtxtTensor matMulLowLow(const CtxtTensor &a, const CtxtTensor &b, u64 in_col_block, u64 in_row_block,
+                            u64 target_level = 4) const;
+    CtxtTensor repackToOneCol(const CtxtTensor &t, u64 out_col_block) const;
+    CtxtTensor repackToMultiCol(const CtxtTensor &t, u64 out_col_block) const;
+    CtxtTensor repackToOneRow(const CtxtTensor &t, u64 out_row_block) const;
+    CtxtTensor repackToMultiRow(const CtxtTensor &t, u64 out_row_block) const;
+    CtxtTensor getLowColBlock(const CtxtTensor &t, u64 col_block) const;
+    CtxtTensor getLowRowBlock(const CtxtTensor &t, u64 row_block) const;
+    // repack of two un-rescaled product halves used by the LoRA path (src/HEMMer.cpp:1055-1091)
+    CtxtTensor repack_loraOpti(CtxtTensor &t1, CtxtTensor &t2) const;
+
     // Schedule of singleCCMatMul / packedMatMul / matMulPre: batched launches with hoisted rotations
     // (default) or one evaluator call per step in the reference's order.  `batch` = shifts per launch.
     void setFused(bool on, u64 batch = 16) {
@@ -144,6 +166,9 @@ private:
     void init();
     const Plaintext &cachedMask(int id, u64 level) const;
     std::vector<u64> transformRotations(MaskKind kind, i64 width) const;
+    // the same for a (possibly rectangular) sigma / tau shape under the current schedule
+    std::vector<u64> transformRotations(MaskKind kind, const TileTensorShape &shape) const;
+    void ensureLogStepKeys(i64 first, i64 bound, i64 unit) const;   // +-i*unit for i = first, 2 first, ... < bound
 
     int device_id_ = 0;
     Context context_;
@@ -156,7 +181,7 @@ private:
     mutable KeyPack pack_;
     HomEvaluator eval_;
     Bootstrapper btp_;
-    Message col_mask_even_, row_mask_even_, mask_left_half_, mask_matmul_;
+    Message col_mask_even_, row_mask_even_, mask_left_half_, mask_matmul_, mask_matmul_half_;
     mutable std::map<std::pair<int, u64>, Plaintext> mask_cache_;
     mutable std::set<u64> have_rot_;
     bool fused_ = true;

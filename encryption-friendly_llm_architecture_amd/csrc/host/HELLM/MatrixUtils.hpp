@@ -113,6 +113,20 @@ CtxtTensor multMatMatPreRev(const HomEvaluator &eval, const CtxtTensor &b, u64 t
 CtxtTensor multMatMatCCReUse(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
                              u64 target_level, MatrixTransformer &transformer);
 
+// LoRA low-rank products: one operand uses only `low_dim` columns (HighLow), rows (LowHigh) or both one thin
+// operand each (LowLow), sitting at the given column / row block of every tile.  `fused` runs the sigma / tau
+// transforms through the batched launches; the few remaining operations are ordinary evaluator calls.
+constexpr i64 LOW_DIM = 2;   // LoRA rank (reference ModelArgs.hpp:67)
+CtxtTensor multMatMatHighLow(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_col_block,
+                             u64 target_level, MatrixTransformer &transformer, i64 low_dim = LOW_DIM,
+                             bool fused = false);
+CtxtTensor multMatMatLowHigh(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_row_block,
+                             u64 target_level, MatrixTransformer &transformer, i64 low_dim = LOW_DIM,
+                             bool fused = false);
+CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_col_block,
+                            u64 in_row_block, u64 target_level, MatrixTransformer &transformer, i64 low_dim = LOW_DIM,
+                            bool fused = false);
+
 // Batched schedules of the same products (same decrypted results, far fewer and larger launches):
 // every column / row shift of the main loop is a direct hoisted rotation of sigma(A) / tau(B) (one ModUp
 // per operand), the two masked halves of a shift are combined before one merged ModDown + rescale, and

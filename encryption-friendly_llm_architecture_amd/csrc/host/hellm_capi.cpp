@@ -536,5 +536,46 @@ int hellm_repack_not_bts(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **o
     *out = new hellm_ct{h->m->repack_notBTS(a->t, b->t)};
     FACADE_CATCH
 }
+int hellm_repack_lora_opti(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->repack_loraOpti(a->t, b->t)};
+    FACADE_CATCH
+}
+int hellm_matmul_high_low(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_col_block,
+                          uint32_t target_level, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->matMulHighLow(a->t, b->t, in_col_block, target_level)};
+    FACADE_CATCH
+}
+int hellm_matmul_low_high(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_row_block,
+                          uint32_t target_level, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->matMulLowHigh(a->t, b->t, in_row_block, target_level)};
+    FACADE_CATCH
+}
+int hellm_matmul_low_low(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_col_block,
+                         uint32_t in_row_block, uint32_t target_level, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_ct{h->m->matMulLowLow(a->t, b->t, in_col_block, in_row_block, target_level)};
+    FACADE_CATCH
+}
+// which: 0 repackToOneCol, 1 repackToMultiCol, 2 repackToOneRow, 3 repackToMultiRow, 4 getLowColBlock, 5 getLowRowBlock
+int hellm_low_rank_block(hellm_hemmer *h, const hellm_ct *a, uint32_t which, uint32_t block, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    need(which < 6, "which must be 0..5");
+    const HELLM::HEMMer &m = *h->m;
+    *out = new hellm_ct{which == 0   ? m.repackToOneCol(a->t, block)
+                        : which == 1 ? m.repackToMultiCol(a->t, block)
+                        : which == 2 ? m.repackToOneRow(a->t, block)
+                        : which == 3 ? m.repackToMultiRow(a->t, block)
+                        : which == 4 ? m.getLowColBlock(a->t, block)
+                                     : m.getLowRowBlock(a->t, block)};
+    FACADE_CATCH
+}
 
 }  // extern "C"

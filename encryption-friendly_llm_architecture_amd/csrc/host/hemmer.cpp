@@ -12,7 +12,7 @@ static MatrixTransformer matrix_transformer;
 void cleanUpMatrixTransformer() { matrix_transformer.cleanUp(); }
 
 namespace {
-enum { MASK_COL_EVEN = 0, MASK_ROW_EVEN = 1, MASK_LEFT_HALF = 2, MASK_MATMUL = 3 };
+enum { MASK_COL_EVEN = 0, MASK_ROW_EVEN = 1, MASK_LEFT_HALF = 2, MASK_MATMUL = 3, MASK_MATMUL_HALF = 4 };
 
 i64 tileDim(u64 log_slots) {
     if (log_slots < 3 || (log_slots & 1) == 0)
@@ -63,6 +63,7 @@ void HEMMer::init() {
     row_mask_even_ = message2(tr_even, tr_even);
     mask_left_half_ = message2(ones, zeros);
     mask_matmul_ = message2(ones, zeros);
+    mask_matmul_half_ = message2(Matrix(n, n, 0.5), zeros);
 }
 
 void HEMMer::save(const std::string &keys_path) {
@@ -77,7 +78,8 @@ const Plaintext &HEMMer::cachedMask(int id, u64 level) const {
     const Message *m = id == MASK_COL_EVEN ? &col_mask_even_
                        : id == MASK_ROW_EVEN ? &row_mask_even_
                        : id == MASK_LEFT_HALF ? &mask_left_half_
-                                              : &mask_matmul_;
+                       : id == MASK_MATMUL_HALF ? &mask_matmul_half_
+                                                : &mask_matmul_;
     return mask_cache_.emplace(key, endec_.encode(*m, level)).first->second;
 }
 
@@ -477,6 +479,204 @@ CtxtTensor HEMMer::matMulPreRev(const CtxtTensor &b, u64 T) const {
 CtxtTensor HEMMer::matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 T) const {
     ensureRotationKeys({(u64)b.getBlockWidth()});
     return multMatMatCCReUse(eval_, tmp, b, T, matrix_transformer);
+}
+
+// ---- LoRA low-rank path --------------------------------------------------------------------------------------
+std::vector<u64> HEMMer::transformRotations(MaskKind kind, const TileTensorShape &shape) const {
+    const u64 slots = u64(1) << log_slots_;
+    const bool vertical = kind == MaskKind::Vertical;
+    const i64 rows = shape.getNumRows(), cols = shape.getNumCols(), step = vertical ? shape.getBlockWidth() : 1;
+    const i64 units = vertical ? rows : cols, sub = std::min(rows, cols);
+    const i64 bs = (i64)std::ceil(std::sqrt((double)(2 * sub - 1))), gs = (i64)std::ceil((double)(sub - 1) / (double)bs);
+    std::vector<u64> r;
+    auto left = [&](i64 v) { r.push_back((u64)(((v % (i64)slots) + (i64)slots) % (i64)slots)); };
+    for (i64 j = 0; j < (fused_ ? bs : 1); j++) left((j + 1) * step);   // hoisted baby steps are direct rotations
+    for (i64 i = 0; i < gs; i++) {
+        left(-(units - i * bs) * step);
+        if (i > 0) left(i * bs * step);
+    }
+    return r;
+}
+void HEMMer::ensureLogStepKeys(i64 first, i64 bound, i64 unit) const {
+    const u64 slots = u64(1) << log_slots_;
+    std::vector<u64> r;
+    for (i64 i = first; i < bound; i <<= 1) {
+        const u64 v = (u64)(i * unit) % slots;
+        r.push_back(v);
+        r.push_back((slots - v) % slots);
+    }
+    ensureRotationKeys(r);
+}
+CtxtTensor HEMMer::matMulHighLow(const CtxtTensor &a, const CtxtTensor &b, u64 in_col_block, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = b.getBlockWidth();
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getShape()));
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, TileTensorShape(b.getHeight(), LOW_DIM, w)));
+    ensureLogStepKeys(LOW_DIM, w / 2, 1);
+    ensureLogStepKeys(LOW_DIM, w / 2, w);
+    ensureRotationKeys({1, (u64)w, slots - (u64)(w / 2), (slots - (u64)(a.getHeight() * w) % slots) % slots});
+    return multMatMatHighLow(eval_, a, b, in_col_block, T, matrix_transformer, LOW_DIM, fused_);
+}
+CtxtTensor HEMMer::matMulLowHigh(const CtxtTensor &a, const CtxtTensor &b, u64 in_row_block, u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = a.getBlockWidth();
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getShape()));
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, b.getShape()));
+    ensureLogStepKeys(LOW_DIM, w / 2, w);
+    ensureRotationKeys({1, (u64)w, slots - (u64)(w / 2), (slots - (u64)(a.getHeight() * w) % slots) % slots});
+    return multMatMatLowHigh(eval_, a, b, in_row_block, T, matrix_transformer, LOW_DIM, fused_);
+}
+CtxtTensor HEMMer::matMulLowLow(const CtxtTensor &a, const CtxtTensor &b, u64 in_col_block, u64 in_row_block,
+                                u64 T) const {
+    const u64 slots = u64(1) << log_slots_;
+    const i64 w = a.getBlockWidth();
+    ensureRotationKeys(transformRotations(MaskKind::Horizontal, TileTensorShape(a.getHeight(), LOW_DIM, w)));
+    ensureRotationKeys(transformRotations(MaskKind::Vertical, TileTensorShape(LOW_DIM, b.getWidth(), w)));
+    ensureLogStepKeys(LOW_DIM, w / 2, 1);
+    ensureLogStepKeys(LOW_DIM, w / 2, w);
+    ensureRotationKeys({1, (u64)w, slots - (u64)(w / 2), (slots - (u64)(a.getHeight() * w) % slots) % slots});
+    return multMatMatLowLow(eval_, a, b, in_col_block, in_row_block, T, matrix_transformer, LOW_DIM, fused_);
+}
+
+namespace {
+// ones on columns [block * low, (block + 1) * low) of the first tile (or of every tile of width `cols`) in `rows` rows
+Message lowColBlockMask(u64 log_slots, u64 rows, u64 cols, u64 w, u64 block, u64 low, bool every_tile) {
+    Message m(log_slots, 0);
+    for (u64 i = 0; i < rows; i++)
+        for (u64 k = 0; k < (every_tile ? w : 1); k += cols)
+            for (u64 j = block * low; j < (block + 1) * low; j++) m[i * w + k + j] = 1;
+    return m;
+}
+// ones on rows [block * low, (block + 1) * low), columns [0, width)
+Message lowRowBlockMask(u64 log_slots, u64 w, u64 block, u64 low, u64 width) {
+    Message m(log_slots, 0);
+    for (u64 i = block * low; i < (block + 1) * low; i++)
+        for (u64 j = 0; j < width; j++) m[i * w + j] = 1;
+    return m;
+}
+}  // namespace
+
+CtxtTensor HEMMer::repackToOneCol(const CtxtTensor &t, u64 out_col_block) const {
+    const u64 rows = (u64)t.getHeight(), cols = (u64)t.getWidth(), w = (u64)t.getBlockWidth();
+    ensureLogStepKeys(LOW_DIM, (i64)w, 1);
+    ensureLogStepKeys((i64)cols, (i64)cols + 1, 1);
+    Ciphertext tmp(context_);
+    CtxtTensor ret{t};
+    u64 pos = out_col_block;
+    for (u64 i = LOW_DIM; i < w; i <<= 1) {
+        if (pos % 2 == 0)
+            eval_.leftRotate(ret.get(), i, tmp);
+        else
+            eval_.rightRotate(ret.get(), i, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+        pos /= 2;
+    }
+    eval_.mult(ret.get(), lowColBlockMask(log_slots_, rows, cols, w, out_col_block, LOW_DIM, false), ret.get());
+    for (u64 i = cols; i < w; i <<= 1) {   // copy to the other tiles of the row
+        eval_.rightRotate(ret.get(), cols, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+    }
+    return ret;
+}
+CtxtTensor HEMMer::repackToMultiCol(const CtxtTensor &t, u64 out_col_block) const {
+    const u64 rows = (u64)t.getHeight(), cols = (u64)t.getWidth(), w = (u64)t.getBlockWidth();
+    ensureLogStepKeys(LOW_DIM, (i64)(w / 2), 1);
+    Ciphertext tmp(context_);
+    CtxtTensor ret{t};
+    u64 pos = out_col_block;
+    for (u64 i = LOW_DIM; i < w / 2; i <<= 1) {
+        if (pos % 2 == 0)
+            eval_.leftRotate(ret.get(), i, tmp);
+        else
+            eval_.rightRotate(ret.get(), i, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+        pos /= 2;
+    }
+    eval_.mult(ret.get(), lowColBlockMask(log_slots_, rows, cols, w, out_col_block, LOW_DIM, true), ret.get());
+    return ret;
+}
+CtxtTensor HEMMer::repackToOneRow(const CtxtTensor &t, u64 out_row_block) const {
+    const u64 rows = (u64)t.getHeight(), cols = (u64)t.getWidth(), w = (u64)t.getBlockWidth();
+    ensureLogStepKeys(LOW_DIM, (i64)rows, (i64)w);
+    ensureLogStepKeys((i64)cols, (i64)cols + 1, 1);
+    Ciphertext tmp(context_);
+    CtxtTensor ret{t};
+    u64 pos = out_row_block;
+    for (u64 i = LOW_DIM; i < rows; i <<= 1) {
+        if (pos % 2 == 0)
+            eval_.leftRotate(ret.get(), i * w, tmp);
+        else
+            eval_.rightRotate(ret.get(), i * w, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+        pos /= 2;
+    }
+    for (u64 i = cols; i < w; i <<= 1) {   // sum the tiles of the row
+        eval_.leftRotate(ret.get(), cols, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+    }
+    eval_.mult(ret.get(), lowRowBlockMask(log_slots_, w, out_row_block, LOW_DIM, cols), ret.get());
+    for (u64 i = cols; i < w; i += cols) {   // copy to the other tiles
+        eval_.rightRotate(ret.get(), cols, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+    }
+    return ret;
+}
+CtxtTensor HEMMer::repackToMultiRow(const CtxtTensor &t, u64 out_row_block) const {
+    const u64 rows = (u64)t.getHeight(), w = (u64)t.getBlockWidth();
+    ensureLogStepKeys(LOW_DIM, (i64)rows, (i64)w);
+    Ciphertext tmp(context_);
+    CtxtTensor ret{t};
+    u64 pos = out_row_block;
+    for (u64 i = LOW_DIM; i < rows; i <<= 1) {
+        if (pos % 2 == 0)
+            eval_.leftRotate(ret.get(), i * w, tmp);
+        else
+            eval_.rightRotate(ret.get(), i * w, tmp);
+        eval_.add(ret.get(), tmp, ret.get());
+        pos /= 2;
+    }
+    eval_.mult(ret.get(), lowRowBlockMask(log_slots_, w, out_row_block, LOW_DIM, w), ret.get());
+    return ret;
+}
+CtxtTensor HEMMer::getLowColBlock(const CtxtTensor &t, u64 col_block) const {
+    CtxtTensor res{t};
+    eval_.mult(t.get(),
+               lowColBlockMask(log_slots_, (u64)t.getHeight(), (u64)t.getWidth(), (u64)t.getBlockWidth(), col_block,
+                               LOW_DIM, true),
+               res.get());
+    return res;
+}
+CtxtTensor HEMMer::getLowRowBlock(const CtxtTensor &t, u64 row_block) const {
+    CtxtTensor res{t};
+    eval_.mult(t.get(), lowRowBlockMask(log_slots_, (u64)t.getBlockWidth(), row_block, LOW_DIM, (u64)t.getBlockWidth()),
+               res.get());
+    return res;
+}
+CtxtTensor HEMMer::repack_loraOpti(CtxtTensor &t1, CtxtTensor &t2) const {
+    const u64 slots = u64(1) << log_slots_, n = (u64)dim_;
+    ensureRotationKeys({n, slots - n});
+    CtxtTensor out(t1), tmp(t2);
+    if (t1.get().getRescaleCounter() > 0) eval_.rescale(t1.get());
+    if (t2.get().getRescaleCounter() > 0) eval_.rescale(t2.get());
+    eval_.conjugate(t1.get(), out.get());
+    eval_.add(t1.get(), out.get(), out.get());
+    eval_.conjugate(t2.get(), tmp.get());
+    eval_.add(t2.get(), tmp.get(), tmp.get());
+    eval_.multImagUnit(tmp.get(), tmp.get());
+    eval_.add(out.get(), tmp.get(), out.get());
+    eval_.leftRotate(out.get(), n, tmp.get());
+    eval_.add(out.get(), tmp.get(), out.get());
+    CtxtTensor conj(out);
+    eval_.conjugate(out.get(), conj.get());
+    eval_.add(out.get(), conj.get(), out.get());
+    eval_.sub(conj.get(), tmp.get(), tmp.get());
+    eval_.multImagUnit(tmp.get(), tmp.get());
+    const Plaintext &m = cachedMask(MASK_MATMUL_HALF, out.getLevel());
+    eval_.mult(tmp.get(), m, tmp.get());
+    eval_.mult(out.get(), m, out.get());
+    eval_.rightRotate(tmp.get(), n, tmp.get());
+    addInplace(out, tmp);
+    return out;
 }
 
 // x + conj(x) = 2 Re(x)

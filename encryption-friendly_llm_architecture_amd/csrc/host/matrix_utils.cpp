@@ -1,6 +1,7 @@
 // sigma / tau / transpose transforms and the matrix products of HELLM/MatrixUtils.hpp.
 // Follows the algorithm of the reference's ciphertext/src/MatrixUtils.cpp (mask families :90-578,
 // transforms :671-1098, products :1100-1679) restated over this build's evaluator.
+#include <algorithm>
 #include <cmath>
 
 #include "HELLM/MatrixUtils.hpp"
@@ -16,9 +17,14 @@ i64 pow2ceil(i64 v) {
 }
 
 // baby-step / giant-step geometry of a transform kind
+// Rectangular tiles (sigma and tau only; reference generateHorizontalMask / generateVerticalMask,
+// ciphertext/src/MatrixUtils.cpp:129-217, 330-419): a diagonal wraps over the columns (sigma) or rows (tau)
+// of the tile while the number of diagonals of one sign is the shorter side.
 struct Geometry {
-    i64 n;       // tile side (values)
-    i64 units;   // diagonals counted in cells: n (plain) or n / 2 (packed)
+    i64 n;       // tile side (values) of a square tile; rows otherwise
+    i64 rows, cols;
+    i64 units;   // length a diagonal wraps over, in cells: n (plain) or n / 2 (packed)
+    i64 sub;     // diagonals of one sign, in cells: min(rows, cols) / cell
     i64 cell;    // 1 or 2
     i64 bs, gs;
     i64 step;    // slots moved per unit diagonal
@@ -27,9 +33,14 @@ struct Geometry {
 Geometry geometry(MaskKind kind, const TileTensorShape &s) {
     Geometry g{};
     const i64 rows = s.getNumRows(), cols = s.getNumCols(), w = s.getBlockWidth();
-    if (rows != cols) throw std::invalid_argument("[MatrixTransformer] only square tiles are supported");
+    const bool plain_sigma_tau = (kind == MaskKind::Horizontal || kind == MaskKind::Vertical);
+    if (rows != cols && !plain_sigma_tau)
+        throw std::invalid_argument("[MatrixTransformer] packed transforms and transpose need square tiles");
     g.n = rows;
+    g.rows = rows;
+    g.cols = cols;
     if (kind == MaskKind::Diagonal) {
+        g.sub = g.n;
         g.units = g.n;
         g.cell = 1;
         const i64 count = 2 * g.n - 1;
@@ -41,9 +52,10 @@ Geometry geometry(MaskKind kind, const TileTensorShape &s) {
     const bool packed = (kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical);
     const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
     g.cell = packed ? 2 : 1;
-    g.units = g.n / g.cell;
-    g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.units - 1)));
-    g.gs = (i64)std::ceil((double)(g.units - 1) / (double)g.bs);
+    g.units = (vertical ? rows : cols) / g.cell;
+    g.sub = std::min(rows, cols) / g.cell;
+    g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.sub - 1)));
+    g.gs = (i64)std::ceil((double)(g.sub - 1) / (double)g.bs);
     g.step = g.cell * (vertical ? w : 1);
     return g;
 }
@@ -57,17 +69,21 @@ Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 lo
     const double value = (kind == MaskKind::PackedHorizontal) ? 0.5 : 1.0;
     for (i64 r = 0; r < height; r++)
         for (i64 c = 0; c < w; c++) {
-            const i64 R = (r % g.n) / g.cell, C = (c % g.n) / g.cell;
+            const i64 R = (r % g.rows) / g.cell, C = (c % g.cols) / g.cell;
             bool on;
             switch (kind) {
                 case MaskKind::Horizontal:
-                case MaskKind::PackedHorizontal:
-                    on = idx >= 0 ? (R == idx && C < g.units - idx) : (R == g.units + idx && C >= -idx);
+                case MaskKind::PackedHorizontal: {
+                    const i64 Rs = R % g.sub;   // a tall tile repeats the pattern every `sub` rows
+                    on = idx >= 0 ? (Rs == idx && C < g.units - idx) : (Rs == g.units + idx && C >= -idx);
                     break;
+                }
                 case MaskKind::Vertical:
-                case MaskKind::PackedVertical:
-                    on = idx >= 0 ? (C == idx && R < g.units - idx) : (C == g.units + idx && R >= -idx);
+                case MaskKind::PackedVertical: {
+                    const i64 Cs = C % g.sub;   // a wide tile repeats it every `sub` columns
+                    on = idx >= 0 ? (Cs == idx && R < g.units - idx) : (Cs == g.units + idx && R >= -idx);
                     break;
+                }
                 default:  // Diagonal: output positions with column - row == idx
                     on = (C - R == idx);
             }
@@ -184,7 +200,7 @@ Ciphertext MatrixTransformer::diagonalTransform(const HomEvaluator &eval, const 
         bool any = false;
         for (i64 j = 0; j < g.bs; j++) {
             const i64 d = 1 + i * g.bs + j - g.units;
-            if (d >= 0) break;
+            if (d >= g.sub - g.units) break;
             eval.multWithoutRescale(baby[(size_t)j], transformMask(eval, kind, shape, level, d), any ? tmp : group);
             if (any) eval.add(group, tmp, group);
             any = true;
@@ -197,7 +213,7 @@ Ciphertext MatrixTransformer::diagonalTransform(const HomEvaluator &eval, const 
         any = false;
         for (i64 j = 0; j < g.bs; j++) {
             const i64 d = 1 + i * g.bs + j;
-            if (d >= g.units) break;
+            if (d >= g.sub) break;
             eval.multWithoutRescale(baby[(size_t)j], transformMask(eval, kind, shape, level, d), any ? tmp : group);
             if (any) eval.add(group, tmp, group);
             any = true;
@@ -389,6 +405,127 @@ CtxtTensor multMatMat<Ciphertext>(const HomEvaluator &eval, const Bootstrapper &
         eval.add(res.get(), t1, res.get());
     }
     return res;
+}
+
+// ---- LoRA low-rank products (reference ciphertext/src/MatrixUtils.cpp:1681-1996) -------------------------
+// One operand has only `low_dim` columns (or rows) in use, sitting at a column (row) block of every tile.  The
+// transforms of the thin operand run on the thin shape, its copies are spread over the blocks by log-step
+// rotations, and the product loop stops after low_dim terms; the outputs of all column blocks still have to
+// be summed (HEMMer::repackTo*).
+namespace {
+Ciphertext sigmaTau(const HomEvaluator &eval, MatrixTransformer &tr, const Ciphertext &in, MaskKind kind,
+                    const TileTensorShape &shape, bool fused) {
+    if (fused) return tr.diagonalTransformFused(eval, in, kind, shape);
+    CtxtTensor t(shape, in);
+    return kind == MaskKind::Horizontal ? tr.diagonalToColumn(eval, t).get() : tr.diagonalToRow(eval, t).get();
+}
+
+// sigma(A) (.) tau(B) and the low_dim - 1 shifted terms (:1716-1766)
+CtxtTensor lowRankTerms(const HomEvaluator &eval, Ciphertext &a, Ciphertext &b, const CtxtTensor &op1,
+                        const CtxtTensor &op2, i64 w, u64 T, i64 low_dim, MatrixTransformer &tr) {
+    const Context &ctx = eval.getContext();
+    const i64 num_rows = op1.getHeight();
+    CtxtTensor res(ctx, op1.getHeight(), op2.getWidth(), op2.getBlockWidth());
+    eval.mult(a, b, res.get());
+    if (low_dim < 2) return res;
+    eval.leftRotate(a, 1, a);
+    eval.leftRotate(b, (u64)w, b);
+    Ciphertext a_wrap(ctx), b_wrap(ctx);
+    eval.rightRotate(a, (u64)(w / 2), a_wrap);
+    eval.rightRotate(b, (u64)(num_rows * w), b_wrap);
+    std::vector<Plaintext> &col_mask = tr.getColMask(eval, op1.getShape(), T + 2);
+    std::vector<Plaintext> &row_mask = tr.getRowMask(eval, op2.getShape(), T + 2);
+    Ciphertext t1(ctx), t2(ctx), acc(ctx);
+    for (i64 i = 1; i < low_dim; i++) {
+        if (i > 1) {
+            eval.leftRotate(a, 1, a);
+            eval.leftRotate(a_wrap, 1, a_wrap);
+            eval.leftRotate(b, (u64)w, b);
+            eval.leftRotate(b_wrap, (u64)w, b_wrap);
+        }
+        eval.maskedSum(a, col_mask[(size_t)(2 * i + 1)], a_wrap, col_mask[(size_t)(2 * i)], t1);
+        eval.rescale(t1);
+        eval.maskedSum(b, row_mask[(size_t)(2 * i + 1)], b_wrap, row_mask[(size_t)(2 * i)], t2);
+        eval.rescale(t2);
+        eval.tensorAccumulate(t1, t2, acc, i == 1);
+    }
+    eval.relinearize(acc, t1);
+    eval.rescale(t1);
+    eval.add(res.get(), t1, res.get());
+    return res;
+}
+}  // namespace
+
+CtxtTensor multMatMatHighLow(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_col_block,
+                             u64 T, MatrixTransformer &tr, i64 low_dim, bool fused) {
+    const Context &ctx = eval.getContext();
+    const i64 w = op2.getBlockWidth();
+    Ciphertext a(ctx), b(ctx), tmp(ctx);
+    eval.levelDown(op1.get(), T + 3, a);
+    eval.levelDown(op2.get(), T + 3, b);
+    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, op1.getShape(), fused);
+    b = sigmaTau(eval, tr, b, MaskKind::Vertical, TileTensorShape(op2.getHeight(), low_dim, w), fused);
+    u64 pos = in_col_block;
+    for (i64 i = low_dim; i < w / 2; i <<= 1) {
+        if (pos % 2 == 0) {
+            eval.leftRotate(b, (u64)(i * w), tmp);
+            eval.rightRotate(tmp, (u64)i, tmp);
+        } else {
+            eval.leftRotate(b, (u64)i, tmp);
+            eval.leftRotate(b, (u64)(i * w), b);
+        }
+        eval.add(b, tmp, b);
+        pos /= 2;
+    }
+    return lowRankTerms(eval, a, b, op1, op2, w, T, low_dim, tr);
+}
+
+CtxtTensor multMatMatLowHigh(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_row_block,
+                             u64 T, MatrixTransformer &tr, i64 low_dim, bool fused) {
+    const Context &ctx = eval.getContext();
+    const i64 w = commonBlockWidth(op1, op2);
+    Ciphertext a(ctx), b(ctx), tmp(ctx);
+    eval.levelDown(op1.get(), T + 3, a);
+    eval.levelDown(op2.get(), T + 3, b);
+    u64 pos = in_row_block;
+    for (i64 i = low_dim; i < w / 2; i <<= 1) {
+        if (pos % 2 == 0)
+            eval.rightRotate(a, (u64)(i * w), tmp);
+        else
+            eval.leftRotate(a, (u64)(i * w), tmp);
+        eval.add(a, tmp, a);
+        pos /= 2;
+    }
+    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, op1.getShape(), fused);
+    b = sigmaTau(eval, tr, b, MaskKind::Vertical, op2.getShape(), fused);
+    return lowRankTerms(eval, a, b, op1, op2, w, T, low_dim, tr);
+}
+
+CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, const CtxtTensor &op2, u64 in_col_block,
+                            u64 in_row_block, u64 T, MatrixTransformer &tr, i64 low_dim, bool fused) {
+    const Context &ctx = eval.getContext();
+    const i64 w = commonBlockWidth(op1, op2);
+    Ciphertext a(ctx), b(ctx), tmp(ctx);
+    eval.levelDown(op1.get(), T + 3, a);
+    eval.levelDown(op2.get(), T + 3, b);
+    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, TileTensorShape(op1.getHeight(), low_dim, w), fused);
+    b = sigmaTau(eval, tr, b, MaskKind::Vertical, TileTensorShape(low_dim, op2.getWidth(), w), fused);
+    u64 cpos = in_col_block, rpos = in_row_block;
+    for (i64 i = low_dim; i < w / 2; i <<= 1) {
+        if (cpos % 2 == 0)
+            eval.rightRotate(a, (u64)i, tmp);
+        else
+            eval.leftRotate(a, (u64)i, tmp);
+        eval.add(a, tmp, a);
+        cpos /= 2;
+        if (rpos % 2 == 0)
+            eval.rightRotate(b, (u64)(i * w), tmp);
+        else
+            eval.leftRotate(b, (u64)(i * w), tmp);
+        eval.add(b, tmp, b);
+        rpos /= 2;
+    }
+    return lowRankTerms(eval, a, b, op1, op2, w, T, low_dim, tr);
 }
 
 template <>

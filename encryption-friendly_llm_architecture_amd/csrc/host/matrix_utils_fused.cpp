@@ -4,6 +4,7 @@
 // 7-limb, ~100-workgroup launch chain; here all independent rotations of a phase share one launch chain.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 
 #include "../../../include/hemm.h"
@@ -37,20 +38,23 @@ i64 pow2ceil(i64 v) {
     return p;
 }
 
+// units: length a diagonal wraps over (columns for sigma, rows for tau); sub: diagonals of one sign (the shorter
+// side of a rectangular tile) -- both in cells
 struct Geo {
-    i64 n, units, cell, bs, gs, step;
+    i64 n, units, sub, cell, bs, gs, step;
 };
 Geo geo(MaskKind kind, const TileTensorShape &s) {
     Geo g{};
-    const i64 w = s.getBlockWidth();
-    if (s.getNumRows() != s.getNumCols()) throw std::invalid_argument("[MatrixTransformer] only square tiles are supported");
-    g.n = s.getNumRows();
+    const i64 w = s.getBlockWidth(), rows = s.getNumRows(), cols = s.getNumCols();
     const bool packed = (kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical);
     const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
+    if (rows != cols && packed) throw std::invalid_argument("[MatrixTransformer] packed transforms need square tiles");
+    g.n = rows;
     g.cell = packed ? 2 : 1;
-    g.units = g.n / g.cell;
-    g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.units - 1)));
-    g.gs = (i64)std::ceil((double)(g.units - 1) / (double)g.bs);
+    g.units = (vertical ? rows : cols) / g.cell;
+    g.sub = std::min(rows, cols) / g.cell;
+    g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.sub - 1)));
+    g.gs = (i64)std::ceil((double)(g.sub - 1) / (double)g.bs);
     g.step = g.cell * (vertical ? w : 1);
     return g;
 }
@@ -232,13 +236,13 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
             std::vector<hemm_lin_term> neg, pos;
             for (i64 j = 0; j < gq.bs; j++) {
                 const i64 d = 1 + i * gq.bs + j - gq.units;
-                if (d >= 0) break;
+                if (d >= gq.sub - gq.units) break;
                 neg.push_back(lin(bb + (size_t)j * ctw, d));
             }
             push_group(std::move(neg), -(gq.units - i * gq.bs) * gq.step);
             for (i64 j = 0; j < gq.bs; j++) {
                 const i64 d = 1 + i * gq.bs + j;
-                if (d >= gq.units) break;
+                if (d >= gq.sub) break;
                 pos.push_back(lin(bb + (size_t)j * ctw, d));
             }
             push_group(std::move(pos), i * gq.bs * gq.step);

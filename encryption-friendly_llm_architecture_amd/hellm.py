@@ -51,8 +51,12 @@ def _L():
                   "hellm_diagonal_to_row"):
             getattr(L, n).argtypes = [vp, vp, pvp]
         for n in ("hellm_mult", "hellm_add", "hellm_complex_packing", "hellm_complex_packing_rev",
-                  "hellm_repack_not_bts"):
+                  "hellm_repack_not_bts", "hellm_repack_lora_opti"):
             getattr(L, n).argtypes = [vp, vp, vp, pvp]
+        L.hellm_matmul_high_low.argtypes = [vp, vp, vp, u32, u32, pvp]
+        L.hellm_matmul_low_high.argtypes = [vp, vp, vp, u32, u32, pvp]
+        L.hellm_matmul_low_low.argtypes = [vp, vp, vp, u32, u32, u32, pvp]
+        L.hellm_low_rank_block.argtypes = [vp, vp, u32, u32, pvp]
         L.hellm_level_down.argtypes = [vp, vp, u32, pvp]
         L.hellm_transpose_inplace.argtypes = [vp, vp, u32]
         L.hellm_complex_packing_inplace.argtypes = [vp, vp]
@@ -401,6 +405,37 @@ class HEMMer:
 
     def repack_not_bts(self, a, b):
         return self._new(Ct, "hellm_repack_not_bts", a.h, b.h)
+
+    def repack_lora_opti(self, a, b):
+        return self._new(Ct, "hellm_repack_lora_opti", a.h, b.h)
+
+    # LoRA low-rank path (rank 2): products with a thin operand and the block repacking around them
+    def matmul_high_low(self, a, b, in_col_block, target_level):
+        return self._new(Ct, "hellm_matmul_high_low", a.h, b.h, in_col_block, target_level)
+
+    def matmul_low_high(self, a, b, in_row_block, target_level):
+        return self._new(Ct, "hellm_matmul_low_high", a.h, b.h, in_row_block, target_level)
+
+    def matmul_low_low(self, a, b, in_col_block, in_row_block, target_level=4):
+        return self._new(Ct, "hellm_matmul_low_low", a.h, b.h, in_col_block, in_row_block, target_level)
+
+    def repack_to_one_col(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 0, block)
+
+    def repack_to_multi_col(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 1, block)
+
+    def repack_to_one_row(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 2, block)
+
+    def repack_to_multi_row(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 3, block)
+
+    def get_low_col_block(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 4, block)
+
+    def get_low_row_block(self, a, block):
+        return self._new(Ct, "hellm_low_rank_block", a.h, 5, block)
 
     def matmul_pre(self, a, target_level=4):
         return self._new(CtVec, "hellm_matmul_pre", a.h, target_level)

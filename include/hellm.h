@@ -134,6 +134,17 @@ int hellm_repack_cc(hellm_hemmer *h, hellm_ct *a, hellm_ct **out);              
 int hellm_complex_packing(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);        /* :176 */
 int hellm_complex_packing_rev(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);    /* :179 */
 int hellm_repack_not_bts(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out);                     /* :186 */
+int hellm_repack_lora_opti(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out);                   /* :184 */
+/* LoRA low-rank products and their repacking (HEMMer.hpp:202-232; rank = 2, reference ModelArgs.hpp:67).
+ * hellm_low_rank_block: which = 0 repackToOneCol, 1 repackToMultiCol, 2 repackToOneRow, 3 repackToMultiRow,
+ * 4 getLowColBlock, 5 getLowRowBlock. */
+int hellm_matmul_high_low(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_col_block,
+                          uint32_t target_level, hellm_ct **out);
+int hellm_matmul_low_high(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_row_block,
+                          uint32_t target_level, hellm_ct **out);
+int hellm_matmul_low_low(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_col_block,
+                         uint32_t in_row_block, uint32_t target_level, hellm_ct **out);
+int hellm_low_rank_block(hellm_hemmer *h, const hellm_ct *a, uint32_t which, uint32_t block, hellm_ct **out);
 int hellm_matmul_pre(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ctvec **out);      /* :190 */
 int hellm_matmul_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const hellm_pt *b, uint32_t target_level,
                        hellm_ct **out); /* :192 */

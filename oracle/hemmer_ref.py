@@ -254,30 +254,52 @@ class OracleEval:
 H, V, PH, PV, DIAG = "horizontal", "vertical", "packed_horizontal", "packed_vertical", "diagonal"
 
 
+def _dims(n):
+    """Tile shape: an int is a square tile, a pair is (rows, cols)."""
+    return (n, n) if isinstance(n, (int, np.integer)) else (int(n[0]), int(n[1]))
+
+
 def geometry(kind, n, w):
-    """(units, cell, bs, gs, step): diagonals in cells, cell size, BSGS sizes, slots per diagonal."""
+    """(units, cell, bs, gs, step): diagonals in cells, cell size, BSGS sizes, slots per diagonal.
+    For a rectangular tile (sigma / tau only, generateHorizontalMask :129-217, generateVerticalMask
+    :330-419) `units` is the length a diagonal wraps over (columns for sigma, rows for tau) and the
+    BSGS sizes come from the shorter side (sub_dim)."""
+    rows, cols = _dims(n)
     if kind == DIAG:
-        count = 2 * n - 1
+        assert rows == cols
+        count = 2 * rows - 1
         bs = math.ceil(math.sqrt(count))
-        return n, 1, bs, math.ceil(count / bs), w - 1
+        return rows, 1, bs, math.ceil(count / bs), w - 1
     cell = 2 if kind in (PH, PV) else 1
-    units = n // cell
-    bs = math.ceil(math.sqrt(2 * units - 1))
-    gs = math.ceil((units - 1) / bs)
+    assert cell == 1 or rows == cols
+    units = (cols if kind in (H, PH) else rows) // cell
+    sub = sub_dim(kind, n)
+    bs = math.ceil(math.sqrt(2 * sub - 1))
+    gs = math.ceil((sub - 1) / bs)
     step = cell * (w if kind in (V, PV) else 1)
     return units, cell, bs, gs, step
 
 
+def sub_dim(kind, n):
+    """Number of diagonals of one sign: the shorter side of the tile, in cells."""
+    rows, cols = _dims(n)
+    return min(rows, cols) // (2 if kind in (PH, PV) else 1)
+
+
 def transform_mask(kind, n, w, slots, idx):
     """Slot pattern of diagonal idx (no pre-rotation)."""
+    rows, cols = _dims(n)
     units, cell, _, _, _ = geometry(kind, n, w)
+    sub = sub_dim(kind, n)
     r = np.arange(slots) // w
     c = np.arange(slots) % w
-    R = (r % n) // cell
-    C = (c % n) // cell
+    R = (r % rows) // cell
+    C = (c % cols) // cell
     if kind in (H, PH):
+        R = R % sub                      # a tall tile repeats the pattern every sub_dim rows
         on = (R == idx) & (C < units - idx) if idx >= 0 else (R == units + idx) & (C >= -idx)
     elif kind in (V, PV):
+        C = C % sub                      # a wide tile repeats it every sub_dim columns
         on = (C == idx) & (R < units - idx) if idx >= 0 else (C == units + idx) & (R >= -idx)
     else:
         on = (C - R) == idx
@@ -288,7 +310,7 @@ def prerotated_mask(kind, n, w, slots, idx):
     units, _, bs, _, step = geometry(kind, n, w)
     m = transform_mask(kind, n, w, slots, idx)
     if kind == DIAG:
-        i = (idx + n - 1) // bs
+        i = (idx + _dims(n)[0] - 1) // bs
         return np.roll(m, i * bs * step)
     if idx > 0:
         i = (idx - 1) // bs
@@ -323,6 +345,7 @@ def row_masks(n, w, slots):
 # --------------------------------------------------------------------------------------------
 def diagonal_transform(ev, ct, kind, n, w):
     units, _, bs, gs, step = geometry(kind, n, w)
+    sub = sub_dim(kind, n)
     level = ev.level_of(ct)
     enc = lambda idx: ev.encode(prerotated_mask(kind, n, w, ev.slots, idx), level)
     baby = []
@@ -333,7 +356,7 @@ def diagonal_transform(ev, ct, kind, n, w):
         group = None
         for j in range(bs):
             d = 1 + i * bs + j - units
-            if d >= 0:
+            if d >= sub - units:
                 break
             t = ev.mult_plain_no_rescale(baby[j], enc(d))
             group = t if group is None else ev.add(group, t)
@@ -342,7 +365,7 @@ def diagonal_transform(ev, ct, kind, n, w):
         group = None
         for j in range(bs):
             d = 1 + i * bs + j
-            if d >= units:
+            if d >= sub:
                 break
             t = ev.mult_plain_no_rescale(baby[j], enc(d))
             group = t if group is None else ev.add(group, t)
@@ -529,6 +552,7 @@ def mult_mat_mat_reuse(ev, tmp, b_pt, T, step=None):
 def diagonal_transform_fused(orc, ct, kind, n, w):
     from .oracle import Ct
     units, _, bs, gs, step = geometry(kind, n, w)
+    sub = sub_dim(kind, n)
     level, nq = ct.level, ct.nq
     enc = lambda idx: orc.encode(prerotated_mask(kind, n, w, orc.slots, idx), level)
     ext = orc.modup(ct.data[1])
@@ -546,9 +570,9 @@ def diagonal_transform_fused(orc, ct, kind, n, w):
             rots.append(r)
 
     for i in range(gs):
-        neg = [(baby[j], 1 + i * bs + j - units) for j in range(bs) if 1 + i * bs + j - units < 0]
+        neg = [(baby[j], 1 + i * bs + j - units) for j in range(bs) if 1 + i * bs + j - units < sub - units]
         push(neg, -(units - i * bs) * step)
-        pos = [(baby[j], 1 + i * bs + j) for j in range(bs) if 1 + i * bs + j < units]
+        pos = [(baby[j], 1 + i * bs + j) for j in range(bs) if 1 + i * bs + j < sub]
         push(pos, i * bs * step)
     sums = []
     for terms in groups:
@@ -678,6 +702,194 @@ def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
         msg[np.arange(h) * 2 * w + c] = np.roll(left[:, c], -c)
         msg[np.arange(h) * 2 * w + w + c] = np.roll(right[:, c], -c)
     return msg
+
+
+# ---- LoRA low-rank products (MatrixUtils.cpp:1681-1996) and their repacking (HEMMer.cpp:1055-1091, 2131-2332) ------
+LOW_DIM = 2            # ModelArgs::LOW_DIM (ModelArgs.hpp:67)
+
+
+def _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim):
+    """Shared tail of the three products: sigma(A) (.) tau(B) plus the low_dim - 1 shifted terms
+    (e.g. :1716-1766): the full product's loop cut after low_dim terms."""
+    cm = col_masks(sa[1], ev.slots)
+    rm = row_masks(sb[0], w, ev.slots)
+    res = ev.mult(a, b)
+    a = ev.left_rotate(a, 1)
+    b = ev.left_rotate(b, w)
+    a_wrap = ev.right_rotate(a, w // 2)
+    b_wrap = ev.right_rotate(b, sa[0] * w)
+    acc = None
+    for i in range(1, low_dim):
+        if i > 1:
+            a = ev.left_rotate(a, 1)
+            a_wrap = ev.left_rotate(a_wrap, 1)
+            b = ev.left_rotate(b, w)
+            b_wrap = ev.left_rotate(b_wrap, w)
+        enc = lambda m: ev.encode(m, T + 2)
+        t1 = ev.rescale(ev.masked_sum(a, enc(cm[2 * i + 1]), a_wrap, enc(cm[2 * i])))
+        t2 = ev.rescale(ev.masked_sum(b, enc(rm[2 * i + 1]), b_wrap, enc(rm[2 * i])))
+        t = ev.tensor(t1, t2)
+        acc = t if acc is None else ev.add(acc, t)
+    if acc is None:
+        return res
+    return ev.add(res, ev.rescale(ev.relinearize(acc)))
+
+
+def mult_mat_mat_high_low(ev, a, b, in_col_block, T, sa, sb, w, low_dim=LOW_DIM, transform=diagonal_transform):
+    """multMatMatHighLow (:1681-1770).  sa, sb = (rows, cols) of the operands' tile shapes.  B holds low_dim
+    columns at column block in_col_block of every tile; tau runs on (rows, low_dim) tiles and the
+    result is spread along the diagonal of column blocks before the truncated product."""
+    a = ev.level_down(a, T + 3)
+    b = ev.level_down(b, T + 3)
+    a = transform(ev, a, H, sa, w)
+    b = transform(ev, b, V, (sb[0], low_dim), w)
+    pos, i = in_col_block, low_dim
+    while i < w // 2:
+        if pos % 2 == 0:
+            tmp = ev.right_rotate(ev.left_rotate(b, i * w), i)
+        else:
+            tmp = ev.left_rotate(b, i)
+            b = ev.left_rotate(b, i * w)
+        b = ev.add(b, tmp)
+        pos //= 2
+        i <<= 1
+    return _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim)
+
+
+def mult_mat_mat_low_high(ev, a, b, in_row_block, T, sa, sb, w, low_dim=LOW_DIM, transform=diagonal_transform):
+    """multMatMatLowHigh (:1772-1876): A holds low_dim rows at row block in_row_block; they are copied to
+    every row block before sigma."""
+    a = ev.level_down(a, T + 3)
+    b = ev.level_down(b, T + 3)
+    pos, i = in_row_block, low_dim
+    while i < w // 2:
+        tmp = ev.right_rotate(a, i * w) if pos % 2 == 0 else ev.left_rotate(a, i * w)
+        a = ev.add(a, tmp)
+        pos //= 2
+        i <<= 1
+    a = transform(ev, a, H, sa, w)
+    b = transform(ev, b, V, sb, w)
+    return _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim)
+
+
+def mult_mat_mat_low_low(ev, a, b, in_col_block, in_row_block, T, sa, sb, w, low_dim=LOW_DIM,
+                         transform=diagonal_transform):
+    """multMatMatLowLow (:1878-1996): A (rows x low_dim at column block in_col_block) times B (low_dim x cols
+    at row block in_row_block); sigma / tau run on the thin shapes and are then copied over the blocks."""
+    a = ev.level_down(a, T + 3)
+    b = ev.level_down(b, T + 3)
+    a = transform(ev, a, H, (sa[0], low_dim), w)
+    b = transform(ev, b, V, (low_dim, sb[1]), w)
+    cpos, rpos, i = in_col_block, in_row_block, low_dim
+    while i < w // 2:
+        tmp = ev.right_rotate(a, i) if cpos % 2 == 0 else ev.left_rotate(a, i)
+        a = ev.add(a, tmp)
+        cpos //= 2
+        tmp = ev.right_rotate(b, i * w) if rpos % 2 == 0 else ev.left_rotate(b, i * w)
+        b = ev.add(b, tmp)
+        rpos //= 2
+        i <<= 1
+    return _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim)
+
+
+def _mult_msg(ev, x, msg):
+    return ev.mult_pt(x, ev.encode(msg, ev.level_of(x)))
+
+
+def low_col_block_mask(rows, cols, w, block, slots, low_dim=LOW_DIM, every_tile=True):
+    m = np.zeros(slots, dtype=np.complex128)
+    for i in range(rows):
+        for k in range(0, w if every_tile else 1, cols):
+            m[i * w + k + block * low_dim: i * w + k + (block + 1) * low_dim] = 1
+    return m
+
+
+def low_row_block_mask(cols, w, block, slots, low_dim=LOW_DIM, width=None):
+    m = np.zeros(slots, dtype=np.complex128)
+    for i in range(block * low_dim, (block + 1) * low_dim):
+        m[i * w: i * w + (w if width is None else width)] = 1
+    return m
+
+
+def get_low_col_block(ev, x, block, rows, cols, w, low_dim=LOW_DIM):
+    """HEMMer::getLowColBlock (HEMMer.cpp:2294-2312)."""
+    return _mult_msg(ev, x, low_col_block_mask(rows, cols, w, block, ev.slots, low_dim))
+
+
+def get_low_row_block(ev, x, block, cols, w, low_dim=LOW_DIM):
+    """HEMMer::getLowRowBlock (HEMMer.cpp:2314-2332)."""
+    return _mult_msg(ev, x, low_row_block_mask(cols, w, block, ev.slots, low_dim))
+
+
+def repack_to_one_col(ev, x, out_block, rows, cols, w, low_dim=LOW_DIM):
+    """HEMMer::repackToOneCol (HEMMer.cpp:2137-2178)."""
+    pos, i = out_block, low_dim
+    while i < w:
+        x = ev.add(x, ev.left_rotate(x, i) if pos % 2 == 0 else ev.right_rotate(x, i))
+        pos //= 2
+        i <<= 1
+    x = _mult_msg(ev, x, low_col_block_mask(rows, cols, w, out_block, ev.slots, low_dim, every_tile=False))
+    i = cols
+    while i < w:
+        x = ev.add(x, ev.right_rotate(x, cols))
+        i <<= 1
+    return x
+
+
+def repack_to_multi_col(ev, x, out_block, rows, cols, w, low_dim=LOW_DIM):
+    """HEMMer::repackToMultiCol (HEMMer.cpp:2180-2215)."""
+    pos, i = out_block, low_dim
+    while i < w // 2:
+        x = ev.add(x, ev.left_rotate(x, i) if pos % 2 == 0 else ev.right_rotate(x, i))
+        pos //= 2
+        i <<= 1
+    return _mult_msg(ev, x, low_col_block_mask(rows, cols, w, out_block, ev.slots, low_dim))
+
+
+def repack_to_one_row(ev, x, out_block, rows, cols, w, low_dim=LOW_DIM):
+    """HEMMer::repackToOneRow (HEMMer.cpp:2217-2259)."""
+    pos, i = out_block, low_dim
+    while i < rows:
+        x = ev.add(x, ev.left_rotate(x, i * w) if pos % 2 == 0 else ev.right_rotate(x, i * w))
+        pos //= 2
+        i <<= 1
+    i = cols
+    while i < w:
+        x = ev.add(x, ev.left_rotate(x, cols))
+        i <<= 1
+    x = _mult_msg(ev, x, low_row_block_mask(cols, w, out_block, ev.slots, low_dim, width=cols))
+    i = cols
+    while i < w:
+        x = ev.add(x, ev.right_rotate(x, cols))
+        i += cols
+    return x
+
+
+def repack_to_multi_row(ev, x, out_block, rows, w, low_dim=LOW_DIM):
+    """HEMMer::repackToMultiRow (HEMMer.cpp:2261-2292)."""
+    pos, i = out_block, low_dim
+    while i < rows:
+        x = ev.add(x, ev.left_rotate(x, i * w) if pos % 2 == 0 else ev.right_rotate(x, i * w))
+        pos //= 2
+        i <<= 1
+    return _mult_msg(ev, x, low_row_block_mask(0, w, out_block, ev.slots, low_dim))
+
+
+def repack_lora_opti(ev, t1, t2, n):
+    """HEMMer::repack_loraOpti (HEMMer.cpp:1055-1091); both inputs arrive un-rescaled."""
+    t1, t2 = ev.rescale(t1), ev.rescale(t2)
+    out = ev.add(t1, ev.conjugate(t1))
+    tmp = ev.mult_imag_unit(ev.add(t2, ev.conjugate(t2)))
+    out = ev.add(out, tmp)
+    tmp = ev.left_rotate(out, n)
+    out = ev.add(out, tmp)
+    conj = ev.conjugate(out)
+    out = ev.add(out, conj)
+    tmp = ev.mult_imag_unit(ev.sub(conj, tmp))
+    half = _message2(np.full((n, n), 0.5), np.zeros((n, n)), ev.slots)
+    tmp = _mult_msg(ev, tmp, half)
+    out = _mult_msg(ev, out, half)
+    return ev.add(out, ev.right_rotate(tmp, n))
 
 
 # ---- rotate-and-sum reductions on the pair layout (HEMMer.cpp:2512-2530, 882-919, 1245-1253, 1699-1760) -----------

@@ -5,6 +5,8 @@
     the hoisted PCMM path (matMulPre once per activation tile pair, matMulReUse per weight tile group), plus
     the rank-8 update X A B with A (768 x 8) and B (8 x 768) zero-padded to 128-wide encrypted tiles
     (two chained CCMMs);
+  * the same rank-2 update through the low-rank path the reference's LoRA layers use (matMulHighLow per
+    activation pair, repackToOneCol, matMulLowLow per output pair; src/TransformerBlock.cpp:1785-1835);
   * one attention head: S = Q K^T (CCMM), a degree-15 Chebyshev polynomial of the scores, then P V (CCMM).
 """
 import numpy as np
@@ -64,6 +66,39 @@ def test_lora_forward_projection(H):
     Bj[:rank] = B[:, :n]
     xab = H.single_cc_matmul(xa, H.encrypt(Bj), 4)
     assert np.abs(H.decrypt(xab) - (X @ A @ B)[:, :n]).max() < TOL
+
+
+def test_lora_low_rank_path(H):
+    """X (128 x 768 as three pair-layout ciphertexts) times A (768 x 2) times B (2 x 768), both factors encrypted
+    in the block layout of the LoRA weights: tile t of A sits in column block t // 2 of the left (even t) or
+    right (odd t) half, tile t of B likewise in row block t // 2.  The reference refreshes X A by bootstrapping
+    between the two products; here the second product simply runs at the levels that are left."""
+    rng = np.random.default_rng(13)
+    n, tiles, rank = 128, 6, 2
+    X = 0.1 * rng.normal(size=(n, n * tiles))
+    A = 0.1 * rng.normal(size=(n * tiles, rank))
+    B = 0.1 * rng.normal(size=(rank, n * tiles))
+    wa = [np.zeros((n, n)), np.zeros((n, n))]
+    wb = [np.zeros((n, n)), np.zeros((n, n))]
+    for t in range(tiles):
+        wa[t % 2][:, (t // 2) * rank:(t // 2 + 1) * rank] = A[t * n:(t + 1) * n]
+        wb[t % 2][(t // 2) * rank:(t // 2 + 1) * rank] = B[:, t * n:(t + 1) * n]
+    cwa, cwb = H.encrypt2(*wa), H.encrypt2(*wb)
+    xa = None
+    for i in range(tiles // 2):
+        cx = H.encrypt2(X[:, 2 * i * n:(2 * i + 1) * n], X[:, (2 * i + 1) * n:(2 * i + 2) * n])
+        t = H.matmul_high_low(cx, H.get_low_col_block(cwa, i), i, 5)
+        xa = t if xa is None else H.add(xa, t)
+    xa = H.repack_to_one_col(xa, 0)
+    assert xa.info()["level"] == 4
+    d = H.decrypt2(xa)
+    assert np.abs(d[0][:, :rank] - X @ A).max() < TOL and np.abs(d[1][:, :rank] - X @ A).max() < TOL
+    want = X @ A @ B
+    for i in range(tiles // 2):
+        y = H.matmul_low_low(xa, H.get_low_row_block(cwb, i), 0, i, 1)
+        d = H.decrypt2(y)
+        assert np.abs(d[0] - want[:, 2 * i * n:(2 * i + 1) * n]).max() < TOL
+        assert np.abs(d[1] - want[:, (2 * i + 1) * n:(2 * i + 2) * n]).max() < TOL
 
 
 def test_attention_head():
