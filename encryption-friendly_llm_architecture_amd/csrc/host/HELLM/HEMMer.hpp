@@ -150,6 +150,19 @@ public:
     // repack of two un-rescaled product halves used by the LoRA path (src/HEMMer.cpp:1055-1091)
     CtxtTensor repack_loraOpti(CtxtTensor &t1, CtxtTensor &t2) const;
 
+    // Rank-2 LoRA through element-wise products, the form the reference's layers run
+    // (src/TransformerBlock.cpp:2199-2365).  Row 2i+j of the weight tile `lora_wa` holds column j of A for the i-th
+    // pair of activation tiles, row 2i+j of `lora_wb` row j of B for the i-th pair of output tiles.
+    //   loraRank2Down: X a_0 and X a_1, each in column 0 of the left tile (two ciphertexts);
+    //   loraRank2Up:   (X A) B as n_out pair-layout ciphertexts.
+    // The weights are first brought to `weight_level` (9 and 6 in the reference).
+    std::vector<CtxtTensor> loraRank2Down(const std::vector<CtxtTensor> &cur, const CtxtTensor &lora_wa,
+                                          u64 weight_level = 9) const;
+    std::vector<CtxtTensor> loraRank2Up(const std::vector<CtxtTensor> &xa, const CtxtTensor &lora_wb, u64 n_out,
+                                        u64 weight_level = 6) const;
+    void maskFirstRowInplace(CtxtTensor &tensor) const;       // src/HEMMer.cpp:1259-1261
+    void maskFirstColOnlyInplace(CtxtTensor &tensor) const;   // src/HEMMer.cpp:1255-1257 (left tile only)
+
     // Schedule of singleCCMatMul / packedMatMul / matMulPre: batched launches with hoisted rotations
     // (default) or one evaluator call per step in the reference's order.  `batch` = shifts per launch.
     void setFused(bool on, u64 batch = 16) {
@@ -168,7 +181,8 @@ private:
     std::vector<u64> transformRotations(MaskKind kind, i64 width) const;
     // the same for a (possibly rectangular) sigma / tau shape under the current schedule
     std::vector<u64> transformRotations(MaskKind kind, const TileTensorShape &shape) const;
-    void ensureLogStepKeys(i64 first, i64 bound, i64 unit) const;   // +-i*unit for i = first, 2 first, ... < bound
+    void ensureLogStepKeys(i64 first, i64 bound, i64 unit) const;
+    std::vector<std::vector<CtxtTensor>> splitWeightRows(const CtxtTensor &weight, u64 count) const;   // +-i*unit for i = first, 2 first, ... < bound
 
     int device_id_ = 0;
     Context context_;

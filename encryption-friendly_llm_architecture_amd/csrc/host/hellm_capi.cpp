@@ -577,5 +577,20 @@ int hellm_low_rank_block(hellm_hemmer *h, const hellm_ct *a, uint32_t which, uin
                                      : m.getLowRowBlock(a->t, block)};
     FACADE_CATCH
 }
+// up = 0: loraRank2Down(cts[0..count), weight) -> out[0..2); up = 1: loraRank2Up(cts[0..2), weight, n_out) -> out[0..n_out)
+int hellm_lora_rank2(hellm_hemmer *h, int up, const hellm_ct *const *cts, uint32_t count, const hellm_ct *weight,
+                     uint32_t n_out, uint32_t weight_level, hellm_ct **out) {
+    FACADE_TRY
+    need(h && cts && weight && out && count >= 1, "null argument");
+    std::vector<HELLM::CtxtTensor> v;
+    for (uint32_t i = 0; i < count; i++) {
+        need(cts[i] != nullptr, "null ciphertext");
+        v.push_back(cts[i]->t);
+    }
+    std::vector<HELLM::CtxtTensor> r =
+        up ? h->m->loraRank2Up(v, weight->t, n_out, weight_level) : h->m->loraRank2Down(v, weight->t, weight_level);
+    for (size_t i = 0; i < r.size(); i++) out[i] = new hellm_ct{r[i]};
+    FACADE_CATCH
+}
 
 }  // extern "C"

@@ -679,6 +679,95 @@ CtxtTensor HEMMer::repack_loraOpti(CtxtTensor &t1, CtxtTensor &t2) const {
     return out;
 }
 
+// ---- rank-2 LoRA through element-wise products ---------------------------------------------------------------
+void HEMMer::maskFirstRowInplace(CtxtTensor &tensor) const {
+    Matrix first(dim_, dim_, 0.0);
+    for (i64 c = 0; c < dim_; c++) first.at(0, c) = 1.0;
+    eval_.mult(tensor.get(), message2(first, first), tensor.get());
+}
+void HEMMer::maskFirstColOnlyInplace(CtxtTensor &tensor) const {
+    Matrix first(dim_, dim_, 0.0), zero(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++) first.at(r, 0) = 1.0;
+    eval_.mult(tensor.get(), message2(first, zero), tensor.get());
+}
+// rows 2i and 2i+1 of the weight tile, each moved to row 0, masked and copied to every row
+std::vector<std::vector<CtxtTensor>> HEMMer::splitWeightRows(const CtxtTensor &weight, u64 count) const {
+    const u64 w = (u64)weight.getBlockWidth(), n = (u64)dim_;
+    std::vector<u64> rots{w};
+    for (u64 i = 1; i < count; i++) rots.push_back(i * 2 * w);
+    ensureRotationKeys(rots);
+    ensureLogStepKeys(1, (i64)n, (i64)w);
+    std::vector<std::vector<CtxtTensor>> out;
+    CtxtTensor tmp{weight};
+    for (u64 i = 0; i < count; i++) {
+        if (i > 0) eval_.leftRotate(weight.get(), i * 2 * w, tmp.get());
+        std::vector<CtxtTensor> pair{tmp, tmp};
+        maskFirstRowInplace(pair[0]);
+        eval_.leftRotate(pair[1].get(), w, pair[1].get());
+        maskFirstRowInplace(pair[1]);
+        out.push_back(std::move(pair));
+    }
+    Ciphertext t(context_);
+    for (auto &pair : out)
+        for (auto &x : pair)
+            for (u64 rot = 1; rot < n; rot <<= 1) {
+                eval_.rightRotate(x.get(), rot * w, t);
+                eval_.add(x.get(), t, x.get());
+            }
+    return out;
+}
+std::vector<CtxtTensor> HEMMer::loraRank2Down(const std::vector<CtxtTensor> &cur, const CtxtTensor &lora_wa,
+                                              u64 weight_level) const {
+    if (cur.empty()) throw std::invalid_argument("[loraRank2Down] no activation tiles");
+    const u64 w = (u64)lora_wa.getBlockWidth();
+    CtxtTensor wa{lora_wa};
+    eval_.levelDown(wa.get(), weight_level, wa.get());
+    auto weights = splitWeightRows(wa, cur.size());
+    ensureLogStepKeys(1, (i64)w, 1);
+    std::vector<CtxtTensor> out;
+    Ciphertext t(context_);
+    for (u64 j = 0; j < 2; j++) {
+        CtxtTensor acc{wa};
+        eval_.mult(cur[0].get(), weights[0][j].get(), acc.get());
+        for (size_t i = 1; i < cur.size(); i++) {
+            eval_.mult(cur[i].get(), weights[i][j].get(), t);
+            eval_.add(acc.get(), t, acc.get());
+        }
+        for (u64 rot = 1; rot < w; rot <<= 1) {
+            eval_.leftRotate(acc.get(), rot, t);
+            eval_.add(acc.get(), t, acc.get());
+        }
+        maskFirstColOnlyInplace(acc);
+        out.push_back(std::move(acc));
+    }
+    return out;
+}
+std::vector<CtxtTensor> HEMMer::loraRank2Up(const std::vector<CtxtTensor> &xa_in, const CtxtTensor &lora_wb, u64 n_out,
+                                            u64 weight_level) const {
+    if (xa_in.size() != 2) throw std::invalid_argument("[loraRank2Up] two column ciphertexts are needed");
+    const u64 w = (u64)lora_wb.getBlockWidth();
+    CtxtTensor wb{lora_wb};
+    eval_.levelDown(wb.get(), weight_level, wb.get());
+    auto weights = splitWeightRows(wb, n_out);
+    ensureLogStepKeys(1, (i64)w, 1);
+    std::vector<CtxtTensor> xa{xa_in};
+    Ciphertext t(context_);
+    for (auto &x : xa)
+        for (u64 rot = 1; rot < w; rot <<= 1) {
+            eval_.rightRotate(x.get(), rot, t);
+            eval_.add(x.get(), t, x.get());
+        }
+    std::vector<CtxtTensor> out;
+    for (u64 i = 0; i < n_out; i++) {
+        CtxtTensor y{wb};
+        eval_.mult(xa[0].get(), weights[i][0].get(), y.get());
+        eval_.mult(xa[1].get(), weights[i][1].get(), t);
+        eval_.add(y.get(), t, y.get());
+        out.push_back(std::move(y));
+    }
+    return out;
+}
+
 // x + conj(x) = 2 Re(x)
 CtxtTensor HEMMer::repackCC(CtxtTensor &t) const {
     CtxtTensor out(t);

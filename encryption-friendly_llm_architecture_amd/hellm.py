@@ -57,6 +57,7 @@ def _L():
         L.hellm_matmul_low_high.argtypes = [vp, vp, vp, u32, u32, pvp]
         L.hellm_matmul_low_low.argtypes = [vp, vp, vp, u32, u32, u32, pvp]
         L.hellm_low_rank_block.argtypes = [vp, vp, u32, u32, pvp]
+        L.hellm_lora_rank2.argtypes = [vp, ctypes.c_int, ctypes.POINTER(vp), u32, vp, u32, u32, ctypes.POINTER(vp)]
         L.hellm_level_down.argtypes = [vp, vp, u32, pvp]
         L.hellm_transpose_inplace.argtypes = [vp, vp, u32]
         L.hellm_complex_packing_inplace.argtypes = [vp, vp]
@@ -436,6 +437,20 @@ class HEMMer:
 
     def get_low_row_block(self, a, block):
         return self._new(Ct, "hellm_low_rank_block", a.h, 5, block)
+
+    def _lora_rank2(self, up, cts, weight, n_out, weight_level):
+        arr = (vp * len(cts))(*[t.h for t in cts])
+        out = (vp * n_out)()
+        check(_L().hellm_lora_rank2(self.h, up, arr, len(cts), weight.h, n_out, weight_level, out))
+        return [Ct(self, vp(out[i])) for i in range(n_out)]
+
+    def lora_rank2_down(self, cur, lora_wa, weight_level=9):
+        """X a_0, X a_1 (column 0 of the left tile) from pair-layout activation tiles and the A weight tile."""
+        return self._lora_rank2(0, cur, lora_wa, 2, weight_level)
+
+    def lora_rank2_up(self, xa, lora_wb, n_out, weight_level=6):
+        """(X A) B as n_out pair-layout ciphertexts from the two outputs of lora_rank2_down and the B weight tile."""
+        return self._lora_rank2(1, xa, lora_wb, n_out, weight_level)
 
     def matmul_pre(self, a, target_level=4):
         return self._new(CtVec, "hellm_matmul_pre", a.h, target_level)

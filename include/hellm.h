@@ -145,6 +145,11 @@ int hellm_matmul_low_high(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b,
 int hellm_matmul_low_low(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, uint32_t in_col_block,
                          uint32_t in_row_block, uint32_t target_level, hellm_ct **out);
 int hellm_low_rank_block(hellm_hemmer *h, const hellm_ct *a, uint32_t which, uint32_t block, hellm_ct **out);
+/* Rank-2 LoRA through element-wise products (the reference runs it inline, src/TransformerBlock.cpp:2199-2365).
+ * up = 0: X a_0, X a_1 from `count` activation ciphertexts and the weight tile of A -> out[0..2);
+ * up = 1: (X A) B from the two ciphertexts of up = 0 and the weight tile of B -> out[0..n_out). */
+int hellm_lora_rank2(hellm_hemmer *h, int up, const hellm_ct *const *cts, uint32_t count, const hellm_ct *weight,
+                     uint32_t n_out, uint32_t weight_level, hellm_ct **out);
 int hellm_matmul_pre(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ctvec **out);      /* :190 */
 int hellm_matmul_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const hellm_pt *b, uint32_t target_level,
                        hellm_ct **out); /* :192 */

@@ -892,6 +892,70 @@ def repack_lora_opti(ev, t1, t2, n):
     return ev.add(out, ev.right_rotate(tmp, n))
 
 
+# ---- rank-2 LoRA through element-wise products (TransformerBlock.cpp:2199-2365) ------------------------------------
+def _first_row_mask(n, slots):
+    m = np.zeros((n, n))
+    m[0] = 1
+    return _message2(m, m, slots)
+
+
+def _first_col_only_mask(n, slots):
+    m = np.zeros((n, n))
+    m[:, 0] = 1
+    return _message2(m, np.zeros((n, n)), slots)
+
+
+def _split_weight_rows(ev, wt, count, n, w):
+    """Rows 2i and 2i+1 of the weight tile, each moved to row 0, masked and copied to all n rows
+    (:2222-2251, :2294-2335)."""
+    first = _first_row_mask(n, ev.slots)
+    out = []
+    for i in range(count):
+        t = wt if i == 0 else ev.left_rotate(wt, i * 2 * w)
+        pair = [_mult_msg(ev, t, first), _mult_msg(ev, ev.left_rotate(t, w), first)]
+        out.append(pair)
+    for pair in out:
+        for j in range(2):
+            rot = 1
+            while rot < n:
+                pair[j] = ev.add(pair[j], ev.right_rotate(pair[j], rot * w))
+                rot <<= 1
+    return out
+
+
+def lora_rank2_down(ev, cur, wa, n, w, weight_level):
+    """X a_0 and X a_1 in column 0 of the left tile: row 2i+j of `wa` holds column j of A for the i-th pair
+    of activation tiles (:2203-2283)."""
+    wa = ev.level_down(wa, weight_level)
+    wts = _split_weight_rows(ev, wa, len(cur), n, w)
+    out = []
+    for j in range(2):
+        acc = None
+        for i, x in enumerate(cur):
+            t = ev.mult(x, wts[i][j])
+            acc = t if acc is None else ev.add(acc, t)
+        rot = 1
+        while rot < w:
+            acc = ev.add(acc, ev.left_rotate(acc, rot))
+            rot <<= 1
+        out.append(_mult_msg(ev, acc, _first_col_only_mask(n, ev.slots)))
+    return out
+
+
+def lora_rank2_up(ev, xa, wb, n_out, n, w, weight_level):
+    """(X A) B for n_out pairs of output tiles: row 2i+j of `wb` holds row j of B for output pair i
+    (:2287-2358)."""
+    wb = ev.level_down(wb, weight_level)
+    wts = _split_weight_rows(ev, wb, n_out, n, w)
+    xa = list(xa)
+    for j in range(2):
+        rot = 1
+        while rot < w:
+            xa[j] = ev.add(xa[j], ev.right_rotate(xa[j], rot))
+            rot <<= 1
+    return [ev.add(ev.mult(xa[0], wts[i][0]), ev.mult(xa[1], wts[i][1])) for i in range(n_out)]
+
+
 # ---- rotate-and-sum reductions on the pair layout (HEMMer.cpp:2512-2530, 882-919, 1245-1253, 1699-1760) -----------
 def _message2(a, b, slots):
     """HEMMer::message2 (HEMMer.cpp:243-262): [A | B] row-major with block width 2 * cols."""

@@ -156,3 +156,35 @@ def test_repack_lora_opti(small):
     out = H.decrypt_slots(got).reshape(n, 2 * n)
     assert np.abs(out[:, :n] - 2 * (A0 + A1)).max() < 2 ** -16
     assert np.abs(out[:, n:] - (2 * A0 + B1 + 1j * A0)).max() < 2 ** -16
+
+
+def test_lora_rank2_elementwise_path(small):
+    """Element-wise rank-2 form: residues against the oracle, values against float64."""
+    H, orc, ev = small
+    n, w, m = N_TILE, W, 2
+    rng = np.random.default_rng(25)
+    X = rng.uniform(-1, 1, (n, 2 * n * m))
+    A = rng.normal(0, 0.3, (2 * n * m, 2))
+    B = rng.normal(0, 0.3, (2, 2 * n * m))
+    wa, wb = np.zeros((n, w)), np.zeros((n, w))
+    for i in range(m):
+        for j in range(2):
+            wa[2 * i + j] = A[2 * n * i:2 * n * (i + 1), j]
+            wb[2 * i + j] = B[j, 2 * n * i:2 * n * (i + 1)]
+    enc2 = lambda M: H.encrypt2(M[:, :n], M[:, n:])
+    cur = [enc2(X[:, 2 * n * i:2 * n * (i + 1)]) for i in range(m)]
+    cwa, cwb = enc2(wa), enc2(wb)
+    ocur, owa, owb = [to_oracle(orc, c) for c in cur], to_oracle(orc, cwa), to_oracle(orc, cwb)
+    xa = H.lora_rank2_down(cur, cwa, weight_level=7)
+    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7)
+    for j in range(2):
+        assert np.array_equal(xa[j].residues(), oxa[j].data)
+        z = H.decrypt_slots(xa[j]).real.reshape(n, w)
+        assert np.abs(z[:, 0] - X @ A[:, j]).max() < 2 ** -16 and np.abs(z[:, 1:]).max() < 2 ** -16
+    out = H.lora_rank2_up(xa, cwb, m, weight_level=4)
+    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4)
+    want = X @ A @ B
+    for i in range(m):
+        assert np.array_equal(out[i].residues(), oout[i].data)
+        z = H.decrypt_slots(out[i]).real.reshape(n, w)
+        assert np.abs(z - want[:, 2 * n * i:2 * n * (i + 1)]).max() < 2 ** -16

@@ -127,3 +127,29 @@ def test_repack_lora_opti_closed_form(sim):
     s1L, s1R, s2L, s2R = 2 * t[0][0].real, 2 * t[0][1].real, 2 * t[1][0].real, 2 * t[1][1].real
     assert np.abs(out[:, :n] - (s1L + s1R)).max() < 1e-12
     assert np.abs(out[:, n:] - (s2R + 0.5 * s2L + 0.5j * s1L)).max() < 1e-12
+
+
+def test_lora_rank2_elementwise_path(sim):
+    """The production rank-2 form (element-wise products and rotate-and-sum, TransformerBlock.cpp:2199-2365):
+    X (n x 6n, three pair-layout tiles) times A (6n x 2) gives two column ciphertexts, then times B (2 x 6n)."""
+    n, w, m = N_TILE, W, 3
+    rng = np.random.default_rng(31)
+    X = rng.normal(size=(n, 2 * n * m))
+    A = rng.normal(size=(2 * n * m, 2))
+    B = rng.normal(size=(2, 2 * n * m))
+    wa, wb = rng.normal(size=(n, w)), rng.normal(size=(n, w))     # unused rows hold other data
+    for i in range(m):
+        for j in range(2):
+            wa[2 * i + j] = A[2 * n * i:2 * n * (i + 1), j]
+            wb[2 * i + j] = B[j, 2 * n * i:2 * n * (i + 1)]
+    cur = [sim.encrypt(X[:, 2 * n * i:2 * n * (i + 1)].reshape(-1)) for i in range(m)]
+    xa = R.lora_rank2_down(sim, cur, sim.encrypt(wa.reshape(-1)), n, w, 9)
+    for j in range(2):
+        z = xa[j].z.real.reshape(n, w)
+        assert np.abs(z[:, 0] - X @ A[:, j]).max() < 1e-12 and np.abs(z[:, 1:]).max() == 0
+        assert xa[j].level == 6                    # 9 -> mask 8 -> product 7 -> mask 6
+    out = R.lora_rank2_up(sim, xa, sim.encrypt(wb.reshape(-1)), m, n, w, 6)
+    want = X @ A @ B
+    for i in range(m):
+        assert np.abs(out[i].z.real.reshape(n, w) - want[:, 2 * n * i:2 * n * (i + 1)]).max() < 1e-12
+        assert out[i].level == 4
