@@ -317,15 +317,14 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
 
 // Validates a list of rotation terms, merges consecutive masked terms of a group that use the same key and
 // Galois element into one two-source term (the kernels then stream that key once for both), and uploads
-// the device descriptors.  *phases = 2 when the first and the second half of the outputs gather from
-// disjoint sets of sources (column shifts of one operand, then row shifts of the other).
+// the device descriptors.
 struct RotDev {
     const u64 *ext, *b, *evk, *mask;
     u32 galois, pad;
     const u64 *ext2, *b2, *mask2;
 };
 static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
-                             uint32_t n_out, hipStream_t stream, void **terms_dev, void **off_dev, int *phases) {
+                             uint32_t n_out, hipStream_t stream, void **terms_dev, void **off_dev) {
     const uint32_t n_terms = group_offsets[n_out];
     std::vector<RotDev> d;
     std::vector<uint32_t> off{0};
@@ -350,19 +349,6 @@ static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, cons
     }
     *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t), off_dev,
                              stream);
-    *phases = 1;
-    if (n_out % 2 == 0 && n_out >= 2) {
-        std::vector<const u64 *> first;
-        bool disjoint = true;
-        for (uint32_t t = 0; t < off[n_out / 2]; t++) first.push_back(d[t].ext);
-        for (uint32_t t = off[n_out / 2]; t < off[n_out] && disjoint; t++)
-            for (const u64 *p : first)
-                if (p == d[t].ext || p == d[t].ext2) {
-                    disjoint = false;
-                    break;
-                }
-        if (disjoint) *phases = 2;
-    }
 }
 
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
@@ -373,10 +359,9 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     need(terms && group_offsets && y && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
     void *terms_dev = nullptr, *off_dev = nullptr;
-    int phases = 1;
-    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev, &phases);
+    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev);
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
-                         phases, (hipStream_t)stream);
+                         (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }
@@ -390,10 +375,9 @@ int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const ui
     need(terms && group_offsets && y_workspace && out && workspace && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
     void *terms_dev = nullptr, *off_dev = nullptr;
-    int phases = 1;
-    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev, &phases);
+    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev);
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y_workspace,
-                         b_premultiplied != 0, phases, (hipStream_t)stream);
+                         b_premultiplied != 0, (hipStream_t)stream);
     launch_moddown_batch(ctx, (u64 *)y_workspace, (int)nq, (int)(2 * n_out), drop_last != 0, (u64 *)out, out_stride,
                          (u64 *)workspace, (hipStream_t)stream);
     check_launch();

@@ -166,20 +166,46 @@ u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
-__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
-                                                            int n_full, int logN, int b_premultiplied, int phases) {
-    // blockIdx.x = output (fastest): workgroups that gather from the same source tile run back to back.
+                                                            int n_full, int logN, int b_premultiplied, int n_out) {
     // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
     // (possibly swapped), so every access is a 16-byte load or store.
-    // The outputs are walked in `phases` equal runs per limb (blockIdx.z = limb * phases + run): when the
-    // runs gather from different sources, only one run's sources (1.5 MiB per source and limb) compete
-    // for an XCD's 4 MiB L2 at a time.
-    const int j = blockIdx.z / phases, o = blockIdx.x + (blockIdx.z % phases) * gridDim.x;
+    // Work is dealt out by SOURCE chunk.  The automorphism maps aligned 512-coefficient chunks onto aligned
+    // chunks, so output chunk c of output o gathers from exactly one source chunk s = pi_o(c).  Workgroups go
+    // round-robin over the 8 XCDs (each with its own L2); XCD x takes the source chunks s = x (mod 8), and for
+    // one (limb, s) all outputs run back to back.  Every XCD then only ever reads its own eighth of the
+    // rotation sources and fetches it once, instead of each L2 pulling in all of them.
+    const int cbits = logN - 9;
+    const u32 chunks = 1u << cbits;
+    u32 o, j, chunk;
+    if (chunks >= 8) {
+        const u32 xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per = chunks >> 3;
+        o = slot % (u32)n_out;
+        const u32 rest = slot / (u32)n_out;
+        const u32 s = (rest % per) * 8u + xcd;
+        j = rest / per;
+        // output chunk whose gather lands in source chunk s: the low cbits+1 bits of the exponent 2 br(i) + 1
+        // are fixed by the chunk; multiply them by g^-1 (mod 2^(cbits+1))
+        u32 g = terms[group_off[o]].galois;
+        if (g == 0) g = 1;
+        u32 ginv = g;                      // g * g = 1 (mod 8); two Newton steps give 12 bits
+        ginv *= 2u - g * ginv;
+        ginv *= 2u - g * ginv;
+        const u32 msk = (2u << cbits) - 1u;
+        const u32 es = 2u * (__brev(s) >> (32 - cbits)) + 1u;
+        const u32 eo = (es * ginv) & msk;
+        chunk = __brev(eo >> 1) >> (32 - cbits);
+    } else {
+        o = blockIdx.x % (u32)n_out;
+        const u32 rest = blockIdx.x / (u32)n_out;
+        chunk = rest % chunks;
+        j = rest / chunks;
+    }
     const int prime = ll.idx[j];
-    const u32 n = (blockIdx.y * 256 + threadIdx.x) * 2;
+    const u32 n = (chunk * 256 + threadIdx.x) * 2;
     const double fq = fp[4 * prime];
     const size_t N = (size_t)1 << logN;
     u64 rb[2], ra[2];
@@ -685,14 +711,14 @@ static CstList p_mod_chain(const hemm_context *c, int nq) {
 }
 
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, int phases, hipStream_t s) {
-    if (phases < 1 || n_out % phases != 0) phases = 1;
+                          bool b_premultiplied, hipStream_t s) {
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     const CstList pm = p_mod_chain(c, nq);
-    dim3 grid(n_out / phases, c->N / 512, E * phases), block(256);
+    if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
+    dim3 grid((unsigned)((size_t)n_out * E * (c->N / 512))), block(256);
     hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
-                       b_premultiplied ? 1 : 0, phases);
+                       b_premultiplied ? 1 : 0, n_out);
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;
