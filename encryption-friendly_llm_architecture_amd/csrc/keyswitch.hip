@@ -166,7 +166,7 @@ u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
+__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
                                                             const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
@@ -467,24 +467,34 @@ static void build_tables(const hemm_context *c, KsTables &t) {
 // tables live beside the context (created on first use, destroyed with it)
 #include <map>
 #include <mutex>
-static std::map<const hemm_context *, KsTables *> g_tabs;
-static std::mutex g_tabs_mu;
+// The registry is never destroyed: contexts can be released from static destructors of other translation
+// units (a cached mask holding the last reference), which may run after this file's statics would be gone.
+struct KsRegistry {
+    std::map<const hemm_context *, KsTables *> tabs;
+    std::mutex mu;
+};
+static KsRegistry &ks_registry() {
+    static KsRegistry *r = new KsRegistry();
+    return *r;
+}
 static KsTables *g_tables_of(const hemm_context *c) {
-    std::lock_guard<std::mutex> lk(g_tabs_mu);
-    auto it = g_tabs.find(c);
-    if (it != g_tabs.end()) return it->second;
+    KsRegistry &r = ks_registry();
+    std::lock_guard<std::mutex> lk(r.mu);
+    auto it = r.tabs.find(c);
+    if (it != r.tabs.end()) return it->second;
     KsTables *t = new KsTables();
     build_tables(c, *t);
-    g_tabs[c] = t;
+    r.tabs[c] = t;
     return t;
 }
 void hemm_keyswitch_tables_free(const hemm_context *c) {
-    std::lock_guard<std::mutex> lk(g_tabs_mu);
-    auto it = g_tabs.find(c);
-    if (it == g_tabs.end()) return;
+    KsRegistry &r = ks_registry();
+    std::lock_guard<std::mutex> lk(r.mu);
+    auto it = r.tabs.find(c);
+    if (it == r.tabs.end()) return;
     (void)hipFree(it->second->dev);
     delete it->second;
-    g_tabs.erase(it);
+    r.tabs.erase(it);
 }
 
 // scratch (u64 words) needed by key switching / rescale at full width
