@@ -420,7 +420,6 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     eval.levelDown(a.get(), T + 3, a.get());
     eval.levelDown(b.get(), T + 3, b.get());
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
-    std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);
     // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
     DeviceBuffer ab(c, 2 * ctw);
@@ -436,11 +435,9 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     // the k = 0 term sigma(A) (x) tau(B) joins the accumulator at the shifts' level T+1
     Ciphertext acc(c);
     acc.allocate(3, T + 1, 1);
-    {
-        DeviceBuffer low(c, 2 * 2 * lo * N);
-        levelDownOneBatch(c, ab.data(), 4, T + 2, low.data());
-        ck(hemm_tensor_batch(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
-    }
+    DeviceBuffer low(c, 2 * 2 * lo * N);   // sigma(A), tau(B) at level T+1
+    levelDownOneBatch(c, ab.data(), 4, T + 2, low.data());
+    ck(hemm_tensor_batch(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
     CtxtTensor res(c, rows, cols, w);
     auto finish = [&]() {
         eval.relinearize(acc, res.get());
@@ -452,6 +449,43 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     }
 
     const i64 n = k;
+    size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
+    if ((u64)(n * w) == c->N / 2) {
+        // the two operands go through separate launch chains here, so each chain takes twice as many shifts
+        G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)(n - 1)));
+        // The tile block fills the slot vector: a row shift of tau(B) is an exact rotation, so it needs no masks
+        // and no level.  The shifts of B start from tau(B) already lowered to T+1 (one limb fewer in every
+        // key-switch) and take a plain ModDown; only the column shifts of sigma(A) are masked.
+        std::vector<Shift> sa;
+        for (i64 i = 1; i < n; i++) sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
+        const Sources xa = extendSources(c, ab.data(), 1, nq);
+        const i64 back = -n;
+        const DeviceBuffer a2 = rotateSources(eval, xa, ab.data(), 1, &back);
+        const Sources xa2 = extendSources(c, a2.data(), 1, nq);
+        const Sources xb = extendSources(c, low.data() + 2 * lo * N, 1, lo);
+        const KeyPack &pack = eval.getKeyPack();
+        const Rot rot(c);
+        DeviceBuffer ya(c, G * 2 * E * N), yb(c, G * 2 * (lo + c->nP) * N), t1(c, G * 2 * lo * N), t2(c, G * 2 * lo * N),
+            ws(c, G * 2 * lo * N);
+        for (size_t first = 0; first < sa.size(); first += G) {
+            const size_t cnt = std::min(G, sa.size() - first);
+            std::vector<hemm_rot_term> terms;
+            std::vector<uint32_t> off{0};
+            pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
+            terms.clear();
+            off.assign(1, 0);
+            for (size_t q = first; q < first + cnt; q++) {
+                terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois((i64)(q + 1) * w), nullptr));
+                off.push_back((uint32_t)terms.size());
+            }
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)lo, 1, 0, yb.data(), t2.data(), lo * N, ws.data(), nullptr));
+            ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(), 1, nullptr));
+        }
+        finish();
+        return res;
+    }
+    std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);
     std::vector<Shift> sa, sb;
     for (i64 i = 1; i < n; i++) {
         sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
@@ -462,7 +496,6 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     const i64 back[2] = {-n, -n * w};
     const DeviceBuffer ab2 = rotateSources(eval, x, ab.data(), 2, back);
     const Sources x2 = extendSources(c, ab2.data(), 2, nq);
-    const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     DeviceBuffer y(c, 2 * G * 2 * E * N), t(c, 2 * G * 2 * lo * N), ws(c, 2 * G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {
         // cnt column shifts of sigma(A), then cnt row shifts of tau(B): one launch chain for all 2 cnt outputs
@@ -530,7 +563,8 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     const Sources xb = extendSources(c, b.get().buf_.data(), 1, nqb);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    const size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
+    // the two operands go through separate launch chains, so each chain takes twice as many shifts
+    const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)sa.size()));
     DeviceBuffer ya(c, G * 2 * (nqa + K) * N), yb(c, G * 2 * (nqb + K) * N), t1(c, G * 2 * lo * N), t2(c, G * 2 * lo * N),
         ws(c, G * 2 * lo * N);
     for (size_t first = 0; first < sa.size(); first += G) {

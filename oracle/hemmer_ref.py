@@ -615,18 +615,28 @@ def _assemble_shifts(orc, src, ext, back, shifts):
 
 
 def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
+    from .oracle import Ct
     ev = OracleEval(orc)
     a = orc.level_down(a, T + 3)
     b = orc.level_down(b, T + 3)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
-    rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
     a = diagonal_transform_fused(orc, a, H, n, w)
     b = diagonal_transform_fused(orc, b, V, n, w)
     # the k = 0 term joins the accumulator at the shifts' level
-    acc = orc.tensor(orc.level_down_one(a), orc.level_down_one(b))
-    ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
+    b_low = orc.level_down_one(b)
+    acc = orc.tensor(orc.level_down_one(a), b_low)
+    ext_a = orc.modup(a.data[1])
     ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
-    tb = _assemble_shifts(orc, b, ext_b, -n * w, [(i * w, rm[2 * i + 1], rm[2 * i]) for i in range(1, n)])
+    if n * w == orc.slots:
+        # the tile block fills the slot vector: row shifts are exact rotations of tau(B) lowered to T+1
+        # (one hoisted term each, no mask, plain ModDown)
+        ext_b = orc.modup(b_low.data[1])
+        tb = [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (i * w) % orc.slots, None)], b_low.nq),
+                                  b_low.nq, False), b_low.scale) for i in range(1, n)]
+    else:
+        rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
+        ext_b = orc.modup(b.data[1])
+        tb = _assemble_shifts(orc, b, ext_b, -n * w, [(i * w, rm[2 * i + 1], rm[2 * i]) for i in range(1, n)])
     for x, y in zip(ta, tb):
         acc = orc.add(acc, orc.tensor(x, y))
     return orc.rescale(orc.relinearize(acc))
