@@ -155,8 +155,8 @@ def gpu_ntt(args, out):
 # HBM bytes per launch of hoisted_terms_kernel at the shape below, from two rocprofv3 --pmc runs of
 # `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # 1 GiB copy this mode also launches (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0):
-# (2 x 778 345.5 + 360 448) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
-HOISTED_TRAFFIC_BYTES = 1963150336
+# (2 x 570 495.7 + 360 448) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
+HOISTED_TRAFFIC_BYTES = 1537473946
 
 
 def gpu_hoisted(args, out):
