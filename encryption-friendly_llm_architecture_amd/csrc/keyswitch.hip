@@ -232,18 +232,19 @@ struct LinTermDev {
     u64 stride;       // polynomial stride of ct
     u64 galois;       // 0: mask used as is; else the mask is read through the automorphism X -> X^galois
 };
-// out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j], p < n_polys (<= 3).  A thread owns one
-// (limb, coefficient) for every polynomial, so each mask residue is read once; products are summed as
-// 128-bit values and reduced every 4 terms.
+// out[o][p][j] = sum_{t in group o} mask_t[j] * ct_t[p][j], p < n_polys (<= 3).  A thread owns the residue pair
+// (n, n+1) of one limb for every polynomial (16-byte accesses; under an automorphism an aligned pair stays an
+// aligned pair, possibly swapped), so each mask residue is read once; integer products are summed as 128-bit
+// values and reduced every 4 terms.
 template <int n_polys>
 __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
                                                          const u32 *__restrict__ group_off, u64 *__restrict__ out,
                                                          const ModQ *__restrict__ modq, const double *__restrict__ fp, int nq, int logN,
                                                          int n_out) {
     // Workgroups go round-robin over the 8 XCDs, each with its own L2.  The outputs of one launch mostly
-    // sum the same ciphertexts under different masks, so all outputs of a (limb, 256-coefficient) tile are
+    // sum the same ciphertexts under different masks, so all outputs of a (limb, 512-coefficient) tile are
     // placed back to back on one XCD: the ciphertext tile is fetched from HBM once instead of once per output.
-    const u32 tiles = (u32)nq << (logN - 8);
+    const u32 tiles = (u32)nq << (logN - 9);
     u32 o, tile;
     if ((tiles & 7u) == 0) {
         const u32 xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
@@ -253,82 +254,108 @@ __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__res
         o = blockIdx.x % (u32)n_out;
         tile = blockIdx.x / (u32)n_out;
     }
-    const int j = (int)(tile >> (logN - 8));
+    const int j = (int)(tile >> (logN - 9));
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN;
-    const size_t e = (size_t)j * N + (size_t)(tile & ((1u << (logN - 8)) - 1)) * 256 + threadIdx.x;
+    const u32 n = ((tile & ((1u << (logN - 9)) - 1)) * 256 + threadIdx.x) * 2;
+    const size_t e = (size_t)j * N + n;
     const double fq = fp[4 * j];
+    // mask residues of the pair (n, n+1), read through the term's automorphism if it has one
+    auto load_mask = [&](const LinTermDev &T) -> ulonglong2 {
+        if (T.galois == 0) return stream_load2(T.mask + e);
+        const u32 np = galois_index(n, (u32)T.galois, logN);
+        ulonglong2 v = *(const ulonglong2 *)(T.mask + (size_t)j * N + (np & ~1u));
+        if (np & 1u) {
+            const u64 tmp = v.x;
+            v.x = v.y;
+            v.y = tmp;
+        }
+        return v;
+    };
     if (fq != 0.0) {
         // primes below 2^44: exact double-precision products (6 FP64 operations each)
         const FpMod f{fq, fp[4 * j + 1]};
-        double facc[n_polys];
+        double facc[n_polys][2];
 #pragma unroll
-        for (int p = 0; p < n_polys; p++) facc[p] = 0.0;
+        for (int p = 0; p < n_polys; p++) facc[p][0] = facc[p][1] = 0.0;
         int since = 0;
         for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
             const LinTermDev T = terms[t];
             if (T.mask != nullptr) {
-                const u64 mk = T.galois ? T.mask[(size_t)j * N + galois_index((u32)(e - (size_t)j * N), (u32)T.galois, logN)]
-                                        : T.mask[e];
-                const double dm = __longlong_as_double((long long)(mk | 0x4330000000000000ull)) - 4503599627370496.0;
+                const ulonglong2 mk = load_mask(T);
+                const double dm0 = u64_to_double(mk.x), dm1 = u64_to_double(mk.y);
 #pragma unroll
                 for (int p = 0; p < n_polys; p++) {
-                    const u64 cv = T.ct[p * T.stride + e];
-                    facc[p] += f.mul(__longlong_as_double((long long)(cv | 0x4330000000000000ull)) - 4503599627370496.0, dm);
+                    const ulonglong2 cv = *(const ulonglong2 *)(T.ct + p * T.stride + e);
+                    facc[p][0] += f.mul(u64_to_double(cv.x), dm0);
+                    facc[p][1] += f.mul(u64_to_double(cv.y), dm1);
                 }
             } else {
 #pragma unroll
                 for (int p = 0; p < n_polys; p++) {
-                    const u64 cv = T.ct[p * T.stride + e];
-                    facc[p] += __longlong_as_double((long long)(cv | 0x4330000000000000ull)) - 4503599627370496.0;
+                    const ulonglong2 cv = *(const ulonglong2 *)(T.ct + p * T.stride + e);
+                    facc[p][0] += u64_to_double(cv.x);
+                    facc[p][1] += u64_to_double(cv.y);
                 }
             }
             if (++since == 64) {  // a term adds at most q: keep the running sums far below 2^52
 #pragma unroll
-                for (int p = 0; p < n_polys; p++) facc[p] = f.reduce(facc[p]);
+                for (int p = 0; p < n_polys; p++) {
+                    facc[p][0] = f.reduce(facc[p][0]);
+                    facc[p][1] = f.reduce(facc[p][1]);
+                }
                 since = 0;
             }
         }
 #pragma unroll
-        for (int p = 0; p < n_polys; p++) out[((size_t)o * n_polys + p) * nq * N + e] = f.canonical(facc[p]);
+        for (int p = 0; p < n_polys; p++)
+            stream_store2(out + ((size_t)o * n_polys + p) * nq * N + e, f.canonical(facc[p][0]), f.canonical(facc[p][1]));
         return;
     }
-    u64 acc[n_polys];
-    u128_t lazy[n_polys];
+    u64 acc[n_polys][2];
+    u128_t lazy[n_polys][2];
 #pragma unroll
-    for (int p = 0; p < n_polys; p++) {
-        acc[p] = 0;
-        lazy[p].lo = lazy[p].hi = 0;
-    }
+    for (int p = 0; p < n_polys; p++)
+        for (int h = 0; h < 2; h++) {
+            acc[p][h] = 0;
+            lazy[p][h].lo = lazy[p][h].hi = 0;
+        }
     int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const LinTermDev T = terms[t];
         if (T.mask != nullptr) {
-            const u64 mk = T.galois ? T.mask[(size_t)j * N + galois_index((u32)(e - (size_t)j * N), (u32)T.galois, logN)]
-                                    : T.mask[e];
-            
-#pragma unroll
-            for (int p = 0; p < n_polys; p++) add128(lazy[p], mul64wide(T.ct[p * T.stride + e], mk));
-            if (++pending == 4) {
-                
+            const ulonglong2 mk = load_mask(T);
 #pragma unroll
             for (int p = 0; p < n_polys; p++) {
-                    acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
-                    lazy[p].lo = lazy[p].hi = 0;
-                }
+                const ulonglong2 cv = *(const ulonglong2 *)(T.ct + p * T.stride + e);
+                add128(lazy[p][0], mul64wide(cv.x, mk.x));
+                add128(lazy[p][1], mul64wide(cv.y, mk.y));
+            }
+            if (++pending == 4) {
+#pragma unroll
+                for (int p = 0; p < n_polys; p++)
+                    for (int h = 0; h < 2; h++) {
+                        acc[p][h] = addmod(acc[p][h], barrett128(lazy[p][h], m), m.q);
+                        lazy[p][h].lo = lazy[p][h].hi = 0;
+                    }
                 pending = 0;
             }
         } else {
-            
-#pragma unroll
-            for (int p = 0; p < n_polys; p++) acc[p] = addmod(acc[p], T.ct[p * T.stride + e], m.q);
-        }
-    }
-    
 #pragma unroll
             for (int p = 0; p < n_polys; p++) {
-        if (pending) acc[p] = addmod(acc[p], barrett128(lazy[p], m), m.q);
-        out[((size_t)o * n_polys + p) * nq * N + e] = acc[p];
+                const ulonglong2 cv = *(const ulonglong2 *)(T.ct + p * T.stride + e);
+                acc[p][0] = addmod(acc[p][0], cv.x, m.q);
+                acc[p][1] = addmod(acc[p][1], cv.y, m.q);
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < n_polys; p++) {
+        if (pending) {
+            acc[p][0] = addmod(acc[p][0], barrett128(lazy[p][0], m), m.q);
+            acc[p][1] = addmod(acc[p][1], barrett128(lazy[p][1], m), m.q);
+        }
+        stream_store2(out + ((size_t)o * n_polys + p) * nq * N + e, acc[p][0], acc[p][1]);
     }
 }
 
@@ -791,7 +818,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s) {
     if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
-    dim3 grid((unsigned)(c->N / 256) * nq * n_out), block(256);
+    if (c->N < 512) throw std::invalid_argument("masked sums need N >= 512");
+    dim3 grid((unsigned)(c->N / 512) * nq * n_out), block(256);
     const LinTermDev *td = (const LinTermDev *)terms_dev;
     if (n_polys == 1)
         hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
