@@ -417,8 +417,6 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     if (min_level < T + 3)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
     // the transforms run at level T+3: lowering first gives the same values with 8 instead of 13 limbs
-    eval.levelDown(a.get(), T + 3, a.get());
-    eval.levelDown(b.get(), T + 3, b.get());
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
     // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
@@ -426,8 +424,24 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     {
         const u64 ctw_in = 2 * (nq + 1) * N;
         DeviceBuffer joint(c, 2 * ctw_in);
-        (void)hipMemcpyAsync(joint.data(), a.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
-        (void)hipMemcpyAsync(joint.data() + ctw_in, b.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        const u64 la = a.getLevel(), lb = b.getLevel();
+        if (la == lb && la > T + 3 && a.get().getRescaleCounter() == 0 && b.get().getRescaleCounter() == 0) {
+            // HomEvaluator::levelDown of both operands at once: multiply by round(Delta_{T+3} q_{T+4} / Delta_level)
+            // over T+5 limbs, then one rescale of the four polynomials straight into the joint buffer
+            const u64 nl = T + 5;
+            const i64 v = (i64)llround(c->delta[T + 3] * (Real)c->q[T + 4] / c->delta[la]);
+            std::vector<u64> sc(nl);
+            for (u64 j = 0; j < nl; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
+            DeviceBuffer t(c, 4 * nl * N);
+            ck(hemm_mul_scalar(c->dev, a.get().buf_.data(), a.get().polyStride(), sc.data(), t.data(), nl * N, (uint32_t)nl, 0, 2, nullptr));
+            ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
+            ck(hemm_rescale(c->dev, t.data(), nl * N, joint.data(), (nl - 1) * N, (uint32_t)nl, 4, nullptr));
+        } else {
+            eval.levelDown(a.get(), T + 3, a.get());
+            eval.levelDown(b.get(), T + 3, b.get());
+            (void)hipMemcpyAsync(joint.data(), a.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(joint.data() + ctw_in, b.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        }
         const MaskKind kinds[2] = {MaskKind::Horizontal, MaskKind::Vertical};
         const TileTensorShape shapes[2] = {a.getShape(), b.getShape()};
         tr.diagonalTransformBatch(eval, joint.data(), 2, T + 3, kinds, shapes, ab.data());
