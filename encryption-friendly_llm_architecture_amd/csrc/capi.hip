@@ -332,11 +332,11 @@ static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, cons
     for (uint32_t o = 0; o < n_out; o++) {
         need(group_offsets[o + 1] >= group_offsets[o], "group offsets must not decrease");
         for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
-            need(terms[t].ext && terms[t].b && terms[t].evk, "null pointer in a rotation term");
+            need(terms[t].ext && terms[t].evk, "null pointer in a rotation term");
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
             RotDev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
                        (const u64 *)terms[t].mask, (u32)terms[t].galois, 0, nullptr, nullptr, nullptr};
-            if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t + 1].ext && terms[t + 1].b &&
+            if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
                 terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois) {
                 cur.ext2 = (const u64 *)terms[t + 1].ext;
                 cur.b2 = (const u64 *)terms[t + 1].b;

@@ -17,7 +17,7 @@ __device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
 
 struct RotTermDev {
     const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
-    const u64 *b;     // [nq][N] b-polynomial of the source
+    const u64 *b;     // [nq][N] b-polynomial of the source (nullptr: none, single-source terms only)
     const u64 *evk;   // [dnum][2][nQ+K][N]
     const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
     u32 galois, pad;
@@ -153,7 +153,7 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         }
         u64 rb[2] = {barrett128(sb[0], m), barrett128(sb[1], m)};
         u64 ra[2] = {barrett128(sa[0], m), barrett128(sa[1], m)};
-        if (j < nq) {
+        if (j < nq && T.b != nullptr) {
             ulonglong2 bv = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
             if (swap) {
                 const u64 tmp = bv.x;
@@ -273,7 +273,7 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 sa0 += f.mul(x.x, ka.x);
                 sa1 += f.mul(x.y, ka.y);
             }
-            if (j < nq) {
+            if (j < nq && T.b != nullptr) {
                 D2 bv = gather_d2(T.b + (size_t)j * N + base, swap);
                 if (!b_premultiplied) {
                     bv.x = f.mul(bv.x, p_mod_q);

@@ -189,11 +189,14 @@ public:
     bool hasGaloisKey(u64 galois) const { return galois_.count(galois) != 0; }
     const u64 *multKey() const;
     const u64 *galoisKey(u64 galois) const;
+    // key switching rho_g(s)^2 -> s: rotates the degree-2 component of an un-relinearised product directly
+    bool hasGaloisSquareKey(u64 galois) const { return galois_sq_.count(galois) != 0; }
+    const u64 *galoisSquareKey(u64 galois) const;
     const Context &getContext() const { return ctx_; }
     // internal
     Context ctx_;
     DeviceBuffer mult_;
-    std::map<u64, DeviceBuffer> galois_;
+    std::map<u64, DeviceBuffer> galois_, galois_sq_;
 };
 
 class KeyGenerator {
@@ -204,6 +207,7 @@ public:
     void genConjKey() const;
     void genLeftRotKey(u64 rot) const;
     void genRightRotKey(u64 rot) const;
+    void genLeftRotSquareKey(u64 rot) const;   // KeyPack::galoisSquareKey of a left rotation (not in HEaaN)
     void genRotKeyBundle() const;   // every power-of-two left and right rotation
     void genCommonKeys() const;     // mult + conj + power-of-two rotations
     void genRotKeysForBootstrap(u64) const {}  // bootstrapping is outside this build

@@ -394,6 +394,11 @@ const u64 *KeyPack::galoisKey(u64 g) const {
     if (it == galois_.end()) throw RuntimeException("no key for Galois element " + std::to_string(g));
     return it->second.data();
 }
+const u64 *KeyPack::galoisSquareKey(u64 g) const {
+    auto it = galois_sq_.find(g);
+    if (it == galois_sq_.end()) throw RuntimeException("no square key for Galois element " + std::to_string(g));
+    return it->second.data();
+}
 void KeyPack::save(const std::string &dir) const {
     const size_t words = ctx_->dnum * 2 * (ctx_->nQ + ctx_->nP) * ctx_->N;
     std::vector<u64> h(words);
@@ -412,6 +417,10 @@ void KeyPack::save(const std::string &dir) const {
         dump("GaloisKey_" + std::to_string(kv.first) + ".bin", kv.second);
         idx << kv.first << "\n";
     }
+    for (auto &kv : galois_sq_) {
+        dump("GaloisSquareKey_" + std::to_string(kv.first) + ".bin", kv.second);
+        idx << "sq" << kv.first << "\n";
+    }
 }
 KeyPack::KeyPack(const Context &c, const std::string &dir) : ctx_(c) {
     const size_t words = c->dnum * 2 * (c->nQ + c->nP) * c->N;
@@ -429,7 +438,10 @@ KeyPack::KeyPack(const Context &c, const std::string &dir) : ctx_(c) {
     while (std::getline(idx, line)) {
         if (line == "mult")
             slurp("MultKey.bin", mult_);
-        else if (!line.empty()) {
+        else if (line.rfind("sq", 0) == 0) {
+            u64 g = std::stoull(line.substr(2));
+            slurp("GaloisSquareKey_" + line.substr(2) + ".bin", galois_sq_[g]);
+        } else if (!line.empty()) {
             u64 g = std::stoull(line);
             slurp("GaloisKey_" + line + ".bin", galois_[g]);
         }
@@ -496,6 +508,18 @@ void KeyGenerator::genLeftRotKey(u64 rot) const {
     DeviceBuffer sg;
     gen_galois(*this, ctx_, sk_, g, sg);
     genSwitchKey(g, sg.data(), pack_.galois_[g]);
+}
+// key id of a square key: the Galois element with bit 40 set (Galois elements are below 2N <= 2^18)
+void KeyGenerator::genLeftRotSquareKey(u64 rot) const {
+    const u64 slots = ctx_->N / 2;
+    rot %= slots;
+    const u64 g = rot == 0 ? 1 : galois_of_rotation(ctx_, rot);
+    if (pack_.hasGaloisSquareKey(g)) return;
+    const size_t T = ctx_->nQ + ctx_->nP;
+    DeviceBuffer s2(ctx_, T * ctx_->N), sg(ctx_, T * ctx_->N);
+    ck(hemm_pointwise(ctx_->dev, HEMM_MUL, sk_.ntt(), 0, sk_.ntt(), 0, s2.data(), 0, (uint32_t)ctx_->nQ, 1, 1, nullptr));
+    ck(hemm_automorphism(ctx_->dev, s2.data(), 0, sg.data(), 0, g, (uint32_t)T, 1, nullptr));
+    genSwitchKey((u64(1) << 40) | g, sg.data(), pack_.galois_sq_[g]);
 }
 void KeyGenerator::genRightRotKey(u64 rot) const {
     const u64 slots = ctx_->N / 2;

@@ -411,7 +411,10 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
     if (fused_) {
-        ensureRotationKeys(fusedRotations(TileTensorShape(n, n, w), log_slots_, false, true));
+        std::vector<u64> square_rots;
+        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots));
+        KeyGenerator keygen(context_, sk_, pack_);
+        for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
         return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
     }
     ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});

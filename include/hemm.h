@@ -124,7 +124,8 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
  * inner product with evk, optional plaintext mask over the extended basis (NULL = 1). */
 typedef struct {
     const uint64_t *ext;  /* [beta][nq+n_p][N] */
-    const uint64_t *b;    /* [nq][N] */
+    const uint64_t *b;    /* [nq][N], or NULL: the term contributes only the key product (used for the
+                           * degree-2 component of a tensor product, with a key for the rotated s^2) */
     const uint64_t *evk;  /* [dnum][2][n_q+n_p][N] */
     const uint64_t *mask; /* [nq+n_p][N] or NULL */
     uint64_t galois;

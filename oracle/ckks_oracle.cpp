@@ -560,7 +560,7 @@ void orc_hoisted_term(void *h, const u64 *ext, const u64 *b, const u64 *evk, con
                 for (int d = 0; d < beta; d++)
                     s = addmod(s, mulmod(ext[((size_t)d * E + j) * N + perm[n]],
                                          evk[(((size_t)d * 2 + pol) * full + pi) * N + n], q), q);
-                if (pol == 0 && j < nq) s = addmod(s, mulmod(b[(size_t)j * N + perm[n]], P, q), q);
+                if (pol == 0 && j < nq && b) s = addmod(s, mulmod(b[(size_t)j * N + perm[n]], P, q), q);
                 if (mask) s = mulmod(s, mask[(size_t)j * N + n], q);
                 o[n] = accumulate ? addmod(o[n], s, q) : s;
             }

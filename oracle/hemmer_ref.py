@@ -589,6 +589,14 @@ def diagonal_transform_fused(orc, ct, kind, n, w):
     return orc.rescale(res)
 
 
+def bsgs_baby_count(n):
+    """Largest power of two g with g * g <= 2 n."""
+    g = 1
+    while 4 * g * g <= 2 * n:
+        g <<= 1
+    return g
+
+
 def _rotated_copy(orc, src, ext, r):
     """rot(src, r) with the automorphism after ModUp (one hoisted term, plain ModDown)."""
     from .oracle import Ct
@@ -626,14 +634,38 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
     b_low = orc.level_down_one(b)
     acc = orc.tensor(orc.level_down_one(a), b_low)
     ext_a = orc.modup(a.data[1])
-    ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
     if n * w == orc.slots:
-        # the tile block fills the slot vector: row shifts are exact rotations of tau(B) lowered to T+1
-        # (one hoisted term each, no mask, plain ModDown)
+        # The tile block fills the slot vector: row shifts are exact rotations rho^(k w) of tau(B) lowered to
+        # T+1 (no mask, plain ModDown), which allows the baby-step / giant-step split k = k1 + g k2:
+        #   C = sum_k2 rho^(g k2 w)(U_k2),  U_k2 = sum_k1 rho^(-g k2 w)(phi^k(sigma A)) (x) rho^(k1 w)(tau B).
+        # The column shifts come out already rotated back by g k2 rows (another Galois element, same masks);
+        # the un-relinearised U_k2 are rotated directly: d1 with the key of rho(s), d2 with a key of
+        # rho(s)^2, all summed in the extended basis before one ModDown merged with the rescale.
+        g = bsgs_baby_count(n)
         ext_b = orc.modup(b_low.data[1])
-        tb = [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (i * w) % orc.slots, None)], b_low.nq),
-                                  b_low.nq, False), b_low.scale) for i in range(1, n)]
+        bb = [b_low] + [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (k1 * w) % orc.slots, None)],
+                                                            b_low.nq), b_low.nq, False), b_low.scale)
+                        for k1 in range(1, g)]
+        ta = _assemble_shifts(orc, a, ext_a, -n,
+                              [((k - g * (k // g) * w) % orc.slots, cm[2 * k + 1], cm[2 * k]) for k in range(1, n)])
+        U = [acc] + [None] * (n // g - 1)
+        for k in range(1, n):
+            t = orc.tensor(ta[k - 1], bb[k % g])
+            U[k // g] = t if U[k // g] is None else orc.add(U[k // g], t)
+        res = orc.rescale(orc.relinearize(U[0]))
+        if n // g > 1:
+            lo = b_low.nq
+            terms = []
+            for k2 in range(1, n // g):
+                gal = orc.galois((k2 * g * w) % orc.slots)
+                u = U[k2]
+                terms.append((orc.modup(u.data[1]), u.data[0], ("g", gal), None))
+                terms.append((orc.modup(u.data[2]), None, ("sq", gal), None))
+            y = orc.hoisted_sum(terms, lo)
+            res = orc.add(res, Ct(orc.moddown_drop(y, lo, True), res.scale))
+        return res
     else:
+        ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
         rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
         ext_b = orc.modup(b.data[1])
         tb = _assemble_shifts(orc, b, ext_b, -n * w, [(i * w, rm[2 * i + 1], rm[2 * i]) for i in range(1, n)])

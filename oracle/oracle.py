@@ -330,6 +330,20 @@ class Oracle:
         if ("gal", g) not in self.keys:
             self.keys[("gal", g)] = self._gen_switch_key(seed, g, self._sk_automorphism(g))
 
+    def gen_rot_square_key(self, seed, g):
+        """Key switching rho_g(s)^2 -> s (key id = Galois element with bit 40 set): rotates the degree-2
+        component of an un-relinearised product directly."""
+        if ("galsq", g) not in self.keys:
+            tot = self.nQ + self.nP
+            s2 = np.empty_like(self.sk)
+            for i in range(tot):
+                self.L.orc_pointwise(self.h, 2, _p(self.sk[i]), _p(self.sk[i]), _p(s2[i]), i)
+            sg = np.empty_like(s2)
+            for i in range(tot):
+                self.L.orc_automorphism_ntt(self.h, _p(s2[i]), _p(sg[i]), g)
+            self.keys[("galsq", g)] = self._gen_switch_key(seed, (1 << 40) | g, sg)
+        return self.keys[("galsq", g)]
+
     def gen_conj_key(self, seed):
         g = 2 * self.N - 1
         self.keys[("gal", g)] = self._gen_switch_key(seed, g, self._sk_automorphism(g))
@@ -581,14 +595,19 @@ class Oracle:
         return self.keys[("gal", g)]
 
     def hoisted_sum(self, terms, nq):
-        """terms: (ext, b, rotation r (left, in slots) or ('g', galois), mask Pt over the extended basis
-        or None).  Returns y[2][nq+K][N] = sum mask * (<galois(ext), evk> + P galois(b))."""
+        """terms: (ext, b or None, rotation r (left, in slots) or ('g', galois) or ('sq', galois): the key of
+        rho_g(s)^2, mask Pt over the extended basis or None).
+        Returns y[2][nq+K][N] = sum mask * (<galois(ext), evk> + P galois(b))."""
         y = np.zeros((2, nq + self.nP, self.N), dtype=np.uint64)
         for i, (ext, b, rot, mask) in enumerate(terms):
             g = rot[1] if isinstance(rot, tuple) else self.galois(rot)
-            evk = self.galois_key(g)
+            if isinstance(rot, tuple) and rot[0] == "sq":
+                evk = self.gen_rot_square_key(self.key_seed, g)
+            else:
+                evk = self.galois_key(g)
             mk = _p(np.ascontiguousarray(mask.data)) if mask is not None else None
-            self.L.orc_hoisted_term(self.h, _p(np.ascontiguousarray(ext)), _p(np.ascontiguousarray(b)),
+            bp = _p(np.ascontiguousarray(b)) if b is not None else None
+            self.L.orc_hoisted_term(self.h, _p(np.ascontiguousarray(ext)), bp,
                                     _p(evk), mk, g, nq, _p(y), int(i > 0))
         return y
 
