@@ -144,6 +144,7 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
 // left rotations (in slots) whose direct keys the batched schedules use
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 // the same for multMatMatFused; square_rots receives the giant steps that also need KeyPack::galoisSquareKey
-std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots);
+std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots,
+                                    bool packed = false);
 
 }  // namespace HELLM

@@ -113,7 +113,7 @@ std::vector<u64> HEMMer::transformRotations(MaskKind kind, i64 width) const {
     const i64 cell = packed ? 2 : 1, units = n / cell, step = cell * (vertical ? width : 1);
     const i64 bs = (i64)std::ceil(std::sqrt((double)(2 * units - 1))),
               gs = (i64)std::ceil((double)(units - 1) / (double)bs);
-    left(step);
+    for (i64 j = 0; j < (fused_ ? bs : 1); j++) left((j + 1) * step);   // hoisted baby steps are direct rotations
     for (i64 i = 0; i < gs; i++) {
         left(-(units - i * bs) * step);
         if (i > 0) left(i * bs * step);
@@ -438,7 +438,10 @@ CtxtTensor HEMMer::packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T)
     ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
     if (fused_ && (u64)(n * w) == slots) {
-        ensureRotationKeys(fusedRotations(TileTensorShape(n, n, w), log_slots_, true, true));
+        std::vector<u64> square_rots;
+        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, true));
+        KeyGenerator keygen(context_, sk_, pack_);
+        for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
         return multPackedMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
     }
     ensureRotationKeys({2, (u64)(2 * w), slots - (u64)n});

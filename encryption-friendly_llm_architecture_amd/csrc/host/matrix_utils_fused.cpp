@@ -150,19 +150,20 @@ std::vector<Plaintext> &MatrixTransformer::getRowMaskExt(const HomEvaluator &eva
     return row_masks_ext_.emplace(key, std::move(v)).first->second;
 }
 
-std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots) {
+std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots,
+                                    bool packed) {
     const i64 slots = i64(1) << log_slots, n = shape.getNumRows(), w = shape.getBlockWidth();
     square_rots.clear();
-    if (n * w != slots) return fusedRotations(shape, log_slots, false, true);
+    if (n * w != slots) return fusedRotations(shape, log_slots, packed, true);
     std::vector<u64> r;
     auto left = [&](i64 v) { return (u64)(((v % slots) + slots) % slots); };
-    const i64 g = bsgsBabyCount(n);
+    const i64 cu = packed ? 2 : 1, units = n / cu, ru = cu * w, g = bsgsBabyCount(units);
     r.push_back(left(-n));
-    for (i64 k = 1; k < n; k++) r.push_back(left(k - g * (k / g) * w));
-    for (i64 k1 = 1; k1 < g; k1++) r.push_back(left(k1 * w));
-    for (i64 k2 = 1; k2 < n / g; k2++) {
-        r.push_back(left(k2 * g * w));
-        square_rots.push_back(left(k2 * g * w));
+    for (i64 i = 1; i < units; i++) r.push_back(left(cu * i - g * (i / g) * ru));
+    for (i64 i1 = 1; i1 < g; i1++) r.push_back(left(i1 * ru));
+    for (i64 i2 = 1; i2 < units / g; i2++) {
+        r.push_back(left(i2 * g * ru));
+        square_rots.push_back(left(i2 * g * ru));
     }
     return r;
 }
@@ -425,6 +426,126 @@ i64 commonBlockWidth(const HETensor<T1> &a, const HETensor<T2> &b) {
 
 }  // namespace
 
+namespace {
+// Sum over the shift index of a product whose row shifts are exact rotations (the tile block fills the slot vector),
+// split into baby and giant steps, i = i1 + g i2 over `units` shifts (column shift of i cells = cu * i slots, row
+// shift of i cells = rho^(i ru)):
+//   C = sum_i2 rho^(g i2 ru)( U_i2 ),   U_i2 = sum_i1 rho^(-g i2 ru)(phi^i(sigma A)) (x) rho^(i1 ru)(tau B)
+// * tau(B), at level T+1, is rotated only g - 1 times (one chain, plain ModDown);
+// * every column shift phi^i(sigma A) is produced already rotated back by g i2 row units: the column masks do not
+//   depend on the row, so this only changes the Galois element of shift i (still one key per shift);
+// * the un-relinearised sums U_i2 (three polynomials) are rotated by the giant steps directly: d1 under the key of
+//   rho(s), d2 under a key of rho(s)^2, all 2 (units/g - 1) terms summed in the extended basis before a single
+//   ModDown merged with the rescale.  U_0 (in `acc`, which arrives holding the i = 0 term) takes the ordinary
+//   relinearisation.
+// units + g + 2 units/g key switches instead of 2 units.
+// sigma_a: [2][T+3][N] at level T+2; tau_b: [2][T+2][N] at level T+1; U_out receives U_1 .. (each [3][T+2][N]).
+void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
+                      std::vector<Plaintext> &cm, i64 n, i64 units, i64 cu, i64 w, u64 batch, DeviceBuffer *U_out,
+                      i64 *g_out) {
+    const Context &c = eval.getContext();
+    const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
+    const i64 ru = cu * w;
+    const i64 g = bsgsBabyCount(units), n_giant = units / g;
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    const u64 ctl = 2 * lo * N;   // words of a two-polynomial ciphertext at level T+1
+    // baby rotations of tau(B): bb[i1] = rho^(i1 ru)(tau B)
+    DeviceBuffer bb(c, (u64)g * ctl);
+    (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, nullptr);
+    if (g > 1) {
+        const Sources xb = extendSources(c, tau_b, 1, lo);
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        for (i64 i1 = 1; i1 < g; i1++) {
+            terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(i1 * ru), nullptr));
+            off.push_back((uint32_t)terms.size());
+        }
+        DeviceBuffer yb(c, (u64)(g - 1) * 2 * (lo + K) * N), ws(c, (u64)(g - 1) * ctl);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)(g - 1), (uint32_t)lo, 1, 0, yb.data(),
+                                bb.data() + ctl, lo * N, ws.data(), nullptr));
+    }
+    // column shifts of sigma(A), shift i rotated back by g (i / g) row units
+    std::vector<Shift> sa;
+    for (i64 i = 1; i < units; i++)
+        sa.push_back(Shift{cu * i - g * (i / g) * ru, &cm[(size_t)(2 * cu * i + 1)], &cm[(size_t)(2 * cu * i)]});
+    const Sources xa = extendSources(c, sigma_a, 1, nq);
+    const i64 back = -n;
+    const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back);
+    const Sources xa2 = extendSources(c, a2.data(), 1, nq);
+    // U[i2 - 1]: [3][lo][N] for i2 >= 1; U_0 is `acc`
+    const u64 uw = 3 * lo * N;
+    U_out->resize(c, (u64)std::max<i64>(1, n_giant - 1) * uw);
+    std::vector<bool> started((size_t)n_giant, false);
+    started[0] = true;
+    const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
+    DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl);
+    for (size_t first = 0; first < sa.size(); first += G) {
+        const size_t cnt = std::min(G, sa.size() - first);
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
+        // shift index q holds i = q + 1: consecutive i with the same i2 pair with consecutive baby rotations
+        size_t q = first;
+        while (q < first + cnt) {
+            const i64 ii = (i64)q + 1, i2 = ii / g, i1 = ii % g;
+            const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - i1));
+            u64 *dst = i2 == 0 ? acc.buf_.data() : U_out->data() + (u64)(i2 - 1) * uw;
+            ck(hemm_tensor_batch(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
+                                 (uint32_t)lo, dst, started[(size_t)i2] ? 1 : 0, nullptr));
+            started[(size_t)i2] = true;
+            q += run;
+        }
+    }
+    *g_out = g;
+}
+
+// res = rescale(relinearize(acc)) + sum_{i2 >= 1} rho^(g i2 ru)(U_i2), the latter through one hoisted launch
+void bsgsGiantSteps(const HomEvaluator &eval, u64 T, const DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
+                    CtxtTensor &res) {
+    const Context &c = eval.getContext();
+    const u64 N = c->N, K = c->nP, lo = T + 2, uw = 3 * lo * N;
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    eval.relinearize(acc, res.get());
+    eval.rescale(res.get());
+    if (n_giant <= 1) return;
+    const u64 m = (u64)(n_giant - 1), beta = (lo + c->alpha - 1) / c->alpha, El = lo + K;
+    DeviceBuffer ext1(c, m * beta * El * N), ext2(c, m * beta * El * N), pb(c, m * lo * N), wsu(c, m * lo * N);
+    ck(hemm_modup_batch(c->dev, U.data() + lo * N, uw, (uint32_t)lo, (uint32_t)m, ext1.data(), wsu.data(), nullptr));
+    ck(hemm_modup_batch(c->dev, U.data() + 2 * lo * N, uw, (uint32_t)lo, (uint32_t)m, ext2.data(), wsu.data(), nullptr));
+    std::vector<u64> sc(lo);
+    for (u64 j = 0; j < lo; j++) {
+        u64 P = 1;
+        for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+        sc[j] = P;
+    }
+    ck(hemm_mul_scalar(c->dev, U.data(), uw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
+    std::vector<hemm_rot_term> terms;
+    for (u64 i = 0; i < m; i++) {
+        const u64 gal = rot.galois((i64)(i + 1) * g * ru);
+        hemm_rot_term t;
+        t.ext = ext1.data() + i * beta * El * N;
+        t.b = pb.data() + i * lo * N;
+        t.evk = pack.galoisKey(gal);
+        t.mask = nullptr;
+        t.galois = gal;
+        terms.push_back(t);
+        t.ext = ext2.data() + i * beta * El * N;
+        t.b = nullptr;
+        t.evk = pack.galoisSquareKey(gal);
+        terms.push_back(t);
+    }
+    const uint32_t off[2] = {0, (uint32_t)terms.size()};
+    Ciphertext giant(c);
+    giant.allocate(2, T, 0);
+    DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * (lo - 1) * N);
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off, 1, (uint32_t)lo, 1, 1, yg.data(), giant.buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
+    eval.add(res.get(), giant, res.get());
+}
+}  // namespace
+
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch) {
     const Context &c = eval.getContext();
@@ -489,105 +610,10 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     const i64 n = k;
     size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     if ((u64)(n * w) == c->N / 2) {
-        // The tile block fills the slot vector, so a row shift of tau(B) is an exact rotation rho^(k w): no masks,
-        // no level.  That allows a baby-step / giant-step split of the sum over k = k1 + g k2:
-        //   C = sum_k2 rho^(g k2 w)( U_k2 ),   U_k2 = sum_k1 rho^(-g k2 w)(phi^k(sigma A)) (x) rho^(k1 w)(tau B)
-        // * tau(B), lowered to T+1, is rotated only g - 1 times (one chain, plain ModDown);
-        // * every column shift phi^k(sigma A) is produced already rotated back by g k2 rows: the column masks do not
-        //   depend on the row, so this only changes the Galois element of shift k (still one key per shift);
-        // * the un-relinearised sums U_k2 (three polynomials) are rotated by the giant steps directly: d1 under the
-        //   key of rho(s), d2 under a key of rho(s)^2, all 2 (n/g - 1) terms summed in the extended basis before a
-        //   single ModDown merged with the rescale.  U_0 takes the ordinary relinearisation.
-        // n + g + 2 n/g key switches instead of 2 n.
-        const i64 g = bsgsBabyCount(n), n_giant = n / g;
-        const u64 slots = c->N / 2, K = c->nP;
-        const KeyPack &pack = eval.getKeyPack();
-        const Rot rot(c);
-        const u64 ctl = 2 * lo * N;   // words of a two-polynomial ciphertext at level T+1
-        // baby rotations of tau(B): bb[k1] = rho^(k1 w)(tau B) at level T+1
-        DeviceBuffer bb(c, (u64)g * ctl);
-        (void)hipMemcpyAsync(bb.data(), low.data() + ctl, ctl * 8, hipMemcpyDeviceToDevice, nullptr);
-        if (g > 1) {
-            const Sources xb = extendSources(c, low.data() + ctl, 1, lo);
-            std::vector<hemm_rot_term> terms;
-            std::vector<uint32_t> off{0};
-            for (i64 k1 = 1; k1 < g; k1++) {
-                terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(k1 * w), nullptr));
-                off.push_back((uint32_t)terms.size());
-            }
-            DeviceBuffer yb(c, (u64)(g - 1) * 2 * (lo + K) * N), ws(c, (u64)(g - 1) * ctl);
-            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)(g - 1), (uint32_t)lo, 1, 0, yb.data(),
-                                    bb.data() + ctl, lo * N, ws.data(), nullptr));
-        }
-        // column shifts of sigma(A), shift k rotated back by g (k / g) rows
-        std::vector<Shift> sa;
-        for (i64 k = 1; k < n; k++)
-            sa.push_back(Shift{k - g * (k / g) * w, &cm[(size_t)(2 * k + 1)], &cm[(size_t)(2 * k)]});
-        const Sources xa = extendSources(c, ab.data(), 1, nq);
-        const i64 back = -n;
-        const DeviceBuffer a2 = rotateSources(eval, xa, ab.data(), 1, &back);
-        const Sources xa2 = extendSources(c, a2.data(), 1, nq);
-        // U[k2]: [3][lo][N]; U[0] is `acc`, which already holds sigma(A) (x) tau(B)
-        const u64 uw = 3 * lo * N;
-        DeviceBuffer U(c, (u64)std::max<i64>(1, n_giant - 1) * uw);
-        std::vector<bool> started((size_t)n_giant, false);
-        started[0] = true;
-        G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)(n - 1)));
-        DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl);
-        for (size_t first = 0; first < sa.size(); first += G) {
-            const size_t cnt = std::min(G, sa.size() - first);
-            std::vector<hemm_rot_term> terms;
-            std::vector<uint32_t> off{0};
-            pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
-            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
-            // shift index q holds k = q + 1: consecutive k with the same k2 pair with consecutive baby rotations
-            size_t q = first;
-            while (q < first + cnt) {
-                const i64 kk = (i64)q + 1, k2 = kk / g, k1 = kk % g;
-                const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - k1));
-                u64 *dst = k2 == 0 ? acc.buf_.data() : U.data() + (u64)(k2 - 1) * uw;
-                ck(hemm_tensor_batch(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)k1 * ctl, (uint32_t)run,
-                                     (uint32_t)lo, dst, started[(size_t)k2] ? 1 : 0, nullptr));
-                started[(size_t)k2] = true;
-                q += run;
-            }
-        }
-        finish();   // U_0: relinearise + rescale -> level T
-        if (n_giant > 1) {
-            const u64 m = (u64)(n_giant - 1), beta = (lo + c->alpha - 1) / c->alpha, El = lo + K;
-            DeviceBuffer ext1(c, m * beta * El * N), ext2(c, m * beta * El * N), pb(c, m * lo * N), wsu(c, m * lo * N);
-            ck(hemm_modup_batch(c->dev, U.data() + lo * N, uw, (uint32_t)lo, (uint32_t)m, ext1.data(), wsu.data(), nullptr));
-            ck(hemm_modup_batch(c->dev, U.data() + 2 * lo * N, uw, (uint32_t)lo, (uint32_t)m, ext2.data(), wsu.data(), nullptr));
-            std::vector<u64> sc(lo);
-            for (u64 j = 0; j < lo; j++) {
-                u64 P = 1;
-                for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
-                sc[j] = P;
-            }
-            ck(hemm_mul_scalar(c->dev, U.data(), uw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
-            std::vector<hemm_rot_term> terms;
-            for (u64 i = 0; i < m; i++) {
-                const u64 gal = rot.galois((i64)(i + 1) * g * w);
-                hemm_rot_term t;
-                t.ext = ext1.data() + i * beta * El * N;
-                t.b = pb.data() + i * lo * N;
-                t.evk = pack.galoisKey(gal);
-                t.mask = nullptr;
-                t.galois = gal;
-                terms.push_back(t);
-                t.ext = ext2.data() + i * beta * El * N;
-                t.b = nullptr;
-                t.evk = pack.galoisSquareKey(gal);
-                terms.push_back(t);
-            }
-            const uint32_t off[2] = {0, (uint32_t)terms.size()};
-            Ciphertext giant(c);
-            giant.allocate(2, T, 0);
-            DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * (lo - 1) * N);
-            ck(hemm_hoisted_moddown(c->dev, terms.data(), off, 1, (uint32_t)lo, 1, 1, yg.data(), giant.buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
-            eval.add(res.get(), giant, res.get());
-        }
-        (void)slots;
+        DeviceBuffer U;
+        i64 g = 1;
+        bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g);
+        bsgsGiantSteps(eval, T, U, g, n / g, w, acc, res);
         return res;
     }
     std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);
@@ -658,39 +684,15 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     }
 
     const i64 n = k;
-    std::vector<Shift> sa;
-    for (i64 i = 1; i < n / 2; i++) sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], &cm[(size_t)(4 * i)]});
-    // rotation sources: sigma(A), its copy rotated by -n columns, and tau(B)
-    const Sources xa = extendSources(c, a.get().buf_.data(), 1, nqa);
-    const i64 back = -n;
-    const DeviceBuffer a2 = rotateSources(eval, xa, a.get().buf_.data(), 1, &back);
-    const Sources xa2 = extendSources(c, a2.data(), 1, nqa);
-    const Sources xb = extendSources(c, b.get().buf_.data(), 1, nqb);
-    const KeyPack &pack = eval.getKeyPack();
-    const Rot rot(c);
-    // the two operands go through separate launch chains, so each chain takes twice as many shifts
-    const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)sa.size()));
-    DeviceBuffer ya(c, G * 2 * (nqa + K) * N), yb(c, G * 2 * (nqb + K) * N), t1(c, G * 2 * lo * N), t2(c, G * 2 * lo * N),
-        ws(c, G * 2 * lo * N);
-    for (size_t first = 0; first < sa.size(); first += G) {
-        const size_t cnt = std::min(G, sa.size() - first);
-        {
-            std::vector<hemm_rot_term> terms;
-            std::vector<uint32_t> off{0};
-            pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
-            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqa, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
-        }
-        // row shifts are exact rotations here: one unmasked hoisted term each, plain ModDown
-        std::vector<hemm_rot_term> terms;
-        std::vector<uint32_t> off{0};
-        for (size_t q = first; q < first + cnt; q++) {
-            terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois((i64)(2 * (q + 1)) * w), nullptr));
-            off.push_back((uint32_t)terms.size());
-        }
-        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nqb, 1, 0, yb.data(), t2.data(), lo * N, ws.data(), nullptr));
-        ck(hemm_tensor_batch(c->dev, t1.data(), t2.data(), (uint32_t)cnt, (uint32_t)lo, acc.buf_.data(), 1, nullptr));
-    }
-    finish();
+    (void)nqa;
+    (void)nqb;
+    (void)N;
+    (void)K;
+    // column shifts of sigma(A) by 2 i, row rotations of tau(B) by 2 i w: baby-step / giant-step over i
+    DeviceBuffer U;
+    i64 g = 1;
+    bsgsShiftProduct(eval, T, a.get().buf_.data(), b.get().buf_.data(), acc, cm, n, n / 2, 2, w, batch, &U, &g);
+    bsgsGiantSteps(eval, T, U, g, (n / 2) / g, 2 * w, acc, res);
     return res;
 }
 

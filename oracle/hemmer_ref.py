@@ -622,6 +622,37 @@ def _assemble_shifts(orc, src, ext, back, shifts):
     return out
 
 
+def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w):
+    """Baby-step / giant-step sum over the shift index i = i1 + g i2 (column shift cu * i slots, row rotation
+    i * cu * w slots); `acc` holds the i = 0 term, a = sigma(A) at T+2, b_low = tau(B) at T+1."""
+    from .oracle import Ct
+    ru = cu * w
+    g = bsgs_baby_count(units)
+    ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b_low.data[1])
+    bb = [b_low] + [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (i1 * ru) % orc.slots, None)],
+                                                        b_low.nq), b_low.nq, False), b_low.scale)
+                    for i1 in range(1, g)]
+    ta = _assemble_shifts(orc, a, ext_a, -n,
+                          [((cu * i - g * (i // g) * ru) % orc.slots, cm[2 * cu * i + 1], cm[2 * cu * i])
+                           for i in range(1, units)])
+    U = [acc] + [None] * (units // g - 1)
+    for i in range(1, units):
+        t = orc.tensor(ta[i - 1], bb[i % g])
+        U[i // g] = t if U[i // g] is None else orc.add(U[i // g], t)
+    res = orc.rescale(orc.relinearize(U[0]))
+    if units // g > 1:
+        lo = b_low.nq
+        terms = []
+        for i2 in range(1, units // g):
+            gal = orc.galois((i2 * g * ru) % orc.slots)
+            u = U[i2]
+            terms.append((orc.modup(u.data[1]), u.data[0], ("g", gal), None))
+            terms.append((orc.modup(u.data[2]), None, ("sq", gal), None))
+        y = orc.hoisted_sum(terms, lo)
+        res = orc.add(res, Ct(orc.moddown_drop(y, lo, True), res.scale))
+    return res
+
+
 def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
     from .oracle import Ct
     ev = OracleEval(orc)
@@ -641,29 +672,7 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
         # The column shifts come out already rotated back by g k2 rows (another Galois element, same masks);
         # the un-relinearised U_k2 are rotated directly: d1 with the key of rho(s), d2 with a key of
         # rho(s)^2, all summed in the extended basis before one ModDown merged with the rescale.
-        g = bsgs_baby_count(n)
-        ext_b = orc.modup(b_low.data[1])
-        bb = [b_low] + [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (k1 * w) % orc.slots, None)],
-                                                            b_low.nq), b_low.nq, False), b_low.scale)
-                        for k1 in range(1, g)]
-        ta = _assemble_shifts(orc, a, ext_a, -n,
-                              [((k - g * (k // g) * w) % orc.slots, cm[2 * k + 1], cm[2 * k]) for k in range(1, n)])
-        U = [acc] + [None] * (n // g - 1)
-        for k in range(1, n):
-            t = orc.tensor(ta[k - 1], bb[k % g])
-            U[k // g] = t if U[k // g] is None else orc.add(U[k // g], t)
-        res = orc.rescale(orc.relinearize(U[0]))
-        if n // g > 1:
-            lo = b_low.nq
-            terms = []
-            for k2 in range(1, n // g):
-                gal = orc.galois((k2 * g * w) % orc.slots)
-                u = U[k2]
-                terms.append((orc.modup(u.data[1]), u.data[0], ("g", gal), None))
-                terms.append((orc.modup(u.data[2]), None, ("sq", gal), None))
-            y = orc.hoisted_sum(terms, lo)
-            res = orc.add(res, Ct(orc.moddown_drop(y, lo, True), res.scale))
-        return res
+        return _bsgs_shift_product(orc, a, b_low, acc, cm, n, n, 1, w)
     else:
         ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
         rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
@@ -684,12 +693,7 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     b = diagonal_transform_fused(orc, b, PV, n, w)
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
-    ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b.data[1])
-    ta = _assemble_shifts(orc, a, ext_a, -n, [(2 * i, cm[4 * i + 1], cm[4 * i]) for i in range(1, n // 2)])
-    for i, x in zip(range(1, n // 2), ta):
-        y = orc.hoisted_sum([(ext_b, b.data[0], (2 * i * w) % orc.slots, None)], b.nq)
-        acc = orc.add(acc, orc.tensor(x, Ct(orc.moddown_drop(y, b.nq, False), b.scale)))
-    return orc.rescale(orc.relinearize(acc))
+    return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w)
 
 
 def mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only=False):
