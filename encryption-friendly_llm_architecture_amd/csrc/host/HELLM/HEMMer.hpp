@@ -170,6 +170,9 @@ public:
         batch_ = batch;
     }
     bool fused() const { return fused_; }
+    // Promise that the operands of singleCCMatMul hold a single tile block (as HEMMer::encrypt produces) and nothing
+    // in the rest of the slot vector; see multMatMatFused.  Off by default.
+    void assumeSingleTile(bool on) { single_tile_ = on; }
 
     // generate (once) the direct rotation keys a routine needs; rotations are left shifts in slots
     void ensureRotationKeys(const std::vector<u64> &left_rotations) const;
@@ -198,7 +201,7 @@ private:
     Message col_mask_even_, row_mask_even_, mask_left_half_, mask_matmul_, mask_matmul_half_;
     mutable std::map<std::pair<int, u64>, Plaintext> mask_cache_;
     mutable std::set<u64> have_rot_;
-    bool fused_ = true;
+    bool fused_ = true, single_tile_ = false;
     u64 batch_ = 16;
 };
 

@@ -131,8 +131,13 @@ CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, con
 // every column / row shift of the main loop is a direct hoisted rotation of sigma(A) / tau(B) (one ModUp
 // per operand), the two masked halves of a shift are combined before one merged ModDown + rescale, and
 // `batch` shifts are processed per launch.
+// single_tile: the caller promises that both operands hold one tile block and nothing else (what HEMMer::encrypt
+// produces).  tau(B) is then copied into every block of the slot vector, which turns its row shifts into exact
+// rotations and opens the baby-step / giant-step route also for a matrix that fills only part of the slots.  With
+// operands that carry further tiles the result would mix them, so the default is off.
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
-                           const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16);
+                           const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16,
+                           bool single_tile = false);
 CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                                  const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer,
                                  u64 batch = 16);
@@ -145,6 +150,6 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 // the same for multMatMatFused; square_rots receives the giant steps that also need KeyPack::galoisSquareKey
 std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots,
-                                    bool packed = false);
+                                    bool packed = false, bool single_tile = false);
 
 }  // namespace HELLM

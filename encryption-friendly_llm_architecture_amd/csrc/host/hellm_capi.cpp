@@ -117,6 +117,12 @@ int hellm_set_schedule(hellm_hemmer *h, int fused, uint32_t batch) {
     h->m->setFused(fused != 0, batch);
     FACADE_CATCH
 }
+int hellm_assume_single_tile(hellm_hemmer *h, int on) {
+    FACADE_TRY
+    need(h != nullptr, "null argument");
+    h->m->assumeSingleTile(on != 0);
+    FACADE_CATCH
+}
 int hellm_sync(void) {
     FACADE_TRY
     CudaTools::cudaDeviceSynchronize();

@@ -412,10 +412,10 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
     if (fused_) {
         std::vector<u64> square_rots;
-        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots));
+        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, false, single_tile_));
         KeyGenerator keygen(context_, sk_, pack_);
         for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
-        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
+        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, single_tile_);
     }
     ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});
     return multMatMat(eval_, btp_, a, b, T, matrix_transformer);

@@ -151,12 +151,15 @@ std::vector<Plaintext> &MatrixTransformer::getRowMaskExt(const HomEvaluator &eva
 }
 
 std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots,
-                                    bool packed) {
+                                    bool packed, bool single_tile) {
     const i64 slots = i64(1) << log_slots, n = shape.getNumRows(), w = shape.getBlockWidth();
     square_rots.clear();
-    if (n * w != slots) return fusedRotations(shape, log_slots, packed, true);
+    const bool spread = single_tile && !packed && n * w < slots && slots % (n * w) == 0;
+    if (n * w != slots && !spread) return fusedRotations(shape, log_slots, packed, true);
     std::vector<u64> r;
     auto left = [&](i64 v) { return (u64)(((v % slots) + slots) % slots); };
+    if (spread)
+        for (i64 blk = n * w; blk < slots; blk <<= 1) r.push_back(left(-blk));
     const i64 cu = packed ? 2 : 1, units = n / cu, ru = cu * w, g = bsgsBabyCount(units);
     r.push_back(left(-n));
     for (i64 i = 1; i < units; i++) r.push_back(left(cu * i - g * (i / g) * ru));
@@ -547,7 +550,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, const DeviceBuffer &U, i64 
 }  // namespace
 
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
-                           const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch) {
+                           const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -609,7 +612,21 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
 
     const i64 n = k;
     size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
-    if ((u64)(n * w) == c->N / 2) {
+    const u64 slots = c->N / 2;
+    const bool spread = single_tile && (u64)(n * w) < slots && slots % (u64)(n * w) == 0;
+    if (spread) {
+        // tau(B) (level T+1) copied into every tile block: X += rho^(-block)(X), block doubling each step.  sigma(A)
+        // stays as it is: rotated back by g k2 rows it spills into the empty block below and the giant step
+        // brings it home, so the product comes out in the first block with the other blocks empty.
+        u64 *tb = low.data() + 2 * lo * N;
+        for (u64 blk = (u64)(n * w); blk < slots; blk <<= 1) {
+            const Sources xb = extendSources(c, tb, 1, lo);
+            const i64 back = -(i64)blk;
+            const DeviceBuffer moved = rotateSources(eval, xb, tb, 1, &back);
+            ck(hemm_pointwise(c->dev, HEMM_ADD, tb, lo * N, moved.data(), lo * N, tb, lo * N, (uint32_t)lo, 0, 2, nullptr));
+        }
+    }
+    if ((u64)(n * w) == slots || spread) {
         DeviceBuffer U;
         i64 g = 1;
         bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g);

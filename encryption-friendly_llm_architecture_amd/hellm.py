@@ -28,6 +28,7 @@ def _L():
         L.hellm_export_key.argtypes = [vp, u64, u64p]
         L.hellm_ensure_rotation_keys.argtypes = [vp, u64p, u32]
         L.hellm_set_schedule.argtypes = [vp, ctypes.c_int, u32]
+        L.hellm_assume_single_tile.argtypes = [vp, ctypes.c_int]
         L.hellm_encrypt.argtypes = [vp, f64p, u32, u32, pvp]
         L.hellm_encrypt2.argtypes = [vp, f64p, f64p, u32, u32, pvp]
         L.hellm_encode.argtypes = [vp, f64p, u32, u32, u32, pvp]
@@ -200,6 +201,10 @@ class HEMMer:
     def set_schedule(self, fused=True, batch=16):
         """fused: batched launches with hoisted rotations (default); False: the reference's call order."""
         check(_L().hellm_set_schedule(self.h, int(fused), batch))
+
+    def assume_single_tile(self, on=True):
+        """Promise that single_cc_matmul operands hold one tile block and nothing else (encrypt() outputs)."""
+        check(_L().hellm_assume_single_tile(self.h, int(on)))
 
     def sync(self):
         check(_L().hellm_sync())

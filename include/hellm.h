@@ -36,6 +36,10 @@ int hellm_sync(void); /* CudaTools::cudaDeviceSynchronize */
 /* schedule of the products: fused != 0 (default) = batched launches with hoisted rotations,
  * 0 = one evaluator call per step in the reference's order; batch = shifts per launch */
 int hellm_set_schedule(hellm_hemmer *h, int fused, uint32_t batch);
+/* HEMMer::assumeSingleTile: the caller promises that the operands of hellm_single_cc_matmul hold one tile block
+ * (what hellm_encrypt produces) and nothing in the rest of the slot vector; the batched schedule then takes the
+ * baby-step / giant-step route for them too.  No counterpart in the reference; off by default. */
+int hellm_assume_single_tile(hellm_hemmer *h, int on);
 
 /* codec: HEMMer::encrypt :90 / encrypt2 :91 / encode :63 / encode2 :65 / encodeDiagonalToRow4 :76 /
  * decrypt :96 / decrypt2 :98 */

@@ -653,7 +653,9 @@ def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w):
     return res
 
 
-def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
+def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
+    """single_tile: both operands hold one tile block and nothing else; tau(B) is then copied into every
+    block (X += rho^(-block)(X), block doubling), which makes its row shifts exact rotations."""
     from .oracle import Ct
     ev = OracleEval(orc)
     a = orc.level_down(a, T + 3)
@@ -665,7 +667,13 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w):
     b_low = orc.level_down_one(b)
     acc = orc.tensor(orc.level_down_one(a), b_low)
     ext_a = orc.modup(a.data[1])
-    if n * w == orc.slots:
+    spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
+    if spread:
+        blk = n * w
+        while blk < orc.slots:
+            b_low = orc.add(b_low, orc.rotate_hoisted(b_low, -blk))
+            blk <<= 1
+    if n * w == orc.slots or spread:
         # The tile block fills the slot vector: row shifts are exact rotations rho^(k w) of tau(B) lowered to
         # T+1 (no mask, plain ModDown), which allows the baby-step / giant-step split k = k1 + g k2:
         #   C = sum_k2 rho^(g k2 w)(U_k2),  U_k2 = sum_k1 rho^(-g k2 w)(phi^k(sigma A)) (x) rho^(k1 w)(tau B).

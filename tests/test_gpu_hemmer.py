@@ -118,6 +118,27 @@ def test_ccmm_residues_bit_exact_and_decrypts(small, fused):
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
 
 
+def test_ccmm_single_tile_promise(small):
+    """With the promise that the operands hold one tile block and nothing else, tau(B) is spread over every block
+    and the product takes the baby-step / giant-step route; the result still lives in the first block only."""
+    H, orc, ev = small
+    rng = np.random.default_rng(15)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    H.set_schedule(True, batch=3)
+    H.assume_single_tile(True)
+    try:
+        c = H.single_cc_matmul(ca, cb, 2)
+    finally:
+        H.assume_single_tile(False)
+        H.set_schedule(True)
+    want = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16, single_tile=True)
+    assert c.info()["level"] == 2
+    assert np.array_equal(c.residues(), want.data)
+    assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
+    assert np.abs(H.decrypt_slots(c)[256:]).max() < 2 ** -20
+
+
 @pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
 def test_ccmm_pair_layout(small, fused):
     """Two products per call on the pair layout [A1 | A2] x [B1 | B2] (rows fill the slot vector, so the
