@@ -171,7 +171,9 @@ public:
     }
     bool fused() const { return fused_; }
     // Promise that the operands of singleCCMatMul hold a single tile block (as HEMMer::encrypt produces) and nothing
-    // in the rest of the slot vector; see multMatMatFused.  Off by default.
+    // in the rest of the slot vector; see multMatMatFused.  Off by default.  Without the promise the same route is
+    // taken when it is known from the operands themselves: Encryptor::encrypt records how many slots of the
+    // plaintext were non-zero and the slot-wise evaluator operations carry that along (Ciphertext::occupiedSlots).
     void assumeSingleTile(bool on) { single_tile_ = on; }
 
     // generate (once) the direct rotation keys a routine needs; rotations are left shifts in slots

@@ -134,7 +134,8 @@ CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, con
 // single_tile: the caller promises that both operands hold one tile block and nothing else (what HEMMer::encrypt
 // produces).  tau(B) is then copied into every block of the slot vector, which turns its row shifts into exact
 // rotations and opens the baby-step / giant-step route also for a matrix that fills only part of the slots.  With
-// operands that carry further tiles the result would mix them, so the default is off.
+// operands that carry further tiles the result would mix them, so the default is off; HEMMer::singleCCMatMul sets
+// it when Ciphertext::occupiedSlots() of both operands shows it to be true.
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16,
                            bool single_tile = false);

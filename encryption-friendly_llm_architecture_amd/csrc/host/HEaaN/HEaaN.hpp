@@ -135,6 +135,7 @@ public:
     DeviceBuffer buf_;  // [level+1][N], NTT form
     u64 level_ = 0, log_slots_ = 0, rescale_counter_ = 0;
     Real scale_ = 0;    // scale of the encoded values; 0 = the fixed scale of (level, rescale counter)
+    u64 occupied_ = ~u64(0);   // slots at and beyond this index were encoded as exact zeros (all ones: unknown)
 };
 
 class Ciphertext {
@@ -158,6 +159,12 @@ public:
     Context ctx_;
     DeviceBuffer buf_;  // [num_poly][level+1][N], NTT form
     u64 level_ = 0, log_slots_ = 0, num_poly_ = 0, rescale_counter_ = 0;
+    // Slots at and beyond this index are known to hold zero (up to noise); all ones = nothing known.  Set by
+    // Encryptor::encrypt from the plaintext, carried through the slot-wise operations of HomEvaluator (add, products,
+    // rescale, levelDown, conjugation ...), forgotten by everything else: rotations, allocate(), load(), and
+    // getPolyData(), which hands out a writable pointer.  Products use it to tell a single tile from stacked tiles.
+    mutable u64 occupied_ = ~u64(0);
+    u64 occupiedSlots() const { return occupied_; }
 };
 
 class SecretKey {

@@ -258,6 +258,7 @@ void Message::load(const std::string &path) {
 void Plaintext::allocate(u64 level, u64 rc) {
     level_ = level;
     rescale_counter_ = rc;
+    occupied_ = ~u64(0);
     log_slots_ = ctx_->logN - 1;
     buf_.resize(ctx_, (level + 1) * ctx_->N);
 }
@@ -276,11 +277,13 @@ void Ciphertext::allocate(u64 num_poly, u64 level, u64 rc) {
     level_ = level;
     rescale_counter_ = rc;
     log_slots_ = ctx_->logN - 1;
+    occupied_ = ~u64(0);
     buf_.resize(ctx_, num_poly * (level + 1) * ctx_->N);
 }
 size_t Ciphertext::polyStride() const { return (size_t)(level_ + 1) * ctx_->N; }
 u64 *Ciphertext::getPolyData(u64 i, u64 level) const {
     if (i >= num_poly_) throw RuntimeException("polynomial index out of range");
+    occupied_ = ~u64(0);   // the caller may write through the pointer
     return buf_.data() + i * polyStride() + level * ctx_->N;
 }
 void Ciphertext::save(const std::string &path) const {
@@ -593,6 +596,9 @@ static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u6
         pt.buf_.resize(c, primes.size() * c->N);
     }
     lift_and_ntt(c, coeffs, primes, pt.buf_.data());
+    size_t occupied = n;
+    while (occupied > 0 && msg[occupied - 1] == Complex(0, 0)) occupied--;
+    pt.occupied_ = occupied;
     return pt;
 }
 Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) const {
@@ -686,6 +692,7 @@ void Encryptor::encrypt(const Plaintext &pt, const SecretKey &sk, Ciphertext &ct
     ck(hemm_pointwise(c->dev, HEMM_MUL, a, 0, sk.ntt(), 0, tmp.data(), 0, (uint32_t)nq, 0, 1, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_SUB, e.data(), 0, tmp.data(), 0, b, 0, (uint32_t)nq, 0, 1, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_ADD, b, 0, pt.buf_.data(), 0, b, 0, (uint32_t)nq, 0, 1, nullptr));
+    out.occupied_ = pt.occupied_;
     ct = std::move(out);
 }
 void Encryptor::encrypt(const Message &msg, const SecretKey &sk, Ciphertext &ct) const {
@@ -701,11 +708,11 @@ void Decryptor::decrypt(const Ciphertext &ct, const SecretKey &sk, Plaintext &pt
     out.allocate(lvl, 0);
     DeviceBuffer tmp(c, nq * N);
     u64 *m = out.buf_.data();
-    ck(hemm_pointwise(c->dev, HEMM_MUL, ct.getPolyData(1), 0, sk.ntt(), 0, tmp.data(), 0, nq, 0, 1, nullptr));
-    ck(hemm_pointwise(c->dev, HEMM_ADD, ct.getPolyData(0), 0, tmp.data(), 0, m, 0, nq, 0, 1, nullptr));
+    ck(hemm_pointwise(c->dev, HEMM_MUL, ct.buf_.data() + ct.polyStride(), 0, sk.ntt(), 0, tmp.data(), 0, nq, 0, 1, nullptr));
+    ck(hemm_pointwise(c->dev, HEMM_ADD, ct.buf_.data(), 0, tmp.data(), 0, m, 0, nq, 0, 1, nullptr));
     if (ct.num_poly_ == 3) {
         ck(hemm_pointwise(c->dev, HEMM_MUL, sk.ntt(), 0, sk.ntt(), 0, tmp.data(), 0, nq, 0, 1, nullptr));
-        ck(hemm_pointwise(c->dev, HEMM_MAC, ct.getPolyData(2), 0, tmp.data(), 0, m, 0, nq, 0, 1, nullptr));
+        ck(hemm_pointwise(c->dev, HEMM_MAC, ct.buf_.data() + 2 * ct.polyStride(), 0, tmp.data(), 0, m, 0, nq, 0, 1, nullptr));
     }
     out.level_ = lvl;
     out.rescale_counter_ = ct.rescale_counter_;

@@ -411,11 +411,15 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
     if (fused_) {
+        // one tile block and nothing else in the slot vector: promised by the caller, or known because both operands
+        // come from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots)
+        const u64 block = (u64)(n * w);
+        const bool single = single_tile_ || (a.get().occupiedSlots() <= block && b.get().occupiedSlots() <= block);
         std::vector<u64> square_rots;
-        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, false, single_tile_));
+        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, false, single));
         KeyGenerator keygen(context_, sk_, pack_);
         for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
-        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, single_tile_);
+        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, single);
     }
     ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});
     return multMatMat(eval_, btp_, a, b, T, matrix_transformer);

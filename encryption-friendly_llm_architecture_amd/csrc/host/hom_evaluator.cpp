@@ -68,16 +68,20 @@ struct OutSlot {
             tmp.allocate(polys, level, rc);
     }
     Ciphertext &get() { return direct ? *dst : tmp; }
-    void commit() {
+    // the result's known-empty slot range is `occupied` (all ones: nothing known); operations that are not
+    // slot-wise leave the default
+    void commit(u64 occupied = ~u64(0)) {
         if (!direct) *dst = std::move(tmp);
+        dst->occupied_ = occupied;
     }
 };
 
 void HomEvaluator::negate(const Ciphertext &a, Ciphertext &out) const {
+    const u64 occ = a.occupied_;
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     ck(hemm_pointwise(ctx_->dev, HEMM_NEG, a.buf_.data(), a.polyStride(), nullptr, 0, o.get().buf_.data(),
                       o.get().polyStride(), (uint32_t)a.level_ + 1, 0, (uint32_t)a.num_poly_, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 
 static void add_sub(const HomEvaluator &ev, const Context &c, int op, const Ciphertext &a0, const Ciphertext &b0,
@@ -95,6 +99,7 @@ static void add_sub(const HomEvaluator &ev, const Context &c, int op, const Ciph
         b = &lb;
     }
     const u64 polys = std::max(a->num_poly_, b->num_poly_), common = std::min(a->num_poly_, b->num_poly_);
+    const u64 occ = std::max(a0.occupied_, b0.occupied_);
     OutSlot o(c, out, polys, a->level_, a->rescale_counter_, true, {&a0, &b0});
     Ciphertext &r = o.get();
     ck(hemm_pointwise(c->dev, op, a->buf_.data(), a->polyStride(), b->buf_.data(), b->polyStride(), r.buf_.data(),
@@ -102,14 +107,14 @@ static void add_sub(const HomEvaluator &ev, const Context &c, int op, const Ciph
     if (polys > common) {  // 3-poly +/- 2-poly: the third polynomial passes through (negated for 2 - 3)
         const Ciphertext *big = a->num_poly_ > b->num_poly_ ? a : b;
         const bool neg = (op == HEMM_SUB && big == b);
-        const u64 *src = big->getPolyData(2);
-        u64 *dst = r.getPolyData(2);
+        const u64 *src = big->buf_.data() + 2 * big->polyStride();
+        u64 *dst = r.buf_.data() + 2 * r.polyStride();
         if (neg)
             ck(hemm_pointwise(c->dev, HEMM_NEG, src, 0, nullptr, 0, dst, 0, (uint32_t)a->level_ + 1, 0, 1, nullptr));
         else if (src != dst)
             (void)hipMemcpyAsync(dst, src, r.polyStride() * 8, hipMemcpyDeviceToDevice, nullptr);
     }
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::add(const Ciphertext &a, const Ciphertext &b, Ciphertext &out) const {
     add_sub(*this, ctx_, HEMM_ADD, a, b, out);
@@ -119,13 +124,14 @@ void HomEvaluator::sub(const Ciphertext &a, const Ciphertext &b, Ciphertext &out
 }
 void HomEvaluator::add(const Ciphertext &a, const Plaintext &b, Ciphertext &out) const {
     if (b.level_ < a.level_) throw RuntimeException("add(ct, pt): plaintext level below the ciphertext level");
+    const u64 occ = std::max(a.occupied_, b.occupied_);
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     Ciphertext &r = o.get();
     if (r.buf_.data() != a.buf_.data())
         (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, nullptr);
     ck(hemm_pointwise(ctx_->dev, HEMM_ADD, r.buf_.data(), 0, b.buf_.data(), 0, r.buf_.data(), 0,
                       (uint32_t)a.level_ + 1, 0, 1, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::add(const Ciphertext &a, const Message &b, Ciphertext &out) const {
     add(a, EnDecoder(ctx_).encode(b, a.level_), out);
@@ -151,10 +157,11 @@ void HomEvaluator::add(const Plaintext &a, const Plaintext &b, Plaintext &out) c
 void HomEvaluator::multWithoutRescale(const Ciphertext &a, const Plaintext &b, Ciphertext &out) const {
     require_rc0(a, "multWithoutRescale");
     if (b.level_ < a.level_) throw RuntimeException("mult(ct, pt): plaintext level below the ciphertext level");
+    const u64 occ = std::min(a.occupied_, b.occupied_);   // a product is empty where either factor is
     OutSlot o(ctx_, out, a.num_poly_, a.level_, 1, true, {&a});
     ck(hemm_pointwise(ctx_->dev, HEMM_MUL, a.buf_.data(), a.polyStride(), b.buf_.data(), 0, o.get().buf_.data(),
                       o.get().polyStride(), (uint32_t)a.level_ + 1, 0, (uint32_t)a.num_poly_, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::mult(const Ciphertext &a, const Plaintext &b, Ciphertext &out) const {
     multWithoutRescale(a, b, out);
@@ -179,17 +186,19 @@ void HomEvaluator::maskedSum(const Ciphertext &a, const Plaintext &ma, const Cip
 }
 
 void HomEvaluator::multInteger(const Ciphertext &a, i64 v, Ciphertext &out) const {
+    const u64 occ = a.occupied_;
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     auto sc = int_residues(ctx_, v, a.level_ + 1);
     ck(hemm_mul_scalar(ctx_->dev, a.buf_.data(), a.polyStride(), sc.data(), o.get().buf_.data(), o.get().polyStride(),
                        (uint32_t)a.level_ + 1, 0, (uint32_t)a.num_poly_, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::multImagUnit(const Ciphertext &a, Ciphertext &out) const {
+    const u64 occ = a.occupied_;
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     ck(hemm_mul_imag_unit(ctx_->dev, a.buf_.data(), a.polyStride(), o.get().buf_.data(), o.get().polyStride(),
                           (uint32_t)a.level_ + 1, (uint32_t)a.num_poly_, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::multWithoutRescale(const Ciphertext &a, const Complex &cst, Ciphertext &out) const {
     require_rc0(a, "multWithoutRescale");
@@ -255,10 +264,11 @@ void HomEvaluator::tensor(const Ciphertext &a, const Ciphertext &b, Ciphertext &
         levelDown(b, lvl, lb);
         pb = &lb;
     }
+    const u64 occ = std::min(a.occupied_, b.occupied_);
     OutSlot o(ctx_, out, 3, lvl, 1, false, {&a, &b});
     ck(hemm_tensor(ctx_->dev, pa->buf_.data(), pa->polyStride(), pb->buf_.data(), pb->polyStride(),
                    o.get().buf_.data(), o.get().polyStride(), (uint32_t)lvl + 1, 0, nullptr));
-    o.commit();
+    o.commit(occ);
 }
 void HomEvaluator::tensorAccumulate(const Ciphertext &a, const Ciphertext &b, Ciphertext &acc, bool first) const {
     if (first) {
@@ -269,6 +279,7 @@ void HomEvaluator::tensorAccumulate(const Ciphertext &a, const Ciphertext &b, Ci
         throw RuntimeException("tensorAccumulate: shape mismatch");
     ck(hemm_tensor(ctx_->dev, a.buf_.data(), a.polyStride(), b.buf_.data(), b.polyStride(), acc.buf_.data(),
                    acc.polyStride(), (uint32_t)a.level_ + 1, 1, nullptr));
+    acc.occupied_ = std::max(acc.occupied_, std::min(a.occupied_, b.occupied_));
 }
 void HomEvaluator::relinearize(const Ciphertext &a, Ciphertext &out) const {
     if (a.num_poly_ != 3) throw RuntimeException("relinearize: operand must have three polynomials");
@@ -276,6 +287,7 @@ void HomEvaluator::relinearize(const Ciphertext &a, Ciphertext &out) const {
     r.allocate(2, a.level_, a.rescale_counter_);
     ck(hemm_relinearize(ctx_->dev, a.buf_.data(), a.polyStride(), pack_.multKey(), (uint32_t)a.level_ + 1,
                         r.buf_.data(), r.polyStride(), nullptr));
+    r.occupied_ = a.occupied_;
     out = std::move(r);
 }
 void HomEvaluator::rescale(Ciphertext &a) const {
@@ -285,6 +297,7 @@ void HomEvaluator::rescale(Ciphertext &a) const {
     r.allocate(a.num_poly_, a.level_ - 1, a.rescale_counter_ - 1);
     ck(hemm_rescale(ctx_->dev, a.buf_.data(), a.polyStride(), r.buf_.data(), r.polyStride(), (uint32_t)a.level_ + 1,
                     (uint32_t)a.num_poly_, nullptr));
+    r.occupied_ = a.occupied_;
     a = std::move(r);
 }
 void HomEvaluator::rescale(Plaintext &a) const {
@@ -319,6 +332,7 @@ void HomEvaluator::levelDown(const Ciphertext &a, u64 target, Ciphertext &out) c
     auto sc = int_residues(ctx_, v, target + 2);
     ck(hemm_mul_scalar(ctx_->dev, a.buf_.data(), a.polyStride(), sc.data(), t.buf_.data(), t.polyStride(),
                        (uint32_t)target + 2, 0, (uint32_t)a.num_poly_, nullptr));
+    t.occupied_ = a.occupied_;
     rescale(t);
     out = std::move(t);
 }
@@ -399,7 +413,11 @@ void HomEvaluator::rightRotate(const Ciphertext &a, u64 rot, Ciphertext &out) co
     const u64 slots = ctx_->N / 2;
     leftRotate(a, (slots - rot % slots) % slots, out);
 }
-void HomEvaluator::conjugate(const Ciphertext &a, Ciphertext &out) const { applyGalois(a, 2 * ctx_->N - 1, out); }
+void HomEvaluator::conjugate(const Ciphertext &a, Ciphertext &out) const {
+    const u64 occ = a.occupied_;   // conjugation acts on every slot by itself
+    applyGalois(a, 2 * ctx_->N - 1, out);
+    out.occupied_ = occ;
+}
 void HomEvaluator::leftRotateReduce(const Ciphertext &a, u64 idx_interval, u64 num_summation, Ciphertext &out) const {
     // sum_{k < num_summation} leftRotate(a, k * idx_interval), num_summation a power of two
     Ciphertext acc(a), t(ctx_);

@@ -631,6 +631,7 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         i64 g = 1;
         bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g);
         bsgsGiantSteps(eval, T, U, g, n / g, w, acc, res);
+        if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
     std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);

@@ -112,7 +112,9 @@ def test_ccmm_residues_bit_exact_and_decrypts(small, fused):
     finally:
         H.set_schedule(True)
     oa, ob = to_oracle(orc, ca), to_oracle(orc, cb)
-    want = R.mult_mat_mat_cc_fused(orc, oa, ob, 2, 16, 16) if fused else R.mult_mat_mat_cc(ev, oa, ob, 2, 16, 16)
+    # operands straight from encrypt() are known to hold a single tile: the batched schedule spreads tau(B)
+    want = (R.mult_mat_mat_cc_fused(orc, oa, ob, 2, 16, 16, single_tile=True) if fused
+            else R.mult_mat_mat_cc(ev, oa, ob, 2, 16, 16))
     assert c.info()["level"] == 2
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
@@ -137,6 +139,31 @@ def test_ccmm_single_tile_promise(small):
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
     assert np.abs(H.decrypt_slots(c)[256:]).max() < 2 ** -20
+
+
+def test_ccmm_stacked_tiles_keep_block_products(small):
+    """Two 16 x 16 tiles stacked in one ciphertext (block width 16, 32 rows): nothing is known about which slots
+    are empty, so the batched schedule must keep the masked row shifts and return both block products."""
+    H, orc, ev = small
+    rng = np.random.default_rng(16)
+    A, B = rng.uniform(-1, 1, (32, 16)), rng.uniform(-1, 1, (32, 16))
+    ea, eb = H.encrypt(A), H.encrypt(B)
+    ca = H.upload(ea.residues(), 16, 16, 16)       # same residues, declared as 16 x 16 tiles
+    cb = H.upload(eb.residues(), 16, 16, 16)
+    H.set_schedule(True, batch=5)
+    c = H.single_cc_matmul(ca, cb, 2)
+    H.set_schedule(True)
+    want = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16)
+    assert np.array_equal(c.residues(), want.data)
+    d = H.decrypt_slots(c).real[:512].reshape(32, 16)
+    assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -20
+    assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -20
+    # a rotation forgets what was known about a single tile: the masked route again
+    ra = H.left_rotate(H.left_rotate(H.encrypt(A[:16]), 3), 512 - 3)
+    c2 = H.single_cc_matmul(ra, H.encrypt(B[:16]), 2)
+    want2 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ra), to_oracle(orc, H.encrypt(B[:16])), 2, 16, 16)
+    assert np.abs(H.decrypt(c2) - A[:16] @ B[:16]).max() < 2 ** -18
+    assert c2.info()["level"] == want2.level
 
 
 @pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
