@@ -26,6 +26,11 @@ enum class MaskKind { Horizontal, Vertical, PackedHorizontal, PackedVertical, Di
 // part.  Vertical (tau): the same with rows and columns swapped.  Packed kinds work on 2 x 2 cells.
 // Diagonal (transpose): output positions (r, c) with r - c == idx.
 Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, i64 idx);
+// Slot pattern of the two-stage transforms: stage 1 selects the rows (sigma) / columns (tau) whose cell index is r
+// mod b, stage 2 those whose cell index div b is r; part 0: all of them, 1: the positions that do not wrap under the
+// stage's rotation (r cells, or r b cells), 2: those that do.  b = twoStageSplit(cells per side).
+Message twoStageMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, int stage, i64 r, int part);
+i64 twoStageSplit(i64 units);   // the smallest power of two b with b * b >= units
 
 class MatrixTransformer {
 public:
@@ -67,6 +72,16 @@ public:
     void diagonalTransformBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
                                 const TileTensorShape *shapes, u64 *out);
 
+    // Two-stage form of the same sigma / tau (square tiles): row i is rotated by i mod b in the first stage and by
+    // b (i div b) in the second (b ~ sqrt(n)), each stage one mask level: in [job][2][level+1][N] -> out
+    // [job][2][level-1][N], TWO levels lower.  2 (b + n/b) keyed rotations with 2 (b + n/b) masks per operand
+    // instead of b + 2 n/b rotations with 2 n - 1 masks, and every stage is a single output of the hoisted launch
+    // (one ModDown per stage).  Used by the batched products when the operands have a level to spare.
+    void diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
+                                   const TileTensorShape *shapes, u64 *out);
+    // left rotations (in slots) the two-stage transform of `kind` uses on tiles in rows of `width` slots
+    static std::vector<u64> twoStageRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots);
+
     void cleanUp();
     size_t cachedMasks() const;
 
@@ -86,6 +101,11 @@ private:
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_, col_masks_ext_first_;
     std::map<std::pair<TileTensorShape, u64>, Plaintext> first_block_masks_;
+    // (kind, shape, level, stage * 4096 + r * 4 + part) -> mask of the two-stage transforms; part 0 is an ordinary
+    // plaintext (the unrotated rows), parts 1 / 2 (main / wrapped columns) are over the extended basis
+    std::map<Key, Plaintext> two_stage_masks_;
+    const Plaintext &twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape, u64 level,
+                                  int stage, i64 r, int part);
 };
 
 // A x B for two encrypted tiles (HEMMer::singleCCMatMul); output level = target_level.

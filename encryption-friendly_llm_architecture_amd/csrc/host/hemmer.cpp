@@ -413,6 +413,8 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     if (fused_) {
         // one tile block and nothing else in the slot vector: promised by the caller, or known because both operands
         // come from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots)
+        ensureRotationKeys(MatrixTransformer::twoStageRotations(MaskKind::Horizontal, TileTensorShape(n, n, w), log_slots_));
+        ensureRotationKeys(MatrixTransformer::twoStageRotations(MaskKind::Vertical, TileTensorShape(n, n, w), log_slots_));
         const u64 block = (u64)(n * w);
         const bool single = single_tile_ || (a.get().occupiedSlots() <= block && b.get().occupiedSlots() <= block);
         std::vector<u64> square_rots;

@@ -403,6 +403,18 @@ void pushShifts(const HomEvaluator &eval, const Sources &x, size_t ix, const Sou
     }
 }
 
+// the same without closing a group per shift: all shifts become terms of the output being assembled
+void pushShiftGroup(const HomEvaluator &eval, const Sources &x, size_t ix, const Sources &x2, size_t ix2,
+                    const std::vector<Shift> &shifts, std::vector<hemm_rot_term> &terms) {
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(eval.getContext());
+    for (const Shift &sft : shifts) {
+        const u64 g = rot.galois(sft.rot);
+        terms.push_back(term(x.extOf(ix), x.pbOf(ix), pack, g, sft.main_mask));
+        terms.push_back(term(x2.extOf(ix2), x2.pbOf(ix2), pack, g, sft.wrap_mask));
+    }
+}
+
 // levelDown by one level of n_polys polynomials [n_polys][level+1][N] -> [n_polys][level][N]:
 // multiply by round(Delta_{level-1} q_level / Delta_level), rescale (HomEvaluator::levelDown on a batch)
 void levelDownOneBatch(const Context &c, const u64 *in, size_t n_polys, u64 level, u64 *out) {
@@ -428,6 +440,122 @@ i64 commonBlockWidth(const HETensor<T1> &a, const HETensor<T2> &b) {
 }
 
 }  // namespace
+
+// ---- two-stage sigma / tau ----------------------------------------------------------------------------------
+i64 twoStageSplit(i64 units) {
+    i64 b = 1;
+    while (b * b < units) b <<= 1;
+    return b;
+}
+
+Message twoStageMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, int stage, i64 r, int part) {
+    const Geo g = geo(kind, shape);
+    if (shape.getNumRows() != shape.getNumCols())
+        throw std::invalid_argument("[MatrixTransformer] the two-stage transforms need square tiles");
+    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
+    const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, height = slots / w, n = g.n, u = g.units;
+    const i64 b = twoStageSplit(u), amount = stage == 1 ? r : r * b;
+    const double value = (kind == MaskKind::PackedHorizontal && stage == 1) ? 0.5 : 1.0;
+    Message m(log_slots, 0);
+    for (i64 row = 0; row < height; row++)
+        for (i64 col = 0; col < w; col++) {
+            const i64 Rc = (row % n) / g.cell, Cc = (col % n) / g.cell;
+            const i64 sel = vertical ? Cc : Rc, pos = vertical ? Rc : Cc;
+            bool on = stage == 1 ? (sel % b == r) : (sel / b == r);
+            if (part == 1) on = on && pos < u - amount;
+            if (part == 2) on = on && pos >= u - amount;
+            if (on) m[(u64)(row * w + col)] = value;
+        }
+    return m;
+}
+
+const Plaintext &MatrixTransformer::twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape,
+                                                 u64 level, int stage, i64 r, int part) {
+    Key key{(int)kind, shape, level, (i64)stage * 4096 + r * 4 + part};
+    auto it = two_stage_masks_.find(key);
+    if (it != two_stage_masks_.end()) return it->second;
+    const Context &ctx = eval.getContext();
+    const Message m = twoStageMaskMessage(kind, shape, getLogFullSlots(ctx), stage, r, part);
+    EnDecoder endec(ctx);
+    return two_stage_masks_.emplace(key, part == 0 ? endec.encode(m, level) : endec.encodeExtended(m, level)).first->second;
+}
+
+std::vector<u64> MatrixTransformer::twoStageRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots) {
+    const Geo g = geo(kind, shape);
+    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
+    const i64 slots = i64(1) << log_slots, b = twoStageSplit(g.units);
+    const i64 wrap = g.n * (vertical ? shape.getBlockWidth() : 1);
+    std::vector<u64> r;
+    auto left = [&](i64 v) { r.push_back((u64)(((v % slots) + slots) % slots)); };
+    left(-wrap);
+    for (i64 i = 1; i < b; i++) left(i * g.step);
+    for (i64 i = 1; i < g.units / b; i++) left(i * b * g.step);
+    return r;
+}
+
+void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
+                                                  const MaskKind *kinds, const TileTensorShape *shapes, u64 *out) {
+    const Context &c = eval.getContext();
+    if (level < 2) throw std::invalid_argument("[diagonalTransform] level >= 2 is needed.");
+    const u64 N = c->N;
+    DeviceBuffer mid(c, n_jobs * 2 * level * N);   // after stage 1: level - 1
+    for (int stage = 1; stage <= 2; stage++) {
+        const u64 lvl = stage == 1 ? level : level - 1, nq = lvl + 1, E = nq + c->nP, ctw = 2 * nq * N;
+        const u64 *src = stage == 1 ? in : mid.data();
+        u64 *dst = stage == 1 ? mid.data() : out;
+        // rotation sources: X and X' = rho^(-one tile side)(X)
+        const Sources x = extendSources(c, src, n_jobs, nq);
+        std::vector<i64> back(n_jobs);
+        std::vector<Geo> g;
+        for (size_t q = 0; q < n_jobs; q++) {
+            g.push_back(geo(kinds[q], shapes[q]));
+            const bool vertical = (kinds[q] == MaskKind::Vertical || kinds[q] == MaskKind::PackedVertical);
+            back[q] = -g[q].n * (vertical ? shapes[q].getBlockWidth() : 1);
+        }
+        const DeviceBuffer src2 = rotateSources(eval, x, src, n_jobs, back.data());
+        const Sources x2 = extendSources(c, src2.data(), n_jobs, nq);
+        // one output per job: sum over the stage's rotations of main_r rot(X) + wrap_r rot(X')
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        std::vector<hemm_lin_term> zero_terms;
+        std::vector<uint32_t> zoff{0};
+        bool any_rotation = false;
+        for (size_t q = 0; q < n_jobs; q++) {
+            const i64 b = twoStageSplit(g[q].units), count = stage == 1 ? b : g[q].units / b, mul = stage == 1 ? 1 : b;
+            std::vector<Shift> sh;
+            std::vector<const Plaintext *> keep;
+            for (i64 r = 1; r < count; r++)
+                sh.push_back(Shift{r * mul * g[q].step, &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 1),
+                                   &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)});
+            pushShiftGroup(eval, x, q, x2, q, sh, terms);
+            off.push_back((uint32_t)terms.size());
+            any_rotation = any_rotation || !sh.empty();
+            hemm_lin_term t;
+            t.ct = src + q * ctw;
+            t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
+            t.stride = nq * N;
+            t.galois = 0;
+            zero_terms.push_back(t);
+            zoff.push_back((uint32_t)zero_terms.size());
+        }
+        // unrotated rows: mask, rescale
+        DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
+        ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), nullptr));
+        ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
+        if (any_rotation) {
+            for (size_t q = 0; q + 1 < off.size(); q++)
+                if (off[q + 1] == off[q])
+                    throw RuntimeException("diagonalTransformTwoStage: jobs with and without rotations cannot share a batch");
+            DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, 1, 1, y.data(), dst,
+                                    (nq - 1) * N, ws.data(), nullptr));
+            ck(hemm_pointwise(c->dev, HEMM_ADD, dst, (nq - 1) * N, zres.data(), (nq - 1) * N, dst, (nq - 1) * N,
+                              (uint32_t)(nq - 1), 0, (uint32_t)(2 * n_jobs), nullptr));
+        } else {
+            (void)hipMemcpyAsync(dst, zres.data(), n_jobs * 2 * (nq - 1) * N * 8, hipMemcpyDeviceToDevice, nullptr);
+        }
+    }
+}
 
 namespace {
 // Sum over the shift index of a product whose row shifts are exact rotations (the tile block fills the slot vector),
@@ -564,20 +692,25 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     if (min_level < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get(), b.get());
     if (min_level < T + 3)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
-    // the transforms run at level T+3: lowering first gives the same values with 8 instead of 13 limbs
+    // The transforms end at level T+2.  With a level to spare they run in two stages from T+4 (far fewer rotations
+    // and masks, MatrixTransformer::diagonalTransformTwoStage), otherwise in one from T+3; lowering the operands first
+    // gives the same values with 9 or 8 instead of 13 limbs.
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
     // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
+    const bool two_stage = min_level >= T + 4 && a.getShape().getNumRows() == a.getShape().getNumCols() &&
+                           b.getShape().getNumRows() == b.getShape().getNumCols();
+    const u64 Lt = two_stage ? T + 4 : T + 3;   // level the transforms start from
     DeviceBuffer ab(c, 2 * ctw);
     {
-        const u64 ctw_in = 2 * (nq + 1) * N;
+        const u64 ctw_in = 2 * (Lt + 1) * N;
         DeviceBuffer joint(c, 2 * ctw_in);
         const u64 la = a.getLevel(), lb = b.getLevel();
-        if (la == lb && la > T + 3 && a.get().getRescaleCounter() == 0 && b.get().getRescaleCounter() == 0) {
-            // HomEvaluator::levelDown of both operands at once: multiply by round(Delta_{T+3} q_{T+4} / Delta_level)
-            // over T+5 limbs, then one rescale of the four polynomials straight into the joint buffer
-            const u64 nl = T + 5;
-            const i64 v = (i64)llround(c->delta[T + 3] * (Real)c->q[T + 4] / c->delta[la]);
+        if (la == lb && la > Lt && a.get().getRescaleCounter() == 0 && b.get().getRescaleCounter() == 0) {
+            // HomEvaluator::levelDown of both operands at once: multiply by round(Delta_Lt q_{Lt+1} / Delta_level)
+            // over Lt+2 limbs, then one rescale of the four polynomials straight into the joint buffer
+            const u64 nl = Lt + 2;
+            const i64 v = (i64)llround(c->delta[Lt] * (Real)c->q[Lt + 1] / c->delta[la]);
             std::vector<u64> sc(nl);
             for (u64 j = 0; j < nl; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
             DeviceBuffer t(c, 4 * nl * N);
@@ -585,14 +718,17 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
             ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
             ck(hemm_rescale(c->dev, t.data(), nl * N, joint.data(), (nl - 1) * N, (uint32_t)nl, 4, nullptr));
         } else {
-            eval.levelDown(a.get(), T + 3, a.get());
-            eval.levelDown(b.get(), T + 3, b.get());
+            eval.levelDown(a.get(), Lt, a.get());
+            eval.levelDown(b.get(), Lt, b.get());
             (void)hipMemcpyAsync(joint.data(), a.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
             (void)hipMemcpyAsync(joint.data() + ctw_in, b.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
         }
         const MaskKind kinds[2] = {MaskKind::Horizontal, MaskKind::Vertical};
         const TileTensorShape shapes[2] = {a.getShape(), b.getShape()};
-        tr.diagonalTransformBatch(eval, joint.data(), 2, T + 3, kinds, shapes, ab.data());
+        if (two_stage)
+            tr.diagonalTransformTwoStage(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
+        else
+            tr.diagonalTransformBatch(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
     }
     // the k = 0 term sigma(A) (x) tau(B) joins the accumulator at the shifts' level T+1
     Ciphertext acc(c);

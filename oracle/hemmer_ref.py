@@ -597,6 +597,65 @@ def bsgs_baby_count(n):
     return g
 
 
+def two_stage_split(units):
+    """Smallest power of two b with b * b >= units."""
+    b = 1
+    while b * b < units:
+        b <<= 1
+    return b
+
+
+def two_stage_mask(kind, n, w, slots, stage, r, part):
+    """Masks of the two-stage sigma / tau: stage 1 selects the rows (sigma) / columns (tau) whose cell index
+    is r mod b, stage 2 those whose cell index div b is r; part 0: all of them, 1: the positions that do
+    not wrap under the stage's rotation (r cells, or r b cells), 2: those that do."""
+    cell = 2 if kind in (PH, PV) else 1
+    u = n // cell
+    b = two_stage_split(u)
+    row, col = np.arange(slots) // w, np.arange(slots) % w
+    Rc, Cc = (row % n) // cell, (col % n) // cell
+    sel, pos = (Cc, Rc) if kind in (V, PV) else (Rc, Cc)
+    on = (sel % b == r) if stage == 1 else (sel // b == r)
+    amount = r if stage == 1 else r * b
+    if part == 1:
+        on = on & (pos < u - amount)
+    elif part == 2:
+        on = on & (pos >= u - amount)
+    return np.where(on, 0.5 if (kind == PH and stage == 1) else 1.0, 0.0).astype(np.complex128)
+
+
+def diagonal_transform_two_stage(orc, ct, kind, n, w):
+    """sigma / tau (square tiles) in two stages of one mask level each: row i is rotated by i mod b, then
+    by b (i div b).  Every stage: X' = rho^(-tile side)(X); one hoisted sum over the stage's rotations of
+    main_r rot(X) + wrap_r rot(X') with ModDown merged with the rescale, plus rescale(mask_0 X) for the
+    rows that stay.  Level L -> L - 2."""
+    from .oracle import Ct
+    cell = 2 if kind in (PH, PV) else 1
+    u = n // cell
+    b = two_stage_split(u)
+    step = cell * (w if kind in (V, PV) else 1)
+    wrap = n * (w if kind in (V, PV) else 1)
+    x = ct
+    for stage, count, mul in ((1, b, 1), (2, u // b, b)):
+        nq = x.nq
+        ext = orc.modup(x.data[1])
+        x2 = _rotated_copy(orc, x, ext, -wrap)
+        ext2 = orc.modup(x2.data[1])
+        zero = orc.rescale(orc.mult_plain_no_rescale(
+            x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), x.level)))
+        terms = []
+        for r in range(1, count):
+            rr = (r * mul * step) % orc.slots
+            terms.append((ext, x.data[0], rr, orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, 1), x.level)))
+            terms.append((ext2, x2.data[0], rr, orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, 2), x.level)))
+        if terms:
+            y = orc.hoisted_sum(terms, nq)
+            x = orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
+        else:
+            x = zero
+    return x
+
+
 def _rotated_copy(orc, src, ext, r):
     """rot(src, r) with the automorphism after ModUp (one hoisted term, plain ModDown)."""
     from .oracle import Ct
@@ -658,11 +717,13 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     block (X += rho^(-block)(X), block doubling), which makes its row shifts exact rotations."""
     from .oracle import Ct
     ev = OracleEval(orc)
-    a = orc.level_down(a, T + 3)
-    b = orc.level_down(b, T + 3)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
-    a = diagonal_transform_fused(orc, a, H, n, w)
-    b = diagonal_transform_fused(orc, b, V, n, w)
+    if min(a.level, b.level) >= T + 4:     # a level to spare: two-stage transforms from T+4
+        a = diagonal_transform_two_stage(orc, orc.level_down(a, T + 4), H, n, w)
+        b = diagonal_transform_two_stage(orc, orc.level_down(b, T + 4), V, n, w)
+    else:
+        a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), H, n, w)
+        b = diagonal_transform_fused(orc, orc.level_down(b, T + 3), V, n, w)
     # the k = 0 term joins the accumulator at the shifts' level
     b_low = orc.level_down_one(b)
     acc = orc.tensor(orc.level_down_one(a), b_low)

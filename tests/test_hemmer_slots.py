@@ -135,3 +135,29 @@ def test_rotate_and_sum_reductions():
     mean, sq = R.row_moments(ev, tiles, 1.0 / rows.shape[1], n)
     assert np.abs(ev.decrypt(mean).real.reshape(n, 2 * n) - rows.mean(axis=1, keepdims=True)).max() < 1e-12
     assert np.abs(ev.decrypt(sq).real.reshape(n, 2 * n) - (rows ** 2).mean(axis=1, keepdims=True)).max() < 1e-12
+
+
+@pytest.mark.parametrize("n,w,log_slots", [(8, 16, 7), (8, 8, 7), (16, 32, 9)])
+def test_two_stage_transform_masks(n, w, log_slots):
+    """The two-stage sigma / tau (rows rotated by i mod b, then by b (i div b)) built from its masks and plain
+    rotations equals the one-stage transform of the reference for all four kinds."""
+    sim = R.SlotSim(log_slots, 12)
+    rng = np.random.default_rng(n * w)
+    x0 = rng.normal(size=sim.slots) + 1j * rng.normal(size=sim.slots)
+    rot = lambda v, r: np.roll(v, -r)
+    for kind in (R.H, R.V, R.PH, R.PV):
+        cell = 2 if kind in (R.PH, R.PV) else 1
+        u = n // cell
+        b = R.two_stage_split(u)
+        step = cell * (w if kind in (R.V, R.PV) else 1)
+        wrap = n * (w if kind in (R.V, R.PV) else 1)
+        x = x0
+        for stage, count, mul in ((1, b, 1), (2, u // b, b)):
+            x2 = rot(x, -wrap)
+            y = R.two_stage_mask(kind, n, w, sim.slots, stage, 0, 0) * x
+            for r in range(1, count):
+                y = y + R.two_stage_mask(kind, n, w, sim.slots, stage, r, 1) * rot(x, r * mul * step)
+                y = y + R.two_stage_mask(kind, n, w, sim.slots, stage, r, 2) * rot(x2, r * mul * step)
+            x = y
+        want = R.diagonal_transform(sim, sim.encrypt(x0), kind, n, w).z
+        assert np.abs(x - want).max() < 1e-12, kind
