@@ -79,6 +79,11 @@ public:
     // (one ModDown per stage).  Used by the batched products when the operands have a level to spare.
     void diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
                                    const TileTensorShape *shapes, u64 *out);
+    // Brings `in` down to the level a transform ending at `end_level` starts from and runs it with the batched
+    // launches: two stages from end_level + 2 when the operand is that high and the tile is square, otherwise one
+    // stage from end_level + 1.
+    Ciphertext lowerAndTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                      const TileTensorShape &shape, u64 end_level);
     // left rotations (in slots) the two-stage transform of `kind` uses on tiles in rows of `width` slots
     static std::vector<u64> twoStageRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots);
 

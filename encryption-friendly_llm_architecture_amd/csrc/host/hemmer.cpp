@@ -98,6 +98,8 @@ void HEMMer::ensureRotationKeys(const std::vector<u64> &rots) const {
 std::vector<u64> HEMMer::transformRotations(MaskKind kind, i64 width) const {
     const u64 slots = u64(1) << log_slots_;
     const i64 n = dim_;
+    if (fused_ && kind != MaskKind::Diagonal)   // the batched products may take the two-stage form
+        ensureRotationKeys(MatrixTransformer::twoStageRotations(kind, TileTensorShape(n, n, width), log_slots_));
     std::vector<u64> r;
     auto left = [&](i64 v) { r.push_back((u64)(((v % (i64)slots) + (i64)slots) % (i64)slots)); };
     if (kind == MaskKind::Diagonal) {
@@ -413,8 +415,6 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     if (fused_) {
         // one tile block and nothing else in the slot vector: promised by the caller, or known because both operands
         // come from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots)
-        ensureRotationKeys(MatrixTransformer::twoStageRotations(MaskKind::Horizontal, TileTensorShape(n, n, w), log_slots_));
-        ensureRotationKeys(MatrixTransformer::twoStageRotations(MaskKind::Vertical, TileTensorShape(n, n, w), log_slots_));
         const u64 block = (u64)(n * w);
         const bool single = single_tile_ || (a.get().occupiedSlots() <= block && b.get().occupiedSlots() <= block);
         std::vector<u64> square_rots;
@@ -496,6 +496,8 @@ CtxtTensor HEMMer::matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtT
 // ---- LoRA low-rank path --------------------------------------------------------------------------------------
 std::vector<u64> HEMMer::transformRotations(MaskKind kind, const TileTensorShape &shape) const {
     const u64 slots = u64(1) << log_slots_;
+    if (fused_ && shape.getNumRows() == shape.getNumCols())   // the batched products may take the two-stage form
+        ensureRotationKeys(MatrixTransformer::twoStageRotations(kind, shape, log_slots_));
     const bool vertical = kind == MaskKind::Vertical;
     const i64 rows = shape.getNumRows(), cols = shape.getNumCols(), step = vertical ? shape.getBlockWidth() : 1;
     const i64 units = vertical ? rows : cols, sub = std::min(rows, cols);

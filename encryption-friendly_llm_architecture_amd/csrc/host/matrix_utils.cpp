@@ -413,11 +413,19 @@ CtxtTensor multMatMat<Ciphertext>(const HomEvaluator &eval, const Bootstrapper &
 // rotations, and the product loop stops after low_dim terms; the outputs of all column blocks still have to
 // be summed (HEMMer::repackTo*).
 namespace {
+// transform of an operand ending at level T+2: batched (two stages when the operand is high enough, see
+// MatrixTransformer::lowerAndTransformFused) or in the reference's order from level T+3
 Ciphertext sigmaTau(const HomEvaluator &eval, MatrixTransformer &tr, const Ciphertext &in, MaskKind kind,
-                    const TileTensorShape &shape, bool fused) {
-    if (fused) return tr.diagonalTransformFused(eval, in, kind, shape);
-    CtxtTensor t(shape, in);
+                    const TileTensorShape &shape, u64 T, bool fused) {
+    if (fused) return tr.lowerAndTransformFused(eval, in, kind, shape, T + 2);
+    Ciphertext x(eval.getContext());
+    eval.levelDown(in, T + 3, x);
+    CtxtTensor t(shape, x);
     return kind == MaskKind::Horizontal ? tr.diagonalToColumn(eval, t).get() : tr.diagonalToRow(eval, t).get();
+}
+// level the operands are lowered to before anything else: the batched transforms may start one level higher
+u64 loraStartLevel(const CtxtTensor &op1, const CtxtTensor &op2, u64 T, bool fused) {
+    return (fused && std::min(op1.getLevel(), op2.getLevel()) >= T + 4) ? T + 4 : T + 3;
 }
 
 // sigma(A) (.) tau(B) and the low_dim - 1 shifted terms (:1716-1766)
@@ -461,10 +469,8 @@ CtxtTensor multMatMatHighLow(const HomEvaluator &eval, const CtxtTensor &op1, co
     const Context &ctx = eval.getContext();
     const i64 w = op2.getBlockWidth();
     Ciphertext a(ctx), b(ctx), tmp(ctx);
-    eval.levelDown(op1.get(), T + 3, a);
-    eval.levelDown(op2.get(), T + 3, b);
-    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, op1.getShape(), fused);
-    b = sigmaTau(eval, tr, b, MaskKind::Vertical, TileTensorShape(op2.getHeight(), low_dim, w), fused);
+    a = sigmaTau(eval, tr, op1.get(), MaskKind::Horizontal, op1.getShape(), T, fused);
+    b = sigmaTau(eval, tr, op2.get(), MaskKind::Vertical, TileTensorShape(op2.getHeight(), low_dim, w), T, fused);
     u64 pos = in_col_block;
     for (i64 i = low_dim; i < w / 2; i <<= 1) {
         if (pos % 2 == 0) {
@@ -485,8 +491,8 @@ CtxtTensor multMatMatLowHigh(const HomEvaluator &eval, const CtxtTensor &op1, co
     const Context &ctx = eval.getContext();
     const i64 w = commonBlockWidth(op1, op2);
     Ciphertext a(ctx), b(ctx), tmp(ctx);
-    eval.levelDown(op1.get(), T + 3, a);
-    eval.levelDown(op2.get(), T + 3, b);
+    const u64 start = loraStartLevel(op1, op2, T, fused);
+    eval.levelDown(op1.get(), start, a);
     u64 pos = in_row_block;
     for (i64 i = low_dim; i < w / 2; i <<= 1) {
         if (pos % 2 == 0)
@@ -496,8 +502,8 @@ CtxtTensor multMatMatLowHigh(const HomEvaluator &eval, const CtxtTensor &op1, co
         eval.add(a, tmp, a);
         pos /= 2;
     }
-    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, op1.getShape(), fused);
-    b = sigmaTau(eval, tr, b, MaskKind::Vertical, op2.getShape(), fused);
+    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, op1.getShape(), T, fused);
+    b = sigmaTau(eval, tr, op2.get(), MaskKind::Vertical, op2.getShape(), T, fused);
     return lowRankTerms(eval, a, b, op1, op2, w, T, low_dim, tr);
 }
 
@@ -506,10 +512,8 @@ CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, con
     const Context &ctx = eval.getContext();
     const i64 w = commonBlockWidth(op1, op2);
     Ciphertext a(ctx), b(ctx), tmp(ctx);
-    eval.levelDown(op1.get(), T + 3, a);
-    eval.levelDown(op2.get(), T + 3, b);
-    a = sigmaTau(eval, tr, a, MaskKind::Horizontal, TileTensorShape(op1.getHeight(), low_dim, w), fused);
-    b = sigmaTau(eval, tr, b, MaskKind::Vertical, TileTensorShape(low_dim, op2.getWidth(), w), fused);
+    a = sigmaTau(eval, tr, op1.get(), MaskKind::Horizontal, TileTensorShape(op1.getHeight(), low_dim, w), T, fused);
+    b = sigmaTau(eval, tr, op2.get(), MaskKind::Vertical, TileTensorShape(low_dim, op2.getWidth(), w), T, fused);
     u64 cpos = in_col_block, rpos = in_row_block;
     for (i64 i = low_dim; i < w / 2; i <<= 1) {
         if (cpos % 2 == 0)

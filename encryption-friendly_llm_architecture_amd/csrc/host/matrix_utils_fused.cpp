@@ -493,6 +493,20 @@ std::vector<u64> MatrixTransformer::twoStageRotations(MaskKind kind, const TileT
     return r;
 }
 
+Ciphertext MatrixTransformer::lowerAndTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
+                                                     const TileTensorShape &shape, u64 end_level) {
+    const Context &c = eval.getContext();
+    if (in.getLevel() < end_level + 1)
+        throw std::invalid_argument("[diagonalTransform] level >= " + std::to_string(end_level + 1) + " is needed.");
+    const bool two_stage = in.getLevel() >= end_level + 2 && shape.getNumRows() == shape.getNumCols();
+    Ciphertext x(c), res(c);
+    eval.levelDown(in, end_level + (two_stage ? 2 : 1), x);
+    if (!two_stage) return diagonalTransformFused(eval, x, kind, shape);
+    res.allocate(2, end_level, 0);
+    diagonalTransformTwoStage(eval, x.buf_.data(), 1, x.getLevel(), &kind, &shape, res.buf_.data());
+    return res;
+}
+
 void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
                                                   const MaskKind *kinds, const TileTensorShape *shapes, u64 *out) {
     const Context &c = eval.getContext();
@@ -814,10 +828,8 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     a.setShape(rows, k);
     b.setShape(k, cols);
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
-    eval.levelDown(a.get(), T + 3, a.get());
-    eval.levelDown(b.get(), T + 2, b.get());
-    a.get() = tr.diagonalTransformFused(eval, a.get(), MaskKind::PackedHorizontal, a.getShape());  // T+2
-    b.get() = tr.diagonalTransformFused(eval, b.get(), MaskKind::PackedVertical, b.getShape());    // T+1
+    a.get() = tr.lowerAndTransformFused(eval, a.get(), MaskKind::PackedHorizontal, a.getShape(), T + 2);
+    b.get() = tr.lowerAndTransformFused(eval, b.get(), MaskKind::PackedVertical, b.getShape(), T + 1);
     const u64 nqa = T + 3, nqb = T + 2, N = c->N, K = c->nP, lo = T + 2;  // both sides end at T+1 (lo limbs)
     // the k = 0 term joins the accumulator at level T+1: sigma(A) lowered one level, tau(B) as it is
     Ciphertext acc(c);
@@ -858,9 +870,8 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
     CtxtTensor a(a_in);
     if (a.getLevel() < T + 3)
         throw std::invalid_argument("[multMatMatPre] level >= " + std::to_string(T + 3) + " is needed.");
-    eval.levelDown(a.get(), T + 3, a.get());
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2, first_block_only);
-    a.get() = tr.diagonalTransformFused(eval, a.get(), MaskKind::Horizontal, a.getShape());
+    a.get() = tr.lowerAndTransformFused(eval, a.get(), MaskKind::Horizontal, a.getShape(), T + 2);
     Ciphertext first_ct(c);
     if (first_block_only)   // shift 0 is masked like the others so that it too is empty outside the first tile block
         eval.mult(a.get(), tr.firstBlockMask(eval, a.getShape(), T + 2), first_ct);

@@ -656,6 +656,15 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
     return x
 
 
+def lower_and_transform_fused(orc, x, kind, n, w, end_level):
+    """Batched transform ending at end_level: two stages from end_level + 2 when the operand is that high and
+    the tile is square, otherwise one stage from end_level + 1."""
+    rows, cols = _dims(n)
+    if x.level >= end_level + 2 and rows == cols:
+        return diagonal_transform_two_stage(orc, orc.level_down(x, end_level + 2), kind, rows, w)
+    return diagonal_transform_fused(orc, orc.level_down(x, end_level + 1), kind, n, w)
+
+
 def _rotated_copy(orc, src, ext, r):
     """rot(src, r) with the automorphism after ModUp (one hoisted term, plain ModDown)."""
     from .oracle import Ct
@@ -718,12 +727,9 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
-    if min(a.level, b.level) >= T + 4:     # a level to spare: two-stage transforms from T+4
-        a = diagonal_transform_two_stage(orc, orc.level_down(a, T + 4), H, n, w)
-        b = diagonal_transform_two_stage(orc, orc.level_down(b, T + 4), V, n, w)
-    else:
-        a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), H, n, w)
-        b = diagonal_transform_fused(orc, orc.level_down(b, T + 3), V, n, w)
+    lvl = min(a.level, b.level)            # both operands take the same route (they share the launches)
+    a = lower_and_transform_fused(orc, orc.level_down(a, min(lvl, T + 4)), H, n, w, T + 2)
+    b = lower_and_transform_fused(orc, orc.level_down(b, min(lvl, T + 4)), V, n, w, T + 2)
     # the k = 0 term joins the accumulator at the shifts' level
     b_low = orc.level_down_one(b)
     acc = orc.tensor(orc.level_down_one(a), b_low)
@@ -756,10 +762,8 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
-    a = orc.level_down(a, T + 3)
-    b = orc.level_down(b, T + 2)
-    a = diagonal_transform_fused(orc, a, PH, n, w)
-    b = diagonal_transform_fused(orc, b, PV, n, w)
+    a = lower_and_transform_fused(orc, a, PH, n, w, T + 2)
+    b = lower_and_transform_fused(orc, b, PV, n, w, T + 1)
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
     return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w)
@@ -773,8 +777,7 @@ def mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only=False):
     if first_block_only:
         masks = [m * block for m in masks]
     cm = [orc.encode_ext(m, T + 2) for m in masks]
-    a = orc.level_down(a, T + 3)
-    a = diagonal_transform_fused(orc, a, H, n, w)
+    a = lower_and_transform_fused(orc, a, H, n, w, T + 2)
     ext = orc.modup(a.data[1])
     first = OracleEval(orc).mult_pt(a, orc.encode(block, T + 2)) if first_block_only else orc.level_down_one(a)
     return [first] + _assemble_shifts(
@@ -850,14 +853,20 @@ def _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim):
     return ev.add(res, ev.rescale(ev.relinearize(acc)))
 
 
-def mult_mat_mat_high_low(ev, a, b, in_col_block, T, sa, sb, w, low_dim=LOW_DIM, transform=diagonal_transform):
+def _lora_transform(ev, x, kind, shape, w, T, fused_orc):
+    """Transform of an operand ending at T+2: reference order from T+3, or the batched form (two stages when
+    the operand is high enough)."""
+    if fused_orc is not None:
+        return lower_and_transform_fused(fused_orc, x, kind, shape, w, T + 2)
+    return diagonal_transform(ev, ev.level_down(x, T + 3), kind, shape, w)
+
+
+def mult_mat_mat_high_low(ev, a, b, in_col_block, T, sa, sb, w, low_dim=LOW_DIM, fused_orc=None):
     """multMatMatHighLow (:1681-1770).  sa, sb = (rows, cols) of the operands' tile shapes.  B holds low_dim
     columns at column block in_col_block of every tile; tau runs on (rows, low_dim) tiles and the
     result is spread along the diagonal of column blocks before the truncated product."""
-    a = ev.level_down(a, T + 3)
-    b = ev.level_down(b, T + 3)
-    a = transform(ev, a, H, sa, w)
-    b = transform(ev, b, V, (sb[0], low_dim), w)
+    a = _lora_transform(ev, a, H, sa, w, T, fused_orc)
+    b = _lora_transform(ev, b, V, (sb[0], low_dim), w, T, fused_orc)
     pos, i = in_col_block, low_dim
     while i < w // 2:
         if pos % 2 == 0:
@@ -871,30 +880,27 @@ def mult_mat_mat_high_low(ev, a, b, in_col_block, T, sa, sb, w, low_dim=LOW_DIM,
     return _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim)
 
 
-def mult_mat_mat_low_high(ev, a, b, in_row_block, T, sa, sb, w, low_dim=LOW_DIM, transform=diagonal_transform):
+def mult_mat_mat_low_high(ev, a, b, in_row_block, T, sa, sb, w, low_dim=LOW_DIM, fused_orc=None):
     """multMatMatLowHigh (:1772-1876): A holds low_dim rows at row block in_row_block; they are copied to
     every row block before sigma."""
-    a = ev.level_down(a, T + 3)
-    b = ev.level_down(b, T + 3)
+    start = T + 4 if fused_orc is not None and min(ev.level_of(a), ev.level_of(b)) >= T + 4 else T + 3
+    a = ev.level_down(a, start)
     pos, i = in_row_block, low_dim
     while i < w // 2:
         tmp = ev.right_rotate(a, i * w) if pos % 2 == 0 else ev.left_rotate(a, i * w)
         a = ev.add(a, tmp)
         pos //= 2
         i <<= 1
-    a = transform(ev, a, H, sa, w)
-    b = transform(ev, b, V, sb, w)
+    a = _lora_transform(ev, a, H, sa, w, T, fused_orc)
+    b = _lora_transform(ev, b, V, sb, w, T, fused_orc)
     return _low_rank_terms(ev, a, b, T, sa, sb, w, low_dim)
 
 
-def mult_mat_mat_low_low(ev, a, b, in_col_block, in_row_block, T, sa, sb, w, low_dim=LOW_DIM,
-                         transform=diagonal_transform):
+def mult_mat_mat_low_low(ev, a, b, in_col_block, in_row_block, T, sa, sb, w, low_dim=LOW_DIM, fused_orc=None):
     """multMatMatLowLow (:1878-1996): A (rows x low_dim at column block in_col_block) times B (low_dim x cols
     at row block in_row_block); sigma / tau run on the thin shapes and are then copied over the blocks."""
-    a = ev.level_down(a, T + 3)
-    b = ev.level_down(b, T + 3)
-    a = transform(ev, a, H, (sa[0], low_dim), w)
-    b = transform(ev, b, V, (low_dim, sb[1]), w)
+    a = _lora_transform(ev, a, H, (sa[0], low_dim), w, T, fused_orc)
+    b = _lora_transform(ev, b, V, (low_dim, sb[1]), w, T, fused_orc)
     cpos, rpos, i = in_col_block, in_row_block, low_dim
     while i < w // 2:
         tmp = ev.right_rotate(a, i) if cpos % 2 == 0 else ev.left_rotate(a, i)

@@ -33,9 +33,8 @@ def to_oracle(orc, ct):
 
 
 def transform_of(orc, fused):
-    if not fused:
-        return R.diagonal_transform
-    return lambda ev, ct, kind, n, w: R.diagonal_transform_fused(orc, ct, kind, n, w)
+    """The oracle runs the batched transforms (through `orc`) or the reference order (None)."""
+    return orc if fused else None
 
 
 def thin_cols(rng, block, n=N_TILE):
