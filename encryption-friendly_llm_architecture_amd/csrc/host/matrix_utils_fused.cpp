@@ -581,8 +581,8 @@ namespace {
 //   depend on the row, so this only changes the Galois element of shift i (still one key per shift);
 // * the un-relinearised sums U_i2 (three polynomials) are rotated by the giant steps directly: d1 under the key of
 //   rho(s), d2 under a key of rho(s)^2, all 2 (units/g - 1) terms summed in the extended basis before a single
-//   ModDown merged with the rescale.  U_0 (in `acc`, which arrives holding the i = 0 term) takes the ordinary
-//   relinearisation.
+//   ModDown merged with the rescale.  U_0 (in `acc`, which arrives holding the i = 0 term) joins the same sum with
+//   its d2 under the multiplication key.
 // units + g + 2 units/g key switches instead of 2 units.
 // sigma_a: [2][T+3][N] at level T+2; tau_b: [2][T+2][N] at level T+1; U_out receives U_1 .. (each [3][T+2][N]).
 void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
@@ -618,9 +618,9 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     const i64 back = -n;
     const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back);
     const Sources xa2 = extendSources(c, a2.data(), 1, nq);
-    // U[i2 - 1]: [3][lo][N] for i2 >= 1; U_0 is `acc`
+    // U[i2]: [3][lo][N] for i2 >= 1 (slot 0 is left for U_0, which is accumulated in `acc`)
     const u64 uw = 3 * lo * N;
-    U_out->resize(c, (u64)std::max<i64>(1, n_giant - 1) * uw);
+    U_out->resize(c, (u64)n_giant * uw);
     std::vector<bool> started((size_t)n_giant, false);
     started[0] = true;
     const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
@@ -636,7 +636,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         while (q < first + cnt) {
             const i64 ii = (i64)q + 1, i2 = ii / g, i1 = ii % g;
             const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - i1));
-            u64 *dst = i2 == 0 ? acc.buf_.data() : U_out->data() + (u64)(i2 - 1) * uw;
+            u64 *dst = i2 == 0 ? acc.buf_.data() : U_out->data() + (u64)i2 * uw;
             ck(hemm_tensor_batch(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
                                  (uint32_t)lo, dst, started[(size_t)i2] ? 1 : 0, nullptr));
             started[(size_t)i2] = true;
@@ -646,19 +646,23 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     *g_out = g;
 }
 
-// res = rescale(relinearize(acc)) + sum_{i2 >= 1} rho^(g i2 ru)(U_i2), the latter through one hoisted launch
-void bsgsGiantSteps(const HomEvaluator &eval, u64 T, const DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
+// res = sum_i2 rho^(g i2 ru)(U_i2) relinearised and rescaled, all through one hoisted launch: U_i2 (i2 >= 1) gives
+// the terms (d1 under the key of rho(s), d2 under the key of rho(s)^2); U_0 gives its d2 under the multiplication key
+// with the identity automorphism, and its d1 is added to the second polynomial of the sum, times P, before the
+// single ModDown merged with the rescale.
+void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
                     CtxtTensor &res) {
     const Context &c = eval.getContext();
     const u64 N = c->N, K = c->nP, lo = T + 2, uw = 3 * lo * N;
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    eval.relinearize(acc, res.get());
-    eval.rescale(res.get());
-    if (n_giant <= 1) return;
-    const u64 m = (u64)(n_giant - 1), beta = (lo + c->alpha - 1) / c->alpha, El = lo + K;
-    DeviceBuffer ext1(c, m * beta * El * N), ext2(c, m * beta * El * N), pb(c, m * lo * N), wsu(c, m * lo * N);
-    ck(hemm_modup_batch(c->dev, U.data() + lo * N, uw, (uint32_t)lo, (uint32_t)m, ext1.data(), wsu.data(), nullptr));
+    // U holds U_1 .. behind a free first slot: U_0 (the accumulator) moves there so one ModUp batch covers all
+    (void)hipMemcpyAsync(U.data(), acc.buf_.data(), uw * 8, hipMemcpyDeviceToDevice, nullptr);
+    const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K;
+    DeviceBuffer ext1(c, std::max<u64>(1, m - 1) * beta * El * N), ext2(c, m * beta * El * N), pb(c, m * lo * N),
+        wsu(c, m * lo * N), pd1(c, lo * N);
+    if (m > 1)
+        ck(hemm_modup_batch(c->dev, U.data() + uw + lo * N, uw, (uint32_t)lo, (uint32_t)(m - 1), ext1.data(), wsu.data(), nullptr));
     ck(hemm_modup_batch(c->dev, U.data() + 2 * lo * N, uw, (uint32_t)lo, (uint32_t)m, ext2.data(), wsu.data(), nullptr));
     std::vector<u64> sc(lo);
     for (u64 j = 0; j < lo; j++) {
@@ -667,11 +671,21 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, const DeviceBuffer &U, i64 
         sc[j] = P;
     }
     ck(hemm_mul_scalar(c->dev, U.data(), uw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
+    ck(hemm_mul_scalar(c->dev, U.data() + lo * N, uw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
     std::vector<hemm_rot_term> terms;
-    for (u64 i = 0; i < m; i++) {
-        const u64 gal = rot.galois((i64)(i + 1) * g * ru);
+    {
         hemm_rot_term t;
-        t.ext = ext1.data() + i * beta * El * N;
+        t.ext = ext2.data();
+        t.b = pb.data();
+        t.evk = pack.multKey();
+        t.mask = nullptr;
+        t.galois = 1;
+        terms.push_back(t);
+    }
+    for (u64 i = 1; i < m; i++) {
+        const u64 gal = rot.galois((i64)i * g * ru);
+        hemm_rot_term t;
+        t.ext = ext1.data() + (i - 1) * beta * El * N;
         t.b = pb.data() + i * lo * N;
         t.evk = pack.galoisKey(gal);
         t.mask = nullptr;
@@ -683,11 +697,11 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, const DeviceBuffer &U, i64 
         terms.push_back(t);
     }
     const uint32_t off[2] = {0, (uint32_t)terms.size()};
-    Ciphertext giant(c);
-    giant.allocate(2, T, 0);
+    res.get().allocate(2, T, 0);
     DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * (lo - 1) * N);
-    ck(hemm_hoisted_moddown(c->dev, terms.data(), off, 1, (uint32_t)lo, 1, 1, yg.data(), giant.buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
-    eval.add(res.get(), giant, res.get());
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 1, nullptr));
+    ck(hemm_pointwise(c->dev, HEMM_ADD, yg.data() + El * N, 0, pd1.data(), 0, yg.data() + El * N, 0, (uint32_t)lo, 0, 1, nullptr));
+    ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 1, res.get().buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
 }
 }  // namespace
 

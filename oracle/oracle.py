@@ -459,6 +459,20 @@ class Oracle:
                                       _p(out[k, i]), i)
         return out
 
+    def add_residues(self, a, b):
+        """Limb-wise a + b of residue arrays [nq][N] over the chain primes 0 .. nq-1."""
+        return self._binary(0, a, b)
+
+    def mul_p_residues(self, a):
+        """a [nq][N] times P = product of the special primes, limb-wise."""
+        P = 1
+        for p in self.p:
+            P *= p
+        out = np.empty_like(a)
+        for i in range(a.shape[0]):
+            self.L.orc_mul_scalar(self.h, _p(np.ascontiguousarray(a[i])), P % self.mods[i], _p(out[i]), i)
+        return out
+
     def mult_integer(self, x, value):
         return Ct(self.mult_scalar_residues(x, value), x.scale)
 
@@ -596,13 +610,15 @@ class Oracle:
 
     def hoisted_sum(self, terms, nq):
         """terms: (ext, b or None, rotation r (left, in slots) or ('g', galois) or ('sq', galois): the key of
-        rho_g(s)^2, mask Pt over the extended basis or None).
+        rho_g(s)^2, or ('mult', 1): the multiplication key without rotation, mask Pt over the extended basis or None).
         Returns y[2][nq+K][N] = sum mask * (<galois(ext), evk> + P galois(b))."""
         y = np.zeros((2, nq + self.nP, self.N), dtype=np.uint64)
         for i, (ext, b, rot, mask) in enumerate(terms):
             g = rot[1] if isinstance(rot, tuple) else self.galois(rot)
             if isinstance(rot, tuple) and rot[0] == "sq":
                 evk = self.gen_rot_square_key(self.key_seed, g)
+            elif isinstance(rot, tuple) and rot[0] == "mult":      # the multiplication key, identity automorphism
+                evk, g = self.keys["mult"], 1
             else:
                 evk = self.galois_key(g)
             mk = _p(np.ascontiguousarray(mask.data)) if mask is not None else None
