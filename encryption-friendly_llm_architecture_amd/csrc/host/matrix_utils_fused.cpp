@@ -158,8 +158,11 @@ std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots,
     if (n * w != slots && !spread) return fusedRotations(shape, log_slots, packed, true);
     std::vector<u64> r;
     auto left = [&](i64 v) { return (u64)(((v % slots) + slots) % slots); };
-    if (spread)
-        for (i64 blk = n * w; blk < slots; blk <<= 1) r.push_back(left(-blk));
+    if (spread) {   // baby rotations gather the block copies as well
+        const i64 gs = bsgsBabyCount(n);
+        for (i64 i1 = 0; i1 < gs; i1++)
+            for (i64 j = 1; j < slots / (n * w); j++) r.push_back(left(i1 * w - j * n * w));
+    }
     const i64 cu = packed ? 2 : 1, units = n / cu, ru = cu * w, g = bsgsBabyCount(units);
     r.push_back(left(-n));
     for (i64 i = 1; i < units; i++) r.push_back(left(cu * i - g * (i / g) * ru));
@@ -585,9 +588,12 @@ namespace {
 //   its d2 under the multiplication key.
 // units + g + 2 units/g key switches instead of 2 units.
 // sigma_a: [2][T+3][N] at level T+2; tau_b: [2][T+2][N] at level T+1; U_out receives U_1 .. (each [3][T+2][N]).
+// spread_block != 0: tau_b holds one tile block of that many slots and nothing else; every baby rotation then also
+// gathers the copies rho^(-j spread_block), j = 1 .. slots / spread_block - 1, as further terms of its output, which
+// is the rotation of tau(B) copied into every block (row shifts of a periodic vector are exact rotations).
 void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
                       std::vector<Plaintext> &cm, i64 n, i64 units, i64 cu, i64 w, u64 batch, DeviceBuffer *U_out,
-                      i64 *g_out) {
+                      i64 *g_out, u64 spread_block = 0) {
     const Context &c = eval.getContext();
     const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
     const i64 ru = cu * w;
@@ -595,21 +601,30 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     const u64 ctl = 2 * lo * N;   // words of a two-polynomial ciphertext at level T+1
-    // baby rotations of tau(B): bb[i1] = rho^(i1 ru)(tau B)
+    // baby rotations of tau(B): bb[i1] = rho^(i1 ru)(tau B), summed over the block copies when tau(B) is spread
     DeviceBuffer bb(c, (u64)g * ctl);
-    (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, nullptr);
-    if (g > 1) {
+    const i64 copies = spread_block ? (i64)((c->N / 2) / spread_block) : 1;
+    if (g > 1 || copies > 1) {
         const Sources xb = extendSources(c, tau_b, 1, lo);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
-        for (i64 i1 = 1; i1 < g; i1++) {
-            terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(i1 * ru), nullptr));
+        const i64 first_out = copies > 1 ? 0 : 1;   // bb[0] needs a launch only for its copies
+        for (i64 i1 = first_out; i1 < g; i1++) {
+            for (i64 j = 0; j < copies; j++) {
+                if (i1 == 0 && j == 0) continue;     // the unrotated operand itself is added below
+                terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(i1 * ru - j * (i64)spread_block), nullptr));
+            }
             off.push_back((uint32_t)terms.size());
         }
-        DeviceBuffer yb(c, (u64)(g - 1) * 2 * (lo + K) * N), ws(c, (u64)(g - 1) * ctl);
-        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)(g - 1), (uint32_t)lo, 1, 0, yb.data(),
-                                bb.data() + ctl, lo * N, ws.data(), nullptr));
+        const u64 n_out = (u64)(g - first_out);
+        DeviceBuffer yb(c, n_out * 2 * (lo + K) * N), ws(c, n_out * ctl);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_out, (uint32_t)lo, 1, 0, yb.data(),
+                                bb.data() + (u64)first_out * ctl, lo * N, ws.data(), nullptr));
     }
+    if (copies > 1)
+        ck(hemm_pointwise(c->dev, HEMM_ADD, bb.data(), lo * N, tau_b, lo * N, bb.data(), lo * N, (uint32_t)lo, 0, 2, nullptr));
+    else
+        (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, nullptr);
     // column shifts of sigma(A), shift i rotated back by g (i / g) row units
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
@@ -778,22 +793,14 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
     const u64 slots = c->N / 2;
     const bool spread = single_tile && (u64)(n * w) < slots && slots % (u64)(n * w) == 0;
-    if (spread) {
-        // tau(B) (level T+1) copied into every tile block: X += rho^(-block)(X), block doubling each step.  sigma(A)
-        // stays as it is: rotated back by g k2 rows it spills into the empty block below and the giant step
-        // brings it home, so the product comes out in the first block with the other blocks empty.
-        u64 *tb = low.data() + 2 * lo * N;
-        for (u64 blk = (u64)(n * w); blk < slots; blk <<= 1) {
-            const Sources xb = extendSources(c, tb, 1, lo);
-            const i64 back = -(i64)blk;
-            const DeviceBuffer moved = rotateSources(eval, xb, tb, 1, &back);
-            ck(hemm_pointwise(c->dev, HEMM_ADD, tb, lo * N, moved.data(), lo * N, tb, lo * N, (uint32_t)lo, 0, 2, nullptr));
-        }
-    }
+    // spread: tau(B) is copied into every tile block on the fly by the baby rotations (bsgsShiftProduct).  sigma(A)
+    // stays as it is: rotated back by g k2 rows it spills into the empty block below and the giant step brings it
+    // home, so the product comes out in the first block with the other blocks empty.
     if ((u64)(n * w) == slots || spread) {
         DeviceBuffer U;
         i64 g = 1;
-        bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g);
+        bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g,
+                         spread ? (u64)(n * w) : 0);
         bsgsGiantSteps(eval, T, U, g, n / g, w, acc, res);
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;

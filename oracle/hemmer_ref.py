@@ -690,16 +690,26 @@ def _assemble_shifts(orc, src, ext, back, shifts):
     return out
 
 
-def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w):
+def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0):
     """Baby-step / giant-step sum over the shift index i = i1 + g i2 (column shift cu * i slots, row rotation
-    i * cu * w slots); `acc` holds the i = 0 term, a = sigma(A) at T+2, b_low = tau(B) at T+1."""
+    i * cu * w slots); `acc` holds the i = 0 term, a = sigma(A) at T+2, b_low = tau(B) at T+1.
+    spread_block: tau(B) holds one tile block of that many slots and nothing else; every baby rotation then
+    also gathers the copies rho^(-j spread_block) (further terms of the same hoisted sum), i.e. it is the
+    rotation of tau(B) copied into every block."""
     from .oracle import Ct
     ru = cu * w
     g = bsgs_baby_count(units)
     ext_a, ext_b = orc.modup(a.data[1]), orc.modup(b_low.data[1])
-    bb = [b_low] + [Ct(orc.moddown_drop(orc.hoisted_sum([(ext_b, b_low.data[0], (i1 * ru) % orc.slots, None)],
-                                                        b_low.nq), b_low.nq, False), b_low.scale)
-                    for i1 in range(1, g)]
+    copies = orc.slots // spread_block if spread_block else 1
+    bb = []
+    for i1 in range(g):
+        terms = [(ext_b, b_low.data[0], (i1 * ru - j * spread_block) % orc.slots, None)
+                 for j in range(copies) if not (i1 == 0 and j == 0)]
+        if not terms:
+            bb.append(b_low)
+            continue
+        moved = Ct(orc.moddown_drop(orc.hoisted_sum(terms, b_low.nq), b_low.nq, False), b_low.scale)
+        bb.append(orc.add(moved, b_low) if i1 == 0 else moved)
     ta = _assemble_shifts(orc, a, ext_a, -n,
                           [((cu * i - g * (i // g) * ru) % orc.slots, cm[2 * cu * i + 1], cm[2 * cu * i])
                            for i in range(1, units)])
@@ -722,8 +732,8 @@ def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w):
 
 
 def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
-    """single_tile: both operands hold one tile block and nothing else; tau(B) is then copied into every
-    block (X += rho^(-block)(X), block doubling), which makes its row shifts exact rotations."""
+    """single_tile: both operands hold one tile block and nothing else; tau(B) is then taken as copied into
+    every block (the copies are gathered by the baby rotations), which makes its row shifts exact rotations."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
@@ -735,11 +745,6 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     acc = orc.tensor(orc.level_down_one(a), b_low)
     ext_a = orc.modup(a.data[1])
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
-    if spread:
-        blk = n * w
-        while blk < orc.slots:
-            b_low = orc.add(b_low, orc.rotate_hoisted(b_low, -blk))
-            blk <<= 1
     if n * w == orc.slots or spread:
         # The tile block fills the slot vector: row shifts are exact rotations rho^(k w) of tau(B) lowered to
         # T+1 (no mask, plain ModDown), which allows the baby-step / giant-step split k = k1 + g k2:
@@ -747,7 +752,7 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
         # The column shifts come out already rotated back by g k2 rows (another Galois element, same masks);
         # the un-relinearised U_k2 are rotated directly: d1 with the key of rho(s), d2 with a key of
         # rho(s)^2, all summed in the extended basis before one ModDown merged with the rescale.
-        return _bsgs_shift_product(orc, a, b_low, acc, cm, n, n, 1, w)
+        return _bsgs_shift_product(orc, a, b_low, acc, cm, n, n, 1, w, n * w if spread else 0)
     else:
         ta = _assemble_shifts(orc, a, ext_a, -n, [(i, cm[2 * i + 1], cm[2 * i]) for i in range(1, n)])
         rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
