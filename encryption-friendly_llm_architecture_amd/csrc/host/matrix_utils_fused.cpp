@@ -466,7 +466,7 @@ Message twoStageMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log
             const i64 sel = vertical ? Cc : Rc, pos = vertical ? Rc : Cc;
             bool on = stage == 1 ? (sel % b == r) : (sel / b == r);
             if (part == 1) on = on && pos < u - amount;
-            if (part == 2) on = on && pos >= u - amount;
+            if (part == 2) on = on && pos >= u - amount;   // part 3: both together (extended basis)
             if (on) m[(u64)(row * w + col)] = value;
         }
     return m;
@@ -490,9 +490,14 @@ std::vector<u64> MatrixTransformer::twoStageRotations(MaskKind kind, const TileT
     const i64 wrap = g.n * (vertical ? shape.getBlockWidth() : 1);
     std::vector<u64> r;
     auto left = [&](i64 v) { r.push_back((u64)(((v % slots) + slots) % slots)); };
-    left(-wrap);
-    for (i64 i = 1; i < b; i++) left(i * g.step);
-    for (i64 i = 1; i < g.units / b; i++) left(i * b * g.step);
+    for (i64 i = 1; i < b; i++) {
+        left(i * g.step);
+        left(i * g.step - wrap);
+    }
+    for (i64 i = 1; i < g.units / b; i++) {
+        left(i * b * g.step);
+        left(i * b * g.step - wrap);
+    }
     return r;
 }
 
@@ -520,33 +525,37 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         const u64 lvl = stage == 1 ? level : level - 1, nq = lvl + 1, E = nq + c->nP, ctw = 2 * nq * N;
         const u64 *src = stage == 1 ? in : mid.data();
         u64 *dst = stage == 1 ? mid.data() : out;
-        // rotation sources: X and X' = rho^(-one tile side)(X)
+        // One rotation source per job (a single ModUp).  A stage's rotation by r cells wraps inside the tile, so it is
+        //   main_r * rho^(r step)(X) + wrap_r * rho^(r step - tile side)(X):
+        // two Galois elements per r with one key each; when they coincide (the tile side is a whole turn of the slot
+        // vector) one term with the mask of both parts.
         const Sources x = extendSources(c, src, n_jobs, nq);
-        std::vector<i64> back(n_jobs);
-        std::vector<Geo> g;
-        for (size_t q = 0; q < n_jobs; q++) {
-            g.push_back(geo(kinds[q], shapes[q]));
-            const bool vertical = (kinds[q] == MaskKind::Vertical || kinds[q] == MaskKind::PackedVertical);
-            back[q] = -g[q].n * (vertical ? shapes[q].getBlockWidth() : 1);
-        }
-        const DeviceBuffer src2 = rotateSources(eval, x, src, n_jobs, back.data());
-        const Sources x2 = extendSources(c, src2.data(), n_jobs, nq);
-        // one output per job: sum over the stage's rotations of main_r rot(X) + wrap_r rot(X')
+        const KeyPack &pack = eval.getKeyPack();
+        const Rot rot(c);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         std::vector<hemm_lin_term> zero_terms;
         std::vector<uint32_t> zoff{0};
         bool any_rotation = false;
         for (size_t q = 0; q < n_jobs; q++) {
-            const i64 b = twoStageSplit(g[q].units), count = stage == 1 ? b : g[q].units / b, mul = stage == 1 ? 1 : b;
-            std::vector<Shift> sh;
-            std::vector<const Plaintext *> keep;
-            for (i64 r = 1; r < count; r++)
-                sh.push_back(Shift{r * mul * g[q].step, &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 1),
-                                   &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)});
-            pushShiftGroup(eval, x, q, x2, q, sh, terms);
+            const Geo g = geo(kinds[q], shapes[q]);
+            const bool vertical = (kinds[q] == MaskKind::Vertical || kinds[q] == MaskKind::PackedVertical);
+            const i64 wrap = g.n * (vertical ? shapes[q].getBlockWidth() : 1);
+            const i64 b = twoStageSplit(g.units), count = stage == 1 ? b : g.units / b, mul = stage == 1 ? 1 : b;
+            for (i64 r = 1; r < count; r++) {
+                const i64 amount = r * mul * g.step;
+                if (rot.norm(amount) == rot.norm(amount - wrap)) {
+                    terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount),
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 3)));
+                } else {
+                    terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount),
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 1)));
+                    terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount - wrap),
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)));
+                }
+                any_rotation = true;
+            }
             off.push_back((uint32_t)terms.size());
-            any_rotation = any_rotation || !sh.empty();
             hemm_lin_term t;
             t.ct = src + q * ctw;
             t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();

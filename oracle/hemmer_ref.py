@@ -608,7 +608,7 @@ def two_stage_split(units):
 def two_stage_mask(kind, n, w, slots, stage, r, part):
     """Masks of the two-stage sigma / tau: stage 1 selects the rows (sigma) / columns (tau) whose cell index
     is r mod b, stage 2 those whose cell index div b is r; part 0: all of them, 1: the positions that do
-    not wrap under the stage's rotation (r cells, or r b cells), 2: those that do."""
+    not wrap under the stage's rotation (r cells, or r b cells), 2: those that do, 3: both."""
     cell = 2 if kind in (PH, PV) else 1
     u = n // cell
     b = two_stage_split(u)
@@ -626,9 +626,9 @@ def two_stage_mask(kind, n, w, slots, stage, r, part):
 
 def diagonal_transform_two_stage(orc, ct, kind, n, w):
     """sigma / tau (square tiles) in two stages of one mask level each: row i is rotated by i mod b, then
-    by b (i div b).  Every stage: X' = rho^(-tile side)(X); one hoisted sum over the stage's rotations of
-    main_r rot(X) + wrap_r rot(X') with ModDown merged with the rescale, plus rescale(mask_0 X) for the
-    rows that stay.  Level L -> L - 2."""
+    by b (i div b).  Every stage is one hoisted sum over its rotations of
+    main_r rho^(r)(X) + wrap_r rho^(r - tile side)(X) (two keys per r, one source) with ModDown merged with
+    the rescale, plus rescale(mask_0 X) for the rows that stay.  Level L -> L - 2."""
     from .oracle import Ct
     cell = 2 if kind in (PH, PV) else 1
     u = n // cell
@@ -639,15 +639,17 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
     for stage, count, mul in ((1, b, 1), (2, u // b, b)):
         nq = x.nq
         ext = orc.modup(x.data[1])
-        x2 = _rotated_copy(orc, x, ext, -wrap)
-        ext2 = orc.modup(x2.data[1])
         zero = orc.rescale(orc.mult_plain_no_rescale(
             x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), x.level)))
+        mask = lambda r, part: orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, part), x.level)
         terms = []
         for r in range(1, count):
-            rr = (r * mul * step) % orc.slots
-            terms.append((ext, x.data[0], rr, orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, 1), x.level)))
-            terms.append((ext2, x2.data[0], rr, orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, 2), x.level)))
+            r_main, r_wrap = (r * mul * step) % orc.slots, (r * mul * step - wrap) % orc.slots
+            if r_main == r_wrap:        # the tile side is a whole turn: one term with both parts of the mask
+                terms.append((ext, x.data[0], r_main, mask(r, 3)))
+            else:
+                terms.append((ext, x.data[0], r_main, mask(r, 1)))
+                terms.append((ext, x.data[0], r_wrap, mask(r, 2)))
         if terms:
             y = orc.hoisted_sum(terms, nq)
             x = orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
