@@ -323,11 +323,12 @@ struct RotDev {
     u32 galois, pad;
     const u64 *ext2, *b2, *mask2;
 };
-static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,
-                             uint32_t n_out, hipStream_t stream, void **terms_dev, void **off_dev) {
+static_assert(sizeof(RotDev) == 64, "RotDev must match the kernels' RotTermDev");
+static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                            std::vector<RotDev> &d, std::vector<uint32_t> &off) {
     const uint32_t n_terms = group_offsets[n_out];
-    std::vector<RotDev> d;
-    std::vector<uint32_t> off{0};
+    d.clear();
+    off.assign(1, 0);
     d.reserve(n_terms);
     for (uint32_t o = 0; o < n_out; o++) {
         need(group_offsets[o + 1] >= group_offsets[o], "group offsets must not decrease");
@@ -347,8 +348,22 @@ static void upload_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, cons
         }
         off.push_back((uint32_t)d.size());
     }
-    *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t), off_dev,
-                             stream);
+}
+// hoisted sums of a validated, merged term list: short lists travel in the kernel arguments, long ones through the
+// staging region
+static void run_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
+                              uint32_t nq, u64 *y, bool b_premultiplied, hipStream_t stream) {
+    std::vector<RotDev> d;
+    std::vector<uint32_t> off;
+    build_rot_terms(ctx, terms, group_offsets, n_out, d, off);
+    if ((int)d.size() <= hoisted_arg_capacity() && (int)n_out <= hoisted_arg_capacity()) {
+        launch_hoisted_terms_args(ctx, d.data(), (int)d.size(), off.data(), (int)n_out, (int)nq, y, b_premultiplied, stream);
+        return;
+    }
+    void *off_dev = nullptr;
+    void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t),
+                                  &off_dev, stream);
+    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, y, b_premultiplied, stream);
 }
 
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
@@ -358,10 +373,7 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     chain_limbs(ctx, nq, 1, &nl);
     need(terms && group_offsets && y && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    void *terms_dev = nullptr, *off_dev = nullptr;
-    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev);
-    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y, b_premultiplied != 0,
-                         (hipStream_t)stream);
+    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y, b_premultiplied != 0, (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }
@@ -374,10 +386,7 @@ int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const ui
     chain_limbs(ctx, nq, 1, &nl);
     need(terms && group_offsets && y_workspace && out && workspace && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    void *terms_dev = nullptr, *off_dev = nullptr;
-    upload_rot_terms(ctx, terms, group_offsets, n_out, (hipStream_t)stream, &terms_dev, &off_dev);
-    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (u64 *)y_workspace,
-                         b_premultiplied != 0, (hipStream_t)stream);
+    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y_workspace, b_premultiplied != 0, (hipStream_t)stream);
     launch_moddown_batch(ctx, (u64 *)y_workspace, (int)nq, (int)(2 * n_out), drop_last != 0, (u64 *)out, out_stride,
                          (u64 *)workspace, (hipStream_t)stream);
     check_launch();

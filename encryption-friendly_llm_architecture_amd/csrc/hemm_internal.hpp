@@ -90,6 +90,9 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
                         hipStream_t s);
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
                           bool b_premultiplied, hipStream_t s);
+int hoisted_arg_capacity();
+void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
+                               int nq, u64 *y, bool b_premultiplied, hipStream_t s);
 void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
                           u64 *conv, hipStream_t s);
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,

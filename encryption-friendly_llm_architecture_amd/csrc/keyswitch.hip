@@ -166,11 +166,11 @@ u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
-__global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__restrict__ terms,
-                                                            const u32 *__restrict__ group_off, u64 *__restrict__ y,
-                                                            const ModQ *__restrict__ modq, const double *__restrict__ fp,
-                                                            LimbList ll, CstList pmod, int nq, int E, int beta,
-                                                            int n_full, int logN, int b_premultiplied, int n_out) {
+__device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict__ terms,
+                                                   const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                   const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                   const LimbList &ll, const CstList &pmod, int nq, int E, int beta,
+                                                   int n_full, int logN, int b_premultiplied, int n_out) {
     // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
     // (possibly swapped), so every access is a 16-byte load or store.
     // Work is dealt out by SOURCE chunk.  The automorphism maps aligned 512-coefficient chunks onto aligned
@@ -224,6 +224,29 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const RotTermDev *__
     }
     stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, rb[0], rb[1]);
     stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, ra[0], ra[1]);
+}
+
+// Term lists of up to HOISTED_ARG_TERMS terms and outputs travel in the kernel arguments (no staging copy before
+// the launch); longer lists are read from device memory.
+static_assert(sizeof(RotTermDev) == 64, "the C ABI builds these records on the host");
+#define HOISTED_ARG_TERMS 32
+struct HoistedArgs {
+    RotTermDev t[HOISTED_ARG_TERMS];
+    u32 off[HOISTED_ARG_TERMS + 1];
+};
+__global__ __launch_bounds__(256) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
+                                                            const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                            LimbList ll, CstList pmod, int nq, int E, int beta,
+                                                            int n_full, int logN, int b_premultiplied, int n_out) {
+    hoisted_terms_body(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out);
+}
+__global__ __launch_bounds__(256) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
+                                                                 const u32 *__restrict__ group_off, u64 *__restrict__ y,
+                                                                 const ModQ *__restrict__ modq,
+                                                                 const double *__restrict__ fp, LimbList ll, CstList pmod,
+                                                                 int nq, int E, int beta, int n_full, int logN,
+                                                                 int b_premultiplied, int n_out) {
+    hoisted_terms_body(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out);
 }
 
 struct LinTermDev {
@@ -753,9 +776,26 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
     dim3 grid((unsigned)((size_t)n_out * E * (c->N / 512))), block(256);
-    hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
+    hipLaunchKernelGGL(hoisted_terms_list_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
                        c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
                        b_premultiplied ? 1 : 0, n_out);
+}
+// the same with the term list (host memory, already merged: n_terms <= HOISTED_ARG_TERMS, n_out <= HOISTED_ARG_TERMS)
+// passed in the kernel arguments
+int hoisted_arg_capacity() { return HOISTED_ARG_TERMS; }
+void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
+                               int nq, u64 *y, bool b_premultiplied, hipStream_t s) {
+    const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+    const CstList pm = p_mod_chain(c, nq);
+    if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
+    if (n_terms > HOISTED_ARG_TERMS || n_out > HOISTED_ARG_TERMS) throw std::invalid_argument("term list too long for the argument path");
+    HoistedArgs a;
+    memset(&a, 0, sizeof(a));
+    memcpy(a.t, terms_host, (size_t)n_terms * sizeof(RotTermDev));
+    memcpy(a.off, group_off_host, (size_t)(n_out + 1) * sizeof(u32));
+    dim3 grid((unsigned)((size_t)n_out * E * (c->N / 512))), block(256);
+    hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, a, y, c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E,
+                       beta, c->nQ + c->nP, c->logN, b_premultiplied ? 1 : 0, n_out);
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;
