@@ -429,12 +429,17 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
 
 int hemm_tensor_batch(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
                       uint64_t *acc3, int accumulate, void *stream) {
+    return hemm_tensor_batch_strided(ctx, t1, t2, n_pairs, nq, acc3, (size_t)nq * (size_t)ctx->N, accumulate, stream);
+}
+int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
+                              uint64_t *acc3, size_t acc_stride, int accumulate, void *stream) {
     HEMM_TRY
     int nl;
     chain_limbs(ctx, nq, 0, &nl);
     need(t1 && t2 && acc3 && n_pairs >= 1, "null operand");
-    launch_tensor_batch(ctx, (const u64 *)t1, (const u64 *)t2, (int)n_pairs, (int)nq, (u64 *)acc3, accumulate != 0,
-                        (hipStream_t)stream);
+    need(acc_stride >= (size_t)nq * (size_t)ctx->N, "accumulator stride below one polynomial");
+    launch_tensor_batch(ctx, (const u64 *)t1, (const u64 *)t2, (int)n_pairs, (int)nq, (u64 *)acc3, acc_stride,
+                        accumulate != 0, (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

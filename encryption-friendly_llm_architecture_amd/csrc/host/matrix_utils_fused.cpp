@@ -642,9 +642,12 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     const i64 back = -n;
     const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back);
     const Sources xa2 = extendSources(c, a2.data(), 1, nq);
-    // U[i2]: [3][lo][N] for i2 >= 1 (slot 0 is left for U_0, which is accumulated in `acc`)
-    const u64 uw = 3 * lo * N;
-    U_out->resize(c, (u64)n_giant * uw);
+    // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
+    // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
+    const u64 pw = lo * N, us = (u64)n_giant * pw;
+    U_out->resize(c, 3 * us);
+    for (u64 p = 0; p < 3; p++)
+        (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, nullptr);
     std::vector<bool> started((size_t)n_giant, false);
     started[0] = true;
     const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
@@ -660,9 +663,9 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         while (q < first + cnt) {
             const i64 ii = (i64)q + 1, i2 = ii / g, i1 = ii % g;
             const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - i1));
-            u64 *dst = i2 == 0 ? acc.buf_.data() : U_out->data() + (u64)i2 * uw;
-            ck(hemm_tensor_batch(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
-                                 (uint32_t)lo, dst, started[(size_t)i2] ? 1 : 0, nullptr));
+            ck(hemm_tensor_batch_strided(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
+                                         (uint32_t)lo, U_out->data() + (u64)i2 * pw, us, started[(size_t)i2] ? 1 : 0,
+                                         nullptr));
             started[(size_t)i2] = true;
             q += run;
         }
@@ -677,29 +680,28 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
 void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
                     CtxtTensor &res) {
     const Context &c = eval.getContext();
-    const u64 N = c->N, K = c->nP, lo = T + 2, uw = 3 * lo * N;
+    const u64 N = c->N, K = c->nP, lo = T + 2;
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    // U holds U_1 .. behind a free first slot: U_0 (the accumulator) moves there so one ModUp batch covers all
-    (void)hipMemcpyAsync(U.data(), acc.buf_.data(), uw * 8, hipMemcpyDeviceToDevice, nullptr);
-    const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K;
-    DeviceBuffer ext1(c, std::max<u64>(1, m - 1) * beta * El * N), ext2(c, m * beta * El * N), pb(c, m * lo * N),
-        wsu(c, m * lo * N), pd1(c, lo * N);
-    if (m > 1)
-        ck(hemm_modup_batch(c->dev, U.data() + uw + lo * N, uw, (uint32_t)lo, (uint32_t)(m - 1), ext1.data(), wsu.data(), nullptr));
-    ck(hemm_modup_batch(c->dev, U.data() + 2 * lo * N, uw, (uint32_t)lo, (uint32_t)m, ext2.data(), wsu.data(), nullptr));
+    // U is polynomial-major ([3][n_giant][lo][N]): d1 and d2 of all partial sums are 2 n_giant polynomials in a row,
+    // extended by ONE ModUp batch (d1 of U_0 rides along unused)
+    (void)acc;
+    const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K, pw = lo * N, us = m * pw;
+    DeviceBuffer ext(c, 2 * m * beta * El * N), pb(c, m * lo * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
+    ck(hemm_modup_batch(c->dev, U.data() + us, pw, (uint32_t)lo, (uint32_t)(2 * m), ext.data(), wsu.data(), nullptr));
+    const u64 *ext1 = ext.data(), *ext2 = ext.data() + m * beta * El * N;   // [i2][beta][El][N] each
     std::vector<u64> sc(lo);
     for (u64 j = 0; j < lo; j++) {
         u64 P = 1;
         for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
         sc[j] = P;
     }
-    ck(hemm_mul_scalar(c->dev, U.data(), uw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
-    ck(hemm_mul_scalar(c->dev, U.data() + lo * N, uw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
+    ck(hemm_mul_scalar(c->dev, U.data(), pw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
+    ck(hemm_mul_scalar(c->dev, U.data() + us, pw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
     std::vector<hemm_rot_term> terms;
     {
         hemm_rot_term t;
-        t.ext = ext2.data();
+        t.ext = ext2;
         t.b = pb.data();
         t.evk = pack.multKey();
         t.mask = nullptr;
@@ -709,13 +711,13 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     for (u64 i = 1; i < m; i++) {
         const u64 gal = rot.galois((i64)i * g * ru);
         hemm_rot_term t;
-        t.ext = ext1.data() + (i - 1) * beta * El * N;
+        t.ext = ext1 + i * beta * El * N;
         t.b = pb.data() + i * lo * N;
         t.evk = pack.galoisKey(gal);
         t.mask = nullptr;
         t.galois = gal;
         terms.push_back(t);
-        t.ext = ext2.data() + i * beta * El * N;
+        t.ext = ext2 + i * beta * El * N;
         t.b = nullptr;
         t.evk = pack.galoisSquareKey(gal);
         terms.push_back(t);

@@ -384,8 +384,9 @@ __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__res
 
 // acc3 (+)= sum_{g < G} (b1 b2, a1 b2 + a2 b1, a1 a2) of t1[g], t2[g], each [2][nq][N]
 __global__ __launch_bounds__(256) void tensor_batch_kernel(const u64 *__restrict__ t1, const u64 *__restrict__ t2,
-                                                           int G, u64 *__restrict__ acc3, int accumulate,
-                                                           const ModQ *__restrict__ modq, int nq, int logN) {
+                                                           int G, u64 *__restrict__ acc3, size_t acc_stride,
+                                                           int accumulate, const ModQ *__restrict__ modq, int nq,
+                                                           int logN) {
     const int j = blockIdx.y;
     const ModQ m = modq[j];
     const size_t N = (size_t)1 << logN, P = (size_t)nq * N;
@@ -393,8 +394,8 @@ __global__ __launch_bounds__(256) void tensor_batch_kernel(const u64 *__restrict
     u64 d0 = 0, d1 = 0, d2 = 0;
     if (accumulate) {
         d0 = acc3[e];
-        d1 = acc3[P + e];
-        d2 = acc3[2 * P + e];
+        d1 = acc3[acc_stride + e];
+        d2 = acc3[2 * acc_stride + e];
     }
     for (int g = 0; g < G; g++) {
         const u64 b1 = t1[(size_t)g * 2 * P + e], a1 = t1[(size_t)g * 2 * P + P + e];
@@ -406,8 +407,8 @@ __global__ __launch_bounds__(256) void tensor_batch_kernel(const u64 *__restrict
         d2 = addmod(d2, mulmod(a1, a2, m), m.q);
     }
     acc3[e] = d0;
-    acc3[P + e] = d1;
-    acc3[2 * P + e] = d2;
+    acc3[acc_stride + e] = d1;
+    acc3[2 * acc_stride + e] = d2;
 }
 
 }  // namespace
@@ -872,9 +873,9 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
                            n_out);
 }
 
-void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, bool accumulate,
-                         hipStream_t s) {
+void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
+                         bool accumulate, hipStream_t s) {
     dim3 grid(c->N / 256, nq), block(256);
-    hipLaunchKernelGGL(tensor_batch_kernel, grid, block, 0, s, t1, t2, G, acc3, accumulate ? 1 : 0, c->d_modq, nq,
-                       c->logN);
+    hipLaunchKernelGGL(tensor_batch_kernel, grid, block, 0, s, t1, t2, G, acc3, acc_stride, accumulate ? 1 : 0, c->d_modq,
+                       nq, c->logN);
 }

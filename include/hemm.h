@@ -162,6 +162,10 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
 /* acc3 [3][nq][N] (+)= sum_g tensor(t1[g], t2[g]); t1, t2: [n_pairs][2][nq][N] */
 int hemm_tensor_batch(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
                       uint64_t *acc3, int accumulate, void *stream);
+/* the same with the three polynomials of the accumulator acc_stride words apart (several accumulators can then be
+ * kept polynomial-major, [3][count][nq][N], so that one hemm_modup_batch covers a polynomial of all of them) */
+int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
+                              uint64_t *acc3, size_t acc_stride, int accumulate, void *stream);
 
 /* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last */
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
