@@ -13,10 +13,6 @@
 #include "hemm_internal.hpp"
 #include "hoisted.cuh"
 
-void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
-                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s);
-bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
-                          size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 
 namespace {
 
@@ -94,6 +90,61 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
         }
         *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
     }
+}
+
+// All digits of a ModUp in one launch (blockIdx.z = digit): the conversion of every digit to the limbs it does not
+// own, plus the copy of its own limbs (already in NTT form in `own`) into its slice of the extended polynomial.
+#define BCONV_MAX_DIGITS 4
+struct BConvDigits {
+    BConvArgs d[BCONV_MAX_DIGITS];
+    const u64 *own;        // [n_polys][.][N] NTT form, polynomial stride own_stride
+    size_t own_stride;
+    uint8_t own_lo[BCONV_MAX_DIGITS], own_hi[BCONV_MAX_DIGITS];
+};
+template <int NS>
+__global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const ModQ *__restrict__ modq) {
+    const BConvArgs &a = g.d[blockIdx.z];
+    const int poly = blockIdx.y;
+    const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const u64 *src = a.src + poly * a.src_poly_stride;
+    u64 *dst = a.dst + poly * a.dst_poly_stride;
+    u64 v0[NS], v1[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        v0[i] = v1[i] = 0;
+        if (i < a.n_src) {
+            const u64 q = modq[a.src_prime[i]].q;
+            const Cst c = a.inv[i];
+            const ulonglong2 x = *(const ulonglong2 *)(src + ((size_t)a.src_slot[i] << a.logN) + n);
+            v0[i] = mul_shoup(x.x, c.w, c.ws, q);
+            v1[i] = mul_shoup(x.y, c.w, c.ws, q);
+        }
+    }
+    for (int j = 0; j < a.n_dst; j++) {
+        const int pj = a.dst_prime[j];
+        const u64 q = modq[pj].q;
+        u64 acc0 = 0, acc1 = 0;
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            if (i < a.n_src) {
+                const Cst c = a.hat[i * a.hat_ld + pj];
+                acc0 += mul_shoup_lazy(v0[i], c.w, c.ws, q);
+                acc1 += mul_shoup_lazy(v1[i], c.w, c.ws, q);
+            }
+            if (i % 3 == 2 || i == NS - 1) {
+                if (acc0 >= 4 * q) acc0 -= 4 * q;
+                if (acc1 >= 4 * q) acc1 -= 4 * q;
+                if (acc0 >= 2 * q) acc0 -= 2 * q;
+                if (acc1 >= 2 * q) acc1 -= 2 * q;
+                if (acc0 >= q) acc0 -= q;
+                if (acc1 >= q) acc1 -= q;
+            }
+        }
+        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
+    }
+    const u64 *own = g.own + poly * g.own_stride;
+    for (int j = g.own_lo[blockIdx.z]; j < g.own_hi[blockIdx.z]; j++)
+        *(ulonglong2 *)(dst + ((size_t)j << a.logN) + n) = *(const ulonglong2 *)(own + ((size_t)j << a.logN) + n);
 }
 
 // grid = (N / 256, n_polys) coefficients x polynomials
@@ -689,13 +740,16 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
     u64 *sc = hemm_scratch(c);
     u64 *last = sc;                               // [n_polys][N]
     u64 *tt = sc + (size_t)n_polys * N;           // [n_polys][nq-1][N]
-    for (int p = 0; p < n_polys; p++)
-        HEMM_HIP(hipMemcpyAsync(last + (size_t)p * N, in + p * in_stride + (size_t)(nq - 1) * N, N * 8,
-                                hipMemcpyDeviceToDevice, s));
-    LimbList pl;
+    LimbList pl, ident;
     memset(&pl, 0, sizeof(pl));
     pl.idx[0] = (uint8_t)(nq - 1);
-    launch_ntt(c, last, pl, 1, n_polys, N, true, s);
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) ident.idx[j] = (uint8_t)j;
+    if (!launch_intt_from(c, in + (size_t)(nq - 1) * N, in_stride, last, pl, ident, 1, n_polys, N, s)) {
+        for (int p = 0; p < n_polys; p++)
+            HEMM_HIP(hipMemcpyAsync(last + (size_t)p * N, in + p * in_stride + (size_t)(nq - 1) * N, N * 8,
+                                    hipMemcpyDeviceToDevice, s));
+        launch_ntt(c, last, pl, 1, n_polys, N, true, s);
+    }
     dim3 grid(N / 256, (nq - 1) * n_polys), block(256);
     hipLaunchKernelGGL(spread_kernel, grid, block, 0, s, last, tt, (size_t)(nq - 1) * N, c->d_modq, nq - 1, c->logN);
     if (launch_ntt_sub_scale(c, tt, nq - 1, n_polys, in, in_stride, out, out_stride, t->dev + t->qlinv_off[nq - 1], s))
@@ -715,9 +769,27 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     KsTables *t = g_tables_of(c);
     const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
     const size_t N = c->N;
-    HEMM_HIP(hipMemcpy2DAsync(coef, (size_t)nq * N * 8, in, in_stride * 8, (size_t)nq * N * 8, n_in,
-                              hipMemcpyDeviceToDevice, s));
-    launch_ntt(c, coef, limbs_default(c, nq, 0), nq, n_in, (size_t)nq * N, true, s);
+    if (alpha > 32) throw std::invalid_argument("digit wider than 32 limbs");
+    const LimbList chain = limbs_default(c, nq, 0);
+    LimbList ident;
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) ident.idx[j] = (uint8_t)j;
+    if (!launch_intt_from(c, in, in_stride, coef, chain, ident, nq, n_in, (size_t)nq * N, s)) {
+        HEMM_HIP(hipMemcpy2DAsync(coef, (size_t)nq * N * 8, in, in_stride * 8, (size_t)nq * N * 8, n_in,
+                                  hipMemcpyDeviceToDevice, s));
+        launch_ntt(c, coef, chain, nq, n_in, (size_t)nq * N, true, s);
+    }
+    // One conversion launch and one forward transform for all digits when the ring size allows: the converted
+    // limbs of every digit are addressed as slots d*E + j of one extended polynomial per input.
+    const bool joint = c->N >= 512 && alpha <= 8 && beta <= BCONV_MAX_DIGITS && beta * E <= 255 &&
+                       beta * E - nq <= HEMM_MAX_PRIMES;
+    BConvDigits g;
+    memset(&g, 0, sizeof(g));
+    g.own = in;
+    g.own_stride = in_stride;
+    LimbList jp, js;
+    memset(&jp, 0, sizeof(jp));
+    memset(&js, 0, sizeof(js));
+    int n_joint = 0;
     for (int d = 0; d < beta; d++) {
         const int lo = d * alpha, hi = std::min(nq, lo + alpha);
         BConvArgs a;
@@ -731,7 +803,6 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         a.n_src = hi - lo;
         a.hat_ld = c->nQ + c->nP;
         a.logN = c->logN;
-        if (a.n_src > 32) throw std::invalid_argument("digit wider than 32 limbs");
         LimbList pl, sl;
         memset(&pl, 0, sizeof(pl));
         memset(&sl, 0, sizeof(sl));
@@ -746,9 +817,20 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
             a.dst_prime[nd] = (uint8_t)(j < nq ? j : c->nQ + (j - nq));
             pl.idx[nd] = a.dst_prime[nd];
             sl.idx[nd] = (uint8_t)j;
+            if (joint) {
+                jp.idx[n_joint] = a.dst_prime[nd];
+                js.idx[n_joint] = (uint8_t)(d * E + j);
+                n_joint++;
+            }
             nd++;
         }
         a.n_dst = nd;
+        if (joint) {
+            g.d[d] = a;
+            g.own_lo[d] = (uint8_t)lo;
+            g.own_hi[d] = (uint8_t)hi;
+            continue;
+        }
         if (nd > 0) {
             launch_bconv(a, c->d_modq, (int)N, n_in, s);
             launch_ntt_slots(c, a.dst, pl, sl, nd, n_in, (size_t)beta * E * N, false, s);
@@ -756,6 +838,16 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         HEMM_HIP(hipMemcpy2DAsync(a.dst + (size_t)lo * N, (size_t)beta * E * N * 8, in + (size_t)lo * N, in_stride * 8,
                                   (size_t)(hi - lo) * N * 8, n_in, hipMemcpyDeviceToDevice, s));
     }
+    if (!joint) return;
+    const dim3 grid((unsigned)(N / 512), n_in, beta), block(256);
+    const int widest = std::min(nq, alpha);
+    if (widest <= 2)
+        hipLaunchKernelGGL(bconv_digits_kernel<2>, grid, block, 0, s, g, c->d_modq);
+    else if (widest <= 5)
+        hipLaunchKernelGGL(bconv_digits_kernel<5>, grid, block, 0, s, g, c->d_modq);
+    else
+        hipLaunchKernelGGL(bconv_digits_kernel<8>, grid, block, 0, s, g, c->d_modq);
+    launch_ntt_slots(c, ext, jp, js, n_joint, n_in, (size_t)beta * E * N, false, s);
 }
 
 // terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]

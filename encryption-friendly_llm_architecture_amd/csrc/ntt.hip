@@ -333,12 +333,14 @@ struct NttEpilogue {
     const Tw *cst;  // per limb: constant and Shoup quotient
     size_t minuend_stride, out_stride;
 };
+// An inverse transform may read its input elsewhere (same slot numbering, own polynomial stride) and leave the
+// result in `data`: the first pass then loads from `minuend` (stride `minuend_stride`) instead of `data`.
 
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
 template <bool INV, bool EPI, class F>
 __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw,
                                           const u32 r, const u64 q, const u64 *__restrict__ mn, u64 *__restrict__ o,
-                                          const Tw cst) {
+                                          const Tw cst, const u64 *__restrict__ ld) {
     typedef typename F::E E;
     const typename F::W *tw = (const typename F::W *)tw_int;
     const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
@@ -369,7 +371,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
         }
     } else {
 #pragma unroll
-        for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = row[c + 16 * k];
+        for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = ld[c + 16 * k];
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = f.from_canonical(lc[padc(16 * c + k)]);
@@ -416,10 +418,13 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
         cst = ep.cst[limb];
     }
     const u64 q = modq[prime].q;
+    const u64 *ld = row;
+    if (INV && ep.minuend != nullptr)
+        ld = ep.minuend + (size_t)poly * ep.minuend_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     if (fp[4 * prime] != 0.0)
-        rows_body<INV, EPI>(row, tw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst);
+        rows_body<INV, EPI>(row, tw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
     else
-        rows_body<INV, EPI>(row, tw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst);
+        rows_body<INV, EPI>(row, tw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
 }
 
 }  // namespace
@@ -442,6 +447,23 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
     (void)none;
     hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl, n_limbs,
                        poly_stride, ep);
+    return true;
+}
+
+bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
+                      const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s) {
+    if (c->logN != 16) return false;
+    if (n_limbs <= 0 || n_polys <= 0) return true;
+    const Tw *tw = (const Tw *)c->d_iw;
+    const int lanes = n_limbs * n_polys;
+    dim3 grid(16, lanes), block(256);
+    NttEpilogue from{};
+    from.minuend = src;
+    from.minuend_stride = src_poly_stride;
+    hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
+                       n_limbs, poly_stride, from);
+    hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ll,
+                       sl, n_limbs, poly_stride);
     return true;
 }
 
