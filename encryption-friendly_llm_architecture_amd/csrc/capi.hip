@@ -296,8 +296,11 @@ static void *upload_desc(hemm_context *ctx, const void *a, size_t na, const void
     if (!ctx->d_desc) HEMM_HIP(hipMalloc(&ctx->d_desc, cap));
     const size_t off_b = (na + 255) & ~(size_t)255;
     if (off_b + nb > cap) throw std::invalid_argument("too many terms in one batched call");
-    HEMM_HIP(hipMemcpyAsync(ctx->d_desc, a, na, hipMemcpyHostToDevice, s));
-    HEMM_HIP(hipMemcpyAsync((char *)ctx->d_desc + off_b, b, nb, hipMemcpyHostToDevice, s));
+    // both lists in one copy (pageable source: the runtime has read it when the call returns)
+    std::vector<char> both(off_b + nb);
+    memcpy(both.data(), a, na);
+    memcpy(both.data() + off_b, b, nb);
+    HEMM_HIP(hipMemcpyAsync(ctx->d_desc, both.data(), both.size(), hipMemcpyHostToDevice, s));
     *second = (char *)ctx->d_desc + off_b;
     return ctx->d_desc;
 }
@@ -417,6 +420,13 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
         need(terms[t].ct != nullptr, "null pointer in a term");
         need(terms[t].galois == 0 || ((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N),
              "galois element must be odd and < 2N");
+    }
+    static_assert(sizeof(hemm_lin_term) == 32, "the kernels read these records as they are");
+    if ((int)n_terms <= masked_arg_capacity() && (int)n_out <= masked_arg_capacity()) {
+        launch_masked_sum_args(ctx, terms, (int)n_terms, group_offsets, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
+                               (hipStream_t)stream);
+        check_launch();
+        return 0;
     }
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, terms, n_terms * sizeof(hemm_lin_term), group_offsets,

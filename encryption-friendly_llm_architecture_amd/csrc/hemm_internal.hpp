@@ -105,5 +105,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
                           u64 *conv, hipStream_t s);
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s);
+int masked_arg_capacity();
+void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
+                            int nq, int n_polys, u64 *out, hipStream_t s);
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
                          bool accumulate, hipStream_t s);

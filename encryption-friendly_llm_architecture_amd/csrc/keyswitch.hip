@@ -311,10 +311,9 @@ struct LinTermDev {
 // aligned pair, possibly swapped), so each mask residue is read once; integer products are summed as 128-bit
 // values and reduced every 4 terms.
 template <int n_polys>
-__global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__restrict__ terms,
-                                                         const u32 *__restrict__ group_off, u64 *__restrict__ out,
-                                                         const ModQ *__restrict__ modq, const double *__restrict__ fp, int nq, int logN,
-                                                         int n_out) {
+__device__ __forceinline__ void masked_sum_body(const LinTermDev *__restrict__ terms, const u32 *__restrict__ group_off,
+                                                u64 *__restrict__ out, const ModQ *__restrict__ modq,
+                                                const double *__restrict__ fp, int nq, int logN, int n_out) {
     // Workgroups go round-robin over the 8 XCDs, each with its own L2.  The outputs of one launch mostly
     // sum the same ciphertexts under different masks, so all outputs of a (limb, 512-coefficient) tile are
     // placed back to back on one XCD: the ciphertext tile is fetched from HBM once instead of once per output.
@@ -431,6 +430,27 @@ __global__ __launch_bounds__(256) void masked_sum_kernel(const LinTermDev *__res
         }
         stream_store2(out + ((size_t)o * n_polys + p) * nq * N + e, acc[p][0], acc[p][1]);
     }
+}
+
+// Short term lists (the usual case: a handful of masked terms per output) travel in the kernel arguments, which
+// saves the staging copy in front of the launch; longer lists are read from device memory.
+#define MASKED_ARG_TERMS 32
+struct MaskedArgs {
+    LinTermDev t[MASKED_ARG_TERMS];
+    u32 off[MASKED_ARG_TERMS + 1];
+};
+template <int n_polys>
+__global__ __launch_bounds__(256) void masked_sum_kernel(const MaskedArgs args, u64 *__restrict__ out,
+                                                         const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                         int nq, int logN, int n_out) {
+    masked_sum_body<n_polys>(args.t, args.off, out, modq, fp, nq, logN, n_out);
+}
+template <int n_polys>
+__global__ __launch_bounds__(256) void masked_sum_list_kernel(const LinTermDev *__restrict__ terms,
+                                                              const u32 *__restrict__ group_off, u64 *__restrict__ out,
+                                                              const ModQ *__restrict__ modq, const double *__restrict__ fp,
+                                                              int nq, int logN, int n_out) {
+    masked_sum_body<n_polys>(terms, group_off, out, modq, fp, nq, logN, n_out);
 }
 
 // acc3 (+)= sum_{g < G} (b1 b2, a1 b2 + a2 b1, a1 a2) of t1[g], t2[g], each [2][nq][N]
@@ -955,14 +975,34 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
     dim3 grid((unsigned)(c->N / 512) * nq * n_out), block(256);
     const LinTermDev *td = (const LinTermDev *)terms_dev;
     if (n_polys == 1)
-        hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
-                           n_out);
+        hipLaunchKernelGGL(masked_sum_list_kernel<1>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq,
+                           c->logN, n_out);
     else if (n_polys == 2)
-        hipLaunchKernelGGL(masked_sum_kernel<2>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
-                           n_out);
+        hipLaunchKernelGGL(masked_sum_list_kernel<2>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq,
+                           c->logN, n_out);
     else
-        hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq, c->logN,
-                           n_out);
+        hipLaunchKernelGGL(masked_sum_list_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq,
+                           c->logN, n_out);
+}
+// the same with the term list in host memory (n_terms, n_out <= masked_arg_capacity()), passed in the kernel arguments
+int masked_arg_capacity() { return MASKED_ARG_TERMS; }
+void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
+                            int nq, int n_polys, u64 *out, hipStream_t s) {
+    if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
+    if (c->N < 512) throw std::invalid_argument("masked sums need N >= 512");
+    if (n_terms > MASKED_ARG_TERMS || n_out > MASKED_ARG_TERMS)
+        throw std::invalid_argument("term list too long for the argument path");
+    MaskedArgs a;
+    memset(&a, 0, sizeof(a));
+    memcpy(a.t, terms_host, (size_t)n_terms * sizeof(LinTermDev));
+    memcpy(a.off, group_off_host, (size_t)(n_out + 1) * sizeof(u32));
+    dim3 grid((unsigned)(c->N / 512) * nq * n_out), block(256);
+    if (n_polys == 1)
+        hipLaunchKernelGGL(masked_sum_kernel<1>, grid, block, 0, s, a, out, c->d_modq, c->d_fp, nq, c->logN, n_out);
+    else if (n_polys == 2)
+        hipLaunchKernelGGL(masked_sum_kernel<2>, grid, block, 0, s, a, out, c->d_modq, c->d_fp, nq, c->logN, n_out);
+    else
+        hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, a, out, c->d_modq, c->d_fp, nq, c->logN, n_out);
 }
 
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
