@@ -37,7 +37,8 @@ vp = ctypes.c_void_p
 
 
 class RotTerm(ctypes.Structure):
-    _fields_ = [("ext", vp), ("b", vp), ("evk", vp), ("mask", vp), ("galois", ctypes.c_uint64)]
+    _fields_ = [("ext", vp), ("b", vp), ("evk", vp), ("mask", vp), ("galois", ctypes.c_uint32),
+                ("mask_shift", ctypes.c_uint32)]
 
 
 class LinTerm(ctypes.Structure):
@@ -74,6 +75,7 @@ def _declare(L):
     L.hemm_hoisted_moddown.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, ci, ci, vp, vp, sz, vp, vp]
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
+    L.hemm_compact_mask.argtypes = [vp, vp, u32, u32, vp, ctypes.POINTER(ci), vp]
 
 
 def check(rc):
@@ -255,14 +257,23 @@ class Context:
                                      vp(ext.data_ptr()), vp(ws.data_ptr()), vp(0)))
         return ext
 
+    def compact_mask(self, mask, shift):
+        """run table [limbs][N >> shift] of a mask [limbs][N] constant over runs of 2^shift residues, or None"""
+        import torch
+        table = torch.empty((mask.shape[0], self.N >> shift), dtype=torch.int64, device=mask.device)
+        ok = ctypes.c_int(0)
+        check(lib().hemm_compact_mask(self.h, vp(mask.data_ptr()), mask.shape[0], shift, vp(table.data_ptr()),
+                                      ctypes.byref(ok), vp(0)))
+        return table if ok.value else None
+
     def hoisted_terms(self, groups, nq, b_premultiplied=False):
-        """groups: list of lists of (ext, b, evk, mask or None, galois) -> y [n_out][2][nq+K][N]"""
+        """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift]) -> y [n_out][2][nq+K][N]"""
         import torch
         flat = [t for g in groups for t in g]
         arr = (RotTerm * len(flat))()
-        for i, (ext, b, evk, mask, gal) in enumerate(flat):
+        for i, (ext, b, evk, mask, gal, *shift) in enumerate(flat):
             arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
-                             mask.data_ptr() if mask is not None else None, gal)
+                             mask.data_ptr() if mask is not None else None, gal, shift[0] if shift else 0)
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))
@@ -276,9 +287,9 @@ class Context:
         import torch
         flat = [t for g in groups for t in g]
         arr = (RotTerm * len(flat))()
-        for i, (ext, b, evk, mask, gal) in enumerate(flat):
+        for i, (ext, b, evk, mask, gal, *shift) in enumerate(flat):
             arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
-                             mask.data_ptr() if mask is not None else None, gal)
+                             mask.data_ptr() if mask is not None else None, gal, shift[0] if shift else 0)
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))

@@ -323,7 +323,7 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
 // the device descriptors.
 struct RotDev {
     const u64 *ext, *b, *evk, *mask;
-    u32 galois, pad;
+    u32 galois, mask_shift;
     const u64 *ext2, *b2, *mask2;
 };
 static_assert(sizeof(RotDev) == 64, "RotDev must match the kernels' RotTermDev");
@@ -338,10 +338,14 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
         for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
             need(terms[t].ext && terms[t].evk, "null pointer in a rotation term");
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
+            need(terms[t].mask_shift == 0 || (terms[t].mask && (int)terms[t].mask_shift < ctx->logN),
+                 "mask_shift needs a run table and must be below log N");
             RotDev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
-                       (const u64 *)terms[t].mask, (u32)terms[t].galois, 0, nullptr, nullptr, nullptr};
+                       (const u64 *)terms[t].mask, (u32)terms[t].galois, terms[t].mask ? (u32)terms[t].mask_shift : 0u,
+                       nullptr, nullptr, nullptr};
             if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
-                terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois) {
+                terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois &&
+                terms[t + 1].mask_shift == terms[t].mask_shift) {
                 cur.ext2 = (const u64 *)terms[t + 1].ext;
                 cur.b2 = (const u64 *)terms[t + 1].b;
                 cur.mask2 = (const u64 *)terms[t + 1].mask;
@@ -433,6 +437,16 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
                                   (n_out + 1) * sizeof(uint32_t), &off_dev, (hipStream_t)stream);
     launch_masked_sum(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
                       (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs, uint32_t shift, uint64_t *table,
+                      int *is_constant, void *stream) {
+    HEMM_TRY
+    need(mask && table && is_constant, "null operand");
+    need(n_limbs >= 1 && shift >= 1 && (int)shift < ctx->logN, "shift must be in [1, log N)");
+    *is_constant = launch_compact_mask(ctx, (const u64 *)mask, (int)n_limbs, (int)shift, (u64 *)table, (hipStream_t)stream) ? 1 : 0;
     check_launch();
     HEMM_CATCH
 }

@@ -106,6 +106,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s);
 int masked_arg_capacity();
+// table[j][r] = mask[j][r << shift]; true when every aligned run of 2^shift residues of the mask is constant
+bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s);
 void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
                             int nq, int n_polys, u64 *out, hipStream_t s);
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,

@@ -20,7 +20,8 @@ struct RotTermDev {
     const u64 *b;     // [nq][N] b-polynomial of the source (nullptr: none, single-source terms only)
     const u64 *evk;   // [dnum][2][nQ+K][N]
     const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
-    u32 galois, pad;
+    u32 galois;
+    u32 mask_shift;   // s > 0: mask (and mask2) are run tables [E][N >> s], one value per 2^s coefficients
     // optional second source rotated by the same Galois element with the same key (ext2 == nullptr: none):
     // the term is mask * rot(source) + mask2 * rot(source 2) and the key is read once for both
     const u64 *ext2, *b2, *mask2;
@@ -34,6 +35,13 @@ __device__ __forceinline__ ulonglong2 stream_load2(const u64 *p) {
     return make_ulonglong2(v.x, v.y);
 }
 __device__ __forceinline__ u64 stream_load1(const u64 *p) { return __builtin_nontemporal_load(p); }
+// mask residues of the pair (n, n+1) of limb j: streamed from a full mask, or one value of a run table (every
+// lane of the workgroup reads the same one or two entries, which stay in cache)
+__device__ __forceinline__ ulonglong2 load_mask2(const u64 *mask, const u32 shift, const int j, const u32 n, const int logN) {
+    if (shift == 0) return stream_load2(mask + ((size_t)j << logN) + n);
+    const u64 v = mask[((size_t)j << (logN - shift)) + (n >> shift)];
+    return make_ulonglong2(v, v);
+}
 __device__ __forceinline__ void stream_store2(u64 *p, u64 a, u64 b) {
     u64x2 v;
     v.x = a;
@@ -81,8 +89,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         const bool swap = (np & 1u) != 0;
         if (T.ext2 != nullptr) {
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
-            const ulonglong2 m1 = stream_load2(T.mask + (size_t)j * N + n);
-            const ulonglong2 m2 = stream_load2(T.mask2 + (size_t)j * N + n);
+            const ulonglong2 m1 = load_mask2(T.mask, T.mask_shift, j, n, logN);
+            const ulonglong2 m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
             u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
             for (int d = 0; d < beta; d++) {
                 ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
@@ -168,7 +176,7 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             rb[1] = addmod(rb[1], bv.y, m.q);
         }
         if (T.mask != nullptr) {
-            const ulonglong2 mk = stream_load2(T.mask + (size_t)j * N + n);
+            const ulonglong2 mk = load_mask2(T.mask, T.mask_shift, j, n, logN);
             add128(lazy_b[0], mul64wide(rb[0], mk.x));
             add128(lazy_b[1], mul64wide(rb[1], mk.y));
             add128(lazy_a[0], mul64wide(ra[0], mk.x));
@@ -237,8 +245,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
         const bool swap = (np & 1u) != 0;
         double sb0 = 0, sb1 = 0, sa0 = 0, sa1 = 0;
         if (T.ext2 != nullptr) {
-            const D2 m1 = to_d2(stream_load2(T.mask + (size_t)j * N + n));
-            const D2 m2 = to_d2(stream_load2(T.mask2 + (size_t)j * N + n));
+            const D2 m1 = to_d2(load_mask2(T.mask, T.mask_shift, j, n, logN));
+            const D2 m2 = to_d2(load_mask2(T.mask2, T.mask_shift, j, n, logN));
             for (int d = 0; d < beta; d++) {
                 const D2 x1 = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
                 const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
@@ -283,7 +291,7 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 sb1 += bv.y;
             }
             if (T.mask != nullptr) {
-                const D2 mk = to_d2(stream_load2(T.mask + (size_t)j * N + n));
+                const D2 mk = to_d2(load_mask2(T.mask, T.mask_shift, j, n, logN));
                 sb0 = f.mul(sb0, mk.x);
                 sb1 = f.mul(sb1, mk.y);
                 sa0 = f.mul(sa0, mk.x);

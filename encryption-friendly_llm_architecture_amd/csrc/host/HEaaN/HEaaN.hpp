@@ -136,6 +136,12 @@ public:
     u64 level_ = 0, log_slots_ = 0, rescale_counter_ = 0;
     Real scale_ = 0;    // scale of the encoded values; 0 = the fixed scale of (level, rescale counter)
     u64 occupied_ = ~u64(0);   // slots at and beyond this index were encoded as exact zeros (all ones: unknown)
+    // Run table of a mask whose residues are constant over aligned runs of 2^compact_shift_ coefficients (the NTT
+    // form of a slot pattern with a power-of-two period): [limbs][N >> shift].  Filled by makeCompact() on masks
+    // that are cached and never written again; allocate() and setLevel() drop it.
+    DeviceBuffer compact_;
+    u32 compact_shift_ = 0;
+    bool makeCompact();        // true when a table was found
 };
 
 class Ciphertext {

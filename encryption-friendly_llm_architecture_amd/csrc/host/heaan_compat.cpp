@@ -261,10 +261,31 @@ void Plaintext::allocate(u64 level, u64 rc) {
     occupied_ = ~u64(0);
     log_slots_ = ctx_->logN - 1;
     buf_.resize(ctx_, (level + 1) * ctx_->N);
+    compact_shift_ = 0;
+    compact_ = DeviceBuffer();
+}
+bool Plaintext::makeCompact() {
+    if (compact_shift_ != 0) return true;
+    const u64 N = ctx_->N, limbs = buf_.words() / N;
+    if (limbs == 0 || ctx_->logN < 10) return false;
+    // slot patterns of period 2^6 .. 2^8 give runs of 2^(logN-7) .. 2^(logN-9) residues: longest runs first
+    for (u32 shift = (u32)ctx_->logN - 7; shift >= (u32)ctx_->logN - 9; shift--) {
+        DeviceBuffer t(ctx_, limbs * (N >> shift));
+        int ok = 0;
+        ck(hemm_compact_mask(ctx_->dev, buf_.data(), (uint32_t)limbs, shift, t.data(), &ok, nullptr));
+        if (ok) {
+            compact_ = std::move(t);
+            compact_shift_ = shift;
+            return true;
+        }
+    }
+    return false;
 }
 void Plaintext::setLevel(u64 level) {
     if (level > level_) throw RuntimeException("Plaintext::setLevel can only lower the level");
     if (level == level_) return;
+    compact_shift_ = 0;
+    compact_ = DeviceBuffer();
     DeviceBuffer nb(ctx_, (level + 1) * ctx_->N);
     hip_ck(hipMemcpyAsync(nb.data(), buf_.data(), (level + 1) * ctx_->N * 8, hipMemcpyDeviceToDevice, nullptr),
            "hipMemcpyAsync");

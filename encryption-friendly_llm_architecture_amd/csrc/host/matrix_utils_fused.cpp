@@ -76,12 +76,17 @@ struct Rot {
 };
 
 hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois, const Plaintext *mask) {
-    hemm_rot_term t;
+    hemm_rot_term t{};
     t.ext = ext;
     t.b = b;
     t.evk = pack.galoisKey(galois);
     t.mask = mask ? mask->buf_.data() : nullptr;
-    t.galois = galois;
+    t.galois = (uint32_t)galois;
+    t.mask_shift = 0;
+    if (mask && mask->compact_shift_ != 0) {
+        t.mask = mask->compact_.data();
+        t.mask_shift = mask->compact_shift_;
+    }
     return t;
 }
 
@@ -123,6 +128,10 @@ std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eva
         v.push_back(endec.encodeExtended(wrap, level));
         v.push_back(endec.encodeExtended(main, level));
     }
+    // column patterns repeat every n slots: in NTT form such a mask is constant over long runs of residues, and
+    // the hoisted sums then read one table entry per run instead of streaming the mask
+    if (!first_block_only && (n & (n - 1)) == 0)
+        for (Plaintext &pt : v) pt.makeCompact();
     return cache.emplace(key, std::move(v)).first->second;
 }
 std::vector<Plaintext> &MatrixTransformer::getRowMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
@@ -700,7 +709,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     ck(hemm_mul_scalar(c->dev, U.data() + us, pw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
     std::vector<hemm_rot_term> terms;
     {
-        hemm_rot_term t;
+        hemm_rot_term t{};
         t.ext = ext2;
         t.b = pb.data();
         t.evk = pack.multKey();
@@ -710,7 +719,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     }
     for (u64 i = 1; i < m; i++) {
         const u64 gal = rot.galois((i64)i * g * ru);
-        hemm_rot_term t;
+        hemm_rot_term t{};
         t.ext = ext1 + i * beta * El * N;
         t.b = pb.data() + i * lo * N;
         t.evk = pack.galoisKey(gal);

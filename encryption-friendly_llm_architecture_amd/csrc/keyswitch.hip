@@ -217,11 +217,17 @@ u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 //                                                         + [pol = 0, j < nq] (P mod q_j) * b_t[j][pi_t(n)] )
 // The automorphism is an index map on the reads (aligned 2^m-blocks map to aligned 2^m-blocks in the
 // bit-reversed order, so a wavefront still reads whole 512-byte runs); the key is streamed once.
+// MODE 1: the launch covers only limbs of primes below 2^44 (double-precision path); MODE 2: only the others
+// (integer path); MODE 0: any limb, path chosen per workgroup.  jmap lists the n_j limbs of the launch.  The integer
+// path keeps 128-bit accumulators and needs more registers, so on large launches the double-precision limbs get a
+// kernel of their own and run at a higher occupancy; small launches stay whole (two part-filled launches cost more).
+template <int MODE>
 __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict__ terms,
                                                    const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                    const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                    const LimbList &ll, const CstList &pmod, int nq, int E, int beta,
-                                                   int n_full, int logN, int b_premultiplied, int n_out) {
+                                                   int n_full, int logN, int b_premultiplied, int n_out,
+                                                   const LimbList &jmap, int n_j) {
     // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
     // (possibly swapped), so every access is a 16-byte load or store.
     // Work is dealt out by SOURCE chunk.  The automorphism maps aligned 512-coefficient chunks onto aligned
@@ -235,9 +241,13 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
     if (chunks >= 8) {
         const u32 xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per = chunks >> 3;
         o = slot % (u32)n_out;
+        // Limbs of 60-bit primes are bound by integer arithmetic, limbs below 2^44 (double precision) by memory:
+        // the limb index runs faster than the chunk index so that both kinds are resident together and the two
+        // limits overlap instead of alternating.
         const u32 rest = slot / (u32)n_out;
-        const u32 s = (rest % per) * 8u + xcd;
-        j = rest / per;
+        const u32 s = (rest / (u32)n_j) * 8u + xcd;
+        j = jmap.idx[rest % (u32)n_j];
+        (void)per;
         // output chunk whose gather lands in source chunk s: the low cbits+1 bits of the exponent 2 br(i) + 1
         // are fixed by the chunk; multiply them by g^-1 (mod 2^(cbits+1))
         u32 g = terms[group_off[o]].galois;
@@ -253,14 +263,14 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
         o = blockIdx.x % (u32)n_out;
         const u32 rest = blockIdx.x / (u32)n_out;
         chunk = rest % chunks;
-        j = rest / chunks;
+        j = jmap.idx[rest / chunks];
     }
     const int prime = ll.idx[j];
     const u32 n = (chunk * 256 + threadIdx.x) * 2;
     const double fq = fp[4 * prime];
     const size_t N = (size_t)1 << logN;
     u64 rb[2], ra[2];
-    if (fq != 0.0 && beta <= 6) {
+    if (MODE == 1 || (MODE == 0 && fq != 0.0 && beta <= 6)) {
         const FpMod f{fq, fp[4 * prime + 1]};
         double fb[2], fa[2];
         hoisted_pair_fp(terms, group_off, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E, beta, n_full, logN,
@@ -285,19 +295,24 @@ struct HoistedArgs {
     RotTermDev t[HOISTED_ARG_TERMS];
     u32 off[HOISTED_ARG_TERMS + 1];
 };
+template <int MODE>
 __global__ __launch_bounds__(256) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
-                                                            int n_full, int logN, int b_premultiplied, int n_out) {
-    hoisted_terms_body(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out);
+                                                            int n_full, int logN, int b_premultiplied, int n_out,
+                                                            LimbList jmap, int n_j) {
+    hoisted_terms_body<MODE>(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
+                           n_j);
 }
+template <int MODE>
 __global__ __launch_bounds__(256) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
                                                                  const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                                  const ModQ *__restrict__ modq,
                                                                  const double *__restrict__ fp, LimbList ll, CstList pmod,
                                                                  int nq, int E, int beta, int n_full, int logN,
-                                                                 int b_premultiplied, int n_out) {
-    hoisted_terms_body(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out);
+                                                                 int b_premultiplied, int n_out, LimbList jmap, int n_j) {
+    hoisted_terms_body<MODE>(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
+                           n_j);
 }
 
 struct LinTermDev {
@@ -883,15 +898,47 @@ static CstList p_mod_chain(const hemm_context *c, int nq) {
     return pm;
 }
 
+// Limbs of the extended basis handled in double precision (primes below 2^44, at most 6 digits) and the others;
+// true when the launch is large enough (in workgroups) for one kernel per kind to pay.
+static bool split_limbs(const hemm_context *c, int nq, int beta, int n_out, LimbList &fpl, int &n_fp, LimbList &il,
+                        int &n_int, LimbList &all) {
+    const LimbList ll = limbs_default(c, nq, 1);
+    const int E = nq + c->nP;
+    memset(&fpl, 0, sizeof(fpl));
+    memset(&il, 0, sizeof(il));
+    n_fp = n_int = 0;
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) all.idx[j] = (uint8_t)j;
+    for (int j = 0; j < E; j++) {
+        if (c->primes[ll.idx[j]] < (1ull << 44) && beta <= 6)
+            fpl.idx[n_fp++] = (uint8_t)j;
+        else
+            il.idx[n_int++] = (uint8_t)j;
+    }
+    return n_fp > 0 && n_int > 0 && (size_t)n_out * E * (c->N / 512) >= 32768;
+}
+
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
                           bool b_premultiplied, hipStream_t s) {
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
-    dim3 grid((unsigned)((size_t)n_out * E * (c->N / 512))), block(256);
-    hipLaunchKernelGGL(hoisted_terms_list_kernel, grid, block, 0, s, (const RotTermDev *)terms_dev, group_off_dev, y,
-                       c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E, beta, c->nQ + c->nP, c->logN,
-                       b_premultiplied ? 1 : 0, n_out);
+    LimbList fpl, il, all;
+    int n_fp, n_int;
+    const bool split = split_limbs(c, nq, beta, n_out, fpl, n_fp, il, n_int, all);
+    const dim3 block(256);
+    const size_t per_limb = (size_t)n_out * (c->N / 512);
+    const LimbList ll = limbs_default(c, nq, 1);
+    const RotTermDev *td = (const RotTermDev *)terms_dev;
+    const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
+    if (!split) {
+        hipLaunchKernelGGL(hoisted_terms_list_kernel<0>, dim3((unsigned)(per_limb * E)), block, 0, s, td, group_off_dev, y,
+                           c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, all, E);
+        return;
+    }
+    hipLaunchKernelGGL(hoisted_terms_list_kernel<1>, dim3((unsigned)(per_limb * n_fp)), block, 0, s, td, group_off_dev, y,
+                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, fpl, n_fp);
+    hipLaunchKernelGGL(hoisted_terms_list_kernel<2>, dim3((unsigned)(per_limb * n_int)), block, 0, s, td, group_off_dev, y,
+                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, il, n_int);
 }
 // the same with the term list (host memory, already merged: n_terms <= HOISTED_ARG_TERMS, n_out <= HOISTED_ARG_TERMS)
 // passed in the kernel arguments
@@ -906,9 +953,22 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     memset(&a, 0, sizeof(a));
     memcpy(a.t, terms_host, (size_t)n_terms * sizeof(RotTermDev));
     memcpy(a.off, group_off_host, (size_t)(n_out + 1) * sizeof(u32));
-    dim3 grid((unsigned)((size_t)n_out * E * (c->N / 512))), block(256);
-    hipLaunchKernelGGL(hoisted_terms_kernel, grid, block, 0, s, a, y, c->d_modq, c->d_fp, limbs_default(c, nq, 1), pm, nq, E,
-                       beta, c->nQ + c->nP, c->logN, b_premultiplied ? 1 : 0, n_out);
+    LimbList fpl, il, all;
+    int n_fp, n_int;
+    const bool split = split_limbs(c, nq, beta, n_out, fpl, n_fp, il, n_int, all);
+    const dim3 block(256);
+    const size_t per_limb = (size_t)n_out * (c->N / 512);
+    const LimbList ll = limbs_default(c, nq, 1);
+    const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
+    if (!split) {
+        hipLaunchKernelGGL(hoisted_terms_kernel<0>, dim3((unsigned)(per_limb * E)), block, 0, s, a, y, c->d_modq, c->d_fp, ll,
+                           pm, nq, E, beta, n_full, c->logN, pre, n_out, all, E);
+        return;
+    }
+    hipLaunchKernelGGL(hoisted_terms_kernel<1>, dim3((unsigned)(per_limb * n_fp)), block, 0, s, a, y, c->d_modq, c->d_fp, ll, pm,
+                       nq, E, beta, n_full, c->logN, pre, n_out, fpl, n_fp);
+    hipLaunchKernelGGL(hoisted_terms_kernel<2>, dim3((unsigned)(per_limb * n_int)), block, 0, s, a, y, c->d_modq, c->d_fp, ll, pm,
+                       nq, E, beta, n_full, c->logN, pre, n_out, il, n_int);
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;
@@ -983,6 +1043,27 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
     else
         hipLaunchKernelGGL(masked_sum_list_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq,
                            c->logN, n_out);
+}
+__global__ __launch_bounds__(256) void compact_mask_kernel(const u64 *__restrict__ mask, u64 *__restrict__ table,
+                                                           size_t total, int shift, u32 *__restrict__ differs) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;        // limb * N + position
+    if (i >= total) return;
+    const size_t run = i >> shift;
+    const u64 v = mask[i], first = mask[run << shift];
+    if ((i & (((size_t)1 << shift) - 1)) == 0) table[run] = v;
+    if (v != first) atomicOr(differs, 1u);
+}
+bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s) {
+    u32 *flag = nullptr, h = 0;
+    HEMM_HIP(hipMalloc((void **)&flag, sizeof(u32)));
+    HEMM_HIP(hipMemcpyAsync(flag, &h, sizeof(u32), hipMemcpyHostToDevice, s));
+    const size_t total = (size_t)n_limbs * c->N;
+    hipLaunchKernelGGL(compact_mask_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, mask, table, total,
+                       shift, flag);
+    HEMM_HIP(hipMemcpyAsync(&h, flag, sizeof(u32), hipMemcpyDeviceToHost, s));
+    HEMM_HIP(hipStreamSynchronize(s));
+    HEMM_HIP(hipFree(flag));
+    return h == 0;
 }
 // the same with the term list in host memory (n_terms, n_out <= masked_arg_capacity()), passed in the kernel arguments
 int masked_arg_capacity() { return MASKED_ARG_TERMS; }

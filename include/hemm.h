@@ -127,9 +127,18 @@ typedef struct {
     const uint64_t *b;    /* [nq][N], or NULL: the term contributes only the key product (used for the
                            * degree-2 component of a tensor product, with a key for the rotated s^2) */
     const uint64_t *evk;  /* [dnum][2][n_q+n_p][N] */
-    const uint64_t *mask; /* [nq+n_p][N] or NULL */
-    uint64_t galois;
+    const uint64_t *mask; /* [nq+n_p][N] or NULL; with mask_shift = s > 0 a run table [nq+n_p][N >> s] */
+    uint32_t galois;
+    uint32_t mask_shift;  /* 0: full mask.  s >= 1: the mask is constant over aligned runs of 2^s coefficients
+                           * (the NTT form of a slot pattern with period 2^(logN-1-s)) and `mask` holds one value
+                           * per run, as written by hemm_compact_mask */
 } hemm_rot_term;
+/* Run table of a mask that is constant over aligned runs of 2^shift coefficients: table[j][r] = mask[j][r << shift]
+ * for n_limbs limbs; *is_constant = 0 (and the table is not to be used) when some run of the mask is not constant.
+ * Synchronises the stream.  No counterpart in HEaaN's interface: it removes the mask traffic of hoisted sums whose
+ * masks select columns of a power-of-two period. */
+int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs, uint32_t shift, uint64_t *table,
+                      int *is_constant, void *stream);
 /* y[o] = sum over terms[group_offsets[o] .. group_offsets[o+1]) of
  *        mask * ( <galois(ext), evk> + P * galois(b) )      in the extended basis, y: [n_out][2][nq+n_p][N].
  * terms / group_offsets are host arrays.  b_premultiplied != 0: every term's b already holds P*b

@@ -258,6 +258,44 @@ def test_batched_hoisted_forms(S):
     assert np.array_equal(host(acc), want3.data)
 
 
+def test_hoisted_terms_with_run_table_masks(S):
+    """A slot pattern of period 128 is, in NTT form, constant over aligned runs of N/256 residues: the hoisted sums
+    read such a mask from its run table and must give the residues of the full mask; a mask without that
+    structure is reported as such."""
+    orc, ctx, N = S.orc, S.ctx, S.N
+    rng = np.random.default_rng(77)
+    nq = orc.nQ - 1
+    orc.key_seed = 6
+    mods = orc.q[:nq]
+    shift = orc.log_n - 8
+    cts = [rand_limbs(rng, mods, (2,), N) for _ in range(2)]
+    dcts = [dev(c) for c in cts]
+    import torch
+    dext = ctx.modup_batch(torch.stack([d[1] for d in dcts]).contiguous(), nq)
+    exts = [orc.modup(c[1]) for c in cts]
+    col = np.arange(orc.slots) % 128
+    m_main = orc.encode_ext((col < 91).astype(float), nq - 1)
+    m_wrap = orc.encode_ext((col >= 91).astype(float), nq - 1)
+    m_rand = orc.encode_ext(rng.uniform(-1, 1, orc.slots), nq - 1)
+    dmain, dwrap, drand = dev(m_main.data), dev(m_wrap.data), dev(m_rand.data)
+    tmain, twrap = ctx.compact_mask(dmain, shift), ctx.compact_mask(dwrap, shift)
+    assert tmain is not None and twrap is not None
+    assert ctx.compact_mask(drand, shift) is None
+    assert np.array_equal(host(tmain), m_main.data[:, ::1 << shift])
+    g1, g2 = orc.galois(37), orc.galois(orc.slots - 91)
+    dk = {g: dev(orc.galois_key(g)) for g in (g1, g2)}
+    # two sources under one key (merged), a single masked term, and a full mask beside a run table in one group
+    groups = [[(dext[0], dcts[0][0], dk[g1], tmain, g1, shift), (dext[1], dcts[1][0], dk[g1], twrap, g1, shift)],
+              [(dext[0], dcts[0][0], dk[g2], twrap, g2, shift)],
+              [(dext[0], dcts[0][0], dk[g1], tmain, g1, shift), (dext[1], dcts[1][0], dk[g1], drand, g1)]]
+    want = [orc.hoisted_sum([(exts[0], cts[0][0], ("g", g1), m_main), (exts[1], cts[1][0], ("g", g1), m_wrap)], nq),
+            orc.hoisted_sum([(exts[0], cts[0][0], ("g", g2), m_wrap)], nq),
+            orc.hoisted_sum([(exts[0], cts[0][0], ("g", g1), m_main), (exts[1], cts[1][0], ("g", g1), m_rand)], nq)]
+    y = host(ctx.hoisted_terms(groups, nq))
+    for k in range(3):
+        assert np.array_equal(y[k], want[k]), k
+
+
 def test_rotation_24_limb_chain_of_60_bit_primes():
     """One key-switched rotation at the shape of the reference's rotation benchmark: N = 2^16, a chain of 24
     60-bit primes + 4 special primes, dnum = 3 (digits of 8 limbs), ciphertext at level 20, steps from the
