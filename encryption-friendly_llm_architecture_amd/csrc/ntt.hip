@@ -357,6 +357,12 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(16 * c + k)];
+        // the minuend of the fused tail is fetched under the second radix-16 block instead of after it
+        u64 mv[EPI ? 16 : 1];
+        if (EPI) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) mv[k] = __builtin_nontemporal_load(mn + c + 16 * k);
+        }
         radix16_fwd(f, x, tw, 16u * (256u + r) + c);
         wave_sync();
 #pragma unroll
@@ -364,7 +370,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
         wave_sync();
         if (EPI) {
 #pragma unroll
-            for (int k = 0; k < 16; k++) o[c + 16 * k] = f.sub_scale(l[padc(c + 16 * k)], mn[c + 16 * k], cst);
+            for (int k = 0; k < 16; k++) o[c + 16 * k] = f.sub_scale(l[padc(c + 16 * k)], mv[k], cst);
         } else {
 #pragma unroll
             for (int k = 0; k < 16; k++) row[c + 16 * k] = f.to_canonical(l[padc(c + 16 * k)]);
