@@ -749,27 +749,34 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     if (min_level < 1 + btp.getMinLevelForBootstrap())
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(1 + btp.getMinLevelForBootstrap()) +
                                     " is needed.");
-    CtxtTensor a{op1}, b{op2};
-    a.setShape(rows, k);
-    b.setShape(k, cols);
-    if (min_level < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get(), b.get());
+    // the operands are only read: no working copies unless they have to be refreshed first
+    const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
+    const Ciphertext *pa = &op1.get(), *pb = &op2.get();
+    Ciphertext own_a(c), own_b(c);
+    if (min_level < 4 + btp.getMinLevelForBootstrap()) {
+        own_a = op1.get();
+        own_b = op2.get();
+        btp.bootstrapExtended(own_a, own_a, own_b);
+        pa = &own_a;
+        pb = &own_b;
+    }
     if (min_level < T + 3)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
     // The transforms end at level T+2.  With a level to spare they run in two stages from T+4 (far fewer rotations
     // and masks, MatrixTransformer::diagonalTransformTwoStage), otherwise in one from T+3; lowering the operands first
     // gives the same values with 9 or 8 instead of 13 limbs.
-    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a.getShape(), T + 2);
+    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
     // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
-    const bool two_stage = min_level >= T + 4 && a.getShape().getNumRows() == a.getShape().getNumCols() &&
-                           b.getShape().getNumRows() == b.getShape().getNumCols();
+    const bool two_stage = min_level >= T + 4 && shape_a.getNumRows() == shape_a.getNumCols() &&
+                           shape_b.getNumRows() == shape_b.getNumCols();
     const u64 Lt = two_stage ? T + 4 : T + 3;   // level the transforms start from
     DeviceBuffer ab(c, 2 * ctw);
     {
         const u64 ctw_in = 2 * (Lt + 1) * N;
         DeviceBuffer joint(c, 2 * ctw_in);
-        const u64 la = a.getLevel(), lb = b.getLevel();
-        if (la == lb && la > Lt && a.get().getRescaleCounter() == 0 && b.get().getRescaleCounter() == 0) {
+        const u64 la = pa->getLevel(), lb = pb->getLevel();
+        if (la == lb && la > Lt && pa->getRescaleCounter() == 0 && pb->getRescaleCounter() == 0) {
             // HomEvaluator::levelDown of both operands at once: multiply by round(Delta_Lt q_{Lt+1} / Delta_level)
             // over Lt+2 limbs, then one rescale of the four polynomials straight into the joint buffer
             const u64 nl = Lt + 2;
@@ -777,17 +784,18 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
             std::vector<u64> sc(nl);
             for (u64 j = 0; j < nl; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
             DeviceBuffer t(c, 4 * nl * N);
-            ck(hemm_mul_scalar(c->dev, a.get().buf_.data(), a.get().polyStride(), sc.data(), t.data(), nl * N, (uint32_t)nl, 0, 2, nullptr));
-            ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
+            ck(hemm_mul_scalar(c->dev, pa->buf_.data(), pa->polyStride(), sc.data(), t.data(), nl * N, (uint32_t)nl, 0, 2, nullptr));
+            ck(hemm_mul_scalar(c->dev, pb->buf_.data(), pb->polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
             ck(hemm_rescale(c->dev, t.data(), nl * N, joint.data(), (nl - 1) * N, (uint32_t)nl, 4, nullptr));
         } else {
-            eval.levelDown(a.get(), Lt, a.get());
-            eval.levelDown(b.get(), Lt, b.get());
-            (void)hipMemcpyAsync(joint.data(), a.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
-            (void)hipMemcpyAsync(joint.data() + ctw_in, b.get().buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+            Ciphertext la_ct(c), lb_ct(c);
+            eval.levelDown(*pa, Lt, la_ct);
+            eval.levelDown(*pb, Lt, lb_ct);
+            (void)hipMemcpyAsync(joint.data(), la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(joint.data() + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
         }
         const MaskKind kinds[2] = {MaskKind::Horizontal, MaskKind::Vertical};
-        const TileTensorShape shapes[2] = {a.getShape(), b.getShape()};
+        const TileTensorShape shapes[2] = {shape_a, shape_b};
         if (two_stage)
             tr.diagonalTransformTwoStage(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
         else
@@ -825,7 +833,7 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
-    std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, b.getShape(), T + 2);
+    std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, shape_b, T + 2);
     std::vector<Shift> sa, sb;
     for (i64 i = 1; i < n; i++) {
         sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
