@@ -19,11 +19,45 @@ struct ContextContent {
     std::vector<Real> delta;             // fixed scale of each level
     std::vector<u64> rot_group;          // 5^j mod 2N
     std::vector<double> ksi_re, ksi_im;  // exp(2 pi i k / 2N)
-    // Freed buffers are kept by size and handed out again: every kernel runs on the one default
-    // stream, so reuse is ordered after the last use without any synchronisation.
+    // Freed buffers are kept by size and handed out again: kernels run on the default stream, so reuse is
+    // ordered after the last use without any synchronisation.  The one exception is a side chain (forkSide /
+    // joinSide below): while it is open, freed buffers are parked and only return to the pool at the join.
     std::multimap<size_t, u64 *> pool;
+    std::vector<std::pair<size_t, u64 *>> parked;
     std::mutex mu;
     size_t pool_bytes = 0;
+    hipStream_t side = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    bool side_open = false;
+
+    // Opens a side chain: work given to the returned stream starts after everything queued on the default stream
+    // so far and runs beside what the default stream is given next.  The stream does not synchronise implicitly
+    // with the default stream; joinSide() makes the default stream wait for it.  Default priority.
+    hipStream_t forkSide() {
+        if (side_open) throw RuntimeException("side chain already open");
+        auto ok = [](hipError_t e, const char *what) {
+            if (e != hipSuccess) throw RuntimeException(std::string(what) + ": " + hipGetErrorString(e));
+        };
+        if (!side) {
+            ok(hipStreamCreateWithFlags(&side, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+            ok(hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming), "hipEventCreateWithFlags");
+            ok(hipEventCreateWithFlags(&ev_join, hipEventDisableTiming), "hipEventCreateWithFlags");
+        }
+        ok(hipEventRecord(ev_fork, nullptr), "hipEventRecord");
+        ok(hipStreamWaitEvent(side, ev_fork, 0), "hipStreamWaitEvent");
+        std::lock_guard<std::mutex> lk(mu);
+        side_open = true;
+        return side;
+    }
+    void joinSide() {
+        if (!side_open) return;
+        (void)hipEventRecord(ev_join, side);
+        (void)hipStreamWaitEvent(nullptr, ev_join, 0);
+        std::lock_guard<std::mutex> lk(mu);
+        side_open = false;
+        for (auto &kv : parked) pool.emplace(kv.first, kv.second);
+        parked.clear();
+    }
 
     u64 prime(size_t i) const { return i < nQ ? q[i] : p[i - nQ]; }
     u64 *alloc(size_t words) {
@@ -44,11 +78,18 @@ struct ContextContent {
     }
     void release(u64 *ptr, size_t words) {
         std::lock_guard<std::mutex> lk(mu);
-        pool.emplace(words, ptr);
+        if (side_open)
+            parked.emplace_back(words, ptr);
+        else
+            pool.emplace(words, ptr);
     }
     ~ContextContent() {
         (void)hipDeviceSynchronize();
         for (auto &kv : pool) (void)hipFree(kv.second);
+        for (auto &kv : parked) (void)hipFree(kv.second);
+        if (side) (void)hipStreamDestroy(side);
+        if (ev_fork) (void)hipEventDestroy(ev_fork);
+        if (ev_join) (void)hipEventDestroy(ev_join);
         if (dev) hemm_context_destroy(dev);
     }
 };

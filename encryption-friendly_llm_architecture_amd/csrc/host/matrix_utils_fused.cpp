@@ -351,23 +351,24 @@ struct Sources {
     const u64 *pbOf(size_t q) const { return pb.data() + q * nq * N_; }
     u64 N_;
 };
-Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq) {
+Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq, hipStream_t stream = nullptr) {
     const u64 N = c->N, E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha, ctw = 2 * nq * N;
     Sources s{DeviceBuffer(c, n * beta * E * N), DeviceBuffer(c, n * nq * N), nq, beta * E * N, N};
     DeviceBuffer ws(c, n * nq * N);
-    ck(hemm_modup_batch(c->dev, cts + nq * N, ctw, (uint32_t)nq, (uint32_t)n, s.ext.data(), ws.data(), nullptr));
+    ck(hemm_modup_batch(c->dev, cts + nq * N, ctw, (uint32_t)nq, (uint32_t)n, s.ext.data(), ws.data(), stream));
     std::vector<u64> sc(nq);
     for (u64 j = 0; j < nq; j++) {
         u64 P = 1;
         for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
         sc[j] = P;
     }
-    ck(hemm_mul_scalar(c->dev, cts, ctw, sc.data(), s.pb.data(), nq * N, (uint32_t)nq, 0, (uint32_t)n, nullptr));
+    ck(hemm_mul_scalar(c->dev, cts, ctw, sc.data(), s.pb.data(), nq * N, (uint32_t)nq, 0, (uint32_t)n, stream));
     return s;
 }
 // The same sources rotated left by rots[q] slots, as ciphertexts [n][2][nq][N]: one hoisted launch and one
 // ModDown for all of them.
-DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u64 *cts, size_t n, const i64 *rots) {
+DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u64 *cts, size_t n, const i64 *rots,
+                           hipStream_t stream = nullptr) {
     const Context &c = eval.getContext();
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
@@ -378,7 +379,7 @@ DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u
     std::vector<size_t> which;
     for (size_t q = 0; q < n; q++) {
         if (rot.norm(rots[q]) == 0) {  // a whole turn (rows of a tile that fills the slots): plain copy
-            (void)hipMemcpyAsync(out.data() + q * ctw, cts + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(out.data() + q * ctw, cts + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, stream);
             continue;
         }
         terms.push_back(term(src.extOf(q), src.pbOf(q), pack, rot.galois(rots[q]), nullptr));
@@ -387,10 +388,16 @@ DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u
     }
     if (which.empty()) return out;
     const size_t m = which.size();
-    DeviceBuffer y(c, m * 2 * E * N), ws(c, m * ctw), tmp(c, m * ctw);
-    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, 1, 0, y.data(), tmp.data(), nq * N, ws.data(), nullptr));
+    DeviceBuffer y(c, m * 2 * E * N), ws(c, m * ctw);
+    if (m == n) {   // every source rotated: the results land where they belong
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, 1, 0, y.data(), out.data(),
+                                nq * N, ws.data(), stream));
+        return out;
+    }
+    DeviceBuffer tmp(c, m * ctw);
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, 1, 0, y.data(), tmp.data(), nq * N, ws.data(), stream));
     for (size_t k = 0; k < m; k++)
-        (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, stream);
     return out;
 }
 
@@ -619,6 +626,17 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     const u64 ctl = 2 * lo * N;   // words of a two-polynomial ciphertext at level T+1
+    // The sources of the column shifts (sigma(A) and its copy rotated by -n, both extended) do not depend on the
+    // baby rotations of tau(B): a chain of small launches that runs on the side stream beside them.
+    const hipStream_t side = c->forkSide();
+    struct JoinOnExit {
+        const Context &c;
+        ~JoinOnExit() { c->joinSide(); }   // also when a launch below throws
+    } join_on_exit{c};
+    const Sources xa = extendSources(c, sigma_a, 1, nq, side);
+    const i64 back = -n;
+    const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back, side);
+    const Sources xa2 = extendSources(c, a2.data(), 1, nq, side);
     // baby rotations of tau(B): bb[i1] = rho^(i1 ru)(tau B), summed over the block copies when tau(B) is spread
     DeviceBuffer bb(c, (u64)g * ctl);
     const i64 copies = spread_block ? (i64)((c->N / 2) / spread_block) : 1;
@@ -647,10 +665,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
         sa.push_back(Shift{cu * i - g * (i / g) * ru, &cm[(size_t)(2 * cu * i + 1)], &cm[(size_t)(2 * cu * i)]});
-    const Sources xa = extendSources(c, sigma_a, 1, nq);
-    const i64 back = -n;
-    const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back);
-    const Sources xa2 = extendSources(c, a2.data(), 1, nq);
+    c->joinSide();
     // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
     // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
     const u64 pw = lo * N, us = (u64)n_giant * pw;
