@@ -545,13 +545,32 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         //   main_r * rho^(r step)(X) + wrap_r * rho^(r step - tile side)(X):
         // two Galois elements per r with one key each; when they coincide (the tile side is a whole turn of the slot
         // vector) one term with the mask of both parts.
+        // unrotated rows: mask, rescale.  They need only the input, so this chain of small launches runs on the side
+        // stream beside the rotations (its masks are looked up, and on first use encoded, before the fork).
+        std::vector<hemm_lin_term> zero_terms;
+        std::vector<uint32_t> zoff{0};
+        for (size_t q = 0; q < n_jobs; q++) {
+            hemm_lin_term t;
+            t.ct = src + q * ctw;
+            t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
+            t.stride = nq * N;
+            t.galois = 0;
+            zero_terms.push_back(t);
+            zoff.push_back((uint32_t)zero_terms.size());
+        }
+        DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
+        const hipStream_t side = c->forkSide();
+        struct JoinOnExit {
+            const Context &c;
+            ~JoinOnExit() { c->joinSide(); }
+        } join_on_exit{c};
+        ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
+        ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
         const Sources x = extendSources(c, src, n_jobs, nq);
         const KeyPack &pack = eval.getKeyPack();
         const Rot rot(c);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
-        std::vector<hemm_lin_term> zero_terms;
-        std::vector<uint32_t> zoff{0};
         bool any_rotation = false;
         for (size_t q = 0; q < n_jobs; q++) {
             const Geo g = geo(kinds[q], shapes[q]);
@@ -572,18 +591,7 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                 any_rotation = true;
             }
             off.push_back((uint32_t)terms.size());
-            hemm_lin_term t;
-            t.ct = src + q * ctw;
-            t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
-            t.stride = nq * N;
-            t.galois = 0;
-            zero_terms.push_back(t);
-            zoff.push_back((uint32_t)zero_terms.size());
         }
-        // unrotated rows: mask, rescale
-        DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
-        ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), nullptr));
-        ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
         if (any_rotation) {
             for (size_t q = 0; q + 1 < off.size(); q++)
                 if (off[q + 1] == off[q])
@@ -591,9 +599,11 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
             DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
             ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, 1, 1, y.data(), dst,
                                     (nq - 1) * N, ws.data(), nullptr));
+            c->joinSide();
             ck(hemm_pointwise(c->dev, HEMM_ADD, dst, (nq - 1) * N, zres.data(), (nq - 1) * N, dst, (nq - 1) * N,
                               (uint32_t)(nq - 1), 0, (uint32_t)(2 * n_jobs), nullptr));
         } else {
+            c->joinSide();
             (void)hipMemcpyAsync(dst, zres.data(), n_jobs * 2 * (nq - 1) * N * 8, hipMemcpyDeviceToDevice, nullptr);
         }
     }
