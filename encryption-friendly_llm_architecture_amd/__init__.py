@@ -38,7 +38,8 @@ vp = ctypes.c_void_p
 
 class RotTerm(ctypes.Structure):
     _fields_ = [("ext", vp), ("b", vp), ("evk", vp), ("mask", vp), ("galois", ctypes.c_uint32),
-                ("mask_shift", ctypes.c_uint32)]
+                ("mask_shift", ctypes.c_uint32), ("pt", vp), ("pt_galois", ctypes.c_uint32),
+                ("reserved", ctypes.c_uint32)]
 
 
 class LinTerm(ctypes.Structure):
@@ -267,13 +268,16 @@ class Context:
         return table if ok.value else None
 
     def hoisted_terms(self, groups, nq, b_premultiplied=False):
-        """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift]) -> y [n_out][2][nq+K][N]"""
+        """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift[, pt, pt_galois]]) -> y [n_out][2][nq+K][N]"""
         import torch
         flat = [t for g in groups for t in g]
         arr = (RotTerm * len(flat))()
-        for i, (ext, b, evk, mask, gal, *shift) in enumerate(flat):
-            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
-                             mask.data_ptr() if mask is not None else None, gal, shift[0] if shift else 0)
+        for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
+            shift = more[0] if more else 0
+            pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
+                             mask.data_ptr() if mask is not None else None, gal, shift,
+                             pt.data_ptr() if pt is not None else None, pt_gal, 0)
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))
@@ -287,9 +291,12 @@ class Context:
         import torch
         flat = [t for g in groups for t in g]
         arr = (RotTerm * len(flat))()
-        for i, (ext, b, evk, mask, gal, *shift) in enumerate(flat):
-            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr(), evk.data_ptr(),
-                             mask.data_ptr() if mask is not None else None, gal, shift[0] if shift else 0)
+        for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
+            shift = more[0] if more else 0
+            pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
+                             mask.data_ptr() if mask is not None else None, gal, shift,
+                             pt.data_ptr() if pt is not None else None, pt_gal, 0)
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))

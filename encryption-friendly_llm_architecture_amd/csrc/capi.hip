@@ -325,8 +325,10 @@ struct RotDev {
     const u64 *ext, *b, *evk, *mask;
     u32 galois, mask_shift;
     const u64 *ext2, *b2, *mask2;
+    const u64 *pt;
+    u32 pt_galois, pad;
 };
-static_assert(sizeof(RotDev) == 64, "RotDev must match the kernels' RotTermDev");
+static_assert(sizeof(RotDev) == 80, "RotDev must match the kernels' RotTermDev");
 static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
                             std::vector<RotDev> &d, std::vector<uint32_t> &off) {
     const uint32_t n_terms = group_offsets[n_out];
@@ -340,12 +342,15 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
             need(terms[t].mask_shift == 0 || (terms[t].mask && (int)terms[t].mask_shift < ctx->logN),
                  "mask_shift needs a run table and must be below log N");
+            need(terms[t].pt == nullptr || ((terms[t].pt_galois & 1) && terms[t].pt_galois < 2 * (uint64_t)ctx->N),
+                 "pt_galois must be odd and < 2N");
             RotDev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
                        (const u64 *)terms[t].mask, (u32)terms[t].galois, terms[t].mask ? (u32)terms[t].mask_shift : 0u,
-                       nullptr, nullptr, nullptr};
+                       nullptr, nullptr, nullptr, (const u64 *)terms[t].pt, terms[t].pt ? (u32)terms[t].pt_galois : 1u, 0u};
             if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
                 terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois &&
-                terms[t + 1].mask_shift == terms[t].mask_shift) {
+                terms[t + 1].mask_shift == terms[t].mask_shift && terms[t + 1].pt == terms[t].pt &&
+                (terms[t].pt == nullptr || terms[t + 1].pt_galois == terms[t].pt_galois)) {
                 cur.ext2 = (const u64 *)terms[t + 1].ext;
                 cur.b2 = (const u64 *)terms[t + 1].b;
                 cur.mask2 = (const u64 *)terms[t + 1].mask;

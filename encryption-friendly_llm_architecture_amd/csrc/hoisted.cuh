@@ -25,6 +25,9 @@ struct RotTermDev {
     // optional second source rotated by the same Galois element with the same key (ext2 == nullptr: none):
     // the term is mask * rot(source) + mask2 * rot(source 2) and the key is read once for both
     const u64 *ext2, *b2, *mask2;
+    // optional plaintext factor [E][N] of the whole term, read through its own automorphism (nullptr: none)
+    const u64 *pt;
+    u32 pt_galois, pad;
 };
 
 // Accesses to data that is touched once per launch (keys, masks, results): marked non-temporal so they do
@@ -41,6 +44,18 @@ __device__ __forceinline__ ulonglong2 load_mask2(const u64 *mask, const u32 shif
     if (shift == 0) return stream_load2(mask + ((size_t)j << logN) + n);
     const u64 v = mask[((size_t)j << (logN - shift)) + (n >> shift)];
     return make_ulonglong2(v, v);
+}
+// residues (n, n+1) of limb j of a plaintext read through the automorphism X -> X^g (an aligned pair stays an aligned
+// pair, possibly swapped)
+__device__ __forceinline__ ulonglong2 load_rotated2(const u64 *pt, const u32 g, const int j, const u32 n, const int logN) {
+    const u32 np = g == 1u ? n : galois_index(n, g, logN);
+    ulonglong2 v = *(const ulonglong2 *)(pt + ((size_t)j << logN) + (np & ~1u));
+    if (np & 1u) {
+        const u64 t = v.x;
+        v.x = v.y;
+        v.y = t;
+    }
+    return v;
 }
 __device__ __forceinline__ void stream_store2(u64 *p, u64 a, u64 b) {
     u64x2 v;
@@ -89,8 +104,15 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         const bool swap = (np & 1u) != 0;
         if (T.ext2 != nullptr) {
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
-            const ulonglong2 m1 = load_mask2(T.mask, T.mask_shift, j, n, logN);
-            const ulonglong2 m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
+            ulonglong2 m1 = load_mask2(T.mask, T.mask_shift, j, n, logN);
+            ulonglong2 m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
+            if (T.pt != nullptr) {
+                const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
+                m1.x = mulmod(m1.x, pv.x, m);
+                m1.y = mulmod(m1.y, pv.y, m);
+                m2.x = mulmod(m2.x, pv.x, m);
+                m2.y = mulmod(m2.y, pv.y, m);
+            }
             u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
             for (int d = 0; d < beta; d++) {
                 ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
@@ -175,8 +197,17 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             rb[0] = addmod(rb[0], bv.x, m.q);
             rb[1] = addmod(rb[1], bv.y, m.q);
         }
-        if (T.mask != nullptr) {
-            const ulonglong2 mk = load_mask2(T.mask, T.mask_shift, j, n, logN);
+        if (T.mask != nullptr || T.pt != nullptr) {
+            ulonglong2 mk = T.mask != nullptr ? load_mask2(T.mask, T.mask_shift, j, n, logN) : make_ulonglong2(1, 1);
+            if (T.pt != nullptr) {
+                const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
+                if (T.mask != nullptr) {
+                    mk.x = mulmod(mk.x, pv.x, m);
+                    mk.y = mulmod(mk.y, pv.y, m);
+                } else {
+                    mk = pv;
+                }
+            }
             add128(lazy_b[0], mul64wide(rb[0], mk.x));
             add128(lazy_b[1], mul64wide(rb[1], mk.y));
             add128(lazy_a[0], mul64wide(ra[0], mk.x));
@@ -245,8 +276,15 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
         const bool swap = (np & 1u) != 0;
         double sb0 = 0, sb1 = 0, sa0 = 0, sa1 = 0;
         if (T.ext2 != nullptr) {
-            const D2 m1 = to_d2(load_mask2(T.mask, T.mask_shift, j, n, logN));
-            const D2 m2 = to_d2(load_mask2(T.mask2, T.mask_shift, j, n, logN));
+            D2 m1 = to_d2(load_mask2(T.mask, T.mask_shift, j, n, logN));
+            D2 m2 = to_d2(load_mask2(T.mask2, T.mask_shift, j, n, logN));
+            if (T.pt != nullptr) {
+                const D2 pv = to_d2(load_rotated2(T.pt, T.pt_galois, j, n, logN));
+                m1.x = f.mul(m1.x, pv.x);
+                m1.y = f.mul(m1.y, pv.y);
+                m2.x = f.mul(m2.x, pv.x);
+                m2.y = f.mul(m2.y, pv.y);
+            }
             for (int d = 0; d < beta; d++) {
                 const D2 x1 = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
                 const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
@@ -296,6 +334,13 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 sb1 = f.mul(sb1, mk.y);
                 sa0 = f.mul(sa0, mk.x);
                 sa1 = f.mul(sa1, mk.y);
+            }
+            if (T.pt != nullptr) {
+                const D2 pv = to_d2(load_rotated2(T.pt, T.pt_galois, j, n, logN));
+                sb0 = f.mul(sb0, pv.x);
+                sb1 = f.mul(sb1, pv.y);
+                sa0 = f.mul(sa0, pv.x);
+                sa1 = f.mul(sa1, pv.y);
             }
         }
         acc_b0 += sb0;

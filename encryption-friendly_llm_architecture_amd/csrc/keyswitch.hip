@@ -289,7 +289,7 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
 
 // Term lists of up to HOISTED_ARG_TERMS terms and outputs travel in the kernel arguments (no staging copy before
 // the launch); longer lists are read from device memory.
-static_assert(sizeof(RotTermDev) == 64, "the C ABI builds these records on the host");
+static_assert(sizeof(RotTermDev) == 80, "the C ABI builds these records on the host");
 #define HOISTED_ARG_TERMS 32
 struct HoistedArgs {
     RotTermDev t[HOISTED_ARG_TERMS];

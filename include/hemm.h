@@ -132,6 +132,10 @@ typedef struct {
     uint32_t mask_shift;  /* 0: full mask.  s >= 1: the mask is constant over aligned runs of 2^s coefficients
                            * (the NTT form of a slot pattern with period 2^(logN-1-s)) and `mask` holds one value
                            * per run, as written by hemm_compact_mask */
+    const uint64_t *pt;   /* [nq+n_p][N] or NULL: a second plaintext factor over the extended basis, read through
+                           * the automorphism pt_galois (the rotated weight of a plaintext-ciphertext product) */
+    uint32_t pt_galois;   /* odd, < 2N; 1 = as stored */
+    uint32_t reserved;    /* 0 */
 } hemm_rot_term;
 /* Run table of a mask that is constant over aligned runs of 2^shift coefficients: table[j][r] = mask[j][r << shift]
  * for n_limbs limbs; *is_constant = 0 (and the table is not to be used) when some run of the mask is not constant.
@@ -140,7 +144,8 @@ typedef struct {
 int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs, uint32_t shift, uint64_t *table,
                       int *is_constant, void *stream);
 /* y[o] = sum over terms[group_offsets[o] .. group_offsets[o+1]) of
- *        mask * ( <galois(ext), evk> + P * galois(b) )      in the extended basis, y: [n_out][2][nq+n_p][N].
+ *        mask * pt_galois(pt) * ( <galois(ext), evk> + P * galois(b) )   in the extended basis (absent factors
+ *        are 1), y: [n_out][2][nq+n_p][N].
  * terms / group_offsets are host arrays.  b_premultiplied != 0: every term's b already holds P*b
  * (hemm_mul_scalar with P mod q_j once per source instead of once per term). */
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets,

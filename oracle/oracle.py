@@ -580,14 +580,33 @@ class Oracle:
         return self.level_down(x, x.level - 1)
 
     # ---- hoisted / merged forms (what the batched GPU launches compute) -------------------------
-    def encode_ext(self, msg, level):
-        """Plaintext over the extended basis: limbs q_0..q_level then the special primes."""
+    def ext_primes(self, level):
+        """Prime indices of the extended basis at `level`: q_0..q_level, then the special primes."""
+        return list(range(level + 1)) + [self.nQ + k for k in range(self.nP)]
+
+    def ext_plain_product(self, mask, pt, g):
+        """mask * (pt read through the automorphism X -> X^g), limb-wise over the extended basis: the plaintext
+        factor a hoisted term applies when it carries both a mask and a rotated plaintext (mask None: factor 1)."""
+        level = pt.data.shape[0] - self.nP - 1
+        out = np.empty_like(pt.data)
+        for j, pi in enumerate(self.ext_primes(level)):
+            rot = np.empty(self.N, dtype=np.uint64)
+            self.L.orc_automorphism_ntt(self.h, _p(np.ascontiguousarray(pt.data[j])), _p(rot), int(g))
+            if mask is None:
+                out[j] = rot
+            else:
+                self.L.orc_pointwise(self.h, 2, _p(np.ascontiguousarray(mask.data[j])), _p(rot), _p(out[j]), pi)
+        return Pt(out, pt.scale * (mask.scale if mask is not None else 1.0))
+
+    def encode_ext(self, msg, level, scale=None):
+        """Plaintext over the extended basis: limbs q_0..q_level then the special primes (scale: the level's fixed
+        scale unless given)."""
         z = np.zeros(self.slots, dtype=np.complex128)
         m = np.asarray(msg)
         z[: m.size] = m.reshape(-1)
         sl = np.ascontiguousarray(z.view(np.float64))
         co = np.empty(self.N, dtype=np.int64)
-        scale = self.delta[level]
+        scale = self.delta[level] if scale is None else scale
         self.L.orc_encode_coeffs(self.h, _p(sl, f64p), float(scale), _p(co, i64p))
         primes = list(range(level + 1)) + [self.nQ + k for k in range(self.nP)]
         out = np.empty((len(primes), self.N), dtype=np.uint64)

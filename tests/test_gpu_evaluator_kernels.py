@@ -296,6 +296,42 @@ def test_hoisted_terms_with_run_table_masks(S):
         assert np.array_equal(y[k], want[k]), k
 
 
+def test_hoisted_terms_with_rotated_plaintext_factor(S):
+    """A term may carry a plaintext over the extended basis, read through its own automorphism, as a further factor
+    (the rotated weight of a plaintext-ciphertext product summed before the ModDown): with a mask, with two masked
+    sources under one key, and alone."""
+    import torch
+    orc, ctx, N = S.orc, S.ctx, S.N
+    rng = np.random.default_rng(78)
+    nq = orc.nQ - 1
+    orc.key_seed = 6
+    mods = orc.q[:nq]
+    shift = orc.log_n - 8
+    cts = [rand_limbs(rng, mods, (2,), N) for _ in range(2)]
+    dcts = [dev(c) for c in cts]
+    dext = ctx.modup_batch(torch.stack([d[1] for d in dcts]).contiguous(), nq)
+    exts = [orc.modup(c[1]) for c in cts]
+    col = np.arange(orc.slots) % 128
+    m_main = orc.encode_ext((col < 91).astype(float), nq - 1)
+    m_wrap = orc.encode_ext((col >= 91).astype(float), nq - 1)
+    weight = orc.encode_ext(rng.uniform(-1, 1, orc.slots), nq - 1)
+    dmain, dwrap, dweight = dev(m_main.data), dev(m_wrap.data), dev(weight.data)
+    tmain, twrap = ctx.compact_mask(dmain, shift), ctx.compact_mask(dwrap, shift)
+    g1, g2 = orc.galois(37), orc.galois(orc.slots - 91)
+    gp = orc.galois(5 * 128 % orc.slots)
+    dk = {g: dev(orc.galois_key(g)) for g in (g1, g2)}
+    groups = [[(dext[0], dcts[0][0], dk[g1], tmain, g1, shift, dweight, gp),
+               (dext[1], dcts[1][0], dk[g1], twrap, g1, shift, dweight, gp)],
+              [(dext[0], dcts[0][0], dk[g2], dwrap, g2, 0, dweight, gp), (dext[1], dcts[1][0], dk[g1], None, g1, 0, dweight, 1)]]
+    e_main, e_wrap = orc.ext_plain_product(m_main, weight, gp), orc.ext_plain_product(m_wrap, weight, gp)
+    want = [orc.hoisted_sum([(exts[0], cts[0][0], ("g", g1), e_main), (exts[1], cts[1][0], ("g", g1), e_wrap)], nq),
+            orc.hoisted_sum([(exts[0], cts[0][0], ("g", g2), e_wrap),
+                             (exts[1], cts[1][0], ("g", g1), orc.ext_plain_product(None, weight, 1))], nq)]
+    y = host(ctx.hoisted_terms(groups, nq))
+    for k in range(2):
+        assert np.array_equal(y[k], want[k]), k
+
+
 def test_rotation_24_limb_chain_of_60_bit_primes():
     """One key-switched rotation at the shape of the reference's rotation benchmark: N = 2^16, a chain of 24
     60-bit primes + 4 special primes, dnum = 3 (digits of 8 limbs), ciphertext at level 20, steps from the
