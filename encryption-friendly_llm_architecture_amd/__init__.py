@@ -77,6 +77,7 @@ def _declare(L):
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
     L.hemm_compact_mask.argtypes = [vp, vp, u32, u32, vp, ctypes.POINTER(ci), vp]
+    L.hemm_sum_parts.argtypes = [vp, vp, u32, u32, u32, vp, vp]
 
 
 def check(rc):
@@ -257,6 +258,14 @@ class Context:
         check(lib().hemm_modup_batch(self.h, vp(polys.data_ptr()), polys.stride(0), nq, n_in,
                                      vp(ext.data_ptr()), vp(ws.data_ptr()), vp(0)))
         return ext
+
+    def sum_parts(self, parts, n_parts, nq):
+        """[n_out * n_parts][2][nq+K][N] partial hoisted sums -> [n_out][2][nq+K][N]"""
+        import torch
+        n_out = parts.shape[0] // n_parts
+        y = torch.empty((n_out,) + tuple(parts.shape[1:]), dtype=torch.int64, device=parts.device)
+        check(lib().hemm_sum_parts(self.h, vp(parts.data_ptr()), n_parts, n_out, nq, vp(y.data_ptr()), vp(0)))
+        return y
 
     def compact_mask(self, mask, shift):
         """run table [limbs][N >> shift] of a mask [limbs][N] constant over runs of 2^shift residues, or None"""

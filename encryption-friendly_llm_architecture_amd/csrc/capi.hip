@@ -446,6 +446,18 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
     HEMM_CATCH
 }
 
+int hemm_sum_parts(hemm_context *ctx, const uint64_t *parts, uint32_t n_parts, uint32_t n_out, uint32_t nq, uint64_t *y,
+                   void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 1, &nl);
+    need(parts && y && n_parts >= 1 && n_out >= 1, "null operand");
+    need(ctx->N >= 2, "ring too small");
+    launch_sum_parts(ctx, (const u64 *)parts, (int)n_parts, (int)n_out, (int)nq, (u64 *)y, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
 int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs, uint32_t shift, uint64_t *table,
                       int *is_constant, void *stream) {
     HEMM_TRY

@@ -105,6 +105,8 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
                           u64 *conv, hipStream_t s);
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s);
+// y[o][p][j] = sum_{q < parts} part[o * parts + q][p][j] over the extended basis, y / part: [.][2][nq+K][N]
+void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s);
 int masked_arg_capacity();
 // table[j][r] = mask[j][r << shift]; true when every aligned run of 2^shift residues of the mask is constant
 bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s);

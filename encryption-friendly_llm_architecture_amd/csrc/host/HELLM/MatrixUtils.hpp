@@ -106,6 +106,19 @@ private:
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_, col_masks_ext_first_;
     std::map<std::pair<TileTensorShape, u64>, Plaintext> first_block_masks_;
+
+public:
+    // tau(B) of a plaintext weight over the extended basis, kept per weight: the key is a hash of the weight's
+    // residues, so a weight whose content changes is prepared again.  layout: 0 = not usable by the batched product,
+    // 1 = equal tile blocks, 2 = only the first block is non-zero.
+    struct WeightTau {
+        Plaintext tau;
+        int layout;
+    };
+    std::map<std::tuple<u64, TileTensorShape, u64>, WeightTau> weight_tau_;
+    std::vector<std::tuple<u64, TileTensorShape, u64>> weight_tau_order_;
+
+private:
     // (kind, shape, level, stage * 4096 + r * 4 + part) -> mask of the two-stage transforms; part 0 is an ordinary
     // plaintext (the unrotated rows), parts 1 / 2 (main / wrapped columns) are over the extended basis
     std::map<Key, Plaintext> two_stage_masks_;

@@ -241,6 +241,8 @@ public:
     // plaintext over the extended basis (limbs q_0..q_level then the special primes), for masks that
     // are applied before ModDown
     Plaintext encodeExtended(const Message &msg, u64 level) const;
+    // the same with the values scaled by `scale` instead of the level's fixed scale
+    Plaintext encodeExtended(const Message &msg, u64 level, Real scale) const;
 
 private:
     Context ctx_;

@@ -577,7 +577,8 @@ void bitrev_perm(std::vector<double> &re, std::vector<double> &im) {
 }
 }  // namespace
 
-static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u64 rescale_counter, bool extended) {
+static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u64 rescale_counter, bool extended,
+                             double scale_override = 0) {
     if (level >= c->nQ) throw RuntimeException("encode: level above the encryption level");
     if (rescale_counter != 0) throw RuntimeException("encode: only rescale counter 0 is supported");
     const size_t n = c->N / 2, M = 2 * c->N;
@@ -603,7 +604,7 @@ static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u6
             }
     }
     bitrev_perm(re, im);
-    const double scale = c->delta[level];
+    const double scale = scale_override != 0 ? scale_override : c->delta[level];
     std::vector<i64> coeffs(c->N);
     for (size_t i = 0; i < n; i++) {
         coeffs[i] = (i64)llround(re[i] / (double)n * scale);
@@ -620,6 +621,7 @@ static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u6
     size_t occupied = n;
     while (occupied > 0 && msg[occupied - 1] == Complex(0, 0)) occupied--;
     pt.occupied_ = occupied;
+    if (scale_override != 0) pt.scale_ = scale_override;
     return pt;
 }
 Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) const {
@@ -627,6 +629,9 @@ Plaintext EnDecoder::encode(const Message &msg, u64 level, u64 rescale_counter) 
 }
 Plaintext EnDecoder::encodeExtended(const Message &msg, u64 level) const {
     return encode_impl(ctx_, msg, level, 0, true);
+}
+Plaintext EnDecoder::encodeExtended(const Message &msg, u64 level, Real scale) const {
+    return encode_impl(ctx_, msg, level, 0, true, (double)scale);
 }
 Plaintext EnDecoder::encode(const Message &msg) const { return encode(msg, getEncryptionLevel(ctx_)); }
 

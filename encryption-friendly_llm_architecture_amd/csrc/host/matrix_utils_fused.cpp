@@ -981,20 +981,43 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
 
 namespace HELLM {
 
-// Plaintext x ciphertext product through the hoisted column shifts of sigma(A) (multMatMatPreFused) and one
-// masked-sum launch that reads tau(B) through each term's automorphism:
-//     rescale(sum_k shift_k(sigma A) (.) rot(tau B, k w)).
-// A row shift of tau(B) is a whole rotation when every tile block of the plaintext (rows * block width slots
-// each) is the same.  The plaintext is known to the host, so the layouts are told apart there:
+// Plaintext x ciphertext product with ONE ModDown.  Every column shift of sigma(A) stays in the extended basis; there
+// it is multiplied by its column mask and by tau(B) rotated k w slots -- tau(B) is a plaintext over the extended basis
+// that the hoisted kernel reads through the term's second automorphism, so the n rotated weights are never
+// materialised -- and all shifts are summed.  The unshifted term P (mask_0 tau(B)) sigma(A) joins on the chain limbs,
+// the sum is divided by P q_{T+2} (ModDown merged with the first rescale) and rescaled once more:
+//     rescale(ModDown(sum_k [mask_k tau(B)_k] (.) KS_k(sigma A))).
+// n - 1 key products, but 1 ModDown instead of n - 1 and no ciphertext ever leaves the extended basis in between.
+// A row shift of tau(B) is a whole rotation when every tile block of the plaintext (rows * block width slots each)
+// is the same.  The plaintext is known to the host, so the layouts are told apart there:
 //   * one tile block fills the slot vector (pair layout), or all blocks are equal: as written above;
 //   * only the first block is non-zero (HEMMer::encode of a single matrix): tau(B) is copied into every block
 //     and the column-shift masks are restricted to the first block, so the product stays empty elsewhere
 //     whatever the ciphertext carries there;
 //   * anything else (different matrices stacked in one plaintext) returns false: the caller takes the
 //     reference-order product.
+// tau(B) is prepared once per weight (decode, permute, encode on the host as MatrixTransformer::diagonalToRow<Plaintext>
+// does) and kept under a hash of the weight's residues.
+namespace {
+u64 hashResidues(const Context &c, const Plaintext &pt) {
+    // limb 0 determines the plaintext (its coefficients are far below q_0 / 2)
+    std::vector<u64> h(c->N);
+    if (hipMemcpy(h.data(), pt.buf_.data(), h.size() * 8, hipMemcpyDeviceToHost) != hipSuccess)
+        throw RuntimeException("hipMemcpy");
+    u64 x = 0xcbf29ce484222325ull ^ pt.getLevel();
+    for (u64 v : h) {
+        x ^= v;
+        x *= 0x100000001b3ull;
+        x ^= x >> 29;
+    }
+    return x;
+}
+}  // namespace
+
 bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const PtxtTensor &op2,
                           u64 T, MatrixTransformer &tr, u64 batch, CtxtTensor &res_out) {
     const Context &c = eval.getContext();
+    (void)batch;
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
     if (std::min(op1.getLevel(), op2.getLevel()) < 1 + btp.getMinLevelForBootstrap())
@@ -1002,38 +1025,109 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
                                     " is needed.");
     const i64 slots = (i64)(c->N / 2), block = k * w;
     if (block > slots || slots % block != 0) return false;
-    CtxtTensor a{op1};
-    PtxtTensor b{op2};
-    a.setShape(rows, k);
-    b.setShape(k, cols);
-    // tau on the plaintext: decode once, permute the values (MatrixTransformer::diagonalToRow<Plaintext>), encode
-    // directly at the level the shifts live at
-    EnDecoder endec(c);
-    const Message src = endec.decode(b.get());
-    // decoded values carry the encoding's rounding noise (about sqrt(N) / 2^43 at this scale): "zero" and "equal"
-    // are taken up to 2^-24
-    const double tol = std::ldexp(1.0, -24);
-    bool rest_zero = true, rest_equal = true;
-    for (i64 j = block; j < slots && (rest_zero || rest_equal); j++) {
-        if (std::abs(src[(u64)j]) >= tol) rest_zero = false;
-        if (std::abs(src[(u64)j] - src[(u64)(j % block)]) >= tol) rest_equal = false;
-    }
-    if (!rest_zero && !rest_equal) return false;
-    const bool first_block_only = rest_zero && block < slots;
-    Message dst(src.getLogSlots(), 0);
-    const i64 height = slots / w;
-    for (i64 r = 0; r < height; r++)
-        for (i64 cc = 0; cc < w; cc++) {
-            const i64 cb = cc - cc % k, i = r % k, j = cc % k;
-            const i64 rb = first_block_only ? 0 : r - r % k;   // single matrix: every block takes the first one's tau
-            dst[(u64)(r * w + cc)] = src[(u64)((rb + (i + j) % k) * w + cb + j)];
+    if (op1.getLevel() < T + 3)
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
+    const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
+    // ---- tau(B) over the extended basis at level T+2, scaled like a plaintext of level T+1
+    const auto key = std::make_tuple(hashResidues(c, op2.get()), shape_b, T);
+    auto it = tr.weight_tau_.find(key);
+    if (it == tr.weight_tau_.end()) {
+        EnDecoder endec(c);
+        const Message src = endec.decode(op2.get());
+        // decoded values carry the encoding's rounding noise (about sqrt(N) / 2^43 at this scale): "zero" and "equal"
+        // are taken up to 2^-24
+        const double tol = std::ldexp(1.0, -24);
+        bool rest_zero = true, rest_equal = true;
+        for (i64 j = block; j < slots && (rest_zero || rest_equal); j++) {
+            if (std::abs(src[(u64)j]) >= tol) rest_zero = false;
+            if (std::abs(src[(u64)j] - src[(u64)(j % block)]) >= tol) rest_equal = false;
         }
-    b.get() = endec.encode(dst, T + 1);
-    if (a.getLevel() < 4 + btp.getMinLevelForBootstrap()) btp.bootstrapExtended(a.get(), a.get());
-    std::vector<Ciphertext> shifts;
-    multMatMatPreFused(eval, a, shifts, T, tr, batch, first_block_only);
+        MatrixTransformer::WeightTau entry{Plaintext(c), 0};
+        if (rest_zero || rest_equal) {
+            const bool first_only = rest_zero && block < slots;
+            Message dst(src.getLogSlots(), 0);
+            const i64 height = slots / w;
+            for (i64 r = 0; r < height; r++)
+                for (i64 cc = 0; cc < w; cc++) {
+                    const i64 cb = cc - cc % k, i = r % k, j = cc % k;
+                    const i64 rb = first_only ? 0 : r - r % k;   // single matrix: every block takes the first one's tau
+                    dst[(u64)(r * w + cc)] = src[(u64)((rb + (i + j) % k) * w + cb + j)];
+                }
+            entry.tau = endec.encodeExtended(dst, T + 2, c->delta[T + 1]);
+            entry.layout = first_only ? 2 : 1;
+        }
+        if (tr.weight_tau_order_.size() >= 256) {   // bounded: the oldest weight is prepared again if it comes back
+            tr.weight_tau_.erase(tr.weight_tau_order_.front());
+            tr.weight_tau_order_.erase(tr.weight_tau_order_.begin());
+        }
+        tr.weight_tau_order_.push_back(key);
+        it = tr.weight_tau_.emplace(key, std::move(entry)).first;
+    }
+    if (it->second.layout == 0) return false;
+    const bool first_block_only = it->second.layout == 2;
+    const Plaintext &tau = it->second.tau;
+    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2, first_block_only);
+    // ---- sigma(A) at level T+2 and its two rotation sources
+    const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
+    Ciphertext own_a(c);
+    const Ciphertext *pa = &op1.get();
+    if (pa->getLevel() < 4 + btp.getMinLevelForBootstrap()) {
+        own_a = *pa;
+        btp.bootstrapExtended(own_a, own_a);
+        pa = &own_a;
+    }
+    const Ciphertext sa = tr.lowerAndTransformFused(eval, *pa, MaskKind::Horizontal, shape_a, T + 2);
+    const Sources x = extendSources(c, sa.buf_.data(), 1, nq);
+    const i64 back = -k;
+    const DeviceBuffer a2 = rotateSources(eval, x, sa.buf_.data(), 1, &back);
+    const Sources x2 = extendSources(c, a2.data(), 1, nq);
+    // ---- all shifts as terms of one sum, dealt to `parts` partial outputs
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    const u64 n_shift = (u64)(k - 1);
+    const u64 parts = std::max<u64>(1, std::min<u64>(16, n_shift));
+    DeviceBuffer y(c, 2 * E * N);
+    if (n_shift > 0) {
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        for (u64 p = 0; p < parts; p++) {
+            for (u64 i = 1 + p * n_shift / parts; i < 1 + (p + 1) * n_shift / parts; i++) {
+                const u64 g = rot.galois((i64)i), gp = rot.galois((i64)i * w);
+                hemm_rot_term t1 = term(x.extOf(0), x.pbOf(0), pack, g, &cm[(size_t)(2 * i + 1)]);
+                hemm_rot_term t2 = term(x2.extOf(0), x2.pbOf(0), pack, g, &cm[(size_t)(2 * i)]);
+                t1.pt = t2.pt = tau.buf_.data();
+                t1.pt_galois = t2.pt_galois = (uint32_t)gp;
+                terms.push_back(t1);
+                terms.push_back(t2);
+            }
+            off.push_back((uint32_t)terms.size());
+        }
+        DeviceBuffer yp(c, parts * 2 * E * N);
+        ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)parts, (uint32_t)nq, yp.data(), 1, nullptr));
+        ck(hemm_sum_parts(c->dev, yp.data(), (uint32_t)parts, 1, (uint32_t)nq, y.data(), nullptr));
+    } else {
+        (void)hipMemsetAsync(y.data(), 0, 2 * E * N * 8, nullptr);
+    }
+    // ---- shift 0: P (mask_0 tau(B)) sigma(A) on the chain limbs
+    {
+        DeviceBuffer m0(c, nq * N), t0(c, 2 * nq * N);
+        ck(hemm_pointwise(c->dev, HEMM_MUL, cm[1].buf_.data(), 0, tau.buf_.data(), 0, m0.data(), 0, (uint32_t)nq, 0, 1, nullptr));
+        ck(hemm_pointwise(c->dev, HEMM_MUL, sa.buf_.data(), nq * N, m0.data(), 0, t0.data(), nq * N, (uint32_t)nq, 0, 2, nullptr));
+        std::vector<u64> sc(nq);
+        for (u64 j = 0; j < nq; j++) {
+            u64 P = 1;
+            for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
+            sc[j] = P;
+        }
+        ck(hemm_mul_scalar(c->dev, t0.data(), nq * N, sc.data(), t0.data(), nq * N, (uint32_t)nq, 0, 2, nullptr));
+        ck(hemm_pointwise(c->dev, HEMM_ADD, y.data(), E * N, t0.data(), nq * N, y.data(), E * N, (uint32_t)nq, 0, 2, nullptr));
+    }
+    // ---- one ModDown merged with the first rescale, then the second rescale
+    DeviceBuffer mid(c, 2 * lo * N), ws(c, 2 * lo * N);
+    ck(hemm_moddown_batch(c->dev, y.data(), (uint32_t)nq, 2, 1, mid.data(), lo * N, ws.data(), nullptr));
     CtxtTensor res(c, rows, cols, w);
-    eval.matmul(shifts, b.get(), res.get(), (u64)w);
+    res.get().allocate(2, T, 0);
+    ck(hemm_rescale(c->dev, mid.data(), lo * N, res.get().buf_.data(), (lo - 1) * N, (uint32_t)lo, 2, nullptr));
     res_out = res;
     return true;
 }

@@ -1065,6 +1065,31 @@ bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shif
     HEMM_HIP(hipFree(flag));
     return h == 0;
 }
+// sum of `parts` consecutive partial results per output over the extended basis, residue pairs, canonical in and out
+__global__ __launch_bounds__(256) void sum_parts_kernel(const u64 *__restrict__ part, int parts, u64 *__restrict__ y,
+                                                        const ModQ *__restrict__ modq, LimbList ll, int E, int logN,
+                                                        size_t pairs) {
+    const size_t N = (size_t)1 << logN, poly_limbs = (size_t)2 * E;
+    const size_t pair = (size_t)blockIdx.x * 256 + threadIdx.x;     // over [n_out][2][E][N/2]
+    if (pair >= pairs) return;
+    const size_t limb = (pair * 2) >> logN;                         // (o * 2 + p) * E + j
+    const size_t o = limb / poly_limbs, within = limb % poly_limbs;
+    const u64 q = modq[ll.idx[within % E]].q;
+    const size_t e = within * N + ((pair * 2) & (N - 1));
+    u64 a0 = 0, a1 = 0;
+    for (int k = 0; k < parts; k++) {
+        const ulonglong2 v = stream_load2(part + ((o * parts + k) * poly_limbs) * N + e);
+        a0 = addmod(a0, v.x, q);
+        a1 = addmod(a1, v.y, q);
+    }
+    stream_store2(y + (o * poly_limbs) * N + e, a0, a1);
+}
+void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s) {
+    const int E = nq + c->nP;
+    const size_t pairs = (size_t)n_out * 2 * E * (c->N / 2);
+    hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s, part, parts, y, c->d_modq,
+                       limbs_default(c, nq, 1), E, c->logN, pairs);
+}
 // the same with the term list in host memory (n_terms, n_out <= masked_arg_capacity()), passed in the kernel arguments
 int masked_arg_capacity() { return MASKED_ARG_TERMS; }
 void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,

@@ -137,6 +137,12 @@ typedef struct {
     uint32_t pt_galois;   /* odd, < 2N; 1 = as stored */
     uint32_t reserved;    /* 0 */
 } hemm_rot_term;
+/* y[o] = sum of the n_parts consecutive partial sums parts[o * n_parts .. ) of hemm_hoisted_terms, limb-wise over the
+ * extended basis; y: [n_out][2][nq+n_p][N], parts: [n_out * n_parts][2][nq+n_p][N].  A sum with one output and many
+ * terms is split over several partial outputs (more workgroups, more keys in flight) and added up here before its
+ * single ModDown.  No counterpart in HEaaN's interface. */
+int hemm_sum_parts(hemm_context *ctx, const uint64_t *parts, uint32_t n_parts, uint32_t n_out, uint32_t nq, uint64_t *y,
+                   void *stream);
 /* Run table of a mask that is constant over aligned runs of 2^shift coefficients: table[j][r] = mask[j][r << shift]
  * for n_limbs limbs; *is_constant = 0 (and the table is not to be used) when some run of the mask is not constant.
  * Synchronises the stream.  No counterpart in HEaaN's interface: it removes the mask traffic of hoisted sums whose

@@ -817,6 +817,56 @@ def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
     return mult_mat_mat_reuse(ev, tmp, b, T, step=w)
 
 
+def mult_mat_mat_pc_lazy(orc, a, b_pt, T, n, w):
+    """Plaintext x ciphertext product with ONE ModDown: every column shift of sigma(A) stays in the extended basis,
+    is multiplied there by its column mask and by tau(B) rotated k w slots (a plaintext over the extended basis,
+    encoded at the scale of level T+1), all n - 1 shifts are summed, the unshifted term P * (mask_0 tau(B)) sigma(A)
+    is added on the chain limbs, and the sum is divided by P q_{T+2} (ModDown merged with the first rescale) and
+    rescaled once more.  Same layout rules as mult_mat_mat_pc_fused; None for other plaintexts."""
+    from .oracle import Ct, Pt
+    ev = OracleEval(orc)
+    slots, block = orc.slots, n * w
+    if block > slots or slots % block:
+        return None
+    v = ev.pt_values(b_pt)
+    blocks = v.reshape(slots // block, block)
+    tol = 2.0 ** -24
+    rest_zero = bool(np.all(np.abs(blocks[1:]) < tol))
+    rest_equal = bool(np.all(np.abs(blocks[1:] - blocks[0]) < tol))
+    if not (rest_zero or rest_equal):
+        return None
+    first_block_only = rest_zero and block < slots
+    if first_block_only:
+        v = np.tile(blocks[0], slots // block)
+    masks = col_masks(n, slots)
+    if first_block_only:
+        keep = np.zeros(slots, dtype=np.complex128)
+        keep[: min(block, slots)] = 1
+        masks = [m * keep for m in masks]
+    cm = [orc.encode_ext(m, T + 2) for m in masks]
+    tau = orc.encode_ext(tau_plain(v, n, w), T + 2, scale=orc.delta[T + 1])
+    a = lower_and_transform_fused(orc, a, H, n, w, T + 2)
+    nq = a.nq
+    ext = orc.modup(a.data[1])
+    a2 = _rotated_copy(orc, a, ext, -n)
+    ext2 = orc.modup(a2.data[1])
+    terms = []
+    for i in range(1, n):
+        gp = orc.galois((i * w) % slots)
+        terms.append((ext, a.data[0], i % slots, orc.ext_plain_product(cm[2 * i + 1], tau, gp)))
+        terms.append((ext2, a2.data[0], i % slots, orc.ext_plain_product(cm[2 * i], tau, gp)))
+    y = orc.hoisted_sum(terms, nq)
+    # shift 0: P * (mask_0 * tau(B)) * sigma(A) on the chain limbs (zero on the special limbs)
+    m0 = orc.ext_plain_product(cm[1], tau, 1)
+    t0 = orc.mult_plain_no_rescale(a, Pt(m0.data[:nq], m0.scale))
+    for pol in range(2):
+        y[pol, :nq] = orc.add_residues(y[pol, :nq], orc.mul_p_residues(np.ascontiguousarray(t0.data[pol])))
+    mid = Ct(orc.moddown_drop(y, nq, True), orc.delta[T + 1] * orc.delta[T + 1])
+    res = orc.rescale(mid)
+    res.scale = orc.delta[T]
+    return res
+
+
 def weights_diagonal_to_row4(w1, w2, w3, w4, slots):
     """HEMMer::msgDiagonalToRow4 (HEMMer.cpp:353-399)."""
     h, w = w1.shape

@@ -198,7 +198,7 @@ def test_pcmm_pair_layout(small, fused):
     H.set_schedule(True)
     opb = O.Pt(pb.residues(), orc.delta[orc.nQ - 1])
     oa = to_oracle(orc, ca)
-    want = R.mult_mat_mat_pc_fused(orc, oa, opb, 2, 16, 32) if fused else R.mult_mat_mat_pc(ev, oa, opb, 2, 16, 32)
+    want = R.mult_mat_mat_pc_lazy(orc, oa, opb, 2, 16, 32) if fused else R.mult_mat_mat_pc(ev, oa, opb, 2, 16, 32)
     assert np.array_equal(c.residues(), want.data)
     d = H.decrypt2(c)
     assert np.abs(d[0] - A1 @ B1).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
@@ -228,7 +228,7 @@ def test_pcmm_and_packed_bit_exact(small, fused):
     c = H.single_matmul(ca, pb, 2)
     opb = O.Pt(pb.residues(), orc.delta[orc.nQ - 1])
     if fused:   # single matrix in the first tile block: tau(B) copied into every block, masks on the first block
-        want = R.mult_mat_mat_pc_fused(orc, to_oracle(orc, ca), opb, 2, 16, 16)
+        want = R.mult_mat_mat_pc_lazy(orc, to_oracle(orc, ca), opb, 2, 16, 16)
     else:
         want = R.mult_mat_mat_pc(ev, to_oracle(orc, ca), opb, 2, 16, 16)
     assert np.array_equal(c.residues(), want.data)
