@@ -152,18 +152,20 @@ def gpu_ntt(args, out):
     }
 
 
-# HBM bytes per launch of hoisted_terms_kernel at the shape below, from two rocprofv3 --pmc runs of
-# `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
+# HBM bytes per call of the hoisted sum at the shape below (its two launches together), from two rocprofv3 --pmc runs
+# of `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # 1 GiB copy this mode also launches (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0):
-# (2 x 570 495.7 + 360 448) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
-HOISTED_TRAFFIC_BYTES = 1537473946
+# (2 x (208 965.9 + 172 138.5) + 196 608 + 163 840) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
+HOISTED_TRAFFIC_BYTES = 1149600563
 
 
 def gpu_hoisted(args, out):
-    """Roofline of the dominant kernel, hoisted_terms_kernel, at the shape of the CCMM's main loop: one
-    launch produces 16 column shifts of sigma(A) and 16 row shifts of tau(B) in the extended basis, each
-    the sum of two masked hoisted rotations (of the operand and of its copy rotated by -n) under one
-    key (7 chain + 4 special limbs, 2 digits)."""
+    """Roofline of the dominant kernels, the hoisted sum of the CCMM's main loop: one call produces 32 column shifts
+    of sigma(A) in the extended basis, each the sum of two masked hoisted rotations (of the operand and of its
+    copy rotated by -n) under one key (7 chain + 4 special limbs, 2 digits).  The column masks are run tables (their
+    NTT form is constant over runs of 256 residues), and a call of this size is two launches over disjoint limbs:
+    hoisted_terms_kernel<1> (the 6 limbs of primes below 2^44, double precision) and hoisted_terms_kernel<2> (the 5
+    limbs of 60-bit primes, integer).  Timed together: the figure is per call."""
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -172,19 +174,18 @@ def gpu_hoisted(args, out):
     qs = [big[0]] + pkg.primes_below(42, 16, 12)
     ps = big[1:]
     ctx = pkg.Context(16, qs, ps, dnum)
-    N, E, T, beta = 1 << 16, nq + K, 13 + K, 2
+    N, E, T, beta, shift = 1 << 16, nq + K, 13 + K, 2, 8
     g = torch.Generator(device="cuda").manual_seed(11)
 
     def rnd(*shape):
         # residues below 2^41 are valid for every prime of the set; the kernel's work does not depend on values
         return torch.randint(0, 2 ** 41, shape, dtype=torch.int64, device="cuda", generator=g)
 
-    src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(4)]
+    src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(2)]
     groups = []
     for o in range(n_out):
-        side = o // (n_out // 2)
         evk, gal = rnd(dnum, 2, T, N), pow(5, o + 1, 2 * N)
-        groups.append([(src[2 * side + t][0], src[2 * side + t][1], evk, rnd(E, N), gal) for t in range(2)])
+        groups.append([(src[t][0], src[t][1], evk, rnd(E, N >> shift), gal, shift) for t in range(2)])
     for _ in range(2):
         ctx.hoisted_terms(groups, nq, b_premultiplied=True)
     torch.cuda.synchronize()
@@ -194,14 +195,15 @@ def gpu_hoisted(args, out):
     for _ in range(iters):
         ctx.hoisted_terms(groups, nq, b_premultiplied=True)
     ms = timer.stop() / iters
-    # algorithmic bytes: per output beta x 2 x E key limbs + 2 x E mask limbs read + 2 x E limbs written;
-    # the four rotation sources (beta x E + nq limbs each) read once per launch
-    limbs = n_out * (beta * 2 * E + 2 * E + 2 * E) + 4 * (beta * E + nq)
-    alg_bytes = limbs * LIMB_BYTES
+    # algorithmic bytes: per output beta x 2 x E key limbs read + 2 x E limbs written (the mask tables are
+    # 2 x E x 2 KiB per output: counted, negligible); the two rotation sources (beta x E + nq limbs each) read once
+    limbs = n_out * (beta * 2 * E + 2 * E) + 2 * (beta * E + nq)
+    alg_bytes = limbs * LIMB_BYTES + n_out * 2 * E * (N >> shift) * 8
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     out["roofline"] = {
-        "kernel": "hoisted_terms_kernel (32 outputs x 2 masked sources under one key, 7+4 limbs, 2 digits: "
-                  "one batch of the CCMM main loop)",
+        "kernel": "hoisted_terms_kernel<1> + hoisted_terms_kernel<2> (one hoisted sum of the CCMM main loop: 32 outputs x "
+                  "2 masked sources under one key, 7+4 limbs, 2 digits, run-table masks; double-precision limbs and "
+                  "integer limbs in one launch each)",
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS, "traffic": HOISTED_TRAFFIC_BYTES,
         "algorithmic_bytes_per_launch": alg_bytes, "avg_ms_per_launch": ms,
