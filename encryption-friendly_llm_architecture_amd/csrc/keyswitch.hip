@@ -761,7 +761,7 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
     u64 *coef = sc;                              // [nq][N]   (reused as conv[2][nq] needs 2*nq)
     u64 *ext = coef + (size_t)2 * (c->nQ) * N;   // [beta][E][N]
     u64 *acc = ext + (size_t)beta * E * N;       // [2][E][N]
-    launch_modup(c, in, nq, ext, coef, false, s);
+    launch_modup_batch(c, in, (size_t)nq * N, nq, 1, ext, coef, s);   // same arithmetic as launch_modup, 5 launches
     launch_inner_product(c, in, ext, evk, nq, acc, s);
     launch_moddown(c, acc, nq, 2, out, out_stride, add_b, 0, add_b ? 1 : 0, coef, s);
 }

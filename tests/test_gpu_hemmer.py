@@ -204,6 +204,27 @@ def test_pcmm_pair_layout(small, fused):
     assert np.abs(d[0] - A1 @ B1).max() < 2 ** -18 and np.abs(d[1] - A2 @ B2).max() < 2 ** -18
 
 
+def test_pcmm_weight_preparation_follows_the_weight_content(small):
+    """The batched plaintext product keeps tau of a weight under a hash of the weight's residues: the same weight gives
+    the same residues on every call, and another weight -- also one that lands in the device buffer the first one
+    left -- gives its own product."""
+    H, orc, ev = small
+    H.set_schedule(True)
+    rng = np.random.default_rng(21)
+    A, B1, B2 = (rng.uniform(-1, 1, (16, 16)) for _ in range(3))
+    ca = H.encrypt(A)
+    p1 = H.encode(B1)
+    first = H.single_matmul(ca, p1, 2).residues()
+    again = H.single_matmul(ca, p1, 2).residues()
+    assert np.array_equal(first, again)
+    del p1
+    p2 = H.encode(B2)
+    c2 = H.single_matmul(ca, p2, 2)
+    assert np.abs(H.decrypt(c2) - A @ B2).max() < 2 ** -20
+    p1 = H.encode(B1)
+    assert np.array_equal(H.single_matmul(ca, p1, 2).residues(), first)
+
+
 def test_batch_size_does_not_change_residues(small):
     H, _, _ = small
     rng = np.random.default_rng(14)
