@@ -185,6 +185,11 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vect
 // plaintext x ciphertext product through the hoisted column shifts (see matrix_utils_fused.cpp for the layouts it takes)
 bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const PtxtTensor &op2,
                           u64 target_level, MatrixTransformer &transformer, u64 batch, CtxtTensor &res);
+// sum_k tmp[k] (x) rho^(k step)(b), relinearised (and rescaled when rescale_after): the ciphertext x ciphertext re-use
+// forms (multMatMatCCReUse: step = block width; multPackedMatMatCCReuse: step = 2 block widths, rescale) with all
+// rotations of b taken from ONE ModUp through direct keys, in batches of hoisted sums
+CtxtTensor multMatMatCCReUseFused(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
+                                  u64 step, bool rescale_after, u64 batch = 16);
 // left rotations (in slots) whose direct keys the batched schedules use
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 // the same for multMatMatFused; square_rots receives the giant steps that also need KeyPack::galoisSquareKey

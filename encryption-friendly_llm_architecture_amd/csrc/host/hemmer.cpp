@@ -464,9 +464,22 @@ void HEMMer::packedMatMulPreRot(const CtxtTensor &a, std::vector<Ciphertext> &tm
 }
 CtxtTensor HEMMer::packedMatMulPreRev(const CtxtTensor &b, u64 T) const {
     ensureRotationKeys(transformRotations(MaskKind::PackedVertical, b.getBlockWidth()));
+    if (fused_ && b.getLevel() >= T + 2) {   // tau through the batched launches (two stages with a level to spare)
+        CtxtTensor res(b);
+        res.setShape(pow2ceil(b.getHeight()), b.getWidth());
+        res.get() = matrix_transformer.lowerAndTransformFused(eval_, b.get(), MaskKind::PackedVertical, res.getShape(), T + 1);
+        return res;
+    }
     return multPackedMatMatPreRev(eval_, b, T, matrix_transformer);
 }
 CtxtTensor HEMMer::packedMatMulCCReuse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 T) const {
+    if (fused_ && tmp.size() > 1) {
+        const u64 step = (u64)(2 * b.getBlockWidth());
+        std::vector<u64> rots;
+        for (size_t k = 1; k < tmp.size(); k++) rots.push_back((k * step) % (u64(1) << log_slots_));
+        ensureRotationKeys(rots);
+        return multMatMatCCReUseFused(eval_, tmp, b, step, true, batch_);
+    }
     ensureRotationKeys({(u64)(2 * b.getBlockWidth())});
     return multPackedMatMatCCReuse(eval_, tmp, b, T, matrix_transformer);
 }
@@ -486,9 +499,21 @@ CtxtTensor HEMMer::matMulReUse(const std::vector<Ciphertext> &tmp, const PtxtTen
 }
 CtxtTensor HEMMer::matMulPreRev(const CtxtTensor &b, u64 T) const {
     ensureRotationKeys(transformRotations(MaskKind::Vertical, b.getBlockWidth()));
+    if (fused_ && b.getLevel() >= T + 2) {
+        CtxtTensor res(b);
+        res.get() = matrix_transformer.lowerAndTransformFused(eval_, b.get(), MaskKind::Vertical, b.getShape(), T + 1);
+        return res;
+    }
     return multMatMatPreRev(eval_, b, T, matrix_transformer);
 }
 CtxtTensor HEMMer::matMulCCReUse(const std::vector<Ciphertext> &tmp, const CtxtTensor &b, u64 T) const {
+    if (fused_ && tmp.size() > 1) {
+        const u64 step = (u64)b.getBlockWidth();
+        std::vector<u64> rots;
+        for (size_t k = 1; k < tmp.size(); k++) rots.push_back((k * step) % (u64(1) << log_slots_));
+        ensureRotationKeys(rots);
+        return multMatMatCCReUseFused(eval_, tmp, b, step, false, batch_);
+    }
     ensureRotationKeys({(u64)b.getBlockWidth()});
     return multMatMatCCReUse(eval_, tmp, b, T, matrix_transformer);
 }

@@ -981,6 +981,51 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
 
 namespace HELLM {
 
+// Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and
+// b = tau(B).  The reference rotates b by `step` in a chain, one key switch after the other; here every rotation
+// comes from the same ModUp of b through its direct key (hoisted), 2 * batch rotations per launch chain with one
+// plain ModDown for all of them.  The accumulator stays un-relinearised until the end.
+CtxtTensor multMatMatCCReUseFused(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
+                                  u64 step, bool rescale_after, u64 batch) {
+    const Context &c = eval.getContext();
+    if (tmp.empty()) throw std::invalid_argument("[multMatMatCCReUse] no shifted operands.");
+    const u64 level = b.getLevel(), nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
+    for (const Ciphertext &t : tmp)
+        if (t.getLevel() != level || t.getNumPoly() != 2 || t.getRescaleCounter() != b.get().getRescaleCounter())
+            throw std::invalid_argument("[multMatMatCCReUse] operands must share one level.");
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    Ciphertext acc(c);
+    acc.allocate(3, level, b.get().getRescaleCounter() + 1);
+    ck(hemm_tensor_batch(c->dev, tmp[0].buf_.data(), b.get().buf_.data(), 1, (uint32_t)nq, acc.buf_.data(), 0, nullptr));
+    const size_t n_rot = tmp.size() - 1;
+    if (n_rot > 0) {
+        const Sources xb = extendSources(c, b.get().buf_.data(), 1, nq);
+        const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)n_rot));
+        DeviceBuffer y(c, G * 2 * E * N), rb(c, G * ctw), ws(c, G * ctw);
+        for (size_t first = 0; first < n_rot; first += G) {
+            const size_t cnt = std::min(G, n_rot - first);
+            std::vector<hemm_rot_term> terms;
+            std::vector<uint32_t> off{0};
+            for (size_t q = 0; q < cnt; q++) {
+                const i64 amount = (i64)((first + q + 1) * step);
+                if (rot.norm(amount) == 0) throw std::invalid_argument("[multMatMatCCReUse] rotation by a whole turn.");
+                terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(amount), nullptr));
+                off.push_back((uint32_t)terms.size());
+            }
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 0, y.data(), rb.data(),
+                                    nq * N, ws.data(), nullptr));
+            for (size_t q = 0; q < cnt; q++)
+                ck(hemm_tensor_batch(c->dev, tmp[first + q + 1].buf_.data(), rb.data() + q * ctw, 1, (uint32_t)nq,
+                                     acc.buf_.data(), 1, nullptr));
+        }
+    }
+    CtxtTensor res(c, b.getHeight(), b.getWidth(), b.getBlockWidth());
+    eval.relinearize(acc, res.get());
+    if (rescale_after) eval.rescale(res.get());
+    return res;
+}
+
 // Plaintext x ciphertext product with ONE ModDown.  Every column shift of sigma(A) stays in the extended basis; there
 // it is multiplied by its column mask and by tau(B) rotated k w slots -- tau(B) is a plaintext over the extended basis
 // that the hoisted kernel reads through the term's second automorphism, so the n rotated weights are never

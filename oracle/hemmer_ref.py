@@ -817,6 +817,20 @@ def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
     return mult_mat_mat_reuse(ev, tmp, b, T, step=w)
 
 
+def mult_mat_mat_cc_reuse_fused(orc, tmp, b, step, rescale_after=False):
+    """Batched ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b), every rotation of b taken from
+    one ModUp through its direct key (automorphism after ModUp, plain ModDown), relinearised at the end (packed
+    form: rescaled as well)."""
+    from .oracle import Ct
+    ext = orc.modup(b.data[1])
+    acc = orc.tensor(tmp[0], b)
+    for k in range(1, len(tmp)):
+        y = orc.hoisted_sum([(ext, b.data[0], (k * step) % orc.slots, None)], b.nq)
+        acc = orc.add(acc, orc.tensor(tmp[k], Ct(orc.moddown_drop(y, b.nq, False), b.scale)))
+    res = orc.relinearize(acc)
+    return orc.rescale(res) if rescale_after else res
+
+
 def mult_mat_mat_pc_lazy(orc, a, b_pt, T, n, w):
     """Plaintext x ciphertext product with ONE ModDown: every column shift of sigma(A) stays in the extended basis,
     is multiplied there by its column mask and by tau(B) rotated k w slots (a plaintext over the extended basis,

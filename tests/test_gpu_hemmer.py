@@ -314,6 +314,11 @@ def test_reuse_variants_and_repacking(small, fused):
     c = H.matmul_cc_reuse(tmp, bt, T)
     d = H.decrypt2(c)
     assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    if fused:   # tau(B) through the batched transform, then all its rotations from one ModUp: residues
+        assert np.array_equal(bt.residues(), R.lower_and_transform_fused(orc, to_oracle(orc, b), R.V, n, 2 * n, T + 1).data)
+        otmp = [to_oracle(orc, tmp.get(k, n, n, 2 * n)) for k in range(len(tmp))]
+        want = R.mult_mat_mat_cc_reuse_fused(orc, otmp, to_oracle(orc, bt), 2 * n)
+        assert np.array_equal(c.residues(), want.data)
     # packed counterparts: the same product as packedMatMul
     pa, pb = H.encrypt2(A0, A1), H.encrypt2(B0, B1)
     H.complex_packing_inplace(pa)
@@ -321,9 +326,15 @@ def test_reuse_variants_and_repacking(small, fused):
     sa = H.packed_matmul_pre(pa, T)
     ptmp = H.packed_matmul_pre_rot(sa, T)
     pbt = H.packed_matmul_pre_rev(pb, T)
-    pc = H.repack_cc(H.packed_matmul_cc_reuse(ptmp, pbt, T))
+    pprod = H.packed_matmul_cc_reuse(ptmp, pbt, T)
+    pc = H.repack_cc(pprod)
     d = H.decrypt2(pc)
     assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    if fused:
+        assert np.array_equal(pbt.residues(), R.lower_and_transform_fused(orc, to_oracle(orc, pb), R.PV, n, 2 * n, T + 1).data)
+        optmp = [to_oracle(orc, ptmp.get(k, n, n, 2 * n)) for k in range(len(ptmp))]
+        want = R.mult_mat_mat_cc_reuse_fused(orc, optmp, to_oracle(orc, pbt), 4 * n, rescale_after=True)
+        assert np.array_equal(pprod.residues(), want.data)
     H.set_schedule(True)
     # splitInTwo: [A0 | A1] -> [A0 | A0], [A1 | A1]
     t1, t2 = H.split_in_two(H.encrypt2(A0, A1))
