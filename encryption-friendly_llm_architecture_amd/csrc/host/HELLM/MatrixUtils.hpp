@@ -19,7 +19,9 @@
 
 namespace HELLM {
 
-enum class MaskKind { Horizontal, Vertical, PackedHorizontal, PackedVertical, Diagonal };
+// DiagonalSigned: the transpose's diagonals grouped the way sigma / tau group theirs (positive and negative diagonals in
+// separate giant-step groups), which is what the batched transform walks; Diagonal keeps the reference's grouping.
+enum class MaskKind { Horizontal, Vertical, PackedHorizontal, PackedVertical, Diagonal, DiagonalSigned };
 
 // 0/1 (or 0.5) slot pattern of diagonal `idx` for a transform kind, before any pre-rotation.
 // Horizontal (sigma): rows r with r mod n == idx take columns [0, n - idx); negative idx = the wrapped

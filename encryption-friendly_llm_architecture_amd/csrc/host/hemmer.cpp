@@ -335,6 +335,26 @@ std::vector<Matrix> HEMMer::decrypt2(const CtxtTensor &t) const {
 
 // ---- packing ---------------------------------------------------------------------------------------------
 void HEMMer::transposeInplace(CtxtTensor &t, u64 target_level) const {
+    if (fused_ && t.getHeight() == t.getWidth() && t.getHeight() == dim_) {
+        // batched: the 2n - 1 diagonals through the same launch chain as sigma / tau (hoisted baby steps, one masked-sum
+        // launch, giant steps summed before one ModDown)
+        const u64 slots = u64(1) << log_slots_;
+        const i64 n = dim_, step = t.getBlockWidth() - 1;
+        const i64 bs = (i64)std::ceil(std::sqrt((double)(2 * n - 1))), gs = (i64)std::ceil((double)(n - 1) / (double)bs);
+        std::vector<u64> r;
+        auto left = [&](i64 v) { r.push_back((u64)(((v % (i64)slots) + (i64)slots) % (i64)slots)); };
+        for (i64 j = 0; j < bs; j++) left((j + 1) * step);
+        for (i64 i = 0; i < gs; i++) {
+            left(-(n - i * bs) * step);
+            if (i > 0) left(i * bs * step);
+        }
+        ensureRotationKeys(r);
+        if (target_level > 0) eval_.levelDown(t.get(), 1 + target_level, t.get());
+        const TileTensorShape shape(t.getWidth(), t.getHeight(), t.getBlockWidth());
+        Ciphertext out = matrix_transformer.diagonalTransformFused(eval_, t.get(), MaskKind::DiagonalSigned, shape);
+        t = CtxtTensor(shape, out);
+        return;
+    }
     ensureRotationKeys(transformRotations(MaskKind::Diagonal, t.getBlockWidth()));
     if (target_level > 0) eval_.levelDown(t.get(), 1 + target_level, t.get());
     t = matrix_transformer.transpose(eval_, t);

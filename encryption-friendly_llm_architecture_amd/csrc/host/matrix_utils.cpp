@@ -56,7 +56,7 @@ Geometry geometry(MaskKind kind, const TileTensorShape &s) {
     g.sub = std::min(rows, cols) / g.cell;
     g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.sub - 1)));
     g.gs = (i64)std::ceil((double)(g.sub - 1) / (double)g.bs);
-    g.step = g.cell * (vertical ? w : 1);
+    g.step = kind == MaskKind::DiagonalSigned ? w - 1 : g.cell * (vertical ? w : 1);
     return g;
 }
 

@@ -62,7 +62,10 @@ Geo geo(MaskKind kind, const TileTensorShape &s) {
     g.sub = std::min(rows, cols) / g.cell;
     g.bs = (i64)std::ceil(std::sqrt((double)(2 * g.sub - 1)));
     g.gs = (i64)std::ceil((double)(g.sub - 1) / (double)g.bs);
-    g.step = g.cell * (vertical ? w : 1);
+    g.step = kind == MaskKind::DiagonalSigned ? w - 1 : g.cell * (vertical ? w : 1);
+    if (kind == MaskKind::Diagonal) throw std::invalid_argument("[MatrixTransformer] the batched transform takes DiagonalSigned");
+    if (kind == MaskKind::DiagonalSigned && rows != cols)
+        throw std::invalid_argument("[MatrixTransformer] transpose needs square tiles");
     return g;
 }
 

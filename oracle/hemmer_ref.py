@@ -252,6 +252,7 @@ class OracleEval:
 # masks  (MatrixUtils.cpp:90-578)
 # --------------------------------------------------------------------------------------------
 H, V, PH, PV, DIAG = "horizontal", "vertical", "packed_horizontal", "packed_vertical", "diagonal"
+DIAG_SIGNED = "diagonal_signed"   # the transpose's diagonals in the grouping of sigma / tau (batched transform)
 
 
 def _dims(n):
@@ -272,11 +273,12 @@ def geometry(kind, n, w):
         return rows, 1, bs, math.ceil(count / bs), w - 1
     cell = 2 if kind in (PH, PV) else 1
     assert cell == 1 or rows == cols
+    assert kind != DIAG_SIGNED or rows == cols
     units = (cols if kind in (H, PH) else rows) // cell
     sub = sub_dim(kind, n)
     bs = math.ceil(math.sqrt(2 * sub - 1))
     gs = math.ceil((sub - 1) / bs)
-    step = cell * (w if kind in (V, PV) else 1)
+    step = w - 1 if kind == DIAG_SIGNED else cell * (w if kind in (V, PV) else 1)
     return units, cell, bs, gs, step
 
 

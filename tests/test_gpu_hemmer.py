@@ -95,8 +95,15 @@ def test_sigma_tau_bit_exact(small):
     i, j = np.meshgrid(np.arange(16), np.arange(16), indexing="ij")
     assert np.abs(H.decrypt(s) - A[i, (i + j) % 16]).max() < 1e-7
     tr = ca.clone()
+    H.set_schedule(False)
     H.transpose_inplace(tr)
+    H.set_schedule(True)
     assert np.array_equal(tr.residues(), R.transpose(ev, oa, 16, 16).data)
+    # batched schedule: the diagonals in sigma / tau's grouping through the batched transform
+    tb = ca.clone()
+    H.transpose_inplace(tb)
+    assert np.array_equal(tb.residues(), R.diagonal_transform_fused(orc, oa, R.DIAG_SIGNED, 16, 16).data)
+    assert np.abs(H.decrypt(tb) - A.T).max() < 1e-7
 
 
 @pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])

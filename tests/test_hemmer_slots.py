@@ -35,6 +35,9 @@ def test_sigma_tau_transpose(n):
         assert np.array_equal(ev.decrypt(t).real.reshape(-1, w)[:n, :n], A[(i + j) % n, j])
         tr = R.transpose(ev, enc(A), n, w)
         assert np.array_equal(ev.decrypt(tr).real.reshape(-1, w)[:n, :n], A.T)
+        # the same diagonals in sigma / tau's grouping (what the batched transform walks)
+        ts = R.diagonal_transform(ev, enc(A), R.DIAG_SIGNED, n, w)
+        assert np.array_equal(ev.decrypt(ts).real.reshape(-1, w), ev.decrypt(tr).real.reshape(-1, w))
         if w == 2 * n:   # the second tile of the pair is transformed independently
             assert np.array_equal(ev.decrypt(tr).real.reshape(-1, w)[:n, n:], 2 * A.T)
 
