@@ -421,10 +421,20 @@ void HEMMer::splitInTwo(CtxtTensor &t, CtxtTensor &t1, CtxtTensor &t2) const {
 // ---- products ---------------------------------------------------------------------------------------------
 CtxtTensor HEMMer::diagonalToColumn(const CtxtTensor &a) const {
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, a.getBlockWidth()));
+    if (fused_) {   // one stage (the level contract: in at l, out at l - 1) through the batched launches
+        CtxtTensor res(a);
+        res.get() = matrix_transformer.diagonalTransformFused(eval_, a.get(), MaskKind::Horizontal, a.getShape());
+        return res;
+    }
     return matrix_transformer.diagonalToColumn(eval_, a);
 }
 CtxtTensor HEMMer::diagonalToRow(const CtxtTensor &b) const {
     ensureRotationKeys(transformRotations(MaskKind::Vertical, b.getBlockWidth()));
+    if (fused_) {
+        CtxtTensor res(b);
+        res.get() = matrix_transformer.diagonalTransformFused(eval_, b.get(), MaskKind::Vertical, b.getShape());
+        return res;
+    }
     return matrix_transformer.diagonalToRow(eval_, b);
 }
 CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T) const {

@@ -88,10 +88,16 @@ def test_sigma_tau_bit_exact(small):
     A = rng.uniform(-1, 1, (16, 16))
     ca = H.encrypt(A)
     oa = to_oracle(orc, ca)
+    H.set_schedule(False)
     s = H.diagonal_to_column(ca)
     assert np.array_equal(s.residues(), R.diagonal_transform(ev, oa, R.H, 16, 16).data)
     t = H.diagonal_to_row(ca)
     assert np.array_equal(t.residues(), R.diagonal_transform(ev, oa, R.V, 16, 16).data)
+    H.set_schedule(True)
+    sb, tb = H.diagonal_to_column(ca), H.diagonal_to_row(ca)
+    assert np.array_equal(sb.residues(), R.diagonal_transform_fused(orc, oa, R.H, 16, 16).data)
+    assert np.array_equal(tb.residues(), R.diagonal_transform_fused(orc, oa, R.V, 16, 16).data)
+    assert np.abs(H.decrypt(sb) - H.decrypt(s)).max() < 1e-7 and np.abs(H.decrypt(tb) - H.decrypt(t)).max() < 1e-7
     i, j = np.meshgrid(np.arange(16), np.arange(16), indexing="ij")
     assert np.abs(H.decrypt(s) - A[i, (i + j) % 16]).max() < 1e-7
     tr = ca.clone()
