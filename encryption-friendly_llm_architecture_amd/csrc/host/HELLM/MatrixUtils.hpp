@@ -187,6 +187,10 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vect
 // plaintext x ciphertext product through the hoisted column shifts (see matrix_utils_fused.cpp for the layouts it takes)
 bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const PtxtTensor &op2,
                           u64 target_level, MatrixTransformer &transformer, u64 batch, CtxtTensor &res);
+// the n/2 column shifts (by two columns each) of a packed sigma(A) at level T+2, as ciphertexts at level T+1
+// (multPackedMatMatPreRot through the hoisted launches)
+void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
+                                 MatrixTransformer &transformer, u64 batch = 16);
 // sum_k tmp[k] (x) rho^(k step)(b), relinearised (and rescaled when rescale_after): the ciphertext x ciphertext re-use
 // forms (multMatMatCCReUse: step = block width; multPackedMatMatCCReuse: step = 2 block widths, rescale) with all
 // rotations of b taken from ONE ModUp through direct keys, in batches of hoisted sums

@@ -485,10 +485,22 @@ CtxtTensor HEMMer::packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T)
 }
 CtxtTensor HEMMer::packedMatMulPre(const CtxtTensor &a, u64 T) const {
     ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, a.getBlockWidth()));
+    if (fused_ && a.getLevel() >= T + 3) {   // sigma through the batched launches (two stages with a level to spare)
+        CtxtTensor res(a);
+        res.get() = matrix_transformer.lowerAndTransformFused(eval_, a.get(), MaskKind::PackedHorizontal, a.getShape(), T + 2);
+        return res;
+    }
     return multPackedMatMatPre(eval_, a, T, matrix_transformer);
 }
 void HEMMer::packedMatMulPreRot(const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 T) const {
     const u64 slots = u64(1) << log_slots_;
+    if (fused_ && a.getLevel() == T + 2 && a.get().getRescaleCounter() == 0) {
+        std::vector<u64> rots{slots - (u64)a.getHeight()};
+        for (i64 i = 1; i < a.getHeight() / 2; i++) rots.push_back((u64)(2 * i));
+        ensureRotationKeys(rots);
+        multPackedMatMatPreRotFused(eval_, a, tmp, T, matrix_transformer, batch_);
+        return;
+    }
     ensureRotationKeys({2, slots - (u64)a.getHeight()});
     multPackedMatMatPreRot(eval_, a, tmp, T, matrix_transformer);
 }

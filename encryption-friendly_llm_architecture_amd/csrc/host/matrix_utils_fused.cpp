@@ -984,6 +984,46 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
 
 namespace HELLM {
 
+// multPackedMatMatPreRot with the batched launches: shift i moves the packed sigma(A) by 2 i columns inside its tile,
+// main and wrapped part under the key of that one rotation (the copy rotated by -n is prepared once), 2 * batch
+// shifts per hoisted launch, ModDown merged with the rescale of the mask product.
+void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::vector<Ciphertext> &tmp, u64 T,
+                                 MatrixTransformer &tr, u64 batch) {
+    const Context &c = eval.getContext();
+    tmp.clear();
+    const i64 n = a_in.getHeight();
+    if (a_in.getLevel() != T + 2 || a_in.get().getRescaleCounter() != 0)
+        throw std::invalid_argument("[multPackedMatMatPreRot] operand must be at level " + std::to_string(T + 2) + ".");
+    std::vector<Plaintext> &cm = tr.getColMaskExt(eval, a_in.getShape(), T + 2);
+    Ciphertext first_ct(c);
+    eval.levelDownOne(a_in.get(), first_ct);
+    tmp.push_back(first_ct);
+    std::vector<Shift> sa;
+    for (i64 i = 1; i < n / 2; i++) sa.push_back(Shift{2 * i, &cm[(size_t)(4 * i + 1)], &cm[(size_t)(4 * i)]});
+    if (sa.empty()) return;
+    const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1;
+    const u64 *src = a_in.get().buf_.data();
+    const Sources x = extendSources(c, src, 1, nq);
+    const i64 back = -n;
+    const DeviceBuffer a2 = rotateSources(eval, x, src, 1, &back);
+    const Sources x2 = extendSources(c, a2.data(), 1, nq);
+    const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)sa.size()));
+    DeviceBuffer y(c, G * 2 * E * N), t(c, G * 2 * lo * N), ws(c, G * 2 * lo * N);
+    for (size_t first = 0; first < sa.size(); first += G) {
+        const size_t cnt = std::min(G, sa.size() - first);
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        pushShifts(eval, x, 0, x2, 0, sa, first, cnt, terms, off);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, y.data(), t.data(), lo * N, ws.data(), nullptr));
+        for (size_t q = 0; q < cnt; q++) {
+            Ciphertext ct(c);
+            ct.allocate(2, T + 1, 0);
+            (void)hipMemcpyAsync(ct.buf_.data(), t.data() + q * 2 * lo * N, 2 * lo * N * 8, hipMemcpyDeviceToDevice, nullptr);
+            tmp.push_back(std::move(ct));
+        }
+    }
+}
+
 // Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and
 // b = tau(B).  The reference rotates b by `step` in a chain, one key switch after the other; here every rotation
 // comes from the same ModUp of b through its direct key (hoisted), 2 * batch rotations per launch chain with one

@@ -819,6 +819,15 @@ def mult_mat_mat_pc_fused(orc, a, b_pt, T, n, w):
     return mult_mat_mat_reuse(ev, tmp, b, T, step=w)
 
 
+def mult_packed_mat_mat_pre_rot_fused(orc, a, T, n, w):
+    """multPackedMatMatPreRot through the hoisted launches: a = packed sigma(A) at level T+2 -> its n/2 column shifts
+    (two columns each) at level T+1."""
+    cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+    ext = orc.modup(a.data[1])
+    return [orc.level_down_one(a)] + _assemble_shifts(
+        orc, a, ext, -n, [(2 * i, cm[4 * i + 1], cm[4 * i]) for i in range(1, n // 2)])
+
+
 def mult_mat_mat_cc_reuse_fused(orc, tmp, b, step, rescale_after=False):
     """Batched ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b), every rotation of b taken from
     one ModUp through its direct key (automorphism after ModUp, plain ModDown), relinearised at the end (packed

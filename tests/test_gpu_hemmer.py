@@ -344,6 +344,12 @@ def test_reuse_variants_and_repacking(small, fused):
     d = H.decrypt2(pc)
     assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
     if fused:
+        osa = R.lower_and_transform_fused(orc, to_oracle(orc, pa), R.PH, n, 2 * n, T + 2)
+        assert np.array_equal(sa.residues(), osa.data)
+        want_rot = R.mult_packed_mat_mat_pre_rot_fused(orc, osa, T, n, 2 * n)
+        assert len(ptmp) == len(want_rot) == n // 2
+        for k in range(len(ptmp)):
+            assert np.array_equal(ptmp.get(k, n, n, 2 * n).residues(), want_rot[k].data), k
         assert np.array_equal(pbt.residues(), R.lower_and_transform_fused(orc, to_oracle(orc, pb), R.PV, n, 2 * n, T + 1).data)
         optmp = [to_oracle(orc, ptmp.get(k, n, n, 2 * n)) for k in range(len(ptmp))]
         want = R.mult_mat_mat_cc_reuse_fused(orc, optmp, to_oracle(orc, pbt), 4 * n, rescale_after=True)
