@@ -97,6 +97,12 @@ def gpu_ccmm(args, out):
     tmp = H.matmul_pre(x, T)
     wp = H.encode_diagonal_to_row4(*[0.02 * rng.normal(size=(128, 128)) for _ in range(4)], level=T + 1)
     out["hoisted_pcmm_reuse_ms"] = ms(lambda: H.matmul_reuse(tmp, wp, T), 10)
+    # the other entry points of the path, batched schedule (pair layout where a layout is needed)
+    out["transpose_ms"] = ms(lambda: H.transpose_inplace(ca.clone(), T))
+    out["diagonal_to_column_level12_ms"] = ms(lambda: H.diagonal_to_column(ca))
+    rev = H.matmul_pre_rev(pb, T)
+    out["ccmm_pre_rev_ms"] = ms(lambda: H.matmul_pre_rev(pb, T))
+    out["ccmm_reuse_ms"] = ms(lambda: H.matmul_cc_reuse(tmp, rev, T))
     return H
 
 

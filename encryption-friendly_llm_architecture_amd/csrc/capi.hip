@@ -446,6 +446,11 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
     HEMM_CATCH
 }
 
+void hemm_abi_sizes(uint32_t *rot_term_bytes, uint32_t *lin_term_bytes) {
+    if (rot_term_bytes) *rot_term_bytes = (uint32_t)sizeof(hemm_rot_term);
+    if (lin_term_bytes) *lin_term_bytes = (uint32_t)sizeof(hemm_lin_term);
+}
+
 int hemm_sum_parts(hemm_context *ctx, const uint64_t *parts, uint32_t n_parts, uint32_t n_out, uint32_t nq, uint64_t *y,
                    void *stream) {
     HEMM_TRY

@@ -127,7 +127,10 @@ public:
     u64 getLogSlots() const { return log_slots_; }
     u64 getRescaleCounter() const { return rescale_counter_; }
     void to(const Device &) {}
-    u64 *getMxData() const { return buf_.data(); }
+    u64 *getMxData() const {
+        hash_state_ = 2;   // a writable pointer is out: the content can change behind this object's back
+        return buf_.data();
+    }
     const Context &getContext() const { return ctx_; }
     // internal
     void allocate(u64 level, u64 rescale_counter);
@@ -142,6 +145,11 @@ public:
     DeviceBuffer compact_;
     u32 compact_shift_ = 0;
     bool makeCompact();        // true when a table was found
+    // Hash of the residues, kept by callers that cache work per plaintext content (the weight preparation of the
+    // plaintext x ciphertext product): 0 = not computed, 1 = content_hash_ is valid (every evaluator operation writes
+    // a plaintext through allocate(), which resets this), 2 = never valid (see getMxData()).
+    mutable u64 content_hash_ = 0;
+    mutable int hash_state_ = 0;
 };
 
 class Ciphertext {

@@ -263,6 +263,7 @@ void Plaintext::allocate(u64 level, u64 rc) {
     buf_.resize(ctx_, (level + 1) * ctx_->N);
     compact_shift_ = 0;
     compact_ = DeviceBuffer();
+    if (hash_state_ == 1) hash_state_ = 0;
 }
 bool Plaintext::makeCompact() {
     if (compact_shift_ != 0) return true;
@@ -286,6 +287,7 @@ void Plaintext::setLevel(u64 level) {
     if (level == level_) return;
     compact_shift_ = 0;
     compact_ = DeviceBuffer();
+    if (hash_state_ == 1) hash_state_ = 0;
     DeviceBuffer nb(ctx_, (level + 1) * ctx_->N);
     hip_ck(hipMemcpyAsync(nb.data(), buf_.data(), (level + 1) * ctx_->N * 8, hipMemcpyDeviceToDevice, nullptr),
            "hipMemcpyAsync");

@@ -1117,7 +1117,19 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
     const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
     // ---- tau(B) over the extended basis at level T+2, scaled like a plaintext of level T+1
-    const auto key = std::make_tuple(hashResidues(c, op2.get()), shape_b, T);
+    // the hash needs a device-to-host copy and with it a drained queue: taken once per plaintext object
+    const Plaintext &weight = op2.get();
+    u64 weight_hash;
+    if (weight.hash_state_ == 1) {
+        weight_hash = weight.content_hash_;
+    } else {
+        weight_hash = hashResidues(c, weight);
+        if (weight.hash_state_ == 0) {
+            weight.content_hash_ = weight_hash;
+            weight.hash_state_ = 1;
+        }
+    }
+    const auto key = std::make_tuple(weight_hash, shape_b, T);
     auto it = tr.weight_tau_.find(key);
     if (it == tr.weight_tau_.end()) {
         EnDecoder endec(c);

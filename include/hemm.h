@@ -137,6 +137,9 @@ typedef struct {
     uint32_t pt_galois;   /* odd, < 2N; 1 = as stored */
     uint32_t reserved;    /* 0 */
 } hemm_rot_term;
+/* sizeof(hemm_rot_term) and sizeof(hemm_lin_term) as this library was built: a binding checks its own record layouts
+ * against them before it passes term lists. */
+void hemm_abi_sizes(uint32_t *rot_term_bytes, uint32_t *lin_term_bytes);
 /* y[o] = sum of the n_parts consecutive partial sums parts[o * n_parts .. ) of hemm_hoisted_terms, limb-wise over the
  * extended basis; y: [n_out][2][nq+n_p][N], parts: [n_out * n_parts][2][nq+n_p][N].  A sum with one output and many
  * terms is split over several partial outputs (more workgroups, more keys in flight) and added up here before its

@@ -29,3 +29,14 @@ def test_primes_helper_matches_oracle_generator():
     from oracle import oracle as O
     assert pkg.primes_below(60, 16, 24) == O.primes_below(60, 16, 24)
     assert pkg.primes_below(42, 10, 5) == O.primes_below(42, 10, 5)
+
+
+def test_term_records_match_the_library_layout():
+    """The ctypes records the Python side fills have the size the library was compiled with."""
+    pkg = load_package()
+    L = ctypes.CDLL(pkg.LIB_PATH)
+    rot, lin = ctypes.c_uint32(0), ctypes.c_uint32(0)
+    L.hemm_abi_sizes.restype = None
+    L.hemm_abi_sizes(ctypes.byref(rot), ctypes.byref(lin))
+    assert rot.value == ctypes.sizeof(pkg.RotTerm) == 56
+    assert lin.value == ctypes.sizeof(pkg.LinTerm) == 32
