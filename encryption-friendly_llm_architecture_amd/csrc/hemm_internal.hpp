@@ -60,14 +60,17 @@ u64 h_invmod(u64 a, u64 q);
 LimbList limbs_default(const hemm_context *c, int nq, int with_p);
 
 // kernel launchers (defined in the .hip files)
+// final_scale (device, one (constant, Shoup quotient) pair per limb of the launch, or nullptr): an inverse transform
+// of N = 2^16 ends with that constant in place of 1/N
 void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
-                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s);
+                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s, const void *final_scale = nullptr);
 bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
                           size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 // inverse transform reading src (same slot numbering as data, polynomial stride src_poly_stride) and leaving the
 // coefficients in data; false when this ring size has no out-of-place form (the caller copies, then transforms)
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
-                      const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s);
+                      const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s,
+                      const void *final_scale = nullptr);
 void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
                 size_t poly_stride, bool inverse, hipStream_t s);
 void launch_binary(const hemm_context *c, int op, const u64 *a, size_t a_stride, const u64 *b, size_t b_stride,

@@ -23,6 +23,7 @@ struct BConvArgs {
     const Cst *inv;        // [n_src]  (S/q_i)^-1 mod q_i
     const Cst *hat;        // [n_src][hat_ld]  (S/q_i) mod prime, indexed by prime
     int n_src, n_dst, hat_ld, logN;
+    int pre_scaled;        // the source residues already carry their (S/q_i)^-1 factor (folded into the inverse transform)
     uint8_t src_slot[32], src_prime[32];
     uint8_t dst_slot[HEMM_MAX_PRIMES], dst_prime[HEMM_MAX_PRIMES];
 };
@@ -38,7 +39,8 @@ __global__ __launch_bounds__(256) void bconv_kernel(BConvArgs a, const ModQ *__r
     for (int i = 0; i < a.n_src; i++) {
         const u64 q = modq[a.src_prime[i]].q;
         const Cst c = a.inv[i];
-        v[i * 256 + threadIdx.x] = mul_shoup(src[((size_t)a.src_slot[i] << a.logN) + n], c.w, c.ws, q);
+        const u64 x = src[((size_t)a.src_slot[i] << a.logN) + n];
+        v[i * 256 + threadIdx.x] = a.pre_scaled ? x : mul_shoup(x, c.w, c.ws, q);
     }
     for (int j = 0; j < a.n_dst; j++) {
         const int pj = a.dst_prime[j];
@@ -67,8 +69,8 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
         const u64 q = modq[a.src_prime[i]].q;
         const Cst c = a.inv[i];
         const ulonglong2 x = *(const ulonglong2 *)(src + ((size_t)a.src_slot[i] << a.logN) + n);
-        v0[i] = mul_shoup(x.x, c.w, c.ws, q);
-        v1[i] = mul_shoup(x.y, c.w, c.ws, q);
+        v0[i] = a.pre_scaled ? x.x : mul_shoup(x.x, c.w, c.ws, q);
+        v1[i] = a.pre_scaled ? x.y : mul_shoup(x.y, c.w, c.ws, q);
     }
     for (int j = 0; j < a.n_dst; j++) {
         const int pj = a.dst_prime[j];
@@ -116,8 +118,8 @@ __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const 
             const u64 q = modq[a.src_prime[i]].q;
             const Cst c = a.inv[i];
             const ulonglong2 x = *(const ulonglong2 *)(src + ((size_t)a.src_slot[i] << a.logN) + n);
-            v0[i] = mul_shoup(x.x, c.w, c.ws, q);
-            v1[i] = mul_shoup(x.y, c.w, c.ws, q);
+            v0[i] = a.pre_scaled ? x.x : mul_shoup(x.x, c.w, c.ws, q);
+            v1[i] = a.pre_scaled ? x.y : mul_shoup(x.y, c.w, c.ws, q);
         }
     }
     for (int j = 0; j < a.n_dst; j++) {
@@ -514,6 +516,10 @@ struct KsTables {
     std::vector<std::vector<Cst>> dropinv;               // [nq][j<nq-1]  (P q_{nq-1})^-1 mod q_j
     size_t pinv_off = 0;                                 // device copies of pinv / dropinv[nq] / qlinv[l]
     std::vector<size_t> dropinv_off, qlinv_off;
+    // (1/N) (S/q_i)^-1 mod q_i in source order: the constant an inverse transform of N = 2^16 ends with when a basis
+    // conversion follows it.  modup: per chain length nq, limbs 0 .. nq-1 (each limb in its own digit's basis).
+    size_t p_invn_off = 0;
+    std::vector<size_t> drop_invn_off, modup_invn_off;   // [nq]
 };
 
 static KsTables *g_tables_of(const hemm_context *c);
@@ -596,6 +602,39 @@ static void build_tables(const hemm_context *c, KsTables &t) {
     for (int l = 0; l < nQ; l++) {
         t.qlinv_off[l] = t.host.size();
         for (auto &x : t.qlinv[l]) t.host.push_back(x);
+    }
+    // inverse-transform constants with 1/N folded in, read back from the inv entries built above
+    auto invn = [&](size_t inv_off, const std::vector<int> &src) {
+        const size_t off = t.host.size();
+        for (size_t i = 0; i < src.size(); i++) {
+            const u64 q = c->primes[src[i]];
+            const u64 v = h_mulmod(t.host[inv_off + i].w, h_invmod((u64)c->N % q, q), q);
+            t.host.push_back(Cst{v, shoup_h(v, q)});
+        }
+        return off;
+    };
+    if (K > 0) {
+        std::vector<int> src;
+        for (int k = 0; k < K; k++) src.push_back(nQ + k);
+        t.p_invn_off = invn(t.p_inv_off, src);
+    }
+    t.drop_invn_off.assign(nQ + 1, 0);
+    if (K > 0)
+        for (int nq = 2; nq <= nQ; nq++) {
+            std::vector<int> src;
+            src.push_back(nq - 1);
+            for (int k = 0; k < K; k++) src.push_back(nQ + k);
+            t.drop_invn_off[nq] = invn(t.drop_inv_off[nq], src);
+        }
+    t.modup_invn_off.assign(nQ + 1, 0);
+    for (int nq = 1; nq <= nQ; nq++) {
+        const int beta = (nq + alpha - 1) / alpha;
+        t.modup_invn_off[nq] = t.host.size();
+        for (int d = 0; d < beta; d++) {
+            std::vector<int> src;
+            for (int j = d * alpha; j < std::min(nq, (d + 1) * alpha); j++) src.push_back(j);
+            invn(t.inv_off[nq][d], src);
+        }
     }
     HEMM_HIP(hipMalloc((void **)&t.dev, t.host.size() * sizeof(Cst)));
     HEMM_HIP(hipMemcpy(t.dev, t.host.data(), t.host.size() * sizeof(Cst), hipMemcpyHostToDevice));
@@ -808,7 +847,9 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     const LimbList chain = limbs_default(c, nq, 0);
     LimbList ident;
     for (int j = 0; j < HEMM_MAX_PRIMES; j++) ident.idx[j] = (uint8_t)j;
-    if (!launch_intt_from(c, in, in_stride, coef, chain, ident, nq, n_in, (size_t)nq * N, s)) {
+    const bool fold = c->logN == 16;
+    if (!launch_intt_from(c, in, in_stride, coef, chain, ident, nq, n_in, (size_t)nq * N, s,
+                          fold ? t->dev + t->modup_invn_off[nq] : nullptr)) {
         HEMM_HIP(hipMemcpy2DAsync(coef, (size_t)nq * N * 8, in, in_stride * 8, (size_t)nq * N * 8, n_in,
                                   hipMemcpyDeviceToDevice, s));
         launch_ntt(c, coef, chain, nq, n_in, (size_t)nq * N, true, s);
@@ -838,6 +879,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         a.n_src = hi - lo;
         a.hat_ld = c->nQ + c->nP;
         a.logN = c->logN;
+        a.pre_scaled = fold ? 1 : 0;
         LimbList pl, sl;
         memset(&pl, 0, sizeof(pl));
         memset(&sl, 0, sizeof(sl));
@@ -1001,7 +1043,10 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
         pl.idx[i] = a.src_prime[i];
         sl.idx[i] = a.src_slot[i];
     }
-    launch_ntt_slots(c, y, pl, sl, ns, n_polys, (size_t)E * N, true, s);
+    const bool fold = c->logN == 16;   // the inverse transform ends with (1/N)(S/q_i)^-1: no scaling pass in the conversion
+    launch_ntt_slots(c, y, pl, sl, ns, n_polys, (size_t)E * N, true, s,
+                     fold ? t->dev + (drop_last ? t->drop_invn_off[nq] : t->p_invn_off) : nullptr);
+    a.pre_scaled = fold ? 1 : 0;
     a.src = y;
     a.src_poly_stride = (size_t)E * N;
     a.dst = conv;

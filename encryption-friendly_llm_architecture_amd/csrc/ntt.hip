@@ -303,16 +303,29 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
                                                          const ModQ *__restrict__ modq,
                                                          const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
                                                          const double *__restrict__ fp, LimbList ll, LimbList sl,
-                                                         int n_limbs, size_t poly_stride) {
+                                                         int n_limbs, size_t poly_stride, const Tw *__restrict__ final_scale) {
     __shared__ u64 lds[256 * 16];
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
     u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + blockIdx.x * 16 + (threadIdx.x & 15);
-    if (fp[4 * prime] != 0.0)
-        cols_body<INV>(base, tw, FpField(modq, ninv, ninv_s, fp, prime), lds);
-    else
-        cols_body<INV>(base, tw, IntField(modq, ninv, ninv_s, fp, prime), lds);
+    // final_scale (inverse transforms only): limb i ends with the constant final_scale[i] in place of 1/N -- a basis
+    // conversion folds its (S/q_i)^-1 factor in here (the caller supplies (1/N)(S/q_i)^-1), at no cost
+    if (fp[4 * prime] != 0.0) {
+        FpField f(modq, ninv, ninv_s, fp, prime);
+        if (INV && final_scale != nullptr) {
+            f.ni = (double)final_scale[limb].w;
+            f.niinv = f.ni * f.qinv;
+        }
+        cols_body<INV>(base, tw, f, lds);
+    } else {
+        IntField f(modq, ninv, ninv_s, fp, prime);
+        if (INV && final_scale != nullptr) {
+            f.ni = final_scale[limb].w;
+            f.nis = final_scale[limb].ws;
+        }
+        cols_body<INV>(base, tw, f, lds);
+    }
 }
 
 // A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
@@ -449,7 +462,7 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
     NttEpilogue none{};
     NttEpilogue ep{minuend, out, (const Tw *)cst_dev, minuend_stride, out_stride};
     hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ll,
-                       sl, n_limbs, poly_stride);
+                       sl, n_limbs, poly_stride, (const Tw *)nullptr);
     (void)none;
     hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl, n_limbs,
                        poly_stride, ep);
@@ -457,7 +470,8 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
 }
 
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
-                      const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s) {
+                      const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s,
+                      const void *final_scale) {
     if (c->logN != 16) return false;
     if (n_limbs <= 0 || n_polys <= 0) return true;
     const Tw *tw = (const Tw *)c->d_iw;
@@ -469,27 +483,29 @@ bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_str
     hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
                        n_limbs, poly_stride, from);
     hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ll,
-                       sl, n_limbs, poly_stride);
+                       sl, n_limbs, poly_stride, (const Tw *)final_scale);
     return true;
 }
 
 void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, const LimbList &sl, int n_limbs,
-                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s) {
+                      int n_polys, size_t poly_stride, bool inverse, hipStream_t s, const void *final_scale) {
     if (n_limbs <= 0 || n_polys <= 0) return;
+    if (final_scale != nullptr && (!inverse || c->logN != 16))
+        throw std::invalid_argument("a final constant is taken by the inverse transform of N = 2^16 only");
     const Tw *tw = (const Tw *)(inverse ? c->d_iw : c->d_w);
     const int lanes = n_limbs * n_polys;
     if (c->logN == 16) {
         dim3 grid(16, lanes), block(256);
         if (!inverse) {
             hipLaunchKernelGGL(ntt16_cols_kernel<false>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
+                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)nullptr);
             hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
                                n_limbs, poly_stride, NttEpilogue{});
         } else {
             hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, data, tw, c->d_modq, c->d_fp, ll, sl,
                                n_limbs, poly_stride, NttEpilogue{});
             hipLaunchKernelGGL(ntt16_cols_kernel<true>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv,
-                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride);
+                               c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)final_scale);
         }
         return;
     }
