@@ -179,9 +179,10 @@ CtxtTensor multMatMatLowLow(const HomEvaluator &eval, const CtxtTensor &op1, con
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer, u64 batch = 16,
                            bool single_tile = false);
+// single_tile: the operands hold one tile block and nothing else (as for multMatMatFused)
 CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                                  const CtxtTensor &op2, u64 target_level, MatrixTransformer &transformer,
-                                 u64 batch = 16);
+                                 u64 batch = 16, bool single_tile = false);
 void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
                         MatrixTransformer &transformer, u64 batch = 16, bool first_block_only = false);
 // plaintext x ciphertext product through the hoisted column shifts (see matrix_utils_fused.cpp for the layouts it takes)

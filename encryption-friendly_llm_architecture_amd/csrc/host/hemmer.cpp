@@ -395,7 +395,23 @@ void HEMMer::complexPackingRowInplace(CtxtTensor &t) const {
     const u64 slots = u64(1) << log_slots_, w = (u64)t.getBlockWidth();
     ensureRotationKeys({w, slots - w});
     Ciphertext odd(context_), even(context_), fus(context_);
-    const Plaintext &m = cachedMask(MASK_ROW_EVEN, t.getLevel());
+    // even rows of rows `w` slots wide: the reference's mask is laid out for the pair layout (w = 2 n); other widths
+    // get their own pattern
+    const Plaintext *mp;
+    if (w == (u64)(2 * dim_)) {
+        mp = &cachedMask(MASK_ROW_EVEN, t.getLevel());
+    } else {
+        const auto key = std::make_pair(1000 + (int)w, t.getLevel());
+        auto it = mask_cache_.find(key);
+        if (it == mask_cache_.end()) {
+            Message msg(log_slots_, 0);
+            for (u64 j = 0; j < slots; j++)
+                if ((j / w) % 2 == 0) msg[j] = 1;
+            it = mask_cache_.emplace(key, endec_.encode(msg, t.getLevel())).first;
+        }
+        mp = &it->second;
+    }
+    const Plaintext &m = *mp;
     eval_.mult(t.get(), m, even);
     eval_.leftRotate(t.get(), w, odd);
     eval_.multImagUnit(odd, odd);
@@ -447,6 +463,26 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
         // come from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots)
         const u64 block = (u64)(n * w);
         const bool single = single_tile_ || (a.get().occupiedSlots() <= block && b.get().occupiedSlots() <= block);
+        // A single tile with a level to spare goes through the complex-packed product: adjacent columns of A and
+        // adjacent rows of B are fused into complex slots (one level), the product then needs n / 2 column shifts
+        // (each a key product and a ModDown) instead of n, and x + conj(x) returns the real product.
+        if (single && block < slots && n >= 4 && a.getHeight() == n && a.getWidth() == n && b.getWidth() == n &&
+            std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
+            b.get().getRescaleCounter() == 0) {
+            CtxtTensor pa(a), pb(b);
+            complexPackingInplace(pa);
+            complexPackingRowInplace(pb);
+            ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
+            ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
+            std::vector<u64> sq;
+            ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, true));
+            KeyGenerator kg(context_, sk_, pack_);
+            for (u64 r : sq) kg.genLeftRotSquareKey(r);
+            CtxtTensor prod = multPackedMatMatFused(eval_, btp_, pa, pb, T, matrix_transformer, batch_, true);
+            CtxtTensor res = repackCC(prod);
+            res.get().occupied_ = block;
+            return res;
+        }
         std::vector<u64> square_rots;
         ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, false, single));
         KeyGenerator keygen(context_, sk_, pack_);
@@ -473,12 +509,15 @@ CtxtTensor HEMMer::packedMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 T)
     const i64 w = a.getBlockWidth(), n = pow2ceil(a.getWidth());
     ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
-    if (fused_ && (u64)(n * w) == slots) {
+    // a single tile in part of the slots is taken only on the caller's promise (assumeSingleTile): the packing that
+    // produced the operands rotates, which forgets what the evaluator knew about empty slots
+    const bool spread = single_tile_ && (u64)(n * w) < slots && slots % (u64)(n * w) == 0;
+    if (fused_ && ((u64)(n * w) == slots || spread)) {
         std::vector<u64> square_rots;
-        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, true));
+        ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, true, spread));
         KeyGenerator keygen(context_, sk_, pack_);
         for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
-        return multPackedMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_);
+        return multPackedMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, spread);
     }
     ensureRotationKeys({2, (u64)(2 * w), slots - (u64)n});
     return multPackedMatMat(eval_, btp_, a, b, T, matrix_transformer);

@@ -166,16 +166,14 @@ std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots,
                                     bool packed, bool single_tile) {
     const i64 slots = i64(1) << log_slots, n = shape.getNumRows(), w = shape.getBlockWidth();
     square_rots.clear();
-    const bool spread = single_tile && !packed && n * w < slots && slots % (n * w) == 0;
+    const bool spread = single_tile && n * w < slots && slots % (n * w) == 0;
     if (n * w != slots && !spread) return fusedRotations(shape, log_slots, packed, true);
     std::vector<u64> r;
     auto left = [&](i64 v) { return (u64)(((v % slots) + slots) % slots); };
-    if (spread) {   // baby rotations gather the block copies as well
-        const i64 gs = bsgsBabyCount(n);
-        for (i64 i1 = 0; i1 < gs; i1++)
-            for (i64 j = 1; j < slots / (n * w); j++) r.push_back(left(i1 * w - j * n * w));
-    }
     const i64 cu = packed ? 2 : 1, units = n / cu, ru = cu * w, g = bsgsBabyCount(units);
+    if (spread)     // baby rotations gather the block copies as well
+        for (i64 i1 = 0; i1 < g; i1++)
+            for (i64 j = 1; j < slots / (n * w); j++) r.push_back(left(i1 * ru - j * n * w));
     r.push_back(left(-n));
     for (i64 i = 1; i < units; i++) r.push_back(left(cu * i - g * (i / g) * ru));
     for (i64 i1 = 1; i1 < g; i1++) r.push_back(left(i1 * ru));
@@ -889,7 +887,7 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
 }
 
 CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
-                                 const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch) {
+                                 const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -899,7 +897,11 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     if (op1.getLevel() < T + 3 || op2.getLevel() < T + 2)
         throw std::invalid_argument("[multPackedMatMat] levels >= " + std::to_string(T + 3) + " / " +
                                     std::to_string(T + 2) + " are needed.");
-    if ((u64)(k * w) != c->N / 2)
+    const u64 slots = c->N / 2;
+    // one tile block in an otherwise empty slot vector: tau(B) is treated as copied into every block (the baby
+    // rotations gather the copies), which makes its row shifts exact rotations, as in multMatMatFused
+    const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
+    if ((u64)(k * w) != slots && !spread)
         throw std::invalid_argument("[multPackedMatMat] the row shift must be cyclic: rows * block width == slots");
     CtxtTensor a{op1}, b{op2};
     a.setShape(rows, k);
@@ -934,8 +936,10 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
     // column shifts of sigma(A) by 2 i, row rotations of tau(B) by 2 i w: baby-step / giant-step over i
     DeviceBuffer U;
     i64 g = 1;
-    bsgsShiftProduct(eval, T, a.get().buf_.data(), b.get().buf_.data(), acc, cm, n, n / 2, 2, w, batch, &U, &g);
+    bsgsShiftProduct(eval, T, a.get().buf_.data(), b.get().buf_.data(), acc, cm, n, n / 2, 2, w, batch, &U, &g,
+                     spread ? (u64)(n * w) : 0);
     bsgsGiantSteps(eval, T, U, g, (n / 2) / g, 2 * w, acc, res);
+    if (spread) res.get().occupied_ = (u64)(n * w);
     return res;
 }
 

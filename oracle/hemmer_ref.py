@@ -767,7 +767,8 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     return orc.rescale(orc.relinearize(acc))
 
 
-def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
+def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False):
+    """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused)."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
@@ -775,7 +776,18 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w):
     b = lower_and_transform_fused(orc, b, PV, n, w, T + 1)
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
-    return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w)
+    spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
+    return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0)
+
+
+def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
+    """One product through the complex-packed route: adjacent columns of A and adjacent rows of B are fused into
+    complex slots (complexPackingInplace / complexPackingRowInplace, one level), the packed product then needs n / 2
+    shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile."""
+    ev = OracleEval(orc)
+    pa = complex_packing_cols(ev, a, n, w)
+    pb = complex_packing_rows(ev, b, n, w)
+    return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=True))
 
 
 def mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only=False):

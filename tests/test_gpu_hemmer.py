@@ -125,8 +125,9 @@ def test_ccmm_residues_bit_exact_and_decrypts(small, fused):
     finally:
         H.set_schedule(True)
     oa, ob = to_oracle(orc, ca), to_oracle(orc, cb)
-    # operands straight from encrypt() are known to hold a single tile: the batched schedule spreads tau(B)
-    want = (R.mult_mat_mat_cc_fused(orc, oa, ob, 2, 16, 16, single_tile=True) if fused
+    # operands straight from encrypt() are known to hold a single tile and have levels to spare: the batched schedule
+    # takes the complex-packed route (half the column shifts) with tau(B) spread over the blocks
+    want = (R.mult_mat_mat_cc_packed_single(orc, oa, ob, 2, 16, 16) if fused
             else R.mult_mat_mat_cc(ev, oa, ob, 2, 16, 16))
     assert c.info()["level"] == 2
     assert np.array_equal(c.residues(), want.data)
@@ -147,11 +148,21 @@ def test_ccmm_single_tile_promise(small):
     finally:
         H.assume_single_tile(False)
         H.set_schedule(True)
-    want = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16, single_tile=True)
+    want = R.mult_mat_mat_cc_packed_single(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16)
     assert c.info()["level"] == 2
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
     assert np.abs(H.decrypt_slots(c)[256:]).max() < 2 ** -20
+    # without a level to spare for the packing (operands at T+3) the unpacked single-tile route runs
+    H.assume_single_tile(True)
+    try:
+        la, lb = H.level_down(ca, 5), H.level_down(cb, 5)
+        c5 = H.single_cc_matmul(la, lb, 2)
+    finally:
+        H.assume_single_tile(False)
+    want5 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16, single_tile=True)
+    assert np.array_equal(c5.residues(), want5.data)
+    assert np.abs(H.decrypt(c5) - A @ B).max() < 2 ** -20
 
 
 def test_ccmm_stacked_tiles_keep_block_products(small):
