@@ -117,6 +117,13 @@ public:
         Plaintext tau;
         int layout;
     };
+    // complexPackingInplace (rows[q] false: adjacent columns -> a + i b) / complexPackingRowInplace (true: adjacent
+    // rows of rows `w` slots wide -> a - i b) of n_jobs ciphertexts at `level` through one launch chain: both
+    // rotations of every job from one ModUp, masks applied in the extended basis, ModDown merged with the rescale.
+    // in: [job][2][level+1][N], out: [job][2][level][N].
+    void complexPackingBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const bool *rows, i64 w,
+                             u64 *out);
+    std::map<std::tuple<int, i64, u64, int>, Plaintext> pack_masks_;   // (rows, w, level, part 0 = Z / 1 = +step / 2 = -step)
     std::map<std::tuple<u64, TileTensorShape, u64>, WeightTau> weight_tau_;
     std::vector<std::tuple<u64, TileTensorShape, u64>> weight_tau_order_;
 
@@ -192,6 +199,10 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
 // (multPackedMatMatPreRot through the hoisted launches)
 void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
                                  MatrixTransformer &transformer, u64 batch = 16);
+// pa = complexPackingInplace(a) (adjacent columns), pb = complexPackingRowInplace(b) (adjacent rows of width w), both at
+// the operands' common level, through MatrixTransformer::complexPackingBatch
+void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &transformer, const Ciphertext &a, const Ciphertext &b,
+                        i64 w, Ciphertext &pa, Ciphertext &pb);
 // sum_k tmp[k] (x) rho^(k step)(b), relinearised (and rescaled when rescale_after): the ciphertext x ciphertext re-use
 // forms (multMatMatCCReUse: step = block width; multPackedMatMatCCReuse: step = 2 block widths, rescale) with all
 // rotations of b taken from ONE ModUp through direct keys, in batches of hoisted sums

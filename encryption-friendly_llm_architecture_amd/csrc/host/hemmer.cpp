@@ -470,8 +470,13 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
             b.get().getRescaleCounter() == 0) {
             CtxtTensor pa(a), pb(b);
-            complexPackingInplace(pa);
-            complexPackingRowInplace(pb);
+            if (a.getLevel() == b.getLevel()) {   // both packings through one launch chain
+                ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});
+                complexPackingPair(eval_, matrix_transformer, a.get(), b.get(), w, pa.get(), pb.get());
+            } else {
+                complexPackingInplace(pa);
+                complexPackingRowInplace(pb);
+            }
             ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
             std::vector<u64> sq;

@@ -610,6 +610,72 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
     }
 }
 
+// The complex packing as a linear map on the slots, out = Z x + M_+ rho^(step)(x) + M_- rho^(-step)(x):
+//   columns (step 1):  fus = m (x + i rho^1 x), out = fus + rho^-1 fus, m = even columns
+//   rows (step w):     fus = m (x - i rho^w x), out = fus + rho^-w fus, m = even rows of width w
+// i.e. Z = m +- i m', M_+ = +- i m, M_- = m' with m'[s] = m[s - step].  One hoisted sum with two terms per job plus
+// rescale(Z x) on the side stream.
+void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
+                                            const bool *rows, i64 w, u64 *out) {
+    const Context &c = eval.getContext();
+    if (level < 1) throw std::invalid_argument("[complexPacking] level >= 1 is needed.");
+    const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N, slots = N / 2;
+    const u64 log_slots = getLogFullSlots(c);
+    auto mask = [&](bool by_rows, int part) -> const Plaintext & {
+        const auto key = std::make_tuple((int)by_rows, w, level, part);
+        auto it = pack_masks_.find(key);
+        if (it != pack_masks_.end()) return it->second;
+        const u64 step = by_rows ? (u64)w : 1;
+        Message m(log_slots, 0);
+        const Complex iu(0, by_rows ? -1.0 : 1.0);
+        for (u64 s = 0; s < slots; s++) {
+            auto even = [&](u64 t) { return by_rows ? ((t / (u64)w) % 2 == 0) : (t % 2 == 0); };
+            const double here = even(s) ? 1.0 : 0.0, prev = even((s + slots - step) % slots) ? 1.0 : 0.0;
+            m[s] = part == 0 ? Complex(here, 0) + iu * prev : part == 1 ? iu * here : Complex(prev, 0);
+        }
+        EnDecoder endec(c);
+        return pack_masks_.emplace(key, part == 0 ? endec.encode(m, level) : endec.encodeExtended(m, level)).first->second;
+    };
+    std::vector<hemm_lin_term> zero_terms;
+    std::vector<uint32_t> zoff{0};
+    for (size_t q = 0; q < n_jobs; q++) {
+        hemm_lin_term t;
+        t.ct = in + q * ctw;
+        t.mask = mask(rows[q], 0).buf_.data();
+        t.stride = nq * N;
+        t.galois = 0;
+        zero_terms.push_back(t);
+        zoff.push_back((uint32_t)zero_terms.size());
+        (void)mask(rows[q], 1);    // encoded before the fork below
+        (void)mask(rows[q], 2);
+    }
+    DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
+    const hipStream_t side = c->forkSide();
+    struct JoinOnExit {
+        const Context &c;
+        ~JoinOnExit() { c->joinSide(); }
+    } join_on_exit{c};
+    ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
+    ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
+    const Sources x = extendSources(c, in, n_jobs, nq);
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    std::vector<hemm_rot_term> terms;
+    std::vector<uint32_t> off{0};
+    for (size_t q = 0; q < n_jobs; q++) {
+        const i64 step = rows[q] ? w : 1;
+        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(step), &mask(rows[q], 1)));
+        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(-step), &mask(rows[q], 2)));
+        off.push_back((uint32_t)terms.size());
+    }
+    DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, 1, 1, y.data(), out,
+                            (nq - 1) * N, ws.data(), nullptr));
+    c->joinSide();
+    ck(hemm_pointwise(c->dev, HEMM_ADD, out, (nq - 1) * N, zres.data(), (nq - 1) * N, out, (nq - 1) * N, (uint32_t)(nq - 1), 0,
+                      (uint32_t)(2 * n_jobs), nullptr));
+}
+
 namespace {
 // Sum over the shift index of a product whose row shifts are exact rotations (the tile block fills the slot vector),
 // split into baby and giant steps, i = i1 + g i2 over `units` shifts (column shift of i cells = cu * i slots, row
@@ -1026,6 +1092,27 @@ void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a_i
             tmp.push_back(std::move(ct));
         }
     }
+}
+
+void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &tr, const Ciphertext &a, const Ciphertext &b, i64 w,
+                        Ciphertext &pa, Ciphertext &pb) {
+    const Context &c = eval.getContext();
+    if (a.getLevel() != b.getLevel() || a.getRescaleCounter() != 0 || b.getRescaleCounter() != 0 || a.getNumPoly() != 2 ||
+        b.getNumPoly() != 2)
+        throw std::invalid_argument("[complexPacking] operands must share one level and be rescaled.");
+    const u64 L = a.getLevel(), N = c->N, ctw = 2 * (L + 1) * N, half = 2 * L * N;
+    DeviceBuffer joint(c, 2 * ctw), packed(c, 2 * half);
+    (void)hipMemcpyAsync(joint.data(), a.buf_.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipMemcpyAsync(joint.data() + ctw, b.buf_.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+    const bool by_rows[2] = {false, true};
+    tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, w, packed.data());
+    Ciphertext ra(c), rb(c);
+    ra.allocate(2, L - 1, 0);
+    rb.allocate(2, L - 1, 0);
+    (void)hipMemcpyAsync(ra.buf_.data(), packed.data(), half * 8, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipMemcpyAsync(rb.buf_.data(), packed.data() + half, half * 8, hipMemcpyDeviceToDevice, nullptr);
+    pa = std::move(ra);
+    pb = std::move(rb);
 }
 
 // Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and

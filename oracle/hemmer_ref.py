@@ -780,13 +780,41 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False):
     return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0)
 
 
+def packing_maps(slots, w, rows):
+    """The complex packing as a linear map on the slots, out = Z x + sum_r M_r rho^r(x):
+    columns: fus = m (x + i rho^1 x), out = fus + rho^-1 fus with m = even columns;
+    rows:    fus = m (x - i rho^w x), out = fus + rho^-w fus with m = even rows of width w.
+    Returns (Z, [(r, M_r)])."""
+    s = np.arange(slots)
+    if rows:
+        m = ((s // w) % 2 == 0).astype(np.complex128)
+        prev = np.roll(m, w)
+        return m - 1j * prev, [(w, -1j * m), (-w, prev)]
+    m = (s % 2 == 0).astype(np.complex128)
+    prev = np.roll(m, 1)
+    return m + 1j * prev, [(1, 1j * m), (-1, prev)]
+
+
+def complex_packing_hoisted(orc, x, w, rows):
+    """complexPackingInplace / complexPackingRowInplace as ONE hoisted sum (both rotations from one ModUp, masks
+    applied in the extended basis, ModDown merged with the rescale) plus rescale(Z x): one level, like the
+    reference's two masked steps."""
+    from .oracle import Ct
+    zmask, terms = packing_maps(orc.slots, w, rows)
+    nq = x.nq
+    ext = orc.modup(x.data[1])
+    zero = orc.rescale(orc.mult_plain_no_rescale(x, orc.encode(zmask, x.level)))
+    y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, x.level)) for r, m in terms], nq)
+    return orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
+
+
 def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
     """One product through the complex-packed route: adjacent columns of A and adjacent rows of B are fused into
     complex slots (complexPackingInplace / complexPackingRowInplace, one level), the packed product then needs n / 2
     shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile."""
     ev = OracleEval(orc)
-    pa = complex_packing_cols(ev, a, n, w)
-    pb = complex_packing_rows(ev, b, n, w)
+    pa = complex_packing_hoisted(orc, a, w, rows=False)
+    pb = complex_packing_hoisted(orc, b, w, rows=True)
     return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=True))
 
 
