@@ -832,8 +832,20 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
 }
 }  // namespace
 
+namespace {
+CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
+                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed);
+}
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
+    return ccmmFused(eval, btp, op1, op2, T, tr, batch, single_tile, false);
+}
+
+namespace {
+// packed: the operands are complex-packed (2 x 2 cells): sigma / tau of the packed kinds, n / 2 shifts of two columns /
+// two rows each; otherwise the same schedule
+CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
+                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -886,7 +898,8 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
             (void)hipMemcpyAsync(joint.data(), la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
             (void)hipMemcpyAsync(joint.data() + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
         }
-        const MaskKind kinds[2] = {MaskKind::Horizontal, MaskKind::Vertical};
+        const MaskKind kinds[2] = {packed ? MaskKind::PackedHorizontal : MaskKind::Horizontal,
+                                   packed ? MaskKind::PackedVertical : MaskKind::Vertical};
         const TileTensorShape shapes[2] = {shape_a, shape_b};
         if (two_stage)
             tr.diagonalTransformTwoStage(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
@@ -904,7 +917,8 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
         eval.relinearize(acc, res.get());
         eval.rescale(res.get());
     };
-    if (k == 1) {
+    const i64 cu = packed ? 2 : 1;
+    if (k / cu <= 1) {
         finish();
         return res;
     }
@@ -919,12 +933,14 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     if ((u64)(n * w) == slots || spread) {
         DeviceBuffer U;
         i64 g = 1;
-        bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n, 1, w, batch, &U, &g,
+        bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n / cu, cu, w, batch, &U, &g,
                          spread ? (u64)(n * w) : 0);
-        bsgsGiantSteps(eval, T, U, g, n / g, w, acc, res);
+        bsgsGiantSteps(eval, T, U, g, (n / cu) / g, cu * w, acc, res);
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
+    if (packed)
+        throw std::invalid_argument("[multPackedMatMat] the row shift must be cyclic: rows * block width == slots");
     std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, shape_b, T + 2);
     std::vector<Shift> sa, sb;
     for (i64 i = 1; i < n; i++) {
@@ -951,10 +967,20 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
     finish();
     return res;
 }
+}  // namespace
 
 CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                                  const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
     const Context &c = eval.getContext();
+    // both operands a level above what the reference asks of B: sigma and tau share one launch chain, as in the
+    // unpacked product (tau(B) is then lowered to T+1 with sigma(A)'s copy for the unshifted term)
+    if (std::min(op1.getLevel(), op2.getLevel()) >= T + 3 && op1.get().getRescaleCounter() == 0 &&
+        op2.get().getRescaleCounter() == 0) {
+        const u64 slots = c->N / 2;
+        const i64 kk = pow2ceil(commonInside(op1, op2)), ww = commonBlockWidth(op1, op2);
+        const bool spread = single_tile && (u64)(kk * ww) < slots && slots % (u64)(kk * ww) == 0;
+        if ((u64)(kk * ww) == slots || spread) return ccmmFused(eval, btp, op1, op2, T, tr, batch, single_tile, true);
+    }
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
     if (std::min(op1.getLevel(), op2.getLevel()) < 1 + btp.getMinLevelForBootstrap())

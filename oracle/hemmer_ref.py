@@ -772,11 +772,19 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False):
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
-    a = lower_and_transform_fused(orc, a, PH, n, w, T + 2)
-    b = lower_and_transform_fused(orc, b, PV, n, w, T + 1)
+    spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
+    lvl = min(a.level, b.level)
+    if lvl >= T + 3:
+        # both operands a level above what B needs: sigma and tau share one launch chain and both end at T+2, as in
+        # the unpacked product; tau(B) is lowered to T+1 with sigma(A)'s copy for the unshifted term
+        a = lower_and_transform_fused(orc, orc.level_down(a, min(lvl, T + 4)), PH, n, w, T + 2)
+        b = lower_and_transform_fused(orc, orc.level_down(b, min(lvl, T + 4)), PV, n, w, T + 2)
+        b = orc.level_down_one(b)
+    else:
+        a = lower_and_transform_fused(orc, a, PH, n, w, T + 2)
+        b = lower_and_transform_fused(orc, b, PV, n, w, T + 1)
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
-    spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0)
 
 
