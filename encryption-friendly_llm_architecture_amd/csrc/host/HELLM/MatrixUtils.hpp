@@ -199,10 +199,10 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
 // (multPackedMatMatPreRot through the hoisted launches)
 void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a, std::vector<Ciphertext> &tmp, u64 target_level,
                                  MatrixTransformer &transformer, u64 batch = 16);
-// pa = complexPackingInplace(a) (adjacent columns), pb = complexPackingRowInplace(b) (adjacent rows of width w), both at
-// the operands' common level, through MatrixTransformer::complexPackingBatch
+// pa = complexPackingInplace(a) (adjacent columns), pb = complexPackingRowInplace(b) (adjacent rows of width w), through
+// MatrixTransformer::complexPackingBatch at min(level of a, level of b, pack_level): operands above it are lowered first
 void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &transformer, const Ciphertext &a, const Ciphertext &b,
-                        i64 w, Ciphertext &pa, Ciphertext &pb);
+                        i64 w, Ciphertext &pa, Ciphertext &pb, u64 pack_level = ~u64(0));
 // sum_k tmp[k] (x) rho^(k step)(b), relinearised (and rescaled when rescale_after): the ciphertext x ciphertext re-use
 // forms (multMatMatCCReUse: step = block width; multPackedMatMatCCReuse: step = 2 block widths, rescale) with all
 // rotations of b taken from ONE ModUp through direct keys, in batches of hoisted sums

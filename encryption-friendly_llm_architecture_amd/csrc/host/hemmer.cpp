@@ -466,26 +466,23 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
         // A single tile with a level to spare goes through the complex-packed product: adjacent columns of A and
         // adjacent rows of B are fused into complex slots (one level), the product then needs n / 2 column shifts
         // (each a key product and a ModDown) instead of n, and x + conj(x) returns the real product.
-        if (single && block < slots && n >= 4 && a.getHeight() == n && a.getWidth() == n && b.getWidth() == n &&
+        if ((block == slots || (single && block < slots)) && n >= 4 && a.getHeight() == n && a.getWidth() == n &&
+            b.getHeight() == n && b.getWidth() == n &&
             std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
             b.get().getRescaleCounter() == 0) {
+            // both packings through one launch chain, at level T+5 (the transforms start from T+4)
             CtxtTensor pa(a), pb(b);
-            if (a.getLevel() == b.getLevel()) {   // both packings through one launch chain
-                ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});
-                complexPackingPair(eval_, matrix_transformer, a.get(), b.get(), w, pa.get(), pb.get());
-            } else {
-                complexPackingInplace(pa);
-                complexPackingRowInplace(pb);
-            }
+            ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});
+            complexPackingPair(eval_, matrix_transformer, a.get(), b.get(), w, pa.get(), pb.get(), T + 5);
             ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
             std::vector<u64> sq;
-            ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, true));
+            ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, block < slots));
             KeyGenerator kg(context_, sk_, pack_);
             for (u64 r : sq) kg.genLeftRotSquareKey(r);
-            CtxtTensor prod = multPackedMatMatFused(eval_, btp_, pa, pb, T, matrix_transformer, batch_, true);
+            CtxtTensor prod = multPackedMatMatFused(eval_, btp_, pa, pb, T, matrix_transformer, batch_, block < slots);
             CtxtTensor res = repackCC(prod);
-            res.get().occupied_ = block;
+            if (block < slots) res.get().occupied_ = block;
             return res;
         }
         std::vector<u64> square_rots;

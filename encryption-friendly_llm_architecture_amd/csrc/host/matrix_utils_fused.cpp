@@ -833,6 +833,33 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
 }  // namespace
 
 namespace {
+// HomEvaluator::levelDown of two ciphertexts to level Lt into one buffer [2 cts][2][Lt+1][N]; when they share a higher
+// level, both at once: multiply by round(Delta_Lt q_{Lt+1} / Delta_level) over Lt+2 limbs, then one rescale of the four
+// polynomials straight into the buffer
+void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphertext &b, u64 Lt, u64 *joint) {
+    const Context &c = eval.getContext();
+    const u64 N = c->N, ctw_in = 2 * (Lt + 1) * N, la = a.getLevel(), lb = b.getLevel();
+    if (la == lb && la > Lt && a.getRescaleCounter() == 0 && b.getRescaleCounter() == 0) {
+        const u64 nl = Lt + 2;
+        const i64 v = (i64)llround(c->delta[Lt] * (Real)c->q[Lt + 1] / c->delta[la]);
+        std::vector<u64> sc(nl);
+        for (u64 j = 0; j < nl; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
+        DeviceBuffer t(c, 4 * nl * N);
+        ck(hemm_mul_scalar(c->dev, a.buf_.data(), a.polyStride(), sc.data(), t.data(), nl * N, (uint32_t)nl, 0, 2, nullptr));
+        ck(hemm_mul_scalar(c->dev, b.buf_.data(), b.polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
+        ck(hemm_rescale(c->dev, t.data(), nl * N, joint, (nl - 1) * N, (uint32_t)nl, 4, nullptr));
+    } else {
+        Ciphertext la_ct(c), lb_ct(c);
+        eval.levelDown(a, Lt, la_ct);
+        eval.levelDown(b, Lt, lb_ct);
+        (void)hipMemcpyAsync(joint, la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(joint + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+    }
+}
+
+}  // namespace
+
+namespace {
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed);
 }
@@ -879,25 +906,8 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     {
         const u64 ctw_in = 2 * (Lt + 1) * N;
         DeviceBuffer joint(c, 2 * ctw_in);
-        const u64 la = pa->getLevel(), lb = pb->getLevel();
-        if (la == lb && la > Lt && pa->getRescaleCounter() == 0 && pb->getRescaleCounter() == 0) {
-            // HomEvaluator::levelDown of both operands at once: multiply by round(Delta_Lt q_{Lt+1} / Delta_level)
-            // over Lt+2 limbs, then one rescale of the four polynomials straight into the joint buffer
-            const u64 nl = Lt + 2;
-            const i64 v = (i64)llround(c->delta[Lt] * (Real)c->q[Lt + 1] / c->delta[la]);
-            std::vector<u64> sc(nl);
-            for (u64 j = 0; j < nl; j++) sc[j] = v >= 0 ? (u64)v % c->q[j] : (c->q[j] - (u64)(-v) % c->q[j]) % c->q[j];
-            DeviceBuffer t(c, 4 * nl * N);
-            ck(hemm_mul_scalar(c->dev, pa->buf_.data(), pa->polyStride(), sc.data(), t.data(), nl * N, (uint32_t)nl, 0, 2, nullptr));
-            ck(hemm_mul_scalar(c->dev, pb->buf_.data(), pb->polyStride(), sc.data(), t.data() + 2 * nl * N, nl * N, (uint32_t)nl, 0, 2, nullptr));
-            ck(hemm_rescale(c->dev, t.data(), nl * N, joint.data(), (nl - 1) * N, (uint32_t)nl, 4, nullptr));
-        } else {
-            Ciphertext la_ct(c), lb_ct(c);
-            eval.levelDown(*pa, Lt, la_ct);
-            eval.levelDown(*pb, Lt, lb_ct);
-            (void)hipMemcpyAsync(joint.data(), la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
-            (void)hipMemcpyAsync(joint.data() + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
-        }
+        (void)ctw_in;
+        jointLevelDown(eval, *pa, *pb, Lt, joint.data());
         const MaskKind kinds[2] = {packed ? MaskKind::PackedHorizontal : MaskKind::Horizontal,
                                    packed ? MaskKind::PackedVertical : MaskKind::Vertical};
         const TileTensorShape shapes[2] = {shape_a, shape_b};
@@ -1121,15 +1131,15 @@ void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a_i
 }
 
 void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &tr, const Ciphertext &a, const Ciphertext &b, i64 w,
-                        Ciphertext &pa, Ciphertext &pb) {
+                        Ciphertext &pa, Ciphertext &pb, u64 pack_level) {
     const Context &c = eval.getContext();
-    if (a.getLevel() != b.getLevel() || a.getRescaleCounter() != 0 || b.getRescaleCounter() != 0 || a.getNumPoly() != 2 ||
-        b.getNumPoly() != 2)
-        throw std::invalid_argument("[complexPacking] operands must share one level and be rescaled.");
-    const u64 L = a.getLevel(), N = c->N, ctw = 2 * (L + 1) * N, half = 2 * L * N;
+    if (a.getRescaleCounter() != 0 || b.getRescaleCounter() != 0 || a.getNumPoly() != 2 || b.getNumPoly() != 2)
+        throw std::invalid_argument("[complexPacking] operands must be rescaled.");
+    // operands above pack_level are lowered first (both at once): the packing then runs on fewer limbs
+    const u64 L = std::min<u64>(std::min(a.getLevel(), b.getLevel()), pack_level);
+    const u64 N = c->N, ctw = 2 * (L + 1) * N, half = 2 * L * N;
     DeviceBuffer joint(c, 2 * ctw), packed(c, 2 * half);
-    (void)hipMemcpyAsync(joint.data(), a.buf_.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
-    (void)hipMemcpyAsync(joint.data() + ctw, b.buf_.data(), ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+    jointLevelDown(eval, a, b, L, joint.data());
     const bool by_rows[2] = {false, true};
     tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, w, packed.data());
     Ciphertext ra(c), rb(c);

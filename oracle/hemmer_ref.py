@@ -821,8 +821,9 @@ def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
     complex slots (complexPackingInplace / complexPackingRowInplace, one level), the packed product then needs n / 2
     shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile."""
     ev = OracleEval(orc)
-    pa = complex_packing_hoisted(orc, a, w, rows=False)
-    pb = complex_packing_hoisted(orc, b, w, rows=True)
+    lvl = min(a.level, b.level, T + 5)        # packing at T+5 at most: the transforms start from T+4
+    pa = complex_packing_hoisted(orc, orc.level_down(a, lvl), w, rows=False)
+    pb = complex_packing_hoisted(orc, orc.level_down(b, lvl), w, rows=True)
     return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=True))
 
 
