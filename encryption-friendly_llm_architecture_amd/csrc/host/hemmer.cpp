@@ -471,16 +471,15 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
             b.get().getRescaleCounter() == 0) {
             // both packings through one launch chain, at level T+5 (the transforms start from T+4)
-            CtxtTensor pa(a), pb(b);
             ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});
-            complexPackingPair(eval_, matrix_transformer, a.get(), b.get(), w, pa.get(), pb.get(), T + 5);
             ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
             std::vector<u64> sq;
             ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, block < slots));
             KeyGenerator kg(context_, sk_, pack_);
             for (u64 r : sq) kg.genLeftRotSquareKey(r);
-            CtxtTensor prod = multPackedMatMatFused(eval_, btp_, pa, pb, T, matrix_transformer, batch_, block < slots);
+            CtxtTensor prod =
+                multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, block < slots);
             CtxtTensor res = repackCC(prod);
             if (block < slots) res.get().occupied_ = block;
             return res;

@@ -861,7 +861,8 @@ void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphert
 
 namespace {
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
-                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed);
+                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre = nullptr,
+                     u64 pre_level = 0);
 }
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
@@ -870,16 +871,19 @@ CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, co
 
 namespace {
 // packed: the operands are complex-packed (2 x 2 cells): sigma / tau of the packed kinds, n / 2 shifts of two columns /
-// two rows each; otherwise the same schedule
+// two rows each; otherwise the same schedule.  pre: both operands already side by side at pre_level (two ciphertexts
+// of two polynomials, the layout the joint transforms read); op1 / op2 then only give the tile shapes.
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
-                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed) {
+                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre, u64 pre_level) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
-    const u64 min_level = std::min(op1.getLevel(), op2.getLevel());
+    const u64 min_level = pre ? pre_level : std::min(op1.getLevel(), op2.getLevel());
     if (min_level < 1 + btp.getMinLevelForBootstrap())
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(1 + btp.getMinLevelForBootstrap()) +
                                     " is needed.");
+    if (pre && min_level < 4 + btp.getMinLevelForBootstrap())
+        throw RuntimeException("bootstrapping is not part of this build");
     // the operands are only read: no working copies unless they have to be refreshed first
     const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
     const Ciphertext *pa = &op1.get(), *pb = &op2.get();
@@ -905,16 +909,21 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     DeviceBuffer ab(c, 2 * ctw);
     {
         const u64 ctw_in = 2 * (Lt + 1) * N;
-        DeviceBuffer joint(c, 2 * ctw_in);
-        (void)ctw_in;
-        jointLevelDown(eval, *pa, *pb, Lt, joint.data());
+        DeviceBuffer joint;
+        const u64 *src = pre;
+        if (!pre || pre_level != Lt) {
+            if (pre) throw std::invalid_argument("[multMatMat] prepared operands must be at the transforms' level.");
+            joint = DeviceBuffer(c, 2 * ctw_in);
+            jointLevelDown(eval, *pa, *pb, Lt, joint.data());
+            src = joint.data();
+        }
         const MaskKind kinds[2] = {packed ? MaskKind::PackedHorizontal : MaskKind::Horizontal,
                                    packed ? MaskKind::PackedVertical : MaskKind::Vertical};
         const TileTensorShape shapes[2] = {shape_a, shape_b};
         if (two_stage)
-            tr.diagonalTransformTwoStage(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
+            tr.diagonalTransformTwoStage(eval, src, 2, Lt, kinds, shapes, ab.data());
         else
-            tr.diagonalTransformBatch(eval, joint.data(), 2, Lt, kinds, shapes, ab.data());
+            tr.diagonalTransformBatch(eval, src, 2, Lt, kinds, shapes, ab.data());
     }
     // the k = 0 term sigma(A) (x) tau(B) joins the accumulator at the shifts' level T+1
     Ciphertext acc(c);
@@ -1149,6 +1158,25 @@ void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &tr, const C
     (void)hipMemcpyAsync(rb.buf_.data(), packed.data() + half, half * 8, hipMemcpyDeviceToDevice, nullptr);
     pa = std::move(ra);
     pb = std::move(rb);
+}
+
+CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &a,
+                                        const CtxtTensor &b, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
+    const Context &c = eval.getContext();
+    if (a.get().getRescaleCounter() != 0 || b.get().getRescaleCounter() != 0 || a.get().getNumPoly() != 2 ||
+        b.get().getNumPoly() != 2)
+        throw std::invalid_argument("[complexPacking] operands must be rescaled.");
+    if (std::min(a.getLevel(), b.getLevel()) < T + 4)
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 4) + " is needed.");
+    // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
+    // is handed to the product where it lies
+    const u64 L = std::min<u64>(std::min(a.getLevel(), b.getLevel()), T + 5);
+    const u64 N = c->N;
+    DeviceBuffer joint(c, 2 * 2 * (L + 1) * N), packed(c, 2 * 2 * L * N);
+    jointLevelDown(eval, a.get(), b.get(), L, joint.data());
+    const bool by_rows[2] = {false, true};
+    tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data());
+    return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1);
 }
 
 // Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and
