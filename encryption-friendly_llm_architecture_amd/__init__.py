@@ -268,9 +268,10 @@ class Context:
         return y
 
     def compact_mask(self, mask, shift):
-        """run table [limbs][N >> shift] of a mask [limbs][N] constant over runs of 2^shift residues, or None"""
+        """run table [limbs][N >> shift][2] = (value, floor(value * 2^64 / prime)) of a mask [limbs][N] over the extended
+        basis that is constant over runs of 2^shift residues, or None"""
         import torch
-        table = torch.empty((mask.shape[0], self.N >> shift), dtype=torch.int64, device=mask.device)
+        table = torch.empty((mask.shape[0], self.N >> shift, 2), dtype=torch.int64, device=mask.device)
         ok = ctypes.c_int(0)
         check(lib().hemm_compact_mask(self.h, vp(mask.data_ptr()), mask.shape[0], shift, vp(table.data_ptr()),
                                       ctypes.byref(ok), vp(0)))

@@ -467,7 +467,8 @@ int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs,
                       int *is_constant, void *stream) {
     HEMM_TRY
     need(mask && table && is_constant, "null operand");
-    need(n_limbs >= 1 && shift >= 1 && (int)shift < ctx->logN, "shift must be in [1, log N)");
+    need((int)n_limbs > ctx->nP && shift >= 1 && (int)shift < ctx->logN,
+         "the mask must cover the extended basis and shift must be in [1, log N)");
     *is_constant = launch_compact_mask(ctx, (const u64 *)mask, (int)n_limbs, (int)shift, (u64 *)table, (hipStream_t)stream) ? 1 : 0;
     check_launch();
     HEMM_CATCH

@@ -151,6 +151,8 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
         m.k = 64 - (u32)__builtin_clzll(q);
         m.mu = (u64)((((u128)1) << (2 * m.k)) / q);
         m.pad = 0;
+        m.mu3 = (m.k == 59 || m.k == 60) ? (u64)((((u128)1) << (2 * m.k + 3)) / q) : 0;
+        m.pad2 = 0;
         c->modq[i] = m;
     }
     auto up = [&](const void *h, size_t bytes) -> void * {

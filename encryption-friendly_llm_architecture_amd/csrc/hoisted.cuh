@@ -39,11 +39,22 @@ __device__ __forceinline__ ulonglong2 stream_load2(const u64 *p) {
 }
 __device__ __forceinline__ u64 stream_load1(const u64 *p) { return __builtin_nontemporal_load(p); }
 // mask residues of the pair (n, n+1) of limb j: streamed from a full mask, or one value of a run table (every
-// lane of the workgroup reads the same one or two entries, which stay in cache)
+// lane of the workgroup reads the same one or two entries, which stay in cache).  A run table holds pairs
+// (value, floor(value * 2^64 / q)): the second word lets integer limbs multiply by the value as by a constant.
 __device__ __forceinline__ ulonglong2 load_mask2(const u64 *mask, const u32 shift, const int j, const u32 n, const int logN) {
     if (shift == 0) return stream_load2(mask + ((size_t)j << logN) + n);
-    const u64 v = mask[((size_t)j << (logN - shift)) + (n >> shift)];
+    const u64 v = mask[(((size_t)j << (logN - shift)) + (n >> shift)) * 2];
     return make_ulonglong2(v, v);
+}
+// (value, Shoup companion) of the run that holds the pair (n, n+1)
+__device__ __forceinline__ ulonglong2 load_mask_run(const u64 *mask, const u32 shift, const int j, const u32 n, const int logN) {
+    return *(const ulonglong2 *)(mask + (((size_t)j << (logN - shift)) + (n >> shift)) * 2);
+}
+// x1 * w1 + x2 * w2 mod q for run-table constants, canonical
+__device__ __forceinline__ u64 shoup_pair(u64 x1, const ulonglong2 w1, u64 x2, const ulonglong2 w2, u64 q) {
+    u64 z = mul_shoup_lazy(x1, w1.x, w1.y, q) + mul_shoup_lazy(x2, w2.x, w2.y, q);   // < 4q < 2^63
+    if (z >= 2 * q) z -= 2 * q;
+    return z >= q ? z - q : z;
 }
 // residues (n, n+1) of limb j of a plaintext read through the automorphism X -> X^g (an aligned pair stays an aligned
 // pair, possibly swapped)
@@ -87,6 +98,101 @@ __device__ __forceinline__ double u64_to_double(u64 v) {  // v < 2^52
     return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - 4503599627370496.0;
 }
 
+// One term with two masked sources under one key (integer path): residues (n, n+1) of limb j of
+// <z, evk> + P (mask b + mask2 b2) with z_d = mask * x_d + mask2 * x2_d, canonical.  RUNS: the masks are run tables
+// without a plaintext factor, i.e. constants with a Shoup companion: no wide product and no Barrett step for z_d.
+template <bool RUNS>
+__device__ __forceinline__ void two_source_int(const RotTermDev &T, const ModQ m, const CstList &pmod, const int j,
+                                               const int prime, const u32 n, const u32 base, const bool swap, int nq,
+                                               int E, int beta, int n_full, int logN, int b_premultiplied,
+                                               u64 (&rb)[2], u64 (&ra)[2]) {
+    const size_t N = (size_t)1 << logN;
+    ulonglong2 m1, m2;   // RUNS: (value, companion) of each mask; otherwise the mask residues of the pair
+    if (RUNS) {
+        m1 = load_mask_run(T.mask, T.mask_shift, j, n, logN);
+        m2 = load_mask_run(T.mask2, T.mask_shift, j, n, logN);
+    } else {
+        m1 = load_mask2(T.mask, T.mask_shift, j, n, logN);
+        m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
+        if (T.pt != nullptr) {
+            const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
+            m1.x = mulmod(m1.x, pv.x, m);
+            m1.y = mulmod(m1.y, pv.y, m);
+            m2.x = mulmod(m2.x, pv.x, m);
+            m2.y = mulmod(m2.y, pv.y, m);
+        }
+    }
+    u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
+    for (int d = 0; d < beta; d++) {
+        ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
+        ulonglong2 x2 = *(const ulonglong2 *)(T.ext2 + ((size_t)d * E + j) * N + base);
+        if (swap) {
+            u64 tmp = x1.x;
+            x1.x = x1.y;
+            x1.y = tmp;
+            tmp = x2.x;
+            x2.x = x2.y;
+            x2.y = tmp;
+        }
+        u64 z0, z1;
+        if (RUNS) {
+            z0 = shoup_pair(x1.x, m1, x2.x, m2, m.q);
+            z1 = shoup_pair(x1.y, m1, x2.y, m2, m.q);
+        } else {
+            u128_t t0 = mul64wide(m1.x, x1.x), t1 = mul64wide(m1.y, x1.y);
+            add128(t0, mul64wide(m2.x, x2.x));
+            add128(t1, mul64wide(m2.y, x2.y));
+            z0 = barrett3(t0, m);
+            z1 = barrett3(t1, m);
+        }
+        const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
+        const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+        add128(pb[0], mul64wide(z0, kb.x));
+        add128(pb[1], mul64wide(z1, kb.y));
+        add128(pa[0], mul64wide(z0, ka.x));
+        add128(pa[1], mul64wide(z1, ka.y));
+    }
+    if (beta <= 3) {   // at most 3 q^2: the short reduction applies
+        rb[0] = barrett3(pb[0], m);
+        rb[1] = barrett3(pb[1], m);
+        ra[0] = barrett3(pa[0], m);
+        ra[1] = barrett3(pa[1], m);
+    } else {
+        rb[0] = barrett128(pb[0], m);
+        rb[1] = barrett128(pb[1], m);
+        ra[0] = barrett128(pa[0], m);
+        ra[1] = barrett128(pa[1], m);
+    }
+    if (j < nq) {
+        ulonglong2 b1 = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
+        ulonglong2 b2 = *(const ulonglong2 *)(T.b2 + (size_t)j * N + base);
+        if (swap) {
+            u64 tmp = b1.x;
+            b1.x = b1.y;
+            b1.y = tmp;
+            tmp = b2.x;
+            b2.x = b2.y;
+            b2.y = tmp;
+        }
+        if (!b_premultiplied) {
+            b1.x = mul_shoup(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b1.y = mul_shoup(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b2.x = mul_shoup(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b2.y = mul_shoup(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+        }
+        if (RUNS) {
+            rb[0] = addmod(rb[0], shoup_pair(b1.x, m1, b2.x, m2, m.q), m.q);
+            rb[1] = addmod(rb[1], shoup_pair(b1.y, m1, b2.y, m2, m.q), m.q);
+        } else {
+            u128_t t0 = mul64wide(m1.x, b1.x), t1 = mul64wide(m1.y, b1.y);
+            add128(t0, mul64wide(m2.x, b2.x));
+            add128(t1, mul64wide(m2.y, b2.y));
+            rb[0] = addmod(rb[0], barrett3(t0, m), m.q);
+            rb[1] = addmod(rb[1], barrett3(t1, m), m.q);
+        }
+    }
+}
+
 // Residues (n, n+1) of limb j of both polynomials of output o (integer path), canonical.
 __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ terms,
                                                  const u32 *__restrict__ group_off, const ModQ m, const CstList &pmod,
@@ -104,66 +210,15 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         const bool swap = (np & 1u) != 0;
         if (T.ext2 != nullptr) {
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
-            ulonglong2 m1 = load_mask2(T.mask, T.mask_shift, j, n, logN);
-            ulonglong2 m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
-            if (T.pt != nullptr) {
-                const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
-                m1.x = mulmod(m1.x, pv.x, m);
-                m1.y = mulmod(m1.y, pv.y, m);
-                m2.x = mulmod(m2.x, pv.x, m);
-                m2.y = mulmod(m2.y, pv.y, m);
-            }
-            u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
-            for (int d = 0; d < beta; d++) {
-                ulonglong2 x1 = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
-                ulonglong2 x2 = *(const ulonglong2 *)(T.ext2 + ((size_t)d * E + j) * N + base);
-                if (swap) {
-                    u64 tmp = x1.x;
-                    x1.x = x1.y;
-                    x1.y = tmp;
-                    tmp = x2.x;
-                    x2.x = x2.y;
-                    x2.y = tmp;
-                }
-                u128_t t0 = mul64wide(m1.x, x1.x), t1 = mul64wide(m1.y, x1.y);
-                add128(t0, mul64wide(m2.x, x2.x));
-                add128(t1, mul64wide(m2.y, x2.y));
-                const u64 z0 = barrett128(t0, m), z1 = barrett128(t1, m);
-                const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-                const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
-                add128(pb[0], mul64wide(z0, kb.x));
-                add128(pb[1], mul64wide(z1, kb.y));
-                add128(pa[0], mul64wide(z0, ka.x));
-                add128(pa[1], mul64wide(z1, ka.y));
-            }
-            u64 rb0 = barrett128(pb[0], m), rb1 = barrett128(pb[1], m);
-            if (j < nq) {
-                ulonglong2 b1 = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
-                ulonglong2 b2 = *(const ulonglong2 *)(T.b2 + (size_t)j * N + base);
-                if (swap) {
-                    u64 tmp = b1.x;
-                    b1.x = b1.y;
-                    b1.y = tmp;
-                    tmp = b2.x;
-                    b2.x = b2.y;
-                    b2.y = tmp;
-                }
-                if (!b_premultiplied) {
-                    b1.x = mul_shoup(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b1.y = mul_shoup(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b2.x = mul_shoup(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                    b2.y = mul_shoup(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-                }
-                u128_t t0 = mul64wide(m1.x, b1.x), t1 = mul64wide(m1.y, b1.y);
-                add128(t0, mul64wide(m2.x, b2.x));
-                add128(t1, mul64wide(m2.y, b2.y));
-                rb0 = addmod(rb0, barrett128(t0, m), m.q);
-                rb1 = addmod(rb1, barrett128(t1, m), m.q);
-            }
-            acc_b[0] = addmod(acc_b[0], rb0, m.q);
-            acc_b[1] = addmod(acc_b[1], rb1, m.q);
-            acc_a[0] = addmod(acc_a[0], barrett128(pa[0], m), m.q);
-            acc_a[1] = addmod(acc_a[1], barrett128(pa[1], m), m.q);
+            u64 rb[2], ra[2];
+            if (T.mask_shift != 0 && T.pt == nullptr)
+                two_source_int<true>(T, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+            else
+                two_source_int<false>(T, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+            acc_b[0] = addmod(acc_b[0], rb[0], m.q);
+            acc_b[1] = addmod(acc_b[1], rb[1], m.q);
+            acc_a[0] = addmod(acc_a[0], ra[0], m.q);
+            acc_a[1] = addmod(acc_a[1], ra[1], m.q);
             continue;
         }
         u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
@@ -181,8 +236,18 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             add128(sa[0], mul64wide(x.x, ka.x));
             add128(sa[1], mul64wide(x.y, ka.y));
         }
-        u64 rb[2] = {barrett128(sb[0], m), barrett128(sb[1], m)};
-        u64 ra[2] = {barrett128(sa[0], m), barrett128(sa[1], m)};
+        u64 rb[2], ra[2];
+        if (beta <= 3) {
+            rb[0] = barrett3(sb[0], m);
+            rb[1] = barrett3(sb[1], m);
+            ra[0] = barrett3(sa[0], m);
+            ra[1] = barrett3(sa[1], m);
+        } else {
+            rb[0] = barrett128(sb[0], m);
+            rb[1] = barrett128(sb[1], m);
+            ra[0] = barrett128(sa[0], m);
+            ra[1] = barrett128(sa[1], m);
+        }
         if (j < nq && T.b != nullptr) {
             ulonglong2 bv = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
             if (swap) {

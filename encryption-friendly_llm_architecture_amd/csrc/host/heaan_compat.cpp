@@ -268,10 +268,10 @@ void Plaintext::allocate(u64 level, u64 rc) {
 bool Plaintext::makeCompact() {
     if (compact_shift_ != 0) return true;
     const u64 N = ctx_->N, limbs = buf_.words() / N;
-    if (limbs == 0 || ctx_->logN < 10) return false;
+    if (limbs != level_ + 1 + ctx_->nP || ctx_->logN < 10) return false;   // masks over the extended basis only
     // slot patterns of period 2^6 .. 2^8 give runs of 2^(logN-7) .. 2^(logN-9) residues: longest runs first
     for (u32 shift = (u32)ctx_->logN - 7; shift >= (u32)ctx_->logN - 9; shift--) {
-        DeviceBuffer t(ctx_, limbs * (N >> shift));
+        DeviceBuffer t(ctx_, 2 * limbs * (N >> shift));   // (value, Shoup companion) per run
         int ok = 0;
         ck(hemm_compact_mask(ctx_->dev, buf_.data(), (uint32_t)limbs, shift, t.data(), &ok, nullptr));
         if (ok) {

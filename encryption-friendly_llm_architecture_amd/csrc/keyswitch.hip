@@ -1089,22 +1089,40 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
         hipLaunchKernelGGL(masked_sum_list_kernel<3>, grid, block, 0, s, td, group_off_dev, out, c->d_modq, c->d_fp, nq,
                            c->logN, n_out);
 }
+// table[run] = (value, floor(value * 2^64 / q)) of each run of a mask over the extended basis; *differs is set when
+// some run is not constant
 __global__ __launch_bounds__(256) void compact_mask_kernel(const u64 *__restrict__ mask, u64 *__restrict__ table,
-                                                           size_t total, int shift, u32 *__restrict__ differs) {
+                                                           size_t total, int shift, int logN,
+                                                           const ModQ *__restrict__ modq, LimbList ll,
+                                                           u32 *__restrict__ differs) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;        // limb * N + position
     if (i >= total) return;
     const size_t run = i >> shift;
     const u64 v = mask[i], first = mask[run << shift];
-    if ((i & (((size_t)1 << shift) - 1)) == 0) table[run] = v;
+    if ((i & (((size_t)1 << shift) - 1)) == 0) {
+        const u64 q = modq[ll.idx[i >> logN]].q;
+        u64 rem = v, ws = 0;                                         // long division of v * 2^64 by q (v < q < 2^61)
+        for (int b = 0; b < 64; b++) {
+            rem <<= 1;
+            ws <<= 1;
+            if (rem >= q) {
+                rem -= q;
+                ws |= 1;
+            }
+        }
+        table[2 * run] = v;
+        table[2 * run + 1] = ws;
+    }
     if (v != first) atomicOr(differs, 1u);
 }
 bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s) {
+    if (n_limbs <= c->nP) throw std::invalid_argument("run tables are built for masks over the extended basis");
     u32 *flag = nullptr, h = 0;
     HEMM_HIP(hipMalloc((void **)&flag, sizeof(u32)));
     HEMM_HIP(hipMemcpyAsync(flag, &h, sizeof(u32), hipMemcpyHostToDevice, s));
     const size_t total = (size_t)n_limbs * c->N;
     hipLaunchKernelGGL(compact_mask_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, mask, table, total,
-                       shift, flag);
+                       shift, c->logN, c->d_modq, limbs_default(c, n_limbs - c->nP, 1), flag);
     HEMM_HIP(hipMemcpyAsync(&h, flag, sizeof(u32), hipMemcpyDeviceToHost, s));
     HEMM_HIP(hipStreamSynchronize(s));
     HEMM_HIP(hipFree(flag));

@@ -36,6 +36,8 @@ struct ModQ {
     u64 mu;    // floor(2^(2k) / q), k = bit length of q
     u32 k;     // bit length of q (q < 2^k, k <= 61)
     u32 pad;
+    u64 mu3;   // floor(2^(2k+3) / q) for k = 59 or 60, else 0 (barrett_tight)
+    u64 pad2;
 };
 
 // x * w mod q for a constant w with ws = floor(w * 2^64 / q); result in [0, 2q).
@@ -60,8 +62,23 @@ __device__ __forceinline__ u64 barrett128(u128_t t, const ModQ &m) {
     if (r >= q) r -= q;
     return r;
 }
+// Barrett reduction of T < 3 * 2^(2k) to [0, q) for primes of 59 or 60 bits (m.mu3 != 0) with the three bits longer
+// constant: qhat = floor(floor(T / 2^(k-2)) * mu3 / 2^(k+5)) misses floor(T / q) by less than
+// T / 2^(2k+3) + 2^(k-2) / q + 1 < 3/8 + 1/2 + 1, i.e. by at most 1: only the high half of one product and a single
+// correction, against a full product and three corrections in barrett128.
+__device__ __forceinline__ u64 barrett_tight(u128_t t, const ModQ &m) {
+    const u32 k = m.k;
+    const u64 t1 = (t.hi << (66 - k)) | (t.lo >> (k - 2));
+    const u64 qhat = __umul64hi(t1, m.mu3) >> (k - 59);
+    const u64 r = t.lo - qhat * m.q;
+    return r >= m.q ? r - m.q : r;
+}
+// T < 3 * 2^(2k)
+__device__ __forceinline__ u64 barrett3(u128_t t, const ModQ &m) {
+    return m.mu3 != 0 ? barrett_tight(t, m) : barrett128(t, m);
+}
 __device__ __forceinline__ u64 mulmod(u64 a, u64 b, const ModQ &m) {
-    return barrett128(mul64wide(a, b), m);
+    return barrett3(mul64wide(a, b), m);
 }
 // reduce an arbitrary 64-bit value
 __device__ __forceinline__ u64 reduce64(u64 a, const ModQ &m) {

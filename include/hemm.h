@@ -127,7 +127,7 @@ typedef struct {
     const uint64_t *b;    /* [nq][N], or NULL: the term contributes only the key product (used for the
                            * degree-2 component of a tensor product, with a key for the rotated s^2) */
     const uint64_t *evk;  /* [dnum][2][n_q+n_p][N] */
-    const uint64_t *mask; /* [nq+n_p][N] or NULL; with mask_shift = s > 0 a run table [nq+n_p][N >> s] */
+    const uint64_t *mask; /* [nq+n_p][N] or NULL; with mask_shift = s > 0 a run table [nq+n_p][N >> s][2] */
     uint32_t galois;
     uint32_t mask_shift;  /* 0: full mask.  s >= 1: the mask is constant over aligned runs of 2^s coefficients
                            * (the NTT form of a slot pattern with period 2^(logN-1-s)) and `mask` holds one value
@@ -146,9 +146,10 @@ void hemm_abi_sizes(uint32_t *rot_term_bytes, uint32_t *lin_term_bytes);
  * single ModDown.  No counterpart in HEaaN's interface. */
 int hemm_sum_parts(hemm_context *ctx, const uint64_t *parts, uint32_t n_parts, uint32_t n_out, uint32_t nq, uint64_t *y,
                    void *stream);
-/* Run table of a mask that is constant over aligned runs of 2^shift coefficients: table[j][r] = mask[j][r << shift]
- * for n_limbs limbs; *is_constant = 0 (and the table is not to be used) when some run of the mask is not constant.
- * Synchronises the stream.  No counterpart in HEaaN's interface: it removes the mask traffic of hoisted sums whose
+/* Run table of a mask over the extended basis (n_limbs = nq + n_p) that is constant over aligned runs of 2^shift
+ * coefficients: table[j][r] = { v = mask[j][r << shift], floor(v * 2^64 / prime_j) } (2 * n_limbs * (N >> shift)
+ * words; the second word lets the 60-bit limbs multiply by v as by a constant); *is_constant = 0 (and the table is
+ * not to be used) when some run of the mask is not constant.  Synchronises the stream.  No counterpart in HEaaN's interface: it removes the mask traffic of hoisted sums whose
  * masks select columns of a power-of-two period. */
 int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs, uint32_t shift, uint64_t *table,
                       int *is_constant, void *stream);

@@ -281,7 +281,12 @@ def test_hoisted_terms_with_run_table_masks(S):
     tmain, twrap = ctx.compact_mask(dmain, shift), ctx.compact_mask(dwrap, shift)
     assert tmain is not None and twrap is not None
     assert ctx.compact_mask(drand, shift) is None
-    assert np.array_equal(host(tmain), m_main.data[:, ::1 << shift])
+    tab = host(tmain)
+    assert np.array_equal(tab[:, :, 0], m_main.data[:, ::1 << shift])
+    primes = [orc.mods[i] for i in orc.ext_primes(nq - 1)]
+    for j in (0, nq - 1, len(primes) - 1):     # Shoup companions floor(v 2^64 / q), checked with Python integers
+        for r in (0, 1, tab.shape[1] - 1):
+            assert int(tab[j, r, 1]) == (int(tab[j, r, 0]) << 64) // int(primes[j])
     g1, g2 = orc.galois(37), orc.galois(orc.slots - 91)
     dk = {g: dev(orc.galois_key(g)) for g in (g1, g2)}
     # two sources under one key (merged), a single masked term, and a full mask beside a run table in one group
