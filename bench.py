@@ -161,8 +161,8 @@ def gpu_ntt(args, out):
 # HBM bytes per call of the hoisted sum at the shape below (its two launches together), from two rocprofv3 --pmc runs
 # of `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # 1 GiB copy this mode also launches (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0):
-# (2 x (208 965.9 + 172 138.5) + 196 608 + 163 840) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
-HOISTED_TRAFFIC_BYTES = 1149600563
+# (2 x (208 852.6 + 172 131.5) + 196 608 + 163 840) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
+HOISTED_TRAFFIC_BYTES = 1149354332
 
 
 def gpu_hoisted(args, out):
@@ -202,9 +202,10 @@ def gpu_hoisted(args, out):
         ctx.hoisted_terms(groups, nq, b_premultiplied=True)
     ms = timer.stop() / iters
     # algorithmic bytes: per output beta x 2 x E key limbs read + 2 x E limbs written (the mask tables are
-    # 2 x E x 2 KiB per output: counted, negligible); the two rotation sources (beta x E + nq limbs each) read once
+    # 2 x E x 4 KiB per output, a value and its Shoup companion per run: counted, negligible); the two rotation
+    # sources (beta x E + nq limbs each) read once
     limbs = n_out * (beta * 2 * E + 2 * E) + 2 * (beta * E + nq)
-    alg_bytes = limbs * LIMB_BYTES + n_out * 2 * E * (N >> shift) * 8
+    alg_bytes = limbs * LIMB_BYTES + n_out * 2 * E * (N >> shift) * 16
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     out["roofline"] = {
         "kernel": "hoisted_terms_kernel<1> + hoisted_terms_kernel<2> (one hoisted sum of the CCMM main loop: 32 outputs x "
