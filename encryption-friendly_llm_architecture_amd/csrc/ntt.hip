@@ -23,19 +23,29 @@ struct __align__(16) Tw {
     u64 w, ws;
 };
 
-__device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q2) {
-    u64 u = x;
-    if (u >= q2) u -= q2;
-    u64 v = mul_shoup_lazy(y, tw.w, tw.ws, q);
-    x = u + v;
-    y = u - v + q2;
+// x * w - hi' * q with the quotient estimate hi' taken from three of the four 32-bit partial products of x * ws:
+// hi' = xh wh + (xh wl >> 32) + (xl wh >> 32) is at most 2 below floor(x ws / 2^64), so the result lies in [0, 4q)
+// instead of [0, 2q) for any 64-bit x.  One multiply-add and the carry chain of the exact high product are saved.
+__device__ __forceinline__ u64 mul_shoup_lazy4(u64 x, u64 w, u64 ws, u64 q) {
+    const u32 xl = (u32)x, xh = (u32)(x >> 32), wl = (u32)ws, wh = (u32)(ws >> 32);
+    const u64 a = (u64)xh * wl, b = (u64)xl * wh;
+    const u64 hi = (u64)xh * wh + (a >> 32) + (b >> 32);
+    return x * w - hi * q;
 }
-__device__ __forceinline__ void gs_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q2) {
-    u64 u = x, v = y;
+// Lazy butterflies (q < 2^61, so 8q < 2^64): forward values stay in [0, 8q), inverse values in [0, 4q); q4 = 4q.
+__device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4) {
+    u64 u = x;
+    if (u >= q4) u -= q4;                                  // < 4q
+    const u64 v = mul_shoup_lazy4(y, tw.w, tw.ws, q);      // < 4q
+    x = u + v;
+    y = u - v + q4;
+}
+__device__ __forceinline__ void gs_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4) {
+    const u64 u = x, v = y;                                // < 4q each
     u64 s = u + v;
-    if (s >= q2) s -= q2;
+    if (s >= q4) s -= q4;
     x = s;
-    y = mul_shoup_lazy(u - v + q2, tw.w, tw.ws, q);
+    y = mul_shoup_lazy4(u - v + q4, tw.w, tw.ws, q);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -61,7 +71,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + (size_t)prime * N;
-    const u64 q = modq[prime].q, q2 = 2 * q;
+    const u64 q = modq[prime].q, q2 = 2 * q, q4 = 4 * q;
     u64 *base = data + (size_t)poly * poly_stride + (size_t)sl.idx[limb] * N;
     const int tile = blockIdx.x;
     // tile origin: strided pass tiles walk the columns; contiguous pass tiles walk the limb
@@ -84,7 +94,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
                 int gidx = r * gp.rowstride + c0 + cc;
                 Tw w = tw[(1 << s) + (gidx / (2 * t))];
                 u64 x = lds[i], y = lds[j];
-                ct_bfly(x, y, w, q, q2);
+                ct_bfly(x, y, w, q, q4);
                 lds[i] = x;
                 lds[j] = y;
             }
@@ -101,7 +111,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
                 int gidx = r * gp.rowstride + c0 + cc;
                 Tw w = tw[(1 << s) + (gidx / (2 * t))];
                 u64 x = lds[i], y = lds[j];
-                gs_bfly(x, y, w, q, q2);
+                gs_bfly(x, y, w, q, q4);
                 lds[i] = x;
                 lds[j] = y;
             }
@@ -115,8 +125,10 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
         if (gp.last) {
             if (INV) {
                 v = mul_shoup_lazy(v, ni, nis, q);
-            } else if (v >= q2)
-                v -= q2;
+            } else {
+                if (v >= q4) v -= q4;
+                if (v >= q2) v -= q2;
+            }
             if (v >= q) v -= q;
         }
         base[(size_t)r * gp.rowstride + c0 + cc] = v;
@@ -144,18 +156,20 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
 struct IntField {
     typedef u64 E;
     typedef Tw W;
-    u64 q, q2, ni, nis;
+    u64 q, q2, q4, ni, nis;
     __device__ __forceinline__ IntField(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
         q = modq[prime].q;
         q2 = 2 * q;
+        q4 = 4 * q;
         ni = ninv[prime];
         nis = ninv_s[prime];
     }
     __device__ __forceinline__ E from_canonical(u64 v) const { return v; }
-    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q2); }
-    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q2); }
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q4); }
+    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q4); }
     __device__ __forceinline__ void before_inverse_block(E (&)[16]) const {}
-    __device__ __forceinline__ u64 to_canonical(E v) const {
+    __device__ __forceinline__ u64 to_canonical(E v) const {   // v < 8q
+        if (v >= q4) v -= q4;
         if (v >= q2) v -= q2;
         return v >= q ? v - q : v;
     }

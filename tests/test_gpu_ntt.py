@@ -45,6 +45,35 @@ def test_ntt_matches_oracle(log_n):
     assert np.array_equal(_to_host(d), want)
 
 
+@pytest.mark.parametrize("log_n", [10, 16])
+def test_ntt_extreme_residues(log_n):
+    """Inputs that push the lazy butterflies towards the top of their ranges (values stay below 8q forward and 4q
+    inverse between corrections): all q-1, alternating 0 / q-1, q-1 in one half; the largest primes below 2^61,
+    below 2^60 and a small one."""
+    pkg = load_package()
+    qs = [O.nearest_prime(2**61 - 2**20, log_n), O.primes_below(60, log_n, 1)[0], O.nearest_prime(2**42, log_n)]
+    assert qs[0] < 2**61
+    ctx = pkg.Context(log_n, qs, [], 1)
+    orc = O.Oracle(log_n, qs, [], 1)
+    N = 1 << log_n
+    pats = []
+    for q in qs:
+        top = np.uint64(q - 1)
+        alt = np.zeros(N, dtype=np.uint64)
+        alt[::2] = top
+        half = np.zeros(N, dtype=np.uint64)
+        half[N // 2:] = top
+        pats.append([np.full(N, top, dtype=np.uint64), alt, half])
+    a = np.ascontiguousarray(np.array(pats).transpose(1, 0, 2))    # [pattern][limb][N]
+    idx = [0, 1, 2]
+    for inverse in (False, True):
+        d = _to_dev(a.copy())
+        ctx.ntt(d, idx, inverse=inverse)
+        want = a.copy()
+        orc.ntt(want, idx, inverse=inverse)
+        assert np.array_equal(_to_host(d), want)
+
+
 def test_ntt_config2_roundtrip_full_batch():
     """32 polys x 24 limbs x 2^16 with the 24 largest 60-bit NTT primes: bit-exact round trip on
     the whole batch, forward output checked against the oracle on a slice of it."""
