@@ -54,9 +54,18 @@ __global__ __launch_bounds__(256) void bconv_kernel(BConvArgs a, const ModQ *__r
     }
 }
 
+// v < 32q (q < 2^59) to [0, q)
+__device__ __forceinline__ u64 reduce_below_32q(u64 v, const u64 q) {
+#pragma unroll
+    for (int m = 16; m >= 1; m >>= 1)
+        if (v >= (u64)m * q) v -= (u64)m * q;
+    return v;
+}
+
 // Register form of the same conversion for up to 8 source limbs: a thread owns two adjacent coefficients
 // (16-byte accesses), keeps the scaled source residues in registers and sums the Shoup products of a
-// target limb lazily (each below 2q; reduced every 3 terms, which cannot overflow for q < 2^61).
+// target limb lazily (each below 2q; reduced every 3 terms, which cannot overflow for q < 2^61).  Targets below 2^59
+// take the cheaper products with a three-term quotient estimate (each below 4q) and reduce once at the end.
 template <int NS>
 __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ *__restrict__ modq) {
     const int poly = blockIdx.y;
@@ -76,6 +85,17 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
         const int pj = a.dst_prime[j];
         const u64 q = modq[pj].q;
         u64 acc0 = 0, acc1 = 0;
+        if (q < (1ull << 59)) {   // up to 8 terms below 4q each cannot overflow: no reductions on the way
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const Cst c = a.hat[i * a.hat_ld + pj];
+                acc0 += mul_shoup_lazy4(v0[i], c.w, c.ws, q);
+                acc1 += mul_shoup_lazy4(v1[i], c.w, c.ws, q);
+            }
+            *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) =
+                make_ulonglong2(reduce_below_32q(acc0, q), reduce_below_32q(acc1, q));
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < NS; i++) {
             const Cst c = a.hat[i * a.hat_ld + pj];
@@ -126,6 +146,19 @@ __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const 
         const int pj = a.dst_prime[j];
         const u64 q = modq[pj].q;
         u64 acc0 = 0, acc1 = 0;
+        if (q < (1ull << 59)) {
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                if (i < a.n_src) {
+                    const Cst c = a.hat[i * a.hat_ld + pj];
+                    acc0 += mul_shoup_lazy4(v0[i], c.w, c.ws, q);
+                    acc1 += mul_shoup_lazy4(v1[i], c.w, c.ws, q);
+                }
+            }
+            *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) =
+                make_ulonglong2(reduce_below_32q(acc0, q), reduce_below_32q(acc1, q));
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < NS; i++) {
             if (i < a.n_src) {

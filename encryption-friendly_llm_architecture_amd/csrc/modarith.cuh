@@ -49,6 +49,15 @@ __device__ __forceinline__ u64 mul_shoup(u64 x, u64 w, u64 ws, u64 q) {
     return r >= q ? r - q : r;
 }
 
+// x * w - hi' * q with the quotient estimate hi' taken from three of the four 32-bit partial products of x * ws:
+// hi' = xh wh + (xh wl >> 32) + (xl wh >> 32) is at most 2 below floor(x ws / 2^64), so the result lies in [0, 4q)
+// instead of [0, 2q) for any 64-bit x.  One multiply-add and the carry chain of the exact high product are saved.
+__device__ __forceinline__ u64 mul_shoup_lazy4(u64 x, u64 w, u64 ws, u64 q) {
+    const u32 xl = (u32)x, xh = (u32)(x >> 32), wl = (u32)ws, wh = (u32)(ws >> 32);
+    const u64 a = (u64)xh * wl, b = (u64)xl * wh;
+    const u64 hi = (u64)xh * wh + (a >> 32) + (b >> 32);
+    return x * w - hi * q;
+}
 // Barrett reduction of a 128-bit value T < 6 * 2^(2k) to [0, q).
 __device__ __forceinline__ u64 barrett128(u128_t t, const ModQ &m) {
     const u32 k = m.k;

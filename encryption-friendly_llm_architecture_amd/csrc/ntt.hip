@@ -23,15 +23,6 @@ struct __align__(16) Tw {
     u64 w, ws;
 };
 
-// x * w - hi' * q with the quotient estimate hi' taken from three of the four 32-bit partial products of x * ws:
-// hi' = xh wh + (xh wl >> 32) + (xl wh >> 32) is at most 2 below floor(x ws / 2^64), so the result lies in [0, 4q)
-// instead of [0, 2q) for any 64-bit x.  One multiply-add and the carry chain of the exact high product are saved.
-__device__ __forceinline__ u64 mul_shoup_lazy4(u64 x, u64 w, u64 ws, u64 q) {
-    const u32 xl = (u32)x, xh = (u32)(x >> 32), wl = (u32)ws, wh = (u32)(ws >> 32);
-    const u64 a = (u64)xh * wl, b = (u64)xl * wh;
-    const u64 hi = (u64)xh * wh + (a >> 32) + (b >> 32);
-    return x * w - hi * q;
-}
 // Lazy butterflies (q < 2^61, so 8q < 2^64): forward values stay in [0, 8q), inverse values in [0, 4q); q4 = 4q.
 __device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4) {
     u64 u = x;
