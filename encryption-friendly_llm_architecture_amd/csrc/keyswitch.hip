@@ -330,8 +330,10 @@ struct HoistedArgs {
     RotTermDev t[HOISTED_ARG_TERMS];
     u32 off[HOISTED_ARG_TERMS + 1];
 };
+// Register budget for five waves per SIMD (96 registers): the double-precision form needs 72 and the integer form 96;
+// the mixed form would take 109 and run at four waves, capped it spills two registers and gains a wave.
 template <int MODE>
-__global__ __launch_bounds__(256) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
                                                             int n_full, int logN, int b_premultiplied, int n_out,
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(256) void hoisted_terms_kernel(const HoistedArgs ar
                            n_j);
 }
 template <int MODE>
-__global__ __launch_bounds__(256) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
                                                                  const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                                  const ModQ *__restrict__ modq,
                                                                  const double *__restrict__ fp, LimbList ll, CstList pmod,
