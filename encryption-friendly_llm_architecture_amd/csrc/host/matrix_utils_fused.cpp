@@ -345,18 +345,28 @@ namespace {
 
 // Rotation sources in the form the hoisted launches read: ModUp of the a-polynomial and P * b of
 // n ciphertexts stored back to back ([n][2][nq][N]).
+// premultiply = false leaves b as it is (pbOf points into the ciphertexts and the hoisted launch multiplies by P
+// itself, `premultiplied()` = 0): one launch less for sources that a single short sum reads.
 struct Sources {
     DeviceBuffer ext, pb;  // [n][beta][E][N], [n][nq][N]
     u64 nq, ext_words;
     const u64 *extOf(size_t q) const { return ext.data() + q * ext_words; }
-    const u64 *pbOf(size_t q) const { return pb.data() + q * nq * N_; }
+    const u64 *pbOf(size_t q) const { return raw ? raw + q * 2 * nq * N_ : pb.data() + q * nq * N_; }
+    int premultiplied() const { return raw ? 0 : 1; }
     u64 N_;
+    const u64 *raw = nullptr;
 };
-Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq, hipStream_t stream = nullptr) {
+Sources extendSources(const Context &c, const u64 *cts, size_t n, u64 nq, hipStream_t stream = nullptr,
+                      bool premultiply = true) {
     const u64 N = c->N, E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha, ctw = 2 * nq * N;
-    Sources s{DeviceBuffer(c, n * beta * E * N), DeviceBuffer(c, n * nq * N), nq, beta * E * N, N};
+    Sources s{DeviceBuffer(c, n * beta * E * N), premultiply ? DeviceBuffer(c, n * nq * N) : DeviceBuffer(), nq,
+              beta * E * N, N};
     DeviceBuffer ws(c, n * nq * N);
     ck(hemm_modup_batch(c->dev, cts + nq * N, ctw, (uint32_t)nq, (uint32_t)n, s.ext.data(), ws.data(), stream));
+    if (!premultiply) {
+        s.raw = cts;
+        return s;
+    }
     std::vector<u64> sc(nq);
     for (u64 j = 0; j < nq; j++) {
         u64 P = 1;
@@ -567,7 +577,7 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         } join_on_exit{c};
         ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
         ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
-        const Sources x = extendSources(c, src, n_jobs, nq);
+        const Sources x = extendSources(c, src, n_jobs, nq, nullptr, false);
         const KeyPack &pack = eval.getKeyPack();
         const Rot rot(c);
         std::vector<hemm_rot_term> terms;
@@ -598,8 +608,8 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                 if (off[q + 1] == off[q])
                     throw RuntimeException("diagonalTransformTwoStage: jobs with and without rotations cannot share a batch");
             DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
-            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, 1, 1, y.data(), dst,
-                                    (nq - 1) * N, ws.data(), nullptr));
+            ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, x.premultiplied(), 1,
+                                    y.data(), dst, (nq - 1) * N, ws.data(), nullptr));
             c->joinSide();
             ck(hemm_pointwise(c->dev, HEMM_ADD, dst, (nq - 1) * N, zres.data(), (nq - 1) * N, dst, (nq - 1) * N,
                               (uint32_t)(nq - 1), 0, (uint32_t)(2 * n_jobs), nullptr));
@@ -657,7 +667,7 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
     } join_on_exit{c};
     ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
     ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
-    const Sources x = extendSources(c, in, n_jobs, nq);
+    const Sources x = extendSources(c, in, n_jobs, nq, nullptr, false);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
     std::vector<hemm_rot_term> terms;
@@ -669,8 +679,8 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
         off.push_back((uint32_t)terms.size());
     }
     DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
-    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, 1, 1, y.data(), out,
-                            (nq - 1) * N, ws.data(), nullptr));
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, x.premultiplied(), 1, y.data(),
+                            out, (nq - 1) * N, ws.data(), nullptr));
     c->joinSide();
     ck(hemm_pointwise(c->dev, HEMM_ADD, out, (nq - 1) * N, zres.data(), (nq - 1) * N, out, (nq - 1) * N, (uint32_t)(nq - 1), 0,
                       (uint32_t)(2 * n_jobs), nullptr));
@@ -718,7 +728,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     DeviceBuffer bb(c, (u64)g * ctl);
     const i64 copies = spread_block ? (i64)((c->N / 2) / spread_block) : 1;
     if (g > 1 || copies > 1) {
-        const Sources xb = extendSources(c, tau_b, 1, lo);
+        const Sources xb = extendSources(c, tau_b, 1, lo, nullptr, false);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         const i64 first_out = copies > 1 ? 0 : 1;   // bb[0] needs a launch only for its copies
@@ -731,8 +741,8 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         }
         const u64 n_out = (u64)(g - first_out);
         DeviceBuffer yb(c, n_out * 2 * (lo + K) * N), ws(c, n_out * ctl);
-        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_out, (uint32_t)lo, 1, 0, yb.data(),
-                                bb.data() + (u64)first_out * ctl, lo * N, ws.data(), nullptr));
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_out, (uint32_t)lo, xb.premultiplied(), 0,
+                                yb.data(), bb.data() + (u64)first_out * ctl, lo * N, ws.data(), nullptr));
     }
     if (copies > 1)
         ck(hemm_pointwise(c->dev, HEMM_ADD, bb.data(), lo * N, tau_b, lo * N, bb.data(), lo * N, (uint32_t)lo, 0, 2, nullptr));
@@ -788,7 +798,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     // extended by ONE ModUp batch (d1 of U_0 rides along unused)
     (void)acc;
     const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K, pw = lo * N, us = m * pw;
-    DeviceBuffer ext(c, 2 * m * beta * El * N), pb(c, m * lo * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
+    DeviceBuffer ext(c, 2 * m * beta * El * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
     ck(hemm_modup_batch(c->dev, U.data() + us, pw, (uint32_t)lo, (uint32_t)(2 * m), ext.data(), wsu.data(), nullptr));
     const u64 *ext1 = ext.data(), *ext2 = ext.data() + m * beta * El * N;   // [i2][beta][El][N] each
     std::vector<u64> sc(lo);
@@ -797,13 +807,13 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
         sc[j] = P;
     }
-    ck(hemm_mul_scalar(c->dev, U.data(), pw, sc.data(), pb.data(), lo * N, (uint32_t)lo, 0, (uint32_t)m, nullptr));
+    // d0 of every partial sum enters its term as it is (the launch multiplies by P); only P d1 of U_0 is made here
     ck(hemm_mul_scalar(c->dev, U.data() + us, pw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
     std::vector<hemm_rot_term> terms;
     {
         hemm_rot_term t{};
         t.ext = ext2;
-        t.b = pb.data();
+        t.b = U.data();
         t.evk = pack.multKey();
         t.mask = nullptr;
         t.galois = 1;
@@ -813,7 +823,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         const u64 gal = rot.galois((i64)i * g * ru);
         hemm_rot_term t{};
         t.ext = ext1 + i * beta * El * N;
-        t.b = pb.data() + i * lo * N;
+        t.b = U.data() + i * pw;
         t.evk = pack.galoisKey(gal);
         t.mask = nullptr;
         t.galois = gal;
@@ -826,7 +836,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     const uint32_t off[2] = {0, (uint32_t)terms.size()};
     res.get().allocate(2, T, 0);
     DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * (lo - 1) * N);
-    ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 1, nullptr));
+    ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 0, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_ADD, yg.data() + El * N, 0, pd1.data(), 0, yg.data() + El * N, 0, (uint32_t)lo, 0, 1, nullptr));
     ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 1, res.get().buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
 }
