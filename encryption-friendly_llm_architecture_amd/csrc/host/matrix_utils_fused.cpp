@@ -705,7 +705,7 @@ namespace {
 // is the rotation of tau(B) copied into every block (row shifts of a periodic vector are exact rotations).
 void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
                       std::vector<Plaintext> &cm, i64 n, i64 units, i64 cu, i64 w, u64 batch, DeviceBuffer *U_out,
-                      i64 *g_out, u64 spread_block = 0) {
+                      i64 *g_out, u64 spread_block = 0, bool u_ready = false) {
     const Context &c = eval.getContext();
     const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
     const i64 ru = cu * w;
@@ -756,9 +756,11 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
     // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
     const u64 pw = lo * N, us = (u64)n_giant * pw;
-    U_out->resize(c, 3 * us);
-    for (u64 p = 0; p < 3; p++)
-        (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, nullptr);
+    if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
+        U_out->resize(c, 3 * us);
+        for (u64 p = 0; p < 3; p++)
+            (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, nullptr);
+    }
     std::vector<bool> started((size_t)n_giant, false);
     started[0] = true;
     const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
@@ -940,13 +942,23 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     acc.allocate(3, T + 1, 1);
     DeviceBuffer low(c, 2 * 2 * lo * N);   // sigma(A), tau(B) at level T+1
     levelDownOneBatch(c, ab.data(), 4, T + 2, low.data());
-    ck(hemm_tensor_batch(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
+    const i64 cu = packed ? 2 : 1;
+    const u64 slots = c->N / 2;
+    const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
+    const bool bsgs = k / cu > 1 && ((u64)(k * w) == slots || spread);
+    DeviceBuffer U;
+    if (bsgs) {   // the term goes straight to the first partial sum of the baby-step / giant-step split
+        const u64 us = (u64)((k / cu) / bsgsBabyCount(k / cu)) * lo * N;
+        U.resize(c, 3 * us);
+        ck(hemm_tensor_batch_strided(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, U.data(), us, 0, nullptr));
+    } else {
+        ck(hemm_tensor_batch(c->dev, low.data(), low.data() + 2 * lo * N, 1, (uint32_t)lo, acc.buf_.data(), 0, nullptr));
+    }
     CtxtTensor res(c, rows, cols, w);
     auto finish = [&]() {
         eval.relinearize(acc, res.get());
         eval.rescale(res.get());
     };
-    const i64 cu = packed ? 2 : 1;
     if (k / cu <= 1) {
         finish();
         return res;
@@ -954,16 +966,13 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
 
     const i64 n = k;
     size_t G = std::max<u64>(1, std::min<u64>(batch, (u64)(n - 1)));
-    const u64 slots = c->N / 2;
-    const bool spread = single_tile && (u64)(n * w) < slots && slots % (u64)(n * w) == 0;
     // spread: tau(B) is copied into every tile block on the fly by the baby rotations (bsgsShiftProduct).  sigma(A)
     // stays as it is: rotated back by g k2 rows it spills into the empty block below and the giant step brings it
     // home, so the product comes out in the first block with the other blocks empty.
-    if ((u64)(n * w) == slots || spread) {
-        DeviceBuffer U;
+    if (bsgs) {
         i64 g = 1;
         bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n / cu, cu, w, batch, &U, &g,
-                         spread ? (u64)(n * w) : 0);
+                         spread ? (u64)(n * w) : 0, true);
         bsgsGiantSteps(eval, T, U, g, (n / cu) / g, cu * w, acc, res);
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
