@@ -121,9 +121,12 @@ public:
     // rows of rows `w` slots wide -> a - i b) of n_jobs ciphertexts at `level` through one launch chain: both
     // rotations of every job from one ModUp, masks applied in the extended basis, ModDown merged with the rescale.
     // in: [job][2][level+1][N], out: [job][2][level][N].
+    // scale_levels (optional): job q is a truncated ciphertext that still carries the fixed scale of level
+    // scale_levels[q] >= level; its masks absorb the change of scale (no levelDown in front)
     void complexPackingBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const bool *rows, i64 w,
-                             u64 *out);
-    std::map<std::tuple<int, i64, u64, int>, Plaintext> pack_masks_;   // (rows, w, level, part 0 = Z / 1 = +step / 2 = -step)
+                             u64 *out, const u64 *scale_levels = nullptr);
+    // (rows, w, level, part 0 = Z / 1 = +step / 2 = -step, level of the input's scale)
+    std::map<std::tuple<int, i64, u64, int, u64>, Plaintext> pack_masks_;
     std::map<std::tuple<u64, TileTensorShape, u64>, WeightTau> weight_tau_;
     std::vector<std::tuple<u64, TileTensorShape, u64>> weight_tau_order_;
 

@@ -626,13 +626,15 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
 // i.e. Z = m +- i m', M_+ = +- i m, M_- = m' with m'[s] = m[s - step].  One hoisted sum with two terms per job plus
 // rescale(Z x) on the side stream.
 void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
-                                            const bool *rows, i64 w, u64 *out) {
+                                            const bool *rows, i64 w, u64 *out, const u64 *scale_levels) {
     const Context &c = eval.getContext();
     if (level < 1) throw std::invalid_argument("[complexPacking] level >= 1 is needed.");
     const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N, slots = N / 2;
     const u64 log_slots = getLogFullSlots(c);
-    auto mask = [&](bool by_rows, int part) -> const Plaintext & {
-        const auto key = std::make_tuple((int)by_rows, w, level, part);
+    // All three masks of a job are encoded over the extended basis (the unrotated term reads the chain limbs only) at
+    // the scale that takes the input's scale to the fixed scale of level - 1 across the rescale.
+    auto mask = [&](bool by_rows, int part, u64 from) -> const Plaintext & {
+        const auto key = std::make_tuple((int)by_rows, w, level, part, from);
         auto it = pack_masks_.find(key);
         if (it != pack_masks_.end()) return it->second;
         const u64 step = by_rows ? (u64)w : 1;
@@ -644,20 +646,23 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
             m[s] = part == 0 ? Complex(here, 0) + iu * prev : part == 1 ? iu * here : Complex(prev, 0);
         }
         EnDecoder endec(c);
-        return pack_masks_.emplace(key, part == 0 ? endec.encode(m, level) : endec.encodeExtended(m, level)).first->second;
+        const Real scale = from == level ? c->delta[level] : c->delta[level - 1] * (Real)c->q[level] / c->delta[from];
+        return pack_masks_.emplace(key, endec.encodeExtended(m, level, scale)).first->second;
     };
+    auto from_of = [&](size_t q) { return scale_levels ? scale_levels[q] : level; };
     std::vector<hemm_lin_term> zero_terms;
     std::vector<uint32_t> zoff{0};
     for (size_t q = 0; q < n_jobs; q++) {
         hemm_lin_term t;
         t.ct = in + q * ctw;
-        t.mask = mask(rows[q], 0).buf_.data();
+        if (from_of(q) < level) throw std::invalid_argument("[complexPacking] the scale must come from the same or a higher level.");
+        t.mask = mask(rows[q], 0, from_of(q)).buf_.data();
         t.stride = nq * N;
         t.galois = 0;
         zero_terms.push_back(t);
         zoff.push_back((uint32_t)zero_terms.size());
-        (void)mask(rows[q], 1);    // encoded before the fork below
-        (void)mask(rows[q], 2);
+        (void)mask(rows[q], 1, from_of(q));    // encoded before the fork below
+        (void)mask(rows[q], 2, from_of(q));
     }
     DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
     const hipStream_t side = c->forkSide();
@@ -674,8 +679,8 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
     std::vector<uint32_t> off{0};
     for (size_t q = 0; q < n_jobs; q++) {
         const i64 step = rows[q] ? w : 1;
-        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(step), &mask(rows[q], 1)));
-        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(-step), &mask(rows[q], 2)));
+        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(step), &mask(rows[q], 1, from_of(q))));
+        terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(-step), &mask(rows[q], 2, from_of(q))));
         off.push_back((uint32_t)terms.size());
     }
     DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
@@ -1188,13 +1193,19 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     if (std::min(a.getLevel(), b.getLevel()) < T + 4)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 4) + " is needed.");
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
-    // is handed to the product where it lies
+    // is handed to the product where it lies.  Operands above the packing level are only truncated to it (a copy of
+    // their first L+1 limbs): the packing masks absorb the change of scale, which saves the levelDown.
     const u64 L = std::min<u64>(std::min(a.getLevel(), b.getLevel()), T + 5);
-    const u64 N = c->N;
-    DeviceBuffer joint(c, 2 * 2 * (L + 1) * N), packed(c, 2 * 2 * L * N);
-    jointLevelDown(eval, a.get(), b.get(), L, joint.data());
+    const u64 N = c->N, ctw = 2 * (L + 1) * N;
+    DeviceBuffer joint(c, 2 * ctw), packed(c, 2 * 2 * L * N);
+    const std::vector<u64> one(L + 1, 1);
+    const Ciphertext *ops[2] = {&a.get(), &b.get()};
+    for (int q = 0; q < 2; q++)
+        ck(hemm_mul_scalar(c->dev, ops[q]->buf_.data(), ops[q]->polyStride(), one.data(), joint.data() + q * ctw, (L + 1) * N,
+                           (uint32_t)(L + 1), 0, 2, nullptr));
     const bool by_rows[2] = {false, true};
-    tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data());
+    const u64 from[2] = {a.getLevel(), b.getLevel()};
+    tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data(), from);
     return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1);
 }
 

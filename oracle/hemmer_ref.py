@@ -806,24 +806,31 @@ def packing_maps(slots, w, rows):
 def complex_packing_hoisted(orc, x, w, rows):
     """complexPackingInplace / complexPackingRowInplace as ONE hoisted sum (both rotations from one ModUp, masks
     applied in the extended basis, ModDown merged with the rescale) plus rescale(Z x): one level, like the
-    reference's two masked steps."""
+    reference's two masked steps.  x may be a truncated ciphertext that still carries the scale of a higher level:
+    the masks are then encoded at Delta_(l-1) q_l / scale(x) instead of Delta_l, so that the result has the fixed
+    scale of level l - 1 without a levelDown in front."""
     from .oracle import Ct
     zmask, terms = packing_maps(orc.slots, w, rows)
-    nq = x.nq
+    nq, lvl = x.nq, x.level
+    ms = orc.delta[lvl] if x.scale == orc.delta[lvl] else orc.delta[lvl - 1] * float(orc.q[lvl]) / x.scale
     ext = orc.modup(x.data[1])
-    zero = orc.rescale(orc.mult_plain_no_rescale(x, orc.encode(zmask, x.level)))
-    y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, x.level)) for r, m in terms], nq)
+    zero = orc.rescale(orc.mult_plain_no_rescale(x, orc.encode(zmask, lvl, ms)))
+    y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, lvl, ms)) for r, m in terms], nq)
+    zero.scale = orc.delta[lvl - 1]
     return orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
 
 
 def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
     """One product through the complex-packed route: adjacent columns of A and adjacent rows of B are fused into
     complex slots (complexPackingInplace / complexPackingRowInplace, one level), the packed product then needs n / 2
-    shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile."""
+    shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile.
+    Operands above the packing level are only truncated to it (the packing masks absorb the change of scale)."""
+    from .oracle import Ct
     ev = OracleEval(orc)
     lvl = min(a.level, b.level, T + 5)        # packing at T+5 at most: the transforms start from T+4
-    pa = complex_packing_hoisted(orc, orc.level_down(a, lvl), w, rows=False)
-    pb = complex_packing_hoisted(orc, orc.level_down(b, lvl), w, rows=True)
+    cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
+    pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
+    pb = complex_packing_hoisted(orc, cut(b), w, rows=True)
     return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=True))
 
 

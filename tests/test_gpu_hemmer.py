@@ -166,20 +166,22 @@ def test_ccmm_single_tile_promise(small):
 
 
 def test_ccmm_packed_route_at_lower_and_mixed_levels(small):
-    """The complex-packed route below its preferred level: operands at T+4 are packed there and the packed transforms
-    run in one stage; operands at different levels are lowered to the smaller one (capped at T+5) first."""
+    """The complex-packed route away from its preferred level: operands at T+4 are packed there and the packed
+    transforms run in one stage; operands above T+5 or at different levels are truncated to the packing level, their
+    packing masks absorbing the change of scale."""
     H, orc, ev = small
     rng = np.random.default_rng(23)
     A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
     ca, cb = H.encrypt(A), H.encrypt(B)
-    T = 2
-    for la, lb in ((T + 4, T + 4), (T + 5, T + 4), (T + 4, T + 5)):
-        a = H.level_down(ca, la) if la < ca.info()["level"] else ca
-        b = H.level_down(cb, lb) if lb < cb.info()["level"] else cb
+    top = ca.info()["level"]
+    assert top == 7
+    for T, la, lb in ((2, 6, 6), (2, 7, 6), (2, 6, 7), (1, 7, 7), (1, 7, 6), (1, 5, 7)):
+        a = H.level_down(ca, la) if la < top else ca
+        b = H.level_down(cb, lb) if lb < top else cb
         c = H.single_cc_matmul(a, b, T)
         want = R.mult_mat_mat_cc_packed_single(orc, to_oracle(orc, a), to_oracle(orc, b), T, 16, 16)
         assert c.info()["level"] == T
-        assert np.array_equal(c.residues(), want.data), (la, lb)
+        assert np.array_equal(c.residues(), want.data), (T, la, lb)
         assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
 
 

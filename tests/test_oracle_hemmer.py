@@ -37,6 +37,21 @@ def test_ccmm_over_oracle(env):
     assert np.abs(z[n * n:]).max() < 2 ** -20
 
 
+@pytest.mark.parametrize("T", [1, 2])
+def test_complex_packed_single_ccmm_over_oracle(env, T):
+    """One product through the complex-packed route.  With T = 1 the fresh operands (level 7) sit above the packing
+    level T + 5: they are only truncated, and the packing masks carry the change of scale."""
+    orc, ev, n = env
+    rng = np.random.default_rng(5)
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    c = R.mult_mat_mat_cc_packed_single(orc, enc(orc, A, 21), enc(orc, B, 22), T, n, n)
+    assert c.level == T and c.scale == orc.delta[T]
+    z = orc.decrypt(c)
+    assert np.abs(z[: n * n].real.reshape(n, n) - A @ B).max() < 2 ** -18
+    assert np.abs(z[: n * n].imag).max() < 2 ** -18
+    assert np.abs(z[n * n:]).max() < 2 ** -18
+
+
 def test_packed_ccmm_over_oracle(env):
     orc, ev, n = env
     rng = np.random.default_rng(1)
