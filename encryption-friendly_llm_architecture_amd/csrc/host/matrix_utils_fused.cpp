@@ -798,13 +798,21 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
 void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
                     CtxtTensor &res) {
     const Context &c = eval.getContext();
-    const u64 N = c->N, K = c->nP, lo = T + 2;
+    const u64 N = c->N, K = c->nP, lo = T + 1;
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
-    // U is polynomial-major ([3][n_giant][lo][N]): d1 and d2 of all partial sums are 2 n_giant polynomials in a row,
-    // extended by ONE ModUp batch (d1 of U_0 rides along unused)
+    // The partial sums (three polynomials each, level T+1) are rescaled first: everything after runs on T+1 instead
+    // of T+2 limbs -- one digit instead of two where that crosses a digit boundary -- and ends in a plain ModDown.
+    // U is polynomial-major ([3][n_giant][.][N]): all 3 n_giant polynomials are rescaled by one launch chain, and d1 and
+    // d2 of all partial sums are 2 n_giant polynomials in a row, extended by ONE ModUp batch (d1 of U_0 rides along
+    // unused).
     (void)acc;
     const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K, pw = lo * N, us = m * pw;
+    {
+        DeviceBuffer Ur(c, 3 * us);
+        ck(hemm_rescale(c->dev, U.data(), (lo + 1) * N, Ur.data(), pw, (uint32_t)(lo + 1), (uint32_t)(3 * m), nullptr));
+        U = std::move(Ur);
+    }
     DeviceBuffer ext(c, 2 * m * beta * El * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
     ck(hemm_modup_batch(c->dev, U.data() + us, pw, (uint32_t)lo, (uint32_t)(2 * m), ext.data(), wsu.data(), nullptr));
     const u64 *ext1 = ext.data(), *ext2 = ext.data() + m * beta * El * N;   // [i2][beta][El][N] each
@@ -842,10 +850,10 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     }
     const uint32_t off[2] = {0, (uint32_t)terms.size()};
     res.get().allocate(2, T, 0);
-    DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * (lo - 1) * N);
+    DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * lo * N);
     ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 0, nullptr));
     ck(hemm_pointwise(c->dev, HEMM_ADD, yg.data() + El * N, 0, pd1.data(), 0, yg.data() + El * N, 0, (uint32_t)lo, 0, 1, nullptr));
-    ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 1, res.get().buf_.data(), (lo - 1) * N, wsg.data(), nullptr));
+    ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 0, res.get().buf_.data(), lo * N, wsg.data(), nullptr));
 }
 }  // namespace
 

@@ -721,9 +721,11 @@ def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0)
     for i in range(1, units):
         t = orc.tensor(ta[i - 1], bb[i % g])
         U[i // g] = t if U[i // g] is None else orc.add(U[i // g], t)
-    # one hoisted sum for everything: U_0 gives its d2 under the multiplication key (no rotation) and its d1,
-    # times P, is added to the second polynomial of the sum before the ModDown merged with the rescale
-    lo = b_low.nq
+    # The partial sums are rescaled first (three polynomials each), then one hoisted sum for everything, a level lower:
+    # U_0 gives its d2 under the multiplication key (no rotation) and its d1, times P, is added to the second polynomial
+    # of the sum before the plain ModDown
+    U = [orc.rescale(u) for u in U]
+    lo = b_low.nq - 1
     terms = [(orc.modup(U[0].data[2]), U[0].data[0], ("mult", 1), None)]
     for i2 in range(1, units // g):
         gal = orc.galois((i2 * g * ru) % orc.slots)
@@ -732,7 +734,7 @@ def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0)
         terms.append((orc.modup(u.data[2]), None, ("sq", gal), None))
     y = orc.hoisted_sum(terms, lo)
     y[1, :lo] = orc.add_residues(y[1, :lo], orc.mul_p_residues(U[0].data[1]))
-    return Ct(orc.moddown_drop(y, lo, True), orc.delta[b_low.level - 1])
+    return Ct(orc.moddown_drop(y, lo, False), orc.delta[b_low.level - 1])
 
 
 def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
