@@ -810,7 +810,13 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     const u64 m = (u64)n_giant, beta = (lo + c->alpha - 1) / c->alpha, El = lo + K, pw = lo * N, us = m * pw;
     {
         DeviceBuffer Ur(c, 3 * us);
-        ck(hemm_rescale(c->dev, U.data(), (lo + 1) * N, Ur.data(), pw, (uint32_t)(lo + 1), (uint32_t)(3 * m), nullptr));
+        // a rescale call works in the context's scratch region of (dnum + 7) (nQ + nP) limbs
+        const u64 cap = std::max<u64>(1, (c->dnum + 7) * (c->nQ + c->nP) / (lo + 1));
+        for (u64 first = 0; first < 3 * m; first += cap) {
+            const u64 cnt = std::min<u64>(cap, 3 * m - first);
+            ck(hemm_rescale(c->dev, U.data() + first * (lo + 1) * N, (lo + 1) * N, Ur.data() + first * pw, pw,
+                            (uint32_t)(lo + 1), (uint32_t)cnt, nullptr));
+        }
         U = std::move(Ur);
     }
     DeviceBuffer ext(c, 2 * m * beta * El * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
