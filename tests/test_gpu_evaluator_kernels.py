@@ -258,6 +258,38 @@ def test_batched_hoisted_forms(S):
     assert np.array_equal(host(acc), want3.data)
 
 
+def test_hoisted_terms_extreme_residues(S):
+    """Every operand of a hoisted sum at q - 1 (sources, b, key, masks): the largest sums of products the
+    reductions of the integer and the double-precision paths ever see, for merged two-source terms (full masks and
+    run tables), single terms and an unmasked term."""
+    orc, ctx, N = S.orc, S.ctx, S.N
+    nq = orc.nQ - 1
+    beta = (nq + orc.alpha - 1) // orc.alpha
+    ext_primes = [orc.mods[i] for i in orc.ext_primes(nq - 1)]
+    top = lambda primes, prefix: np.stack([np.full(tuple(prefix) + (N,), q - 1, dtype=np.uint64) for q in primes],
+                                          axis=len(prefix))
+    ext = np.ascontiguousarray(top(ext_primes, (beta,)))                   # [beta][E][N]
+    b = np.ascontiguousarray(top(orc.q[:nq], ()))                          # [nq][N]
+    evk = np.ascontiguousarray(top(orc.mods, (orc.dnum, 2)))               # [dnum][2][nQ+nP][N]
+    mask = O.Pt(np.ascontiguousarray(top(ext_primes, ())), 1.0)            # [E][N]
+    g1, g2 = orc.galois(5), orc.galois(orc.slots - 3)
+    dext, db, dk, dm = dev(ext), dev(b), dev(evk), dev(mask.data)
+    groups = [[(dext, db, dk, dm, g1), (dext, db, dk, dm, g1)],            # merged: two sources under one key
+              [(dext, db, dk, dm, g2), (dext, db, dk, None, g1)]]          # single terms, masked and unmasked
+    shift = orc.log_n - 8
+    tm = ctx.compact_mask(dm, shift)                                       # the same masks as run tables
+    assert tm is not None
+    groups.append([(dext, db, dk, tm, g1, shift), (dext, db, dk, tm, g1, shift)])
+    y = host(ctx.hoisted_terms(groups, nq))
+    L, h = orc.L, orc.h
+    for k, terms in enumerate([[(mask, g1), (mask, g1)], [(mask, g2), (None, g1)], [(mask, g1), (mask, g1)]]):
+        want = np.zeros((2, nq + orc.nP, N), dtype=np.uint64)
+        for i, (mk, g) in enumerate(terms):
+            L.orc_hoisted_term(h, O._p(ext), O._p(b), O._p(evk), O._p(mk.data) if mk is not None else None, g, nq,
+                               O._p(want), int(i > 0))
+        assert np.array_equal(y[k], want), k
+
+
 def test_hoisted_terms_with_run_table_masks(S):
     """A slot pattern of period 128 is, in NTT form, constant over aligned runs of N/256 residues: the hoisted sums
     read such a mask from its run table and must give the residues of the full mask; a mask without that
