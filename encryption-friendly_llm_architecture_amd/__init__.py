@@ -68,6 +68,7 @@ def _declare(L):
     L.hemm_rotate.argtypes = [vp, vp, sz, vp, u64, u32, vp, sz, vp]
     L.hemm_relinearize.argtypes = [vp, vp, sz, vp, u32, vp, sz, vp]
     L.hemm_rescale.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
+    L.hemm_rescale_static.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
     L.hemm_sample_uniform.argtypes = [vp, u64p, u32p, u32, vp, vp]
     L.hemm_sample_error.argtypes = [vp, u64, u32p, u32, vp, vp]
     L.hemm_modup_batch.argtypes = [vp, vp, sz, u32, u32, vp, vp, vp]
@@ -245,6 +246,12 @@ class Context:
         out = self._new(ct.shape[0], nq - 1, ct)
         check(lib().hemm_rescale(self.h, vp(ct.data_ptr()), self._ps(ct), vp(out.data_ptr()),
                                  self._ps(out), nq, ct.shape[0], vp(0)))
+        return out
+
+    def rescale_static(self, ct, nq, out):
+        """hemm_rescale_static: the caller brings the output buffer, the call allocates nothing."""
+        check(lib().hemm_rescale_static(self.h, vp(ct.data_ptr()), self._ps(ct), vp(out.data_ptr()),
+                                        self._ps(out), nq, ct.shape[0], vp(0)))
         return out
 
 

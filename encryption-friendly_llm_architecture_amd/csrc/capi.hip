@@ -9,6 +9,10 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
 void hemm_context_free(hemm_context *c);
 void hemm_primes_below_impl(int bits, int logN, int count, u64 *out);
 void hemm_keyswitch_tables_free(const hemm_context *c);
+void hemm_static_setup(hemm_context *c);
+size_t hemm_static_scratch_words();
+void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
+                           int n_polys, hipStream_t s);
 
 static thread_local std::string g_err;
 void hemm_set_error(const std::string &m) { g_err = m; }
@@ -39,7 +43,15 @@ int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64
                         hemm_context **out) {
     HEMM_TRY
     need(out && primes, "null argument");
-    *out = hemm_context_build((int)log_n, (int)n_q, (int)n_p, (const u64 *)primes, (int)dnum);
+    hemm_context *c = hemm_context_build((int)log_n, (int)n_q, (int)n_p, (const u64 *)primes, (int)dnum);
+    try {
+        hemm_static_setup(c);   // constant tables and the address of the static scratch: hemm_rescale_static allocates nothing
+    } catch (...) {
+        hemm_keyswitch_tables_free(c);
+        hemm_context_free(c);
+        throw;
+    }
+    *out = c;
     HEMM_CATCH
 }
 void hemm_context_destroy(hemm_context *ctx) {
@@ -502,6 +514,20 @@ int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64
          "n_polys * nq limbs must fit the context's scratch ((dnum + 7) * (nQ + nP) limbs)");
     launch_rescale(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
                    (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_rescale_static(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out, size_t out_stride,
+                        uint32_t nq, uint32_t n_polys, void *stream) {
+    HEMM_TRY
+    need(ctx && in && out, "null operand");
+    need(ctx->logN >= 9, "residue kernels need log_n >= 9");
+    need(nq >= 2 && nq <= (uint32_t)ctx->nQ, "nq must be in [2, n_q]");
+    need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_static_scratch_words(),
+         "n_polys * nq * N must not exceed HEMM_STATIC_SCRATCH_WORDS");
+    launch_rescale_static(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
+                          (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

@@ -840,13 +840,11 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
     launch_moddown(c, acc, nq, 2, out, out_stride, add_b, 0, add_b ? 1 : 0, coef, s);
 }
 
-// in: [n_polys][nq][N] -> out: [n_polys][nq-1][N]
-void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
-                    int n_polys, hipStream_t s) {
-    if (nq < 2) throw std::invalid_argument("rescale needs at least two limbs");
-    KsTables *t = g_tables_of(c);
+// in: [n_polys][nq][N] -> out: [n_polys][nq-1][N]; sc: scratch of n_polys * nq * N words, fully written before it
+// is read
+static void rescale_with(hemm_context *c, KsTables *t, u64 *sc, const u64 *in, size_t in_stride, u64 *out,
+                         size_t out_stride, int nq, int n_polys, hipStream_t s) {
     const size_t N = c->N;
-    u64 *sc = hemm_scratch(c);
     u64 *last = sc;                               // [n_polys][N]
     u64 *tt = sc + (size_t)n_polys * N;           // [n_polys][nq-1][N]
     LimbList pl, ident;
@@ -868,6 +866,60 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
     for (int j = 0; j < nq - 1; j++) cl.c[j] = t->qlinv[nq - 1][j];
     hipLaunchKernelGGL(sub_scale_kernel, grid, block, 0, s, in, in_stride, tt, (size_t)(nq - 1) * N,
                        (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq - 1, c->logN);
+}
+
+void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
+                    int n_polys, hipStream_t s) {
+    if (nq < 2) throw std::invalid_argument("rescale needs at least two limbs");
+    rescale_with(c, g_tables_of(c), hemm_scratch(c), in, in_stride, out, out_stride, nq, n_polys, s);
+}
+
+// ---- rescale for callers that cannot allocate ----------------------------------------------------
+// The scratch of the call below lives in the library's own device image: 32 limbs of N = 2^16 (16 MiB) per GPU the
+// library runs on, held until the process ends.  Host code never passes the array's name to a kernel or a copy: the
+// name is only a handle for hipGetSymbolAddress, which yields the array's address on the device that is current,
+// and each device has its own.
+#define HEMM_STATIC_SCRATCH_WORDS ((size_t)32 << 16)
+#define HEMM_MAX_DEVICES 64
+static __device__ __align__(256) u64 scratch[HEMM_STATIC_SCRATCH_WORDS];
+static u64 *g_static_scratch[HEMM_MAX_DEVICES];   // per device, filled by hemm_static_setup
+
+size_t hemm_static_scratch_words() { return HEMM_STATIC_SCRATCH_WORDS; }
+
+// Set-up for launch_rescale_static, run by hemm_context_create with the context's device current: resolves the
+// device address of the scratch array on that device (once per device) and builds the context's constant tables,
+// so that the call itself has nothing left to allocate.
+void hemm_static_setup(hemm_context *c) {
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lk(mu);
+    if (c->device < 0 || c->device >= HEMM_MAX_DEVICES) throw std::invalid_argument("device index out of range");
+    if (g_static_scratch[c->device] == nullptr) {
+        u64 *ptr = nullptr;
+        HEMM_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) throw std::runtime_error("hipGetSymbolAddress returned no address for the scratch array");
+        g_static_scratch[c->device] = ptr;
+    }
+    (void)g_tables_of(c);
+}
+
+void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
+                           int n_polys, hipStream_t s) {
+    if (nq < 2) throw std::invalid_argument("rescale needs at least two limbs");
+    if (n_polys < 1 || (size_t)n_polys * (size_t)nq * (size_t)c->N > HEMM_STATIC_SCRATCH_WORDS)
+        throw std::invalid_argument("n_polys * nq * N exceeds the static scratch of 2097152 words (32 limbs of N = 2^16)");
+    int dev = -1;
+    HEMM_HIP(hipGetDevice(&dev));
+    if (dev != c->device) throw std::invalid_argument("the context belongs to another device than the current one");
+    KsTables *t = nullptr;
+    {
+        KsRegistry &r = ks_registry();
+        std::lock_guard<std::mutex> lk(r.mu);
+        auto it = r.tabs.find(c);
+        if (it != r.tabs.end()) t = it->second;
+    }
+    u64 *sc = g_static_scratch[dev];
+    if (t == nullptr || sc == nullptr) throw std::runtime_error("context was not set up by hemm_context_create");
+    rescale_with(c, t, sc, in, in_stride, out, out_stride, nq, n_polys, s);
 }
 
 // ---- batched / hoisted forms ---------------------------------------------------------------------

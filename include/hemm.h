@@ -195,6 +195,20 @@ int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint6
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
                  size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
 
+
+/* hemm_rescale for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and same
+ * result as hemm_rescale, but its scratch (n_polys * nq * N words) is a fixed array inside the library's device image
+ * instead of the context's lazily allocated buffer, and the constant tables it reads were built by
+ * hemm_context_create: the call itself makes no hipMalloc / hipFree.  Limit: n_polys * nq * N <=
+ * HEMM_STATIC_SCRATCH_WORDS (16 MiB: a two-polynomial ciphertext of up to 16 limbs at N = 2^16), larger inputs are
+ * rejected with return value 1.  The array is held once per GPU until the process ends and is shared by every call
+ * on that GPU: calls that overlap on one GPU (two streams, two contexts) race.  Nothing in it has to start at zero;
+ * every word a call reads was written by that call.  The context's device must be the current one. */
+#define HEMM_STATIC_SCRATCH_WORDS (32u << 16)
+int hemm_rescale_static(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
+                        size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
