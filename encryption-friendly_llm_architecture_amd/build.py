@@ -41,7 +41,23 @@ def build(verbose=False):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB)
+    build_examples(verbose)
     return LIB
+
+
+def build_examples(verbose=False):
+    """C++ callers of the host layer, compiled as plain C++ (no HIP) and linked with libhemm.so only."""
+    ex = os.path.join(HERE, "examples")
+    for src in sorted(glob.glob(os.path.join(ex, "*.cpp"))):
+        out = os.path.splitext(src)[0]
+        cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", src, "-I", os.path.join(CSRC, "host"),
+               "-I", os.path.join(HERE, "..", "include"), "-L", HERE, "-lhemm", "-L/opt/rocm/lib",
+               "-Wl,-rpath-link,/opt/rocm/lib", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath,/opt/rocm/lib", "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("example build failed for %s:\n%s" % (src, r.stderr))
+        if verbose:
+            print("built", out)
 
 
 if __name__ == "__main__":

@@ -7,7 +7,7 @@
 #include <string>
 #include <vector>
 
-#include "modarith.cuh"
+#include "modarith.h"
 
 #define HEMM_MAX_PRIMES 64
 

@@ -127,8 +127,8 @@ public:
                              u64 *out, const u64 *scale_levels = nullptr);
     // (rows, w, level, part 0 = Z / 1 = +step / 2 = -step, level of the input's scale)
     std::map<std::tuple<int, i64, u64, int, u64>, Plaintext> pack_masks_;
-    std::map<std::tuple<u64, TileTensorShape, u64>, WeightTau> weight_tau_;
-    std::vector<std::tuple<u64, TileTensorShape, u64>> weight_tau_order_;
+    std::map<std::tuple<u64, u64, TileTensorShape, u64>, WeightTau> weight_tau_;
+    std::vector<std::tuple<u64, u64, TileTensorShape, u64>> weight_tau_order_;
 
 private:
     // (kind, shape, level, stage * 4096 + r * 4 + part) -> mask of the two-stage transforms; part 0 is an ordinary

@@ -148,7 +148,7 @@ public:
     // Hash of the residues, kept by callers that cache work per plaintext content (the weight preparation of the
     // plaintext x ciphertext product): 0 = not computed, 1 = content_hash_ is valid (every evaluator operation writes
     // a plaintext through allocate(), which resets this), 2 = never valid (see getMxData()).
-    mutable u64 content_hash_ = 0;
+    mutable u64 content_hash_ = 0, content_hash2_ = 0;   // two independent 64-bit digests: a 128-bit key
     mutable int hash_state_ = 0;
 };
 

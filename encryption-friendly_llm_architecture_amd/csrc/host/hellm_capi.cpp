@@ -417,6 +417,16 @@ int hellm_eval_chebyshev(hellm_hemmer *h, const hellm_ct *a, const double *coeff
     FACADE_CATCH
 }
 
+int hellm_linear_transform(hellm_hemmer *h, const hellm_ct *a, double left, double right, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    r->t.get() = HEaaN::Math::linearTransform(h->m->getEval(), h->m->getBtp(), a->t.get(),
+                                              HEaaN::Math::InputInterval(left, right));
+    *out = r;
+    FACADE_CATCH
+}
+
 int hellm_transpose_inplace(hellm_hemmer *h, hellm_ct *a, uint32_t T) {
     FACADE_TRY
     need(h && a, "null argument");

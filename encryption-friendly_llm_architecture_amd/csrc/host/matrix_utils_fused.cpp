@@ -1286,18 +1286,22 @@ CtxtTensor multMatMatCCReUseFused(const HomEvaluator &eval, const std::vector<Ci
 // tau(B) is prepared once per weight (decode, permute, encode on the host as MatrixTransformer::diagonalToRow<Plaintext>
 // does) and kept under a hash of the weight's residues.
 namespace {
-u64 hashResidues(const Context &c, const Plaintext &pt) {
+// two independent 64-bit digests of a plaintext's content (together a 128-bit key: an accidental collision between
+// two weights is out of reach)
+std::pair<u64, u64> hashResidues(const Context &c, const Plaintext &pt) {
     // limb 0 determines the plaintext (its coefficients are far below q_0 / 2)
     std::vector<u64> h(c->N);
     if (hipMemcpy(h.data(), pt.buf_.data(), h.size() * 8, hipMemcpyDeviceToHost) != hipSuccess)
         throw RuntimeException("hipMemcpy");
-    u64 x = 0xcbf29ce484222325ull ^ pt.getLevel();
+    u64 x = 0xcbf29ce484222325ull ^ pt.getLevel(), y = 0x9e3779b97f4a7c15ull + pt.getLevel();
     for (u64 v : h) {
         x ^= v;
         x *= 0x100000001b3ull;
         x ^= x >> 29;
+        y = (y ^ (v + 0x632be59bd9b4e019ull)) * 0xff51afd7ed558ccdull;   // another multiplier, another mixing shift
+        y ^= y >> 32;
     }
-    return x;
+    return {x, y};
 }
 }  // namespace
 
@@ -1318,17 +1322,18 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
     // ---- tau(B) over the extended basis at level T+2, scaled like a plaintext of level T+1
     // the hash needs a device-to-host copy and with it a drained queue: taken once per plaintext object
     const Plaintext &weight = op2.get();
-    u64 weight_hash;
+    std::pair<u64, u64> weight_hash;
     if (weight.hash_state_ == 1) {
-        weight_hash = weight.content_hash_;
+        weight_hash = {weight.content_hash_, weight.content_hash2_};
     } else {
         weight_hash = hashResidues(c, weight);
         if (weight.hash_state_ == 0) {
-            weight.content_hash_ = weight_hash;
+            weight.content_hash_ = weight_hash.first;
+            weight.content_hash2_ = weight_hash.second;
             weight.hash_state_ = 1;
         }
     }
-    const auto key = std::make_tuple(weight_hash, shape_b, T);
+    const auto key = std::make_tuple(weight_hash.first, weight_hash.second, shape_b, T);
     auto it = tr.weight_tau_.find(key);
     if (it == tr.weight_tau_.end()) {
         EnDecoder endec(c);

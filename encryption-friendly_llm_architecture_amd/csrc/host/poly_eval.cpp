@@ -111,113 +111,118 @@ namespace HEaaN {
 namespace Math {
 namespace {
 
-typedef std::map<u64, Ciphertext> Basis;
-
-// T_1 .. T_baby and T_{2 baby}, T_{4 baby}, ... up to `top`
-Basis chebBasis(const HomEvaluator &eval, const Ciphertext &u, u64 baby, u64 top) {
-    Basis t;
-    t.emplace(1, u);
-    Ciphertext p(eval.getContext()), r(eval.getContext());
-    for (u64 i = 2; i <= baby; i++) {
-        const u64 hi = (i + 1) / 2, lo = i / 2;
-        eval.mult(t.at(hi), t.at(lo), p);
-        eval.add(p, p, p);
-        if (hi == lo)
-            eval.add(p, Complex(-1.0, 0.0), r);
-        else
-            eval.sub(p, t.at(1), r);
-        t.emplace(i, r);
+// A block of plain Chebyshev coefficients c[0 .. 2m) (coefficient of T_j) rewritten over products of T_1, T_2, T_4,
+// ..., T_m: out[b] multiplies prod_k T_{2^k}^{bit k of b}.  One step: c_k T_k = 2 c_k T_m T_{k-m} - c_k T_{2m-k} for
+// m < k < 2m and c_m T_m = c_m T_m T_0, i.e. c = r + T_m q with q[0] = c_m, q[k-m] = 2 c_k, r[2m-k] -= c_k.
+void toBinaryProductBasis(std::vector<Real> c, Real *out) {
+    const size_t len = c.size();
+    if (len == 1) {
+        out[0] = c[0];
+        return;
     }
-    for (u64 m = baby; 2 * m <= top; m *= 2) {
-        eval.mult(t.at(m), t.at(m), p);
-        eval.add(p, p, p);
-        eval.add(p, Complex(-1.0, 0.0), r);
-        t.emplace(2 * m, r);
+    const size_t m = len / 2;
+    std::vector<Real> q(m, 0.0), r(c.begin(), c.begin() + (long)m);
+    q[0] = c[m];
+    for (size_t k = m + 1; k < len; k++) {
+        q[k - m] = 2.0 * c[k];
+        r[2 * m - k] -= c[k];
     }
-    return t;
+    toBinaryProductBasis(std::move(r), out);
+    toBinaryProductBasis(std::move(q), out + m);
 }
 
 struct Value {
     bool has_ct = false;
     Ciphertext ct;
-    bool has_const = false;
-    Real cst = 0;
+    Real cst = 0;     // the value when !has_ct
     explicit Value(const Context &c) : ct(c) {}
 };
 
-// sum_k c[k] T_k for len(c) <= baby + 1 (no ciphertext when every non-constant coefficient is zero)
-Value chebCombination(const HomEvaluator &eval, const Basis &t, const std::vector<Real> &c) {
+// sum over b in [lo, lo + len) of e[b] prod_k T_{2^k}^{bit k of (b - lo)}; pw[k] = T_{2^k}.  A node of 2^k
+// coefficients sits k levels below the input: leaves e0 + e1 T_1 take one level (the constant is multiplied at the
+// scale of the level and rescaled, however small it is), each product with T_{len/2} one more.
+Value productTree(const HomEvaluator &eval, const std::vector<Ciphertext> &pw, const Real *e, size_t len) {
     Value v(eval.getContext());
-    Ciphertext term(eval.getContext());
-    for (size_t k = 1; k < c.size(); k++) {
-        if (c[k] == 0.0) continue;
-        eval.mult(t.at(k), Complex(c[k], 0.0), term);
-        if (!v.has_ct) {
-            v.ct = term;
-            v.has_ct = true;
-        } else {
-            eval.add(v.ct, term, v.ct);
-        }
+    if (len == 1) {
+        v.cst = e[0];
+        return v;
     }
-    if (v.has_ct && c[0] != 0.0) eval.add(v.ct, Complex(c[0], 0.0), v.ct);
-    return v;
-}
-
-Value chebRecursive(const HomEvaluator &eval, const Basis &t, std::vector<Real> c, u64 baby) {
-    size_t deg = c.size() - 1;
-    while (deg > 0 && c[deg] == 0.0) deg--;
-    c.resize(deg + 1);
-    if (deg < baby) {
-        Value v = chebCombination(eval, t, c);
-        if (!v.has_ct && deg == 0) {
-            v.has_const = true;
-            v.cst = c[0];
+    if (len == 2) {
+        v.cst = e[0];
+        if (e[1] != 0.0) {
+            eval.multWithoutRescale(pw[0], Complex(e[1], 0.0), v.ct);
+            eval.rescale(v.ct);
+            if (e[0] != 0.0) eval.add(v.ct, Complex(e[0], 0.0), v.ct);
+            v.has_ct = true;
         }
         return v;
     }
-    u64 m = baby;
-    while (2 * m <= deg) m *= 2;
-    // c_k T_k = 2 c_k T_m T_{k-m} - c_k T_{2m-k} for m < k < 2m;  c_m T_m = c_m T_m T_0
-    std::vector<Real> q(deg - m + 1, 0.0), r(c.begin(), c.begin() + (long)m);
-    q[0] = c[m];
-    for (size_t k = m + 1; k <= deg; k++) {
-        q[k - m] = 2.0 * c[k];
-        r[2 * m - k] -= c[k];
+    const size_t h = len / 2;
+    size_t k = 0;
+    while (((size_t)1 << k) < h) k++;
+    Value lo = productTree(eval, pw, e, h), hi = productTree(eval, pw, e + h, h);
+    if (hi.has_ct) {
+        eval.mult(hi.ct, pw[k], v.ct);
+        v.has_ct = true;
+    } else if (hi.cst != 0.0) {
+        eval.multWithoutRescale(pw[k], Complex(hi.cst, 0.0), v.ct);
+        eval.rescale(v.ct);
+        v.has_ct = true;
     }
-    Value qv = chebRecursive(eval, t, q, baby), rv = chebRecursive(eval, t, r, baby);
-    Value out(eval.getContext());
-    if (!qv.has_ct) {
-        if (qv.has_const && qv.cst != 0.0) {
-            eval.mult(t.at(m), Complex(qv.cst, 0.0), out.ct);
-            out.has_ct = true;
-        }
-    } else {
-        eval.mult(qv.ct, t.at(m), out.ct);
-        out.has_ct = true;
-    }
-    if (!rv.has_ct) {
-        if (out.has_ct && rv.has_const && rv.cst != 0.0) eval.add(out.ct, Complex(rv.cst, 0.0), out.ct);
-        return out;
-    }
-    if (out.has_ct)
-        eval.add(out.ct, rv.ct, out.ct);
-    else
-        out = rv;
-    return out;
+    if (!v.has_ct) return lo;
+    if (lo.has_ct)
+        eval.add(v.ct, lo.ct, v.ct);
+    else if (lo.cst != 0.0)
+        eval.add(v.ct, Complex(lo.cst, 0.0), v.ct);
+    return v;
 }
 
 }  // namespace
 
+Ciphertext linearTransform(const HomEvaluator &eval, const Bootstrapper &, const Ciphertext &ctxt,
+                           const InputInterval &iv) {
+    if (!(iv.right_end > iv.left_end)) throw std::invalid_argument("[linearTransform] empty interval");
+    Ciphertext r(eval.getContext());
+    const Real mid = 0.5 * (iv.right_end + iv.left_end);
+    if (mid != 0.0)
+        eval.add(ctxt, Complex(-mid, 0.0), r);
+    else
+        r = ctxt;
+    eval.mult(r, Complex(2.0 / (iv.right_end - iv.left_end), 0.0), r);
+    return r;
+}
+
 Ciphertext evaluateChebyshevExpansion(const HomEvaluator &eval, const Bootstrapper &, const Ciphertext &ctxt,
-                                      const ChebyshevCoefficients &cc, Real multiplier) {
-    const u64 baby = cc.num_baby_step;
-    if (baby < 2 || (baby & (baby - 1)) != 0 || cc.coeffs.size() < 2)
-        throw std::invalid_argument("[evaluateChebyshevExpansion] baby steps must be a power of two >= 2, degree >= 1");
-    std::vector<Real> c(cc.coeffs);
-    if (multiplier != 1.0)
-        for (auto &x : c) x *= multiplier;
-    const Basis t = chebBasis(eval, ctxt, baby, std::max<u64>(c.size() - 1, 1));
-    Value v = chebRecursive(eval, t, c, baby);
+                                      const ChebyshevCoefficients &cc, const Real multiplier) {
+    if (cc.basis != PolynomialBasis::basic)
+        throw std::invalid_argument("[evaluateChebyshevExpansion] only the basic polynomial basis is built");
+    if (cc.coeffs.size() < 2) throw std::invalid_argument("[evaluateChebyshevExpansion] constant polynomial");
+    u64 bs = cc.num_bs, gs = cc.num_gs;
+    if (gs > 1 && (bs & (bs - 1)) != 0)
+        throw std::invalid_argument("[evaluateChebyshevExpansion] the number of baby steps must be a power of two");
+    const u64 B = (u64)1 << cc.log_bs, G = (u64)1 << cc.log_gs;
+    // every block of bs plain coefficients over products of T_1 .. T_{B/2}; block i then multiplies the product of
+    // T_{2^k bs} over the bits of i: one coefficient vector over products of T_1, T_2, T_4, ..., T_{B G / 2}
+    std::vector<Real> e(B * G, 0.0);
+    for (u64 i = 0; i < gs; i++) {
+        std::vector<Real> block(B, 0.0);
+        for (u64 j = 0; j < bs && i * bs + j < cc.coeffs.size(); j++) block[j] = multiplier * cc.coeffs[i * bs + j];
+        toBinaryProductBasis(std::move(block), e.data() + i * B);
+    }
+    size_t top = e.size();
+    while (top > 1 && e[top - 1] == 0.0) top--;
+    size_t len = 2;
+    while (len < top) len *= 2;
+    std::vector<Ciphertext> pw;      // T_1, T_2, T_4, ... as far as the tree multiplies by them
+    pw.push_back(ctxt);
+    Ciphertext p(eval.getContext());
+    for (size_t m = 2; m < len; m *= 2) {
+        eval.mult(pw.back(), pw.back(), p);
+        eval.add(p, p, p);
+        eval.add(p, Complex(-1.0, 0.0), p);
+        pw.push_back(p);
+    }
+    Value v = productTree(eval, pw, e.data(), len);
     if (!v.has_ct) throw std::invalid_argument("[evaluateChebyshevExpansion] constant polynomial");
     return v.ct;
 }

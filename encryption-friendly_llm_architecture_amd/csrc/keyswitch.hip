@@ -11,7 +11,7 @@
 #include <cstring>
 
 #include "hemm_internal.hpp"
-#include "hoisted.cuh"
+#include "hoisted.h"
 
 
 namespace {

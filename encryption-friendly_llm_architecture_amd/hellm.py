@@ -86,6 +86,7 @@ def _L():
         L.hellm_exp_iter.argtypes = [vp, vp, ctypes.c_int, pvp]
         L.hellm_eval_odd_polynomial.argtypes = [vp, vp, dp, u32, ctypes.c_int, ctypes.c_int, pvp]
         L.hellm_eval_chebyshev.argtypes = [vp, vp, dp, u32, u32, ctypes.c_double, pvp]
+        L.hellm_linear_transform.argtypes = [vp, vp, ctypes.c_double, ctypes.c_double, pvp]
         _declared = True
     return L
 
@@ -348,9 +349,15 @@ class HEMMer:
         return self._new(Ct, "hellm_eval_odd_polynomial", a.h, c, len(coeffs), k, l)
 
     def eval_chebyshev(self, a, coeffs, baby_steps, multiplier=1.0):
-        """multiplier * sum_k coeffs[k] T_k(a) for slot values in [-1, 1]"""
+        """HEaaN::Math::evaluateChebyshevExpansion on ChebyshevCoefficients{coeffs, baby_steps}: coefficients in the
+        baby-step / giant-step product basis (entry bs * i + j multiplies T_j * prod_k T_{2^k bs}^{bit k of i}), slot
+        values in [-1, 1]; baby_steps = 0: one block, i.e. a plain Chebyshev series"""
         c = (ctypes.c_double * len(coeffs))(*[float(x) for x in coeffs])
         return self._new(Ct, "hellm_eval_chebyshev", a.h, c, len(coeffs), baby_steps, float(multiplier))
+
+    def linear_transform(self, a, left, right):
+        """HEaaN::Math::linearTransform: [left, right] -> [-1, 1]"""
+        return self._new(Ct, "hellm_linear_transform", a.h, float(left), float(right))
 
     def level_down(self, a, target):
         return self._new(Ct, "hellm_level_down", a.h, target)

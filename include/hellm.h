@@ -107,13 +107,17 @@ int hellm_ct_load(hellm_hemmer *h, const char *file, hellm_ct **out);
  * exp_iter: HELLM::Exp::exp_iter (src/Exp.cpp:41-52), (1 + x / 2^k)^(2^k);
  * eval_odd_polynomial: HELLM::ReLU::evalOddPolynomial (src/ReLU.cpp:165-188), coeffs[i] = coefficient of x^i,
  *   k baby steps (power of two), l giant-step powers;
- * eval_chebyshev: HEaaN::Math::evaluateChebyshevExpansion (external/include/HEaaN-math/tools/PolynomialEvaluator.hpp:49-63),
- *   multiplier * sum_k coeffs[k] T_k(x) for slot values in [-1, 1]. */
+ * eval_chebyshev: HEaaN::Math::evaluateChebyshevExpansion (external/include/HEaaN-math/tools/PolynomialEvaluator.hpp:49-63)
+ *   on ChebyshevCoefficients{coeffs, baby_steps} (:21-40) in the header's baby-step / giant-step product basis:
+ *   multiplier * sum_i (sum_j coeffs[bs i + j] T_j(x)) * prod_k T_{2^k bs}(x)^{bit k of i} for slot values in [-1, 1]
+ *   (the layout of the tables in include/HELLM/*RemezCoeff.hpp); baby_steps = 0 means one block: a plain series;
+ * linear_transform: HEaaN::Math::linearTransform (:42-47), (2 / (right - left)) * (x - (right + left) / 2). */
 int hellm_exp_iter(hellm_hemmer *h, const hellm_ct *a, int num_iter, hellm_ct **out);
 int hellm_eval_odd_polynomial(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, int k, int l,
                               hellm_ct **out);
 int hellm_eval_chebyshev(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs,
                          uint32_t baby_steps, double multiplier, hellm_ct **out);
+int hellm_linear_transform(hellm_hemmer *h, const hellm_ct *a, double left, double right, hellm_ct **out);
 
 /* transforms and products */
 int hellm_diagonal_to_column(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out); /* MatrixTransformer :776 */

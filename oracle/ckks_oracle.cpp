@@ -90,6 +90,7 @@ struct Ctx {
     std::vector<Prime> pr;       // nQ chain primes then nP special primes
     std::vector<u64> rot_group;  // 5^j mod 2N
     std::vector<double> ksi_re, ksi_im;
+    int threads = 1;             // limbs / coefficients are independent: the loops over them may run in parallel
 };
 
 inline u64 shoup(u64 w, u64 q) { return (u64)(((u128)w << 64) / q); }
@@ -226,8 +227,10 @@ BConv make_bconv(const Ctx *c, const std::vector<int> &src, const std::vector<in
 void run_bconv(const Ctx *c, const BConv &b, const u64 *const *in, u64 *const *out) {
     const int N = c->N;
     const size_t ns = b.src.size();
-    std::vector<u64> v(ns);
+    if (ns > 64) abort();
+#pragma omp parallel for num_threads(c->threads) schedule(static)
     for (int n = 0; n < N; n++) {
+        u64 v[64];
         for (size_t i = 0; i < ns; i++) v[i] = mulmod(in[i][n], b.qhat_inv[i], c->pr[b.src[i]].q);
         for (size_t d = 0; d < b.dst.size(); d++) {
             u64 t = c->pr[b.dst[d]].q;
@@ -269,6 +272,8 @@ void *orc_create(int logN, int nQ, int nP, const u64 *primes, int dnum) {
     return c;
 }
 void orc_destroy(void *h) { delete (Ctx *)h; }
+// worker threads for the loops over independent limbs / coefficients (results do not depend on it)
+void orc_set_threads(void *h, int threads) { ((Ctx *)h)->threads = threads < 1 ? 1 : threads; }
 u64 orc_psi(void *h, int pi) { return ((Ctx *)h)->pr[pi].psi; }
 int orc_alpha(void *h) { return ((Ctx *)h)->alpha; }
 
@@ -413,6 +418,7 @@ void orc_modup(void *h, const u64 *in, int nq, u64 *out) {
     const int beta = (nq + c->alpha - 1) / c->alpha;
     std::vector<u64> coef((size_t)nq * N);
     memcpy(coef.data(), in, sizeof(u64) * (size_t)nq * N);
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (int j = 0; j < nq; j++) ntt_inv(c->pr[j], coef.data() + (size_t)j * N, N);
     for (int d = 0; d < beta; d++) {
         int lo = d * c->alpha, hi = std::min(nq, lo + c->alpha);
@@ -430,6 +436,7 @@ void orc_modup(void *h, const u64 *in, int nq, u64 *out) {
         u64 *od = out + (size_t)d * ext * N;
         for (size_t k = 0; k < dst.size(); k++) op.push_back(od + (size_t)dst_limb[k] * N);
         run_bconv(c, b, ip.data(), op.data());
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
         for (size_t k = 0; k < dst.size(); k++) ntt_fwd(c->pr[dst[k]], op[k], N);
         for (int j = lo; j < hi; j++)
             memcpy(od + (size_t)j * N, in + (size_t)j * N, sizeof(u64) * N);
@@ -440,6 +447,7 @@ void orc_inner_product(void *h, const u64 *ext, const u64 *evk, int nq, u64 *acc
     Ctx *c = (Ctx *)h;
     const int N = c->N, K = c->nP, e = nq + K, full = c->nQ + c->nP;
     const int beta = (nq + c->alpha - 1) / c->alpha;
+#pragma omp parallel for num_threads(c->threads) collapse(2) schedule(dynamic)
     for (int pol = 0; pol < 2; pol++)
         for (int j = 0; j < e; j++) {
             int pi = prime_of(c, j, nq);
@@ -463,10 +471,9 @@ void orc_moddown(void *h, const u64 *acc, int nq, u64 *out) {
     std::vector<u64> pc((size_t)K * N);
     memcpy(pc.data(), acc + (size_t)nq * N, sizeof(u64) * (size_t)K * N);
     std::vector<int> src, dst;
-    for (int k = 0; k < K; k++) {
-        ntt_inv(c->pr[c->nQ + k], pc.data() + (size_t)k * N, N);
-        src.push_back(c->nQ + k);
-    }
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
+    for (int k = 0; k < K; k++) ntt_inv(c->pr[c->nQ + k], pc.data() + (size_t)k * N, N);
+    for (int k = 0; k < K; k++) src.push_back(c->nQ + k);
     for (int j = 0; j < nq; j++) dst.push_back(j);
     BConv b = make_bconv(c, src, dst);
     std::vector<const u64 *> ip;
@@ -474,6 +481,7 @@ void orc_moddown(void *h, const u64 *acc, int nq, u64 *out) {
     for (int k = 0; k < K; k++) ip.push_back(pc.data() + (size_t)k * N);
     for (int j = 0; j < nq; j++) op.push_back(out + (size_t)j * N);
     run_bconv(c, b, ip.data(), op.data());
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (int j = 0; j < nq; j++) {
         const u64 q = c->pr[j].q;
         ntt_fwd(c->pr[j], op[j], N);
@@ -504,6 +512,7 @@ void orc_rescale(void *h, const u64 *in, int nq, u64 *out) {
     memcpy(lc.data(), in + (size_t)last * N, sizeof(u64) * N);
     ntt_inv(c->pr[last], lc.data(), N);
     const u64 ql = c->pr[last].q;
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic) firstprivate(t)
     for (int j = 0; j < last; j++) {
         const u64 q = c->pr[j].q;
         for (int n = 0; n < N; n++) t[n] = lc[n] % q;
@@ -519,6 +528,7 @@ void orc_rescale(void *h, const u64 *in, int nq, u64 *out) {
 void orc_tensor(void *h, const u64 *ct1, const u64 *ct2, int nq, u64 *out) {
     Ctx *c = (Ctx *)h;
     const int N = c->N;
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (int j = 0; j < nq; j++) {
         const u64 q = c->pr[j].q;
         const u64 *b1 = ct1 + (size_t)j * N, *a1 = ct1 + ((size_t)nq + j) * N;
@@ -548,6 +558,7 @@ void orc_hoisted_term(void *h, const u64 *ext, const u64 *b, const u64 *evk, con
         u64 e = (2 * (u64)bitrev((unsigned)k, c->logN) + 1) * g % M;
         perm[k] = (int)bitrev((unsigned)((e - 1) / 2), c->logN);
     }
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (int j = 0; j < E; j++) {
         const int pi = prime_of(c, j, nq);
         const u64 q = c->pr[pi].q;
@@ -585,17 +596,19 @@ void orc_moddown_drop(void *h, const u64 *y, int nq, int drop_last, u64 *out) {
     std::vector<u64> dc(src.size() * (size_t)N);
     std::vector<const u64 *> ip;
     std::vector<u64 *> op;
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (size_t i = 0; i < src.size(); i++) {
         memcpy(dc.data() + i * N, y + (size_t)slot[i] * N, sizeof(u64) * N);
         ntt_inv(c->pr[src[i]], dc.data() + i * N, N);
-        ip.push_back(dc.data() + i * N);
     }
+    for (size_t i = 0; i < src.size(); i++) ip.push_back(dc.data() + i * N);
     for (int j = 0; j < nq_out; j++) {
         dst.push_back(j);
         op.push_back(out + (size_t)j * N);
     }
     BConv bc = make_bconv(c, src, dst);
     run_bconv(c, bc, ip.data(), op.data());
+#pragma omp parallel for num_threads(c->threads) schedule(dynamic)
     for (int j = 0; j < nq_out; j++) {
         const u64 q = c->pr[j].q;
         ntt_fwd(c->pr[j], op[j], N);

@@ -103,6 +103,11 @@ class SlotSim:
         assert x.rc == 0 and x.level >= 1
         return SimCt(x.z * c, x.level - 1, 0)
 
+    def mult_const_rescale(self, x, c):
+        """multWithoutRescale(ct, constant) + rescale: always one level, however small or integral the constant."""
+        assert x.rc == 0 and x.level >= 1
+        return SimCt(x.z * c, x.level - 1, 0)
+
     def add_const(self, x, c):
         return SimCt(x.z + c, x.level, x.rc)
 
@@ -203,6 +208,13 @@ class OracleEval:
         r = math.floor(c + 0.5)
         if abs(c - r) <= 1e-8:
             return self.o.mult_integer(x, int(r))
+        d = c * self.o.delta[x.level]
+        v = int(math.floor(abs(d) + 0.5)) * (1 if d >= 0 else -1)      # llround: halves away from zero
+        return self.o.rescale(Ct(self.o.mult_scalar_residues(x, v), x.scale * self.o.delta[x.level]))
+
+    def mult_const_rescale(self, x, c):
+        """multWithoutRescale(ct, real constant) + rescale: round(c * Delta_level) on the residues, one level."""
+        from .oracle import Ct
         d = c * self.o.delta[x.level]
         v = int(math.floor(abs(d) + 0.5)) * (1 if d >= 0 else -1)      # llround: halves away from zero
         return self.o.rescale(Ct(self.o.mult_scalar_residues(x, v), x.scale * self.o.delta[x.level]))
@@ -544,6 +556,55 @@ def mult_mat_mat_reuse(ev, tmp, b_pt, T, step=None):
         t = ev.mult_plain_no_rescale(c, ev.left_rotate(b_pt, k * step))
         acc = t if acc is None else ev.add(acc, t)
     return ev.rescale(acc)
+
+
+def mult_mat_mat_pre_rev(ev, b, T, n, w, kind=V):
+    """multMatMatPreRev (:1641-1649) / multPackedMatMatPreRev (:1266-1274, kind=PV): tau(B) after a levelDown to
+    T+2; multPackedMatMatPre (:1218-1227) is the same at T+3 with kind=PH (pass T+1)."""
+    return diagonal_transform(ev, ev.level_down(b, T + 2), kind, n, w)
+
+
+def mult_mat_mat_cc_reuse(ev, tmp, b, step, rescale_after=False):
+    """multMatMatCCReUse (:1651-1679; step = block width, no rescale) / multPackedMatMatCCReuse (:1276-1305;
+    step = 2 * block width, rescale after the relinearisation): sum_k tmp[k] (x) leftRotate^k(tau B, step), the
+    rotations chained one after the other."""
+    acc = ev.tensor(tmp[0], b)
+    for k in range(1, len(tmp)):
+        b = ev.left_rotate(b, step)
+        acc = ev.add(acc, ev.tensor(tmp[k], b))
+    out = ev.relinearize(acc)
+    return ev.rescale(out) if rescale_after else out
+
+
+def mult_packed_mat_mat_pre_rot(ev, a, T, n, w):
+    """multPackedMatMatPreRot (:1229-1264): the n/2 shifts by two columns of packed sigma(A), at level T+1."""
+    cm = [ev.encode(m, T + 2) for m in col_masks(n, ev.slots)]
+    tmp = [ev.level_down_one(a)]
+    a = ev.left_rotate(a, 2)
+    a_wrap = ev.right_rotate(a, n)
+    for i in range(1, n // 2):
+        if i > 1:
+            a = ev.left_rotate(a, 2)
+            a_wrap = ev.left_rotate(a_wrap, 2)
+        tmp.append(ev.rescale(ev.masked_sum(a, cm[4 * i + 1], a_wrap, cm[4 * i])))
+    return tmp
+
+
+def transpose_complex_packing(ev, t, n, w, target_level=0, fused_orc=None):
+    """HEMMer::transposeComplexPackingInplace (HEMMer.cpp:779-799): columns (2c, 2c+1) -> a - i b in both, an
+    optional levelDown to target_level + 1, then the transpose (reference order, or the batched transform over
+    `fused_orc` as the default schedule runs it)."""
+    even = (np.arange(ev.slots) % 2 == 0).astype(np.complex128)
+    m = ev.encode(even, ev.level_of(t))
+    e = ev.mult_pt(t, m)
+    o = ev.mult_pt(ev.negate(ev.mult_imag_unit(ev.left_rotate(t, 1))), m)
+    fus = ev.add(o, e)
+    out = ev.add(ev.right_rotate(fus, 1), fus)
+    if target_level > 0:
+        out = ev.level_down(out, 1 + target_level)
+    if fused_orc is not None:
+        return diagonal_transform_fused(fused_orc, out, DIAG_SIGNED, n, w)
+    return transpose(ev, out, n, w)
 
 
 # --------------------------------------------------------------------------------------------

@@ -48,6 +48,7 @@ def lib():
         L.orc_psi.restype = ctypes.c_uint64
         L.orc_psi.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.orc_alpha.argtypes = [ctypes.c_void_p]
+        L.orc_set_threads.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.orc_sm64.restype = ctypes.c_uint64
         L.orc_sm64.argtypes = [ctypes.c_uint64]
         L.orc_stream_key.restype = ctypes.c_uint64
@@ -220,6 +221,7 @@ class Oracle:
         self.h = self.L.orc_create(log_n, self.nQ, self.nP, arr, dnum)
         self.alpha = self.L.orc_alpha(self.h)
         self.threads = threads
+        self.L.orc_set_threads(self.h, threads)
         # fixed per-level scale: Delta_L = 2^log_scale, Delta_{l-1} = Delta_l^2 / q_l
         self.delta = [0.0] * self.nQ
         self.delta[self.nQ - 1] = float(1 << log_scale)
@@ -297,18 +299,20 @@ class Oracle:
         P = 1
         for p in self.p:
             P *= p
-        tmp = np.empty(self.N, dtype=np.uint64)
+        def limb(d, i, e_i):
+            tmp = np.empty(self.N, dtype=np.uint64)
+            a = self.uniform(self.stream(seed, TAG_EVK_A, key_id, d * tot + i), i)
+            evk[d, 1, i] = a
+            self.L.orc_pointwise(self.h, 2, _p(a), _p(self.sk[i]), _p(tmp), i)   # a*s
+            self.L.orc_pointwise(self.h, 1, _p(e_i), _p(tmp), _p(evk[d, 0, i]), i)  # e - a*s
+            if i < self.nQ and d * self.alpha <= i < (d + 1) * self.alpha:
+                self.L.orc_mul_scalar(self.h, _p(s_from[i]), P % self.mods[i], _p(tmp), i)
+                self.L.orc_pointwise(self.h, 0, _p(evk[d, 0, i]), _p(tmp), _p(evk[d, 0, i]), i)
+
         for d in range(self.dnum):
             e = self.small_to_ntt(self.error(self.stream(seed, TAG_EVK_E, key_id, d)),
                                   list(range(tot)))
-            for i in range(tot):
-                a = self.uniform(self.stream(seed, TAG_EVK_A, key_id, d * tot + i), i)
-                evk[d, 1, i] = a
-                self.L.orc_pointwise(self.h, 2, _p(a), _p(self.sk[i]), _p(tmp), i)   # a*s
-                self.L.orc_pointwise(self.h, 1, _p(e[i]), _p(tmp), _p(evk[d, 0, i]), i)  # e - a*s
-                if i < self.nQ and d * self.alpha <= i < (d + 1) * self.alpha:
-                    self.L.orc_mul_scalar(self.h, _p(s_from[i]), P % self.mods[i], _p(tmp), i)
-                    self.L.orc_pointwise(self.h, 0, _p(evk[d, 0, i]), _p(tmp), _p(evk[d, 0, i]), i)
+            self._for_each(lambda i: limb(d, i, e[i]), range(tot))
         return evk
 
     def gen_mult_key(self, seed):
@@ -318,10 +322,21 @@ class Oracle:
             self.L.orc_pointwise(self.h, 2, _p(self.sk[i]), _p(self.sk[i]), _p(s2[i]), i)
         self.keys["mult"] = self._gen_switch_key(seed, 0, s2)
 
+    def _for_each(self, fn, items):
+        """fn over independent items (limbs), on self.threads worker threads (ctypes calls release the GIL)."""
+        items = list(items)
+        if self.threads <= 1 or len(items) <= 1:
+            for it in items:
+                fn(it)
+            return
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=min(self.threads, len(items))) as ex:
+            list(ex.map(fn, items))
+
     def _sk_automorphism(self, g):
         out = np.empty_like(self.sk)
-        for i in range(self.nQ + self.nP):
-            self.L.orc_automorphism_ntt(self.h, _p(self.sk[i]), _p(out[i]), g)
+        self._for_each(lambda i: self.L.orc_automorphism_ntt(self.h, _p(self.sk[i]), _p(out[i]), g),
+                       range(self.nQ + self.nP))
         return out
 
     def gen_rot_key(self, seed, r):

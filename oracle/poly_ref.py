@@ -4,11 +4,14 @@
   * eval_odd_polynomial  reference ciphertext/src/ReLU.cpp:53-188 (Han-Ki baby-step / giant-step for odd
                          polynomials given by monomial coefficients; products stay un-relinearised until
                          a giant-step multiplication needs them)
-  * eval_chebyshev       HEaaN::Math::evaluateChebyshevExpansion is closed (PolynomialEvaluator.hpp:49-63
-                         is only a declaration); this is the textbook baby-step / giant-step evaluation in
-                         the Chebyshev basis, stated here and mirrored operation by operation by the product.
-                         Parity with HEaaN's own residues is unpinned; what is pinned is the value
-                         (numpy.polynomial.chebyshev.chebval) and GPU == this restatement.
+  * eval_chebyshev       HEaaN::Math::evaluateChebyshevExpansion is closed (PolynomialEvaluator.hpp:49-63 is
+                         only a declaration).  Its coefficient convention -- the baby-step / giant-step product
+                         basis the header comment spells out -- is followed; the order of operations is this
+                         build's and is mirrored operation by operation by the product.  Pins: the reference's
+                         own EXP_15_4 table (include/HELLM/LossRemezCoeff.hpp:18-35) evaluates to exp on
+                         [-2, 2] (src/Loss.cpp:41-56) to 1e-10; plain Chebyshev series converted to the product
+                         basis agree with numpy's chebval; GPU == this restatement.  Parity with HEaaN's own
+                         residues is unpinned.
 
 Every function takes an evaluator `ev` with mult / tensor / rescale / relinearize / add / sub / mult_const /
 add_const / level_of (hemmer_ref.SlotSim for exact slot arithmetic, hemmer_ref.OracleEval for the CKKS oracle).
@@ -73,75 +76,125 @@ def eval_odd_polynomial(ev, x, poly, k, l):
     return ev.relinearize(_odd_giant_step(ev, odd, giant, list(poly), k, l))
 
 
-# ---- Chebyshev basis -------------------------------------------------------------------------------
-def _cheb_basis(ev, u, baby, top):
-    """T_1 .. T_baby and T_{2 baby}, T_{4 baby}, ... up to `top`, from T_2m = 2 T_m^2 - 1 and
-    T_{m+n} = 2 T_m T_n - T_{m-n}."""
-    t = {1: u}
-    for i in range(2, baby + 1):
-        hi, lo = (i + 1) // 2, i // 2
-        p = ev.mult(t[hi], t[lo])
-        p = ev.add(p, p)
-        t[i] = ev.add_const(p, -1.0) if hi == lo else ev.sub(p, t[1])
-    m = baby
-    while 2 * m <= top:
-        p = ev.mult(t[m], t[m])
-        t[2 * m] = ev.add_const(ev.add(p, p), -1.0)
-        m *= 2
-    return t
+# ---- Chebyshev expansions in the baby-step / giant-step product basis ---------------------------------
+def cheb_product_value(d, bs, t):
+    """Value of the expansion the reference's tables hold (PolynomialEvaluator.hpp:49-58), straight from its
+    definition: sum_i (sum_j d[bs i + j] T_j(t)) * prod_k T_{2^k bs}(t)^{bit k of i}.  numpy, for the tests."""
+    import numpy as np
+    from numpy.polynomial import chebyshev as C
+    t = np.asarray(t, dtype=np.float64)
+    d = [float(x) for x in d]
+    bs = bs if bs > 0 else len(d)
+    gs = -(-len(d) // bs)
+    total = np.zeros_like(t)
+    for i in range(gs):
+        block = d[bs * i: bs * (i + 1)]
+        term = C.chebval(t, block)
+        k = 0
+        while (i >> k) != 0:
+            if (i >> k) & 1:
+                term = term * C.chebval(t, [0.0] * ((1 << k) * bs) + [1.0])
+            k += 1
+        total = total + term
+    return total
 
 
-def _cheb_combination(ev, t, c):
-    """sum_k c[k] T_k for len(c) <= baby + 1, None when every coefficient is zero."""
-    r = None
-    for k in range(1, len(c)):
-        if c[k] == 0.0:
-            continue
-        term = ev.mult_const(t[k], c[k])
-        r = term if r is None else ev.add(r, term)
-    if r is None:
-        return None
-    return ev.add_const(r, c[0]) if c[0] != 0.0 else r
+def cheb_plain_to_product(c, bs):
+    """Plain Chebyshev series c (coefficient of T_k) -> the product basis with bs baby steps (bs a power of two):
+    c_k T_k = 2 c_k T_m T_{k-m} - c_k T_{2m-k} for m < k < 2m, applied from the top giant step down to m = bs."""
+    c = [float(x) for x in c]
+    size = bs
+    while size < len(c):
+        size *= 2
+    c = c + [0.0] * (size - len(c))
+
+    def split(c):
+        if len(c) <= bs:
+            return c
+        m = len(c) // 2
+        q, r = [0.0] * m, c[:m]
+        q[0] = c[m]
+        for k in range(m + 1, len(c)):
+            q[k - m] = 2.0 * c[k]
+            r[2 * m - k] -= c[k]
+        return split(r) + split(q)
+
+    return split(c)
 
 
-def _cheb_recursive(ev, t, c, baby):
-    deg = len(c) - 1
-    while deg > 0 and c[deg] == 0.0:
-        deg -= 1
-    c = c[: deg + 1]
-    if deg < baby:
-        return _cheb_combination(ev, t, c), (c[0] if deg == 0 else None)
-    m = baby
-    while 2 * m <= deg:
-        m *= 2
-    # c_k T_k = 2 c_k T_m T_{k-m} - c_k T_{2m-k}  for m < k < 2m;  c_m T_m = c_m T_m T_0
-    q = [0.0] * (deg - m + 1)
-    r = list(c[:m])
+def _to_binary_product_basis(c):
+    """c[0 .. 2m) plain -> coefficients over products of T_1, T_2, T_4, ..., T_m (bit k of the index <-> T_{2^k})."""
+    if len(c) == 1:
+        return [c[0]]
+    m = len(c) // 2
+    q, r = [0.0] * m, list(c[:m])
     q[0] = c[m]
-    for k in range(m + 1, deg + 1):
+    for k in range(m + 1, len(c)):
         q[k - m] = 2.0 * c[k]
         r[2 * m - k] -= c[k]
-    qv, qconst = _cheb_recursive(ev, t, q, baby)
-    rv, rconst = _cheb_recursive(ev, t, r, baby)
-    # q(u) * T_m: a constant q multiplies T_m by a scalar
-    if qv is None:
-        prod = ev.mult_const(t[m], qconst) if qconst not in (None, 0.0) else None
+    return _to_binary_product_basis(r) + _to_binary_product_basis(q)
+
+
+def _product_tree(ev, pw, e):
+    """(ciphertext or None, constant): sum_b e[b] prod_k T_{2^k}^{bit k of b}, pw[k] = T_{2^k}."""
+    if len(e) == 1:
+        return None, e[0]
+    if len(e) == 2:
+        if e[1] == 0.0:
+            return None, e[0]
+        v = ev.mult_const_rescale(pw[0], e[1])
+        return (ev.add_const(v, e[0]) if e[0] != 0.0 else v), e[0]
+    h = len(e) // 2
+    k = h.bit_length() - 1
+    lo, lo_c = _product_tree(ev, pw, e[:h])
+    hi, hi_c = _product_tree(ev, pw, e[h:])
+    if hi is not None:
+        v = ev.mult(hi, pw[k])
+    elif hi_c != 0.0:
+        v = ev.mult_const_rescale(pw[k], hi_c)
     else:
-        prod = ev.mult(qv, t[m])
-    if rv is None:
-        out = prod
-        if rconst not in (None, 0.0):
-            out = ev.add_const(out, rconst)
-        return out, None
-    return (ev.add(prod, rv) if prod is not None else rv), None
+        return lo, lo_c
+    if lo is not None:
+        return ev.add(v, lo), 0.0
+    return (ev.add_const(v, lo_c) if lo_c != 0.0 else v), 0.0
 
 
-def eval_chebyshev(ev, u, coeffs, baby):
-    """sum_k coeffs[k] T_k(u) for u with values in [-1, 1]; baby = number of baby steps (power of two)."""
-    coeffs = [float(x) for x in coeffs]
-    deg = len(coeffs) - 1
-    t = _cheb_basis(ev, u, baby, max(deg, 1))
-    v, const = _cheb_recursive(ev, t, coeffs, baby)
+def linear_transform(ev, x, left, right):
+    """HEaaN::Math::linearTransform (PolynomialEvaluator.hpp:42-47): (2 / (right - left)) (x - (right + left) / 2)."""
+    mid = 0.5 * (right + left)
+    r = ev.add_const(x, -mid) if mid != 0.0 else x
+    return ev.mult_const(r, 2.0 / (right - left))
+
+
+def eval_chebyshev(ev, u, coeffs, baby, multiplier=1.0):
+    """HEaaN::Math::evaluateChebyshevExpansion on ChebyshevCoefficients{coeffs, baby} (PolynomialEvaluator.hpp:
+    19-63): multiplier * sum_i (sum_j coeffs[bs i + j] T_j(u)) prod_k T_{2^k bs}(u)^{bit k of i}, u in [-1, 1].
+    The blocks are rewritten over products of T_1, T_2, T_4, ... so that constants only multiply T_1; the tree then
+    uses ceil(log2 bs) + ceil(log2 gs) levels, the header's level_cost."""
+    d = [float(x) for x in coeffs]
+    bs = baby if baby > 0 else len(d)
+    gs = -(-len(d) // bs)
+    if gs > 1 and bs & (bs - 1):
+        raise ValueError("the number of baby steps must be a power of two")
+    B = 1 << max(0, (bs - 1).bit_length())
+    G = 1 << max(0, (gs - 1).bit_length())
+    e = []
+    for i in range(G):
+        block = [multiplier * x for x in d[bs * i: bs * (i + 1)]] if i < gs else []
+        e += _to_binary_product_basis(block + [0.0] * (B - len(block)))
+    top = len(e)
+    while top > 1 and e[top - 1] == 0.0:
+        top -= 1
+    size = 2
+    while size < top:
+        size *= 2
+    pw = [u]
+    m = 2
+    while m < size:
+        p = ev.mult(pw[-1], pw[-1])
+        pw.append(ev.add_const(ev.add(p, p), -1.0))
+        m *= 2
+    v, _ = _product_tree(ev, pw, e[:size])
     if v is None:
         raise ValueError("constant polynomial")
     return v

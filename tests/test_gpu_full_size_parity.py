@@ -1,0 +1,257 @@
+"""Bit-exact GPU-vs-oracle checks at the full ring (N = 2^16) and at the shapes the benchmark times:
+
+* the hoisted sum of the CCMM main loop at its benchmark shape (32 outputs, two masked sources under one key,
+  7 + 4 limbs, 2 digits, run-table masks), which is large enough to be launched as two kernels (double-precision
+  limbs / integer limbs), through the kernel-argument path and the staged-list path, and with every operand at q - 1;
+* masked sums at N = 2^16 through both paths and for 1, 2 and 3 polynomials;
+* one whole 128 x 128 singleCCMatMul on the preset, residue for residue against the oracle running the same
+  schedule (keys derived from the same seed on both sides);
+* one key-switched rotation per step of the set {1, 2, 4, ..., 64} and multiples of 128, ciphertext at level 20 of a
+  chain of 24 60-bit primes + 4 special primes, dnum 3, with the ModUp / inner product / ModDown stages at that shape."""
+import os
+
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle import hemmer_ref as R
+from oracle import oracle as O
+from oracle.oracle import _p
+
+pytestmark = pytest.mark.gpu
+THREADS = max(1, min(16, os.cpu_count() or 1))
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int64)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy().view(np.uint64)
+
+
+def rand_limbs(rng, mods, shape_prefix, N):
+    out = np.empty(tuple(shape_prefix) + (len(mods), N), dtype=np.uint64)
+    for j, q in enumerate(mods):
+        out[..., j, :] = rng.integers(0, q, tuple(shape_prefix) + (N,), dtype=np.uint64)
+    return out
+
+
+class Bench:
+    """Preset-sized context (13 + 4 primes, dnum 3) with random sources, keys and column masks at nq = 7."""
+
+    def __init__(self):
+        pkg = load_package()
+        self.log_n, self.N, self.nq = 16, 1 << 16, 7
+        qs, ps = O.ckks_chain(16, 13, 4)
+        self.orc = O.Oracle(16, qs, ps, 3, threads=THREADS)
+        self.ctx = pkg.Context(16, qs, ps, 3)
+        orc, nq, N = self.orc, self.nq, self.N
+        self.beta = (nq + orc.alpha - 1) // orc.alpha
+        assert self.beta == 2 and orc.nP == 4
+        self.ext_mods = [orc.mods[i] for i in orc.ext_primes(nq - 1)]
+        rng = np.random.default_rng(2024)
+        self.ext = [np.ascontiguousarray(rand_limbs(rng, self.ext_mods, (self.beta,), N)) for _ in range(4)]
+        self.b = [rand_limbs(rng, orc.q[:nq], (), N) for _ in range(4)]
+        self.evk = [np.ascontiguousarray(rand_limbs(rng, orc.mods, (orc.dnum, 2), N)) for _ in range(4)]
+        self.gal = [orc.galois(r) for r in (1, 37, orc.slots - 128, 2048)]
+        col = np.arange(orc.slots) % 128
+        self.shift = self.log_n - 8
+        self.masks = []
+        for k in (1, 37, 64, 127):
+            main = orc.encode_ext((col < 128 - k).astype(float), nq - 1)
+            wrap = orc.encode_ext((col >= 128 - k).astype(float), nq - 1)
+            self.masks.append((main, wrap))
+        self.d_ext = [dev(x) for x in self.ext]
+        self.d_b = [dev(x) for x in self.b]
+        self.d_evk = [dev(x) for x in self.evk]
+        self.d_full = [(dev(m.data), dev(w.data)) for m, w in self.masks]
+        self.d_tab = [(self.ctx.compact_mask(m, self.shift), self.ctx.compact_mask(w, self.shift)) for m, w in self.d_full]
+        assert all(t is not None for pair in self.d_tab for t in pair)
+
+    def want(self, spec):
+        """spec: tuple of (source, key, mask pair, half) -> y[2][E][N] on the oracle."""
+        orc = self.orc
+        y = np.zeros((2, self.nq + orc.nP, self.N), dtype=np.uint64)
+        for i, (s, k, m, half) in enumerate(spec):
+            orc.L.orc_hoisted_term(orc.h, _p(self.ext[s]), _p(self.b[s]), _p(self.evk[k]), _p(self.masks[m][half].data),
+                                   self.gal[k], self.nq, _p(y), int(i > 0))
+        return y
+
+    def term(self, s, k, m, half, table=True):
+        mask = self.d_tab[m][half] if table else self.d_full[m][half]
+        return (self.d_ext[s], self.d_b[s], self.d_evk[k], mask, self.gal[k], self.shift if table else 0)
+
+
+@pytest.fixture(scope="module")
+def bench():
+    return Bench()
+
+
+def check_outputs(bench, specs, y):
+    cache = {}
+    for o, spec in enumerate(specs):
+        if spec not in cache:
+            cache[spec] = bench.want(spec)
+        assert np.array_equal(y[o], cache[spec]), (o, spec)
+
+
+def test_hoisted_sum_at_the_main_loop_shape_two_launches(bench):
+    """32 outputs x (main, wrap) halves of one shift under one key: one merged two-source term per output, list and
+    outputs within the kernel-argument capacity, 32 * 11 * 128 = 45056 workgroups -> one launch for the
+    double-precision limbs and one for the integer limbs."""
+    specs = []
+    for o in range(32):
+        k, m = o % 4, (o // 4) % 4
+        s0, s1 = (o // 2) % 4, (o // 2 + 1 + o % 3) % 4
+        specs.append(((s0, k, m, 0), (s1, k, m, 1)))
+    groups = [[bench.term(*t) for t in spec] for spec in specs]
+    y = host(bench.ctx.hoisted_terms(groups, bench.nq))
+    check_outputs(bench, specs, y)
+
+
+def test_hoisted_sum_staged_term_list_two_launches(bench):
+    """The same size with two shifts per output (64 merged terms: beyond the kernel-argument capacity, so the term
+    list is staged in device memory), full masks beside run tables, and a third, single term on some outputs."""
+    specs = []
+    for o in range(32):
+        k, m = o % 4, (o // 4) % 4
+        k2, m2 = (k + 1) % 4, (m + 2) % 4
+        s0, s1 = (o // 2) % 4, (o // 2 + 1) % 4
+        spec = [(s0, k, m, 0), (s1, k, m, 1), (s1, k2, m2, 0), (s0, k2, m2, 1)]
+        if o % 5 == 0:
+            spec.append((o % 4, (k + 2) % 4, m, 1))
+        specs.append(tuple(spec))
+    # the two halves of a shift use the same kind of mask (run table or full), so that they merge under their key
+    groups = [[bench.term(*t, table=((i // 2) + o) % 3 != 0) for i, t in enumerate(spec)] for o, spec in enumerate(specs)]
+    y = host(bench.ctx.hoisted_terms(groups, bench.nq))
+    check_outputs(bench, specs, y)
+
+
+def test_hoisted_sum_two_launches_every_operand_at_q_minus_one(bench):
+    """Largest sums the reductions of both launches see: sources, b, key and masks all q - 1, at the split size."""
+    orc, ctx, N, nq = bench.orc, bench.ctx, bench.N, bench.nq
+    top = lambda primes, prefix: np.ascontiguousarray(
+        np.stack([np.full(tuple(prefix) + (N,), q - 1, dtype=np.uint64) for q in primes], axis=len(prefix)))
+    ext, b = top(bench.ext_mods, (bench.beta,)), top(orc.q[:nq], ())
+    evk, mask = top(orc.mods, (orc.dnum, 2)), top(bench.ext_mods, ())
+    dext, db, dk, dm = dev(ext), dev(b), dev(evk), dev(mask)
+    tm = ctx.compact_mask(dm, bench.shift)
+    assert tm is not None
+    g1, g2 = bench.gal[1], bench.gal[2]
+    kinds = [[(dext, db, dk, tm, g1, bench.shift), (dext, db, dk, tm, g1, bench.shift)],      # merged, run tables
+             [(dext, db, dk, dm, g2), (dext, db, dk, dm, g2)],                                # merged, full masks
+             [(dext, db, dk, dm, g1), (dext, db, dk, None, g2)]]                              # single terms
+    groups = [kinds[o % 3] for o in range(32)]
+    y = host(ctx.hoisted_terms(groups, nq))
+    want = []
+    for terms in ([(mask, g1), (mask, g1)], [(mask, g2), (mask, g2)], [(mask, g1), (None, g2)]):
+        w = np.zeros((2, nq + orc.nP, N), dtype=np.uint64)
+        for i, (mk, g) in enumerate(terms):
+            orc.L.orc_hoisted_term(orc.h, _p(ext), _p(b), _p(evk), _p(mk) if mk is not None else None, g, nq, _p(w),
+                                   int(i > 0))
+        want.append(w)
+    for o in range(32):
+        assert np.array_equal(y[o], want[o % 3]), o
+
+
+@pytest.mark.parametrize("n_polys", [1, 2, 3])
+def test_masked_sums_full_ring_both_paths(bench, n_polys):
+    """out[o] = sum_t mask_t * ct_t over nq limbs at N = 2^16: a short list (kernel arguments) and a long one (staged),
+    with unmasked terms and a mask read through an automorphism."""
+    orc, ctx, N, nq = bench.orc, bench.ctx, bench.N, bench.nq
+    rng = np.random.default_rng(5 + n_polys)
+    mods = orc.q[:nq]
+    cts = [rand_limbs(rng, mods, (n_polys,), N) for _ in range(3)]
+    dcts = [dev(c) for c in cts]
+    pts = [orc.encode(rng.uniform(-1, 1, orc.slots), nq - 1) for _ in range(3)]
+    dpts = [dev(p.data) for p in pts]
+    g = orc.galois(5)
+
+    def one(spec):
+        acc = None
+        for (ci, pi, gal) in spec:
+            x = O.Ct(cts[ci], 1.0)
+            if pi is not None:
+                p = pts[pi] if not gal else orc.left_rotate(pts[pi], 5)
+                x = orc.mult_plain_no_rescale(x, p)
+            acc = x if acc is None else orc.add(acc, x)
+        return acc.data
+
+    short = [((0, 0, 0), (1, None, 0)), ((2, 1, 1),), ((1, 2, 0), (2, 0, 0), (0, 1, 1))]
+    long_ = [tuple(((o + t) % 3, (o + 2 * t) % 3 if (o + t) % 4 else None, (t % 5 == 1) and (o + t) % 4 != 0)
+                   for t in range(5)) for o in range(8)]
+    for specs in (short, long_):
+        groups = [[(dcts[ci], dpts[pi] if pi is not None else None, g if gal else 0) for (ci, pi, gal) in spec]
+                  for spec in specs]
+        got = host(ctx.masked_sum_batch(groups, nq, n_polys))
+        for o, spec in enumerate(specs):
+            assert np.array_equal(got[o], one(spec)), (o, spec)
+
+
+def test_preset_ccmm_residues_bit_exact():
+    """singleCCMatMul of two fresh 128 x 128 tiles on the preset (N = 2^16, 13 + 4 primes, dnum 3, target level 4):
+    every residue of the result equals the oracle's, which runs the same schedule with keys from the same seed."""
+    load_package()
+    from efla_amd import hellm
+    H = hellm.HEMMer(preset=True, seed=3)
+    qs, ps = O.ckks_chain(16, 13, 4)
+    orc = O.Oracle(16, qs, ps, dnum=3, threads=THREADS)
+    orc.gen_secret(3)
+    orc.gen_mult_key(3)
+    orc.gen_conj_key(3)
+    orc.key_seed = 3
+    assert np.array_equal(H.secret_coeffs(), orc.sk_coeffs)
+    rng = np.random.default_rng(1)
+    A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    c = H.single_cc_matmul(ca, cb, 4)
+    top = orc.delta[orc.nQ - 1]
+    want = R.mult_mat_mat_cc_packed_single(orc, O.Ct(ca.residues(), top), O.Ct(cb.residues(), top), 4, 128, 128)
+    assert c.info()["level"] == 4 == want.level
+    assert np.array_equal(c.residues(), want.data)
+    assert np.abs(H.decrypt(c) - A @ B).max() < 2.0 ** -12
+
+
+@pytest.fixture(scope="module")
+def chain24():
+    pkg = load_package()
+    primes = pkg.primes_below(60, 16, 28)
+    qs, ps = primes[:24], primes[24:]
+    orc = O.Oracle(16, qs, ps, 3, threads=THREADS)
+    ctx = pkg.Context(16, qs, ps, 3)
+    orc.gen_secret(3)
+    rng = np.random.default_rng(20)
+    ct = rand_limbs(rng, qs[:21], (2,), 1 << 16)
+    return orc, ctx, ct, dev(ct)
+
+
+def test_rotation_stages_at_level_20_of_24(chain24):
+    """ModUp, key inner product and ModDown one at a time at 21 active limbs + 4 special primes (3 digits of 8)."""
+    orc, ctx, ct, dct = chain24
+    nq, N = 21, 1 << 16
+    E = nq + orc.nP
+    orc.gen_rot_key(6, 1)
+    evk = orc.keys[("gal", orc.galois(1))]
+    ext = orc.modup(ct[1])
+    dext = ctx.modup(dct[1].contiguous(), nq)
+    assert np.array_equal(host(dext), ext)
+    acc = np.empty((2, E, N), dtype=np.uint64)
+    orc.L.orc_inner_product(orc.h, _p(ext), _p(evk), nq, _p(acc))
+    dacc = ctx.inner_product(dext, dev(evk), nq)
+    assert np.array_equal(host(dacc), acc)
+    want = np.empty((2, nq, N), dtype=np.uint64)
+    for p in range(2):
+        orc.L.orc_moddown(orc.h, _p(acc[p]), nq, _p(want[p]))
+    assert np.array_equal(host(ctx.moddown(dacc, nq)), want)
+
+
+@pytest.mark.parametrize("step", [1, 2, 4, 8, 16, 32, 64] + [128 * j for j in (1, 2, 16, 48, 112, 128, 255)])
+def test_rotation_step_set_at_level_20_of_24(chain24, step):
+    orc, ctx, ct, dct = chain24
+    orc.gen_rot_key(6, step)
+    g = orc.galois(step)
+    want = orc.left_rotate(O.Ct(ct, 1.0), step)
+    got = host(ctx.rotate(dct, dev(orc.keys.pop(("gal", g))), g, 21))
+    assert np.array_equal(got, want.data)

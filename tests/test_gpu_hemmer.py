@@ -359,11 +359,14 @@ def test_reuse_variants_and_repacking(small, fused):
     c = H.matmul_cc_reuse(tmp, bt, T)
     d = H.decrypt2(c)
     assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    otmp = [to_oracle(orc, tmp.get(k, n, n, 2 * n)) for k in range(len(tmp))]
     if fused:   # tau(B) through the batched transform, then all its rotations from one ModUp: residues
         assert np.array_equal(bt.residues(), R.lower_and_transform_fused(orc, to_oracle(orc, b), R.V, n, 2 * n, T + 1).data)
-        otmp = [to_oracle(orc, tmp.get(k, n, n, 2 * n)) for k in range(len(tmp))]
         want = R.mult_mat_mat_cc_reuse_fused(orc, otmp, to_oracle(orc, bt), 2 * n)
         assert np.array_equal(c.residues(), want.data)
+    else:       # reference order: levelDown + tau, then the chained rotations of tau(B)
+        assert np.array_equal(bt.residues(), R.mult_mat_mat_pre_rev(ev, to_oracle(orc, b), T, n, 2 * n).data)
+        assert np.array_equal(c.residues(), R.mult_mat_mat_cc_reuse(ev, otmp, to_oracle(orc, bt), 2 * n).data)
     # packed counterparts: the same product as packedMatMul
     pa, pb = H.encrypt2(A0, A1), H.encrypt2(B0, B1)
     H.complex_packing_inplace(pa)
@@ -375,6 +378,16 @@ def test_reuse_variants_and_repacking(small, fused):
     pc = H.repack_cc(pprod)
     d = H.decrypt2(pc)
     assert np.abs(d[0] - A0 @ B0).max() < 2 ** -18 and np.abs(d[1] - A1 @ B1).max() < 2 ** -18
+    if not fused:
+        osa = R.mult_mat_mat_pre_rev(ev, to_oracle(orc, pa), T + 1, n, 2 * n, kind=R.PH)   # multPackedMatMatPre: T + 3
+        assert np.array_equal(sa.residues(), osa.data)
+        want_rot = R.mult_packed_mat_mat_pre_rot(ev, osa, T, n, 2 * n)
+        assert len(ptmp) == len(want_rot) == n // 2
+        for k in range(len(ptmp)):
+            assert np.array_equal(ptmp.get(k, n, n, 2 * n).residues(), want_rot[k].data), k
+        assert np.array_equal(pbt.residues(), R.mult_mat_mat_pre_rev(ev, to_oracle(orc, pb), T, n, 2 * n, kind=R.PV).data)
+        want = R.mult_mat_mat_cc_reuse(ev, want_rot, to_oracle(orc, pbt), 4 * n, rescale_after=True)
+        assert np.array_equal(pprod.residues(), want.data)
     if fused:
         osa = R.lower_and_transform_fused(orc, to_oracle(orc, pa), R.PH, n, 2 * n, T + 2)
         assert np.array_equal(sa.residues(), osa.data)
@@ -408,6 +421,34 @@ def test_reuse_variants_and_repacking(small, fused):
     m = np.concatenate([np.ones((n, n)), np.zeros((n, n))], axis=1).ravel()
     want = (o + rot) * m + np.roll(rot * m, n)
     assert np.abs(out - want).max() < 2 ** -18
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+@pytest.mark.parametrize("target_level", [0, 3])
+def test_transpose_complex_packing_inplace(small, fused, target_level):
+    """HEMMer::transposeComplexPackingInplace: columns (2c, 2c+1) -> a - i b written to both, optional levelDown,
+    transpose; residues against the restatement, slots against the closed form."""
+    H, orc, ev = small
+    n = 16
+    rng = np.random.default_rng(21)
+    A0, A1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    x = H.encrypt2(A0, A1)
+    ox = to_oracle(orc, x)
+    H.set_schedule(fused)
+    try:
+        H.transpose_complex_packing_inplace(x, target_level)
+    finally:
+        H.set_schedule(True)
+    want = R.transpose_complex_packing(ev, ox, n, 2 * n, target_level, fused_orc=orc if fused else None)
+    assert x.info()["level"] == want.level
+    assert np.array_equal(x.residues(), want.data)
+    M = np.concatenate([A0, A1], axis=1)                      # rows of the pair layout, 2n wide
+    P = np.empty_like(M, dtype=np.complex128)
+    P[:, 0::2] = M[:, 0::2] - 1j * M[:, 1::2]
+    P[:, 1::2] = P[:, 0::2]
+    z = H.decrypt_slots(x).reshape(n, 2 * n)
+    for half in (0, 1):
+        assert np.abs(z[:, half * n:(half + 1) * n] - P[:, half * n:(half + 1) * n].T).max() < 2 ** -18
 
 
 def test_rotate_and_sum_reductions(small):

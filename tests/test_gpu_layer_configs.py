@@ -102,7 +102,7 @@ def test_lora_low_rank_path(H):
 
 
 def test_attention_head():
-    # 12 levels hold scores (3) + polynomial (5) + scores x V (3) only if the products may run down to level 1:
+    # 12 levels hold scores (3) + polynomial (4) + scores x V (3 or 4) only if the products may run down to level 1:
     # the preset keeps the reference's rule "bootstrap below level 4 + 3", so this uses the same primes with the
     # minimum bootstrap level set to 0
     load_package()
@@ -122,8 +122,9 @@ def test_attention_head():
     # Gaussian-kernel score (any smooth kernel exercises the same evaluation)
     f = lambda t: np.exp(-2.0 * (1.0 - t) ** 2)
     coef = C.chebinterpolate(f, 15)
-    p = H.eval_chebyshev(s, list(coef), 4)
-    assert p.info()["level"] == 4
+    from oracle import poly_ref as P
+    p = H.eval_chebyshev(s, P.cheb_plain_to_product(coef, 4), 4)   # tables are in the baby-step / giant-step product basis
+    assert p.info()["level"] == 9 - 4                              # level_cost = log2(4) + log2(4)
     assert np.abs(H.decrypt(p) - f(S)).max() < 2 ** -9
     out = H.single_cc_matmul(p, cv, 1)
     assert out.info()["level"] == 1

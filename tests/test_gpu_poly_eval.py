@@ -8,7 +8,7 @@ from __graft_entry__ import load_package
 from oracle import hemmer_ref as R
 from oracle import oracle as O
 from oracle import poly_ref as P
-from tests.test_poly_eval import EXP_2
+from tests.test_poly_eval import EXP_15_4, EXP_2
 
 pytestmark = pytest.mark.gpu
 
@@ -42,12 +42,24 @@ def test_residues_match_oracle(small):
         want = P.eval_odd_polynomial(ev, oct_, poly, k, l)
         assert np.array_equal(got.residues(), want.data), (k, l)
         assert np.abs(H.decrypt(got) - np.polynomial.polynomial.polyval(M, poly)).max() < 2 ** -16
-    for coef, baby in ((EXP_2, 4), (list(rng.normal(size=16)), 4), (list(rng.normal(size=8)), 2),
-                       ([0.5, 0, 0, 0, 2.0], 4)):
-        got = H.eval_chebyshev(ct, coef, baby)
-        want = P.eval_chebyshev(ev, oct_, coef, baby)
+    # tables in the product basis of HEaaN-math: the reference's own EXP_15_4, random tables, a plain series as one
+    # block, a sparse one
+    for coef, baby in ((EXP_15_4, 4), (list(rng.normal(size=16)), 4), (list(rng.normal(size=8)), 2),
+                       (list(rng.normal(size=11)), 8), (list(rng.normal(size=6)), 0), ([0.5, 0, 0, 0, 2.0], 4)):
+        got = H.eval_chebyshev(ct, coef, baby, 0.5)
+        want = P.eval_chebyshev(ev, oct_, coef, baby, 0.5)
         assert np.array_equal(got.residues(), want.data), (len(coef), baby)
-        assert np.abs(H.decrypt(got) - C.chebval(M, coef)).max() < 2 ** -14
+        assert np.abs(H.decrypt(got) - 0.5 * P.cheb_product_value(coef, baby, M)).max() < 2 ** -14
+    # exp on [-2, 2] as the reference computes it (src/Loss.cpp:41-56): linearTransform, then the table
+    M2 = rng.uniform(-2, 2, (16, 16))
+    c2 = H.encrypt(M2)
+    o2 = O.Ct(c2.residues(), orc.delta[c2.info()["level"]])
+    u, ou = H.linear_transform(c2, -2.0, 2.0), P.linear_transform(ev, o2, -2.0, 2.0)
+    assert np.array_equal(u.residues(), ou.data)
+    got, want = H.eval_chebyshev(u, EXP_15_4, 4), P.eval_chebyshev(ev, ou, EXP_15_4, 4)
+    assert np.array_equal(got.residues(), want.data)
+    assert got.info()["level"] == u.info()["level"] - 4
+    assert np.abs(H.decrypt(got) - np.exp(M2)).max() < 2 ** -16
     with pytest.raises(ValueError):
         H.eval_chebyshev(ct, EXP_2, 3)          # baby steps must be a power of two
     low = H.level_down(ct, 2)
@@ -62,8 +74,8 @@ def test_full_ring_values():
     rng = np.random.default_rng(3)
     M = rng.uniform(-1, 1, (128, 128))
     ct = H.encrypt(M)
-    e = H.eval_chebyshev(ct, EXP_2, 4)
-    assert e.info()["level"] == 12 - 4      # its three last coefficients are below 1e-8: integer-0 products, no level
+    e = H.eval_chebyshev(ct, EXP_15_4, 4)   # the reference's table, 4 levels (its level_cost)
+    assert e.info()["level"] == 12 - 4
     assert np.abs(H.decrypt(e) - np.exp(2 * M)).max() < 2 ** -12
     r = H.exp_iter(ct, 6)
     assert np.abs(H.decrypt(r) - (1 + M / 64) ** 64).max() < 2 ** -12
