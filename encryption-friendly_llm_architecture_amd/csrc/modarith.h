@@ -53,10 +53,16 @@ __device__ __forceinline__ u64 mul_shoup(u64 x, u64 w, u64 ws, u64 q) {
 // hi' = xh wh + (xh wl >> 32) + (xl wh >> 32) is at most 2 below floor(x ws / 2^64), so the result lies in [0, 4q)
 // instead of [0, 2q) for any 64-bit x.  One multiply-add and the carry chain of the exact high product are saved.
 __device__ __forceinline__ u64 mul_shoup_lazy4(u64 x, u64 w, u64 ws, u64 q) {
-    const u32 xl = (u32)x, xh = (u32)(x >> 32), wl = (u32)ws, wh = (u32)(ws >> 32);
-    const u64 a = (u64)xh * wl, b = (u64)xl * wh;
-    const u64 hi = (u64)xh * wh + (a >> 32) + (b >> 32);
-    return x * w - hi * q;
+    const u32 xl = (u32)x, xh = (u32)(x >> 32), sl = (u32)ws, sh = (u32)(ws >> 32);
+    const u64 hi = ((u64)xh * sh + __umulhi(xh, sl)) + __umulhi(xl, sh);
+    // x * w - hi * q = x * w + hi * (2^64 - q) mod 2^64 as one chain of 32-bit multiply-adds: the two low products
+    // accumulate in one 64-bit register (a carry out of bit 64 is dropped, as it should be), the four cross products
+    // only feed the high word; no 64-bit subtraction and none of its carry hazards
+    const u64 nq = 0 - q;
+    const u32 hl = (u32)hi, hh = (u32)(hi >> 32), wl = (u32)w, wh = (u32)(w >> 32), nl = (u32)nq, nh = (u32)(nq >> 32);
+    const u64 t = (u64)hl * nl + (u64)xl * wl;
+    const u32 top = (u32)(t >> 32) + xl * wh + xh * wl + hl * nh + hh * nl;
+    return ((u64)top << 32) | (u32)t;
 }
 // Barrett reduction of a 128-bit value T < 6 * 2^(2k) to [0, q).
 __device__ __forceinline__ u64 barrett128(u128_t t, const ModQ &m) {

@@ -24,18 +24,27 @@ struct __align__(16) Tw {
 };
 
 // Lazy butterflies (q < 2^61, so 8q < 2^64): forward values stay in [0, 8q), inverse values in [0, 4q); q4 = 4q.
-__device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4) {
-    u64 u = x;
-    if (u >= q4) u -= q4;                                  // < 4q
+// u -= 4q when u >= 4q, written as an addition of -4q and a select: no borrow chain
+__device__ __forceinline__ u64 csub(u64 u, const u64 m, const u64 neg_m) {
+    u64 t = u + neg_m;
+    asm("" : "+v"(t));          // keeps the compiler from turning this back into a subtraction of a selected 0 / m
+    return u >= m ? t : u;
+}
+// 2^64 - m as a value the compiler cannot see through (it would turn x + (2^64 - m) back into a subtraction)
+__device__ __forceinline__ u64 opaque_neg(u64 m) {
+    u64 n = 0 - m;
+    asm("" : "+s"(n));
+    return n;
+}
+__device__ __forceinline__ void ct_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4, const u64 nq4) {
+    const u64 u = csub(x, q4, nq4);                        // < 4q
     const u64 v = mul_shoup_lazy4(y, tw.w, tw.ws, q);      // < 4q
     x = u + v;
     y = u - v + q4;
 }
-__device__ __forceinline__ void gs_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4) {
+__device__ __forceinline__ void gs_bfly(u64 &x, u64 &y, const Tw tw, const u64 q, const u64 q4, const u64 nq4) {
     const u64 u = x, v = y;                                // < 4q each
-    u64 s = u + v;
-    if (s >= q4) s -= q4;
-    x = s;
+    x = csub(u + v, q4, nq4);
     y = mul_shoup_lazy4(u - v + q4, tw.w, tw.ws, q);
 }
 
@@ -62,7 +71,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + (size_t)prime * N;
-    const u64 q = modq[prime].q, q2 = 2 * q, q4 = 4 * q;
+    const u64 q = modq[prime].q, q2 = 2 * q, q4 = 4 * q, nq4 = opaque_neg(q4);
     u64 *base = data + (size_t)poly * poly_stride + (size_t)sl.idx[limb] * N;
     const int tile = blockIdx.x;
     // tile origin: strided pass tiles walk the columns; contiguous pass tiles walk the limb
@@ -85,7 +94,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
                 int gidx = r * gp.rowstride + c0 + cc;
                 Tw w = tw[(1 << s) + (gidx / (2 * t))];
                 u64 x = lds[i], y = lds[j];
-                ct_bfly(x, y, w, q, q4);
+                ct_bfly(x, y, w, q, q4, nq4);
                 lds[i] = x;
                 lds[j] = y;
             }
@@ -102,7 +111,7 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
                 int gidx = r * gp.rowstride + c0 + cc;
                 Tw w = tw[(1 << s) + (gidx / (2 * t))];
                 u64 x = lds[i], y = lds[j];
-                gs_bfly(x, y, w, q, q4);
+                gs_bfly(x, y, w, q, q4, nq4);
                 lds[i] = x;
                 lds[j] = y;
             }
@@ -147,33 +156,32 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
 struct IntField {
     typedef u64 E;
     typedef Tw W;
-    u64 q, q2, q4, ni, nis;
+    u64 q, q2, q4, nq4, nq2, nq1, ni, nis;
     __device__ __forceinline__ IntField(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
         q = modq[prime].q;
         q2 = 2 * q;
         q4 = 4 * q;
+        nq4 = opaque_neg(q4);
+        nq2 = opaque_neg(q2);
+        nq1 = opaque_neg(q);
         ni = ninv[prime];
         nis = ninv_s[prime];
     }
     __device__ __forceinline__ E from_canonical(u64 v) const { return v; }
-    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q4); }
-    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q4); }
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q4, nq4); }
+    __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q4, nq4); }
     __device__ __forceinline__ void before_inverse_block(E (&)[16]) const {}
     __device__ __forceinline__ u64 to_canonical(E v) const {   // v < 8q
-        if (v >= q4) v -= q4;
-        if (v >= q2) v -= q2;
-        return v >= q ? v - q : v;
+        return csub(csub(csub(v, q4, nq4), q2, nq2), q, nq1);
     }
     __device__ __forceinline__ u64 scale_to_canonical(E v) const {
-        u64 t = mul_shoup_lazy(v, ni, nis, q);
-        return t >= q ? t - q : t;
+        return csub(mul_shoup_lazy(v, ni, nis, q), q, nq1);
     }
     // (y - v) * cst mod q for a transformed value v and a canonical minuend y
     __device__ __forceinline__ u64 sub_scale(E v, u64 y, const Tw cst) const {
         const u64 c = to_canonical(v);
         const u64 d = y >= c ? y - c : y + q - c;
-        const u64 t = mul_shoup_lazy(d, cst.w, cst.ws, q);
-        return t >= q ? t - q : t;
+        return csub(mul_shoup_lazy(d, cst.w, cst.ws, q), q, nq1);
     }
 };
 
