@@ -24,6 +24,8 @@ struct BConvArgs {
     const Cst *hat;        // [n_src][hat_ld]  (S/q_i) mod prime, indexed by prime
     int n_src, n_dst, hat_ld, logN;
     int pre_scaled;        // the source residues already carry their (S/q_i)^-1 factor (folded into the inverse transform)
+    int split;             // register kernels: the target limbs are dealt to this many workgroups per coefficient block
+                           // (blockIdx.y = polynomial * split + part); 0 counts as 1
     uint8_t src_slot[32], src_prime[32];
     uint8_t dst_slot[HEMM_MAX_PRIMES], dst_prime[HEMM_MAX_PRIMES];
 };
@@ -68,7 +70,9 @@ __device__ __forceinline__ u64 reduce_below_32q(u64 v, const u64 q) {
 // take the cheaper products with a three-term quotient estimate (each below 4q) and reduce once at the end.
 template <int NS>
 __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ *__restrict__ modq) {
-    const int poly = blockIdx.y;
+    const int S = a.split > 1 ? a.split : 1;
+    const int poly = blockIdx.y / S, part = blockIdx.y % S;
+    const int per = (a.n_dst + S - 1) / S, j_lo = part * per, j_hi = min(a.n_dst, j_lo + per);
     const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
     const u64 *src = a.src + poly * a.src_poly_stride;
     u64 *dst = a.dst + poly * a.dst_poly_stride;
@@ -81,7 +85,7 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
         v0[i] = a.pre_scaled ? x.x : mul_shoup(x.x, c.w, c.ws, q);
         v1[i] = a.pre_scaled ? x.y : mul_shoup(x.y, c.w, c.ws, q);
     }
-    for (int j = 0; j < a.n_dst; j++) {
+    for (int j = j_lo; j < j_hi; j++) {
         const int pj = a.dst_prime[j];
         const u64 q = modq[pj].q;
         u64 acc0 = 0, acc1 = 0;
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
 // own, plus the copy of its own limbs (already in NTT form in `own`) into its slice of the extended polynomial.
 #define BCONV_MAX_DIGITS 4
 struct BConvDigits {
-    BConvArgs d[BCONV_MAX_DIGITS];
+    BConvArgs d[BCONV_MAX_DIGITS];  // d[0].split applies to every digit
     const u64 *own;        // [n_polys][.][N] NTT form, polynomial stride own_stride
     size_t own_stride;
     uint8_t own_lo[BCONV_MAX_DIGITS], own_hi[BCONV_MAX_DIGITS];
@@ -126,7 +130,9 @@ struct BConvDigits {
 template <int NS>
 __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const ModQ *__restrict__ modq) {
     const BConvArgs &a = g.d[blockIdx.z];
-    const int poly = blockIdx.y;
+    const int S = g.d[0].split > 1 ? g.d[0].split : 1;
+    const int poly = blockIdx.y / S, part = blockIdx.y % S;
+    const int per = (a.n_dst + S - 1) / S, j_lo = part * per, j_hi = min(a.n_dst, j_lo + per);
     const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
     const u64 *src = a.src + poly * a.src_poly_stride;
     u64 *dst = a.dst + poly * a.dst_poly_stride;
@@ -142,7 +148,7 @@ __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const 
             v1[i] = a.pre_scaled ? x.y : mul_shoup(x.y, c.w, c.ws, q);
         }
     }
-    for (int j = 0; j < a.n_dst; j++) {
+    for (int j = j_lo; j < j_hi; j++) {
         const int pj = a.dst_prime[j];
         const u64 q = modq[pj].q;
         u64 acc0 = 0, acc1 = 0;
@@ -178,13 +184,25 @@ __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const 
         *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
     }
     const u64 *own = g.own + poly * g.own_stride;
-    for (int j = g.own_lo[blockIdx.z]; j < g.own_hi[blockIdx.z]; j++)
+    for (int j = g.own_lo[blockIdx.z] + part; j < g.own_hi[blockIdx.z]; j += S)
         *(ulonglong2 *)(dst + ((size_t)j << a.logN) + n) = *(const ulonglong2 *)(own + ((size_t)j << a.logN) + n);
 }
 
 // grid = (N / 256, n_polys) coefficients x polynomials
-void launch_bconv(const BConvArgs &a, const ModQ *modq, int N, int n_polys, hipStream_t s) {
-    dim3 block(256), wide(N / 256, n_polys), pair(N / 512, n_polys);
+// A conversion over few polynomials has too few coefficient blocks to fill the GPU (N / 512 workgroups per polynomial
+// and digit, each thread walking every target limb in turn): its target limbs are then dealt to `split` workgroups.
+static int bconv_split(int N, int n_units, int n_dst) {
+    const int blocks = (N / 512) * n_units;
+    int S = (1536 + blocks - 1) / blocks;
+    if (S > 8) S = 8;
+    if (S > n_dst) S = n_dst;
+    return S < 1 ? 1 : S;
+}
+
+void launch_bconv(const BConvArgs &a_in, const ModQ *modq, int N, int n_polys, hipStream_t s) {
+    BConvArgs a = a_in;
+    a.split = (a.n_src <= 8 && N >= 512) ? bconv_split(N, n_polys, a.n_dst) : 1;
+    dim3 block(256), wide(N / 256, n_polys), pair(N / 512, n_polys * a.split);
     switch (a.n_src) {
 #define BCONV_CASE(K) case K: hipLaunchKernelGGL(bconv_reg_kernel<K>, pair, block, 0, s, a, modq); break;
         BCONV_CASE(1) BCONV_CASE(2) BCONV_CASE(3) BCONV_CASE(4) BCONV_CASE(5) BCONV_CASE(6) BCONV_CASE(7) BCONV_CASE(8)
@@ -836,6 +854,22 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
     u64 *ext = coef + (size_t)2 * (c->nQ) * N;   // [beta][E][N]
     u64 *acc = ext + (size_t)beta * E * N;       // [2][E][N]
     launch_modup_batch(c, in, (size_t)nq * N, nq, 1, ext, coef, s);   // same arithmetic as launch_modup, 5 launches
+    if (N >= 512) {
+        // the key product as a hoisted sum of one term under the identity automorphism: P * add_b joins the sum in
+        // the extended basis, so the ModDown needs no addend and ends in the forward transform's fused tail
+        // (identical residues: every step is exact modular arithmetic in the same order)
+        RotTermDev term;
+        memset(&term, 0, sizeof(term));
+        term.ext = ext;
+        term.b = add_b;
+        term.evk = evk;
+        term.galois = 1;
+        term.pt_galois = 1;
+        const u32 off[2] = {0, 1};
+        launch_hoisted_terms_args(c, &term, 1, off, 1, nq, acc, false, s);
+        launch_moddown_batch(c, acc, nq, 2, 0, out, out_stride, coef, s);
+        return;
+    }
     launch_inner_product(c, in, ext, evk, nq, acc, s);
     launch_moddown(c, acc, nq, 2, out, out_stride, add_b, 0, add_b ? 1 : 0, coef, s);
 }
@@ -1003,7 +1037,8 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
                                   (size_t)(hi - lo) * N * 8, n_in, hipMemcpyDeviceToDevice, s));
     }
     if (!joint) return;
-    const dim3 grid((unsigned)(N / 512), n_in, beta), block(256);
+    g.d[0].split = bconv_split((int)N, n_in * beta, E - alpha);
+    const dim3 grid((unsigned)(N / 512), n_in * g.d[0].split, beta), block(256);
     const int widest = std::min(nq, alpha);
     if (widest <= 2)
         hipLaunchKernelGGL(bconv_digits_kernel<2>, grid, block, 0, s, g, c->d_modq);
