@@ -56,6 +56,18 @@ def gpu_ccmm(args, out):
     out["gpu_event_ms_per_step"] = ev_ms / args.steps
     out["max_abs_err"] = err
     out["max_abs_err_ok"] = bool(err <= 2.0 ** -12)
+    # algorithmic bytes of one product, counted by the library as it queues the launches: per launch the operands it
+    # must read once plus the results it must write once (a two-launch transform = one read and one write per limb)
+    H.traffic(reset=True)
+    c = H.single_cc_matmul(ca, cb, T)
+    H.sync()
+    by, ln = H.traffic(reset=True)
+    total = sum(by.values())
+    out["ccmm_algorithmic_bytes"] = {
+        "total": total, "by_kind": by, "launches_by_kind": ln, "launches": sum(ln.values()),
+        "achieved_GBps": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9,
+        "frac_of_hbm_peak": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
     # one rotation (automorphism + hybrid key switch) at the top level
     r = H.left_rotate(ca, 1)
     H.sync()
@@ -137,6 +149,16 @@ def gpu_ntt(args, out):
         inv_ms = timer.stop() / iters
         res[bits] = (fwd_ms, inv_ms)
         del ctx, d, ref
+    a = torch.empty((32, 24, 1 << 16), dtype=torch.int64, device="cuda").fill_(1)
+    b = torch.empty_like(a)
+    b.copy_(a)
+    timer = pkg.Timer()
+    timer.start()
+    for _ in range(10):
+        b.copy_(a)
+        a.copy_(b)
+    copy_ms = timer.stop() / 10
+    del a, b
     fwd_ms, inv_ms = res[60]
     out["ntt_forward_limbs_per_s"] = limbs / fwd_ms * 1e3
     out["ntt_inverse_limbs_per_s"] = limbs / inv_ms * 1e3
@@ -155,6 +177,9 @@ def gpu_ntt(args, out):
         "frac_42bit": alg_bytes / (res[42][0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_launch_pair": alg_bytes, "avg_ms_per_launch_pair": fwd_ms,
         "avg_ms_per_launch_pair_42bit": res[42][0],
+        # the floor of a two-launch transform on this box: two plain device copies of the same 384 MiB
+        "two_device_copies_of_the_batch_ms": copy_ms,
+        "frac_of_two_copies": copy_ms / fwd_ms, "frac_of_two_copies_42bit": copy_ms / res[42][0],
     }
 
 
@@ -215,6 +240,54 @@ def gpu_hoisted(args, out):
         "frac": achieved / HBM_PEAK_GBS, "traffic": HOISTED_TRAFFIC_BYTES,
         "algorithmic_bytes_per_launch": alg_bytes, "avg_ms_per_launch": ms,
     }
+    # (b) the hoisted sum of one sigma / tau transform stage, the largest single launch of the product
+    # (hoisted_terms_kernel<0>): 2 outputs (one per operand) at level T+4, each 7 rotations of two masked sources
+    # under one key, full masks over the extended basis (9 + 4 limbs, 2 digits)
+    nq2, E2 = 9, 9 + K
+    src2 = [[(rnd(beta, E2, N), rnd(nq2, N)) for _ in range(2)] for _ in range(2)]
+    groups2 = []
+    for o in range(2):
+        grp = []
+        for r in range(7):
+            evk, gal = rnd(dnum, 2, T, N), pow(5, 8 * o + r + 1, 2 * N)
+            grp += [(src2[o][t][0], src2[o][t][1], evk, rnd(E2, N), gal, 0) for t in range(2)]
+        groups2.append(grp)
+    ctx.traffic(reset=True)
+    ctx.hoisted_terms(groups2, nq2, b_premultiplied=True)
+    stage_bytes = sum(ctx.traffic(reset=True)[0].values())
+    torch.cuda.synchronize()
+    timer.start()
+    for _ in range(iters):
+        ctx.hoisted_terms(groups2, nq2, b_premultiplied=True)
+    ms2 = timer.stop() / iters
+    out["roofline_transform_stage"] = {
+        "kernel": "hoisted_terms_kernel<0> (hoisted sum of one sigma/tau transform stage: 2 outputs x 7 keys x 2 "
+                  "masked sources, full masks, 9+4 limbs, 2 digits)",
+        "bound": "hbm", "achieved": stage_bytes / (ms2 * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": stage_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_launch": stage_bytes,
+        "avg_ms_per_launch": ms2,
+    }
+    # (c) the ModDown merged with the rescale of one main-loop batch: 64 polynomials from 7+4 to 6 limbs in five
+    # launches (inverse transform of the 5 dropped limbs, basis conversion, forward transform with the fused
+    # (y - conv) / (P q_6) tail)
+    y = rnd(64, E, N)
+    ctx.traffic(reset=True)
+    ctx.moddown_batch(y, nq, True)
+    md_by = ctx.traffic(reset=True)[0]
+    md_bytes = sum(md_by.values())
+    torch.cuda.synchronize()
+    timer.start()
+    for _ in range(iters):
+        ctx.moddown_batch(y, nq, True)
+    ms3 = timer.stop() / iters
+    out["roofline_moddown_chain"] = {
+        "kernel": "ntt16_rows_kernel<true,false> + ntt16_cols_kernel<true> + bconv_reg_kernel<5> + "
+                  "ntt16_cols_kernel<false> + ntt16_rows_kernel<false,true> (ModDown + rescale of 64 polynomials, "
+                  "7+4 -> 6 limbs)",
+        "bound": "hbm", "achieved": md_bytes / (ms3 * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": md_bytes / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_chain": md_bytes,
+        "algorithmic_bytes_by_kind": {k: v for k, v in md_by.items() if v}, "avg_ms_per_chain": ms3,
+    }
     if args.roofline_only:
         # a plain copy of known size in the same process: the scale reference for the --pmc counters
         a = torch.empty(1 << 27, dtype=torch.int64, device="cuda").fill_(1)
@@ -246,23 +319,54 @@ def gpu_rotation_60bit(args, out):
     out["rotation_24x60bit_level20_us"] = timer.stop() / 30 * 1e3
 
 
-def cpu_baseline(out, budget_s=25.0):
-    """The CPU oracle (scalar C++ port, one thread) on a bounded sample of the CCMM's operation mix,
-    scaled by the per-product operation counts."""
+def cpu_baseline(out):
+    """The CPU oracle (C++ port of the same arithmetic) on the GPU box's host cores.
+
+    cpu_baseline: ONE whole product of the headline workload -- the oracle's restatement of exactly the launch
+    schedule the GPU runs (complex-packed single-tile CCMM, same operation order, same residues) -- on all the cores
+    this job may use (the oracle threads over limbs).  cpu_baseline_1_thread: a bounded sample of the reference's
+    operation order on one thread, scaled by the operation counts of one product (a whole product would take
+    about two minutes on one thread)."""
     import numpy as np
+    from oracle import hemmer_ref as R
     from oracle import oracle as O
+    cores = max(1, min(16, os.cpu_count() or 1))
     qs, ps = O.ckks_chain(16, 13, 4)
-    orc = O.Oracle(16, qs, ps, dnum=3, threads=1)
+    orc = O.Oracle(16, qs, ps, dnum=3, threads=cores)
     orc.gen_secret(3)
     orc.key_seed = 3
     orc.gen_mult_key(3)
-    rng = np.random.default_rng(0)
-    z = rng.uniform(-1, 1, orc.slots).astype(np.complex128)
-    ct12 = orc.encrypt(orc.encode(z, 12), 4)
-    ct6 = orc.level_down(ct12, 6)
-    ct5 = orc.level_down(ct12, 5)
-    m12, m6 = orc.encode(z, 12), orc.encode(z, 6)
-    orc.left_rotate(ct6, 1)   # derive the key outside the timed region
+    orc.gen_conj_key(3)
+    rng = np.random.default_rng(1)
+    n = 128
+    A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+
+    def enc(M, seed):
+        z = np.zeros(orc.slots, dtype=np.complex128)
+        z[:M.size] = M.reshape(-1)
+        return orc.encrypt(orc.encode(z, orc.nQ - 1), seed)
+
+    ca, cb = enc(A, 11), enc(B, 12)
+    t0 = time.perf_counter()
+    c = R.mult_mat_mat_cc_packed_single(orc, ca, cb, 4, n, n)   # keys are derived on first use, inside the timed region
+    full_s = time.perf_counter() - t0
+    err = float(np.abs(orc.decrypt(c)[:n * n].real.reshape(n, n) - A @ B).max())
+    out["cpu_baseline"] = {
+        "value": full_s * 1e3, "unit": "ms", "cores": cores, "kind": "port",
+        "sample": "one whole 128x128 singleCCMatMul on the CPU oracle (restatement of the batched complex-packed "
+                  "schedule the GPU runs, N=2^16, 13+4 primes, level 12 -> 4; about 330 evaluation keys derived on "
+                  "first use inside the timed region), %d threads over limbs; max abs error %.2e" % (cores, err),
+    }
+    orc1 = O.Oracle(16, qs, ps, dnum=3, threads=1)
+    orc1.gen_secret(3)
+    orc1.key_seed = 3
+    orc1.gen_mult_key(3)
+    z = rng.uniform(-1, 1, orc1.slots).astype(np.complex128)
+    ct12 = orc1.encrypt(orc1.encode(z, 12), 4)
+    ct6 = orc1.level_down(ct12, 6)
+    ct5 = orc1.level_down(ct12, 5)
+    m12, m6 = orc1.encode(z, 12), orc1.encode(z, 6)
+    orc1.left_rotate(ct6, 1)   # derive the key outside the timed region
 
     def t(fn, reps):
         t0 = time.perf_counter()
@@ -270,25 +374,26 @@ def cpu_baseline(out, budget_s=25.0):
             fn()
         return (time.perf_counter() - t0) / reps
 
-    t_rot12 = t(lambda: orc.left_rotate(ct12, 1), 2)
-    t_rot6 = t(lambda: orc.left_rotate(ct6, 1), 4)
-    t_mul12 = t(lambda: orc.mult_plain_no_rescale(ct12, m12), 2)
-    t_mul6 = t(lambda: orc.mult_plain_no_rescale(ct6, m6), 4)
-    pre = orc.mult_plain_no_rescale(ct6, m6)
-    t_res6 = t(lambda: orc.rescale(pre), 4)
-    t_tensor5 = t(lambda: orc.tensor(ct5, ct5), 4)
-    t3 = orc.tensor(ct5, ct5)
-    t_relin5 = t(lambda: orc.relinearize(t3), 2)
-    # operation counts of one 128 x 128 CCMM: 2 transforms (32 rotations + 255 mask products each at
-    # level 12), 508 rotations + 508 mask products + 254 rescales at level 6, 127 tensor products,
-    # 2 relinearisations
+    t_rot12 = t(lambda: orc1.left_rotate(ct12, 1), 1)
+    t_rot6 = t(lambda: orc1.left_rotate(ct6, 1), 2)
+    t_mul12 = t(lambda: orc1.mult_plain_no_rescale(ct12, m12), 2)
+    t_mul6 = t(lambda: orc1.mult_plain_no_rescale(ct6, m6), 2)
+    pre = orc1.mult_plain_no_rescale(ct6, m6)
+    t_res6 = t(lambda: orc1.rescale(pre), 2)
+    t_tensor5 = t(lambda: orc1.tensor(ct5, ct5), 2)
+    t3 = orc1.tensor(ct5, ct5)
+    t_relin5 = t(lambda: orc1.relinearize(t3), 1)
+    # operation counts of one 128 x 128 CCMM in the reference's order: 2 transforms (32 rotations + 255 mask
+    # products each at level 12), 508 rotations + 508 mask products + 254 rescales at level 6, 127 tensor
+    # products, 2 relinearisations
     total = (64 * t_rot12 + 510 * t_mul12 + 508 * t_rot6 + 508 * t_mul6 + 254 * t_res6 +
              128 * t_tensor5 + 2 * t_relin5)
-    out["cpu_baseline"] = {
+    out["cpu_baseline_1_thread"] = {
         "value": total * 1e3, "unit": "ms", "cores": 1, "kind": "port",
-        "sample": "CPU oracle, 1 thread: timed 2 rotations + 2 mask products at level 12, 4 rotations, "
-                  "4 mask products, 4 rescales at level 6, 4 tensor products + 2 relinearisations at "
-                  "level 5; scaled by the operation counts of one CCMM (64/510/508/508/254/128/2)",
+        "sample": "CPU oracle, 1 thread, the reference's operation order: timed 1 rotation + 2 mask products at "
+                  "level 12, 2 rotations, 2 mask products, 2 rescales at level 6, 2 tensor products + 1 "
+                  "relinearisation at level 5; scaled by the operation counts of one CCMM "
+                  "(64/510/508/508/254/128/2)",
         "rotation_level12_ms": t_rot12 * 1e3, "rotation_level6_ms": t_rot6 * 1e3,
     }
 

@@ -117,6 +117,16 @@ class Context:
     def psi(self, idx):
         return lib().hemm_context_psi(self.h, idx)
 
+    TRAFFIC_KINDS = ("transforms", "key_products", "basis_conversions", "tensor_accumulation", "masked_sums", "pointwise")
+
+    def traffic(self, reset=False):
+        """Algorithmic bytes and launch counts queued on this context since the last reset, by kind of work."""
+        b = (ctypes.c_uint64 * 8)()
+        n = (ctypes.c_uint64 * 8)()
+        check(lib().hemm_traffic(self.h, b, n, int(reset)))
+        return ({k: int(b[i]) for i, k in enumerate(self.TRAFFIC_KINDS)},
+                {k: int(n[i]) for i, k in enumerate(self.TRAFFIC_KINDS)})
+
     def ntt(self, data, prime_idx, inverse=False, stream=None):
         """In-place transform of a CUDA int64 tensor shaped [..., n_limbs, N]."""
         n_limbs = len(prime_idx)

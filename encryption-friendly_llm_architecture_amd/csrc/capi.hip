@@ -387,7 +387,8 @@ static void run_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, con
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t),
                                   &off_dev, stream);
-    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, y, b_premultiplied, stream);
+    launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, y, b_premultiplied, stream, d.data(),
+                         (int)d.size());
 }
 
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
@@ -453,8 +454,22 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
     void *terms_dev = upload_desc(ctx, terms, n_terms * sizeof(hemm_lin_term), group_offsets,
                                   (n_out + 1) * sizeof(uint32_t), &off_dev, (hipStream_t)stream);
     launch_masked_sum(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
-                      (hipStream_t)stream);
+                      (hipStream_t)stream, terms, (int)n_terms);
     check_launch();
+    HEMM_CATCH
+}
+
+int hemm_traffic(hemm_context *ctx, uint64_t *bytes, uint64_t *launches, int reset) {
+    HEMM_TRY
+    need(ctx != nullptr, "null context");
+    for (int k = 0; k < HEMM_TRAFFIC_KINDS; k++) {
+        if (bytes) bytes[k] = k < TR_KINDS ? ctx->traffic[k] : 0;
+        if (launches) launches[k] = k < TR_KINDS ? ctx->launches[k] : 0;
+    }
+    if (reset) {
+        memset(ctx->traffic, 0, sizeof(ctx->traffic));
+        memset(ctx->launches, 0, sizeof(ctx->launches));
+    }
     HEMM_CATCH
 }
 

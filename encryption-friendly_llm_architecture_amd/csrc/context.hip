@@ -173,6 +173,8 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_scratch = nullptr;
     c->d_desc = nullptr;
     c->scratch_bytes = 0;
+    memset(c->traffic, 0, sizeof(c->traffic));
+    memset(c->launches, 0, sizeof(c->launches));
     return c;
 }
 

@@ -36,7 +36,18 @@ struct hemm_context {
     u64 *d_scratch;
     size_t scratch_bytes;
     void *d_desc;                   // staging for the term lists of batched calls
+    // Algorithmic bytes of everything launched on this context since the last reset, by kind of work: for each
+    // launch the operands it has to read once plus the results it has to write once (what a launch of that kind
+    // cannot avoid moving), counted on the host when the launch is queued.  A 2^16-point transform counts one
+    // read and one write of every limb although it runs as two launches.
+    unsigned long long traffic[8], launches[8];
 };
+enum { TR_NTT = 0, TR_KEYPROD, TR_BCONV, TR_TENSOR, TR_MASKED, TR_POINTWISE, TR_KINDS };
+inline void account(const hemm_context *c, int kind, size_t bytes, int n_launches = 1) {
+    hemm_context *m = const_cast<hemm_context *>(c);
+    m->traffic[kind] += bytes;
+    m->launches[kind] += (unsigned long long)n_launches;
+}
 
 // a constant and its Shoup quotient floor(w * 2^64 / q)
 struct __align__(16) Cst {
@@ -99,15 +110,16 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
                     int n_polys, hipStream_t s);
 void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
                         hipStream_t s);
+// terms_host / n_terms: the host copy of the list (only read for the byte accounting; may be nullptr)
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, hipStream_t s);
+                          bool b_premultiplied, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0);
 int hoisted_arg_capacity();
 void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
                                int nq, u64 *y, bool b_premultiplied, hipStream_t s);
 void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
                           u64 *conv, hipStream_t s);
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
-                       u64 *out, hipStream_t s);
+                       u64 *out, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0);
 // y[o][p][j] = sum_{q < parts} part[o * parts + q][p][j] over the extended basis, y / part: [.][2][nq+K][N]
 void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s);
 int masked_arg_capacity();

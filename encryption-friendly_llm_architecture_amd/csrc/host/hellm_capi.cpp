@@ -129,6 +129,13 @@ int hellm_sync(void) {
     FACADE_CATCH
 }
 
+int hellm_traffic(hellm_hemmer *h, uint64_t *bytes, uint64_t *launches, int reset) {
+    FACADE_TRY
+    need(h, "null argument");
+    if (hemm_traffic(h->m->getContext()->dev, bytes, launches, reset) != 0) throw RuntimeException(hemm_last_error());
+    FACADE_CATCH
+}
+
 int hellm_encrypt(hellm_hemmer *h, const double *m, uint32_t rows, uint32_t cols, hellm_ct **out) {
     FACADE_TRY
     need(h && out, "null argument");

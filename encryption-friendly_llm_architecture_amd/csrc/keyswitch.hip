@@ -199,8 +199,9 @@ static int bconv_split(int N, int n_units, int n_dst) {
     return S < 1 ? 1 : S;
 }
 
-void launch_bconv(const BConvArgs &a_in, const ModQ *modq, int N, int n_polys, hipStream_t s) {
+void launch_bconv(const hemm_context *c, const BConvArgs &a_in, const ModQ *modq, int N, int n_polys, hipStream_t s) {
     BConvArgs a = a_in;
+    account(c, TR_BCONV, (size_t)(a.n_src + a.n_dst) * n_polys * N * 8);
     a.split = (a.n_src <= 8 && N >= 512) ? bconv_split(N, n_polys, a.n_dst) : 1;
     dim3 block(256), wide(N / 256, n_polys), pair(N / 512, n_polys * a.split);
     switch (a.n_src) {
@@ -747,6 +748,7 @@ void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, b
     const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
     const size_t N = c->N;
     HEMM_HIP(hipMemcpyAsync(coef, in, (size_t)nq * N * 8, hipMemcpyDeviceToDevice, s));
+    account(c, TR_POINTWISE, (size_t)2 * nq * N * 8);
     launch_ntt(c, coef, limbs_default(c, nq, 0), nq, 1, (size_t)nq * N, true, s);
     for (int d = 0; d < beta; d++) {
         const int lo = d * alpha, hi = std::min(nq, lo + alpha);
@@ -778,7 +780,7 @@ void launch_modup(hemm_context *c, const u64 *in, int nq, u64 *ext, u64 *coef, b
         }
         a.n_dst = nd;
         if (nd > 0) {
-            launch_bconv(a, c->d_modq, (int)N, 1, s);
+            launch_bconv(c, a, c->d_modq, (int)N, 1, s);
             launch_ntt_slots(c, a.dst, pl, sl, nd, 1, (size_t)E * N, false, s);
         }
         if (fill_own)
@@ -796,6 +798,7 @@ void launch_inner_product(hemm_context *c, const u64 *in, const u64 *ext, const 
     if (in != nullptr)
         for (int j = 0; j < nq; j++) dm.digit_of[j] = (uint8_t)(j / alpha);
     dim3 grid(c->N / 256, E), block(256);
+    account(c, TR_KEYPROD, (size_t)(3 * beta * E + 2 * E) * c->N * 8);
     hipLaunchKernelGGL(inner_product_kernel, grid, block, 0, s, in, ext, evk, acc, c->d_modq,
                        limbs_default(c, nq, 1), dm, beta, E, c->nQ + c->nP, c->logN);
 }
@@ -832,12 +835,13 @@ void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, si
         a.dst_slot[j] = (uint8_t)j;
         a.dst_prime[j] = (uint8_t)j;
     }
-    launch_bconv(a, c->d_modq, (int)N, n_polys, s);
+    launch_bconv(c, a, c->d_modq, (int)N, n_polys, s);
     const dim3 block(256);
     launch_ntt(c, conv, limbs_default(c, nq, 0), nq, n_polys, (size_t)nq * N, false, s);
     CstList cl;
     for (int j = 0; j < nq; j++) cl.c[j] = t->pinv[j];
     dim3 g2(N / 256, nq * n_polys);
+    account(c, TR_POINTWISE, (size_t)(3 * n_polys + add_polys) * nq * N * 8);
     hipLaunchKernelGGL(sub_scale_kernel, g2, block, 0, s, acc, (size_t)E * N, conv, (size_t)nq * N, add, add_stride,
                        add_polys, out, out_stride, c->d_modq, cl, nq, c->logN);
 }
@@ -892,12 +896,14 @@ static void rescale_with(hemm_context *c, KsTables *t, u64 *sc, const u64 *in, s
         launch_ntt(c, last, pl, 1, n_polys, N, true, s);
     }
     dim3 grid(N / 256, (nq - 1) * n_polys), block(256);
+    account(c, TR_POINTWISE, (size_t)n_polys * nq * N * 8);
     hipLaunchKernelGGL(spread_kernel, grid, block, 0, s, last, tt, (size_t)(nq - 1) * N, c->d_modq, nq - 1, c->logN);
     if (launch_ntt_sub_scale(c, tt, nq - 1, n_polys, in, in_stride, out, out_stride, t->dev + t->qlinv_off[nq - 1], s))
         return;
     launch_ntt(c, tt, limbs_default(c, nq - 1, 0), nq - 1, n_polys, (size_t)(nq - 1) * N, false, s);
     CstList cl;
     for (int j = 0; j < nq - 1; j++) cl.c[j] = t->qlinv[nq - 1][j];
+    account(c, TR_POINTWISE, (size_t)3 * n_polys * (nq - 1) * N * 8);
     hipLaunchKernelGGL(sub_scale_kernel, grid, block, 0, s, in, in_stride, tt, (size_t)(nq - 1) * N,
                        (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq - 1, c->logN);
 }
@@ -1030,7 +1036,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
             continue;
         }
         if (nd > 0) {
-            launch_bconv(a, c->d_modq, (int)N, n_in, s);
+            launch_bconv(c, a, c->d_modq, (int)N, n_in, s);
             launch_ntt_slots(c, a.dst, pl, sl, nd, n_in, (size_t)beta * E * N, false, s);
         }
         HEMM_HIP(hipMemcpy2DAsync(a.dst + (size_t)lo * N, (size_t)beta * E * N * 8, in + (size_t)lo * N, in_stride * 8,
@@ -1040,6 +1046,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     g.d[0].split = bconv_split((int)N, n_in * beta, E - alpha);
     const dim3 grid((unsigned)(N / 512), n_in * g.d[0].split, beta), block(256);
     const int widest = std::min(nq, alpha);
+    account(c, TR_BCONV, (size_t)n_in * (beta * E + nq) * N * 8);   // every digit's sources and its whole slice
     if (widest <= 2)
         hipLaunchKernelGGL(bconv_digits_kernel<2>, grid, block, 0, s, g, c->d_modq);
     else if (widest <= 5)
@@ -1047,6 +1054,36 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     else
         hipLaunchKernelGGL(bconv_digits_kernel<8>, grid, block, 0, s, g, c->d_modq);
     launch_ntt_slots(c, ext, jp, js, n_joint, n_in, (size_t)beta * E * N, false, s);
+}
+
+
+// Algorithmic bytes of one hoisted sum: every distinct source once (its extended digits and, where present, its b),
+// every term's key once, full masks and plaintext factors once per distinct pointer (run tables by their own size),
+// every output once.
+static size_t hoisted_bytes(const hemm_context *c, const RotTermDev *t, int n_terms, int n_out, int nq) {
+    const size_t limb = (size_t)c->N * 8;
+    const int E = nq + c->nP, beta = (nq + c->alpha - 1) / c->alpha;
+    std::vector<const u64 *> seen;
+    auto first = [&](const u64 *p) {
+        if (p == nullptr) return false;
+        for (const u64 *q : seen)
+            if (q == p) return false;
+        seen.push_back(p);
+        return true;
+    };
+    size_t bytes = (size_t)n_out * 2 * E * limb;
+    for (int i = 0; i < n_terms; i++) {
+        bytes += (size_t)2 * beta * E * limb;   // the key of the term
+        if (first(t[i].ext)) bytes += (size_t)beta * E * limb;
+        if (first(t[i].b)) bytes += (size_t)nq * limb;
+        if (first(t[i].ext2)) bytes += (size_t)beta * E * limb;
+        if (first(t[i].b2)) bytes += (size_t)nq * limb;
+        const size_t mask_bytes = t[i].mask_shift ? (size_t)E * 2 * (limb >> t[i].mask_shift) : (size_t)E * limb;
+        if (first(t[i].mask)) bytes += mask_bytes;
+        if (first(t[i].mask2)) bytes += mask_bytes;
+        if (first(t[i].pt)) bytes += (size_t)E * limb;
+    }
+    return bytes;
 }
 
 // terms / group_off are DEVICE arrays (n_out + 1 offsets); y: [n_out][2][nq+K][N]
@@ -1082,8 +1119,9 @@ static bool split_limbs(const hemm_context *c, int nq, int beta, int n_out, Limb
 }
 
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, hipStream_t s) {
+                          bool b_premultiplied, hipStream_t s, const void *terms_host, int n_terms) {
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
+    if (terms_host != nullptr) account(c, TR_KEYPROD, hoisted_bytes(c, (const RotTermDev *)terms_host, n_terms, n_out, nq));
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
     LimbList fpl, il, all;
@@ -1113,6 +1151,7 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
     if (n_terms > HOISTED_ARG_TERMS || n_out > HOISTED_ARG_TERMS) throw std::invalid_argument("term list too long for the argument path");
+    account(c, TR_KEYPROD, hoisted_bytes(c, (const RotTermDev *)terms_host, n_terms, n_out, nq));
     HoistedArgs a;
     memset(&a, 0, sizeof(a));
     memcpy(a.t, terms_host, (size_t)n_terms * sizeof(RotTermDev));
@@ -1183,7 +1222,7 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
         a.dst_slot[j] = (uint8_t)j;
         a.dst_prime[j] = (uint8_t)j;
     }
-    launch_bconv(a, c->d_modq, (int)N, n_polys, s);
+    launch_bconv(c, a, c->d_modq, (int)N, n_polys, s);
     const dim3 block(256);
     const Cst *cst_dev = t->dev + (drop_last ? t->dropinv_off[nq] : t->pinv_off);
     if (launch_ntt_sub_scale(c, conv, nq_out, n_polys, y, (size_t)E * N, out, out_stride, cst_dev, s)) return;
@@ -1191,13 +1230,35 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
     CstList cl;
     for (int j = 0; j < nq_out; j++) cl.c[j] = drop_last ? t->dropinv[nq][j] : t->pinv[j];
     dim3 g2(N / 256, nq_out * n_polys);
+    account(c, TR_POINTWISE, (size_t)3 * n_polys * nq_out * N * 8);
     hipLaunchKernelGGL(sub_scale_kernel, g2, block, 0, s, y, (size_t)E * N, conv, (size_t)nq_out * N,
                        (const u64 *)nullptr, (size_t)0, 0, out, out_stride, c->d_modq, cl, nq_out, c->logN);
 }
 
+
+// Algorithmic bytes of a masked sum: distinct ciphertexts and masks once, outputs once.
+static size_t masked_bytes(const hemm_context *c, const LinTermDev *t, int n_terms, int n_out, int nq, int n_polys) {
+    const size_t limb = (size_t)c->N * 8;
+    std::vector<const u64 *> seen;
+    auto first = [&](const u64 *p) {
+        if (p == nullptr) return false;
+        for (const u64 *q : seen)
+            if (q == p) return false;
+        seen.push_back(p);
+        return true;
+    };
+    size_t bytes = (size_t)n_out * n_polys * nq * limb;
+    for (int i = 0; i < n_terms; i++) {
+        if (first(t[i].ct)) bytes += (size_t)n_polys * nq * limb;
+        if (first(t[i].mask)) bytes += (size_t)nq * limb;
+    }
+    return bytes;
+}
+
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
-                       u64 *out, hipStream_t s) {
+                       u64 *out, hipStream_t s, const void *terms_host, int n_terms) {
     if (n_polys > 3) throw std::invalid_argument("masked sums take at most 3 polynomials");
+    if (terms_host != nullptr) account(c, TR_MASKED, masked_bytes(c, (const LinTermDev *)terms_host, n_terms, n_out, nq, n_polys));
     if (c->N < 512) throw std::invalid_argument("masked sums need N >= 512");
     dim3 grid((unsigned)(c->N / 512) * nq * n_out), block(256);
     const LinTermDev *td = (const LinTermDev *)terms_dev;
@@ -1272,6 +1333,7 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(const u64 *__restrict__ 
 void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s) {
     const int E = nq + c->nP;
     const size_t pairs = (size_t)n_out * 2 * E * (c->N / 2);
+    account(c, TR_KEYPROD, (size_t)(parts + 1) * n_out * 2 * (nq + c->nP) * c->N * 8);
     hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s, part, parts, y, c->d_modq,
                        limbs_default(c, nq, 1), E, c->logN, pairs);
 }
@@ -1283,6 +1345,7 @@ void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms
     if (c->N < 512) throw std::invalid_argument("masked sums need N >= 512");
     if (n_terms > MASKED_ARG_TERMS || n_out > MASKED_ARG_TERMS)
         throw std::invalid_argument("term list too long for the argument path");
+    account(c, TR_MASKED, masked_bytes(c, (const LinTermDev *)terms_host, n_terms, n_out, nq, n_polys));
     MaskedArgs a;
     memset(&a, 0, sizeof(a));
     memcpy(a.t, terms_host, (size_t)n_terms * sizeof(LinTermDev));
@@ -1299,6 +1362,7 @@ void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
                          bool accumulate, hipStream_t s) {
     dim3 grid(c->N / 256, nq), block(256);
+    account(c, TR_TENSOR, (size_t)(4 * G + (accumulate ? 6 : 3)) * nq * c->N * 8);
     hipLaunchKernelGGL(tensor_batch_kernel, grid, block, 0, s, t1, t2, G, acc3, acc_stride, accumulate ? 1 : 0, c->d_modq,
                        nq, c->logN);
 }

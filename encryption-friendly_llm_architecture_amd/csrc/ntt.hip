@@ -479,6 +479,7 @@ static int polys_per_run(int n_limbs, int n_polys, bool inverse) {
 bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
                           size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s) {
     if (c->logN != 16) return false;
+    account(c, TR_NTT, (size_t)3 * n_limbs * n_polys * c->N * 8, 2);   // limbs in, minuend in, result out
     LimbList ll, sl;
     for (int j = 0; j < HEMM_MAX_PRIMES; j++) ll.idx[j] = sl.idx[j] = (uint8_t)j;
     const Tw *tw = (const Tw *)c->d_w;
@@ -503,6 +504,7 @@ bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_str
                       const void *final_scale) {
     if (c->logN != 16) return false;
     if (n_limbs <= 0 || n_polys <= 0) return true;
+    account(c, TR_NTT, (size_t)2 * n_limbs * n_polys * c->N * 8, 2);
     const Tw *tw = (const Tw *)c->d_iw;
     const dim3 block(256);
     const int run = polys_per_run(n_limbs, n_polys, true);
@@ -526,6 +528,7 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
     if (n_limbs <= 0 || n_polys <= 0) return;
     if (final_scale != nullptr && (!inverse || c->logN != 16))
         throw std::invalid_argument("a final constant is taken by the inverse transform of N = 2^16 only");
+    account(c, TR_NTT, (size_t)2 * n_limbs * n_polys * c->N * 8, c->logN > 12 ? 2 : 1);
     const Tw *tw = (const Tw *)(inverse ? c->d_iw : c->d_w);
     const int lanes = n_limbs * n_polys;
     if (c->logN == 16) {

@@ -114,6 +114,7 @@ void launch_binary(const hemm_context *c, int op, const u64 *a, size_t a_stride,
                    u64 *out, size_t out_stride, const LimbList &ll, int n_limbs, int n_polys, hipStream_t s) {
     dim3 grid(c->N / 512, n_limbs * n_polys), block(256);
     Operand A{a, a_stride}, B{b, b_stride};
+    account(c, TR_POINTWISE, (size_t)(op == OP_NEG ? 2 : op == OP_MAC ? 4 : 3) * n_limbs * n_polys * c->N * 8);
     switch (op) {
         case OP_ADD: hipLaunchKernelGGL(binary_kernel<OP_ADD>, grid, block, 0, s, A, B, out, out_stride, c->d_modq, ll, n_limbs, c->logN); break;
         case OP_SUB: hipLaunchKernelGGL(binary_kernel<OP_SUB>, grid, block, 0, s, A, B, out, out_stride, c->d_modq, ll, n_limbs, c->logN); break;
@@ -137,6 +138,7 @@ void launch_mul_scalar(const hemm_context *c, const u64 *a, size_t a_stride, con
     }
     dim3 grid(c->N / 512, n_limbs * n_polys), block(256);
     Operand A{a, a_stride};
+    account(c, TR_POINTWISE, (size_t)2 * n_limbs * n_polys * c->N * 8);
     hipLaunchKernelGGL(scalar_kernel<false>, grid, block, 0, s, A, out, out_stride, c->d_modq, ll, sc, n_limbs, c->logN);
 }
 
@@ -150,6 +152,7 @@ void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *
     }
     dim3 grid(c->N / 512, n_limbs * n_polys), block(256);
     Operand A{a, a_stride};
+    account(c, TR_POINTWISE, (size_t)2 * n_limbs * n_polys * c->N * 8);
     hipLaunchKernelGGL(scalar_kernel<true>, grid, block, 0, s, A, out, out_stride, c->d_modq, ll, sc, n_limbs, c->logN);
 }
 
@@ -157,6 +160,7 @@ void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c
                    size_t out_stride, int nq, bool accumulate, hipStream_t s) {
     dim3 grid(c->N / 256, nq), block(256);
     Operand A{c1, s1}, B{c2, s2};
+    account(c, TR_TENSOR, (size_t)(accumulate ? 10 : 7) * nq * c->N * 8);
     if (accumulate)
         hipLaunchKernelGGL(tensor_kernel<true>, grid, block, 0, s, A, B, out, out_stride, c->d_modq, c->logN);
     else
@@ -167,5 +171,6 @@ void launch_galois(const hemm_context *c, const u64 *a, size_t a_stride, u64 *ou
                    int n_limbs, int n_polys, hipStream_t s) {
     dim3 grid(c->N / 256, n_limbs * n_polys), block(256);
     Operand A{a, a_stride};
+    account(c, TR_POINTWISE, (size_t)2 * n_limbs * n_polys * c->N * 8);
     hipLaunchKernelGGL(galois_kernel, grid, block, 0, s, A, out, out_stride, (u32)g, n_limbs, c->logN);
 }

@@ -29,6 +29,7 @@ def _L():
         L.hellm_ensure_rotation_keys.argtypes = [vp, u64p, u32]
         L.hellm_set_schedule.argtypes = [vp, ctypes.c_int, u32]
         L.hellm_assume_single_tile.argtypes = [vp, ctypes.c_int]
+        L.hellm_traffic.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ctypes.c_int]
         L.hellm_encrypt.argtypes = [vp, f64p, u32, u32, pvp]
         L.hellm_encrypt2.argtypes = [vp, f64p, f64p, u32, u32, pvp]
         L.hellm_encode.argtypes = [vp, f64p, u32, u32, u32, pvp]
@@ -209,6 +210,16 @@ class HEMMer:
 
     def sync(self):
         check(_L().hellm_sync())
+
+    TRAFFIC_KINDS = ("transforms", "key_products", "basis_conversions", "tensor_accumulation", "masked_sums", "pointwise")
+
+    def traffic(self, reset=False):
+        """Algorithmic bytes and launch counts queued on the device context since the last reset, by kind of work."""
+        b = (ctypes.c_uint64 * 8)()
+        n = (ctypes.c_uint64 * 8)()
+        check(_L().hellm_traffic(self.h, b, n, int(reset)))
+        return ({k: int(b[i]) for i, k in enumerate(self.TRAFFIC_KINDS)},
+                {k: int(n[i]) for i, k in enumerate(self.TRAFFIC_KINDS)})
 
     def secret_coeffs(self):
         out = np.empty(self.N, dtype=np.int32)

@@ -33,6 +33,8 @@ int hellm_secret_coeffs(hellm_hemmer *h, int32_t *out /* N */);
 int hellm_export_key(hellm_hemmer *h, uint64_t galois, uint64_t *out);
 int hellm_ensure_rotation_keys(hellm_hemmer *h, const uint64_t *left_rotations, uint32_t count);
 int hellm_sync(void); /* CudaTools::cudaDeviceSynchronize */
+/* hemm_traffic of the device context under this HEMMer (arrays of 8 entries, see hemm.h); no counterpart in HEMMer */
+int hellm_traffic(hellm_hemmer *h, uint64_t *bytes, uint64_t *launches, int reset);
 /* schedule of the products: fused != 0 (default) = batched launches with hoisted rotations,
  * 0 = one evaluator call per step in the reference's order; batch = shifts per launch */
 int hellm_set_schedule(hellm_hemmer *h, int fused, uint32_t batch);

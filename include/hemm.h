@@ -137,6 +137,14 @@ typedef struct {
     uint32_t pt_galois;   /* odd, < 2N; 1 = as stored */
     uint32_t reserved;    /* 0 */
 } hemm_rot_term;
+/* Algorithmic bytes of everything queued on this context since the last reset, by kind of work (for each launch: the
+ * operands it must read once plus the results it must write once; a two-launch 2^16-point transform counts one read
+ * and one write per limb), and the number of launches; counted on the host, costs nothing on the device.  Kinds:
+ * 0 transforms, 1 key products (inner products, hoisted sums), 2 basis conversions, 3 tensor products and their
+ * accumulation, 4 masked sums, 5 other pointwise work and copies; entries 6, 7 are 0.  Either array may be NULL.
+ * No counterpart in HEaaN's interface: it is the per-kernel byte breakdown a roofline report needs. */
+#define HEMM_TRAFFIC_KINDS 8
+int hemm_traffic(hemm_context *ctx, uint64_t *bytes, uint64_t *launches, int reset);
 /* sizeof(hemm_rot_term) and sizeof(hemm_lin_term) as this library was built: a binding checks its own record layouts
  * against them before it passes term lists. */
 void hemm_abi_sizes(uint32_t *rot_term_bytes, uint32_t *lin_term_bytes);
