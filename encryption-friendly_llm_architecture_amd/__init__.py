@@ -58,6 +58,8 @@ def _declare(L):
     sz, u32, u64, ci = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int
     L.hemm_pointwise.argtypes = [vp, ci, vp, sz, vp, sz, vp, sz, u32, ci, u32, vp]
     L.hemm_mul_scalar.argtypes = [vp, vp, sz, u64p, vp, sz, u32, ci, u32, vp]
+    L.hemm_encode.argtypes = [vp, vp, ctypes.c_double, u32, ci, u32, vp, vp]
+    L.hemm_decode.argtypes = [vp, vp, u32, ctypes.c_double, vp, vp, vp]
     L.hemm_mul_imag_unit.argtypes = [vp, vp, sz, vp, sz, u32, u32, vp]
     L.hemm_tensor.argtypes = [vp, vp, sz, vp, sz, vp, sz, u32, ci, vp]
     L.hemm_automorphism.argtypes = [vp, vp, sz, vp, sz, u64, u32, u32, vp]
@@ -138,6 +140,25 @@ class Context:
                              vp(stream or 0)))
         return data
 
+
+    def encode(self, slots, scale, nq, with_p=False):
+        """slots: complex128 CUDA tensor [n_msgs][N/2] (or [N/2]) -> int64 [n_msgs][nq (+ n_p)][N] (NTT form)."""
+        import torch
+        z = slots.reshape(-1, self.N // 2).clone().contiguous()
+        limbs = nq + (self.nP if with_p else 0)
+        out = torch.empty((z.shape[0], limbs, self.N), dtype=torch.int64, device=z.device)
+        check(lib().hemm_encode(self.h, vp(z.data_ptr()), ctypes.c_double(scale), nq, int(with_p), z.shape[0],
+                                vp(out.data_ptr()), vp(0)))
+        return out
+
+    def decode(self, pt, scale, n_limbs=2):
+        """pt: int64 CUDA tensor [>= n_limbs][N] (NTT form) -> complex128 CUDA tensor [N/2]."""
+        import torch
+        ws = torch.empty((n_limbs, self.N), dtype=torch.int64, device=pt.device)
+        z = torch.empty(self.N // 2, dtype=torch.complex128, device=pt.device)
+        check(lib().hemm_decode(self.h, vp(pt.data_ptr()), n_limbs, ctypes.c_double(scale), vp(ws.data_ptr()),
+                                vp(z.data_ptr()), vp(0)))
+        return z
 
     # ---- evaluator-level kernels on [polys][limbs][N] int64 CUDA tensors ---------------------
     def _new(self, polys, limbs, like):

@@ -48,6 +48,7 @@ int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64
         hemm_static_setup(c);   // constant tables and the address of the static scratch: hemm_rescale_static allocates nothing
     } catch (...) {
         hemm_keyswitch_tables_free(c);
+        hemm_embedding_tables_free(c);
         hemm_context_free(c);
         throw;
     }
@@ -55,7 +56,10 @@ int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64
     HEMM_CATCH
 }
 void hemm_context_destroy(hemm_context *ctx) {
-    if (ctx) hemm_keyswitch_tables_free(ctx);
+    if (ctx) {
+        hemm_keyswitch_tables_free(ctx);
+        hemm_embedding_tables_free(ctx);
+    }
     hemm_context_free(ctx);
 }
 uint64_t hemm_context_psi(const hemm_context *ctx, uint32_t idx) { return ctx->psi.at(idx); }
@@ -181,6 +185,41 @@ int hemm_mul_scalar(hemm_context *ctx, const uint64_t *a, size_t a_stride, const
     need(a && out && scalars, "null operand");
     launch_mul_scalar(ctx, (const u64 *)a, a_stride, (const u64 *)scalars, (u64 *)out, out_stride, ll, nl,
                       (int)n_polys, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_encode(hemm_context *ctx, double *slots, double scale, uint32_t nq, int with_p, uint32_t n_msgs, uint64_t *out,
+                void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
+    need(slots && out && n_msgs >= 1, "null operand");
+    need(scale > 0, "scale must be positive");
+    launch_encode(ctx, slots, scale, ll, nl, (int)n_msgs, (u64 *)out, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_decode(hemm_context *ctx, const uint64_t *pt, uint32_t n_limbs, double scale, uint64_t *workspace, double *slots,
+                void *stream) {
+    HEMM_TRY
+    need(pt && workspace && slots, "null operand");
+    need(n_limbs >= 1 && n_limbs <= 2 && (int)n_limbs <= ctx->nQ, "decode reads one or two limbs");
+    need(scale > 0, "scale must be positive");
+    launch_decode(ctx, (const u64 *)pt, (int)n_limbs, scale, (u64 *)workspace, slots, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_add_scalar(hemm_context *ctx, const uint64_t *a, const uint64_t *re, const uint64_t *im, uint64_t *out,
+                    uint32_t nq, int with_p, void *stream) {
+    HEMM_TRY
+    int nl;
+    LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
+    need(a && out && re, "null operand");
+    need(ctx->N >= 512, "needs N >= 512");
+    launch_add_scalar(ctx, (const u64 *)a, (const u64 *)re, (const u64 *)im, (u64 *)out, ll, nl, (hipStream_t)stream);
     check_launch();
     HEMM_CATCH
 }

@@ -88,6 +88,12 @@ void launch_binary(const hemm_context *c, int op, const u64 *a, size_t a_stride,
                    u64 *out, size_t out_stride, const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
 void launch_mul_scalar(const hemm_context *c, const u64 *a, size_t a_stride, const u64 *scalars, u64 *out,
                        size_t out_stride, const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
+void launch_add_scalar(const hemm_context *c, const u64 *a, const u64 *re, const u64 *im, u64 *out, const LimbList &ll,
+                       int n_limbs, hipStream_t s);
+void launch_encode(const hemm_context *c, double *slots, double scale, const LimbList &ll, int n_limbs, int n_msgs, u64 *out,
+                   hipStream_t s);
+void launch_decode(const hemm_context *c, const u64 *pt, int n_limbs, double scale, u64 *work, double *slots, hipStream_t s);
+void hemm_embedding_tables_free(const hemm_context *c);
 void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride,
                      const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
 void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c2, size_t s2, u64 *out,

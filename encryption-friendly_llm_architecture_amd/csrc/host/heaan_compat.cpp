@@ -122,11 +122,9 @@ Context makeContextCustom(u64 log_degree, const std::vector<u64> &chain, const s
     }
     c->ksi_re.resize(M + 1);
     c->ksi_im.resize(M + 1);
-    for (u64 k = 0; k <= M; k++) {
-        double ang = 2.0 * M_PI * (double)k / (double)M;
-        c->ksi_re[k] = cos(ang);
-        c->ksi_im[k] = sin(ang);
-    }
+    // separate loops: a cos / sin pair on one value may be merged into one sincos call, which rounds differently
+    for (u64 k = 0; k <= M; k++) c->ksi_re[k] = cos(2.0 * M_PI * (double)k / (double)M);
+    for (u64 k = 0; k <= M; k++) c->ksi_im[k] = sin(2.0 * M_PI * (double)k / (double)M);
     return c;
 }
 
@@ -585,6 +583,24 @@ static Plaintext encode_impl(const Context &c, const Message &msg, u64 level, u6
     if (rescale_counter != 0) throw RuntimeException("encode: only rescale counter 0 is supported");
     const size_t n = c->N / 2, M = 2 * c->N;
     if (msg.getSize() != n) throw RuntimeException("encode: message must fill all N/2 slots");
+    if (c->N >= 512) {
+        // on the device: the same butterflies in the same order (one IEEE operation per step), so the same residues
+        // as the host loop below
+        static_assert(sizeof(Complex) == 16, "a message is an array of (re, im) doubles");
+        const double scale = scale_override != 0 ? scale_override : c->delta[level];
+        Plaintext pt(c);
+        pt.allocate(level, 0);
+        const size_t limbs = level + 1 + (extended ? c->nP : 0);
+        if (extended) pt.buf_.resize(c, limbs * c->N);
+        DeviceBuffer z(c, c->N);
+        hip_ck(hipMemcpy(z.data(), &msg[0], n * sizeof(Complex), hipMemcpyHostToDevice), "hipMemcpy");
+        ck(hemm_encode(c->dev, (double *)z.data(), scale, (uint32_t)level + 1, extended ? 1 : 0, 1, pt.buf_.data(), nullptr));
+        size_t occupied = n;
+        while (occupied > 0 && msg[occupied - 1] == Complex(0, 0)) occupied--;
+        pt.occupied_ = occupied;
+        if (scale_override != 0) pt.scale_ = scale_override;
+        return pt;
+    }
     std::vector<double> re(n), im(n);
     for (size_t i = 0; i < n; i++) {
         re[i] = msg[i].real();
@@ -641,6 +657,18 @@ Message EnDecoder::decode(const Plaintext &pt) const {
     const Context &c = ctx_;
     const size_t N = c->N, n = N / 2, M = 2 * N;
     const u64 two = pt.level_ >= 1 ? 1 : 0;
+    if (N >= 512) {
+        double scale = pt.scale_;
+        if (scale == 0) {
+            scale = c->delta[pt.level_];
+            for (u64 k = 0; k < pt.rescale_counter_; k++) scale *= c->delta[pt.level_];
+        }
+        DeviceBuffer work(c, (two + 1) * N), z(c, N);
+        ck(hemm_decode(c->dev, pt.buf_.data(), (uint32_t)(two + 1), scale, work.data(), (double *)z.data(), nullptr));
+        Message m(c->logN - 1);
+        hip_ck(hipMemcpy(&m[0], z.data(), n * sizeof(Complex), hipMemcpyDeviceToHost), "hipMemcpy");
+        return m;
+    }
     DeviceBuffer tmp(c, (two + 1) * N);
     hip_ck(hipMemcpyAsync(tmp.data(), pt.buf_.data(), (two + 1) * N * 8, hipMemcpyDeviceToDevice, nullptr), "memcpy");
     ck(hemm_ntt(c->dev, tmp.data(), chain_primes(two + 1).data(), (uint32_t)(two + 1), 1, 1, nullptr));

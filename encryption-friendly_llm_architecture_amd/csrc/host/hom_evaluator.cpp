@@ -137,8 +137,24 @@ void HomEvaluator::add(const Ciphertext &a, const Message &b, Ciphertext &out) c
     add(a, EnDecoder(ctx_).encode(b, a.level_), out);
 }
 void HomEvaluator::add(const Ciphertext &a, const Complex &cst, Ciphertext &out) const {
-    Message m(getLogFullSlots(ctx_), cst);
-    add(a, m, out);
+    if (ctx_->N < 512) {
+        Message m(getLogFullSlots(ctx_), cst);
+        add(a, m, out);
+        return;
+    }
+    // a constant in every slot is the polynomial round(re Delta) + round(im Delta) X^(N/2): added to the residues of
+    // the first polynomial directly, no plaintext is encoded
+    const Real delta = ctx_->delta[a.level_];
+    const i64 re = (i64)llround(cst.real() * delta), im = (i64)llround(cst.imag() * delta);
+    const u64 occ = (re != 0 || im != 0) ? (u64)ctx_->N / 2 : a.occupied_;
+    OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
+    Ciphertext &r = o.get();
+    if (r.buf_.data() != a.buf_.data())
+        (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, nullptr);
+    const auto rr = int_residues(ctx_, re, a.level_ + 1), ri = int_residues(ctx_, im, a.level_ + 1);
+    ck(hemm_add_scalar(ctx_->dev, r.buf_.data(), rr.data(), im != 0 ? ri.data() : nullptr, r.buf_.data(),
+                       (uint32_t)a.level_ + 1, 0, nullptr));
+    o.commit(occ);
 }
 void HomEvaluator::sub(const Ciphertext &a, const Message &b, Ciphertext &out) const {
     Message nb(b);

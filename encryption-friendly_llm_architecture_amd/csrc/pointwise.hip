@@ -70,6 +70,22 @@ __global__ __launch_bounds__(256) void scalar_kernel(Operand a, u64 *__restrict_
     *(ulonglong2 *)(out + poly * out_stride + e) = r;
 }
 
+// out = a + re[limb] + im[limb] * (-1)^{bitrev(k) & 1}: the NTT form of the constant polynomial re + im' X^(N/2)
+// (im[limb] = im' psi^(N/2), the sign flips on the upper half of the bit-reversed index range), i.e. a complex
+// constant in every slot, added without encoding a plaintext.
+__global__ __launch_bounds__(256) void scalar_add_kernel(Operand a, u64 *__restrict__ out, size_t out_stride,
+                                                         const ModQ *__restrict__ modq, LimbList ll, ScalarList sc,
+                                                         int n_limbs, int logN) {
+    const int limb = blockIdx.y;
+    const u64 q = modq[ll.idx[limb]].q;
+    const size_t k = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const size_t e = ((size_t)limb << logN) + k;
+    const ulonglong2 x = *(const ulonglong2 *)(a.p + e);
+    const u64 im = (k >> (logN - 1)) ? negmod(sc.ws[limb], q) : sc.ws[limb];
+    const u64 c = addmod(sc.w[limb], im, q);
+    *(ulonglong2 *)(out + e) = make_ulonglong2(addmod(x.x, c, q), addmod(x.y, c, q));
+}
+
 // (b1,a1) x (b2,a2) -> (b1 b2, a1 b2 + a2 b1, a1 a2); ACC adds into out.
 template <bool ACC>
 __global__ __launch_bounds__(256) void tensor_kernel(Operand c1, Operand c2, u64 *__restrict__ out, size_t out_stride,
@@ -154,6 +170,22 @@ void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *
     Operand A{a, a_stride};
     account(c, TR_POINTWISE, (size_t)2 * n_limbs * n_polys * c->N * 8);
     hipLaunchKernelGGL(scalar_kernel<true>, grid, block, 0, s, A, out, out_stride, c->d_modq, ll, sc, n_limbs, c->logN);
+}
+
+// re / im: one residue per limb (im may be nullptr); one polynomial
+void launch_add_scalar(const hemm_context *c, const u64 *a, const u64 *re, const u64 *im, u64 *out, const LimbList &ll,
+                       int n_limbs, hipStream_t s) {
+    ScalarList sc;
+    for (int j = 0; j < n_limbs; j++) {
+        const u64 q = c->primes[ll.idx[j]];
+        sc.w[j] = re[j] % q;
+        // im' X^(N/2) evaluates to im' psi^(N/2) (2 bitrev(k) + 1 odd): the kernel flips its sign by slot
+        sc.ws[j] = im ? h_mulmod(im[j] % q, h_powmod(c->psi[ll.idx[j]], (u64)c->N / 2, q), q) : 0;
+    }
+    dim3 grid(c->N / 512, n_limbs), block(256);
+    Operand A{a, 0};
+    account(c, TR_POINTWISE, (size_t)2 * n_limbs * c->N * 8);
+    hipLaunchKernelGGL(scalar_add_kernel, grid, block, 0, s, A, out, (size_t)0, c->d_modq, ll, sc, n_limbs, c->logN);
 }
 
 void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c2, size_t s2, u64 *out,

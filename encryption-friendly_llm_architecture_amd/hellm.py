@@ -165,6 +165,30 @@ class CtVec(_Handle):
         return Ct(self.owner, h)
 
 
+def chebyshev_product_basis(coeffs, baby_steps):
+    """Plain Chebyshev series (coeffs[k] multiplies T_k) -> the coefficient table HEaaN::Math::ChebyshevCoefficients
+    holds for `baby_steps` baby steps (a power of two): entry bs * i + j multiplies T_j * prod_k T_{2^k bs}^{bit k of i}.
+    Uses T_k = 2 T_m T_{k-m} - T_{2m-k} (m < k < 2m) from the top giant step down, so numpy's fits can be fed to
+    eval_chebyshev the way the reference's Remez tables are."""
+    bs = int(baby_steps)
+    assert bs >= 1 and bs & (bs - 1) == 0, "baby_steps must be a power of two"
+    c = [float(x) for x in coeffs]
+    size = bs
+    while size < len(c):
+        size *= 2
+    c += [0.0] * (size - len(c))
+
+    def split(c):
+        if len(c) == bs:
+            return c
+        m = len(c) // 2
+        low = [c[0]] + [c[j] - c[2 * m - j] for j in range(1, m)]
+        high = [c[m]] + [2.0 * c[m + j] for j in range(1, m)]
+        return split(low) + split(high)
+
+    return split(c)
+
+
 class HEMMer:
     """HELLM::HEMMer on the GPU.  preset=True builds the FGb-sized context (N = 2^16)."""
 

@@ -78,6 +78,23 @@ int hemm_pointwise(hemm_context *ctx, int op, const uint64_t *a, size_t a_stride
 int hemm_mul_scalar(hemm_context *ctx, const uint64_t *a, size_t a_stride, const uint64_t *scalars,
                     uint64_t *out, size_t out_stride, uint32_t nq, int with_p, uint32_t n_polys,
                     void *stream);
+/* EnDecoder::encode (EnDecoder.hpp:51): n_msgs messages of N/2 complex slots each (device memory, interleaved
+ * re, im doubles, [n_msgs][N/2][2]; CLOBBERED) -> plaintexts out [n_msgs][nq (+ n_p)][N] in NTT form, coefficient
+ * i = round(scale * c_i) for the inverse canonical embedding c of the slots on the orbit zeta^(5^j).  Double precision
+ * with one IEEE operation per step in a fixed order: the same bits as a host loop over the same butterflies. */
+int hemm_encode(hemm_context *ctx, double *slots, double scale, uint32_t nq, int with_p, uint32_t n_msgs, uint64_t *out,
+                void *stream);
+/* EnDecoder::decode (EnDecoder.hpp:66): plaintext pt [>= n_limbs][N] (NTT form, limbs of chain primes 0 .. n_limbs-1,
+ * n_limbs = 1 or 2: the centred value is recovered from that many limbs) -> slots [N/2][2] doubles on the device;
+ * workspace: n_limbs * N words. */
+int hemm_decode(hemm_context *ctx, const uint64_t *pt, uint32_t n_limbs, double scale, uint64_t *workspace, double *slots,
+                void *stream);
+/* HomEvaluator::add(Ciphertext, Complex) :159 / sub :207 without a plaintext: out[j][k] = a[j][k] + re[j] +- im[j] I_j,
+ * the NTT form of the constant polynomial re + im X^(N/2) (a complex constant in every slot; I_j = psi_j^(N/2), the
+ * sign flips on the upper half of the bit-reversed index range).  One polynomial [nq (+ n_p)][N]; re / im hold one
+ * residue per limb on the host, im may be NULL.  N >= 512. */
+int hemm_add_scalar(hemm_context *ctx, const uint64_t *a, const uint64_t *re, const uint64_t *im, uint64_t *out,
+                    uint32_t nq, int with_p, void *stream);
 /* HomEvaluator::multImagUnit :330: multiply by the monomial X^(N/2) in NTT form. */
 int hemm_mul_imag_unit(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out,
                        size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);

@@ -264,11 +264,10 @@ void *orc_create(int logN, int nQ, int nP, const u64 *primes, int dnum) {
     }
     c->ksi_re.resize(M + 1);
     c->ksi_im.resize(M + 1);
-    for (int k = 0; k <= M; k++) {
-        double ang = 2.0 * M_PI * (double)k / (double)M;
-        c->ksi_re[k] = cos(ang);
-        c->ksi_im[k] = sin(ang);
-    }
+    // cos and sin in separate loops: called on one value side by side, an optimising compiler may replace the pair by a
+    // single sincos call, whose results differ from cos / sin in the last bit for a few arguments
+    for (int k = 0; k <= M; k++) c->ksi_re[k] = cos(2.0 * M_PI * (double)k / (double)M);
+    for (int k = 0; k <= M; k++) c->ksi_im[k] = sin(2.0 * M_PI * (double)k / (double)M);
     return c;
 }
 void orc_destroy(void *h) { delete (Ctx *)h; }

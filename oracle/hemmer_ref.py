@@ -220,8 +220,13 @@ class OracleEval:
         return self.o.rescale(Ct(self.o.mult_scalar_residues(x, v), x.scale * self.o.delta[x.level]))
 
     def add_const(self, x, c):
-        import numpy as _np
-        return self.o.add(x, self.o.encode(_np.full(self.o.slots, c, dtype=_np.complex128), x.level))
+        """HomEvaluator::add(ct, Complex): the constant polynomial round(re Delta) + round(im Delta) X^(N/2) added to
+        the first polynomial (what encoding a constant message gives, without the transform)."""
+        from .oracle import Ct
+        if self.o.N < 512:
+            import numpy as _np
+            return self.o.add(x, self.o.encode(_np.full(self.o.slots, c, dtype=_np.complex128), x.level))
+        return Ct(self.o.add_constant_residues(x.data, complex(c), x.level), x.scale)
 
     def mult_imag_unit(self, x):
         return self.o.mult_imag_unit(x)

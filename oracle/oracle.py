@@ -474,6 +474,27 @@ class Oracle:
                                       _p(out[k, i]), i)
         return out
 
+    def add_constant_residues(self, data, c, level):
+        """data [polys][nq][N] + the NTT form of round(re Delta_level) + round(im Delta_level) X^(N/2) on polynomial 0:
+        slot k of limb j gets re + im psi_j^(N/2) (-1)^(bitrev(k) & 1), i.e. the sign flips on the upper half."""
+        def rnd(v):
+            return int(math.floor(abs(v) + 0.5)) * (1 if v >= 0 else -1)      # llround: halves away from zero
+        re, im = rnd(c.real * self.delta[level]), rnd(c.imag * self.delta[level])
+        out = data.copy()
+        nq = out.shape[1]
+        cols = np.empty((nq, self.N), dtype=np.uint64)
+        for j in range(nq):
+            cols[j] = re % int(self.q[j])
+        if im != 0:
+            v = np.empty((nq, self.N), dtype=np.uint64)
+            w = np.empty_like(v)
+            for j in range(nq):
+                v[j] = im % int(self.q[j])
+                self.L.orc_mul_imag_unit(self.h, _p(v[j]), _p(w[j]), j)      # im X^(N/2) in NTT form
+            cols = self._binary(0, cols, w)
+        out[0] = self._binary(0, np.ascontiguousarray(out[0]), cols)
+        return out
+
     def add_residues(self, a, b):
         """Limb-wise a + b of residue arrays [nq][N] over the chain primes 0 .. nq-1."""
         return self._binary(0, a, b)

@@ -97,3 +97,15 @@ def test_mult_rescale_leveldown(orc, z):
     assert np.abs(orc.decrypt(orc.mult_integer(ct, -2)) + 2 * z).max() < 1e-7
     assert np.abs(orc.decrypt(orc.sub(ct, ct))).max() < 1e-7
     assert np.abs(orc.decrypt(orc.negate(ct)) + z).max() < 1e-7
+
+
+@pytest.mark.parametrize("c", [0.37, -1.25, 0.5 - 0.75j, -3.0j])
+def test_constant_added_on_the_residues_equals_an_encoded_constant_message(orc, z, c):
+    """add(ct, constant) without a plaintext: the residues must be those of adding the encoding of the message that
+    holds the constant in every slot (the embedding of a constant is re Delta + im Delta X^(N/2)), and the
+    ciphertext must decrypt to z + c."""
+    ct = orc.encrypt(orc.encode(z, orc.nQ - 1), 21)
+    direct = orc.add_constant_residues(ct.data, complex(c), ct.level)
+    via_message = orc.add(ct, orc.encode(np.full(orc.slots, c, dtype=np.complex128), ct.level))
+    assert np.array_equal(direct, via_message.data)
+    assert np.abs(orc.decrypt(O.Ct(direct, ct.scale)) - (z + c)).max() < 1e-6
