@@ -466,7 +466,7 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
         // A single tile with a level to spare goes through the complex-packed product: adjacent columns of A and
         // adjacent rows of B are fused into complex slots (one level), the product then needs n / 2 column shifts
         // (each a key product and a ModDown) instead of n, and x + conj(x) returns the real product.
-        if ((block == slots || (single && block < slots)) && n >= 4 && a.getHeight() == n && a.getWidth() == n &&
+        if (block <= slots && slots % block == 0 && n >= 4 && a.getHeight() == n && a.getWidth() == n &&
             b.getHeight() == n && b.getWidth() == n &&
             std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
             b.get().getRescaleCounter() == 0) {
@@ -475,13 +475,15 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
             std::vector<u64> sq;
-            ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, block < slots));
+            // stacked tiles / unknown content keep their per-block products: the packed cells then shift through
+            // masked pairs (no baby-step / giant-step split, which needs exact row rotations)
+            const bool spread = single && block < slots;
+            ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, spread));
             KeyGenerator kg(context_, sk_, pack_);
             for (u64 r : sq) kg.genLeftRotSquareKey(r);
-            CtxtTensor prod =
-                multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, block < slots);
+            CtxtTensor prod = multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, spread);
             CtxtTensor res = repackCC(prod);
-            if (block < slots) res.get().occupied_ = block;
+            if (spread) res.get().occupied_ = block;
             return res;
         }
         std::vector<u64> square_rots;

@@ -190,7 +190,7 @@ std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, boo
     auto left = [&](i64 v) { r.push_back((u64)(((v % slots) + slots) % slots)); };
     const i64 stride = packed ? 2 : 1, count = packed ? n / 2 : n;
     left(-n);
-    if (need_rows && !packed) left(-n * w);
+    if (need_rows) left(-n * w);
     for (i64 i = 1; i < count; i++) {
         left(stride * i);
         if (need_rows) left(stride * i * w);
@@ -996,14 +996,16 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
-    if (packed)
-        throw std::invalid_argument("[multPackedMatMat] the row shift must be cyclic: rows * block width == slots");
+    // Row shifts that wrap inside a tile block (stacked tiles, or content that is not known to be a single tile):
+    // every shift of tau(B) is a masked pair like the column shifts of sigma(A).  Complex-packed operands shift by
+    // cells of two columns / two rows, so they need half as many.
     std::vector<Plaintext> &rm = tr.getRowMaskExt(eval, shape_b, T + 2);
     std::vector<Shift> sa, sb;
-    for (i64 i = 1; i < n; i++) {
-        sa.push_back(Shift{i, &cm[(size_t)(2 * i + 1)], &cm[(size_t)(2 * i)]});
-        sb.push_back(Shift{i * w, &rm[(size_t)(2 * i + 1)], &rm[(size_t)(2 * i)]});
+    for (i64 i = 1; i < n / cu; i++) {
+        sa.push_back(Shift{cu * i, &cm[(size_t)(2 * cu * i + 1)], &cm[(size_t)(2 * cu * i)]});
+        sb.push_back(Shift{cu * i * w, &rm[(size_t)(2 * cu * i + 1)], &rm[(size_t)(2 * cu * i)]});
     }
+    G = std::max<u64>(1, std::min<u64>(batch, (u64)sa.size()));
     // rotation sources: sigma(A), tau(B) and their copies rotated by -n columns / -n rows
     const Sources x = extendSources(c, ab.data(), 2, nq);
     const i64 back[2] = {-n, -n * w};

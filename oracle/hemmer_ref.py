@@ -847,6 +847,18 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False):
         # the unpacked product; tau(B) is lowered to T+1 with sigma(A)'s copy for the unshifted term
         a = lower_and_transform_fused(orc, orc.level_down(a, min(lvl, T + 4)), PH, n, w, T + 2)
         b = lower_and_transform_fused(orc, orc.level_down(b, min(lvl, T + 4)), PV, n, w, T + 2)
+        if n * w != orc.slots and not spread:
+            # row shifts wrap inside a tile block (stacked tiles, content not known to be a single tile): every shift
+            # of tau(B) by a cell of two rows is a masked pair like the column shifts of sigma(A), n / 2 - 1 of each
+            acc = orc.tensor(orc.level_down_one(a), orc.level_down_one(b))
+            rm = [orc.encode_ext(m, T + 2) for m in row_masks(n, w, orc.slots)]
+            ta = _assemble_shifts(orc, a, orc.modup(a.data[1]), -n,
+                                  [(2 * i, cm[4 * i + 1], cm[4 * i]) for i in range(1, n // 2)])
+            tb = _assemble_shifts(orc, b, orc.modup(b.data[1]), -n * w,
+                                  [(2 * i * w, rm[4 * i + 1], rm[4 * i]) for i in range(1, n // 2)])
+            for x, y in zip(ta, tb):
+                acc = orc.add(acc, orc.tensor(x, y))
+            return orc.rescale(orc.relinearize(acc))
         b = orc.level_down_one(b)
     else:
         a = lower_and_transform_fused(orc, a, PH, n, w, T + 2)
@@ -886,6 +898,19 @@ def complex_packing_hoisted(orc, x, w, rows):
     y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, lvl, ms)) for r, m in terms], nq)
     zero.scale = orc.delta[lvl - 1]
     return orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
+
+
+def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
+    """mult_mat_mat_cc_packed_single for operands that may hold stacked tiles (single_tile = False): the packing and
+    the transforms act on every tile block alike, the cells shift through masked pairs, and each block of the result
+    is the product of the operands' blocks."""
+    from .oracle import Ct
+    ev = OracleEval(orc)
+    lvl = min(a.level, b.level, T + 5)
+    cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
+    pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
+    pb = complex_packing_hoisted(orc, cut(b), w, rows=True)
+    return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile))
 
 
 def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):

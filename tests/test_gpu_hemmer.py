@@ -197,17 +197,27 @@ def test_ccmm_stacked_tiles_keep_block_products(small):
     H.set_schedule(True, batch=5)
     c = H.single_cc_matmul(ca, cb, 2)
     H.set_schedule(True)
-    want = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16)
+    # four levels to spare: the complex-packed product with masked shifts of its two-column / two-row cells
+    want = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ca), to_oracle(orc, cb), 2, 16, 16, single_tile=False)
     assert np.array_equal(c.residues(), want.data)
     d = H.decrypt_slots(c).real[:512].reshape(32, 16)
+    assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -18
+    assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -18
+    # three levels to spare: the unpacked product with masked row shifts
+    la, lb = H.level_down(ca, 5), H.level_down(cb, 5)
+    c1 = H.single_cc_matmul(la, lb, 2)
+    want1 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16)
+    assert np.array_equal(c1.residues(), want1.data)
+    d = H.decrypt_slots(c1).real[:512].reshape(32, 16)
     assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -20
     assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -20
     # a rotation forgets what was known about a single tile: the masked route again
     ra = H.left_rotate(H.left_rotate(H.encrypt(A[:16]), 3), 512 - 3)
-    c2 = H.single_cc_matmul(ra, H.encrypt(B[:16]), 2)
-    want2 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, ra), to_oracle(orc, H.encrypt(B[:16])), 2, 16, 16)
+    eb16 = H.encrypt(B[:16])
+    c2 = H.single_cc_matmul(ra, eb16, 2)
+    want2 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ra), to_oracle(orc, eb16), 2, 16, 16, single_tile=False)
+    assert np.array_equal(c2.residues(), want2.data)
     assert np.abs(H.decrypt(c2) - A[:16] @ B[:16]).max() < 2 ** -18
-    assert c2.info()["level"] == want2.level
 
 
 @pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
