@@ -21,7 +21,15 @@ namespace HELLM {
 
 // DiagonalSigned: the transpose's diagonals grouped the way sigma / tau group theirs (positive and negative diagonals in
 // separate giant-step groups), which is what the batched transform walks; Diagonal keeps the reference's grouping.
-enum class MaskKind { Horizontal, Vertical, PackedHorizontal, PackedVertical, Diagonal, DiagonalSigned };
+enum class MaskKind {
+    Horizontal, Vertical, PackedHorizontal, PackedVertical, Diagonal, DiagonalSigned,
+    // the complex packing followed by the packed transform as ONE linear map (one level instead of two): diagonal r of
+    // the composite collects mask_d (.) rho^(2 d unit)(M_e) over 2 d + e = r, e in {0, +1, -1} the packing's three terms
+    PackingHorizontal, PackingVertical
+};
+// The complex packing as a linear map on the slots, out = Z x + M_+ rho^(step)(x) + M_- rho^(-step)(x) (step 1 for
+// columns, the block width for rows): part 0 = Z, 1 = M_+, 2 = M_-.
+Message packingMaskMessage(bool by_rows, i64 block_width, u64 log_slots, int part);
 
 // 0/1 (or 0.5) slot pattern of diagonal `idx` for a transform kind, before any pre-rotation.
 // Horizontal (sigma): rows r with r mod n == idx take columns [0, n - idx); negative idx = the wrapped

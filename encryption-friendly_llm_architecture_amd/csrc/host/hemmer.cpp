@@ -468,7 +468,7 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
         // (each a key product and a ModDown) instead of n, and x + conj(x) returns the real product.
         if (block <= slots && slots % block == 0 && n >= 4 && a.getHeight() == n && a.getWidth() == n &&
             b.getHeight() == n && b.getWidth() == n &&
-            std::min(a.getLevel(), b.getLevel()) >= T + 4 && a.get().getRescaleCounter() == 0 &&
+            std::min(a.getLevel(), b.getLevel()) >= T + 3 && a.get().getRescaleCounter() == 0 &&
             b.get().getRescaleCounter() == 0) {
             // both packings through one launch chain, at level T+5 (the transforms start from T+4)
             ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});

@@ -34,6 +34,7 @@ Geometry geometry(MaskKind kind, const TileTensorShape &s) {
     Geometry g{};
     const i64 rows = s.getNumRows(), cols = s.getNumCols(), w = s.getBlockWidth();
     const bool plain_sigma_tau = (kind == MaskKind::Horizontal || kind == MaskKind::Vertical);
+    const bool packing = (kind == MaskKind::PackingHorizontal || kind == MaskKind::PackingVertical);
     if (rows != cols && !plain_sigma_tau)
         throw std::invalid_argument("[MatrixTransformer] packed transforms and transpose need square tiles");
     g.n = rows;
@@ -50,7 +51,8 @@ Geometry geometry(MaskKind kind, const TileTensorShape &s) {
         return g;
     }
     const bool packed = (kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical);
-    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
+    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical || kind == MaskKind::PackingVertical);
+    (void)packing;   // the composite kinds move by single columns / rows: the geometry of the plain transforms
     g.cell = packed ? 2 : 1;
     g.units = (vertical ? rows : cols) / g.cell;
     g.sub = std::min(rows, cols) / g.cell;
@@ -62,7 +64,39 @@ Geometry geometry(MaskKind kind, const TileTensorShape &s) {
 
 }  // namespace
 
+Message packingMaskMessage(bool by_rows, i64 w, u64 log_slots, int part) {
+    const u64 slots = u64(1) << log_slots, step = by_rows ? (u64)w : 1;
+    Message m(log_slots, 0);
+    const Complex iu(0, by_rows ? -1.0 : 1.0);
+    for (u64 s = 0; s < slots; s++) {
+        auto even = [&](u64 t) { return by_rows ? ((t / (u64)w) % 2 == 0) : (t % 2 == 0); };
+        const double here = even(s) ? 1.0 : 0.0, prev = even((s + slots - step) % slots) ? 1.0 : 0.0;
+        m[s] = part == 0 ? Complex(here, 0) + iu * prev : part == 1 ? iu * here : Complex(prev, 0);
+    }
+    return m;
+}
+
 Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log_slots, i64 idx) {
+    if (kind == MaskKind::PackingHorizontal || kind == MaskKind::PackingVertical) {
+        // T_packed(P(x)) = sum_d mask_d (.) rho^(2 d unit)(Z x + M_+ rho^unit x + M_- rho^-unit x): the coefficient of
+        // rho^(idx unit)(x) collects the three ways of writing idx = 2 d + e
+        const bool rows = kind == MaskKind::PackingVertical;
+        const MaskKind base = rows ? MaskKind::PackedVertical : MaskKind::PackedHorizontal;
+        const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, unit = rows ? w : 1;
+        const i64 cells = (rows ? shape.getNumRows() : shape.getNumCols()) / 2;
+        Message m(log_slots, 0);
+        const int parts[3] = {0, 1, 2};
+        const i64 shift[3] = {0, 1, -1};
+        for (int k = 0; k < 3; k++) {
+            if (((idx - shift[k]) % 2) != 0) continue;
+            const i64 d = (idx - shift[k]) / 2;
+            if (d <= -cells || d >= cells) continue;
+            const Message t = transformMaskMessage(base, shape, log_slots, d), pm = packingMaskMessage(rows, w, log_slots, parts[k]);
+            const i64 r = ((2 * d * unit) % slots + slots) % slots;
+            for (i64 s = 0; s < slots; s++) m[(u64)s] += t[(u64)s] * pm[(u64)((s + r) % slots)];
+        }
+        return m;
+    }
     const Geometry g = geometry(kind, shape);
     const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, height = slots / w;
     Message m(log_slots, 0);

@@ -54,8 +54,9 @@ Geo geo(MaskKind kind, const TileTensorShape &s) {
     Geo g{};
     const i64 w = s.getBlockWidth(), rows = s.getNumRows(), cols = s.getNumCols();
     const bool packed = (kind == MaskKind::PackedHorizontal || kind == MaskKind::PackedVertical);
-    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical);
-    if (rows != cols && packed) throw std::invalid_argument("[MatrixTransformer] packed transforms need square tiles");
+    const bool vertical = (kind == MaskKind::Vertical || kind == MaskKind::PackedVertical || kind == MaskKind::PackingVertical);
+    const bool packing = (kind == MaskKind::PackingHorizontal || kind == MaskKind::PackingVertical);
+    if (rows != cols && (packed || packing)) throw std::invalid_argument("[MatrixTransformer] packed transforms need square tiles");
     g.n = rows;
     g.cell = packed ? 2 : 1;
     g.units = (vertical ? rows : cols) / g.cell;
@@ -629,7 +630,7 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
                                             const bool *rows, i64 w, u64 *out, const u64 *scale_levels) {
     const Context &c = eval.getContext();
     if (level < 1) throw std::invalid_argument("[complexPacking] level >= 1 is needed.");
-    const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N, slots = N / 2;
+    const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
     const u64 log_slots = getLogFullSlots(c);
     // All three masks of a job are encoded over the extended basis (the unrotated term reads the chain limbs only) at
     // the scale that takes the input's scale to the fixed scale of level - 1 across the rescale.
@@ -637,14 +638,7 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
         const auto key = std::make_tuple((int)by_rows, w, level, part, from);
         auto it = pack_masks_.find(key);
         if (it != pack_masks_.end()) return it->second;
-        const u64 step = by_rows ? (u64)w : 1;
-        Message m(log_slots, 0);
-        const Complex iu(0, by_rows ? -1.0 : 1.0);
-        for (u64 s = 0; s < slots; s++) {
-            auto even = [&](u64 t) { return by_rows ? ((t / (u64)w) % 2 == 0) : (t % 2 == 0); };
-            const double here = even(s) ? 1.0 : 0.0, prev = even((s + slots - step) % slots) ? 1.0 : 0.0;
-            m[s] = part == 0 ? Complex(here, 0) + iu * prev : part == 1 ? iu * here : Complex(prev, 0);
-        }
+        const Message m = packingMaskMessage(by_rows, w, log_slots, part);
         EnDecoder endec(c);
         const Real scale = from == level ? c->delta[level] : c->delta[level - 1] * (Real)c->q[level] / c->delta[from];
         return pack_masks_.emplace(key, endec.encodeExtended(m, level, scale)).first->second;
@@ -893,7 +887,7 @@ void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphert
 namespace {
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre = nullptr,
-                     u64 pre_level = 0);
+                     u64 pre_level = 0, bool merge_packing = false);
 }
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
@@ -904,8 +898,12 @@ namespace {
 // packed: the operands are complex-packed (2 x 2 cells): sigma / tau of the packed kinds, n / 2 shifts of two columns /
 // two rows each; otherwise the same schedule.  pre: both operands already side by side at pre_level (two ciphertexts
 // of two polynomials, the layout the joint transforms read); op1 / op2 then only give the tile shapes.
+// merge_packing (with packed): the operands are NOT packed yet; the complex packing and the packed transform run as one
+// composite one-stage transform from T+3 (MaskKind::PackingHorizontal / PackingVertical), for operands with only
+// three levels above the target.
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
-                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre, u64 pre_level) {
+                     MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre, u64 pre_level,
+                     bool merge_packing) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -934,7 +932,7 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
     // sigma(A) and tau(B) through one launch chain; `ab` holds both results [2 cts][2][nq][N]
     const u64 nq = T + 3, N = c->N, E = nq + c->nP, lo = nq - 1, ctw = 2 * nq * N;
-    const bool two_stage = min_level >= T + 4 && shape_a.getNumRows() == shape_a.getNumCols() &&
+    const bool two_stage = !merge_packing && min_level >= T + 4 && shape_a.getNumRows() == shape_a.getNumCols() &&
                            shape_b.getNumRows() == shape_b.getNumCols();
     const u64 Lt = two_stage ? T + 4 : T + 3;   // level the transforms start from
     DeviceBuffer ab(c, 2 * ctw);
@@ -948,8 +946,12 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
             jointLevelDown(eval, *pa, *pb, Lt, joint.data());
             src = joint.data();
         }
-        const MaskKind kinds[2] = {packed ? MaskKind::PackedHorizontal : MaskKind::Horizontal,
-                                   packed ? MaskKind::PackedVertical : MaskKind::Vertical};
+        const MaskKind kinds[2] = {merge_packing ? MaskKind::PackingHorizontal
+                                   : packed      ? MaskKind::PackedHorizontal
+                                                 : MaskKind::Horizontal,
+                                   merge_packing ? MaskKind::PackingVertical
+                                   : packed      ? MaskKind::PackedVertical
+                                                 : MaskKind::Vertical};
         const TileTensorShape shapes[2] = {shape_a, shape_b};
         if (two_stage)
             tr.diagonalTransformTwoStage(eval, src, 2, Lt, kinds, shapes, ab.data());
@@ -1206,8 +1208,11 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     if (a.get().getRescaleCounter() != 0 || b.get().getRescaleCounter() != 0 || a.get().getNumPoly() != 2 ||
         b.get().getNumPoly() != 2)
         throw std::invalid_argument("[complexPacking] operands must be rescaled.");
-    if (std::min(a.getLevel(), b.getLevel()) < T + 4)
-        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 4) + " is needed.");
+    if (std::min(a.getLevel(), b.getLevel()) < T + 3)
+        throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
+    // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
+    if (std::min(a.getLevel(), b.getLevel()) == T + 3)
+        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true);
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
     // is handed to the product where it lies.  Operands above the packing level are only truncated to it (a copy of
     // their first L+1 limbs): the packing masks absorb the change of scale, which saves the levelDown.

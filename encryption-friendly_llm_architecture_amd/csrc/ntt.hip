@@ -470,6 +470,9 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
 // Measured on 32 x 24 limbs: forward transforms are fastest at 192 limbs per run (60-bit primes 0.52 -> 0.43 ms,
 // primes below 2^44 0.41 -> 0.36 ms), inverse ones at 384 (0.48 -> 0.44 ms, 0.37 -> 0.34 ms).
 static int polys_per_run(int n_limbs, int n_polys, bool inverse) {
+    // batches of up to 448 limbs (224 MiB: what one chain of the matrix products transforms at once, whose input a
+    // producer has just written) are fastest as one run: 480 us for the ModDown of 64 polynomials against 497 us cut
+    if (n_limbs * n_polys <= 448) return n_polys;
     const int limbs = inverse ? 384 : 192;
     int p = limbs / n_limbs;
     if (p < 1) p = 1;

@@ -270,6 +270,8 @@ class OracleEval:
 # --------------------------------------------------------------------------------------------
 H, V, PH, PV, DIAG = "horizontal", "vertical", "packed_horizontal", "packed_vertical", "diagonal"
 DIAG_SIGNED = "diagonal_signed"   # the transpose's diagonals in the grouping of sigma / tau (batched transform)
+# the complex packing followed by the packed transform as ONE linear map (one level instead of two)
+PKH, PKV = "packing_horizontal", "packing_vertica"
 
 
 def _dims(n):
@@ -290,12 +292,12 @@ def geometry(kind, n, w):
         return rows, 1, bs, math.ceil(count / bs), w - 1
     cell = 2 if kind in (PH, PV) else 1
     assert cell == 1 or rows == cols
-    assert kind != DIAG_SIGNED or rows == cols
-    units = (cols if kind in (H, PH) else rows) // cell
+    assert kind not in (DIAG_SIGNED, PKH, PKV) or rows == cols
+    units = (cols if kind in (H, PH, PKH) else rows) // cell
     sub = sub_dim(kind, n)
     bs = math.ceil(math.sqrt(2 * sub - 1))
     gs = math.ceil((sub - 1) / bs)
-    step = w - 1 if kind == DIAG_SIGNED else cell * (w if kind in (V, PV) else 1)
+    step = w - 1 if kind == DIAG_SIGNED else cell * (w if kind in (V, PV, PKV) else 1)
     return units, cell, bs, gs, step
 
 
@@ -308,6 +310,22 @@ def sub_dim(kind, n):
 def transform_mask(kind, n, w, slots, idx):
     """Slot pattern of diagonal idx (no pre-rotation)."""
     rows, cols = _dims(n)
+    if kind in (PKH, PKV):
+        # T_packed(P(x)) = sum_d mask_d rho^(2 d unit)(Z x + M_+ rho^unit x + M_- rho^-unit x): the coefficient of
+        # rho^(idx unit)(x) collects the three ways of writing idx = 2 d + e, e in {0, +1, -1}
+        by_rows = kind == PKV
+        base, unit, cells = (PV if by_rows else PH), (w if by_rows else 1), (rows if by_rows else cols) // 2
+        zmask, terms = packing_maps(slots, w, by_rows)
+        part = {0: zmask, 1: terms[0][1], -1: terms[1][1]}
+        m = np.zeros(slots, dtype=np.complex128)
+        for e in (0, 1, -1):
+            if (idx - e) % 2:
+                continue
+            d = (idx - e) // 2
+            if d <= -cells or d >= cells:
+                continue
+            m += transform_mask(base, n, w, slots, d) * np.roll(part[e], -2 * d * unit)
+        return m
     units, cell, _, _, _ = geometry(kind, n, w)
     sub = sub_dim(kind, n)
     r = np.arange(slots) // w
@@ -835,18 +853,24 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     return orc.rescale(orc.relinearize(acc))
 
 
-def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False):
-    """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused)."""
+def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False):
+    """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused).
+    merge_packing: a and b are NOT packed yet; the packing and the packed transform run as one composite one-stage
+    transform from T+3 (kinds PKH / PKV)."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     lvl = min(a.level, b.level)
-    if lvl >= T + 3:
+    if merge_packing or lvl >= T + 3:
+        if merge_packing:
+            a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)
+            b = diagonal_transform_fused(orc, orc.level_down(b, T + 3), PKV, n, w)
         # both operands a level above what B needs: sigma and tau share one launch chain and both end at T+2, as in
         # the unpacked product; tau(B) is lowered to T+1 with sigma(A)'s copy for the unshifted term
-        a = lower_and_transform_fused(orc, orc.level_down(a, min(lvl, T + 4)), PH, n, w, T + 2)
-        b = lower_and_transform_fused(orc, orc.level_down(b, min(lvl, T + 4)), PV, n, w, T + 2)
+        else:
+            a = lower_and_transform_fused(orc, orc.level_down(a, min(lvl, T + 4)), PH, n, w, T + 2)
+            b = lower_and_transform_fused(orc, orc.level_down(b, min(lvl, T + 4)), PV, n, w, T + 2)
         if n * w != orc.slots and not spread:
             # row shifts wrap inside a tile block (stacked tiles, content not known to be a single tile): every shift
             # of tau(B) by a cell of two rows is a masked pair like the column shifts of sigma(A), n / 2 - 1 of each
@@ -906,6 +930,8 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     is the product of the operands' blocks."""
     from .oracle import Ct
     ev = OracleEval(orc)
+    if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
+        return repack_cc(ev, mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True))
     lvl = min(a.level, b.level, T + 5)
     cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
     pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
@@ -917,14 +943,9 @@ def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
     """One product through the complex-packed route: adjacent columns of A and adjacent rows of B are fused into
     complex slots (complexPackingInplace / complexPackingRowInplace, one level), the packed product then needs n / 2
     shifts instead of n, and x + conj(x) returns the real product (repackCC).  For operands that hold a single tile.
-    Operands above the packing level are only truncated to it (the packing masks absorb the change of scale)."""
-    from .oracle import Ct
-    ev = OracleEval(orc)
-    lvl = min(a.level, b.level, T + 5)        # packing at T+5 at most: the transforms start from T+4
-    cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
-    pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
-    pb = complex_packing_hoisted(orc, cut(b), w, rows=True)
-    return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=True))
+    Operands above the packing level are only truncated to it (the packing masks absorb the change of scale);
+    operands three levels above the target take the packing and the packed transform as one composite transform."""
+    return mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile=True)
 
 
 def mult_mat_mat_pre_fused(orc, a, T, n, w, first_block_only=False):

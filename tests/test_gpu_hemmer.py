@@ -153,14 +153,15 @@ def test_ccmm_single_tile_promise(small):
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -20
     assert np.abs(H.decrypt_slots(c)[256:]).max() < 2 ** -20
-    # without a level to spare for the packing (operands at T+3) the unpacked single-tile route runs
+    # without a level to spare for a separate packing (operands at T+3) the packing and the packed transform run as
+    # one composite transform
     H.assume_single_tile(True)
     try:
         la, lb = H.level_down(ca, 5), H.level_down(cb, 5)
         c5 = H.single_cc_matmul(la, lb, 2)
     finally:
         H.assume_single_tile(False)
-    want5 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16, single_tile=True)
+    want5 = R.mult_mat_mat_cc_packed_single(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16)
     assert np.array_equal(c5.residues(), want5.data)
     assert np.abs(H.decrypt(c5) - A @ B).max() < 2 ** -20
 
@@ -203,14 +204,18 @@ def test_ccmm_stacked_tiles_keep_block_products(small):
     d = H.decrypt_slots(c).real[:512].reshape(32, 16)
     assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -18
     assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -18
-    # three levels to spare: the unpacked product with masked row shifts
+    # three levels to spare: packing and packed transform as one composite transform, then the same masked shifts
     la, lb = H.level_down(ca, 5), H.level_down(cb, 5)
     c1 = H.single_cc_matmul(la, lb, 2)
-    want1 = R.mult_mat_mat_cc_fused(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16)
+    want1 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, la), to_oracle(orc, lb), 2, 16, 16, single_tile=False)
     assert np.array_equal(c1.residues(), want1.data)
     d = H.decrypt_slots(c1).real[:512].reshape(32, 16)
-    assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -20
-    assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -20
+    assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -18
+    assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -18
+    # mixed levels with the lower operand three above the target
+    c3 = H.single_cc_matmul(ca, lb, 2)
+    want3 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ca), to_oracle(orc, lb), 2, 16, 16, single_tile=False)
+    assert np.array_equal(c3.residues(), want3.data)
     # a rotation forgets what was known about a single tile: the masked route again
     ra = H.left_rotate(H.left_rotate(H.encrypt(A[:16]), 3), 512 - 3)
     eb16 = H.encrypt(B[:16])

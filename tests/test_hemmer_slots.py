@@ -164,3 +164,35 @@ def test_two_stage_transform_masks(n, w, log_slots):
             x = y
         want = R.diagonal_transform(sim, sim.encrypt(x0), kind, n, w).z
         assert np.abs(x - want).max() < 1e-12, kind
+
+
+@pytest.mark.parametrize("n,w,log_slots", [(8, 16, 7), (8, 8, 7), (16, 32, 9), (16, 16, 9)])
+def test_composite_packing_transform_masks(n, w, log_slots):
+    """The complex packing followed by the packed sigma / tau as ONE one-stage transform (kinds PKH / PKV, diagonals
+    over single columns / rows): equal to the packing and then the packed transform on arbitrary slot vectors,
+    stacked tile blocks included."""
+    sim = R.SlotSim(log_slots, 12)
+    rng = np.random.default_rng(n + w)
+    x0 = rng.normal(size=sim.slots) + 1j * rng.normal(size=sim.slots)
+    for merged, packed, pack in ((R.PKH, R.PH, R.complex_packing_cols), (R.PKV, R.PV, R.complex_packing_rows)):
+        two_steps = R.diagonal_transform(sim, pack(sim, sim.encrypt(x0), n, w), packed, n, w)
+        one_step = R.diagonal_transform(sim, sim.encrypt(x0), merged, n, w)
+        assert np.abs(one_step.z - two_steps.z).max() < 1e-12, merged
+        assert sim.level_of(one_step) == sim.level_of(two_steps) + 1      # one level instead of two
+
+
+def test_composite_packed_ccmm_three_levels_above_the_target():
+    """A whole product through the composite transform on the slot simulator: operands three levels above the target,
+    single tile and stacked tiles."""
+    n = 8
+    sim = R.SlotSim(7, 12)
+    rng = np.random.default_rng(3)
+    A, B = rng.uniform(-1, 1, (2 * n, n)), rng.uniform(-1, 1, (2 * n, n))
+    a, b = sim.encrypt(A.reshape(-1), 5), sim.encrypt(B.reshape(-1), 5)
+    for kind, unit in ((R.PKH, 1), (R.PKV, n)):
+        assert R.geometry(kind, n, n)[4] == unit
+    pa = R.diagonal_transform(sim, a, R.PKH, n, n)
+    pb = R.diagonal_transform(sim, b, R.PKV, n, n)
+    want_a = R.diagonal_transform(sim, R.complex_packing_cols(sim, a, n, n), R.PH, n, n)
+    want_b = R.diagonal_transform(sim, R.complex_packing_rows(sim, b, n, n), R.PV, n, n)
+    assert np.abs(pa.z - want_a.z).max() < 1e-12 and np.abs(pb.z - want_b.z).max() < 1e-12

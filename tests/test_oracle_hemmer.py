@@ -104,3 +104,22 @@ def test_complex_packed_ccmm_on_stacked_tiles_over_oracle(env):
     assert np.abs(d[:n] - A[:n] @ B[:n]).max() < 2 ** -18
     assert np.abs(d[n:] - A[n:] @ B[n:]).max() < 2 ** -18
     assert np.abs(z.imag).max() < 2 ** -18
+
+
+@pytest.mark.parametrize("single_tile", [True, False])
+def test_complex_packed_ccmm_three_levels_above_target_over_oracle(env, single_tile):
+    """Operands only three levels above the target: the packing and the packed transform run as one composite transform
+    (one level), the rest of the complex-packed product is unchanged."""
+    orc, ev, n = env
+    rng = np.random.default_rng(8)
+    rows = n if single_tile else 2 * n
+    A, B = rng.uniform(-1, 1, (rows, n)), rng.uniform(-1, 1, (rows, n))
+    a, b = orc.level_down(enc(orc, A, 25), 5), orc.level_down(enc(orc, B, 26), 5)
+    c = R.mult_mat_mat_cc_packed(orc, a, b, 2, n, n, single_tile=single_tile)
+    assert c.level == 2 and c.scale == orc.delta[2]
+    z = orc.decrypt(c)
+    d = z[: rows * n].real.reshape(rows, n)
+    assert np.abs(d[:n] - A[:n] @ B[:n]).max() < 2 ** -18
+    if not single_tile:
+        assert np.abs(d[n:] - A[n:] @ B[n:]).max() < 2 ** -18
+    assert np.abs(z.imag).max() < 2 ** -18
