@@ -9,8 +9,8 @@ dominant kernel (the hoisted key-switch inner product, HBM bound) and of the NTT
 the CPU oracle timed on the host cores.
 
 A "step" is one full CCMM.  Everything runs on one GPU; --gpus above 1 is refused.
---roofline-only runs just the roofline legs (used for the committed rocprofv3 summaries, so that a
-kernel's average in the profile is the average of exactly the launches timed here).
+--roofline-only runs just the roofline legs and --ccmm-only just the headline product loop (used for the committed
+rocprofv3 summaries, so that a kernel's average in the profile is the average of exactly the launches timed here).
 """
 import argparse
 import json
@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 LIMB_BYTES = (1 << 16) * 8
 
 
-def gpu_ccmm(args, out):
+def gpu_ccmm(args, out, headline_only=False):
     import numpy as np
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -68,6 +68,8 @@ def gpu_ccmm(args, out):
         "achieved_GBps": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9,
         "frac_of_hbm_peak": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
+    if headline_only:
+        return H
     # one rotation (automorphism + hybrid key switch) at the top level
     r = H.left_rotate(ca, 1)
     H.sync()
@@ -524,6 +526,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--roofline-only", action="store_true", help="run only the roofline legs")
+    ap.add_argument("--ccmm-only", action="store_true", help="run only the headline product loop (for kernel traces)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run it with --gpus 1 "
@@ -546,7 +549,10 @@ def main():
         gpu_ntt(args, out)
         print(json.dumps(out))
         return
-    H = gpu_ccmm(args, out)
+    H = gpu_ccmm(args, out, headline_only=args.ccmm_only)
+    if args.ccmm_only:
+        print(json.dumps(out))
+        return
     gpu_layer_configs(args, out, H)
     del H
     gpu_hoisted(args, out)

@@ -273,6 +273,8 @@ __device__ __forceinline__ void radix16_inv(const F &f, typename F::E (&x)[16], 
                     // (stride 17 words) hits 16 distinct bank pairs
 __device__ __forceinline__ int padc(int c) { return c + (c >> 4); }
 
+__device__ __forceinline__ int swz_row(int r) { return r ^ ((r >> 4) & 1); }
+
 // forward pass 1 / inverse pass 2 work on a 256-row x 16-column slab.
 template <bool INV, class F>
 __device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw) {
@@ -286,11 +288,13 @@ __device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__re
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = f.from_canonical(base[(size_t)(rh + 16 * k) << 8]);
         radix16_fwd(f, x, tw, 1u);
+        // row r of the slab is kept at row r ^ (bit 4 of r): the rows 16 apart that one wavefront reads together
+        // after the exchange then alternate between the two halves of the 64 LDS banks instead of sharing 32 of them
 #pragma unroll
-        for (int k = 0; k < 16; k++) lds[(rh + 16 * k) * 16 + cc] = x[k];
+        for (int k = 0; k < 16; k++) lds[swz_row(rh + 16 * k) * 16 + cc] = x[k];
         __syncthreads();
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = lds[(16 * rh + k) * 16 + cc];
+        for (int k = 0; k < 16; k++) x[k] = lds[swz_row(16 * rh + k) * 16 + cc];
         radix16_fwd(f, x, tw, 16u + rh);
 #pragma unroll
         for (int k = 0; k < 16; k++) mem[(size_t)(16 * rh + k) << 8] = x[k];
