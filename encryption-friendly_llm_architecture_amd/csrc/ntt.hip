@@ -153,11 +153,15 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
 // Between the two launches of one transform the buffer holds the raw doubles.
 #pragma clang fp contract(off)
 
-struct IntField {
+// LAZY16 (primes below 2^60, so 16q < 2^64; forward transforms only): forward values stay in [0, 16q) and only every
+// other stage corrects its first operand -- by 8q, which takes values below 16q to below 8q; the stage after it adds up
+// to 4q twice without a correction.  One conditional subtraction per two butterflies instead of one per butterfly.
+template <bool LAZY16>
+struct IntFieldT {
     typedef u64 E;
     typedef Tw W;
     u64 q, q2, q4, nq4, nq2, nq1, ni, nis;
-    __device__ __forceinline__ IntField(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
+    __device__ __forceinline__ IntFieldT(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
         q = modq[prime].q;
         q2 = 2 * q;
         q4 = 4 * q;
@@ -168,10 +172,21 @@ struct IntField {
         nis = ninv_s[prime];
     }
     __device__ __forceinline__ E from_canonical(u64 v) const { return v; }
-    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const { ct_bfly(x, y, tw, q, q4, nq4); }
+    // odd: the stage's index within its radix-16 block is odd
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw, const bool odd) const {
+        if (!LAZY16) {
+            ct_bfly(x, y, tw, q, q4, nq4);
+            return;
+        }
+        const u64 u = odd ? x : csub(x, 2 * q4, opaque_neg(2 * q4));   // < 12q on odd stages, < 8q on even ones
+        const u64 v = mul_shoup_lazy4(y, tw.w, tw.ws, q);              // < 4q
+        x = u + v;
+        y = u - v + q4;
+    }
     __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q4, nq4); }
-    __device__ __forceinline__ void before_inverse_block(E (&)[16]) const {}
-    __device__ __forceinline__ u64 to_canonical(E v) const {   // v < 8q
+    __device__ __forceinline__ void after_inverse_block(E (&)[16]) const {}
+    __device__ __forceinline__ u64 to_canonical(E v) const {   // v < 8q (16q with LAZY16)
+        if (LAZY16) v = csub(v, 2 * q4, opaque_neg(2 * q4));
         return csub(csub(csub(v, q4, nq4), q2, nq2), q, nq1);
     }
     __device__ __forceinline__ u64 scale_to_canonical(E v) const {
@@ -184,6 +199,8 @@ struct IntField {
         return csub(mul_shoup_lazy(d, cst.w, cst.ws, q), q, nq1);
     }
 };
+
+typedef IntFieldT<false> IntField;
 
 struct __align__(16) TwF {
     double w, winv;
@@ -209,7 +226,7 @@ struct FpField {
     __device__ __forceinline__ E from_canonical(u64 v) const {
         return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - 4503599627370496.0;
     }
-    __device__ __forceinline__ void ct(E &x, E &y, const W tw) const {
+    __device__ __forceinline__ void ct(E &x, E &y, const W tw, const bool) const {
         const double v = mulmod(y, tw.w, tw.winv);
         const double u = x;
         x = u + v;
@@ -220,9 +237,13 @@ struct FpField {
         x = u + v;
         y = mulmod(u - v, tw.w, tw.winv);
     }
-    __device__ __forceinline__ void before_inverse_block(E (&x)[16]) const {
-#pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = reduce(x[k]);
+    // A Gentleman-Sande block of four stages doubles the sums: from inputs bounded by B its outputs are bounded by
+    // 16 B (element 0), 8 r (element 1), 4 r, 4 r, 2 r x 4, r x 8 with r = 0.55 q the bound of a product, and the
+    // largest value it multiplies is 16 B.  With only elements 0 and 1 reduced after each block every block starts
+    // from B <= 2.2 q, so nothing exceeds 36 q < 2^50, where the products are still exact.
+    __device__ __forceinline__ void after_inverse_block(E (&x)[16]) const {
+        x[0] = reduce(x[0]);
+        x[1] = reduce(x[1]);
     }
     __device__ __forceinline__ u64 centred_to_canonical(E r) const {
         r += r < 0.0 ? q : 0.0;
@@ -248,7 +269,7 @@ __device__ __forceinline__ void radix16_fwd(const F &f, typename F::E (&x)[16], 
         for (int g = 0; g < (1 << s); g++) {
             const typename F::W w = tw[(X << s) + g];
 #pragma unroll
-            for (int j = 0; j < d; j++) f.ct(x[g * 2 * d + j], x[g * 2 * d + j + d], w);
+            for (int j = 0; j < d; j++) f.ct(x[g * 2 * d + j], x[g * 2 * d + j + d], w, (s & 1) != 0);
         }
     }
 }
@@ -301,14 +322,13 @@ __device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__re
     } else {
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = mem[(size_t)(16 * rh + k) << 8];
-        f.before_inverse_block(x);
         radix16_inv(f, x, tw, 16u + rh);
+        f.after_inverse_block(x);
 #pragma unroll
         for (int k = 0; k < 16; k++) lds[(16 * rh + k) * 16 + cc] = x[k];
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = lds[(rh + 16 * k) * 16 + cc];
-        f.before_inverse_block(x);
         radix16_inv(f, x, tw, 1u);
 #pragma unroll
         for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = f.scale_to_canonical(x[k]);
@@ -335,13 +355,15 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
             f.niinv = f.ni * f.qinv;
         }
         cols_body<INV>(base, tw, f, lds);
-    } else {
+    } else if (INV || (modq[prime].q >> 60) != 0) {
         IntField f(modq, ninv, ninv_s, fp, prime);
         if (INV && final_scale != nullptr) {
             f.ni = final_scale[limb].w;
             f.nis = final_scale[limb].ws;
         }
         cols_body<INV>(base, tw, f, lds);
+    } else {
+        cols_body<INV>(base, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds);
     }
 }
 
@@ -412,14 +434,15 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = f.from_canonical(lc[padc(16 * c + k)]);
         radix16_inv(f, x, tw, 16u * (256u + r) + c);
+        f.after_inverse_block(x);
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = l[padc(c + 16 * k)];
-        f.before_inverse_block(x);
         radix16_inv(f, x, tw, 256u + r);
+        f.after_inverse_block(x);
 #pragma unroll
         for (int k = 0; k < 16; k++) mem[c + 16 * k] = x[k];
     }
@@ -459,8 +482,10 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
         ld = ep.minuend + (size_t)poly * ep.minuend_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     if (fp[4 * prime] != 0.0)
         rows_body<INV, EPI>(row, tw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
-    else
+    else if (INV || (q >> 60) != 0)
         rows_body<INV, EPI>(row, tw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+    else
+        rows_body<INV, EPI>(row, tw, IntFieldT<true>(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
 }
 
 }  // namespace
