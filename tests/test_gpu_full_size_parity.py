@@ -212,6 +212,16 @@ def test_preset_ccmm_residues_bit_exact():
     assert c.info()["level"] == 4 == want.level
     assert np.array_equal(c.residues(), want.data)
     assert np.abs(H.decrypt(c) - A @ B).max() < 2.0 ** -12
+    # the same operands three levels above the target with nothing known about their content (a raw upload): the
+    # complex packing and the packed transform as one composite transform, then 63 + 63 masked cell shifts
+    la, lb = H.level_down(ca, 7), H.level_down(cb, 7)
+    ua, ub = H.upload(la.residues(), 128, 128, 128), H.upload(lb.residues(), 128, 128, 128)
+    c3 = H.single_cc_matmul(ua, ub, 4)
+    d7 = orc.delta[7]
+    want3 = R.mult_mat_mat_cc_packed(orc, O.Ct(ua.residues(), d7), O.Ct(ub.residues(), d7), 4, 128, 128, single_tile=False)
+    assert c3.info()["level"] == 4 == want3.level
+    assert np.array_equal(c3.residues(), want3.data)
+    assert np.abs(H.decrypt(c3) - A @ B).max() < 2.0 ** -12
 
 
 @pytest.fixture(scope="module")
