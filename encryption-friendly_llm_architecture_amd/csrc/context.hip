@@ -84,9 +84,11 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     const int N = 1 << logN, T = nQ + nP;
     for (int i = 0; i < T; i++) {
         u64 q = primes[i];
-        if (q >= (1ull << 61) || q < (1ull << 20) || (q - 1) % (2 * (u64)N) != 0 || !h_is_prime(q))
+        // Below 2^31 the one-step reductions of a 60-bit residue (or of a 128-bit product) to this prime would leave more
+        // than the few multiples of q that their conditional subtractions remove.
+        if (q >= (1ull << 61) || q < (1ull << 31) || (q - 1) % (2 * (u64)N) != 0 || !h_is_prime(q))
             throw std::invalid_argument("prime " + std::to_string(i) +
-                                        " must be a prime < 2^61 congruent to 1 mod 2N");
+                                        " must be a prime in [2^31, 2^61) congruent to 1 mod 2N");
         for (int j = 0; j < i; j++)
             if (primes[j] == q) throw std::invalid_argument("primes must be distinct");
     }
@@ -152,7 +154,7 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
         m.mu = (u64)((((u128)1) << (2 * m.k)) / q);
         m.pad = 0;
         m.mu3 = (m.k == 59 || m.k == 60) ? (u64)((((u128)1) << (2 * m.k + 3)) / q) : 0;
-        m.pad2 = 0;
+        m.r64 = (u64)((((u128)1) << 64) % q);
         c->modq[i] = m;
     }
     auto up = [&](const void *h, size_t bytes) -> void * {

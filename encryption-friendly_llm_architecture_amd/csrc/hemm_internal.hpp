@@ -77,6 +77,29 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
                       int n_polys, size_t poly_stride, bool inverse, hipStream_t s, const void *final_scale = nullptr);
 bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_polys, const u64 *minuend,
                           size_t minuend_stride, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
+// A forward transform of N = 2^16 whose input is a fast basis conversion: limb l of the launch is the conversion of
+// the coefficient-form sources of digit digit_of[l] (already carrying their (S/q_i)^-1 factors) to prime ll[l],
+// computed while the first pass loads its slab instead of being written by a conversion launch and read back.
+#define CONV_MAX_DIGITS 4
+#define CONV_MAX_SOURCES 8
+struct ConvSources {
+    struct Digit {
+        const u64 *src;             // coefficient form, [n_polys][.][N]
+        const Cst *hat;             // [n_src][hat_ld]  (S/q_i) mod prime, indexed by prime
+        size_t src_poly_stride;
+        int n_src;
+        uint8_t src_slot[CONV_MAX_SOURCES];
+    } d[CONV_MAX_DIGITS];
+    int hat_ld;
+    uint8_t digit_of[HEMM_MAX_PRIMES];
+};
+// data: [n_polys][.][N] (polynomial stride poly_stride), limb l written to slot sl[l].  With ep_* set the second pass
+// ends with out = (minuend - transform) * cst[l] (slots of minuend / out = l) and data is only a workspace.
+// false when the ring size or the source counts have no such form (nothing was launched).
+bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *data, const LimbList &ll, const LimbList &sl,
+                          int n_limbs, int n_polys, size_t poly_stride, hipStream_t s, const u64 *ep_minuend = nullptr,
+                          size_t ep_minuend_stride = 0, u64 *ep_out = nullptr, size_t ep_out_stride = 0,
+                          const void *ep_cst_dev = nullptr);
 // inverse transform reading src (same slot numbering as data, polynomial stride src_poly_stride) and leaving the
 // coefficients in data; false when this ring size has no out-of-place form (the caller copies, then transforms)
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,

@@ -56,18 +56,9 @@ __global__ __launch_bounds__(256) void bconv_kernel(BConvArgs a, const ModQ *__r
     }
 }
 
-// v < 32q (q < 2^59) to [0, q)
-__device__ __forceinline__ u64 reduce_below_32q(u64 v, const u64 q) {
-#pragma unroll
-    for (int m = 16; m >= 1; m >>= 1)
-        if (v >= (u64)m * q) v -= (u64)m * q;
-    return v;
-}
-
-// Register form of the same conversion for up to 8 source limbs: a thread owns two adjacent coefficients
-// (16-byte accesses), keeps the scaled source residues in registers and sums the Shoup products of a
-// target limb lazily (each below 2q; reduced every 3 terms, which cannot overflow for q < 2^61).  Targets below 2^59
-// take the cheaper products with a three-term quotient estimate (each below 4q) and reduce once at the end.
+// Register form of the same conversion for up to 8 source limbs and primes below 2^60: a thread owns two adjacent
+// coefficients (16-byte accesses), keeps the scaled source residues in registers and takes every target residue as a
+// lazy dot product (four 32-bit multiply-adds per term) with one reduction at the end.
 template <int NS>
 __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ *__restrict__ modq) {
     const int S = a.split > 1 ? a.split : 1;
@@ -87,34 +78,17 @@ __global__ __launch_bounds__(256) void bconv_reg_kernel(BConvArgs a, const ModQ 
     }
     for (int j = j_lo; j < j_hi; j++) {
         const int pj = a.dst_prime[j];
-        const u64 q = modq[pj].q;
-        u64 acc0 = 0, acc1 = 0;
-        if (q < (1ull << 59)) {   // up to 8 terms below 4q each cannot overflow: no reductions on the way
-#pragma unroll
-            for (int i = 0; i < NS; i++) {
-                const Cst c = a.hat[i * a.hat_ld + pj];
-                acc0 += mul_shoup_lazy4(v0[i], c.w, c.ws, q);
-                acc1 += mul_shoup_lazy4(v1[i], c.w, c.ws, q);
-            }
-            *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) =
-                make_ulonglong2(reduce_below_32q(acc0, q), reduce_below_32q(acc1, q));
-            continue;
-        }
+        const ModQ m = modq[pj];
+        Dot3 d0, d1;
+        dot3_clear(d0);
+        dot3_clear(d1);
 #pragma unroll
         for (int i = 0; i < NS; i++) {
-            const Cst c = a.hat[i * a.hat_ld + pj];
-            acc0 += mul_shoup_lazy(v0[i], c.w, c.ws, q);
-            acc1 += mul_shoup_lazy(v1[i], c.w, c.ws, q);
-            if (i % 3 == 2 || i == NS - 1) {
-                if (acc0 >= 4 * q) acc0 -= 4 * q;
-                if (acc1 >= 4 * q) acc1 -= 4 * q;
-                if (acc0 >= 2 * q) acc0 -= 2 * q;
-                if (acc1 >= 2 * q) acc1 -= 2 * q;
-                if (acc0 >= q) acc0 -= q;
-                if (acc1 >= q) acc1 -= q;
-            }
+            const u64 h = a.hat[i * a.hat_ld + pj].w;
+            dot3_add(d0, v0[i], h);
+            dot3_add(d1, v1[i], h);
         }
-        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
+        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(dot3_reduce(d0, m), dot3_reduce(d1, m));
     }
 }
 
@@ -150,38 +124,19 @@ __global__ __launch_bounds__(256) void bconv_digits_kernel(BConvDigits g, const 
     }
     for (int j = j_lo; j < j_hi; j++) {
         const int pj = a.dst_prime[j];
-        const u64 q = modq[pj].q;
-        u64 acc0 = 0, acc1 = 0;
-        if (q < (1ull << 59)) {
-#pragma unroll
-            for (int i = 0; i < NS; i++) {
-                if (i < a.n_src) {
-                    const Cst c = a.hat[i * a.hat_ld + pj];
-                    acc0 += mul_shoup_lazy4(v0[i], c.w, c.ws, q);
-                    acc1 += mul_shoup_lazy4(v1[i], c.w, c.ws, q);
-                }
-            }
-            *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) =
-                make_ulonglong2(reduce_below_32q(acc0, q), reduce_below_32q(acc1, q));
-            continue;
-        }
+        const ModQ m = modq[pj];
+        Dot3 d0, d1;
+        dot3_clear(d0);
+        dot3_clear(d1);
 #pragma unroll
         for (int i = 0; i < NS; i++) {
             if (i < a.n_src) {
-                const Cst c = a.hat[i * a.hat_ld + pj];
-                acc0 += mul_shoup_lazy(v0[i], c.w, c.ws, q);
-                acc1 += mul_shoup_lazy(v1[i], c.w, c.ws, q);
-            }
-            if (i % 3 == 2 || i == NS - 1) {
-                if (acc0 >= 4 * q) acc0 -= 4 * q;
-                if (acc1 >= 4 * q) acc1 -= 4 * q;
-                if (acc0 >= 2 * q) acc0 -= 2 * q;
-                if (acc1 >= 2 * q) acc1 -= 2 * q;
-                if (acc0 >= q) acc0 -= q;
-                if (acc1 >= q) acc1 -= q;
+                const u64 h = a.hat[i * a.hat_ld + pj].w;
+                dot3_add(d0, v0[i], h);
+                dot3_add(d1, v1[i], h);
             }
         }
-        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(acc0, acc1);
+        *(ulonglong2 *)(dst + ((size_t)a.dst_slot[j] << a.logN) + n) = make_ulonglong2(dot3_reduce(d0, m), dot3_reduce(d1, m));
     }
     const u64 *own = g.own + poly * g.own_stride;
     for (int j = g.own_lo[blockIdx.z] + part; j < g.own_hi[blockIdx.z]; j += S)
@@ -199,12 +154,20 @@ static int bconv_split(int N, int n_units, int n_dst) {
     return S < 1 ? 1 : S;
 }
 
+// the lazy dot products of the register kernels hold 8 terms of 60 x 60 bits
+static bool lazy_dot_ok(const hemm_context *c) {
+    for (u64 q : c->primes)
+        if ((q >> 60) != 0) return false;
+    return true;
+}
+
 void launch_bconv(const hemm_context *c, const BConvArgs &a_in, const ModQ *modq, int N, int n_polys, hipStream_t s) {
     BConvArgs a = a_in;
     account(c, TR_BCONV, (size_t)(a.n_src + a.n_dst) * n_polys * N * 8);
-    a.split = (a.n_src <= 8 && N >= 512) ? bconv_split(N, n_polys, a.n_dst) : 1;
+    const bool reg = a.n_src <= 8 && N >= 512 && lazy_dot_ok(c);
+    a.split = reg ? bconv_split(N, n_polys, a.n_dst) : 1;
     dim3 block(256), wide(N / 256, n_polys), pair(N / 512, n_polys * a.split);
-    switch (a.n_src) {
+    switch (reg ? a.n_src : 0) {
 #define BCONV_CASE(K) case K: hipLaunchKernelGGL(bconv_reg_kernel<K>, pair, block, 0, s, a, modq); break;
         BCONV_CASE(1) BCONV_CASE(2) BCONV_CASE(3) BCONV_CASE(4) BCONV_CASE(5) BCONV_CASE(6) BCONV_CASE(7) BCONV_CASE(8)
 #undef BCONV_CASE
@@ -984,7 +947,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     // One conversion launch and one forward transform for all digits when the ring size allows: the converted
     // limbs of every digit are addressed as slots d*E + j of one extended polynomial per input.
     const bool joint = c->N >= 512 && alpha <= 8 && beta <= BCONV_MAX_DIGITS && beta * E <= 255 &&
-                       beta * E - nq <= HEMM_MAX_PRIMES;
+                       beta * E - nq <= HEMM_MAX_PRIMES && lazy_dot_ok(c);
     BConvDigits g;
     memset(&g, 0, sizeof(g));
     g.own = in;
@@ -1222,9 +1185,26 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
         a.dst_slot[j] = (uint8_t)j;
         a.dst_prime[j] = (uint8_t)j;
     }
-    launch_bconv(c, a, c->d_modq, (int)N, n_polys, s);
     const dim3 block(256);
     const Cst *cst_dev = t->dev + (drop_last ? t->dropinv_off[nq] : t->pinv_off);
+    if (fold && ns <= CONV_MAX_SOURCES && lazy_dot_ok(c)) {
+        // the conversion is computed inside the first pass of the forward transform: no conversion launch, and the
+        // converted limbs are neither written in coefficient form nor read back
+        ConvSources cs;
+        memset(&cs, 0, sizeof(cs));
+        cs.d[0].src = y;
+        cs.d[0].hat = a.hat;
+        cs.d[0].src_poly_stride = a.src_poly_stride;
+        cs.d[0].n_src = ns;
+        for (int i = 0; i < ns; i++) cs.d[0].src_slot[i] = a.src_slot[i];
+        cs.hat_ld = a.hat_ld;
+        LimbList cl = limbs_default(c, nq_out, 0), ident;
+        for (int j = 0; j < HEMM_MAX_PRIMES; j++) ident.idx[j] = (uint8_t)j;
+        if (launch_ntt_converted(c, cs, conv, cl, ident, nq_out, n_polys, (size_t)nq_out * N, s, y, (size_t)E * N, out,
+                                 out_stride, cst_dev))
+            return;
+    }
+    launch_bconv(c, a, c->d_modq, (int)N, n_polys, s);
     if (launch_ntt_sub_scale(c, conv, nq_out, n_polys, y, (size_t)E * N, out, out_stride, cst_dev, s)) return;
     launch_ntt(c, conv, limbs_default(c, nq_out, 0), nq_out, n_polys, (size_t)nq_out * N, false, s);
     CstList cl;

@@ -37,7 +37,7 @@ struct ModQ {
     u32 k;     // bit length of q (q < 2^k, k <= 61)
     u32 pad;
     u64 mu3;   // floor(2^(2k+3) / q) for k = 59 or 60, else 0 (barrett_tight)
-    u64 pad2;
+    u64 r64;   // 2^64 mod q
 };
 
 // x * w mod q for a constant w with ws = floor(w * 2^64 / q); result in [0, 2q).
@@ -63,6 +63,13 @@ __device__ __forceinline__ u64 mul_shoup_lazy4(u64 x, u64 w, u64 ws, u64 q) {
     const u64 t = (u64)hl * nl + (u64)xl * wl;
     const u32 top = (u32)(t >> 32) + xl * wh + xh * wl + hl * nh + hh * nl;
     return ((u64)top << 32) | (u32)t;
+}
+// v < 32q (q < 2^59) to [0, q)
+__device__ __forceinline__ u64 reduce_below_32q(u64 v, const u64 q) {
+#pragma unroll
+    for (int m = 16; m >= 1; m >>= 1)
+        if (v >= (u64)m * q) v -= (u64)m * q;
+    return v;
 }
 // Barrett reduction of a 128-bit value T < 6 * 2^(2k) to [0, q).
 __device__ __forceinline__ u64 barrett128(u128_t t, const ModQ &m) {
@@ -101,6 +108,45 @@ __device__ __forceinline__ u64 reduce64(u64 a, const ModQ &m) {
     t.lo = a;
     t.hi = 0;
     return barrett128(t, m);
+}
+// Lazy dot product sum_i v_i * h_i of up to 8 residues v_i < 2^60 with constants h_i < 2^60 (a target residue of a
+// fast basis conversion).  The 32-bit halves are multiplied into three 64-bit accumulators -- s0 (weight 1, with a
+// carry count), s1 (weight 2^32: 16 terms below 2^60 cannot overflow), s2 (weight 2^64) -- four multiply-adds per
+// term and no reduction until the end, against a Shoup product with its own quotient per term.
+struct Dot3 {
+    u64 s0, s1, s2;
+    u32 c;
+};
+__device__ __forceinline__ void dot3_clear(Dot3 &d) {
+    d.s0 = d.s1 = d.s2 = 0;
+    d.c = 0;
+}
+__device__ __forceinline__ void dot3_add(Dot3 &d, const u64 v, const u64 h) {
+    const u32 vl = (u32)v, vh = (u32)(v >> 32), hl = (u32)h, hh = (u32)(h >> 32);
+    const u64 p = (u64)vl * hl;
+    d.s0 += p;
+    d.c += d.s0 < p ? 1u : 0u;
+    d.s1 += (u64)vl * hh;
+    d.s1 += (u64)vh * hl;
+    d.s2 += (u64)vh * hh;
+}
+// the sum as a 128-bit value (below 8 * 2^(60 + k) for constants below 2^k)
+__device__ __forceinline__ u128_t dot3_value(const Dot3 &d) {
+    u128_t t;
+    const u64 mid = d.s1 << 32;
+    t.lo = d.s0 + mid;
+    t.hi = d.s2 + d.c + (d.s1 >> 32) + (t.lo < mid ? 1ull : 0ull);
+    return t;
+}
+// ... reduced to [0, q): the high word (below 2^(k-1)) is folded with 2^64 mod q, which leaves a value below
+// 2^(2k-1) + 2^64 < 6 * 2^(2k) for k >= 31, then one Barrett step
+__device__ __forceinline__ u64 dot3_reduce(const Dot3 &d, const ModQ &m) {
+    const u128_t t = dot3_value(d);
+    u128_t u = mul64wide(t.hi, m.r64);
+    const u64 lo = u.lo + t.lo;
+    u.hi += lo < t.lo ? 1ull : 0ull;
+    u.lo = lo;
+    return barrett128(u, m);
 }
 __device__ __forceinline__ u64 addmod(u64 a, u64 b, u64 q) {
     u64 s = a + b;

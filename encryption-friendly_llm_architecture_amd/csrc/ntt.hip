@@ -15,6 +15,8 @@
 //
 // Other sizes (2^6 .. 2^15, used by the small-parameter tests) run a plain LDS kernel with the
 // same butterfly network, so residues are identical for every N.
+#include <algorithm>
+
 #include "hemm_internal.hpp"
 
 namespace {
@@ -160,11 +162,12 @@ template <bool LAZY16>
 struct IntFieldT {
     typedef u64 E;
     typedef Tw W;
-    u64 q, q2, q4, nq4, nq2, nq1, ni, nis;
+    u64 q, q2, q4, nq8, nq4, nq2, nq1, ni, nis;
     __device__ __forceinline__ IntFieldT(const ModQ *modq, const u64 *ninv, const u64 *ninv_s, const double *, int prime) {
         q = modq[prime].q;
         q2 = 2 * q;
         q4 = 4 * q;
+        nq8 = opaque_neg(2 * q4);
         nq4 = opaque_neg(q4);
         nq2 = opaque_neg(q2);
         nq1 = opaque_neg(q);
@@ -172,13 +175,14 @@ struct IntFieldT {
         nis = ninv_s[prime];
     }
     __device__ __forceinline__ E from_canonical(u64 v) const { return v; }
+    __device__ __forceinline__ E from_dot(const Dot3 &d, const ModQ &m) const { return dot3_reduce(d, m); }
     // odd: the stage's index within its radix-16 block is odd
     __device__ __forceinline__ void ct(E &x, E &y, const W tw, const bool odd) const {
         if (!LAZY16) {
             ct_bfly(x, y, tw, q, q4, nq4);
             return;
         }
-        const u64 u = odd ? x : csub(x, 2 * q4, opaque_neg(2 * q4));   // < 12q on odd stages, < 8q on even ones
+        const u64 u = odd ? x : csub(x, 2 * q4, nq8);   // < 12q on odd stages, < 8q on even ones
         const u64 v = mul_shoup_lazy4(y, tw.w, tw.ws, q);              // < 4q
         x = u + v;
         y = u - v + q4;
@@ -186,7 +190,7 @@ struct IntFieldT {
     __device__ __forceinline__ void gs(E &x, E &y, const W tw) const { gs_bfly(x, y, tw, q, q4, nq4); }
     __device__ __forceinline__ void after_inverse_block(E (&)[16]) const {}
     __device__ __forceinline__ u64 to_canonical(E v) const {   // v < 8q (16q with LAZY16)
-        if (LAZY16) v = csub(v, 2 * q4, opaque_neg(2 * q4));
+        if (LAZY16) v = csub(v, 2 * q4, nq8);
         return csub(csub(csub(v, q4, nq4), q2, nq2), q, nq1);
     }
     __device__ __forceinline__ u64 scale_to_canonical(E v) const {
@@ -225,6 +229,17 @@ struct FpField {
     __device__ __forceinline__ E reduce(E x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
     __device__ __forceinline__ E from_canonical(u64 v) const {
         return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - 4503599627370496.0;
+    }
+    // A lazy dot product (three accumulators of weights 1, 2^32, 2^64 and a carry count of weight 2^64) as a residue of
+    // magnitude below q: regrouped into pieces of weights 1, 2^32, 2^64 below 2^32, 2^33 and 2^45 (constants below
+    // 2^44, residues below 2^60, 8 terms), each exact in a double; the two upper ones are multiplied by 2^32 and 2^64
+    // mod q.  No integer reduction and no conversion from canonical form.
+    __device__ __forceinline__ E from_dot(const Dot3 &d, const ModQ &) const {
+        const u64 p1 = (d.s0 >> 32) + (d.s1 & 0xffffffffull), p2 = (d.s1 >> 32) + d.s2 + d.c;
+        const double r32 = reduce(4294967296.0), r64 = reduce(18446744073709551616.0);
+        const double a = (double)(u32)d.s0 + mulmod(from_canonical(p1), r32, r32 * qinv) +
+                         mulmod(from_canonical(p2), r64, r64 * qinv);
+        return reduce(a);
     }
     __device__ __forceinline__ void ct(E &x, E &y, const W tw, const bool) const {
         const double v = mulmod(y, tw.w, tw.winv);
@@ -365,6 +380,85 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
     } else {
         cols_body<INV>(base, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds);
     }
+}
+
+// Forward pass 1 over a slab whose input is a basis conversion computed on the fly: the thread's 16 coefficients of
+// the target limb are sum_i v_i * hat_i mod q over the NS source limbs of the limb's digit (sources pre-scaled, the
+// same lazy sums and reductions as the stand-alone conversion kernels, so the residues are the same).  The workgroups
+// of the target limbs that share a (polynomial, slab) pair have consecutive blockIdx.y and the same blockIdx.x, so
+// they sit on one XCD at about the same time and all but the first find the source slabs in its L2.
+template <int NS, class F>
+__device__ __forceinline__ void cols_converted_body(u64 *__restrict__ base, const Tw *__restrict__ tw_int, const F f,
+                                                    u64 *lds_raw, const u64 *const (&sp)[NS], const u64 (&h)[NS],
+                                                    const int n_src, const ModQ m) {
+    typedef typename F::E E;
+    const typename F::W *tw = (const typename F::W *)tw_int;
+    E *lds = (E *)lds_raw;
+    E *mem = (E *)base;
+    const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
+    E x[16];
+    // eight coefficients at a time (three accumulators each), source by source, so that the eight loads of one source
+    // limb are in flight together
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        Dot3 d[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) dot3_clear(d[k]);
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            if (i < n_src) {
+                u64 v[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) v[k] = sp[i][(size_t)(rh + 16 * (8 * half + k)) << 8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) dot3_add(d[k], v[k], h[i]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) x[8 * half + k] = f.from_dot(d[k], m);
+    }
+    radix16_fwd(f, x, tw, 1u);
+#pragma unroll
+    for (int k = 0; k < 16; k++) lds[swz_row(rh + 16 * k) * 16 + cc] = x[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = lds[swz_row(16 * rh + k) * 16 + cc];
+    radix16_fwd(f, x, tw, 16u + rh);
+#pragma unroll
+    for (int k = 0; k < 16; k++) mem[(size_t)(16 * rh + k) << 8] = x[k];
+}
+
+template <int NS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ntt16_cols_converted_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                                   const ModQ *__restrict__ modq,
+                                                                   const u64 *__restrict__ ninv,
+                                                                   const u64 *__restrict__ ninv_s,
+                                                                   const double *__restrict__ fp, LimbList ll, LimbList sl,
+                                                                   int n_limbs, size_t poly_stride, ConvSources cs) {
+    __shared__ u64 lds[256 * 16];
+    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const size_t col = blockIdx.x * 16 + (threadIdx.x & 15);
+    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + col;
+    const int dg = cs.digit_of[limb], n_src = cs.d[dg].n_src;
+    const u64 *src = cs.d[dg].src + (size_t)poly * cs.d[dg].src_poly_stride + col;
+    const Cst *hat = cs.d[dg].hat + prime;
+    const ModQ m = modq[prime];
+    const u64 *sp[NS];
+    u64 h[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        const int ii = i < n_src ? i : 0;
+        sp[i] = src + ((size_t)cs.d[dg].src_slot[ii] << 16);
+        h[i] = hat[(size_t)ii * cs.hat_ld].w;
+    }
+    if (fp[4 * prime] != 0.0)
+        cols_converted_body<NS>(base, tw, FpField(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
+    else if ((m.q >> 60) != 0)
+        cols_converted_body<NS>(base, tw, IntField(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
+    else
+        cols_converted_body<NS>(base, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
 }
 
 // A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
@@ -527,6 +621,51 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
                            c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)nullptr);
         hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * np), block, 0, s, d, tw, c->d_modq,
                            c->d_fp, ll, sl, n_limbs, poly_stride, ep);
+    }
+    return true;
+}
+
+bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *data, const LimbList &ll, const LimbList &sl,
+                          int n_limbs, int n_polys, size_t poly_stride, hipStream_t s, const u64 *ep_minuend,
+                          size_t ep_minuend_stride, u64 *ep_out, size_t ep_out_stride, const void *ep_cst_dev) {
+    if (c->logN != 16) return false;
+    int widest = 0;
+    for (int l = 0; l < n_limbs; l++) {
+        if (cs.digit_of[l] >= CONV_MAX_DIGITS) throw std::invalid_argument("conversion digit out of range");
+        widest = std::max(widest, cs.d[cs.digit_of[l]].n_src);
+    }
+    if (widest < 1 || widest > CONV_MAX_SOURCES) return false;
+    if (n_limbs <= 0 || n_polys <= 0) return true;
+    const bool tail = ep_out != nullptr;
+    // sources of every digit in use once, limbs out (through the tail: minuend in, result out)
+    size_t src_limbs = 0;
+    bool seen[CONV_MAX_DIGITS] = {false, false, false, false};
+    for (int l = 0; l < n_limbs; l++)
+        if (!seen[cs.digit_of[l]]) {
+            seen[cs.digit_of[l]] = true;
+            src_limbs += (size_t)cs.d[cs.digit_of[l]].n_src;
+        }
+    account(c, TR_BCONV, src_limbs * n_polys * c->N * 8, 0);
+    account(c, TR_NTT, (size_t)(tail ? 2 : 1) * n_limbs * n_polys * c->N * 8, 2);
+    const Tw *tw = (const Tw *)c->d_w;
+    const dim3 block(256), grid(16, n_limbs * n_polys);
+#define CONV_CASE(K)                                                                                                    \
+    hipLaunchKernelGGL(ntt16_cols_converted_kernel<K>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, \
+                       c->d_fp, ll, sl, n_limbs, poly_stride, cs)
+    if (widest <= 2)
+        CONV_CASE(2);
+    else if (widest <= 5)
+        CONV_CASE(5);
+    else
+        CONV_CASE(8);
+#undef CONV_CASE
+    if (tail) {
+        NttEpilogue ep{ep_minuend, ep_out, (const Tw *)ep_cst_dev, ep_minuend_stride, ep_out_stride};
+        hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw,
+                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, ep);
+    } else {
+        hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw,
+                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
     }
     return true;
 }

@@ -9,6 +9,14 @@
  * uses chain prime j for j < nq and special prime (j - nq) after that.  `stream` is a
  * hipStream_t (NULL = default stream); calls are asynchronous on it.
  *
+ * One stream per context at a time.  A context owns one device scratch region and one staging
+ * region for term lists longer than 32.  hemm_modup, hemm_moddown, hemm_keyswitch, hemm_rotate,
+ * hemm_relinearize and hemm_rescale work in the scratch region, and the batched
+ * calls (hemm_hoisted_*, hemm_masked_sum_batch) copy long term lists through the staging region,
+ * so two such calls queued on DIFFERENT streams of one context race unless the caller orders
+ * them with events.  Calls that take a `workspace` argument use only that memory.  Callers that
+ * want concurrent streams build one context per stream.
+ *
  * Return value: 0 = ok, 1 = invalid argument, 2 = HIP/runtime failure; the text is in
  * hemm_last_error().
  */
@@ -26,7 +34,7 @@ typedef struct hemm_context hemm_context;
 const char *hemm_last_error(void);
 
 /* HEaaN::makeContext (Context.hpp:39,88): ring degree 2^log_n, n_q chain primes followed by
- * n_p special (key-switching) primes, all < 2^61 and = 1 mod 2^(log_n+1); dnum = number of
+ * n_p special (key-switching) primes, all in [2^31, 2^61) and = 1 mod 2^(log_n+1); dnum = number of
  * key-switching digits.  Twiddle tables are built on the current device. */
 int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64_t *primes,
                         uint32_t dnum, hemm_context **out);
