@@ -1006,6 +1006,30 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
                                   (size_t)(hi - lo) * N * 8, n_in, hipMemcpyDeviceToDevice, s));
     }
     if (!joint) return;
+    if (fold && n_joint + nq <= HEMM_MAX_PRIMES) {
+        // the conversions of all digits inside the first pass of the forward transform; the same launch copies every
+        // digit's own limbs into its slice
+        ConvSources cs;
+        memset(&cs, 0, sizeof(cs));
+        cs.hat_ld = c->nQ + c->nP;
+        int l = 0;
+        for (int d = 0; d < beta; d++) {
+            cs.d[d].src = g.d[d].src;
+            cs.d[d].hat = g.d[d].hat;
+            cs.d[d].src_poly_stride = g.d[d].src_poly_stride;
+            cs.d[d].n_src = g.d[d].n_src;
+            for (int i = 0; i < g.d[d].n_src; i++) cs.d[d].src_slot[i] = g.d[d].src_slot[i];
+            for (int j = 0; j < g.d[d].n_dst; j++) cs.digit_of[l++] = (uint8_t)d;
+        }
+        cs.copy_src = in;
+        cs.copy_src_stride = in_stride;
+        cs.n_copy = nq;
+        for (int j = 0; j < nq; j++) {
+            cs.copy_src_slot[j] = (uint8_t)j;
+            js.idx[n_joint + j] = (uint8_t)((j / alpha) * E + j);
+        }
+        if (launch_ntt_converted(c, cs, ext, jp, js, n_joint, n_in, (size_t)beta * E * N, s)) return;
+    }
     g.d[0].split = bconv_split((int)N, n_in * beta, E - alpha);
     const dim3 grid((unsigned)(N / 512), n_in * g.d[0].split, beta), block(256);
     const int widest = std::min(nq, alpha);

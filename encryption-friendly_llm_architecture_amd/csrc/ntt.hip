@@ -436,11 +436,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                                                                    const double *__restrict__ fp, LimbList ll, LimbList sl,
                                                                    int n_limbs, size_t poly_stride, ConvSources cs) {
     __shared__ u64 lds[256 * 16];
-    const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
-    const int prime = ll.idx[limb];
-    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const int per_poly = n_limbs + cs.n_copy;
+    const int limb = blockIdx.y % per_poly, poly = blockIdx.y / per_poly;
     const size_t col = blockIdx.x * 16 + (threadIdx.x & 15);
     u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + col;
+    if (limb >= n_limbs) {   // a limb that is only copied into its slot
+        const u64 *from = cs.copy_src + (size_t)poly * cs.copy_src_stride +
+                          ((size_t)cs.copy_src_slot[limb - n_limbs] << 16) + col;
+        const int rh = threadIdx.x >> 4;
+        u64 t[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) t[k] = from[(size_t)(rh + 16 * k) << 8];
+#pragma unroll
+        for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = t[k];
+        return;
+    }
+    const int prime = ll.idx[limb];
+    const Tw *tw = tw_all + ((size_t)prime << 16);
     const int dg = cs.digit_of[limb], n_src = cs.d[dg].n_src;
     const u64 *src = cs.d[dg].src + (size_t)poly * cs.d[dg].src_poly_stride + col;
     const Cst *hat = cs.d[dg].hat + prime;
@@ -645,10 +657,11 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
             seen[cs.digit_of[l]] = true;
             src_limbs += (size_t)cs.d[cs.digit_of[l]].n_src;
         }
-    account(c, TR_BCONV, src_limbs * n_polys * c->N * 8, 0);
+    if (cs.n_copy < 0 || n_limbs + cs.n_copy > HEMM_MAX_PRIMES) throw std::invalid_argument("too many copied limbs");
+    account(c, TR_BCONV, (src_limbs + 2 * (size_t)cs.n_copy) * n_polys * c->N * 8, 0);
     account(c, TR_NTT, (size_t)(tail ? 2 : 1) * n_limbs * n_polys * c->N * 8, 2);
     const Tw *tw = (const Tw *)c->d_w;
-    const dim3 block(256), grid(16, n_limbs * n_polys);
+    const dim3 block(256), grid(16, (n_limbs + cs.n_copy) * n_polys);
 #define CONV_CASE(K)                                                                                                    \
     hipLaunchKernelGGL(ntt16_cols_converted_kernel<K>, grid, block, 0, s, data, tw, c->d_modq, c->d_ninv, c->d_ninv_s, \
                        c->d_fp, ll, sl, n_limbs, poly_stride, cs)
