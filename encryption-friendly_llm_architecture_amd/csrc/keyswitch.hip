@@ -537,6 +537,8 @@ struct KsTables {
     // conversion follows it.  modup: per chain length nq, limbs 0 .. nq-1 (each limb in its own digit's basis).
     size_t p_invn_off = 0;
     std::vector<size_t> drop_invn_off, modup_invn_off;   // [nq]
+    size_t ones_off = 0;                                 // the constant 1 for every prime (a one-source conversion
+                                                         // with it is a plain reduction into the target prime)
 };
 
 static KsTables *g_tables_of(const hemm_context *c);
@@ -653,6 +655,8 @@ static void build_tables(const hemm_context *c, KsTables &t) {
             invn(t.inv_off[nq][d], src);
         }
     }
+    t.ones_off = t.host.size();
+    for (int pj = 0; pj < T; pj++) t.host.push_back(Cst{1, 0});
     HEMM_HIP(hipMalloc((void **)&t.dev, t.host.size() * sizeof(Cst)));
     HEMM_HIP(hipMemcpy(t.dev, t.host.data(), t.host.size() * sizeof(Cst), hipMemcpyHostToDevice));
 }
@@ -857,6 +861,20 @@ static void rescale_with(hemm_context *c, KsTables *t, u64 *sc, const u64 *in, s
             HEMM_HIP(hipMemcpyAsync(last + (size_t)p * N, in + p * in_stride + (size_t)(nq - 1) * N, N * 8,
                                     hipMemcpyDeviceToDevice, s));
         launch_ntt(c, last, pl, 1, n_polys, N, true, s);
+    }
+    if (c->logN == 16 && lazy_dot_ok(c)) {
+        // the reduction of the last limb's coefficients into every remaining prime is a one-source conversion with
+        // the constant 1: computed inside the first pass of the forward transform
+        ConvSources cs;
+        memset(&cs, 0, sizeof(cs));
+        cs.d[0].src = last;
+        cs.d[0].hat = t->dev + t->ones_off;
+        cs.d[0].src_poly_stride = N;
+        cs.d[0].n_src = 1;
+        cs.hat_ld = c->nQ + c->nP;
+        if (launch_ntt_converted(c, cs, tt, limbs_default(c, nq - 1, 0), ident, nq - 1, n_polys, (size_t)(nq - 1) * N, s,
+                                 in, in_stride, out, out_stride, t->dev + t->qlinv_off[nq - 1]))
+            return;
     }
     dim3 grid(N / 256, (nq - 1) * n_polys), block(256);
     account(c, TR_POINTWISE, (size_t)n_polys * nq * N * 8);
