@@ -130,3 +130,14 @@ def test_attention_head():
     assert out.info()["level"] == 1
     want = (f(S) @ pad(V))[:, :d]
     assert np.abs(H.decrypt(out)[:, :d] - want).max() < 2 ** -8
+
+
+def test_whole_layer_workloads(H):
+    """Both layer-level workloads at their full extent -- every output column group of the LoRA projection (36 weight
+    tile products, 12 CCMMs) and all 12 attention heads (24 CCMMs + 12 polynomial evaluations) -- exactly as the
+    benchmark runs them, every decrypted output against float64 algebra."""
+    import bench
+    out = {}
+    bench.gpu_layer_configs(None, out, H)
+    assert out["config4_max_abs_err"] < 2.0 ** -12
+    assert out["config5_max_abs_err"] < 2.0 ** -12
