@@ -92,12 +92,12 @@ struct ConvSources {
     } d[CONV_MAX_DIGITS];
     int hat_ld;
     uint8_t digit_of[HEMM_MAX_PRIMES];
-    // limbs n_limbs .. n_limbs + n_copy - 1 of the launch's lists are plain copies (first pass only, no transform):
-    // slot copy_src_slot[i] of copy_src (NTT form, polynomial stride copy_src_stride) to slot sl[n_limbs + i] of data
+    // n_copy further limbs of the launch are plain copies (first pass only, no transform): slot copy_src_slot[i] of
+    // copy_src (NTT form, polynomial stride copy_src_stride) to slot copy_dst_slot[i] of data
     const u64 *copy_src;
     size_t copy_src_stride;
     int n_copy;
-    uint8_t copy_src_slot[HEMM_MAX_PRIMES];
+    uint8_t copy_src_slot[HEMM_MAX_PRIMES], copy_dst_slot[HEMM_MAX_PRIMES];
 };
 // data: [n_polys][.][N] (polynomial stride poly_stride), limb l written to slot sl[l].  With ep_* set the second pass
 // ends with out = (minuend - transform) * cst[l] (slots of minuend / out = l) and data is only a workspace.

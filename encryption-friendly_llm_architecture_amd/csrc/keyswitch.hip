@@ -1024,7 +1024,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
                                   (size_t)(hi - lo) * N * 8, n_in, hipMemcpyDeviceToDevice, s));
     }
     if (!joint) return;
-    if (fold && n_joint + nq <= HEMM_MAX_PRIMES) {
+    if (fold) {
         // the conversions of all digits inside the first pass of the forward transform; the same launch copies every
         // digit's own limbs into its slice
         ConvSources cs;
@@ -1044,7 +1044,7 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         cs.n_copy = nq;
         for (int j = 0; j < nq; j++) {
             cs.copy_src_slot[j] = (uint8_t)j;
-            js.idx[n_joint + j] = (uint8_t)((j / alpha) * E + j);
+            cs.copy_dst_slot[j] = (uint8_t)((j / alpha) * E + j);
         }
         if (launch_ntt_converted(c, cs, ext, jp, js, n_joint, n_in, (size_t)beta * E * N, s)) return;
     }

@@ -439,10 +439,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int per_poly = n_limbs + cs.n_copy;
     const int limb = blockIdx.y % per_poly, poly = blockIdx.y / per_poly;
     const size_t col = blockIdx.x * 16 + (threadIdx.x & 15);
-    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + col;
     if (limb >= n_limbs) {   // a limb that is only copied into its slot
         const u64 *from = cs.copy_src + (size_t)poly * cs.copy_src_stride +
                           ((size_t)cs.copy_src_slot[limb - n_limbs] << 16) + col;
+        u64 *base = data + (size_t)poly * poly_stride + ((size_t)cs.copy_dst_slot[limb - n_limbs] << 16) + col;
         const int rh = threadIdx.x >> 4;
         u64 t[16];
 #pragma unroll
@@ -451,6 +451,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = t[k];
         return;
     }
+    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + col;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
     const int dg = cs.digit_of[limb], n_src = cs.d[dg].n_src;
@@ -657,7 +658,8 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
             seen[cs.digit_of[l]] = true;
             src_limbs += (size_t)cs.d[cs.digit_of[l]].n_src;
         }
-    if (cs.n_copy < 0 || n_limbs + cs.n_copy > HEMM_MAX_PRIMES) throw std::invalid_argument("too many copied limbs");
+    if (n_limbs > HEMM_MAX_PRIMES || cs.n_copy < 0 || cs.n_copy > HEMM_MAX_PRIMES)
+        throw std::invalid_argument("too many limbs in one converted transform");
     account(c, TR_BCONV, (src_limbs + 2 * (size_t)cs.n_copy) * n_polys * c->N * 8, 0);
     account(c, TR_NTT, (size_t)(tail ? 2 : 1) * n_limbs * n_polys * c->N * 8, 2);
     const Tw *tw = (const Tw *)c->d_w;
