@@ -140,6 +140,37 @@ def test_keyswitch_stages(S, drop):
     assert np.array_equal(want[0], ob) and np.array_equal(want[1], oa)
 
 
+@pytest.mark.parametrize("log_n", [10, 16])
+def test_keyswitch_and_rescale_with_primes_above_2_60(log_n):
+    """Primes of 2^60 and more leave the lazy dot products of the conversion kernels (8 terms of 60 x 60 bits) and the
+    conversions inside the transforms: the generic conversion kernel and the separate launches must give the
+    oracle's residues too."""
+    pkg = load_package()
+    big = O.primes_below(61, log_n, 6)
+    assert all(q >> 60 for q in big)
+    qs, ps = big[:4], big[4:]
+    orc = O.Oracle(log_n, qs, ps, 2)
+    ctx = pkg.Context(log_n, qs, ps, 2)
+    N = 1 << log_n
+    rng = np.random.default_rng(61 + log_n)
+    orc.gen_secret(3, hw=min(192, N // 4))
+    orc.gen_mult_key(6)
+    evk = orc.keys["mult"]
+    for nq in (4, 3):
+        E = nq + orc.nP
+        x = rand_limbs(rng, orc.q[:nq], (), N)
+        beta = (nq + orc.alpha - 1) // orc.alpha
+        ext = np.empty((beta, E, N), dtype=np.uint64)
+        orc.L.orc_modup(orc.h, _p(x), nq, _p(ext))
+        assert np.array_equal(host(ctx.modup(dev(x), nq)), ext)
+        ob, oa = orc.keyswitch(x, evk)
+        got = host(ctx.keyswitch(dev(x), dev(evk), nq))
+        assert np.array_equal(got[0], ob) and np.array_equal(got[1], oa)
+        ct = rand_limbs(rng, orc.q[:nq], (2,), N)
+        want = orc.rescale(O.Ct(ct, 1.0)).data
+        assert np.array_equal(host(ctx.rescale(dev(ct), nq)), want)
+
+
 def test_rotate_relinearize_rescale(S):
     orc, ctx, N = S.orc, S.ctx, S.N
     nq = orc.nQ - 1
