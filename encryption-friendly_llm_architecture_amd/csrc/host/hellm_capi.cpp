@@ -553,6 +553,12 @@ int hellm_complex_packing_rev(hellm_hemmer *h, const hellm_ct *a, const hellm_ct
     *out = new hellm_ct{h->m->complexPackingRev(a->t, b->t)};
     FACADE_CATCH
 }
+int hellm_complex_packing_pt(hellm_hemmer *h, const hellm_pt *a, const hellm_pt *b, hellm_pt **out) {
+    FACADE_TRY
+    need(h && a && b && out, "null argument");
+    *out = new hellm_pt{h->m->complexPacking(a->t, b->t)};
+    FACADE_CATCH
+}
 int hellm_repack_not_bts(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out) {
     FACADE_TRY
     need(h && a && b && out, "null argument");

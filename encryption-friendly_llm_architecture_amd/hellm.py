@@ -53,7 +53,7 @@ def _L():
                   "hellm_diagonal_to_row"):
             getattr(L, n).argtypes = [vp, vp, pvp]
         for n in ("hellm_mult", "hellm_add", "hellm_complex_packing", "hellm_complex_packing_rev",
-                  "hellm_repack_not_bts", "hellm_repack_lora_opti"):
+                  "hellm_complex_packing_pt", "hellm_repack_not_bts", "hellm_repack_lora_opti"):
             getattr(L, n).argtypes = [vp, vp, vp, pvp]
         L.hellm_matmul_high_low.argtypes = [vp, vp, vp, u32, u32, pvp]
         L.hellm_matmul_low_high.argtypes = [vp, vp, vp, u32, u32, pvp]
@@ -450,6 +450,10 @@ class HEMMer:
 
     def complex_packing_rev(self, a, b):
         return self._new(Ct, "hellm_complex_packing_rev", a.h, b.h)
+
+    def complex_packing_pt(self, a, b):
+        """plaintexts: 0.5 a - 0.5 i b (HEMMer::complexPacking(PtxtTensor, PtxtTensor))"""
+        return self._new(Pt, "hellm_complex_packing_pt", a.h, b.h)
 
     def repack_not_bts(self, a, b):
         return self._new(Ct, "hellm_repack_not_bts", a.h, b.h)

@@ -143,6 +143,8 @@ int hellm_packed_matmul_cc_reuse(hellm_hemmer *h, const hellm_ctvec *tmp, const 
 int hellm_repack_cc(hellm_hemmer *h, hellm_ct *a, hellm_ct **out);                                       /* :172 */
 int hellm_complex_packing(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);        /* :176 */
 int hellm_complex_packing_rev(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);    /* :179 */
+/* plaintext pair 0.5 a - 0.5 i b on the decoded values, encoded at the lower of the two levels (HEMMer.hpp:174, src/HEMMer.cpp:971-978) */
+int hellm_complex_packing_pt(hellm_hemmer *h, const hellm_pt *a, const hellm_pt *b, hellm_pt **out);
 int hellm_repack_not_bts(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out);                     /* :186 */
 int hellm_repack_lora_opti(hellm_hemmer *h, hellm_ct *a, hellm_ct *b, hellm_ct **out);                   /* :184 */
 /* LoRA low-rank products and their repacking (HEMMer.hpp:202-232; rank = 2, reference ModelArgs.hpp:67).

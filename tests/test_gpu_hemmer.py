@@ -66,6 +66,22 @@ def test_keys_and_encoding_match_oracle(small):
         assert np.array_equal(H.encode(M, level).residues(), orc.encode(z, level).data)
 
 
+def test_plaintext_pair_packing_bit_exact(small):
+    """HEMMer::complexPacking(PtxtTensor, PtxtTensor): 0.5 a - 0.5 i b, decoded, combined and encoded again at the lower
+    level -- the oracle's decode / encode of the same residues gives the same plaintext."""
+    H, orc, _ = small
+    rng = np.random.default_rng(17)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    a, b = H.encode(A, 5), H.encode(B, 3)
+    p = H.complex_packing_pt(a, b)
+    za = orc.decode(O.Pt(a.residues(), orc.delta[5]))
+    zb = orc.decode(O.Pt(b.residues(), orc.delta[3]))
+    want = orc.encode(0.5 * za - 0.5j * zb, 3)
+    assert np.array_equal(p.residues(), want.data)
+    got = orc.decode(O.Pt(p.residues(), orc.delta[3]))[:256].reshape(16, 16)
+    assert np.abs(got - (0.5 * A - 0.5j * B)).max() < 1e-9
+
+
 def test_evaluator_calls_bit_exact(small):
     H, orc, ev = small
     rng = np.random.default_rng(2)
