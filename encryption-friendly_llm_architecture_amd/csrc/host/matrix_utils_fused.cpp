@@ -763,25 +763,56 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     std::vector<bool> started((size_t)n_giant, false);
     started[0] = true;
     const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
-    DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl);
-    for (size_t first = 0; first < sa.size(); first += G) {
-        const size_t cnt = std::min(G, sa.size() - first);
-        std::vector<hemm_rot_term> terms;
-        std::vector<uint32_t> off{0};
-        pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
-        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, ya.data(), t1.data(), lo * N, ws.data(), nullptr));
+    // Chains of G shifts.  When the shifts split into exactly two chains, they are cut on a giant-step boundary (so
+    // that they accumulate into different partial sums) and the second runs on the side stream beside the first, with
+    // buffers of its own: each launch of one chain fills the part-empty last round of workgroups of the other's
+    // (measured -1.3 % per product; staggering the chains so that one's inverse transforms meet the other's key
+    // product gained nothing).
+    std::vector<std::pair<size_t, size_t>> chains;   // (first, count)
+    for (size_t first = 0; first < sa.size(); first += G) chains.push_back({first, std::min(G, sa.size() - first)});
+    bool two_streams = false;
+    if (chains.size() == 2) {
+        const size_t cut = ((chains[0].second + 1) / (size_t)g) * (size_t)g;   // shift index q holds i = q + 1
+        if (cut >= 1 && cut - 1 >= 1 && cut - 1 < sa.size() && sa.size() - (cut - 1) <= G && cut - 1 <= G) {
+            chains[0] = {0, cut - 1};
+            chains[1] = {cut - 1, sa.size() - (cut - 1)};
+            two_streams = true;
+        }
+    }
+    DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl), ya2, t12, ws2;
+    if (two_streams) {
+        ya2 = DeviceBuffer(c, G * 2 * E * N);
+        t12 = DeviceBuffer(c, G * ctl);
+        ws2 = DeviceBuffer(c, G * ctl);
+    }
+    auto accumulate = [&](size_t first, size_t cnt, const u64 *tb, hipStream_t st) {
         // shift index q holds i = q + 1: consecutive i with the same i2 pair with consecutive baby rotations
         size_t q = first;
         while (q < first + cnt) {
             const i64 ii = (i64)q + 1, i2 = ii / g, i1 = ii % g;
             const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - i1));
-            ck(hemm_tensor_batch_strided(c->dev, t1.data() + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
+            ck(hemm_tensor_batch_strided(c->dev, tb + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
                                          (uint32_t)lo, U_out->data() + (u64)i2 * pw, us, started[(size_t)i2] ? 1 : 0,
-                                         nullptr));
+                                         st));
             started[(size_t)i2] = true;
             q += run;
         }
+    };
+    // forked before the first chain is queued: the side stream waits only for what both chains depend on
+    const hipStream_t side2 = two_streams ? c->forkSide() : nullptr;
+    for (size_t ch = 0; ch < chains.size(); ch++) {
+        const size_t first = chains[ch].first, cnt = chains[ch].second;
+        const bool on_side = two_streams && ch == 1;
+        const hipStream_t st = on_side ? side2 : nullptr;
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1,
+                                on_side ? ya2.data() : ya.data(), on_side ? t12.data() : t1.data(), lo * N,
+                                on_side ? ws2.data() : ws.data(), st));
+        accumulate(first, cnt, on_side ? t12.data() : t1.data(), st);
     }
+    if (two_streams) c->joinSide();
     *g_out = g;
 }
 
