@@ -522,8 +522,8 @@ def cpu_baseline(out):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--roofline-only", action="store_true", help="run only the roofline legs")
     ap.add_argument("--ccmm-only", action="store_true", help="run only the headline product loop (for kernel traces)")
