@@ -215,10 +215,13 @@ void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a, 
 void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &transformer, const Ciphertext &a, const Ciphertext &b,
                         i64 w, Ciphertext &pa, Ciphertext &pb, u64 pack_level = ~u64(0));
 // complexPackingPair at min(levels, target_level + 5) followed by multPackedMatMatFused, the packed pair passed on in
-// place: the complex product of two plain n x n tiles (its real part, x + conj(x), is A B); needs level >= T+4
+// place: the complex product of two plain n x n tiles (its real part, x + conj(x), is A B); needs level >= T+3.
+// add_conj: returns x + conj(x) itself; where the schedule ends in a giant-step sum the conjugated terms join that sum
+// (keys of every giant rotation's Galois element times 2N - 1, plain and square, and the square key of 2N - 1:
+// KeyGenerator::genGaloisKey / genGaloisSquareKey), otherwise the result is conjugated and added.
 CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &a,
                                         const CtxtTensor &b, u64 target_level, MatrixTransformer &transformer,
-                                        u64 batch = 16, bool single_tile = false);
+                                        u64 batch = 16, bool single_tile = false, bool add_conj = false);
 // sum_k tmp[k] (x) rho^(k step)(b), relinearised (and rescaled when rescale_after): the ciphertext x ciphertext re-use
 // forms (multMatMatCCReUse: step = block width; multPackedMatMatCCReuse: step = 2 block widths, rescale) with all
 // rotations of b taken from ONE ModUp through direct keys, in batches of hoisted sums

@@ -229,6 +229,9 @@ public:
     void genLeftRotKey(u64 rot) const;
     void genRightRotKey(u64 rot) const;
     void genLeftRotSquareKey(u64 rot) const;   // KeyPack::galoisSquareKey of a left rotation (not in HEaaN)
+    // keys by Galois element (not in HEaaN): of X -> X^g for any odd g, e.g. a rotation followed by the conjugation
+    void genGaloisKey(u64 galois) const;
+    void genGaloisSquareKey(u64 galois) const;
     void genRotKeyBundle() const;   // every power-of-two left and right rotation
     void genCommonKeys() const;     // mult + conj + power-of-two rotations
     void genRotKeysForBootstrap(u64) const {}  // bootstrapping is outside this build

@@ -533,11 +533,21 @@ void KeyGenerator::genLeftRotKey(u64 rot) const {
     gen_galois(*this, ctx_, sk_, g, sg);
     genSwitchKey(g, sg.data(), pack_.galois_[g]);
 }
-// key id of a square key: the Galois element with bit 40 set (Galois elements are below 2N <= 2^18)
+void KeyGenerator::genGaloisKey(u64 g) const {
+    if (g % 2 == 0 || g >= 2 * ctx_->N) throw RuntimeException("a Galois element is odd and below 2N");
+    if (g == 1 || pack_.hasGaloisKey(g)) return;
+    DeviceBuffer sg;
+    gen_galois(*this, ctx_, sk_, g, sg);
+    genSwitchKey(g, sg.data(), pack_.galois_[g]);
+}
 void KeyGenerator::genLeftRotSquareKey(u64 rot) const {
     const u64 slots = ctx_->N / 2;
     rot %= slots;
-    const u64 g = rot == 0 ? 1 : galois_of_rotation(ctx_, rot);
+    genGaloisSquareKey(rot == 0 ? 1 : galois_of_rotation(ctx_, rot));
+}
+// key id of a square key: the Galois element with bit 40 set (Galois elements are below 2N <= 2^18)
+void KeyGenerator::genGaloisSquareKey(u64 g) const {
+    if (g % 2 == 0 || g >= 2 * ctx_->N) throw RuntimeException("a Galois element is odd and below 2N");
     if (pack_.hasGaloisSquareKey(g)) return;
     const size_t T = ctx_->nQ + ctx_->nP;
     DeviceBuffer s2(ctx_, T * ctx_->N), sg(ctx_, T * ctx_->N);

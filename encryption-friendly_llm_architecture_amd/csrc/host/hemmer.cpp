@@ -481,8 +481,25 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, sq, true, spread));
             KeyGenerator kg(context_, sk_, pack_);
             for (u64 r : sq) kg.genLeftRotSquareKey(r);
-            CtxtTensor prod = multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, spread);
-            CtxtTensor res = repackCC(prod);
+            // x + conj(x) inside the product: its giant-step sum (exact row rotations: the block fills the slot vector
+            // or is spread over it) takes every term a second time under the Galois element times 2N - 1
+            if (block == slots || spread) {
+                const u64 two_n = 4 * slots, cj = two_n - 1;   // 2N with N = 2 * slots
+                auto galois = [&](u64 r) {   // 5^r mod 2N
+                    u64 g = 1, b = 5 % two_n;
+                    for (r %= slots; r; r >>= 1, b = b * b % two_n)
+                        if (r & 1) g = g * b % two_n;
+                    return g;
+                };
+                kg.genConjKey();
+                kg.genGaloisSquareKey(cj);
+                for (u64 r : sq) {
+                    const u64 gc = (galois(r) * cj) % two_n;
+                    kg.genGaloisKey(gc);
+                    kg.genGaloisSquareKey(gc);
+                }
+            }
+            CtxtTensor res = multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, spread, true);
             if (spread) res.get().occupied_ = block;
             return res;
         }

@@ -820,8 +820,11 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
 // the terms (d1 under the key of rho(s), d2 under the key of rho(s)^2); U_0 gives its d2 under the multiplication key
 // with the identity automorphism, and its d1 is added to the second polynomial of the sum, times P, before the
 // single ModDown merged with the rescale.
+// add_conj: the result is x + conj(x) for the sum x described above -- every term enters a second time under its
+// Galois element times 2N - 1 (keys of the composite elements; d1 of U_0, which needs no key switch in x, is switched
+// under the conjugation key), so the real part of a complex-packed product needs no key-switch round of its own.
 void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64 n_giant, i64 ru, Ciphertext &acc,
-                    CtxtTensor &res) {
+                    CtxtTensor &res, bool add_conj = false) {
     const Context &c = eval.getContext();
     const u64 N = c->N, K = c->nP, lo = T + 1;
     const KeyPack &pack = eval.getKeyPack();
@@ -879,6 +882,23 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         t.evk = pack.galoisSquareKey(gal);
         terms.push_back(t);
     }
+    if (add_conj) {
+        const u64 cj = 2 * N - 1;
+        for (u64 i = 0; i < m; i++) {
+            const u64 gal = i == 0 ? 1 : rot.galois((i64)i * g * ru), gc = (gal * cj) % (2 * N);
+            hemm_rot_term t{};
+            t.ext = ext1 + i * beta * El * N;
+            t.b = U.data() + i * pw;
+            t.evk = pack.galoisKey(gc);
+            t.mask = nullptr;
+            t.galois = gc;
+            terms.push_back(t);
+            t.ext = ext2 + i * beta * El * N;
+            t.b = nullptr;
+            t.evk = pack.galoisSquareKey(gc);
+            terms.push_back(t);
+        }
+    }
     const uint32_t off[2] = {0, (uint32_t)terms.size()};
     res.get().allocate(2, T, 0);
     DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * lo * N);
@@ -918,7 +938,7 @@ void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphert
 namespace {
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre = nullptr,
-                     u64 pre_level = 0, bool merge_packing = false);
+                     u64 pre_level = 0, bool merge_packing = false, bool add_conj = false);
 }
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
@@ -932,9 +952,11 @@ namespace {
 // merge_packing (with packed): the operands are NOT packed yet; the complex packing and the packed transform run as one
 // composite one-stage transform from T+3 (MaskKind::PackingHorizontal / PackingVertical), for operands with only
 // three levels above the target.
+// add_conj: the result is x + conj(x) of the product x (the real part, twice, of a complex-packed product): inside the
+// giant-step sum where the schedule has one, by a conjugation afterwards otherwise.
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre, u64 pre_level,
-                     bool merge_packing) {
+                     bool merge_packing, bool add_conj) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -1010,6 +1032,11 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     auto finish = [&]() {
         eval.relinearize(acc, res.get());
         eval.rescale(res.get());
+        if (add_conj) {
+            Ciphertext cj(c);
+            eval.conjugate(res.get(), cj);
+            eval.add(res.get(), cj, res.get());
+        }
     };
     if (k / cu <= 1) {
         finish();
@@ -1025,7 +1052,7 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
         i64 g = 1;
         bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n / cu, cu, w, batch, &U, &g,
                          spread ? (u64)(n * w) : 0, true);
-        bsgsGiantSteps(eval, T, U, g, (n / cu) / g, cu * w, acc, res);
+        bsgsGiantSteps(eval, T, U, g, (n / cu) / g, cu * w, acc, res, add_conj);
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
@@ -1234,7 +1261,8 @@ void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &tr, const C
 }
 
 CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &a,
-                                        const CtxtTensor &b, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
+                                        const CtxtTensor &b, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile,
+                                        bool add_conj) {
     const Context &c = eval.getContext();
     if (a.get().getRescaleCounter() != 0 || b.get().getRescaleCounter() != 0 || a.get().getNumPoly() != 2 ||
         b.get().getNumPoly() != 2)
@@ -1243,7 +1271,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
     // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
     if (std::min(a.getLevel(), b.getLevel()) == T + 3)
-        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true);
+        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true, add_conj);
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
     // is handed to the product where it lies.  Operands above the packing level are only truncated to it (a copy of
     // their first L+1 limbs): the packing masks absorb the change of scale, which saves the levelDown.
@@ -1258,7 +1286,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     const bool by_rows[2] = {false, true};
     const u64 from[2] = {a.getLevel(), b.getLevel()};
     tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data(), from);
-    return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1);
+    return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1, false, add_conj);
 }
 
 // Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and

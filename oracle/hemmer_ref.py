@@ -778,12 +778,14 @@ def _assemble_shifts(orc, src, ext, back, shifts):
     return out
 
 
-def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0):
+def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0, with_conj=False):
     """Baby-step / giant-step sum over the shift index i = i1 + g i2 (column shift cu * i slots, row rotation
     i * cu * w slots); `acc` holds the i = 0 term, a = sigma(A) at T+2, b_low = tau(B) at T+1.
     spread_block: tau(B) holds one tile block of that many slots and nothing else; every baby rotation then
     also gathers the copies rho^(-j spread_block) (further terms of the same hoisted sum), i.e. it is the
-    rotation of tau(B) copied into every block."""
+    rotation of tau(B) copied into every block.
+    with_conj: returns x + conj(x) of that sum x: every term of the giant-step sum enters a second time under its
+    Galois element times 2N - 1 (d1 of U_0, which needs no key switch in x, under the conjugation key)."""
     from .oracle import Ct
     ru = cu * w
     g = bsgs_baby_count(units)
@@ -816,6 +818,13 @@ def _bsgs_shift_product(orc, a, b_low, acc, cm, n, units, cu, w, spread_block=0)
         u = U[i2]
         terms.append((orc.modup(u.data[1]), u.data[0], ("g", gal), None))
         terms.append((orc.modup(u.data[2]), None, ("sq", gal), None))
+    if with_conj:
+        cj, two_n = 2 * orc.N - 1, 2 * orc.N
+        for i2 in range(units // g):
+            gal = 1 if i2 == 0 else orc.galois((i2 * g * ru) % orc.slots)
+            u = U[i2]
+            terms.append((orc.modup(u.data[1]), u.data[0], ("g", gal * cj % two_n), None))
+            terms.append((orc.modup(u.data[2]), None, ("sq", gal * cj % two_n), None))
     y = orc.hoisted_sum(terms, lo)
     y[1, :lo] = orc.add_residues(y[1, :lo], orc.mul_p_residues(U[0].data[1]))
     return Ct(orc.moddown_drop(y, lo, False), orc.delta[b_low.level - 1])
@@ -853,10 +862,12 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     return orc.rescale(orc.relinearize(acc))
 
 
-def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False):
+def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False, with_conj=False):
     """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused).
     merge_packing: a and b are NOT packed yet; the packing and the packed transform run as one composite one-stage
-    transform from T+3 (kinds PKH / PKV)."""
+    transform from T+3 (kinds PKH / PKV).
+    with_conj: returns x + conj(x) of the product x -- inside the giant-step sum where the schedule has one, by a
+    conjugation afterwards otherwise."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
@@ -882,14 +893,15 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packi
                                   [(2 * i * w, rm[4 * i + 1], rm[4 * i]) for i in range(1, n // 2)])
             for x, y in zip(ta, tb):
                 acc = orc.add(acc, orc.tensor(x, y))
-            return orc.rescale(orc.relinearize(acc))
+            res = orc.rescale(orc.relinearize(acc))
+            return repack_cc(ev, res) if with_conj else res
         b = orc.level_down_one(b)
     else:
         a = lower_and_transform_fused(orc, a, PH, n, w, T + 2)
         b = lower_and_transform_fused(orc, b, PV, n, w, T + 1)
     # the k = 0 term joins the accumulator at the shifts' level
     acc = orc.tensor(orc.level_down_one(a), b)
-    return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0)
+    return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0, with_conj)
 
 
 def packing_maps(slots, w, rows):
@@ -931,12 +943,12 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     from .oracle import Ct
     ev = OracleEval(orc)
     if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
-        return repack_cc(ev, mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True))
+        return mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True, with_conj=True)
     lvl = min(a.level, b.level, T + 5)
     cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
     pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
     pb = complex_packing_hoisted(orc, cut(b), w, rows=True)
-    return repack_cc(ev, mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile))
+    return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True)
 
 
 def mult_mat_mat_cc_packed_single(orc, a, b, T, n, w):
