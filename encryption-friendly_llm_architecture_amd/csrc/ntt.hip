@@ -642,6 +642,8 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
                           int n_limbs, int n_polys, size_t poly_stride, hipStream_t s, const u64 *ep_minuend,
                           size_t ep_minuend_stride, u64 *ep_out, size_t ep_out_stride, const void *ep_cst_dev) {
     if (c->logN != 16) return false;
+    if (n_limbs > HEMM_MAX_PRIMES || cs.n_copy < 0 || cs.n_copy > HEMM_MAX_PRIMES)
+        throw std::invalid_argument("too many limbs in one converted transform");
     int widest = 0;
     for (int l = 0; l < n_limbs; l++) {
         if (cs.digit_of[l] >= CONV_MAX_DIGITS) throw std::invalid_argument("conversion digit out of range");
@@ -658,8 +660,8 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
             seen[cs.digit_of[l]] = true;
             src_limbs += (size_t)cs.d[cs.digit_of[l]].n_src;
         }
-    if (n_limbs > HEMM_MAX_PRIMES || cs.n_copy < 0 || cs.n_copy > HEMM_MAX_PRIMES)
-        throw std::invalid_argument("too many limbs in one converted transform");
+    if ((size_t)(n_limbs + cs.n_copy) * (size_t)n_polys > 65535)
+        return false;   // more workgroup rows than one launch holds: the caller converts and transforms separately
     account(c, TR_BCONV, (src_limbs + 2 * (size_t)cs.n_copy) * n_polys * c->N * 8, 0);
     account(c, TR_NTT, (size_t)(tail ? 2 : 1) * n_limbs * n_polys * c->N * 8, 2);
     const Tw *tw = (const Tw *)c->d_w;
