@@ -591,6 +591,29 @@ def test_full_ccmm_128(full, fused):
     assert np.abs(H.decrypt(c2) - 2 * (A @ B)).max() < TOL
 
 
+def test_full_ccmm_batch_sizes_give_the_same_residues(full):
+    """The batch size only decides how the shifts are cut into launch chains (two concurrent chains of kernel-argument
+    term lists at the default 16; one chain with a staged term list at 32; four chains one after the other at 8): every
+    residue of the product is the same."""
+    H = full
+    rng = np.random.default_rng(5)
+    A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    ref = None
+    try:
+        for batch in (16, 32, 8):
+            H.set_schedule(True, batch=batch)
+            c = H.single_cc_matmul(ca, cb, 4)
+            r = c.residues()
+            if ref is None:
+                ref = r
+                assert np.abs(H.decrypt(c) - A @ B).max() < TOL
+            else:
+                assert np.array_equal(r, ref), batch
+    finally:
+        H.set_schedule(True)
+
+
 def test_full_pcmm_packed_and_hoisted(full):
     H = full
     rng = np.random.default_rng(2)
