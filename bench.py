@@ -527,6 +527,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--roofline-only", action="store_true", help="run only the roofline legs")
     ap.add_argument("--ccmm-only", action="store_true", help="run only the headline product loop (for kernel traces)")
+    ap.add_argument("--rotation-only", action="store_true",
+                    help="run only the single key-switched rotation at the 24 x 60-bit shape (for kernel traces)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only: run it with --gpus 1 "
@@ -544,6 +546,10 @@ def main():
                                "+ 4 special 60-bit primes, dnum=3, scale 2^42, inputs fresh at level 12, "
                                "target level 4, all keys and masks resident in HBM"},
     }
+    if args.rotation_only:
+        gpu_rotation_60bit(args, out)
+        print(json.dumps(out))
+        return
     if args.roofline_only:
         gpu_hoisted(args, out)
         gpu_ntt(args, out)
