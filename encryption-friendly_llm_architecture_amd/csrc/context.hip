@@ -125,7 +125,8 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
         }
         u64 *wt = w.data() + (size_t)i * N * 2, *iwt = iw.data() + (size_t)i * N * 2;
         // Primes below 2^44 run the 2^16-point transform in double precision (exact: see ntt.hip); their
-        // table entries are the doubles (w, w / q) instead of (w, Shoup quotient).
+        // table is the N twiddles as doubles, packed into the first half of the prime's region (8 bytes per twiddle
+        // instead of 16: the row passes read as many twiddle bytes as data, and the quotient w / q costs one multiply).
         const bool fp = (logN == 16) && (q >> 44) == 0;
         auto as_bits = [](double d) {
             u64 b;
@@ -134,10 +135,16 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
         };
         for (int j = 0; j < N; j++) {
             unsigned r = bitrev((unsigned)j, logN);
-            wt[2 * j] = fp ? as_bits((double)pw[r]) : pw[r];
-            wt[2 * j + 1] = fp ? as_bits((double)pw[r] / (double)q) : h_shoup(pw[r], q);
-            iwt[2 * j] = fp ? as_bits((double)ipw[r]) : ipw[r];
-            iwt[2 * j + 1] = fp ? as_bits((double)ipw[r] / (double)q) : h_shoup(ipw[r], q);
+            if (fp) {
+                wt[j] = as_bits((double)pw[r]);
+                iwt[j] = as_bits((double)ipw[r]);
+                wt[N + j] = iwt[N + j] = 0;
+                continue;
+            }
+            wt[2 * j] = pw[r];
+            wt[2 * j + 1] = h_shoup(pw[r], q);
+            iwt[2 * j] = ipw[r];
+            iwt[2 * j + 1] = h_shoup(ipw[r], q);
         }
         ninv[i] = h_invmod((u64)N, q);
         const bool small = (q >> 44) == 0;  // residues and products-by-parts are exact in double precision

@@ -148,9 +148,11 @@ __global__ __launch_bounds__(256) void ntt_generic_kernel(u64 *__restrict__ data
 // has to assemble every 64-bit integer product from 32-bit pieces, so for residues that fit a double
 // exactly the floating-point butterfly is about a third of the instructions.  A product y*w mod q is
 //     c = rint(y * (w/q));  h = fl(y*w);  l = fma(y, w, -h)  [exact low part];  r = fma(-c, q, h) + l
-// Both h - c*q and the final sum are integers far below 2^53, so r is the exact centred residue
-// (|r| <= 0.54 q for |y| < 2^48).  Values stay signed and unreduced through the forward stages (growth
-// 0.54 q per stage); the inverse stages double the sums, so a radix-16 block first reduces its inputs.
+// Both h - c*q and the final sum are integers far below 2^53, so r is an exact residue of y*w, whatever c is.  The
+// quotient w/q is formed as fl(w * fl(1/q)): y * (w/q) is then off by at most |y| * 1.5 * 2^-52, so
+// |r| <= (0.5 + |y| * 1.5 * 2^-52) q -- 0.57 q for |y| < 2^47.5, 0.8 q for |y| < 2^49.7.  Values stay signed and
+// unreduced through the forward stages (growth 0.57 q per stage: below 11 q < 2^48 after all 16); the inverse
+// stages double the sums, so a radix-16 block first reduces its inputs.
 // The last pass maps to [0, q), which makes the stored result identical to the integer path's.
 // Between the two launches of one transform the buffer holds the raw doubles.
 #pragma clang fp contract(off)
@@ -206,13 +208,10 @@ struct IntFieldT {
 
 typedef IntFieldT<false> IntField;
 
-struct __align__(16) TwF {
-    double w, winv;
-};
 
 struct FpField {
     typedef double E;
-    typedef TwF W;
+    typedef double W;   // the twiddle as a double; its quotient w / q is formed on the fly as w * (1 / q)
     double q, qinv, ni, niinv;
     __device__ __forceinline__ FpField(const ModQ *, const u64 *, const u64 *, const double *fp, int prime) {
         q = fp[4 * prime];
@@ -242,7 +241,7 @@ struct FpField {
         return reduce(a);
     }
     __device__ __forceinline__ void ct(E &x, E &y, const W tw, const bool) const {
-        const double v = mulmod(y, tw.w, tw.winv);
+        const double v = mulmod(y, tw, tw * qinv);
         const double u = x;
         x = u + v;
         y = u - v;
@@ -250,12 +249,13 @@ struct FpField {
     __device__ __forceinline__ void gs(E &x, E &y, const W tw) const {
         const double u = x, v = y;
         x = u + v;
-        y = mulmod(u - v, tw.w, tw.winv);
+        y = mulmod(u - v, tw, tw * qinv);
     }
     // A Gentleman-Sande block of four stages doubles the sums: from inputs bounded by B its outputs are bounded by
-    // 16 B (element 0), 8 r (element 1), 4 r, 4 r, 2 r x 4, r x 8 with r = 0.55 q the bound of a product, and the
-    // largest value it multiplies is 16 B.  With only elements 0 and 1 reduced after each block every block starts
-    // from B <= 2.2 q, so nothing exceeds 36 q < 2^50, where the products are still exact.
+    // 16 B (element 0), 8 r (element 1), 4 r, 4 r, 2 r x 4, r x 8 with r the bound of a product, and the largest
+    // value it multiplies is 16 B.  With only elements 0 and 1 reduced after each block every block starts from
+    // B <= 4 r: r <= 0.8 q gives B <= 3.2 q and 16 B <= 51 q < 2^49.7 (q < 2^44), for which r <= 0.8 q holds again;
+    // products of values below 2^50 are still exact.
     __device__ __forceinline__ void after_inverse_block(E (&x)[16]) const {
         x[0] = reduce(x[0]);
         x[1] = reduce(x[1]);
