@@ -200,8 +200,8 @@ def gpu_ntt(args, out):
 # HBM bytes per call of the hoisted sum at the shape below (its two launches together), from two rocprofv3 --pmc runs
 # of `bench.py --roofline-only` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # 1 GiB copy this mode also launches (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0):
-# (2 x (208 852.6 + 172 131.5) + 196 608 + 163 840) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
-HOISTED_TRAFFIC_BYTES = 1149354332
+# (2 x (159 700.4 + 172 140.0) + 196 608 + 163 840) KiB, see profiles/hoisted_terms_and_ntt_roofline_shapes.txt.
+HOISTED_TRAFFIC_BYTES = 1048707891
 
 
 def gpu_hoisted(args, out):
@@ -209,8 +209,8 @@ def gpu_hoisted(args, out):
     of sigma(A) in the extended basis, each the sum of two masked hoisted rotations (of the operand and of its
     copy rotated by -n) under one key (7 chain + 4 special limbs, 2 digits).  The column masks are run tables (their
     NTT form is constant over runs of 256 residues), and a call of this size is two launches over disjoint limbs:
-    hoisted_terms_kernel<1> (the 6 limbs of primes below 2^44, double precision) and hoisted_terms_kernel<2> (the 5
-    limbs of 60-bit primes, integer).  Timed together: the figure is per call."""
+    hoisted_terms_kernel<1, true> (the 6 limbs of primes below 2^44, double precision) and hoisted_terms_kernel<2, true>
+    (the 5 limbs of 60-bit primes, integer); the second template argument says that the keys are in the compact layout.  Timed together: the figure is per call."""
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -229,33 +229,36 @@ def gpu_hoisted(args, out):
     src = [(rnd(beta, E, N), rnd(nq, N)) for _ in range(2)]
     groups = []
     for o in range(n_out):
-        evk, gal = rnd(dnum, 2, T, N), pow(5, o + 1, 2 * N)
+        # keys in the compact layout, as the product's schedule passes them (6 bytes per residue of a prime below 2^44)
+        evk, gal = ctx.compact_key(rnd(dnum, 2, T, N)), pow(5, o + 1, 2 * N)
         groups.append([(src[t][0], src[t][1], evk, rnd(E, N >> shift), gal, shift) for t in range(2)])
     for _ in range(2):
-        ctx.hoisted_terms(groups, nq, b_premultiplied=True)
+        ctx.hoisted_terms(groups, nq, b_premultiplied=True, compact_keys=True)
     torch.cuda.synchronize()
     timer = pkg.Timer()
     iters = 10
     timer.start()
     for _ in range(iters):
-        ctx.hoisted_terms(groups, nq, b_premultiplied=True)
+        ctx.hoisted_terms(groups, nq, b_premultiplied=True, compact_keys=True)
     ms = timer.stop() / iters
-    # algorithmic bytes: per output beta x 2 x E key limbs read + 2 x E limbs written (the mask tables are
-    # 2 x E x 4 KiB per output, a value and its Shoup companion per run: counted, negligible); the two rotation
-    # sources (beta x E + nq limbs each) read once
-    limbs = n_out * (beta * 2 * E + 2 * E) + 2 * (beta * E + nq)
-    alg_bytes = limbs * LIMB_BYTES + n_out * 2 * E * (N >> shift) * 16
+    # algorithmic bytes: per output beta x 2 x E key limbs read (6 of them 6 bytes per residue, 5 of them 8) + 2 x E
+    # limbs written (the mask tables are 2 x E x 4 KiB per output, a value and its Shoup companion per run: counted,
+    # negligible); the two rotation sources (beta x E + nq limbs each) read once
+    n_small = sum(1 for q in qs[:nq] if q < 2 ** 44)
+    key_bytes = beta * 2 * (n_small * 6 + (E - n_small) * 8) * N
+    limbs = n_out * 2 * E + 2 * (beta * E + nq)
+    alg_bytes = n_out * key_bytes + limbs * LIMB_BYTES + n_out * 2 * E * (N >> shift) * 16
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     out["roofline"] = {
-        "kernel": "hoisted_terms_kernel<1> + hoisted_terms_kernel<2> (one hoisted sum of the CCMM main loop: 32 outputs x "
-                  "2 masked sources under one key, 7+4 limbs, 2 digits, run-table masks; double-precision limbs and "
-                  "integer limbs in one launch each)",
+        "kernel": "hoisted_terms_kernel<1, true> + hoisted_terms_kernel<2, true> (one hoisted sum of the CCMM main loop: 32 "
+                  "outputs x 2 masked sources under one compact key, 7+4 limbs, 2 digits, run-table masks; "
+                  "double-precision limbs and integer limbs in one launch each)",
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS, "traffic": HOISTED_TRAFFIC_BYTES,
         "algorithmic_bytes_per_launch": alg_bytes, "avg_ms_per_launch": ms,
     }
     # (b) the hoisted sum of one sigma / tau transform stage, the largest single launch of the product
-    # (hoisted_terms_kernel<0>): 2 outputs (one per operand) at level T+4, each 7 rotations of two masked sources
+    # (hoisted_terms_kernel<0, true>): 2 outputs (one per operand) at level T+4, each 7 rotations of two masked sources
     # under one key, full masks over the extended basis (9 + 4 limbs, 2 digits)
     nq2, E2 = 9, 9 + K
     src2 = [[(rnd(beta, E2, N), rnd(nq2, N)) for _ in range(2)] for _ in range(2)]
@@ -263,19 +266,19 @@ def gpu_hoisted(args, out):
     for o in range(2):
         grp = []
         for r in range(7):
-            evk, gal = rnd(dnum, 2, T, N), pow(5, 8 * o + r + 1, 2 * N)
+            evk, gal = ctx.compact_key(rnd(dnum, 2, T, N)), pow(5, 8 * o + r + 1, 2 * N)
             grp += [(src2[o][t][0], src2[o][t][1], evk, rnd(E2, N), gal, 0) for t in range(2)]
         groups2.append(grp)
     ctx.traffic(reset=True)
-    ctx.hoisted_terms(groups2, nq2, b_premultiplied=True)
+    ctx.hoisted_terms(groups2, nq2, b_premultiplied=True, compact_keys=True)
     stage_bytes = sum(ctx.traffic(reset=True)[0].values())
     torch.cuda.synchronize()
     timer.start()
     for _ in range(iters):
-        ctx.hoisted_terms(groups2, nq2, b_premultiplied=True)
+        ctx.hoisted_terms(groups2, nq2, b_premultiplied=True, compact_keys=True)
     ms2 = timer.stop() / iters
     out["roofline_transform_stage"] = {
-        "kernel": "hoisted_terms_kernel<0> (hoisted sum of one sigma/tau transform stage: 2 outputs x 7 keys x 2 "
+        "kernel": "hoisted_terms_kernel<0, true> (hoisted sum of one sigma/tau transform stage: 2 outputs x 7 compact keys x 2 "
                   "masked sources, full masks, 9+4 limbs, 2 digits)",
         "bound": "hbm", "achieved": stage_bytes / (ms2 * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": stage_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_launch": stage_bytes,

@@ -39,7 +39,7 @@ vp = ctypes.c_void_p
 class RotTerm(ctypes.Structure):
     _fields_ = [("ext", vp), ("b", vp), ("evk", vp), ("mask", vp), ("galois", ctypes.c_uint32),
                 ("mask_shift", ctypes.c_uint32), ("pt", vp), ("pt_galois", ctypes.c_uint32),
-                ("reserved", ctypes.c_uint32)]
+                ("flags", ctypes.c_uint32)]
 
 
 class LinTerm(ctypes.Structure):
@@ -80,6 +80,9 @@ def _declare(L):
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
     L.hemm_compact_mask.argtypes = [vp, vp, u32, u32, vp, ctypes.POINTER(ci), vp]
+    L.hemm_key_compact_words.argtypes = [vp]
+    L.hemm_key_compact_words.restype = ctypes.c_size_t
+    L.hemm_key_compact.argtypes = [vp, vp, vp, vp]
     L.hemm_sum_parts.argtypes = [vp, vp, u32, u32, u32, vp, vp]
 
 
@@ -315,17 +318,27 @@ class Context:
                                       ctypes.byref(ok), vp(0)))
         return table if ok.value else None
 
-    def hoisted_terms(self, groups, nq, b_premultiplied=False):
+    def compact_key(self, evk):
+        """The compact form of a key [dnum][2][nQ+nP][N] that the hoisted sums read (6 bytes per residue of a prime
+        below 2^44): pass it as evk with compact_keys=True (or a list of flags, one per term in order; the library takes
+        one layout per call)."""
+        import torch
+        out = torch.empty(lib().hemm_key_compact_words(self.h), dtype=torch.int64, device=evk.device)
+        check(lib().hemm_key_compact(self.h, vp(evk.data_ptr()), vp(out.data_ptr()), vp(0)))
+        return out
+
+    def hoisted_terms(self, groups, nq, b_premultiplied=False, compact_keys=False):
         """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift[, pt, pt_galois]]) -> y [n_out][2][nq+K][N]"""
         import torch
         flat = [t for g in groups for t in g]
+        flag = (lambda i: compact_keys[i]) if isinstance(compact_keys, (list, tuple)) else (lambda i: compact_keys)
         arr = (RotTerm * len(flat))()
         for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
             shift = more[0] if more else 0
             pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
             arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
                              mask.data_ptr() if mask is not None else None, gal, shift,
-                             pt.data_ptr() if pt is not None else None, pt_gal, 0)
+                             pt.data_ptr() if pt is not None else None, pt_gal, int(flag(i)))
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))
@@ -334,17 +347,18 @@ class Context:
         check(lib().hemm_hoisted_terms(self.h, arr, off, len(groups), nq, vp(y.data_ptr()), int(b_premultiplied), vp(0)))
         return y
 
-    def hoisted_moddown(self, groups, nq, drop_last, b_premultiplied=False):
+    def hoisted_moddown(self, groups, nq, drop_last, b_premultiplied=False, compact_keys=False):
         """hoisted_terms + moddown_batch in one call -> [n_out][2][nq - drop_last][N]"""
         import torch
         flat = [t for g in groups for t in g]
+        flag = (lambda i: compact_keys[i]) if isinstance(compact_keys, (list, tuple)) else (lambda i: compact_keys)
         arr = (RotTerm * len(flat))()
         for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
             shift = more[0] if more else 0
             pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
             arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
                              mask.data_ptr() if mask is not None else None, gal, shift,
-                             pt.data_ptr() if pt is not None else None, pt_gal, 0)
+                             pt.data_ptr() if pt is not None else None, pt_gal, int(flag(i)))
         offs = [0]
         for g in groups:
             offs.append(offs[-1] + len(g))

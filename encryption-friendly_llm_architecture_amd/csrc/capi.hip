@@ -377,7 +377,7 @@ struct RotDev {
     u32 galois, mask_shift;
     const u64 *ext2, *b2, *mask2;
     const u64 *pt;
-    u32 pt_galois, pad;
+    u32 pt_galois, flags;
 };
 static_assert(sizeof(RotDev) == 80, "RotDev must match the kernels' RotTermDev");
 static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
@@ -395,9 +395,11 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
                  "mask_shift needs a run table and must be below log N");
             need(terms[t].pt == nullptr || ((terms[t].pt_galois & 1) && terms[t].pt_galois < 2 * (uint64_t)ctx->N),
                  "pt_galois must be odd and < 2N");
+            need((terms[t].flags & ~(uint32_t)HEMM_ROT_COMPACT_KEY) == 0, "unknown flag in a rotation term");
             RotDev cur{(const u64 *)terms[t].ext, (const u64 *)terms[t].b, (const u64 *)terms[t].evk,
                        (const u64 *)terms[t].mask, (u32)terms[t].galois, terms[t].mask ? (u32)terms[t].mask_shift : 0u,
-                       nullptr, nullptr, nullptr, (const u64 *)terms[t].pt, terms[t].pt ? (u32)terms[t].pt_galois : 1u, 0u};
+                       nullptr, nullptr, nullptr, (const u64 *)terms[t].pt, terms[t].pt ? (u32)terms[t].pt_galois : 1u,
+                       (u32)terms[t].flags};
             if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
                 terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois &&
                 terms[t + 1].mask_shift == terms[t].mask_shift && terms[t + 1].pt == terms[t].pt &&
@@ -419,6 +421,8 @@ static void run_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, con
     std::vector<RotDev> d;
     std::vector<uint32_t> off;
     build_rot_terms(ctx, terms, group_offsets, n_out, d, off);
+    for (const RotDev &t : d)
+        need(t.flags == d[0].flags, "all terms of a hoisted sum must use the same key layout");
     if ((int)d.size() <= hoisted_arg_capacity() && (int)n_out <= hoisted_arg_capacity()) {
         launch_hoisted_terms_args(ctx, d.data(), (int)d.size(), off.data(), (int)n_out, (int)nq, y, b_premultiplied, stream);
         return;
@@ -427,7 +431,16 @@ static void run_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, con
     void *terms_dev = upload_desc(ctx, d.data(), d.size() * sizeof(RotDev), off.data(), (n_out + 1) * sizeof(uint32_t),
                                   &off_dev, stream);
     launch_hoisted_terms(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, y, b_premultiplied, stream, d.data(),
-                         (int)d.size());
+                         (int)d.size(), !d.empty() && (d[0].flags & HEMM_ROT_COMPACT_KEY) != 0);
+}
+
+size_t hemm_key_compact_words(const hemm_context *ctx) { return ctx ? key_compact_words(ctx) : 0; }
+int hemm_key_compact(hemm_context *ctx, const uint64_t *evk, uint64_t *out, void *stream) {
+    HEMM_TRY
+    need(ctx && evk && out, "null operand");
+    launch_key_compact(ctx, (const u64 *)evk, (u64 *)out, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
 }
 
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,

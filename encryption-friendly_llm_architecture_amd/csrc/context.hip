@@ -170,6 +170,10 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
         HEMM_HIP(hipMemcpy(d, h, bytes, hipMemcpyHostToDevice));
         return d;
     };
+    c->key_off.assign(T + 1, 0);
+    for (int i = 0; i < T; i++)
+        c->key_off[i + 1] = c->key_off[i] + (fpc[4 * i] != 0.0 ? 3u : 4u);
+    c->d_key_off = (u32 *)up(c->key_off.data(), c->key_off.size() * 4);
     c->d_w = (u64 *)up(w.data(), w.size() * 8);
     c->d_iw = (u64 *)up(iw.data(), iw.size() * 8);
     c->d_ws = c->d_iws = nullptr;
@@ -189,6 +193,7 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
 
 void hemm_context_free(hemm_context *c) {
     if (!c) return;
+    hipFree(c->d_key_off);
     hipFree(c->d_w);
     hipFree(c->d_iw);
     hipFree(c->d_ninv);

@@ -36,6 +36,10 @@ struct hemm_context {
     u64 *d_scratch;
     size_t scratch_bytes;
     void *d_desc;                   // staging for the term lists of batched calls
+    // compact evaluation keys: offset of every prime's limb inside a (digit, polynomial) slice and, last entry, the
+    // slice size, in units of 2N bytes (a prime below 2^44 takes 6 bytes per residue = 3 units, any other 4)
+    std::vector<u32> key_off;
+    u32 *d_key_off;
     // Algorithmic bytes of everything launched on this context since the last reset, by kind of work: for each
     // launch the operands it has to read once plus the results it has to write once (what a launch of that kind
     // cannot avoid moving), counted on the host when the launch is queued.  A 2^16-point transform counts one
@@ -146,8 +150,10 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
 void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
                         hipStream_t s);
 // terms_host / n_terms: the host copy of the list (only read for the byte accounting; may be nullptr)
+// compact: every term's key is in the compact layout (all terms of a launch use the same layout)
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0);
+                          bool b_premultiplied, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0,
+                          bool compact = false);
 int hoisted_arg_capacity();
 void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
                                int nq, u64 *y, bool b_premultiplied, hipStream_t s);
@@ -157,6 +163,8 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
                        u64 *out, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0);
 // y[o][p][j] = sum_{q < parts} part[o * parts + q][p][j] over the extended basis, y / part: [.][2][nq+K][N]
 void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s);
+size_t key_compact_words(const hemm_context *c);
+void launch_key_compact(const hemm_context *c, const u64 *evk, u64 *out, hipStream_t s);
 int masked_arg_capacity();
 // table[j][r] = mask[j][r << shift]; true when every aligned run of 2^shift residues of the mask is constant
 bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s);

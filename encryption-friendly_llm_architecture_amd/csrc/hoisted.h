@@ -27,8 +27,10 @@ struct RotTermDev {
     const u64 *ext2, *b2, *mask2;
     // optional plaintext factor [E][N] of the whole term, read through its own automorphism (nullptr: none)
     const u64 *pt;
-    u32 pt_galois, pad;
+    u32 pt_galois;
+    u32 flags;        // bit 0: evk is a compact key (see key_limb)
 };
+#define ROT_TERM_COMPACT_KEY 1u
 
 // Accesses to data that is touched once per launch (keys, masks, results): marked non-temporal so they do
 // not push the rotation sources, which every output gathers from, out of the L2.
@@ -98,11 +100,34 @@ __device__ __forceinline__ double u64_to_double(u64 v) {  // v < 2^52
     return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - 4503599627370496.0;
 }
 
+// Evaluation keys come in two layouts.  Plain: [dnum][2][n_full][N] words.  Compact: every residue of a prime below
+// 2^44 takes 6 bytes instead of 8 -- per (digit, polynomial) the limbs sit back to back, a limb of such a prime as
+// N / 2 records of 12 bytes, one per residue pair (n, n+1): the two 32-bit low words, then the two 16-bit high
+// halves in one word; every other limb as N words.  koff[prime] is the limb's offset and koff[n_full] the size of a
+// (digit, polynomial) slice, both in units of 2N bytes.  A key is read once per launch and is most of what a key
+// product moves: a quarter less of it for the double-precision limbs, in one 12-byte load per thread and stream
+// (low and high parts in separate arrays, two loads per stream, ran 15 % slower than plain keys: the kernel is bound
+// by the loads in flight, not by the bytes).
+// (the layout is a property of the launch -- every term of a launch uses the same one -- and a template parameter of
+// the kernels: with both forms behind a run-time test the mixed kernel spilled 24 registers)
+template <bool COMPACT>
+__device__ __forceinline__ const char *key_limb(const RotTermDev &T, const u32 *__restrict__ koff, const int d,
+                                                const int pol, const int prime, const size_t N, const int n_full) {
+    if (COMPACT) return (const char *)T.evk + ((size_t)(d * 2 + pol) * koff[n_full] + koff[prime]) * (2 * N);
+    return (const char *)(T.evk + ((size_t)(d * 2 + pol) * n_full + prime) * N);
+}
+// residues (n, n+1) of a limb of any prime (compact keys: of a prime of 2^44 or more)
+__device__ __forceinline__ ulonglong2 key_pair_u64(const char *limb, const u32 n) {
+    return stream_load2((const u64 *)limb + n);
+}
+typedef u32 u32x3 __attribute__((ext_vector_type(3), aligned(4)));
+
 // One term with two masked sources under one key (integer path): residues (n, n+1) of limb j of
 // <z, evk> + P (mask b + mask2 b2) with z_d = mask * x_d + mask2 * x2_d, canonical.  RUNS: the masks are run tables
 // without a plaintext factor, i.e. constants with a Shoup companion: no wide product and no Barrett step for z_d.
-template <bool RUNS>
-__device__ __forceinline__ void two_source_int(const RotTermDev &T, const ModQ m, const CstList &pmod, const int j,
+template <bool RUNS, bool COMPACT>
+__device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *__restrict__ koff, const ModQ m,
+                                               const CstList &pmod, const int j,
                                                const int prime, const u32 n, const u32 base, const bool swap, int nq,
                                                int E, int beta, int n_full, int logN, int b_premultiplied,
                                                u64 (&rb)[2], u64 (&ra)[2]) {
@@ -145,8 +170,8 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const ModQ m
             z0 = barrett3(t0, m);
             z1 = barrett3(t1, m);
         }
-        const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-        const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+        const ulonglong2 kb = key_pair_u64(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n);
+        const ulonglong2 ka = key_pair_u64(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n);
         add128(pb[0], mul64wide(z0, kb.x));
         add128(pb[1], mul64wide(z1, kb.y));
         add128(pa[0], mul64wide(z0, ka.x));
@@ -194,8 +219,10 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const ModQ m
 }
 
 // Residues (n, n+1) of limb j of both polynomials of output o (integer path), canonical.
+template <bool COMPACT>
 __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ terms,
-                                                 const u32 *__restrict__ group_off, const ModQ m, const CstList &pmod,
+                                                 const u32 *__restrict__ group_off, const u32 *__restrict__ koff,
+                                                 const ModQ m, const CstList &pmod,
                                                  const int j, const int o, const int prime, const u32 n, int nq, int E,
                                                  int beta, int n_full, int logN, int b_premultiplied, u64 (&out_b)[2],
                                                  u64 (&out_a)[2]) {
@@ -212,9 +239,9 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
             u64 rb[2], ra[2];
             if (T.mask_shift != 0 && T.pt == nullptr)
-                two_source_int<true>(T, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+                two_source_int<true, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
             else
-                two_source_int<false>(T, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+                two_source_int<false, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
             acc_b[0] = addmod(acc_b[0], rb[0], m.q);
             acc_b[1] = addmod(acc_b[1], rb[1], m.q);
             acc_a[0] = addmod(acc_a[0], ra[0], m.q);
@@ -229,8 +256,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                 x.x = x.y;
                 x.y = tmp;
             }
-            const ulonglong2 kb = stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n);
-            const ulonglong2 ka = stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n);
+            const ulonglong2 kb = key_pair_u64(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n);
+            const ulonglong2 ka = key_pair_u64(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n);
             add128(sb[0], mul64wide(x.x, kb.x));
             add128(sb[1], mul64wide(x.y, kb.y));
             add128(sa[0], mul64wide(x.x, ka.x));
@@ -324,10 +351,23 @@ __device__ __forceinline__ D2 gather_d2(const u64 *p, const bool swap) {
     }
     return to_d2(v);
 }
+// residues (n, n+1) of a key limb of a prime below 2^44 as doubles
+template <bool COMPACT>
+__device__ __forceinline__ D2 key_pair_fp(const char *limb, const u32 n, const size_t N) {
+    if (!COMPACT) return to_d2(stream_load2((const u64 *)limb + n));
+    // uniform base + 32-bit byte offset: the offsets n * 4 and n * 2 are shared by every key stream of the thread
+    const u32x3 v = __builtin_nontemporal_load((const u32x3 *)(limb + n * 6u));   // one 12-byte load
+    D2 r;
+    r.x = __hiloint2double((int)((v.z & 0xffffu) | 0x43300000u), (int)v.x) - 4503599627370496.0;
+    r.y = __hiloint2double((int)((v.z >> 16) | 0x43300000u), (int)v.y) - 4503599627370496.0;
+    return r;
+}
 #pragma clang fp contract(off)
 // The same residues in double precision (primes below 2^44); out_* are unreduced centred doubles.
+template <bool COMPACT>
 __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ terms,
-                                                const u32 *__restrict__ group_off, const FpMod f, const double p_mod_q,
+                                                const u32 *__restrict__ group_off, const u32 *__restrict__ koff,
+                                                const FpMod f, const double p_mod_q,
                                                 const int j, const int o, const int prime, const u32 n, int nq, int E,
                                                 int beta, int n_full, int logN, int b_premultiplied, double (&out_b)[2],
                                                 double (&out_a)[2]) {
@@ -355,8 +395,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
                 const double z0 = f.mul(m1.x, x1.x) + f.mul(m2.x, x2.x);
                 const double z1 = f.mul(m1.y, x1.y) + f.mul(m2.y, x2.y);
-                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
-                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
+                const D2 kb = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n, N);
+                const D2 ka = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n, N);
                 sb0 += f.mul(z0, kb.x);
                 sb1 += f.mul(z1, kb.y);
                 sa0 += f.mul(z0, ka.x);
@@ -377,8 +417,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
         } else {
             for (int d = 0; d < beta; d++) {
                 const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
-                const D2 kb = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 0) * n_full + prime) * N + n));
-                const D2 ka = to_d2(stream_load2(T.evk + (((size_t)d * 2 + 1) * n_full + prime) * N + n));
+                const D2 kb = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n, N);
+                const D2 ka = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n, N);
                 sb0 += f.mul(x.x, kb.x);
                 sb1 += f.mul(x.y, kb.y);
                 sa0 += f.mul(x.x, ka.x);

@@ -214,10 +214,15 @@ public:
     bool hasGaloisSquareKey(u64 galois) const { return galois_sq_.count(galois) != 0; }
     const u64 *galoisSquareKey(u64 galois) const;
     const Context &getContext() const { return ctx_; }
+    // The compact form of a key for the hoisted sums (hemm_key_compact: 6 bytes per residue of a prime below 2^44),
+    // made on first request and kept beside the plain key.  kind: 0 multiplication key, 1 key of X -> X^galois,
+    // 2 its square key.
+    const u64 *compactKey(int kind, u64 galois) const;
     // internal
     Context ctx_;
     DeviceBuffer mult_;
     std::map<u64, DeviceBuffer> galois_, galois_sq_;
+    mutable std::map<std::pair<int, u64>, DeviceBuffer> compact_;
 };
 
 class KeyGenerator {

@@ -423,6 +423,20 @@ const u64 *KeyPack::galoisSquareKey(u64 g) const {
     if (it == galois_sq_.end()) throw RuntimeException("no square key for Galois element " + std::to_string(g));
     return it->second.data();
 }
+const u64 *KeyPack::compactKey(int kind, u64 g) const {
+    const auto id = std::make_pair(kind, kind == 0 ? u64(0) : g);
+    auto it = compact_.find(id);
+    if (it == compact_.end()) {
+        const u64 *plain = kind == 0 ? multKey() : kind == 1 ? galoisKey(g) : galoisSquareKey(g);
+        DeviceBuffer c(ctx_, hemm_key_compact_words(ctx_->dev));
+        ck(hemm_key_compact(ctx_->dev, plain, c.data(), nullptr));
+        // made once per key, on the default stream: finished before the caller queues its sum on whichever stream (the
+        // side stream does not wait for later work of the default one)
+        hip_ck(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+        it = compact_.emplace(id, std::move(c)).first;
+    }
+    return it->second.data();
+}
 void KeyPack::save(const std::string &dir) const {
     const size_t words = ctx_->dnum * 2 * (ctx_->nQ + ctx_->nP) * ctx_->N;
     std::vector<u64> h(words);

@@ -79,11 +79,24 @@ struct Rot {
     u64 galois(i64 r) const { return powmod(5, norm(r), M); }
 };
 
+// The key of a term of a hoisted sum (kind: 0 multiplication key, 1 key of X -> X^galois, 2 its square key): the
+// compact form, a quarter less to read for the limbs of primes below 2^44, wherever the kernels take it (up to 6
+// digits), else the plain one.
+void set_key(hemm_rot_term &t, const KeyPack &pack, int kind, u64 galois) {
+    if (pack.getContext()->dnum <= 6) {
+        t.evk = pack.compactKey(kind, galois);
+        t.flags = HEMM_ROT_COMPACT_KEY;
+    } else {
+        t.evk = kind == 0 ? pack.multKey() : kind == 1 ? pack.galoisKey(galois) : pack.galoisSquareKey(galois);
+        t.flags = 0;
+    }
+}
+
 hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois, const Plaintext *mask) {
     hemm_rot_term t{};
     t.ext = ext;
     t.b = b;
-    t.evk = pack.galoisKey(galois);
+    set_key(t, pack, 1, galois);
     t.mask = mask ? mask->buf_.data() : nullptr;
     t.galois = (uint32_t)galois;
     t.mask_shift = 0;
@@ -864,7 +877,7 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         hemm_rot_term t{};
         t.ext = ext2;
         t.b = U.data();
-        t.evk = pack.multKey();
+        set_key(t, pack, 0, 0);
         t.mask = nullptr;
         t.galois = 1;
         terms.push_back(t);
@@ -874,13 +887,13 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         hemm_rot_term t{};
         t.ext = ext1 + i * beta * El * N;
         t.b = U.data() + i * pw;
-        t.evk = pack.galoisKey(gal);
+        set_key(t, pack, 1, gal);
         t.mask = nullptr;
         t.galois = gal;
         terms.push_back(t);
         t.ext = ext2 + i * beta * El * N;
         t.b = nullptr;
-        t.evk = pack.galoisSquareKey(gal);
+        set_key(t, pack, 2, gal);
         terms.push_back(t);
     }
     if (add_conj) {
@@ -890,13 +903,13 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
             hemm_rot_term t{};
             t.ext = ext1 + i * beta * El * N;
             t.b = U.data() + i * pw;
-            t.evk = pack.galoisKey(gc);
+            set_key(t, pack, 1, gc);
             t.mask = nullptr;
             t.galois = gc;
             terms.push_back(t);
             t.ext = ext2 + i * beta * El * N;
             t.b = nullptr;
-            t.evk = pack.galoisSquareKey(gc);
+            set_key(t, pack, 2, gc);
             terms.push_back(t);
         }
     }

@@ -238,13 +238,13 @@ u64 shoup_h(u64 w, u64 q) { return (u64)((((unsigned __int128)w) << 64) / q); }
 // (integer path); MODE 0: any limb, path chosen per workgroup.  jmap lists the n_j limbs of the launch.  The integer
 // path keeps 128-bit accumulators and needs more registers, so on large launches the double-precision limbs get a
 // kernel of their own and run at a higher occupancy; small launches stay whole (two part-filled launches cost more).
-template <int MODE>
+template <int MODE, bool COMPACT>
 __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict__ terms,
                                                    const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                    const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                    const LimbList &ll, const CstList &pmod, int nq, int E, int beta,
                                                    int n_full, int logN, int b_premultiplied, int n_out,
-                                                   const LimbList &jmap, int n_j) {
+                                                   const LimbList &jmap, int n_j, const u32 *__restrict__ koff) {
     // A thread owns the residue pair (n, n+1): the automorphism maps an aligned pair to an aligned pair
     // (possibly swapped), so every access is a 16-byte load or store.
     // Work is dealt out by SOURCE chunk.  The automorphism maps aligned 512-coefficient chunks onto aligned
@@ -290,14 +290,14 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
     if (MODE == 1 || (MODE == 0 && fq != 0.0 && beta <= 6)) {
         const FpMod f{fq, fp[4 * prime + 1]};
         double fb[2], fa[2];
-        hoisted_pair_fp(terms, group_off, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E, beta, n_full, logN,
+        hoisted_pair_fp<COMPACT>(terms, group_off, koff, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E, beta, n_full, logN,
                         b_premultiplied, fb, fa);
         rb[0] = f.canonical(fb[0]);
         rb[1] = f.canonical(fb[1]);
         ra[0] = f.canonical(fa[0]);
         ra[1] = f.canonical(fa[1]);
     } else {
-        hoisted_pair_int(terms, group_off, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN, b_premultiplied,
+        hoisted_pair_int<COMPACT>(terms, group_off, koff, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN, b_premultiplied,
                          rb, ra);
     }
     stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, rb[0], rb[1]);
@@ -314,24 +314,25 @@ struct HoistedArgs {
 };
 // Register budget for five waves per SIMD (96 registers): the double-precision form needs 72 and the integer form 96;
 // the mixed form would take 109 and run at four waves, capped it spills two registers and gains a wave.
-template <int MODE>
+template <int MODE, bool COMPACT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
                                                             const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                             LimbList ll, CstList pmod, int nq, int E, int beta,
                                                             int n_full, int logN, int b_premultiplied, int n_out,
-                                                            LimbList jmap, int n_j) {
-    hoisted_terms_body<MODE>(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
-                           n_j);
+                                                            LimbList jmap, int n_j, const u32 *__restrict__ koff) {
+    hoisted_terms_body<MODE, COMPACT>(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
+                           n_j, koff);
 }
-template <int MODE>
+template <int MODE, bool COMPACT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
                                                                  const u32 *__restrict__ group_off, u64 *__restrict__ y,
                                                                  const ModQ *__restrict__ modq,
                                                                  const double *__restrict__ fp, LimbList ll, CstList pmod,
                                                                  int nq, int E, int beta, int n_full, int logN,
-                                                                 int b_premultiplied, int n_out, LimbList jmap, int n_j) {
-    hoisted_terms_body<MODE>(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
-                           n_j);
+                                                                 int b_premultiplied, int n_out, LimbList jmap, int n_j,
+                                                                 const u32 *__restrict__ koff) {
+    hoisted_terms_body<MODE, COMPACT>(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
+                           n_j, koff);
 }
 
 struct LinTermDev {
@@ -943,6 +944,36 @@ void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64
     rescale_with(c, t, sc, in, in_stride, out, out_stride, nq, n_polys, s);
 }
 
+// ---- compact evaluation keys -----------------------------------------------------------------------
+// out: the compact layout the hoisted kernels read (hoisted.h, key_limb) of a plain key [dnum][2][n_full][N]
+__global__ __launch_bounds__(256) void key_compact_kernel(const u64 *__restrict__ evk, char *__restrict__ out,
+                                                          const u32 *__restrict__ koff, const double *__restrict__ fp,
+                                                          int n_full, int logN) {
+    const size_t N = (size_t)1 << logN;
+    const int prime = blockIdx.y % n_full, slice = blockIdx.y / n_full;   // slice = digit * 2 + polynomial
+    const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const ulonglong2 v = *(const ulonglong2 *)(evk + ((size_t)slice * n_full + prime) * N + n);
+    char *limb = out + ((size_t)slice * koff[n_full] + koff[prime]) * (2 * N);
+    if (fp[4 * prime] != 0.0) {
+        u32 *pair = (u32 *)(limb + n * 6);
+        pair[0] = (u32)v.x;
+        pair[1] = (u32)v.y;
+        pair[2] = (u32)(v.x >> 32) | ((u32)(v.y >> 32) << 16);
+    } else {
+        *(ulonglong2 *)(limb + n * 8) = v;
+    }
+}
+size_t key_compact_words(const hemm_context *c) {
+    return (size_t)c->dnum * 2 * c->key_off[c->nQ + c->nP] * (2 * (size_t)c->N) / 8;
+}
+void launch_key_compact(const hemm_context *c, const u64 *evk, u64 *out, hipStream_t s) {
+    if (c->N < 512) throw std::invalid_argument("compact keys need N >= 512");
+    const int n_full = c->nQ + c->nP;
+    account(c, TR_POINTWISE, (size_t)c->dnum * 2 * n_full * c->N * 8 + key_compact_words(c) * 8);
+    hipLaunchKernelGGL(key_compact_kernel, dim3(c->N / 512, c->dnum * 2 * n_full), dim3(256), 0, s, evk, (char *)out,
+                       c->d_key_off, c->d_fp, n_full, c->logN);
+}
+
 // ---- batched / hoisted forms ---------------------------------------------------------------------
 // in: [n_in][.][N] (polynomial stride in_stride, first nq limbs used) -> ext [n_in][beta][nq+K][N], own
 // limbs of every digit filled.  coef: workspace [n_in][nq][N].
@@ -1077,8 +1108,14 @@ static size_t hoisted_bytes(const hemm_context *c, const RotTermDev *t, int n_te
         return true;
     };
     size_t bytes = (size_t)n_out * 2 * E * limb;
+    // key bytes of the launch's limbs per (digit, polynomial): 6 bytes per residue of a prime below 2^44 in a compact key
+    size_t compact_slice = 0;
+    for (int j = 0; j < E; j++) {
+        const int prime = j < nq ? j : c->nQ + (j - nq);
+        compact_slice += (size_t)c->N * ((c->primes[prime] >> 44) == 0 ? 6 : 8);
+    }
     for (int i = 0; i < n_terms; i++) {
-        bytes += (size_t)2 * beta * E * limb;   // the key of the term
+        bytes += (size_t)2 * beta * ((t[i].flags & ROT_TERM_COMPACT_KEY) ? compact_slice : (size_t)E * limb);   // the key
         if (first(t[i].ext)) bytes += (size_t)beta * E * limb;
         if (first(t[i].b)) bytes += (size_t)nq * limb;
         if (first(t[i].ext2)) bytes += (size_t)beta * E * limb;
@@ -1124,11 +1161,13 @@ static bool split_limbs(const hemm_context *c, int nq, int beta, int n_out, Limb
 }
 
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
-                          bool b_premultiplied, hipStream_t s, const void *terms_host, int n_terms) {
+                          bool b_premultiplied, hipStream_t s, const void *terms_host, int n_terms, bool compact) {
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     if (terms_host != nullptr) account(c, TR_KEYPROD, hoisted_bytes(c, (const RotTermDev *)terms_host, n_terms, n_out, nq));
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
+    // with more than 6 digits the limbs of primes below 2^44 go through the integer path, which reads whole words
+    if (compact && beta > 6) throw std::invalid_argument("compact keys need at most 6 digits");
     LimbList fpl, il, all;
     int n_fp, n_int;
     const bool split = split_limbs(c, nq, beta, n_out, fpl, n_fp, il, n_int, all);
@@ -1137,15 +1176,24 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     const LimbList ll = limbs_default(c, nq, 1);
     const RotTermDev *td = (const RotTermDev *)terms_dev;
     const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
+#define HOISTED_LIST(MODE, COMPACT, GRID, JM, NJ)                                                                    \
+    hipLaunchKernelGGL((hoisted_terms_list_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, td, group_off_dev, y, \
+                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
     if (!split) {
-        hipLaunchKernelGGL(hoisted_terms_list_kernel<0>, dim3((unsigned)(per_limb * E)), block, 0, s, td, group_off_dev, y,
-                           c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, all, E);
+        if (compact)
+            HOISTED_LIST(0, true, per_limb * E, all, E);
+        else
+            HOISTED_LIST(0, false, per_limb * E, all, E);
         return;
     }
-    hipLaunchKernelGGL(hoisted_terms_list_kernel<1>, dim3((unsigned)(per_limb * n_fp)), block, 0, s, td, group_off_dev, y,
-                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, fpl, n_fp);
-    hipLaunchKernelGGL(hoisted_terms_list_kernel<2>, dim3((unsigned)(per_limb * n_int)), block, 0, s, td, group_off_dev, y,
-                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, il, n_int);
+    if (compact) {
+        HOISTED_LIST(1, true, per_limb * n_fp, fpl, n_fp);
+        HOISTED_LIST(2, true, per_limb * n_int, il, n_int);
+    } else {
+        HOISTED_LIST(1, false, per_limb * n_fp, fpl, n_fp);
+        HOISTED_LIST(2, false, per_limb * n_int, il, n_int);
+    }
+#undef HOISTED_LIST
 }
 // the same with the term list (host memory, already merged: n_terms <= HOISTED_ARG_TERMS, n_out <= HOISTED_ARG_TERMS)
 // passed in the kernel arguments
@@ -1168,15 +1216,26 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     const size_t per_limb = (size_t)n_out * (c->N / 512);
     const LimbList ll = limbs_default(c, nq, 1);
     const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
+    const bool compact = n_terms > 0 && (((const RotTermDev *)terms_host)[0].flags & ROT_TERM_COMPACT_KEY) != 0;
+    if (compact && beta > 6) throw std::invalid_argument("compact keys need at most 6 digits");
+#define HOISTED_ARGS(MODE, COMPACT, GRID, JM, NJ)                                                                     \
+    hipLaunchKernelGGL((hoisted_terms_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, a, y, c->d_modq, c->d_fp, \
+                       ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
     if (!split) {
-        hipLaunchKernelGGL(hoisted_terms_kernel<0>, dim3((unsigned)(per_limb * E)), block, 0, s, a, y, c->d_modq, c->d_fp, ll,
-                           pm, nq, E, beta, n_full, c->logN, pre, n_out, all, E);
+        if (compact)
+            HOISTED_ARGS(0, true, per_limb * E, all, E);
+        else
+            HOISTED_ARGS(0, false, per_limb * E, all, E);
         return;
     }
-    hipLaunchKernelGGL(hoisted_terms_kernel<1>, dim3((unsigned)(per_limb * n_fp)), block, 0, s, a, y, c->d_modq, c->d_fp, ll, pm,
-                       nq, E, beta, n_full, c->logN, pre, n_out, fpl, n_fp);
-    hipLaunchKernelGGL(hoisted_terms_kernel<2>, dim3((unsigned)(per_limb * n_int)), block, 0, s, a, y, c->d_modq, c->d_fp, ll, pm,
-                       nq, E, beta, n_full, c->logN, pre, n_out, il, n_int);
+    if (compact) {
+        HOISTED_ARGS(1, true, per_limb * n_fp, fpl, n_fp);
+        HOISTED_ARGS(2, true, per_limb * n_int, il, n_int);
+    } else {
+        HOISTED_ARGS(1, false, per_limb * n_fp, fpl, n_fp);
+        HOISTED_ARGS(2, false, per_limb * n_int, il, n_int);
+    }
+#undef HOISTED_ARGS
 }
 
 // y: [n_polys][nq+K][N] NTT (dropped limbs are clobbered).  drop_last = 0: out[p] = y[p] / P over nq limbs;

@@ -160,8 +160,18 @@ typedef struct {
     const uint64_t *pt;   /* [nq+n_p][N] or NULL: a second plaintext factor over the extended basis, read through
                            * the automorphism pt_galois (the rotated weight of a plaintext-ciphertext product) */
     uint32_t pt_galois;   /* odd, < 2N; 1 = as stored */
-    uint32_t reserved;    /* 0 */
+    uint32_t flags;       /* 0, or HEMM_ROT_COMPACT_KEY: evk is the compact form written by hemm_key_compact */
 } hemm_rot_term;
+#define HEMM_ROT_COMPACT_KEY 1u
+/* Compact form of an evaluation key for the hoisted sums (hemm_hoisted_terms / hemm_hoisted_moddown), which read a key
+ * once per launch and move little else: residues of primes below 2^44 take 6 bytes instead of 8 (per digit and
+ * polynomial the limbs back to back; such a limb as N/2 records of 12 bytes, one per residue pair: two 32-bit low
+ * words, then the two 16-bit high halves in one word; any other limb as N words).  Needs N >= 512 and at most 6
+ * digits per key switch.  All terms of one call use the same layout.  out: hemm_key_compact_words(ctx) words.  The
+ * plain key stays valid and is what every other call takes.
+ * No counterpart in HEaaN's interface (its key storage is not exposed). */
+size_t hemm_key_compact_words(const hemm_context *ctx);
+int hemm_key_compact(hemm_context *ctx, const uint64_t *evk, uint64_t *out, void *stream);
 /* Algorithmic bytes of everything queued on this context since the last reset, by kind of work (for each launch: the
  * operands it must read once plus the results it must write once; a two-launch 2^16-point transform counts one read
  * and one write per limb), and the number of launches; counted on the host, costs nothing on the device.  Kinds:

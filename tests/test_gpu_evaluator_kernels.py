@@ -253,6 +253,18 @@ def test_batched_hoisted_forms(S):
     shared_pb = [[(dext[0], pbs[0], dk[g1], dm1, g1), (dext[1], pbs[1], dk[g1], dm2, g1),
                   (dext[2], pbs[2], dk[g3], dm1, g3)]]
     assert np.array_equal(host(ctx.hoisted_terms(shared_pb, nq, b_premultiplied=True)[0]), want_shared)
+    # compact keys (6 bytes per residue of a prime below 2^44): the same sums, kernel-argument and staged term lists
+    ck = {g: ctx.compact_key(k) for g, k in dk.items()}
+    assert all(c.numel() < k.numel() for c, k in zip(ck.values(), dk.values()))
+    swap = lambda gs: [[(t[0], t[1], ck[t[4]], t[3], t[4]) + tuple(t[5:]) for t in g] for g in gs]
+    assert torch.equal(ctx.hoisted_terms(swap(groups), nq, compact_keys=True), y)
+    assert np.array_equal(host(ctx.hoisted_terms(swap(shared), nq, compact_keys=True)[0]), want_shared)
+    many = (groups + shared) * 12    # more than 32 terms: the staged list
+    assert torch.equal(ctx.hoisted_terms(swap(many), nq, compact_keys=True), ctx.hoisted_terms(many, nq))
+    # one layout per call: a mix is refused before anything is launched
+    n_terms = sum(len(g) for g in groups)
+    with pytest.raises(ValueError, match="same key layout"):
+        ctx.hoisted_terms(swap(groups), nq, compact_keys=[True] + [False] * (n_terms - 1))
     # plain ModDown and ModDown merged with the rescale, batched over all outputs
     for drop in (False, True):
         got = host(ctx.moddown_batch(y.clone(), nq, drop))
