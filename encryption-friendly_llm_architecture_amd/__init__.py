@@ -42,6 +42,10 @@ class RotTerm(ctypes.Structure):
                 ("flags", ctypes.c_uint32)]
 
 
+class TensorGroup(ctypes.Structure):
+    _fields_ = [("t1", vp), ("t2", vp), ("acc3", vp), ("n_pairs", ctypes.c_uint32), ("accumulate", ctypes.c_uint32)]
+
+
 class LinTerm(ctypes.Structure):
     _fields_ = [("ct", vp), ("mask", vp), ("stride", ctypes.c_uint64), ("galois", ctypes.c_uint64)]
 
@@ -79,6 +83,7 @@ def _declare(L):
     L.hemm_hoisted_moddown.argtypes = [vp, ctypes.POINTER(RotTerm), u32p, u32, u32, ci, ci, vp, vp, sz, vp, vp]
     L.hemm_masked_sum_batch.argtypes = [vp, ctypes.POINTER(LinTerm), u32p, u32, u32, u32, vp, vp]
     L.hemm_tensor_batch.argtypes = [vp, vp, vp, u32, u32, vp, ci, vp]
+    L.hemm_tensor_batch_groups.argtypes = [vp, ctypes.POINTER(TensorGroup), u32, u32, sz, vp]
     L.hemm_compact_mask.argtypes = [vp, vp, u32, u32, vp, ctypes.POINTER(ci), vp]
     L.hemm_key_compact_words.argtypes = [vp]
     L.hemm_key_compact_words.restype = ctypes.c_size_t
@@ -407,6 +412,15 @@ class Context:
             acc = torch.empty((3, nq, self.N), dtype=torch.int64, device=t1.device)
         check(lib().hemm_tensor_batch(self.h, vp(t1.data_ptr()), vp(t2.data_ptr()), t1.shape[0], nq,
                                       vp(acc.data_ptr()), int(accumulate), vp(0)))
+        return acc
+
+    def tensor_batch_groups(self, groups, nq, acc):
+        """groups: list of (t1 [n_pairs][2][nq][N], t2 the same, index of the accumulator, accumulate) -- one launch;
+        acc: [3][n_acc][nq][N], polynomial-major (accumulator i is acc[:, i])."""
+        arr = (TensorGroup * len(groups))()
+        for i, (t1, t2, idx, accumulate) in enumerate(groups):
+            arr[i] = TensorGroup(t1.data_ptr(), t2.data_ptr(), acc[0, idx].data_ptr(), t1.shape[0], int(accumulate))
+        check(lib().hemm_tensor_batch_groups(self.h, arr, len(groups), nq, acc.shape[1] * nq * self.N, vp(0)))
         return acc
 
 

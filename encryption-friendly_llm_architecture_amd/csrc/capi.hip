@@ -570,6 +570,33 @@ int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint6
     HEMM_CATCH
 }
 
+int hemm_tensor_batch_groups(hemm_context *ctx, const hemm_tensor_group *groups, uint32_t n_groups, uint32_t nq,
+                             size_t acc_stride, void *stream) {
+    HEMM_TRY
+    int nl;
+    chain_limbs(ctx, nq, 0, &nl);
+    need(groups != nullptr && n_groups >= 1 && (int)n_groups <= tensor_max_groups(), "between 1 and 8 groups per call");
+    need(acc_stride >= (size_t)nq * (size_t)ctx->N, "accumulator stride below one polynomial");
+    std::vector<TensorGroupHost> g(n_groups);
+    const size_t poly = (size_t)nq * (size_t)ctx->N;
+    for (uint32_t i = 0; i < n_groups; i++) {
+        need(groups[i].t1 && groups[i].t2 && groups[i].acc3 && groups[i].n_pairs >= 1, "null operand");
+        need(groups[i].accumulate <= 1, "accumulate is 0 or 1");
+        // polynomial p of accumulator i covers [acc3 + p * stride, + poly): no two of one call may overlap
+        for (uint32_t k = 0; k < i; k++)
+            for (int p = 0; p < 3; p++)
+                for (int r = 0; r < 3; r++) {
+                    const uint64_t *a = groups[i].acc3 + p * acc_stride, *b = groups[k].acc3 + r * acc_stride;
+                    need(a + poly <= b || b + poly <= a, "accumulators of one call overlap");
+                }
+        g[i] = TensorGroupHost{(const u64 *)groups[i].t1, (const u64 *)groups[i].t2, (u64 *)groups[i].acc3,
+                               (int)groups[i].n_pairs, groups[i].accumulate != 0};
+    }
+    launch_tensor_groups(ctx, g.data(), (int)n_groups, (int)nq, acc_stride, (hipStream_t)stream);
+    check_launch();
+    HEMM_CATCH
+}
+
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out, size_t out_stride,
                  uint32_t nq, uint32_t n_polys, void *stream) {
     HEMM_TRY

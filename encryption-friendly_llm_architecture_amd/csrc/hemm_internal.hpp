@@ -170,5 +170,16 @@ int masked_arg_capacity();
 bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s);
 void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
                             int nq, int n_polys, u64 *out, hipStream_t s);
+// several tensor sums in one launch: acc[i] (+)= sum over n_pairs[i] pairs of t1[i], t2[i] (distinct accumulators)
+#define TENSOR_MAX_GROUPS 8
+struct TensorGroupHost {
+    const u64 *t1, *t2;
+    u64 *acc;
+    int n_pairs;
+    bool accumulate;
+};
+int tensor_max_groups();
+void launch_tensor_groups(hemm_context *c, const TensorGroupHost *g, int n_groups, int nq, size_t acc_stride,
+                          hipStream_t s);
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
                          bool accumulate, hipStream_t s);

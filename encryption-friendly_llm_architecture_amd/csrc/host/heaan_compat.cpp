@@ -524,6 +524,7 @@ void KeyGenerator::genMultKey() const {
     DeviceBuffer s2(ctx_, T * ctx_->N);
     ck(hemm_pointwise(ctx_->dev, HEMM_MUL, sk_.ntt(), 0, sk_.ntt(), 0, s2.data(), 0, (uint32_t)ctx_->nQ, 1, 1, nullptr));
     genSwitchKey(0, s2.data(), pack_.mult_);
+    pack_.compact_.erase(std::make_pair(0, u64(0)));   // a compact form of an earlier multiplication key is stale
 }
 static void gen_galois(const KeyGenerator &, const Context &c, const SecretKey &sk, u64 g, DeviceBuffer &sg) {
     const size_t T = c->nQ + c->nP;

@@ -780,7 +780,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     // that they accumulate into different partial sums) and the second runs on the side stream beside the first, with
     // buffers of its own: each launch of one chain fills the part-empty last round of workgroups of the other's
     // (measured -1.3 % per product; staggering the chains so that one's inverse transforms meet the other's key
-    // product gained nothing).
+    // product gained nothing; three and four chains on as many streams cost 1.0 % and 2.3 %).
     std::vector<std::pair<size_t, size_t>> chains;   // (first, count)
     for (size_t first = 0; first < sa.size(); first += G) chains.push_back({first, std::min(G, sa.size() - first)});
     bool two_streams = false;
@@ -801,16 +801,37 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     }
     auto accumulate = [&](size_t first, size_t cnt, const u64 *tb, hipStream_t st) {
         // shift index q holds i = q + 1: consecutive i with the same i2 pair with consecutive baby rotations
+        // one launch for the giant-step groups of the chain (each group its own accumulator)
         size_t q = first;
+        std::vector<hemm_tensor_group> groups;
+        auto flush = [&]() {
+            if (!groups.empty())
+                ck(hemm_tensor_batch_groups(c->dev, groups.data(), (uint32_t)groups.size(), (uint32_t)lo, us, st));
+            groups.clear();
+        };
         while (q < first + cnt) {
             const i64 ii = (i64)q + 1, i2 = ii / g, i1 = ii % g;
             const size_t run = std::min<size_t>(first + cnt - q, (size_t)(g - i1));
-            ck(hemm_tensor_batch_strided(c->dev, tb + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
-                                         (uint32_t)lo, U_out->data() + (u64)i2 * pw, us, started[(size_t)i2] ? 1 : 0,
-                                         st));
+            if (N < 512) {
+                ck(hemm_tensor_batch_strided(c->dev, tb + (q - first) * ctl, bb.data() + (u64)i1 * ctl, (uint32_t)run,
+                                             (uint32_t)lo, U_out->data() + (u64)i2 * pw, us,
+                                             started[(size_t)i2] ? 1 : 0, st));
+            } else {
+                // a group that continues an accumulator already in the list would race with it: close the list first
+                for (const hemm_tensor_group &h : groups)
+                    if (h.acc3 == U_out->data() + (u64)i2 * pw) {
+                        flush();
+                        break;
+                    }
+                groups.push_back(hemm_tensor_group{tb + (q - first) * ctl, bb.data() + (u64)i1 * ctl,
+                                                   U_out->data() + (u64)i2 * pw, (uint32_t)run,
+                                                   started[(size_t)i2] ? 1u : 0u});
+                if (groups.size() == 8) flush();
+            }
             started[(size_t)i2] = true;
             q += run;
         }
+        flush();
     };
     // forked before the first chain is queued: the side stream waits only for what both chains depend on
     const hipStream_t side2 = two_streams ? c->forkSide() : nullptr;
@@ -818,13 +839,14 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         const size_t first = chains[ch].first, cnt = chains[ch].second;
         const bool on_side = two_streams && ch == 1;
         const hipStream_t st = on_side ? side2 : nullptr;
+        u64 *yap = on_side ? ya2.data() : ya.data(), *t1p = on_side ? t12.data() : t1.data(),
+            *wsp = on_side ? ws2.data() : ws.data();
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
-        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1,
-                                on_side ? ya2.data() : ya.data(), on_side ? t12.data() : t1.data(), lo * N,
-                                on_side ? ws2.data() : ws.data(), st));
-        accumulate(first, cnt, on_side ? t12.data() : t1.data(), st);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, yap, t1p, lo * N,
+                                wsp, st));
+        accumulate(first, cnt, t1p, st);
     }
     if (two_streams) c->joinSide();
     *g_out = g;

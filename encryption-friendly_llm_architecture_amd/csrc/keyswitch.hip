@@ -517,6 +517,49 @@ __global__ __launch_bounds__(256) void tensor_batch_kernel(const u64 *__restrict
     acc3[2 * acc_stride + e] = d2;
 }
 
+// The same for up to TENSOR_MAX_GROUPS accumulators in one launch (blockIdx.z = group): the giant-step groups of a
+// chain of shifts are a few such sums of at most g pairs each, and one launch over all of them fills the GPU where
+// a launch per group is a single part-filled round of workgroups.  A thread owns the residue pair (n, n+1).
+struct TensorGroups {
+    const u64 *t1[TENSOR_MAX_GROUPS], *t2[TENSOR_MAX_GROUPS];
+    u64 *acc[TENSOR_MAX_GROUPS];
+    int n_pairs[TENSOR_MAX_GROUPS], accumulate[TENSOR_MAX_GROUPS];
+};
+__global__ __launch_bounds__(256) void tensor_groups_kernel(TensorGroups gr, size_t acc_stride,
+                                                            const ModQ *__restrict__ modq, int nq, int logN) {
+    const int j = blockIdx.y, z = blockIdx.z;
+    const ModQ m = modq[j];
+    const size_t N = (size_t)1 << logN, P = (size_t)nq * N;
+    const size_t e = (size_t)j * N + ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const u64 *__restrict__ t1 = gr.t1[z], *__restrict__ t2 = gr.t2[z];
+    u64 *__restrict__ acc3 = gr.acc[z];
+    const int G = gr.n_pairs[z];
+    ulonglong2 d0 = make_ulonglong2(0, 0), d1 = d0, d2 = d0;
+    if (gr.accumulate[z]) {
+        d0 = *(const ulonglong2 *)(acc3 + e);
+        d1 = *(const ulonglong2 *)(acc3 + acc_stride + e);
+        d2 = *(const ulonglong2 *)(acc3 + 2 * acc_stride + e);
+    }
+    for (int g = 0; g < G; g++) {
+        const ulonglong2 b1 = stream_load2(t1 + (size_t)g * 2 * P + e), a1 = stream_load2(t1 + (size_t)g * 2 * P + P + e);
+        const ulonglong2 b2 = *(const ulonglong2 *)(t2 + (size_t)g * 2 * P + e);
+        const ulonglong2 a2 = *(const ulonglong2 *)(t2 + (size_t)g * 2 * P + P + e);
+        d0.x = addmod(d0.x, mulmod(b1.x, b2.x, m), m.q);
+        d0.y = addmod(d0.y, mulmod(b1.y, b2.y, m), m.q);
+        u128_t t = mul64wide(a1.x, b2.x);
+        add128(t, mul64wide(a2.x, b1.x));
+        d1.x = addmod(d1.x, barrett128(t, m), m.q);
+        t = mul64wide(a1.y, b2.y);
+        add128(t, mul64wide(a2.y, b1.y));
+        d1.y = addmod(d1.y, barrett128(t, m), m.q);
+        d2.x = addmod(d2.x, mulmod(a1.x, a2.x, m), m.q);
+        d2.y = addmod(d2.y, mulmod(a1.y, a2.y, m), m.q);
+    }
+    *(ulonglong2 *)(acc3 + e) = d0;
+    *(ulonglong2 *)(acc3 + acc_stride + e) = d1;
+    *(ulonglong2 *)(acc3 + 2 * acc_stride + e) = d2;
+}
+
 }  // namespace
 
 // ---- tables -----------------------------------------------------------------------------------
@@ -1440,6 +1483,26 @@ void launch_masked_sum_args(hemm_context *c, const void *terms_host, int n_terms
         hipLaunchKernelGGL(masked_sum_kernel<3>, grid, block, 0, s, a, out, c->d_modq, c->d_fp, nq, c->logN, n_out);
 }
 
+int tensor_max_groups() { return TENSOR_MAX_GROUPS; }
+void launch_tensor_groups(hemm_context *c, const TensorGroupHost *g, int n_groups, int nq, size_t acc_stride,
+                          hipStream_t s) {
+    if (n_groups < 1 || n_groups > TENSOR_MAX_GROUPS) throw std::invalid_argument("between 1 and 8 groups per launch");
+    if (c->N < 512) throw std::invalid_argument("grouped tensor sums need N >= 512");
+    TensorGroups gr;
+    memset(&gr, 0, sizeof(gr));
+    size_t bytes = 0;
+    for (int i = 0; i < n_groups; i++) {
+        gr.t1[i] = g[i].t1;
+        gr.t2[i] = g[i].t2;
+        gr.acc[i] = g[i].acc;
+        gr.n_pairs[i] = g[i].n_pairs;
+        gr.accumulate[i] = g[i].accumulate ? 1 : 0;
+        bytes += (size_t)(4 * g[i].n_pairs + (g[i].accumulate ? 6 : 3)) * nq * c->N * 8;
+    }
+    account(c, TR_TENSOR, bytes);
+    hipLaunchKernelGGL(tensor_groups_kernel, dim3(c->N / 512, nq, n_groups), dim3(256), 0, s, gr, acc_stride, c->d_modq,
+                       nq, c->logN);
+}
 void launch_tensor_batch(hemm_context *c, const u64 *t1, const u64 *t2, int G, int nq, u64 *acc3, size_t acc_stride,
                          bool accumulate, hipStream_t s) {
     dim3 grid(c->N / 256, nq), block(256);

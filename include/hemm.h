@@ -233,6 +233,18 @@ int hemm_tensor_batch(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2,
  * kept polynomial-major, [3][count][nq][N], so that one hemm_modup_batch covers a polynomial of all of them) */
 int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint64_t *t2, uint32_t n_pairs, uint32_t nq,
                               uint64_t *acc3, size_t acc_stride, int accumulate, void *stream);
+/* several such sums in one launch (at most 8; N >= 512): group i adds the n_pairs tensor products of t1[k], t2[k],
+ * k < n_pairs, to its own accumulator acc3 (or stores them when accumulate is 0).  The accumulators of one call must
+ * not overlap.  One launch over the giant-step groups of a chain of shifts fills the GPU where a launch per group
+ * does not.  No counterpart in HEaaN's interface (HomEvaluator::tensor :518 takes one pair). */
+typedef struct {
+    const uint64_t *t1, *t2; /* [n_pairs][2][nq][N] each */
+    uint64_t *acc3;          /* three polynomials acc_stride words apart */
+    uint32_t n_pairs;
+    uint32_t accumulate;     /* 0 or 1 */
+} hemm_tensor_group;
+int hemm_tensor_batch_groups(hemm_context *ctx, const hemm_tensor_group *groups, uint32_t n_groups, uint32_t nq,
+                             size_t acc_stride, void *stream);
 
 /* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last */
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,

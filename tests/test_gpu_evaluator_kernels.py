@@ -299,6 +299,19 @@ def test_batched_hoisted_forms(S):
         t = orc.tensor(O.Ct(a, 1.0), O.Ct(b, 1.0))
         want3 = t if want3 is None else orc.add(want3, t)
     assert np.array_equal(host(acc), want3.data)
+    # several sums in one launch, accumulators polynomial-major: group 0 stores 3 pairs into accumulator 1, group 1
+    # adds 2 pairs to accumulator 0 (which holds the sum above), group 2 stores one pair into accumulator 2
+    acc3 = torch.zeros((3, 3, nq, S.N), dtype=torch.int64, device="cuda")
+    acc3[:, 0] = acc
+    ctx.tensor_batch_groups([(t1, t2, 1, False), (t1[1:].contiguous(), t2[:2].contiguous(), 0, True),
+                             (t2[:1].contiguous(), t2[:1].contiguous(), 2, False)], nq, acc3)
+    single = [ctx.tensor_batch(t1, t2, nq),
+              ctx.tensor_batch(t1[1:].contiguous(), t2[:2].contiguous(), nq, acc=acc.clone()),
+              ctx.tensor_batch(t2[:1].contiguous(), t2[:1].contiguous(), nq)]
+    for idx, want in zip((1, 0, 2), single):
+        assert torch.equal(acc3[:, idx], want)
+    with pytest.raises(ValueError, match="overlap"):
+        ctx.tensor_batch_groups([(t1, t2, 1, False), (t1, t2, 1, True)], nq, acc3)
 
 
 def test_hoisted_terms_extreme_residues(S):
