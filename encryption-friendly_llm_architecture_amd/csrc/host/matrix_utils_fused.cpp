@@ -854,8 +854,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
 
 // res = sum_i2 rho^(g i2 ru)(U_i2) relinearised and rescaled, all through one hoisted launch: U_i2 (i2 >= 1) gives
 // the terms (d1 under the key of rho(s), d2 under the key of rho(s)^2); U_0 gives its d2 under the multiplication key
-// with the identity automorphism, and its d1 is added to the second polynomial of the sum, times P, before the
-// single ModDown merged with the rescale.
+// with the identity automorphism, and its d1 is added to the second polynomial after the single ModDown.
 // add_conj: the result is x + conj(x) for the sum x described above -- every term enters a second time under its
 // Galois element times 2N - 1 (keys of the composite elements; d1 of U_0, which needs no key switch in x, is switched
 // under the conjugation key), so the real part of a complex-packed product needs no key-switch round of its own.
@@ -883,17 +882,12 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
         }
         U = std::move(Ur);
     }
-    DeviceBuffer ext(c, 2 * m * beta * El * N), wsu(c, 2 * m * lo * N), pd1(c, lo * N);
+    DeviceBuffer ext(c, 2 * m * beta * El * N), wsu(c, 2 * m * lo * N);
     ck(hemm_modup_batch(c->dev, U.data() + us, pw, (uint32_t)lo, (uint32_t)(2 * m), ext.data(), wsu.data(), nullptr));
     const u64 *ext1 = ext.data(), *ext2 = ext.data() + m * beta * El * N;   // [i2][beta][El][N] each
-    std::vector<u64> sc(lo);
-    for (u64 j = 0; j < lo; j++) {
-        u64 P = 1;
-        for (u64 p : c->p) P = (u64)((u128)P * (p % c->q[j]) % c->q[j]);
-        sc[j] = P;
-    }
-    // d0 of every partial sum enters its term as it is (the launch multiplies by P); only P d1 of U_0 is made here
-    ck(hemm_mul_scalar(c->dev, U.data() + us, pw, sc.data(), pd1.data(), lo * N, (uint32_t)lo, 0, 1, nullptr));
+    // d0 of every partial sum enters its term as it is (the launch multiplies by P); d1 of U_0, which needs no key
+    // switch, is added after the ModDown: (y + P d1 - conv) / P = (y - conv) / P + d1 on every chain limb, and P d1
+    // vanishes on the special limbs the conversion reads
     std::vector<hemm_rot_term> terms;
     {
         hemm_rot_term t{};
@@ -939,8 +933,9 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     res.get().allocate(2, T, 0);
     DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * lo * N);
     ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 0, nullptr));
-    ck(hemm_pointwise(c->dev, HEMM_ADD, yg.data() + El * N, 0, pd1.data(), 0, yg.data() + El * N, 0, (uint32_t)lo, 0, 1, nullptr));
     ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 0, res.get().buf_.data(), lo * N, wsg.data(), nullptr));
+    u64 *res1 = res.get().buf_.data() + lo * N;
+    ck(hemm_pointwise(c->dev, HEMM_ADD, res1, 0, U.data() + us, 0, res1, 0, (uint32_t)lo, 0, 1, nullptr));
 }
 }  // namespace
 
