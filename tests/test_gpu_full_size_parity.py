@@ -66,6 +66,7 @@ class Bench:
         self.d_ext = [dev(x) for x in self.ext]
         self.d_b = [dev(x) for x in self.b]
         self.d_evk = [dev(x) for x in self.evk]
+        self.d_evk_compact = [self.ctx.compact_key(k) for k in self.d_evk]   # 6 bytes per residue of a prime below 2^44
         self.d_full = [(dev(m.data), dev(w.data)) for m, w in self.masks]
         self.d_tab = [(self.ctx.compact_mask(m, self.shift), self.ctx.compact_mask(w, self.shift)) for m, w in self.d_full]
         assert all(t is not None for pair in self.d_tab for t in pair)
@@ -79,9 +80,10 @@ class Bench:
                                    self.gal[k], self.nq, _p(y), int(i > 0))
         return y
 
-    def term(self, s, k, m, half, table=True):
+    def term(self, s, k, m, half, table=True, compact=False):
         mask = self.d_tab[m][half] if table else self.d_full[m][half]
-        return (self.d_ext[s], self.d_b[s], self.d_evk[k], mask, self.gal[k], self.shift if table else 0)
+        key = self.d_evk_compact[k] if compact else self.d_evk[k]
+        return (self.d_ext[s], self.d_b[s], key, mask, self.gal[k], self.shift if table else 0)
 
 
 @pytest.fixture(scope="module")
@@ -109,6 +111,9 @@ def test_hoisted_sum_at_the_main_loop_shape_two_launches(bench):
     groups = [[bench.term(*t) for t in spec] for spec in specs]
     y = host(bench.ctx.hoisted_terms(groups, bench.nq))
     check_outputs(bench, specs, y)
+    # the same sums on compact keys (the layout the products use): the <1, true> / <2, true> launches
+    groups = [[bench.term(*t, compact=True) for t in spec] for spec in specs]
+    assert np.array_equal(host(bench.ctx.hoisted_terms(groups, bench.nq, compact_keys=True)), y)
 
 
 def test_hoisted_sum_staged_term_list_two_launches(bench):
@@ -127,6 +132,9 @@ def test_hoisted_sum_staged_term_list_two_launches(bench):
     groups = [[bench.term(*t, table=((i // 2) + o) % 3 != 0) for i, t in enumerate(spec)] for o, spec in enumerate(specs)]
     y = host(bench.ctx.hoisted_terms(groups, bench.nq))
     check_outputs(bench, specs, y)
+    groups = [[bench.term(*t, table=((i // 2) + o) % 3 != 0, compact=True) for i, t in enumerate(spec)]
+              for o, spec in enumerate(specs)]
+    assert np.array_equal(host(bench.ctx.hoisted_terms(groups, bench.nq, compact_keys=True)), y)
 
 
 def test_hoisted_sum_two_launches_every_operand_at_q_minus_one(bench):
@@ -154,6 +162,10 @@ def test_hoisted_sum_two_launches_every_operand_at_q_minus_one(bench):
         want.append(w)
     for o in range(32):
         assert np.array_equal(y[o], want[o % 3]), o
+    # compact key with every residue q - 1: the high halves of the 12-byte records at their largest
+    dkc = ctx.compact_key(dk)
+    groups_c = [[(t[0], t[1], dkc) + tuple(t[3:]) for t in g] for g in groups]
+    assert np.array_equal(host(ctx.hoisted_terms(groups_c, nq, compact_keys=True)), y)
 
 
 @pytest.mark.parametrize("n_polys", [1, 2, 3])
