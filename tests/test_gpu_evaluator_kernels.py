@@ -466,3 +466,31 @@ def test_device_samplers_match_oracle(S):
     got = host(ctx.sample_error(ek, idx))
     for j in idx:
         assert np.array_equal(got[j], np.mod(e.astype(np.int64), orc.mods[j]).astype(np.uint64)), j
+
+
+def test_batched_entry_points_refuse_what_the_kernels_cannot_take():
+    """Compact keys with more than six digits (there the limbs of primes below 2^44 run through the integer path,
+    which reads whole words), more groups than one grouped tensor launch holds, and a flag the library does not know:
+    each refused on the host, nothing launched."""
+    import torch
+    pkg = load_package()
+    log_n, N = 10, 1 << 10
+    qs, ps = O.ckks_chain(log_n, 8, 1)
+    ctx = pkg.Context(log_n, qs, ps, 8)            # digits of one limb: a sum at nq = 8 has 8 digits
+    nq, E = 8, 9
+    z = lambda *shape: torch.zeros(shape, dtype=torch.int64, device="cuda")
+    ext, b, evk = z(8, E, N), z(nq, N), z(8, 2, 9, N)
+    groups = [[(ext, b, evk, None, 5)]]
+    assert int(ctx.hoisted_terms(groups, nq).abs().sum().item()) == 0          # the plain layout runs
+    ck = ctx.compact_key(evk)
+    with pytest.raises(ValueError, match="at most 6 digits"):
+        ctx.hoisted_terms([[(ext, b, ck, None, 5)]], nq, compact_keys=True)
+    with pytest.raises(ValueError, match="unknown flag"):
+        ctx.hoisted_terms(groups, nq, compact_keys=[2])
+    t = z(1, 2, nq, N)
+    acc = z(3, 9, nq, N)
+    with pytest.raises(ValueError, match="groups per call"):
+        ctx.tensor_batch_groups([(t, t, i, False) for i in range(9)], nq, acc)
+    ctx.tensor_batch_groups([(t, t, i, False) for i in range(8)], nq, acc)
+    torch.cuda.synchronize()
+    assert int(acc.abs().sum().item()) == 0
