@@ -239,9 +239,11 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
             u64 rb[2], ra[2];
             if (T.mask_shift != 0 && T.pt == nullptr)
-                two_source_int<true, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+                two_source_int<true, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN,
+                                              b_premultiplied, rb, ra);
             else
-                two_source_int<false, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN, b_premultiplied, rb, ra);
+                two_source_int<false, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN,
+                                               b_premultiplied, rb, ra);
             acc_b[0] = addmod(acc_b[0], rb[0], m.q);
             acc_b[1] = addmod(acc_b[1], rb[1], m.q);
             acc_a[0] = addmod(acc_a[0], ra[0], m.q);

@@ -290,15 +290,15 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
     if (MODE == 1 || (MODE == 0 && fq != 0.0 && beta <= 6)) {
         const FpMod f{fq, fp[4 * prime + 1]};
         double fb[2], fa[2];
-        hoisted_pair_fp<COMPACT>(terms, group_off, koff, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E, beta, n_full, logN,
-                        b_premultiplied, fb, fa);
+        hoisted_pair_fp<COMPACT>(terms, group_off, koff, f, j < nq ? (double)pmod.c[j].w : 0.0, j, o, prime, n, nq, E,
+                                 beta, n_full, logN, b_premultiplied, fb, fa);
         rb[0] = f.canonical(fb[0]);
         rb[1] = f.canonical(fb[1]);
         ra[0] = f.canonical(fa[0]);
         ra[1] = f.canonical(fa[1]);
     } else {
-        hoisted_pair_int<COMPACT>(terms, group_off, koff, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN, b_premultiplied,
-                         rb, ra);
+        hoisted_pair_int<COMPACT>(terms, group_off, koff, modq[prime], pmod, j, o, prime, n, nq, E, beta, n_full, logN,
+                                  b_premultiplied, rb, ra);
     }
     stream_store2(y + (((size_t)o * 2 + 0) * E + j) * N + n, rb[0], rb[1]);
     stream_store2(y + (((size_t)o * 2 + 1) * E + j) * N + n, ra[0], ra[1]);
@@ -312,28 +312,28 @@ struct HoistedArgs {
     RotTermDev t[HOISTED_ARG_TERMS];
     u32 off[HOISTED_ARG_TERMS + 1];
 };
-// Register budget for five waves per SIMD (96 registers): the double-precision form needs 72 and the integer form 96;
-// the mixed form would take 109 and run at four waves, capped it spills two registers and gains a wave.
+// Register budget for five waves per SIMD (96 registers): the double-precision form needs 72 (74 on compact keys) and
+// the integer form 93 - 96; the mixed form would take 109 and run at four waves, capped it spills two or three registers
+// and gains a wave.  COMPACT: the key layout of the launch (hoisted.h, key_limb).
+#define HOISTED_KERNEL __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void
 template <int MODE, bool COMPACT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y,
-                                                            const ModQ *__restrict__ modq, const double *__restrict__ fp,
-                                                            LimbList ll, CstList pmod, int nq, int E, int beta,
-                                                            int n_full, int logN, int b_premultiplied, int n_out,
-                                                            LimbList jmap, int n_j, const u32 *__restrict__ koff) {
-    hoisted_terms_body<MODE, COMPACT>(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
-                           n_j, koff);
+HOISTED_KERNEL hoisted_terms_kernel(const HoistedArgs args, u64 *__restrict__ y, const ModQ *__restrict__ modq,
+                                    const double *__restrict__ fp, LimbList ll, CstList pmod, int nq, int E, int beta,
+                                    int n_full, int logN, int b_premultiplied, int n_out, LimbList jmap, int n_j,
+                                    const u32 *__restrict__ koff) {
+    hoisted_terms_body<MODE, COMPACT>(args.t, args.off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN,
+                                      b_premultiplied, n_out, jmap, n_j, koff);
 }
 template <int MODE, bool COMPACT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms,
-                                                                 const u32 *__restrict__ group_off, u64 *__restrict__ y,
-                                                                 const ModQ *__restrict__ modq,
-                                                                 const double *__restrict__ fp, LimbList ll, CstList pmod,
-                                                                 int nq, int E, int beta, int n_full, int logN,
-                                                                 int b_premultiplied, int n_out, LimbList jmap, int n_j,
-                                                                 const u32 *__restrict__ koff) {
-    hoisted_terms_body<MODE, COMPACT>(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN, b_premultiplied, n_out, jmap,
-                           n_j, koff);
+HOISTED_KERNEL hoisted_terms_list_kernel(const RotTermDev *__restrict__ terms, const u32 *__restrict__ group_off,
+                                         u64 *__restrict__ y, const ModQ *__restrict__ modq,
+                                         const double *__restrict__ fp, LimbList ll, CstList pmod, int nq, int E,
+                                         int beta, int n_full, int logN, int b_premultiplied, int n_out, LimbList jmap,
+                                         int n_j, const u32 *__restrict__ koff) {
+    hoisted_terms_body<MODE, COMPACT>(terms, group_off, y, modq, fp, ll, pmod, nq, E, beta, n_full, logN,
+                                      b_premultiplied, n_out, jmap, n_j, koff);
 }
+#undef HOISTED_KERNEL
 
 struct LinTermDev {
     const u64 *ct;    // [n_polys][.][N]
@@ -1219,9 +1219,10 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     const LimbList ll = limbs_default(c, nq, 1);
     const RotTermDev *td = (const RotTermDev *)terms_dev;
     const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
-#define HOISTED_LIST(MODE, COMPACT, GRID, JM, NJ)                                                                    \
-    hipLaunchKernelGGL((hoisted_terms_list_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, td, group_off_dev, y, \
-                       c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
+#define HOISTED_LIST(MODE, COMPACT, GRID, JM, NJ)                                                                  \
+    hipLaunchKernelGGL((hoisted_terms_list_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, td,        \
+                       group_off_dev, y, c->d_modq, c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, \
+                       NJ, c->d_key_off)
     if (!split) {
         if (compact)
             HOISTED_LIST(0, true, per_limb * E, all, E);
@@ -1246,7 +1247,8 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     const CstList pm = p_mod_chain(c, nq);
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
-    if (n_terms > HOISTED_ARG_TERMS || n_out > HOISTED_ARG_TERMS) throw std::invalid_argument("term list too long for the argument path");
+    if (n_terms > HOISTED_ARG_TERMS || n_out > HOISTED_ARG_TERMS)
+        throw std::invalid_argument("term list too long for the argument path");
     account(c, TR_KEYPROD, hoisted_bytes(c, (const RotTermDev *)terms_host, n_terms, n_out, nq));
     HoistedArgs a;
     memset(&a, 0, sizeof(a));
@@ -1261,9 +1263,9 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
     const bool compact = n_terms > 0 && (((const RotTermDev *)terms_host)[0].flags & ROT_TERM_COMPACT_KEY) != 0;
     if (compact && beta > 6) throw std::invalid_argument("compact keys need at most 6 digits");
-#define HOISTED_ARGS(MODE, COMPACT, GRID, JM, NJ)                                                                     \
-    hipLaunchKernelGGL((hoisted_terms_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, a, y, c->d_modq, c->d_fp, \
-                       ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
+#define HOISTED_ARGS(MODE, COMPACT, GRID, JM, NJ)                                                                  \
+    hipLaunchKernelGGL((hoisted_terms_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, a, y, c->d_modq, \
+                       c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
     if (!split) {
         if (compact)
             HOISTED_ARGS(0, true, per_limb * E, all, E);
