@@ -282,7 +282,12 @@ __device__ __forceinline__ void hoisted_terms_body(const RotTermDev *__restrict_
         chunk = rest % chunks;
         j = jmap.idx[rest / chunks];
     }
-    const int prime = ll.idx[j];
+    // output, limb and chunk are the same for the whole workgroup; the byte tables above are read with vector loads,
+    // so say it: everything derived from them (the bases of all streams) then lives in scalar registers
+    o = __builtin_amdgcn_readfirstlane(o);
+    j = __builtin_amdgcn_readfirstlane(j);
+    chunk = __builtin_amdgcn_readfirstlane(chunk);
+    const int prime = __builtin_amdgcn_readfirstlane((int)ll.idx[j]);
     const u32 n = (chunk * 256 + threadIdx.x) * 2;
     const double fq = fp[4 * prime];
     const size_t N = (size_t)1 << logN;
