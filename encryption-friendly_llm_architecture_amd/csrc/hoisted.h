@@ -110,14 +110,35 @@ __device__ __forceinline__ double u64_to_double(u64 v) {  // v < 2^52
 // by the loads in flight, not by the bytes).
 // (the layout is a property of the launch -- every term of a launch uses the same one -- and a template parameter of
 // the kernels: with both forms behind a run-time test the mixed kernel spilled 24 registers)
-template <bool COMPACT>
-__device__ __forceinline__ const char *key_limb(const RotTermDev &T, const u32 *__restrict__ koff, const int d,
-                                                const int pol, const int prime, const size_t N, const int n_full) {
-    if (COMPACT) return (const char *)T.evk + ((size_t)(d * 2 + pol) * koff[n_full] + koff[prime]) * (2 * N);
-    return (const char *)(T.evk + ((size_t)(d * 2 + pol) * n_full + prime) * N);
+//
+// The double-precision path reads a key through a buffer resource: the key's base and the offset of the limb sit in scalar registers and a
+// thread supplies only the 32-bit byte offset of its residue pair, shared by all key streams of the thread (with
+// 64-bit addresses in vector registers every stream costs two registers and an add with carry per load): 70
+// registers instead of 74, i.e. seven waves per SIMD instead of six.  The host checks that a key is below 4 GiB.
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t key_rsrc(const RotTermDev &T) {
+    // raw buffer (stride 0), no range limit, 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc((void *)T.evk, 0, -1, 0x00020000);
 }
-// residues (n, n+1) of a limb of any prime (compact keys: of a prime of 2^44 or more)
-__device__ __forceinline__ ulonglong2 key_pair_u64(const char *limb, const u32 n) {
+// byte offset of limb `prime` of polynomial pol of digit d inside the key (keys are far below 4 GiB)
+template <bool COMPACT>
+__device__ __forceinline__ u32 key_limb(const u32 *__restrict__ koff, const int d, const int pol, const int prime,
+                                        const int logN, const int n_full) {
+    if (COMPACT) return (((u32)(d * 2 + pol) * koff[n_full] + koff[prime]) << (logN + 1));
+    return ((u32)((d * 2 + pol) * n_full + prime)) << (logN + 3);
+}
+// residues (n, n+1) of a limb of any prime (compact keys: of a prime of 2^44 or more); streamed (non-temporal)
+__device__ __forceinline__ ulonglong2 key_pair_u64(const __amdgpu_buffer_rsrc_t key, const u32 limb, const u32 n) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(key, n * 8u, limb, 2);
+    return make_ulonglong2(((u64)v.y << 32) | v.x, ((u64)v.w << 32) | v.z);
+}
+// The integer path keeps plain pointers: it is short of scalar registers (106 of 102 usable with a resource per term,
+// which spilled 18 vector registers), not of vector registers.
+template <bool COMPACT>
+__device__ __forceinline__ ulonglong2 key_pair_ptr(const RotTermDev &T, const u32 *__restrict__ koff, const int d,
+                                                   const int pol, const int prime, const int logN, const int n_full,
+                                                   const u32 n) {
+    const char *limb = (const char *)T.evk + key_limb<COMPACT>(koff, d, pol, prime, logN, n_full);
     return stream_load2((const u64 *)limb + n);
 }
 typedef u32 u32x3 __attribute__((ext_vector_type(3), aligned(4)));
@@ -170,8 +191,8 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *_
             z0 = barrett3(t0, m);
             z1 = barrett3(t1, m);
         }
-        const ulonglong2 kb = key_pair_u64(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n);
-        const ulonglong2 ka = key_pair_u64(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n);
+        const ulonglong2 kb = key_pair_ptr<COMPACT>(T, koff, d, 0, prime, logN, n_full, n);
+        const ulonglong2 ka = key_pair_ptr<COMPACT>(T, koff, d, 1, prime, logN, n_full, n);
         add128(pb[0], mul64wide(z0, kb.x));
         add128(pb[1], mul64wide(z1, kb.y));
         add128(pa[0], mul64wide(z0, ka.x));
@@ -258,8 +279,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                 x.x = x.y;
                 x.y = tmp;
             }
-            const ulonglong2 kb = key_pair_u64(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n);
-            const ulonglong2 ka = key_pair_u64(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n);
+            const ulonglong2 kb = key_pair_ptr<COMPACT>(T, koff, d, 0, prime, logN, n_full, n);
+            const ulonglong2 ka = key_pair_ptr<COMPACT>(T, koff, d, 1, prime, logN, n_full, n);
             add128(sb[0], mul64wide(x.x, kb.x));
             add128(sb[1], mul64wide(x.y, kb.y));
             add128(sa[0], mul64wide(x.x, ka.x));
@@ -355,10 +376,9 @@ __device__ __forceinline__ D2 gather_d2(const u64 *p, const bool swap) {
 }
 // residues (n, n+1) of a key limb of a prime below 2^44 as doubles
 template <bool COMPACT>
-__device__ __forceinline__ D2 key_pair_fp(const char *limb, const u32 n, const size_t N) {
-    if (!COMPACT) return to_d2(stream_load2((const u64 *)limb + n));
-    // uniform base + 32-bit byte offset: the offsets n * 4 and n * 2 are shared by every key stream of the thread
-    const u32x3 v = __builtin_nontemporal_load((const u32x3 *)(limb + n * 6u));   // one 12-byte load
+__device__ __forceinline__ D2 key_pair_fp(const __amdgpu_buffer_rsrc_t key, const u32 limb, const u32 n) {
+    if (!COMPACT) return to_d2(key_pair_u64(key, limb, n));
+    const u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(key, n * 6u, limb, 2);   // one 12-byte load
     D2 r;
     r.x = __hiloint2double((int)((v.z & 0xffffu) | 0x43300000u), (int)v.x) - 4503599627370496.0;
     r.y = __hiloint2double((int)((v.z >> 16) | 0x43300000u), (int)v.y) - 4503599627370496.0;
@@ -378,6 +398,7 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
     int since = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const RotTermDev T = terms[t];
+        const __amdgpu_buffer_rsrc_t kr = key_rsrc(T);
         const u32 np = galois_index(n, T.galois, logN);
         const u32 base = np & ~1u;
         const bool swap = (np & 1u) != 0;
@@ -397,8 +418,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 const D2 x2 = gather_d2(T.ext2 + ((size_t)d * E + j) * N + base, swap);
                 const double z0 = f.mul(m1.x, x1.x) + f.mul(m2.x, x2.x);
                 const double z1 = f.mul(m1.y, x1.y) + f.mul(m2.y, x2.y);
-                const D2 kb = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n, N);
-                const D2 ka = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n, N);
+                const D2 kb = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 0, prime, logN, n_full), n);
+                const D2 ka = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 1, prime, logN, n_full), n);
                 sb0 += f.mul(z0, kb.x);
                 sb1 += f.mul(z1, kb.y);
                 sa0 += f.mul(z0, ka.x);
@@ -419,8 +440,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
         } else {
             for (int d = 0; d < beta; d++) {
                 const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
-                const D2 kb = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 0, prime, N, n_full), n, N);
-                const D2 ka = key_pair_fp<COMPACT>(key_limb<COMPACT>(T, koff, d, 1, prime, N, n_full), n, N);
+                const D2 kb = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 0, prime, logN, n_full), n);
+                const D2 ka = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 1, prime, logN, n_full), n);
                 sb0 += f.mul(x.x, kb.x);
                 sb1 += f.mul(x.y, kb.y);
                 sa0 += f.mul(x.x, ka.x);

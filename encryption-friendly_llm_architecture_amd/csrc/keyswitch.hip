@@ -1216,6 +1216,9 @@ void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *gro
     if (c->N < 512) throw std::invalid_argument("hoisted terms need N >= 512");
     // with more than 6 digits the limbs of primes below 2^44 go through the integer path, which reads whole words
     if (compact && beta > 6) throw std::invalid_argument("compact keys need at most 6 digits");
+    // the kernels address a key by 32-bit byte offsets
+    if ((size_t)c->dnum * 2 * (c->nQ + c->nP) * c->N * 8 >= ((size_t)1 << 32))
+        throw std::invalid_argument("hoisted terms need keys below 4 GiB");
     LimbList fpl, il, all;
     int n_fp, n_int;
     const bool split = split_limbs(c, nq, beta, n_out, fpl, n_fp, il, n_int, all);
@@ -1268,6 +1271,8 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
     const int n_full = c->nQ + c->nP, pre = b_premultiplied ? 1 : 0;
     const bool compact = n_terms > 0 && (((const RotTermDev *)terms_host)[0].flags & ROT_TERM_COMPACT_KEY) != 0;
     if (compact && beta > 6) throw std::invalid_argument("compact keys need at most 6 digits");
+    if ((size_t)c->dnum * 2 * (c->nQ + c->nP) * c->N * 8 >= ((size_t)1 << 32))
+        throw std::invalid_argument("hoisted terms need keys below 4 GiB");
 #define HOISTED_ARGS(MODE, COMPACT, GRID, JM, NJ)                                                                  \
     hipLaunchKernelGGL((hoisted_terms_kernel<MODE, COMPACT>), dim3((unsigned)(GRID)), block, 0, s, a, y, c->d_modq, \
                        c->d_fp, ll, pm, nq, E, beta, n_full, c->logN, pre, n_out, JM, NJ, c->d_key_off)
