@@ -20,6 +20,30 @@
 #include "hemm_internal.hpp"
 
 namespace {
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+// Column passes address a limb through a buffer resource: the limb's base sits in scalar registers, the slab row
+// (a step of 2 KiB or 32 KiB) goes into the scalar offset of each access and a thread supplies one 32-bit byte offset
+// for all of its 16 accesses -- with 64-bit addresses in vector registers every access costs an add with carry.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t limb_rsrc(const void *p) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, -1, 0x00020000);   // raw, no range limit, 32-bit format
+}
+template <class E>
+__device__ __forceinline__ E buf_load(const __amdgpu_buffer_rsrc_t r, const u32 voff, const u32 soff) {
+    const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    const u64 u = ((u64)w.y << 32) | w.x;
+    E v;
+    __builtin_memcpy(&v, &u, 8);
+    return v;
+}
+template <class E>
+__device__ __forceinline__ void buf_store(const __amdgpu_buffer_rsrc_t r, const u32 voff, const u32 soff, const E v) {
+    u64 u;
+    __builtin_memcpy(&u, &v, 8);
+    u32x2 w;
+    w.x = (u32)u;
+    w.y = (u32)(u >> 32);
+    __builtin_amdgcn_raw_buffer_store_b64(w, r, voff, soff, 0);
+}
 
 struct __align__(16) Tw {
     u64 w, ws;
@@ -313,16 +337,18 @@ __device__ __forceinline__ int swz_row(int r) { return r ^ ((r >> 4) & 1); }
 
 // forward pass 1 / inverse pass 2 work on a 256-row x 16-column slab.
 template <bool INV, class F>
-__device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw) {
+__device__ __forceinline__ void cols_body(const __amdgpu_buffer_rsrc_t limb, const u32 col, const Tw *__restrict__ tw_int,
+                                          const F f, u64 *lds_raw) {
     typedef typename F::E E;
     const typename F::W *tw = (const typename F::W *)tw_int;
     E *lds = (E *)lds_raw;
-    E *mem = (E *)base;
     const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
+    // byte offsets of (row rh, col) and (row 16 rh, col); rows 16 k resp. k further on go into the scalar offset
+    const u32 v_outer = (col + ((u32)rh << 8)) * 8u, v_inner = (col + ((u32)rh << 12)) * 8u;
     E x[16];
     if (!INV) {
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = f.from_canonical(base[(size_t)(rh + 16 * k) << 8]);
+        for (int k = 0; k < 16; k++) x[k] = f.from_canonical(buf_load<u64>(limb, v_outer, (u32)k << 15));
         radix16_fwd(f, x, tw, 1u);
         // row r of the slab is kept at row r ^ (bit 4 of r): the rows 16 apart that one wavefront reads together
         // after the exchange then alternate between the two halves of the 64 LDS banks instead of sharing 32 of them
@@ -333,10 +359,10 @@ __device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__re
         for (int k = 0; k < 16; k++) x[k] = lds[swz_row(16 * rh + k) * 16 + cc];
         radix16_fwd(f, x, tw, 16u + rh);
 #pragma unroll
-        for (int k = 0; k < 16; k++) mem[(size_t)(16 * rh + k) << 8] = x[k];
+        for (int k = 0; k < 16; k++) buf_store<E>(limb, v_inner, (u32)k << 11, x[k]);
     } else {
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = mem[(size_t)(16 * rh + k) << 8];
+        for (int k = 0; k < 16; k++) x[k] = buf_load<E>(limb, v_inner, (u32)k << 11);
         radix16_inv(f, x, tw, 16u + rh);
         f.after_inverse_block(x);
 #pragma unroll
@@ -346,7 +372,7 @@ __device__ __forceinline__ void cols_body(u64 *__restrict__ base, const Tw *__re
         for (int k = 0; k < 16; k++) x[k] = lds[(rh + 16 * k) * 16 + cc];
         radix16_inv(f, x, tw, 1u);
 #pragma unroll
-        for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = f.scale_to_canonical(x[k]);
+        for (int k = 0; k < 16; k++) buf_store<u64>(limb, v_outer, (u32)k << 15, f.scale_to_canonical(x[k]));
     }
 }
 
@@ -360,7 +386,9 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
     const int limb = blockIdx.y % n_limbs, poly = blockIdx.y / n_limbs;
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
-    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + blockIdx.x * 16 + (threadIdx.x & 15);
+    const __amdgpu_buffer_rsrc_t base = limb_rsrc(
+        data + (size_t)poly * poly_stride + ((size_t)__builtin_amdgcn_readfirstlane((int)sl.idx[limb]) << 16));
+    const u32 col = blockIdx.x * 16 + (threadIdx.x & 15);
     // final_scale (inverse transforms only): limb i ends with the constant final_scale[i] in place of 1/N -- a basis
     // conversion folds its (S/q_i)^-1 factor in here (the caller supplies (1/N)(S/q_i)^-1), at no cost
     if (fp[4 * prime] != 0.0) {
@@ -369,16 +397,16 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
             f.ni = (double)final_scale[limb].w;
             f.niinv = f.ni * f.qinv;
         }
-        cols_body<INV>(base, tw, f, lds);
+        cols_body<INV>(base, col, tw, f, lds);
     } else if (INV || (modq[prime].q >> 60) != 0) {
         IntField f(modq, ninv, ninv_s, fp, prime);
         if (INV && final_scale != nullptr) {
             f.ni = final_scale[limb].w;
             f.nis = final_scale[limb].ws;
         }
-        cols_body<INV>(base, tw, f, lds);
+        cols_body<INV>(base, col, tw, f, lds);
     } else {
-        cols_body<INV>(base, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds);
+        cols_body<INV>(base, col, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds);
     }
 }
 
@@ -388,13 +416,14 @@ __global__ __launch_bounds__(256) void ntt16_cols_kernel(u64 *__restrict__ data,
 // of the target limbs that share a (polynomial, slab) pair have consecutive blockIdx.y and the same blockIdx.x, so
 // they sit on one XCD at about the same time and all but the first find the source slabs in its L2.
 template <int NS, class F>
-__device__ __forceinline__ void cols_converted_body(u64 *__restrict__ base, const Tw *__restrict__ tw_int, const F f,
-                                                    u64 *lds_raw, const u64 *const (&sp)[NS], const u64 (&h)[NS],
-                                                    const int n_src, const ModQ m) {
+__device__ __forceinline__ void cols_converted_body(const __amdgpu_buffer_rsrc_t limb, const u32 col,
+                                                    const Tw *__restrict__ tw_int, const F f, u64 *lds_raw,
+                                                    const __amdgpu_buffer_rsrc_t src, const u32 voff,
+                                                    const u32 (&so)[NS], const u64 (&h)[NS], const int n_src,
+                                                    const ModQ m) {
     typedef typename F::E E;
     const typename F::W *tw = (const typename F::W *)tw_int;
     E *lds = (E *)lds_raw;
-    E *mem = (E *)base;
     const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
     E x[16];
     // eight coefficients at a time (three accumulators each), source by source, so that the eight loads of one source
@@ -409,7 +438,11 @@ __device__ __forceinline__ void cols_converted_body(u64 *__restrict__ base, cons
             if (i < n_src) {
                 u64 v[8];
 #pragma unroll
-                for (int k = 0; k < 8; k++) v[k] = sp[i][(size_t)(rh + 16 * (8 * half + k)) << 8];
+                for (int k = 0; k < 8; k++) {
+                    // row rh + 16 (8 half + k) of the slab: the row step of 32 KiB goes into the scalar offset
+                    const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(src, voff, so[i] + ((u32)(8 * half + k) << 15), 0);
+                    v[k] = ((u64)w.y << 32) | w.x;
+                }
 #pragma unroll
                 for (int k = 0; k < 8; k++) dot3_add(d[k], v[k], h[i]);
             }
@@ -424,8 +457,9 @@ __device__ __forceinline__ void cols_converted_body(u64 *__restrict__ base, cons
 #pragma unroll
     for (int k = 0; k < 16; k++) x[k] = lds[swz_row(16 * rh + k) * 16 + cc];
     radix16_fwd(f, x, tw, 16u + rh);
+    const u32 v_inner = (col + ((u32)rh << 12)) * 8u;   // (row 16 rh, col); row k further on in the scalar offset
 #pragma unroll
-    for (int k = 0; k < 16; k++) mem[(size_t)(16 * rh + k) << 8] = x[k];
+    for (int k = 0; k < 16; k++) buf_store<E>(limb, v_inner, (u32)k << 11, x[k]);
 }
 
 // Register budget of three waves per SIMD (168): left alone the compiler takes 170 - 176 registers, which leaves two
@@ -451,27 +485,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = t[k];
         return;
     }
-    u64 *base = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + col;
+    const __amdgpu_buffer_rsrc_t base = limb_rsrc(
+        data + (size_t)poly * poly_stride + ((size_t)__builtin_amdgcn_readfirstlane((int)sl.idx[limb]) << 16));
     const int prime = ll.idx[limb];
     const Tw *tw = tw_all + ((size_t)prime << 16);
-    const int dg = cs.digit_of[limb], n_src = cs.d[dg].n_src;
-    const u64 *src = cs.d[dg].src + (size_t)poly * cs.d[dg].src_poly_stride + col;
+    const int dg = __builtin_amdgcn_readfirstlane((int)cs.digit_of[limb]), n_src = cs.d[dg].n_src;
+    // The sources are read through a buffer resource: base (the polynomial's source limbs; far below 4 GiB), source slot
+    // and slab row sit in scalar registers, a thread supplies one 32-bit offset for all of its 16 n_src loads.
+    const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(cs.d[dg].src + (size_t)poly * cs.d[dg].src_poly_stride), 0, -1, 0x00020000);
+    const u32 voff = (u32)(col + ((threadIdx.x >> 4) << 8)) * 8u;
     const Cst *hat = cs.d[dg].hat + prime;
     const ModQ m = modq[prime];
-    const u64 *sp[NS];
+    u32 so[NS];
     u64 h[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) {
         const int ii = i < n_src ? i : 0;
-        sp[i] = src + ((size_t)cs.d[dg].src_slot[ii] << 16);
+        so[i] = __builtin_amdgcn_readfirstlane((u32)cs.d[dg].src_slot[ii]) << 19;
         h[i] = hat[(size_t)ii * cs.hat_ld].w;
     }
     if (fp[4 * prime] != 0.0)
-        cols_converted_body<NS>(base, tw, FpField(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
+        cols_converted_body<NS>(base, (u32)col, tw, FpField(modq, ninv, ninv_s, fp, prime), lds, src, voff, so, h, n_src, m);
     else if ((m.q >> 60) != 0)
-        cols_converted_body<NS>(base, tw, IntField(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
+        cols_converted_body<NS>(base, (u32)col, tw, IntField(modq, ninv, ninv_s, fp, prime), lds, src, voff, so, h, n_src, m);
     else
-        cols_converted_body<NS>(base, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds, sp, h, n_src, m);
+        cols_converted_body<NS>(base, (u32)col, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds, src, voff, so, h, n_src, m);
 }
 
 // A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
