@@ -377,14 +377,15 @@ class Context:
                                          vp(y.data_ptr()), vp(out.data_ptr()), nq_out * self.N, vp(ws.data_ptr()), vp(0)))
         return out
 
-    def moddown_batch(self, y, nq, drop_last):
-        """y: [..., nq+K, N] (clobbered) -> [..., nq - drop_last, N]"""
+    def moddown_batch(self, y, nq, drop_last, column_slab=False):
+        """y: [..., nq+K, N] (clobbered) -> [..., nq - drop_last, N]; column_slab: the three-launch form
+        (HEMM_MODDOWN_COLUMN_SLAB), same residues"""
         import torch
         n_polys = y.numel() // ((nq + self.nP) * self.N)
         nq_out = nq - 1 if drop_last else nq
         out = torch.empty(tuple(y.shape[:-2]) + (nq_out, self.N), dtype=torch.int64, device=y.device)
         ws = torch.empty_like(out)
-        check(lib().hemm_moddown_batch(self.h, vp(y.data_ptr()), nq, n_polys, int(drop_last),
+        check(lib().hemm_moddown_batch(self.h, vp(y.data_ptr()), nq, n_polys, int(bool(drop_last)) | (2 if column_slab else 0),
                                        vp(out.data_ptr()), nq_out * self.N, vp(ws.data_ptr()), vp(0)))
         return out
 

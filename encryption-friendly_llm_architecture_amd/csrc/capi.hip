@@ -477,8 +477,9 @@ int hemm_moddown_batch(hemm_context *ctx, uint64_t *y, uint32_t nq, uint32_t n_p
     chain_limbs(ctx, nq, 1, &nl);
     need(y && out && workspace && n_polys >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    launch_moddown_batch(ctx, (u64 *)y, (int)nq, (int)n_polys, drop_last != 0, (u64 *)out, out_stride,
-                         (u64 *)workspace, (hipStream_t)stream);
+    need((drop_last & ~(1 | HEMM_MODDOWN_COLUMN_SLAB)) == 0, "unknown ModDown flag");
+    launch_moddown_batch(ctx, (u64 *)y, (int)nq, (int)n_polys, (drop_last & 1) != 0, (u64 *)out, out_stride,
+                         (u64 *)workspace, (hipStream_t)stream, (drop_last & HEMM_MODDOWN_COLUMN_SLAB) != 0);
     check_launch();
     HEMM_CATCH
 }

@@ -110,6 +110,13 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
                           int n_limbs, int n_polys, size_t poly_stride, hipStream_t s, const u64 *ep_minuend = nullptr,
                           size_t ep_minuend_stride = 0, u64 *ep_out = nullptr, size_t ep_out_stride = 0,
                           const void *ep_cst_dev = nullptr);
+// out[p][j] = (y[p][j] - conversion of the n_src listed limbs of y[p] to prime j) * cst[j], j < nq_out, as inverse row
+// pass (in place on the listed limbs), one column-slab kernel (second inverse pass, conversion as lazy dot products, first
+// forward pass into conv[n_polys][nq_out][N]) and forward row pass with the fused tail.  final_scale / hat / cst: device
+// tables in source order, [n_src][hat_ld] by prime, by target limb.  false when the shape has no such form.
+bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const uint8_t *src_slot, const uint8_t *src_prime,
+                         int n_src, const void *final_scale_dev, const void *hat_dev, int hat_ld, u64 *conv, int nq_out,
+                         int n_polys, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 // inverse transform reading src (same slot numbering as data, polynomial stride src_poly_stride) and leaving the
 // coefficients in data; false when this ring size has no out-of-place form (the caller copies, then transforms)
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
@@ -158,7 +165,7 @@ int hoisted_arg_capacity();
 void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_terms, const u32 *group_off_host, int n_out,
                                int nq, u64 *y, bool b_premultiplied, hipStream_t s);
 void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
-                          u64 *conv, hipStream_t s);
+                          u64 *conv, hipStream_t s, bool slab = false);
 void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, int n_polys,
                        u64 *out, hipStream_t s, const void *terms_host = nullptr, int n_terms = 0);
 // y[o][p][j] = sum_{q < parts} part[o * parts + q][p][j] over the extended basis, y / part: [.][2][nq+K][N]

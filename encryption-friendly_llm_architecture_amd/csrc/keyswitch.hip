@@ -1297,7 +1297,7 @@ void launch_hoisted_terms_args(hemm_context *c, const void *terms_host, int n_te
 // drop_last = 1: out[p] = y[p] / (P q_{nq-1}) over nq-1 limbs (ModDown and rescale in one conversion).
 // conv: workspace [n_polys][nq_out][N].
 void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop_last, u64 *out, size_t out_stride,
-                          u64 *conv, hipStream_t s) {
+                          u64 *conv, hipStream_t s, bool slab) {
     KsTables *t = g_tables_of(c);
     const int K = c->nP, E = nq + K, nq_out = drop_last ? nq - 1 : nq;
     const size_t N = c->N;
@@ -1324,6 +1324,17 @@ void launch_moddown_batch(hemm_context *c, u64 *y, int nq, int n_polys, int drop
         sl.idx[i] = a.src_slot[i];
     }
     const bool fold = c->logN == 16;   // the inverse transform ends with (1/N)(S/q_i)^-1: no scaling pass in the conversion
+    // the three-launch form with one column-slab kernel in the middle, only on request: it moves a fifth less data but
+    // runs at two waves per SIMD and is slower on every batch size measured
+    if (slab && !(fold && lazy_dot_ok(c))) throw std::invalid_argument("the column-slab ModDown needs N = 2^16 and primes below 2^60");
+    if (slab) {
+        if (!launch_moddown_slab(c, y, (size_t)E * N, a.src_slot, a.src_prime, ns,
+                            t->dev + (drop_last ? t->drop_invn_off[nq] : t->p_invn_off),
+                            t->dev + (drop_last ? t->drop_hat_off[nq] : t->p_hat_off), c->nQ + c->nP, conv, nq_out, n_polys,
+                            out, out_stride, t->dev + (drop_last ? t->dropinv_off[nq] : t->pinv_off), s))
+            throw std::invalid_argument("the column-slab ModDown takes 4 or 5 dropped limbs");
+        return;
+    }
     launch_ntt_slots(c, y, pl, sl, ns, n_polys, (size_t)E * N, true, s,
                      fold ? t->dev + (drop_last ? t->drop_invn_off[nq] : t->p_invn_off) : nullptr);
     a.pre_scaled = fold ? 1 : 0;

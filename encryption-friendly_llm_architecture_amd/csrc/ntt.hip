@@ -16,6 +16,7 @@
 // Other sizes (2^6 .. 2^15, used by the small-parameter tests) run a plain LDS kernel with the
 // same butterfly network, so residues are identical for every N.
 #include <algorithm>
+#include <cstring>
 
 #include "hemm_internal.hpp"
 
@@ -513,6 +514,152 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         cols_converted_body<NS>(base, (u32)col, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds, src, voff, so, h, n_src, m);
 }
 
+// ------------------------------------------------------------------------------------------
+// Column-slab kernel of a ModDown (or any conversion of a few source limbs): for one (polynomial, 16-column slab) a
+// workgroup runs the second pass of the inverse transform of every source limb, keeps the canonical coefficients on
+// chip -- the last four sources in registers, one more in LDS -- and then, target limb by target limb, takes the
+// basis conversion as lazy dot products and runs the first pass of the forward transform.  The inverse result is
+// never written and the sources are never read back: the three steps are local to the slab, only the row passes on
+// either side need the other half of the 256 x 256 view.  Arithmetic, order of operations and stored values are those
+// of ntt16_cols_kernel<true> followed by ntt16_cols_converted_kernel.
+// 128 registers of sources per thread leave room for two waves per SIMD; LDS: 32 KiB exchange + 32 KiB source.
+// ------------------------------------------------------------------------------------------
+#define SLAB_REG_SOURCES 4
+struct SlabSources {
+    const u64 *src;            // first-pass output of the inverse transform (raw field values), [n_polys][.][N]
+    size_t src_poly_stride;
+    const Cst *hat;            // [n_src][hat_ld]  (S/q_i) mod prime, indexed by prime
+    const Tw *final_scale;     // [n_src]  (1/N)(S/q_i)^-1 mod q_i
+    int hat_ld, n_src, n_dst;
+    uint8_t src_slot[SLAB_REG_SOURCES + 1], src_prime[SLAB_REG_SOURCES + 1];
+    uint8_t dst_slot[HEMM_MAX_PRIMES], dst_prime[HEMM_MAX_PRIMES];
+};
+
+template <class F>
+__device__ __forceinline__ void slab_inverse(const __amdgpu_buffer_rsrc_t limb, const u32 v_inner,
+                                             const Tw *__restrict__ tw_int, const F f, u64 *lds_raw, u64 (&r)[16]) {
+    typedef typename F::E E;
+    const typename F::W *tw = (const typename F::W *)tw_int;
+    E *lds = (E *)lds_raw;
+    const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
+    E x[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = buf_load<E>(limb, v_inner, (u32)k << 11);
+    radix16_inv(f, x, tw, 16u + rh);
+    f.after_inverse_block(x);
+    __syncthreads();   // the previous exchange has been read by every wave
+#pragma unroll
+    for (int k = 0; k < 16; k++) lds[(16 * rh + k) * 16 + cc] = x[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = lds[(rh + 16 * k) * 16 + cc];
+    radix16_inv(f, x, tw, 1u);
+#pragma unroll
+    for (int k = 0; k < 16; k++) r[k] = f.scale_to_canonical(x[k]);
+}
+
+template <int NREG, bool LDS, class F>
+__device__ __forceinline__ void slab_forward(const __amdgpu_buffer_rsrc_t limb, const u32 v_inner,
+                                             const Tw *__restrict__ tw_int, const F f, u64 *lds_raw,
+                                             const u64 *__restrict__ lsrc, const u64 hl,
+                                             const u64 (&c)[SLAB_REG_SOURCES][16], const u64 (&h)[SLAB_REG_SOURCES],
+                                             const ModQ m) {
+    typedef typename F::E E;
+    const typename F::W *tw = (const typename F::W *)tw_int;
+    E *lds = (E *)lds_raw;
+    const int cc = threadIdx.x & 15, rh = threadIdx.x >> 4;
+    E x[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        Dot3 d;
+        dot3_clear(d);
+        if (LDS) dot3_add(d, lsrc[k * 256 + threadIdx.x], hl);
+#pragma unroll
+        for (int j = SLAB_REG_SOURCES - NREG; j < SLAB_REG_SOURCES; j++) dot3_add(d, c[j][k], h[j]);
+        x[k] = f.from_dot(d, m);
+    }
+    radix16_fwd(f, x, tw, 1u);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; k++) lds[swz_row(rh + 16 * k) * 16 + cc] = x[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = lds[swz_row(16 * rh + k) * 16 + cc];
+    radix16_fwd(f, x, tw, 16u + rh);
+#pragma unroll
+    for (int k = 0; k < 16; k++) buf_store<E>(limb, v_inner, (u32)k << 11, x[k]);
+}
+
+template <int NREG, bool LDS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void ntt16_slab_convert_kernel(
+    u64 *__restrict__ data, const size_t poly_stride, const Tw *__restrict__ tw_all, const Tw *__restrict__ itw_all,
+    const ModQ *__restrict__ modq, const u64 *__restrict__ ninv, const u64 *__restrict__ ninv_s,
+    const double *__restrict__ fp, const SlabSources ss) {
+    __shared__ u64 lds[256 * 16];
+    __shared__ u64 lsrc[256 * 16];
+    const int poly = blockIdx.y;
+    const u32 col = blockIdx.x * 16 + (threadIdx.x & 15);
+    const u32 v_inner = (col + ((u32)(threadIdx.x >> 4) << 12)) * 8u;   // (row 16 rh, col); row k further: scalar offset
+    constexpr int n_lds = LDS ? 1 : 0, n_src = NREG + n_lds, first_reg = SLAB_REG_SOURCES - NREG;
+    u64 c[SLAB_REG_SOURCES][16];
+#pragma unroll
+    for (int j = 0; j < SLAB_REG_SOURCES; j++)
+#pragma unroll
+        for (int k = 0; k < 16; k++) c[j][k] = 0;
+    // source i < n_lds goes to LDS, the others shift through the register sets: the last source ends in c[3]
+#pragma unroll 1
+    for (int i = 0; i < n_src; i++) {
+        const int prime = __builtin_amdgcn_readfirstlane((int)ss.src_prime[i]);
+        const __amdgpu_buffer_rsrc_t limb = limb_rsrc(
+            ss.src + (size_t)poly * ss.src_poly_stride + ((size_t)__builtin_amdgcn_readfirstlane((int)ss.src_slot[i]) << 16));
+        const Tw *tw = itw_all + ((size_t)prime << 16);
+        const Tw fs = ss.final_scale[i];
+        if (i >= n_lds) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                c[0][k] = c[1][k];
+                c[1][k] = c[2][k];
+                c[2][k] = c[3][k];
+            }
+        }
+        if (fp[4 * prime] != 0.0) {
+            FpField f(modq, ninv, ninv_s, fp, prime);
+            f.ni = (double)fs.w;
+            f.niinv = f.ni * f.qinv;
+            slab_inverse(limb, v_inner, tw, f, lds, c[3]);
+        } else {
+            IntField f(modq, ninv, ninv_s, fp, prime);
+            f.ni = fs.w;
+            f.nis = fs.ws;
+            slab_inverse(limb, v_inner, tw, f, lds, c[3]);
+        }
+        if (i < n_lds) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) lsrc[k * 256 + threadIdx.x] = c[3][k];
+        }
+    }
+#pragma unroll 1
+    for (int t = 0; t < ss.n_dst; t++) {
+        const int prime = __builtin_amdgcn_readfirstlane((int)ss.dst_prime[t]);
+        const __amdgpu_buffer_rsrc_t limb = limb_rsrc(
+            data + (size_t)poly * poly_stride + ((size_t)__builtin_amdgcn_readfirstlane((int)ss.dst_slot[t]) << 16));
+        const Tw *tw = tw_all + ((size_t)prime << 16);
+        const ModQ m = modq[prime];
+        const Cst *hat = ss.hat + prime;
+        u64 h[SLAB_REG_SOURCES];
+#pragma unroll
+        for (int j = 0; j < SLAB_REG_SOURCES; j++) {
+            const int i = n_lds + j - first_reg;
+            h[j] = j >= first_reg ? hat[(size_t)i * ss.hat_ld].w : 0;
+        }
+        const u64 hl = LDS ? hat[0].w : 0;
+        if (fp[4 * prime] != 0.0)
+            slab_forward<NREG, LDS>(limb, v_inner, tw, FpField(modq, ninv, ninv_s, fp, prime), lds, lsrc, hl, c, h, m);
+        else
+            slab_forward<NREG, LDS>(limb, v_inner, tw, IntFieldT<true>(modq, ninv, ninv_s, fp, prime), lds, lsrc, hl, c, h, m);
+    }
+}
+
 // A row's 16 threads sit in one wavefront (thread = row * 16 + column group), so the LDS exchanges of
 // the row kernel never cross a wavefront: ordering them needs no workgroup barrier, only a fence that
 // keeps the compiler from moving LDS accesses across it.
@@ -722,6 +869,67 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
     } else {
         hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw,
                            c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
+    }
+    return true;
+}
+
+// out[p][j] = (y[p][j] - conversion of the n_src listed limbs of y[p] to prime j) * cst[j] for j < nq_out, in three
+// launches: first pass of the inverse transform of the listed limbs (in place), the column-slab kernel (second inverse
+// pass, conversion, first forward pass into conv), second forward pass with the fused tail.  Same residues as the
+// four-launch chain.  false when the shape has no such form (nothing was launched).
+bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const uint8_t *src_slot, const uint8_t *src_prime,
+                         int n_src, const void *final_scale_dev, const void *hat_dev, int hat_ld, u64 *conv, int nq_out,
+                         int n_polys, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s) {
+    if (c->logN != 16 || n_src < 4 || n_src > 5 || nq_out < 1 || nq_out > HEMM_MAX_PRIMES) return false;
+    if (n_polys <= 0) return true;
+    SlabSources ss;
+    memset(&ss, 0, sizeof(ss));
+    LimbList sp, ssl, cl, ident;
+    memset(&sp, 0, sizeof(sp));
+    memset(&ssl, 0, sizeof(ssl));
+    for (int j = 0; j < HEMM_MAX_PRIMES; j++) cl.idx[j] = ident.idx[j] = (uint8_t)j;
+    for (int i = 0; i < n_src; i++) {
+        ss.src_slot[i] = ssl.idx[i] = src_slot[i];
+        ss.src_prime[i] = sp.idx[i] = src_prime[i];
+    }
+    for (int j = 0; j < nq_out; j++) {
+        ss.dst_slot[j] = (uint8_t)j;
+        ss.dst_prime[j] = (uint8_t)j;
+    }
+    ss.hat = (const Cst *)hat_dev;
+    ss.final_scale = (const Tw *)final_scale_dev;
+    ss.hat_ld = hat_ld;
+    ss.n_src = n_src;
+    ss.n_dst = nq_out;
+    ss.src_poly_stride = y_stride;
+    // same algorithmic bytes as the separate launches: the dropped limbs in and out of the inverse transform, the
+    // conversion's sources, the minuend in and the result out of the forward transform
+    account(c, TR_NTT, (size_t)2 * n_src * n_polys * c->N * 8, 1);
+    account(c, TR_BCONV, (size_t)n_src * n_polys * c->N * 8, 1);
+    account(c, TR_NTT, (size_t)2 * nq_out * n_polys * c->N * 8, 1);
+    const dim3 block(256);
+    const size_t conv_stride = (size_t)nq_out << 16;
+    const int widest = n_src > nq_out ? n_src : nq_out;
+    int run = 448 / widest;
+    if (run < 1) run = 1;
+    for (int p0 = 0; p0 < n_polys; p0 += run) {
+        const int np = n_polys - p0 < run ? n_polys - p0 : run;
+        u64 *yp = y + (size_t)p0 * y_stride;
+        u64 *cp = conv + (size_t)p0 * conv_stride;
+        ss.src = yp;
+        hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * n_src * np), block, 0, s, yp, (const Tw *)c->d_iw,
+                           c->d_modq, c->d_fp, sp, ssl, n_src, y_stride, NttEpilogue{});
+#define SLAB_CASE(NREG, LDS)                                                                                             \
+    hipLaunchKernelGGL((ntt16_slab_convert_kernel<NREG, LDS>), dim3(16, np), block, 0, s, cp, conv_stride,             \
+                       (const Tw *)c->d_w, (const Tw *)c->d_iw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ss)
+        if (n_src == 5)
+            SLAB_CASE(4, true);
+        else
+            SLAB_CASE(4, false);
+#undef SLAB_CASE
+        NttEpilogue ep{yp, out + (size_t)p0 * out_stride, (const Tw *)cst_dev, y_stride, out_stride};
+        hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * nq_out * np), block, 0, s, cp, (const Tw *)c->d_w,
+                           c->d_modq, c->d_fp, cl, ident, nq_out, conv_stride, ep);
     }
     return true;
 }

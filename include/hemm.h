@@ -213,7 +213,13 @@ int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const ui
 
 /* y [n_polys][nq+n_p][N] (clobbered) -> out [n_polys][nq - drop_last][N]: division by P (drop_last = 0)
  * or by P*q_{nq-1} (drop_last = 1, ModDown and rescale in one basis conversion);
- * workspace >= n_polys*(nq-drop_last)*N words. */
+ * workspace >= n_polys*(nq-drop_last)*N words.
+ * drop_last | HEMM_MODDOWN_COLUMN_SLAB (N = 2^16, 4 or 5 dropped limbs, primes below 2^60) runs the same arithmetic
+ * in three launches instead of four: the second pass of the inverse transform, the basis conversion and the first
+ * pass of the forward transform in one kernel per 16-column slab, so the dropped limbs are not written in
+ * coefficient form and read back (identical residues; a fifth less memory traffic, but slower where measured, so
+ * nothing in the library selects it by itself). */
+#define HEMM_MODDOWN_COLUMN_SLAB 2
 int hemm_moddown_batch(hemm_context *ctx, uint64_t *y, uint32_t nq, uint32_t n_polys, int drop_last,
                        uint64_t *out, size_t out_stride, uint64_t *workspace, void *stream);
 typedef struct {

@@ -251,6 +251,116 @@ def test_rescale_is_exact_division(mid):
             assert int(out[j, n]) == want % mods[j]
 
 
+@pytest.mark.parametrize("drop_last", [0, 1])
+def test_moddown_drop_vs_crt(mid, drop_last):
+    """Division by P, or by P q_last in one conversion, against big integers: with D the product of the dropped
+    primes and s the float-free lift of the dropped residues (s = y mod D up to a multiple u D, 0 <= u < number of
+    dropped limbs), every kept limb is (y_j - s) / D mod q_j -- the floor of y / D shifted down by u, never rounded."""
+    rng = np.random.default_rng(17)
+    N, nq = mid.N, 5
+    primes = [mid.prime_of(j, nq) for j in range(nq + mid.nP)]
+    coef = np.stack([rand_res(rng, mid.mods[pi], N) for pi in primes])
+    y = coef.copy()
+    mid.ntt(y, primes)
+    nq_out = nq - drop_last
+    out = np.empty((nq_out, N), dtype=np.uint64)
+    mid.L.orc_moddown_drop(mid.h, _p(y), nq, drop_last, _p(out))
+    mid.ntt(out, list(range(nq_out)), inverse=True)
+    dropped = ([nq - 1] if drop_last else []) + list(range(nq, nq + mid.nP))      # limb slots
+    dmods = [mid.mods[primes[l]] for l in dropped]
+    D = 1
+    for m in dmods:
+        D *= m
+    kept = [mid.q[j] for j in range(nq_out)]
+    for n in range(0, N, 23):
+        s = 0
+        for l, m in zip(dropped, dmods):
+            dh = D // m
+            s += (int(coef[l, n]) * pow(dh, -1, m) % m) * dh
+        exact, _ = crt([coef[l, n] for l in dropped], dmods)
+        u = (s - exact) // D
+        assert s % D == exact and 0 <= u < len(dropped)
+        full, _ = crt([coef[j, n] for j in range(nq_out)] + [coef[l, n] for l in dropped], kept + dmods)
+        assert (full - exact) % D == 0
+        for j, q in enumerate(kept):
+            assert int(out[j, n]) == (int(coef[j, n]) - s) * pow(D, -1, q) % q
+            assert int(out[j, n]) == ((full - exact) // D - u) % q          # floor(y / D) - u
+
+
+def test_inner_product_vs_bigint(mid):
+    rng = np.random.default_rng(18)
+    N, nq = mid.N, 5
+    E, full = nq + mid.nP, mid.nQ + mid.nP
+    beta = (nq + mid.alpha - 1) // mid.alpha
+    primes = [mid.prime_of(j, nq) for j in range(E)]
+    ext = np.stack([[rand_res(rng, mid.mods[pi], N) for pi in primes] for _ in range(beta)])
+    evk = np.stack([[[rand_res(rng, m, N) for m in mid.mods] for _ in range(2)] for _ in range(mid.dnum)])
+    ext[0, 0, :4] = np.uint64(mid.mods[0] - 1)          # both factors at q - 1
+    evk[0, :, 0, :4] = np.uint64(mid.mods[0] - 1)
+    acc = np.empty((2, E, N), dtype=np.uint64)
+    mid.L.orc_inner_product(mid.h, _p(ext), _p(evk), nq, _p(acc))
+    for pol in range(2):
+        for j, pi in enumerate(primes):
+            q = mid.mods[pi]
+            for n in list(range(4)) + list(range(5, N, 97)):
+                want = sum(int(ext[d, j, n]) * int(evk[d, pol, pi, n]) for d in range(beta)) % q
+                assert int(acc[pol, j, n]) == want
+
+
+def test_hoisted_term_vs_bigint(small):
+    """y (+)= mask * (<rot_g(ext), evk> + P rot_g(b)): the automorphism is checked through the coefficient domain
+    (X -> X^g by brute-force substitution), the products with big integers."""
+    o = small
+    rng = np.random.default_rng(19)
+    N, nq = o.N, 5                    # two digits
+    E, full = nq + o.nP, o.nQ + o.nP
+    beta = (nq + o.alpha - 1) // o.alpha
+    assert beta == 2
+    primes = [o.prime_of(j, nq) for j in range(E)]
+    g = pow(5, 7, 2 * N)
+    P = 1
+    for p in o.p:
+        P *= p
+
+    def substitute(poly, q):          # X -> X^g on coefficients, sign from X^N = -1
+        out = [0] * N
+        for i, v in enumerate(poly):
+            e = i * g % (2 * N)
+            out[e % N] = int(v) % q if e < N else (q - int(v)) % q
+        return np.array(out, dtype=np.uint64)
+
+    def rotated_ntt(x, pi):           # NTT form of the substituted polynomial
+        c = x.copy()
+        o.ntt(c.reshape(1, N), [pi], inverse=True)
+        c = substitute(c, o.mods[pi])
+        o.ntt(c.reshape(1, N), [pi])
+        return c
+
+    ext = np.stack([[rand_res(rng, o.mods[pi], N) for pi in primes] for _ in range(beta)])
+    b = np.stack([rand_res(rng, o.q[j], N) for j in range(nq)])
+    evk = np.stack([[[rand_res(rng, m, N) for m in o.mods] for _ in range(2)] for _ in range(o.dnum)])
+    mask = np.stack([rand_res(rng, o.mods[pi], N) for pi in primes])
+    y0 = np.stack([[rand_res(rng, o.mods[pi], N) for pi in primes] for _ in range(2)])
+    for accumulate, with_b, with_mask in ((0, True, True), (1, True, False), (1, False, True)):
+        y = y0.copy()
+        o.L.orc_hoisted_term(o.h, _p(ext), _p(b) if with_b else None, _p(evk), _p(mask) if with_mask else None,
+                             g, nq, _p(y), accumulate)
+        for j, pi in enumerate(primes):
+            q = o.mods[pi]
+            rext = [rotated_ntt(ext[d, j], pi) for d in range(beta)]
+            rb = rotated_ntt(b[j], pi) if (with_b and j < nq) else None
+            for pol in range(2):
+                for n in range(N):
+                    s = sum(int(rext[d][n]) * int(evk[d, pol, pi, n]) for d in range(beta))
+                    if pol == 0 and rb is not None:
+                        s += P * int(rb[n])
+                    if with_mask:
+                        s *= int(mask[j, n])
+                    if accumulate:
+                        s += int(y0[pol, j, n])
+                    assert int(y[pol, j, n]) == s % q, (accumulate, j, pol, n)
+
+
 def test_tensor_and_imag_unit(mid):
     rng = np.random.default_rng(9)
     N, nq = mid.N, 3
