@@ -277,3 +277,88 @@ def test_rotation_step_set_at_level_20_of_24(chain24, step):
     want = orc.left_rotate(O.Ct(ct, 1.0), step)
     got = host(ctx.rotate(dct, dev(orc.keys.pop(("gal", g))), g, 21))
     assert np.array_equal(got, want.data)
+
+
+# ---- basis conversions at the upper end of their lazy accumulators ------------------------------------------------
+def _product(ms):
+    out = 1
+    for m in ms:
+        out *= int(m)
+    return out
+
+
+def _worst_case_limb(orc, prime_idx, basis):
+    """NTT form of the polynomial whose every coefficient c satisfies [c (S / q)^-1]_q = q - 1 for the basis product
+    S: the residue a fast basis conversion multiplies its constants with is then q - 1 at every position."""
+    q = orc.mods[prime_idx]
+    hat = _product(b for b in basis if b != q) % q
+    x = np.full((1, orc.N), (q - 1) * hat % q, dtype=np.uint64)
+    # what the conversion will see, checked before the transform hides it
+    assert int(x[0, 0]) * pow(hat, -1, q) % q == q - 1
+    orc.ntt(x, [prime_idx])
+    return x[0]
+
+
+def _mixed_chain():
+    """8 chain primes just below 2^60 and 8 near 2^42 with 8 special primes below 2^60, two digits of 8 limbs: the
+    widest conversions the fused transform pass takes, in both directions (eight 60-bit sources into primes below
+    2^44, which finish in double precision, and into 60-bit primes)."""
+    pkg = load_package()
+    big = pkg.primes_below(60, 16, 16)
+    qs = big[:8] + pkg.primes_below(42, 16, 8)
+    ps = big[8:]
+    return O.Oracle(16, qs, ps, 2, threads=THREADS), pkg.Context(16, qs, ps, 2)
+
+
+def test_conversions_with_every_source_residue_at_q_minus_1(bench):
+    """ModUp, ModDown merged with the rescale, plain ModDown and rescale on inputs whose scaled coefficient-form
+    residues are q_i - 1 in every source limb and at every position: the lazy dot products of the fused conversion
+    pass (16 products of 32 x 28 bits per 64-bit accumulator, finished in double precision for targets below 2^44)
+    at the largest sources they can meet, 5 sources on the preset and 8 on a chain of two 8-limb digits."""
+    rng = np.random.default_rng(77)
+    for orc, ctx, nq in ((bench.orc, bench.ctx, 7), (bench.orc, bench.ctx, 13)) + tuple(
+            (o, c, 16) for o, c in (_mixed_chain(),)):
+        N, K, alpha = orc.N, orc.nP, orc.alpha
+        # ModUp: limb j carries -(Q_d / q_j) for its digit d
+        poly = np.empty((nq, N), dtype=np.uint64)
+        for j in range(nq):
+            d = j // alpha
+            basis = orc.q[d * alpha:min(nq, (d + 1) * alpha)]
+            poly[j] = _worst_case_limb(orc, j, basis)
+        want = orc.modup(poly)
+        assert np.array_equal(host(ctx.modup(dev(poly), nq)), want)
+        assert np.array_equal(host(ctx.modup_batch(dev(np.stack([poly, poly])), nq)[1]), want)
+        # ModDown (with and without the rescale merged in): dropped limbs at the worst case, the others random
+        E = nq + K
+        ext_mods = [orc.mods[orc.prime_of(j, nq)] for j in range(E)]
+        for drop in (True, False):
+            y = rand_limbs(rng, ext_mods, (2,), N)
+            slots = ([nq - 1] if drop else []) + list(range(nq, E))
+            basis = [ext_mods[l] for l in slots]
+            for l in slots:
+                y[:, l] = _worst_case_limb(orc, orc.prime_of(l, nq), basis)
+            want = orc.moddown_drop(y, nq, drop)
+            assert np.array_equal(host(ctx.moddown_batch(dev(y), nq, drop)), want), (nq, drop)
+            if len(slots) in (4, 5):
+                assert np.array_equal(host(ctx.moddown_batch(dev(y), nq, drop, column_slab=True)), want), (nq, drop)
+        # rescale: the last limb's coefficients all q_last - 1
+        ct = rand_limbs(rng, orc.q[:nq], (2,), N)
+        ct[:, nq - 1] = _worst_case_limb(orc, nq - 1, [orc.q[nq - 1]])
+        want = orc.rescale(O.Ct(ct, 1.0)).data
+        assert np.array_equal(host(ctx.rescale(dev(ct), nq)), want)
+
+
+def test_moddown_column_slab_form_same_residues(bench, chain24):
+    """HEMM_MODDOWN_COLUMN_SLAB: the three-launch ModDown (inverse column pass, conversion and forward column pass in
+    one kernel per slab) against the four-launch chain and the oracle; 4 and 5 dropped limbs, a 42-bit and a 60-bit
+    last limb (the fifth source goes through LDS in either arithmetic)."""
+    import torch
+    rng = np.random.default_rng(78)
+    for orc, ctx, nq, n_polys in ((bench.orc, bench.ctx, 7, 64), (bench.orc, bench.ctx, 13, 3), (chain24[0], chain24[1], 21, 2)):
+        N, E = orc.N, nq + orc.nP
+        ext_mods = [orc.mods[orc.prime_of(j, nq)] for j in range(E)]
+        y = rand_limbs(rng, ext_mods, (n_polys,), N)
+        for drop in (True, False):
+            slab = ctx.moddown_batch(dev(y), nq, drop, column_slab=True)
+            assert torch.equal(slab, ctx.moddown_batch(dev(y), nq, drop))
+            assert np.array_equal(host(slab[-2:]), orc.moddown_drop(y[-2:], nq, drop))
