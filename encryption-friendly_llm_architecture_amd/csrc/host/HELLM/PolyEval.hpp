@@ -1,5 +1,7 @@
 // Polynomial evaluation on ciphertexts.
 //   HELLM::Exp::exp_iter            reference ciphertext/src/Exp.cpp:41-52, include/HELLM/Exp.hpp
+//   HELLM::Exp::exp_iter_Parallel   reference ciphertext/src/Exp.cpp:55-77 (called by HEMMer::expParallelInplace,
+//                                   src/HEMMer.cpp:1416, with 14 iterations on the six score tensors of a layer)
 //   HELLM::ReLU::evalOddPolynomial  reference ciphertext/src/ReLU.cpp:53-188 (Han-Ki baby-step / giant-step)
 //   HEaaN::Math::ChebyshevCoefficients / linearTransform / evaluateChebyshevExpansion
 //                                   declared by the closed HEaaN-math (PolynomialEvaluator.hpp:19-63, used as
@@ -13,6 +15,7 @@
 #include <vector>
 
 #include "HEaaN/HEaaN.hpp"
+#include "HELLM/HETensor.hpp"
 
 namespace HEaaN {
 namespace Math {
@@ -26,17 +29,26 @@ struct Interval {
 using InputInterval = Interval;
 using DiffInterval = Interval;
 
-// HEaaN-math/tools/PolynomialEvaluator.hpp:19-40: same members, same constructor arithmetic.  The coefficients are
-// NOT a plain Chebyshev series: entry bs * i + j multiplies T_j times the product of T_{2^k bs} over the set bits k
-// of i (the tables of include/HELLM/*RemezCoeff.hpp are stored that way).
+// The coefficient holder HEaaN-math declares (tools/PolynomialEvaluator.hpp:19-40): member names and constructor
+// arguments are that interface, so callers written against it compile.  The coefficients are NOT a plain Chebyshev
+// series: entry bs * i + j multiplies T_j times the product of T_{2^k bs} over the set bits k of i (the tables of
+// include/HELLM/*RemezCoeff.hpp are stored that way).  Derived sizes: the table is cut into blocks of num_bs entries
+// (all of it when no block size is given), num_gs blocks in all; a block needs ceil(log2 num_bs) levels, combining
+// the blocks ceil(log2 num_gs) more.
 enum PolynomialBasis { basic, odd };
 struct ChebyshevCoefficients {
+    static u64 ceilLog2(u64 v) {
+        u64 bits = 0;
+        while ((u64(1) << bits) < v) bits++;
+        return bits;
+    }
     ChebyshevCoefficients(std::vector<Real> coefficient, u64 num_baby_step, PolynomialBasis base = PolynomialBasis::basic)
         : coeffs{std::move(coefficient)}, basis{base} {
-        num_bs = (num_baby_step > 0) ? num_baby_step : coeffs.size();
-        num_gs = static_cast<u64>(std::ceil(static_cast<Real>(coeffs.size()) / static_cast<Real>(num_bs)));
-        log_bs = static_cast<u64>(std::ceil(std::log2(num_bs)));
-        log_gs = static_cast<u64>(std::ceil(std::log2(num_gs)));
+        const u64 n = coeffs.size();
+        num_bs = num_baby_step != 0 ? num_baby_step : n;
+        num_gs = num_bs != 0 ? (n + num_bs - 1) / num_bs : 0;
+        log_bs = ceilLog2(num_bs);
+        log_gs = ceilLog2(num_gs);
         level_cost = log_bs + log_gs;
     }
     std::vector<Real> coeffs;
@@ -68,6 +80,12 @@ namespace Exp {
 // (1 + op / 2^num_iter)^(2^num_iter): num_iter + 1 levels
 void exp_iter(const HEaaN::HomEvaluator &eval, const HEaaN::Bootstrapper &btp, const HEaaN::Ciphertext &op,
               HEaaN::Ciphertext &res, int num_iter);
+// The same on every tensor of op, in place, the squarings interleaved pair by pair: tensors 2j and 2j+1 are squared
+// together in each of the num_iter rounds, and a pair that has reached the bootstrap level is first merged into one
+// complex ciphertext and bootstrapped as one (here: raises).  As in the reference, a trailing tensor without a partner
+// is scaled and shifted but never squared.
+void exp_iter_Parallel(const HEaaN::HomEvaluator &eval, const HEaaN::Bootstrapper &btp, std::vector<HELLM::CtxtTensor> &op,
+                       int num_iter);
 }  // namespace Exp
 namespace ReLU {
 // sum over odd i of polynomial[i] ctxt^i; k baby steps (power of two), l giant-step powers ctxt^k, ctxt^2k, ...

@@ -352,6 +352,7 @@ public:
     explicit Bootstrapper(const HomEvaluator &, u64 min_level = 3) : min_level_(min_level) {}
     u64 getMinLevelForBootstrap() const { return min_level_; }
     void bootstrap(const Ciphertext &, Ciphertext &) const;
+    void bootstrap(const Ciphertext &, Ciphertext &, Ciphertext &) const;   // complex input -> real and imaginary part
     void bootstrapExtended(const Ciphertext &, Ciphertext &) const;
     void bootstrapExtended(const Ciphertext &, Ciphertext &, Ciphertext &) const;
 

@@ -377,6 +377,22 @@ int hellm_mult(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct *
     *out = r;
     FACADE_CATCH
 }
+int hellm_mult_const(hellm_hemmer *h, const hellm_ct *a, double re, double im, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().mult(a->t.get(), HEaaN::Complex(re, im), r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
+int hellm_add_const(hellm_hemmer *h, const hellm_ct *a, double re, double im, hellm_ct **out) {
+    FACADE_TRY
+    need(h && a && out, "null argument");
+    hellm_ct *r = new hellm_ct{a->t};
+    h->m->getEval().add(a->t.get(), HEaaN::Complex(re, im), r->t.get());
+    *out = r;
+    FACADE_CATCH
+}
 int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out) {
     FACADE_TRY
     need(h && a && b && out, "null argument");
@@ -400,6 +416,19 @@ int hellm_exp_iter(hellm_hemmer *h, const hellm_ct *a, int num_iter, hellm_ct **
     hellm_ct *r = new hellm_ct{a->t};
     HELLM::Exp::exp_iter(h->m->getEval(), h->m->getBtp(), a->t.get(), r->t.get(), num_iter);
     *out = r;
+    FACADE_CATCH
+}
+int hellm_exp_iter_parallel(hellm_hemmer *h, hellm_ct **cts, uint32_t n, int num_iter) {
+    FACADE_TRY
+    need(h && cts && num_iter >= 0, "bad argument");
+    std::vector<HELLM::CtxtTensor> op;
+    op.reserve(n);
+    for (uint32_t i = 0; i < n; i++) {
+        need(cts[i] != nullptr, "null ciphertext");
+        op.push_back(cts[i]->t);
+    }
+    HELLM::Exp::exp_iter_Parallel(h->m->getEval(), h->m->getBtp(), op, num_iter);
+    for (uint32_t i = 0; i < n; i++) cts[i]->t = op[i];
     FACADE_CATCH
 }
 int hellm_eval_odd_polynomial(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, int k, int l,

@@ -473,6 +473,9 @@ void HomEvaluator::matmul(const std::vector<Ciphertext> &cts, const Plaintext &p
 void Bootstrapper::bootstrap(const Ciphertext &, Ciphertext &) const {
     throw RuntimeException("bootstrapping is not part of this build");
 }
+void Bootstrapper::bootstrap(const Ciphertext &, Ciphertext &, Ciphertext &) const {
+    throw RuntimeException("bootstrapping is not part of this build");
+}
 void Bootstrapper::bootstrapExtended(const Ciphertext &, Ciphertext &) const {
     throw RuntimeException("bootstrapping is not part of this build");
 }

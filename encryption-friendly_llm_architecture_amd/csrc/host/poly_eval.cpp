@@ -20,6 +20,24 @@ void exp_iter(const HomEvaluator &eval, const Bootstrapper &btp, const Ciphertex
     res = std::move(r);
 }
 
+void exp_iter_Parallel(const HomEvaluator &eval, const Bootstrapper &btp, std::vector<HELLM::CtxtTensor> &op, int num_iter) {
+    for (auto &t : op) {
+        eval.mult(t.get(), Complex(1.0 / std::pow(2, num_iter), 0.0), t.get());
+        eval.add(t.get(), Complex(1.0, 0.0), t.get());
+    }
+    for (int i = 0; i < num_iter; i++)
+        for (size_t j = 0; j < op.size() / 2; j++) {
+            Ciphertext &a = op[2 * j].get(), &b = op[2 * j + 1].get();
+            if (a.getLevel() == btp.getMinLevelForBootstrap()) {
+                eval.multImagUnit(b, b);
+                eval.add(a, b, a);
+                btp.bootstrap(a, a, b);
+            }
+            eval.square(a, a);
+            eval.square(b, b);
+        }
+}
+
 }  // namespace Exp
 
 namespace ReLU {

@@ -55,6 +55,8 @@ def _L():
         for n in ("hellm_mult", "hellm_add", "hellm_complex_packing", "hellm_complex_packing_rev",
                   "hellm_complex_packing_pt", "hellm_repack_not_bts", "hellm_repack_lora_opti"):
             getattr(L, n).argtypes = [vp, vp, vp, pvp]
+        for n in ("hellm_mult_const", "hellm_add_const"):
+            getattr(L, n).argtypes = [vp, vp, ctypes.c_double, ctypes.c_double, pvp]
         L.hellm_matmul_high_low.argtypes = [vp, vp, vp, u32, u32, pvp]
         L.hellm_matmul_low_high.argtypes = [vp, vp, vp, u32, u32, pvp]
         L.hellm_matmul_low_low.argtypes = [vp, vp, vp, u32, u32, u32, pvp]
@@ -85,6 +87,7 @@ def _L():
         L.hellm_ct_save.argtypes = [vp, vp, ctypes.c_char_p]
         L.hellm_ct_load.argtypes = [vp, ctypes.c_char_p, pvp]
         L.hellm_exp_iter.argtypes = [vp, vp, ctypes.c_int, pvp]
+        L.hellm_exp_iter_parallel.argtypes = [vp, pvp, ctypes.c_uint32, ctypes.c_int]
         L.hellm_eval_odd_polynomial.argtypes = [vp, vp, dp, u32, ctypes.c_int, ctypes.c_int, pvp]
         L.hellm_eval_chebyshev.argtypes = [vp, vp, dp, u32, u32, ctypes.c_double, pvp]
         L.hellm_linear_transform.argtypes = [vp, vp, ctypes.c_double, ctypes.c_double, pvp]
@@ -326,6 +329,15 @@ class HEMMer:
     def add(self, a, b):
         return self._new(Ct, "hellm_add", a.h, b.h)
 
+    def mult_const(self, a, c):
+        """HomEvaluator::mult(ct, constant): a Gaussian-integer constant does not consume a level"""
+        c = complex(c)
+        return self._new(Ct, "hellm_mult_const", a.h, c.real, c.imag)
+
+    def add_const(self, a, c):
+        c = complex(c)
+        return self._new(Ct, "hellm_add_const", a.h, c.real, c.imag)
+
     def reduce_row_sum_with_scaled_mask(self, a, mask_left, mask_right):
         import numpy as np
         ml = np.ascontiguousarray(mask_left, dtype=np.float64)
@@ -377,6 +389,11 @@ class HEMMer:
     def exp_iter(self, a, num_iter):
         """(1 + a / 2^num_iter)^(2^num_iter) on the slots (HELLM::Exp::exp_iter)"""
         return self._new(Ct, "hellm_exp_iter", a.h, num_iter)
+
+    def exp_iter_parallel(self, cts, num_iter):
+        """HELLM::Exp::exp_iter_Parallel: exp_iter on every tensor of the list in place, squared pair by pair"""
+        arr = (vp * len(cts))(*[c.h for c in cts])
+        check(_L().hellm_exp_iter_parallel(self.h, arr, len(cts), num_iter))
 
     def eval_odd_polynomial(self, a, coeffs, k, l):
         """sum over odd i of coeffs[i] a^i (HELLM::ReLU::evalOddPolynomial)"""

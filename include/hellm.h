@@ -76,6 +76,10 @@ int hellm_left_rotate(hellm_hemmer *h, const hellm_ct *a, uint64_t rot, hellm_ct
 int hellm_conjugate(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);
 int hellm_mult(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);
 int hellm_add(hellm_hemmer *h, const hellm_ct *a, const hellm_ct *b, hellm_ct **out);
+/* HomEvaluator::mult / add with a complex constant (HEaaN/HomEvaluator.hpp:168-176, 119-127): a constant that is a
+ * Gaussian integer multiplies without consuming a level (the reference's mult(ct, -2), TransformerBlock.cpp:2487) */
+int hellm_mult_const(hellm_hemmer *h, const hellm_ct *a, double re, double im, hellm_ct **out);
+int hellm_add_const(hellm_hemmer *h, const hellm_ct *a, double re, double im, hellm_ct **out);
 int hellm_level_down(hellm_hemmer *h, const hellm_ct *a, uint32_t target_level, hellm_ct **out);
 int hellm_mult_imag_unit(hellm_hemmer *h, const hellm_ct *a, hellm_ct **out);
 
@@ -107,6 +111,9 @@ int hellm_ct_load(hellm_hemmer *h, const char *file, hellm_ct **out);
 
 /* polynomial evaluation on the slots
  * exp_iter: HELLM::Exp::exp_iter (src/Exp.cpp:41-52), (1 + x / 2^k)^(2^k);
+ * exp_iter_parallel: HELLM::Exp::exp_iter_Parallel (src/Exp.cpp:55-77) on n tensors in place, squared pair by pair
+ *   (an unpaired last tensor is scaled and shifted but not squared, as in the reference); fails where the reference
+ *   would bootstrap;
  * eval_odd_polynomial: HELLM::ReLU::evalOddPolynomial (src/ReLU.cpp:165-188), coeffs[i] = coefficient of x^i,
  *   k baby steps (power of two), l giant-step powers;
  * eval_chebyshev: HEaaN::Math::evaluateChebyshevExpansion (external/include/HEaaN-math/tools/PolynomialEvaluator.hpp:49-63)
@@ -115,6 +122,7 @@ int hellm_ct_load(hellm_hemmer *h, const char *file, hellm_ct **out);
  *   (the layout of the tables in include/HELLM/*RemezCoeff.hpp); baby_steps = 0 means one block: a plain series;
  * linear_transform: HEaaN::Math::linearTransform (:42-47), (2 / (right - left)) * (x - (right + left) / 2). */
 int hellm_exp_iter(hellm_hemmer *h, const hellm_ct *a, int num_iter, hellm_ct **out);
+int hellm_exp_iter_parallel(hellm_hemmer *h, hellm_ct **cts, uint32_t n, int num_iter);
 int hellm_eval_odd_polynomial(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs, int k, int l,
                               hellm_ct **out);
 int hellm_eval_chebyshev(hellm_hemmer *h, const hellm_ct *a, const double *coeffs, uint32_t n_coeffs,

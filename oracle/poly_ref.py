@@ -1,6 +1,7 @@
 """TEST INFRASTRUCTURE ONLY -- CPU restatement of the polynomial evaluation routines built on the evaluator:
 
   * exp_iter             reference ciphertext/src/Exp.cpp:41-52   ((1 + x / 2^k)^(2^k) by repeated squaring)
+  * exp_iter_parallel    reference ciphertext/src/Exp.cpp:55-77   (the same on a list of tensors, pair by pair)
   * eval_odd_polynomial  reference ciphertext/src/ReLU.cpp:53-188 (Han-Ki baby-step / giant-step for odd
                          polynomials given by monomial coefficients; products stay un-relinearised until
                          a giant-step multiplication needs them)
@@ -25,6 +26,17 @@ def exp_iter(ev, x, num_iter):
     for _ in range(num_iter):
         r = ev.mult(r, r)
     return r
+
+
+def exp_iter_parallel(ev, xs, num_iter):
+    """reference ciphertext/src/Exp.cpp:55-77: every tensor scaled and shifted, then num_iter rounds in which the
+    pairs (2j, 2j+1) are squared; a trailing tensor without a partner is never squared."""
+    xs = [ev.add_const(ev.mult_const(x, 1.0 / math.pow(2, num_iter)), 1.0) for x in xs]
+    for _ in range(num_iter):
+        for j in range(len(xs) // 2):
+            xs[2 * j] = ev.mult(xs[2 * j], xs[2 * j])
+            xs[2 * j + 1] = ev.mult(xs[2 * j + 1], xs[2 * j + 1])
+    return xs
 
 
 # ---- odd polynomials, monomial basis (ReLU.cpp) ----------------------------------------------------

@@ -7,11 +7,11 @@
     (two chained CCMMs);
   * the same rank-2 update through the low-rank path the reference's LoRA layers use (matMulHighLow per
     activation pair, repackToOneCol, matMulLowLow per output pair; src/TransformerBlock.cpp:1785-1835);
-  * one attention head: S = Q K^T (CCMM), a degree-15 Chebyshev polynomial of the scores, then P V (CCMM).
+  * attention heads with the Gaussian-kernel score of the reference's layer: norms by squaring and rotate-and-sum,
+    -2 Q K^T + |q|^2 + |k|^2 (CCMM), a degree-15 Chebyshev table of exp(-x / 16), then scores x V (CCMM).
 """
 import numpy as np
 import pytest
-from numpy.polynomial import chebyshev as C
 
 from __graft_entry__ import load_package
 
@@ -101,35 +101,46 @@ def test_lora_low_rank_path(H):
         assert np.abs(d[1] - want[:, (2 * i + 1) * n:(2 * i + 2) * n]).max() < TOL
 
 
-def test_attention_head():
-    # 12 levels hold scores (3) + polynomial (4) + scores x V (3 or 4) only if the products may run down to level 1:
-    # the preset keeps the reference's rule "bootstrap below level 4 + 3", so this uses the same primes with the
-    # minimum bootstrap level set to 0
+def test_attention_heads_gaussian_kernel():
+    """Four heads (one pair-layout ciphertext of Q, K, V) through the score of the reference's attention layer:
+    maskRightLeft, squares, oneMatRotSumInplace, transposed key norms, -2 Q K^T + |q|^2 + |k|^2, the degree-15
+    table of exp(-x / 16), scores x V; every stage against float64.  12 levels hold masks (1) + scores (3) +
+    polynomial (4) + scores x V (3) only if the products may run down to level 1: the preset keeps the reference's
+    rule "bootstrap below level 4 + 3", so this uses the same primes with the minimum bootstrap level set to 0."""
     load_package()
+    import bench
     from efla_amd import hellm
     from oracle import oracle as O
     qs, ps = O.ckks_chain(16, 13, 4)
     H = hellm.HEMMer(16, qs, ps, dnum=3, min_bootstrap_level=0, seed=3)
     rng = np.random.default_rng(12)
     n, d = 128, 64
-    Q, K, V = (0.1 * rng.normal(size=(n, d)) for _ in range(3))
-    pad = lambda M: np.pad(M, ((0, n - M.shape[0]), (0, n - M.shape[1])))
-    cq, ckt, cv = H.encrypt(pad(Q)), H.encrypt(pad(K.T)), H.encrypt(pad(V))
-    s = H.single_cc_matmul(cq, ckt, 9)                       # scores, level 9
-    S = Q @ K.T
-    assert np.abs(H.decrypt(s) - S).max() < TOL
-    # degree-15 Chebyshev interpolant of exp(-(1 - t)^2 / 2 * 4) on [-1, 1] as a stand-in for the paper's
-    # Gaussian-kernel score (any smooth kernel exercises the same evaluation)
-    f = lambda t: np.exp(-2.0 * (1.0 - t) ** 2)
-    coef = C.chebinterpolate(f, 15)
-    from oracle import poly_ref as P
-    p = H.eval_chebyshev(s, P.cheb_plain_to_product(coef, 4), 4)   # tables are in the baby-step / giant-step product basis
-    assert p.info()["level"] == 9 - 4                              # level_cost = log2(4) + log2(4)
-    assert np.abs(H.decrypt(p) - f(S)).max() < 2 ** -9
-    out = H.single_cc_matmul(p, cv, 1)
-    assert out.info()["level"] == 1
-    want = (f(S) @ pad(V))[:, :d]
-    assert np.abs(H.decrypt(out)[:, :d] - want).max() < 2 ** -8
+    Q, K, V = (0.1 * rng.normal(size=(n, 12 * d)) for _ in range(3))
+    (q, k, kt, v), = bench.gk_attention_inputs(H, Q, K, V, [1])
+    # the stages of the first half (heads 8 and 10: left halves of tiles 2 and 3)
+    mq, mk = H.mask_right_left(q), H.mask_right_left(k)
+    sq, sk = [H.mult(x, x) for x in mq], [H.mult(x, x) for x in mk]
+    H.one_mat_rot_sum_inplace(sq[0], sq[1])
+    H.one_mat_rot_sum_inplace(sk[0], sk[1])
+    H.transpose_inplace(sk[0], 8)
+    s = H.single_cc_matmul(mq[0], kt, 8)
+    x = H.add(H.add(H.mult_const(s, -2.0), H.level_down(sq[0], 8)), sk[0])
+    assert x.info()["level"] == 8 == s.info()["level"]          # the integer constant took no level
+    zx, zn = H.decrypt2(x), H.decrypt2(sq[1])
+    for t in (0, 1):
+        h = 2 * (2 + t)
+        qh, kh = Q[:, h * d:(h + 1) * d], K[:, h * d:(h + 1) * d]
+        dist = (qh * qh).sum(1)[:, None] + (kh * kh).sum(1)[None, :] - 2.0 * qh @ kh.T
+        assert bench.GK_INTERVAL[0] < dist.min() and dist.max() < bench.GK_INTERVAL[1] + 0.25
+        assert np.abs(zx[t] - dist).max() < TOL
+        qr = Q[:, (h + 1) * d:(h + 2) * d]                       # the right half's norms, spread over the tile row
+        assert np.abs(zn[t] - (qr * qr).sum(1)[:, None]).max() < TOL
+    p = H.eval_chebyshev(H.linear_transform(x, *bench.GK_INTERVAL), bench.gk_table(), 4)
+    assert p.info()["level"] == 4                                # the interval map is a subtraction; level_cost = 2 + 2
+    # all four heads end to end
+    outs = bench.gk_attention(H, [(q, k, kt, v)])
+    assert all(o.info()["level"] == 1 for o in outs)
+    assert bench.gk_attention_error(H, outs, Q, K, V, [1]) < 2.0 ** -12
 
 
 def test_whole_layer_workloads(H):

@@ -36,6 +36,16 @@ def test_residues_match_oracle(small):
     want = P.exp_iter(ev, oct_, 4)
     assert np.array_equal(got.residues(), want.data)
     assert np.abs(H.decrypt(got) - (1 + M / 16) ** 16).max() < 2 ** -18
+    # HELLM::Exp::exp_iter_Parallel on three tensors: one pair and an unpaired last one
+    Ms = [rng.uniform(-1, 1, (16, 16)) for _ in range(3)]
+    cts = [H.encrypt(m) for m in Ms]
+    octs = [O.Ct(c.residues(), orc.delta[c.info()["level"]]) for c in cts]
+    H.exp_iter_parallel(cts, 4)
+    wants = P.exp_iter_parallel(ev, octs, 4)
+    for c, w in zip(cts, wants):
+        assert np.array_equal(c.residues(), w.data)
+    assert np.abs(H.decrypt(cts[1]) - (1 + Ms[1] / 16) ** 16).max() < 2 ** -18
+    assert np.abs(H.decrypt(cts[2]) - (1 + Ms[2] / 16)).max() < 2 ** -20
     poly = [0, 1.5, 0, -0.7, 0, 0.3, 0, -0.11, 0, 0.05, 0, -0.02, 0, 0.008, 0, -0.003]
     for k, l in ((2, 3), (4, 2)):
         got = H.eval_odd_polynomial(ct, poly, k, l)
@@ -65,6 +75,8 @@ def test_residues_match_oracle(small):
     low = H.level_down(ct, 2)
     with pytest.raises(load_package().HemmError):
         H.exp_iter(low, 4)                      # not enough levels: the reference would bootstrap here
+    with pytest.raises(load_package().HemmError):
+        H.exp_iter_parallel([H.level_down(ct, 2), H.level_down(ct, 2)], 4)
 
 
 def test_full_ring_values():

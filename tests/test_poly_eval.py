@@ -61,6 +61,13 @@ def test_slot_values():
     r = P.exp_iter(ev, ct, 6)
     assert r.level == 12 - 7
     assert np.abs(ev.decrypt(r).real - (1 + x / 64) ** 64).max() < 1e-12
+    # the list form squares pair by pair; a trailing tensor without a partner is only scaled and shifted
+    ys = [rng.uniform(-1, 1, 512) for _ in range(5)]
+    rs = P.exp_iter_parallel(ev, [ev.encrypt(y) for y in ys], 5)
+    for y, r in zip(ys[:4], rs[:4]):
+        assert r.level == 12 - 6
+        assert np.abs(ev.decrypt(r).real - (1 + y / 32) ** 32).max() < 1e-12
+    assert rs[4].level == 12 - 1 and np.abs(ev.decrypt(rs[4]).real - (1 + ys[4] / 32)).max() < 1e-12
     poly = [0, 1.5, 0, -0.7, 0, 0.3, 0, -0.11, 0, 0.05, 0, -0.02, 0, 0.008, 0, -0.003]
     for k, l in ((2, 3), (4, 2), (8, 1)):
         r = P.eval_odd_polynomial(ev, ct, poly, k, l)
