@@ -17,6 +17,12 @@ void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64
 static thread_local std::string g_err;
 void hemm_set_error(const std::string &m) { g_err = m; }
 
+// A null stream argument means the context's stream (the legacy default stream unless hemm_context_set_stream named
+// another one -- stream capture cannot use the legacy default stream).
+static inline hipStream_t on_stream(const hemm_context *ctx, void *stream) {
+    return stream != nullptr ? (hipStream_t)stream : ctx->stream;
+}
+
 #define HEMM_TRY try {
 #define HEMM_CATCH                                \
     }                                             \
@@ -118,7 +124,7 @@ int hemm_ntt(hemm_context *ctx, uint64_t *data, const uint32_t *prime_idx, uint3
         ll.idx[j] = (uint8_t)prime_idx[j];
     }
     launch_ntt(ctx, (u64 *)data, ll, (int)n_limbs, (int)n_polys, (size_t)n_limbs * ctx->N, inverse != 0,
-               (hipStream_t)stream);
+               on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -141,7 +147,7 @@ int hemm_sample_uniform(hemm_context *ctx, const uint64_t *stream_keys, const ui
     HEMM_TRY
     const LimbList ll = explicit_limbs(ctx, prime_idx, n_limbs);
     need(stream_keys && out, "null operand");
-    launch_sample_uniform(ctx, (const u64 *)stream_keys, ll, (int)n_limbs, (u64 *)out, (hipStream_t)stream);
+    launch_sample_uniform(ctx, (const u64 *)stream_keys, ll, (int)n_limbs, (u64 *)out, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -151,7 +157,7 @@ int hemm_sample_error(hemm_context *ctx, uint64_t stream_key, const uint32_t *pr
     HEMM_TRY
     const LimbList ll = explicit_limbs(ctx, prime_idx, n_limbs);
     need(out, "null operand");
-    launch_sample_error(ctx, (u64)stream_key, ll, (int)n_limbs, (u64 *)out, (hipStream_t)stream);
+    launch_sample_error(ctx, (u64)stream_key, ll, (int)n_limbs, (u64 *)out, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -172,7 +178,7 @@ int hemm_pointwise(hemm_context *ctx, int op, const uint64_t *a, size_t a_stride
     need(a && out && (b || op == HEMM_NEG), "null operand");
     need(op >= 0 && op <= 4, "unknown op");
     launch_binary(ctx, op, (const u64 *)a, a_stride, (const u64 *)b, b_stride, (u64 *)out, out_stride, ll, nl,
-                  (int)n_polys, (hipStream_t)stream);
+                  (int)n_polys, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -184,7 +190,7 @@ int hemm_mul_scalar(hemm_context *ctx, const uint64_t *a, size_t a_stride, const
     LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
     need(a && out && scalars, "null operand");
     launch_mul_scalar(ctx, (const u64 *)a, a_stride, (const u64 *)scalars, (u64 *)out, out_stride, ll, nl,
-                      (int)n_polys, (hipStream_t)stream);
+                      (int)n_polys, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -196,7 +202,7 @@ int hemm_encode(hemm_context *ctx, double *slots, double scale, uint32_t nq, int
     LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
     need(slots && out && n_msgs >= 1, "null operand");
     need(scale > 0, "scale must be positive");
-    launch_encode(ctx, slots, scale, ll, nl, (int)n_msgs, (u64 *)out, (hipStream_t)stream);
+    launch_encode(ctx, slots, scale, ll, nl, (int)n_msgs, (u64 *)out, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -207,7 +213,7 @@ int hemm_decode(hemm_context *ctx, const uint64_t *pt, uint32_t n_limbs, double 
     need(pt && workspace && slots, "null operand");
     need(n_limbs >= 1 && n_limbs <= 2 && (int)n_limbs <= ctx->nQ, "decode reads one or two limbs");
     need(scale > 0, "scale must be positive");
-    launch_decode(ctx, (const u64 *)pt, (int)n_limbs, scale, (u64 *)workspace, slots, (hipStream_t)stream);
+    launch_decode(ctx, (const u64 *)pt, (int)n_limbs, scale, (u64 *)workspace, slots, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -219,7 +225,16 @@ int hemm_add_scalar(hemm_context *ctx, const uint64_t *a, const uint64_t *re, co
     LimbList ll = chain_limbs(ctx, nq, with_p, &nl);
     need(a && out && re, "null operand");
     need(ctx->N >= 512, "needs N >= 512");
-    launch_add_scalar(ctx, (const u64 *)a, (const u64 *)re, (const u64 *)im, (u64 *)out, ll, nl, (hipStream_t)stream);
+    launch_add_scalar(ctx, (const u64 *)a, (const u64 *)re, (const u64 *)im, (u64 *)out, ll, nl, on_stream(ctx, stream));
+    check_launch();
+    HEMM_CATCH
+}
+
+int hemm_zero(hemm_context *ctx, uint64_t *out, size_t words, void *stream) {
+    HEMM_TRY
+    need(ctx && out, "null operand");
+    need((words & 1) == 0 && ((uintptr_t)out & 15) == 0, "an even number of words at a 16-byte boundary is needed");
+    if (words) launch_zero(ctx, (u64 *)out, words, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -230,7 +245,7 @@ int hemm_mul_imag_unit(hemm_context *ctx, const uint64_t *a, size_t a_stride, ui
     int nl;
     LimbList ll = chain_limbs(ctx, nq, 0, &nl);
     need(a && out, "null operand");
-    launch_mul_imag(ctx, (const u64 *)a, a_stride, (u64 *)out, out_stride, ll, nl, (int)n_polys, (hipStream_t)stream);
+    launch_mul_imag(ctx, (const u64 *)a, a_stride, (u64 *)out, out_stride, ll, nl, (int)n_polys, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -242,7 +257,7 @@ int hemm_tensor(hemm_context *ctx, const uint64_t *ct1, size_t stride1, const ui
     chain_limbs(ctx, nq, 0, &nl);
     need(ct1 && ct2 && out, "null operand");
     launch_tensor(ctx, (const u64 *)ct1, stride1, (const u64 *)ct2, stride2, (u64 *)out, out_stride, (int)nq,
-                  accumulate != 0, (hipStream_t)stream);
+                  accumulate != 0, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -255,7 +270,7 @@ int hemm_automorphism(hemm_context *ctx, const uint64_t *a, size_t a_stride, uin
     need(a != out, "automorphism cannot run in place");
     need((galois & 1) && galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
     launch_galois(ctx, (const u64 *)a, a_stride, (u64 *)out, out_stride, galois, (int)n_limbs, (int)n_polys,
-                  (hipStream_t)stream);
+                  on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -266,7 +281,7 @@ int hemm_modup(hemm_context *ctx, const uint64_t *in, uint32_t nq, uint64_t *ext
     chain_limbs(ctx, nq, 1, &nl);
     need(in && ext, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    launch_modup(ctx, (const u64 *)in, (int)nq, (u64 *)ext, hemm_scratch(ctx), true, (hipStream_t)stream);
+    launch_modup(ctx, (const u64 *)in, (int)nq, (u64 *)ext, hemm_scratch(ctx), true, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -277,7 +292,7 @@ int hemm_inner_product(hemm_context *ctx, const uint64_t *ext, const uint64_t *e
     int nl;
     chain_limbs(ctx, nq, 1, &nl);
     need(ext && evk && acc, "null operand");
-    launch_inner_product(ctx, nullptr, (const u64 *)ext, (const u64 *)evk, (int)nq, (u64 *)acc, (hipStream_t)stream);
+    launch_inner_product(ctx, nullptr, (const u64 *)ext, (const u64 *)evk, (int)nq, (u64 *)acc, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -291,7 +306,7 @@ int hemm_moddown(hemm_context *ctx, uint64_t *acc, uint32_t nq, uint32_t n_polys
     need(ctx->nP >= 1, "key switching needs special primes");
     need(n_polys >= 1 && n_polys <= 2, "n_polys must be 1 or 2");
     launch_moddown(ctx, (u64 *)acc, (int)nq, (int)n_polys, (u64 *)out, out_stride, nullptr, 0, 0, hemm_scratch(ctx),
-                   (hipStream_t)stream);
+                   on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -303,7 +318,7 @@ int hemm_keyswitch(hemm_context *ctx, const uint64_t *in, const uint64_t *evk, u
     chain_limbs(ctx, nq, 1, &nl);
     need(in && evk && out, "null operand");
     launch_keyswitch(ctx, (const u64 *)in, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, (const u64 *)add_b,
-                     (hipStream_t)stream);
+                     on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -317,9 +332,9 @@ int hemm_rotate(hemm_context *ctx, const uint64_t *ct, size_t ct_stride, const u
     need((galois & 1) && galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
     const size_t N = ctx->N;
     u64 *rot = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
-    launch_galois(ctx, (const u64 *)ct, ct_stride, rot, (size_t)nq * N, galois, (int)nq, 2, (hipStream_t)stream);
+    launch_galois(ctx, (const u64 *)ct, ct_stride, rot, (size_t)nq * N, galois, (int)nq, 2, on_stream(ctx, stream));
     launch_keyswitch(ctx, rot + (size_t)nq * N, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, rot,
-                     (hipStream_t)stream);
+                     on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -333,9 +348,9 @@ int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, c
     const size_t N = ctx->N;
     u64 *tmp = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
     launch_keyswitch(ctx, (const u64 *)ct3 + 2 * ct_stride, (const u64 *)evk, (int)nq, tmp, (size_t)nq * N, nullptr,
-                     (hipStream_t)stream);
+                     on_stream(ctx, stream));
     launch_binary(ctx, HEMM_ADD, (const u64 *)ct3, ct_stride, tmp, (size_t)nq * N, (u64 *)out, out_stride, ll, nl, 2,
-                  (hipStream_t)stream);
+                  on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -347,6 +362,10 @@ static void *upload_desc(hemm_context *ctx, const void *a, size_t na, const void
     if (!ctx->d_desc) HEMM_HIP(hipMalloc(&ctx->d_desc, cap));
     const size_t off_b = (na + 255) & ~(size_t)255;
     if (off_b + nb > cap) throw std::invalid_argument("too many terms in one batched call");
+    // the list is copied from pageable host memory that is gone when the call returns: nothing a graph could replay
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (s != nullptr && hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+        throw std::invalid_argument("a term list too long for the kernel arguments cannot be recorded into a graph");
     // both lists in one copy (pageable source: the runtime has read it when the call returns)
     std::vector<char> both(off_b + nb);
     memcpy(both.data(), a, na);
@@ -364,7 +383,7 @@ int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, ui
     need(in && ext && workspace && n_in >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
     launch_modup_batch(ctx, (const u64 *)in, in_stride, (int)nq, (int)n_in, (u64 *)ext, (u64 *)workspace,
-                       (hipStream_t)stream);
+                       on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -438,7 +457,7 @@ size_t hemm_key_compact_words(const hemm_context *ctx) { return ctx ? key_compac
 int hemm_key_compact(hemm_context *ctx, const uint64_t *evk, uint64_t *out, void *stream) {
     HEMM_TRY
     need(ctx && evk && out, "null operand");
-    launch_key_compact(ctx, (const u64 *)evk, (u64 *)out, (hipStream_t)stream);
+    launch_key_compact(ctx, (const u64 *)evk, (u64 *)out, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -450,7 +469,7 @@ int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint
     chain_limbs(ctx, nq, 1, &nl);
     need(terms && group_offsets && y && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y, b_premultiplied != 0, (hipStream_t)stream);
+    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y, b_premultiplied != 0, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -463,9 +482,9 @@ int hemm_hoisted_moddown(hemm_context *ctx, const hemm_rot_term *terms, const ui
     chain_limbs(ctx, nq, 1, &nl);
     need(terms && group_offsets && y_workspace && out && workspace && n_out >= 1, "null operand");
     need(ctx->nP >= 1, "key switching needs special primes");
-    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y_workspace, b_premultiplied != 0, (hipStream_t)stream);
+    run_hoisted_terms(ctx, terms, group_offsets, n_out, nq, (u64 *)y_workspace, b_premultiplied != 0, on_stream(ctx, stream));
     launch_moddown_batch(ctx, (u64 *)y_workspace, (int)nq, (int)(2 * n_out), drop_last != 0, (u64 *)out, out_stride,
-                         (u64 *)workspace, (hipStream_t)stream);
+                         (u64 *)workspace, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -479,7 +498,7 @@ int hemm_moddown_batch(hemm_context *ctx, uint64_t *y, uint32_t nq, uint32_t n_p
     need(ctx->nP >= 1, "key switching needs special primes");
     need((drop_last & ~(1 | HEMM_MODDOWN_COLUMN_SLAB)) == 0, "unknown ModDown flag");
     launch_moddown_batch(ctx, (u64 *)y, (int)nq, (int)n_polys, (drop_last & 1) != 0, (u64 *)out, out_stride,
-                         (u64 *)workspace, (hipStream_t)stream, (drop_last & HEMM_MODDOWN_COLUMN_SLAB) != 0);
+                         (u64 *)workspace, on_stream(ctx, stream), (drop_last & HEMM_MODDOWN_COLUMN_SLAB) != 0);
     check_launch();
     HEMM_CATCH
 }
@@ -499,18 +518,26 @@ int hemm_masked_sum_batch(hemm_context *ctx, const hemm_lin_term *terms, const u
     static_assert(sizeof(hemm_lin_term) == 32, "the kernels read these records as they are");
     if ((int)n_terms <= masked_arg_capacity() && (int)n_out <= masked_arg_capacity()) {
         launch_masked_sum_args(ctx, terms, (int)n_terms, group_offsets, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
-                               (hipStream_t)stream);
+                               on_stream(ctx, stream));
         check_launch();
         return 0;
     }
     void *off_dev = nullptr;
     void *terms_dev = upload_desc(ctx, terms, n_terms * sizeof(hemm_lin_term), group_offsets,
-                                  (n_out + 1) * sizeof(uint32_t), &off_dev, (hipStream_t)stream);
+                                  (n_out + 1) * sizeof(uint32_t), &off_dev, on_stream(ctx, stream));
     launch_masked_sum(ctx, terms_dev, (const u32 *)off_dev, (int)n_out, (int)nq, (int)n_polys, (u64 *)out,
-                      (hipStream_t)stream, terms, (int)n_terms);
+                      on_stream(ctx, stream), terms, (int)n_terms);
     check_launch();
     HEMM_CATCH
 }
+
+int hemm_context_set_stream(hemm_context *ctx, void *stream) {
+    HEMM_TRY
+    need(ctx != nullptr, "null context");
+    ctx->stream = (hipStream_t)stream;
+    HEMM_CATCH
+}
+void *hemm_context_stream(const hemm_context *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
 int hemm_traffic(hemm_context *ctx, uint64_t *bytes, uint64_t *launches, int reset) {
     HEMM_TRY
@@ -538,7 +565,7 @@ int hemm_sum_parts(hemm_context *ctx, const uint64_t *parts, uint32_t n_parts, u
     chain_limbs(ctx, nq, 1, &nl);
     need(parts && y && n_parts >= 1 && n_out >= 1, "null operand");
     need(ctx->N >= 2, "ring too small");
-    launch_sum_parts(ctx, (const u64 *)parts, (int)n_parts, (int)n_out, (int)nq, (u64 *)y, (hipStream_t)stream);
+    launch_sum_parts(ctx, (const u64 *)parts, (int)n_parts, (int)n_out, (int)nq, (u64 *)y, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -549,7 +576,7 @@ int hemm_compact_mask(hemm_context *ctx, const uint64_t *mask, uint32_t n_limbs,
     need(mask && table && is_constant, "null operand");
     need((int)n_limbs > ctx->nP && shift >= 1 && (int)shift < ctx->logN,
          "the mask must cover the extended basis and shift must be in [1, log N)");
-    *is_constant = launch_compact_mask(ctx, (const u64 *)mask, (int)n_limbs, (int)shift, (u64 *)table, (hipStream_t)stream) ? 1 : 0;
+    *is_constant = launch_compact_mask(ctx, (const u64 *)mask, (int)n_limbs, (int)shift, (u64 *)table, on_stream(ctx, stream)) ? 1 : 0;
     check_launch();
     HEMM_CATCH
 }
@@ -566,7 +593,7 @@ int hemm_tensor_batch_strided(hemm_context *ctx, const uint64_t *t1, const uint6
     need(t1 && t2 && acc3 && n_pairs >= 1, "null operand");
     need(acc_stride >= (size_t)nq * (size_t)ctx->N, "accumulator stride below one polynomial");
     launch_tensor_batch(ctx, (const u64 *)t1, (const u64 *)t2, (int)n_pairs, (int)nq, (u64 *)acc3, acc_stride,
-                        accumulate != 0, (hipStream_t)stream);
+                        accumulate != 0, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -593,7 +620,7 @@ int hemm_tensor_batch_groups(hemm_context *ctx, const hemm_tensor_group *groups,
         g[i] = TensorGroupHost{(const u64 *)groups[i].t1, (const u64 *)groups[i].t2, (u64 *)groups[i].acc3,
                                (int)groups[i].n_pairs, groups[i].accumulate != 0};
     }
-    launch_tensor_groups(ctx, g.data(), (int)n_groups, (int)nq, acc_stride, (hipStream_t)stream);
+    launch_tensor_groups(ctx, g.data(), (int)n_groups, (int)nq, acc_stride, on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -608,7 +635,7 @@ int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64
     need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_scratch_words(ctx),
          "n_polys * nq limbs must fit the context's scratch ((dnum + 7) * (nQ + nP) limbs)");
     launch_rescale(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
-                   (hipStream_t)stream);
+                   on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }
@@ -622,7 +649,7 @@ int hemm_rescale_static(hemm_context *ctx, const uint64_t *in, size_t in_stride,
     need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_static_scratch_words(),
          "n_polys * nq * N must not exceed HEMM_STATIC_SCRATCH_WORDS");
     launch_rescale_static(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
-                          (hipStream_t)stream);
+                          on_stream(ctx, stream));
     check_launch();
     HEMM_CATCH
 }

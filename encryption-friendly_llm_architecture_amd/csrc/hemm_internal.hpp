@@ -36,6 +36,7 @@ struct hemm_context {
     u64 *d_scratch;
     size_t scratch_bytes;
     void *d_desc;                   // staging for the term lists of batched calls
+    hipStream_t stream = nullptr;   // what a null stream argument of an entry point means for this context
     // compact evaluation keys: offset of every prime's limb inside a (digit, polynomial) slice and, last entry, the
     // slice size, in units of 2N bytes (a prime below 2^44 takes 6 bytes per residue = 3 units, any other 4)
     std::vector<u32> key_off;
@@ -134,6 +135,7 @@ void launch_encode(const hemm_context *c, double *slots, double scale, const Lim
                    hipStream_t s);
 void launch_decode(const hemm_context *c, const u64 *pt, int n_limbs, double scale, u64 *work, double *slots, hipStream_t s);
 void hemm_embedding_tables_free(const hemm_context *c);
+void launch_zero(const hemm_context *c, u64 *out, size_t words, hipStream_t s);
 void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride,
                      const LimbList &ll, int n_limbs, int n_polys, hipStream_t s);
 void launch_tensor(const hemm_context *c, const u64 *c1, size_t s1, const u64 *c2, size_t s2, u64 *out,

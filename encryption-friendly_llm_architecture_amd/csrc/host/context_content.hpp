@@ -5,6 +5,7 @@
 
 #include <map>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "../../../include/hemm.h"
@@ -29,6 +30,10 @@ struct ContextContent {
     hipStream_t side = nullptr;
     hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     bool side_open = false;
+    // the stream the host layer queues on: the device context's (hemm_context_set_stream), by default the legacy
+    // default stream; on(s) resolves a stream argument whose null value means that stream
+    hipStream_t stream() const { return (hipStream_t)hemm_context_stream(dev); }
+    hipStream_t on(hipStream_t s) const { return s != nullptr ? s : stream(); }
 
     // Opens a side chain: work given to the returned stream starts after everything queued on the default stream
     // so far and runs beside what the default stream is given next.  The stream does not synchronise implicitly
@@ -43,7 +48,7 @@ struct ContextContent {
             ok(hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming), "hipEventCreateWithFlags");
             ok(hipEventCreateWithFlags(&ev_join, hipEventDisableTiming), "hipEventCreateWithFlags");
         }
-        ok(hipEventRecord(ev_fork, nullptr), "hipEventRecord");
+        ok(hipEventRecord(ev_fork, stream()), "hipEventRecord");
         ok(hipStreamWaitEvent(side, ev_fork, 0), "hipStreamWaitEvent");
         std::lock_guard<std::mutex> lk(mu);
         side_open = true;
@@ -52,11 +57,27 @@ struct ContextContent {
     void joinSide() {
         if (!side_open) return;
         (void)hipEventRecord(ev_join, side);
-        (void)hipStreamWaitEvent(nullptr, ev_join, 0);
+        (void)hipStreamWaitEvent(stream(), ev_join, 0);
         std::lock_guard<std::mutex> lk(mu);
         side_open = false;
         for (auto &kv : parked) pool.emplace(kv.first, kv.second);
         parked.clear();
+    }
+
+    // Optional phase trace of the batched products: while it is on, mark() records an event on the default stream at
+    // a named point of the schedule; the report gives the time between consecutive marks.
+    bool trace_on = false;
+    std::vector<std::pair<std::string, hipEvent_t>> trace_marks;
+    void mark(const char *name) {
+        if (!trace_on) return;
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return;
+        (void)hipEventRecord(e, stream());
+        trace_marks.emplace_back(name, e);
+    }
+    void traceClear() {
+        for (auto &m : trace_marks) (void)hipEventDestroy(m.second);
+        trace_marks.clear();
     }
 
     u64 prime(size_t i) const { return i < nQ ? q[i] : p[i - nQ]; }
@@ -76,17 +97,26 @@ struct ContextContent {
         pool_bytes += words * 8;
         return d;
     }
+    // Stream capture of a sequence of calls (hellm_graph_begin / _end): a buffer released while the capture is open
+    // stays with the graph being recorded -- its replays write that memory -- and returns to the pool when the graph
+    // is destroyed.
+    bool capture_open = false;
+    std::vector<std::pair<size_t, u64 *>> captured;
     void release(u64 *ptr, size_t words) {
         std::lock_guard<std::mutex> lk(mu);
-        if (side_open)
+        if (capture_open)
+            captured.emplace_back(words, ptr);
+        else if (side_open)
             parked.emplace_back(words, ptr);
         else
             pool.emplace(words, ptr);
     }
     ~ContextContent() {
         (void)hipDeviceSynchronize();
+        traceClear();
         for (auto &kv : pool) (void)hipFree(kv.second);
         for (auto &kv : parked) (void)hipFree(kv.second);
+        for (auto &kv : captured) (void)hipFree(kv.second);
         if (side) (void)hipStreamDestroy(side);
         if (ev_fork) (void)hipEventDestroy(ev_fork);
         if (ev_join) (void)hipEventDestroy(ev_join);

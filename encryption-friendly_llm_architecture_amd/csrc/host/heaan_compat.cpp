@@ -205,7 +205,7 @@ DeviceBuffer &DeviceBuffer::operator=(const DeviceBuffer &o) {
         return *this;
     }
     resize(o.ctx_, o.words_);
-    hip_ck(hipMemcpyAsync(ptr_, o.ptr_, words_ * 8, hipMemcpyDeviceToDevice, nullptr), "hipMemcpyAsync");
+    hip_ck(hipMemcpyAsync(ptr_, o.ptr_, words_ * 8, hipMemcpyDeviceToDevice, ctx_->stream()), "hipMemcpyAsync");
     return *this;
 }
 DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
@@ -287,7 +287,7 @@ void Plaintext::setLevel(u64 level) {
     compact_ = DeviceBuffer();
     if (hash_state_ == 1) hash_state_ = 0;
     DeviceBuffer nb(ctx_, (level + 1) * ctx_->N);
-    hip_ck(hipMemcpyAsync(nb.data(), buf_.data(), (level + 1) * ctx_->N * 8, hipMemcpyDeviceToDevice, nullptr),
+    hip_ck(hipMemcpyAsync(nb.data(), buf_.data(), (level + 1) * ctx_->N * 8, hipMemcpyDeviceToDevice, ctx_->stream()),
            "hipMemcpyAsync");
     buf_ = std::move(nb);
     level_ = level;
@@ -432,7 +432,7 @@ const u64 *KeyPack::compactKey(int kind, u64 g) const {
         ck(hemm_key_compact(ctx_->dev, plain, c.data(), nullptr));
         // made once per key, on the default stream: finished before the caller queues its sum on whichever stream (the
         // side stream does not wait for later work of the default one)
-        hip_ck(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+        hip_ck(hipStreamSynchronize(ctx_->stream()), "hipStreamSynchronize");
         it = compact_.emplace(id, std::move(c)).first;
     }
     return it->second.data();
@@ -695,7 +695,7 @@ Message EnDecoder::decode(const Plaintext &pt) const {
         return m;
     }
     DeviceBuffer tmp(c, (two + 1) * N);
-    hip_ck(hipMemcpyAsync(tmp.data(), pt.buf_.data(), (two + 1) * N * 8, hipMemcpyDeviceToDevice, nullptr), "memcpy");
+    hip_ck(hipMemcpyAsync(tmp.data(), pt.buf_.data(), (two + 1) * N * 8, hipMemcpyDeviceToDevice, c->stream()), "memcpy");
     ck(hemm_ntt(c->dev, tmp.data(), chain_primes(two + 1).data(), (uint32_t)(two + 1), 1, 1, nullptr));
     std::vector<u64> h((two + 1) * N);
     hip_ck(hipMemcpy(h.data(), tmp.data(), h.size() * 8, hipMemcpyDeviceToHost), "hipMemcpy");

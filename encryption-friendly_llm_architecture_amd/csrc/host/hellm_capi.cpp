@@ -1,6 +1,7 @@
 // extern "C" facade over HELLM::HEMMer (declared in include/hellm.h).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
 
 #include "../../../include/hellm.h"
@@ -127,6 +128,135 @@ int hellm_sync(void) {
     FACADE_TRY
     CudaTools::cudaDeviceSynchronize();
     FACADE_CATCH
+}
+
+int hellm_phase_trace(hellm_hemmer *h, int on) {
+    FACADE_TRY
+    need(h, "null argument");
+    auto &c = *h->m->getContext();
+    c.traceClear();
+    c.trace_on = on != 0;
+    FACADE_CATCH
+}
+int hellm_phase_report(hellm_hemmer *h, char *text, size_t capacity) {
+    FACADE_TRY
+    need(h && text && capacity > 0, "null argument");
+    auto &c = *h->m->getContext();
+    if (hipDeviceSynchronize() != hipSuccess) throw RuntimeException("hipDeviceSynchronize failed");
+    std::string out;
+    for (size_t i = 1; i < c.trace_marks.size(); i++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, c.trace_marks[i - 1].second, c.trace_marks[i].second) != hipSuccess)
+            throw RuntimeException("hipEventElapsedTime failed");
+        out += c.trace_marks[i].first + "\t" + std::to_string(ms) + "\n";
+    }
+    need(out.size() + 1 <= capacity, "report does not fit the buffer");
+    memcpy(text, out.c_str(), out.size() + 1);
+    c.traceClear();
+    FACADE_CATCH
+}
+// ---- a sequence of calls recorded once and replayed (HIP graph) ----------------------------------------------------
+struct hellm_graph {
+    HEaaN::Context ctx;
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<size_t, HEaaN::u64 *>> owned;   // intermediates of the recorded calls
+    size_t nodes = 0;
+};
+namespace {
+void hipck(hipError_t e, const char *what) {
+    if (e != hipSuccess) throw RuntimeException(std::string(what) + ": " + hipGetErrorString(e));
+}
+thread_local hellm_graph *g_recording = nullptr;
+}  // namespace
+int hellm_graph_begin(hellm_hemmer *h) {
+    FACADE_TRY
+    need(h, "null argument");
+    if (g_recording) throw RuntimeException("a recording is already open on this thread");
+    HEaaN::Context c = h->m->getContext();
+    if (c->side_open || c->capture_open || c->stream() != nullptr)
+        throw RuntimeException("the context is busy with another stream");
+    auto *g = new hellm_graph();
+    g->ctx = c;
+    try {
+        hipck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        hipck(hipStreamCreateWithFlags(&g->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+        if (hemm_context_set_stream(c->dev, g->stream) != 0) throw RuntimeException(hemm_last_error());
+        hipck(hipStreamBeginCapture(g->stream, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture");
+    } catch (...) {
+        (void)hemm_context_set_stream(c->dev, nullptr);
+        if (g->stream) (void)hipStreamDestroy(g->stream);
+        delete g;
+        throw;
+    }
+    c->capture_open = true;
+    g_recording = g;
+    FACADE_CATCH
+}
+int hellm_graph_end(hellm_hemmer *h, hellm_graph **out) {
+    FACADE_TRY
+    need(h && out, "null argument");
+    hellm_graph *g = g_recording;
+    if (!g || g->ctx != h->m->getContext()) throw RuntimeException("no recording is open on this context");
+    g_recording = nullptr;
+    HEaaN::Context c = g->ctx;
+    const hipError_t e = hipStreamEndCapture(g->stream, &g->graph);
+    (void)hemm_context_set_stream(c->dev, nullptr);
+    {
+        std::lock_guard<std::mutex> lk(c->mu);
+        c->capture_open = false;
+        g->owned.swap(c->captured);
+    }
+    auto drop = [&]() {
+        std::lock_guard<std::mutex> lk(c->mu);
+        for (auto &kv : g->owned) c->pool.emplace(kv.first, kv.second);
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        (void)hipStreamDestroy(g->stream);
+        delete g;
+    };
+    if (e != hipSuccess) {
+        drop();
+        throw RuntimeException(std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+    }
+    if (hipGraphGetNodes(g->graph, nullptr, &g->nodes) != hipSuccess) g->nodes = 0;
+    const hipError_t ei = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (ei != hipSuccess) {
+        drop();
+        throw RuntimeException(std::string("hipGraphInstantiate: ") + hipGetErrorString(ei));
+    }
+    *out = g;
+    FACADE_CATCH
+}
+int hellm_graph_launch(hellm_graph *g) {
+    FACADE_TRY
+    need(g && g->exec, "null argument");
+    hipck(hipGraphLaunch(g->exec, g->stream), "hipGraphLaunch");
+    FACADE_CATCH
+}
+int hellm_graph_sync(hellm_graph *g) {
+    FACADE_TRY
+    need(g, "null argument");
+    hipck(hipStreamSynchronize(g->stream), "hipStreamSynchronize");
+    FACADE_CATCH
+}
+int hellm_graph_nodes(const hellm_graph *g, uint64_t *out) {
+    FACADE_TRY
+    need(g && out, "null argument");
+    *out = g->nodes;
+    FACADE_CATCH
+}
+void hellm_graph_destroy(hellm_graph *g) {
+    if (!g) return;
+    (void)hipStreamSynchronize(g->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    (void)hipStreamDestroy(g->stream);
+    {
+        std::lock_guard<std::mutex> lk(g->ctx->mu);
+        for (auto &kv : g->owned) g->ctx->pool.emplace(kv.first, kv.second);
+    }
+    delete g;
 }
 
 int hellm_traffic(hellm_hemmer *h, uint64_t *bytes, uint64_t *launches, int reset) {
@@ -314,6 +444,21 @@ int hellm_ct_clone(const hellm_ct *ct, hellm_ct **out) {
     FACADE_TRY
     need(ct && out, "null argument");
     *out = new hellm_ct{ct->t};
+    FACADE_CATCH
+}
+int hellm_ct_assign(hellm_hemmer *h, hellm_ct *dst, const hellm_ct *src) {
+    FACADE_TRY
+    need(h && dst && src, "null argument");
+    HEaaN::Ciphertext &d = dst->t.get();
+    const HEaaN::Ciphertext &s = src->t.get();
+    if (d.getNumPoly() != s.getNumPoly() || d.getLevel() != s.getLevel() || d.getRescaleCounter() != s.getRescaleCounter() ||
+        d.buf_.words() != s.buf_.words())
+        throw std::invalid_argument("[assign] the two ciphertexts differ in polynomials, level or pending rescales");
+    if (d.buf_.data() != s.buf_.data() &&
+        hipMemcpyAsync(d.buf_.data(), s.buf_.data(), s.buf_.words() * 8, hipMemcpyDeviceToDevice, h->m->getContext()->stream()) !=
+            hipSuccess)
+        throw RuntimeException("hipMemcpyAsync failed");
+    d.occupied_ = std::max(d.occupied_, s.occupied_);   // never claims more empty slots than either had
     FACADE_CATCH
 }
 void hellm_ct_destroy(hellm_ct *ct) { delete ct; }

@@ -112,7 +112,7 @@ static void add_sub(const HomEvaluator &ev, const Context &c, int op, const Ciph
         if (neg)
             ck(hemm_pointwise(c->dev, HEMM_NEG, src, 0, nullptr, 0, dst, 0, (uint32_t)a->level_ + 1, 0, 1, nullptr));
         else if (src != dst)
-            (void)hipMemcpyAsync(dst, src, r.polyStride() * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(dst, src, r.polyStride() * 8, hipMemcpyDeviceToDevice, c->stream());
     }
     o.commit(occ);
 }
@@ -128,7 +128,7 @@ void HomEvaluator::add(const Ciphertext &a, const Plaintext &b, Ciphertext &out)
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     Ciphertext &r = o.get();
     if (r.buf_.data() != a.buf_.data())
-        (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, ctx_->stream());
     ck(hemm_pointwise(ctx_->dev, HEMM_ADD, r.buf_.data(), 0, b.buf_.data(), 0, r.buf_.data(), 0,
                       (uint32_t)a.level_ + 1, 0, 1, nullptr));
     o.commit(occ);
@@ -150,7 +150,7 @@ void HomEvaluator::add(const Ciphertext &a, const Complex &cst, Ciphertext &out)
     OutSlot o(ctx_, out, a.num_poly_, a.level_, a.rescale_counter_, true, {&a});
     Ciphertext &r = o.get();
     if (r.buf_.data() != a.buf_.data())
-        (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(r.buf_.data(), a.buf_.data(), a.buf_.words() * 8, hipMemcpyDeviceToDevice, ctx_->stream());
     const auto rr = int_residues(ctx_, re, a.level_ + 1), ri = int_residues(ctx_, im, a.level_ + 1);
     ck(hemm_add_scalar(ctx_->dev, r.buf_.data(), rr.data(), im != 0 ? ri.data() : nullptr, r.buf_.data(),
                        (uint32_t)a.level_ + 1, 0, nullptr));

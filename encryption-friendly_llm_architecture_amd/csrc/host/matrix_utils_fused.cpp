@@ -338,7 +338,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
         ck(hemm_pointwise(c->dev, HEMM_ADD, res.data(), nq * N, sums.data(), nq * N, res.data(), nq * N, (uint32_t)nq, 0,
                           (uint32_t)(2 * n_jobs), nullptr));
     } else if (ng == 0) {
-        (void)hipMemcpyAsync(res.data(), sums.data(), n_jobs * ctw * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(res.data(), sums.data(), n_jobs * ctw * 8, hipMemcpyDeviceToDevice, c->stream());
     } else {
         throw RuntimeException("diagonalTransformBatch: jobs with and without giant steps cannot share a batch");
     }
@@ -404,7 +404,7 @@ DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u
     std::vector<size_t> which;
     for (size_t q = 0; q < n; q++) {
         if (rot.norm(rots[q]) == 0) {  // a whole turn (rows of a tile that fills the slots): plain copy
-            (void)hipMemcpyAsync(out.data() + q * ctw, cts + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, stream);
+            (void)hipMemcpyAsync(out.data() + q * ctw, cts + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, c->on(stream));
             continue;
         }
         terms.push_back(term(src.extOf(q), src.pbOf(q), pack, rot.galois(rots[q]), nullptr));
@@ -422,7 +422,7 @@ DeviceBuffer rotateSources(const HomEvaluator &eval, const Sources &src, const u
     DeviceBuffer tmp(c, m * ctw);
     ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)m, (uint32_t)nq, 1, 0, y.data(), tmp.data(), nq * N, ws.data(), stream));
     for (size_t k = 0; k < m; k++)
-        (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, stream);
+        (void)hipMemcpyAsync(out.data() + which[k] * ctw, tmp.data() + k * ctw, ctw * 8, hipMemcpyDeviceToDevice, c->on(stream));
     return out;
 }
 
@@ -629,8 +629,9 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                               (uint32_t)(nq - 1), 0, (uint32_t)(2 * n_jobs), nullptr));
         } else {
             c->joinSide();
-            (void)hipMemcpyAsync(dst, zres.data(), n_jobs * 2 * (nq - 1) * N * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(dst, zres.data(), n_jobs * 2 * (nq - 1) * N * 8, hipMemcpyDeviceToDevice, c->stream());
         }
+        c->mark(stage == 1 ? "transform stage 1" : "transform stage 2");
     }
 }
 
@@ -759,19 +760,20 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     if (copies > 1)
         ck(hemm_pointwise(c->dev, HEMM_ADD, bb.data(), lo * N, tau_b, lo * N, bb.data(), lo * N, (uint32_t)lo, 0, 2, nullptr));
     else
-        (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, c->stream());
     // column shifts of sigma(A), shift i rotated back by g (i / g) row units
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
         sa.push_back(Shift{cu * i - g * (i / g) * ru, &cm[(size_t)(2 * cu * i + 1)], &cm[(size_t)(2 * cu * i)]});
     c->joinSide();
+    c->mark("rotation sources and baby rotations");
     // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
     // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
     const u64 pw = lo * N, us = (u64)n_giant * pw;
     if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
         U_out->resize(c, 3 * us);
         for (u64 p = 0; p < 3; p++)
-            (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, c->stream());
     }
     std::vector<bool> started((size_t)n_giant, false);
     started[0] = true;
@@ -959,8 +961,8 @@ void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphert
         Ciphertext la_ct(c), lb_ct(c);
         eval.levelDown(a, Lt, la_ct);
         eval.levelDown(b, Lt, lb_ct);
-        (void)hipMemcpyAsync(joint, la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
-        (void)hipMemcpyAsync(joint + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, nullptr);
+        (void)hipMemcpyAsync(joint, la_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, c->stream());
+        (void)hipMemcpyAsync(joint + ctw_in, lb_ct.buf_.data(), ctw_in * 8, hipMemcpyDeviceToDevice, c->stream());
     }
 }
 
@@ -1081,9 +1083,12 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
     // home, so the product comes out in the first block with the other blocks empty.
     if (bsgs) {
         i64 g = 1;
+        c->mark("unshifted term");
         bsgsShiftProduct(eval, T, ab.data(), low.data() + 2 * lo * N, acc, cm, n, n / cu, cu, w, batch, &U, &g,
                          spread ? (u64)(n * w) : 0, true);
+        c->mark("main loop");
         bsgsGiantSteps(eval, T, U, g, (n / cu) / g, cu * w, acc, res, add_conj);
+        c->mark("giant steps");
         if (spread) res.get().occupied_ = (u64)(n * w);   // the product sits in the first block, the rest is empty
         return res;
     }
@@ -1220,7 +1225,7 @@ void multMatMatPreFused(const HomEvaluator &eval, const CtxtTensor &a_in, std::v
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);
             (void)hipMemcpyAsync(ct.buf_.data(), t.data() + q * 2 * lo * N, 2 * lo * N * 8, hipMemcpyDeviceToDevice,
-                                 nullptr);
+                                 c->stream());
             tmp.push_back(std::move(ct));
         }
     }
@@ -1264,7 +1269,7 @@ void multPackedMatMatPreRotFused(const HomEvaluator &eval, const CtxtTensor &a_i
         for (size_t q = 0; q < cnt; q++) {
             Ciphertext ct(c);
             ct.allocate(2, T + 1, 0);
-            (void)hipMemcpyAsync(ct.buf_.data(), t.data() + q * 2 * lo * N, 2 * lo * N * 8, hipMemcpyDeviceToDevice, nullptr);
+            (void)hipMemcpyAsync(ct.buf_.data(), t.data() + q * 2 * lo * N, 2 * lo * N * 8, hipMemcpyDeviceToDevice, c->stream());
             tmp.push_back(std::move(ct));
         }
     }
@@ -1285,8 +1290,8 @@ void complexPackingPair(const HomEvaluator &eval, MatrixTransformer &tr, const C
     Ciphertext ra(c), rb(c);
     ra.allocate(2, L - 1, 0);
     rb.allocate(2, L - 1, 0);
-    (void)hipMemcpyAsync(ra.buf_.data(), packed.data(), half * 8, hipMemcpyDeviceToDevice, nullptr);
-    (void)hipMemcpyAsync(rb.buf_.data(), packed.data() + half, half * 8, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipMemcpyAsync(ra.buf_.data(), packed.data(), half * 8, hipMemcpyDeviceToDevice, c->stream());
+    (void)hipMemcpyAsync(rb.buf_.data(), packed.data() + half, half * 8, hipMemcpyDeviceToDevice, c->stream());
     pa = std::move(ra);
     pb = std::move(rb);
 }
@@ -1295,6 +1300,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                                         const CtxtTensor &b, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile,
                                         bool add_conj) {
     const Context &c = eval.getContext();
+    c->mark("start");
     if (a.get().getRescaleCounter() != 0 || b.get().getRescaleCounter() != 0 || a.get().getNumPoly() != 2 ||
         b.get().getNumPoly() != 2)
         throw std::invalid_argument("[complexPacking] operands must be rescaled.");
@@ -1317,6 +1323,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     const bool by_rows[2] = {false, true};
     const u64 from[2] = {a.getLevel(), b.getLevel()};
     tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data(), from);
+    c->mark("complex packing");
     return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1, false, add_conj);
 }
 
@@ -1507,7 +1514,7 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
         ck(hemm_hoisted_terms(c->dev, terms.data(), off.data(), (uint32_t)parts, (uint32_t)nq, yp.data(), 1, nullptr));
         ck(hemm_sum_parts(c->dev, yp.data(), (uint32_t)parts, 1, (uint32_t)nq, y.data(), nullptr));
     } else {
-        (void)hipMemsetAsync(y.data(), 0, 2 * E * N * 8, nullptr);
+        ck(hemm_zero(c->dev, y.data(), 2 * E * N, nullptr));
     }
     // ---- shift 0: P (mask_0 tau(B)) sigma(A) on the chain limbs
     {

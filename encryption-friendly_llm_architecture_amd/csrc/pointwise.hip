@@ -2,6 +2,8 @@
 // constant multiplies, the 3-polynomial tensor product and the NTT-domain Galois permutation.
 // One workgroup covers 512 consecutive residues of one limb with 16-byte accesses; blockIdx.y
 // walks (poly, limb) so every wavefront streams one contiguous 4 KiB run.
+#include <algorithm>
+
 #include "hemm_internal.hpp"
 
 namespace {
@@ -156,6 +158,18 @@ void launch_mul_scalar(const hemm_context *c, const u64 *a, size_t a_stride, con
     Operand A{a, a_stride};
     account(c, TR_POINTWISE, (size_t)2 * n_limbs * n_polys * c->N * 8);
     hipLaunchKernelGGL(scalar_kernel<false>, grid, block, 0, s, A, out, out_stride, c->d_modq, ll, sc, n_limbs, c->logN);
+}
+
+// out[0 .. words) = 0 (words a multiple of 2): a fill kernel where a memset node would be recorded into a captured graph
+__global__ __launch_bounds__(256) void zero_kernel(ulonglong2 *__restrict__ out, size_t pairs) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < pairs; i += (size_t)gridDim.x * 256)
+        out[i] = make_ulonglong2(0, 0);
+}
+void launch_zero(const hemm_context *c, u64 *out, size_t words, hipStream_t s) {
+    const size_t pairs = words / 2;
+    const unsigned blocks = (unsigned)std::min<size_t>((pairs + 255) / 256, 4096);
+    account(c, TR_POINTWISE, words * 8);
+    hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, s, (ulonglong2 *)out, pairs);
 }
 
 void launch_mul_imag(const hemm_context *c, const u64 *a, size_t a_stride, u64 *out, size_t out_stride,

@@ -28,6 +28,15 @@ def _L():
         L.hellm_export_key.argtypes = [vp, u64, u64p]
         L.hellm_ensure_rotation_keys.argtypes = [vp, u64p, u32]
         L.hellm_set_schedule.argtypes = [vp, ctypes.c_int, u32]
+        L.hellm_graph_begin.argtypes = [vp]
+        L.hellm_graph_end.argtypes = [vp, pvp]
+        L.hellm_graph_launch.argtypes = [vp]
+        L.hellm_graph_sync.argtypes = [vp]
+        L.hellm_graph_nodes.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
+        L.hellm_graph_destroy.argtypes = [vp]
+        L.hellm_graph_destroy.restype = None
+        L.hellm_phase_trace.argtypes = [vp, ctypes.c_int]
+        L.hellm_phase_report.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
         L.hellm_assume_single_tile.argtypes = [vp, ctypes.c_int]
         L.hellm_traffic.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ctypes.c_int]
         L.hellm_encrypt.argtypes = [vp, f64p, u32, u32, pvp]
@@ -42,6 +51,7 @@ def _L():
         L.hellm_ct_download.argtypes = [vp, u64p]
         L.hellm_ct_upload.argtypes = [vp, u64p, u32, u32, u32, u32, u32, u32, pvp]
         L.hellm_ct_clone.argtypes = [vp, pvp]
+        L.hellm_ct_assign.argtypes = [vp, vp, vp]
         L.hellm_ct_destroy.argtypes = [vp]
         L.hellm_pt_destroy.argtypes = [vp]
         L.hellm_pt_download.argtypes = [vp, u32p, u64p]
@@ -192,6 +202,36 @@ def chebyshev_product_basis(coeffs, baby_steps):
     return split(c)
 
 
+class Graph:
+    """A recorded sequence of HEMMer calls (hellm_graph_*): launch() replays it asynchronously on its own stream,
+    sync() waits for it."""
+
+    def __init__(self, owner, h, keep):
+        self.owner, self.h, self.keep = owner, h, keep
+
+    def launch(self):
+        check(_L().hellm_graph_launch(self.h))
+
+    def sync(self):
+        check(_L().hellm_graph_sync(self.h))
+
+    def nodes(self):
+        n = ctypes.c_uint64()
+        check(_L().hellm_graph_nodes(self.h, ctypes.byref(n)))
+        return n.value
+
+    def free(self):
+        if self.h:
+            _L().hellm_graph_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
 class HEMMer:
     """HELLM::HEMMer on the GPU.  preset=True builds the FGb-sized context (N = 2^16)."""
 
@@ -239,6 +279,32 @@ class HEMMer:
         check(_L().hellm_sync())
 
     TRAFFIC_KINDS = ("transforms", "key_products", "basis_conversions", "tensor_accumulation", "masked_sums", "pointwise")
+
+    def assign(self, dst, src):
+        """dst's residues = src's, in place (hellm_ct_assign)"""
+        check(_L().hellm_ct_assign(self.h, dst.h, src.h))
+
+    def record(self, fn):
+        """Runs fn() with the calls on this HEMMer recorded into a HIP graph instead of executed; returns
+        (Graph, fn's result).  fn's result and operands are kept alive by the graph object."""
+        check(_L().hellm_graph_begin(self.h))
+        try:
+            res = fn()
+        finally:
+            g = vp()
+            rc = _L().hellm_graph_end(self.h, ctypes.byref(g))
+        check(rc)
+        return Graph(self, g, res), res
+
+    def phase_trace(self, on=True):
+        """Record an event at each named point of the batched schedules from now on (off: stop and forget)."""
+        check(_L().hellm_phase_trace(self.h, int(on)))
+
+    def phase_report(self):
+        """[(name, ms since the previous mark)] of the marks recorded so far; waits for the device."""
+        buf = ctypes.create_string_buffer(1 << 16)
+        check(_L().hellm_phase_report(self.h, buf, len(buf)))
+        return [(l.split("\t")[0], float(l.split("\t")[1])) for l in buf.value.decode().splitlines()]
 
     def traffic(self, reset=False):
         """Algorithmic bytes and launch counts queued on the device context since the last reset, by kind of work."""

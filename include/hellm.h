@@ -33,6 +33,27 @@ int hellm_secret_coeffs(hellm_hemmer *h, int32_t *out /* N */);
 int hellm_export_key(hellm_hemmer *h, uint64_t galois, uint64_t *out);
 int hellm_ensure_rotation_keys(hellm_hemmer *h, const uint64_t *left_rotations, uint32_t count);
 int hellm_sync(void); /* CudaTools::cudaDeviceSynchronize */
+/* Phase trace of the batched products (no counterpart in HEMMer): while it is on, the schedule records an event on the
+ * default stream at each named point it passes (packing, transform stages, rotation sources, main loop, giant steps);
+ * the report waits for the device, writes one "name<TAB>milliseconds since the previous mark" line per mark into
+ * text and forgets the marks. */
+int hellm_phase_trace(hellm_hemmer *h, int on);
+int hellm_phase_report(hellm_hemmer *h, char *text, size_t capacity);
+/* A sequence of calls on one HEMMer recorded once into a HIP graph and replayed (no counterpart in HEMMer; for loops
+ * that run the same products on operands rewritten in place).  Between begin and end the calls of this thread on h are
+ * recorded instead of run: every buffer they use must exist already, so run the same sequence once before (keys,
+ * masks and scratch are made on first use).  Operand and result ciphertexts of the recorded calls must stay alive and
+ * in place while the graph is replayed; intermediates belong to the graph until it is destroyed.  A replay runs on
+ * the graph's own stream and is asynchronous: hellm_graph_sync before anything else touches its operands or results,
+ * and before other work on h (the context's scratch has one user at a time).  Term lists too long for the kernel
+ * arguments (more than 32 merged terms per launch) are refused while recording. */
+typedef struct hellm_graph hellm_graph;
+int hellm_graph_begin(hellm_hemmer *h);
+int hellm_graph_end(hellm_hemmer *h, hellm_graph **out);
+int hellm_graph_launch(hellm_graph *g);
+int hellm_graph_sync(hellm_graph *g);
+int hellm_graph_nodes(const hellm_graph *g, uint64_t *out);
+void hellm_graph_destroy(hellm_graph *g);
 /* hemm_traffic of the device context under this HEMMer (arrays of 8 entries, see hemm.h); no counterpart in HEMMer */
 int hellm_traffic(hellm_hemmer *h, uint64_t *bytes, uint64_t *launches, int reset);
 /* schedule of the products: fused != 0 (default) = batched launches with hoisted rotations,
@@ -63,6 +84,9 @@ int hellm_ct_download(const hellm_ct *ct, uint64_t *out /* [num_poly][level+1][N
 int hellm_ct_upload(hellm_hemmer *h, const uint64_t *residues, uint32_t num_poly, uint32_t level,
                     uint32_t rescale_counter, uint32_t rows, uint32_t cols, uint32_t block_width, hellm_ct **out);
 int hellm_ct_clone(const hellm_ct *ct, hellm_ct **out);
+/* dst's residues = src's, in place (same polynomials, level and pending rescales): how a loop feeds new operands to a
+ * recorded graph, whose launches read fixed addresses */
+int hellm_ct_assign(hellm_hemmer *h, hellm_ct *dst, const hellm_ct *src);
 void hellm_ct_destroy(hellm_ct *ct);
 void hellm_pt_destroy(hellm_pt *pt);
 int hellm_pt_download(const hellm_pt *pt, uint32_t *level, uint64_t *out /* [level+1][N] or NULL */);

@@ -39,6 +39,12 @@ const char *hemm_last_error(void);
 int hemm_context_create(uint32_t log_n, uint32_t n_q, uint32_t n_p, const uint64_t *primes,
                         uint32_t dnum, hemm_context **out);
 void hemm_context_destroy(hemm_context *ctx);
+/* The stream that a null `stream` argument of the entry points below stands for on this context: the legacy default
+ * stream until another one is named here.  For callers that record the library's launches into a HIP graph (stream
+ * capture cannot use the legacy default stream) or keep the library off the default stream altogether.  The context's
+ * scratch and staging regions have one user at a time: calls on different streams of one context must not overlap. */
+int hemm_context_set_stream(hemm_context *ctx, void *stream);
+void *hemm_context_stream(const hemm_context *ctx);
 /* primitive 2N-th root of unity used for prime `idx` (smallest g^((q-1)/2N) of order 2N) */
 uint64_t hemm_context_psi(const hemm_context *ctx, uint32_t idx);
 
@@ -104,6 +110,9 @@ int hemm_decode(hemm_context *ctx, const uint64_t *pt, uint32_t n_limbs, double 
 int hemm_add_scalar(hemm_context *ctx, const uint64_t *a, const uint64_t *re, const uint64_t *im, uint64_t *out,
                     uint32_t nq, int with_p, void *stream);
 /* HomEvaluator::multImagUnit :330: multiply by the monomial X^(N/2) in NTT form. */
+/* out[0 .. words) = 0 by a kernel (an even number of words, 16-byte aligned): the clearing step of an accumulation,
+ * safe to record into a HIP graph where a memset node is not.  No counterpart in HEaaN. */
+int hemm_zero(hemm_context *ctx, uint64_t *out, size_t words, void *stream);
 int hemm_mul_imag_unit(hemm_context *ctx, const uint64_t *a, size_t a_stride, uint64_t *out,
                        size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
 /* HomEvaluator::tensor :518: (b1,a1) x (b2,a2) -> (b1 b2, a1 b2 + a2 b1, a1 a2); accumulate != 0
