@@ -202,9 +202,9 @@ def test_masked_sums_full_ring_both_paths(bench, n_polys):
             assert np.array_equal(got[o], one(spec)), (o, spec)
 
 
-def test_preset_ccmm_residues_bit_exact():
-    """singleCCMatMul of two fresh 128 x 128 tiles on the preset (N = 2^16, 13 + 4 primes, dnum 3, target level 4):
-    every residue of the result equals the oracle's, which runs the same schedule with keys from the same seed."""
+@pytest.fixture(scope="module")
+def preset():
+    """The preset evaluator and the oracle over the same primes with keys from the same seed."""
     load_package()
     from efla_amd import hellm
     H = hellm.HEMMer(preset=True, seed=3)
@@ -215,6 +215,97 @@ def test_preset_ccmm_residues_bit_exact():
     orc.gen_conj_key(3)
     orc.key_seed = 3
     assert np.array_equal(H.secret_coeffs(), orc.sk_coeffs)
+    return H, orc, R.OracleEval(orc)
+
+
+def as_oracle(orc, ct):
+    i = ct.info()
+    assert i["rescale_counter"] == 0
+    return O.Ct(ct.residues(), orc.delta[i["level"]])
+
+
+def test_preset_pcmm_residues_bit_exact(preset):
+    """singleMatMul at N = 2^16 (the 127 shifts as terms of one sum dealt to 16 partial outputs, the weight read
+    through a second automorphism, one ModDown): a single tile in the first block and the pair layout, residue for
+    residue against the oracle's restatement of that schedule."""
+    H, orc, ev = preset
+    rng = np.random.default_rng(31)
+    A, B, A2, B2 = (rng.uniform(-1, 1, (128, 128)) for _ in range(4))
+    top = orc.delta[orc.nQ - 1]
+    ca, pb = H.encrypt(A), H.encode(B)
+    c = H.single_matmul(ca, pb, 4)
+    want = R.mult_mat_mat_pc_lazy(orc, as_oracle(orc, ca), O.Pt(pb.residues(), top), 4, 128, 128)
+    assert c.info()["level"] == 4 == want.level
+    assert np.array_equal(c.residues(), want.data)
+    assert np.abs(H.decrypt(c) - A @ B).max() < 2.0 ** -12
+    ca2, pb2 = H.encrypt2(A, A2), H.encode2(B, B2)
+    c2 = H.single_matmul(ca2, pb2, 4)
+    want2 = R.mult_mat_mat_pc_lazy(orc, as_oracle(orc, ca2), O.Pt(pb2.residues(), top), 4, 128, 256)
+    assert np.array_equal(c2.residues(), want2.data)
+    d = H.decrypt2(c2)
+    assert np.abs(d[0] - A @ B).max() < 2.0 ** -12 and np.abs(d[1] - A2 @ B2).max() < 2.0 ** -12
+
+
+def test_preset_pair_layout_and_packed_ccmm_residues_bit_exact(preset):
+    """singleCCMatMul on the pair layout (two products per call) and packedMatMul + repackCC at N = 2^16."""
+    H, orc, ev = preset
+    rng = np.random.default_rng(32)
+    A, B, A2, B2 = (rng.uniform(-1, 1, (128, 128)) for _ in range(4))
+    pa, pb = H.encrypt2(A, A2), H.encrypt2(B, B2)
+    oa, ob = as_oracle(orc, pa), as_oracle(orc, pb)
+    c = H.single_cc_matmul(pa, pb, 4)
+    assert np.array_equal(c.residues(), R.mult_mat_mat_cc_packed_single(orc, oa, ob, 4, 128, 256).data)
+    d = H.decrypt2(c)
+    assert np.abs(d[0] - A @ B).max() < 2.0 ** -12 and np.abs(d[1] - A2 @ B2).max() < 2.0 ** -12
+    H.complex_packing_inplace(pa)
+    H.complex_packing_row_inplace(pb)
+    oa, ob = R.complex_packing_cols(ev, oa, 128, 256), R.complex_packing_rows(ev, ob, 128, 256)
+    assert np.array_equal(pa.residues(), oa.data) and np.array_equal(pb.residues(), ob.data)
+    prod = H.packed_matmul(pa, pb, 4)
+    want = R.mult_packed_mat_mat_fused(orc, oa, ob, 4, 128, 256)
+    assert np.array_equal(prod.residues(), want.data)
+    pc = H.repack_cc(prod)
+    assert np.array_equal(pc.residues(), R.repack_cc(ev, want).data)
+    d = H.decrypt2(pc)
+    assert np.abs(d[0] - A @ B).max() < 2.0 ** -12 and np.abs(d[1] - A2 @ B2).max() < 2.0 ** -12
+
+
+def test_preset_hoisted_pcmm_and_transpose_residues_bit_exact(preset):
+    """matMulPre (all 128 shifted copies) + matMulReUse on a complex-packed activation pair, and transposeInplace of a
+    pair-layout ciphertext, at N = 2^16."""
+    H, orc, ev = preset
+    n = 128
+    rng = np.random.default_rng(33)
+    X0, X1 = 0.1 * rng.normal(size=(n, n)), 0.1 * rng.normal(size=(n, n))
+    W = [rng.normal(0, 0.02, (n, n)) for _ in range(4)]
+    x = H.complex_packing(H.encrypt2(X0, X0), H.encrypt2(X1, X1))
+    ox = as_oracle(orc, x)
+    tmp = H.matmul_pre(x, 4)
+    otmp = R.mult_mat_mat_pre_fused(orc, ox, 4, n, 2 * n)
+    assert len(tmp) == n == len(otmp)
+    for k in range(n):
+        assert np.array_equal(tmp.get(k, n, n, 2 * n).residues(), otmp[k].data), k
+    wp = H.encode_diagonal_to_row4(*W, level=5)
+    owp = orc.encode(R.weights_diagonal_to_row4(*W, orc.slots), 5)
+    assert np.array_equal(wp.residues(), owp.data)
+    y = H.matmul_reuse(tmp, wp, 4)
+    assert np.array_equal(y.residues(), R.mult_mat_mat_reuse(ev, otmp, owp, 4).data)
+    z = H.decrypt2(H.repack_cc(y))
+    assert np.abs(z[0] - (X0 @ W[0] + X1 @ W[2])).max() < 2.0 ** -12
+    assert np.abs(z[1] - (X0 @ W[1] + X1 @ W[3])).max() < 2.0 ** -12
+    A, A2 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    t = H.encrypt2(A, A2)
+    want = R.diagonal_transform_fused(orc, as_oracle(orc, t), R.DIAG_SIGNED, n, 2 * n)
+    H.transpose_inplace(t)
+    assert np.array_equal(t.residues(), want.data)
+    d = H.decrypt2(t)
+    assert np.abs(d[0] - A.T).max() < 2.0 ** -12 and np.abs(d[1] - A2.T).max() < 2.0 ** -12
+
+
+def test_preset_ccmm_residues_bit_exact(preset):
+    """singleCCMatMul of two fresh 128 x 128 tiles on the preset (N = 2^16, 13 + 4 primes, dnum 3, target level 4):
+    every residue of the result equals the oracle's, which runs the same schedule with keys from the same seed."""
+    H, orc, _ = preset
     rng = np.random.default_rng(1)
     A, B = rng.uniform(-1, 1, (128, 128)), rng.uniform(-1, 1, (128, 128))
     ca, cb = H.encrypt(A), H.encrypt(B)
