@@ -68,6 +68,9 @@ def gpu_ccmm(args, out, headline_only=False):
         "achieved_GBps": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9,
         "frac_of_hbm_peak": total / (out["gpu_event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
+    # device memory after the product: evaluation keys by form (the hoisted sums read the compact one) and the buffer
+    # pool of the context as a whole (keys, masks, ciphertexts, workspaces)
+    out["resident_bytes_after_ccmm"] = H.key_bytes()
     if headline_only:
         return H
     # one rotation (automorphism + hybrid key switch) at the top level

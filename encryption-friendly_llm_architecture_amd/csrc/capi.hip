@@ -462,6 +462,14 @@ int hemm_key_compact(hemm_context *ctx, const uint64_t *evk, uint64_t *out, void
     HEMM_CATCH
 }
 
+int hemm_key_expand(hemm_context *ctx, const uint64_t *compact, uint64_t *evk, void *stream) {
+    HEMM_TRY
+    need(ctx && compact && evk, "null operand");
+    launch_key_expand(ctx, (const u64 *)compact, (u64 *)evk, on_stream(ctx, stream));
+    check_launch();
+    HEMM_CATCH
+}
+
 int hemm_hoisted_terms(hemm_context *ctx, const hemm_rot_term *terms, const uint32_t *group_offsets, uint32_t n_out,
                        uint32_t nq, uint64_t *y, int b_premultiplied, void *stream) {
     HEMM_TRY

@@ -174,6 +174,7 @@ void launch_masked_sum(hemm_context *c, const void *terms_dev, const u32 *group_
 void launch_sum_parts(hemm_context *c, const u64 *part, int parts, int n_out, int nq, u64 *y, hipStream_t s);
 size_t key_compact_words(const hemm_context *c);
 void launch_key_compact(const hemm_context *c, const u64 *evk, u64 *out, hipStream_t s);
+void launch_key_expand(const hemm_context *c, const u64 *compact, u64 *evk, hipStream_t s);
 int masked_arg_capacity();
 // table[j][r] = mask[j][r << shift]; true when every aligned run of 2^shift residues of the mask is constant
 bool launch_compact_mask(hemm_context *c, const u64 *mask, int n_limbs, int shift, u64 *table, hipStream_t s);

@@ -168,6 +168,9 @@ public:
     void setFused(bool on, u64 batch = 16) {
         fused_ = on;
         batch_ = batch;
+        // the batched schedules read rotation keys through the hoisted sums only: keys derived from now on are kept in
+        // the compact form (KeyPack::compactKey), one plain form at a time while they are generated
+        pack_.compact_on_generate_ = on;
     }
     bool fused() const { return fused_; }
     // Promise that the operands of singleCCMatMul hold a single tile block (as HEMMer::encrypt produces) and nothing

@@ -207,22 +207,34 @@ public:
     void save(const std::string &dir) const;
     void to(const Device &) {}
     bool hasMultKey() const { return mult_.words() != 0; }
-    bool hasGaloisKey(u64 galois) const { return galois_.count(galois) != 0; }
+    bool hasGaloisKey(u64 galois) const { return galois_.count(galois) != 0 || compact_.count({1, galois}) != 0; }
     const u64 *multKey() const;
     const u64 *galoisKey(u64 galois) const;
     // key switching rho_g(s)^2 -> s: rotates the degree-2 component of an un-relinearised product directly
-    bool hasGaloisSquareKey(u64 galois) const { return galois_sq_.count(galois) != 0; }
+    bool hasGaloisSquareKey(u64 galois) const { return galois_sq_.count(galois) != 0 || compact_.count({2, galois}) != 0; }
     const u64 *galoisSquareKey(u64 galois) const;
     const Context &getContext() const { return ctx_; }
     // The compact form of a key for the hoisted sums (hemm_key_compact: 6 bytes per residue of a prime below 2^44),
-    // made on first request and kept beside the plain key.  kind: 0 multiplication key, 1 key of X -> X^galois,
-    // 2 its square key.
+    // made on first request.  kind: 0 multiplication key, 1 key of X -> X^galois, 2 its square key.
+    // A Galois or square key that has a compact form gives up its plain form (the sums read only the compact one, and
+    // there are hundreds of such keys); galoisKey / galoisSquareKey rebuild the plain form on request
+    // (hemm_key_expand, lossless) and keep the few most recent ones.  The multiplication key keeps both forms.
     const u64 *compactKey(int kind, u64 galois) const;
+    // device bytes held by the keys: plain forms, compact forms
+    std::pair<u64, u64> keyBytes() const;
     // internal
     Context ctx_;
     DeviceBuffer mult_;
-    std::map<u64, DeviceBuffer> galois_, galois_sq_;
+    mutable std::map<u64, DeviceBuffer> galois_, galois_sq_;
     mutable std::map<std::pair<int, u64>, DeviceBuffer> compact_;
+    mutable std::vector<std::pair<int, u64>> rebuilt_;   // plain forms rebuilt from compact ones, oldest first
+    // set by a holder whose work goes through the hoisted sums: KeyGenerator then compacts a Galois or square key as
+    // soon as it is generated, so that at most one plain form exists at a time while hundreds of keys are derived
+    bool compact_on_generate_ = false;
+    bool compactible() const;   // the hoisted kernels take compact keys for this context (N >= 512, at most 6 digits)
+
+private:
+    const u64 *plainOrRebuilt(int kind, u64 galois) const;
 };
 
 class KeyGenerator {

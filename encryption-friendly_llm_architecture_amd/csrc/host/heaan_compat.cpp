@@ -1,5 +1,6 @@
 // Implementation of the HEaaN-compatible host surface (host/HEaaN/HEaaN.hpp): object lifetime,
 // level / scale bookkeeping, host-side encoding and sampling; every ring operation is a C-ABI call.
+#include <algorithm>
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -413,16 +414,26 @@ const u64 *KeyPack::multKey() const {
     if (!hasMultKey()) throw RuntimeException("multiplication key has not been generated");
     return mult_.data();
 }
-const u64 *KeyPack::galoisKey(u64 g) const {
-    auto it = galois_.find(g);
-    if (it == galois_.end()) throw RuntimeException("no key for Galois element " + std::to_string(g));
-    return it->second.data();
+const u64 *KeyPack::plainOrRebuilt(int kind, u64 g) const {
+    auto &plain = kind == 1 ? galois_ : galois_sq_;
+    auto it = plain.find(g);
+    if (it != plain.end()) return it->second.data();
+    auto ct = compact_.find({kind, g});
+    if (ct == compact_.end())
+        throw RuntimeException(std::string(kind == 1 ? "no key" : "no square key") + " for Galois element " + std::to_string(g));
+    // rebuilt plain forms are few at a time: a chain of single rotations uses a handful of steps over and over
+    const size_t keep = 4;
+    while (rebuilt_.size() >= keep) {
+        (rebuilt_.front().first == 1 ? galois_ : galois_sq_).erase(rebuilt_.front().second);
+        rebuilt_.erase(rebuilt_.begin());
+    }
+    DeviceBuffer b(ctx_, ctx_->dnum * 2 * (ctx_->nQ + ctx_->nP) * ctx_->N);
+    ck(hemm_key_expand(ctx_->dev, ct->second.data(), b.data(), nullptr));
+    rebuilt_.emplace_back(kind, g);
+    return plain.emplace(g, std::move(b)).first->second.data();
 }
-const u64 *KeyPack::galoisSquareKey(u64 g) const {
-    auto it = galois_sq_.find(g);
-    if (it == galois_sq_.end()) throw RuntimeException("no square key for Galois element " + std::to_string(g));
-    return it->second.data();
-}
+const u64 *KeyPack::galoisKey(u64 g) const { return plainOrRebuilt(1, g); }
+const u64 *KeyPack::galoisSquareKey(u64 g) const { return plainOrRebuilt(2, g); }
 const u64 *KeyPack::compactKey(int kind, u64 g) const {
     const auto id = std::make_pair(kind, kind == 0 ? u64(0) : g);
     auto it = compact_.find(id);
@@ -430,12 +441,28 @@ const u64 *KeyPack::compactKey(int kind, u64 g) const {
         const u64 *plain = kind == 0 ? multKey() : kind == 1 ? galoisKey(g) : galoisSquareKey(g);
         DeviceBuffer c(ctx_, hemm_key_compact_words(ctx_->dev));
         ck(hemm_key_compact(ctx_->dev, plain, c.data(), nullptr));
-        // made once per key, on the default stream: finished before the caller queues its sum on whichever stream (the
-        // side stream does not wait for later work of the default one)
+        // made once per key, on the context's stream: finished before the caller queues its sum on whichever stream (the
+        // side stream does not wait for later work of that one)
         hip_ck(hipStreamSynchronize(ctx_->stream()), "hipStreamSynchronize");
         it = compact_.emplace(id, std::move(c)).first;
+        if (kind != 0) {   // the plain form goes back to the pool (the next key generated takes its place)
+            (kind == 1 ? galois_ : galois_sq_).erase(g);
+            for (size_t i = 0; i < rebuilt_.size(); i++)
+                if (rebuilt_[i] == std::make_pair(kind, g)) {
+                    rebuilt_.erase(rebuilt_.begin() + (long)i);
+                    break;
+                }
+        }
     }
     return it->second.data();
+}
+bool KeyPack::compactible() const { return ctx_->dnum <= 6 && ctx_->N >= 512; }
+std::pair<u64, u64> KeyPack::keyBytes() const {
+    u64 plain = mult_.words() * 8, compact = 0;
+    for (auto &kv : galois_) plain += kv.second.words() * 8;
+    for (auto &kv : galois_sq_) plain += kv.second.words() * 8;
+    for (auto &kv : compact_) compact += kv.second.words() * 8;
+    return {plain, compact};
 }
 void KeyPack::save(const std::string &dir) const {
     const size_t words = ctx_->dnum * 2 * (ctx_->nQ + ctx_->nP) * ctx_->N;
@@ -451,13 +478,29 @@ void KeyPack::save(const std::string &dir) const {
         dump("MultKey.bin", mult_);
         idx << "mult\n";
     }
-    for (auto &kv : galois_) {
-        dump("GaloisKey_" + std::to_string(kv.first) + ".bin", kv.second);
-        idx << kv.first << "\n";
+    // every key, whichever form it is held in (a plain form that was given up is rebuilt for the dump)
+    std::vector<u64> gal, sq;
+    for (auto &kv : galois_) gal.push_back(kv.first);
+    for (auto &kv : galois_sq_) sq.push_back(kv.first);
+    for (auto &kv : compact_) {
+        if (kv.first.first == 1 && !galois_.count(kv.first.second)) gal.push_back(kv.first.second);
+        if (kv.first.first == 2 && !galois_sq_.count(kv.first.second)) sq.push_back(kv.first.second);
     }
-    for (auto &kv : galois_sq_) {
-        dump("GaloisSquareKey_" + std::to_string(kv.first) + ".bin", kv.second);
-        idx << "sq" << kv.first << "\n";
+    std::sort(gal.begin(), gal.end());
+    std::sort(sq.begin(), sq.end());
+    auto dump_ptr = [&](const std::string &name, const u64 *src) {
+        hip_ck(hipMemcpy(h.data(), src, words * 8, hipMemcpyDeviceToHost), "hipMemcpy");
+        std::ofstream f(dir + "/" + name, std::ios::binary);
+        if (!f) throw RuntimeException("cannot open " + dir + "/" + name);
+        f.write((const char *)h.data(), (std::streamsize)(words * 8));
+    };
+    for (u64 g : gal) {
+        dump_ptr("GaloisKey_" + std::to_string(g) + ".bin", galoisKey(g));
+        idx << g << "\n";
+    }
+    for (u64 g : sq) {
+        dump_ptr("GaloisSquareKey_" + std::to_string(g) + ".bin", galoisSquareKey(g));
+        idx << "sq" << g << "\n";
     }
 }
 KeyPack::KeyPack(const Context &c, const std::string &dir) : ctx_(c) {
@@ -547,6 +590,7 @@ void KeyGenerator::genLeftRotKey(u64 rot) const {
     DeviceBuffer sg;
     gen_galois(*this, ctx_, sk_, g, sg);
     genSwitchKey(g, sg.data(), pack_.galois_[g]);
+    if (pack_.compact_on_generate_ && pack_.compactible()) (void)pack_.compactKey(1, g);
 }
 void KeyGenerator::genGaloisKey(u64 g) const {
     if (g % 2 == 0 || g >= 2 * ctx_->N) throw RuntimeException("a Galois element is odd and below 2N");
@@ -554,6 +598,7 @@ void KeyGenerator::genGaloisKey(u64 g) const {
     DeviceBuffer sg;
     gen_galois(*this, ctx_, sk_, g, sg);
     genSwitchKey(g, sg.data(), pack_.galois_[g]);
+    if (pack_.compact_on_generate_ && pack_.compactible()) (void)pack_.compactKey(1, g);
 }
 void KeyGenerator::genLeftRotSquareKey(u64 rot) const {
     const u64 slots = ctx_->N / 2;
@@ -569,6 +614,7 @@ void KeyGenerator::genGaloisSquareKey(u64 g) const {
     ck(hemm_pointwise(ctx_->dev, HEMM_MUL, sk_.ntt(), 0, sk_.ntt(), 0, s2.data(), 0, (uint32_t)ctx_->nQ, 1, 1, nullptr));
     ck(hemm_automorphism(ctx_->dev, s2.data(), 0, sg.data(), 0, g, (uint32_t)T, 1, nullptr));
     genSwitchKey((u64(1) << 40) | g, sg.data(), pack_.galois_sq_[g]);
+    if (pack_.compact_on_generate_ && pack_.compactible()) (void)pack_.compactKey(2, g);
 }
 void KeyGenerator::genRightRotKey(u64 rot) const {
     const u64 slots = ctx_->N / 2;

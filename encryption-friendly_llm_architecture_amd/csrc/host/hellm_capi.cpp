@@ -130,6 +130,15 @@ int hellm_sync(void) {
     FACADE_CATCH
 }
 
+int hellm_key_bytes(hellm_hemmer *h, uint64_t *plain, uint64_t *compact, uint64_t *pool) {
+    FACADE_TRY
+    need(h, "null argument");
+    const auto kb = h->m->keyPack().keyBytes();
+    if (plain) *plain = kb.first;
+    if (compact) *compact = kb.second;
+    if (pool) *pool = h->m->getContext()->pool_bytes;
+    FACADE_CATCH
+}
 int hellm_phase_trace(hellm_hemmer *h, int on) {
     FACADE_TRY
     need(h, "null argument");

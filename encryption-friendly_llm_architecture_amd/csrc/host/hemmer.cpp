@@ -49,6 +49,7 @@ HEMMer::HEMMer(const std::string &key_path, int device_id, ParameterPreset prese
 HEMMer::~HEMMer() = default;
 
 void HEMMer::init() {
+    pack_.compact_on_generate_ = fused_;
     KeyGenerator keygen(context_, sk_, pack_);
     if (!pack_.hasMultKey()) keygen.genMultKey();
     keygen.genConjKey();

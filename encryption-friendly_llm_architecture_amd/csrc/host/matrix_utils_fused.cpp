@@ -83,7 +83,7 @@ struct Rot {
 // compact form, a quarter less to read for the limbs of primes below 2^44, wherever the kernels take it (up to 6
 // digits), else the plain one.
 void set_key(hemm_rot_term &t, const KeyPack &pack, int kind, u64 galois) {
-    if (pack.getContext()->dnum <= 6) {
+    if (pack.compactible()) {
         t.evk = pack.compactKey(kind, galois);
         t.flags = HEMM_ROT_COMPACT_KEY;
     } else {

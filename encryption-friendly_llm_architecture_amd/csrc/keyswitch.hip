@@ -1011,6 +1011,25 @@ __global__ __launch_bounds__(256) void key_compact_kernel(const u64 *__restrict_
         *(ulonglong2 *)(limb + n * 8) = v;
     }
 }
+// the inverse: the plain key [dnum][2][n_full][N] of a compact one (lossless: 6 bytes hold any residue below 2^48)
+__global__ __launch_bounds__(256) void key_expand_kernel(const char *__restrict__ in, u64 *__restrict__ evk,
+                                                         const u32 *__restrict__ koff, const double *__restrict__ fp,
+                                                         int n_full, int logN) {
+    const size_t N = (size_t)1 << logN;
+    const int prime = blockIdx.y % n_full, slice = blockIdx.y / n_full;
+    const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    const char *limb = in + ((size_t)slice * koff[n_full] + koff[prime]) * (2 * N);
+    ulonglong2 v;
+    if (fp[4 * prime] != 0.0) {
+        const u32 *pair = (const u32 *)(limb + n * 6);
+        const u32 hi = pair[2];
+        v.x = ((u64)(hi & 0xffffu) << 32) | pair[0];
+        v.y = ((u64)(hi >> 16) << 32) | pair[1];
+    } else {
+        v = *(const ulonglong2 *)(limb + n * 8);
+    }
+    *(ulonglong2 *)(evk + ((size_t)slice * n_full + prime) * N + n) = v;
+}
 size_t key_compact_words(const hemm_context *c) {
     return (size_t)c->dnum * 2 * c->key_off[c->nQ + c->nP] * (2 * (size_t)c->N) / 8;
 }
@@ -1019,6 +1038,14 @@ void launch_key_compact(const hemm_context *c, const u64 *evk, u64 *out, hipStre
     const int n_full = c->nQ + c->nP;
     account(c, TR_POINTWISE, (size_t)c->dnum * 2 * n_full * c->N * 8 + key_compact_words(c) * 8);
     hipLaunchKernelGGL(key_compact_kernel, dim3(c->N / 512, c->dnum * 2 * n_full), dim3(256), 0, s, evk, (char *)out,
+                       c->d_key_off, c->d_fp, n_full, c->logN);
+}
+
+void launch_key_expand(const hemm_context *c, const u64 *compact, u64 *evk, hipStream_t s) {
+    if (c->N < 512) throw std::invalid_argument("compact keys need N >= 512");
+    const int n_full = c->nQ + c->nP;
+    account(c, TR_POINTWISE, (size_t)c->dnum * 2 * n_full * c->N * 8 + key_compact_words(c) * 8);
+    hipLaunchKernelGGL(key_expand_kernel, dim3(c->N / 512, c->dnum * 2 * n_full), dim3(256), 0, s, (const char *)compact, evk,
                        c->d_key_off, c->d_fp, n_full, c->logN);
 }
 

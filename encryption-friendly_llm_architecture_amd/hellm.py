@@ -35,6 +35,7 @@ def _L():
         L.hellm_graph_nodes.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
         L.hellm_graph_destroy.argtypes = [vp]
         L.hellm_graph_destroy.restype = None
+        L.hellm_key_bytes.argtypes = [vp] + [ctypes.POINTER(ctypes.c_uint64)] * 3
         L.hellm_phase_trace.argtypes = [vp, ctypes.c_int]
         L.hellm_phase_report.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
         L.hellm_assume_single_tile.argtypes = [vp, ctypes.c_int]
@@ -295,6 +296,12 @@ class HEMMer:
             rc = _L().hellm_graph_end(self.h, ctypes.byref(g))
         check(rc)
         return Graph(self, g, res), res
+
+    def key_bytes(self):
+        """{'plain', 'compact', 'pool'}: device bytes of the evaluation keys by form and of the context's buffer pool"""
+        a, b, c = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
+        check(_L().hellm_key_bytes(self.h, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+        return {"plain": a.value, "compact": b.value, "pool": c.value}
 
     def phase_trace(self, on=True):
         """Record an event at each named point of the batched schedules from now on (off: stop and forget)."""

@@ -33,6 +33,10 @@ int hellm_secret_coeffs(hellm_hemmer *h, int32_t *out /* N */);
 int hellm_export_key(hellm_hemmer *h, uint64_t galois, uint64_t *out);
 int hellm_ensure_rotation_keys(hellm_hemmer *h, const uint64_t *left_rotations, uint32_t count);
 int hellm_sync(void); /* CudaTools::cudaDeviceSynchronize */
+/* Device bytes held by this HEMMer's evaluation keys (plain forms, compact forms) and by the buffer pool of its context
+ * as a whole (every buffer it ever took from the device: keys, masks, ciphertexts, workspaces; freed buffers stay in
+ * the pool for reuse).  No counterpart in HEMMer. */
+int hellm_key_bytes(hellm_hemmer *h, uint64_t *plain, uint64_t *compact, uint64_t *pool);
 /* Phase trace of the batched products (no counterpart in HEMMer): while it is on, the schedule records an event on the
  * default stream at each named point it passes (packing, transform stages, rotation sources, main loop, giant steps);
  * the report waits for the device, writes one "name<TAB>milliseconds since the previous mark" line per mark into

@@ -177,10 +177,12 @@ typedef struct {
  * polynomial the limbs back to back; such a limb as N/2 records of 12 bytes, one per residue pair: two 32-bit low
  * words, then the two 16-bit high halves in one word; any other limb as N words).  Needs N >= 512 and at most 6
  * digits per key switch.  All terms of one call use the same layout.  out: hemm_key_compact_words(ctx) words.  The
- * plain key stays valid and is what every other call takes.
+ * plain key is what every other call takes.
  * No counterpart in HEaaN's interface (its key storage is not exposed). */
 size_t hemm_key_compact_words(const hemm_context *ctx);
 int hemm_key_compact(hemm_context *ctx, const uint64_t *evk, uint64_t *out, void *stream);
+/* the plain key [dnum][2][n_q+n_p][N] back from its compact form (lossless), for holders that keep only the latter */
+int hemm_key_expand(hemm_context *ctx, const uint64_t *compact, uint64_t *evk, void *stream);
 /* Algorithmic bytes of everything queued on this context since the last reset, by kind of work (for each launch: the
  * operands it must read once plus the results it must write once; a two-launch 2^16-point transform counts one read
  * and one write per limb), and the number of launches; counted on the host, costs nothing on the device.  Kinds:
