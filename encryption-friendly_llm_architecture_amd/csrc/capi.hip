@@ -355,11 +355,19 @@ int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, c
     HEMM_CATCH
 }
 
-// descriptor staging: one device region reused by every call (copies and kernels are ordered on the stream)
+// descriptor staging: one device region per stream, reused by every call on it (copies and kernels are ordered on the
+// stream)
 static void *upload_desc(hemm_context *ctx, const void *a, size_t na, const void *b, size_t nb, void **second,
                          hipStream_t s) {
     const size_t cap = 4u << 20;
-    if (!ctx->d_desc) HEMM_HIP(hipMalloc(&ctx->d_desc, cap));
+    void *region = nullptr;
+    for (auto &kv : ctx->d_desc)
+        if (kv.first == s) region = kv.second;
+    if (region == nullptr) {
+        if (ctx->d_desc.size() >= 8) throw std::invalid_argument("term lists were staged on more than 8 streams of one context");
+        HEMM_HIP(hipMalloc(&region, cap));
+        ctx->d_desc.emplace_back(s, region);
+    }
     const size_t off_b = (na + 255) & ~(size_t)255;
     if (off_b + nb > cap) throw std::invalid_argument("too many terms in one batched call");
     // the list is copied from pageable host memory that is gone when the call returns: nothing a graph could replay
@@ -370,9 +378,9 @@ static void *upload_desc(hemm_context *ctx, const void *a, size_t na, const void
     std::vector<char> both(off_b + nb);
     memcpy(both.data(), a, na);
     memcpy(both.data() + off_b, b, nb);
-    HEMM_HIP(hipMemcpyAsync(ctx->d_desc, both.data(), both.size(), hipMemcpyHostToDevice, s));
-    *second = (char *)ctx->d_desc + off_b;
-    return ctx->d_desc;
+    HEMM_HIP(hipMemcpyAsync(region, both.data(), both.size(), hipMemcpyHostToDevice, s));
+    *second = (char *)region + off_b;
+    return region;
 }
 
 int hemm_modup_batch(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint32_t nq, uint32_t n_in,
@@ -633,6 +641,24 @@ int hemm_tensor_batch_groups(hemm_context *ctx, const hemm_tensor_group *groups,
     HEMM_CATCH
 }
 
+// Strides of a batch must hold a whole polynomial, and the output may only share memory with the input when both lay
+// their polynomials out alike (out == in, equal strides: polynomial p of the result then overwrites the first nq - 1
+// limbs of polynomial p of the input, which the call has read by then); any other overlap would let one polynomial's
+// result land in another's unread input.
+static void check_rescale_layout(const hemm_context *ctx, const uint64_t *in, size_t in_stride, const uint64_t *out,
+                                 size_t out_stride, uint32_t nq, uint32_t n_polys) {
+    const size_t N = ctx->N, in_words = (size_t)nq * N, out_words = (size_t)(nq - 1) * N;
+    if (n_polys > 1) {
+        need(in_stride >= in_words, "in_stride is shorter than a polynomial of nq limbs");
+        need(out_stride >= out_words, "out_stride is shorter than a polynomial of nq - 1 limbs");
+    }
+    const uint64_t *in_end = in + (size_t)(n_polys - 1) * in_stride + in_words;
+    const uint64_t *out_end = out + (size_t)(n_polys - 1) * out_stride + out_words;
+    const bool overlap = out < in_end && in < out_end;
+    need(!overlap || (out == in && (n_polys == 1 || out_stride == in_stride)),
+         "out overlaps in (only out == in with equal strides is allowed)");
+}
+
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out, size_t out_stride,
                  uint32_t nq, uint32_t n_polys, void *stream) {
     HEMM_TRY
@@ -642,6 +668,7 @@ int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64
     need(nq >= 2, "rescale needs at least two limbs");
     need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_scratch_words(ctx),
          "n_polys * nq limbs must fit the context's scratch ((dnum + 7) * (nQ + nP) limbs)");
+    check_rescale_layout(ctx, in, in_stride, out, out_stride, nq, n_polys);
     launch_rescale(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
                    on_stream(ctx, stream));
     check_launch();
@@ -656,6 +683,7 @@ int hemm_rescale_static(hemm_context *ctx, const uint64_t *in, size_t in_stride,
     need(nq >= 2 && nq <= (uint32_t)ctx->nQ, "nq must be in [2, n_q]");
     need(n_polys >= 1 && (size_t)n_polys * nq * ctx->N <= hemm_static_scratch_words(),
          "n_polys * nq * N must not exceed HEMM_STATIC_SCRATCH_WORDS");
+    check_rescale_layout(ctx, in, in_stride, out, out_stride, nq, n_polys);
     launch_rescale_static(ctx, (const u64 *)in, in_stride, (u64 *)out, out_stride, (int)nq, (int)n_polys,
                           on_stream(ctx, stream));
     check_launch();
@@ -663,3 +691,5 @@ int hemm_rescale_static(hemm_context *ctx, const uint64_t *in, size_t in_stride,
 }
 
 }  // extern "C"
+
+static_assert(HEMM_STATIC_SCRATCH_WORDS == ((size_t)32 << 16), "hemm.h documents 32 limbs of N = 2^16");

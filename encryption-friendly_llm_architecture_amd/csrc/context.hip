@@ -184,7 +184,6 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_modq = (ModQ *)up(c->modq.data(), T * sizeof(ModQ));
     c->d_fp = (double *)up(fpc.data(), fpc.size() * 8);
     c->d_scratch = nullptr;
-    c->d_desc = nullptr;
     c->scratch_bytes = 0;
     memset(c->traffic, 0, sizeof(c->traffic));
     memset(c->launches, 0, sizeof(c->launches));
@@ -203,6 +202,6 @@ void hemm_context_free(hemm_context *c) {
     hipFree(c->d_modq);
     hipFree(c->d_fp);
     if (c->d_scratch) hipFree(c->d_scratch);
-    if (c->d_desc) hipFree(c->d_desc);
+    for (auto &kv : c->d_desc) (void)hipFree(kv.second);
     delete c;
 }

@@ -35,7 +35,9 @@ struct hemm_context {
     // scratch owned by the context (single stream use)
     u64 *d_scratch;
     size_t scratch_bytes;
-    void *d_desc;                   // staging for the term lists of batched calls
+    // staging for the term lists of batched calls: one region per stream that has staged a list (a region has one
+    // user at a time: the copy into it and the kernel that reads it are ordered on that stream)
+    std::vector<std::pair<hipStream_t, void *>> d_desc;
     hipStream_t stream = nullptr;   // what a null stream argument of an entry point means for this context
     // compact evaluation keys: offset of every prime's limb inside a (digit, polynomial) slice and, last entry, the
     // slice size, in units of 2N bytes (a prime below 2^44 takes 6 bytes per residue = 3 units, any other 4)

@@ -786,7 +786,8 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     std::vector<std::pair<size_t, size_t>> chains;   // (first, count)
     for (size_t first = 0; first < sa.size(); first += G) chains.push_back({first, std::min(G, sa.size() - first)});
     bool two_streams = false;
-    // (term lists of more than 32 terms go through the context's one staging region, which two streams may not share)
+    // (chains of up to 32 shifts: their term lists travel in the kernel arguments; longer lists would be staged, each
+    // stream through a region of its own, and copied from pageable memory, which waits for the stream)
     if (chains.size() == 2 && G <= 32) {
         const size_t cut = ((chains[0].second + 1) / (size_t)g) * (size_t)g;   // shift index q holds i = q + 1
         if (cut >= 1 && cut - 1 >= 1 && cut - 1 < sa.size() && sa.size() - (cut - 1) <= G && cut - 1 <= G) {

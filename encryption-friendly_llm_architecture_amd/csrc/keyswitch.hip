@@ -949,7 +949,7 @@ void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, 
 // library runs on, held until the process ends.  Host code never passes the array's name to a kernel or a copy: the
 // name is only a handle for hipGetSymbolAddress, which yields the array's address on the device that is current,
 // and each device has its own.
-#define HEMM_STATIC_SCRATCH_WORDS ((size_t)32 << 16)
+#include "../../include/hemm.h"   // HEMM_STATIC_SCRATCH_WORDS: the limit callers size against is the array's size
 #define HEMM_MAX_DEVICES 64
 static __device__ __align__(256) u64 scratch[HEMM_STATIC_SCRATCH_WORDS];
 static u64 *g_static_scratch[HEMM_MAX_DEVICES];   // per device, filled by hemm_static_setup
@@ -959,9 +959,12 @@ size_t hemm_static_scratch_words() { return HEMM_STATIC_SCRATCH_WORDS; }
 // Set-up for launch_rescale_static, run by hemm_context_create with the context's device current: resolves the
 // device address of the scratch array on that device (once per device) and builds the context's constant tables,
 // so that the call itself has nothing left to allocate.
+static std::mutex &static_setup_mutex() {
+    static std::mutex *mu = new std::mutex();
+    return *mu;
+}
 void hemm_static_setup(hemm_context *c) {
-    static std::mutex mu;
-    std::lock_guard<std::mutex> lk(mu);
+    std::lock_guard<std::mutex> lk(static_setup_mutex());
     if (c->device < 0 || c->device >= HEMM_MAX_DEVICES) throw std::invalid_argument("device index out of range");
     if (g_static_scratch[c->device] == nullptr) {
         u64 *ptr = nullptr;
@@ -976,7 +979,8 @@ void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64
                            int n_polys, hipStream_t s) {
     if (nq < 2) throw std::invalid_argument("rescale needs at least two limbs");
     if (n_polys < 1 || (size_t)n_polys * (size_t)nq * (size_t)c->N > HEMM_STATIC_SCRATCH_WORDS)
-        throw std::invalid_argument("n_polys * nq * N exceeds the static scratch of 2097152 words (32 limbs of N = 2^16)");
+        throw std::invalid_argument("n_polys * nq * N exceeds the static scratch of " +
+                                    std::to_string((size_t)HEMM_STATIC_SCRATCH_WORDS) + " words (HEMM_STATIC_SCRATCH_WORDS)");
     int dev = -1;
     HEMM_HIP(hipGetDevice(&dev));
     if (dev != c->device) throw std::invalid_argument("the context belongs to another device than the current one");
@@ -987,7 +991,12 @@ void launch_rescale_static(hemm_context *c, const u64 *in, size_t in_stride, u64
         auto it = r.tabs.find(c);
         if (it != r.tabs.end()) t = it->second;
     }
-    u64 *sc = g_static_scratch[dev];
+    if (dev < 0 || dev >= HEMM_MAX_DEVICES) throw std::invalid_argument("device index out of range");
+    u64 *sc = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(static_setup_mutex());
+        sc = g_static_scratch[dev];
+    }
     if (t == nullptr || sc == nullptr) throw std::runtime_error("context was not set up by hemm_context_create");
     rescale_with(c, t, sc, in, in_stride, out, out_stride, nq, n_polys, s);
 }

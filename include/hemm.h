@@ -9,13 +9,12 @@
  * uses chain prime j for j < nq and special prime (j - nq) after that.  `stream` is a
  * hipStream_t (NULL = default stream); calls are asynchronous on it.
  *
- * One stream per context at a time.  A context owns one device scratch region and one staging
- * region for term lists longer than 32.  hemm_modup, hemm_moddown, hemm_keyswitch, hemm_rotate,
- * hemm_relinearize and hemm_rescale work in the scratch region, and the batched
- * calls (hemm_hoisted_*, hemm_masked_sum_batch) copy long term lists through the staging region,
- * so two such calls queued on DIFFERENT streams of one context race unless the caller orders
- * them with events.  Calls that take a `workspace` argument use only that memory.  Callers that
- * want concurrent streams build one context per stream.
+ * A context owns one device scratch region.  hemm_modup, hemm_moddown, hemm_keyswitch,
+ * hemm_rotate, hemm_relinearize and hemm_rescale work in it, so two such calls queued on
+ * DIFFERENT streams of one context race unless the caller orders them with events.  Calls that
+ * take a `workspace` argument use only that memory; the batched calls (hemm_hoisted_*,
+ * hemm_masked_sum_batch) copy term lists longer than 32 through a staging region of their own
+ * per stream (up to 8 streams per context), so they may run side by side on two streams.
  *
  * Return value: 0 = ok, 1 = invalid argument, 2 = HIP/runtime failure; the text is in
  * hemm_last_error().
@@ -263,7 +262,9 @@ typedef struct {
 int hemm_tensor_batch_groups(hemm_context *ctx, const hemm_tensor_group *groups, uint32_t n_groups, uint32_t nq,
                              size_t acc_stride, void *stream);
 
-/* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last */
+/* HomEvaluator::rescale :540: [n_polys][nq][N] -> [n_polys][nq-1][N], (c_i - [c_last]_{q_i}) / q_last.
+ * With more than one polynomial, in_stride >= nq * N and out_stride >= (nq - 1) * N; out may not overlap in, except
+ * out == in with equal strides (each result then takes the place of its own input); anything else is refused. */
 int hemm_rescale(hemm_context *ctx, const uint64_t *in, size_t in_stride, uint64_t *out,
                  size_t out_stride, uint32_t nq, uint32_t n_polys, void *stream);
 
