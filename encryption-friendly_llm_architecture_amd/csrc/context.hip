@@ -176,7 +176,33 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_key_off = (u32 *)up(c->key_off.data(), c->key_off.size() * 4);
     c->d_w = (u64 *)up(w.data(), w.size() * 8);
     c->d_iw = (u64 *)up(iw.data(), iw.size() * 8);
-    c->d_ws = c->d_iws = nullptr;
+    c->d_rw = c->d_irw = nullptr;
+    if (logN == 16) {
+        // per prime the same storage convention as the stage-ordered tables: 16-byte entries, or doubles packed into
+        // the first half of the prime's region
+        std::vector<u64> rw((size_t)T * N * 2, 0), irw((size_t)T * N * 2, 0);
+        for (int i = 0; i < T; i++) {
+            const bool fp = fpc[4 * i] != 0.0;
+            const u64 *src[2] = {w.data() + (size_t)i * N * 2, iw.data() + (size_t)i * N * 2};
+            u64 *dst[2] = {rw.data() + (size_t)i * N * 2, irw.data() + (size_t)i * N * 2};
+            for (int dir = 0; dir < 2; dir++)
+                for (u32 r = 0; r < 256; r++)
+                    for (u32 l = 0; l < 4; l++)
+                        for (u32 g = 0; g < (1u << l); g++)
+                            for (u32 cc = 0; cc < 16; cc++) {
+                                const size_t from = ((size_t)(16 * (256 + r) + cc) << l) + g;
+                                const size_t to = ((size_t)r * 15 + (1u << l) - 1 + g) * 16 + cc;
+                                if (fp) {
+                                    dst[dir][to] = src[dir][from];
+                                } else {
+                                    dst[dir][2 * to] = src[dir][2 * from];
+                                    dst[dir][2 * to + 1] = src[dir][2 * from + 1];
+                                }
+                            }
+        }
+        c->d_rw = (u64 *)up(rw.data(), rw.size() * 8);
+        c->d_irw = (u64 *)up(irw.data(), irw.size() * 8);
+    }
     c->d_ninv = (u64 *)up(ninv.data(), T * 8);
     c->d_ninv_s = (u64 *)up(ninv_s.data(), T * 8);
     c->d_imag = (u64 *)up(im.data(), T * 8);
@@ -195,6 +221,8 @@ void hemm_context_free(hemm_context *c) {
     hipFree(c->d_key_off);
     hipFree(c->d_w);
     hipFree(c->d_iw);
+    if (c->d_rw) hipFree(c->d_rw);
+    if (c->d_irw) hipFree(c->d_irw);
     hipFree(c->d_ninv);
     hipFree(c->d_ninv_s);
     hipFree(c->d_imag);

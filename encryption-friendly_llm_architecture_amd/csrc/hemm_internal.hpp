@@ -25,8 +25,10 @@ struct hemm_context {
     std::vector<u64> psi;           // primitive 2N-th roots
     std::vector<ModQ> modq;         // host copy
     // device tables, all [prime][N] unless noted
-    u64 *d_w, *d_ws;                // psi^bitrev(i) and Shoup quotients (forward)
-    u64 *d_iw, *d_iws;              // inverse-transform twiddles
+    u64 *d_w, *d_iw;                // (psi^bitrev(i), Shoup quotient), forward and inverse transform
+    u64 *d_rw, *d_irw;              // N = 2^16: the twiddles of the row passes' inner radix-16 blocks in the order their
+                                    // threads read them, entry (r * 15 + 2^l - 1 + g) * 16 + c = entry
+                                    // ((16 (256 + r) + c) << l) + g of d_w / d_iw (nullptr for other ring sizes)
     u64 *d_ninv, *d_ninv_s;         // [prime]
     ModQ *d_modq;                   // [prime]
     double *d_fp;                   // [prime][4]: q, 1/q, 1/N mod q, that / q as doubles; q = 0 marks a prime of

@@ -330,6 +330,37 @@ __device__ __forceinline__ void radix16_inv(const F &f, typename F::E (&x)[16], 
     }
 }
 
+// The inner radix-16 block of a row pass (X = 16 (256 + r) + c: a different X for every thread) reads its 15 twiddles
+// from a table laid out for it: entry ((r * 15 + slot) * 16 + c), slot = 2^l - 1 + g for twiddle (X << l) + g, so that
+// the 16 threads of a row read 16 consecutive entries per (l, g) -- from the stage-ordered table they would read 16
+// entries 2^l apart, up to 64 cache lines per load instruction of a wavefront instead of 8.
+template <class F>
+__device__ __forceinline__ void radix16_fwd_rows(const F &f, typename F::E (&x)[16], const typename F::W *__restrict__ rt) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int d = 8 >> s;
+#pragma unroll
+        for (int g = 0; g < (1 << s); g++) {
+            const typename F::W w = rt[((1 << s) - 1 + g) * 16];
+#pragma unroll
+            for (int j = 0; j < d; j++) f.ct(x[g * 2 * d + j], x[g * 2 * d + j + d], w, (s & 1) != 0);
+        }
+    }
+}
+template <class F>
+__device__ __forceinline__ void radix16_inv_rows(const F &f, typename F::E (&x)[16], const typename F::W *__restrict__ rt) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const int d = 1 << s;
+#pragma unroll
+        for (int g = 0; g < (8 >> s); g++) {
+            const typename F::W w = rt[((8 >> s) - 1 + g) * 16];
+#pragma unroll
+            for (int j = 0; j < d; j++) f.gs(x[g * 2 * d + j], x[g * 2 * d + j + d], w);
+        }
+    }
+}
+
 #define ROWPAD 272  // 256 residues of a row + one pad word per 16, so a 16-lane column read
                     // (stride 17 words) hits 16 distinct bank pairs
 __device__ __forceinline__ int padc(int c) { return c + (c >> 4); }
@@ -683,12 +714,14 @@ struct NttEpilogue {
 
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
 template <bool INV, bool EPI, class F>
-__device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__restrict__ tw_int, const F f, u64 *lds_raw,
-                                          const u32 r, const u64 q, const u64 *__restrict__ mn, u64 *__restrict__ o,
-                                          const Tw cst, const u64 *__restrict__ ld) {
+__device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__restrict__ tw_int,
+                                          const Tw *__restrict__ rtw_int, const F f, u64 *lds_raw, const u32 r, const u64 q,
+                                          const u64 *__restrict__ mn, u64 *__restrict__ o, const Tw cst,
+                                          const u64 *__restrict__ ld) {
     typedef typename F::E E;
     const typename F::W *tw = (const typename F::W *)tw_int;
     const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
+    const typename F::W *rt = (const typename F::W *)rtw_int + (r * 15u * 16u + (u32)c);
     E *l = (E *)lds_raw + rr * ROWPAD;
     u64 *lc = lds_raw + rr * ROWPAD;
     E *mem = (E *)row;
@@ -708,7 +741,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
 #pragma unroll
             for (int k = 0; k < 16; k++) mv[k] = __builtin_nontemporal_load(mn + c + 16 * k);
         }
-        radix16_fwd(f, x, tw, 16u * (256u + r) + c);
+        radix16_fwd_rows(f, x, rt);
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) l[padc(16 * c + k)] = x[k];
@@ -726,7 +759,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = f.from_canonical(lc[padc(16 * c + k)]);
-        radix16_inv(f, x, tw, 16u * (256u + r) + c);
+        radix16_inv_rows(f, x, rt);
         f.after_inverse_block(x);
         wave_sync();
 #pragma unroll
@@ -743,6 +776,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
 
 template <bool INV, bool EPI>
 __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
+                                                         const Tw *__restrict__ rtw_all,
                                                          const ModQ *__restrict__ modq, const double *__restrict__ fp,
                                                          LimbList ll, LimbList sl, int n_limbs, size_t poly_stride,
                                                          NttEpilogue ep) {
@@ -757,7 +791,7 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
     const int limb = (int)(group >> 4);
     const u32 slab = group & 15u;
     const int prime = ll.idx[limb];
-    const Tw *tw = tw_all + ((size_t)prime << 16);
+    const Tw *tw = tw_all + ((size_t)prime << 16), *rtw = rtw_all + ((size_t)prime << 16);
     const u32 r = slab * 16 + (threadIdx.x >> 4);  // global row
     u64 *row = data + (size_t)poly * poly_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     const u64 *mn = nullptr;
@@ -774,11 +808,11 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
     if (INV && ep.minuend != nullptr)
         ld = ep.minuend + (size_t)poly * ep.minuend_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
     if (fp[4 * prime] != 0.0)
-        rows_body<INV, EPI>(row, tw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI>(row, tw, rtw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
     else if (INV || (q >> 60) != 0)
-        rows_body<INV, EPI>(row, tw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI>(row, tw, rtw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
     else
-        rows_body<INV, EPI>(row, tw, IntFieldT<true>(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI>(row, tw, rtw, IntFieldT<true>(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
 }
 
 }  // namespace
@@ -818,8 +852,8 @@ bool launch_ntt_sub_scale(const hemm_context *c, u64 *data, int n_limbs, int n_p
                        minuend_stride, out_stride};
         hipLaunchKernelGGL(ntt16_cols_kernel<false>, dim3(16, n_limbs * np), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                            c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)nullptr);
-        hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * np), block, 0, s, d, tw, c->d_modq,
-                           c->d_fp, ll, sl, n_limbs, poly_stride, ep);
+        hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * np), block, 0, s, d, tw, (const Tw *)c->d_rw,
+                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, ep);
     }
     return true;
 }
@@ -865,10 +899,10 @@ bool launch_ntt_converted(const hemm_context *c, const ConvSources &cs, u64 *dat
     if (tail) {
         NttEpilogue ep{ep_minuend, ep_out, (const Tw *)ep_cst_dev, ep_minuend_stride, ep_out_stride};
         hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw,
-                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, ep);
+                           (const Tw *)c->d_rw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, ep);
     } else {
         hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * n_limbs * n_polys), block, 0, s, data, tw,
-                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
+                           (const Tw *)c->d_rw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
     }
     return true;
 }
@@ -918,7 +952,7 @@ bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const u
         u64 *cp = conv + (size_t)p0 * conv_stride;
         ss.src = yp;
         hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * n_src * np), block, 0, s, yp, (const Tw *)c->d_iw,
-                           c->d_modq, c->d_fp, sp, ssl, n_src, y_stride, NttEpilogue{});
+                           (const Tw *)c->d_irw, c->d_modq, c->d_fp, sp, ssl, n_src, y_stride, NttEpilogue{});
 #define SLAB_CASE(NREG, LDS)                                                                                             \
     hipLaunchKernelGGL((ntt16_slab_convert_kernel<NREG, LDS>), dim3(16, np), block, 0, s, cp, conv_stride,             \
                        (const Tw *)c->d_w, (const Tw *)c->d_iw, c->d_modq, c->d_ninv, c->d_ninv_s, c->d_fp, ss)
@@ -929,7 +963,7 @@ bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const u
 #undef SLAB_CASE
         NttEpilogue ep{yp, out + (size_t)p0 * out_stride, (const Tw *)cst_dev, y_stride, out_stride};
         hipLaunchKernelGGL((ntt16_rows_kernel<false, true>), dim3(16 * nq_out * np), block, 0, s, cp, (const Tw *)c->d_w,
-                           c->d_modq, c->d_fp, cl, ident, nq_out, conv_stride, ep);
+                           (const Tw *)c->d_rw, c->d_modq, c->d_fp, cl, ident, nq_out, conv_stride, ep);
     }
     return true;
 }
@@ -950,8 +984,8 @@ bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_str
         NttEpilogue from{};
         from.minuend = src + (size_t)p0 * src_poly_stride;
         from.minuend_stride = src_poly_stride;
-        hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, d, tw, c->d_modq, c->d_fp, ll,
-                           sl, n_limbs, poly_stride, from);
+        hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, d, tw, (const Tw *)c->d_irw,
+                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, from);
         hipLaunchKernelGGL(ntt16_cols_kernel<true>, dim3(16, lanes), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                            c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)final_scale);
     }
@@ -976,11 +1010,11 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
             if (!inverse) {
                 hipLaunchKernelGGL(ntt16_cols_kernel<false>, dim3(16, ln), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                                    c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)nullptr);
-                hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * ln), block, 0, s, d, tw, c->d_modq,
-                                   c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
+                hipLaunchKernelGGL((ntt16_rows_kernel<false, false>), dim3(16 * ln), block, 0, s, d, tw,
+                                   (const Tw *)c->d_rw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
             } else {
-                hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * ln), block, 0, s, d, tw, c->d_modq,
-                                   c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
+                hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * ln), block, 0, s, d, tw,
+                                   (const Tw *)c->d_irw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, NttEpilogue{});
                 hipLaunchKernelGGL(ntt16_cols_kernel<true>, dim3(16, ln), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                                    c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)final_scale);
             }
