@@ -460,10 +460,17 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
     ensureRotationKeys(transformRotations(MaskKind::Horizontal, w));
     ensureRotationKeys(transformRotations(MaskKind::Vertical, w));
     if (fused_) {
-        // one tile block and nothing else in the slot vector: promised by the caller, or known because both operands
-        // come from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots)
+        // One tile block and nothing else in the slot vector: promised by the caller, or known because the operand
+        // comes from Encryptor::encrypt through slot-wise operations only (Ciphertext::occupiedSlots).  Only B has to
+        // be such a tile: its row shifts become exact rotations once tau(B) is copied into every block, and each
+        // slot of the sum over the shifts of sigma(A) then holds what it should whatever A carries in its other
+        // blocks (column shifts stay inside a row; the rotations of the baby-step / giant-step split cancel slot by
+        // slot).  What A carries there shows up in the other blocks of the result, so the result is known to be a
+        // single tile only when A is one as well.
         const u64 block = (u64)(n * w);
-        const bool single = single_tile_ || (a.get().occupiedSlots() <= block && b.get().occupiedSlots() <= block);
+        const bool a_single = single_tile_ || a.get().occupiedSlots() <= block;
+        const bool single = single_tile_ || b.get().occupiedSlots() <= block;
+        const u64 unknown = ~u64(0);
         // A single tile with a level to spare goes through the complex-packed product: adjacent columns of A and
         // adjacent rows of B are fused into complex slots (one level), the product then needs n / 2 column shifts
         // (each a key product and a ModDown) instead of n, and x + conj(x) returns the real product.
@@ -501,14 +508,16 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
                 }
             }
             CtxtTensor res = multMatMatComplexPackedFused(eval_, btp_, a, b, T, matrix_transformer, batch_, spread, true);
-            if (spread) res.get().occupied_ = block;
+            if (spread) res.get().occupied_ = a_single ? block : unknown;
             return res;
         }
         std::vector<u64> square_rots;
         ensureRotationKeys(fusedCcmmRotations(TileTensorShape(n, n, w), log_slots_, square_rots, false, single));
         KeyGenerator keygen(context_, sk_, pack_);
         for (u64 r : square_rots) keygen.genLeftRotSquareKey(r);
-        return multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, single);
+        CtxtTensor res = multMatMatFused(eval_, btp_, a, b, T, matrix_transformer, batch_, single);
+        if (!a_single) res.get().occupied_ = unknown;
+        return res;
     }
     ensureRotationKeys({1, (u64)w, slots - (u64)n, slots - (u64)((n * w) % (i64)slots)});
     return multMatMat(eval_, btp_, a, b, T, matrix_transformer);

@@ -232,13 +232,41 @@ def test_ccmm_stacked_tiles_keep_block_products(small):
     c3 = H.single_cc_matmul(ca, lb, 2)
     want3 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ca), to_oracle(orc, lb), 2, 16, 16, single_tile=False)
     assert np.array_equal(c3.residues(), want3.data)
-    # a rotation forgets what was known about a single tile: the masked route again
-    ra = H.left_rotate(H.left_rotate(H.encrypt(A[:16]), 3), 512 - 3)
-    eb16 = H.encrypt(B[:16])
-    c2 = H.single_cc_matmul(ra, eb16, 2)
-    want2 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ra), to_oracle(orc, eb16), 2, 16, 16, single_tile=False)
+    # a rotation forgets what was known about a single tile: with such a B the masked route again
+    ea16 = H.encrypt(A[:16])
+    rb = H.left_rotate(H.left_rotate(H.encrypt(B[:16]), 3), 512 - 3)
+    c2 = H.single_cc_matmul(ea16, rb, 2)
+    want2 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, ea16), to_oracle(orc, rb), 2, 16, 16, single_tile=False)
     assert np.array_equal(c2.residues(), want2.data)
     assert np.abs(H.decrypt(c2) - A[:16] @ B[:16]).max() < 2 ** -18
+
+
+def test_ccmm_only_the_right_operand_has_to_be_a_known_single_tile(small):
+    """A carries a second tile (or anything else) beyond its first block and nothing is known about it; B comes from
+    encrypt.  tau(B) can still be spread over the blocks, so the product takes the single-tile route (residues of the
+    oracle's restatement of it), the first block of the result is A1 B, and the result is not taken for a single
+    tile afterwards: used as the right operand of another product it goes through the masked route."""
+    H, orc, ev = small
+    rng = np.random.default_rng(41)
+    A, B, C = rng.uniform(-1, 1, (32, 16)), rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    ea = H.encrypt(A)
+    ca = H.upload(ea.residues(), 16, 16, 16)        # two stacked tiles declared as one 16 x 16 tensor
+    cb = H.encrypt(B)
+    for la, lb in ((7, 7), (6, 7), (5, 5)):          # separate packing at T+5 / T+4, composite transform at T+3
+        a = H.level_down(ca, la) if la < 7 else ca
+        b = H.level_down(cb, lb) if lb < 7 else cb
+        c = H.single_cc_matmul(a, b, 2)
+        want = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, a), to_oracle(orc, b), 2, 16, 16, single_tile=True)
+        assert np.array_equal(c.residues(), want.data), (la, lb)
+        assert np.abs(H.decrypt(c) - A[:16] @ B).max() < 2 ** -18
+    assert np.abs(H.decrypt_slots(c)[256:]).max() > 2 ** -6          # the other block is not empty ...
+    cc = H.encrypt(C)
+    # ... and the result does not pass for a single tile: as a right operand it takes the masked route
+    hi = H.single_cc_matmul(ca, cb, 4)
+    d = H.single_cc_matmul(H.level_down(cc, 4), hi, 1)
+    want = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, H.level_down(cc, 4)), to_oracle(orc, hi), 1, 16, 16, single_tile=False)
+    assert np.array_equal(d.residues(), want.data)
+    assert np.abs(H.decrypt(d) - C @ (A[:16] @ B)).max() < 2 ** -16
 
 
 @pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
