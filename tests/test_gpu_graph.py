@@ -51,3 +51,32 @@ def test_recorded_product_full_ring():
     from efla_amd import hellm
     H = hellm.HEMMer(preset=True, seed=3)
     run(H, 128, 4, 3)
+
+
+def test_two_contexts_replay_side_by_side():
+    """Two HEMMers of one process (same seed, so the same keys; nothing is shared between their contexts) replay their
+    recorded products at the same time on their own streams: each replay gives the residues of its eager product."""
+    load_package()
+    from efla_amd import hellm
+    qs, ps = O.ckks_chain(10, 8, 3)
+    rng = np.random.default_rng(9)
+    lanes = []
+    for k in range(2):
+        H = hellm.HEMMer(10, qs, ps, dnum=3, min_bootstrap_level=0, seed=7)
+        a, b = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+        ca, cb = H.encrypt(a), H.encrypt(b)
+        want = H.single_cc_matmul(ca, cb, 2).residues()
+        H.sync()
+        graph, res = H.record(lambda: H.single_cc_matmul(ca, cb, 2))
+        lanes.append((H, graph, res, want, a @ b, (ca, cb)))
+    assert not np.array_equal(lanes[0][3], lanes[1][3])
+    for _ in range(3):
+        for _, graph, _, _, _, _ in lanes:
+            graph.launch()
+            graph.launch()      # two replays in a row on each stream, the two streams side by side
+        for H, graph, res, want, prod, _ in lanes:
+            graph.sync()
+            assert np.array_equal(res.residues(), want)
+            assert np.abs(H.decrypt(res) - prod).max() < 2.0 ** -12
+    for _, graph, _, _, _, _ in lanes:
+        graph.free()
