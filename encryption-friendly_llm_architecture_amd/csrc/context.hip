@@ -211,6 +211,9 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_fp = (double *)up(fpc.data(), fpc.size() * 8);
     c->d_scratch = nullptr;
     c->scratch_bytes = 0;
+    HEMM_HIP(hipStreamCreateWithFlags(&c->aux, hipStreamNonBlocking));
+    HEMM_HIP(hipEventCreateWithFlags(&c->aux_fork, hipEventDisableTiming));
+    HEMM_HIP(hipEventCreateWithFlags(&c->aux_join, hipEventDisableTiming));
     memset(c->traffic, 0, sizeof(c->traffic));
     memset(c->launches, 0, sizeof(c->launches));
     return c;
@@ -231,5 +234,8 @@ void hemm_context_free(hemm_context *c) {
     hipFree(c->d_fp);
     if (c->d_scratch) hipFree(c->d_scratch);
     for (auto &kv : c->d_desc) (void)hipFree(kv.second);
+    if (c->aux) (void)hipStreamDestroy(c->aux);
+    if (c->aux_fork) (void)hipEventDestroy(c->aux_fork);
+    if (c->aux_join) (void)hipEventDestroy(c->aux_join);
     delete c;
 }

@@ -41,6 +41,10 @@ struct hemm_context {
     // user at a time: the copy into it and the kernel that reads it are ordered on that stream)
     std::vector<std::pair<hipStream_t, void *>> d_desc;
     hipStream_t stream = nullptr;   // what a null stream argument of an entry point means for this context
+    // a second stream (non-blocking, default priority) for the runs of a large transform batch: the odd runs go there,
+    // forked from and joined back into the caller's stream with the two events inside the same call
+    hipStream_t aux = nullptr;
+    hipEvent_t aux_fork = nullptr, aux_join = nullptr;
     // compact evaluation keys: offset of every prime's limb inside a (digit, polynomial) slice and, last entry, the
     // slice size, in units of 2N bytes (a prime below 2^44 takes 6 bytes per residue = 3 units, any other 4)
     std::vector<u32> key_off;

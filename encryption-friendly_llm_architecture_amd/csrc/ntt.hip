@@ -823,13 +823,17 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
 // A transform is two launches, and the second reads what the first wrote.  On a large batch the first launch has
 // pushed its early output out of the 256 MB memory-side cache by the time the second one starts, so batches are cut
 // into runs of whole polynomials of about this many limbs (0.5 MiB each) and the two launches alternate run by run.
-// Measured on 32 x 24 limbs: forward transforms are fastest at 192 limbs per run (60-bit primes 0.52 -> 0.43 ms,
-// primes below 2^44 0.41 -> 0.36 ms), inverse ones at 384 (0.48 -> 0.44 ms, 0.37 -> 0.34 ms).
-static int polys_per_run(int n_limbs, int n_polys, bool inverse) {
+// Measured on 32 x 24 limbs, one stream: forward transforms are fastest at 192 limbs per run (60-bit primes 0.52 ->
+// 0.43 ms, primes below 2^44 0.41 -> 0.36 ms), inverse ones at 384 (0.48 -> 0.44 ms, 0.37 -> 0.34 ms).  A plain batch
+// of several runs (launch_ntt_slots) deals them out over two streams, the caller's and the context's second one:
+// a launch of one run fills the part-empty last round of workgroups of the other's.  Same box, runs of 192 limbs in
+// both directions: forward 0.378 -> 0.350 ms (60-bit) and 0.309 -> 0.278 ms (42-bit), inverse 0.390 -> 0.383 and
+// 0.285 -> 0.278 ms; runs of 96, 128 or 256 limbs on two streams are 1 - 8 % slower than that.
+static int polys_per_run(int n_limbs, int n_polys, bool inverse, bool two_streams = false) {
     // batches of up to 448 limbs (224 MiB: what one chain of the matrix products transforms at once, whose input a
     // producer has just written) are fastest as one run: 480 us for the ModDown of 64 polynomials against 497 us cut
     if (n_limbs * n_polys <= 448) return n_polys;
-    const int limbs = inverse ? 384 : 192;
+    const int limbs = inverse && !two_streams ? 384 : 192;
     int p = limbs / n_limbs;
     if (p < 1) p = 1;
     return p < n_polys ? p : n_polys;
@@ -1002,11 +1006,21 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
     const int lanes = n_limbs * n_polys;
     if (c->logN == 16) {
         const dim3 block(256);
-        const int run = polys_per_run(n_limbs, n_polys, inverse);
-        for (int p0 = 0; p0 < n_polys; p0 += run) {
+        const int run = polys_per_run(n_limbs, n_polys, inverse, c->aux != nullptr);
+        // several runs: the odd ones on the context's second stream, which starts after what the caller's stream holds
+        // so far and is waited for before the call returns to it
+        const bool two = c->aux != nullptr && run < n_polys;
+        const hipStream_t own = s;
+        if (two) {
+            HEMM_HIP(hipEventRecord(c->aux_fork, own));
+            HEMM_HIP(hipStreamWaitEvent(c->aux, c->aux_fork, 0));
+        }
+        int run_index = 0;
+        for (int p0 = 0; p0 < n_polys; p0 += run, run_index++) {
             const int np = n_polys - p0 < run ? n_polys - p0 : run;
             const int ln = n_limbs * np;
             u64 *d = data + (size_t)p0 * poly_stride;
+            s = two && (run_index & 1) ? c->aux : own;
             if (!inverse) {
                 hipLaunchKernelGGL(ntt16_cols_kernel<false>, dim3(16, ln), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                                    c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)nullptr);
@@ -1018,6 +1032,10 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
                 hipLaunchKernelGGL(ntt16_cols_kernel<true>, dim3(16, ln), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                                    c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)final_scale);
             }
+        }
+        if (two) {
+            HEMM_HIP(hipEventRecord(c->aux_join, c->aux));
+            HEMM_HIP(hipStreamWaitEvent(own, c->aux_join, 0));
         }
         return;
     }
