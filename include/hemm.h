@@ -71,7 +71,10 @@ int hemm_sample_error(hemm_context *ctx, uint64_t stream_key, const uint32_t *pr
 
 /* Batched negacyclic NTT (inverse = 0: natural -> bit-reversed order) or INTT (inverse = 1,
  * including 1/N) in place over data[n_polys][n_limbs][N]; limb j uses prime prime_idx[j]
- * (host array).  Every NTT-form operand of HomEvaluator goes through this. */
+ * (host array).  Every NTT-form operand of HomEvaluator goes through this.  At N = 2^16 a batch of more than 448
+ * limbs is cut into runs of 192 limbs that alternate between `stream` and a second stream of the context; the second
+ * stream starts after what `stream` holds so far and `stream` waits for it before the call's work counts as done, so
+ * the call stays ordered on `stream` like any other. */
 int hemm_ntt(hemm_context *ctx, uint64_t *data, const uint32_t *prime_idx, uint32_t n_limbs,
              uint32_t n_polys, int inverse, void *stream);
 
