@@ -333,7 +333,8 @@ class Context:
         return out
 
     def hoisted_terms(self, groups, nq, b_premultiplied=False, compact_keys=False):
-        """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift[, pt, pt_galois]]) -> y [n_out][2][nq+K][N]"""
+        """groups: list of lists of (ext, b, evk, mask or None, galois[, mask_shift[, pt, pt_galois]]) -> y [n_out][2][nq+K][N];
+        evk None: a term without a key switch, mask * P * (b, a) with the a-polynomial [nq][N] as ext."""
         import torch
         flat = [t for g in groups for t in g]
         flag = (lambda i: compact_keys[i]) if isinstance(compact_keys, (list, tuple)) else (lambda i: compact_keys)
@@ -341,7 +342,7 @@ class Context:
         for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
             shift = more[0] if more else 0
             pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
-            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr() if evk is not None else None,
                              mask.data_ptr() if mask is not None else None, gal, shift,
                              pt.data_ptr() if pt is not None else None, pt_gal, int(flag(i)))
         offs = [0]
@@ -361,7 +362,7 @@ class Context:
         for i, (ext, b, evk, mask, gal, *more) in enumerate(flat):
             shift = more[0] if more else 0
             pt, pt_gal = (more[1], more[2]) if len(more) >= 3 else (None, 1)
-            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr(),
+            arr[i] = RotTerm(ext.data_ptr(), b.data_ptr() if b is not None else None, evk.data_ptr() if evk is not None else None,
                              mask.data_ptr() if mask is not None else None, gal, shift,
                              pt.data_ptr() if pt is not None else None, pt_gal, int(flag(i)))
         offs = [0]

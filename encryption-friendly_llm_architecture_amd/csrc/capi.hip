@@ -416,7 +416,10 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
     for (uint32_t o = 0; o < n_out; o++) {
         need(group_offsets[o + 1] >= group_offsets[o], "group offsets must not decrease");
         for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
-            need(terms[t].ext && terms[t].evk, "null pointer in a rotation term");
+            need(terms[t].ext != nullptr, "null pointer in a rotation term");
+            // a term without a key: mask * P * (b, a), the a-polynomial in `ext`; it rotates nothing
+            need(terms[t].evk != nullptr || (terms[t].b != nullptr && terms[t].galois == 1 && terms[t].pt == nullptr),
+                 "a term without a key needs b, the identity automorphism and no plaintext factor");
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
             need(terms[t].mask_shift == 0 || (terms[t].mask && (int)terms[t].mask_shift < ctx->logN),
                  "mask_shift needs a run table and must be below log N");
@@ -427,7 +430,7 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
                        (const u64 *)terms[t].mask, (u32)terms[t].galois, terms[t].mask ? (u32)terms[t].mask_shift : 0u,
                        nullptr, nullptr, nullptr, (const u64 *)terms[t].pt, terms[t].pt ? (u32)terms[t].pt_galois : 1u,
                        (u32)terms[t].flags};
-            if (t + 1 < group_offsets[o + 1] && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
+            if (t + 1 < group_offsets[o + 1] && terms[t].evk && terms[t].mask && terms[t + 1].mask && terms[t].b && terms[t + 1].ext && terms[t + 1].b &&
                 terms[t + 1].evk == terms[t].evk && terms[t + 1].galois == terms[t].galois &&
                 terms[t + 1].mask_shift == terms[t].mask_shift && terms[t + 1].pt == terms[t].pt &&
                 (terms[t].pt == nullptr || terms[t + 1].pt_galois == terms[t].pt_galois)) {
@@ -440,6 +443,15 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
         }
         off.push_back((uint32_t)d.size());
     }
+    // the key layout is a property of the launch: terms without a key follow the others
+    u32 layout = 0;
+    for (const RotDev &t : d)
+        if (t.evk != nullptr) {
+            layout = t.flags;
+            break;
+        }
+    for (RotDev &t : d)
+        if (t.evk == nullptr) t.flags = layout;
 }
 // hoisted sums of a validated, merged term list: short lists travel in the kernel arguments, long ones through the
 // staging region

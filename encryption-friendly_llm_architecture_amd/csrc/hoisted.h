@@ -18,7 +18,8 @@ __device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
 struct RotTermDev {
     const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
     const u64 *b;     // [nq][N] b-polynomial of the source (nullptr: none, single-source terms only)
-    const u64 *evk;   // [dnum][2][nQ+K][N]
+    const u64 *evk;   // [dnum][2][nQ+K][N]; nullptr: a term without a key switch, mask * P * (b, a) on the chain limbs with
+                      // the a-polynomial [nq][N] in `ext` (single-source terms only; its mask needs nq limbs)
     const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
     u32 galois;
     u32 mask_shift;   // s > 0: mask (and mask2) are run tables [E][N >> s], one value per 2^s coefficients
@@ -253,6 +254,9 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
     int pending = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const RotTermDev T = terms[t];
+        // a term without a key lives on the chain limbs: its polynomials and its mask have nq limbs, nothing of it
+        // is read for a special limb
+        if (T.evk == nullptr && j >= nq) continue;
         const u32 np = galois_index(n, T.galois, logN);
         const u32 base = np & ~1u;
         const bool swap = (np & 1u) != 0;
@@ -272,7 +276,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             continue;
         }
         u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
-        for (int d = 0; d < beta; d++) {
+        const bool keyless = T.evk == nullptr;
+        for (int d = 0; d < (keyless ? 0 : beta); d++) {
             ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
             if (swap) {
                 const u64 tmp = x.x;
@@ -311,6 +316,20 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             }
             rb[0] = addmod(rb[0], bv.x, m.q);
             rb[1] = addmod(rb[1], bv.y, m.q);
+        }
+        if (keyless) {   // the a-polynomial enters as it is (times P): no key product above (j < nq here)
+            ulonglong2 av = *(const ulonglong2 *)(T.ext + (size_t)j * N + base);
+            if (swap) {
+                const u64 tmp = av.x;
+                av.x = av.y;
+                av.y = tmp;
+            }
+            if (!b_premultiplied) {
+                av.x = mul_shoup(av.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+                av.y = mul_shoup(av.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            }
+            ra[0] = av.x;
+            ra[1] = av.y;
         }
         if (T.mask != nullptr || T.pt != nullptr) {
             ulonglong2 mk = T.mask != nullptr ? load_mask2(T.mask, T.mask_shift, j, n, logN) : make_ulonglong2(1, 1);
@@ -398,6 +417,7 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
     int since = 0;
     for (u32 t = group_off[o]; t < group_off[o + 1]; t++) {
         const RotTermDev T = terms[t];
+        if (T.evk == nullptr && j >= nq) continue;   // a term without a key: chain limbs only, mask included
         const __amdgpu_buffer_rsrc_t kr = key_rsrc(T);
         const u32 np = galois_index(n, T.galois, logN);
         const u32 base = np & ~1u;
@@ -438,7 +458,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 sb1 += f.mul(m1.y, b1.y) + f.mul(m2.y, b2.y);
             }
         } else {
-            for (int d = 0; d < beta; d++) {
+            const bool keyless = T.evk == nullptr;
+            for (int d = 0; d < (keyless ? 0 : beta); d++) {
                 const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
                 const D2 kb = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 0, prime, logN, n_full), n);
                 const D2 ka = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 1, prime, logN, n_full), n);
@@ -455,6 +476,15 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
                 }
                 sb0 += bv.x;
                 sb1 += bv.y;
+            }
+            if (keyless) {   // the a-polynomial enters as it is (times P); j < nq here
+                D2 av = gather_d2(T.ext + (size_t)j * N + base, swap);
+                if (!b_premultiplied) {
+                    av.x = f.mul(av.x, p_mod_q);
+                    av.y = f.mul(av.y, p_mod_q);
+                }
+                sa0 = av.x;
+                sa1 = av.y;
             }
             if (T.mask != nullptr) {
                 const D2 mk = to_d2(load_mask2(T.mask, T.mask_shift, j, n, logN));

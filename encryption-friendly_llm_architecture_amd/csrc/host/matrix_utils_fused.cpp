@@ -107,6 +107,18 @@ hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois
     return t;
 }
 
+// mask * P * (b, a) of the ciphertext at ct (polynomial stride given), on the chain limbs: a term of a hoisted sum that
+// needs no key switch (the launch must not take its b polynomials as premultiplied)
+hemm_rot_term keylessTerm(const u64 *ct, u64 poly_stride, const Plaintext &mask) {
+    hemm_rot_term t{};
+    t.ext = ct + poly_stride;
+    t.b = ct;
+    t.evk = nullptr;
+    t.mask = mask.buf_.data();
+    t.galois = 1;
+    return t;
+}
+
 }  // namespace
 
 const Plaintext &MatrixTransformer::firstBlockMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level) {
@@ -570,34 +582,20 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         //   main_r * rho^(r step)(X) + wrap_r * rho^(r step - tile side)(X):
         // two Galois elements per r with one key each; when they coincide (the tile side is a whole turn of the slot
         // vector) one term with the mask of both parts.
-        // unrotated rows: mask, rescale.  They need only the input, so this chain of small launches runs on the side
-        // stream beside the rotations (its masks are looked up, and on first use encoded, before the fork).
-        std::vector<hemm_lin_term> zero_terms;
-        std::vector<uint32_t> zoff{0};
+        // The rows that stay, mask_0 * X, need no key switch: they join the same sum as a term without a key
+        // (mask_0 * P * (b, a) on the chain limbs) and share its ModDown and rescale.
+        bool any_rotation = false;
         for (size_t q = 0; q < n_jobs; q++) {
-            hemm_lin_term t;
-            t.ct = src + q * ctw;
-            t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
-            t.stride = nq * N;
-            t.galois = 0;
-            zero_terms.push_back(t);
-            zoff.push_back((uint32_t)zero_terms.size());
+            const Geo g = geo(kinds[q], shapes[q]);
+            const i64 b = twoStageSplit(g.units);
+            any_rotation = any_rotation || (stage == 1 ? b : g.units / b) > 1;
         }
-        DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
-        const hipStream_t side = c->forkSide();
-        struct JoinOnExit {
-            const Context &c;
-            ~JoinOnExit() { c->joinSide(); }
-        } join_on_exit{c};
-        ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
-        ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
-        const Sources x = extendSources(c, src, n_jobs, nq, nullptr, false);
+        const Sources x = any_rotation ? extendSources(c, src, n_jobs, nq, nullptr, false) : Sources{};
         const KeyPack &pack = eval.getKeyPack();
         const Rot rot(c);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
-        bool any_rotation = false;
-        for (size_t q = 0; q < n_jobs; q++) {
+        for (size_t q = 0; any_rotation && q < n_jobs; q++) {
             const Geo g = geo(kinds[q], shapes[q]);
             const bool vertical = (kinds[q] == MaskKind::Vertical || kinds[q] == MaskKind::PackedVertical);
             const i64 wrap = g.n * (vertical ? shapes[q].getBlockWidth() : 1);
@@ -613,23 +611,32 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                     terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount - wrap),
                                          &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)));
                 }
-                any_rotation = true;
             }
+            terms.push_back(keylessTerm(src + q * ctw, nq * N, twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0)));
             off.push_back((uint32_t)terms.size());
         }
         if (any_rotation) {
             for (size_t q = 0; q + 1 < off.size(); q++)
-                if (off[q + 1] == off[q])
+                if (off[q + 1] == off[q] + 1)
                     throw RuntimeException("diagonalTransformTwoStage: jobs with and without rotations cannot share a batch");
             DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
             ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, x.premultiplied(), 1,
                                     y.data(), dst, (nq - 1) * N, ws.data(), nullptr));
-            c->joinSide();
-            ck(hemm_pointwise(c->dev, HEMM_ADD, dst, (nq - 1) * N, zres.data(), (nq - 1) * N, dst, (nq - 1) * N,
-                              (uint32_t)(nq - 1), 0, (uint32_t)(2 * n_jobs), nullptr));
-        } else {
-            c->joinSide();
-            (void)hipMemcpyAsync(dst, zres.data(), n_jobs * 2 * (nq - 1) * N * 8, hipMemcpyDeviceToDevice, c->stream());
+        } else {   // no rotation in this stage: mask and rescale
+            std::vector<hemm_lin_term> zero_terms;
+            std::vector<uint32_t> zoff{0};
+            for (size_t q = 0; q < n_jobs; q++) {
+                hemm_lin_term t;
+                t.ct = src + q * ctw;
+                t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
+                t.stride = nq * N;
+                t.galois = 0;
+                zero_terms.push_back(t);
+                zoff.push_back((uint32_t)zero_terms.size());
+            }
+            DeviceBuffer zsum(c, n_jobs * ctw);
+            ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), nullptr));
+            ck(hemm_rescale(c->dev, zsum.data(), nq * N, dst, (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
         }
         c->mark(stage == 1 ? "transform stage 1" : "transform stage 2");
     }
@@ -638,8 +645,8 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
 // The complex packing as a linear map on the slots, out = Z x + M_+ rho^(step)(x) + M_- rho^(-step)(x):
 //   columns (step 1):  fus = m (x + i rho^1 x), out = fus + rho^-1 fus, m = even columns
 //   rows (step w):     fus = m (x - i rho^w x), out = fus + rho^-w fus, m = even rows of width w
-// i.e. Z = m +- i m', M_+ = +- i m, M_- = m' with m'[s] = m[s - step].  One hoisted sum with two terms per job plus
-// rescale(Z x) on the side stream.
+// i.e. Z = m +- i m', M_+ = +- i m, M_- = m' with m'[s] = m[s - step].  One hoisted sum with three terms per job: the two
+// rotations and Z x, which needs no key switch (a term without a key).
 void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
                                             const bool *rows, i64 w, u64 *out, const u64 *scale_levels) {
     const Context &c = eval.getContext();
@@ -658,28 +665,8 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
         return pack_masks_.emplace(key, endec.encodeExtended(m, level, scale)).first->second;
     };
     auto from_of = [&](size_t q) { return scale_levels ? scale_levels[q] : level; };
-    std::vector<hemm_lin_term> zero_terms;
-    std::vector<uint32_t> zoff{0};
-    for (size_t q = 0; q < n_jobs; q++) {
-        hemm_lin_term t;
-        t.ct = in + q * ctw;
+    for (size_t q = 0; q < n_jobs; q++)
         if (from_of(q) < level) throw std::invalid_argument("[complexPacking] the scale must come from the same or a higher level.");
-        t.mask = mask(rows[q], 0, from_of(q)).buf_.data();
-        t.stride = nq * N;
-        t.galois = 0;
-        zero_terms.push_back(t);
-        zoff.push_back((uint32_t)zero_terms.size());
-        (void)mask(rows[q], 1, from_of(q));    // encoded before the fork below
-        (void)mask(rows[q], 2, from_of(q));
-    }
-    DeviceBuffer zsum(c, n_jobs * ctw), zres(c, n_jobs * 2 * (nq - 1) * N);
-    const hipStream_t side = c->forkSide();
-    struct JoinOnExit {
-        const Context &c;
-        ~JoinOnExit() { c->joinSide(); }
-    } join_on_exit{c};
-    ck(hemm_masked_sum_batch(c->dev, zero_terms.data(), zoff.data(), (uint32_t)n_jobs, (uint32_t)nq, 2, zsum.data(), side));
-    ck(hemm_rescale(c->dev, zsum.data(), nq * N, zres.data(), (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), side));
     const Sources x = extendSources(c, in, n_jobs, nq, nullptr, false);
     const KeyPack &pack = eval.getKeyPack();
     const Rot rot(c);
@@ -689,14 +676,12 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
         const i64 step = rows[q] ? w : 1;
         terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(step), &mask(rows[q], 1, from_of(q))));
         terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(-step), &mask(rows[q], 2, from_of(q))));
+        terms.push_back(keylessTerm(in + q * ctw, nq * N, mask(rows[q], 0, from_of(q))));   // Z x needs no key switch
         off.push_back((uint32_t)terms.size());
     }
     DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
     ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, x.premultiplied(), 1, y.data(),
                             out, (nq - 1) * N, ws.data(), nullptr));
-    c->joinSide();
-    ck(hemm_pointwise(c->dev, HEMM_ADD, out, (nq - 1) * N, zres.data(), (nq - 1) * N, out, (nq - 1) * N, (uint32_t)(nq - 1), 0,
-                      (uint32_t)(2 * n_jobs), nullptr));
 }
 
 namespace {

@@ -1199,8 +1199,12 @@ static size_t hoisted_bytes(const hemm_context *c, const RotTermDev *t, int n_te
         compact_slice += (size_t)c->N * ((c->primes[prime] >> 44) == 0 ? 6 : 8);
     }
     for (int i = 0; i < n_terms; i++) {
-        bytes += (size_t)2 * beta * ((t[i].flags & ROT_TERM_COMPACT_KEY) ? compact_slice : (size_t)E * limb);   // the key
-        if (first(t[i].ext)) bytes += (size_t)beta * E * limb;
+        if (t[i].evk == nullptr) {   // no key: the two polynomials on the chain limbs
+            if (first(t[i].ext)) bytes += (size_t)nq * limb;
+        } else {
+            bytes += (size_t)2 * beta * ((t[i].flags & ROT_TERM_COMPACT_KEY) ? compact_slice : (size_t)E * limb);   // the key
+            if (first(t[i].ext)) bytes += (size_t)beta * E * limb;
+        }
         if (first(t[i].b)) bytes += (size_t)nq * limb;
         if (first(t[i].ext2)) bytes += (size_t)beta * E * limb;
         if (first(t[i].b2)) bytes += (size_t)nq * limb;

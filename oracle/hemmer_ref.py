@@ -713,8 +713,8 @@ def two_stage_mask(kind, n, w, slots, stage, r, part):
 def diagonal_transform_two_stage(orc, ct, kind, n, w):
     """sigma / tau (square tiles) in two stages of one mask level each: row i is rotated by i mod b, then
     by b (i div b).  Every stage is one hoisted sum over its rotations of
-    main_r rho^(r)(X) + wrap_r rho^(r - tile side)(X) (two keys per r, one source) with ModDown merged with
-    the rescale, plus rescale(mask_0 X) for the rows that stay.  Level L -> L - 2."""
+    main_r rho^(r)(X) + wrap_r rho^(r - tile side)(X) (two keys per r, one source) and of mask_0 X for the rows that
+    stay (a term without a key switch), with ModDown merged with the rescale.  Level L -> L - 2."""
     from .oracle import Ct
     cell = 2 if kind in (PH, PV) else 1
     u = n // cell
@@ -724,10 +724,12 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
     x = ct
     for stage, count, mul in ((1, b, 1), (2, u // b, b)):
         nq = x.nq
-        ext = orc.modup(x.data[1])
-        zero = orc.rescale(orc.mult_plain_no_rescale(
-            x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), x.level)))
         mask = lambda r, part: orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, part), x.level)
+        if count <= 1:      # no rotation in this stage: mask and rescale
+            x = orc.rescale(orc.mult_plain_no_rescale(
+                x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), x.level)))
+            continue
+        ext = orc.modup(x.data[1])
         terms = []
         for r in range(1, count):
             r_main, r_wrap = (r * mul * step) % orc.slots, (r * mul * step - wrap) % orc.slots
@@ -736,11 +738,9 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
             else:
                 terms.append((ext, x.data[0], r_main, mask(r, 1)))
                 terms.append((ext, x.data[0], r_wrap, mask(r, 2)))
-        if terms:
-            y = orc.hoisted_sum(terms, nq)
-            x = orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
-        else:
-            x = zero
+        terms.append((x.data[1], x.data[0], ("none",), mask(0, 0)))
+        y = orc.hoisted_sum(terms, nq)
+        x = Ct(orc.moddown_drop(y, nq, True), x.scale * orc.delta[x.level] / float(orc.q[x.level]))
     return x
 
 
@@ -920,9 +920,9 @@ def packing_maps(slots, w, rows):
 
 
 def complex_packing_hoisted(orc, x, w, rows):
-    """complexPackingInplace / complexPackingRowInplace as ONE hoisted sum (both rotations from one ModUp, masks
-    applied in the extended basis, ModDown merged with the rescale) plus rescale(Z x): one level, like the
-    reference's two masked steps.  x may be a truncated ciphertext that still carries the scale of a higher level:
+    """complexPackingInplace / complexPackingRowInplace as ONE hoisted sum (both rotations from one ModUp and Z x as a
+    term without a key switch, masks applied in the extended basis, ModDown merged with the rescale): one level, like
+    the reference's two masked steps.  x may be a truncated ciphertext that still carries the scale of a higher level:
     the masks are then encoded at Delta_(l-1) q_l / scale(x) instead of Delta_l, so that the result has the fixed
     scale of level l - 1 without a levelDown in front."""
     from .oracle import Ct
@@ -930,10 +930,9 @@ def complex_packing_hoisted(orc, x, w, rows):
     nq, lvl = x.nq, x.level
     ms = orc.delta[lvl] if x.scale == orc.delta[lvl] else orc.delta[lvl - 1] * float(orc.q[lvl]) / x.scale
     ext = orc.modup(x.data[1])
-    zero = orc.rescale(orc.mult_plain_no_rescale(x, orc.encode(zmask, lvl, ms)))
-    y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, lvl, ms)) for r, m in terms], nq)
-    zero.scale = orc.delta[lvl - 1]
-    return orc.add(Ct(orc.moddown_drop(y, nq, True), zero.scale), zero)
+    y = orc.hoisted_sum([(ext, x.data[0], r % orc.slots, orc.encode_ext(m, lvl, ms)) for r, m in terms] +
+                        [(x.data[1], x.data[0], ("none",), orc.encode_ext(zmask, lvl, ms))], nq)
+    return Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
 
 
 def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):

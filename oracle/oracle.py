@@ -665,9 +665,12 @@ class Oracle:
 
     def hoisted_sum(self, terms, nq):
         """terms: (ext, b or None, rotation r (left, in slots) or ('g', galois) or ('sq', galois): the key of
-        rho_g(s)^2, or ('mult', 1): the multiplication key without rotation, mask Pt over the extended basis or None).
+        rho_g(s)^2, or ('mult', 1): the multiplication key without rotation, or ('none',): no key switch at all, ext
+        being the a-polynomial on the chain limbs; mask Pt over the extended basis or None).
         Returns y[2][nq+K][N] = sum mask * (<galois(ext), evk> + P galois(b))."""
         y = np.zeros((2, nq + self.nP, self.N), dtype=np.uint64)
+        keyless = [t for t in terms if isinstance(t[2], tuple) and t[2][0] == "none"]
+        terms = [t for t in terms if not (isinstance(t[2], tuple) and t[2][0] == "none")]
         for i, (ext, b, rot, mask) in enumerate(terms):
             g = rot[1] if isinstance(rot, tuple) else self.galois(rot)
             if isinstance(rot, tuple) and rot[0] == "sq":
@@ -680,6 +683,14 @@ class Oracle:
             bp = _p(np.ascontiguousarray(b)) if b is not None else None
             self.L.orc_hoisted_term(self.h, _p(np.ascontiguousarray(ext)), bp,
                                     _p(evk), mk, g, nq, _p(y), int(i > 0))
+        # ('none',): a term without a key switch -- ext is the a-polynomial [nq][N] itself and the term is
+        # mask * P * (b, a) on the chain limbs (exact residue arithmetic: where it joins the sum does not matter)
+        for a, b, _, mask in keyless:
+            for pol, src in ((0, b), (1, a)):
+                t = self.mul_p_residues(np.ascontiguousarray(src[:nq]))
+                if mask is not None:
+                    t = self._binary(2, t, np.ascontiguousarray(mask.data[:nq]))
+                y[pol, :nq] = self.add_residues(np.ascontiguousarray(y[pol, :nq]), t)
         return y
 
     def moddown_drop(self, y, nq, drop_last):

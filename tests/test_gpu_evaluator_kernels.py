@@ -425,6 +425,54 @@ def test_hoisted_terms_with_rotated_plaintext_factor(S):
         assert np.array_equal(y[k], want[k]), k
 
 
+def test_hoisted_terms_without_a_key(S):
+    """A term with no key is mask * P * (b, a) on the chain limbs and nothing on the special limbs (the part of a masked
+    sum that is not rotated joins the rotated parts before their common ModDown): alone, behind keyed terms of a
+    group (plain and compact keys, argument and staged lists), and through the ModDown merged with the rescale."""
+    import torch
+    orc, ctx, N = S.orc, S.ctx, S.N
+    rng = np.random.default_rng(79)
+    nq = orc.nQ - 1
+    orc.key_seed = 6
+    ct = rand_limbs(rng, orc.q[:nq], (2,), N)
+    dct = dev(ct)
+    ext = orc.modup(ct[1])
+    dext = ctx.modup_batch(dct[1:2].contiguous(), nq)[0]
+    masks = [orc.encode_ext(rng.uniform(-1, 1, orc.slots), nq - 1) for _ in range(3)]
+    dmasks = [dev(m.data) for m in masks]
+    g1, g2 = orc.galois(3), orc.galois(orc.slots - 7)
+    keys = {g: orc.galois_key(g) for g in (g1, g2)}
+    dk = {g: dev(keys[g]) for g in keys}
+    none = ("none",)
+    want = [orc.hoisted_sum([(ct[1], ct[0], none, masks[0])], nq),
+            orc.hoisted_sum([(ext, ct[0], ("g", g1), masks[1]), (ext, ct[0], ("g", g2), masks[2]),
+                             (ct[1], ct[0], none, masks[0])], nq),
+            orc.hoisted_sum([(ct[1], ct[0], none, None), (ext, ct[0], ("g", g1), None)], nq)]
+    assert not want[0][:, nq:].any() and want[0][:, :nq].any()
+    chain_mask = dev(np.ascontiguousarray(masks[0].data[:nq]))       # a term without a key reads nq limbs of its mask
+    groups = [[(dct[1], dct[0], None, chain_mask, 1)],
+              [(dext, dct[0], dk[g1], dmasks[1], g1), (dext, dct[0], dk[g2], dmasks[2], g2), (dct[1], dct[0], None, chain_mask, 1)],
+              [(dct[1], dct[0], None, None, 1), (dext, dct[0], dk[g1], None, g1)]]
+    y = host(ctx.hoisted_terms(groups, nq))
+    for k in range(3):
+        assert np.array_equal(y[k], want[k]), k
+    # compact keys; a list too long for the kernel arguments (staged); the merged ModDown + rescale behind the sum
+    ck = {g: ctx.compact_key(dk[g]) for g in dk}
+    groups_c = [[(dext, dct[0], ck[g1], dmasks[1], g1), (dext, dct[0], ck[g2], dmasks[2], g2), (dct[1], dct[0], None, dmasks[0], 1)]]
+    assert np.array_equal(host(ctx.hoisted_terms(groups_c, nq, compact_keys=True))[0], want[1])
+    long_group = [(dext, dct[0], dk[g1], dmasks[1], g1), (dext, dct[0], dk[g2], dmasks[2], g2)] * 20 + [(dct[1], dct[0], None, dmasks[0], 1)]
+    long_want = orc.hoisted_sum([(ext, ct[0], ("g", g1), masks[1]), (ext, ct[0], ("g", g2), masks[2])] * 20 +
+                                [(ct[1], ct[0], none, masks[0])], nq)
+    assert np.array_equal(host(ctx.hoisted_terms([long_group], nq))[0], long_want)
+    got = host(ctx.hoisted_moddown(groups[1:2], nq, True))[0]
+    assert np.array_equal(got, orc.moddown_drop(want[1], nq, True))
+    # what a term without a key may not carry
+    with pytest.raises(ValueError, match="without a key"):
+        ctx.hoisted_terms([[(dct[1], dct[0], None, dmasks[0], g1)]], nq)
+    with pytest.raises(ValueError, match="without a key"):
+        ctx.hoisted_terms([[(dct[1], None, None, dmasks[0], 1)]], nq)
+
+
 def test_rotation_24_limb_chain_of_60_bit_primes():
     """One key-switched rotation at the shape of the reference's rotation benchmark: N = 2^16, a chain of 24
     60-bit primes + 4 special primes, dnum = 3 (digits of 8 limbs), ciphertext at level 20, steps from the
