@@ -417,9 +417,8 @@ static void build_rot_terms(hemm_context *ctx, const hemm_rot_term *terms, const
         need(group_offsets[o + 1] >= group_offsets[o], "group offsets must not decrease");
         for (uint32_t t = group_offsets[o]; t < group_offsets[o + 1]; t++) {
             need(terms[t].ext != nullptr, "null pointer in a rotation term");
-            // a term without a key: mask * P * (b, a), the a-polynomial in `ext`; it rotates nothing
-            need(terms[t].evk != nullptr || (terms[t].b != nullptr && terms[t].galois == 1 && terms[t].pt == nullptr),
-                 "a term without a key needs b, the identity automorphism and no plaintext factor");
+            // a term without a key: mask * pt * P * (b, a), the a-polynomial in `ext`; it rotates nothing
+            need(terms[t].evk != nullptr || terms[t].galois == 1, "a term without a key takes the identity automorphism");
             need((terms[t].galois & 1) && terms[t].galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
             need(terms[t].mask_shift == 0 || (terms[t].mask && (int)terms[t].mask_shift < ctx->logN),
                  "mask_shift needs a run table and must be below log N");

@@ -18,8 +18,9 @@ __device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
 struct RotTermDev {
     const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
     const u64 *b;     // [nq][N] b-polynomial of the source (nullptr: none, single-source terms only)
-    const u64 *evk;   // [dnum][2][nQ+K][N]; nullptr: a term without a key switch, mask * P * (b, a) on the chain limbs with
-                      // the a-polynomial [nq][N] in `ext` (single-source terms only; its mask needs nq limbs)
+    const u64 *evk;   // [dnum][2][nQ+K][N]; nullptr: a term without a key switch, mask * pt * P * (b, a) on the chain
+                      // limbs with the a-polynomial [nq][N] in `ext`, always as it is (b may be premultiplied like any
+                      // other b, or absent); single-source terms only; its mask needs nq limbs
     const u64 *mask;  // [E][N] plaintext over the extended basis, or nullptr
     u32 galois;
     u32 mask_shift;   // s > 0: mask (and mask2) are run tables [E][N >> s], one value per 2^s coefficients
@@ -324,10 +325,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                 av.x = av.y;
                 av.y = tmp;
             }
-            if (!b_premultiplied) {
-                av.x = mul_shoup(av.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                av.y = mul_shoup(av.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-            }
+            av.x = mul_shoup(av.x, pmod.c[j].w, pmod.c[j].ws, m.q);   // never premultiplied, whatever b is
+            av.y = mul_shoup(av.y, pmod.c[j].w, pmod.c[j].ws, m.q);
             ra[0] = av.x;
             ra[1] = av.y;
         }
@@ -479,10 +478,8 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
             }
             if (keyless) {   // the a-polynomial enters as it is (times P); j < nq here
                 D2 av = gather_d2(T.ext + (size_t)j * N + base, swap);
-                if (!b_premultiplied) {
-                    av.x = f.mul(av.x, p_mod_q);
-                    av.y = f.mul(av.y, p_mod_q);
-                }
+                av.x = f.mul(av.x, p_mod_q);   // never premultiplied, whatever b is
+                av.y = f.mul(av.y, p_mod_q);
                 sa0 = av.x;
                 sa1 = av.y;
             }

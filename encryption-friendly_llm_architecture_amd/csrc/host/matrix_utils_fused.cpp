@@ -107,15 +107,22 @@ hemm_rot_term term(const u64 *ext, const u64 *b, const KeyPack &pack, u64 galois
     return t;
 }
 
-// mask * P * (b, a) of the ciphertext at ct (polynomial stride given), on the chain limbs: a term of a hoisted sum that
-// needs no key switch (the launch must not take its b polynomials as premultiplied)
-hemm_rot_term keylessTerm(const u64 *ct, u64 poly_stride, const Plaintext &mask) {
+// mask * P * (b, a) on the chain limbs: a term of a hoisted sum that needs no key switch.  a is always given as it is;
+// b as the launch takes every b (premultiplied or not), or nullptr
+hemm_rot_term keylessTerm(const u64 *b, const u64 *a, const Plaintext *mask) {
     hemm_rot_term t{};
-    t.ext = ct + poly_stride;
-    t.b = ct;
+    t.ext = a;
+    t.b = b;
     t.evk = nullptr;
-    t.mask = mask.buf_.data();
     t.galois = 1;
+    t.pt_galois = 1;
+    if (mask) {
+        t.mask = mask->buf_.data();
+        if (mask->compact_shift_ != 0) {
+            t.mask = mask->compact_.data();
+            t.mask_shift = mask->compact_shift_;
+        }
+    }
     return t;
 }
 
@@ -612,7 +619,7 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                                          &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)));
                 }
             }
-            terms.push_back(keylessTerm(src + q * ctw, nq * N, twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0)));
+            terms.push_back(keylessTerm(src + q * ctw, src + q * ctw + nq * N, &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0)));
             off.push_back((uint32_t)terms.size());
         }
         if (any_rotation) {
@@ -676,7 +683,7 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
         const i64 step = rows[q] ? w : 1;
         terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(step), &mask(rows[q], 1, from_of(q))));
         terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(-step), &mask(rows[q], 2, from_of(q))));
-        terms.push_back(keylessTerm(in + q * ctw, nq * N, mask(rows[q], 0, from_of(q))));   // Z x needs no key switch
+        terms.push_back(keylessTerm(in + q * ctw, in + q * ctw + nq * N, &mask(rows[q], 0, from_of(q))));   // Z x: no key switch
         off.push_back((uint32_t)terms.size());
     }
     DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
@@ -874,9 +881,9 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     ck(hemm_modup_batch(c->dev, U.data() + us, pw, (uint32_t)lo, (uint32_t)(2 * m), ext.data(), wsu.data(), nullptr));
     const u64 *ext1 = ext.data(), *ext2 = ext.data() + m * beta * El * N;   // [i2][beta][El][N] each
     // d0 of every partial sum enters its term as it is (the launch multiplies by P); d1 of U_0, which needs no key
-    // switch, is added after the ModDown: (y + P d1 - conv) / P = (y - conv) / P + d1 on every chain limb, and P d1
-    // vanishes on the special limbs the conversion reads
+    // switch, joins the second polynomial as a term without a key (P d1 on the chain limbs)
     std::vector<hemm_rot_term> terms;
+    terms.push_back(keylessTerm(nullptr, U.data() + us, nullptr));
     {
         hemm_rot_term t{};
         t.ext = ext2;
@@ -922,8 +929,6 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     DeviceBuffer yg(c, 2 * El * N), wsg(c, 2 * lo * N);
     ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 0, nullptr));
     ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 0, res.get().buf_.data(), lo * N, wsg.data(), nullptr));
-    u64 *res1 = res.get().buf_.data() + lo * N;
-    ck(hemm_pointwise(c->dev, HEMM_ADD, res1, 0, U.data() + us, 0, res1, 0, (uint32_t)lo, 0, 1, nullptr));
 }
 }  // namespace
 
@@ -1494,6 +1499,11 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
                 terms.push_back(t1);
                 terms.push_back(t2);
             }
+            if (p == 0) {   // shift 0 needs no key switch: P (mask_0 tau(B)) sigma(A) on the chain limbs
+                hemm_rot_term t0 = keylessTerm(x.pbOf(0), sa.buf_.data() + nq * N, &cm[1]);
+                t0.pt = tau.buf_.data();
+                terms.push_back(t0);
+            }
             off.push_back((uint32_t)terms.size());
         }
         DeviceBuffer yp(c, parts * 2 * E * N);
@@ -1501,9 +1511,7 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
         ck(hemm_sum_parts(c->dev, yp.data(), (uint32_t)parts, 1, (uint32_t)nq, y.data(), nullptr));
     } else {
         ck(hemm_zero(c->dev, y.data(), 2 * E * N, nullptr));
-    }
-    // ---- shift 0: P (mask_0 tau(B)) sigma(A) on the chain limbs
-    {
+        // ---- no shift at all: P (mask_0 tau(B)) sigma(A) on the chain limbs
         DeviceBuffer m0(c, nq * N), t0(c, 2 * nq * N);
         ck(hemm_pointwise(c->dev, HEMM_MUL, cm[1].buf_.data(), 0, tau.buf_.data(), 0, m0.data(), 0, (uint32_t)nq, 0, 1, nullptr));
         ck(hemm_pointwise(c->dev, HEMM_MUL, sa.buf_.data(), nq * N, m0.data(), 0, t0.data(), nq * N, (uint32_t)nq, 0, 2, nullptr));

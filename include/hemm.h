@@ -162,10 +162,10 @@ typedef struct {
     const uint64_t *ext;  /* [beta][nq+n_p][N] */
     const uint64_t *b;    /* [nq][N], or NULL: the term contributes only the key product (used for the
                            * degree-2 component of a tensor product, with a key for the rotated s^2) */
-    const uint64_t *evk;  /* [dnum][2][n_q+n_p][N], or NULL: a term that needs no key switch, mask * P * (b, a) on the chain
-                           * limbs with the a-polynomial [nq][N] in `ext` (galois = 1, b set, no pt; of its mask only the
-                           * nq chain limbs are read): the unrotated part of a masked sum joins its rotated parts before
-                           * their common ModDown */
+    const uint64_t *evk;  /* [dnum][2][n_q+n_p][N], or NULL: a term that needs no key switch, mask * pt * P * (b, a) on the
+                           * chain limbs with the a-polynomial [nq][N] in `ext` (always as it is, also where b is
+                           * premultiplied; b may be NULL; galois = 1; of its mask only the nq chain limbs are read): the
+                           * unrotated part of a masked sum joins its rotated parts before their common ModDown */
     const uint64_t *mask; /* [nq+n_p][N] or NULL; with mask_shift = s > 0 a run table [nq+n_p][N >> s][2] */
     uint32_t galois;
     uint32_t mask_shift;  /* 0: full mask.  s >= 1: the mask is constant over aligned runs of 2^s coefficients

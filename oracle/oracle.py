@@ -687,6 +687,8 @@ class Oracle:
         # mask * P * (b, a) on the chain limbs (exact residue arithmetic: where it joins the sum does not matter)
         for a, b, _, mask in keyless:
             for pol, src in ((0, b), (1, a)):
+                if src is None:
+                    continue
                 t = self.mul_p_residues(np.ascontiguousarray(src[:nq]))
                 if mask is not None:
                     t = self._binary(2, t, np.ascontiguousarray(mask.data[:nq]))

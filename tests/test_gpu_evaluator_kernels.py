@@ -426,7 +426,7 @@ def test_hoisted_terms_with_rotated_plaintext_factor(S):
 
 
 def test_hoisted_terms_without_a_key(S):
-    """A term with no key is mask * P * (b, a) on the chain limbs and nothing on the special limbs (the part of a masked
+    """A term with no key is mask * pt * P * (b, a) on the chain limbs and nothing on the special limbs (the part of a masked
     sum that is not rotated joins the rotated parts before their common ModDown): alone, behind keyed terms of a
     group (plain and compact keys, argument and staged lists), and through the ModDown merged with the rescale."""
     import torch
@@ -444,6 +444,8 @@ def test_hoisted_terms_without_a_key(S):
     keys = {g: orc.galois_key(g) for g in (g1, g2)}
     dk = {g: dev(keys[g]) for g in keys}
     none = ("none",)
+    weight = orc.encode_ext(rng.uniform(-1, 1, orc.slots), nq - 1)
+    dweight = dev(weight.data)
     want = [orc.hoisted_sum([(ct[1], ct[0], none, masks[0])], nq),
             orc.hoisted_sum([(ext, ct[0], ("g", g1), masks[1]), (ext, ct[0], ("g", g2), masks[2]),
                              (ct[1], ct[0], none, masks[0])], nq),
@@ -456,6 +458,14 @@ def test_hoisted_terms_without_a_key(S):
     y = host(ctx.hoisted_terms(groups, nq))
     for k in range(3):
         assert np.array_equal(y[k], want[k]), k
+    # without b (only the second polynomial receives P a); with a plaintext factor; with b premultiplied by the caller
+    # (a is always taken as it is)
+    pb = dev(orc.mul_p_residues(np.ascontiguousarray(ct[0])))
+    got = host(ctx.hoisted_terms([[(dct[1], None, None, None, 1)], [(dct[1], dct[0], None, dmasks[0], 1, 0, dweight, 1)]], nq))
+    assert np.array_equal(got[0], orc.hoisted_sum([(ct[1], None, none, None)], nq)) and not got[0][0].any()
+    assert np.array_equal(got[1], orc.hoisted_sum([(ct[1], ct[0], none, orc.ext_plain_product(masks[0], weight, 1))], nq))
+    got = host(ctx.hoisted_terms([[(dct[1], pb, None, chain_mask, 1)]], nq, b_premultiplied=True))
+    assert np.array_equal(got[0], want[0])
     # compact keys; a list too long for the kernel arguments (staged); the merged ModDown + rescale behind the sum
     ck = {g: ctx.compact_key(dk[g]) for g in dk}
     groups_c = [[(dext, dct[0], ck[g1], dmasks[1], g1), (dext, dct[0], ck[g2], dmasks[2], g2), (dct[1], dct[0], None, dmasks[0], 1)]]
@@ -469,8 +479,6 @@ def test_hoisted_terms_without_a_key(S):
     # what a term without a key may not carry
     with pytest.raises(ValueError, match="without a key"):
         ctx.hoisted_terms([[(dct[1], dct[0], None, dmasks[0], g1)]], nq)
-    with pytest.raises(ValueError, match="without a key"):
-        ctx.hoisted_terms([[(dct[1], None, None, dmasks[0], 1)]], nq)
 
 
 def test_rotation_24_limb_chain_of_60_bit_primes():
