@@ -235,7 +235,8 @@ std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, boo
 //   1 ModUp of A, all bs baby rotations as hoisted terms in one launch + one batched ModDown;
 //   one masked-sum launch for every (giant index, sign) group;
 //   1 batched ModUp of the group sums, every giant rotation as a hoisted term of ONE output, so the
-//   groups are summed in the extended basis and share a single ModDown; one rescale at the end.
+//   groups are summed in the extended basis together with the group that is not rotated (a term without a key) and
+//   share a single ModDown merged with the rescale.
 // Several transforms of operands at the same level (sigma(A) and tau(B) of one product) go through the
 // same launches: `in` holds n_jobs ciphertexts [job][2][nq][N], `out` receives [job][2][nq-1][N].
 void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
@@ -337,8 +338,8 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
     DeviceBuffer sums(c, n_groups * ctw);
     ck(hemm_masked_sum_batch(c->dev, lt.data(), loff.data(), (uint32_t)n_groups, (uint32_t)nq, 2, sums.data(), nullptr));
 
-    // 3. giant steps: every rotated group is a term of its job's output
-    DeviceBuffer res(c, n_jobs * ctw);
+    // 3. giant steps: every rotated group is a term of its job's output; the group that is not rotated joins the same
+    // sum as a term without a key, and the sum takes one ModDown merged with the rescale
     bool every_job_rotates = ng > 0;
     for (size_t q = 0; q < n_jobs; q++) every_job_rotates = every_job_rotates && rotated_first[q + 1] > rotated_first[q];
     if (every_job_rotates) {
@@ -350,18 +351,17 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
         for (size_t q = 0; q < n_jobs; q++) {
             for (size_t k = rotated_first[q]; k < rotated_first[q + 1]; k++)
                 gt.push_back(term(ext2.data() + k * beta * E * N, rs + k * ctw, pack, rot.galois(rotated_by[k]), nullptr));
+            gt.push_back(keylessTerm(sums.data() + q * ctw, sums.data() + q * ctw + nq * N, nullptr));
             goff.push_back((uint32_t)gt.size());
         }
         DeviceBuffer y2(c, n_jobs * 2 * E * N), ws3(c, n_jobs * ctw);
-        ck(hemm_hoisted_moddown(c->dev, gt.data(), goff.data(), (uint32_t)n_jobs, (uint32_t)nq, 0, 0, y2.data(), res.data(), nq * N, ws3.data(), nullptr));
-        ck(hemm_pointwise(c->dev, HEMM_ADD, res.data(), nq * N, sums.data(), nq * N, res.data(), nq * N, (uint32_t)nq, 0,
-                          (uint32_t)(2 * n_jobs), nullptr));
+        ck(hemm_hoisted_moddown(c->dev, gt.data(), goff.data(), (uint32_t)n_jobs, (uint32_t)nq, 0, 1, y2.data(), out,
+                                (nq - 1) * N, ws3.data(), nullptr));
     } else if (ng == 0) {
-        (void)hipMemcpyAsync(res.data(), sums.data(), n_jobs * ctw * 8, hipMemcpyDeviceToDevice, c->stream());
+        ck(hemm_rescale(c->dev, sums.data(), nq * N, out, (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
     } else {
         throw RuntimeException("diagonalTransformBatch: jobs with and without giant steps cannot share a batch");
     }
-    ck(hemm_rescale(c->dev, res.data(), nq * N, out, (nq - 1) * N, (uint32_t)nq, (uint32_t)(2 * n_jobs), nullptr));
 }
 
 Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,

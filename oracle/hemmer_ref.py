@@ -669,9 +669,11 @@ def diagonal_transform_fused(orc, ct, kind, n, w):
         sums.append(acc)
     res = sums[0]
     if len(sums) > 1:
+        # the group that is not rotated joins the rotated ones as a term without a key; one ModDown merged with the rescale
         terms = [(orc.modup(s.data[1]), s.data[0], r % orc.slots, None) for s, r in zip(sums[1:], rots[1:])]
+        terms.append((res.data[1], res.data[0], ("none",), None))
         y = orc.hoisted_sum(terms, nq)
-        res = orc.add(Ct(orc.moddown_drop(y, nq, False), res.scale), res)
+        return Ct(orc.moddown_drop(y, nq, True), res.scale / float(orc.q[nq - 1]))
     return orc.rescale(res)
 
 
