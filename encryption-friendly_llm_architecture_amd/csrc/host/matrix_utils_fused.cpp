@@ -739,9 +739,10 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         const i64 first_out = copies > 1 ? 0 : 1;   // bb[0] needs a launch only for its copies
         for (i64 i1 = first_out; i1 < g; i1++) {
             for (i64 j = 0; j < copies; j++) {
-                if (i1 == 0 && j == 0) continue;     // the unrotated operand itself is added below
+                if (i1 == 0 && j == 0) continue;     // the operand itself joins below
                 terms.push_back(term(xb.extOf(0), xb.pbOf(0), pack, rot.galois(i1 * ru - j * (i64)spread_block), nullptr));
             }
+            if (i1 == 0) terms.push_back(keylessTerm(tau_b, tau_b + lo * N, nullptr));   // no key switch for itself
             off.push_back((uint32_t)terms.size());
         }
         const u64 n_out = (u64)(g - first_out);
@@ -749,10 +750,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_out, (uint32_t)lo, xb.premultiplied(), 0,
                                 yb.data(), bb.data() + (u64)first_out * ctl, lo * N, ws.data(), nullptr));
     }
-    if (copies > 1)
-        ck(hemm_pointwise(c->dev, HEMM_ADD, bb.data(), lo * N, tau_b, lo * N, bb.data(), lo * N, (uint32_t)lo, 0, 2, nullptr));
-    else
-        (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, c->stream());
+    if (copies <= 1) (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, c->stream());
     // column shifts of sigma(A), shift i rotated back by g (i / g) row units
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
