@@ -211,9 +211,6 @@ hemm_context *hemm_context_build(int logN, int nQ, int nP, const u64 *primes, in
     c->d_fp = (double *)up(fpc.data(), fpc.size() * 8);
     c->d_scratch = nullptr;
     c->scratch_bytes = 0;
-    HEMM_HIP(hipStreamCreateWithFlags(&c->aux, hipStreamNonBlocking));
-    HEMM_HIP(hipEventCreateWithFlags(&c->aux_fork, hipEventDisableTiming));
-    HEMM_HIP(hipEventCreateWithFlags(&c->aux_join, hipEventDisableTiming));
     memset(c->traffic, 0, sizeof(c->traffic));
     memset(c->launches, 0, sizeof(c->launches));
     return c;

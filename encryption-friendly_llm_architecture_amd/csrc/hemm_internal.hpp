@@ -42,7 +42,8 @@ struct hemm_context {
     std::vector<std::pair<hipStream_t, void *>> d_desc;
     hipStream_t stream = nullptr;   // what a null stream argument of an entry point means for this context
     // a second stream (non-blocking, default priority) for the runs of a large transform batch: the odd runs go there,
-    // forked from and joined back into the caller's stream with the two events inside the same call
+    // forked from and joined back into the caller's stream with the two events inside the same call.  Made on first
+    // use: a process has few hardware queues, and a stream that is never used would still share one with a busy stream
     hipStream_t aux = nullptr;
     hipEvent_t aux_fork = nullptr, aux_join = nullptr;
     // compact evaluation keys: offset of every prime's limb inside a (digit, polynomial) slice and, last entry, the

@@ -1006,11 +1006,17 @@ void launch_ntt_slots(const hemm_context *c, u64 *data, const LimbList &ll, cons
     const int lanes = n_limbs * n_polys;
     if (c->logN == 16) {
         const dim3 block(256);
-        const int run = polys_per_run(n_limbs, n_polys, inverse, c->aux != nullptr);
+        const int run = polys_per_run(n_limbs, n_polys, inverse, true);
         // several runs: the odd ones on the context's second stream, which starts after what the caller's stream holds
         // so far and is waited for before the call returns to it
-        const bool two = c->aux != nullptr && run < n_polys;
+        const bool two = run < n_polys;
         const hipStream_t own = s;
+        if (two && c->aux == nullptr) {
+            hemm_context *m = const_cast<hemm_context *>(c);
+            HEMM_HIP(hipStreamCreateWithFlags(&m->aux, hipStreamNonBlocking));
+            HEMM_HIP(hipEventCreateWithFlags(&m->aux_fork, hipEventDisableTiming));
+            HEMM_HIP(hipEventCreateWithFlags(&m->aux_join, hipEventDisableTiming));
+        }
         if (two) {
             HEMM_HIP(hipEventRecord(c->aux_fork, own));
             HEMM_HIP(hipStreamWaitEvent(c->aux, c->aux_fork, 0));
