@@ -327,6 +327,65 @@ def test_preset_ccmm_residues_bit_exact(preset):
     assert np.abs(H.decrypt(c3) - A @ B).max() < 2.0 ** -12
 
 
+def test_preset_polynomials_reductions_and_low_rank_product_residues_bit_exact(preset):
+    """The rows around the matrix products at N = 2^16 on the preset, residue for residue against the oracle's
+    restatements: Exp::exp_iter and its pairwise form, the reference's EXP_15_4 Chebyshev table (4 baby steps), the
+    rotate-and-sum reductions of the pair layout, and a LoRA low-rank product (multMatMatHighLow) with its repacking."""
+    from oracle import poly_ref as P
+    from tests.test_poly_eval import EXP_15_4
+    H, orc, ev = preset
+    n, w, ld = 128, 256, R.LOW_DIM
+    rng = np.random.default_rng(34)
+    # polynomial evaluation
+    M = rng.uniform(-1, 1, (n, n))
+    ct = H.level_down(H.encrypt(M), 8)
+    oct_ = as_oracle(orc, ct)
+    got = H.exp_iter(ct, 3)
+    assert np.array_equal(got.residues(), P.exp_iter(ev, oct_, 3).data)
+    assert np.abs(H.decrypt(got) - (1 + M / 8) ** 8).max() < 2.0 ** -16
+    pair = [H.level_down(H.encrypt(rng.uniform(-1, 1, (n, n))), 6) for _ in range(2)]
+    opair = [as_oracle(orc, c) for c in pair]
+    H.exp_iter_parallel(pair, 2)
+    for c, want in zip(pair, P.exp_iter_parallel(ev, opair, 2)):
+        assert np.array_equal(c.residues(), want.data)
+    got = H.eval_chebyshev(ct, EXP_15_4, 4, 0.5)
+    want = P.eval_chebyshev(ev, oct_, EXP_15_4, 4, 0.5)
+    assert got.info()["level"] == want.level and np.array_equal(got.residues(), want.data)
+    # reductions on the pair layout
+    A, B = rng.normal(size=(n, n)), rng.normal(size=(n, n))
+    x = H.encrypt2(A, B)
+    ox = as_oracle(orc, x)
+    scaled = np.zeros((n, n))
+    scaled[:, 0] = 1.0 / (2 * n)
+    red = x.clone()
+    H.reduce_row_sum_with_scaled_mask(red, scaled, np.zeros((n, n)))
+    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n)
+    assert np.array_equal(red.residues(), want.data)
+    mean = np.concatenate([A, B], axis=1).mean(axis=1, keepdims=True)
+    assert np.abs(H.decrypt2(red)[0] - mean).max() < 2.0 ** -18
+    a, b = x.clone(), x.clone()
+    H.one_mat_rot_sum_inplace(a, b)
+    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n)
+    assert np.array_equal(a.residues(), wa.data) and np.array_equal(b.residues(), wb.data)
+    # a low-rank product: X (two tiles) times the block of ld columns of the LoRA factor, then repacked into one column block
+    blk = 3
+    thin = lambda: np.pad(rng.normal(0, 0.5, (n, ld)), ((0, 0), (blk * ld, n - (blk + 1) * ld)))
+    X0, X1, A0, A1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n)), thin(), thin()
+    cx, ca = H.encrypt2(X0, X1), H.encrypt2(A0, A1)
+    ocx, oca = as_oracle(orc, cx), as_oracle(orc, ca)
+    low = H.get_low_col_block(ca, blk)
+    olow = R.get_low_col_block(ev, oca, blk, n, n, w, ld)
+    assert np.array_equal(low.residues(), olow.data)
+    prod = H.matmul_high_low(cx, low, blk, 3)
+    want = R.mult_mat_mat_high_low(ev, ocx, olow, blk, 3, (n, n), (n, n), w, ld, orc)
+    assert prod.info()["level"] == 3 and np.array_equal(prod.residues(), want.data)
+    one = H.repack_to_one_col(prod, 0)
+    assert np.array_equal(one.residues(), R.repack_to_one_col(ev, want, 0, n, n, w, ld).data)
+    XA = X0 @ A0[:, blk * ld:(blk + 1) * ld] + X1 @ A1[:, blk * ld:(blk + 1) * ld]
+    for half in H.decrypt2(one):
+        assert np.abs(half[:, :ld] - XA).max() < 2.0 ** -12 and np.abs(half[:, ld:]).max() < 2.0 ** -12
+
+
 @pytest.fixture(scope="module")
 def chain24():
     pkg = load_package()
