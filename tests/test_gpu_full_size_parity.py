@@ -386,6 +386,65 @@ def test_preset_polynomials_reductions_and_low_rank_product_residues_bit_exact(p
         assert np.abs(half[:, :ld] - XA).max() < 2.0 ** -12 and np.abs(half[:, ld:]).max() < 2.0 ** -12
 
 
+def test_preset_other_low_rank_forms_residues_bit_exact(preset):
+    """multMatMatLowHigh with repackToMultiRow / OneRow, multMatMatLowLow and the element-wise rank-2 LoRA path
+    (down and up projection) at N = 2^16 on the preset, residue for residue against the oracle."""
+    H, orc, ev = preset
+    n, w, ld = 128, 256, R.LOW_DIM
+    rng = np.random.default_rng(35)
+    rows_of = lambda blk: np.pad(rng.normal(0, 0.5, (ld, n)), ((blk * ld, n - (blk + 1) * ld), (0, 0)))
+    cols_of = lambda blk: np.pad(rng.normal(0, 0.5, (n, ld)), ((0, 0), (blk * ld, n - (blk + 1) * ld)))
+    blk = 2
+    L0 = rows_of(blk)
+    G0, G1 = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    ca, cg = H.encrypt2(L0, L0), H.encrypt2(G0, G1)
+    oa, og = as_oracle(orc, ca), as_oracle(orc, cg)
+    low = H.get_low_row_block(ca, blk)
+    olow = R.get_low_row_block(ev, oa, blk, n, w, ld)
+    assert np.array_equal(low.residues(), olow.data)
+    got = H.matmul_low_high(low, cg, blk, 3)
+    want = R.mult_mat_mat_low_high(ev, olow, og, blk, 3, (n, n), (n, n), w, ld, orc)
+    assert np.array_equal(got.residues(), want.data)
+    multi = H.repack_to_multi_row(got, 5)
+    assert np.array_equal(multi.residues(), R.repack_to_multi_row(ev, want, 5, n, w, ld).data)
+    thin = L0[blk * ld:(blk + 1) * ld]
+    d = H.decrypt2(multi)
+    assert np.abs(d[0][5 * ld:6 * ld] - thin @ G0).max() < 2.0 ** -12 and np.abs(d[1][5 * ld:6 * ld] - thin @ G1).max() < 2.0 ** -12
+    one = H.repack_to_one_row(got, 1)
+    assert np.array_equal(one.residues(), R.repack_to_one_row(ev, want, 1, n, n, w, ld).data)
+    # low x low
+    cb, rb = 0, 4
+    A = cols_of(cb)
+    B0, B1 = rows_of(rb), rows_of(rb)
+    ca, cw = H.encrypt2(A, A), H.encrypt2(B0, B1)
+    got = H.matmul_low_low(ca, cw, cb, rb, 2)
+    want = R.mult_mat_mat_low_low(ev, as_oracle(orc, ca), as_oracle(orc, cw), cb, rb, 2, (n, n), (n, n), w, ld, orc)
+    assert got.info()["level"] == 2 and np.array_equal(got.residues(), want.data)
+    d = H.decrypt2(got)
+    assert np.abs(d[0] - A[:, cb * ld:(cb + 1) * ld] @ B0[rb * ld:(rb + 1) * ld]).max() < 2.0 ** -12
+    # the element-wise rank-2 path on one pair of tiles
+    m = 1
+    X = rng.uniform(-1, 1, (n, 2 * n * m))
+    A2 = rng.normal(0, 0.3, (2 * n * m, 2))
+    B2 = rng.normal(0, 0.3, (2, 2 * n * m))
+    wa, wb = np.zeros((n, w)), np.zeros((n, w))
+    for j in range(2):
+        wa[j] = A2[:, j]
+        wb[j] = B2[j]
+    enc2 = lambda M: H.encrypt2(M[:, :n], M[:, n:])
+    cur, cwa, cwb = [enc2(X)], enc2(wa), enc2(wb)
+    ocur, owa, owb = [as_oracle(orc, c) for c in cur], as_oracle(orc, cwa), as_oracle(orc, cwb)
+    xa = H.lora_rank2_down(cur, cwa, weight_level=7)
+    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7)
+    for j in range(2):
+        assert np.array_equal(xa[j].residues(), oxa[j].data)
+    out = H.lora_rank2_up(xa, cwb, m, weight_level=4)
+    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4)
+    assert np.array_equal(out[0].residues(), oout[0].data)
+    z = H.decrypt_slots(out[0]).real.reshape(n, w)
+    assert np.abs(z - X @ A2 @ B2).max() < 2.0 ** -10
+
+
 @pytest.fixture(scope="module")
 def chain24():
     pkg = load_package()
