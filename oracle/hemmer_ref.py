@@ -1278,6 +1278,34 @@ def repack_lora_opti(ev, t1, t2, n):
     return ev.add(out, ev.right_rotate(tmp, n))
 
 
+def repack_not_bts(ev, t1, t2, n, rescale_first=True):
+    """HEMMer::repack_notBTS (HEMMer.cpp:1025-1053): 2 Re(t1) + 2i Re(t2), the halves folded by a rotation of n,
+    the left columns kept and the second half put back beside them.  rescale_first: the reference rescales both inputs
+    (they arrive un-rescaled from a product); callers with rescaled inputs skip that step."""
+    if rescale_first:
+        t1, t2 = ev.rescale(t1), ev.rescale(t2)
+    out = ev.add(t1, ev.conjugate(t1))
+    tmp = ev.mult_imag_unit(ev.add(t2, ev.conjugate(t2)))
+    out = ev.add(out, tmp)
+    tmp = ev.left_rotate(out, n)
+    out = ev.add(out, tmp)
+    left = _message2(np.ones((n, n)), np.zeros((n, n)), ev.slots)        # mask_matmul_ (HEMMer.cpp:167-176)
+    tmp = _mult_msg(ev, tmp, left)
+    out = _mult_msg(ev, out, left)
+    return ev.add(out, ev.right_rotate(tmp, n))
+
+
+def split_in_two(ev, t, n):
+    """HEMMer::splitInTwo (HEMMer.cpp:819-831): [A | B] -> [A | A], [B | B] (the unmasked operand is lowered to the
+    product's level before the subtraction, as HomEvaluator::sub does with operands of two levels)."""
+    left = _message2(np.ones((n, n)), np.zeros((n, n)), ev.slots)        # mask_left_half_
+    tmp = _mult_msg(ev, t, left)
+    t2 = ev.sub(ev.level_down(t, ev.level_of(tmp)), tmp)
+    t1 = ev.add(ev.right_rotate(tmp, n), tmp)
+    t2 = ev.add(t2, ev.left_rotate(t2, n))
+    return t1, t2
+
+
 # ---- rank-2 LoRA through element-wise products (TransformerBlock.cpp:2199-2365) ------------------------------------
 def _first_row_mask(n, slots):
     m = np.zeros((n, n))

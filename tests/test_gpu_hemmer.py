@@ -460,19 +460,29 @@ def test_reuse_variants_and_repacking(small, fused):
         assert np.array_equal(pprod.residues(), want.data)
     H.set_schedule(True)
     # splitInTwo: [A0 | A1] -> [A0 | A0], [A1 | A1]
-    t1, t2 = H.split_in_two(H.encrypt2(A0, A1))
+    both = H.encrypt2(A0, A1)
+    t1, t2 = H.split_in_two(both)
+    w1, w2 = R.split_in_two(ev, to_oracle(orc, both), n)
+    assert np.array_equal(t1.residues(), w1.data) and np.array_equal(t2.residues(), w2.data)
     d1, d2 = H.decrypt2(t1), H.decrypt2(t2)
     for got, want in ((d1[0], A0), (d1[1], A0), (d2[0], A1), (d2[1], A1)):
         assert np.abs(got - want).max() < 2 ** -20
     # complexPackingRev: x - i y
-    z = H.decrypt_slots(H.complex_packing_rev(H.encrypt2(A0, A1), H.encrypt2(B0, B1)))
+    ra, rb = H.encrypt2(A0, A1), H.encrypt2(B0, B1)
+    rev = H.complex_packing_rev(ra, rb)
+    # HEMMer::complexPackingRev (HEMMer.cpp:987-994): multImagUnit of the second operand, subtracted from the first
+    assert np.array_equal(rev.residues(), ev.sub(to_oracle(orc, ra), ev.mult_imag_unit(to_oracle(orc, rb))).data)
+    z = H.decrypt_slots(rev)
     want = np.concatenate([A0, A1], axis=1).ravel() - 1j * np.concatenate([B0, B1], axis=1).ravel()
     assert np.abs(z - want).max() < 2 ** -20
     # repack_notBTS: o = 2 Re(t1) + 2i Re(t2); left half <- o + rot(o, n) on the left columns, right half <-
     # the left columns of rot(o, n)
     x1 = H.complex_packing(H.encrypt2(A0, A1), H.encrypt2(B0, B1))     # A + iB
     x2 = H.complex_packing(H.encrypt2(B1, A0), H.encrypt2(A1, B0))
-    out = H.decrypt_slots(H.repack_not_bts(x1, x2))
+    repacked = H.repack_not_bts(x1, x2)
+    want_ct = R.repack_not_bts(ev, to_oracle(orc, x1), to_oracle(orc, x2), n, rescale_first=False)
+    assert np.array_equal(repacked.residues(), want_ct.data)
+    out = H.decrypt_slots(repacked)
     s1 = np.concatenate([A0, A1], axis=1).ravel()
     s2 = np.concatenate([B1, A0], axis=1).ravel()
     o = 2 * s1 + 2j * s2

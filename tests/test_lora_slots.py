@@ -129,6 +129,25 @@ def test_repack_lora_opti_closed_form(sim):
     assert np.abs(out[:, n:] - (s2R + 0.5 * s2L + 0.5j * s1L)).max() < 1e-12
 
 
+def test_repack_not_bts_and_split_in_two_closed_forms(sim):
+    """repack_notBTS (HEMMer.cpp:1025-1053): with o = 2 Re(t1) + 2i Re(t2) and L / R its left and right tiles the result
+    is [o_L + o_R | o_R]; splitInTwo (HEMMer.cpp:819-831): [A | B] -> [A | A] and [B | B].  Worked out by hand from the
+    reference's rotations and masks."""
+    n = N_TILE
+    rng = np.random.default_rng(6)
+    t = [rng.normal(size=(2, n, n)) + 1j * rng.normal(size=(2, n, n)) for _ in range(2)]
+    t1 = R.SimCt(tile2(sim, t[0][0], t[0][1]), 5, rc=1)
+    t2 = R.SimCt(tile2(sim, t[1][0], t[1][1]), 5, rc=1)
+    out = R.repack_not_bts(sim, t1, t2, n).z.reshape(n, W)
+    oL, oR = 2 * t[0][0].real + 2j * t[1][0].real, 2 * t[0][1].real + 2j * t[1][1].real
+    assert np.abs(out[:, :n] - (oL + oR)).max() < 1e-12 and np.abs(out[:, n:] - oR).max() < 1e-12
+    A, B = rng.normal(size=(n, n)), rng.normal(size=(n, n))
+    a, b = R.split_in_two(sim, sim.encrypt(tile2(sim, A, B)), n)
+    for got, want in ((a, A), (b, B)):
+        left, right = halves(got.z)
+        assert np.abs(left - want).max() < 1e-12 and np.abs(right - want).max() < 1e-12
+
+
 def test_lora_rank2_elementwise_path(sim):
     """The production rank-2 form (element-wise products and rotate-and-sum, TransformerBlock.cpp:2199-2365):
     X (n x 6n, three pair-layout tiles) times A (6n x 2) gives two column ciphertexts, then times B (2 x 6n)."""
