@@ -1298,6 +1298,80 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
     if (std::min(a.getLevel(), b.getLevel()) == T + 3)
         return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true, add_conj);
+    {
+        const i64 rows = a.getHeight(), cols = b.getWidth(), k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
+        const u64 slots = c->N / 2;
+        const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
+        const bool bsgs = k / 2 > 1 && ((u64)(k * w) == slots || spread);
+        // With a level more to spare the two operands go their own ways: B is packed at T+4 and its transform ends at
+        // T+1, where the product needs it (no level-down in front of the baby rotations), on the side stream; A is packed
+        // at T+5 and transformed to T+2 on the context's stream, and only its copy for the unshifted term is lowered.
+        if (bsgs && rows == k && cols == k && a.getLevel() >= T + 5 && b.getLevel() >= T + 4 &&
+            std::min(a.getLevel(), b.getLevel()) >= 4 + btp.getMinLevelForBootstrap()) {
+            const u64 N = c->N, La = T + 5, Lb = T + 4, lo = T + 2;
+            const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
+            std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
+            DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
+            const std::vector<u64> one(La + 1, 1);
+            void *own = hemm_context_stream(c->dev);
+            {
+                const hipStream_t side = c->forkSide();
+                // (the phase marks of the two chains would interleave: one mark after both)
+                struct Back {
+                    const Context &c;
+                    void *own;
+                    bool trace;
+                    ~Back() {
+                        (void)hemm_context_set_stream(c->dev, own);
+                        c->joinSide();
+                        c->trace_on = trace;
+                    }
+                } back{c, own, c->trace_on};
+                c->trace_on = false;
+                // B one level below A, on the side stream: truncated to T+4, packed by rows (T+3), tau in two stages (T+1)
+                ck(hemm_context_set_stream(c->dev, side));
+                {
+                    DeviceBuffer jb(c, 2 * (Lb + 1) * N), pk(c, 2 * Lb * N);
+                    ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), one.data(), jb.data(), (Lb + 1) * N,
+                                       (uint32_t)(Lb + 1), 0, 2, nullptr));
+                    const bool by_rows = true;
+                    const u64 from = b.getLevel();
+                    tr.complexPackingBatch(eval, jb.data(), 1, Lb, &by_rows, w, pk.data(), &from);
+                    const MaskKind kind = MaskKind::PackedVertical;
+                    tr.diagonalTransformTwoStage(eval, pk.data(), 1, Lb - 1, &kind, &shape_b, tb.data());
+                }
+                ck(hemm_context_set_stream(c->dev, own));
+                // A on the context's stream: truncated to T+5, packed by columns (T+4), sigma in two stages (T+2)
+                {
+                    DeviceBuffer ja(c, 2 * (La + 1) * N), pk(c, 2 * La * N);
+                    ck(hemm_mul_scalar(c->dev, a.get().buf_.data(), a.get().polyStride(), one.data(), ja.data(), (La + 1) * N,
+                                       (uint32_t)(La + 1), 0, 2, nullptr));
+                    const bool by_rows = false;
+                    const u64 from = a.getLevel();
+                    tr.complexPackingBatch(eval, ja.data(), 1, La, &by_rows, w, pk.data(), &from);
+                    const MaskKind kind = MaskKind::PackedHorizontal;
+                    tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
+                }
+                levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
+            }
+            c->mark("packing and transforms");
+            const i64 g0 = bsgsBabyCount(k / 2);
+            const u64 us = (u64)((k / 2) / g0) * lo * N;
+            DeviceBuffer U(c, 3 * us);
+            ck(hemm_tensor_batch_strided(c->dev, low_a.data(), tb.data(), 1, (uint32_t)lo, U.data(), us, 0, nullptr));
+            Ciphertext acc(c);
+            acc.allocate(3, T + 1, 1);
+            CtxtTensor res(c, rows, cols, w);
+            i64 g = 1;
+            c->mark("unshifted term");
+            bsgsShiftProduct(eval, T, sa.data(), tb.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g, spread ? (u64)(k * w) : 0, true);
+            c->mark("main loop");
+            bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
+            c->mark("giant steps");
+            if (spread) res.get().occupied_ = (u64)(k * w);
+            return res;
+        }
+    }
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
     // is handed to the product where it lies.  Operands above the packing level are only truncated to it (a copy of
     // their first L+1 limbs): the packing masks absorb the change of scale, which saves the levelDown.

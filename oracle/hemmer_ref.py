@@ -864,18 +864,21 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
     return orc.rescale(orc.relinearize(acc))
 
 
-def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False, with_conj=False):
+def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False, with_conj=False,
+                              own_levels=False):
     """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused).
     merge_packing: a and b are NOT packed yet; the packing and the packed transform run as one composite one-stage
     transform from T+3 (kinds PKH / PKV).
     with_conj: returns x + conj(x) of the product x -- inside the giant-step sum where the schedule has one, by a
-    conjugation afterwards otherwise."""
+    conjugation afterwards otherwise.
+    own_levels: sigma(A) ends at T+2 and tau(B) at T+1 from whatever levels they arrive at (the form for operands one
+    level apart)."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     lvl = min(a.level, b.level)
-    if merge_packing or lvl >= T + 3:
+    if not own_levels and (merge_packing or lvl >= T + 3):
         if merge_packing:
             a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)
             b = diagonal_transform_fused(orc, orc.level_down(b, T + 3), PKV, n, w)
@@ -945,10 +948,18 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     ev = OracleEval(orc)
     if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
         return mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True, with_conj=True)
+    cut = lambda x, lvl: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
+    spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
+    rows, cols = _dims(n)
+    if a.level >= T + 5 and b.level >= T + 4 and rows == cols and n // 2 > 1 and (n * w == orc.slots or spread):
+        # a level more to spare: B is packed at T+4 and transformed straight to T+1, A packed at T+5 and transformed to
+        # T+2 (the two chains run side by side on the GPU); only A's copy for the unshifted term is lowered
+        pa = complex_packing_hoisted(orc, cut(a, T + 5), w, rows=False)
+        pb = complex_packing_hoisted(orc, cut(b, T + 4), w, rows=True)
+        return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True, own_levels=True)
     lvl = min(a.level, b.level, T + 5)
-    cut = lambda x: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
-    pa = complex_packing_hoisted(orc, cut(a), w, rows=False)
-    pb = complex_packing_hoisted(orc, cut(b), w, rows=True)
+    pa = complex_packing_hoisted(orc, cut(a, lvl), w, rows=False)
+    pb = complex_packing_hoisted(orc, cut(b, lvl), w, rows=True)
     return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True)
 
 
