@@ -710,7 +710,8 @@ namespace {
 // is the rotation of tau(B) copied into every block (row shifts of a periodic vector are exact rotations).
 void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
                       std::vector<Plaintext> &cm, i64 n, i64 units, i64 cu, i64 w, u64 batch, DeviceBuffer *U_out,
-                      i64 *g_out, u64 spread_block = 0, bool u_ready = false) {
+                      i64 *g_out, u64 spread_block = 0, bool u_ready = false, hipStream_t b_stream = nullptr,
+                      const u64 *low_a = nullptr) {
     const Context &c = eval.getContext();
     const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
     const i64 ru = cu * w;
@@ -719,21 +720,23 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     const Rot rot(c);
     const u64 ctl = 2 * lo * N;   // words of a two-polynomial ciphertext at level T+1
     // The sources of the column shifts (sigma(A) and its copy rotated by -n, both extended) do not depend on the
-    // baby rotations of tau(B): a chain of small launches that runs on the side stream beside them.
-    const hipStream_t side = c->forkSide();
+    // baby rotations of tau(B): two chains of small launches side by side.  b_stream: the side chain is already open
+    // and tau(B) is being produced on it; the baby rotations then follow it there and the sources of sigma(A) take the
+    // context's stream, with no join in between.  Otherwise the side chain is opened here for the sources of sigma(A).
+    const hipStream_t s_b = b_stream, s_a = b_stream ? nullptr : c->forkSide();
     struct JoinOnExit {
         const Context &c;
         ~JoinOnExit() { c->joinSide(); }   // also when a launch below throws
     } join_on_exit{c};
-    const Sources xa = extendSources(c, sigma_a, 1, nq, side);
+    const Sources xa = extendSources(c, sigma_a, 1, nq, s_a);
     const i64 back = -n;
-    const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back, side);
-    const Sources xa2 = extendSources(c, a2.data(), 1, nq, side);
+    const DeviceBuffer a2 = rotateSources(eval, xa, sigma_a, 1, &back, s_a);
+    const Sources xa2 = extendSources(c, a2.data(), 1, nq, s_a);
     // baby rotations of tau(B): bb[i1] = rho^(i1 ru)(tau B), summed over the block copies when tau(B) is spread
     DeviceBuffer bb(c, (u64)g * ctl);
     const i64 copies = spread_block ? (i64)((c->N / 2) / spread_block) : 1;
     if (g > 1 || copies > 1) {
-        const Sources xb = extendSources(c, tau_b, 1, lo, nullptr, false);
+        const Sources xb = extendSources(c, tau_b, 1, lo, s_b, false);
         std::vector<hemm_rot_term> terms;
         std::vector<uint32_t> off{0};
         const i64 first_out = copies > 1 ? 0 : 1;   // bb[0] needs a launch only for its copies
@@ -748,9 +751,9 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         const u64 n_out = (u64)(g - first_out);
         DeviceBuffer yb(c, n_out * 2 * (lo + K) * N), ws(c, n_out * ctl);
         ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_out, (uint32_t)lo, xb.premultiplied(), 0,
-                                yb.data(), bb.data() + (u64)first_out * ctl, lo * N, ws.data(), nullptr));
+                                yb.data(), bb.data() + (u64)first_out * ctl, lo * N, ws.data(), s_b));
     }
-    if (copies <= 1) (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, c->stream());
+    if (copies <= 1) (void)hipMemcpyAsync(bb.data(), tau_b, ctl * 8, hipMemcpyDeviceToDevice, c->on(s_b));
     // column shifts of sigma(A), shift i rotated back by g (i / g) row units
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
@@ -760,7 +763,10 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
     // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
     const u64 pw = lo * N, us = (u64)n_giant * pw;
-    if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
+    if (low_a != nullptr) {   // the i = 0 term, sigma(A) lowered to T+1 times tau(B), now that both chains have joined
+        U_out->resize(c, 3 * us);
+        ck(hemm_tensor_batch_strided(c->dev, low_a, tau_b, 1, (uint32_t)lo, U_out->data(), us, 0, nullptr));
+    } else if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
         U_out->resize(c, 3 * us);
         for (u64 p = 0; p < 3; p++)
             (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, c->stream());
@@ -1353,23 +1359,23 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                     tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
                 }
                 levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
+                // the side chain stays open: the baby rotations of tau(B) follow its transform there while the sources
+                // of sigma(A) are made here, and the two meet in front of the main loop
+                c->trace_on = back.trace;
+                c->mark("packing and transforms of A");
+                DeviceBuffer U;
+                Ciphertext acc(c);
+                acc.allocate(3, T + 1, 1);
+                CtxtTensor res(c, rows, cols, w);
+                i64 g = 1;
+                bsgsShiftProduct(eval, T, sa.data(), tb.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g,
+                                 spread ? (u64)(k * w) : 0, false, side, low_a.data());
+                c->mark("main loop");
+                bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
+                c->mark("giant steps");
+                if (spread) res.get().occupied_ = (u64)(k * w);
+                return res;
             }
-            c->mark("packing and transforms");
-            const i64 g0 = bsgsBabyCount(k / 2);
-            const u64 us = (u64)((k / 2) / g0) * lo * N;
-            DeviceBuffer U(c, 3 * us);
-            ck(hemm_tensor_batch_strided(c->dev, low_a.data(), tb.data(), 1, (uint32_t)lo, U.data(), us, 0, nullptr));
-            Ciphertext acc(c);
-            acc.allocate(3, T + 1, 1);
-            CtxtTensor res(c, rows, cols, w);
-            i64 g = 1;
-            c->mark("unshifted term");
-            bsgsShiftProduct(eval, T, sa.data(), tb.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g, spread ? (u64)(k * w) : 0, true);
-            c->mark("main loop");
-            bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
-            c->mark("giant steps");
-            if (spread) res.get().occupied_ = (u64)(k * w);
-            return res;
         }
     }
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
