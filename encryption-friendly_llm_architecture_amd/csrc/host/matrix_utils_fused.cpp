@@ -1312,9 +1312,10 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
         // With a level more to spare the two operands go their own ways: B is packed at T+4 and its transform ends at
         // T+1, where the product needs it (no level-down in front of the baby rotations), on the side stream; A is packed
         // at T+5 and transformed to T+2 on the context's stream, and only its copy for the unshifted term is lowered.
-        if (bsgs && rows == k && cols == k && a.getLevel() >= T + 5 && b.getLevel() >= T + 4 &&
+        // (an A with only four levels above the target is packed at T+4 and takes the one-stage transform from T+3)
+        if (bsgs && rows == k && cols == k && a.getLevel() >= T + 4 && b.getLevel() >= T + 4 &&
             std::min(a.getLevel(), b.getLevel()) >= 4 + btp.getMinLevelForBootstrap()) {
-            const u64 N = c->N, La = T + 5, Lb = T + 4, lo = T + 2;
+            const u64 N = c->N, La = std::min<u64>(a.getLevel(), T + 5), Lb = T + 4, lo = T + 2;
             const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
             std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
             DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
@@ -1347,7 +1348,8 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                     tr.diagonalTransformTwoStage(eval, pk.data(), 1, Lb - 1, &kind, &shape_b, tb.data());
                 }
                 ck(hemm_context_set_stream(c->dev, own));
-                // A on the context's stream: truncated to T+5, packed by columns (T+4), sigma in two stages (T+2)
+                // A on the context's stream: truncated to T+5, packed by columns (T+4), sigma in two stages (T+2); from T+4:
+                // packed to T+3, sigma in one stage
                 {
                     DeviceBuffer ja(c, 2 * (La + 1) * N), pk(c, 2 * La * N);
                     ck(hemm_mul_scalar(c->dev, a.get().buf_.data(), a.get().polyStride(), one.data(), ja.data(), (La + 1) * N,
@@ -1356,8 +1358,12 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                     const u64 from = a.getLevel();
                     tr.complexPackingBatch(eval, ja.data(), 1, La, &by_rows, w, pk.data(), &from);
                     const MaskKind kind = MaskKind::PackedHorizontal;
-                    tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
+                    if (La == T + 5)
+                        tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
+                    else
+                        tr.diagonalTransformBatch(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
                 }
+                // (the only call that works in the context's scratch region while the side chain is open)
                 levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
                 // the side chain stays open: the baby rotations of tau(B) follow its transform there while the sources
                 // of sigma(A) are made here, and the two meet in front of the main loop

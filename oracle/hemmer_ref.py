@@ -951,10 +951,11 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     cut = lambda x, lvl: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     rows, cols = _dims(n)
-    if a.level >= T + 5 and b.level >= T + 4 and rows == cols and n // 2 > 1 and (n * w == orc.slots or spread):
-        # a level more to spare: B is packed at T+4 and transformed straight to T+1, A packed at T+5 and transformed to
-        # T+2 (the two chains run side by side on the GPU); only A's copy for the unshifted term is lowered
-        pa = complex_packing_hoisted(orc, cut(a, T + 5), w, rows=False)
+    if a.level >= T + 4 and b.level >= T + 4 and rows == cols and n // 2 > 1 and (n * w == orc.slots or spread):
+        # the operands go their own ways: B is packed at T+4 and transformed straight to T+1 (two stages), A packed at
+        # T+5 and transformed to T+2 in two stages, or packed at T+4 and transformed in one (the two chains run side by
+        # side on the GPU); only A's copy for the unshifted term is lowered
+        pa = complex_packing_hoisted(orc, cut(a, min(a.level, T + 5)), w, rows=False)
         pb = complex_packing_hoisted(orc, cut(b, T + 4), w, rows=True)
         return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True, own_levels=True)
     lvl = min(a.level, b.level, T + 5)
