@@ -87,8 +87,11 @@ public:
     // [job][2][level-1][N], TWO levels lower.  2 (b + n/b) keyed rotations with 2 (b + n/b) masks per operand
     // instead of b + 2 n/b rotations with 2 n - 1 masks, and every stage is a single output of the hoisted launch
     // (one ModDown per stage).  Used by the batched products when the operands have a level to spare.
+    // scale_levels (optional, one per job): the level whose fixed scale job q's input carries -- an operand truncated to
+    // `level` from a higher one; the masks of the first stage are then encoded at Delta_(level-1) q_level /
+    // Delta_(scale level), which lands the result on the fixed scale of level - 1 without a levelDown in front.
     void diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
-                                   const TileTensorShape *shapes, u64 *out);
+                                   const TileTensorShape *shapes, u64 *out, const u64 *scale_levels = nullptr);
     // Brings `in` down to the level a transform ending at `end_level` starts from and runs it with the batched
     // launches: two stages from end_level + 2 when the operand is that high and the tile is square, otherwise one
     // stage from end_level + 1.
@@ -139,11 +142,12 @@ public:
     std::vector<std::tuple<u64, u64, TileTensorShape, u64>> weight_tau_order_;
 
 private:
-    // (kind, shape, level, stage * 4096 + r * 4 + part) -> mask of the two-stage transforms; part 0 is an ordinary
-    // plaintext (the unrotated rows), parts 1 / 2 (main / wrapped columns) are over the extended basis
+    // (kind, shape, level, (scale level * 4 + stage) * 4096 + r * 4 + part) -> mask of the two-stage transforms; part 0 is
+    // an ordinary plaintext (the unrotated rows), parts 1 / 2 (main / wrapped columns) are over the extended basis; masks
+    // that absorb a change of scale (scale level != 0) are all over the extended basis
     std::map<Key, Plaintext> two_stage_masks_;
     const Plaintext &twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape, u64 level,
-                                  int stage, i64 r, int part);
+                                  int stage, i64 r, int part, u64 from = 0);
 };
 
 // A x B for two encrypted tiles (HEMMer::singleCCMatMul); output level = target_level.

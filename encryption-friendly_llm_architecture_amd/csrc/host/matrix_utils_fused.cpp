@@ -533,13 +533,18 @@ Message twoStageMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log
 }
 
 const Plaintext &MatrixTransformer::twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape,
-                                                 u64 level, int stage, i64 r, int part) {
-    Key key{(int)kind, shape, level, (i64)stage * 4096 + r * 4 + part};
+                                                 u64 level, int stage, i64 r, int part, u64 from) {
+    if (from == level) from = 0;   // the level's own scale
+    Key key{(int)kind, shape, level, ((i64)from * 4 + stage) * 4096 + r * 4 + part};
     auto it = two_stage_masks_.find(key);
     if (it != two_stage_masks_.end()) return it->second;
     const Context &ctx = eval.getContext();
     const Message m = twoStageMaskMessage(kind, shape, getLogFullSlots(ctx), stage, r, part);
     EnDecoder endec(ctx);
+    if (from != 0) {
+        const Real scale = ctx->delta[level - 1] * (Real)ctx->q[level] / ctx->delta[from];
+        return two_stage_masks_.emplace(key, endec.encodeExtended(m, level, scale)).first->second;
+    }
     return two_stage_masks_.emplace(key, part == 0 ? endec.encode(m, level) : endec.encodeExtended(m, level)).first->second;
 }
 
@@ -568,6 +573,18 @@ Ciphertext MatrixTransformer::lowerAndTransformFused(const HomEvaluator &eval, c
         throw std::invalid_argument("[diagonalTransform] level >= " + std::to_string(end_level + 1) + " is needed.");
     const bool two_stage = in.getLevel() >= end_level + 2 && shape.getNumRows() == shape.getNumCols();
     Ciphertext x(c), res(c);
+    if (two_stage && in.getLevel() > end_level + 2 && in.getRescaleCounter() == 0 && in.getNumPoly() == 2) {
+        // an operand above the starting level is only truncated to it (a copy of its first limbs): the masks of the
+        // first stage absorb the change of scale, which saves the multiply-and-rescale of a levelDown
+        const u64 L = end_level + 2, N = c->N, from = in.getLevel();
+        DeviceBuffer cut(c, 2 * (L + 1) * N);
+        const std::vector<u64> one(L + 1, 1);
+        ck(hemm_mul_scalar(c->dev, in.buf_.data(), in.polyStride(), one.data(), cut.data(), (L + 1) * N, (uint32_t)(L + 1), 0, 2,
+                           nullptr));
+        res.allocate(2, end_level, 0);
+        diagonalTransformTwoStage(eval, cut.data(), 1, L, &kind, &shape, res.buf_.data(), &from);
+        return res;
+    }
     eval.levelDown(in, end_level + (two_stage ? 2 : 1), x);
     if (!two_stage) return diagonalTransformFused(eval, x, kind, shape);
     res.allocate(2, end_level, 0);
@@ -576,7 +593,8 @@ Ciphertext MatrixTransformer::lowerAndTransformFused(const HomEvaluator &eval, c
 }
 
 void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
-                                                  const MaskKind *kinds, const TileTensorShape *shapes, u64 *out) {
+                                                  const MaskKind *kinds, const TileTensorShape *shapes, u64 *out,
+                                                  const u64 *scale_levels) {
     const Context &c = eval.getContext();
     if (level < 2) throw std::invalid_argument("[diagonalTransform] level >= 2 is needed.");
     const u64 N = c->N;
@@ -585,6 +603,7 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         const u64 lvl = stage == 1 ? level : level - 1, nq = lvl + 1, E = nq + c->nP, ctw = 2 * nq * N;
         const u64 *src = stage == 1 ? in : mid.data();
         u64 *dst = stage == 1 ? mid.data() : out;
+        auto from_of = [&](size_t q) -> u64 { return stage == 1 && scale_levels ? scale_levels[q] : 0; };
         // One rotation source per job (a single ModUp).  A stage's rotation by r cells wraps inside the tile, so it is
         //   main_r * rho^(r step)(X) + wrap_r * rho^(r step - tile side)(X):
         // two Galois elements per r with one key each; when they coincide (the tile side is a whole turn of the slot
@@ -611,15 +630,15 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
                 const i64 amount = r * mul * g.step;
                 if (rot.norm(amount) == rot.norm(amount - wrap)) {
                     terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount),
-                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 3)));
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 3, from_of(q))));
                 } else {
                     terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount),
-                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 1)));
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 1, from_of(q))));
                     terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount - wrap),
-                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2)));
+                                         &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, r, 2, from_of(q))));
                 }
             }
-            terms.push_back(keylessTerm(src + q * ctw, src + q * ctw + nq * N, &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0)));
+            terms.push_back(keylessTerm(src + q * ctw, src + q * ctw + nq * N, &twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0, from_of(q))));
             off.push_back((uint32_t)terms.size());
         }
         if (any_rotation) {
@@ -635,7 +654,7 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
             for (size_t q = 0; q < n_jobs; q++) {
                 hemm_lin_term t;
                 t.ct = src + q * ctw;
-                t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0).buf_.data();
+                t.mask = twoStageMask(eval, kinds[q], shapes[q], lvl, stage, 0, 0, from_of(q)).buf_.data();
                 t.stride = nq * N;
                 t.galois = 0;
                 zero_terms.push_back(t);

@@ -712,11 +712,13 @@ def two_stage_mask(kind, n, w, slots, stage, r, part):
     return np.where(on, 0.5 if (kind == PH and stage == 1) else 1.0, 0.0).astype(np.complex128)
 
 
-def diagonal_transform_two_stage(orc, ct, kind, n, w):
+def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None):
     """sigma / tau (square tiles) in two stages of one mask level each: row i is rotated by i mod b, then
     by b (i div b).  Every stage is one hoisted sum over its rotations of
     main_r rho^(r)(X) + wrap_r rho^(r - tile side)(X) (two keys per r, one source) and of mask_0 X for the rows that
-    stay (a term without a key switch), with ModDown merged with the rescale.  Level L -> L - 2."""
+    stay (a term without a key switch), with ModDown merged with the rescale.  Level L -> L - 2.
+    from_level: the level whose scale the input still carries when it was only truncated from there (the masks of
+    the first stage are then encoded at Delta_{L-1} q_L / Delta_from, so the stage ends at the scale of L - 1)."""
     from .oracle import Ct
     cell = 2 if kind in (PH, PV) else 1
     u = n // cell
@@ -725,11 +727,14 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
     wrap = n * (w if kind in (V, PV) else 1)
     x = ct
     for stage, count, mul in ((1, b, 1), (2, u // b, b)):
-        nq = x.nq
-        mask = lambda r, part: orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, part), x.level)
+        nq, lvl = x.nq, x.level
+        own = stage == 2 or from_level is None or from_level == lvl
+        ms = orc.delta[lvl] if own else orc.delta[lvl - 1] * float(orc.q[lvl]) / orc.delta[from_level]
+        mask = lambda r, part: orc.encode_ext(two_stage_mask(kind, n, w, orc.slots, stage, r, part), lvl, ms)
         if count <= 1:      # no rotation in this stage: mask and rescale
             x = orc.rescale(orc.mult_plain_no_rescale(
-                x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), x.level)))
+                x, orc.encode(two_stage_mask(kind, n, w, orc.slots, stage, 0, 0), lvl, ms)))
+            x.scale = orc.delta[lvl - 1]
             continue
         ext = orc.modup(x.data[1])
         terms = []
@@ -742,16 +747,20 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w):
                 terms.append((ext, x.data[0], r_wrap, mask(r, 2)))
         terms.append((x.data[1], x.data[0], ("none",), mask(0, 0)))
         y = orc.hoisted_sum(terms, nq)
-        x = Ct(orc.moddown_drop(y, nq, True), x.scale * orc.delta[x.level] / float(orc.q[x.level]))
+        x = Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
     return x
 
 
 def lower_and_transform_fused(orc, x, kind, n, w, end_level):
     """Batched transform ending at end_level: two stages from end_level + 2 when the operand is that high and
     the tile is square, otherwise one stage from end_level + 1."""
+    from .oracle import Ct
     rows, cols = _dims(n)
     if x.level >= end_level + 2 and rows == cols:
-        return diagonal_transform_two_stage(orc, orc.level_down(x, end_level + 2), kind, rows, w)
+        # an operand above the starting level is only truncated to it: the masks of the first stage absorb the change
+        # of scale (no levelDown)
+        cut = Ct(np.ascontiguousarray(x.data[:, : end_level + 3]), x.scale)
+        return diagonal_transform_two_stage(orc, cut, kind, rows, w, from_level=x.level)
     return diagonal_transform_fused(orc, orc.level_down(x, end_level + 1), kind, n, w)
 
 
