@@ -1141,6 +1141,56 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
 CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                                  const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
     const Context &c = eval.getContext();
+    // Square tiles with A four levels and B three levels above the target: the operands go their own ways, as in the
+    // complex-packed product.  tau(B) runs from T+3 to T+1 on the side stream, where the baby rotations follow it;
+    // sigma(A) runs from T+4 to T+2 on the context's stream.  Operands above these levels are only truncated (the
+    // first stage's masks absorb the change of scale), so nothing but sigma(A)'s copy for the unshifted term passes
+    // through the context's scratch region while the side chain is open.
+    if (op1.getLevel() >= T + 4 && op2.getLevel() >= T + 3 && op1.get().getRescaleCounter() == 0 &&
+        op2.get().getRescaleCounter() == 0 && op1.get().getNumPoly() == 2 && op2.get().getNumPoly() == 2 &&
+        std::min(op1.getLevel(), op2.getLevel()) >= 4 + btp.getMinLevelForBootstrap()) {
+        const i64 rows = op1.getHeight(), cols = op2.getWidth();
+        const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
+        const u64 slots = c->N / 2, N = c->N, lo = T + 2;
+        const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
+        if (rows == k && cols == k && k / 2 >= 4 && ((u64)(k * w) == slots || spread)) {
+            const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
+            std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
+            void *own = hemm_context_stream(c->dev);
+            const hipStream_t side = c->forkSide();
+            struct Back {   // (the phase marks of the two chains would interleave: none while both run)
+                const Context &c;
+                void *own;
+                bool trace;
+                ~Back() {
+                    (void)hemm_context_set_stream(c->dev, own);
+                    c->joinSide();
+                    c->trace_on = trace;
+                }
+            } back{c, own, c->trace_on};
+            c->trace_on = false;
+            ck(hemm_context_set_stream(c->dev, side));
+            const Ciphertext tb = tr.lowerAndTransformFused(eval, op2.get(), MaskKind::PackedVertical, shape_b, T + 1);
+            ck(hemm_context_set_stream(c->dev, own));
+            const Ciphertext sa = tr.lowerAndTransformFused(eval, op1.get(), MaskKind::PackedHorizontal, shape_a, T + 2);
+            DeviceBuffer low_a(c, 2 * lo * N);
+            levelDownOneBatch(c, sa.buf_.data(), 2, T + 2, low_a.data());
+            c->trace_on = back.trace;
+            c->mark("transforms");
+            DeviceBuffer U;
+            Ciphertext acc(c);
+            acc.allocate(3, T + 1, 1);
+            CtxtTensor res(c, rows, cols, w);
+            i64 g = 1;
+            bsgsShiftProduct(eval, T, sa.buf_.data(), tb.buf_.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g,
+                             spread ? (u64)(k * w) : 0, false, side, low_a.data());
+            c->mark("main loop");
+            bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res);
+            c->mark("giant steps");
+            if (spread) res.get().occupied_ = (u64)(k * w);
+            return res;
+        }
+    }
     // both operands a level above what the reference asks of B: sigma and tau share one launch chain, as in the
     // unpacked product (tau(B) is then lowered to T+1 with sigma(A)'s copy for the unshifted term)
     if (std::min(op1.getLevel(), op2.getLevel()) >= T + 3 && op1.get().getRescaleCounter() == 0 &&
@@ -1332,7 +1382,9 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
         // T+1, where the product needs it (no level-down in front of the baby rotations), on the side stream; A is packed
         // at T+5 and transformed to T+2 on the context's stream, and only its copy for the unshifted term is lowered.
         // (an A with only four levels above the target is packed at T+4 and takes the one-stage transform from T+3)
-        if (bsgs && rows == k && cols == k && a.getLevel() >= T + 4 && b.getLevel() >= T + 4 &&
+        // (k / 2 >= 4: every transform stage then has rotations; a stage without any rescales through the context's
+        // scratch region, which only one of the two chains may use)
+        if (bsgs && k / 2 >= 4 && rows == k && cols == k && a.getLevel() >= T + 4 && b.getLevel() >= T + 4 &&
             std::min(a.getLevel(), b.getLevel()) >= 4 + btp.getMinLevelForBootstrap()) {
             const u64 N = c->N, La = std::min<u64>(a.getLevel(), T + 5), Lb = T + 4, lo = T + 2;
             const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);

@@ -887,6 +887,11 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packi
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     lvl = min(a.level, b.level)
+    rows, cols = _dims(n)
+    # square tiles with A four and B three levels above the target take their own ways too (truncated to T+4 / T+3)
+    if (not merge_packing and a.level >= T + 4 and b.level >= T + 3 and rows == cols and n // 2 >= 4
+            and (n * w == orc.slots or spread)):
+        own_levels = True
     if not own_levels and (merge_packing or lvl >= T + 3):
         if merge_packing:
             a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)
@@ -960,7 +965,7 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     cut = lambda x, lvl: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     rows, cols = _dims(n)
-    if a.level >= T + 4 and b.level >= T + 4 and rows == cols and n // 2 > 1 and (n * w == orc.slots or spread):
+    if a.level >= T + 4 and b.level >= T + 4 and rows == cols and n // 2 >= 4 and (n * w == orc.slots or spread):
         # the operands go their own ways: B is packed at T+4 and transformed straight to T+1 (two stages), A packed at
         # T+5 and transformed to T+2 in two stages, or packed at T+4 and transformed in one (the two chains run side by
         # side on the GPU); only A's copy for the unshifted term is lowered
