@@ -327,6 +327,30 @@ def test_preset_ccmm_residues_bit_exact(preset):
     assert np.abs(H.decrypt(c3) - A @ B).max() < 2.0 ** -12
 
 
+def test_preset_two_stream_products_repeat_bit_for_bit(preset):
+    """The products whose operands take their own ways on two streams (singleCCMatMul of single tiles, packedMatMul)
+    and the one-ModDown PCMM, called eight times in turn on the same operands: every call returns the residues of
+    the first.  A launch of one chain that read what the other had not finished writing, or two users of one
+    workspace, would show up as a call that differs."""
+    H, orc, _ = preset
+    rng = np.random.default_rng(41)
+    A, B, A2, B2 = (rng.uniform(-1, 1, (128, 128)) for _ in range(4))
+    ca, cb = H.encrypt(A), H.encrypt(B)
+    pa, pb = H.encrypt2(A, A2), H.encrypt2(B, B2)
+    H.complex_packing_inplace(pa)
+    H.complex_packing_row_inplace(pb)
+    wb = H.encode(B)
+    first = None
+    for it in range(8):
+        got = (H.single_cc_matmul(ca, cb, 4).residues(), H.packed_matmul(pa, pb, 4).residues(),
+               H.single_matmul(ca, wb, 4).residues())
+        if first is None:
+            first = got
+            continue
+        for k, (x, y) in enumerate(zip(got, first)):
+            assert np.array_equal(x, y), (it, k)
+
+
 def test_preset_polynomials_reductions_and_low_rank_product_residues_bit_exact(preset):
     """The rows around the matrix products at N = 2^16 on the preset, residue for residue against the oracle's
     restatements: Exp::exp_iter and its pairwise form, the reference's EXP_15_4 Chebyshev table (4 baby steps), the
