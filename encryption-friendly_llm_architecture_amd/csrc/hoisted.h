@@ -146,8 +146,9 @@ __device__ __forceinline__ ulonglong2 key_pair_ptr(const RotTermDev &T, const u3
 typedef u32 u32x3 __attribute__((ext_vector_type(3), aligned(4)));
 
 // One term with two masked sources under one key (integer path): residues (n, n+1) of limb j of
-// <z, evk> + P (mask b + mask2 b2) with z_d = mask * x_d + mask2 * x2_d, canonical.  RUNS: the masks are run tables
-// without a plaintext factor, i.e. constants with a Shoup companion: no wide product and no Barrett step for z_d.
+// <z, evk> + P (mask b + mask2 b2) with z_d = mask * x_d + mask2 * x2_d, canonical.  RUNS: the masks are run tables,
+// i.e. constants with a Shoup companion: no wide product and no Barrett step for z_d; a plaintext factor of the term is
+// then left to the caller, which multiplies the finished pair by it.
 template <bool RUNS, bool COMPACT>
 __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *__restrict__ koff, const ModQ m,
                                                const CstList &pmod, const int j,
@@ -264,12 +265,22 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         if (T.ext2 != nullptr) {
             // two masked sources under one key: z_d = mask * x_d + mask2 * x2_d, then one pass over the key
             u64 rb[2], ra[2];
-            if (T.mask_shift != 0 && T.pt == nullptr)
+            if (T.mask_shift != 0) {
+                // run-table masks are constants: the plaintext factor of the term, if it has one, is common to both
+                // sources and multiplies the finished pair once (same residues as masks multiplied by it beforehand)
                 two_source_int<true, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN,
                                               b_premultiplied, rb, ra);
-            else
+                if (T.pt != nullptr) {
+                    const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
+                    rb[0] = mulmod(rb[0], pv.x, m);
+                    rb[1] = mulmod(rb[1], pv.y, m);
+                    ra[0] = mulmod(ra[0], pv.x, m);
+                    ra[1] = mulmod(ra[1], pv.y, m);
+                }
+            } else {
                 two_source_int<false, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN,
                                                b_premultiplied, rb, ra);
+            }
             acc_b[0] = addmod(acc_b[0], rb[0], m.q);
             acc_b[1] = addmod(acc_b[1], rb[1], m.q);
             acc_a[0] = addmod(acc_a[0], ra[0], m.q);

@@ -1245,7 +1245,7 @@ static bool split_limbs(const hemm_context *c, int nq, int beta, int n_out, Limb
         else
             il.idx[n_int++] = (uint8_t)j;
     }
-    return n_fp > 0 && n_int > 0 && (size_t)n_out * E * (c->N / 512) >= 32768;
+    return n_fp > 0 && n_int > 0 && (size_t)n_out * E * (c->N / 512) >= 16384;
 }
 
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,
