@@ -953,6 +953,56 @@ void bsgsGiantSteps(const HomEvaluator &eval, u64 T, DeviceBuffer &U, i64 g, i64
     ck(hemm_hoisted_terms(c->dev, terms.data(), off, 1, (uint32_t)lo, yg.data(), 0, nullptr));
     ck(hemm_moddown_batch(c->dev, yg.data(), (uint32_t)lo, 2, 0, res.get().buf_.data(), lo * N, wsg.data(), nullptr));
 }
+
+// The operands of a product on their own ways: B's chain is queued on the side stream -- the context's stream is
+// pointed there for as long as B's calls are made -- and A's on the context's own.  On leaving (also by an exception)
+// the context's stream is its own again, the side chain has joined and the phase marks, which the two interleaved
+// chains would garble, are back on.
+class OwnWays {
+  public:
+    explicit OwnWays(const Context &c)
+        : c_(c), own_(hemm_context_stream(c->dev)), trace_(c->trace_on), side_(c->forkSide()) {
+        c->trace_on = false;
+    }
+    ~OwnWays() {
+        (void)hemm_context_set_stream(c_->dev, own_);
+        c_->joinSide();
+        c_->trace_on = trace_;
+    }
+    OwnWays(const OwnWays &) = delete;
+    OwnWays &operator=(const OwnWays &) = delete;
+    void toSide() const { ck(hemm_context_set_stream(c_->dev, side_)); }
+    void toOwn() const { ck(hemm_context_set_stream(c_->dev, own_)); }
+    void marksOn() const { c_->trace_on = trace_; }
+    hipStream_t side() const { return side_; }
+
+  private:
+    const Context &c_;
+    void *own_;
+    bool trace_;
+    hipStream_t side_;
+};
+
+// What follows the two chains: the baby rotations of tau(B) (level T+1) go on where it was made, on the side stream,
+// while the rotation sources of sigma(A) (level T+2) are made on the context's; the chains meet in front of the main
+// loop, where the unshifted term low_a (x) tau(B) is taken.  Complex-packed cells: k / 2 shifts of two columns / rows.
+CtxtTensor ownWaysShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, const u64 *low_a,
+                               std::vector<Plaintext> &cm, i64 rows, i64 cols, i64 k, i64 w, u64 batch, bool spread,
+                               hipStream_t side, bool add_conj) {
+    const Context &c = eval.getContext();
+    DeviceBuffer U;
+    Ciphertext acc(c);
+    acc.allocate(3, T + 1, 1);
+    CtxtTensor res(c, rows, cols, w);
+    i64 g = 1;
+    bsgsShiftProduct(eval, T, sigma_a, tau_b, acc, cm, k, k / 2, 2, w, batch, &U, &g, spread ? (u64)(k * w) : 0, false,
+                     side, low_a);
+    c->mark("main loop");
+    bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
+    c->mark("giant steps");
+    if (spread) res.get().occupied_ = (u64)(k * w);   // the product sits in the first block, the rest is empty
+    return res;
+}
 }  // namespace
 
 namespace {
@@ -1156,39 +1206,17 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
         if (rows == k && cols == k && k / 2 >= 4 && ((u64)(k * w) == slots || spread)) {
             const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
             std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
-            void *own = hemm_context_stream(c->dev);
-            const hipStream_t side = c->forkSide();
-            struct Back {   // (the phase marks of the two chains would interleave: none while both run)
-                const Context &c;
-                void *own;
-                bool trace;
-                ~Back() {
-                    (void)hemm_context_set_stream(c->dev, own);
-                    c->joinSide();
-                    c->trace_on = trace;
-                }
-            } back{c, own, c->trace_on};
-            c->trace_on = false;
-            ck(hemm_context_set_stream(c->dev, side));
+            OwnWays ways(c);
+            ways.toSide();
             const Ciphertext tb = tr.lowerAndTransformFused(eval, op2.get(), MaskKind::PackedVertical, shape_b, T + 1);
-            ck(hemm_context_set_stream(c->dev, own));
+            ways.toOwn();
             const Ciphertext sa = tr.lowerAndTransformFused(eval, op1.get(), MaskKind::PackedHorizontal, shape_a, T + 2);
             DeviceBuffer low_a(c, 2 * lo * N);
             levelDownOneBatch(c, sa.buf_.data(), 2, T + 2, low_a.data());
-            c->trace_on = back.trace;
+            ways.marksOn();
             c->mark("transforms");
-            DeviceBuffer U;
-            Ciphertext acc(c);
-            acc.allocate(3, T + 1, 1);
-            CtxtTensor res(c, rows, cols, w);
-            i64 g = 1;
-            bsgsShiftProduct(eval, T, sa.buf_.data(), tb.buf_.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g,
-                             spread ? (u64)(k * w) : 0, false, side, low_a.data());
-            c->mark("main loop");
-            bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res);
-            c->mark("giant steps");
-            if (spread) res.get().occupied_ = (u64)(k * w);
-            return res;
+            return ownWaysShiftProduct(eval, T, sa.buf_.data(), tb.buf_.data(), low_a.data(), cm, rows, cols, k, w, batch,
+                                       spread, ways.side(), false);
         }
     }
     // both operands a level above what the reference asks of B: sigma and tau share one launch chain, as in the
@@ -1391,23 +1419,10 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
             std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
             DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
             const std::vector<u64> one(La + 1, 1);
-            void *own = hemm_context_stream(c->dev);
             {
-                const hipStream_t side = c->forkSide();
-                // (the phase marks of the two chains would interleave: one mark after both)
-                struct Back {
-                    const Context &c;
-                    void *own;
-                    bool trace;
-                    ~Back() {
-                        (void)hemm_context_set_stream(c->dev, own);
-                        c->joinSide();
-                        c->trace_on = trace;
-                    }
-                } back{c, own, c->trace_on};
-                c->trace_on = false;
+                OwnWays ways(c);
                 // B one level below A, on the side stream: truncated to T+4, packed by rows (T+3), tau in two stages (T+1)
-                ck(hemm_context_set_stream(c->dev, side));
+                ways.toSide();
                 {
                     DeviceBuffer jb(c, 2 * (Lb + 1) * N), pk(c, 2 * Lb * N);
                     ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), one.data(), jb.data(), (Lb + 1) * N,
@@ -1418,7 +1433,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                     const MaskKind kind = MaskKind::PackedVertical;
                     tr.diagonalTransformTwoStage(eval, pk.data(), 1, Lb - 1, &kind, &shape_b, tb.data());
                 }
-                ck(hemm_context_set_stream(c->dev, own));
+                ways.toOwn();
                 // A on the context's stream: truncated to T+5, packed by columns (T+4), sigma in two stages (T+2); from T+4:
                 // packed to T+3, sigma in one stage
                 {
@@ -1438,20 +1453,10 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                 levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
                 // the side chain stays open: the baby rotations of tau(B) follow its transform there while the sources
                 // of sigma(A) are made here, and the two meet in front of the main loop
-                c->trace_on = back.trace;
+                ways.marksOn();
                 c->mark("packing and transforms of A");
-                DeviceBuffer U;
-                Ciphertext acc(c);
-                acc.allocate(3, T + 1, 1);
-                CtxtTensor res(c, rows, cols, w);
-                i64 g = 1;
-                bsgsShiftProduct(eval, T, sa.data(), tb.data(), acc, cm, k, k / 2, 2, w, batch, &U, &g,
-                                 spread ? (u64)(k * w) : 0, false, side, low_a.data());
-                c->mark("main loop");
-                bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
-                c->mark("giant steps");
-                if (spread) res.get().occupied_ = (u64)(k * w);
-                return res;
+                return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
+                                           ways.side(), add_conj);
             }
         }
     }
