@@ -232,6 +232,20 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
 CtxtTensor multMatMatCCReUseFused(const HomEvaluator &eval, const std::vector<Ciphertext> &tmp, const CtxtTensor &b,
                                   u64 step, bool rescale_after, u64 batch = 16);
 // left rotations (in slots) whose direct keys the batched schedules use
+// Rotate-and-sum as hoisted sums.  The reference adds log2(count) rotations one after the other (x += rot(x, 2^k unit));
+// the same sum, out = sum_{i < count} leftRotate(in, i * unit) (unit < 0: to the right; count a power of two), is taken
+// here in at most two stages -- i = i0 + b i1 -- each ONE ModUp, ONE sum of the stage's rotations (its unrotated input a
+// term without a key) and ONE ModDown, for all jobs of the call together.  The jobs share level and count; `in` may be
+// `out`.
+struct RotateSumJob {
+    const Ciphertext *in;
+    i64 unit;
+    Ciphertext *out;
+};
+void rotateSumFused(const HomEvaluator &eval, const std::vector<RotateSumJob> &jobs, u64 count);
+// left rotation amounts whose keys rotateSumFused needs for (unit, count)
+std::vector<u64> rotateSumRotations(i64 unit, u64 count, u64 log_slots);
+
 std::vector<u64> fusedRotations(const TileTensorShape &shape, u64 log_slots, bool packed, bool need_rows);
 // the same for multMatMatFused; square_rots receives the giant steps that also need KeyPack::galoisSquareKey
 std::vector<u64> fusedCcmmRotations(const TileTensorShape &shape, u64 log_slots, std::vector<u64> &square_rots,

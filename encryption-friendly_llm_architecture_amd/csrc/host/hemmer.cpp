@@ -182,6 +182,14 @@ std::vector<u64> logSteps(u64 bound, u64 slots) {
 
 void HEMMer::reduceRowSumWithScaledMask(CtxtTensor &tensor, const Message &mask) const {
     const u64 w = (u64)tensor.getBlockWidth(), slots = u64(1) << log_slots_;
+    if (fused_ && (w & (w - 1)) == 0) {   // the same sums, each as hoisted sums of its rotations
+        ensureRotationKeys(rotateSumRotations(1, w, log_slots_));
+        ensureRotationKeys(rotateSumRotations(-1, w, log_slots_));
+        rotateSumFused(eval_, {{&tensor.get(), 1, &tensor.get()}}, w);
+        eval_.mult(tensor.get(), mask, tensor.get());
+        rotateSumFused(eval_, {{&tensor.get(), -1, &tensor.get()}}, w);
+        return;
+    }
     ensureRotationKeys(logSteps(w, slots));
     Ciphertext tmp(context_);
     for (u64 i = 1; i < w; i <<= 1) {
@@ -197,6 +205,23 @@ void HEMMer::reduceRowSumWithScaledMask(CtxtTensor &tensor, const Message &mask)
 
 void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
     const u64 n = (u64)dim_, slots = u64(1) << log_slots_;
+    Matrix first(dim_, dim_, 0.0), last(dim_, dim_, 0.0);
+    for (i64 r = 0; r < dim_; r++) {
+        first.at(r, 0) = 1.0;
+        last.at(r, dim_ - 1) = 1.0;
+    }
+    if (fused_ && n >= 4 && (n & (n - 1)) == 0 && a.getLevel() == b.getLevel()) {
+        // both tensors through the same launch chains: a to the left and b to the right, then the other way round
+        for (i64 unit : {i64(1), i64(-1)}) {
+            ensureRotationKeys(rotateSumRotations(unit, n / 2, log_slots_));
+            ensureRotationKeys(rotateSumRotations(unit, n, log_slots_));
+        }
+        rotateSumFused(eval_, {{&a.get(), 1, &a.get()}, {&b.get(), -1, &b.get()}}, n / 2);
+        eval_.mult(a.get(), message2(first, first), a.get());
+        eval_.mult(b.get(), message2(last, last), b.get());
+        rotateSumFused(eval_, {{&a.get(), -1, &a.get()}, {&b.get(), 1, &b.get()}}, n);
+        return;
+    }
     ensureRotationKeys(logSteps(n, slots));
     Ciphertext tmp(context_);
     for (u64 rot = 1; rot < n / 2; rot <<= 1) {
@@ -204,11 +229,6 @@ void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
         eval_.add(a.get(), tmp, a.get());
         eval_.rightRotate(b.get(), rot, tmp);
         eval_.add(b.get(), tmp, b.get());
-    }
-    Matrix first(dim_, dim_, 0.0), last(dim_, dim_, 0.0);
-    for (i64 r = 0; r < dim_; r++) {
-        first.at(r, 0) = 1.0;
-        last.at(r, dim_ - 1) = 1.0;
     }
     eval_.mult(a.get(), message2(first, first), a.get());
     eval_.mult(b.get(), message2(last, last), b.get());
@@ -237,8 +257,6 @@ void HEMMer::maskFirstColInplace(CtxtTensor &tensor) const {
 void HEMMer::rowMoments(const std::vector<CtxtTensor> &tiles, Real inv_count, CtxtTensor &mean,
                         CtxtTensor &mean_square) const {
     if (tiles.empty()) throw std::invalid_argument("[rowMoments] no tiles");
-    const u64 w = (u64)tiles[0].getBlockWidth(), slots = u64(1) << log_slots_;
-    ensureRotationKeys(logSteps(w, slots));
     Ciphertext tmp(context_);
     mean.get() = tiles[0].get();
     eval_.tensor(tiles[0].get(), tiles[0].get(), mean_square.get());
@@ -846,7 +864,7 @@ std::vector<std::vector<CtxtTensor>> HEMMer::splitWeightRows(const CtxtTensor &w
     std::vector<u64> rots{w};
     for (u64 i = 1; i < count; i++) rots.push_back(i * 2 * w);
     ensureRotationKeys(rots);
-    ensureLogStepKeys(1, (i64)n, (i64)w);
+    if (!(fused_ && (n & (n - 1)) == 0)) ensureLogStepKeys(1, (i64)n, (i64)w);
     std::vector<std::vector<CtxtTensor>> out;
     CtxtTensor tmp{weight};
     for (u64 i = 0; i < count; i++) {
@@ -856,6 +874,14 @@ std::vector<std::vector<CtxtTensor>> HEMMer::splitWeightRows(const CtxtTensor &w
         eval_.leftRotate(pair[1].get(), w, pair[1].get());
         maskFirstRowInplace(pair[1]);
         out.push_back(std::move(pair));
+    }
+    if (fused_ && (n & (n - 1)) == 0) {   // row 0 copied to every row: all 2 * count tensors through the same launch chains
+        ensureRotationKeys(rotateSumRotations(-(i64)w, n, log_slots_));
+        std::vector<RotateSumJob> jobs;
+        for (auto &pair : out)
+            for (auto &x : pair) jobs.push_back({&x.get(), -(i64)w, &x.get()});
+        rotateSumFused(eval_, jobs, n);
+        return out;
     }
     Ciphertext t(context_);
     for (auto &pair : out)
@@ -873,7 +899,7 @@ std::vector<CtxtTensor> HEMMer::loraRank2Down(const std::vector<CtxtTensor> &cur
     CtxtTensor wa{lora_wa};
     eval_.levelDown(wa.get(), weight_level, wa.get());
     auto weights = splitWeightRows(wa, cur.size());
-    ensureLogStepKeys(1, (i64)w, 1);
+    if (!(fused_ && (w & (w - 1)) == 0)) ensureLogStepKeys(1, (i64)w, 1);
     std::vector<CtxtTensor> out;
     Ciphertext t(context_);
     for (u64 j = 0; j < 2; j++) {
@@ -883,9 +909,14 @@ std::vector<CtxtTensor> HEMMer::loraRank2Down(const std::vector<CtxtTensor> &cur
             eval_.mult(cur[i].get(), weights[i][j].get(), t);
             eval_.add(acc.get(), t, acc.get());
         }
-        for (u64 rot = 1; rot < w; rot <<= 1) {
-            eval_.leftRotate(acc.get(), rot, t);
-            eval_.add(acc.get(), t, acc.get());
+        if (fused_ && (w & (w - 1)) == 0) {
+            ensureRotationKeys(rotateSumRotations(1, w, log_slots_));
+            rotateSumFused(eval_, {{&acc.get(), 1, &acc.get()}}, w);
+        } else {
+            for (u64 rot = 1; rot < w; rot <<= 1) {
+                eval_.leftRotate(acc.get(), rot, t);
+                eval_.add(acc.get(), t, acc.get());
+            }
         }
         maskFirstColOnlyInplace(acc);
         out.push_back(std::move(acc));
@@ -899,14 +930,20 @@ std::vector<CtxtTensor> HEMMer::loraRank2Up(const std::vector<CtxtTensor> &xa_in
     CtxtTensor wb{lora_wb};
     eval_.levelDown(wb.get(), weight_level, wb.get());
     auto weights = splitWeightRows(wb, n_out);
-    ensureLogStepKeys(1, (i64)w, 1);
+    if (!(fused_ && (w & (w - 1)) == 0)) ensureLogStepKeys(1, (i64)w, 1);
     std::vector<CtxtTensor> xa{xa_in};
     Ciphertext t(context_);
-    for (auto &x : xa)
-        for (u64 rot = 1; rot < w; rot <<= 1) {
-            eval_.rightRotate(x.get(), rot, t);
-            eval_.add(x.get(), t, x.get());
-        }
+    if (fused_ && (w & (w - 1)) == 0 && xa[0].getLevel() == xa[1].getLevel() &&
+        xa[0].get().getRescaleCounter() == xa[1].get().getRescaleCounter()) {
+        ensureRotationKeys(rotateSumRotations(-1, w, log_slots_));
+        rotateSumFused(eval_, {{&xa[0].get(), -1, &xa[0].get()}, {&xa[1].get(), -1, &xa[1].get()}}, w);
+    } else {
+        for (auto &x : xa)
+            for (u64 rot = 1; rot < w; rot <<= 1) {
+                eval_.rightRotate(x.get(), rot, t);
+                eval_.add(x.get(), t, x.get());
+            }
+    }
     std::vector<CtxtTensor> out;
     for (u64 i = 0; i < n_out; i++) {
         CtxtTensor y{wb};

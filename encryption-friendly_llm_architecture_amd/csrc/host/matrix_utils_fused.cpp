@@ -1478,6 +1478,78 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1, false, add_conj);
 }
 
+namespace {
+// stages (rotations per stage, multiplier of the unit): one stage up to four terms, else i = i0 + b i1 with
+// b = 2^ceil(log2(count) / 2)
+std::vector<std::pair<u64, u64>> rotateSumStages(u64 count) {
+    if (count == 0 || (count & (count - 1)) != 0) throw std::invalid_argument("[rotateSum] the count must be a power of two");
+    if (count <= 4) return {{count, 1}};
+    u64 b = 1;
+    while (b * b < count) b <<= 1;
+    return {{b, 1}, {count / b, b}};
+}
+}  // namespace
+
+std::vector<u64> rotateSumRotations(i64 unit, u64 count, u64 log_slots) {
+    const i64 slots = i64(1) << log_slots;
+    std::vector<u64> r;
+    for (const auto &st : rotateSumStages(count))
+        for (u64 i = 1; i < st.first; i++) {
+            const u64 v = (u64)((((i64)(i * st.second) * unit) % slots + slots) % slots);
+            if (v != 0) r.push_back(v);
+        }
+    return r;
+}
+
+void rotateSumFused(const HomEvaluator &eval, const std::vector<RotateSumJob> &jobs, u64 count) {
+    if (jobs.empty()) return;
+    const Context &c = eval.getContext();
+    const KeyPack &pack = eval.getKeyPack();
+    const Rot rot(c);
+    const size_t n = jobs.size();
+    const u64 level = jobs[0].in->getLevel(), rc = jobs[0].in->getRescaleCounter();
+    const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
+    for (const RotateSumJob &j : jobs)
+        if (j.in == nullptr || j.out == nullptr || j.in->getNumPoly() != 2 || j.in->getLevel() != level ||
+            j.in->getRescaleCounter() != rc)
+            throw std::invalid_argument("[rotateSum] the operands must share one level and have two polynomials.");
+    const auto stages = rotateSumStages(count);
+    DeviceBuffer cur(c, n * ctw), nxt(c, n * ctw);
+    for (size_t q = 0; q < n; q++)
+        for (u64 p = 0; p < 2; p++)
+            (void)hipMemcpyAsync(cur.data() + q * ctw + p * nq * N, jobs[q].in->buf_.data() + p * jobs[q].in->polyStride(),
+                                 nq * N * 8, hipMemcpyDeviceToDevice, c->stream());
+    for (const auto &st : stages) {
+        if (st.first <= 1) continue;
+        // raw b polynomials: the launch multiplies them by P itself (one launch less than premultiplied sources)
+        const Sources x = extendSources(c, cur.data(), n, nq, nullptr, false);
+        std::vector<hemm_rot_term> terms;
+        std::vector<uint32_t> off{0};
+        for (size_t q = 0; q < n; q++) {
+            const u64 *b = cur.data() + q * ctw, *a = b + nq * N;
+            for (u64 i = 1; i < st.first; i++) {
+                const i64 amount = (i64)(i * st.second) * jobs[q].unit;
+                if (rot.norm(amount) == 0)   // a whole turn: the input itself once more
+                    terms.push_back(keylessTerm(b, a, nullptr));
+                else
+                    terms.push_back(term(x.extOf(q), x.pbOf(q), pack, rot.galois(amount), nullptr));
+            }
+            terms.push_back(keylessTerm(b, a, nullptr));   // i = 0: no key switch
+            off.push_back((uint32_t)terms.size());
+        }
+        DeviceBuffer y(c, n * 2 * E * N), ws(c, n * ctw);
+        ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n, (uint32_t)nq, x.premultiplied(), 0, y.data(),
+                                nxt.data(), nq * N, ws.data(), nullptr));
+        std::swap(cur, nxt);
+    }
+    for (size_t q = 0; q < n; q++) {
+        Ciphertext res(c);
+        res.allocate(2, level, rc);
+        (void)hipMemcpyAsync(res.buf_.data(), cur.data() + q * ctw, ctw * 8, hipMemcpyDeviceToDevice, c->stream());
+        *jobs[q].out = std::move(res);   // (occupied slots: unknown, as allocate leaves them)
+    }
+}
+
 // Ciphertext x ciphertext re-use product: sum_k tmp[k] (x) rho^(k step)(b) with tmp from multMatMatPre(Fused) and
 // b = tau(B).  The reference rotates b by `step` in a chain, one key switch after the other; here every rotation
 // comes from the same ModUp of b through its direct key (hoisted), 2 * batch rotations per launch chain with one

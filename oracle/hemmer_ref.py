@@ -30,6 +30,18 @@ def pow2ceil(v):
 # --------------------------------------------------------------------------------------------
 # slot simulator
 # --------------------------------------------------------------------------------------------
+def rotate_sum_stages(count):
+    """(rotations per stage, multiplier of the unit): one stage up to four terms, else i = i0 + b i1 with
+    b = 2^ceil(log2(count) / 2)."""
+    assert count >= 1 and count & (count - 1) == 0
+    if count <= 4:
+        return [(count, 1)]
+    b = 1
+    while b * b < count:
+        b <<= 1
+    return [(b, 1), (count // b, b)]
+
+
 class SimCt:
     def __init__(self, z, level, rc=0):
         self.z, self.level, self.rc = np.asarray(z, dtype=np.complex128), level, rc
@@ -122,6 +134,13 @@ class SlotSim:
 
     def right_rotate(self, x, r):
         return SimCt(np.roll(x.z, r % self.slots), x.level, x.rc)
+
+    def rotate_sum(self, x, unit, count):
+        """sum_{i < count} leftRotate(x, i * unit) (unit < 0: to the right)."""
+        z = np.zeros_like(x.z)
+        for i in range(count):
+            z = z + np.roll(x.z, -((i * unit) % self.slots))
+        return SimCt(z, x.level, x.rc)
 
     def conjugate(self, x):
         return SimCt(np.conj(x.z), x.level, x.rc)
@@ -236,6 +255,25 @@ class OracleEval:
 
     def right_rotate(self, x, r):
         return self.o.right_rotate(x, r)
+
+    def rotate_sum(self, x, unit, count):
+        """sum_{i < count} leftRotate(x, i * unit) (unit < 0: to the right) as hoisted sums (rotateSumFused): at most
+        two stages, i = i0 + b i1, each one ModUp, one sum of the stage's rotations with the unrotated input as a term
+        without a key, and one ModDown."""
+        from .oracle import Ct
+        o = self.o
+        for cnt, mul in rotate_sum_stages(count):
+            if cnt <= 1:
+                continue
+            ext = o.modup(x.data[1])
+            terms = []
+            for i in range(1, cnt):
+                r = (i * mul * unit) % o.slots
+                terms.append((x.data[1], x.data[0], ("none",), None) if r == 0 else (ext, x.data[0], r, None))
+            terms.append((x.data[1], x.data[0], ("none",), None))
+            y = o.hoisted_sum(terms, x.nq)
+            x = Ct(o.moddown_drop(y, x.nq, False), x.scale)
+        return x
 
     def conjugate(self, x):
         return self.o.conjugate(x)
@@ -1345,7 +1383,7 @@ def _first_col_only_mask(n, slots):
     return _message2(m, np.zeros((n, n)), slots)
 
 
-def _split_weight_rows(ev, wt, count, n, w):
+def _split_weight_rows(ev, wt, count, n, w, hoisted=False):
     """Rows 2i and 2i+1 of the weight tile, each moved to row 0, masked and copied to all n rows
     (:2222-2251, :2294-2335)."""
     first = _first_row_mask(n, ev.slots)
@@ -1356,6 +1394,9 @@ def _split_weight_rows(ev, wt, count, n, w):
         out.append(pair)
     for pair in out:
         for j in range(2):
+            if hoisted:
+                pair[j] = ev.rotate_sum(pair[j], -w, n)
+                continue
             rot = 1
             while rot < n:
                 pair[j] = ev.add(pair[j], ev.right_rotate(pair[j], rot * w))
@@ -1363,32 +1404,38 @@ def _split_weight_rows(ev, wt, count, n, w):
     return out
 
 
-def lora_rank2_down(ev, cur, wa, n, w, weight_level):
+def lora_rank2_down(ev, cur, wa, n, w, weight_level, hoisted=False):
     """X a_0 and X a_1 in column 0 of the left tile: row 2i+j of `wa` holds column j of A for the i-th pair
-    of activation tiles (:2203-2283)."""
+    of activation tiles (:2203-2283).  hoisted: every rotate-and-sum as hoisted sums (the batched schedule)."""
     wa = ev.level_down(wa, weight_level)
-    wts = _split_weight_rows(ev, wa, len(cur), n, w)
+    wts = _split_weight_rows(ev, wa, len(cur), n, w, hoisted)
     out = []
     for j in range(2):
         acc = None
         for i, x in enumerate(cur):
             t = ev.mult(x, wts[i][j])
             acc = t if acc is None else ev.add(acc, t)
-        rot = 1
-        while rot < w:
-            acc = ev.add(acc, ev.left_rotate(acc, rot))
-            rot <<= 1
+        if hoisted:
+            acc = ev.rotate_sum(acc, 1, w)
+        else:
+            rot = 1
+            while rot < w:
+                acc = ev.add(acc, ev.left_rotate(acc, rot))
+                rot <<= 1
         out.append(_mult_msg(ev, acc, _first_col_only_mask(n, ev.slots)))
     return out
 
 
-def lora_rank2_up(ev, xa, wb, n_out, n, w, weight_level):
+def lora_rank2_up(ev, xa, wb, n_out, n, w, weight_level, hoisted=False):
     """(X A) B for n_out pairs of output tiles: row 2i+j of `wb` holds row j of B for output pair i
     (:2287-2358)."""
     wb = ev.level_down(wb, weight_level)
-    wts = _split_weight_rows(ev, wb, n_out, n, w)
+    wts = _split_weight_rows(ev, wb, n_out, n, w, hoisted)
     xa = list(xa)
     for j in range(2):
+        if hoisted:
+            xa[j] = ev.rotate_sum(xa[j], -1, w)
+            continue
         rot = 1
         while rot < w:
             xa[j] = ev.add(xa[j], ev.right_rotate(xa[j], rot))
@@ -1405,7 +1452,11 @@ def _message2(a, b, slots):
     return m
 
 
-def reduce_row_sum_with_scaled_mask(ev, x, mask_msg, w):
+def reduce_row_sum_with_scaled_mask(ev, x, mask_msg, w, hoisted=False):
+    if hoisted:
+        x = ev.rotate_sum(x, 1, w)
+        x = ev.mult_pt(x, ev.encode(mask_msg, ev.level_of(x)))
+        return ev.rotate_sum(x, -1, w)
     i = 1
     while i < w:
         x = ev.add(x, ev.left_rotate(x, i))
@@ -1418,15 +1469,20 @@ def reduce_row_sum_with_scaled_mask(ev, x, mask_msg, w):
     return x
 
 
-def one_mat_rot_sum(ev, a, b, n):
+def one_mat_rot_sum(ev, a, b, n, hoisted=False):
+    first, last = np.zeros((n, n)), np.zeros((n, n))
+    first[:, 0] = 1.0
+    last[:, n - 1] = 1.0
+    if hoisted:
+        a, b = ev.rotate_sum(a, 1, n // 2), ev.rotate_sum(b, -1, n // 2)
+        a = ev.mult_pt(a, ev.encode(_message2(first, first, ev.slots), ev.level_of(a)))
+        b = ev.mult_pt(b, ev.encode(_message2(last, last, ev.slots), ev.level_of(b)))
+        return ev.rotate_sum(a, -1, n), ev.rotate_sum(b, 1, n)
     rot = 1
     while rot < n // 2:
         a = ev.add(a, ev.left_rotate(a, rot))
         b = ev.add(b, ev.right_rotate(b, rot))
         rot <<= 1
-    first, last = np.zeros((n, n)), np.zeros((n, n))
-    first[:, 0] = 1.0
-    last[:, n - 1] = 1.0
     a = ev.mult_pt(a, ev.encode(_message2(first, first, ev.slots), ev.level_of(a)))
     b = ev.mult_pt(b, ev.encode(_message2(last, last, ev.slots), ev.level_of(b)))
     rot = 1
@@ -1445,7 +1501,7 @@ def mask_right_left(ev, x, n):
             ev.mult_pt(x, ev.encode(_message2(right, right, ev.slots), ev.level_of(x))))
 
 
-def row_moments(ev, tiles, inv_count, n):
+def row_moments(ev, tiles, inv_count, n, hoisted=False):
     mean = tiles[0]
     sq = ev.tensor(tiles[0], tiles[0])
     for t in tiles[1:]:
@@ -1455,5 +1511,5 @@ def row_moments(ev, tiles, inv_count, n):
     scaled = np.zeros((n, n))
     scaled[:, 0] = inv_count
     mask = _message2(scaled, np.zeros((n, n)), ev.slots)
-    return (reduce_row_sum_with_scaled_mask(ev, mean, mask, 2 * n),
-            reduce_row_sum_with_scaled_mask(ev, sq, mask, 2 * n))
+    return (reduce_row_sum_with_scaled_mask(ev, mean, mask, 2 * n, hoisted),
+            reduce_row_sum_with_scaled_mask(ev, sq, mask, 2 * n, hoisted))

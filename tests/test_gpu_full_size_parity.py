@@ -383,13 +383,13 @@ def test_preset_polynomials_reductions_and_low_rank_product_residues_bit_exact(p
     scaled[:, 0] = 1.0 / (2 * n)
     red = x.clone()
     H.reduce_row_sum_with_scaled_mask(red, scaled, np.zeros((n, n)))
-    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n)
+    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n, True)
     assert np.array_equal(red.residues(), want.data)
     mean = np.concatenate([A, B], axis=1).mean(axis=1, keepdims=True)
     assert np.abs(H.decrypt2(red)[0] - mean).max() < 2.0 ** -18
     a, b = x.clone(), x.clone()
     H.one_mat_rot_sum_inplace(a, b)
-    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n)
+    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n, True)
     assert np.array_equal(a.residues(), wa.data) and np.array_equal(b.residues(), wb.data)
     # a low-rank product: X (two tiles) times the block of ld columns of the LoRA factor, then repacked into one column block
     blk = 3
@@ -459,11 +459,11 @@ def test_preset_other_low_rank_forms_residues_bit_exact(preset):
     cur, cwa, cwb = [enc2(X)], enc2(wa), enc2(wb)
     ocur, owa, owb = [as_oracle(orc, c) for c in cur], as_oracle(orc, cwa), as_oracle(orc, cwb)
     xa = H.lora_rank2_down(cur, cwa, weight_level=7)
-    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7)
+    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7, True)
     for j in range(2):
         assert np.array_equal(xa[j].residues(), oxa[j].data)
     out = H.lora_rank2_up(xa, cwb, m, weight_level=4)
-    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4)
+    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4, True)
     assert np.array_equal(out[0].residues(), oout[0].data)
     z = H.decrypt_slots(out[0]).real.reshape(n, w)
     assert np.abs(z - X @ A2 @ B2).max() < 2.0 ** -10

@@ -520,9 +520,20 @@ def test_transpose_complex_packing_inplace(small, fused, target_level):
         assert np.abs(z[:, half * n:(half + 1) * n] - P[:, half * n:(half + 1) * n].T).max() < 2 ** -18
 
 
-def test_rotate_and_sum_reductions(small):
-    """Row reductions on the pair layout: residues against the oracle restatement, values against numpy."""
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_rotate_and_sum_reductions(small, fused):
+    """Row reductions on the pair layout: residues against the oracle restatement, values against numpy.  The
+    reference's order adds log2 rotations one after the other; the batched schedule takes the same sums as hoisted sums
+    of all their rotations (HELLM::rotateSumFused)."""
     H, orc, ev = small
+    H.set_schedule(fused)
+    try:
+        _rotate_and_sum_reductions(H, orc, ev, fused)
+    finally:
+        H.set_schedule(True)
+
+
+def _rotate_and_sum_reductions(H, orc, ev, fused):
     n = 16
     rng = np.random.default_rng(13)
     A, B = rng.normal(size=(n, n)), rng.normal(size=(n, n))
@@ -532,14 +543,14 @@ def test_rotate_and_sum_reductions(small):
     scaled[:, 0] = 1.0 / (2 * n)
     got = x.clone()
     H.reduce_row_sum_with_scaled_mask(got, scaled, np.zeros((n, n)))
-    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n)
+    want = R.reduce_row_sum_with_scaled_mask(ev, ox, R._message2(scaled, np.zeros((n, n)), orc.slots), 2 * n, fused)
     assert np.array_equal(got.residues(), want.data)
     d = H.decrypt2(got)
     mean = np.concatenate([A, B], axis=1).mean(axis=1, keepdims=True)
     assert np.abs(d[0] - mean).max() < 2 ** -20 and np.abs(d[1] - mean).max() < 2 ** -20
     a, b = x.clone(), x.clone()
     H.one_mat_rot_sum_inplace(a, b)
-    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n)
+    wa, wb = R.one_mat_rot_sum(ev, ox, ox, n, fused)
     assert np.array_equal(a.residues(), wa.data) and np.array_equal(b.residues(), wb.data)
     assert np.abs(H.decrypt2(a)[1] - B[:, : n // 2].sum(axis=1, keepdims=True)).max() < 2 ** -18
     l, r = H.mask_right_left(x)
@@ -550,7 +561,7 @@ def test_rotate_and_sum_reductions(small):
     tiles = [H.encrypt2(rng.normal(size=(n, n)), rng.normal(size=(n, n))) for _ in range(3)]
     rows = np.concatenate([np.concatenate(H.decrypt2(t), axis=1) for t in tiles], axis=1)
     m, sq = H.row_moments(tiles, 1.0 / rows.shape[1])
-    wm, wsq = R.row_moments(ev, [to_oracle(orc, t) for t in tiles], 1.0 / rows.shape[1], n)
+    wm, wsq = R.row_moments(ev, [to_oracle(orc, t) for t in tiles], 1.0 / rows.shape[1], n, fused)
     assert np.array_equal(m.residues(), wm.data) and np.array_equal(sq.residues(), wsq.data)
     assert np.abs(H.decrypt2(m)[0] - rows.mean(axis=1, keepdims=True)).max() < 2 ** -18
     assert np.abs(H.decrypt2(sq)[1] - (rows ** 2).mean(axis=1, keepdims=True)).max() < 2 ** -16

@@ -157,9 +157,19 @@ def test_repack_lora_opti(small):
     assert np.abs(out[:, n:] - (2 * A0 + B1 + 1j * A0)).max() < 2 ** -16
 
 
-def test_lora_rank2_elementwise_path(small):
-    """Element-wise rank-2 form: residues against the oracle, values against float64."""
+@pytest.mark.parametrize("fused", [False, True], ids=["reference-order", "batched"])
+def test_lora_rank2_elementwise_path(small, fused):
+    """Element-wise rank-2 form: residues against the oracle, values against float64; the rotate-and-sum steps in the
+    reference's order and as hoisted sums."""
     H, orc, ev = small
+    H.set_schedule(fused)
+    try:
+        _lora_rank2_elementwise_path(H, orc, ev, fused)
+    finally:
+        H.set_schedule(True)
+
+
+def _lora_rank2_elementwise_path(H, orc, ev, fused):
     n, w, m = N_TILE, W, 2
     rng = np.random.default_rng(25)
     X = rng.uniform(-1, 1, (n, 2 * n * m))
@@ -175,13 +185,13 @@ def test_lora_rank2_elementwise_path(small):
     cwa, cwb = enc2(wa), enc2(wb)
     ocur, owa, owb = [to_oracle(orc, c) for c in cur], to_oracle(orc, cwa), to_oracle(orc, cwb)
     xa = H.lora_rank2_down(cur, cwa, weight_level=7)
-    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7)
+    oxa = R.lora_rank2_down(ev, ocur, owa, n, w, 7, fused)
     for j in range(2):
         assert np.array_equal(xa[j].residues(), oxa[j].data)
         z = H.decrypt_slots(xa[j]).real.reshape(n, w)
         assert np.abs(z[:, 0] - X @ A[:, j]).max() < 2 ** -16 and np.abs(z[:, 1:]).max() < 2 ** -16
     out = H.lora_rank2_up(xa, cwb, m, weight_level=4)
-    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4)
+    oout = R.lora_rank2_up(ev, oxa, owb, m, n, w, 4, fused)
     want = X @ A @ B
     for i in range(m):
         assert np.array_equal(out[i].residues(), oout[i].data)

@@ -113,8 +113,10 @@ def test_assemble_masks_are_complementary():
         assert cm[2 * i].sum() == i * slots // n and rm[2 * i].sum() == i * slots // n
 
 
-def test_rotate_and_sum_reductions():
-    """Row reductions on the pair layout against numpy (exact slot arithmetic)."""
+@pytest.mark.parametrize("hoisted", [False, True], ids=["log-steps", "hoisted-sums"])
+def test_rotate_and_sum_reductions(hoisted):
+    """Row reductions on the pair layout against numpy (exact slot arithmetic), in the reference's order (log2 steps)
+    and as the sums of all rotations the batched schedule takes."""
     n = 8
     ev = R.SlotSim(7, 12)                     # 2 n^2 = 128 slots
     rng = np.random.default_rng(5)
@@ -122,11 +124,11 @@ def test_rotate_and_sum_reductions():
     x = ev.encrypt(R._message2(A, B, ev.slots))
     scaled = np.zeros((n, n))
     scaled[:, 0] = 1.0 / (2 * n)
-    out = R.reduce_row_sum_with_scaled_mask(ev, x, R._message2(scaled, np.zeros((n, n)), ev.slots), 2 * n)
+    out = R.reduce_row_sum_with_scaled_mask(ev, x, R._message2(scaled, np.zeros((n, n)), ev.slots), 2 * n, hoisted)
     z = ev.decrypt(out).real.reshape(n, 2 * n)
     want = np.concatenate([A, B], axis=1).mean(axis=1, keepdims=True)
     assert np.abs(z - want).max() < 1e-12       # every slot of a row holds the row mean over both halves
-    a, b = R.one_mat_rot_sum(ev, x, x, n)
+    a, b = R.one_mat_rot_sum(ev, x, x, n, hoisted)
     za, zb = ev.decrypt(a).real.reshape(n, 2 * n), ev.decrypt(b).real.reshape(n, 2 * n)
     # a: sums of the first half of each tile row, spread over the tile row; b: sums of the second half
     assert np.abs(za[:, :n] - A[:, : n // 2].sum(axis=1, keepdims=True)).max() < 1e-12
@@ -135,7 +137,7 @@ def test_rotate_and_sum_reductions():
     assert np.abs(zb[:, n:] - B[:, n // 2:].sum(axis=1, keepdims=True)).max() < 1e-12
     tiles = [ev.encrypt(R._message2(rng.normal(size=(n, n)), rng.normal(size=(n, n)), ev.slots)) for _ in range(3)]
     rows = np.concatenate([ev.decrypt(t).real.reshape(n, 2 * n) for t in tiles], axis=1)
-    mean, sq = R.row_moments(ev, tiles, 1.0 / rows.shape[1], n)
+    mean, sq = R.row_moments(ev, tiles, 1.0 / rows.shape[1], n, hoisted)
     assert np.abs(ev.decrypt(mean).real.reshape(n, 2 * n) - rows.mean(axis=1, keepdims=True)).max() < 1e-12
     assert np.abs(ev.decrypt(sq).real.reshape(n, 2 * n) - (rows ** 2).mean(axis=1, keepdims=True)).max() < 1e-12
 

@@ -148,7 +148,8 @@ def test_repack_not_bts_and_split_in_two_closed_forms(sim):
         assert np.abs(left - want).max() < 1e-12 and np.abs(right - want).max() < 1e-12
 
 
-def test_lora_rank2_elementwise_path(sim):
+@pytest.mark.parametrize("hoisted", [False, True], ids=["log-steps", "hoisted-sums"])
+def test_lora_rank2_elementwise_path(sim, hoisted):
     """The production rank-2 form (element-wise products and rotate-and-sum, TransformerBlock.cpp:2199-2365):
     X (n x 6n, three pair-layout tiles) times A (6n x 2) gives two column ciphertexts, then times B (2 x 6n)."""
     n, w, m = N_TILE, W, 3
@@ -162,12 +163,12 @@ def test_lora_rank2_elementwise_path(sim):
             wa[2 * i + j] = A[2 * n * i:2 * n * (i + 1), j]
             wb[2 * i + j] = B[j, 2 * n * i:2 * n * (i + 1)]
     cur = [sim.encrypt(X[:, 2 * n * i:2 * n * (i + 1)].reshape(-1)) for i in range(m)]
-    xa = R.lora_rank2_down(sim, cur, sim.encrypt(wa.reshape(-1)), n, w, 9)
+    xa = R.lora_rank2_down(sim, cur, sim.encrypt(wa.reshape(-1)), n, w, 9, hoisted)
     for j in range(2):
         z = xa[j].z.real.reshape(n, w)
         assert np.abs(z[:, 0] - X @ A[:, j]).max() < 1e-12 and np.abs(z[:, 1:]).max() == 0
         assert xa[j].level == 6                    # 9 -> mask 8 -> product 7 -> mask 6
-    out = R.lora_rank2_up(sim, xa, sim.encrypt(wb.reshape(-1)), m, n, w, 6)
+    out = R.lora_rank2_up(sim, xa, sim.encrypt(wb.reshape(-1)), m, n, w, 6, hoisted)
     want = X @ A @ B
     for i in range(m):
         assert np.abs(out[i].z.real.reshape(n, w) - want[:, 2 * n * i:2 * n * (i + 1)]).max() < 1e-12

@@ -123,3 +123,19 @@ def test_complex_packed_ccmm_three_levels_above_target_over_oracle(env, single_t
     if not single_tile:
         assert np.abs(d[n:] - A[n:] @ B[n:]).max() < 2 ** -18
     assert np.abs(z.imag).max() < 2 ** -18
+
+
+@pytest.mark.parametrize("unit,count", [(1, 16), (-1, 32), (-16, 8), (3, 4), (5, 2), (32, 16)])
+def test_rotate_sum_as_hoisted_sums_over_oracle(env, unit, count):
+    """OracleEval.rotate_sum (at most two stages of one hoisted sum each, the unrotated input as a term without a
+    key) decrypts to the sum of the count rotations of its input; (32, 16) wraps round the 512 slots, so one of its
+    rotations is a whole turn."""
+    orc, ev, _ = env
+    rng = np.random.default_rng(9)
+    z = rng.uniform(-1, 1, orc.slots) + 1j * rng.uniform(-1, 1, orc.slots)
+    x = orc.encrypt(orc.encode(z, 5), 31)
+    got = orc.decrypt(ev.rotate_sum(x, unit, count))
+    want = sum(np.roll(z, -((i * unit) % orc.slots)) for i in range(count))
+    assert np.abs(got - want).max() < 2 ** -20
+    assert [c for c, _ in R.rotate_sum_stages(count)] == ([count] if count <= 4 else
+                                                          [1 << ((count.bit_length()) // 2), count >> ((count.bit_length()) // 2)])
