@@ -90,8 +90,20 @@ public:
     // scale_levels (optional, one per job): the level whose fixed scale job q's input carries -- an operand truncated to
     // `level` from a higher one; the masks of the first stage are then encoded at Delta_(level-1) q_level /
     // Delta_(scale level), which lands the result on the fixed scale of level - 1 without a levelDown in front.
+    // first_stage = 2: only the second stage; `in` is then what a first stage from `level` left at level - 1.
     void diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
-                                   const TileTensorShape *shapes, u64 *out, const u64 *scale_levels = nullptr);
+                                   const TileTensorShape *shapes, u64 *out, const u64 *scale_levels = nullptr,
+                                   int first_stage = 1);
+    // The complex packing (by rows for PackedVertical, by columns for PackedHorizontal) and the FIRST stage of the
+    // two-stage transform of `kind` as one linear map on the slots -- one hoisted sum, one mask level: the term that
+    // rotates by a slots carries sum over (stage rotation r, packing shift e) with r + e = a of
+    // stage mask_r (.) rho^r(packing mask_e).  in [2][level+1][N] (not packed yet) -> out [2][level][N], which the
+    // second stage takes to level - 1: packing and transform in two levels, for an operand with one level less than
+    // packing, stage 1 and stage 2 need on their own.
+    void packingStageOne(const HomEvaluator &eval, const u64 *in, u64 level, MaskKind kind, const TileTensorShape &shape,
+                         u64 *out);
+    // left rotations (in slots) packingStageOne uses
+    static std::vector<u64> packingStageOneRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots);
     // Brings `in` down to the level a transform ending at `end_level` starts from and runs it with the batched
     // launches: two stages from end_level + 2 when the operand is that high and the tile is square, otherwise one
     // stage from end_level + 1.
@@ -146,6 +158,8 @@ private:
     // an ordinary plaintext (the unrotated rows), parts 1 / 2 (main / wrapped columns) are over the extended basis; masks
     // that absorb a change of scale (scale level != 0) are all over the extended basis
     std::map<Key, Plaintext> two_stage_masks_;
+    // (kind, shape, level, 0) -> (left rotation in slots, mask over the extended basis) of packingStageOne
+    std::map<Key, std::vector<std::pair<u64, Plaintext>>> packing_stage_one_masks_;
     const Plaintext &twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape, u64 level,
                                   int stage, i64 r, int part, u64 from = 0);
 };

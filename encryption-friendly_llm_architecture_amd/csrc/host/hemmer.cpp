@@ -500,6 +500,11 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             ensureRotationKeys({1, slots - 1, (u64)w, slots - (u64)w});
             ensureRotationKeys(transformRotations(MaskKind::PackedHorizontal, w));
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
+            // three levels above the target with exact row rotations: B's packing and first tau stage are one composite
+            // map (MatrixTransformer::packingStageOne), with rotations of its own
+            if (std::min(a.getLevel(), b.getLevel()) == T + 3 && n >= 8 && (block == slots || (single && block < slots)))
+                ensureRotationKeys(MatrixTransformer::packingStageOneRotations(MaskKind::PackedVertical,
+                                                                               TileTensorShape(n, n, w), log_slots_));
             std::vector<u64> sq;
             // stacked tiles / unknown content keep their per-block products: the packed cells then shift through
             // masked pairs (no baby-step / giant-step split, which needs exact row rotations)

@@ -6,6 +6,8 @@
 
 #include <algorithm>
 #include <cmath>
+#include <map>
+#include <set>
 
 #include "../../../include/hemm.h"
 #include "HELLM/MatrixUtils.hpp"
@@ -594,14 +596,16 @@ Ciphertext MatrixTransformer::lowerAndTransformFused(const HomEvaluator &eval, c
 
 void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
                                                   const MaskKind *kinds, const TileTensorShape *shapes, u64 *out,
-                                                  const u64 *scale_levels) {
+                                                  const u64 *scale_levels, int first_stage) {
     const Context &c = eval.getContext();
     if (level < 2) throw std::invalid_argument("[diagonalTransform] level >= 2 is needed.");
     const u64 N = c->N;
-    DeviceBuffer mid(c, n_jobs * 2 * level * N);   // after stage 1: level - 1
-    for (int stage = 1; stage <= 2; stage++) {
+    if (first_stage != 1 && first_stage != 2) throw std::invalid_argument("[diagonalTransform] stage 1 or 2");
+    DeviceBuffer mid;   // after stage 1: level - 1
+    if (first_stage == 1) mid = DeviceBuffer(c, n_jobs * 2 * level * N);
+    for (int stage = first_stage; stage <= 2; stage++) {
         const u64 lvl = stage == 1 ? level : level - 1, nq = lvl + 1, E = nq + c->nP, ctw = 2 * nq * N;
-        const u64 *src = stage == 1 ? in : mid.data();
+        const u64 *src = stage == first_stage ? in : mid.data();
         u64 *dst = stage == 1 ? mid.data() : out;
         auto from_of = [&](size_t q) -> u64 { return stage == 1 && scale_levels ? scale_levels[q] : 0; };
         // One rotation source per job (a single ModUp).  A stage's rotation by r cells wraps inside the tile, so it is
@@ -666,6 +670,91 @@ void MatrixTransformer::diagonalTransformTwoStage(const HomEvaluator &eval, cons
         }
         c->mark(stage == 1 ? "transform stage 1" : "transform stage 2");
     }
+}
+
+namespace {
+// (left rotation in slots, mask) of the composite of the complex packing and the first transform stage
+std::vector<std::pair<u64, Message>> packingStageOneMessages(MaskKind kind, const TileTensorShape &shape, u64 log_slots) {
+    if (kind != MaskKind::PackedHorizontal && kind != MaskKind::PackedVertical)
+        throw std::invalid_argument("[packingStageOne] a packed kind is needed");
+    const Geo g = geo(kind, shape);
+    const bool vertical = kind == MaskKind::PackedVertical;
+    const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, unit = vertical ? w : 1;
+    const i64 b = twoStageSplit(g.units), wrap = g.n * (vertical ? w : 1);
+    auto norm = [&](i64 v) { return (u64)(((v % slots) + slots) % slots); };
+    const Message pm[3] = {packingMaskMessage(vertical, w, log_slots, 0), packingMaskMessage(vertical, w, log_slots, 1),
+                           packingMaskMessage(vertical, w, log_slots, 2)};
+    const i64 shift[3] = {0, unit, -unit};
+    std::map<u64, Message> acc;
+    auto add = [&](const Message &stage_mask, i64 a) {
+        const u64 ra = norm(a);
+        for (int e = 0; e < 3; e++) {
+            auto it = acc.find(norm(a + shift[e]));
+            if (it == acc.end()) it = acc.emplace(norm(a + shift[e]), Message(log_slots, 0)).first;
+            Message &m = it->second;
+            for (u64 s = 0; s < (u64)slots; s++) m[s] += stage_mask[s] * pm[e][(s + ra) % (u64)slots];
+        }
+    };
+    add(twoStageMaskMessage(kind, shape, log_slots, 1, 0, 0), 0);
+    for (i64 r = 1; r < b; r++) {
+        add(twoStageMaskMessage(kind, shape, log_slots, 1, r, 1), r * g.step);
+        add(twoStageMaskMessage(kind, shape, log_slots, 1, r, 2), r * g.step - wrap);
+    }
+    std::vector<std::pair<u64, Message>> out;
+    for (auto &am : acc) {
+        bool any = false;
+        for (u64 s = 0; s < (u64)slots && !any; s++) any = am.second[s] != Complex(0, 0);
+        if (any) out.emplace_back(am.first, std::move(am.second));   // (a rotation whose masks cancel is left out)
+    }
+    return out;
+}
+}  // namespace
+
+std::vector<u64> MatrixTransformer::packingStageOneRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots) {
+    // every stage rotation (0, r step, r step - wrap) shifted by the packing's 0, +unit, -unit
+    const Geo g = geo(kind, shape);
+    const bool vertical = kind == MaskKind::PackedVertical;
+    const i64 w = shape.getBlockWidth(), slots = i64(1) << log_slots, unit = vertical ? w : 1;
+    const i64 b = twoStageSplit(g.units), wrap = g.n * (vertical ? w : 1);
+    std::set<u64> r;
+    for (i64 i = 0; i < b; i++)
+        for (i64 a : {i * g.step, i * g.step - wrap})
+            for (i64 e : {i64(0), unit, -unit}) {
+                const u64 v = (u64)((((a + e) % slots) + slots) % slots);
+                if (v != 0 && (i > 0 || a == 0)) r.insert(v);
+            }
+    return std::vector<u64>(r.begin(), r.end());
+}
+
+void MatrixTransformer::packingStageOne(const HomEvaluator &eval, const u64 *in, u64 level, MaskKind kind,
+                                        const TileTensorShape &shape, u64 *out) {
+    const Context &c = eval.getContext();
+    if (level < 1) throw std::invalid_argument("[packingStageOne] level >= 1 is needed.");
+    const u64 nq = level + 1, N = c->N, E = nq + c->nP;
+    Key key{(int)kind, shape, level, 0};
+    auto it = packing_stage_one_masks_.find(key);
+    if (it == packing_stage_one_masks_.end()) {
+        EnDecoder endec(c);
+        std::vector<std::pair<u64, Plaintext>> v;
+        for (const auto &am : packingStageOneMessages(kind, shape, getLogFullSlots(c)))
+            v.emplace_back(am.first, endec.encodeExtended(am.second, level));
+        it = packing_stage_one_masks_.emplace(key, std::move(v)).first;
+    }
+    const Sources x = extendSources(c, in, 1, nq, nullptr, false);
+    const KeyPack &pack = eval.getKeyPack();
+    const u64 M = 2 * N;
+    std::vector<hemm_rot_term> terms;
+    for (const auto &am : it->second) {
+        if (am.first == 0)
+            terms.push_back(keylessTerm(in, in + nq * N, &am.second));
+        else
+            terms.push_back(term(x.extOf(0), x.pbOf(0), pack, powmod(5, am.first, M), &am.second));
+    }
+    const uint32_t off[2] = {0, (uint32_t)terms.size()};
+    DeviceBuffer y(c, 2 * E * N), ws(c, 2 * (nq - 1) * N);
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off, 1, (uint32_t)nq, x.premultiplied(), 1, y.data(), out, (nq - 1) * N,
+                            ws.data(), nullptr));
+    c->mark("packing and transform stage 1");
 }
 
 // The complex packing as a linear map on the slots, out = Z x + M_+ rho^(step)(x) + M_- rho^(-step)(x):
@@ -1399,8 +1488,43 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
     if (std::min(a.getLevel(), b.getLevel()) < T + 3)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
     // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
-    if (std::min(a.getLevel(), b.getLevel()) == T + 3)
+    if (std::min(a.getLevel(), b.getLevel()) == T + 3) {
+        const i64 rows = a.getHeight(), cols = b.getWidth(), k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
+        const u64 slots = c->N / 2;
+        const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
+        // B's row shifts are exact rotations (its tile fills the slot vector or is spread over it): tau(B) is needed at
+        // T+1 only, which leaves B two levels -- the packing with the FIRST stage of the two-stage tau as one composite
+        // map, then the second stage, on the side stream; A has one level for packing and sigma together (the composite
+        // one-stage transform) and takes it on the context's stream at the same time.
+        if (k / 2 >= 4 && rows == k && cols == k && ((u64)(k * w) == slots || spread) &&
+            T + 3 >= 4 + btp.getMinLevelForBootstrap()) {
+            const u64 N = c->N, L = T + 3, lo = T + 2, ctw = 2 * (L + 1) * N;
+            const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
+            std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
+            DeviceBuffer joint(c, 2 * ctw), sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
+            jointLevelDown(eval, a.get(), b.get(), L, joint.data());
+            c->mark("level down");
+            {
+                OwnWays ways(c);
+                ways.toSide();
+                {
+                    DeviceBuffer mid(c, 2 * L * N);
+                    const MaskKind kind = MaskKind::PackedVertical;
+                    tr.packingStageOne(eval, joint.data() + ctw, L, kind, shape_b, mid.data());
+                    tr.diagonalTransformTwoStage(eval, mid.data(), 1, L, &kind, &shape_b, tb.data(), nullptr, 2);
+                }
+                ways.toOwn();
+                const MaskKind kind = MaskKind::PackingHorizontal;
+                tr.diagonalTransformBatch(eval, joint.data(), 1, L, &kind, &shape_a, sa.data());
+                levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
+                ways.marksOn();
+                c->mark("packing and transform of A");
+                return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
+                                           ways.side(), add_conj);
+            }
+        }
         return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true, add_conj);
+    }
     {
         const i64 rows = a.getHeight(), cols = b.getWidth(), k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
         const u64 slots = c->N / 2;

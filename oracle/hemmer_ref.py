@@ -750,13 +750,14 @@ def two_stage_mask(kind, n, w, slots, stage, r, part):
     return np.where(on, 0.5 if (kind == PH and stage == 1) else 1.0, 0.0).astype(np.complex128)
 
 
-def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None):
+def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None, first_stage=1):
     """sigma / tau (square tiles) in two stages of one mask level each: row i is rotated by i mod b, then
     by b (i div b).  Every stage is one hoisted sum over its rotations of
     main_r rho^(r)(X) + wrap_r rho^(r - tile side)(X) (two keys per r, one source) and of mask_0 X for the rows that
     stay (a term without a key switch), with ModDown merged with the rescale.  Level L -> L - 2.
     from_level: the level whose scale the input still carries when it was only truncated from there (the masks of
-    the first stage are then encoded at Delta_{L-1} q_L / Delta_from, so the stage ends at the scale of L - 1)."""
+    the first stage are then encoded at Delta_{L-1} q_L / Delta_from, so the stage ends at the scale of L - 1).
+    first_stage = 2: only the second stage (ct is what a first stage left)."""
     from .oracle import Ct
     cell = 2 if kind in (PH, PV) else 1
     u = n // cell
@@ -765,6 +766,8 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None):
     wrap = n * (w if kind in (V, PV) else 1)
     x = ct
     for stage, count, mul in ((1, b, 1), (2, u // b, b)):
+        if stage < first_stage:
+            continue
         nq, lvl = x.nq, x.level
         own = stage == 2 or from_level is None or from_level == lvl
         ms = orc.delta[lvl] if own else orc.delta[lvl - 1] * float(orc.q[lvl]) / orc.delta[from_level]
@@ -787,6 +790,43 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None):
         y = orc.hoisted_sum(terms, nq)
         x = Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
     return x
+
+
+def packing_stage_one(orc, x, kind, n, w):
+    """The complex packing (by rows for PV, by columns for PH) and the FIRST stage of the two-stage transform of `kind`
+    as one linear map on the slots (MatrixTransformer::packingStageOne): one hoisted sum, one level.  The term that
+    rotates by a slots carries the sum over (stage rotation r, packing shift e) with r + e = a of
+    stage mask_r (.) rho^r(packing mask_e); a = 0 is the term without a key; rotations whose masks cancel are left out."""
+    from .oracle import Ct
+    assert kind in (PH, PV)
+    slots = orc.slots
+    u = n // 2
+    b = two_stage_split(u)
+    unit = w if kind == PV else 1
+    step, wrap = 2 * unit, n * unit
+    zmask, pterms = packing_maps(slots, w, rows=(kind == PV))
+    pack = [(0, zmask)] + pterms
+    acc = {}
+
+    def add(stage_mask, a):
+        for e, pm in pack:
+            t = (a + e) % slots
+            acc[t] = acc.get(t, 0) + stage_mask * np.roll(pm, -(a % slots))     # rho^a(pm)[s] = pm[s + a]
+
+    add(two_stage_mask(kind, n, w, slots, 1, 0, 0), 0)
+    for r in range(1, b):
+        add(two_stage_mask(kind, n, w, slots, 1, r, 1), r * step)
+        add(two_stage_mask(kind, n, w, slots, 1, r, 2), r * step - wrap)
+    nq, lvl = x.nq, x.level
+    ext = orc.modup(x.data[1])
+    terms = []
+    for a in sorted(acc):
+        if not np.any(acc[a]):
+            continue
+        m = orc.encode_ext(acc[a], lvl)
+        terms.append((x.data[1], x.data[0], ("none",), m) if a == 0 else (ext, x.data[0], a, m))
+    y = orc.hoisted_sum(terms, nq)
+    return Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
 
 
 def lower_and_transform_fused(orc, x, kind, n, w, end_level):
@@ -930,6 +970,14 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packi
     if (not merge_packing and a.level >= T + 4 and b.level >= T + 3 and rows == cols and n // 2 >= 4
             and (n * w == orc.slots or spread)):
         own_levels = True
+    if merge_packing and rows == cols and n // 2 >= 4 and (n * w == orc.slots or spread):
+        # exact row rotations: tau(B) is needed at T+1 only, which leaves B two levels -- the packing with the first
+        # stage of tau as one composite map, then the second stage -- while A takes the composite one-stage transform
+        a, b = orc.level_down(a, T + 3), orc.level_down(b, T + 3)
+        a = diagonal_transform_fused(orc, a, PKH, n, w)
+        b = diagonal_transform_two_stage(orc, packing_stage_one(orc, b, PV, n, w), PV, n, w, first_stage=2)
+        acc = orc.tensor(orc.level_down_one(a), b)
+        return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0, with_conj)
     if not own_levels and (merge_packing or lvl >= T + 3):
         if merge_packing:
             a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)

@@ -325,6 +325,13 @@ def test_preset_ccmm_residues_bit_exact(preset):
     assert c3.info()["level"] == 4 == want3.level
     assert np.array_equal(c3.residues(), want3.data)
     assert np.abs(H.decrypt(c3) - A @ B).max() < 2.0 ** -12
+    # three levels above the target as known single tiles: B's row shifts are exact rotations, so B takes the packing
+    # and the first stage of tau as one composite map and then the second stage, beside A's composite transform
+    c4 = H.single_cc_matmul(la, lb, 4)
+    want4 = R.mult_mat_mat_cc_packed(orc, O.Ct(la.residues(), d7), O.Ct(lb.residues(), d7), 4, 128, 128, single_tile=True)
+    assert c4.info()["level"] == 4 == want4.level
+    assert np.array_equal(c4.residues(), want4.data)
+    assert np.abs(H.decrypt(c4) - A @ B).max() < 2.0 ** -12
 
 
 def test_preset_two_stream_products_repeat_bit_for_bit(preset):
