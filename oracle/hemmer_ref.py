@@ -798,10 +798,20 @@ def packing_stage_one(orc, x, kind, n, w):
     rotates by a slots carries the sum over (stage rotation r, packing shift e) with r + e = a of
     stage mask_r (.) rho^r(packing mask_e); a = 0 is the term without a key; rotations whose masks cancel are left out."""
     from .oracle import Ct
+    nq, lvl = x.nq, x.level
+    ext = orc.modup(x.data[1])
+    terms = []
+    for a, mask in packing_stage_one_maps(kind, n, w, orc.slots):
+        m = orc.encode_ext(mask, lvl)
+        terms.append((x.data[1], x.data[0], ("none",), m) if a == 0 else (ext, x.data[0], a, m))
+    y = orc.hoisted_sum(terms, nq)
+    return Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
+
+
+def packing_stage_one_maps(kind, n, w, slots):
+    """[(left rotation a in slots, mask)] with stage_1(packing(x)) = sum_a mask_a (.) rho^a(x), in increasing a."""
     assert kind in (PH, PV)
-    slots = orc.slots
-    u = n // 2
-    b = two_stage_split(u)
+    b = two_stage_split(n // 2)
     unit = w if kind == PV else 1
     step, wrap = 2 * unit, n * unit
     zmask, pterms = packing_maps(slots, w, rows=(kind == PV))
@@ -817,16 +827,7 @@ def packing_stage_one(orc, x, kind, n, w):
     for r in range(1, b):
         add(two_stage_mask(kind, n, w, slots, 1, r, 1), r * step)
         add(two_stage_mask(kind, n, w, slots, 1, r, 2), r * step - wrap)
-    nq, lvl = x.nq, x.level
-    ext = orc.modup(x.data[1])
-    terms = []
-    for a in sorted(acc):
-        if not np.any(acc[a]):
-            continue
-        m = orc.encode_ext(acc[a], lvl)
-        terms.append((x.data[1], x.data[0], ("none",), m) if a == 0 else (ext, x.data[0], a, m))
-    y = orc.hoisted_sum(terms, nq)
-    return Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
+    return [(a, acc[a]) for a in sorted(acc) if np.any(acc[a])]
 
 
 def lower_and_transform_fused(orc, x, kind, n, w, end_level):

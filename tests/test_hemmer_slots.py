@@ -183,6 +183,33 @@ def test_composite_packing_transform_masks(n, w, log_slots):
         assert sim.level_of(one_step) == sim.level_of(two_steps) + 1      # one level instead of two
 
 
+@pytest.mark.parametrize("n,w,log_slots", [(8, 16, 7), (8, 8, 7), (16, 32, 9), (16, 16, 9)])
+def test_packing_and_first_stage_as_one_map(n, w, log_slots):
+    """packing_stage_one_maps: sum_a mask_a (.) rho^a(x) equals the complex packing followed by the first stage of
+    the two-stage packed transform, and the second stage then completes the packed transform of the packed operand
+    (arbitrary slot vectors; tiles that fill the slot vector, where main and wrapped rotations coincide, and tiles
+    that leave other blocks)."""
+    sim = R.SlotSim(log_slots, 12)
+    rng = np.random.default_rng(3 * n + w)
+    x0 = rng.normal(size=sim.slots) + 1j * rng.normal(size=sim.slots)
+    rot = lambda v, r: np.roll(v, -r)
+    for kind, pack in ((R.PH, R.complex_packing_cols), (R.PV, R.complex_packing_rows)):
+        maps = R.packing_stage_one_maps(kind, n, w, sim.slots)
+        assert len({a for a, _ in maps}) == len(maps) and all(0 <= a < sim.slots for a, _ in maps)
+        x = sum(m * rot(x0, a) for a, m in maps)
+        # the second stage alone (its masks and rotations as in the two-stage transform)
+        u = n // 2
+        b = R.two_stage_split(u)
+        step = 2 * (w if kind == R.PV else 1)
+        wrap = n * (w if kind == R.PV else 1)
+        y = R.two_stage_mask(kind, n, w, sim.slots, 2, 0, 0) * x
+        for r in range(1, u // b):
+            y = y + R.two_stage_mask(kind, n, w, sim.slots, 2, r, 1) * rot(x, r * b * step)
+            y = y + R.two_stage_mask(kind, n, w, sim.slots, 2, r, 2) * rot(x, r * b * step - wrap)
+        want = R.diagonal_transform(sim, pack(sim, sim.encrypt(x0), n, w), kind, n, w).z
+        assert np.abs(y - want).max() < 1e-12, kind
+
+
 def test_composite_packed_ccmm_three_levels_above_the_target():
     """A whole product through the composite transform on the slot simulator: operands three levels above the target,
     single tile and stacked tiles."""
