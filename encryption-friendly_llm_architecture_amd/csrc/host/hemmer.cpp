@@ -502,9 +502,15 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             ensureRotationKeys(transformRotations(MaskKind::PackedVertical, w));
             // three levels above the target with exact row rotations: B's packing and first tau stage are one composite
             // map (MatrixTransformer::packingStageOne), with rotations of its own
-            if (std::min(a.getLevel(), b.getLevel()) == T + 3 && n >= 8 && (block == slots || (single && block < slots)))
+            // operands with a level less than a separate packing needs (A below T+5 or B below T+4) and exact row
+            // rotations: the packing and the first transform stage are one composite map, with rotations of its own
+            if (n >= 8 && (block == slots || (single && block < slots)) && !(a.getLevel() >= T + 5 && b.getLevel() >= T + 4)) {
                 ensureRotationKeys(MatrixTransformer::packingStageOneRotations(MaskKind::PackedVertical,
                                                                                TileTensorShape(n, n, w), log_slots_));
+                if (a.getLevel() >= T + 4)
+                    ensureRotationKeys(MatrixTransformer::packingStageOneRotations(MaskKind::PackedHorizontal,
+                                                                                   TileTensorShape(n, n, w), log_slots_));
+            }
             std::vector<u64> sq;
             // stacked tiles / unknown content keep their per-block products: the packed cells then shift through
             // masked pairs (no baby-step / giant-step split, which needs exact row rotations)

@@ -727,17 +727,21 @@ std::vector<u64> MatrixTransformer::packingStageOneRotations(MaskKind kind, cons
 }
 
 void MatrixTransformer::packingStageOne(const HomEvaluator &eval, const u64 *in, u64 level, MaskKind kind,
-                                        const TileTensorShape &shape, u64 *out) {
+                                        const TileTensorShape &shape, u64 *out, u64 scale_level) {
     const Context &c = eval.getContext();
     if (level < 1) throw std::invalid_argument("[packingStageOne] level >= 1 is needed.");
+    if (scale_level == 0) scale_level = level;
+    if (scale_level < level) throw std::invalid_argument("[packingStageOne] the scale must come from the same or a higher level.");
     const u64 nq = level + 1, N = c->N, E = nq + c->nP;
-    Key key{(int)kind, shape, level, 0};
+    Key key{(int)kind, shape, level, (i64)(scale_level == level ? 0 : scale_level)};
     auto it = packing_stage_one_masks_.find(key);
     if (it == packing_stage_one_masks_.end()) {
         EnDecoder endec(c);
+        // an input truncated from scale_level: the masks carry the change of scale (as in complexPackingBatch)
+        const Real scale = scale_level == level ? c->delta[level] : c->delta[level - 1] * (Real)c->q[level] / c->delta[scale_level];
         std::vector<std::pair<u64, Plaintext>> v;
         for (const auto &am : packingStageOneMessages(kind, shape, getLogFullSlots(c)))
-            v.emplace_back(am.first, endec.encodeExtended(am.second, level));
+            v.emplace_back(am.first, endec.encodeExtended(am.second, level, scale));
         it = packing_stage_one_masks_.emplace(key, std::move(v)).first;
     }
     const Sources x = extendSources(c, in, 1, nq, nullptr, false);
@@ -1487,103 +1491,88 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
         throw std::invalid_argument("[complexPacking] operands must be rescaled.");
     if (std::min(a.getLevel(), b.getLevel()) < T + 3)
         throw std::invalid_argument("[multMatMat] level >= " + std::to_string(T + 3) + " is needed.");
-    // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
-    if (std::min(a.getLevel(), b.getLevel()) == T + 3) {
-        const i64 rows = a.getHeight(), cols = b.getWidth(), k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
-        const u64 slots = c->N / 2;
-        const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
-        // B's row shifts are exact rotations (its tile fills the slot vector or is spread over it): tau(B) is needed at
-        // T+1 only, which leaves B two levels -- the packing with the FIRST stage of the two-stage tau as one composite
-        // map, then the second stage, on the side stream; A has one level for packing and sigma together (the composite
-        // one-stage transform) and takes it on the context's stream at the same time.
-        if (k / 2 >= 4 && rows == k && cols == k && ((u64)(k * w) == slots || spread) &&
-            T + 3 >= 4 + btp.getMinLevelForBootstrap()) {
-            const u64 N = c->N, L = T + 3, lo = T + 2, ctw = 2 * (L + 1) * N;
-            const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
-            std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
-            DeviceBuffer joint(c, 2 * ctw), sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
-            jointLevelDown(eval, a.get(), b.get(), L, joint.data());
-            c->mark("level down");
-            {
-                OwnWays ways(c);
-                ways.toSide();
-                {
-                    DeviceBuffer mid(c, 2 * L * N);
-                    const MaskKind kind = MaskKind::PackedVertical;
-                    tr.packingStageOne(eval, joint.data() + ctw, L, kind, shape_b, mid.data());
-                    tr.diagonalTransformTwoStage(eval, mid.data(), 1, L, &kind, &shape_b, tb.data(), nullptr, 2);
-                }
-                ways.toOwn();
-                const MaskKind kind = MaskKind::PackingHorizontal;
-                tr.diagonalTransformBatch(eval, joint.data(), 1, L, &kind, &shape_a, sa.data());
-                levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
-                ways.marksOn();
-                c->mark("packing and transform of A");
-                return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
-                                           ways.side(), add_conj);
-            }
-        }
-        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true, add_conj);
-    }
     {
         const i64 rows = a.getHeight(), cols = b.getWidth(), k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
-        const u64 slots = c->N / 2;
+        const u64 slots = c->N / 2, la = a.getLevel(), lb = b.getLevel();
         const bool spread = single_tile && (u64)(k * w) < slots && slots % (u64)(k * w) == 0;
         const bool bsgs = k / 2 > 1 && ((u64)(k * w) == slots || spread);
-        // With a level more to spare the two operands go their own ways: B is packed at T+4 and its transform ends at
-        // T+1, where the product needs it (no level-down in front of the baby rotations), on the side stream; A is packed
-        // at T+5 and transformed to T+2 on the context's stream, and only its copy for the unshifted term is lowered.
-        // (an A with only four levels above the target is packed at T+4 and takes the one-stage transform from T+3)
+        // Exact row rotations (B's tile fills the slot vector or is spread over it) on square tiles: the product needs
+        // sigma(A') at T+2 but tau(B') at T+1, and the two operands go their own ways there on two streams -- B on the
+        // side stream, where the baby rotations follow its transform, A on the context's, where only its copy for the
+        // unshifted term is lowered; the chains meet in front of the main loop.  Operands above the level their way
+        // starts from are only truncated to it (the first masks on the way carry the change of scale).  The ways:
+        //   * separate packing (A >= T+5, B >= T+4): packed at T+5 / T+4, then the two-stage transform -- three launch
+        //     chains of few terms each;
+        //   * packing and the first transform stage as one composite map (MatrixTransformer::packingStageOne), then the
+        //     second stage: two chains, the first with about twice the terms -- for an A at T+4 and a B at T+3, which
+        //     have a level less than the separate packing needs;
+        //   * an A at T+3 has one level for packing and sigma together: the composite one-stage transform.
         // (k / 2 >= 4: every transform stage then has rotations; a stage without any rescales through the context's
         // scratch region, which only one of the two chains may use)
-        if (bsgs && k / 2 >= 4 && rows == k && cols == k && a.getLevel() >= T + 4 && b.getLevel() >= T + 4 &&
-            std::min(a.getLevel(), b.getLevel()) >= 4 + btp.getMinLevelForBootstrap()) {
-            const u64 N = c->N, La = std::min<u64>(a.getLevel(), T + 5), Lb = T + 4, lo = T + 2;
+        if (bsgs && k / 2 >= 4 && rows == k && cols == k && std::min(la, lb) >= 4 + btp.getMinLevelForBootstrap()) {
+            const bool separate = la >= T + 5 && lb >= T + 4;
+            const u64 N = c->N, lo = T + 2;
             const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
             std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
             DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
-            const std::vector<u64> one(La + 1, 1);
+            const std::vector<u64> one(T + 6, 1);
+            // the first L + 1 limbs of both polynomials of x, back to back
+            auto truncated = [&](const Ciphertext &x, u64 L) {
+                DeviceBuffer t(c, 2 * (L + 1) * N);
+                ck(hemm_mul_scalar(c->dev, x.buf_.data(), x.polyStride(), one.data(), t.data(), (L + 1) * N, (uint32_t)(L + 1), 0,
+                                   2, nullptr));
+                return t;
+            };
+            OwnWays ways(c);
+            ways.toSide();
             {
-                OwnWays ways(c);
-                // B one level below A, on the side stream: truncated to T+4, packed by rows (T+3), tau in two stages (T+1)
-                ways.toSide();
-                {
-                    DeviceBuffer jb(c, 2 * (Lb + 1) * N), pk(c, 2 * Lb * N);
-                    ck(hemm_mul_scalar(c->dev, b.get().buf_.data(), b.get().polyStride(), one.data(), jb.data(), (Lb + 1) * N,
-                                       (uint32_t)(Lb + 1), 0, 2, nullptr));
+                const MaskKind kind = MaskKind::PackedVertical;
+                if (separate) {   // truncated to T+4, packed by rows (T+3), tau in two stages (T+1)
+                    const u64 Lb = T + 4;
+                    const DeviceBuffer jb = truncated(b.get(), Lb);
+                    DeviceBuffer pk(c, 2 * Lb * N);
                     const bool by_rows = true;
-                    const u64 from = b.getLevel();
-                    tr.complexPackingBatch(eval, jb.data(), 1, Lb, &by_rows, w, pk.data(), &from);
-                    const MaskKind kind = MaskKind::PackedVertical;
+                    tr.complexPackingBatch(eval, jb.data(), 1, Lb, &by_rows, w, pk.data(), &lb);
                     tr.diagonalTransformTwoStage(eval, pk.data(), 1, Lb - 1, &kind, &shape_b, tb.data());
+                } else {          // truncated to T+3, packing + first stage (T+2), second stage (T+1)
+                    const u64 Lb = T + 3;
+                    const DeviceBuffer jb = truncated(b.get(), Lb);
+                    DeviceBuffer mid(c, 2 * Lb * N);
+                    tr.packingStageOne(eval, jb.data(), Lb, kind, shape_b, mid.data(), lb);
+                    tr.diagonalTransformTwoStage(eval, mid.data(), 1, Lb, &kind, &shape_b, tb.data(), nullptr, 2);
                 }
-                ways.toOwn();
-                // A on the context's stream: truncated to T+5, packed by columns (T+4), sigma in two stages (T+2); from T+4:
-                // packed to T+3, sigma in one stage
-                {
-                    DeviceBuffer ja(c, 2 * (La + 1) * N), pk(c, 2 * La * N);
-                    ck(hemm_mul_scalar(c->dev, a.get().buf_.data(), a.get().polyStride(), one.data(), ja.data(), (La + 1) * N,
-                                       (uint32_t)(La + 1), 0, 2, nullptr));
-                    const bool by_rows = false;
-                    const u64 from = a.getLevel();
-                    tr.complexPackingBatch(eval, ja.data(), 1, La, &by_rows, w, pk.data(), &from);
-                    const MaskKind kind = MaskKind::PackedHorizontal;
-                    if (La == T + 5)
-                        tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
-                    else
-                        tr.diagonalTransformBatch(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
-                }
-                // (the only call that works in the context's scratch region while the side chain is open)
-                levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
-                // the side chain stays open: the baby rotations of tau(B) follow its transform there while the sources
-                // of sigma(A) are made here, and the two meet in front of the main loop
-                ways.marksOn();
-                c->mark("packing and transforms of A");
-                return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
-                                           ways.side(), add_conj);
             }
+            ways.toOwn();
+            if (separate) {       // truncated to T+5, packed by columns (T+4), sigma in two stages (T+2)
+                const u64 La = T + 5;
+                const DeviceBuffer ja = truncated(a.get(), La);
+                DeviceBuffer pk(c, 2 * La * N);
+                const bool by_rows = false;
+                const MaskKind kind = MaskKind::PackedHorizontal;
+                tr.complexPackingBatch(eval, ja.data(), 1, La, &by_rows, w, pk.data(), &la);
+                tr.diagonalTransformTwoStage(eval, pk.data(), 1, La - 1, &kind, &shape_a, sa.data());
+            } else if (la >= T + 4) {   // truncated to T+4, packing + first stage (T+3), second stage (T+2)
+                const u64 La = T + 4;
+                const DeviceBuffer ja = truncated(a.get(), La);
+                DeviceBuffer mid(c, 2 * La * N);
+                const MaskKind kind = MaskKind::PackedHorizontal;
+                tr.packingStageOne(eval, ja.data(), La, kind, shape_a, mid.data(), la);
+                tr.diagonalTransformTwoStage(eval, mid.data(), 1, La, &kind, &shape_a, sa.data(), nullptr, 2);
+            } else {              // at T+3: packing and sigma as one composite one-stage transform (T+2)
+                const MaskKind kind = MaskKind::PackingHorizontal;
+                tr.diagonalTransformBatch(eval, a.get().buf_.data(), 1, T + 3, &kind, &shape_a, sa.data());
+            }
+            // (the only call that works in the context's scratch region while the side chain is open)
+            levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
+            ways.marksOn();
+            c->mark("packing and transforms of A");
+            return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
+                                       ways.side(), add_conj);
         }
     }
+    // one level short of a separate packing: the packing and the packed transform as one composite transform from T+3
+    if (std::min(a.getLevel(), b.getLevel()) == T + 3)
+        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, nullptr, 0, true, add_conj);
     // pack at T+5 when the operands allow it, so that the transforms keep their two stages from T+4; the packed pair
     // is handed to the product where it lies.  Operands above the packing level are only truncated to it (a copy of
     // their first L+1 limbs): the packing masks absorb the change of scale, which saves the levelDown.

@@ -792,17 +792,20 @@ def diagonal_transform_two_stage(orc, ct, kind, n, w, from_level=None, first_sta
     return x
 
 
-def packing_stage_one(orc, x, kind, n, w):
+def packing_stage_one(orc, x, kind, n, w, from_level=None):
     """The complex packing (by rows for PV, by columns for PH) and the FIRST stage of the two-stage transform of `kind`
     as one linear map on the slots (MatrixTransformer::packingStageOne): one hoisted sum, one level.  The term that
     rotates by a slots carries the sum over (stage rotation r, packing shift e) with r + e = a of
-    stage mask_r (.) rho^r(packing mask_e); a = 0 is the term without a key; rotations whose masks cancel are left out."""
+    stage mask_r (.) rho^r(packing mask_e); a = 0 is the term without a key; rotations whose masks cancel are left out.
+    from_level: the level whose scale a truncated input still carries (the masks then carry the change of scale)."""
     from .oracle import Ct
     nq, lvl = x.nq, x.level
+    own = from_level is None or from_level == lvl
+    ms = orc.delta[lvl] if own else orc.delta[lvl - 1] * float(orc.q[lvl]) / orc.delta[from_level]
     ext = orc.modup(x.data[1])
     terms = []
     for a, mask in packing_stage_one_maps(kind, n, w, orc.slots):
-        m = orc.encode_ext(mask, lvl)
+        m = orc.encode_ext(mask, lvl, ms)
         terms.append((x.data[1], x.data[0], ("none",), m) if a == 0 else (ext, x.data[0], a, m))
     y = orc.hoisted_sum(terms, nq)
     return Ct(orc.moddown_drop(y, nq, True), orc.delta[lvl - 1])
@@ -971,14 +974,6 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packi
     if (not merge_packing and a.level >= T + 4 and b.level >= T + 3 and rows == cols and n // 2 >= 4
             and (n * w == orc.slots or spread)):
         own_levels = True
-    if merge_packing and rows == cols and n // 2 >= 4 and (n * w == orc.slots or spread):
-        # exact row rotations: tau(B) is needed at T+1 only, which leaves B two levels -- the packing with the first
-        # stage of tau as one composite map, then the second stage -- while A takes the composite one-stage transform
-        a, b = orc.level_down(a, T + 3), orc.level_down(b, T + 3)
-        a = diagonal_transform_fused(orc, a, PKH, n, w)
-        b = diagonal_transform_two_stage(orc, packing_stage_one(orc, b, PV, n, w), PV, n, w, first_stage=2)
-        acc = orc.tensor(orc.level_down_one(a), b)
-        return _bsgs_shift_product(orc, a, b, acc, cm, n, n // 2, 2, w, n * w if spread else 0, with_conj)
     if not own_levels and (merge_packing or lvl >= T + 3):
         if merge_packing:
             a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)
@@ -1047,18 +1042,34 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     is the product of the operands' blocks."""
     from .oracle import Ct
     ev = OracleEval(orc)
-    if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
-        return mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True, with_conj=True)
     cut = lambda x, lvl: Ct(np.ascontiguousarray(x.data[:, : lvl + 1]), x.scale)
     spread = single_tile and n * w < orc.slots and orc.slots % (n * w) == 0
     rows, cols = _dims(n)
-    if a.level >= T + 4 and b.level >= T + 4 and rows == cols and n // 2 >= 4 and (n * w == orc.slots or spread):
-        # the operands go their own ways: B is packed at T+4 and transformed straight to T+1 (two stages), A packed at
-        # T+5 and transformed to T+2 in two stages, or packed at T+4 and transformed in one (the two chains run side by
-        # side on the GPU); only A's copy for the unshifted term is lowered
-        pa = complex_packing_hoisted(orc, cut(a, min(a.level, T + 5)), w, rows=False)
-        pb = complex_packing_hoisted(orc, cut(b, T + 4), w, rows=True)
-        return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True, own_levels=True)
+    assert min(a.level, b.level) >= T + 3
+    if rows == cols and n // 2 >= 4 and (n * w == orc.slots or spread):
+        # exact row rotations: the operands go their own ways to T+2 (sigma(A)) and T+1 (tau(B)) -- side by side on the
+        # GPU -- and only A's copy for the unshifted term is lowered.  Operands above the level their way starts from
+        # are only truncated to it.
+        if a.level >= T + 5 and b.level >= T + 4:
+            # separate packing: B packed at T+4 and transformed in two stages, A packed at T+5 and transformed in two
+            pa = complex_packing_hoisted(orc, cut(a, T + 5), w, rows=False)
+            pb = complex_packing_hoisted(orc, cut(b, T + 4), w, rows=True)
+            return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True,
+                                             own_levels=True)
+        # a level less than that: the packing and the first transform stage as one composite map, then the second
+        # stage (B from T+3, A from T+4); an A at T+3 has one level for both: the composite one-stage transform
+        tb = diagonal_transform_two_stage(orc, packing_stage_one(orc, cut(b, T + 3), PV, n, w, b.level), PV, n, w,
+                                          first_stage=2)
+        if a.level >= T + 4:
+            sa = diagonal_transform_two_stage(orc, packing_stage_one(orc, cut(a, T + 4), PH, n, w, a.level), PH, n, w,
+                                              first_stage=2)
+        else:
+            sa = diagonal_transform_fused(orc, a, PKH, n, w)
+        cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
+        acc = orc.tensor(orc.level_down_one(sa), tb)
+        return _bsgs_shift_product(orc, sa, tb, acc, cm, n, n // 2, 2, w, n * w if spread else 0, True)
+    if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
+        return mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True, with_conj=True)
     lvl = min(a.level, b.level, T + 5)
     pa = complex_packing_hoisted(orc, cut(a, lvl), w, rows=False)
     pb = complex_packing_hoisted(orc, cut(b, lvl), w, rows=True)

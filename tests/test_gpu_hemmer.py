@@ -183,16 +183,18 @@ def test_ccmm_single_tile_promise(small):
 
 
 def test_ccmm_packed_route_at_lower_and_mixed_levels(small):
-    """The complex-packed route away from its preferred level: operands at T+4 are packed there and the packed
-    transforms run in one stage; operands above T+5 or at different levels are truncated to the packing level, their
-    packing masks absorbing the change of scale."""
+    """The complex-packed route away from its preferred levels (A >= T+5, B >= T+4: separate packing, two-stage
+    transforms).  An A at T+4 or a B at T+3 takes the packing and the first transform stage as one composite map and
+    then the second stage, an A at T+3 the composite one-stage transform; operands above the level their way starts
+    from are truncated to it, the first masks on the way absorbing the change of scale."""
     H, orc, ev = small
     rng = np.random.default_rng(23)
     A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
     ca, cb = H.encrypt(A), H.encrypt(B)
     top = ca.info()["level"]
     assert top == 7
-    for T, la, lb in ((2, 6, 6), (2, 7, 6), (2, 6, 7), (1, 7, 7), (1, 7, 6), (1, 5, 7)):
+    for T, la, lb in ((2, 6, 6), (2, 7, 6), (2, 6, 7), (1, 7, 7), (1, 7, 6), (1, 5, 7), (2, 7, 5), (2, 6, 5), (2, 5, 7),
+                      (3, 7, 6)):
         a = H.level_down(ca, la) if la < top else ca
         b = H.level_down(cb, lb) if lb < top else cb
         c = H.single_cc_matmul(a, b, T)

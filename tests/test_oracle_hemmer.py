@@ -37,10 +37,11 @@ def test_ccmm_over_oracle(env):
     assert np.abs(z[n * n:]).max() < 2 ** -20
 
 
-@pytest.mark.parametrize("T", [1, 2])
+@pytest.mark.parametrize("T", [1, 2, 3])
 def test_complex_packed_single_ccmm_over_oracle(env, T):
     """One product through the complex-packed route.  With T = 1 the fresh operands (level 7) sit above the packing
-    level T + 5: they are only truncated, and the packing masks carry the change of scale."""
+    level T + 5: they are only truncated, and the packing masks carry the change of scale.  With T = 3 they sit at
+    T + 4: the packing and the first transform stage are one composite map."""
     orc, ev, n = env
     rng = np.random.default_rng(5)
     A, B = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
