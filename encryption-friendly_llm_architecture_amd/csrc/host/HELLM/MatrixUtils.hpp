@@ -100,9 +100,11 @@ public:
     // stage mask_r (.) rho^r(packing mask_e).  in [2][level+1][N] (not packed yet) -> out [2][level][N], which the
     // second stage takes to level - 1: packing and transform in two levels, for an operand with one level less than
     // packing, stage 1 and stage 2 need on their own.
-    // scale_level (0: `level`): the level whose fixed scale the input carries when it was only truncated to `level`.
-    void packingStageOne(const HomEvaluator &eval, const u64 *in, u64 level, MaskKind kind, const TileTensorShape &shape,
-                         u64 *out, u64 scale_level = 0);
+    // n_jobs operands through the same launch chain, in [job][2][level+1][N] -> out [job][2][level][N].
+    // scale_levels (optional, one per job; 0: `level`): the level whose fixed scale the job's input carries when it was
+    // only truncated to `level`.
+    void packingStageOne(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level, const MaskKind *kinds,
+                         const TileTensorShape *shapes, u64 *out, const u64 *scale_levels = nullptr);
     // left rotations (in slots) packingStageOne uses
     static std::vector<u64> packingStageOneRotations(MaskKind kind, const TileTensorShape &shape, u64 log_slots);
     // Brings `in` down to the level a transform ending at `end_level` starts from and runs it with the batched

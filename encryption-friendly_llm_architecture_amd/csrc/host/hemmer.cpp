@@ -504,7 +504,10 @@ CtxtTensor HEMMer::singleCCMatMul(const CtxtTensor &a, const CtxtTensor &b, u64 
             // map (MatrixTransformer::packingStageOne), with rotations of its own
             // operands with a level less than a separate packing needs (A below T+5 or B below T+4) and exact row
             // rotations: the packing and the first transform stage are one composite map, with rotations of its own
-            if (n >= 8 && (block == slots || (single && block < slots)) && !(a.getLevel() >= T + 5 && b.getLevel() >= T + 4)) {
+            // (with masked row shifts both operands end at T+2: composite maps when the lower one is at T+4)
+            const bool exact_rows = block == slots || (single && block < slots);
+            const bool separate = a.getLevel() >= T + 5 && b.getLevel() >= T + 4;
+            if (n >= 8 && ((exact_rows && !separate) || (!exact_rows && std::min(a.getLevel(), b.getLevel()) == T + 4))) {
                 ensureRotationKeys(MatrixTransformer::packingStageOneRotations(MaskKind::PackedVertical,
                                                                                TileTensorShape(n, n, w), log_slots_));
                 if (a.getLevel() >= T + 4)

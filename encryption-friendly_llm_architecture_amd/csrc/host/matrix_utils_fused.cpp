@@ -726,38 +726,45 @@ std::vector<u64> MatrixTransformer::packingStageOneRotations(MaskKind kind, cons
     return std::vector<u64>(r.begin(), r.end());
 }
 
-void MatrixTransformer::packingStageOne(const HomEvaluator &eval, const u64 *in, u64 level, MaskKind kind,
-                                        const TileTensorShape &shape, u64 *out, u64 scale_level) {
+void MatrixTransformer::packingStageOne(const HomEvaluator &eval, const u64 *in, size_t n_jobs, u64 level,
+                                        const MaskKind *kinds, const TileTensorShape *shapes, u64 *out,
+                                        const u64 *scale_levels) {
     const Context &c = eval.getContext();
     if (level < 1) throw std::invalid_argument("[packingStageOne] level >= 1 is needed.");
-    if (scale_level == 0) scale_level = level;
-    if (scale_level < level) throw std::invalid_argument("[packingStageOne] the scale must come from the same or a higher level.");
-    const u64 nq = level + 1, N = c->N, E = nq + c->nP;
-    Key key{(int)kind, shape, level, (i64)(scale_level == level ? 0 : scale_level)};
-    auto it = packing_stage_one_masks_.find(key);
-    if (it == packing_stage_one_masks_.end()) {
-        EnDecoder endec(c);
-        // an input truncated from scale_level: the masks carry the change of scale (as in complexPackingBatch)
-        const Real scale = scale_level == level ? c->delta[level] : c->delta[level - 1] * (Real)c->q[level] / c->delta[scale_level];
-        std::vector<std::pair<u64, Plaintext>> v;
-        for (const auto &am : packingStageOneMessages(kind, shape, getLogFullSlots(c)))
-            v.emplace_back(am.first, endec.encodeExtended(am.second, level, scale));
-        it = packing_stage_one_masks_.emplace(key, std::move(v)).first;
-    }
-    const Sources x = extendSources(c, in, 1, nq, nullptr, false);
+    const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
+    const Sources x = extendSources(c, in, n_jobs, nq, nullptr, false);
     const KeyPack &pack = eval.getKeyPack();
     const u64 M = 2 * N;
     std::vector<hemm_rot_term> terms;
-    for (const auto &am : it->second) {
-        if (am.first == 0)
-            terms.push_back(keylessTerm(in, in + nq * N, &am.second));
-        else
-            terms.push_back(term(x.extOf(0), x.pbOf(0), pack, powmod(5, am.first, M), &am.second));
+    std::vector<uint32_t> off{0};
+    for (size_t q = 0; q < n_jobs; q++) {
+        const u64 scale_level = scale_levels && scale_levels[q] != 0 ? scale_levels[q] : level;
+        if (scale_level < level)
+            throw std::invalid_argument("[packingStageOne] the scale must come from the same or a higher level.");
+        Key key{(int)kinds[q], shapes[q], level, (i64)(scale_level == level ? 0 : scale_level)};
+        auto it = packing_stage_one_masks_.find(key);
+        if (it == packing_stage_one_masks_.end()) {
+            EnDecoder endec(c);
+            // an input truncated from scale_level: the masks carry the change of scale (as in complexPackingBatch)
+            const Real scale =
+                scale_level == level ? c->delta[level] : c->delta[level - 1] * (Real)c->q[level] / c->delta[scale_level];
+            std::vector<std::pair<u64, Plaintext>> v;
+            for (const auto &am : packingStageOneMessages(kinds[q], shapes[q], getLogFullSlots(c)))
+                v.emplace_back(am.first, endec.encodeExtended(am.second, level, scale));
+            it = packing_stage_one_masks_.emplace(key, std::move(v)).first;
+        }
+        const u64 *ct = in + q * ctw;
+        for (const auto &am : it->second) {
+            if (am.first == 0)
+                terms.push_back(keylessTerm(ct, ct + nq * N, &am.second));
+            else
+                terms.push_back(term(x.extOf(q), x.pbOf(q), pack, powmod(5, am.first, M), &am.second));
+        }
+        off.push_back((uint32_t)terms.size());
     }
-    const uint32_t off[2] = {0, (uint32_t)terms.size()};
-    DeviceBuffer y(c, 2 * E * N), ws(c, 2 * (nq - 1) * N);
-    ck(hemm_hoisted_moddown(c->dev, terms.data(), off, 1, (uint32_t)nq, x.premultiplied(), 1, y.data(), out, (nq - 1) * N,
-                            ws.data(), nullptr));
+    DeviceBuffer y(c, n_jobs * 2 * E * N), ws(c, n_jobs * 2 * (nq - 1) * N);
+    ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_jobs, (uint32_t)nq, x.premultiplied(), 1, y.data(),
+                            out, (nq - 1) * N, ws.data(), nullptr));
     c->mark("packing and transform stage 1");
 }
 
@@ -1128,7 +1135,7 @@ void jointLevelDown(const HomEvaluator &eval, const Ciphertext &a, const Ciphert
 namespace {
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre = nullptr,
-                     u64 pre_level = 0, bool merge_packing = false, bool add_conj = false);
+                     u64 pre_level = 0, bool merge_packing = false, bool add_conj = false, int first_stage = 1);
 }
 CtxtTensor multMatMatFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1,
                            const CtxtTensor &op2, u64 T, MatrixTransformer &tr, u64 batch, bool single_tile) {
@@ -1144,9 +1151,11 @@ namespace {
 // three levels above the target.
 // add_conj: the result is x + conj(x) of the product x (the real part, twice, of a complex-packed product): inside the
 // giant-step sum where the schedule has one, by a conjugation afterwards otherwise.
+// first_stage = 2 (with pre at T+3): pre is what the first stage of the two-stage transforms from T+4 left -- taken
+// together with the packing, MatrixTransformer::packingStageOne -- and only the second stage runs here.
 CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const CtxtTensor &op1, const CtxtTensor &op2, u64 T,
                      MatrixTransformer &tr, u64 batch, bool single_tile, bool packed, const u64 *pre, u64 pre_level,
-                     bool merge_packing, bool add_conj) {
+                     bool merge_packing, bool add_conj, int first_stage) {
     const Context &c = eval.getContext();
     const i64 rows = op1.getHeight(), cols = op2.getWidth();
     const i64 k = pow2ceil(commonInside(op1, op2)), w = commonBlockWidth(op1, op2);
@@ -1179,7 +1188,13 @@ CtxtTensor ccmmFused(const HomEvaluator &eval, const Bootstrapper &btp, const Ct
                            shape_b.getNumRows() == shape_b.getNumCols();
     const u64 Lt = two_stage ? T + 4 : T + 3;   // level the transforms start from
     DeviceBuffer ab(c, 2 * ctw);
-    {
+    if (first_stage == 2) {   // the first stage came with the packing: the second one from T+3
+        if (!pre || pre_level != T + 3 || !packed || merge_packing)
+            throw std::invalid_argument("[multMatMat] a second stage alone takes packed operands prepared at T+3.");
+        const MaskKind kinds[2] = {MaskKind::PackedHorizontal, MaskKind::PackedVertical};
+        const TileTensorShape shapes[2] = {shape_a, shape_b};
+        tr.diagonalTransformTwoStage(eval, pre, 2, T + 4, kinds, shapes, ab.data(), nullptr, 2);
+    } else {
         const u64 ctw_in = 2 * (Lt + 1) * N;
         DeviceBuffer joint;
         const u64 *src = pre;
@@ -1538,7 +1553,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                     const u64 Lb = T + 3;
                     const DeviceBuffer jb = truncated(b.get(), Lb);
                     DeviceBuffer mid(c, 2 * Lb * N);
-                    tr.packingStageOne(eval, jb.data(), Lb, kind, shape_b, mid.data(), lb);
+                    tr.packingStageOne(eval, jb.data(), 1, Lb, &kind, &shape_b, mid.data(), &lb);
                     tr.diagonalTransformTwoStage(eval, mid.data(), 1, Lb, &kind, &shape_b, tb.data(), nullptr, 2);
                 }
             }
@@ -1556,7 +1571,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                 const DeviceBuffer ja = truncated(a.get(), La);
                 DeviceBuffer mid(c, 2 * La * N);
                 const MaskKind kind = MaskKind::PackedHorizontal;
-                tr.packingStageOne(eval, ja.data(), La, kind, shape_a, mid.data(), la);
+                tr.packingStageOne(eval, ja.data(), 1, La, &kind, &shape_a, mid.data(), &la);
                 tr.diagonalTransformTwoStage(eval, mid.data(), 1, La, &kind, &shape_a, sa.data(), nullptr, 2);
             } else {              // at T+3: packing and sigma as one composite one-stage transform (T+2)
                 const MaskKind kind = MaskKind::PackingHorizontal;
@@ -1586,6 +1601,16 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                            (uint32_t)(L + 1), 0, 2, nullptr));
     const bool by_rows[2] = {false, true};
     const u64 from[2] = {a.getLevel(), b.getLevel()};
+    if (L == T + 4 && a.getHeight() == a.getWidth() && b.getHeight() == b.getWidth() && a.getHeight() == b.getHeight() &&
+        pow2ceil(commonInside(a, b)) / 2 >= 4) {
+        // a level short of a separate packing in front of two-stage transforms: the packing and the first stage as one
+        // composite map for both operands (T+4 -> T+3); the product runs the second stage
+        const MaskKind kinds[2] = {MaskKind::PackedHorizontal, MaskKind::PackedVertical};
+        const i64 k = pow2ceil(commonInside(a, b)), w = commonBlockWidth(a, b);
+        const TileTensorShape shapes[2] = {TileTensorShape(a.getHeight(), k, w), TileTensorShape(k, b.getWidth(), w)};
+        tr.packingStageOne(eval, joint.data(), 2, L, kinds, shapes, packed.data(), from);
+        return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1, false, add_conj, 2);
+    }
     tr.complexPackingBatch(eval, joint.data(), 2, L, by_rows, a.getBlockWidth(), packed.data(), from);
     c->mark("complex packing");
     return ccmmFused(eval, btp, a, b, T, tr, batch, single_tile, true, packed.data(), L - 1, false, add_conj);

@@ -956,14 +956,15 @@ def mult_mat_mat_cc_fused(orc, a, b, T, n, w, single_tile=False):
 
 
 def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packing=False, with_conj=False,
-                              own_levels=False):
+                              own_levels=False, first_stage=1):
     """single_tile: the operands hold one tile block and nothing else (see mult_mat_mat_cc_fused).
     merge_packing: a and b are NOT packed yet; the packing and the packed transform run as one composite one-stage
     transform from T+3 (kinds PKH / PKV).
     with_conj: returns x + conj(x) of the product x -- inside the giant-step sum where the schedule has one, by a
     conjugation afterwards otherwise.
     own_levels: sigma(A) ends at T+2 and tau(B) at T+1 from whatever levels they arrive at (the form for operands one
-    level apart)."""
+    level apart).
+    first_stage = 2: a and b (at T+3) are what packing_stage_one left; only the second transform stage runs here."""
     from .oracle import Ct
     ev = OracleEval(orc)
     cm = [orc.encode_ext(m, T + 2) for m in col_masks(n, orc.slots)]
@@ -971,13 +972,17 @@ def mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=False, merge_packi
     lvl = min(a.level, b.level)
     rows, cols = _dims(n)
     # square tiles with A four and B three levels above the target take their own ways too (truncated to T+4 / T+3)
-    if (not merge_packing and a.level >= T + 4 and b.level >= T + 3 and rows == cols and n // 2 >= 4
-            and (n * w == orc.slots or spread)):
+    if (first_stage == 1 and not merge_packing and a.level >= T + 4 and b.level >= T + 3 and rows == cols
+            and n // 2 >= 4 and (n * w == orc.slots or spread)):
         own_levels = True
     if not own_levels and (merge_packing or lvl >= T + 3):
         if merge_packing:
             a = diagonal_transform_fused(orc, orc.level_down(a, T + 3), PKH, n, w)
             b = diagonal_transform_fused(orc, orc.level_down(b, T + 3), PKV, n, w)
+        elif first_stage == 2:
+            assert a.level == T + 3 == b.level
+            a = diagonal_transform_two_stage(orc, a, PH, n, w, first_stage=2)
+            b = diagonal_transform_two_stage(orc, b, PV, n, w, first_stage=2)
         # both operands a level above what B needs: sigma and tau share one launch chain and both end at T+2, as in
         # the unpacked product; tau(B) is lowered to T+1 with sigma(A)'s copy for the unshifted term
         else:
@@ -1071,6 +1076,12 @@ def mult_mat_mat_cc_packed(orc, a, b, T, n, w, single_tile):
     if min(a.level, b.level) == T + 3:   # one level short of a separate packing: packing and transform as one map
         return mult_packed_mat_mat_fused(orc, a, b, T, n, w, single_tile=single_tile, merge_packing=True, with_conj=True)
     lvl = min(a.level, b.level, T + 5)
+    if lvl == T + 4 and rows == cols and n // 2 >= 4:
+        # a level short of a separate packing in front of two-stage transforms: the packing and the first stage as one
+        # composite map for both operands (T+4 -> T+3); the product runs the second stage
+        pa = packing_stage_one(orc, cut(a, lvl), PH, n, w, a.level)
+        pb = packing_stage_one(orc, cut(b, lvl), PV, n, w, b.level)
+        return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True, first_stage=2)
     pa = complex_packing_hoisted(orc, cut(a, lvl), w, rows=False)
     pb = complex_packing_hoisted(orc, cut(b, lvl), w, rows=True)
     return mult_packed_mat_mat_fused(orc, pa, pb, T, n, w, single_tile=single_tile, with_conj=True)

@@ -222,6 +222,12 @@ def test_ccmm_stacked_tiles_keep_block_products(small):
     d = H.decrypt_slots(c).real[:512].reshape(32, 16)
     assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -18
     assert np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -18
+    # (the same at T+4: packing and first transform stage as one composite map for both operands, then the second stage)
+    c4 = H.single_cc_matmul(H.level_down(ca, 6), cb, 2)
+    want4 = R.mult_mat_mat_cc_packed(orc, to_oracle(orc, H.level_down(ca, 6)), to_oracle(orc, cb), 2, 16, 16, single_tile=False)
+    assert np.array_equal(c4.residues(), want4.data)
+    d = H.decrypt_slots(c4).real[:512].reshape(32, 16)
+    assert np.abs(d[:16] - A[:16] @ B[:16]).max() < 2 ** -18 and np.abs(d[16:] - A[16:] @ B[16:]).max() < 2 ** -18
     # three levels to spare: packing and packed transform as one composite transform, then the same masked shifts
     la, lb = H.level_down(ca, 5), H.level_down(cb, 5)
     c1 = H.single_cc_matmul(la, lb, 2)

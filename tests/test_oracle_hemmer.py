@@ -92,14 +92,16 @@ def test_lazy_pcmm_over_oracle(env):
     assert R.mult_mat_mat_pc_lazy(orc, enc(orc, A, 17), orc.encode(zfull, orc.nQ - 1), 2, n, n) is None
 
 
-def test_complex_packed_ccmm_on_stacked_tiles_over_oracle(env):
+@pytest.mark.parametrize("T", [2, 3])
+def test_complex_packed_ccmm_on_stacked_tiles_over_oracle(env, T):
     """Two tiles stacked in one ciphertext (block width n, 2 n rows) through the complex-packed product with masked
-    shifts of its two-column / two-row cells: each tile block of the result is the product of the operands' blocks."""
+    shifts of its two-column / two-row cells: each tile block of the result is the product of the operands' blocks.
+    T = 3 leaves the fresh operands (level 7) four levels: the packing and the first transform stage are one map."""
     orc, ev, n = env
     rng = np.random.default_rng(6)
     A, B = rng.uniform(-1, 1, (2 * n, n)), rng.uniform(-1, 1, (2 * n, n))
-    c = R.mult_mat_mat_cc_packed(orc, enc(orc, A, 23), enc(orc, B, 24), 2, n, n, single_tile=False)
-    assert c.level == 2 and c.scale == orc.delta[2]
+    c = R.mult_mat_mat_cc_packed(orc, enc(orc, A, 23), enc(orc, B, 24), T, n, n, single_tile=False)
+    assert c.level == T and c.scale == orc.delta[T]
     z = orc.decrypt(c)
     d = z[: 2 * n * n].real.reshape(2 * n, n)
     assert np.abs(d[:n] - A[:n] @ B[:n]).max() < 2 ** -18
