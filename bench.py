@@ -392,6 +392,29 @@ def gpu_rotation_60bit(args, out):
     out["rotation_24x60bit_level20_us"] = timer.stop() / 30 * 1e3
 
 
+def gpu_pcmm_loop(args, out):
+    """A loop of singleMatMul on the pair layout (two 128 x 128 products per call, the weight's tau prepared by the
+    warm-up calls), for kernel traces and counters; the figure is an extra key, not the headline."""
+    import numpy as np
+    from __graft_entry__ import load_package
+    load_package()
+    from efla_amd import hellm
+    H = hellm.HEMMer(preset=True, seed=3)
+    rng = np.random.default_rng(1)
+    A, A2, B, B2 = (rng.uniform(-1, 1, (128, 128)) for _ in range(4))
+    pa, pb = H.encrypt2(A, A2), H.encode2(B, B2)
+    for _ in range(max(1, args.warmup)):
+        c = H.single_matmul(pa, pb, 4)
+    H.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        c = H.single_matmul(pa, pb, 4)
+    H.sync()
+    out["pcmm_pair_layout_two_products_ms"] = (time.perf_counter() - t0) * 1e3 / args.steps
+    d = H.decrypt2(c)
+    out["pcmm_max_abs_err"] = float(max(np.abs(d[0] - A @ B).max(), np.abs(d[1] - A2 @ B2).max()))
+
+
 def gpu_layer_configs(args, out, H):
     """The two layer-level workloads, timed as extra keys (not the headline): the LoRA forward projection and one
     attention block of 12 heads, each with its max abs error against float64 algebra.  Inputs, keys, masks and
@@ -634,6 +657,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--roofline-only", action="store_true", help="run only the roofline legs")
     ap.add_argument("--ccmm-only", action="store_true", help="run only the headline product loop (for kernel traces)")
+    ap.add_argument("--pcmm-only", action="store_true",
+                    help="run only a loop of pair-layout plaintext x ciphertext products (for kernel traces)")
     ap.add_argument("--rotation-only", action="store_true",
                     help="run only the single key-switched rotation at the 24 x 60-bit shape (for kernel traces)")
     args = ap.parse_args()
@@ -660,6 +685,10 @@ def main():
     if args.roofline_only:
         gpu_hoisted(args, out)
         gpu_ntt(args, out)
+        print(json.dumps(out))
+        return
+    if args.pcmm_only:
+        gpu_pcmm_loop(args, out)
         print(json.dumps(out))
         return
     H = gpu_ccmm(args, out, headline_only=args.ccmm_only)
