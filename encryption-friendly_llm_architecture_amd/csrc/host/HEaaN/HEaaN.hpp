@@ -312,6 +312,15 @@ public:
     void sub(const Ciphertext &a, const Message &b, Ciphertext &out) const;
 
     void mult(const Ciphertext &a, const Ciphertext &b, Ciphertext &out) const;
+    // out[i] = mult(*a[i], *b[i]) for products that do not depend on one another -- the same residues as the calls one
+    // by one, through shared launches when the operands sit at one level: the tensor products, ONE ModUp of all the
+    // third polynomials, ONE sum with the multiplication key, ONE ModDown and ONE rescale.  (No counterpart in HEaaN's
+    // interface: the polynomial evaluators issue the independent products of a step together.)
+    void multBatch(const std::vector<const Ciphertext *> &a, const std::vector<const Ciphertext *> &b,
+                   std::vector<Ciphertext> &out) const;
+    // out[i] = rescale(multWithoutRescale(a, csts[i])) for real constants, the products through ONE rescale (same
+    // residues as the calls one by one; a is rescaled, two polynomials, above level 0)
+    void multRealBatch(const Ciphertext &a, const std::vector<Real> &csts, std::vector<Ciphertext> &out) const;
     void mult(const Ciphertext &a, const Plaintext &b, Ciphertext &out) const;
     void mult(const Ciphertext &a, const Message &b, Ciphertext &out) const;
     void mult(const Ciphertext &a, const Complex &c, Ciphertext &out) const;

@@ -1,6 +1,7 @@
 // HomEvaluator: level / scale bookkeeping on the host, arithmetic through the C ABI.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 
 #include "../../../include/hemm.h"
@@ -331,6 +332,116 @@ void HomEvaluator::mult(const Ciphertext &a, const Ciphertext &b, Ciphertext &ou
     out = std::move(t);
 }
 void HomEvaluator::square(const Ciphertext &a, Ciphertext &out) const { mult(a, a, out); }
+
+namespace {
+// hemm_rescale of n_polys polynomials stored back to back, in as few calls as the context's scratch region allows
+// ((dnum + 7) (nQ + nP) limbs per call)
+void rescale_many(const Context &c, const u64 *in, u64 *out, u64 nq, size_t n_polys) {
+    const u64 N = c->N;
+    const size_t per_call = std::max<size_t>(1, (size_t)((c->dnum + 7) * (c->nQ + c->nP) / nq));
+    for (size_t p0 = 0; p0 < n_polys; p0 += per_call) {
+        const size_t np = std::min(per_call, n_polys - p0);
+        ck(hemm_rescale(c->dev, in + p0 * nq * N, nq * N, out + p0 * (nq - 1) * N, (nq - 1) * N, (uint32_t)nq, (uint32_t)np,
+                        nullptr));
+    }
+}
+}  // namespace
+
+void HomEvaluator::multRealBatch(const Ciphertext &a, const std::vector<Real> &csts, std::vector<Ciphertext> &out) const {
+    require_rc0(a, "multRealBatch");
+    if (a.num_poly_ != 2 || a.level_ == 0) throw RuntimeException("multRealBatch: two polynomials above level 0 are needed");
+    const size_t n = csts.size();
+    const u64 lvl = a.level_, nq = lvl + 1, N = ctx_->N;
+    const Real delta = ctx_->delta[lvl];
+    std::vector<Ciphertext> res;
+    res.reserve(n);
+    if (n == 0) {
+        out = std::move(res);
+        return;
+    }
+    DeviceBuffer t(ctx_, n * 2 * nq * N), low(ctx_, n * 2 * lvl * N);
+    for (size_t i = 0; i < n; i++) {
+        const auto sc = int_residues(ctx_, (i64)llround(csts[i] * delta), nq);
+        ck(hemm_mul_scalar(ctx_->dev, a.buf_.data(), a.polyStride(), sc.data(), t.data() + i * 2 * nq * N, nq * N, (uint32_t)nq,
+                           0, 2, nullptr));
+    }
+    rescale_many(ctx_, t.data(), low.data(), nq, 2 * n);
+    for (size_t i = 0; i < n; i++) {
+        res.emplace_back(ctx_);
+        res.back().allocate(2, lvl - 1, 0);
+        (void)hipMemcpyAsync(res.back().buf_.data(), low.data() + i * 2 * lvl * N, 2 * lvl * N * 8, hipMemcpyDeviceToDevice,
+                             ctx_->stream());
+        res.back().occupied_ = a.occupied_;
+    }
+    out = std::move(res);
+}
+
+void HomEvaluator::multBatch(const std::vector<const Ciphertext *> &a, const std::vector<const Ciphertext *> &b,
+                             std::vector<Ciphertext> &out) const {
+    const size_t n = a.size();
+    if (n == 0 || n != b.size()) throw RuntimeException("multBatch: operand lists of different lengths");
+    bool shared = n > 1 && ctx_->N >= 512;   // (the hoisted sums need N >= 512)
+    for (size_t i = 0; i < n; i++) {
+        if (a[i] == nullptr || b[i] == nullptr) throw RuntimeException("multBatch: null operand");
+        shared = shared && a[i]->level_ == a[0]->level_ && b[i]->level_ == a[0]->level_ && a[i]->level_ > 0 &&
+                 a[i]->rescale_counter_ == 0 && b[i]->rescale_counter_ == 0 && a[i]->num_poly_ == 2 && b[i]->num_poly_ == 2;
+    }
+    std::vector<Ciphertext> res;
+    res.reserve(n);
+    if (!shared) {
+        for (size_t i = 0; i < n; i++) {
+            res.emplace_back(ctx_);
+            mult(*a[i], *b[i], res.back());
+        }
+        out = std::move(res);
+        return;
+    }
+    const u64 lvl = a[0]->level_, nq = lvl + 1, N = ctx_->N, E = nq + ctx_->nP, beta = (nq + ctx_->alpha - 1) / ctx_->alpha;
+    const u64 t3w = 3 * nq * N, ctw = 2 * nq * N;
+    // tensor products, three polynomials each
+    DeviceBuffer t3(ctx_, n * t3w);
+    for (size_t i = 0; i < n; i++)
+        ck(hemm_tensor(ctx_->dev, a[i]->buf_.data(), a[i]->polyStride(), b[i]->buf_.data(), b[i]->polyStride(),
+                       t3.data() + i * t3w, nq * N, (uint32_t)nq, 0, nullptr));
+    // relinearisation of all of them: d2 extended in one ModUp, <ext(d2), evk> + P (d0, d1) in one sum, one ModDown
+    // (ModDown(P d + k) = d + ModDown(k) residue for residue: what relinearize() adds after its ModDown)
+    DeviceBuffer ext(ctx_, n * beta * E * N), ws(ctx_, n * nq * N);
+    ck(hemm_modup_batch(ctx_->dev, t3.data() + 2 * nq * N, t3w, (uint32_t)nq, (uint32_t)n, ext.data(), ws.data(), nullptr));
+    std::vector<hemm_rot_term> terms;
+    std::vector<uint32_t> off{0};
+    for (size_t i = 0; i < n; i++) {
+        hemm_rot_term t{};
+        t.ext = ext.data() + i * beta * E * N;
+        t.b = t3.data() + i * t3w;
+        if (pack_.compactible()) {
+            t.evk = pack_.compactKey(0, 0);
+            t.flags = HEMM_ROT_COMPACT_KEY;
+        } else {
+            t.evk = pack_.multKey();
+        }
+        t.galois = 1;
+        t.pt_galois = 1;
+        terms.push_back(t);
+        hemm_rot_term d1{};   // the second polynomial needs no key: P d1 on the chain limbs
+        d1.ext = t3.data() + i * t3w + nq * N;
+        d1.galois = 1;
+        d1.pt_galois = 1;
+        terms.push_back(d1);
+        off.push_back((uint32_t)terms.size());
+    }
+    DeviceBuffer y(ctx_, n * 2 * E * N), r(ctx_, n * ctw), ws2(ctx_, n * ctw), low(ctx_, n * 2 * lvl * N);
+    ck(hemm_hoisted_moddown(ctx_->dev, terms.data(), off.data(), (uint32_t)n, (uint32_t)nq, 0, 0, y.data(), r.data(), nq * N,
+                            ws2.data(), nullptr));
+    rescale_many(ctx_, r.data(), low.data(), nq, 2 * n);
+    for (size_t i = 0; i < n; i++) {
+        res.emplace_back(ctx_);
+        res.back().allocate(2, lvl - 1, 0);
+        (void)hipMemcpyAsync(res.back().buf_.data(), low.data() + i * 2 * lvl * N, 2 * lvl * N * 8, hipMemcpyDeviceToDevice,
+                             ctx_->stream());
+        res.back().occupied_ = std::min(a[i]->occupied_, b[i]->occupied_);
+    }
+    out = std::move(res);
+}
 
 // Drop to target_level keeping the fixed per-level scale: read the first target+2 limbs, multiply by
 // round(Delta_target * q_{target+1} / Delta_level) and rescale by q_{target+1}.

@@ -156,43 +156,91 @@ struct Value {
     explicit Value(const Context &c) : ct(c) {}
 };
 
-// sum over b in [lo, lo + len) of e[b] prod_k T_{2^k}^{bit k of (b - lo)}; pw[k] = T_{2^k}.  A node of 2^k
-// coefficients sits k levels below the input: leaves e0 + e1 T_1 take one level (the constant is multiplied at the
-// scale of the level and rescaled, however small it is), each product with T_{len/2} one more.
-Value productTree(const HomEvaluator &eval, const std::vector<Ciphertext> &pw, const Real *e, size_t len) {
-    Value v(eval.getContext());
+// sum over b in [0, len) of e[b] prod_k T_{2^k}^{bit k of b}, pw[k] = T_{2^k}, as a binary tree: a node of 2^(k+1)
+// coefficients is lo + hi T_{2^k} with lo, hi its halves and sits k + 1 levels below the input: leaves e0 + e1 T_1 take
+// one level (the constant is multiplied at the scale of the level and rescaled, however small it is), each product
+// with T_{2^k} one more.  The tree is taken level by level: the products of one level do not depend on one another and
+// go through HomEvaluator::multBatch together with the square that makes T_{2^(k+1)} for the next level (same residues
+// as one product after the other).  pw holds T_1 on entry and is extended as far as the tree multiplies.
+Value productTree(const HomEvaluator &eval, std::vector<Ciphertext> &pw, const Real *e, size_t len) {
+    const Context &ctx = eval.getContext();
     if (len == 1) {
+        Value v(ctx);
         v.cst = e[0];
         return v;
     }
-    if (len == 2) {
-        v.cst = e[0];
-        if (e[1] != 0.0) {
-            eval.multWithoutRescale(pw[0], Complex(e[1], 0.0), v.ct);
-            eval.rescale(v.ct);
-            if (e[0] != 0.0) eval.add(v.ct, Complex(e[0], 0.0), v.ct);
-            v.has_ct = true;
+    std::vector<Value> cur;
+    {   // leaves e0 + e1 T_1: the products by the constants through one rescale
+        std::vector<Real> csts;
+        for (size_t j = 0; j < len / 2; j++)
+            if (e[2 * j + 1] != 0.0) csts.push_back(e[2 * j + 1]);
+        std::vector<Ciphertext> scaled;
+        eval.multRealBatch(pw[0], csts, scaled);
+        size_t taken = 0;
+        for (size_t j = 0; j < len / 2; j++) {
+            Value v(ctx);
+            v.cst = e[2 * j];
+            if (e[2 * j + 1] != 0.0) {
+                v.ct = std::move(scaled[taken++]);
+                if (e[2 * j] != 0.0) eval.add(v.ct, Complex(e[2 * j], 0.0), v.ct);
+                v.has_ct = true;
+            }
+            cur.push_back(std::move(v));
         }
-        return v;
     }
-    const size_t h = len / 2;
-    size_t k = 0;
-    while (((size_t)1 << k) < h) k++;
-    Value lo = productTree(eval, pw, e, h), hi = productTree(eval, pw, e + h, h);
-    if (hi.has_ct) {
-        eval.mult(hi.ct, pw[k], v.ct);
-        v.has_ct = true;
-    } else if (hi.cst != 0.0) {
-        eval.multWithoutRescale(pw[k], Complex(hi.cst, 0.0), v.ct);
-        eval.rescale(v.ct);
-        v.has_ct = true;
+    auto next_power = [&](const Ciphertext &square) {   // T_{2m} = 2 T_m^2 - 1
+        Ciphertext p(square);
+        eval.add(p, p, p);
+        eval.add(p, Complex(-1.0, 0.0), p);
+        pw.push_back(std::move(p));
+    };
+    if (cur.size() > 1) {   // T_2, which the first level of products multiplies by
+        Ciphertext sq(ctx);
+        eval.mult(pw[0], pw[0], sq);
+        next_power(sq);
     }
-    if (!v.has_ct) return lo;
-    if (lo.has_ct)
-        eval.add(v.ct, lo.ct, v.ct);
-    else if (lo.cst != 0.0)
-        eval.add(v.ct, Complex(lo.cst, 0.0), v.ct);
-    return v;
+    for (size_t k = 1; cur.size() > 1; k++) {
+        const size_t n_nodes = cur.size() / 2;
+        const bool more = n_nodes > 1;   // the next level multiplies by T_{2^(k+1)}
+        std::vector<const Ciphertext *> fa, fb;
+        for (size_t j = 0; j < n_nodes; j++)
+            if (cur[2 * j + 1].has_ct) {
+                fa.push_back(&cur[2 * j + 1].ct);
+                fb.push_back(&pw[k]);
+            }
+        if (more) {
+            fa.push_back(&pw[k]);
+            fb.push_back(&pw[k]);
+        }
+        std::vector<Ciphertext> prod;
+        if (!fa.empty()) eval.multBatch(fa, fb, prod);
+        std::vector<Value> next;
+        size_t taken = 0;
+        for (size_t j = 0; j < n_nodes; j++) {
+            Value &lo = cur[2 * j], &hi = cur[2 * j + 1];
+            Value v(ctx);
+            if (hi.has_ct) {
+                v.ct = std::move(prod[taken++]);
+                v.has_ct = true;
+            } else if (hi.cst != 0.0) {
+                eval.multWithoutRescale(pw[k], Complex(hi.cst, 0.0), v.ct);
+                eval.rescale(v.ct);
+                v.has_ct = true;
+            }
+            if (!v.has_ct) {
+                next.push_back(std::move(lo));
+                continue;
+            }
+            if (lo.has_ct)
+                eval.add(v.ct, lo.ct, v.ct);
+            else if (lo.cst != 0.0)
+                eval.add(v.ct, Complex(lo.cst, 0.0), v.ct);
+            next.push_back(std::move(v));
+        }
+        if (more) next_power(prod[taken]);
+        cur = std::move(next);
+    }
+    return std::move(cur[0]);
 }
 
 }  // namespace
@@ -231,15 +279,8 @@ Ciphertext evaluateChebyshevExpansion(const HomEvaluator &eval, const Bootstrapp
     while (top > 1 && e[top - 1] == 0.0) top--;
     size_t len = 2;
     while (len < top) len *= 2;
-    std::vector<Ciphertext> pw;      // T_1, T_2, T_4, ... as far as the tree multiplies by them
+    std::vector<Ciphertext> pw;      // T_1; the tree adds T_2, T_4, ... as far as it multiplies by them
     pw.push_back(ctxt);
-    Ciphertext p(eval.getContext());
-    for (size_t m = 2; m < len; m *= 2) {
-        eval.mult(pw.back(), pw.back(), p);
-        eval.add(p, p, p);
-        eval.add(p, Complex(-1.0, 0.0), p);
-        pw.push_back(p);
-    }
     Value v = productTree(eval, pw, e.data(), len);
     if (!v.has_ct) throw std::invalid_argument("[evaluateChebyshevExpansion] constant polynomial");
     return v.ct;
