@@ -25,7 +25,7 @@ void exp_iter_Parallel(const HomEvaluator &eval, const Bootstrapper &btp, std::v
         eval.mult(t.get(), Complex(1.0 / std::pow(2, num_iter), 0.0), t.get());
         eval.add(t.get(), Complex(1.0, 0.0), t.get());
     }
-    for (int i = 0; i < num_iter; i++)
+    for (int i = 0; i < num_iter; i++) {
         for (size_t j = 0; j < op.size() / 2; j++) {
             Ciphertext &a = op[2 * j].get(), &b = op[2 * j + 1].get();
             if (a.getLevel() == btp.getMinLevelForBootstrap()) {
@@ -33,9 +33,15 @@ void exp_iter_Parallel(const HomEvaluator &eval, const Bootstrapper &btp, std::v
                 eval.add(a, b, a);
                 btp.bootstrap(a, a, b);
             }
-            eval.square(a, a);
-            eval.square(b, b);
         }
+        // the squares of a round do not depend on one another: one launch chain for all of them (same residues)
+        std::vector<const Ciphertext *> xs;
+        for (size_t j = 0; j < 2 * (op.size() / 2); j++) xs.push_back(&op[j].get());
+        if (xs.empty()) continue;
+        std::vector<Ciphertext> sq;
+        eval.multBatch(xs, xs, sq);
+        for (size_t j = 0; j < sq.size(); j++) op[j].get() = std::move(sq[j]);
+    }
 }
 
 }  // namespace Exp
