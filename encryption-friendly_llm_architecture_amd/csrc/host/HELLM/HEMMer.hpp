@@ -186,6 +186,9 @@ public:
 private:
     void init();
     const Plaintext &cachedMask(int id, u64 level) const;
+    // the 0/1 masks of the reductions and the rank-2 LoRA path (column 0, column n-1, left / right half of the columns,
+    // row 0; on both tiles of the pair layout or on the left one only), encoded once per level
+    const Plaintext &selectorMask(int which, u64 level) const;
     std::vector<u64> transformRotations(MaskKind kind, i64 width) const;
     // the same for a (possibly rectangular) sigma / tau shape under the current schedule
     std::vector<u64> transformRotations(MaskKind kind, const TileTensorShape &shape) const;

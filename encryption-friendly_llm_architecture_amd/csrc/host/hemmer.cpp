@@ -84,6 +84,33 @@ const Plaintext &HEMMer::cachedMask(int id, u64 level) const {
     return mask_cache_.emplace(key, endec_.encode(*m, level)).first->second;
 }
 
+namespace {
+enum { SEL_FIRST_COL = 100, SEL_LAST_COL, SEL_LEFT_COLS, SEL_RIGHT_COLS, SEL_FIRST_ROW, SEL_FIRST_COL_LEFT_TILE };
+}
+const Plaintext &HEMMer::selectorMask(int which, u64 level) const {
+    auto key = std::make_pair(which, level);
+    auto it = mask_cache_.find(key);
+    if (it != mask_cache_.end()) return it->second;
+    const i64 n = dim_;
+    Matrix m(n, n, 0.0), zero(n, n, 0.0);
+    for (i64 r = 0; r < n; r++)
+        for (i64 c = 0; c < n; c++) {
+            bool on = false;
+            switch (which) {
+                case SEL_FIRST_COL:
+                case SEL_FIRST_COL_LEFT_TILE: on = c == 0; break;
+                case SEL_LAST_COL: on = c == n - 1; break;
+                case SEL_LEFT_COLS: on = c < n / 2; break;
+                case SEL_RIGHT_COLS: on = c >= n / 2; break;
+                case SEL_FIRST_ROW: on = r == 0; break;
+                default: throw std::invalid_argument("[selectorMask] unknown mask");
+            }
+            if (on) m.at(r, c) = 1.0;
+        }
+    const Message msg = which == SEL_FIRST_COL_LEFT_TILE ? message2(m, zero) : message2(m, m);
+    return mask_cache_.emplace(key, endec_.encode(msg, level)).first->second;
+}
+
 void HEMMer::ensureRotationKeys(const std::vector<u64> &rots) const {
     const u64 slots = u64(1) << log_slots_;
     KeyGenerator keygen(context_, sk_, pack_);
@@ -205,11 +232,6 @@ void HEMMer::reduceRowSumWithScaledMask(CtxtTensor &tensor, const Message &mask)
 
 void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
     const u64 n = (u64)dim_, slots = u64(1) << log_slots_;
-    Matrix first(dim_, dim_, 0.0), last(dim_, dim_, 0.0);
-    for (i64 r = 0; r < dim_; r++) {
-        first.at(r, 0) = 1.0;
-        last.at(r, dim_ - 1) = 1.0;
-    }
     if (fused_ && n >= 4 && (n & (n - 1)) == 0 && a.getLevel() == b.getLevel()) {
         // both tensors through the same launch chains: a to the left and b to the right, then the other way round
         for (i64 unit : {i64(1), i64(-1)}) {
@@ -217,8 +239,8 @@ void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
             ensureRotationKeys(rotateSumRotations(unit, n, log_slots_));
         }
         rotateSumFused(eval_, {{&a.get(), 1, &a.get()}, {&b.get(), -1, &b.get()}}, n / 2);
-        eval_.mult(a.get(), message2(first, first), a.get());
-        eval_.mult(b.get(), message2(last, last), b.get());
+        eval_.mult(a.get(), selectorMask(SEL_FIRST_COL, a.getLevel()), a.get());
+        eval_.mult(b.get(), selectorMask(SEL_LAST_COL, b.getLevel()), b.get());
         rotateSumFused(eval_, {{&a.get(), -1, &a.get()}, {&b.get(), 1, &b.get()}}, n);
         return;
     }
@@ -230,8 +252,8 @@ void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
         eval_.rightRotate(b.get(), rot, tmp);
         eval_.add(b.get(), tmp, b.get());
     }
-    eval_.mult(a.get(), message2(first, first), a.get());
-    eval_.mult(b.get(), message2(last, last), b.get());
+    eval_.mult(a.get(), selectorMask(SEL_FIRST_COL, a.getLevel()), a.get());
+    eval_.mult(b.get(), selectorMask(SEL_LAST_COL, b.getLevel()), b.get());
     for (u64 rot = 1; rot < n; rot <<= 1) {
         eval_.rightRotate(a.get(), rot, tmp);
         eval_.add(a.get(), tmp, a.get());
@@ -241,17 +263,12 @@ void HEMMer::oneMatRotSumInplace(CtxtTensor &a, CtxtTensor &b) const {
 }
 
 void HEMMer::maskRightLeft(const CtxtTensor &tensor, CtxtTensor &out_left, CtxtTensor &out_right) const {
-    Matrix left(dim_, dim_, 0.0), right(dim_, dim_, 0.0);
-    for (i64 r = 0; r < dim_; r++)
-        for (i64 c = 0; c < dim_; c++) (c < dim_ / 2 ? left : right).at(r, c) = 1.0;
-    eval_.mult(tensor.get(), message2(left, left), out_left.get());
-    eval_.mult(tensor.get(), message2(right, right), out_right.get());
+    eval_.mult(tensor.get(), selectorMask(SEL_LEFT_COLS, tensor.getLevel()), out_left.get());
+    eval_.mult(tensor.get(), selectorMask(SEL_RIGHT_COLS, tensor.getLevel()), out_right.get());
 }
 
 void HEMMer::maskFirstColInplace(CtxtTensor &tensor) const {
-    Matrix first(dim_, dim_, 0.0);
-    for (i64 r = 0; r < dim_; r++) first.at(r, 0) = 1.0;
-    eval_.mult(tensor.get(), message2(first, first), tensor.get());
+    eval_.mult(tensor.get(), selectorMask(SEL_FIRST_COL, tensor.getLevel()), tensor.get());
 }
 
 void HEMMer::rowMoments(const std::vector<CtxtTensor> &tiles, Real inv_count, CtxtTensor &mean,
@@ -863,14 +880,10 @@ CtxtTensor HEMMer::repack_loraOpti(CtxtTensor &t1, CtxtTensor &t2) const {
 
 // ---- rank-2 LoRA through element-wise products ---------------------------------------------------------------
 void HEMMer::maskFirstRowInplace(CtxtTensor &tensor) const {
-    Matrix first(dim_, dim_, 0.0);
-    for (i64 c = 0; c < dim_; c++) first.at(0, c) = 1.0;
-    eval_.mult(tensor.get(), message2(first, first), tensor.get());
+    eval_.mult(tensor.get(), selectorMask(SEL_FIRST_ROW, tensor.getLevel()), tensor.get());
 }
 void HEMMer::maskFirstColOnlyInplace(CtxtTensor &tensor) const {
-    Matrix first(dim_, dim_, 0.0), zero(dim_, dim_, 0.0);
-    for (i64 r = 0; r < dim_; r++) first.at(r, 0) = 1.0;
-    eval_.mult(tensor.get(), message2(first, zero), tensor.get());
+    eval_.mult(tensor.get(), selectorMask(SEL_FIRST_COL_LEFT_TILE, tensor.getLevel()), tensor.get());
 }
 // rows 2i and 2i+1 of the weight tile, each moved to row 0, masked and copied to every row
 std::vector<std::vector<CtxtTensor>> HEMMer::splitWeightRows(const CtxtTensor &weight, u64 count) const {
