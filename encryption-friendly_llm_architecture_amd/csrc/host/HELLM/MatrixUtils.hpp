@@ -117,6 +117,9 @@ public:
 
     void cleanUp();
     size_t cachedMasks() const;
+    // The caches hold masks of ONE parameter set (ring size, chain and special primes, scale factors): contexts over the
+    // same set share them; the first call with a context over another set empties them.  Every cached lookup starts here.
+    void useChainOf(const Context &c);
 
 private:
     struct Key {
@@ -130,6 +133,8 @@ private:
     };
     Ciphertext diagonalTransform(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
                                  const TileTensorShape &shape);
+    std::vector<u64> chain_;   // N, nQ, the primes and the bit patterns of the scale factors the caches belong to
+    Context last_context_;     // the context of the last lookup (held, so that its address cannot be taken by another)
     std::map<Key, Plaintext> masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_, row_masks_;
     std::map<std::pair<TileTensorShape, u64>, std::vector<Plaintext>> col_masks_ext_, row_masks_ext_, col_masks_ext_first_;

@@ -3,6 +3,7 @@
 // transforms :671-1098, products :1100-1679) restated over this build's evaluator.
 #include <algorithm>
 #include <cmath>
+#include <cstring>
 
 #include "HELLM/MatrixUtils.hpp"
 
@@ -128,6 +129,7 @@ Message transformMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 lo
 
 const Plaintext &MatrixTransformer::transformMask(const HomEvaluator &eval, MaskKind kind,
                                                   const TileTensorShape &shape, u64 level, i64 idx) {
+    useChainOf(eval.getContext());
     Key key{(int)kind, shape, level, idx};
     auto it = masks_.find(key);
     if (it != masks_.end()) return it->second;
@@ -152,6 +154,7 @@ const Plaintext &MatrixTransformer::transformMask(const HomEvaluator &eval, Mask
 
 std::vector<Plaintext> &MatrixTransformer::getColMask(const HomEvaluator &eval, const TileTensorShape &shape,
                                                       u64 level) {
+    useChainOf(eval.getContext());
     auto key = std::make_pair(shape, level);
     auto it = col_masks_.find(key);
     if (it != col_masks_.end()) return it->second;
@@ -177,6 +180,7 @@ std::vector<Plaintext> &MatrixTransformer::getColMask(const HomEvaluator &eval, 
 
 std::vector<Plaintext> &MatrixTransformer::getRowMask(const HomEvaluator &eval, const TileTensorShape &shape,
                                                       u64 level) {
+    useChainOf(eval.getContext());
     auto key = std::make_pair(shape, level);
     auto it = row_masks_.find(key);
     if (it != row_masks_.end()) return it->second;
@@ -204,12 +208,44 @@ void MatrixTransformer::cleanUp() {
     masks_.clear();
     col_masks_.clear();
     row_masks_.clear();
+    col_masks_ext_.clear();
+    row_masks_ext_.clear();
+    col_masks_ext_first_.clear();
+    first_block_masks_.clear();
+    two_stage_masks_.clear();
+    packing_stage_one_masks_.clear();
+    pack_masks_.clear();
+    weight_tau_.clear();
+    weight_tau_order_.clear();
+    chain_.clear();
+    last_context_ = Context();
 }
 size_t MatrixTransformer::cachedMasks() const {
-    size_t n = masks_.size();
+    size_t n = masks_.size() + first_block_masks_.size() + two_stage_masks_.size() + pack_masks_.size();
     for (auto &kv : col_masks_) n += kv.second.size();
     for (auto &kv : row_masks_) n += kv.second.size();
+    for (auto &kv : col_masks_ext_) n += kv.second.size();
+    for (auto &kv : row_masks_ext_) n += kv.second.size();
+    for (auto &kv : col_masks_ext_first_) n += kv.second.size();
+    for (auto &kv : packing_stage_one_masks_) n += kv.second.size();
     return n;
+}
+void MatrixTransformer::useChainOf(const Context &c) {
+    if (c.get() == last_context_.get()) return;
+    last_context_ = c;
+    std::vector<u64> sig{getDegree(c), getEncryptionLevel(c)};
+    const std::vector<u64> primes = getPrimeList(c);
+    sig.insert(sig.end(), primes.begin(), primes.end());
+    for (Real d : getDefaultScaleFactorList(c)) {
+        u64 bits;
+        static_assert(sizeof(bits) == sizeof(d), "scale factors are doubles");
+        std::memcpy(&bits, &d, sizeof(bits));
+        sig.push_back(bits);
+    }
+    if (sig == chain_) return;
+    if (!chain_.empty()) cleanUp();
+    chain_ = std::move(sig);
+    last_context_ = c;
 }
 
 // T(A) = M_0 * A + sum_{d != 0} M_d * rot_{d step}(A), d in (-units, units), grouped so that only

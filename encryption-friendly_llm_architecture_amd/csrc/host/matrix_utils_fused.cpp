@@ -131,6 +131,7 @@ hemm_rot_term keylessTerm(const u64 *b, const u64 *a, const Plaintext *mask) {
 }  // namespace
 
 const Plaintext &MatrixTransformer::firstBlockMask(const HomEvaluator &eval, const TileTensorShape &shape, u64 level) {
+    useChainOf(eval.getContext());
     auto key = std::make_pair(shape, level);
     auto it = first_block_masks_.find(key);
     if (it != first_block_masks_.end()) return it->second;
@@ -144,6 +145,7 @@ const Plaintext &MatrixTransformer::firstBlockMask(const HomEvaluator &eval, con
 
 std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
                                                          u64 level, bool first_block_only) {
+    useChainOf(eval.getContext());
     auto key = std::make_pair(shape, level);
     auto &cache = first_block_only ? col_masks_ext_first_ : col_masks_ext_;
     auto it = cache.find(key);
@@ -174,6 +176,7 @@ std::vector<Plaintext> &MatrixTransformer::getColMaskExt(const HomEvaluator &eva
 }
 std::vector<Plaintext> &MatrixTransformer::getRowMaskExt(const HomEvaluator &eval, const TileTensorShape &shape,
                                                          u64 level) {
+    useChainOf(eval.getContext());
     auto key = std::make_pair(shape, level);
     auto it = row_masks_ext_.find(key);
     if (it != row_masks_ext_.end()) return it->second;
@@ -536,6 +539,7 @@ Message twoStageMaskMessage(MaskKind kind, const TileTensorShape &shape, u64 log
 
 const Plaintext &MatrixTransformer::twoStageMask(const HomEvaluator &eval, MaskKind kind, const TileTensorShape &shape,
                                                  u64 level, int stage, i64 r, int part, u64 from) {
+    useChainOf(eval.getContext());
     if (from == level) from = 0;   // the level's own scale
     Key key{(int)kind, shape, level, ((i64)from * 4 + stage) * 4096 + r * 4 + part};
     auto it = two_stage_masks_.find(key);
@@ -732,6 +736,7 @@ void MatrixTransformer::packingStageOne(const HomEvaluator &eval, const u64 *in,
     const Context &c = eval.getContext();
     if (level < 1) throw std::invalid_argument("[packingStageOne] level >= 1 is needed.");
     const u64 nq = level + 1, N = c->N, E = nq + c->nP, ctw = 2 * nq * N;
+    useChainOf(c);
     const Sources x = extendSources(c, in, n_jobs, nq, nullptr, false);
     const KeyPack &pack = eval.getKeyPack();
     const u64 M = 2 * N;
@@ -781,6 +786,7 @@ void MatrixTransformer::complexPackingBatch(const HomEvaluator &eval, const u64 
     const u64 log_slots = getLogFullSlots(c);
     // All three masks of a job are encoded over the extended basis (the unrotated term reads the chain limbs only) at
     // the scale that takes the input's scale to the fixed scale of level - 1 across the rescale.
+    useChainOf(c);
     auto mask = [&](bool by_rows, int part, u64 from) -> const Plaintext & {
         const auto key = std::make_tuple((int)by_rows, w, level, part, from);
         auto it = pack_masks_.find(key);
@@ -1798,6 +1804,7 @@ bool multMatMatPlainFused(const HomEvaluator &eval, const Bootstrapper &btp, con
             weight.hash_state_ = 1;
         }
     }
+    tr.useChainOf(c);
     const auto key = std::make_tuple(weight_hash.first, weight_hash.second, shape_b, T);
     auto it = tr.weight_tau_.find(key);
     if (it == tr.weight_tau_.end()) {

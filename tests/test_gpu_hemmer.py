@@ -695,3 +695,29 @@ def test_full_pcmm_packed_and_hoisted(full):
     H.transpose_inplace(t)
     d = H.decrypt2(t)
     assert np.abs(d[0] - A.T).max() < TOL and np.abs(d[1] - A2.T).max() < TOL
+
+
+def test_two_parameter_sets_take_turns(small):
+    """Two HEMMers over different prime chains with the same tile shape, used in turn: the mask caches behind the
+    products belong to one parameter set at a time (masks are keyed by kind, shape and level, all of which the two sets
+    share), so each product must still give the residues of its own oracle."""
+    from efla_amd import hellm
+    H1, orc1, _ = small
+    qs, ps = O.ckks_chain(10, 9, 3)
+    assert len(qs) == len(orc1.q) + 1
+    H2 = hellm.HEMMer(10, qs, ps, dnum=3, min_bootstrap_level=0, seed=9)
+    orc2 = O.Oracle(10, qs, ps, dnum=3)
+    gen_oracle_keys(orc2, 9, H2.dim)
+    rng = np.random.default_rng(77)
+    A, B = rng.uniform(-1, 1, (16, 16)), rng.uniform(-1, 1, (16, 16))
+    for H, orc in ((H1, orc1), (H2, orc2), (H1, orc1), (H2, orc2)):
+        ca, cb = H.encrypt(A), H.encrypt(B)
+        a = H.level_down(ca, 6) if ca.info()["level"] > 6 else ca
+        b = H.level_down(cb, 6) if cb.info()["level"] > 6 else cb
+        c = H.single_cc_matmul(a, b, 2)
+        want = R.mult_mat_mat_cc_packed_single(orc, to_oracle(orc, a), to_oracle(orc, b), 2, 16, 16)
+        assert np.array_equal(c.residues(), want.data)
+        assert np.abs(H.decrypt(c) - A @ B).max() < 2 ** -18
+        w = H.encode(B)
+        p = H.single_matmul(ca, w, 2)
+        assert np.abs(H.decrypt(p) - A @ B).max() < 2 ** -18
