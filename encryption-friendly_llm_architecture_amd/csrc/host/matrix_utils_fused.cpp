@@ -283,6 +283,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
         }
     DeviceBuffer y(c, n_baby * 2 * E * N), baby(c, n_baby * ctw), ws(c, n_baby * ctw);
     ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)n_baby, (uint32_t)nq, 1, 0, y.data(), baby.data(), nq * N, ws.data(), nullptr));
+    c->mark("one-stage transform: baby rotations");
 
     // 2. group sums: a job's group 0 needs no rotation (d = 0, the positive diagonals of giant index 0, and
     //    any group whose rotation is a whole turn).  The unrotated groups of all jobs come first in `sums`,
@@ -342,6 +343,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
     const size_t ng = rotated.size(), n_groups = n_jobs + ng;
     DeviceBuffer sums(c, n_groups * ctw);
     ck(hemm_masked_sum_batch(c->dev, lt.data(), loff.data(), (uint32_t)n_groups, (uint32_t)nq, 2, sums.data(), nullptr));
+    c->mark("one-stage transform: masked group sums");
 
     // 3. giant steps: every rotated group is a term of its job's output; the group that is not rotated joins the same
     // sum as a term without a key, and the sum takes one ModDown merged with the rescale
@@ -367,6 +369,7 @@ void MatrixTransformer::diagonalTransformBatch(const HomEvaluator &eval, const u
     } else {
         throw RuntimeException("diagonalTransformBatch: jobs with and without giant steps cannot share a batch");
     }
+    c->mark("one-stage transform: giant steps");
 }
 
 Ciphertext MatrixTransformer::diagonalTransformFused(const HomEvaluator &eval, const Ciphertext &in, MaskKind kind,
