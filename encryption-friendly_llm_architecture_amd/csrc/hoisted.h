@@ -56,9 +56,8 @@ __device__ __forceinline__ ulonglong2 load_mask_run(const u64 *mask, const u32 s
 }
 // x1 * w1 + x2 * w2 mod q for run-table constants, canonical
 __device__ __forceinline__ u64 shoup_pair(u64 x1, const ulonglong2 w1, u64 x2, const ulonglong2 w2, u64 q) {
-    u64 z = mul_shoup_lazy(x1, w1.x, w1.y, q) + mul_shoup_lazy(x2, w2.x, w2.y, q);   // < 4q < 2^63
-    if (z >= 2 * q) z -= 2 * q;
-    return z >= q ? z - q : z;
+    const u64 z = mul_shoup_lazy_u(x1, w1.x, w1.y, q) + mul_shoup_lazy_u(x2, w2.x, w2.y, q);   // < 4q < 2^63
+    return cond_sub_u(cond_sub_u(z, 2 * q), q);
 }
 // residues (n, n+1) of limb j of a plaintext read through the automorphism X -> X^g (an aligned pair stays an aligned
 // pair, possibly swapped)
@@ -165,10 +164,10 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *_
         m2 = load_mask2(T.mask2, T.mask_shift, j, n, logN);
         if (T.pt != nullptr) {
             const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
-            m1.x = mulmod(m1.x, pv.x, m);
-            m1.y = mulmod(m1.y, pv.y, m);
-            m2.x = mulmod(m2.x, pv.x, m);
-            m2.y = mulmod(m2.y, pv.y, m);
+            m1.x = mulmod_u(m1.x, pv.x, m);
+            m1.y = mulmod_u(m1.y, pv.y, m);
+            m2.x = mulmod_u(m2.x, pv.x, m);
+            m2.y = mulmod_u(m2.y, pv.y, m);
         }
     }
     u128_t pb[2] = {{0, 0}, {0, 0}}, pa[2] = {{0, 0}, {0, 0}};
@@ -191,8 +190,8 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *_
             u128_t t0 = mul64wide(m1.x, x1.x), t1 = mul64wide(m1.y, x1.y);
             add128(t0, mul64wide(m2.x, x2.x));
             add128(t1, mul64wide(m2.y, x2.y));
-            z0 = barrett3(t0, m);
-            z1 = barrett3(t1, m);
+            z0 = barrett3_u(t0, m);
+            z1 = barrett3_u(t1, m);
         }
         const ulonglong2 kb = key_pair_ptr<COMPACT>(T, koff, d, 0, prime, logN, n_full, n);
         const ulonglong2 ka = key_pair_ptr<COMPACT>(T, koff, d, 1, prime, logN, n_full, n);
@@ -202,15 +201,15 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *_
         add128(pa[1], mul64wide(z1, ka.y));
     }
     if (beta <= 3) {   // at most 3 q^2: the short reduction applies
-        rb[0] = barrett3(pb[0], m);
-        rb[1] = barrett3(pb[1], m);
-        ra[0] = barrett3(pa[0], m);
-        ra[1] = barrett3(pa[1], m);
+        rb[0] = barrett3_u(pb[0], m);
+        rb[1] = barrett3_u(pb[1], m);
+        ra[0] = barrett3_u(pa[0], m);
+        ra[1] = barrett3_u(pa[1], m);
     } else {
-        rb[0] = barrett128(pb[0], m);
-        rb[1] = barrett128(pb[1], m);
-        ra[0] = barrett128(pa[0], m);
-        ra[1] = barrett128(pa[1], m);
+        rb[0] = barrett128_u(pb[0], m);
+        rb[1] = barrett128_u(pb[1], m);
+        ra[0] = barrett128_u(pa[0], m);
+        ra[1] = barrett128_u(pa[1], m);
     }
     if (j < nq) {
         ulonglong2 b1 = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
@@ -224,20 +223,20 @@ __device__ __forceinline__ void two_source_int(const RotTermDev &T, const u32 *_
             b2.y = tmp;
         }
         if (!b_premultiplied) {
-            b1.x = mul_shoup(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-            b1.y = mul_shoup(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
-            b2.x = mul_shoup(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-            b2.y = mul_shoup(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b1.x = mul_shoup_u(b1.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b1.y = mul_shoup_u(b1.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b2.x = mul_shoup_u(b2.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+            b2.y = mul_shoup_u(b2.y, pmod.c[j].w, pmod.c[j].ws, m.q);
         }
         if (RUNS) {
-            rb[0] = addmod(rb[0], shoup_pair(b1.x, m1, b2.x, m2, m.q), m.q);
-            rb[1] = addmod(rb[1], shoup_pair(b1.y, m1, b2.y, m2, m.q), m.q);
+            rb[0] = addmod_u(rb[0], shoup_pair(b1.x, m1, b2.x, m2, m.q), m.q);
+            rb[1] = addmod_u(rb[1], shoup_pair(b1.y, m1, b2.y, m2, m.q), m.q);
         } else {
             u128_t t0 = mul64wide(m1.x, b1.x), t1 = mul64wide(m1.y, b1.y);
             add128(t0, mul64wide(m2.x, b2.x));
             add128(t1, mul64wide(m2.y, b2.y));
-            rb[0] = addmod(rb[0], barrett3(t0, m), m.q);
-            rb[1] = addmod(rb[1], barrett3(t1, m), m.q);
+            rb[0] = addmod_u(rb[0], barrett3_u(t0, m), m.q);
+            rb[1] = addmod_u(rb[1], barrett3_u(t1, m), m.q);
         }
     }
 }
@@ -272,19 +271,19 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                                               b_premultiplied, rb, ra);
                 if (T.pt != nullptr) {
                     const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
-                    rb[0] = mulmod(rb[0], pv.x, m);
-                    rb[1] = mulmod(rb[1], pv.y, m);
-                    ra[0] = mulmod(ra[0], pv.x, m);
-                    ra[1] = mulmod(ra[1], pv.y, m);
+                    rb[0] = mulmod_u(rb[0], pv.x, m);
+                    rb[1] = mulmod_u(rb[1], pv.y, m);
+                    ra[0] = mulmod_u(ra[0], pv.x, m);
+                    ra[1] = mulmod_u(ra[1], pv.y, m);
                 }
             } else {
                 two_source_int<false, COMPACT>(T, koff, m, pmod, j, prime, n, base, swap, nq, E, beta, n_full, logN,
                                                b_premultiplied, rb, ra);
             }
-            acc_b[0] = addmod(acc_b[0], rb[0], m.q);
-            acc_b[1] = addmod(acc_b[1], rb[1], m.q);
-            acc_a[0] = addmod(acc_a[0], ra[0], m.q);
-            acc_a[1] = addmod(acc_a[1], ra[1], m.q);
+            acc_b[0] = addmod_u(acc_b[0], rb[0], m.q);
+            acc_b[1] = addmod_u(acc_b[1], rb[1], m.q);
+            acc_a[0] = addmod_u(acc_a[0], ra[0], m.q);
+            acc_a[1] = addmod_u(acc_a[1], ra[1], m.q);
             continue;
         }
         u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
@@ -305,15 +304,15 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         }
         u64 rb[2], ra[2];
         if (beta <= 3) {
-            rb[0] = barrett3(sb[0], m);
-            rb[1] = barrett3(sb[1], m);
-            ra[0] = barrett3(sa[0], m);
-            ra[1] = barrett3(sa[1], m);
+            rb[0] = barrett3_u(sb[0], m);
+            rb[1] = barrett3_u(sb[1], m);
+            ra[0] = barrett3_u(sa[0], m);
+            ra[1] = barrett3_u(sa[1], m);
         } else {
-            rb[0] = barrett128(sb[0], m);
-            rb[1] = barrett128(sb[1], m);
-            ra[0] = barrett128(sa[0], m);
-            ra[1] = barrett128(sa[1], m);
+            rb[0] = barrett128_u(sb[0], m);
+            rb[1] = barrett128_u(sb[1], m);
+            ra[0] = barrett128_u(sa[0], m);
+            ra[1] = barrett128_u(sa[1], m);
         }
         if (j < nq && T.b != nullptr) {
             ulonglong2 bv = *(const ulonglong2 *)(T.b + (size_t)j * N + base);
@@ -323,11 +322,11 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                 bv.y = tmp;
             }
             if (!b_premultiplied) {
-                bv.x = mul_shoup(bv.x, pmod.c[j].w, pmod.c[j].ws, m.q);
-                bv.y = mul_shoup(bv.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+                bv.x = mul_shoup_u(bv.x, pmod.c[j].w, pmod.c[j].ws, m.q);
+                bv.y = mul_shoup_u(bv.y, pmod.c[j].w, pmod.c[j].ws, m.q);
             }
-            rb[0] = addmod(rb[0], bv.x, m.q);
-            rb[1] = addmod(rb[1], bv.y, m.q);
+            rb[0] = addmod_u(rb[0], bv.x, m.q);
+            rb[1] = addmod_u(rb[1], bv.y, m.q);
         }
         if (keyless) {   // the a-polynomial enters as it is (times P): no key product above (j < nq here)
             ulonglong2 av = *(const ulonglong2 *)(T.ext + (size_t)j * N + base);
@@ -336,8 +335,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
                 av.x = av.y;
                 av.y = tmp;
             }
-            av.x = mul_shoup(av.x, pmod.c[j].w, pmod.c[j].ws, m.q);   // never premultiplied, whatever b is
-            av.y = mul_shoup(av.y, pmod.c[j].w, pmod.c[j].ws, m.q);
+            av.x = mul_shoup_u(av.x, pmod.c[j].w, pmod.c[j].ws, m.q);   // never premultiplied, whatever b is
+            av.y = mul_shoup_u(av.y, pmod.c[j].w, pmod.c[j].ws, m.q);
             ra[0] = av.x;
             ra[1] = av.y;
         }
@@ -346,8 +345,8 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             if (T.pt != nullptr) {
                 const ulonglong2 pv = load_rotated2(T.pt, T.pt_galois, j, n, logN);
                 if (T.mask != nullptr) {
-                    mk.x = mulmod(mk.x, pv.x, m);
-                    mk.y = mulmod(mk.y, pv.y, m);
+                    mk.x = mulmod_u(mk.x, pv.x, m);
+                    mk.y = mulmod_u(mk.y, pv.y, m);
                 } else {
                     mk = pv;
                 }
@@ -358,23 +357,23 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
             add128(lazy_a[1], mul64wide(ra[1], mk.y));
             if (++pending == 4) {
                 for (int i = 0; i < 2; i++) {
-                    acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
-                    acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
+                    acc_b[i] = addmod_u(acc_b[i], barrett128_u(lazy_b[i], m), m.q);
+                    acc_a[i] = addmod_u(acc_a[i], barrett128_u(lazy_a[i], m), m.q);
                     lazy_b[i].lo = lazy_b[i].hi = lazy_a[i].lo = lazy_a[i].hi = 0;
                 }
                 pending = 0;
             }
         } else {
             for (int i = 0; i < 2; i++) {
-                acc_b[i] = addmod(acc_b[i], rb[i], m.q);
-                acc_a[i] = addmod(acc_a[i], ra[i], m.q);
+                acc_b[i] = addmod_u(acc_b[i], rb[i], m.q);
+                acc_a[i] = addmod_u(acc_a[i], ra[i], m.q);
             }
         }
     }
     if (pending) {
         for (int i = 0; i < 2; i++) {
-            acc_b[i] = addmod(acc_b[i], barrett128(lazy_b[i], m), m.q);
-            acc_a[i] = addmod(acc_a[i], barrett128(lazy_a[i], m), m.q);
+            acc_b[i] = addmod_u(acc_b[i], barrett128_u(lazy_b[i], m), m.q);
+            acc_a[i] = addmod_u(acc_a[i], barrett128_u(lazy_a[i], m), m.q);
         }
     }
     out_b[0] = acc_b[0];

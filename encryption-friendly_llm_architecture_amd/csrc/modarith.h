@@ -153,4 +153,46 @@ __device__ __forceinline__ u64 addmod(u64 a, u64 b, u64 q) {
     return s >= q ? s - q : s;
 }
 __device__ __forceinline__ u64 submod(u64 a, u64 b, u64 q) { return a >= b ? a - b : a + q - b; }
+
+// ---- the same reductions for a modulus that is uniform over the wavefront (the prime of a workgroup's limb) ----------
+// A 64-bit subtraction is a borrow chain of two instructions with a wait state between them on gfx950, an addition is one
+// instruction: a value is reduced by ADDING 2^64 - m, kept in scalar registers where the compiler cannot see through it
+// and turn the sum back into a subtraction, and selecting.  Same values as the forms above.
+__device__ __forceinline__ u64 neg_uniform(u64 m) {
+    u64 n = 0 - m;
+    asm("" : "+s"(n));
+    return n;
+}
+// u >= m ? u - m : u
+__device__ __forceinline__ u64 cond_sub_u(u64 u, const u64 m) {
+    u64 t = u + neg_uniform(m);
+    asm("" : "+v"(t));
+    return u >= m ? t : u;
+}
+__device__ __forceinline__ u64 mul_shoup_lazy_u(u64 x, u64 w, u64 ws, u64 q) {
+    return x * w + __umul64hi(x, ws) * neg_uniform(q);
+}
+__device__ __forceinline__ u64 mul_shoup_u(u64 x, u64 w, u64 ws, u64 q) {
+    return cond_sub_u(mul_shoup_lazy_u(x, w, ws, q), q);
+}
+__device__ __forceinline__ u64 barrett128_u(u128_t t, const ModQ &m) {
+    const u32 k = m.k;
+    const u64 t1 = (t.hi << (65 - k)) | (t.lo >> (k - 1));
+    const u128_t p = mul64wide(t1, m.mu);
+    const u64 qhat = (p.hi << (63 - k)) | (p.lo >> (k + 1));
+    const u64 q = m.q;
+    const u64 r = t.lo + qhat * neg_uniform(q);
+    return cond_sub_u(cond_sub_u(cond_sub_u(r, 4 * q), 2 * q), q);
+}
+__device__ __forceinline__ u64 barrett_tight_u(u128_t t, const ModQ &m) {
+    const u32 k = m.k;
+    const u64 t1 = (t.hi << (66 - k)) | (t.lo >> (k - 2));
+    const u64 qhat = __umul64hi(t1, m.mu3) >> (k - 59);
+    return cond_sub_u(t.lo + qhat * neg_uniform(m.q), m.q);
+}
+__device__ __forceinline__ u64 barrett3_u(u128_t t, const ModQ &m) {
+    return m.mu3 != 0 ? barrett_tight_u(t, m) : barrett128_u(t, m);
+}
+__device__ __forceinline__ u64 mulmod_u(u64 a, u64 b, const ModQ &m) { return barrett3_u(mul64wide(a, b), m); }
+__device__ __forceinline__ u64 addmod_u(u64 a, u64 b, u64 q) { return cond_sub_u(a + b, q); }
 __device__ __forceinline__ u64 negmod(u64 a, u64 q) { return a ? q - a : 0; }
