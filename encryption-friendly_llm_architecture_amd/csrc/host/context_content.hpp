@@ -28,7 +28,7 @@ struct ContextContent {
     std::mutex mu;
     size_t pool_bytes = 0;
     hipStream_t side = nullptr;
-    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr, ev_main = nullptr, ev_side = nullptr;
     bool side_open = false;
     // the stream the host layer queues on: the device context's (hemm_context_set_stream), by default the legacy
     // default stream; on(s) resolves a stream argument whose null value means that stream
@@ -47,12 +47,31 @@ struct ContextContent {
             ok(hipStreamCreateWithFlags(&side, hipStreamNonBlocking), "hipStreamCreateWithFlags");
             ok(hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming), "hipEventCreateWithFlags");
             ok(hipEventCreateWithFlags(&ev_join, hipEventDisableTiming), "hipEventCreateWithFlags");
+            ok(hipEventCreateWithFlags(&ev_main, hipEventDisableTiming), "hipEventCreateWithFlags");
+            ok(hipEventCreateWithFlags(&ev_side, hipEventDisableTiming), "hipEventCreateWithFlags");
         }
         ok(hipEventRecord(ev_fork, stream()), "hipEventRecord");
         ok(hipStreamWaitEvent(side, ev_fork, 0), "hipStreamWaitEvent");
         std::lock_guard<std::mutex> lk(mu);
         side_open = true;
         return side;
+    }
+    // While a side chain is open, the two streams can also wait for each other half way without closing it:
+    // sideWaitsForMain() orders what the side stream is given next after everything queued on the default stream so
+    // far; markSide() notes the side stream's position and waitSideMark() makes the default stream wait for the last
+    // such note (work queued on the side stream after the note is not waited for).
+    void sideWaitsForMain() {
+        if (!side_open) throw RuntimeException("no side chain open");
+        (void)hipEventRecord(ev_main, stream());
+        (void)hipStreamWaitEvent(side, ev_main, 0);
+    }
+    void markSide() {
+        if (!side_open) throw RuntimeException("no side chain open");
+        (void)hipEventRecord(ev_side, side);
+    }
+    void waitSideMark() {
+        if (!side_open) throw RuntimeException("no side chain open");
+        (void)hipStreamWaitEvent(stream(), ev_side, 0);
     }
     void joinSide() {
         if (!side_open) return;
@@ -120,6 +139,8 @@ struct ContextContent {
         if (side) (void)hipStreamDestroy(side);
         if (ev_fork) (void)hipEventDestroy(ev_fork);
         if (ev_join) (void)hipEventDestroy(ev_join);
+        if (ev_main) (void)hipEventDestroy(ev_main);
+        if (ev_side) (void)hipEventDestroy(ev_side);
         if (dev) hemm_context_destroy(dev);
     }
 };

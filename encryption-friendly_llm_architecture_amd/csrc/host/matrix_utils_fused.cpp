@@ -839,7 +839,7 @@ namespace {
 void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, Ciphertext &acc,
                       std::vector<Plaintext> &cm, i64 n, i64 units, i64 cu, i64 w, u64 batch, DeviceBuffer *U_out,
                       i64 *g_out, u64 spread_block = 0, bool u_ready = false, hipStream_t b_stream = nullptr,
-                      const u64 *low_a = nullptr) {
+                      bool unshifted_last = false) {
     const Context &c = eval.getContext();
     const u64 nq = T + 3, N = c->N, K = c->nP, E = nq + K, lo = nq - 1;
     const i64 ru = cu * w;
@@ -886,21 +886,6 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
     std::vector<Shift> sa;
     for (i64 i = 1; i < units; i++)
         sa.push_back(Shift{cu * i - g * (i / g) * ru, &cm[(size_t)(2 * cu * i + 1)], &cm[(size_t)(2 * cu * i)]});
-    c->joinSide();
-    c->mark("rotation sources and baby rotations");
-    // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
-    // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
-    const u64 pw = lo * N, us = (u64)n_giant * pw;
-    if (low_a != nullptr) {   // the i = 0 term, sigma(A) lowered to T+1 times tau(B), now that both chains have joined
-        U_out->resize(c, 3 * us);
-        ck(hemm_tensor_batch_strided(c->dev, low_a, tau_b, 1, (uint32_t)lo, U_out->data(), us, 0, nullptr));
-    } else if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
-        U_out->resize(c, 3 * us);
-        for (u64 p = 0; p < 3; p++)
-            (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, c->stream());
-    }
-    std::vector<bool> started((size_t)n_giant, false);
-    started[0] = true;
     const size_t G = std::max<u64>(1, std::min<u64>(2 * batch, (u64)std::max<i64>(1, units - 1)));
     // Chains of G shifts.  When the shifts split into exactly two chains, they are cut on a giant-step boundary (so
     // that they accumulate into different partial sums) and the second runs on the side stream beside the first, with
@@ -920,7 +905,33 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
             two_streams = true;
         }
     }
-    DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl), ya2, t12, ws2;
+    // The operands have come their own ways and the shifts run as two chains: the streams do not meet here.  The first
+    // chain's sums (which need only the sources of sigma(A)) follow them on the context's stream and wait for the baby
+    // rotations just before their products with them; the second chain follows the baby rotations on the side stream
+    // once the sources of sigma(A) are there.  The large launches of a chain so fill the gaps of the other operand's
+    // chain of small ones.
+    const bool no_meeting = b_stream != nullptr && two_streams && unshifted_last;
+    if (no_meeting) {
+        c->markSide();
+        c->sideWaitsForMain();
+    } else {
+        c->joinSide();
+    }
+    c->mark("rotation sources and baby rotations");
+    // U, polynomial-major: polynomial p of U_i2 at (p * n_giant + i2) * lo * N, so that one ModUp batch later
+    // covers d1 and d2 of all of them.  U_0 starts from `acc`, which holds the i = 0 term.
+    const u64 pw = lo * N, us = (u64)n_giant * pw;
+    if (unshifted_last) {     // the i = 0 term joins U_0 behind the first chain of shifts
+        U_out->resize(c, 3 * us);
+    } else if (!u_ready) {   // otherwise the caller has put the i = 0 term where U_0 lives
+        U_out->resize(c, 3 * us);
+        for (u64 p = 0; p < 3; p++)
+            (void)hipMemcpyAsync(U_out->data() + p * us, acc.buf_.data() + p * pw, pw * 8, hipMemcpyDeviceToDevice, c->stream());
+    }
+    std::vector<bool> started((size_t)n_giant, false);
+    started[0] = !unshifted_last;
+    DeviceBuffer ya(c, G * 2 * E * N), t1(c, G * ctl), ws(c, G * ctl), ya2, t12, ws2, low_a;
+    if (unshifted_last) low_a = DeviceBuffer(c, ctl);
     if (two_streams) {
         ya2 = DeviceBuffer(c, G * 2 * E * N);
         t12 = DeviceBuffer(c, G * ctl);
@@ -961,7 +972,7 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         flush();
     };
     // forked before the first chain is queued: the side stream waits only for what both chains depend on
-    const hipStream_t side2 = two_streams ? c->forkSide() : nullptr;
+    const hipStream_t side2 = !two_streams ? nullptr : no_meeting ? b_stream : c->forkSide();
     for (size_t ch = 0; ch < chains.size(); ch++) {
         const size_t first = chains[ch].first, cnt = chains[ch].second;
         const bool on_side = two_streams && ch == 1;
@@ -973,7 +984,17 @@ void bsgsShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const
         pushShifts(eval, xa, 0, xa2, 0, sa, first, cnt, terms, off);
         ck(hemm_hoisted_moddown(c->dev, terms.data(), off.data(), (uint32_t)cnt, (uint32_t)nq, 1, 1, yap, t1p, lo * N,
                                 wsp, st));
+        if (no_meeting && !on_side) c->waitSideMark();
         accumulate(first, cnt, t1p, st);
+    }
+    if (unshifted_last) {
+        // sigma(A) lowered to T+1 times tau(B), on the context's stream behind the chain that owns U_0: lowering it in
+        // front of the rotation sources would lengthen the chain of small launches that the main loop waits for, here
+        // it runs beside the second chain (sums of residues do not depend on their order).  The lowering is the only
+        // call that works in the context's scratch region while the side chain is open.
+        levelDownOneBatch(c, sigma_a, 2, T + 2, low_a.data());
+        ck(hemm_tensor_batch_strided(c->dev, low_a.data(), tau_b, 1, (uint32_t)lo, U_out->data(), us,
+                                     started[0] ? 1 : 0, nullptr));
     }
     if (two_streams) c->joinSide();
     *g_out = g;
@@ -1094,8 +1115,9 @@ class OwnWays {
 
 // What follows the two chains: the baby rotations of tau(B) (level T+1) go on where it was made, on the side stream,
 // while the rotation sources of sigma(A) (level T+2) are made on the context's; the chains meet in front of the main
-// loop, where the unshifted term low_a (x) tau(B) is taken.  Complex-packed cells: k / 2 shifts of two columns / rows.
-CtxtTensor ownWaysShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b, const u64 *low_a,
+// loop; the unshifted term, sigma(A) lowered to T+1 times tau(B), is taken behind the loop's first chain.
+// Complex-packed cells: k / 2 shifts of two columns / rows.
+CtxtTensor ownWaysShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma_a, const u64 *tau_b,
                                std::vector<Plaintext> &cm, i64 rows, i64 cols, i64 k, i64 w, u64 batch, bool spread,
                                hipStream_t side, bool add_conj) {
     const Context &c = eval.getContext();
@@ -1105,7 +1127,7 @@ CtxtTensor ownWaysShiftProduct(const HomEvaluator &eval, u64 T, const u64 *sigma
     CtxtTensor res(c, rows, cols, w);
     i64 g = 1;
     bsgsShiftProduct(eval, T, sigma_a, tau_b, acc, cm, k, k / 2, 2, w, batch, &U, &g, spread ? (u64)(k * w) : 0, false,
-                     side, low_a);
+                     side, true);
     c->mark("main loop");
     bsgsGiantSteps(eval, T, U, g, (k / 2) / g, 2 * w, acc, res, add_conj);
     c->mark("giant steps");
@@ -1328,11 +1350,9 @@ CtxtTensor multPackedMatMatFused(const HomEvaluator &eval, const Bootstrapper &b
             const Ciphertext tb = tr.lowerAndTransformFused(eval, op2.get(), MaskKind::PackedVertical, shape_b, T + 1);
             ways.toOwn();
             const Ciphertext sa = tr.lowerAndTransformFused(eval, op1.get(), MaskKind::PackedHorizontal, shape_a, T + 2);
-            DeviceBuffer low_a(c, 2 * lo * N);
-            levelDownOneBatch(c, sa.buf_.data(), 2, T + 2, low_a.data());
             ways.marksOn();
             c->mark("transforms");
-            return ownWaysShiftProduct(eval, T, sa.buf_.data(), tb.buf_.data(), low_a.data(), cm, rows, cols, k, w, batch,
+            return ownWaysShiftProduct(eval, T, sa.buf_.data(), tb.buf_.data(), cm, rows, cols, k, w, batch,
                                        spread, ways.side(), false);
         }
     }
@@ -1538,7 +1558,7 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
             const u64 N = c->N, lo = T + 2;
             const TileTensorShape shape_a(rows, k, w), shape_b(k, cols, w);
             std::vector<Plaintext> &cm = tr.getColMaskExt(eval, shape_a, T + 2);
-            DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N), low_a(c, 2 * lo * N);
+            DeviceBuffer sa(c, 2 * (T + 3) * N), tb(c, 2 * lo * N);
             const std::vector<u64> one(T + 6, 1);
             // the first L + 1 limbs of both polynomials of x, back to back
             auto truncated = [&](const Ciphertext &x, u64 L) {
@@ -1586,11 +1606,9 @@ CtxtTensor multMatMatComplexPackedFused(const HomEvaluator &eval, const Bootstra
                 const MaskKind kind = MaskKind::PackingHorizontal;
                 tr.diagonalTransformBatch(eval, a.get().buf_.data(), 1, T + 3, &kind, &shape_a, sa.data());
             }
-            // (the only call that works in the context's scratch region while the side chain is open)
-            levelDownOneBatch(c, sa.data(), 2, T + 2, low_a.data());
             ways.marksOn();
             c->mark("packing and transforms of A");
-            return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), low_a.data(), cm, rows, cols, k, w, batch, spread,
+            return ownWaysShiftProduct(eval, T, sa.data(), tb.data(), cm, rows, cols, k, w, batch, spread,
                                        ways.side(), add_conj);
         }
     }
