@@ -332,9 +332,17 @@ int hemm_rotate(hemm_context *ctx, const uint64_t *ct, size_t ct_stride, const u
     need((galois & 1) && galois < 2 * (uint64_t)ctx->N, "galois element must be odd and < 2N");
     const size_t N = ctx->N;
     u64 *rot = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
-    launch_galois(ctx, (const u64 *)ct, ct_stride, rot, (size_t)nq * N, galois, (int)nq, 2, on_stream(ctx, stream));
-    launch_keyswitch(ctx, rot + (size_t)nq * N, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, rot,
-                     on_stream(ctx, stream));
+    const hipStream_t s = on_stream(ctx, stream);
+    if (modup_through_automorphism_ok(ctx, (int)nq)) {
+        // No launch that rotates: the ModUp reads the second polynomial through the automorphism (first inverse pass
+        // and the copies of the digits' own limbs) and the key product reads the first one through it -- the same
+        // residues as rotating both first.
+        launch_keyswitch(ctx, (const u64 *)ct + ct_stride, (const u64 *)evk, (int)nq, (u64 *)out, out_stride,
+                         (const u64 *)ct, s, (u32)galois, true);
+    } else {
+        launch_galois(ctx, (const u64 *)ct, ct_stride, rot, (size_t)nq * N, galois, (int)nq, 2, s);
+        launch_keyswitch(ctx, rot + (size_t)nq * N, (const u64 *)evk, (int)nq, (u64 *)out, out_stride, rot, s);
+    }
     check_launch();
     HEMM_CATCH
 }

@@ -68,6 +68,13 @@ struct __align__(16) Cst {
     u64 w, ws;
 };
 
+// NTT-domain index of the automorphism X -> X^g: out[k] = in[galois_index(k)]
+__device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
+    const u32 br = __brev(k) >> (32 - logN);
+    const u32 e = ((2 * br + 1) * g) & ((2u << logN) - 1);
+    return __brev(e >> 1) >> (32 - logN);
+}
+
 void hemm_set_error(const std::string &msg);
 
 #define HEMM_HIP(call)                                                                       \
@@ -111,6 +118,7 @@ struct ConvSources {
     const u64 *copy_src;
     size_t copy_src_stride;
     int n_copy;
+    u32 copy_galois;            // != 0: the copies read their source through this automorphism (N = 2^16)
     uint8_t copy_src_slot[HEMM_MAX_PRIMES], copy_dst_slot[HEMM_MAX_PRIMES];
 };
 // data: [n_polys][.][N] (polynomial stride poly_stride), limb l written to slot sl[l].  With ep_* set the second pass
@@ -129,9 +137,11 @@ bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const u
                          int n_polys, u64 *out, size_t out_stride, const void *cst_dev, hipStream_t s);
 // inverse transform reading src (same slot numbering as data, polynomial stride src_poly_stride) and leaving the
 // coefficients in data; false when this ring size has no out-of-place form (the caller copies, then transforms)
+// galois != 0: src is read through that automorphism (the transform of the rotated polynomial, without a launch
+// that rotates it first)
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
                       const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s,
-                      const void *final_scale = nullptr);
+                      const void *final_scale = nullptr, u32 galois = 0);
 void launch_ntt(const hemm_context *c, u64 *data, const LimbList &ll, int n_limbs, int n_polys,
                 size_t poly_stride, bool inverse, hipStream_t s);
 void launch_binary(const hemm_context *c, int op, const u64 *a, size_t a_stride, const u64 *b, size_t b_stride,
@@ -161,12 +171,16 @@ void launch_inner_product(hemm_context *c, const u64 *in, const u64 *ext, const 
                           hipStream_t s);
 void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, size_t out_stride, const u64 *add,
                     size_t add_stride, int add_polys, u64 *conv, hipStream_t s);
+// galois != 0 (N = 2^16): the key switch of the automorphism of `in`, which is read through it where the ModUp reads
+// it; b_rotates: add_b is read through the same automorphism where the key product adds it
 void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
-                      const u64 *add_b, hipStream_t s);
+                      const u64 *add_b, hipStream_t s, u32 galois = 0, bool b_rotates = false);
 void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
                     int n_polys, hipStream_t s);
 void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
-                        hipStream_t s);
+                        hipStream_t s, u32 galois = 0);
+// whether launch_modup_batch at this level takes a non-zero `galois` (its input read through that automorphism)
+bool modup_through_automorphism_ok(const hemm_context *c, int nq);
 // terms_host / n_terms: the host copy of the list (only read for the byte accounting; may be nullptr)
 // compact: every term's key is in the compact layout (all terms of a launch use the same layout)
 void launch_hoisted_terms(hemm_context *c, const void *terms_dev, const u32 *group_off_dev, int n_out, int nq, u64 *y,

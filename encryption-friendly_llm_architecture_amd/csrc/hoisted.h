@@ -8,13 +8,6 @@ struct CstList {
     Cst c[HEMM_MAX_PRIMES];
 };
 
-// NTT-domain index of the automorphism X -> X^g: out[k] = in[galois_index(k)]
-__device__ __forceinline__ u32 galois_index(u32 k, u32 g, int logN) {
-    const u32 br = __brev(k) >> (32 - logN);
-    const u32 e = ((2 * br + 1) * g) & ((2u << logN) - 1);
-    return __brev(e >> 1) >> (32 - logN);
-}
-
 struct RotTermDev {
     const u64 *ext;   // [beta][E][N] extended digits of the source a-polynomial
     const u64 *b;     // [nq][N] b-polynomial of the source (nullptr: none, single-source terms only)
@@ -30,9 +23,12 @@ struct RotTermDev {
     // optional plaintext factor [E][N] of the whole term, read through its own automorphism (nullptr: none)
     const u64 *pt;
     u32 pt_galois;
-    u32 flags;        // bit 0: evk is a compact key (see key_limb)
+    u32 flags;        // bit 0: evk is a compact key (see key_limb); bit 1 (single-source terms with a plain key only): ext
+                      // already holds the digits of the rotated polynomial and is read as it is, only b is read through
+                      // the automorphism
 };
 #define ROT_TERM_COMPACT_KEY 1u
+#define ROT_TERM_EXT_ROTATED 2u
 
 // Accesses to data that is touched once per launch (keys, masks, results): marked non-temporal so they do
 // not push the rotation sources, which every output gathers from, out of the L2.
@@ -288,9 +284,10 @@ __device__ __forceinline__ void hoisted_pair_int(const RotTermDev *__restrict__ 
         }
         u128_t sb[2] = {{0, 0}, {0, 0}}, sa[2] = {{0, 0}, {0, 0}};
         const bool keyless = T.evk == nullptr;
+        const bool ext_as_is = !COMPACT && (T.flags & ROT_TERM_EXT_ROTATED) != 0;
         for (int d = 0; d < (keyless ? 0 : beta); d++) {
-            ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + base);
-            if (swap) {
+            ulonglong2 x = *(const ulonglong2 *)(T.ext + ((size_t)d * E + j) * N + (ext_as_is ? n : base));
+            if (swap && !ext_as_is) {
                 const u64 tmp = x.x;
                 x.x = x.y;
                 x.y = tmp;
@@ -468,8 +465,9 @@ __device__ __forceinline__ void hoisted_pair_fp(const RotTermDev *__restrict__ t
             }
         } else {
             const bool keyless = T.evk == nullptr;
+            const bool ext_as_is = !COMPACT && (T.flags & ROT_TERM_EXT_ROTATED) != 0;
             for (int d = 0; d < (keyless ? 0 : beta); d++) {
-                const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + base, swap);
+                const D2 x = gather_d2(T.ext + ((size_t)d * E + j) * N + (ext_as_is ? n : base), swap && !ext_as_is);
                 const D2 kb = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 0, prime, logN, n_full), n);
                 const D2 ka = key_pair_fp<COMPACT>(kr, key_limb<COMPACT>(koff, d, 1, prime, logN, n_full), n);
                 sb0 += f.mul(x.x, kb.x);

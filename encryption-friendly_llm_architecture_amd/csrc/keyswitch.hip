@@ -865,7 +865,7 @@ void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, si
 // Full key switch of `in` ([nq][N], NTT) with `evk` ([dnum][2][nQ+K][N]):
 // out[0] = ks_b (+ add_b), out[1] = ks_a; out poly stride out_stride.
 void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
-                      const u64 *add_b, hipStream_t s) {
+                      const u64 *add_b, hipStream_t s, u32 galois, bool b_rotates) {
     if (c->nP < 1) throw std::invalid_argument("key switching needs special primes");
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     const size_t N = c->N;
@@ -873,7 +873,8 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
     u64 *coef = sc;                              // [nq][N]   (reused as conv[2][nq] needs 2*nq)
     u64 *ext = coef + (size_t)2 * (c->nQ) * N;   // [beta][E][N]
     u64 *acc = ext + (size_t)beta * E * N;       // [2][E][N]
-    launch_modup_batch(c, in, (size_t)nq * N, nq, 1, ext, coef, s);   // same arithmetic as launch_modup, 5 launches
+    launch_modup_batch(c, in, (size_t)nq * N, nq, 1, ext, coef, s, galois);   // same arithmetic as launch_modup
+    if (b_rotates && (galois == 0 || N < 512)) throw std::invalid_argument("add_b rotates only with the key switch's input");
     if (N >= 512) {
         // the key product as a hoisted sum of one term under the identity automorphism: P * add_b joins the sum in
         // the extended basis, so the ModDown needs no addend and ends in the forward transform's fused tail
@@ -885,6 +886,10 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
         term.evk = evk;
         term.galois = 1;
         term.pt_galois = 1;
+        if (galois != 0 && b_rotates) {   // ext holds the rotated digits already: only add_b goes through the automorphism
+            term.galois = galois;
+            term.flags = ROT_TERM_EXT_ROTATED;
+        }
         const u32 off[2] = {0, 1};
         launch_hoisted_terms_args(c, &term, 1, off, 1, nq, acc, false, s);
         launch_moddown_batch(c, acc, nq, 2, 0, out, out_stride, coef, s);
@@ -1061,8 +1066,16 @@ void launch_key_expand(const hemm_context *c, const u64 *compact, u64 *evk, hipS
 // ---- batched / hoisted forms ---------------------------------------------------------------------
 // in: [n_in][.][N] (polynomial stride in_stride, first nq limbs used) -> ext [n_in][beta][nq+K][N], own
 // limbs of every digit filled.  coef: workspace [n_in][nq][N].
+// The form of launch_modup_batch in which the conversions of all digits and the copies of their own limbs are one
+// launch (the first pass of the forward transform) is the one that can read its input through an automorphism.
+bool modup_through_automorphism_ok(const hemm_context *c, int nq) {
+    const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
+    return c->logN == 16 && alpha <= 8 && alpha <= CONV_MAX_SOURCES && beta <= BCONV_MAX_DIGITS &&
+           beta <= CONV_MAX_DIGITS && beta * E <= 255 && beta * E - nq <= HEMM_MAX_PRIMES && lazy_dot_ok(c);
+}
+
 void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,
-                        hipStream_t s) {
+                        hipStream_t s, u32 galois) {
     KsTables *t = g_tables_of(c);
     const int K = c->nP, E = nq + K, alpha = c->alpha, beta = (nq + alpha - 1) / alpha;
     const size_t N = c->N;
@@ -1071,8 +1084,10 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
     LimbList ident;
     for (int j = 0; j < HEMM_MAX_PRIMES; j++) ident.idx[j] = (uint8_t)j;
     const bool fold = c->logN == 16;
+    if (galois != 0 && !modup_through_automorphism_ok(c, nq))
+        throw std::invalid_argument("this ModUp shape has no form that reads its input through an automorphism");
     if (!launch_intt_from(c, in, in_stride, coef, chain, ident, nq, n_in, (size_t)nq * N, s,
-                          fold ? t->dev + t->modup_invn_off[nq] : nullptr)) {
+                          fold ? t->dev + t->modup_invn_off[nq] : nullptr, galois)) {
         HEMM_HIP(hipMemcpy2DAsync(coef, (size_t)nq * N * 8, in, in_stride * 8, (size_t)nq * N * 8, n_in,
                                   hipMemcpyDeviceToDevice, s));
         launch_ntt(c, coef, chain, nq, n_in, (size_t)nq * N, true, s);
@@ -1157,12 +1172,14 @@ void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq
         cs.copy_src = in;
         cs.copy_src_stride = in_stride;
         cs.n_copy = nq;
+        cs.copy_galois = galois;
         for (int j = 0; j < nq; j++) {
             cs.copy_src_slot[j] = (uint8_t)j;
             cs.copy_dst_slot[j] = (uint8_t)((j / alpha) * E + j);
         }
         if (launch_ntt_converted(c, cs, ext, jp, js, n_joint, n_in, (size_t)beta * E * N, s)) return;
     }
+    if (galois != 0) throw std::invalid_argument("this ModUp shape has no form that reads through an automorphism");
     g.d[0].split = bconv_split((int)N, n_in * beta, E - alpha);
     const dim3 grid((unsigned)(N / 512), n_in * g.d[0].split, beta), block(256);
     const int widest = std::min(nq, alpha);

@@ -511,8 +511,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         u64 *base = data + (size_t)poly * poly_stride + ((size_t)cs.copy_dst_slot[limb - n_limbs] << 16) + col;
         const int rh = threadIdx.x >> 4;
         u64 t[16];
+        if (cs.copy_galois != 0) {   // the copy of the source's automorphism
+            const u64 *fl = from - col;
 #pragma unroll
-        for (int k = 0; k < 16; k++) t[k] = from[(size_t)(rh + 16 * k) << 8];
+            for (int k = 0; k < 16; k++)
+                t[k] = fl[galois_index(((u32)(rh + 16 * k) << 8) + (u32)col, cs.copy_galois, 16)];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) t[k] = from[(size_t)(rh + 16 * k) << 8];
+        }
 #pragma unroll
         for (int k = 0; k < 16; k++) base[(size_t)(rh + 16 * k) << 8] = t[k];
         return;
@@ -708,16 +715,19 @@ struct NttEpilogue {
     u64 *out;
     const Tw *cst;  // per limb: constant and Shoup quotient
     size_t minuend_stride, out_stride;
+    u32 galois;     // inverse transforms that read their input elsewhere: != 0 reads it through this automorphism
 };
 // An inverse transform may read its input elsewhere (same slot numbering, own polynomial stride) and leave the
 // result in `data`: the first pass then loads from `minuend` (stride `minuend_stride`) instead of `data`.
 
 // forward pass 2 / inverse pass 1 work on 16 whole rows (16 x 256 contiguous residues).
-template <bool INV, bool EPI, class F>
+// GAL (inverse only): ld is the base of the source limb and residue k of the input is ld[galois_index(k)] -- an aligned
+// group of 16 residues stays an aligned group under the automorphism, so the loads touch the same number of lines
+template <bool INV, bool EPI, bool GAL, class F>
 __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__restrict__ tw_int,
                                           const Tw *__restrict__ rtw_int, const F f, u64 *lds_raw, const u32 r, const u64 q,
                                           const u64 *__restrict__ mn, u64 *__restrict__ o, const Tw cst,
-                                          const u64 *__restrict__ ld) {
+                                          const u64 *__restrict__ ld, const u32 gal = 0) {
     typedef typename F::E E;
     const typename F::W *tw = (const typename F::W *)tw_int;
     const int c = threadIdx.x & 15, rr = threadIdx.x >> 4;
@@ -754,8 +764,13 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
             for (int k = 0; k < 16; k++) row[c + 16 * k] = f.to_canonical(l[padc(c + 16 * k)]);
         }
     } else {
+        if (GAL) {
 #pragma unroll
-        for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = ld[c + 16 * k];
+            for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = ld[galois_index((r << 8) + (u32)(c + 16 * k), gal, 16)];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) lc[padc(c + 16 * k)] = ld[c + 16 * k];
+        }
         wave_sync();
 #pragma unroll
         for (int k = 0; k < 16; k++) x[k] = f.from_canonical(lc[padc(16 * c + k)]);
@@ -774,7 +789,7 @@ __device__ __forceinline__ void rows_body(u64 *__restrict__ row, const Tw *__res
     }
 }
 
-template <bool INV, bool EPI>
+template <bool INV, bool EPI, bool GAL = false>
 __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data, const Tw *__restrict__ tw_all,
                                                          const Tw *__restrict__ rtw_all,
                                                          const ModQ *__restrict__ modq, const double *__restrict__ fp,
@@ -806,13 +821,15 @@ __global__ __launch_bounds__(256) void ntt16_rows_kernel(u64 *__restrict__ data,
     const u64 q = modq[prime].q;
     const u64 *ld = row;
     if (INV && ep.minuend != nullptr)
-        ld = ep.minuend + (size_t)poly * ep.minuend_stride + ((size_t)sl.idx[limb] << 16) + ((size_t)r << 8);
+        ld = ep.minuend + (size_t)poly * ep.minuend_stride + ((size_t)sl.idx[limb] << 16) + (GAL ? 0 : (size_t)r << 8);
+    const u32 gal = GAL ? ep.galois : 0u;
     if (fp[4 * prime] != 0.0)
-        rows_body<INV, EPI>(row, tw, rtw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI, GAL>(row, tw, rtw, FpField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld, gal);
     else if (INV || (q >> 60) != 0)
-        rows_body<INV, EPI>(row, tw, rtw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI, GAL>(row, tw, rtw, IntField(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld, gal);
     else
-        rows_body<INV, EPI>(row, tw, rtw, IntFieldT<true>(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld);
+        rows_body<INV, EPI, GAL>(row, tw, rtw, IntFieldT<true>(modq, nullptr, nullptr, fp, prime), lds, r, q, mn, o, cst, ld,
+                                 gal);
 }
 
 }  // namespace
@@ -974,8 +991,11 @@ bool launch_moddown_slab(const hemm_context *c, u64 *y, size_t y_stride, const u
 
 bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_stride, u64 *data, const LimbList &ll,
                       const LimbList &sl, int n_limbs, int n_polys, size_t poly_stride, hipStream_t s,
-                      const void *final_scale) {
-    if (c->logN != 16) return false;
+                      const void *final_scale, u32 galois) {
+    if (c->logN != 16) {
+        if (galois != 0) throw std::invalid_argument("a transform reads through an automorphism at N = 2^16 only");
+        return false;
+    }
     if (n_limbs <= 0 || n_polys <= 0) return true;
     account(c, TR_NTT, (size_t)2 * n_limbs * n_polys * c->N * 8, 2);
     const Tw *tw = (const Tw *)c->d_iw;
@@ -988,8 +1008,13 @@ bool launch_intt_from(const hemm_context *c, const u64 *src, size_t src_poly_str
         NttEpilogue from{};
         from.minuend = src + (size_t)p0 * src_poly_stride;
         from.minuend_stride = src_poly_stride;
-        hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, d, tw, (const Tw *)c->d_irw,
-                           c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, from);
+        from.galois = galois;
+        if (galois != 0)
+            hipLaunchKernelGGL((ntt16_rows_kernel<true, false, true>), dim3(16 * lanes), block, 0, s, d, tw,
+                               (const Tw *)c->d_irw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, from);
+        else
+            hipLaunchKernelGGL((ntt16_rows_kernel<true, false>), dim3(16 * lanes), block, 0, s, d, tw,
+                               (const Tw *)c->d_irw, c->d_modq, c->d_fp, ll, sl, n_limbs, poly_stride, from);
         hipLaunchKernelGGL(ntt16_cols_kernel<true>, dim3(16, lanes), block, 0, s, d, tw, c->d_modq, c->d_ninv,
                            c->d_ninv_s, c->d_fp, ll, sl, n_limbs, poly_stride, (const Tw *)final_scale);
     }
