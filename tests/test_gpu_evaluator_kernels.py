@@ -190,6 +190,12 @@ def test_rotate_relinearize_rescale(S):
     orc.gen_conj_key(6)
     g = 2 * N - 1
     assert np.array_equal(host(ctx.rotate(dct, dev(orc.keys[("gal", g)]), g, nq)), orc.conjugate(ct).data)
+    # the result may replace the operand: every read of it is queued before the launch that writes the result
+    # (at N = 2^16 no launch copies the rotated polynomials first: the ModUp and the key product read them through
+    # the automorphism)
+    same = dct.clone()
+    ctx.rotate(same, dev(orc.keys[("gal", g)]), g, nq, out=same)
+    assert np.array_equal(host(same), orc.conjugate(ct).data)
     t3 = orc.tensor(ct, ct)
     d3 = ctx.tensor(dct, dct, nq)
     assert np.array_equal(host(d3), t3.data)
