@@ -354,6 +354,14 @@ int hemm_relinearize(hemm_context *ctx, const uint64_t *ct3, size_t ct_stride, c
     LimbList ll = chain_limbs(ctx, nq, 0, &nl);
     need(ct3 && evk && out, "null operand");
     const size_t N = ctx->N;
+    if (N >= 512) {
+        // (d0, d1) joins the key product of d2 in the extended basis as a term without a key: the ModDown leaves the
+        // finished pair, no addition launch (P d + x divided by P is d + x / P exactly)
+        launch_keyswitch(ctx, (const u64 *)ct3 + 2 * ct_stride, (const u64 *)evk, (int)nq, (u64 *)out, out_stride,
+                         (const u64 *)ct3, on_stream(ctx, stream), 0, false, (const u64 *)ct3 + ct_stride);
+        check_launch();
+        return 0;
+    }
     u64 *tmp = hemm_scratch(ctx) + hemm_scratch_words(ctx) - (size_t)2 * ctx->nQ * N;  // [2][nq][N]
     launch_keyswitch(ctx, (const u64 *)ct3 + 2 * ct_stride, (const u64 *)evk, (int)nq, tmp, (size_t)nq * N, nullptr,
                      on_stream(ctx, stream));

@@ -172,9 +172,11 @@ void launch_inner_product(hemm_context *c, const u64 *in, const u64 *ext, const 
 void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, size_t out_stride, const u64 *add,
                     size_t add_stride, int add_polys, u64 *conv, hipStream_t s);
 // galois != 0 (N = 2^16): the key switch of the automorphism of `in`, which is read through it where the ModUp reads
-// it; b_rotates: add_b is read through the same automorphism where the key product adds it
+// it; b_rotates: add_b is read through the same automorphism where the key product adds it; add_a (N >= 512, with
+// add_b): out[1] = ks_a + add_a as well, both addends entering the sum in the extended basis
 void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
-                      const u64 *add_b, hipStream_t s, u32 galois = 0, bool b_rotates = false);
+                      const u64 *add_b, hipStream_t s, u32 galois = 0, bool b_rotates = false,
+                      const u64 *add_a = nullptr);
 void launch_rescale(hemm_context *c, const u64 *in, size_t in_stride, u64 *out, size_t out_stride, int nq,
                     int n_polys, hipStream_t s);
 void launch_modup_batch(hemm_context *c, const u64 *in, size_t in_stride, int nq, int n_in, u64 *ext, u64 *coef,

@@ -865,7 +865,7 @@ void launch_moddown(hemm_context *c, u64 *acc, int nq, int n_polys, u64 *out, si
 // Full key switch of `in` ([nq][N], NTT) with `evk` ([dnum][2][nQ+K][N]):
 // out[0] = ks_b (+ add_b), out[1] = ks_a; out poly stride out_stride.
 void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u64 *out, size_t out_stride,
-                      const u64 *add_b, hipStream_t s, u32 galois, bool b_rotates) {
+                      const u64 *add_b, hipStream_t s, u32 galois, bool b_rotates, const u64 *add_a) {
     if (c->nP < 1) throw std::invalid_argument("key switching needs special primes");
     const int K = c->nP, E = nq + K, beta = (nq + c->alpha - 1) / c->alpha;
     const size_t N = c->N;
@@ -875,23 +875,34 @@ void launch_keyswitch(hemm_context *c, const u64 *in, const u64 *evk, int nq, u6
     u64 *acc = ext + (size_t)beta * E * N;       // [2][E][N]
     launch_modup_batch(c, in, (size_t)nq * N, nq, 1, ext, coef, s, galois);   // same arithmetic as launch_modup
     if (b_rotates && (galois == 0 || N < 512)) throw std::invalid_argument("add_b rotates only with the key switch's input");
+    if (add_a != nullptr && (N < 512 || add_b == nullptr || b_rotates))
+        throw std::invalid_argument("an addend for the second polynomial needs N >= 512 and one for the first");
     if (N >= 512) {
         // the key product as a hoisted sum of one term under the identity automorphism: P * add_b joins the sum in
         // the extended basis, so the ModDown needs no addend and ends in the forward transform's fused tail
         // (identical residues: every step is exact modular arithmetic in the same order)
-        RotTermDev term;
-        memset(&term, 0, sizeof(term));
-        term.ext = ext;
-        term.b = add_b;
-        term.evk = evk;
-        term.galois = 1;
-        term.pt_galois = 1;
+        RotTermDev term[2];
+        memset(term, 0, sizeof(term));
+        term[0].ext = ext;
+        term[0].b = add_b;
+        term[0].evk = evk;
+        term[0].galois = 1;
+        term[0].pt_galois = 1;
         if (galois != 0 && b_rotates) {   // ext holds the rotated digits already: only add_b goes through the automorphism
-            term.galois = galois;
-            term.flags = ROT_TERM_EXT_ROTATED;
+            term[0].galois = galois;
+            term[0].flags = ROT_TERM_EXT_ROTATED;
         }
-        const u32 off[2] = {0, 1};
-        launch_hoisted_terms_args(c, &term, 1, off, 1, nq, acc, false, s);
+        int n_terms = 1;
+        if (add_a != nullptr) {   // (add_b, add_a) as a term without a key: P times both joins the sum on the chain limbs
+            term[0].b = nullptr;
+            term[1].ext = add_a;
+            term[1].b = add_b;
+            term[1].galois = 1;
+            term[1].pt_galois = 1;
+            n_terms = 2;
+        }
+        const u32 off[2] = {0, (u32)n_terms};
+        launch_hoisted_terms_args(c, term, n_terms, off, 1, nq, acc, false, s);
         launch_moddown_batch(c, acc, nq, 2, 0, out, out_stride, coef, s);
         return;
     }
